@@ -1,0 +1,263 @@
+"""ctypes front-end of the CPU oracle (oracle/qlinear_oracle.c).  TEST INFRASTRUCTURE ONLY.
+
+Only tests, the smoke check and the benchmark's cpu_baseline leg may import this module; the shipped
+package never does.  All arrays are numpy, C-contiguous.
+
+Weight blocks are passed in the reference's array-of-structures layout (mllm/core/DataTypes.hpp:110-121,164-170)
+as a uint8 array [N, K/32, 18] (Q4_0) or [N, K/32, 34] (Q8_0); the 2-byte `d` field is an IEEE fp16 bit pattern.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+Q4_0, Q8_0 = 0, 1
+SCALE_IEEE, SCALE_X86_REF = 0, 1
+BLOCK_BYTES = {Q4_0: 18, Q8_0: 34}
+
+_lib = None
+_ref = None
+
+
+def _p(a, t):
+    return a.ctypes.data_as(C.POINTER(t)) if a is not None else None
+
+
+def lib():
+    """Load liboracle.so, building it with the committed Makefile when it is not there yet."""
+    global _lib
+    if _lib is None:
+        so = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(so):
+            subprocess.check_call(["make", "-C", _HERE, "liboracle.so"])
+        L = C.CDLL(so)
+        L.orc_fp16_to_fp32.restype = C.c_float
+        L.orc_fp16_to_fp32.argtypes = [C.c_uint16]
+        L.orc_fp32_to_fp16.restype = C.c_uint16
+        L.orc_fp32_to_fp16.argtypes = [C.c_float]
+        L.orc_bf16_to_fp32.restype = C.c_float
+        L.orc_bf16_to_fp32.argtypes = [C.c_uint16]
+        L.orc_fp32_to_bf16.restype = C.c_uint16
+        L.orc_fp32_to_bf16.argtypes = [C.c_float]
+        L.orc_x86_scale_bits.restype = C.c_uint16
+        L.orc_x86_scale_bits.argtypes = [C.c_uint16]
+        L.orc_vec_dot.restype = C.c_float
+        L.orc_silu.restype = C.c_float
+        L.orc_silu.argtypes = [C.c_float]
+        L.orc_linear_q.restype = C.c_int
+        L.orc_w4a16_gemm.restype = C.c_int
+        L.orc_moe_ffn.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def ref_available():
+    return os.path.exists(os.path.join(_HERE, "_ref", "libmllm_ref.so"))
+
+
+def ref():
+    """The reference's own kernels compiled into oracle/_ref (only where `make -C oracle ref` has been run)."""
+    global _ref
+    if _ref is None:
+        L = C.CDLL(os.path.join(_HERE, "_ref", "libmllm_ref.so"))
+        L.ref_fp32_to_fp16_bits.restype = C.c_uint16
+        L.ref_fp32_to_fp16_bits.argtypes = [C.c_float]
+        L.ref_fp16_bits_to_fp32.restype = C.c_float
+        L.ref_fp16_bits_to_fp32.argtypes = [C.c_uint16]
+        L.ref_scale_store_load.restype = C.c_float
+        L.ref_scale_store_load.argtypes = [C.c_uint16]
+        _ref = L
+    return _ref
+
+
+# ----------------------------------------------------------------------------- scalar helpers (vectorised in numpy)
+def fp16_bits_to_fp32(bits):
+    return np.asarray(bits, dtype=np.uint16).view(np.float16).astype(np.float32)
+
+
+def x86_scale_bits(bits):
+    f = np.vectorize(lambda b: lib().orc_x86_scale_bits(int(b)), otypes=[np.uint16])
+    return f(np.asarray(bits, dtype=np.uint16))
+
+
+def bf16_bits_to_fp32(bits):
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
+def fp32_to_bf16_bits(x):
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    r = (u + 0x7FFF + ((u >> 16) & 1)) >> 16
+    return r.astype(np.uint16)
+
+
+# ----------------------------------------------------------------------------- Q8_0 activation quantisation
+def quantize_rows_q8_0(x):
+    """x fp32 [M, K] -> (codes int8 [M, K], scale bit patterns uint16 [M, K/32])."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    M, K = x.shape
+    qs = np.empty((M, K), np.int8)
+    d = np.empty((M, K // 32), np.uint16)
+    for m in range(M):
+        lib().orc_quantize_row_q8_0(_p(x[m], C.c_float), _p(qs[m], C.c_int8), _p(d[m], C.c_uint16), C.c_int(K))
+    return qs, d
+
+
+def dequantize(W, wtype, scale_mode=SCALE_IEEE):
+    """W uint8 [N, K/32, blk] -> fp32 [N, K]."""
+    W = np.ascontiguousarray(W, dtype=np.uint8)
+    N, nb, _ = W.shape
+    y = np.empty((N, nb * 32), np.float32)
+    for n in range(N):
+        lib().orc_dequantize_row(_p(W[n], C.c_uint8), C.c_int(wtype), _p(y[n], C.c_float), C.c_int(nb * 32),
+                                 C.c_int(scale_mode))
+    return y
+
+
+def block_isums(W, wtype, xq):
+    """exact int32 block dot products [N, M, K/32]."""
+    W = np.ascontiguousarray(W, dtype=np.uint8)
+    xq = np.ascontiguousarray(xq, dtype=np.int8)
+    N, nb, _ = W.shape
+    M = xq.shape[0]
+    out = np.empty((N, M, nb), np.int32)
+    lib().orc_block_isums(_p(W, C.c_uint8), C.c_int(wtype), _p(xq, C.c_int8), C.c_int(M), C.c_int(N),
+                          C.c_int(nb * 32), _p(out, C.c_int32))
+    return out
+
+
+def linear_q(x, W, wtype, bias=None, scale_mode=SCALE_X86_REF, return_xq=False):
+    """Quantized Linear as the reference CPU path computes it.  x fp32 [M, K]; returns y fp32 [M, N]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    W = np.ascontiguousarray(W, dtype=np.uint8)
+    M, K = x.shape
+    N, nb, bb = W.shape
+    assert nb * 32 == K and bb == BLOCK_BYTES[wtype]
+    y = np.empty((M, N), np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    xq = np.empty((M, K), np.int8)
+    xd = np.empty((M, nb), np.uint16)
+    rc = lib().orc_linear_q(_p(x, C.c_float), _p(W, C.c_uint8), C.c_int(wtype), _p(b, C.c_float), _p(y, C.c_float),
+                            C.c_int(M), C.c_int(N), C.c_int(K), C.c_int(scale_mode), _p(xq, C.c_int8),
+                            _p(xd, C.c_uint16))
+    assert rc == 0, rc
+    return (y, xq, xd) if return_xq else y
+
+
+# ----------------------------------------------------------------------------- W4A16
+def w4a16_dequant(qw, s_bits, zp, group=128):
+    """qw uint8 [N, K/2], s uint16 [N, G], zp uint8 [N, ceil(G/2)] -> bf16 bit patterns [N, K]."""
+    qw = np.ascontiguousarray(qw, dtype=np.uint8)
+    s_bits = np.ascontiguousarray(s_bits, dtype=np.uint16)
+    zp = np.ascontiguousarray(zp, dtype=np.uint8)
+    N, K = qw.shape[0], qw.shape[1] * 2
+    w = np.empty((N, K), np.uint16)
+    lib().orc_w4a16_dequant(_p(qw, C.c_uint8), _p(s_bits, C.c_uint16), _p(zp, C.c_uint8), C.c_int(N), C.c_int(K),
+                            C.c_int(group), _p(w, C.c_uint16))
+    return w
+
+
+def w4a16_gemm(a_bits, qw, s_bits, zp, bias_bits=None, group=128):
+    """A bf16 bits [M, K] -> C bf16 bits [M, N]."""
+    a_bits = np.ascontiguousarray(a_bits, dtype=np.uint16)
+    qw = np.ascontiguousarray(qw, dtype=np.uint8)
+    s_bits = np.ascontiguousarray(s_bits, dtype=np.uint16)
+    zp = np.ascontiguousarray(zp, dtype=np.uint8)
+    M, K = a_bits.shape
+    N = qw.shape[0]
+    c = np.empty((M, N), np.uint16)
+    bb = None if bias_bits is None else np.ascontiguousarray(bias_bits, dtype=np.uint16)
+    rc = lib().orc_w4a16_gemm(_p(a_bits, C.c_uint16), _p(qw, C.c_uint8), _p(s_bits, C.c_uint16), _p(zp, C.c_uint8),
+                              _p(bb, C.c_uint16), _p(c, C.c_uint16), C.c_int(M), C.c_int(N), C.c_int(K), C.c_int(group))
+    assert rc == 0, rc
+    return c
+
+
+# ----------------------------------------------------------------------------- W8A8
+def per_token_quant_int8(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    M, K = x.shape
+    q = np.empty((M, K), np.int8)
+    s = np.empty((M,), np.float32)
+    lib().orc_per_token_quant_int8(_p(x, C.c_float), _p(q, C.c_int8), _p(s, C.c_float), C.c_int(M), C.c_int(K))
+    return q, s
+
+
+def w8a8_gemm(xq, x_scale, W, w_scale, bias=None):
+    """returns (acc int32 [M, N], y bf16 bits [M, N])."""
+    xq = np.ascontiguousarray(xq, dtype=np.int8)
+    W = np.ascontiguousarray(W, dtype=np.int8)
+    x_scale = np.ascontiguousarray(x_scale, dtype=np.float32)
+    w_scale = np.ascontiguousarray(w_scale, dtype=np.float32)
+    M, K = xq.shape
+    N = W.shape[0]
+    acc = np.empty((M, N), np.int32)
+    y = np.empty((M, N), np.uint16)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    lib().orc_w8a8_gemm(_p(xq, C.c_int8), _p(x_scale, C.c_float), _p(W, C.c_int8), _p(w_scale, C.c_float),
+                        _p(b, C.c_float), _p(acc, C.c_int32), _p(y, C.c_uint16), C.c_int(M), C.c_int(N), C.c_int(K))
+    return acc, y
+
+
+# ----------------------------------------------------------------------------- MoE
+def moe_ffn(x, topk_ids, topk_w, Wg, Wu, Wd, wtype, scale_mode=SCALE_X86_REF):
+    """x fp32 [T, H]; ids int32 [T, k]; w fp32 [T, k]; Wg/Wu uint8 [E, I, H/32, blk]; Wd uint8 [E, H, I/32, blk]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    ids = np.ascontiguousarray(topk_ids, dtype=np.int32)
+    tw = np.ascontiguousarray(topk_w, dtype=np.float32)
+    Wg = np.ascontiguousarray(Wg, dtype=np.uint8)
+    Wu = np.ascontiguousarray(Wu, dtype=np.uint8)
+    Wd = np.ascontiguousarray(Wd, dtype=np.uint8)
+    T, H = x.shape
+    E, I = Wg.shape[0], Wg.shape[1]
+    k = ids.shape[1]
+    y = np.empty((T, H), np.float32)
+    rc = lib().orc_moe_ffn(_p(x, C.c_float), _p(ids, C.c_int32), _p(tw, C.c_float), _p(Wg, C.c_uint8),
+                           _p(Wu, C.c_uint8), _p(Wd, C.c_uint8), C.c_int(wtype), _p(y, C.c_float), C.c_int(T),
+                           C.c_int(H), C.c_int(I), C.c_int(E), C.c_int(k), C.c_int(scale_mode))
+    assert rc == 0, rc
+    return y
+
+
+# ----------------------------------------------------------------------------- compiled reference (oracle/_ref)
+def ref_quantize_rows_q8_0(x):
+    """reference quantize_row_q8_0 -> (codes int8 [M, K], EFFECTIVE scale values fp32 [M, K/32])."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    M, K = x.shape
+    qs = np.empty((M, K), np.int8)
+    d = np.empty((M, K // 32), np.float32)
+    for m in range(M):
+        ref().ref_quantize_row_q8_0(_p(x[m], C.c_float), _p(qs[m], C.c_int8), _p(d[m], C.c_float), C.c_int(K))
+    return qs, d
+
+
+def ref_dequantize(W, wtype):
+    W = np.ascontiguousarray(W, dtype=np.uint8)
+    N, nb, _ = W.shape
+    y = np.empty((N, nb * 32), np.float32)
+    for n in range(N):
+        ref().ref_dequantize_row(_p(W[n], C.c_uint8), C.c_int(wtype), _p(y[n], C.c_float), C.c_int(nb * 32))
+    return y
+
+
+def ref_linear_q(x, W, wtype, bias=None):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    W = np.ascontiguousarray(W, dtype=np.uint8)
+    M, K = x.shape
+    N = W.shape[0]
+    y = np.empty((M, N), np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    ref().ref_linear_q(_p(x, C.c_float), _p(W, C.c_uint8), C.c_int(wtype), _p(b, C.c_float), _p(y, C.c_float),
+                       C.c_int(M), C.c_int(N), C.c_int(K))
+    return y
+
+
+def ref_quantize_rows_q4_0(x):
+    """reference quantize_row_q4_0 (the offline weight quantizer) -> canonical blocks uint8 [N, K/32, 18]."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    N, K = x.shape
+    out = np.empty((N, K // 32, 18), np.uint8)
+    for n in range(N):
+        ref().ref_quantize_row_q4_0(_p(x[n], C.c_float), _p(out[n], C.c_uint8), C.c_int(K))
+    return out

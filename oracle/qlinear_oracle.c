@@ -1,0 +1,397 @@
+/*
+ * CPU oracle for the quantized-Linear path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This file restates, in plain C, the arithmetic the reference's x86 CPU backend
+ * performs for a Linear layer with Q4_0 / Q8_0 weights, plus closed-form
+ * restatements of the W4A16 (group-128, zero-point) and W8A8 (per-token dynamic)
+ * paths and of the MoE expert loop.  It is the checker the GPU kernels are
+ * compared against.  Nothing in the shipped library links, loads or calls it:
+ * only tests, the smoke check and the benchmark's cpu_baseline leg may.
+ *
+ * Every function cites the reference file:line it follows (paths are relative
+ * to the reference checkout root).
+ *
+ * Pinning status (what independently fixes each function; see tests/test_oracle_*.py):
+ *   orc_fp16_to_fp32 / orc_fp32_to_fp16      exhaustive vs numpy float16 and vs the compiled reference macros
+ *   orc_x86_scale_bits                       exhaustive (65 536 patterns) vs the compiled reference's store/load round trip
+ *   orc_quantize_row_q8_0                    bit-exact vs the compiled reference quantize_row_q8_0 (AVX2 branch)
+ *   orc_dequantize_row_q4_0 / _q8_0          bit-exact vs the compiled reference
+ *   orc_vec_dot_q4_0_q8_0 / _q8_0_q8_0       bit-exact vs the compiled reference vec_dot_* (same 8-lane fma + hsum order)
+ *   orc_linear_q                             composition of the above; llamafile_sgemm itself is unbuildable here
+ *                                            (needs fmt through mllm/utils/Common.hpp), its tile kernel is restated and
+ *                                            pinned through vec_dot (identical lane layout, fma and hsum) and a double
+ *                                            precision brute force
+ *   orc_w4a16_*  orc_w8a8_*  orc_per_token_quant_int8
+ *                                            the reference has no CPU implementation (CUDA-only third-party kernels):
+ *                                            parity unpinned by the reference; pinned here by the closed forms its tests
+ *                                            state, brute force in int64/float64 and special cases
+ *   orc_moe_ffn                              composition + permutation invariance + hand-built micro case
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define QK 32
+#define ORC_API __attribute__((visibility("default")))
+
+enum { ORC_Q4_0 = 0, ORC_Q8_0 = 1 };
+enum { ORC_SCALE_IEEE = 0, ORC_SCALE_X86_REF = 1 };
+
+static inline float u2f(uint32_t u) { float f; memcpy(&f, &u, 4); return f; }
+static inline uint32_t f2u(float f) { uint32_t u; memcpy(&u, &f, 4); return u; }
+
+/* ------------------------------------------------------------------------------------------------
+ * fp16 <-> fp32.  The x86 reference uses F16C: _cvtsh_ss / _cvtss_sh(x, 0) (round to nearest even)
+ * mllm/backends/cpu/kernels/common/ggml/quantize/quantize.hpp:108-109
+ * ---------------------------------------------------------------------------------------------- */
+ORC_API float orc_fp16_to_fp32(uint16_t h) {
+  uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+  uint32_t e = (h >> 10) & 0x1f, m = h & 0x3ff;
+  if (e == 0) {
+    float v = (float)m * 0x1p-24f; /* subnormal or zero: exact */
+    return sign ? -v : v;
+  }
+  if (e == 31) return u2f(sign | 0x7f800000u | (m << 13));
+  return u2f(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+ORC_API uint16_t orc_fp32_to_fp16(float f) {
+  uint32_t x = f2u(f);
+  uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+  x &= 0x7fffffffu;
+  if (x > 0x7f800000u) return (uint16_t)(sign | 0x7e00u | ((x >> 13) & 0x3ffu)); /* NaN -> quiet NaN */
+  if (x >= 0x477ff000u) return (uint16_t)(sign | 0x7c00u);                        /* >= 65520 rounds to inf */
+  if (x < 0x38800000u) {                                                          /* below 2^-14: subnormal half */
+    float v = u2f(x) * 0x1p24f;                                                   /* exact scaling */
+    return (uint16_t)(sign | (uint16_t)lrintf(v));                                /* RNE in the default rounding mode */
+  }
+  uint32_t e = (x >> 23) - 112u, m = x & 0x7fffffu;
+  uint32_t h = (e << 10) | (m >> 13), rem = m & 0x1fffu;
+  if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++; /* a carry into the exponent is the right answer */
+  return (uint16_t)(sign | h);
+}
+
+/* bf16 helpers (the prefill paths take bf16 activations; the decode path up-casts bf16 exactly) */
+ORC_API float orc_bf16_to_fp32(uint16_t b) { return u2f((uint32_t)b << 16); }
+ORC_API uint16_t orc_fp32_to_bf16(float f) {
+  uint32_t x = f2u(f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+  x += 0x7fffu + ((x >> 16) & 1u);
+  return (uint16_t)(x >> 16);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * The x86 build of the reference stores a block scale through two mismatched types: the macro
+ * MLLM_FP32_TO_FP16 yields the raw 16-bit pattern `b` as an integer (quantize.hpp:109,133), which is
+ * assigned to a half_float::half field (mllm/core/DataTypes.hpp:26) -> the field holds the NUMBER b rounded
+ * to half precision (11 significant bits, nearest even).  Reading goes half -> float -> uint16_t -> table
+ * lookup (quantize.hpp:114-130), so the scale that takes part in the arithmetic is fp16_to_fp32(b') with
+ * b' = RNE(b to 11 significant bits).  Patterns >= 65520 become +inf as a half; converting that to uint16_t
+ * is undefined in C++ and never occurs for finite scales (b < 0x7c00), we return 0xffff for them.
+ * ---------------------------------------------------------------------------------------------- */
+ORC_API uint16_t orc_x86_scale_bits(uint16_t b) {
+  if (b < 2048) return b;
+  if (b >= 65520) return 0xffff;
+  int p = 31 - __builtin_clz((unsigned)b); /* b in [2^p, 2^(p+1)) */
+  int sh = p - 10;
+  uint32_t q = b >> sh, rem = b & ((1u << sh) - 1u), half = 1u << (sh - 1);
+  if (rem > half || (rem == half && (q & 1u))) q++;
+  return (uint16_t)(q << sh);
+}
+
+static inline float scale_value(uint16_t bits, int scale_mode) {
+  return orc_fp16_to_fp32(scale_mode == ORC_SCALE_X86_REF ? orc_x86_scale_bits(bits) : bits);
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Q8_0 activation quantization, AVX2 branch of quantize_row_q8_0
+ * mllm/backends/cpu/kernels/common/ggml/quantize/quantize_q8.cpp:106-190
+ *   amax = max|x| ; d = amax/127 ; id = amax != 0 ? 127/amax : 0 ; q = int8_sat(rne(x*id)) ; d -> fp16 RNE
+ * Output is structure-of-arrays: codes[k], scale bit patterns[k/32] as the F16C conversion produces them
+ * (the x86 storage rounding is applied where the scale is USED, see scale_value()).
+ * ---------------------------------------------------------------------------------------------- */
+ORC_API void orc_quantize_row_q8_0(const float* x, int8_t* qs, uint16_t* d_bits, int k) {
+  int nb = k / QK;
+  for (int i = 0; i < nb; i++) {
+    const float* xb = x + (size_t)i * QK;
+    float amax = 0.0f;
+    for (int j = 0; j < QK; j++) {
+      float a = fabsf(xb[j]);
+      amax = a > amax ? a : amax;
+    }
+    const float d = amax / 127.f;
+    const float id = (amax != 0.0f) ? 127.f / amax : 0.0f;
+    d_bits[i] = orc_fp32_to_fp16(d);
+    for (int j = 0; j < QK; j++) {
+      float v = rintf(xb[j] * id); /* _mm256_round_ps(_MM_ROUND_NEAREST) = half to even */
+      int q = (int)v;
+      q = q > 127 ? 127 : (q < -128 ? -128 : q); /* packs_epi32 / packs_epi16 saturate */
+      qs[(size_t)i * QK + j] = (int8_t)q;
+    }
+  }
+}
+
+/* Reference array-of-structures block layouts, mllm/core/DataTypes.hpp:110-121,164-170 (pack(1)):
+ *   block_q4_0 = { fp16 d; uint8 qs[16] }  18 bytes; element j in the low nibble of qs[j], element j+16 in the high one
+ *   block_q8_0 = { fp16 d; int8 qs[32] }   34 bytes
+ * Here `d` is always the IEEE fp16 bit pattern. */
+static inline uint16_t blk_d(const uint8_t* blk) { uint16_t d; memcpy(&d, blk, 2); return d; }
+static inline int blk_bytes(int wtype) { return wtype == ORC_Q4_0 ? 18 : 34; }
+
+static inline void unpack_block(const uint8_t* blk, int wtype, int8_t w[QK]) {
+  if (wtype == ORC_Q4_0) {
+    for (int j = 0; j < 16; j++) {
+      w[j] = (int8_t)((blk[2 + j] & 0x0f) - 8);
+      w[j + 16] = (int8_t)((blk[2 + j] >> 4) - 8);
+    }
+  } else {
+    memcpy(w, blk + 2, QK);
+  }
+}
+
+/* dequantize_row_q4_0: quantize_q4.cpp:74-93 ; dequantize_row_q8_0: quantize_q8.cpp:197-211 */
+ORC_API void orc_dequantize_row(const uint8_t* blocks, int wtype, float* y, int k, int scale_mode) {
+  int nb = k / QK, bb = blk_bytes(wtype);
+  for (int i = 0; i < nb; i++) {
+    const uint8_t* blk = blocks + (size_t)i * bb;
+    float d = scale_value(blk_d(blk), scale_mode);
+    int8_t w[QK];
+    unpack_block(blk, wtype, w);
+    for (int j = 0; j < QK; j++) y[(size_t)i * QK + j] = (float)w[j] * d;
+  }
+}
+
+/* One weight row times one quantized activation row.
+ *   vec_dot_q4_0_q8_0 (AVX2): ggml/vec_dot.cpp:132-162, helpers ggml/vec_dot.hpp:244-295
+ *   vec_dot_q8_0_q8_0 (AVX2): ggml/vec_dot.cpp:1572-1593
+ *   tinyBLAS_Q0_AVX::gemm   : llamafile/llamafile_sgemm.cpp:697-743 (identical per-output arithmetic)
+ * Eight fp32 lanes; lane L holds sum_blocks fma(dW*dX, float(int32 sum of elements 4L..4L+3), lane) and the
+ * horizontal sum is ((l0+l4)+(l2+l6)) + ((l1+l5)+(l3+l7)).  isum (optional) receives the exact per-block int32 sums. */
+static float dot_row(const uint8_t* wrow, int wtype, const int8_t* xq, const uint16_t* xd, int nb, int scale_mode,
+                     int32_t* isum) {
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  int bb = blk_bytes(wtype);
+  for (int b = 0; b < nb; b++) {
+    const uint8_t* blk = wrow + (size_t)b * bb;
+    int8_t w[QK];
+    unpack_block(blk, wtype, w);
+    const int8_t* xb = xq + (size_t)b * QK;
+    const float d = scale_value(blk_d(blk), scale_mode) * scale_value(xd[b], scale_mode);
+    int32_t tot = 0;
+    for (int L = 0; L < 8; L++) {
+      int32_t s = 0;
+      for (int j = 0; j < 4; j++) s += (int32_t)w[4 * L + j] * (int32_t)xb[4 * L + j];
+      tot += s;
+      acc[L] = fmaf(d, (float)s, acc[L]);
+    }
+    if (isum) isum[b] = tot;
+  }
+  float t0 = acc[4] + acc[0], t1 = acc[5] + acc[1], t2 = acc[6] + acc[2], t3 = acc[7] + acc[3];
+  float u0 = t0 + t2, u1 = t1 + t3;
+  return u0 + u1;
+}
+
+ORC_API float orc_vec_dot(const uint8_t* wrow, int wtype, const int8_t* xq, const uint16_t* xd, int k, int scale_mode) {
+  return dot_row(wrow, wtype, xq, xd, k / QK, scale_mode, NULL);
+}
+
+/* Exact per-block integer dot products isum[n][m][b] (the int32 accumulators the GPU must match bit for bit). */
+ORC_API void orc_block_isums(const uint8_t* W, int wtype, const int8_t* xq, int M, int N, int K, int32_t* isum) {
+  int nb = K / QK, bb = blk_bytes(wtype);
+#pragma omp parallel for schedule(static)
+  for (int n = 0; n < N; n++)
+    for (int m = 0; m < M; m++)
+      for (int b = 0; b < nb; b++) {
+        int8_t w[QK];
+        unpack_block(W + ((size_t)n * nb + b) * bb, wtype, w);
+        const int8_t* xb = xq + ((size_t)m * nb + b) * QK;
+        int32_t s = 0;
+        for (int j = 0; j < QK; j++) s += (int32_t)w[j] * (int32_t)xb[j];
+        isum[((size_t)n * M + m) * nb + b] = s;
+      }
+}
+
+/* Quantized Linear as the x86 CPU backend runs it:
+ *   CPULinearOp::forward -> ggml::mat_mul(x, W, y, bias, false, true)      backends/cpu/ops/LinearOp.cpp:100-128,282-288
+ *   mat_mul: quantize every activation row to Q8_0, then llamafile_sgemm   ggml/matmul.cpp:148-206
+ *   y[m][n] = bias[n] + hsum(...)                                          llamafile_sgemm.cpp:735-741
+ * x fp32 [M][K]; W reference blocks [N][K/32]; bias fp32 [N] or NULL; y fp32 [M][N].
+ * xq_out / xd_out (optional) receive the activation codes [M][K] and scale patterns [M][K/32]. */
+ORC_API int orc_linear_q(const float* x, const uint8_t* W, int wtype, const float* bias, float* y, int M, int N, int K,
+                         int scale_mode, int8_t* xq_out, uint16_t* xd_out) {
+  if (K % QK != 0 || M < 0 || N < 0) return -1;
+  int nb = K / QK, bb = blk_bytes(wtype);
+  int8_t* xq = xq_out ? xq_out : (int8_t*)malloc((size_t)M * K);
+  uint16_t* xd = xd_out ? xd_out : (uint16_t*)malloc((size_t)M * nb * 2);
+  if (!xq || !xd) return -2;
+#pragma omp parallel for schedule(static)
+  for (int m = 0; m < M; m++) orc_quantize_row_q8_0(x + (size_t)m * K, xq + (size_t)m * K, xd + (size_t)m * nb, K);
+#pragma omp parallel for schedule(static)
+  for (int n = 0; n < N; n++) {
+    const uint8_t* wrow = W + (size_t)n * nb * bb;
+    for (int m = 0; m < M; m++) {
+      float v = dot_row(wrow, wtype, xq + (size_t)m * K, xd + (size_t)m * nb, nb, scale_mode, NULL);
+      y[(size_t)m * N + n] = bias ? bias[n] + v : v;
+    }
+  }
+  if (!xq_out) free(xq);
+  if (!xd_out) free(xd);
+  return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * W4A16, group 128 along K, uint4 codes with uint4 zero-points and fp16 scales (AWQ/Marlin semantics):
+ *   w = (q - zp) * scale, computed in the activation dtype   mllm-kernel/mllm_kernel/cuda/csrc/gemm/marlin/dequant.h:18-26,
+ *                                                            marlin_template.h:153-168
+ *   test formula (q - 8) * scale for the symmetric variant   mllm-kernel/tests/test_gptq_marlin.py:143-146
+ * Canonical restatement used by the GPU kernel and by this oracle:
+ *   w_bf16[n][k] = bf16_rne( float(q[n][k] - zp[n][k/128]) * fp16_to_fp32(s[n][k/128]) )
+ *   C[m][n]      = bf16_rne( sum_k float(A[m][k]) * float(w_bf16[n][k]) )      (products are exact in fp32)
+ * The sum is taken in double here (order-free anchor); the kernel accumulates in fp32.
+ * Storage: qw u8 [N][K/2], element 2j in the low nibble of byte j; zp u8 [N][ceil(G/2)], group 2g low nibble;
+ * s fp16 bits [N][G], G = K/128.
+ * ---------------------------------------------------------------------------------------------- */
+static inline int nib(const uint8_t* p, size_t i) { return (i & 1) ? (p[i >> 1] >> 4) : (p[i >> 1] & 0x0f); }
+
+ORC_API void orc_w4a16_dequant(const uint8_t* qw, const uint16_t* s, const uint8_t* zp, int N, int K, int group,
+                               uint16_t* w_bf16) {
+  int G = K / group, zpb = (G + 1) / 2;
+#pragma omp parallel for schedule(static)
+  for (int n = 0; n < N; n++)
+    for (int k = 0; k < K; k++) {
+      int g = k / group;
+      int q = nib(qw + (size_t)n * (K / 2), (size_t)k);
+      int z = nib(zp + (size_t)n * zpb, (size_t)g);
+      float w = (float)(q - z) * orc_fp16_to_fp32(s[(size_t)n * G + g]);
+      w_bf16[(size_t)n * K + k] = orc_fp32_to_bf16(w);
+    }
+}
+
+ORC_API int orc_w4a16_gemm(const uint16_t* A_bf16, const uint8_t* qw, const uint16_t* s, const uint8_t* zp,
+                           const uint16_t* bias_bf16, uint16_t* C_bf16, int M, int N, int K, int group) {
+  if (K % group != 0 || K % 2 != 0) return -1;
+  uint16_t* w = (uint16_t*)malloc((size_t)N * K * 2);
+  float* af = (float*)malloc((size_t)M * K * 4);
+  if (!w || !af) return -2;
+  orc_w4a16_dequant(qw, s, zp, N, K, group, w);
+  for (size_t i = 0; i < (size_t)M * K; i++) af[i] = orc_bf16_to_fp32(A_bf16[i]);
+#pragma omp parallel for schedule(static)
+  for (int n = 0; n < N; n++) {
+    float* wf = (float*)malloc((size_t)K * 4);
+    for (int k = 0; k < K; k++) wf[k] = orc_bf16_to_fp32(w[(size_t)n * K + k]);
+    for (int m = 0; m < M; m++) {
+      double acc = 0.0;
+      const float* a = af + (size_t)m * K;
+      for (int k = 0; k < K; k++) acc += (double)a[k] * (double)wf[k];
+      float r = (float)acc;
+      if (bias_bf16) r += orc_bf16_to_fp32(bias_bf16[n]);
+      C_bf16[(size_t)m * N + n] = orc_fp32_to_bf16(r);
+    }
+    free(wf);
+  }
+  free(w);
+  free(af);
+  return 0;
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * Per-token dynamic int8 activation quantization (torch form):
+ *   absmax = max(amax|x|, 1e-10); scale = absmax / 127; q = clamp(round_half_even(x / scale), -128, 127)
+ *   pymllm/tests/bench_w8a8_activation_quant.py:20-26
+ * x fp32 [M][K] (a bf16 activation is up-cast exactly first); q int8 [M][K]; scale fp32 [M].
+ * ---------------------------------------------------------------------------------------------- */
+ORC_API void orc_per_token_quant_int8(const float* x, int8_t* q, float* scale, int M, int K) {
+#pragma omp parallel for schedule(static)
+  for (int m = 0; m < M; m++) {
+    const float* xr = x + (size_t)m * K;
+    float amax = 0.0f;
+    for (int k = 0; k < K; k++) {
+      float a = fabsf(xr[k]);
+      amax = a > amax ? a : amax;
+    }
+    if (amax < 1e-10f) amax = 1e-10f;
+    const float sc = amax / 127.0f;
+    scale[m] = sc;
+    for (int k = 0; k < K; k++) {
+      float v = rintf(xr[k] / sc);
+      v = v > 127.f ? 127.f : (v < -128.f ? -128.f : v);
+      q[(size_t)m * K + k] = (int8_t)v;
+    }
+  }
+}
+
+/* W8A8 GEMM: acc[m][n] = sum_k xq[m][k] * W[n][k] in int32 (exact), then
+ *   y = out_dtype( float(acc) * (w_scale[n] * x_scale[m]) + bias[n] )
+ *   mllm-kernel/mllm_kernel/cuda/csrc/cutlass_extensions/epilogue/epilogue_per_row_per_col_scale.h:234-253,273-280
+ *   CPU-style references: tests/ascend/AscendLinearKernelTest.hpp:289-303, mllm-kernel/tests/test_int8_scaled_mm_cutlass.py:22-35
+ * acc_out (optional) int32 [M][N]; y bf16 bits [M][N] (optional). */
+ORC_API void orc_w8a8_gemm(const int8_t* xq, const float* x_scale, const int8_t* W, const float* w_scale,
+                           const float* bias, int32_t* acc_out, uint16_t* y_bf16, int M, int N, int K) {
+#pragma omp parallel for schedule(static)
+  for (int m = 0; m < M; m++)
+    for (int n = 0; n < N; n++) {
+      const int8_t* a = xq + (size_t)m * K;
+      const int8_t* w = W + (size_t)n * K;
+      int32_t acc = 0;
+      for (int k = 0; k < K; k++) acc += (int32_t)a[k] * (int32_t)w[k];
+      if (acc_out) acc_out[(size_t)m * N + n] = acc;
+      if (y_bf16) {
+        float r = (float)acc * (w_scale[n] * x_scale[m]);
+        if (bias) r += bias[n];
+        y_bf16[(size_t)m * N + n] = orc_fp32_to_bf16(r);
+      }
+    }
+}
+
+/* ------------------------------------------------------------------------------------------------
+ * MoE expert FFN over expert-sorted tokens.
+ *   Qwen3MoE::moeInfer      mllm/models/qwen3_moe/modeling_qwen3_moe_fa2.hpp:175-238
+ *   Qwen3MoeMLP::forward    :98-100     down(silu(gate(x)) * up(x)), every Linear = orc_linear_q
+ *   SiLU scalar form        mllm/backends/cpu/kernels/x86/silu.cpp:41   x / (1 + exp(-x))
+ * x fp32 [T][H]; topk_ids int32 [T][k]; topk_w fp32 [T][k]; expert e weights: Wg,Wu blocks [I][H/32], Wd blocks [H][I/32],
+ * stored per expert contiguously.  y fp32 [T][H] = sum_j topk_w[t][j] * expert_{ids[t][j]}(x[t]), j ascending.
+ * ---------------------------------------------------------------------------------------------- */
+ORC_API float orc_silu(float x) { return x / (1.0f + expf(-x)); }
+
+ORC_API int orc_moe_ffn(const float* x, const int32_t* topk_ids, const float* topk_w, const uint8_t* Wg,
+                        const uint8_t* Wu, const uint8_t* Wd, int wtype, float* y, int T, int H, int I, int E, int k,
+                        int scale_mode) {
+  if (H % QK || I % QK) return -1;
+  int bb = blk_bytes(wtype);
+  size_t gu_bytes = (size_t)I * (H / QK) * bb, d_bytes = (size_t)H * (I / QK) * bb;
+  float* per = (float*)calloc((size_t)T * k * H, 4); /* output of the expert for (token, slot) */
+  if (!per) return -2;
+  for (int e = 0; e < E; e++) {
+    int cnt = 0;
+    for (int i = 0; i < T * k; i++) cnt += (topk_ids[i] == e);
+    if (!cnt) continue;
+    int* rows = (int*)malloc(sizeof(int) * cnt);
+    float* xe = (float*)malloc((size_t)cnt * H * 4);
+    float* g = (float*)malloc((size_t)cnt * I * 4);
+    float* u = (float*)malloc((size_t)cnt * I * 4);
+    float* o = (float*)malloc((size_t)cnt * H * 4);
+    int c = 0;
+    for (int i = 0; i < T * k; i++)
+      if (topk_ids[i] == e) {
+        rows[c] = i;
+        memcpy(xe + (size_t)c * H, x + (size_t)(i / k) * H, (size_t)H * 4);
+        c++;
+      }
+    orc_linear_q(xe, Wg + e * gu_bytes, wtype, NULL, g, cnt, I, H, scale_mode, NULL, NULL);
+    orc_linear_q(xe, Wu + e * gu_bytes, wtype, NULL, u, cnt, I, H, scale_mode, NULL, NULL);
+    for (size_t i = 0; i < (size_t)cnt * I; i++) g[i] = orc_silu(g[i]) * u[i];
+    orc_linear_q(g, Wd + e * d_bytes, wtype, NULL, o, cnt, H, I, scale_mode, NULL, NULL);
+    for (c = 0; c < cnt; c++) memcpy(per + (size_t)rows[c] * H, o + (size_t)c * H, (size_t)H * 4);
+    free(rows); free(xe); free(g); free(u); free(o);
+  }
+#pragma omp parallel for schedule(static)
+  for (int t = 0; t < T; t++)
+    for (int h = 0; h < H; h++) {
+      float acc = 0.0f;
+      for (int j = 0; j < k; j++) acc += per[((size_t)t * k + j) * H + h] * topk_w[(size_t)t * k + j];
+      y[(size_t)t * H + h] = acc;
+    }
+  free(per);
+  return 0;
+}

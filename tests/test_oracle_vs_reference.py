@@ -1,0 +1,103 @@
+"""Pins oracle/qlinear_oracle.c against the reference's own compiled kernels (oracle/_ref).
+
+Skipped where oracle/_ref was not built (it needs the reference checkout); tests/test_oracle_golden.py covers the same
+ground from committed fixtures there.
+"""
+import numpy as np
+import pytest
+
+from mllm_amd import synth
+from oracle import oracle as orc
+
+pytestmark = pytest.mark.skipif(not orc.ref_available(), reason="oracle/_ref not built (reference checkout absent)")
+
+
+def test_fp16_conversions_match_reference_macros():
+    L, R = orc.lib(), orc.ref()
+    for b in range(65536):
+        a, r = np.float32(L.orc_fp16_to_fp32(b)), np.float32(R.ref_fp16_bits_to_fp32(b))
+        assert a.view(np.uint32) == r.view(np.uint32) or (np.isnan(a) and np.isnan(r)), hex(b)
+    rng = np.random.default_rng(1)
+    halves = np.arange(0, 0x7c00, dtype=np.uint16).view(np.float16).astype(np.float32)
+    mids = (halves[:-1].astype(np.float64) + halves[1:].astype(np.float64)) / 2
+    samples = np.concatenate([halves, mids.astype(np.float32), np.nextafter(mids.astype(np.float32), np.float32(1e9)),
+                              np.nextafter(mids.astype(np.float32), np.float32(-1e9)),
+                              rng.standard_normal(20000).astype(np.float32) * np.float32(0.01),
+                              np.float32([65504, 65519.99, 65520, 1e6, 3e-8, 2.9802322e-8, 2.98e-8, 0.0])])
+    samples = np.concatenate([samples, -samples])
+    for f in samples[::3]:
+        assert L.orc_fp32_to_fp16(float(f)) == R.ref_fp32_to_fp16_bits(float(f)), float(f)
+
+
+def test_x86_scale_roundtrip_exhaustive():
+    L, R = orc.lib(), orc.ref()
+    changed = 0
+    for b in range(65520):
+        eff = L.orc_x86_scale_bits(b)
+        want = np.float32(R.ref_scale_store_load(b))
+        got = np.float32(L.orc_fp16_to_fp32(eff))
+        assert got.view(np.uint32) == want.view(np.uint32) or (np.isnan(got) and np.isnan(want)), hex(b)
+        changed += eff != b
+    assert changed > 50000  # the quirk is real: most patterns do not survive
+
+
+def _rows(rng, K):
+    import importlib.util, os
+    spec = importlib.util.spec_from_file_location(
+        "make_golden", os.path.join(os.path.dirname(__file__), "golden", "make_golden.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod.actquant_rows(rng, K)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_quantize_row_q8_0_bit_exact(seed):
+    rng = np.random.default_rng(seed)
+    x = np.concatenate([_rows(rng, 512), rng.standard_normal((64, 512)).astype(np.float32) * 3])
+    qs, d_bits = orc.quantize_rows_q8_0(x)
+    rqs, rd = orc.ref_quantize_rows_q8_0(x)
+    assert np.array_equal(qs, rqs)
+    eff = orc.fp16_bits_to_fp32(orc.x86_scale_bits(d_bits))
+    assert np.array_equal(eff.view(np.uint32), rd.view(np.uint32))
+
+
+@pytest.mark.parametrize("wtype", [orc.Q4_0, orc.Q8_0])
+def test_dequantize_bit_exact(wtype):
+    rng = np.random.default_rng(3)
+    W = synth.make_weight(rng, wtype, 16, 256)
+    assert np.array_equal(orc.dequantize(W, wtype, orc.SCALE_X86_REF).view(np.uint32),
+                          orc.ref_dequantize(W, wtype).view(np.uint32))
+    # un-snapped scales: only the x86 reading reproduces the reference, the IEEE reading must differ somewhere
+    W2 = W.copy()
+    W2[:, :, 0] |= 0x05
+    assert np.array_equal(orc.dequantize(W2, wtype, orc.SCALE_X86_REF).view(np.uint32),
+                          orc.ref_dequantize(W2, wtype).view(np.uint32))
+    assert not np.array_equal(orc.dequantize(W2, wtype, orc.SCALE_IEEE), orc.ref_dequantize(W2, wtype))
+
+
+@pytest.mark.parametrize("wtype", [orc.Q4_0, orc.Q8_0])
+@pytest.mark.parametrize("M", [1, 3, 4, 8])
+@pytest.mark.parametrize("bias", [False, True])
+def test_linear_bit_exact_vs_reference_vec_dot(wtype, M, bias):
+    rng = np.random.default_rng(100 + M)
+    N, K = 48, 320
+    W = synth.make_weight(rng, wtype, N, K)
+    x = synth.make_x_fp32(rng, M, K)
+    b = rng.standard_normal(N).astype(np.float32) if bias else None
+    y = orc.linear_q(x, W, wtype, b, orc.SCALE_X86_REF)
+    r = orc.ref_linear_q(x, W, wtype, b)
+    assert np.array_equal(y.view(np.uint32), r.view(np.uint32))
+
+
+def test_q4_0_weights_from_reference_quantizer():
+    """weights written by the reference's own quantize_row_q4_0 (negative scales included) run through the oracle."""
+    rng = np.random.default_rng(5)
+    Wf = (rng.standard_normal((32, 256)) * 0.05).astype(np.float32)
+    W = orc.ref_quantize_rows_q4_0(Wf)
+    x = synth.make_x_fp32(rng, 2, 256)
+    y = orc.linear_q(x, W, orc.Q4_0, None, orc.SCALE_X86_REF)
+    r = orc.ref_linear_q(x, W, orc.Q4_0)
+    assert np.array_equal(y.view(np.uint32), r.view(np.uint32))
+    # and the quantized Linear approximates the fp32 one
+    ref = x @ Wf.T
+    assert np.linalg.norm(y - ref) / np.linalg.norm(ref) < 0.15
