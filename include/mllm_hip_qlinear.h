@@ -1,0 +1,95 @@
+/*
+ * mllm_hip_qlinear.h -- C ABI of the MI355X (gfx950) quantized-Linear kernels.
+ *
+ * This is the seam a HIP backend's Linear / MatMul ops call: plain pointers and sizes, no C++ or torch types.
+ * The C++ ops that sit on top of it (HipLinearOp etc., mllm_amd/csrc/host) mirror the reference's
+ * BaseOp::{load,reshape,setup,forward} contract; this header is what their forward()/load() bind.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the name ends in _host
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); calls are asynchronous on it
+ *   - return value: 0 on success; a positive value is a hipError_t; a negative value is MLLM_HIP_E_* below
+ *   - matrices are row-major; a Linear weight is [N out_channels][K in_channels] like the reference's
+ *     `weight_.view({out_channels, in_channels})` (mllm/backends/cpu/ops/LinearOp.cpp:13-40)
+ *   - nothing here allocates device memory: workspaces are sized by a *_bytes() call and passed in
+ */
+#ifndef MLLM_HIP_QLINEAR_H
+#define MLLM_HIP_QLINEAR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLLM_HIP_E_BADARG (-1)   /* null pointer, negative size, unknown enum            */
+#define MLLM_HIP_E_SHAPE (-2)    /* K not a multiple of the block / group size, M too big */
+#define MLLM_HIP_E_ALIGN (-3)    /* pointer not aligned as documented                     */
+#define MLLM_HIP_E_NODEVICE (-4) /* no gfx950 device / kernel image not loadable          */
+
+/* weight block formats: mllm/core/DataTypes.hpp:110-121 (block_q4_0, 18 B), :164-170 (block_q8_0, 34 B) */
+enum { MLLM_HIP_Q4_0 = 0, MLLM_HIP_Q8_0 = 1 };
+/* activation element types */
+enum { MLLM_HIP_F32 = 0, MLLM_HIP_BF16 = 1 };
+/* How a block scale is read.
+ *   IEEE     the 2-byte `d` field is an IEEE fp16 bit pattern (ARM builds of the reference, GGUF files)
+ *   X86_REF  the x86 build of the reference: the field is a half-precision NUMBER equal to the bit pattern
+ *            (mllm/core/DataTypes.hpp:26 with quantize.hpp:108-134), i.e. the pattern rounded to 11 significant
+ *            bits.  For weights this selects how prepack decodes the stored field; for the activation scale
+ *            computed inside the GEMV it selects whether that rounding is reproduced. */
+enum { MLLM_HIP_SCALE_IEEE = 0, MLLM_HIP_SCALE_X86_REF = 1 };
+
+/* library / device ------------------------------------------------------------------------------------ */
+const char* mllm_hip_version(void);
+/* Selects nothing and allocates nothing; returns 0 when device `device` is a gfx950 part and the kernels load. */
+int mllm_hip_init(int device);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * Q4_0 / Q8_0 Linear  (decode GEMV, M = 1..8)
+ * replaces: CPULinearOp::forward -> ggml::mat_mul -> quantize_row_q8_0 + llamafile_sgemm
+ *           mllm/backends/cpu/ops/LinearOp.cpp:100-128,282-288 ; ggml/matmul.cpp:148-206 ;
+ *           ggml/quantize/quantize_q8.cpp:106-190 ; llamafile/llamafile_sgemm.cpp:697-743
+ * ------------------------------------------------------------------------------------------------------- */
+
+/* Size of the pre-packed (structure-of-arrays) form of an [N][K] weight: 16-byte code vectors first, fp16 scales after. */
+size_t mllm_hip_q_packed_bytes(int wtype, int64_t N, int64_t K);
+
+/* load()-time repack of reference blocks (array of 18 / 34-byte structs, row-major [N][K/32], on the device) into the
+ * coalesced layout the kernels read.  `weight_scale_mode` says how the stored `d` field is to be decoded.
+ * replaces: CPULinearOp::load (LinearOp.cpp:13-98) + the X2X host->device copy of the weight. */
+int mllm_hip_q_prepack(int wtype, const void* blocks, int weight_scale_mode, void* packed, int64_t N, int64_t K,
+                       void* stream);
+
+/* y[m][n] = bias[n] + sum_b fp32(dW[n][b] * dX[m][b]) * int32(sum_32 qW * qX),   qX,dX = Q8_0 quantization of x[m]
+ * x: [M][K] fp32 or bf16 (x_dtype), y: fp32 [M][N], bias: fp32 [N] or NULL, 1 <= M <= 8, K % 32 == 0.
+ * The activation quantization is fused into the kernel. */
+int mllm_hip_linear_q_gemv(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y,
+                           int M, int64_t N, int64_t K, int act_scale_mode, void* stream);
+
+/* Same for any M: quantizes the activations with a stand-alone kernel into `workspace`
+ * (mllm_hip_linear_q_workspace_bytes) and runs the tiled block-dot kernel.  Used by prefill and by the MoE path. */
+size_t mllm_hip_linear_q_workspace_bytes(int64_t M, int64_t K);
+int mllm_hip_linear_q(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y,
+                      int64_t M, int64_t N, int64_t K, int act_scale_mode, void* workspace, void* stream);
+
+/* Stand-alone Q8_0 activation quantization (quantize_row_q8_0, AVX2 branch, quantize_q8.cpp:106-190).
+ * codes int8 [M][K]; d_bits uint16 [M][K/32] = the fp16 pattern of amax/127 (before any x86 storage rounding). */
+int mllm_hip_quantize_q8_0(const void* x, int x_dtype, int8_t* codes, uint16_t* d_bits, int64_t M, int64_t K,
+                           void* stream);
+
+/* Parity probes (used by the tests, cheap enough to ship):
+ *   dequantize: w[n][k] = code * fp32(scale)       dequantize_row_q4_0 / _q8_0 (quantize_q4.cpp:74-93, quantize_q8.cpp:197-211)
+ *   block_isums: exact int32 dot product of every weight block with every activation block, [N][M][K/32] */
+int mllm_hip_q_dequantize(int wtype, const void* packed, float* w, int64_t N, int64_t K, void* stream);
+int mllm_hip_q_block_isums(int wtype, const void* packed, const int8_t* codes, int32_t* isums, int64_t M, int64_t N,
+                           int64_t K, void* stream);
+
+/* GEMV launch-shape override for tuning sweeps: lanes per weight row (8/16/32/64), rows per lane group (1/2/4),
+ * waves per workgroup (1..4); 0 restores the built-in heuristic. */
+int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_per_wg);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLLM_HIP_QLINEAR_H */

@@ -1,0 +1,54 @@
+"""Loads the in-tree HIP library through its C ABI (include/mllm_hip_qlinear.h).
+
+There is no fallback: if the library is missing or a call fails, an exception is raised.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libmllm_hip_qlinear.so")
+
+_lib = None
+
+
+class HipQLinearError(RuntimeError):
+    pass
+
+
+_ERRS = {-1: "bad argument", -2: "unsupported shape", -3: "misaligned pointer", -4: "no gfx950 device"}
+
+
+def check(rc, what):
+    if rc != 0:
+        msg = _ERRS.get(rc, "hipError_t %d" % rc if rc > 0 else "error %d" % rc)
+        raise HipQLinearError("%s failed: %s" % (what, msg))
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise HipQLinearError(
+                "%s not found: build it with `python -m mllm_amd.build` (hipcc, gfx950)" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        i64, vp, ci = C.c_int64, C.c_void_p, C.c_int
+        L.mllm_hip_version.restype = C.c_char_p
+        L.mllm_hip_init.argtypes = [ci]
+        L.mllm_hip_q_packed_bytes.restype = C.c_size_t
+        L.mllm_hip_q_packed_bytes.argtypes = [ci, i64, i64]
+        L.mllm_hip_q_prepack.argtypes = [ci, vp, ci, vp, i64, i64, vp]
+        L.mllm_hip_linear_q_gemv.argtypes = [ci, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]
+        L.mllm_hip_quantize_q8_0.argtypes = [vp, ci, vp, vp, i64, i64, vp]
+        L.mllm_hip_q_dequantize.argtypes = [ci, vp, vp, i64, i64, vp]
+        L.mllm_hip_q_block_isums.argtypes = [ci, vp, vp, vp, i64, i64, i64, vp]
+        L.mllm_hip_gemv_set_tuning.argtypes = [ci, ci, ci]
+        _lib = L
+    return _lib
+
+
+# every symbol include/mllm_hip_qlinear.h declares (checked by the CPU test-suite against the header text)
+def exported_symbols():
+    import re
+    hdr = os.path.join(os.path.dirname(_HERE), "include", "mllm_hip_qlinear.h")
+    txt = open(hdr).read()
+    return sorted(set(re.findall(r"\b(mllm_hip_[a-z0-9_]+)\s*\(", txt)))

@@ -1,0 +1,128 @@
+// Device-side helpers shared by the gfx950 quantized-Linear kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mllm_hip_qlinear.h"
+
+#define QK 32
+#define MLLM_API extern "C" __attribute__((visibility("default")))
+
+#define HIP_RET(expr)                    \
+  do {                                   \
+    hipError_t e__ = (expr);             \
+    if (e__ != hipSuccess) return (int)e__; \
+  } while (0)
+
+namespace mllmhip {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte load
+
+// ---- bit casts / small conversions ---------------------------------------------------------------------
+__device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest even, NaN kept quiet
+  uint32_t x = __float_as_uint(f);
+  if ((x & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((x >> 16) | 0x40u);
+  x += 0x7fffu + ((x >> 16) & 1u);
+  return (uint16_t)(x >> 16);
+}
+__device__ __forceinline__ float f16bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
+__device__ __forceinline__ uint16_t f32_to_f16bits(float f) {  // v_cvt_f16_f32, round to nearest even
+  return __builtin_bit_cast(uint16_t, (_Float16)f);
+}
+// What an fp16 scale pattern reads back as after the reference's x86 build stored it in a block: the pattern, taken as
+// a number, rounded to half precision (11 significant bits).  Mirrors the mechanism itself: number -> half -> number.
+__device__ __forceinline__ uint16_t x86_scale_bits(uint16_t b) {
+  return (uint16_t)(uint32_t)(float)(_Float16)(float)(uint32_t)b;
+}
+
+// ---- wavefront reductions with DPP (64-wide waves; a DPP row is 16 lanes) -------------------------------
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+// Sum over aligned groups of G consecutive lanes; every lane of the group ends up with the total.
+template <int G>
+__device__ __forceinline__ float group_sum(float v) {
+  if (G >= 2) v += dpp_f<0xB1>(v);   // quad_perm [1,0,3,2]
+  if (G >= 4) v += dpp_f<0x4E>(v);   // quad_perm [2,3,0,1]
+  if (G >= 8) v += dpp_f<0x141>(v);  // row_half_mirror
+  if (G >= 16) v += dpp_f<0x140>(v); // row_mirror
+  if (G >= 32) v += __shfl_xor(v, 16, 64);
+  if (G >= 64) v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+// ---- Q8_0 quantization of one 32-element block held in registers ----------------------------------------
+// quantize_row_q8_0, AVX2 branch (mllm/backends/cpu/kernels/common/ggml/quantize/quantize_q8.cpp:106-190):
+//   amax = max|v| ; d = amax / 127 ; id = amax != 0 ? 127 / amax : 0 ; q = sat_int8(round_half_even(v * id)).
+// q[8] receives the codes, four per dword in element order; returns the fp16 pattern of d; sum = sum of the codes.
+__device__ __forceinline__ uint16_t quantize_block_q8_0(const float (&v)[32], uint32_t (&q)[8], int& sum) {
+  float amax = 0.f;
+#pragma unroll
+  for (int j = 0; j < 32; j++) amax = fmaxf(amax, fabsf(v[j]));
+  const float d = amax / 127.f;
+  const float id = (amax != 0.f) ? 127.f / amax : 0.f;
+  int s = 0;
+#pragma unroll
+  for (int w = 0; w < 8; w++) {
+    uint32_t pk = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      int qi = (int)rintf(v[4 * w + j] * id);
+      qi = min(127, max(-128, qi));
+      s += qi;
+      pk |= ((uint32_t)qi & 0xffu) << (8 * j);
+    }
+    q[w] = pk;
+  }
+  sum = s;
+  return f32_to_f16bits(d);
+}
+
+// Loads one 32-element activation block as fp32 (fp32 input: 8 x 16 B, bf16 input: 4 x 16 B; bf16 -> fp32 is exact).
+__device__ __forceinline__ void load_block_f32(const void* x, int x_dtype, int64_t elem_offset, float (&v)[32]) {
+  if (x_dtype == MLLM_HIP_F32) {
+    const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(x) + elem_offset);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      float4 t = p[i];
+      v[4 * i + 0] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
+    }
+  } else {
+    const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(x) + elem_offset);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      uint4 t = p[i];
+      uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        v[8 * i + 2 * j + 0] = __uint_as_float(w[j] << 16);
+        v[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      }
+    }
+  }
+}
+
+// packed weight layout: code planes of 16 B per block (Q4_0: one plane, Q8_0: two), then the fp16 scales
+struct PackedView {
+  const u32x4* q0;      // Q4_0: 32 nibbles of the block; Q8_0: elements 0..15
+  const u32x4* q1;      // Q8_0: elements 16..31 (unused for Q4_0)
+  const uint16_t* d;    // IEEE fp16 patterns
+};
+__host__ __device__ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+__host__ __device__ inline size_t packed_plane_bytes(int64_t N, int64_t K) { return align_up((size_t)N * (K / QK) * 16, 256); }
+__host__ __device__ inline size_t packed_bytes(int wtype, int64_t N, int64_t K) {
+  return packed_plane_bytes(N, K) * (wtype == MLLM_HIP_Q4_0 ? 1 : 2) + align_up((size_t)N * (K / QK) * 2, 256);
+}
+__host__ __device__ inline PackedView packed_view(int wtype, const void* packed, int64_t N, int64_t K) {
+  const char* p = reinterpret_cast<const char*>(packed);
+  size_t pl = packed_plane_bytes(N, K);
+  PackedView v;
+  v.q0 = reinterpret_cast<const u32x4*>(p);
+  v.q1 = reinterpret_cast<const u32x4*>(p + pl);
+  v.d = reinterpret_cast<const uint16_t*>(p + pl * (wtype == MLLM_HIP_Q4_0 ? 1 : 2));
+  return v;
+}
+
+}  // namespace mllmhip

@@ -1,0 +1,82 @@
+"""Host-side convenience layer over the C ABI for callers that hold torch tensors on the GPU.
+
+torch is used for device memory and the current stream only; every computation is a call into
+libmllm_hip_qlinear.so.  Enumerations mirror include/mllm_hip_qlinear.h.
+"""
+import torch
+
+from . import _lib
+
+Q4_0, Q8_0 = 0, 1
+F32, BF16 = 0, 1
+SCALE_IEEE, SCALE_X86_REF = 0, 1
+BLOCK_BYTES = {Q4_0: 18, Q8_0: 34}
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _xdtype(x):
+    if x.dtype == torch.float32:
+        return F32
+    if x.dtype == torch.bfloat16:
+        return BF16
+    raise TypeError("activations must be float32 or bfloat16, got %s" % x.dtype)
+
+
+class PackedQWeight:
+    """A Q4_0 / Q8_0 weight [N, K] repacked on the device into the layout the kernels read."""
+
+    def __init__(self, wtype, blocks, weight_scale_mode=SCALE_IEEE):
+        """blocks: uint8 tensor [N, K/32, 18|34] of reference blocks (host or device)."""
+        assert blocks.dtype == torch.uint8 and blocks.dim() == 3 and blocks.shape[2] == BLOCK_BYTES[wtype]
+        self.wtype, self.N, self.K = wtype, blocks.shape[0], blocks.shape[1] * 32
+        L = _lib.lib()
+        nbytes = L.mllm_hip_q_packed_bytes(wtype, self.N, self.K)
+        if nbytes == 0:
+            raise _lib.HipQLinearError("unsupported weight shape N=%d K=%d" % (self.N, self.K))
+        dev_blocks = blocks.contiguous().cuda()
+        self.buf = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        _lib.check(L.mllm_hip_q_prepack(wtype, dev_blocks.data_ptr(), weight_scale_mode, self.buf.data_ptr(), self.N,
+                                        self.K, _stream()), "mllm_hip_q_prepack")
+        torch.cuda.current_stream().synchronize()  # dev_blocks may be released after this
+
+    @property
+    def ptr(self):
+        return self.buf.data_ptr()
+
+    def dequantize(self):
+        out = torch.empty((self.N, self.K), dtype=torch.float32, device="cuda")
+        _lib.check(_lib.lib().mllm_hip_q_dequantize(self.wtype, self.ptr, out.data_ptr(), self.N, self.K, _stream()),
+                   "mllm_hip_q_dequantize")
+        return out
+
+    def block_isums(self, codes):
+        M = codes.shape[0]
+        out = torch.empty((self.N, M, self.K // 32), dtype=torch.int32, device="cuda")
+        _lib.check(_lib.lib().mllm_hip_q_block_isums(self.wtype, self.ptr, codes.data_ptr(), out.data_ptr(), M, self.N,
+                                                     self.K, _stream()), "mllm_hip_q_block_isums")
+        return out
+
+
+def linear_q_gemv(w, x, bias=None, act_scale_mode=SCALE_X86_REF, out=None):
+    """y = Linear(x) with Q4_0/Q8_0 weights, 1 <= M <= 8.  x [M, K] fp32/bf16 on the GPU -> y fp32 [M, N]."""
+    assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
+    M = x.shape[0]
+    y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_linear_q_gemv(w.wtype, w.ptr, x.data_ptr(), _xdtype(x),
+                                                 bias.data_ptr() if bias is not None else None, y.data_ptr(), M, w.N,
+                                                 w.K, act_scale_mode, _stream()), "mllm_hip_linear_q_gemv")
+    return y
+
+
+def quantize_q8_0(x):
+    """x [M, K] -> (codes int8 [M, K], scale patterns int16-viewed-as-uint16 [M, K/32])."""
+    assert x.is_cuda and x.is_contiguous() and x.dim() == 2
+    M, K = x.shape
+    codes = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    d = torch.empty((M, K // 32), dtype=torch.int16, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_quantize_q8_0(x.data_ptr(), _xdtype(x), codes.data_ptr(), d.data_ptr(), M, K,
+                                                 _stream()), "mllm_hip_quantize_q8_0")
+    return codes, d

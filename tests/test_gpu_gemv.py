@@ -1,0 +1,198 @@
+"""GPU parity of the Q4_0 / Q8_0 decode GEMV against the CPU oracle and the committed golden vectors.
+
+Bars: activation codes, scale patterns, dequantized weights and int32 block sums bit-exact; fp32 outputs rel-L2 <= 1e-3
+(the kernel sums the per-block terms in a different order than the CPU's 8-lane accumulators).
+"""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from mllm_amd import _lib, qlinear as ql, synth
+from oracle import oracle as orc
+from gpu_util import announce, bf16_dev, rel_l2, to_dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3  # rel-L2, the bar of the fp32 outputs
+
+
+def _mode(m):
+    return ql.SCALE_X86_REF if m == orc.SCALE_X86_REF else ql.SCALE_IEEE
+
+
+def test_init_and_version():
+    L = _lib.lib()
+    assert b"gfx950" in L.mllm_hip_version()
+    _lib.check(L.mllm_hip_init(0), "mllm_hip_init")
+    assert L.mllm_hip_init(99) == -4
+
+
+@pytest.mark.parametrize("wname,wtype", [("q4_0", 0), ("q8_0", 1)])
+def test_golden_gemv(golden_dir, wname, wtype):
+    g = np.load(os.path.join(golden_dir, "gemv_kat.npz"))
+    announce("golden gemv", wname)
+    w = ql.PackedQWeight(wtype, torch.from_numpy(g[f"{wname}_W"]))
+    bias = to_dev(g[f"{wname}_bias"])
+    for M in (1, 3, 4, 8):
+        x = to_dev(g[f"{wname}_x{M}"])
+        y = ql.linear_q_gemv(w, x, None, ql.SCALE_X86_REF).cpu().numpy()
+        yb = ql.linear_q_gemv(w, x, bias, ql.SCALE_X86_REF).cpu().numpy()
+        assert rel_l2(y, g[f"{wname}_y{M}"]) < 1e-5, M
+        assert rel_l2(yb, g[f"{wname}_yb{M}"]) < 1e-5, M
+
+
+def test_golden_actquant_bit_exact(golden_dir):
+    g = np.load(os.path.join(golden_dir, "q8_0_actquant.npz"))
+    announce("golden actquant")
+    codes, d = ql.quantize_q8_0(to_dev(g["x"]))
+    assert np.array_equal(codes.cpu().numpy(), g["qs"])
+    d_bits = d.cpu().numpy().view(np.uint16)
+    eff = orc.fp16_bits_to_fp32(orc.x86_scale_bits(d_bits))
+    assert np.array_equal(eff.view(np.uint32), g["d_eff"].view(np.uint32))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_actquant_bit_exact_vs_oracle(dtype):
+    rng = synth.rng_for(1, 11)
+    M, K = 8, 9728
+    if dtype == "bf16":
+        bits, xf = synth.make_x_bf16(rng, M, K)
+        xd = bf16_dev(bits)
+    else:
+        xf = (synth.make_x_fp32(rng, M, K) * rng.uniform(0.001, 50, (M, 1))).astype(np.float32)
+        xf[2, 96:128] = 0
+        xd = to_dev(xf)
+    announce("actquant", dtype, M, K)
+    codes, d = ql.quantize_q8_0(xd)
+    qs, db = orc.quantize_rows_q8_0(xf)
+    assert np.array_equal(codes.cpu().numpy(), qs)
+    assert np.array_equal(d.cpu().numpy().view(np.uint16), db)
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+def test_dequant_and_block_isums_bit_exact(wtype, golden_dir):
+    rng = synth.rng_for(1, 12)
+    N, K, M = 96, 640, 5
+    W = synth.make_weight(rng, wtype, N, K)
+    W[:, :, 0] |= 0x05  # scales off the snapped grid: the two decodings of the weight scale now differ
+    announce("dequant/isums", wtype)
+    for mode in (orc.SCALE_IEEE, orc.SCALE_X86_REF):
+        # x86 mode: the file holds the pattern as a half-precision number -> encode it that way for prepack
+        Wd = W.copy()
+        if mode == orc.SCALE_X86_REF:
+            b = W[:, :, 0:2].copy().view(np.uint16)[:, :, 0]
+            enc = b.astype(np.float32).astype(np.float16).view(np.uint16)  # half(float(pattern))
+            Wd[:, :, 0:2] = enc.reshape(N, -1, 1).view(np.uint8)
+        w = ql.PackedQWeight(wtype, torch.from_numpy(Wd), _mode(mode))
+        want = orc.dequantize(W, wtype, mode)
+        assert np.array_equal(w.dequantize().cpu().numpy().view(np.uint32), want.view(np.uint32)), mode
+    g = np.load(os.path.join(golden_dir, "dequant_kat.npz"))
+    wg = ql.PackedQWeight(wtype, torch.from_numpy(g["W4" if wtype == 0 else "W8"]))
+    assert np.array_equal(wg.dequantize().cpu().numpy(), g["y4" if wtype == 0 else "y8"])
+    x = synth.make_x_fp32(rng, M, K)
+    qs, _ = orc.quantize_rows_q8_0(x)
+    w = ql.PackedQWeight(wtype, torch.from_numpy(W))
+    got = w.block_isums(to_dev(qs)).cpu().numpy()
+    assert np.array_equal(got, orc.block_isums(W, wtype, qs))
+
+
+SHAPES = [("c1", 6144, 2048)] + [(k, n, kk) for k, (n, kk) in synth.QWEN3_4B_LAYER.items() if k != "v_proj"]
+
+
+@pytest.mark.parametrize("name,N,K", SHAPES)
+@pytest.mark.parametrize("wtype", [0, 1])
+def test_gemv_full_shapes(name, N, K, wtype):
+    rng = synth.rng_for(1, hash((name, wtype)) % 1000)
+    W = synth.make_weight(rng, wtype, N, K)
+    w = ql.PackedQWeight(wtype, torch.from_numpy(W))
+    bias = rng.standard_normal(N).astype(np.float32)
+    for M in (1, 4, 8):
+        bits, xf = synth.make_x_bf16(rng, M, K)
+        announce("gemv", name, N, K, "wtype", wtype, "M", M)
+        for mode in (orc.SCALE_X86_REF, orc.SCALE_IEEE):
+            y = ql.linear_q_gemv(w, bf16_dev(bits), None, _mode(mode)).cpu().numpy()
+            want = orc.linear_q(xf, W, wtype, None, mode)
+            assert rel_l2(y, want) < TOL, (M, mode, rel_l2(y, want))
+            assert rel_l2(y, want) < 2e-6, (M, mode, rel_l2(y, want))  # in practice only the summation order differs
+        yb = ql.linear_q_gemv(w, to_dev(xf), to_dev(bias), ql.SCALE_X86_REF).cpu().numpy()
+        assert rel_l2(yb, orc.linear_q(xf, W, wtype, bias, orc.SCALE_X86_REF)) < 2e-6
+
+
+@pytest.mark.parametrize("N,K", [(1, 32), (37, 96), (1000, 800), (65, 2048), (7, 4096 + 32)])
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 6, 7, 8])
+def test_gemv_ragged(N, K, M):
+    rng = synth.rng_for(1, N + K + M)
+    for wtype in (0, 1):
+        W = synth.make_weight(rng, wtype, N, K)
+        w = ql.PackedQWeight(wtype, torch.from_numpy(W))
+        xf = synth.make_x_fp32(rng, M, K)
+        announce("ragged", N, K, M, wtype)
+        y = ql.linear_q_gemv(w, to_dev(xf), None, ql.SCALE_X86_REF).cpu().numpy()
+        assert rel_l2(y, orc.linear_q(xf, W, wtype, None, orc.SCALE_X86_REF)) < 2e-6
+
+
+def test_gemv_every_launch_shape():
+    rng = synth.rng_for(1, 99)
+    N, K = 520, 2560
+    L = _lib.lib()
+    try:
+        for wtype in (0, 1):
+            W = synth.make_weight(rng, wtype, N, K)
+            w = ql.PackedQWeight(wtype, torch.from_numpy(W))
+            for M in (1, 2, 4, 8):
+                xf = synth.make_x_fp32(rng, M, K)
+                want = orc.linear_q(xf, W, wtype, None, orc.SCALE_X86_REF)
+                xd = to_dev(xf)
+                for G in (8, 16, 32, 64):
+                    for R in (1, 2, 4):
+                        for NW in (1, 4):
+                            announce("launch shape", wtype, M, G, R, NW)
+                            assert L.mllm_hip_gemv_set_tuning(G, R, NW) == 0
+                            y = ql.linear_q_gemv(w, xd, None, ql.SCALE_X86_REF).cpu().numpy()
+                            assert rel_l2(y, want) < 2e-6, (wtype, M, G, R, NW)
+    finally:
+        L.mllm_hip_gemv_set_tuning(0, 0, 0)
+
+
+def test_gemv_special_inputs():
+    """all-zero activations -> bias only; a x20 outlier; a single hot element"""
+    rng = synth.rng_for(1, 5)
+    N, K = 256, 1024
+    W = synth.make_q4_0(rng, N, K)
+    w = ql.PackedQWeight(0, torch.from_numpy(W))
+    bias = rng.standard_normal(N).astype(np.float32)
+    announce("special inputs")
+    y0 = ql.linear_q_gemv(w, torch.zeros((2, K), device="cuda"), to_dev(bias)).cpu().numpy()
+    assert np.array_equal(y0, np.stack([bias, bias]))
+    x = synth.make_x_fp32(rng, 1, K)
+    x[0, 17] *= 20
+    y = ql.linear_q_gemv(w, to_dev(x)).cpu().numpy()
+    assert rel_l2(y, orc.linear_q(x, W, 0)) < 2e-6
+    e = np.zeros((1, K), np.float32)
+    e[0, 40] = 3.0
+    y = ql.linear_q_gemv(w, to_dev(e), None, ql.SCALE_IEEE).cpu().numpy()
+    col = orc.dequantize(W, 0)[:, 40] / np.float32(1)  # one hot: y = W[:, 40] * dequant(q8(3.0)) = w * 127 * d
+    d = np.float32(np.float16(np.float32(3.0) / np.float32(127)))
+    assert np.allclose(y[0], col * (np.float32(127) * d), rtol=1e-6, atol=0)
+
+
+def test_gemv_argument_errors():
+    L = _lib.lib()
+    rng = synth.rng_for(1, 6)
+    W = synth.make_q4_0(rng, 8, 64)
+    w = ql.PackedQWeight(0, torch.from_numpy(W))
+    x = torch.zeros((8, 64), device="cuda")
+    y = torch.zeros((8, 8), device="cuda")
+    f = L.mllm_hip_linear_q_gemv
+    assert f(0, w.ptr, x.data_ptr(), 0, None, y.data_ptr(), 0, 8, 64, 0, None) == -2   # M = 0
+    assert f(0, w.ptr, x.data_ptr(), 0, None, y.data_ptr(), 9, 8, 64, 0, None) == -2   # M = 9
+    assert f(0, w.ptr, x.data_ptr(), 0, None, y.data_ptr(), 1, 8, 48, 0, None) == -2   # K % 32
+    assert f(5, w.ptr, x.data_ptr(), 0, None, y.data_ptr(), 1, 8, 64, 0, None) == -1   # weight type
+    assert f(0, None, x.data_ptr(), 0, None, y.data_ptr(), 1, 8, 64, 0, None) == -1    # null weight
+    assert f(0, w.ptr, None, 0, None, y.data_ptr(), 1, 8, 64, 0, None) == -1           # null x
+    assert f(0, w.ptr, x.data_ptr(), 7, None, y.data_ptr(), 1, 8, 64, 0, None) == -1   # x dtype
+    assert f(0, w.ptr + 4, x.data_ptr(), 0, None, y.data_ptr(), 1, 8, 64, 0, None) == -3  # alignment
+    assert L.mllm_hip_q_packed_bytes(0, 8, 48) == 0
+    with pytest.raises(_lib.HipQLinearError):
+        _lib.check(-2, "probe")
