@@ -86,7 +86,7 @@ int mllm_hip_q_block_isums(int wtype, const void* packed, const int8_t* codes, i
                            int64_t K, void* stream);
 
 /* GEMV launch-shape override for tuning sweeps: lanes per weight row (8/16/32/64), rows per lane group (1/2/4),
- * waves per workgroup (1..4); 0 restores the built-in heuristic. */
+ * waves per workgroup (1..16); 0 restores the built-in heuristic. */
 int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_per_wg);
 
 #ifdef __cplusplus

@@ -80,21 +80,32 @@ __device__ __forceinline__ uint16_t quantize_block_q8_0(const float (&v)[32], ui
   return f32_to_f16bits(d);
 }
 
-// Loads one 32-element activation block as fp32 (fp32 input: 8 x 16 B, bf16 input: 4 x 16 B; bf16 -> fp32 is exact).
-__device__ __forceinline__ void load_block_f32(const void* x, int x_dtype, int64_t elem_offset, float (&v)[32]) {
-  if (x_dtype == MLLM_HIP_F32) {
-    const float4* p = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(x) + elem_offset);
+// One 32-element activation block, raw: fp32 input = 8 x 16 B, bf16 input = 4 x 16 B.  Loading and converting are
+// separate steps so that a caller can issue other loads in between.
+template <int XT>
+__device__ __forceinline__ void load_block_raw_t(const void* x, int64_t elem_offset, u32x4 (&raw)[XT == MLLM_HIP_F32 ? 8 : 4]) {
+  if (XT == MLLM_HIP_F32) {
+    const u32x4* p = reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(x) + elem_offset);
+#pragma unroll
+    for (int i = 0; i < 8; i++) raw[i] = p[i];
+  } else {
+    const u32x4* p = reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(x) + elem_offset);
+#pragma unroll
+    for (int i = 0; i < 4; i++) raw[i] = p[i];
+  }
+}
+template <int XT>
+__device__ __forceinline__ void block_raw_to_f32_t(const u32x4 (&raw)[XT == MLLM_HIP_F32 ? 8 : 4], float (&v)[32]) {
+  if (XT == MLLM_HIP_F32) {
 #pragma unroll
     for (int i = 0; i < 8; i++) {
-      float4 t = p[i];
-      v[4 * i + 0] = t.x; v[4 * i + 1] = t.y; v[4 * i + 2] = t.z; v[4 * i + 3] = t.w;
+      v[4 * i + 0] = __uint_as_float(raw[i].x); v[4 * i + 1] = __uint_as_float(raw[i].y);
+      v[4 * i + 2] = __uint_as_float(raw[i].z); v[4 * i + 3] = __uint_as_float(raw[i].w);
     }
-  } else {
-    const uint4* p = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(x) + elem_offset);
+  } else {  // bf16 -> fp32 is exact
 #pragma unroll
     for (int i = 0; i < 4; i++) {
-      uint4 t = p[i];
-      uint32_t w[4] = {t.x, t.y, t.z, t.w};
+      const uint32_t w[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
 #pragma unroll
       for (int j = 0; j < 4; j++) {
         v[8 * i + 2 * j + 0] = __uint_as_float(w[j] << 16);
@@ -103,8 +114,43 @@ __device__ __forceinline__ void load_block_f32(const void* x, int x_dtype, int64
     }
   }
 }
+__device__ __forceinline__ void load_block_raw(const void* x, int x_dtype, int64_t elem_offset, u32x4 (&raw)[8]) {
+  if (x_dtype == MLLM_HIP_F32) {
+    const u32x4* p = reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(x) + elem_offset);
+#pragma unroll
+    for (int i = 0; i < 8; i++) raw[i] = p[i];
+  } else {
+    const u32x4* p = reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(x) + elem_offset);
+#pragma unroll
+    for (int i = 0; i < 4; i++) raw[i] = p[i];
+  }
+}
+__device__ __forceinline__ void block_raw_to_f32(const u32x4 (&raw)[8], int x_dtype, float (&v)[32]) {
+  if (x_dtype == MLLM_HIP_F32) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      v[4 * i + 0] = __uint_as_float(raw[i].x); v[4 * i + 1] = __uint_as_float(raw[i].y);
+      v[4 * i + 2] = __uint_as_float(raw[i].z); v[4 * i + 3] = __uint_as_float(raw[i].w);
+    }
+  } else {  // bf16 -> fp32 is exact
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+      const uint32_t w[4] = {raw[i].x, raw[i].y, raw[i].z, raw[i].w};
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        v[8 * i + 2 * j + 0] = __uint_as_float(w[j] << 16);
+        v[8 * i + 2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      }
+    }
+  }
+}
+__device__ __forceinline__ void load_block_f32(const void* x, int x_dtype, int64_t elem_offset, float (&v)[32]) {
+  u32x4 raw[8];
+  load_block_raw(x, x_dtype, elem_offset, raw);
+  block_raw_to_f32(raw, x_dtype, v);
+}
 
-// packed weight layout: code planes of 16 B per block (Q4_0: one plane, Q8_0: two), then the fp16 scales
+// packed weight layout: code planes of 16 B per block (Q4_0: one plane, Q8_0: two), then the fp16 scales [N][nbp]
 struct PackedView {
   const u32x4* q0;      // Q4_0: 32 nibbles of the block; Q8_0: elements 0..15
   const u32x4* q1;      // Q8_0: elements 16..31 (unused for Q4_0)
@@ -112,8 +158,10 @@ struct PackedView {
 };
 __host__ __device__ inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 __host__ __device__ inline size_t packed_plane_bytes(int64_t N, int64_t K) { return align_up((size_t)N * (K / QK) * 16, 256); }
+// scale rows are padded to a multiple of 8 entries (16 bytes) so that a row's scales can be fetched with 16-byte loads
+__host__ __device__ inline int64_t scale_row_stride(int64_t K) { return (int64_t)align_up((size_t)(K / QK), 8); }
 __host__ __device__ inline size_t packed_bytes(int wtype, int64_t N, int64_t K) {
-  return packed_plane_bytes(N, K) * (wtype == MLLM_HIP_Q4_0 ? 1 : 2) + align_up((size_t)N * (K / QK) * 2, 256);
+  return packed_plane_bytes(N, K) * (wtype == MLLM_HIP_Q4_0 ? 1 : 2) + align_up((size_t)N * scale_row_stride(K) * 2, 256);
 }
 __host__ __device__ inline PackedView packed_view(int wtype, const void* packed, int64_t N, int64_t K) {
   const char* p = reinterpret_cast<const char*>(packed);

@@ -1,0 +1,6 @@
+// GEMV kernel instances for one (weight type, activation type) pair; split out so that the pairs compile in parallel.
+#include "qgemv_kernel.h"
+
+namespace mllmhip {
+int launch_gemv_q4_f32(const GemvArgs& a, int MT, GemvShape s, hipStream_t st) { return launch_gemv<MLLM_HIP_Q4_0, MLLM_HIP_F32>(a, MT, s, st); }
+}  // namespace mllmhip

@@ -42,6 +42,19 @@ class PackedQWeight:
                                         self.K, _stream()), "mllm_hip_q_prepack")
         torch.cuda.current_stream().synchronize()  # dev_blocks may be released after this
 
+    @classmethod
+    def synthetic(cls, wtype, N, K, generator=None):
+        """Random weight drawn on the device (benchmark pools): codes uniform, fp16 block scales |N(0,0.02)|/7 with the low
+        three pattern bits cleared so that the IEEE and the x86 reading of the scale agree.  Goes through prepack."""
+        nb = K // 32
+        blocks = torch.randint(0, 256, (N, nb, BLOCK_BYTES[wtype]), dtype=torch.uint8, device="cuda", generator=generator)
+        if wtype == Q8_0:
+            blocks[blocks == 0x80] = 0x81  # int8 codes in [-127, 127]
+        s = (torch.randn((N, nb), device="cuda", generator=generator) * 0.02).abs() / 7.0
+        bits = s.to(torch.float16).view(torch.int16) & ~7
+        blocks[:, :, 0:2] = bits.view(torch.uint8).view(N, nb, 2)
+        return cls(wtype, blocks)
+
     @property
     def ptr(self):
         return self.buf.data_ptr()

@@ -146,7 +146,7 @@ def test_gemv_every_launch_shape():
                 xd = to_dev(xf)
                 for G in (8, 16, 32, 64):
                     for R in (1, 2, 4):
-                        for NW in (1, 4):
+                        for NW in (1, 4, 16):
                             announce("launch shape", wtype, M, G, R, NW)
                             assert L.mllm_hip_gemv_set_tuning(G, R, NW) == 0
                             y = ql.linear_q_gemv(w, xd, None, ql.SCALE_X86_REF).cpu().numpy()
