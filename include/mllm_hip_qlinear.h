@@ -89,6 +89,34 @@ int mllm_hip_q_block_isums(int wtype, const void* packed, const int8_t* codes, i
  * waves per workgroup (1..16); 0 restores the built-in heuristic. */
 int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_per_wg);
 
+/* ---------------------------------------------------------------------------------------------------------
+ * W8A8 Linear (prefill): per-token dynamic int8 activations x int8 weights with per-channel scales
+ * replaces: CompressedTensorsW8A8Int8Scheme.apply = per_token_quant_int8 + int8_scaled_mm
+ *           pymllm/quantization/methods/compressed_tensors.py:450-468
+ *           pymllm/quantization/kernels/int8_activation_triton.py:13-42 (rounding rule of
+ *           pymllm/tests/bench_w8a8_activation_quant.py:20-26: half to even)
+ *           mllm-kernel/mllm_kernel/cuda/csrc/gemm/int8/int8_scaled_mm_cutlass.cu:40-154
+ * ------------------------------------------------------------------------------------------------------- */
+
+/* q[m][k] = clamp(round_half_even(x[m][k] / scale[m]), -128, 127), scale[m] = max(amax|x[m]|, 1e-10) / 127.
+ * x: [M][K] fp32 or bf16; q: int8 [M][K]; scale: fp32 [M]. */
+int mllm_hip_per_token_quant_int8(const void* x, int x_dtype, int8_t* q, float* scale, int64_t M, int64_t K,
+                                  void* stream);
+
+/* acc[m][n] = sum_k xq[m][k] * W[n][k] (int32, exact);  out = bf16( float(acc) * (w_scale[n] * x_scale[m]) + bias[n] ).
+ * xq int8 [M][K]; W int8 [N][K] (the checkpoint's [out, in] layout); w_scale fp32 [N]; x_scale fp32 [M]; bias fp32 [N] or
+ * NULL; out_bf16 [M][N] and/or acc_out int32 [M][N] (either may be NULL, not both).  K % 16 == 0. */
+int mllm_hip_w8a8_gemm(const int8_t* xq, const float* x_scale, const int8_t* W, const float* w_scale, const float* bias,
+                       void* out_bf16, int32_t* acc_out, int64_t M, int64_t N, int64_t K, void* stream);
+
+/* The two steps back to back; `workspace` (mllm_hip_w8a8_workspace_bytes) holds the quantized activations. */
+size_t mllm_hip_w8a8_workspace_bytes(int64_t M, int64_t K);
+int mllm_hip_w8a8_linear(const void* x, int x_dtype, const int8_t* W, const float* w_scale, const float* bias,
+                         void* out_bf16, int64_t M, int64_t N, int64_t K, void* workspace, void* stream);
+
+/* GEMM tile override for tuning sweeps: 0 heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64 workgroup tiles. */
+int mllm_hip_w8a8_set_tuning(int tile);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,6 +42,12 @@ def lib():
         L.mllm_hip_q_dequantize.argtypes = [ci, vp, vp, i64, i64, vp]
         L.mllm_hip_q_block_isums.argtypes = [ci, vp, vp, vp, i64, i64, i64, vp]
         L.mllm_hip_gemv_set_tuning.argtypes = [ci, ci, ci]
+        L.mllm_hip_per_token_quant_int8.argtypes = [vp, ci, vp, vp, i64, i64, vp]
+        L.mllm_hip_w8a8_gemm.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, vp]
+        L.mllm_hip_w8a8_workspace_bytes.restype = C.c_size_t
+        L.mllm_hip_w8a8_workspace_bytes.argtypes = [i64, i64]
+        L.mllm_hip_w8a8_linear.argtypes = [vp, ci, vp, vp, vp, vp, i64, i64, i64, vp, vp]
+        L.mllm_hip_w8a8_set_tuning.argtypes = [ci]
         _lib = L
     return _lib
 

@@ -93,3 +93,44 @@ def quantize_q8_0(x):
     _lib.check(_lib.lib().mllm_hip_quantize_q8_0(x.data_ptr(), _xdtype(x), codes.data_ptr(), d.data_ptr(), M, K,
                                                  _stream()), "mllm_hip_quantize_q8_0")
     return codes, d
+
+
+# ----------------------------------------------------------------------------- W8A8 (per-token dynamic int8)
+def _p(t):
+    return t.data_ptr() if t is not None else None
+
+
+def per_token_quant_int8(x):
+    """x [M, K] fp32/bf16 -> (q int8 [M, K], scale fp32 [M])."""
+    assert x.is_cuda and x.is_contiguous() and x.dim() == 2
+    M, K = x.shape
+    q = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    s = torch.empty((M,), dtype=torch.float32, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_per_token_quant_int8(x.data_ptr(), _xdtype(x), q.data_ptr(), s.data_ptr(), M, K,
+                                                        _stream()), "mllm_hip_per_token_quant_int8")
+    return q, s
+
+
+def w8a8_gemm(xq, x_scale, W, w_scale, bias=None, want_acc=False, out=None):
+    """xq int8 [M, K], W int8 [N, K] -> bf16 [M, N] (and the int32 accumulators when want_acc)."""
+    M, K = xq.shape
+    N = W.shape[0]
+    assert W.shape[1] == K and xq.is_contiguous() and W.is_contiguous()
+    y = out if out is not None else torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    acc = torch.empty((M, N), dtype=torch.int32, device="cuda") if want_acc else None
+    _lib.check(_lib.lib().mllm_hip_w8a8_gemm(xq.data_ptr(), _p(x_scale), W.data_ptr(), _p(w_scale), _p(bias),
+                                             y.data_ptr(), _p(acc), M, N, K, _stream()), "mllm_hip_w8a8_gemm")
+    return (y, acc) if want_acc else y
+
+
+def w8a8_linear(x, W, w_scale, bias=None, workspace=None, out=None):
+    """bf16/fp32 x [M, K] -> bf16 [M, N]: per-token quantization + int8 GEMM, two launches."""
+    M, K = x.shape
+    N = W.shape[0]
+    L = _lib.lib()
+    if workspace is None:
+        workspace = torch.empty(L.mllm_hip_w8a8_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+    y = out if out is not None else torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    _lib.check(L.mllm_hip_w8a8_linear(x.data_ptr(), _xdtype(x), W.data_ptr(), w_scale.data_ptr(), _p(bias),
+                                      y.data_ptr(), M, N, K, workspace.data_ptr(), _stream()), "mllm_hip_w8a8_linear")
+    return y
