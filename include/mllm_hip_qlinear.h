@@ -117,6 +117,27 @@ int mllm_hip_w8a8_linear(const void* x, int x_dtype, const int8_t* W, const floa
 /* GEMM tile override for tuning sweeps: 0 heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64 workgroup tiles. */
 int mllm_hip_w8a8_set_tuning(int tile);
 
+/* ---------------------------------------------------------------------------------------------------------
+ * W4A16 Linear (prefill): bf16 activations x uint4 weights, per-group fp16 scale and uint4 zero-point
+ * replaces: AWQMarlinLinearMethod.apply -> gptq_marlin_gemm with zero points
+ *           pymllm/quantization/methods/awq_marlin.py:274-449
+ *           mllm-kernel/mllm_kernel/cuda/csrc/gemm/marlin/marlin_template.h:255-... , dequant.h:18-26
+ * ------------------------------------------------------------------------------------------------------- */
+
+/* C[m][n] = bf16( sum_k A[m][k] * w[n][k] + bias[n] ),  w[n][k] = bf16( (q[n][k] - zp[n][k/group]) * scale[n][k/group] ).
+ * a_bf16 [M][K]; qw uint8 [N][K/2] (element 2j in the low nibble of byte j); scales fp16 [N][K/group];
+ * zeros uint8 [N][ceil(K/group/2)] (group 2i in the low nibble of byte i); bias_bf16 [N] or NULL; c_bf16 [M][N].
+ * group % 64 == 0 and K % group == 0 (128 in the checkpoints). */
+int mllm_hip_w4a16_gemm(const void* a_bf16, const uint8_t* qw, const uint16_t* scales, const uint8_t* zeros,
+                        const void* bias_bf16, void* c_bf16, int64_t M, int64_t N, int64_t K, int group, void* stream);
+
+/* Parity probe: the dequantized weight table w_bf16 [N][K] exactly as the GEMM forms it. */
+int mllm_hip_w4a16_dequantize(const uint8_t* qw, const uint16_t* scales, const uint8_t* zeros, void* w_bf16, int64_t N,
+                              int64_t K, int group, void* stream);
+
+/* GEMM tile override for tuning sweeps: 0 heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64 workgroup tiles. */
+int mllm_hip_w4a16_set_tuning(int tile);
+
 #ifdef __cplusplus
 }
 #endif

@@ -48,6 +48,9 @@ def lib():
         L.mllm_hip_w8a8_workspace_bytes.argtypes = [i64, i64]
         L.mllm_hip_w8a8_linear.argtypes = [vp, ci, vp, vp, vp, vp, i64, i64, i64, vp, vp]
         L.mllm_hip_w8a8_set_tuning.argtypes = [ci]
+        L.mllm_hip_w4a16_gemm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp]
+        L.mllm_hip_w4a16_dequantize.argtypes = [vp, vp, vp, vp, i64, i64, ci, vp]
+        L.mllm_hip_w4a16_set_tuning.argtypes = [ci]
         _lib = L
     return _lib
 

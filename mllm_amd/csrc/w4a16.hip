@@ -1,0 +1,278 @@
+// W4A16 Linear for prefill on gfx950: bf16 activations x uint4 weights with per-group fp16 scales and uint4 zero-points
+// (group size a multiple of 64 along K, 128 in the checkpoints), fp32 accumulation, bf16 output.
+//
+// Semantics (the reference runs this on CUDA through Marlin; restated in closed form):
+//   dequantization      mllm-kernel/mllm_kernel/cuda/csrc/gemm/marlin/dequant.h:18-26 (q - zp), marlin_template.h:153-168 (x scale)
+//   checkpoint scheme   pymllm/quantization/methods/awq_marlin.py:274-449
+//   test formula        mllm-kernel/tests/test_gptq_marlin.py:143-146
+//   w_bf16[n][k] = bf16_rne( float(q[n][k] - zp[n][k/g]) * fp32(scale[n][k/g]) )   (the product is exact in fp32: <= 16 bits)
+//   C[m][n]      = bf16_rne( sum_k A[m][k] * w_bf16[n][k]  (+ bias[n]) ),  fp32 accumulate on the matrix cores
+// Storage: qw uint8 [N][K/2], element 2j in the low nibble of byte j; scales fp16 [N][K/g]; zero-points uint8
+// [N][ceil(K/g/2)], group 2i in the low nibble of byte i.
+//
+// Weights are fetched packed (16 bytes = 32 elements per lane), dequantized once per workgroup in registers and staged
+// as bf16 in LDS next to the activation tile; the matrix cores read both operands from LDS.
+#include "qcommon.h"
+
+namespace mllmhip {
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, nearest even
+}
+
+// eight elements of one packed dword -> four dwords of bf16 pairs, element order kept.
+// (q - zp) * s == fma(q, s, -zp*s) exactly: both products and their sum need at most 16 significant bits.
+__device__ __forceinline__ void dequant8(uint32_t w, float s, float nzs, uint32_t (&out)[4]) {
+  const uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;  // bytes: elements 0,2,4,6 / 1,3,5,7
+#pragma unroll
+  for (int b = 0; b < 4; b++) {
+    const float e0 = fmaf((float)((lo >> (8 * b)) & 0xffu), s, nzs);
+    const float e1 = fmaf((float)((hi >> (8 * b)) & 0xffu), s, nzs);
+    out[b] = pack_bf16(e0, e1);
+  }
+}
+
+struct W4A16Args {
+  const uint16_t* A;    // bf16 [M][K]
+  const uint8_t* qw;    // [N][K/2]
+  const uint16_t* s;    // fp16 [N][G]
+  const uint8_t* zp;    // [N][(G+1)/2]
+  const uint16_t* bias; // bf16 [N] or null
+  uint16_t* C;          // bf16 [M][N]
+  int M, N, K, group;
+};
+
+// Workgroup tile BM x BN, K step 64 elements; waves (BM/WM) x (BN/WN), each WM x WN as 32x32 tiles of
+// v_mfma_f32_32x32x16_bf16 (every lane supplies 8 consecutive k of one row of A and of one row of W).
+// LDS rows hold 64 bf16 = 128 bytes, padded to 144 so that 16-byte reads of 16 neighbouring rows hit distinct banks.
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__((BM / WM) * (BN / WN) * 64) void w4a16_gemm_kernel(W4A16Args a) {
+  constexpr int BK = 64, LDK = 144;
+  constexpr int NT = (BM / WM) * (BN / WN) * 64;
+  constexpr int CA = BM * 8 / NT;                 // 16-byte activation chunks (8 bf16) per thread and K step
+  constexpr int CB = (BN * 2 + NT - 1) / NT;      // 16-byte packed weight chunks (32 elements) per thread and K step
+  static_assert(BM * 8 % NT == 0, "activation tile must split evenly over the threads");
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int STAGE = (BM + BN) * LDK;
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / (BN / WN), wn = wave % (BN / WN);
+  const int G = a.K / a.group, zpb = (G + 1) / 2;
+
+  const int tilesN = (a.N + BN - 1) / BN, tilesM = (a.M + BM - 1) / BM;
+  const int total = tilesM * tilesN;
+  int tile = blockIdx.x;
+  if (total % 8 == 0) tile = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;  // one run of tiles per XCD
+  const int m0 = (tile / tilesN) * BM, n0 = (tile % tilesN) * BN;
+
+  const __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.A), 0, (uint32_t)((int64_t)a.M * a.K * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rW = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.qw), 0, (uint32_t)((int64_t)a.N * a.K / 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rS = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.s), 0, (uint32_t)((int64_t)a.N * G * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rZ = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.zp), 0, (uint32_t)((int64_t)a.N * zpb), 0x00020000);
+
+  // activation chunk c: row = idx / 8, 16-byte column = idx % 8 ; weight chunk c: row = idx / 2, half = idx % 2
+  uint32_t offA[CA];
+#pragma unroll
+  for (int c = 0; c < CA; c++) {
+    const int idx = tid + c * NT, row = m0 + idx / 8;
+    offA[c] = row < a.M ? (uint32_t)(((int64_t)row * a.K + (idx % 8) * 8) * 2) : 0xffffffffu;
+  }
+  int wrow[CB];
+  bool wok[CB];
+#pragma unroll
+  for (int c = 0; c < CB; c++) {
+    const int idx = tid + c * NT;
+    wrow[c] = n0 + idx / 2;
+    wok[c] = idx < BN * 2 && wrow[c] < a.N;
+  }
+  u32x4 gA[CA], gW[CB];
+  uint16_t gS[CB];
+  uint8_t gZ[CB];
+  auto gload = [&](int k0) {
+#pragma unroll
+    for (int c = 0; c < CA; c++) {
+      const bool ok = offA[c] != 0xffffffffu && k0 + ((tid + c * NT) % 8) * 8 < a.K;
+      gA[c] = __builtin_amdgcn_raw_buffer_load_b128(rA, ok ? offA[c] + (uint32_t)k0 * 2u : 0xffffffffu, 0, 0);
+    }
+    const int g = k0 / a.group;
+#pragma unroll
+    for (int c = 0; c < CB; c++) {
+      const int half = (tid + c * NT) & 1;
+      const bool ok = wok[c] && k0 + half * 32 < a.K;
+      gW[c] = __builtin_amdgcn_raw_buffer_load_b128(rW, ok ? (uint32_t)(((int64_t)wrow[c] * a.K + k0 + half * 32) / 2) : 0xffffffffu, 0, 0);
+      gS[c] = __builtin_amdgcn_raw_buffer_load_b16(rS, ok ? (uint32_t)(((int64_t)wrow[c] * G + g) * 2) : 0xffffffffu, 0, 0);
+      gZ[c] = __builtin_amdgcn_raw_buffer_load_b8(rZ, ok ? (uint32_t)((int64_t)wrow[c] * zpb + (g >> 1)) : 0xffffffffu, 0, 0);
+    }
+  };
+  auto sstore = [&](int buf, int k0) {
+    unsigned char* base = smem + buf * STAGE;
+#pragma unroll
+    for (int c = 0; c < CA; c++) {
+      const int idx = tid + c * NT;
+      *reinterpret_cast<u32x4*>(base + (idx / 8) * LDK + (idx % 8) * 16) = gA[c];
+    }
+    const int g = k0 / a.group;
+#pragma unroll
+    for (int c = 0; c < CB; c++) {
+      const int idx = tid + c * NT;
+      if (idx < BN * 2) {
+        const float s = f16bits_to_f32(gS[c]);
+        const float z = (float)((g & 1) ? (gZ[c] >> 4) : (gZ[c] & 15));
+        const float nzs = -(z * s);  // exact: 4-bit integer times an 11-bit significand
+        const uint32_t w[4] = {gW[c].x, gW[c].y, gW[c].z, gW[c].w};
+        unsigned char* dst = base + (BM + idx / 2) * LDK + (idx & 1) * 64;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+          uint32_t o[4];
+          dequant8(w[j], s, nzs, o);
+          *reinterpret_cast<u32x4*>(dst + j * 16) = u32x4{o[0], o[1], o[2], o[3]};
+        }
+      }
+    }
+  };
+
+  v16f acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; i++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  const int KT = (a.K + BK - 1) / BK;
+  gload(0);
+  sstore(0, 0);
+  __syncthreads();
+  const int lrow = lane & 31, lk = (lane >> 5) * 16;
+  for (int kt = 0; kt < KT; kt++) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) gload((kt + 1) * BK);
+    const unsigned char* base = smem + buf * STAGE;
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) {
+      bf16x8 fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+        fa[i] = *reinterpret_cast<const bf16x8*>(base + (wm * WM + i * 32 + lrow) * LDK + ks * 32 + lk);
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+        fb[j] = *reinterpret_cast<const bf16x8*>(base + (BM + wn * WN + j * 32 + lrow) * LDK + ks * 32 + lk);
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < KT) sstore(buf ^ 1, (kt + 1) * BK);
+    __syncthreads();
+  }
+
+  // epilogue.  32x32 accumulator layout: register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int n = n0 + wn * WN + j * 32 + lrow;
+    const bool nok = n < a.N;
+    const float bn = (nok && a.bias) ? bf16_to_f32(a.bias[n]) : 0.f;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int m = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+        if (nok && m < a.M) {
+          float f = acc[i][j][r];
+          if (a.bias) f += bn;
+          a.C[(int64_t)m * a.N + n] = f32_to_bf16(f);
+        }
+      }
+    }
+  }
+}
+
+// dequantized weight table (parity probe and the definition of "dequantized weight values")
+__global__ void w4a16_dequant_kernel(const uint8_t* __restrict__ qw, const uint16_t* __restrict__ s,
+                                     const uint8_t* __restrict__ zp, uint16_t* __restrict__ w, int64_t N, int64_t K, int group) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // one packed dword = 8 elements
+  if (i >= N * K / 8) return;
+  const int64_t n = i / (K / 8), k = (i % (K / 8)) * 8;
+  const int G = (int)(K / group), zpb = (G + 1) / 2, g = (int)(k / group);
+  const float sc = f16bits_to_f32(s[n * G + g]);
+  const uint8_t zb = zp[n * zpb + (g >> 1)];
+  const float z = (float)((g & 1) ? (zb >> 4) : (zb & 15));
+  const uint32_t word = *reinterpret_cast<const uint32_t*>(qw + (n * K + k) / 2);
+  uint32_t o[4];
+  dequant8(word, sc, -(z * sc), o);
+  *reinterpret_cast<u32x4*>(w + n * K + k) = u32x4{o[0], o[1], o[2], o[3]};
+}
+
+template <int BM, int BN, int WM, int WN>
+static int launch_w4a16(const W4A16Args& a, hipStream_t st) {
+  constexpr int NT = (BM / WM) * (BN / WN) * 64;
+  const size_t lds = 2 * (size_t)(BM + BN) * 144;
+  const unsigned grid = (unsigned)(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN));
+  auto kern = w4a16_gemm_kernel<BM, BN, WM, WN>;
+  if (lds > 64 * 1024)
+    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds, st, a);
+  return (int)hipGetLastError();
+}
+
+static int g_w4a16_tile = 0;  // 0 = heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64
+
+}  // namespace mllmhip
+
+using namespace mllmhip;
+
+MLLM_API int mllm_hip_w4a16_set_tuning(int tile) {
+  if (tile < 0 || tile > 3) return MLLM_HIP_E_BADARG;
+  g_w4a16_tile = tile;
+  return 0;
+}
+
+static int check_w4a16(const void* qw, const void* s, const void* zp, int64_t N, int64_t K, int group) {
+  if (!qw || !s || !zp || N <= 0 || K <= 0 || group <= 0) return MLLM_HIP_E_BADARG;
+  if (group % 64 || K % group) return MLLM_HIP_E_SHAPE;
+  if (N * K / 2 >= ((int64_t)1 << 32) || N > INT32_MAX || K > INT32_MAX) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(qw) % 16) return MLLM_HIP_E_ALIGN;
+  return 0;
+}
+
+MLLM_API int mllm_hip_w4a16_gemm(const void* a_bf16, const uint8_t* qw, const uint16_t* scales, const uint8_t* zeros,
+                                 const void* bias_bf16, void* c_bf16, int64_t M, int64_t N, int64_t K, int group,
+                                 void* stream) {
+  int rc = check_w4a16(qw, scales, zeros, N, K, group);
+  if (rc) return rc;
+  if (!a_bf16 || !c_bf16 || M <= 0) return MLLM_HIP_E_BADARG;
+  if (M * K * 2 >= ((int64_t)1 << 32) || M > INT32_MAX) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(a_bf16) % 16) return MLLM_HIP_E_ALIGN;
+  W4A16Args a{(const uint16_t*)a_bf16, qw, scales, zeros, (const uint16_t*)bias_bf16, (uint16_t*)c_bf16,
+              (int)M, (int)N, (int)K, group};
+  hipStream_t st = (hipStream_t)stream;
+  int tile = g_w4a16_tile;
+  if (!tile) {
+    const int64_t big = ((M + 255) / 256) * ((N + 191) / 192);
+    const int64_t mid = ((M + 127) / 128) * ((N + 127) / 128);
+    tile = (M >= 256 && big >= 192) ? 1 : (mid >= 128 ? 2 : 3);
+  }
+  switch (tile) {
+    case 1: return launch_w4a16<256, 192, 128, 96>(a, st);
+    case 2: return launch_w4a16<128, 128, 64, 64>(a, st);
+    default: return launch_w4a16<64, 64, 32, 32>(a, st);
+  }
+}
+
+MLLM_API int mllm_hip_w4a16_dequantize(const uint8_t* qw, const uint16_t* scales, const uint8_t* zeros, void* w_bf16,
+                                       int64_t N, int64_t K, int group, void* stream) {
+  int rc = check_w4a16(qw, scales, zeros, N, K, group);
+  if (rc) return rc;
+  if (!w_bf16) return MLLM_HIP_E_BADARG;
+  const int64_t words = N * K / 8;
+  hipLaunchKernelGGL(w4a16_dequant_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, (hipStream_t)stream, qw,
+                     scales, zeros, (uint16_t*)w_bf16, N, K, group);
+  return (int)hipGetLastError();
+}

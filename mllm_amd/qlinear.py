@@ -134,3 +134,24 @@ def w8a8_linear(x, W, w_scale, bias=None, workspace=None, out=None):
     _lib.check(L.mllm_hip_w8a8_linear(x.data_ptr(), _xdtype(x), W.data_ptr(), w_scale.data_ptr(), _p(bias),
                                       y.data_ptr(), M, N, K, workspace.data_ptr(), _stream()), "mllm_hip_w8a8_linear")
     return y
+
+
+# ----------------------------------------------------------------------------- W4A16 (group-wise uint4 + zero point)
+def w4a16_gemm(a, qw, scales, zeros, bias=None, group=128, out=None):
+    """a bf16 [M, K]; qw uint8 [N, K/2]; scales fp16 [N, K/group]; zeros uint8 [N, ceil(K/group/2)] -> bf16 [M, N]."""
+    assert a.dtype == torch.bfloat16 and a.is_contiguous() and qw.dtype == torch.uint8 and scales.dtype == torch.float16
+    M, K = a.shape
+    N = qw.shape[0]
+    assert qw.shape[1] * 2 == K
+    y = out if out is not None else torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_w4a16_gemm(a.data_ptr(), qw.data_ptr(), scales.data_ptr(), zeros.data_ptr(), _p(bias),
+                                              y.data_ptr(), M, N, K, group, _stream()), "mllm_hip_w4a16_gemm")
+    return y
+
+
+def w4a16_dequantize(qw, scales, zeros, group=128):
+    N, K = qw.shape[0], qw.shape[1] * 2
+    w = torch.empty((N, K), dtype=torch.bfloat16, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_w4a16_dequantize(qw.data_ptr(), scales.data_ptr(), zeros.data_ptr(), w.data_ptr(), N, K,
+                                                    group, _stream()), "mllm_hip_w4a16_dequantize")
+    return w
