@@ -138,6 +138,29 @@ int mllm_hip_w4a16_dequantize(const uint8_t* qw, const uint16_t* scales, const u
 /* GEMM tile override for tuning sweeps: 0 heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64 workgroup tiles. */
 int mllm_hip_w4a16_set_tuning(int tile);
 
+/* ---------------------------------------------------------------------------------------------------------
+ * MoE expert FFN over expert-sorted tokens, Q4_0 / Q8_0 expert weights
+ * replaces: Qwen3MoE::moeInfer + Qwen3MoeMLP::forward (one CPULinearOp::forward per expert and projection)
+ *           mllm/models/qwen3_moe/modeling_qwen3_moe_fa2.hpp:98-100,175-238
+ * ------------------------------------------------------------------------------------------------------- */
+
+/* y[t] = sum_j topk_w[t][j] * down_e( silu(gate_e(x[t])) * up_e(x[t]) ),  e = topk_ids[t][j], j ascending.
+ * Every projection is the block-quantized Linear above (activations re-quantized to Q8_0 in front of each one).
+ * gate_packed / up_packed: E pre-packed [I][H] matrices back to back, expert e at + e * mllm_hip_q_packed_bytes(wtype, I, H);
+ * down_packed: E pre-packed [H][I] matrices, stride mllm_hip_q_packed_bytes(wtype, H, I).
+ * x [T][H] fp32 or bf16; topk_ids int32 [T][k] (entries outside [0, E) contribute nothing); topk_w fp32 [T][k];
+ * y fp32 [T][H].  H % 32 == 0, I % 32 == 0, E <= 4096.  workspace: mllm_hip_moe_workspace_bytes. */
+size_t mllm_hip_moe_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k);
+int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x,
+                       int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H,
+                       int64_t I, int E, int k, int act_scale_mode, void* workspace, void* stream);
+
+/* Routing probe: tokens per expert (counts [E]), exclusive prefix (offsets [E+1]) and the flat (t*k + j) index at every
+ * expert-sorted position (sorted_idx [T*k]); any output may be NULL.  workspace as for mllm_hip_moe_ffn_q.
+ * replaces: the histogram + argsort at modeling_qwen3_moe_fa2.hpp:178-197 */
+int mllm_hip_moe_route(const int32_t* topk_ids, int64_t T, int E, int k, int32_t* counts, int32_t* offsets,
+                       int32_t* sorted_idx, void* workspace, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

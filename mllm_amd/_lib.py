@@ -51,6 +51,13 @@ def lib():
         L.mllm_hip_w4a16_gemm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp]
         L.mllm_hip_w4a16_dequantize.argtypes = [vp, vp, vp, vp, i64, i64, ci, vp]
         L.mllm_hip_w4a16_set_tuning.argtypes = [ci]
+        L.mllm_hip_linear_q_workspace_bytes.restype = C.c_size_t
+        L.mllm_hip_linear_q_workspace_bytes.argtypes = [i64, i64]
+        L.mllm_hip_linear_q.argtypes = [ci, vp, vp, ci, vp, vp, i64, i64, i64, ci, vp, vp]
+        L.mllm_hip_moe_workspace_bytes.restype = C.c_size_t
+        L.mllm_hip_moe_workspace_bytes.argtypes = [i64, i64, i64, ci, ci]
+        L.mllm_hip_moe_ffn_q.argtypes = [ci, vp, vp, vp, vp, ci, vp, vp, vp, i64, i64, i64, ci, ci, ci, vp, vp]
+        L.mllm_hip_moe_route.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, vp]
         _lib = L
     return _lib
 

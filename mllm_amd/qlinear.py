@@ -155,3 +155,78 @@ def w4a16_dequantize(qw, scales, zeros, group=128):
     _lib.check(_lib.lib().mllm_hip_w4a16_dequantize(qw.data_ptr(), scales.data_ptr(), zeros.data_ptr(), w.data_ptr(), N, K,
                                                     group, _stream()), "mllm_hip_w4a16_dequantize")
     return w
+
+
+# ----------------------------------------------------------------------------- any-M quantized Linear and the MoE FFN
+def linear_q(w, x, bias=None, act_scale_mode=SCALE_X86_REF, workspace=None, out=None):
+    """Q4_0/Q8_0 Linear for any number of rows: stand-alone Q8_0 activation quantization + MFMA block-dot tiles."""
+    assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
+    M = x.shape[0]
+    L = _lib.lib()
+    if workspace is None:
+        workspace = torch.empty(L.mllm_hip_linear_q_workspace_bytes(M, w.K), dtype=torch.uint8, device="cuda")
+    y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")
+    _lib.check(L.mllm_hip_linear_q(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K,
+                                   act_scale_mode, workspace.data_ptr(), _stream()), "mllm_hip_linear_q")
+    return y
+
+
+class PackedExperts:
+    """E pre-packed [N, K] weight matrices back to back (the layout mllm_hip_moe_ffn_q takes)."""
+
+    def __init__(self, wtype, blocks, weight_scale_mode=SCALE_IEEE):
+        """blocks: uint8 [E, N, K/32, 18|34] (host or device)."""
+        assert blocks.dtype == torch.uint8 and blocks.dim() == 4
+        self.wtype, self.E, self.N, self.K = wtype, blocks.shape[0], blocks.shape[1], blocks.shape[2] * 32
+        L = _lib.lib()
+        self.stride = L.mllm_hip_q_packed_bytes(wtype, self.N, self.K)
+        self.buf = torch.empty(self.E * self.stride, dtype=torch.uint8, device="cuda")
+        for e in range(self.E):
+            dev = blocks[e].contiguous().cuda()
+            _lib.check(L.mllm_hip_q_prepack(wtype, dev.data_ptr(), weight_scale_mode,
+                                            self.buf.data_ptr() + e * self.stride, self.N, self.K, _stream()),
+                       "mllm_hip_q_prepack")
+            torch.cuda.current_stream().synchronize()
+
+    @classmethod
+    def synthetic(cls, wtype, E, N, K, generator=None):
+        nb = K // 32
+        blocks = torch.randint(0, 256, (E, N, nb, BLOCK_BYTES[wtype]), dtype=torch.uint8, device="cuda", generator=generator)
+        if wtype == Q8_0:
+            blocks[blocks == 0x80] = 0x81
+        s = (torch.randn((E, N, nb), device="cuda", generator=generator) * 0.02).abs() / 7.0
+        bits = s.to(torch.float16).view(torch.int16) & ~7
+        blocks[:, :, :, 0:2] = bits.view(torch.uint8).view(E, N, nb, 2)
+        return cls(wtype, blocks)
+
+    @property
+    def ptr(self):
+        return self.buf.data_ptr()
+
+
+def moe_ffn_q(gate, up, down, x, topk_ids, topk_w, act_scale_mode=SCALE_X86_REF, workspace=None, out=None):
+    """x [T, H]; topk_ids int32 [T, k]; topk_w fp32 [T, k]; gate/up PackedExperts [E, I, H]; down [E, H, I] -> y fp32 [T, H]."""
+    T, H = x.shape
+    k = topk_ids.shape[1]
+    E, I = gate.E, gate.N
+    assert gate.K == H and up.N == I and down.N == H and down.K == I and topk_ids.dtype == torch.int32
+    L = _lib.lib()
+    if workspace is None:
+        workspace = torch.empty(L.mllm_hip_moe_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
+    y = out if out is not None else torch.empty((T, H), dtype=torch.float32, device="cuda")
+    _lib.check(L.mllm_hip_moe_ffn_q(gate.wtype, gate.ptr, up.ptr, down.ptr, x.data_ptr(), _xdtype(x), topk_ids.data_ptr(),
+                                    topk_w.data_ptr(), y.data_ptr(), T, H, I, E, k, act_scale_mode, workspace.data_ptr(),
+                                    _stream()), "mllm_hip_moe_ffn_q")
+    return y
+
+
+def moe_route(topk_ids, E):
+    T, k = topk_ids.shape
+    L = _lib.lib()
+    ws = torch.empty(L.mllm_hip_moe_workspace_bytes(T, 32, 32, E, k), dtype=torch.uint8, device="cuda")
+    counts = torch.empty(E, dtype=torch.int32, device="cuda")
+    offsets = torch.empty(E + 1, dtype=torch.int32, device="cuda")
+    sidx = torch.empty(T * k, dtype=torch.int32, device="cuda")
+    _lib.check(L.mllm_hip_moe_route(topk_ids.data_ptr(), T, E, k, counts.data_ptr(), offsets.data_ptr(), sidx.data_ptr(),
+                                    ws.data_ptr(), _stream()), "mllm_hip_moe_route")
+    return counts, offsets, sidx
