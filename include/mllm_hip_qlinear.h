@@ -161,6 +161,14 @@ int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed
 int mllm_hip_moe_route(const int32_t* topk_ids, int64_t T, int E, int k, int32_t* counts, int32_t* offsets,
                        int32_t* sorted_idx, void* workspace, void* stream);
 
+/* ---------------------------------------------------------------------------------------------------------
+ * fp32 activation x activation MatMul (the backend's kMatMul slot; not a quantized path)
+ * replaces: CPUMatMulOp::forward  mllm/backends/cpu/ops/MatMulOp.cpp:47-61
+ * C[M][N] = op(A) * op(B), op(X) = X or X^T; A is [M][K] ([K][M] when transposed), B is [K][N] ([N][K] when transposed).
+ * ------------------------------------------------------------------------------------------------------- */
+int mllm_hip_matmul_f32(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K, int transpose_a,
+                        int transpose_b, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -12,6 +12,8 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libmllm_hip_qlinear.so")
+HOST_LIB = os.path.join(LIBDIR, "libmllm_hip_backend.so")  # C++ op-factory layer on top of the C ABI
+HOST = os.path.join(CSRC, "host")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # no fast-math: the activation quantization needs correctly rounded fp32 division and plain multiplies;
@@ -47,7 +49,23 @@ def build(keep_asm=False, jobs=8):
                        capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n" + r.stderr)
+    build_host()
     return LIB
+
+
+def build_host():
+    """The C++ host layer (mllm-compatible Backend / ops) as its own library, linked against the kernel library."""
+    srcs = sorted(os.path.join(HOST, f) for f in os.listdir(HOST) if f.endswith(".cpp"))
+    cmd = [HIPCC, "-x", "hip", "--offload-arch=gfx950", "-O2", "-std=c++20", "-fPIC", "-shared", "-fvisibility=hidden",
+           "-I" + os.path.join(ROOT, "include"), "-I" + HOST, "-Wall", "-o", HOST_LIB] + srcs + [
+           "-L" + LIBDIR, "-lmllm_hip_qlinear", "-Wl,-rpath,$ORIGIN", "-ldl"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if r.returncode != 0:
+        raise RuntimeError("host layer build failed:\n" + err)
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return HOST_LIB
 
 
 if __name__ == "__main__":

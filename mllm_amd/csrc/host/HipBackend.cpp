@@ -1,0 +1,253 @@
+#include "HipBackend.hpp"
+
+#include <hip/hip_runtime_api.h>
+
+#include <cstring>
+
+#include "mllm_hip_qlinear.h"
+
+namespace mllm::hip {
+
+#define MLLM_HIP_CHECK(expr)                                                                              \
+  do {                                                                                                    \
+    hipError_t e__ = (expr);                                                                              \
+    if (e__ != hipSuccess) MLLM_ERROR_EXIT(ExitCode::kHIPError, "%s failed: %s", #expr, hipGetErrorString(e__)); \
+  } while (0)
+// kernels report through return codes; the op turns a failure into the runtime's fatal path
+#define MLLM_HIP_KERNEL_CHECK(expr)                                                                     \
+  do {                                                                                                  \
+    int rc__ = (expr);                                                                                  \
+    if (rc__ != 0) MLLM_ERROR_EXIT(ExitCode::kHIPError, "%s failed with code %d", #expr, rc__);          \
+  } while (0)
+
+// ---- allocator ------------------------------------------------------------------------------------------------
+bool HipAllocator::alloc(Storage* storage) {
+  void* p = nullptr;
+  if (hipMalloc(&p, storage->size_ ? storage->size_ : 256) != hipSuccess) return false;
+  storage->ptr_ = p;
+  return true;
+}
+void HipAllocator::free(Storage* storage) {
+  if (storage->ptr_) (void)hipFree(storage->ptr_);
+  storage->ptr_ = nullptr;
+}
+bool HipAllocator::generalAlloc(void** ptr, size_t cap, size_t) { return hipMalloc(ptr, cap) == hipSuccess; }
+void HipAllocator::generalFree(void* ptr) { (void)hipFree(ptr); }
+size_t HipAllocator::allocSize(Storage* storage) { return (storage->size_ + 255) / 256 * 256; }
+
+// ---- backend ---------------------------------------------------------------------------------------------------
+HipBackend::HipBackend(const HipBackendConfig& cfg) : Backend(kHIP, std::make_shared<HipAllocator>()), cfg_(cfg) {
+  MLLM_HIP_CHECK(hipSetDevice(cfg_.device));
+  MLLM_HIP_KERNEL_CHECK(mllm_hip_init(cfg_.device));
+  hipStream_t st;
+  MLLM_HIP_CHECK(hipStreamCreate(&st));
+  stream_ = st;
+  regOpFactory<HipLinearOpFactory, HipMatMulOpFactory, HipX2XOpFactory>();
+}
+HipBackend::~HipBackend() {
+  if (stream_) (void)hipStreamDestroy((hipStream_t)stream_);
+}
+void HipBackend::synchronize() const { MLLM_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream_)); }
+
+std::shared_ptr<HipBackend> initHipBackend() {
+  auto& ctx = Context::instance();
+  if (ctx.hasBackend(kHIP)) return std::static_pointer_cast<HipBackend>(ctx.getBackend(kHIP));
+  HipBackendConfig cfg;
+  if (const char* m = std::getenv("MLLM_HIP_SCALE_MODE")) {
+    if (std::strcmp(m, "x86") == 0) cfg.weight_scale_mode = cfg.act_scale_mode = MLLM_HIP_SCALE_X86_REF;
+  }
+  auto backend = std::make_shared<HipBackend>(cfg);
+  ctx.registerBackend(backend);
+  ctx.memoryManager()->registerAllocator(kHIP, backend->allocator());
+  return backend;
+}
+
+static HipBackend& backend() { return *std::static_pointer_cast<HipBackend>(Context::instance().getBackend(kHIP)); }
+
+// ---- X2X -------------------------------------------------------------------------------------------------------
+void HipX2XOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  MLLM_RT_ASSERT_EQ(inputs.size(), 1u);
+  MLLM_RT_ASSERT_EQ(outputs.size(), 1u);
+  const auto& in = inputs[0];
+  auto& out = outputs[0];
+  const size_t n = in.bytes();
+  auto st = (hipStream_t)backend().stream();
+  if (in.device() == kCPU && out.device() == kHIP) {
+    MLLM_HIP_CHECK(hipMemcpyAsync(out.ptr<void>(), in.ptr<void>(), n, hipMemcpyHostToDevice, st));
+    MLLM_HIP_CHECK(hipStreamSynchronize(st));  // the host buffer may be released by the caller right after
+  } else if (in.device() == kHIP && out.device() == kCPU) {
+    MLLM_HIP_CHECK(hipStreamSynchronize(st));  // everything queued on the device is finished before the copy back
+    MLLM_HIP_CHECK(hipMemcpy(out.ptr<void>(), in.ptr<void>(), n, hipMemcpyDeviceToHost));
+  } else if (in.device() == kHIP && out.device() == kHIP) {
+    if (in.ptr<void>() != out.ptr<void>()) MLLM_HIP_CHECK(hipMemcpyAsync(out.ptr<void>(), in.ptr<void>(), n, hipMemcpyDeviceToDevice, st));
+  } else {
+    NYI("X2X between devices %d and %d", (int)in.device(), (int)out.device());
+  }
+}
+
+// ---- MatMul -----------------------------------------------------------------------------------------------------
+void HipMatMulOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  const auto& a = inputs[0];
+  const auto& b = inputs[1];
+  auto& c = outputs[0];
+  if (a.dtype() != kFloat32 || b.dtype() != kFloat32) NYI("HipMatMulOp supports fp32 operands only");
+  const auto& cs = c.shape();
+  const int64_t M = cs[cs.size() - 2], N = cs[cs.size() - 1];
+  const auto& as = a.shape();
+  const int64_t K = options_.transpose_a ? as[as.size() - 2] : as[as.size() - 1];
+  int64_t batch = 1;
+  for (size_t i = 0; i + 2 < cs.size(); i++) batch *= cs[i];
+  const bool b_batched = b.rank() == a.rank() && b.rank() > 2;
+  for (int64_t i = 0; i < batch; i++) {
+    MLLM_HIP_KERNEL_CHECK(mllm_hip_matmul_f32(a.ptr<float>() + i * M * K, b.ptr<float>() + (b_batched ? i * N * K : 0),
+                                              c.ptr<float>() + i * M * N, M, N, K, options_.transpose_a, options_.transpose_b,
+                                              backend().stream()));
+  }
+}
+
+// ---- Linear ------------------------------------------------------------------------------------------------------
+HipLinearOp::HipLinearOp(const aops::LinearOpOptions& options) : aops::LinearOp(options) {}
+
+static Tensor onDevice(const Tensor& t) { return t.device() == kHIP ? t : t.to(kHIP); }
+
+void HipLinearOp::load(const ParameterFile::ptr_t& ploader) {
+  aops::LinearOp::load(ploader);  // "<name>.weight" viewed [out, in], "<name>.bias"
+  const int64_t N = options_.out_channels, K = options_.in_channels;
+  auto& be = backend();
+  switch (weight_.dtype()) {  // the weight's dtype selects the path, as the reference's device backends do
+    case kGGUF_Q4_0:
+    case kGGUF_Q8_0: {
+      scheme_ = weight_.dtype() == kGGUF_Q4_0 ? Scheme::kQ4_0 : Scheme::kQ8_0;
+      const int wt = scheme_ == Scheme::kQ4_0 ? MLLM_HIP_Q4_0 : MLLM_HIP_Q8_0;
+      MLLM_RT_ASSERT_EQ((int64_t)weight_.numel(), N * K);
+      const size_t pb = mllm_hip_q_packed_bytes(wt, N, K);
+      if (pb == 0) MLLM_ERROR_EXIT(ExitCode::kCoreError, "Linear %s: in_channels %d is not a multiple of 32", getName().c_str(), (int)K);
+      Tensor dev_blocks = onDevice(weight_);
+      packed_ = Tensor::empty({(int32_t)pb}, kByte, kHIP).alloc();
+      MLLM_HIP_KERNEL_CHECK(mllm_hip_q_prepack(wt, dev_blocks.ptr<void>(), be.config().weight_scale_mode, packed_.ptr<void>(), N, K, be.stream()));
+      be.synchronize();  // dev_blocks is released when it goes out of scope
+      if (options_.bias) bias_dev_ = onDevice(bias_);
+      break;
+    }
+    case kInt8: {
+      scheme_ = Scheme::kW8A8;
+      weight_ = onDevice(weight_);
+      weight_scale_ = onDevice(ploader->pull(getName() + ".weight.scale"));
+      MLLM_RT_ASSERT_EQ(weight_scale_.dtype(), kFloat32);
+      MLLM_RT_ASSERT_EQ((int64_t)weight_scale_.numel(), N);
+      if (options_.bias) bias_dev_ = onDevice(bias_);
+      break;
+    }
+    case kUInt8:
+    case kByte: {
+      scheme_ = Scheme::kW4A16;  // two uint4 codes per byte, [N][K/2]
+      MLLM_RT_ASSERT_EQ((int64_t)weight_.numel(), N * K / 2);
+      weight_ = onDevice(weight_);
+      weight_scale_ = onDevice(ploader->pull(getName() + ".weight.scale"));
+      weight_zp_ = onDevice(ploader->pull(getName() + ".weight.zero_point"));
+      MLLM_RT_ASSERT_EQ(weight_scale_.dtype(), kFloat16);
+      const int64_t G = (int64_t)weight_scale_.numel() / N;
+      MLLM_RT_ASSERT(G > 0 && K % G == 0);
+      group_ = (int)(K / G);
+      if (options_.bias) {
+        MLLM_RT_ASSERT_EQ(bias_.dtype(), kBFloat16);
+        bias_dev_ = onDevice(bias_);
+      }
+      break;
+    }
+    default: NYI("HipLinearOp: weight dtype %d", (int)weight_.dtype());
+  }
+}
+
+void HipLinearOp::reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  if (options_.isRedirect()) {
+    outputs.emplace_back(inputs[1]);
+    return;
+  }
+  const auto& i = inputs[0];
+  auto o_shape = i.shape();
+  MLLM_RT_ASSERT_EQ(o_shape[o_shape.size() - 1], options_.in_channels);
+  o_shape[o_shape.size() - 1] = options_.out_channels;
+  // block-quantized weights produce fp32 like the CPU backend's kGGUF path (mllm/backends/cpu/ops/LinearOp.cpp:357-360)
+  const DataTypes o_dtype = (scheme_ == Scheme::kQ4_0 || scheme_ == Scheme::kQ8_0) ? kFloat32 : kBFloat16;
+  outputs.emplace_back(Tensor::empty(o_shape, o_dtype, i.device()));
+}
+
+void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  const auto& x = inputs[0];
+  auto& y = outputs[0];
+  MLLM_RT_ASSERT_EQ(x.device(), kHIP);
+  const int64_t K = options_.in_channels, N = options_.out_channels;
+  const int64_t M = (int64_t)x.numel() / K;  // all leading dimensions are rows
+  auto& be = backend();
+  void* st = be.stream();
+  auto xdt = [&]() {
+    if (x.dtype() == kFloat32) return MLLM_HIP_F32;
+    if (x.dtype() == kBFloat16) return MLLM_HIP_BF16;
+    MLLM_ERROR_EXIT(ExitCode::kCoreError, "HipLinearOp: activation dtype %d not supported", (int)x.dtype());
+  };
+  auto workspace = [&](size_t bytes) {
+    if (workspace_.isNil() || workspace_.bytes() < bytes) workspace_ = Tensor::empty({(int32_t)bytes}, kByte, kHIP).alloc();
+    return workspace_.ptr<void>();
+  };
+  const float* bias = bias_dev_.isNil() ? nullptr : bias_dev_.ptr<float>();
+  switch (scheme_) {
+    case Scheme::kQ4_0:
+    case Scheme::kQ8_0: {
+      const int wt = scheme_ == Scheme::kQ4_0 ? MLLM_HIP_Q4_0 : MLLM_HIP_Q8_0;
+      if (M <= 8) {
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), (int)M, N, K,
+                                                     be.config().act_scale_mode, st));
+      } else {
+        void* ws = workspace(mllm_hip_linear_q_workspace_bytes(M, K));
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K,
+                                                be.config().act_scale_mode, ws, st));
+      }
+      break;
+    }
+    case Scheme::kW8A8: {
+      void* ws = workspace(mllm_hip_w8a8_workspace_bytes(M, K));
+      MLLM_HIP_KERNEL_CHECK(mllm_hip_w8a8_linear(x.ptr<void>(), xdt(), weight_.ptr<int8_t>(), weight_scale_.ptr<float>(), bias, y.ptr<void>(), M,
+                                                 N, K, ws, st));
+      break;
+    }
+    case Scheme::kW4A16: {
+      MLLM_RT_ASSERT_EQ(x.dtype(), kBFloat16);
+      MLLM_HIP_KERNEL_CHECK(mllm_hip_w4a16_gemm(x.ptr<void>(), weight_.ptr<uint8_t>(), weight_scale_.ptr<uint16_t>(), weight_zp_.ptr<uint8_t>(),
+                                                bias_dev_.isNil() ? nullptr : bias_dev_.ptr<void>(), y.ptr<void>(), M, N, K, group_, st));
+      break;
+    }
+    default: MLLM_ERROR_EXIT(ExitCode::kCoreError, "HipLinearOp::forward before load()");
+  }
+}
+
+ParameterFile::ptr_t HipLinearOp::getParams() {
+  auto p = aops::LinearOp::getParams();
+  if (!weight_scale_.isNil()) p->push(getName() + ".weight.scale", weight_scale_);
+  if (!weight_zp_.isNil()) p->push(getName() + ".weight.zero_point", weight_zp_);
+  return p;
+}
+
+}  // namespace mllm::hip
+
+// ---- out-of-tree route: the plugin C ABI (adds the ops under names; it cannot replace kLinear, see PluginSystem.cpp:82-90)
+extern "C" {
+static void* createHipLinearFactory() { return new mllm::hip::HipLinearOpFactory(); }
+static void freeHipLinearFactory(void* f) { delete static_cast<mllm::hip::HipLinearOpFactory*>(f); }
+static void* createHipMatMulFactory() { return new mllm::hip::HipMatMulOpFactory(); }
+static void freeHipMatMulFactory(void* f) { delete static_cast<mllm::hip::HipMatMulOpFactory*>(f); }
+
+__attribute__((visibility("default"))) void* opPackageDescriptor() {
+  auto* pkg = new PluginOpPackageDescriptor();
+  std::snprintf(pkg->name, sizeof(pkg->name), "MllmHipQLinear");
+  pkg->device_type = (int32_t)mllm::kHIP;
+  pkg->op_factories_count = 2;
+  std::snprintf(pkg->op_factories_names[0], MLLM_PLUGIN_OP_PACKAGE_NAME_LEN, "hip_linear");
+  std::snprintf(pkg->op_factories_names[1], MLLM_PLUGIN_OP_PACKAGE_NAME_LEN, "hip_matmul");
+  pkg->op_factory_create_funcs[0] = createHipLinearFactory;
+  pkg->op_factory_create_funcs[1] = createHipMatMulFactory;
+  pkg->op_factory_free_funcs[0] = freeHipLinearFactory;
+  pkg->op_factory_free_funcs[1] = freeHipMatMulFactory;
+  return pkg;
+}
+}

@@ -1,0 +1,99 @@
+// HIP backend for mllm's op-factory boundary: allocator, backend, and the Linear / MatMul / X2X ops, on top of the C ABI
+// in include/mllm_hip_qlinear.h.
+//
+// Follows the pattern of the reference's device backends:
+//   registration      mllm/backends/opencl/OpenCLBackend.cpp:32-44, mllm/backends/ascend/Register.cpp:15-42
+//   factories         mllm/backends/cpu/ops/LinearOp.hpp:21-26, mllm/backends/ascend/AscendBackend.cpp:31-50
+//   device allocator  mllm/backends/cuda/CudaAllocator.cpp:10-65
+//   weight-side names mllm/backends/ascend/ops/AscendLinearOp.cpp:42-48 ("<name>.weight.scale")
+#pragma once
+#include "mllm_core.hpp"
+
+namespace mllm::hip {
+
+class HipAllocator final : public Allocator {
+ public:
+  bool ctrlByMemManager() override { return false; }
+  bool alloc(Storage* storage) override;
+  bool alloc(const Storage::ptr_t& storage) override { return alloc(storage.get()); }
+  void free(Storage* storage) override;
+  void free(const Storage::ptr_t& storage) override { free(storage.get()); }
+  bool generalAlloc(void** ptr, size_t cap, size_t align) override;
+  void generalFree(void* ptr) override;
+  size_t allocSize(Storage* storage) override;
+  size_t allocSize(const Storage::ptr_t& storage) override { return allocSize(storage.get()); }
+  [[nodiscard]] size_t alignSize() const override { return 256; }
+};
+
+// How fp16 block scales are read (see MLLM_HIP_SCALE_* in the C header): IEEE bit patterns, or the x86 reference build's
+// number-valued field.  Chosen per process: environment MLLM_HIP_SCALE_MODE = "ieee" (default) | "x86".
+struct HipBackendConfig {
+  int weight_scale_mode = 0;
+  int act_scale_mode = 0;
+  int device = 0;
+};
+
+class HipBackend final : public Backend {
+ public:
+  explicit HipBackend(const HipBackendConfig& cfg = HipBackendConfig());
+  ~HipBackend() override;
+  [[nodiscard]] void* stream() const { return stream_; }  // hipStream_t; default priority
+  [[nodiscard]] const HipBackendConfig& config() const { return cfg_; }
+  void setScaleModes(int weight_scale_mode, int act_scale_mode) {
+    cfg_.weight_scale_mode = weight_scale_mode;
+    cfg_.act_scale_mode = act_scale_mode;
+  }
+  void synchronize() const;
+
+ private:
+  HipBackendConfig cfg_;
+  void* stream_ = nullptr;
+};
+
+// Registers backend + allocator with the Context (idempotent).  The counterpart of initOpenCLBackend() / initAscendBackend().
+std::shared_ptr<HipBackend> initHipBackend();
+
+class HipLinearOp final : public aops::LinearOp {
+ public:
+  explicit HipLinearOp(const aops::LinearOpOptions& options);
+  void load(const ParameterFile::ptr_t& ploader) override;
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+  void forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+  ParameterFile::ptr_t getParams() override;
+
+ private:
+  enum class Scheme { kNone, kQ4_0, kQ8_0, kW8A8, kW4A16 };
+  Scheme scheme_ = Scheme::kNone;
+  Tensor packed_;        // Q4_0 / Q8_0: the repacked device copy the kernels read
+  Tensor weight_scale_;  // "<name>.weight.scale": fp32 [N] (W8A8) or fp16 [N][K/group] (W4A16)
+  Tensor weight_zp_;     // "<name>.weight.zero_point": uint8 [N][ceil(K/group/2)] (W4A16)
+  Tensor bias_dev_;      // bias in the form the kernel takes (fp32; bf16 for W4A16)
+  Tensor workspace_;
+  int group_ = 0;
+};
+class HipLinearOpFactory final : public TypedOpFactory<OpTypes::kLinear, aops::LinearOpOptions> {
+ public:
+  std::shared_ptr<BaseOp> createOpImpl(const aops::LinearOpOptions& options) override { return std::make_shared<HipLinearOp>(options); }
+};
+
+class HipMatMulOp final : public aops::MatMulOp {
+ public:
+  explicit HipMatMulOp(const aops::MatMulOpOptions& options) : aops::MatMulOp(options) {}
+  void forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+};
+class HipMatMulOpFactory final : public TypedOpFactory<OpTypes::kMatMul, aops::MatMulOpOptions> {
+ public:
+  std::shared_ptr<BaseOp> createOpImpl(const aops::MatMulOpOptions& options) override { return std::make_shared<HipMatMulOp>(options); }
+};
+
+class HipX2XOp final : public aops::X2XOp {
+ public:
+  explicit HipX2XOp(const aops::X2XOpOptions& options) : aops::X2XOp(options) {}
+  void forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+};
+class HipX2XOpFactory final : public TypedOpFactory<OpTypes::kX2X, aops::X2XOpOptions> {
+ public:
+  std::shared_ptr<BaseOp> createOpImpl(const aops::X2XOpOptions& options) override { return std::make_shared<HipX2XOp>(options); }
+};
+
+}  // namespace mllm::hip

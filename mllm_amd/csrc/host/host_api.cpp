@@ -1,0 +1,120 @@
+// A plain-C doorway into the C++ backend for callers (and tests) that cannot include the C++ headers: runs one Linear
+// through exactly the sequence mllm's runtime uses for a device op,
+//   initializeContext + initHipBackend -> Backend::createOp(kLinear, LinearOpOptions) -> load(ParameterFile)
+//   -> Tensor::to(kHIP) (X2X) -> reshape -> setup -> forward -> Tensor::to(kCPU)
+// (mllm/nn/Layer.cpp:13-34,53-82, mllm/backends/cpu/CPUDispatcher.cpp:56-62).
+#include <cstring>
+#include <string>
+
+#include "HipBackend.hpp"
+#include "mllm_hip_qlinear.h"
+
+using namespace mllm;
+
+namespace {
+DataTypes weight_dtype(const std::string& scheme) {
+  if (scheme == "q4_0") return kGGUF_Q4_0;
+  if (scheme == "q8_0") return kGGUF_Q8_0;
+  if (scheme == "w8a8") return kInt8;
+  if (scheme == "w4a16") return kUInt8;
+  MLLM_ERROR_EXIT(ExitCode::kCoreError, "unknown scheme '%s'", scheme.c_str());
+}
+}  // namespace
+
+extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_linear(
+    const char* scheme_c, const void* weight_host, const void* scale_host, const void* zp_host, const void* bias_host,
+    const void* x_host, int x_is_bf16, void* y_host, int M, int N, int K, int group, int weight_scale_x86, int act_scale_x86, int via_plugin,
+    const char* plugin_path) {
+  const std::string scheme(scheme_c);
+  initializeContext();
+  auto be = hip::initHipBackend();
+  be->setScaleModes(weight_scale_x86 ? MLLM_HIP_SCALE_X86_REF : MLLM_HIP_SCALE_IEEE,
+                    act_scale_x86 ? MLLM_HIP_SCALE_X86_REF : MLLM_HIP_SCALE_IEEE);
+  auto& ctx = Context::instance();
+
+  // a parameter file holding host tensors that borrow the caller's memory
+  auto params = ParameterFile::create(ModelFileVersion::kV2);
+  const std::string name = "model.layers.0.proj";
+  const DataTypes wdt = weight_dtype(scheme);
+  if (wdt == kUInt8)
+    params->push(name + ".weight", Tensor::fromExternal(const_cast<void*>(weight_host), {N, K / 2}, kUInt8, kCPU));
+  else
+    params->push(name + ".weight", Tensor::fromExternal(const_cast<void*>(weight_host), {N, K}, wdt, kCPU));
+  if (scheme == "w8a8") params->push(name + ".weight.scale", Tensor::fromExternal(const_cast<void*>(scale_host), {N}, kFloat32, kCPU));
+  if (scheme == "w4a16") {
+    const int G = K / group;
+    params->push(name + ".weight.scale", Tensor::fromExternal(const_cast<void*>(scale_host), {N, G}, kFloat16, kCPU));
+    params->push(name + ".weight.zero_point", Tensor::fromExternal(const_cast<void*>(zp_host), {N, (G + 1) / 2}, kUInt8, kCPU));
+  }
+  if (bias_host)
+    params->push(name + ".bias", Tensor::fromExternal(const_cast<void*>(bias_host), {N}, scheme == "w4a16" ? kBFloat16 : kFloat32, kCPU));
+
+  aops::LinearOpOptions opts;
+  opts.in_channels = K;
+  opts.out_channels = N;
+  opts.bias = bias_host != nullptr;
+  opts.impl_type = aops::LinearImplTypes::kDefault;
+
+  BaseOp::ptr_t op;
+  if (via_plugin) {
+    // out-of-tree route: the op package is looked up by name after dlopen (tests/plugin/HostTest.cpp:5-12 in the reference)
+    static bool loaded = false;
+    if (!loaded) {
+      loadOpPackage(plugin_path);
+      loaded = true;
+    }
+    op = ctx.getBackend(kHIP)->createOp((OpTypes)ctx.lookupCustomizedOpId(kHIP, "hip_linear"), opts);
+  } else {
+    op = ctx.getBackend(kHIP)->createOp(OpTypes::kLinear, opts);
+  }
+  op->setName(name);
+  op->load(params);
+
+  Tensor x = Tensor::fromExternal(const_cast<void*>(x_host), {1, M, K}, x_is_bf16 ? kBFloat16 : kFloat32, kCPU).to(kHIP);
+  std::vector<Tensor> inputs{x}, outputs;
+  op->reshape(inputs, outputs);
+  op->setup(inputs, outputs);
+  op->forward(inputs, outputs);
+  Tensor y = outputs[0].to(kCPU);
+  if ((int)y.shape().size() != 3 || y.shape()[1] != M || y.shape()[2] != N) return -10;
+  std::memcpy(y_host, y.ptr<void>(), y.bytes());
+  // getParams() must hand back every tensor load() needs
+  auto back = op->getParams();
+  if (!back->has(name + ".weight")) return -11;
+  if ((scheme == "w8a8" || scheme == "w4a16") && !back->has(name + ".weight.scale")) return -12;
+  return (int)y.dtype();
+}
+
+// fp32 MatMul through the kMatMul factory slot
+extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_matmul(const float* a_host, const float* b_host, float* c_host,
+                                                                                  int M, int N, int K, int transpose_b) {
+  initializeContext();
+  hip::initHipBackend();
+  auto& ctx = Context::instance();
+  Tensor a = Tensor::fromExternal(const_cast<float*>(a_host), {M, K}, kFloat32, kCPU).to(kHIP);
+  Tensor b = Tensor::fromExternal(const_cast<float*>(b_host), transpose_b ? Tensor::shape_t{N, K} : Tensor::shape_t{K, N}, kFloat32, kCPU).to(kHIP);
+  aops::MatMulOpOptions o;
+  o.transpose_b = transpose_b != 0;
+  auto outs = ctx.buildOpAndSubmitTask(OpTypes::kMatMul, o, {a, b});
+  Tensor c = outs[0].to(kCPU);
+  std::memcpy(c_host, c.ptr<void>(), c.bytes());
+  return 0;
+}
+
+// error-path probe for the CPU tests: asks a backend that was never registered for an op (the runtime's behaviour is to
+// terminate the process, mllm/engine/Context.cpp:37-42) -- run in a child process.
+extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_probe_missing_backend() {
+  initializeContext();
+  Context::instance().getBackend(kHIP);
+  return 0;
+}
+// type-erased options of the wrong type must throw std::bad_cast (mllm/core/BaseOp.hpp:132-136)
+extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_probe_bad_cast() {
+  hip::HipLinearOpFactory f;
+  try {
+    f.create(aops::MatMulOpOptions{});
+  } catch (const std::bad_cast&) {
+    return 1;
+  }
+  return 0;
+}
