@@ -37,6 +37,86 @@ def parse():
     return ap.parse_args()
 
 
+def side_workloads(torch, ql, synth, gen):
+    """The other configurations of the metric: W8A8 / W4A16 prefill GEMMs (MFMA-bound) and the MoE expert FFN."""
+    def ev_time(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / reps
+
+    out = {}
+    # W8A8 prefill: A bf16 [2048,2048] with 1 % outliers x20, W int8 [6144,2048]
+    M, N, K = 2048, 6144, 2048
+    a = torch.randn((M, K), device="cuda", generator=gen)
+    a = torch.where(torch.rand((M, K), device="cuda", generator=gen) < 0.01, a * 20, a).to(torch.bfloat16)
+    Ws = [torch.randint(-127, 128, (N, K), dtype=torch.int8, device="cuda", generator=gen) for _ in range(4)]
+    ws = (torch.rand(N, device="cuda", generator=gen) + 0.01) * 0.01
+    q, sc = ql.per_token_quant_int8(a)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    wsp = torch.empty(_lib_ws(ql, "w8a8", M, K), dtype=torch.uint8, device="cuda")
+    i = [0]
+
+    def gemm():
+        ql.w8a8_gemm(q, sc, Ws[i[0] % 4], ws, None, out=y)
+        i[0] += 1
+
+    def fused():
+        ql.w8a8_linear(a, Ws[i[0] % 4], ws, None, workspace=wsp, out=y)
+        i[0] += 1
+    tg, tq, tf = ev_time(gemm, 20), ev_time(lambda: ql.per_token_quant_int8(a), 20), ev_time(fused, 20)
+    ops = 2.0 * M * N * K
+    out["w8a8_prefill_2048x6144x2048"] = {
+        "gemm_us": tg * 1e6, "gemm_TOPS": ops / tg / 1e12, "gemm_frac_of_5000_TOPS": ops / tg / 5e15,
+        "quant_us": tq * 1e6, "quant_GBps": (M * K * 3 + M * 4) / tq / 1e9,
+        "quant_plus_gemm_us": tf * 1e6, "quant_plus_gemm_TOPS": ops / tf / 1e12}
+    del Ws
+    # W4A16 prefill: A bf16 [2048,2560], W uint4 [9728,2560] g128
+    M, N, K = 2048, 9728, 2560
+    a = torch.randn((M, K), device="cuda", generator=gen).to(torch.bfloat16)
+    qws = [torch.randint(0, 256, (N, K // 2), dtype=torch.uint8, device="cuda", generator=gen) for _ in range(3)]
+    s4 = (torch.randn((N, K // 128), device="cuda", generator=gen).abs() * 0.01).to(torch.float16)
+    zp = torch.randint(0, 256, (N, K // 256), dtype=torch.uint8, device="cuda", generator=gen)
+    y = torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+
+    def g4():
+        ql.w4a16_gemm(a, qws[i[0] % 3], s4, zp, None, 128, out=y)
+        i[0] += 1
+    t4 = ev_time(g4, 10)
+    fl = 2.0 * M * N * K
+    out["w4a16_prefill_2048x9728x2560"] = {"us": t4 * 1e6, "TFLOPS": fl / t4 / 1e12, "frac_of_2500_TFLOPS": fl / t4 / 2.5e15}
+    del qws
+    # MoE FFN: 512 tokens, hidden 2048, 128 experts, top-8 Zipf(1.1), intermediate 768, Q4_0
+    import numpy as np
+    T, H, I, E, k = 512, 2048, 768, 128, 8
+    ids_np, w_np = synth.make_moe_routing(synth.rng_for(4), T, E, k)
+    ids, tw = torch.from_numpy(ids_np).cuda(), torch.from_numpy(w_np).cuda()
+    gate = ql.PackedExperts.synthetic(ql.Q4_0, E, I, H, gen)
+    up = ql.PackedExperts.synthetic(ql.Q4_0, E, I, H, gen)
+    down = ql.PackedExperts.synthetic(ql.Q4_0, E, H, I, gen)
+    x = torch.randn((T, H), device="cuda", generator=gen).to(torch.bfloat16)
+    wsm = torch.empty(_lib_ws(ql, "moe", T, H, I, E, k), dtype=torch.uint8, device="cuda")
+    ym = torch.empty((T, H), dtype=torch.float32, device="cuda")
+    tm = ev_time(lambda: ql.moe_ffn_q(gate, up, down, x, ids, tw, workspace=wsm, out=ym), 10)
+    active = int((np.bincount(ids_np.reshape(-1), minlength=E) > 0).sum())
+    wbytes = active * (2 * I * (H // 32) * 18 + H * (I // 32) * 18)
+    flops = T * k * (2.0 * H * I * 2 + 2.0 * I * H)
+    out["moe_ffn_512tok_128e_top8_q4_0"] = {"us": tm * 1e6, "active_experts": active, "weight_GBps": wbytes / tm / 1e9,
+                                            "frac_of_hbm_peak": wbytes / tm / 8e12, "TOPS": flops / tm / 1e12}
+    return out
+
+
+def _lib_ws(ql, which, *a):
+    from mllm_amd import _lib
+    L = _lib.lib()
+    return L.mllm_hip_w8a8_workspace_bytes(*a) if which == "w8a8" else L.mllm_hip_moe_workspace_bytes(*a)
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -150,6 +230,9 @@ def main():
                                             "gate_proj": measure_shape(other, M, "gate_proj", pool2, 3)}
         del pool2
         torch.cuda.empty_cache()
+
+    if not args.no_extra:
+        extra["prefill_and_moe"] = side_workloads(torch, ql, synth, gen)
 
     cpu = None
     if not args.no_cpu:
