@@ -67,6 +67,18 @@ int mllm_hip_q_prepack(int wtype, const void* blocks, int weight_scale_mode, voi
 int mllm_hip_linear_q_gemv(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y,
                            int M, int64_t N, int64_t K, int act_scale_mode, void* stream);
 
+/* Up to four Linears that share the activations and K in ONE launch (sibling projections: q/k/v, gate/up).  Per part the
+ * result equals mllm_hip_linear_q_gemv on that part; the point is fewer, larger launches (a decode-size matrix is a few
+ * MB, far below what hides the fixed cost of a launch).  `parts` is a host array, read during the call. */
+typedef struct {
+  const void* packed; /* pre-packed [N][K] weight                      */
+  const float* bias;  /* fp32 [N] or NULL                              */
+  float* y;           /* fp32 [M][N]                                   */
+  int64_t N;
+} mllm_hip_gemv_part;
+int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M,
+                                 int64_t K, int act_scale_mode, void* stream);
+
 /* Same for any M: quantizes the activations with a stand-alone kernel into `workspace`
  * (mllm_hip_linear_q_workspace_bytes) and runs the tiled block-dot kernel.  Used by prefill and by the MoE path. */
 size_t mllm_hip_linear_q_workspace_bytes(int64_t M, int64_t K);

@@ -11,6 +11,11 @@ LIB_PATH = os.path.join(_HERE, "lib", "libmllm_hip_qlinear.so")
 _lib = None
 
 
+class GemvPart(C.Structure):
+    """mllm_hip_gemv_part"""
+    _fields_ = [("packed", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p), ("N", C.c_int64)]
+
+
 class HipQLinearError(RuntimeError):
     pass
 
@@ -38,6 +43,7 @@ def lib():
         L.mllm_hip_q_packed_bytes.argtypes = [ci, i64, i64]
         L.mllm_hip_q_prepack.argtypes = [ci, vp, ci, vp, i64, i64, vp]
         L.mllm_hip_linear_q_gemv.argtypes = [ci, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]
+        L.mllm_hip_linear_q_gemv_multi.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_quantize_q8_0.argtypes = [vp, ci, vp, vp, i64, i64, vp]
         L.mllm_hip_q_dequantize.argtypes = [ci, vp, vp, i64, i64, vp]
         L.mllm_hip_q_block_isums.argtypes = [ci, vp, vp, vp, i64, i64, i64, vp]

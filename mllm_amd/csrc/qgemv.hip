@@ -202,30 +202,44 @@ MLLM_API int mllm_hip_q_prepack(int wtype, const void* blocks, int weight_scale_
   return (int)hipGetLastError();
 }
 
-MLLM_API int mllm_hip_linear_q_gemv(int wtype, const void* packed, const void* x, int x_dtype, const float* bias,
-                                    float* y, int M, int64_t N, int64_t K, int act_scale_mode, void* stream) {
-  int rc = check_w(wtype, packed, N, K);
-  if (rc) return rc;
-  if (!x || !y || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16)) return MLLM_HIP_E_BADARG;
+MLLM_API int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,
+                                          int M, int64_t K, int act_scale_mode, void* stream) {
+  if (nparts < 1 || nparts > GEMV_MAX_PARTS || !parts) return MLLM_HIP_E_BADARG;
+  if (!x || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16)) return MLLM_HIP_E_BADARG;
   if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
   if (M < 1 || M > 8) return MLLM_HIP_E_SHAPE;
   if (reinterpret_cast<uintptr_t>(x) % 16) return MLLM_HIP_E_ALIGN;
-  GemvArgs a;
-  a.w = packed_view(wtype, packed, N, K);
+  GemvArgs a{};
+  int64_t nmax = 0;
+  for (int p = 0; p < nparts; p++) {
+    int rc = check_w(wtype, parts[p].packed, parts[p].N, K);
+    if (rc) return rc;
+    if (!parts[p].y) return MLLM_HIP_E_BADARG;
+    a.part[p].w = packed_view(wtype, parts[p].packed, parts[p].N, K);
+    a.part[p].bias = parts[p].bias;
+    a.part[p].y = parts[p].y;
+    a.part[p].N = (int)parts[p].N;
+    nmax += parts[p].N;
+  }
+  a.nparts = nparts;
   a.x = x;
-  a.bias = bias;
-  a.y = y;
   a.M = M;
-  a.N = (int)N;
   a.nb = (int)(K / QK);
   a.nbp = (int)scale_row_stride(K);
   a.x86_scale = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8));
-  const GemvShape s = pick_shape(MT, N, a.nb);
+  const GemvShape s = pick_shape(MT, nmax, a.nb);
   hipStream_t st = (hipStream_t)stream;
   if (wtype == MLLM_HIP_Q4_0)
     return x_dtype == MLLM_HIP_F32 ? launch_gemv_q4_f32(a, MT, s, st) : launch_gemv_q4_bf16(a, MT, s, st);
   return x_dtype == MLLM_HIP_F32 ? launch_gemv_q8_f32(a, MT, s, st) : launch_gemv_q8_bf16(a, MT, s, st);
+}
+
+MLLM_API int mllm_hip_linear_q_gemv(int wtype, const void* packed, const void* x, int x_dtype, const float* bias,
+                                    float* y, int M, int64_t N, int64_t K, int act_scale_mode, void* stream) {
+  if (!y) return MLLM_HIP_E_BADARG;
+  mllm_hip_gemv_part part{packed, bias, y, N};
+  return mllm_hip_linear_q_gemv_multi(wtype, 1, &part, x, x_dtype, M, K, act_scale_mode, stream);
 }
 
 MLLM_API int mllm_hip_quantize_q8_0(const void* x, int x_dtype, int8_t* codes, uint16_t* d_bits, int64_t M, int64_t K,

@@ -15,13 +15,21 @@
 
 namespace mllmhip {
 
-struct GemvArgs {
+// One launch serves up to four weight matrices that share the activations and K (sibling projections: q/k/v, gate/up):
+// workgroups [wg_start[p], wg_start[p+1]) belong to part p.
+constexpr int GEMV_MAX_PARTS = 4;
+struct GemvPart {
   PackedView w;
-  const void* x;
   const float* bias;
   float* y;
-  int M;          // actual rows of x (<= MT)
   int N;
+};
+struct GemvArgs {
+  GemvPart part[GEMV_MAX_PARTS];
+  int wg_start[GEMV_MAX_PARTS + 1];
+  int nparts;
+  const void* x;
+  int M;          // actual rows of x (<= MT)
   int nb;         // K / 32
   int nbp;        // scale row stride (nb rounded up to 8)
   int x86_scale;  // reproduce the x86 storage rounding of the activation scale
@@ -147,6 +155,13 @@ template <int WT, int XT, int MT, int G, int R, int U, bool SCL>
 __global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int nb = a.nb, nbp = a.nbp;
+  int pidx = 0;  // uniform: which matrix this workgroup works on
+#pragma unroll
+  for (int p = 1; p < GEMV_MAX_PARTS; p++)
+    if (p < a.nparts && (int)blockIdx.x >= a.wg_start[p]) pidx = p;
+  const GemvPart& pt = a.part[pidx];
+  const int bid = blockIdx.x - a.wg_start[pidx];
+  const int N = pt.N;
   const int mnb = MT * nb;
   u32x4* s_lo = reinterpret_cast<u32x4*>(smem);
   u32x4* s_hi = s_lo + mnb;
@@ -162,7 +177,7 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
   constexpr int ROWS_W = GROUPS * R;  // weight rows of one wave
   const int grp = lane / G;
   const int c0 = lane % G;
-  const int64_t wrow0 = ((int64_t)blockIdx.x * nwaves + wave) * ROWS_W;
+  const int64_t wrow0 = ((int64_t)bid * nwaves + wave) * ROWS_W;
   const int64_t row0 = wrow0 + (int64_t)grp * R;
   uint16_t* s_ws = reinterpret_cast<uint16_t*>(smem + align_up((size_t)mnb * 40, 16)) + (size_t)wave * ROWS_W * nbp;
 
@@ -175,7 +190,7 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
   load_x8<XT>(a.x, (int64_t)min(tid + nthreads, valid_items - 1) * 8, raw1);
 
   // ---- 2. block scales of this wave's rows: chunks of 8 scales (16 bytes), lane L takes chunks L and L+64 ------
-  const WRsrc wr = make_wrsrc(a.w, WT, a.N, nb, nbp);
+  const WRsrc wr = make_wrsrc(pt.w, WT, N, nb, nbp);
   const int cpr = nbp >> 3;  // chunks per row
   u32x4 sc[2];
   if (SCL) {
@@ -183,7 +198,7 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
     for (int k = 0; k < 2; k++) {
       const int ch = lane + 64 * k;
       const int rw = ch / cpr, cc = ch - rw * cpr;
-      const bool ok = rw < ROWS_W && wrow0 + rw < a.N;
+      const bool ok = rw < ROWS_W && wrow0 + rw < N;
       sc[k] = __builtin_amdgcn_raw_buffer_load_b128(wr.d, ok ? (uint32_t)(((wrow0 + rw) * nbp + cc * 8) * 2) : BUF_OOB, 0, BUF_NT);
     }
   }
@@ -195,7 +210,7 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
   uint32_t rbase[R], dbase[R];
 #pragma unroll
   for (int r = 0; r < R; r++) {
-    rbase[r] = (row0 + r < a.N) ? (uint32_t)((row0 + r) * nb) : BUF_OOB;
+    rbase[r] = (row0 + r < N) ? (uint32_t)((row0 + r) * nb) : BUF_OOB;
     dbase[r] = (uint32_t)((row0 + r) * nbp);
   }
   WChunk<WT, R, U, SCL> cur;
@@ -304,17 +319,23 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
     for (int m = 0; m < MT; m++) {
       float v = group_sum<G>(acc[r][m]);
       const int64_t row = row0 + r;
-      if (c0 == 0 && row < a.N && m < a.M) a.y[(int64_t)m * a.N + row] = a.bias ? a.bias[row] + v : v;
+      if (c0 == 0 && row < N && m < a.M) pt.y[(int64_t)m * N + row] = pt.bias ? pt.bias[row] + v : v;
     }
 }
 
 // ---- launchers ---------------------------------------------------------------------------------------------------
 template <int WT, int XT, int MT, int G, int R>
-static int launch_gemv_u(const GemvArgs& a, int NW, hipStream_t st) {
+static int launch_gemv_u(const GemvArgs& a_in, int NW, hipStream_t st) {
   constexpr int U = ((R >= 4) ? 1 : (R == 2 ? 2 : 4)) * (WT == MLLM_HIP_Q4_0 ? 2 : 1);
   constexpr int ROWS_W = (64 / G) * R;
   const int rows_per_wg = NW * ROWS_W;
-  const unsigned grid = (unsigned)((a.N + rows_per_wg - 1) / rows_per_wg);
+  GemvArgs a = a_in;
+  unsigned grid = 0;
+  for (int p = 0; p < a.nparts; p++) {
+    a.wg_start[p] = (int)grid;
+    grid += (unsigned)((a.part[p].N + rows_per_wg - 1) / rows_per_wg);
+  }
+  a.wg_start[a.nparts] = (int)grid;
   const bool scl = ROWS_W * (a.nbp / 8) <= 128;
   const size_t lds = align_up((size_t)MT * a.nb * 40, 16) + (scl ? (size_t)NW * ROWS_W * a.nbp * 2 : 0);
   if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;

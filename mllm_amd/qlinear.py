@@ -84,6 +84,22 @@ def linear_q_gemv(w, x, bias=None, act_scale_mode=SCALE_X86_REF, out=None):
     return y
 
 
+def linear_q_gemv_multi(ws, x, biases=None, act_scale_mode=SCALE_X86_REF, outs=None):
+    """Sibling projections (same x, same K) in one launch.  ws: list of PackedQWeight; returns the list of outputs."""
+    assert 1 <= len(ws) <= 4 and x.is_cuda and x.is_contiguous() and x.dim() == 2
+    M, K = x.shape
+    if outs is None:
+        outs = [torch.empty((M, w.N), dtype=torch.float32, device="cuda") for w in ws]
+    parts = (_lib.GemvPart * len(ws))()
+    for i, w in enumerate(ws):
+        assert w.K == K and w.wtype == ws[0].wtype
+        b = biases[i] if biases is not None else None
+        parts[i] = _lib.GemvPart(w.ptr, b.data_ptr() if b is not None else None, outs[i].data_ptr(), w.N)
+    _lib.check(_lib.lib().mllm_hip_linear_q_gemv_multi(ws[0].wtype, len(ws), parts, x.data_ptr(), _xdtype(x), M, K,
+                                                       act_scale_mode, _stream()), "mllm_hip_linear_q_gemv_multi")
+    return outs
+
+
 def quantize_q8_0(x):
     """x [M, K] -> (codes int8 [M, K], scale patterns int16-viewed-as-uint16 [M, K/32])."""
     assert x.is_cuda and x.is_contiguous() and x.dim() == 2

@@ -196,3 +196,26 @@ def test_gemv_argument_errors():
     assert L.mllm_hip_q_packed_bytes(0, 8, 48) == 0
     with pytest.raises(_lib.HipQLinearError):
         _lib.check(-2, "probe")
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M", [1, 3, 8])
+def test_gemv_multi_equals_single(wtype, M):
+    """sibling projections in one launch give exactly the bits of one launch each (q/k/v and gate/up shapes)"""
+    rng = synth.rng_for(1, 70 + M + wtype)
+    for shapes in ([(4096, 2560), (1024, 2560), (1024, 2560)], [(9728, 2560), (9728, 2560)], [(40, 96), (7, 96), (33, 96), (1, 96)]):
+        K = shapes[0][1]
+        Ws = [synth.make_weight(rng, wtype, n, K) for n, _ in shapes]
+        ws = [ql.PackedQWeight(wtype, torch.from_numpy(W)) for W in Ws]
+        biases = [to_dev(rng.standard_normal(n).astype(np.float32)) for n, _ in shapes]
+        bits, xf = synth.make_x_bf16(rng, M, K)
+        xd = bf16_dev(bits)
+        announce("gemv multi", wtype, M, shapes)
+        outs = ql.linear_q_gemv_multi(ws, xd, biases)
+        for w, W, b, o in zip(ws, Ws, biases, outs):
+            single = ql.linear_q_gemv(w, xd, b)
+            assert torch.equal(o, single)
+            assert rel_l2(o.cpu().numpy(), orc.linear_q(xf, W, wtype, b.cpu().numpy(), orc.SCALE_X86_REF)) < 2e-6
+    L = _lib.lib()
+    assert L.mllm_hip_linear_q_gemv_multi(0, 5, None, None, 0, 1, 64, 0, None) == -1
+    assert L.mllm_hip_linear_q_gemv_multi(0, 0, None, None, 0, 1, 64, 0, None) == -1
