@@ -2,13 +2,14 @@
 """Benchmark of the quantized-Linear hot path on one MI355X.
 
 Workload (the configuration the metric is quoted on): the seven Linear projections of a Qwen3-4B decoder layer as decode
-GEMVs with Q4_0 weights, bf16 activations, M = 1.  One step = one decode token through all 36 layers = 252 GEMV launches
-over 2.04 GB of distinct weights (far larger than the 256 MB last-level cache, so every step streams from HBM).
-The launches of a step are captured once into a HIP graph and replayed.
+GEMVs with Q4_0 weights, bf16 activations, M = 1.  One step = one decode token through all 36 layers over 2.04 GB of
+distinct weights (far larger than the 256 MB last-level cache, so every step streams from HBM).  Projections that read
+the same activations share a launch (q/k/v, gate/up): 4 launches per layer, 144 per step; --per-op gives one launch per
+projection (252 per step).  The launches of a step are captured once into a HIP graph and replayed.
 
 Prints ONE JSON line.  `value` is whole-job algorithmic GB/s (weights 18 B per 32-element block + activations + outputs,
-divided by wall time of the timed steps, inputs resident in HBM).  `roofline` is the dominant GEMV shape alone
-(gate/up projection), timed with HIP events on the launch stream.  `cpu_baseline` times the CPU oracle of the same path on a
+divided by wall time of the timed steps, inputs resident in HBM).  `roofline` is the dominant GEMV launch alone
+(gate+up projection), timed with HIP events on the launch stream.  `cpu_baseline` times the CPU oracle of the same path on a
 bounded sample on the host cores.
 """
 import argparse
@@ -31,6 +32,11 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--wtype", choices=["q4_0", "q8_0"], default="q4_0")
     ap.add_argument("--m", type=int, default=1, help="activation rows of the headline workload (1..8)")
+    ap.add_argument("--per-op", action="store_true",
+                    help="one launch per projection (7 per layer) instead of sibling projections sharing a launch (4 per layer)")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="counter run: 20 launches of the dominant GEMV launch and 20 of a plain copy of the same byte count, "
+                         "nothing else; meant to run under rocprofv3 --pmc FETCH_SIZE (or WRITE_SIZE)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the M=4/8 and Q8_0 side measurements")
@@ -149,9 +155,19 @@ def main():
         return N_LAYERS * sum(synth.gemv_algorithmic_bytes(wtype, M, n, k, 2) for n, k in shapes.values())
 
     def run_step(pool, xs, ys):
-        for layer in pool:
-            for name, w in layer.items():
-                ql.linear_q_gemv(w, xs[w.K], None, ql.SCALE_X86_REF, out=ys[name])
+        """one decode token: per layer q/k/v in one launch, o, gate/up in one launch, down (4 launches)"""
+        if args.per_op:
+            for layer in pool:
+                for name, w in layer.items():
+                    ql.linear_q_gemv(w, xs[w.K], None, ql.SCALE_X86_REF, out=ys[name])
+            return
+        for l in pool:
+            ql.linear_q_gemv_multi([l["q_proj"], l["k_proj"], l["v_proj"]], xs[2560], None, ql.SCALE_X86_REF,
+                                   [ys["q_proj"], ys["k_proj"], ys["v_proj"]])
+            ql.linear_q_gemv(l["o_proj"], xs[4096], None, ql.SCALE_X86_REF, out=ys["o_proj"])
+            ql.linear_q_gemv_multi([l["gate_proj"], l["up_proj"]], xs[2560], None, ql.SCALE_X86_REF,
+                                   [ys["gate_proj"], ys["up_proj"]])
+            ql.linear_q_gemv(l["down_proj"], xs[9728], None, ql.SCALE_X86_REF, out=ys["down_proj"])
 
     def timed(fn, steps, warmup):
         """warmup, then `steps` calls bracketed by synchronize; returns (wall seconds, HIP-event seconds)"""
@@ -186,39 +202,61 @@ def main():
                 "bytes_per_step": nbytes}
 
     def measure_shape(wtype, M, name, pool, reps=5):
-        """one GEMV shape alone over every layer's distinct copy of it: HIP-event average per launch"""
-        n, k = shapes[name]
+        """one GEMV launch shape alone over every layer's distinct copy of it: HIP-event average per launch.
+        "gate_up" / "qkv" are the sibling launches (two / three matrices, one launch)."""
+        groups = {"gate_up": ["gate_proj", "up_proj"], "qkv": ["q_proj", "k_proj", "v_proj"]}.get(name, [name])
+        k = shapes[groups[0]][1]
         x = torch.randn((M, k), device="cuda", generator=gen).to(torch.bfloat16)
-        y = torch.empty((M, n), dtype=torch.float32, device="cuda")
-        ws = [layer[name] for layer in pool]
+        ys = [torch.empty((M, shapes[g][0]), dtype=torch.float32, device="cuda") for g in groups]
+        sets = [[layer[g] for g in groups] for layer in pool]
         if name == "gate_proj":
-            ws += [layer["up_proj"] for layer in pool]
+            sets += [[layer["up_proj"]] for layer in pool]
 
         def fn():
-            for w in ws:
-                ql.linear_q_gemv(w, x, None, ql.SCALE_X86_REF, out=y)
+            for ws in sets:
+                if len(ws) == 1:
+                    ql.linear_q_gemv(ws[0], x, None, ql.SCALE_X86_REF, out=ys[0])
+                else:
+                    ql.linear_q_gemv_multi(ws, x, None, ql.SCALE_X86_REF, ys)
         replay = graphed(fn)
         _, ev = timed(replay, reps, 2)
-        per = ev / (reps * len(ws))
-        nbytes = synth.gemv_algorithmic_bytes(wtype, M, n, k, 2)
-        return {"us": per * 1e6, "GBps": nbytes / per / 1e9, "bytes": nbytes, "launches": reps * len(ws)}
+        per = ev / (reps * len(sets))
+        nbytes = sum(synth.gemv_algorithmic_bytes(wtype, M, shapes[g][0], k, 2) for g in groups) - (len(groups) - 1) * M * k * 2
+        return {"us": per * 1e6, "GBps": nbytes / per / 1e9, "bytes": nbytes, "launches": reps * len(sets)}
 
     wtype = ql.Q4_0 if args.wtype == "q4_0" else ql.Q8_0
+    if args.pmc_probe:
+        pool = make_pool(wtype, 20)
+        x = torch.randn((args.m, 2560), device="cuda", generator=gen).to(torch.bfloat16)
+        ys = [torch.empty((args.m, 9728), dtype=torch.float32, device="cuda") for _ in range(2)]
+        nbytes = 2 * synth.gemv_algorithmic_bytes(wtype, args.m, 9728, 2560, 2) // 16 * 16
+        src = torch.randint(0, 255, (20, nbytes), dtype=torch.uint8, device="cuda", generator=gen)
+        dst = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        torch.cuda.synchronize()
+        for l in pool:
+            ql.linear_q_gemv_multi([l["gate_proj"], l["up_proj"]], x, None, ql.SCALE_X86_REF, ys)
+        for i in range(20):
+            _lib.check(_lib.lib().mllm_hip_probe_copy(dst.data_ptr(), src[i].data_ptr(), nbytes, stream.cuda_stream), "probe_copy")
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc_probe": True, "gemv_algorithmic_bytes": nbytes, "copy_bytes_read": nbytes, "copy_bytes_written": nbytes}))
+        return
     pool = make_pool(wtype, N_LAYERS)
     torch.cuda.synchronize()
 
     head = measure_workload(wtype, args.m, pool, args.steps, args.warmup)
-    per_shape = {name: measure_shape(wtype, args.m, name, pool) for name in ("gate_proj", "down_proj", "q_proj", "o_proj", "k_proj")}
-    dom = per_shape["gate_proj"]
+    per_shape = {name: measure_shape(wtype, args.m, name, pool)
+                 for name in ("gate_up", "qkv", "gate_proj", "down_proj", "q_proj", "o_proj", "k_proj")}
+    dom_name = "gate_proj" if args.per_op else "gate_up"
+    dom = per_shape[dom_name]
 
     extra = {"per_shape": per_shape, "event_ms_per_step": head["event_ms_per_step"],
-             "graph": not args.no_graph, "layers": N_LAYERS, "launches_per_step": N_LAYERS * len(shapes)}
+             "graph": not args.no_graph, "layers": N_LAYERS, "launches_per_step": N_LAYERS * (len(shapes) if args.per_op else 4)}
     if not args.no_extra:
         for M in (4, 8):
             if M != args.m:
                 r = measure_workload(wtype, M, pool, max(5, args.steps // 3), 2)
                 extra["%s_m%d" % (args.wtype, M)] = {"GBps": r["GBps"], "ms_per_step": r["ms_per_step"],
-                                                     "gate_proj": measure_shape(wtype, M, "gate_proj", pool, 3)}
+                                                     dom_name: measure_shape(wtype, M, dom_name, pool, 3)}
         del pool
         torch.cuda.empty_cache()
         other = ql.Q8_0 if wtype == ql.Q4_0 else ql.Q4_0
@@ -227,11 +265,26 @@ def main():
         for M in (1, 4, 8):
             r = measure_workload(other, M, pool2, max(5, args.steps // 3), 2)
             extra["%s_m%d" % (oname, M)] = {"GBps": r["GBps"], "ms_per_step": r["ms_per_step"],
-                                            "gate_proj": measure_shape(other, M, "gate_proj", pool2, 3)}
+                                            dom_name: measure_shape(other, M, dom_name, pool2, 3)}
         del pool2
         torch.cuda.empty_cache()
 
     if not args.no_extra:
+        # what a stream of launches of this size can reach at all: a read-only 16-byte streaming kernel over distinct buffers
+        floor = {}
+        big = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device="cuda", generator=gen)
+        for nb_ in (1483776, 5919744, 14052352, 28099584, 56199168):
+            n = nb_ // 16 * 16
+            offs = [(i * 57000000) % ((1 << 30) - n) // 256 * 256 for i in range(40)]
+
+            def fl():
+                for o in offs:
+                    _lib.lib().mllm_hip_probe_copy(None, big.data_ptr() + o, n, stream.cuda_stream)
+            rp = graphed(fl)
+            _, ev = timed(rp, 5, 2)
+            floor[str(n)] = {"us": ev / (5 * 40) * 1e6, "GBps": n / (ev / (5 * 40)) / 1e9}
+        del big
+        extra["read_only_floor"] = floor
         extra["prefill_and_moe"] = side_workloads(torch, ql, synth, gen)
 
     cpu = None
@@ -263,12 +316,19 @@ def main():
         "ms_per_step": round(head["ms_per_step"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": "Qwen3-4B decoder-layer decode GEMVs (q/k/v/o/gate/up/down), %s weights, bf16 x, M=%d; "
-                               "one step = 36 layers x 7 projections = 252 launches over %.2f GB of distinct weights"
-                               % (args.wtype.upper(), args.m, head["bytes_per_step"] / 1e9),
+                               "one step = one decode token through 36 layers, %s, over %.2f GB of distinct weights"
+                               % (args.wtype.upper(), args.m,
+                                  "one launch per projection (252 launches)" if args.per_op else
+                                  "sibling projections share a launch: qkv | o | gate+up | down (144 launches)",
+                                  head["bytes_per_step"] / 1e9),
                    "M": args.m, "weights": args.wtype, "percent_of_hbm_peak": round(100 * head["GBps"] / HBM_PEAK_GBS, 2)},
         "roofline": {"bound": "hbm", "achieved": round(dom["GBps"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(dom["GBps"] / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "gemv_q_kernel gate/up_proj N=9728 K=2560 M=%d" % args.m, "us_per_launch": round(dom["us"], 3),
+                     "frac": round(dom["GBps"] / HBM_PEAK_GBS, 4),
+                     # FETCH_SIZE + WRITE_SIZE per dispatch from two rocprofv3 --pmc runs of `bench.py --pmc-probe`, each scaled
+                     # by what the counter reads for the library's plain copy kernel of the same size
+                     "traffic": 28159986 if (wtype == ql.Q4_0 and args.m == 1 and not args.per_op) else None,
+                     "kernel": ("gemv_q_kernel gate_proj N=9728 K=2560 M=%d" if args.per_op else
+                                "gemv_q_kernel gate+up in one launch, 2 x (N=9728 K=2560), M=%d") % args.m, "us_per_launch": round(dom["us"], 3),
                      "algorithmic_bytes_per_launch": dom["bytes"]},
         "cpu_baseline": cpu,
         "extra": extra,

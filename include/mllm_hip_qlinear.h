@@ -97,6 +97,10 @@ int mllm_hip_q_dequantize(int wtype, const void* packed, float* w, int64_t N, in
 int mllm_hip_q_block_isums(int wtype, const void* packed, const int8_t* codes, int32_t* isums, int64_t M, int64_t N,
                            int64_t K, void* stream);
 
+/* Measurement yardstick: copies `bytes` (a multiple of 16) from src to dst with 16-byte accesses, or only reads src when
+ * dst is NULL.  Used to calibrate HBM traffic counters and to measure the fixed cost of a launch of a given size. */
+int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
+
 /* GEMV launch-shape override for tuning sweeps: lanes per weight row (8/16/32/64), rows per lane group (1/2/4),
  * waves per workgroup (1..16); 0 restores the built-in heuristic. */
 int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_per_wg);

@@ -108,6 +108,30 @@ __global__ void block_isums_kernel(int wtype, PackedView w, const int8_t* __rest
   out[i] = isum;
 }
 
+// plain copy / read kernels of known size: the yardstick for HBM counters and for the per-launch floor of a stream
+__global__ __launch_bounds__(256) void probe_copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, size_t n16) {
+  const size_t base = (size_t)blockIdx.x * 256 * 8 + threadIdx.x;
+  u32x4 v[8];
+#pragma unroll
+  for (int u = 0; u < 8; u++) {
+    const size_t i = base + (size_t)u * 256;
+    v[u] = u32x4{0, 0, 0, 0};
+    if (i < n16) v[u] = __builtin_nontemporal_load(&src[i]);
+  }
+  if (dst) {
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const size_t i = base + (size_t)u * 256;
+      if (i < n16) dst[i] = v[u];
+    }
+  } else {  // read only: keep the loads alive without writing
+    uint32_t a = 0;
+#pragma unroll
+    for (int u = 0; u < 8; u++) a ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    __asm__ volatile("" ::"v"(a));
+  }
+}
+
 // ---- launch-shape selection ------------------------------------------------------------------------------
 static int g_tune_G = 0, g_tune_R = 0, g_tune_NW = 0;
 
@@ -156,6 +180,15 @@ MLLM_API int mllm_hip_init(int device) {
   HIP_RET(hipGetDeviceProperties(&prop, device));
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return MLLM_HIP_E_NODEVICE;
   return 0;
+}
+
+MLLM_API int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream) {
+  if (!src || bytes == 0 || bytes % 16) return MLLM_HIP_E_BADARG;
+  if (reinterpret_cast<uintptr_t>(src) % 16 || reinterpret_cast<uintptr_t>(dst) % 16) return MLLM_HIP_E_ALIGN;
+  const size_t n16 = bytes / 16;
+  hipLaunchKernelGGL(probe_copy_kernel, dim3((unsigned)((n16 + 2047) / 2048)), dim3(256), 0, (hipStream_t)stream, (u32x4*)dst,
+                     (const u32x4*)src, n16);
+  return (int)hipGetLastError();
 }
 
 MLLM_API int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_per_wg) {
