@@ -17,9 +17,9 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int TOK_TILE = 128;   // activation rows per workgroup tile (4 MFMA row tiles)
+constexpr int TOK_TILE = 64;    // activation rows per workgroup tile (2 MFMA row tiles)
 constexpr int TT = TOK_TILE / 32;
-constexpr int KCH = 64;         // blocks of activation scales staged in LDS at a time
+constexpr int KCH = 8;          // blocks per K chunk staged in LDS
 
 // ---------------------------------------------------------------------------------------------------------
 // routing: histogram, offsets, expert-sorted order and the tile list, one workgroup
@@ -51,15 +51,23 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const int32_t* __restri
       o.counts[e] = c;
       o.offsets[e] = off;
       s_cur[e] = off;
-      for (int r = 0; r < c; r += TOK_TILE) {
-        o.tile_expert[nt] = e;
-        o.tile_row0[nt] = off + r;
-        o.tile_rows[nt] = min(TOK_TILE, c - r);
-        nt++;
-      }
       off += c;
     }
     o.offsets[E] = off;
+    // tile list, full tiles first so that the long-running workgroups start early
+    for (int pass = 0; pass < 2; pass++)
+      for (int e = 0; e < E; e++) {
+        const int c = s_cnt[e], base = o.offsets[e];
+        for (int r = 0; r < c; r += TOK_TILE) {
+          const int rows = min(TOK_TILE, c - r);
+          if ((rows == TOK_TILE) == (pass == 0)) {
+            o.tile_expert[nt] = e;
+            o.tile_row0[nt] = base + r;
+            o.tile_rows[nt] = rows;
+            nt++;
+          }
+        }
+      }
     o.ntiles[0] = nt;
   }
   __syncthreads();
@@ -126,138 +134,200 @@ struct QGemmArgs {
   int x86_scale;
 };
 
-// weight operand of one block for the lane's output channel: lanes 0..31 supply elements 0..15, lanes 32..63 elements
-// 16..31 (Q4_0: low / high nibbles of the same 16 bytes; Q8_0: first / second code plane), as signed int8.
+// weight codes of one block for the lane's output channel as signed int8: lanes 0..31 supply elements 0..15, lanes 32..63
+// elements 16..31 (Q4_0: low / high nibbles of the same 16 bytes; Q8_0: first / second code plane).
 template <int WT>
-__device__ __forceinline__ v4i weight_operand(const PackedView& w, int64_t blk, int hi) {
+__device__ __forceinline__ v4i weight_operand(const u32x4& q, int hi) {
   if (WT == MLLM_HIP_Q4_0) {
-    const u32x4 q = w.q0[blk];
     const uint32_t sh = hi ? 4u : 0u;
-    v4i r;
     const uint32_t d[4] = {q.x, q.y, q.z, q.w};
+    v4i r;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
-      const uint32_t nib = (d[j] >> sh) & 0x0f0f0f0fu;               // bytes 0..15
-      r[j] = (int)((((nib | 0x80808080u) - 0x08080808u)) ^ 0x80808080u);  // per-byte (v - 8), no borrow between bytes
+      const uint32_t nib = (d[j] >> sh) & 0x0f0f0f0fu;                    // bytes 0..15
+      r[j] = (int)(((nib | 0x80808080u) - 0x08080808u) ^ 0x80808080u);    // per-byte (v - 8), no borrow between bytes
     }
     return r;
   } else {
-    const u32x4 q = hi ? w.q1[blk] : w.q0[blk];
     return v4i{(int)q.x, (int)q.y, (int)q.z, (int)q.w};
   }
 }
 
 __device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
 
-// MODE 0: out[o_index[pos]][n] = acc (+ bias)          one weight matrix
-// MODE 1: h = silu(acc0) * acc1, quantized to Q8_0     two weight matrices (gate, up) sharing the activations
+constexpr int PLANE = TOK_TILE * 16 + 16;          // LDS bytes of one (block, half) plane of activation codes, padded
+constexpr int SA_BYTES = KCH * 2 * PLANE;
+constexpr int SDX_BYTES = KCH * TOK_TILE * 4;
+constexpr int SU_LD = 128 + 4;                     // row stride (floats) of the up -> gate hand-over tile
+constexpr int SU_BYTES = TOK_TILE * SU_LD * 4;
+
+// Workgroup tile: up to TOK_TILE activation rows x 128 output channels; a wave owns 32 channels (one MFMA column tile) and
+// all 32-row tiles.  K is walked in chunks of 8 blocks:
+//   * the rows' int8 codes (128 x 256 B) and fp32 scales of the chunk are staged in LDS once per workgroup, laid out as
+//     [block][half][row] 16-byte words so that operand reads of neighbouring rows are neighbouring words;
+//   * each lane keeps its channel's 8 weight blocks and 8 scales of the chunk in registers;
+//   * the next chunk's global loads (activations and weights) are in flight while the current chunk is computed.
+// MODE 0: one weight matrix, out[o_index[pos]][n] = acc (+ bias).
+// MODE 1: eight waves; waves 0..3 run the gate matrix, waves 4..7 the up matrix over the same channels; the up
+//         accumulators are handed over through LDS and the gate waves emit h = silu(g) * u quantized to Q8_0 (the 32
+//         channels of a wave are exactly one block of the next Linear's input).
 template <int WT, int MODE>
-__global__ __launch_bounds__(256) void qgemm_tile_kernel(QGemmArgs a) {
-  __shared__ __align__(16) float s_dx[KCH][TOK_TILE];  // activation scales of the tile, [block][row]: 32 KB
+__global__ __launch_bounds__(MODE == 1 ? 512 : 256) void qgemm_tile_kernel(QGemmArgs a) {
+  constexpr int NT = MODE == 1 ? 512 : 256;
+  constexpr int UA = TOK_TILE * 16 / NT;  // 16-byte activation words per thread and chunk
+  extern __shared__ __align__(16) unsigned char smem[];
+  unsigned char* sA = smem;
+  float* sDx = reinterpret_cast<float*>(smem + SA_BYTES);
+  float* sU = reinterpret_cast<float*>(smem);  // MODE 1 hand-over tile, reuses the staging area after the last chunk
+
   const int tile = blockIdx.x;
   if (tile >= a.ntiles[0]) return;
   const int e = a.tile_expert[tile], row0 = a.tile_row0[tile], rows = a.tile_rows[tile];
   const int ntt = (rows + 31) >> 5;
+  const int last_njg = (rows - 32 * (ntt - 1) + 7) >> 3;  // 8-row groups in the last 32-row tile
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lrow = lane & 31, hi = lane >> 5;
-  const int nb = a.K / QK;
-  const int nt = blockIdx.y * 4 + wave;      // this wave's tile of 32 output channels
+  const int nb = a.K / QK, nbp = (int)scale_row_stride(a.K);
+  const int mat = MODE == 1 ? (wave >> 2) : 0;
+  const int nt = blockIdx.y * 4 + (wave & 3);  // this wave's tile of 32 output channels
   const bool nvalid = nt * 32 < a.N;
   const int n = min(nt * 32 + lrow, a.N - 1);
 
-  const PackedView w0 = packed_view(WT, a.W0 + (size_t)e * a.wstride, a.N, a.K);
-  const PackedView w1 = packed_view(WT, (MODE == 1 ? a.W1 : a.W0) + (size_t)e * a.wstride, a.N, a.K);
-  const int nbp = (int)scale_row_stride(a.K);
+  const PackedView w = packed_view(WT, (mat ? a.W1 : a.W0) + (size_t)e * a.wstride, a.N, a.K);
+  const u32x4* wq = (WT == MLLM_HIP_Q8_0 && hi) ? w.q1 : w.q0;
 
-  // activation row of the lane in each of the four row tiles (-1: padding)
-  int arow[TT];
-#pragma unroll
-  for (int tt = 0; tt < TT; tt++) {
-    const int p = tt * 32 + lrow;
-    int r = -1;
-    if (p < rows) r = a.a_index ? a.a_index[row0 + p] / a.a_div : row0 + p;
-    arow[tt] = r;
-  }
   const __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.aq), 0, (uint32_t)((int64_t)a.a_rows * a.K), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rD = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(a.ad), 0, (uint32_t)((int64_t)a.a_rows * nb * 4), 0x00020000);
 
-  float acc0[TT][16], acc1[MODE == 1 ? TT : 1][16];
+  // staging assignment: word u = tid + i*NT of the chunk -> row u/16, 16-byte column u%16 (= block*2 + half)
+  uint32_t abase[UA];
+#pragma unroll
+  for (int i = 0; i < UA; i++) {
+    const int u = tid + i * NT, p = u >> 4;
+    uint32_t off = 0xffffffffu;
+    if (p < rows) {
+      const int r = a.a_index ? a.a_index[row0 + p] / a.a_div : row0 + p;
+      off = (uint32_t)((int64_t)r * a.K + (u & 15) * 16);
+    }
+    abase[i] = off;
+  }
+  // scales: thread t < 2*TOK_TILE -> row t/2, blocks (t%2)*4 .. +4 of the chunk
+  uint32_t dbase = 0xffffffffu;
+  if (tid < 2 * TOK_TILE && (tid >> 1) < rows) {
+    const int p = tid >> 1;
+    const int r = a.a_index ? a.a_index[row0 + p] / a.a_div : row0 + p;
+    dbase = (uint32_t)(((int64_t)r * nb + (tid & 1) * 4) * 4);
+  }
+
+  u32x4 pa[UA];
+  float pd[4];
+  u32x4 bq[KCH], bqn[KCH], bs, bsn;
+  auto gload_act = [&](int b0) {
+#pragma unroll
+    for (int i = 0; i < UA; i++) {
+      const int blk = ((tid + i * NT) & 15) >> 1;
+      const bool ok = abase[i] != 0xffffffffu && b0 + blk < nb;
+      pa[i] = __builtin_amdgcn_raw_buffer_load_b128(rA, ok ? abase[i] + (uint32_t)b0 * QK : 0xffffffffu, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      const bool ok = dbase != 0xffffffffu && b0 + (tid & 1) * 4 + j < nb;
+      pd[j] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rD, ok ? dbase + (uint32_t)(b0 + j) * 4 : 0xffffffffu, 0, 0));
+    }
+  };
+  auto sstore_act = [&]() {
+#pragma unroll
+    for (int i = 0; i < UA; i++) {
+      const int u = tid + i * NT;
+      *reinterpret_cast<u32x4*>(sA + (u & 15) * PLANE + (u >> 4) * 16) = pa[i];
+    }
+    if (tid < 2 * TOK_TILE) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) sDx[((tid & 1) * 4 + j) * TOK_TILE + (tid >> 1)] = pd[j];
+    }
+  };
+  auto gload_w = [&](int b0, u32x4 (&q)[KCH], u32x4& sc) {
+#pragma unroll
+    for (int k = 0; k < KCH; k++) q[k] = wq[(int64_t)n * nb + min(b0 + k, nb - 1)];
+    sc = *reinterpret_cast<const u32x4*>(w.d + (int64_t)n * nbp + min(b0, nbp - KCH));
+  };
+
+  float acc[TT][16];
 #pragma unroll
   for (int tt = 0; tt < TT; tt++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      acc0[tt][r] = 0.f;
-      if (MODE == 1) acc1[tt][r] = 0.f;
-    }
+    for (int r = 0; r < 16; r++) acc[tt][r] = 0.f;
+
+  gload_act(0);
+  gload_w(0, bq, bs);
+  sstore_act();
+  __syncthreads();
 
   for (int b0 = 0; b0 < nb; b0 += KCH) {
-    const int nbc = min(KCH, nb - b0);
-    __syncthreads();  // previous chunk fully consumed
-    for (int i = tid; i < nbc * TOK_TILE; i += 256) {
-      const int p = i % TOK_TILE, b = i / TOK_TILE;
-      float v = 0.f;
-      if (p < rows) {
-        const int r = a.a_index ? a.a_index[row0 + p] / a.a_div : row0 + p;
-        v = a.ad[(int64_t)r * nb + b0 + b];
-      }
-      s_dx[b][p] = v;
-    }
-    __syncthreads();
+    // the next chunk's loads are issued unconditionally (past the end they are clamped or out of range and unused): a
+    // branch around them would leave the number of loads in flight unknown and force a full wait before the MFMAs
+    const bool more = b0 + KCH < nb;
+    gload_act(b0 + KCH);
+    gload_w(b0 + KCH, bqn, bsn);
     if (nvalid) {
-      for (int b = 0; b < nbc; b++) {
-        const int64_t blk = (int64_t)n * nb + b0 + b;
-        const v4i fb0 = weight_operand<WT>(w0, blk, hi);
-        const float dw0 = f16bits_to_f32(w0.d[(int64_t)n * nbp + b0 + b]);
-        v4i fb1;
-        float dw1 = 0.f;
-        if (MODE == 1) {
-          fb1 = weight_operand<WT>(w1, blk, hi);
-          dw1 = f16bits_to_f32(w1.d[(int64_t)n * nbp + b0 + b]);
-        }
+      const uint32_t sw[4] = {bs.x, bs.y, bs.z, bs.w};
 #pragma unroll
-        for (int tt = 0; tt < TT; tt++) {
-          if (tt < ntt) {
-            const uint32_t off = arow[tt] >= 0 ? (uint32_t)((int64_t)arow[tt] * a.K + (b0 + b) * QK + hi * 16) : 0xffffffffu;
-            const u32x4 aw = __builtin_amdgcn_raw_buffer_load_b128(rA, off, 0, 0);
-            const v4i fa = v4i{(int)aw.x, (int)aw.y, (int)aw.z, (int)aw.w};
-            v16i z;
+      for (int k = 0; k < KCH; k++) {
+        if (b0 + k < nb) {
+          const v4i fb = weight_operand<WT>(bq[k], hi);
+          const float dw = f16bits_to_f32((uint16_t)(sw[k >> 1] >> (16 * (k & 1))));
 #pragma unroll
-            for (int r = 0; r < 16; r++) z[r] = 0;
-            const v16i i0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb0, z, 0, 0, 0);
-            v16i i1 = z;
-            if (MODE == 1) i1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb1, z, 0, 0, 0);
-            // accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32
+          for (int tt = 0; tt < TT; tt++) {
+            if (tt < ntt) {
+              const v4i fa = *reinterpret_cast<const v4i*>(sA + (k * 2 + hi) * PLANE + (tt * 32 + lrow) * 16);
+              v16i z;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-              const f32x4 dx = *reinterpret_cast<const f32x4*>(&s_dx[b][tt * 32 + 8 * j + 4 * hi]);
+              for (int r = 0; r < 16; r++) z[r] = 0;
+              const v16i is = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, z, 0, 0, 0);
+              const int njg = (tt == ntt - 1) ? last_njg : 4;
+              // accumulator register r of lane l: row 8*(r/4) + 4*(l/32) + r%4, column l%32
 #pragma unroll
-              for (int i = 0; i < 4; i++) {
-                acc0[tt][4 * j + i] = fmaf(dw0 * dx[i], (float)i0[4 * j + i], acc0[tt][4 * j + i]);
-                if (MODE == 1) acc1[tt][4 * j + i] = fmaf(dw1 * dx[i], (float)i1[4 * j + i], acc1[tt][4 * j + i]);
+              for (int j = 0; j < 4; j++) {
+                if (j < njg) {
+                  const f32x4 dx = *reinterpret_cast<const f32x4*>(&sDx[k * TOK_TILE + tt * 32 + 8 * j + 4 * hi]);
+#pragma unroll
+                  for (int i = 0; i < 4; i++) acc[tt][4 * j + i] = fmaf(dw * dx[i], (float)is[4 * j + i], acc[tt][4 * j + i]);
+                }
               }
             }
           }
         }
       }
     }
+    __syncthreads();  // every wave is done with the staged chunk
+    if (more) {
+      sstore_act();
+#pragma unroll
+      for (int k = 0; k < KCH; k++) bq[k] = bqn[k];
+      bs = bsn;
+    }
+    __syncthreads();
   }
-  if (!nvalid) return;
 
+  if (MODE == 1) {
+    // up waves hand their accumulators to the gate waves of the same channels (the staging area is free now)
+    if (mat == 1 && nvalid) {
 #pragma unroll
-  for (int tt = 0; tt < TT; tt++) {
-    if (tt >= ntt) continue;
+      for (int tt = 0; tt < TT; tt++)
+        if (tt < ntt)
 #pragma unroll
-    for (int r = 0; r < 16; r++) {
-      const int p = tt * 32 + 8 * (r / 4) + 4 * hi + (r % 4);  // row within the tile, same for the 32 lanes of a half
-      if (MODE == 0) {
-        if (p < rows && nt * 32 + lrow < a.N) {
-          const int64_t orow = a.o_index ? a.o_index[row0 + p] : row0 + p;
-          float v = acc0[tt][r];
-          if (a.bias) v = a.bias[n] + v;
-          a.out[orow * a.N + n] = v;
-        }
-      } else {
-        // the 32 channels of this wave are exactly one Q8_0 block of the next Linear's input
-        const float h = silu_f(acc0[tt][r]) * acc1[tt][r];
+          for (int r = 0; r < 16; r++)
+            sU[(tt * 32 + 8 * (r / 4) + 4 * hi + (r % 4)) * SU_LD + (wave & 3) * 32 + lrow] = acc[tt][r];
+    }
+    __syncthreads();
+    if (mat == 1 || !nvalid) return;
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) {
+      if (tt >= ntt) continue;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int p = tt * 32 + 8 * (r / 4) + 4 * hi + (r % 4);  // row within the tile, same for the 32 lanes of a half
+        const float h = silu_f(acc[tt][r]) * sU[p * SU_LD + (wave & 3) * 32 + lrow];
         float amax = fabsf(h);
         amax = fmaxf(amax, dpp_f<0xB1>(amax));
         amax = fmaxf(amax, dpp_f<0x4E>(amax));
@@ -275,6 +345,22 @@ __global__ __launch_bounds__(256) void qgemm_tile_kernel(QGemmArgs a) {
             if (a.x86_scale) bits = x86_scale_bits(bits);
             a.hd[(int64_t)(row0 + p) * (a.N / QK) + nt] = f16bits_to_f32(bits);
           }
+        }
+      }
+    }
+  } else {
+    if (!nvalid) return;
+#pragma unroll
+    for (int tt = 0; tt < TT; tt++) {
+      if (tt >= ntt) continue;
+#pragma unroll
+      for (int r = 0; r < 16; r++) {
+        const int p = tt * 32 + 8 * (r / 4) + 4 * hi + (r % 4);
+        if (p < rows && nt * 32 + lrow < a.N) {
+          const int64_t orow = a.o_index ? a.o_index[row0 + p] : row0 + p;
+          float v = acc[tt][r];
+          if (a.bias) v = a.bias[n] + v;
+          a.out[orow * a.N + n] = v;
         }
       }
     }
@@ -324,11 +410,14 @@ static RouteOut carve_route(Carver& c, int E, int64_t entries) {
 template <int MODE>
 static int launch_tiles(int wtype, const QGemmArgs& a, unsigned max_tiles, hipStream_t st) {
   const dim3 grid(max_tiles, (unsigned)((a.N + 127) / 128));
-  if (wtype == MLLM_HIP_Q4_0)
-    hipLaunchKernelGGL((qgemm_tile_kernel<MLLM_HIP_Q4_0, MODE>), grid, dim3(256), 0, st, a);
-  else
-    hipLaunchKernelGGL((qgemm_tile_kernel<MLLM_HIP_Q8_0, MODE>), grid, dim3(256), 0, st, a);
-  return (int)hipGetLastError();
+  const size_t lds = (MODE == 1 && SU_BYTES > SA_BYTES + SDX_BYTES) ? (size_t)SU_BYTES : (size_t)(SA_BYTES + SDX_BYTES);
+  auto launch = [&](auto kern) -> int {
+    if (lds > 64 * 1024)
+      HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, grid, dim3(MODE == 1 ? 512 : 256), lds, st, a);
+    return (int)hipGetLastError();
+  };
+  return wtype == MLLM_HIP_Q4_0 ? launch(qgemm_tile_kernel<MLLM_HIP_Q4_0, MODE>) : launch(qgemm_tile_kernel<MLLM_HIP_Q8_0, MODE>);
 }
 
 }  // namespace mllmhip
