@@ -130,7 +130,21 @@ size_t mllm_hip_w8a8_workspace_bytes(int64_t M, int64_t K);
 int mllm_hip_w8a8_linear(const void* x, int x_dtype, const int8_t* W, const float* w_scale, const float* bias,
                          void* out_bf16, int64_t M, int64_t N, int64_t K, void* workspace, void* stream);
 
-/* GEMM tile override for tuning sweeps: 0 heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64 workgroup tiles. */
+/* Weights repacked once after loading (the step the reference does in process_weights_after_loading,
+ * pymllm/quantization/methods/compressed_tensors.py:429-448, where it re-lays the matrix for its CUTLASS kernel): the
+ * [N][K] int8 matrix in the operand order of v_mfma_i32_32x32x32_i8, N padded to 32 and K to 128 with zeros, so that the
+ * GEMM's waves fetch their weight operands from global memory with fully contiguous 1 KB loads and skip LDS for them.
+ * Same arithmetic and results as mllm_hip_w8a8_gemm / _linear; this is the fast path for prefill-sized M. */
+size_t mllm_hip_w8a8_packed_bytes(int64_t N, int64_t K);
+int mllm_hip_w8a8_prepack(const int8_t* W, int64_t N, int64_t K, void* packed, void* stream);
+int mllm_hip_w8a8_gemm_packed(const int8_t* xq, const float* x_scale, const void* W_packed, const float* w_scale,
+                              const float* bias, void* out_bf16, int32_t* acc_out, int64_t M, int64_t N, int64_t K,
+                              void* stream);
+int mllm_hip_w8a8_linear_packed(const void* x, int x_dtype, const void* W_packed, const float* w_scale, const float* bias,
+                                void* out_bf16, int64_t M, int64_t N, int64_t K, void* workspace, void* stream);
+
+/* GEMM tile override for tuning sweeps (plain-layout entry points): 0 heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64
+ * workgroup tiles through LDS, 4 = weight operands fetched straight from global memory (K % 128 == 0, else 2). */
 int mllm_hip_w8a8_set_tuning(int tile);
 
 /* ---------------------------------------------------------------------------------------------------------

@@ -55,6 +55,11 @@ def lib():
         L.mllm_hip_w8a8_workspace_bytes.argtypes = [i64, i64]
         L.mllm_hip_w8a8_linear.argtypes = [vp, ci, vp, vp, vp, vp, i64, i64, i64, vp, vp]
         L.mllm_hip_w8a8_set_tuning.argtypes = [ci]
+        L.mllm_hip_w8a8_packed_bytes.restype = C.c_size_t
+        L.mllm_hip_w8a8_packed_bytes.argtypes = [i64, i64]
+        L.mllm_hip_w8a8_prepack.argtypes = [vp, i64, i64, vp, vp]
+        L.mllm_hip_w8a8_gemm_packed.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, vp]
+        L.mllm_hip_w8a8_linear_packed.argtypes = [vp, ci, vp, vp, vp, vp, i64, i64, i64, vp, vp]
         L.mllm_hip_w4a16_gemm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp]
         L.mllm_hip_w4a16_dequantize.argtypes = [vp, vp, vp, vp, i64, i64, ci, vp]
         L.mllm_hip_w4a16_set_tuning.argtypes = [ci]

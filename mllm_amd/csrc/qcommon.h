@@ -26,6 +26,12 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest 
   x += 0x7fffu + ((x >> 16) & 1u);
   return (uint16_t)(x >> 16);
 }
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {  // two floats -> one dword of bf16, a in the low half
+  f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, nearest even
+}
 __device__ __forceinline__ float f16bits_to_f32(uint16_t h) { return (float)__builtin_bit_cast(_Float16, h); }
 __device__ __forceinline__ uint16_t f32_to_f16bits(float f) {  // v_cvt_f16_f32, round to nearest even
   return __builtin_bit_cast(uint16_t, (_Float16)f);

@@ -16,15 +16,8 @@
 
 namespace mllmhip {
 
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-  f32x2 v = {a, b};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, nearest even
-}
 
 // eight elements of one packed dword -> four dwords of bf16 pairs, element order kept.
 // (q - zp) * s == fma(q, s, -zp*s) exactly: both products and their sum need at most 16 significant bits.

@@ -152,6 +152,42 @@ def w8a8_linear(x, W, w_scale, bias=None, workspace=None, out=None):
     return y
 
 
+def w8a8_prepack(W):
+    """W int8 [N, K] -> the matrix in MFMA operand order (uint8, mllm_hip_w8a8_packed_bytes long), done once per weight."""
+    assert W.is_cuda and W.is_contiguous() and W.dtype == torch.int8 and W.dim() == 2
+    N, K = W.shape
+    L = _lib.lib()
+    packed = torch.empty(L.mllm_hip_w8a8_packed_bytes(N, K), dtype=torch.uint8, device="cuda")
+    _lib.check(L.mllm_hip_w8a8_prepack(W.data_ptr(), N, K, packed.data_ptr(), _stream()), "mllm_hip_w8a8_prepack")
+    return packed
+
+
+def w8a8_gemm_packed(xq, x_scale, W_packed, N, w_scale, bias=None, want_acc=False, out=None):
+    """As w8a8_gemm, with the weights from w8a8_prepack (N = their row count)."""
+    M, K = xq.shape
+    L = _lib.lib()
+    assert xq.is_contiguous() and W_packed.numel() == L.mllm_hip_w8a8_packed_bytes(N, K)
+    y = out if out is not None else torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    acc = torch.empty((M, N), dtype=torch.int32, device="cuda") if want_acc else None
+    _lib.check(L.mllm_hip_w8a8_gemm_packed(xq.data_ptr(), _p(x_scale), W_packed.data_ptr(), _p(w_scale), _p(bias),
+                                           y.data_ptr(), _p(acc), M, N, K, _stream()), "mllm_hip_w8a8_gemm_packed")
+    return (y, acc) if want_acc else y
+
+
+def w8a8_linear_packed(x, W_packed, N, w_scale, bias=None, workspace=None, out=None):
+    """As w8a8_linear, with the weights from w8a8_prepack."""
+    M, K = x.shape
+    L = _lib.lib()
+    assert W_packed.numel() == L.mllm_hip_w8a8_packed_bytes(N, K)
+    if workspace is None:
+        workspace = torch.empty(L.mllm_hip_w8a8_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+    y = out if out is not None else torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    _lib.check(L.mllm_hip_w8a8_linear_packed(x.data_ptr(), _xdtype(x), W_packed.data_ptr(), w_scale.data_ptr(), _p(bias),
+                                             y.data_ptr(), M, N, K, workspace.data_ptr(), _stream()),
+               "mllm_hip_w8a8_linear_packed")
+    return y
+
+
 # ----------------------------------------------------------------------------- W4A16 (group-wise uint4 + zero point)
 def w4a16_gemm(a, qw, scales, zeros, bias=None, group=128, out=None):
     """a bf16 [M, K]; qw uint8 [N, K/2]; scales fp16 [N, K/group]; zeros uint8 [N, ceil(K/group/2)] -> bf16 [M, N]."""

@@ -49,7 +49,7 @@ REF_SHAPES = [(1, 64, 32), (1, 2048, 2048), (8, 128, 64), (16, 6144, 2048), (32,
 
 
 @pytest.mark.parametrize("M,N,K", REF_SHAPES + [(300, 200, 48), (257, 193, 80)])
-@pytest.mark.parametrize("tile", [0, 1, 2, 3])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
 def test_gemm_bit_exact(M, N, K, tile):
     rng = synth.rng_for(3, M * 7 + N + K)
     xq = rng.integers(-127, 128, (M, K), dtype=np.int8)
@@ -71,6 +71,43 @@ def test_gemm_bit_exact(M, N, K, tile):
     assert np.array_equal(_bits(y), wy)
     assert np.array_equal(_bits(yb), wyb)
     assert rel_l2(synth.bf16_bits_to_fp32(_bits(y)), synth.bf16_bits_to_fp32(wy)) <= 1e-3
+
+
+def _pack_reference(W):
+    """The packed layout restated with numpy: block (nb, kb) of 32 rows x 32 bytes, lane l = (row l%32, half l/32)."""
+    N, K = W.shape
+    Np, Kp = (N + 31) // 32 * 32, (K + 127) // 128 * 128
+    Wp = np.zeros((Np, Kp), dtype=np.int8)
+    Wp[:N, :K] = W
+    # [nb][row][kb][half][16] -> [nb][kb][half][row][16]
+    return Wp.reshape(Np // 32, 32, Kp // 32, 2, 16).transpose(0, 2, 3, 1, 4).reshape(-1)
+
+
+# shapes that reach each tile of the weights-from-global kernel: 128x384, 64x384, 128x128, 64x128, and ragged edges
+PACKED_SHAPES = REF_SHAPES + [(300, 200, 48), (257, 193, 80), (1536, 6144, 256), (512, 9216, 128), (1024, 3072, 128),
+                              (200, 800, 144)]
+
+
+@pytest.mark.parametrize("M,N,K", PACKED_SHAPES)
+def test_gemm_packed_bit_exact(M, N, K):
+    rng = synth.rng_for(3, M * 11 + N + K)
+    xq = rng.integers(-127, 128, (M, K), dtype=np.int8)
+    W = rng.integers(-127, 128, (N, K), dtype=np.int8)
+    xs = ((rng.random(M) + 0.01) * 0.01).astype(np.float32)
+    ws = ((rng.random(N) + 0.01) * 0.01).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.01).astype(np.float32)
+    announce("w8a8 packed gemm", M, N, K)
+    Wp = ql.w8a8_prepack(to_dev(W))
+    assert np.array_equal(Wp.cpu().numpy().view(np.int8), _pack_reference(W))
+    y, acc = ql.w8a8_gemm_packed(to_dev(xq), to_dev(xs), Wp, N, to_dev(ws), None, want_acc=True)
+    y1 = ql.w8a8_gemm_packed(to_dev(xq), to_dev(xs), Wp, N, to_dev(ws), None)      # bf16 only: the fast store path
+    yb = ql.w8a8_gemm_packed(to_dev(xq), to_dev(xs), Wp, N, to_dev(ws), to_dev(bias))
+    wacc, wy = orc.w8a8_gemm(xq, xs, W, ws, None)
+    _, wyb = orc.w8a8_gemm(xq, xs, W, ws, bias)
+    assert np.array_equal(acc.cpu().numpy(), wacc)
+    assert np.array_equal(_bits(y), wy)
+    assert np.array_equal(_bits(y1), wy)
+    assert np.array_equal(_bits(yb), wyb)
 
 
 def test_full_size_prefill():
@@ -97,6 +134,13 @@ def test_full_size_prefill():
     # the fused entry point (quantize + GEMM) gives the same bits
     y2 = ql.w8a8_linear(xd, Wd, wsd)
     assert torch.equal(y2.view(torch.int16), y.view(torch.int16))
+    # and so does the prepacked-weight path, on every element
+    Wp = ql.w8a8_prepack(Wd)
+    y3, acc3 = ql.w8a8_gemm_packed(q, s, Wp, N, wsd, None, want_acc=True)
+    assert np.array_equal(acc3.cpu().numpy(), acc)
+    y4 = ql.w8a8_linear_packed(xd, Wp, N, wsd)
+    assert torch.equal(y3.view(torch.int16), y.view(torch.int16))
+    assert torch.equal(y4.view(torch.int16), y.view(torch.int16))
 
 
 def test_argument_errors():
@@ -111,3 +155,6 @@ def test_argument_errors():
     assert g(t.data_ptr() + 1, f.data_ptr(), t.data_ptr(), f.data_ptr(), None, o.data_ptr(), None, 8, 8, 64, None) == -3
     assert L.mllm_hip_per_token_quant_int8(None, 1, t.data_ptr(), f.data_ptr(), 4, 64, None) == -1
     assert L.mllm_hip_w8a8_set_tuning(9) == -1
+    assert L.mllm_hip_w8a8_prepack(t.data_ptr(), 64, 40, o.data_ptr(), None) == -2
+    assert L.mllm_hip_w8a8_prepack(None, 64, 64, o.data_ptr(), None) == -1
+    assert L.mllm_hip_w8a8_packed_bytes(33, 130) == 64 * 256
