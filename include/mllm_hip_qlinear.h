@@ -168,6 +168,24 @@ int mllm_hip_w4a16_dequantize(const uint8_t* qw, const uint16_t* scales, const u
 /* GEMM tile override for tuning sweeps: 0 heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64 workgroup tiles. */
 int mllm_hip_w4a16_set_tuning(int tile);
 
+/* Weights repacked once after loading (the step the reference does in AWQMarlinLinearMethod.process_weights_after_loading,
+ * pymllm/quantization/methods/awq_marlin.py:366-410: awq_marlin_repack, marlin_permute_scales,
+ * awq_to_marlin_zero_points): the 4-bit codes in the operand order of v_mfma_f32_32x32x16_bf16 (N padded to 32, K to 128),
+ * followed by one (scale, -zero_point * scale) fp32 pair per row and group.  The GEMM's waves then fetch their weight
+ * operands from global memory with contiguous 1 KB loads and dequantize them in registers; same arithmetic
+ * (w = bf16(fma(q, scale, -zp*scale)) = bf16((q - zp) * scale), fp32 accumulation) as mllm_hip_w4a16_gemm.
+ * This is the fast path for prefill-sized M. */
+size_t mllm_hip_w4a16_packed_bytes(int64_t N, int64_t K, int group);
+int mllm_hip_w4a16_prepack(const uint8_t* qw, const uint16_t* scales, const uint8_t* zeros, int64_t N, int64_t K, int group,
+                           void* packed, void* stream);
+int mllm_hip_w4a16_gemm_packed(const void* a_bf16, const void* packed, const void* bias_bf16, void* c_bf16, int64_t M,
+                               int64_t N, int64_t K, int group, void* stream);
+/* Parity probe: the dequantized weight table w_bf16 [N][K] exactly as the packed GEMM forms it. */
+int mllm_hip_w4a16_dequantize_packed(const void* packed, void* w_bf16, int64_t N, int64_t K, int group, void* stream);
+/* Tile override for the packed GEMM: 0 heuristic, 1 = 128x384, 2 = 64x384, 3 = 128x128, 4 = 64x128, 5 = 128x256;
+ * + 16 switches off the half-height tiles that shorten a partly filled last round. */
+int mllm_hip_w4a16_packed_set_tuning(int tile);
+
 /* ---------------------------------------------------------------------------------------------------------
  * MoE expert FFN over expert-sorted tokens, Q4_0 / Q8_0 expert weights
  * replaces: Qwen3MoE::moeInfer + Qwen3MoeMLP::forward (one CPULinearOp::forward per expert and projection)

@@ -63,6 +63,12 @@ def lib():
         L.mllm_hip_w4a16_gemm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp]
         L.mllm_hip_w4a16_dequantize.argtypes = [vp, vp, vp, vp, i64, i64, ci, vp]
         L.mllm_hip_w4a16_set_tuning.argtypes = [ci]
+        L.mllm_hip_w4a16_packed_set_tuning.argtypes = [ci]
+        L.mllm_hip_w4a16_packed_bytes.restype = C.c_size_t
+        L.mllm_hip_w4a16_packed_bytes.argtypes = [i64, i64, ci]
+        L.mllm_hip_w4a16_prepack.argtypes = [vp, vp, vp, i64, i64, ci, vp, vp]
+        L.mllm_hip_w4a16_gemm_packed.argtypes = [vp, vp, vp, vp, i64, i64, i64, ci, vp]
+        L.mllm_hip_w4a16_dequantize_packed.argtypes = [vp, vp, i64, i64, ci, vp]
         L.mllm_hip_linear_q_workspace_bytes.restype = C.c_size_t
         L.mllm_hip_linear_q_workspace_bytes.argtypes = [i64, i64]
         L.mllm_hip_linear_q.argtypes = [ci, vp, vp, ci, vp, vp, i64, i64, i64, ci, vp, vp]

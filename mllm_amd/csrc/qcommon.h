@@ -28,6 +28,7 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {  // round to nearest 
 }
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {  // two floats -> one dword of bf16, a in the low half
   f32x2 v = {a, b};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // v_cvt_pk_bf16_f32, nearest even

@@ -21,8 +21,13 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 
 // eight elements of one packed dword -> four dwords of bf16 pairs, element order kept.
 // (q - zp) * s == fma(q, s, -zp*s) exactly: both products and their sum need at most 16 significant bits.
+// One conversion (v_cvt_f32_ubyteN reads byte N of a dword), one fma and half a pack per element.  The empty asm hides
+// from the optimizer that only four bits of each byte can be set; knowing it, the compiler replaces mask + byte
+// conversion by one bit-field extract PER ELEMENT plus the conversion.
 __device__ __forceinline__ void dequant8(uint32_t w, float s, float nzs, uint32_t (&out)[4]) {
-  const uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;  // bytes: elements 0,2,4,6 / 1,3,5,7
+  uint32_t lo = w & 0x0f0f0f0fu, hi = (w >> 4) & 0x0f0f0f0fu;  // bytes: elements 0,2,4,6 / 1,3,5,7
+  asm("" : "+v"(lo));
+  asm("" : "+v"(hi));
 #pragma unroll
   for (int b = 0; b < 4; b++) {
     const float e0 = fmaf((float)((lo >> (8 * b)) & 0xffu), s, nzs);
@@ -203,19 +208,363 @@ __global__ void w4a16_dequant_kernel(const uint8_t* __restrict__ qw, const uint1
   *reinterpret_cast<u32x4*>(w + n * K + k) = u32x4{o[0], o[1], o[2], o[3]};
 }
 
-template <int BM, int BN, int WM, int WN>
-static int launch_w4a16(const W4A16Args& a, hipStream_t st) {
-  constexpr int NT = (BM / WM) * (BN / WN) * 64;
-  const size_t lds = 2 * (size_t)(BM + BN) * 144;
-  const unsigned grid = (unsigned)(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN));
-  auto kern = w4a16_gemm_kernel<BM, BN, WM, WN>;
-  if (lds > 64 * 1024)
-    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds, st, a);
+// ---------------------------------------------------------------------------------------------------------
+// Prepacked weights + weights-from-global kernel (the fast path for prefill-sized M).
+//
+// Measured on this part: a 16-byte LDS read of a whole wave occupies the CU's LDS pipe for 16 cycles (64 B/clk/CU) while
+// one v_mfma_f32_32x32x16_bf16 occupies a SIMD for 32, so a wave that pulls both operands of a 64x64 tile through LDS is
+// LDS-bound at under half the matrix rate, and dequantized weights staged in LDS cost that bandwidth twice (write +
+// reads).  Here only the activation tile goes through LDS.  The four waves of a workgroup sit side by side along N, each
+// owns (32 TM) x (32 TN) outputs, loads ITS packed 4-bit weights straight from global memory (16 bytes per lane = the
+// lane's operands of four MFMA K steps), dequantizes them in registers one MFMA step ahead of their use, and no weight
+// is dequantized twice inside a workgroup.
+//
+// Packed layout (one pass over the checkpoint tensors, mllm_hip_w4a16_prepack):
+//   q   [N/32][K/64][64 lanes][16 bytes]: lane l = (row l%32, half l/32); dword d of its 16 bytes holds the eight
+//       elements k = 64 kb + 16 d + 8 (l/32) + 0..7 of its row, element e in nibble e (the checkpoint's own dword).
+//       N is padded to 32 rows and K to 128 elements with zeros.
+//   sz  [N/32][K/group][32 rows][2 floats]: (scale, -zero_point * scale) of the row's group, both exact in fp32.
+__host__ __device__ inline int64_t w4a16_packed_n(int64_t N) { return (N + 31) / 32 * 32; }
+__host__ __device__ inline int64_t w4a16_packed_k(int64_t K) { return (K + 127) / 128 * 128; }
+__host__ __device__ inline int64_t w4a16_packed_qbytes(int64_t N, int64_t K) { return w4a16_packed_n(N) * w4a16_packed_k(K) / 2; }
+
+__global__ __launch_bounds__(256) void w4a16_prepack_q_kernel(const uint8_t* __restrict__ qw, uint32_t* __restrict__ P, int N,
+                                                              int K, int64_t words) {
+  const int64_t w = (int64_t)blockIdx.x * 256 + threadIdx.x;  // one dword = 8 elements of the packed matrix
+  if (w >= words) return;
+  const int kbs = (int)(w4a16_packed_k(K) / 64);
+  const int d = (int)(w % 4), l = (int)((w / 4) % 64);
+  const int64_t blk = w / 256;
+  const int kb = (int)(blk % kbs), nb = (int)(blk / kbs);
+  const int n = nb * 32 + (l & 31), k = kb * 64 + d * 16 + (l >> 5) * 8;
+  uint32_t v = 0;
+  if (n < N && k < K) v = *reinterpret_cast<const uint32_t*>(qw + ((int64_t)n * K + k) / 2);
+  P[w] = v;
+}
+__global__ __launch_bounds__(256) void w4a16_prepack_sz_kernel(const uint16_t* __restrict__ s, const uint8_t* __restrict__ zp,
+                                                               float2* __restrict__ SZ, int N, int G, int64_t count) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (nb, g, row)
+  if (i >= count) return;
+  const int row = (int)(i % 32), g = (int)((i / 32) % G), nb = (int)(i / 32 / G);
+  const int n = nb * 32 + row;
+  float2 v = {0.f, 0.f};
+  if (n < N) {
+    const float sc = f16bits_to_f32(s[(int64_t)n * G + g]);
+    const uint8_t zb = zp[(int64_t)n * ((G + 1) / 2) + (g >> 1)];
+    const float z = (float)((g & 1) ? (zb >> 4) : (zb & 15));
+    v = float2{sc, -(z * sc)};
+  }
+  SZ[i] = v;
+}
+
+struct W4A16PArgs {
+  const uint16_t* A;     // bf16 [M][K]
+  const uint8_t* P;      // packed q then sz
+  const uint16_t* bias;  // bf16 [N] or null
+  uint16_t* C;           // bf16 [M][N]
+  int M, N, K, group;
+};
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+// One output tile (32 TM rows from m0) x (128 TN columns from n0) by the four waves of a workgroup.
+template <int TM, int TN, int BK>
+__device__ __forceinline__ void w4a16_nsplit_tile(const W4A16PArgs& a, const int m0, const int n0, unsigned char* smem) {
+  static_assert(BK == 64 || BK == 128, "K step of one or two 64-element weight blocks");
+  constexpr int LDK = 2 * BK + 16, KS = BK / 16, NH = BK / 64;  // LDS row in bytes; MFMA steps; weight blocks per K step
+  constexpr int CPRA = BK / 8;                                  // 16-byte activation chunks per row and K step
+  constexpr int BM = TM * 32, WN = TN * 32, BN = 4 * WN;
+  constexpr int CA = BM * (2 * BK / 16) / 256;  // 16-byte activation chunks per thread and K step
+  static_assert(CA >= 1, "tile too small for 256 threads");
+  constexpr int STAGE = BM * LDK;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lrow = lane & 31, hi = lane >> 5;
+
+  const int Kp = (int)w4a16_packed_k(a.K), kbs = Kp / 64, G = a.K / a.group, g64 = a.group / 64;
+  const int64_t qbytes = w4a16_packed_qbytes(a.N, a.K);
+  const int nbs = (int)(w4a16_packed_n(a.N) / 32);
+  const __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.A), 0, (uint32_t)((int64_t)a.M * a.K * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rQ = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.P), 0, (uint32_t)qbytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rS = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(a.P + qbytes), 0, (uint32_t)((int64_t)nbs * G * 256), 0x00020000);
+
+  // activation chunk: row idx / CPRA, 16-byte column idx % CPRA.  Rows past M are clamped (never stored); columns past K
+  // read as zeros so that the zero-padded tail of the weights never meets another row's values.
+  uint32_t offA[CA];
+  int colA[CA];
+#pragma unroll
+  for (int c = 0; c < CA; c++) {
+    const int idx = tid + c * 256;
+    colA[c] = (idx % CPRA) * 8;
+    offA[c] = (uint32_t)(((int64_t)min(m0 + idx / CPRA, a.M - 1) * a.K + colA[c]) * 2);
+  }
+  uint32_t offQ[TN], offS[TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int nb = min((n0 + wave * WN) / 32 + j, nbs - 1);
+    offQ[j] = (uint32_t)((int64_t)nb * kbs * 1024 + lane * 16);
+    offS[j] = (uint32_t)(((int64_t)nb * G * 32 + lrow) * 8);
+  }
+  auto loadA = [&](int k0, u32x4 (&ga)[CA]) {
+#pragma unroll
+    for (int c = 0; c < CA; c++)
+      ga[c] = __builtin_amdgcn_raw_buffer_load_b128(rA, k0 + colA[c] < a.K ? offA[c] : 0xffffffffu, k0 * 2, 0);
+  };
+  auto storeA = [&](int buf, const u32x4 (&ga)[CA]) {
+#pragma unroll
+    for (int c = 0; c < CA; c++) {
+      const int idx = tid + c * 256;
+      *reinterpret_cast<u32x4*>(smem + buf * STAGE + (idx / CPRA) * LDK + (idx % CPRA) * 16) = ga[c];
+    }
+  };
+  auto readA = [&](int buf, int ks, bf16x8 (&fa)[TM]) {
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+      fa[i] = *reinterpret_cast<const bf16x8*>(smem + buf * STAGE + (i * 32 + lrow) * LDK + ks * 32 + hi * 16);
+  };
+  // the packed weights and the (scale, -zp*scale) pair of 64-element block kb of column block j
+  auto loadQ = [&](int kb, int j) -> u32x4 { return __builtin_amdgcn_raw_buffer_load_b128(rQ, offQ[j], kb * 1024, 0); };
+  auto loadS = [&](int kb, int j) -> u32x2 {
+    return __builtin_amdgcn_raw_buffer_load_b64(rS, offS[j], min(kb / g64, G - 1) * 256, 0);
+  };
+  auto dequant = [&](const u32x4& q, const u32x2& sz, int d) -> bf16x8 {
+    uint32_t o[4];
+    dequant8(q[d], __uint_as_float(sz.x), __uint_as_float(sz.y), o);
+    return __builtin_bit_cast(bf16x8, u32x4{o[0], o[1], o[2], o[3]});
+  };
+
+  v16f acc[TN][TM];
+#pragma unroll
+  for (int j = 0; j < TN; j++)
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[j][i][r] = 0.f;
+
+  const int KT = Kp / BK;
+  u32x4 ga[CA];
+  u32x4 rq[NH][TN];  // packed weights of the 64-element blocks of a K step
+  u32x2 rs[NH][TN];
+  bf16x8 fb[2][TN];  // dequantized operands of MFMA step ks (set ks & 1)
+  bf16x8 fa[2][TM];
+  loadA(0, ga);
+#pragma unroll
+  for (int h = 0; h < NH; h++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      rq[h][j] = loadQ(h, j);
+      rs[h][j] = loadS(h, j);
+    }
+  storeA(0, ga);
+  __syncthreads();
+  readA(0, 0, fa[0]);
+#pragma unroll
+  for (int j = 0; j < TN; j++) fb[0][j] = dequant(rq[0][j], rs[0][j], 0);
+
+  for (int kt = 0; kt < KT; kt++) {
+    const int buf = kt & 1, k1 = (kt + 1) * BK;
+    loadA(k1, ga);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      if (ks < KS - 1) {
+        readA(buf, ks + 1, fa[(ks + 1) & 1]);  // the next step's activations while this one's MFMAs run
+      } else {
+        storeA(buf ^ 1, ga);  // free since the previous barrier; its loads were issued a whole K step ago
+        __syncthreads();
+        readA(buf ^ 1, 0, fa[(ks + 1) & 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const int nh = ((ks + 1) / 4) % NH, nd = (ks + 1) % 4;  // block and dword of the NEXT MFMA step's weights
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        // One wave per SIMD issues in order: the dequantization of the next step's operand (23 VALU instructions) is
+        // cut into TM pieces, one in the shadow of each MFMA (32 cycles), and pinned there; left to the scheduler, the
+        // MFMAs queue up back to back and the matrix pipe idles behind them while the VALU work runs.
+        uint32_t lo = rq[nh][j][nd] & 0x0f0f0f0fu, hi = (rq[nh][j][nd] >> 4) & 0x0f0f0f0fu;
+        asm("" : "+v"(lo));
+        asm("" : "+v"(hi));
+        const float sc = __uint_as_float(rs[nh][j].x), nzs = __uint_as_float(rs[nh][j].y);
+        uint32_t o[4];
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks & 1][j], fa[ks & 1][i], acc[j][i], 0, 0, 0);
+#pragma unroll
+          for (int b = i * 4 / TM; b < (i + 1) * 4 / TM; b++)
+            o[b] = pack_bf16(fmaf((float)((lo >> (8 * b)) & 0xffu), sc, nzs), fmaf((float)((hi >> (8 * b)) & 0xffu), sc, nzs));
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        fb[(ks + 1) & 1][j] = __builtin_bit_cast(bf16x8, u32x4{o[0], o[1], o[2], o[3]});
+        if (nd == 3) {  // last dword of that half consumed: fetch the same half of the next K step into its registers
+          rq[nh][j] = loadQ((kt + 1) * NH + nh, j);
+          rs[nh][j] = loadS((kt + 1) * NH + nh, j);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  }
+  __syncthreads();  // all LDS reads done before the epilogue reuses the tiles
+
+  // acc[j][i][4g+e] = C[m0 + 32i + lrow][n0 + wave*WN + 32j + 8g + 4hi + e]
+  float* sBi = reinterpret_cast<float*>(smem);
+  for (int i = tid; i < BN; i += 256) sBi[i] = (a.bias && n0 + i < a.N) ? bf16_to_f32(a.bias[n0 + i]) : 0.f;
+  __syncthreads();
+  constexpr int ROWB = 2 * BN + 16;
+  unsigned char* patch = smem + 4096;
+  static_assert(BN * 4 <= 4096, "bias overlaps the store patch");
+  const bool has_bias = a.bias != nullptr;
+  const bool full = m0 + BM <= a.M && n0 + BN <= a.N && a.N % 8 == 0 && reinterpret_cast<uintptr_t>(a.C) % 16 == 0;
+  if (full) {
+    // branch-free path: each 32-row slab of results is turned through LDS so that a wave stores whole rows of the
+    // workgroup's BN columns (runs of whole cache lines, 16 bytes per lane)
+    f32x4 bi4[TN][4];
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) bi4[j][g] = *reinterpret_cast<const f32x4*>(&sBi[wave * WN + j * 32 + 8 * g + 4 * hi]);
+    constexpr int CPR = BN / 8;  // 16-byte pieces per row
+    static_assert((8 * CPR) % 64 == 0, "a wave stores whole rows");
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+          float f[4];
+#pragma unroll
+          for (int e = 0; e < 4; e++) f[e] = acc[j][i][4 * g + e];
+          if (has_bias) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) f[e] += bi4[j][g][e];
+          }
+          *reinterpret_cast<uint2*>(patch + lrow * ROWB + (wave * WN + j * 32 + 8 * g + 4 * hi) * 2) =
+              uint2{pack_bf16(f[0], f[1]), pack_bf16(f[2], f[3])};
+        }
+      __syncthreads();
+#pragma unroll
+      for (int t = 0; t < 8 * CPR / 64; t++) {  // wave w stores rows 8w .. 8w+7
+        const int c = lane + 64 * t;
+        const int row = wave * 8 + c / CPR, cc = c % CPR;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(patch + row * ROWB + cc * 16);
+        *reinterpret_cast<u32x4*>(&a.C[(int64_t)(m0 + i * 32 + row) * a.N + n0 + cc * 8]) = v;
+      }
+      if (i + 1 < TM) __syncthreads();
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < TM; i++) {
+    const int m = m0 + i * 32 + lrow;
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int g = 0; g < 4; g++) {
+        const int cn = wave * WN + j * 32 + 8 * g + 4 * hi;
+        const f32x4 bi4 = *reinterpret_cast<const f32x4*>(&sBi[cn]);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+          if (m < a.M && n0 + cn + e < a.N) {
+            float f = acc[j][i][4 * g + e];
+            if (has_bias) f += bi4[e];
+            a.C[(int64_t)m * a.N + n0 + cn + e] = (uint16_t)pack_bf16(f, 0.f);
+          }
+      }
+  }
+}
+
+// Tile schedule.  Workgroups [0, nbig) own full tiles (32 TM rows) over the first `big_cols` column tiles; the rest own
+// half-height tiles over the remaining column tiles.  The host picks big_cols so that the full tiles fill whole rounds of
+// the chip's workgroup slots and the remainder, which would otherwise occupy a whole further round at a fraction of the
+// chip, runs as twice as many tiles of half the duration.
+// WPS: waves per SIMD the register budget is held to (workgroups of 4 waves: WPS workgroups per CU).
+template <int TM, int TN, int BK, int WPS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPS, WPS))) void w4a16_gemm_nsplit_kernel(W4A16PArgs a, int big_cols) {
+  constexpr int BM = TM * 32, BN = 4 * TN * 32;
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int tilesM = (a.M + BM - 1) / BM;
+  const int nbig = tilesM * big_cols;
+  int b = blockIdx.x;
+  if (b < nbig) {
+    if (nbig % 8 == 0) b = (b % 8) * (nbig / 8) + b / 8;  // one run of tiles per XCD that shares a slice of the weights
+    w4a16_nsplit_tile<TM, TN, BK>(a, (b % tilesM) * BM, (b / tilesM) * BN, smem);
+  } else {
+    if constexpr (TM >= 2) {
+      constexpr int HM = BM / 2;
+      const int tilesH = (a.M + HM - 1) / HM;
+      b -= nbig;
+      w4a16_nsplit_tile<TM / 2, TN, BK>(a, (b % tilesH) * HM, (big_cols + b / tilesH) * BN, smem);
+    }
+  }
+}
+
+// dequantized weight table from the PACKED form, through the same dequant8 and (scale, -zp*scale) pairs as the GEMM
+__global__ void w4a16_dequant_packed_kernel(const uint8_t* __restrict__ P, uint16_t* __restrict__ w, int N, int K, int group) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // one dword = 8 elements of the table
+  if (i >= (int64_t)N * K / 8) return;
+  const int n = (int)(i / (K / 8)), k = (int)(i % (K / 8)) * 8;
+  const int kbs = (int)(w4a16_packed_k(K) / 64), G = K / group;
+  const int nb = n / 32, row = n % 32, kb = k / 64, d = (k % 64) / 16, hi = (k % 16) / 8;
+  const uint32_t word = reinterpret_cast<const uint32_t*>(P)[(((int64_t)nb * kbs + kb) * 64 + hi * 32 + row) * 4 + d];
+  const float2 sz = reinterpret_cast<const float2*>(P + w4a16_packed_qbytes(N, K))[((int64_t)nb * G + k / group) * 32 + row];
+  uint32_t o[4];
+  dequant8(word, sz.x, sz.y, o);
+  *reinterpret_cast<u32x4*>(w + (int64_t)n * K + k) = u32x4{o[0], o[1], o[2], o[3]};
+}
+
+static int g_w4a16_tail = 1;  // half-height tiles for a short last round (0 switches the schedule off: tuning/tests)
+
+template <int TM, int TN, int BK, int WPS>
+static int launch_w4a16_nsplit(const W4A16PArgs& a, hipStream_t st) {
+  constexpr int BM = TM * 32, BN = 4 * TN * 32;
+  constexpr size_t stage = 2 * (size_t)BM * (2 * BK + 16), patch = 4096 + 32 * (2 * (size_t)BN + 16);
+  const size_t lds = stage > patch ? stage : patch;
+  auto kern = w4a16_gemm_nsplit_kernel<TM, TN, BK, WPS>;
+  static int slots = 0;  // workgroups the chip holds at once
+  if (!slots) {
+    if (lds > 64 * 1024)
+      HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    int dev = 0, cus = 0, per_cu = 0;
+    HIP_RET(hipGetDevice(&dev));
+    HIP_RET(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+    HIP_RET(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(kern), 256, lds));
+    slots = cus * (per_cu > 0 ? per_cu : 1);
+  }
+  const int tilesM = (a.M + BM - 1) / BM, tilesN = (a.N + BN - 1) / BN;
+  const int64_t total = (int64_t)tilesM * tilesN;
+  int big_cols = tilesN;
+  if (g_w4a16_tail && TM >= 2 && total > slots && total % slots) {
+    // columns whose full tiles fit into whole rounds; the remaining columns as half tiles if that ends earlier
+    const int cols = (int)(total / slots * slots / tilesM);
+    const int64_t halves = (int64_t)(tilesN - cols) * ((a.M + BM / 2 - 1) / (BM / 2));
+    const double as_full = (double)((total + slots - 1) / slots);
+    // a half tile takes about 0.6 of a full one: it dequantizes the same weights for half the rows
+    const double with_tail = (double)(((int64_t)cols * tilesM + slots - 1) / slots) + 0.6 * (double)((halves + slots - 1) / slots);
+    if (with_tail < as_full) big_cols = cols;
+  }
+  const int64_t grid = (int64_t)tilesM * big_cols + (int64_t)(tilesN - big_cols) * ((a.M + BM / 2 - 1) / (BM / 2));
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), lds, st, a, big_cols);
   return (int)hipGetLastError();
 }
 
-static int g_w4a16_tile = 0;  // 0 = heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64
+static int g_w4a16_ptile = 0;  // packed path: 0 = heuristic, 1 = 128x384, 2 = 64x384, 3 = 128x128, 4 = 64x128, 5 = 128x256
+
+// Tile choice for the weights-from-global kernel.  128x256 with two workgroups per CU measured best on large problems
+// (one wave's dequantization runs beside the other's MFMAs); smaller tiles only to give every CU work.
+static int launch_w4a16_nsplit_auto(const W4A16PArgs& a, hipStream_t st) {
+  auto tiles = [&](int bm, int bn) { return (int64_t)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
+  int t = g_w4a16_ptile;
+  if (!t) {
+    if (a.M > 64) t = tiles(128, 256) >= 256 ? 5 : tiles(128, 128) >= 128 ? 3 : 4;
+    else t = tiles(64, 384) >= 192 ? 2 : 4;
+  }
+  switch (t) {
+    case 1: return launch_w4a16_nsplit<4, 3, 128, 1>(a, st);
+    case 2: return launch_w4a16_nsplit<2, 3, 128, 2>(a, st);
+    case 3: return launch_w4a16_nsplit<4, 1, 64, 3>(a, st);
+    case 5: return launch_w4a16_nsplit<4, 2, 64, 2>(a, st);
+    default: return launch_w4a16_nsplit<2, 1, 128, 2>(a, st);
+  }
+}
 
 }  // namespace mllmhip
 
@@ -224,6 +573,13 @@ using namespace mllmhip;
 MLLM_API int mllm_hip_w4a16_set_tuning(int tile) {
   if (tile < 0 || tile > 3) return MLLM_HIP_E_BADARG;
   g_w4a16_tile = tile;
+  return 0;
+}
+
+MLLM_API int mllm_hip_w4a16_packed_set_tuning(int tile) {
+  if (tile < 0 || (tile & 15) > 5 || tile > 31) return MLLM_HIP_E_BADARG;
+  g_w4a16_ptile = tile & 15;
+  g_w4a16_tail = !(tile & 16);
   return 0;
 }
 
@@ -268,5 +624,50 @@ MLLM_API int mllm_hip_w4a16_dequantize(const uint8_t* qw, const uint16_t* scales
   const int64_t words = N * K / 8;
   hipLaunchKernelGGL(w4a16_dequant_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, (hipStream_t)stream, qw,
                      scales, zeros, (uint16_t*)w_bf16, N, K, group);
+  return (int)hipGetLastError();
+}
+
+MLLM_API size_t mllm_hip_w4a16_packed_bytes(int64_t N, int64_t K, int group) {
+  if (N <= 0 || K <= 0 || group <= 0 || group % 64 || K % group) return 0;
+  return (size_t)(w4a16_packed_qbytes(N, K) + w4a16_packed_n(N) * (K / group) * 8);
+}
+
+MLLM_API int mllm_hip_w4a16_prepack(const uint8_t* qw, const uint16_t* scales, const uint8_t* zeros, int64_t N, int64_t K,
+                                    int group, void* packed, void* stream) {
+  int rc = check_w4a16(qw, scales, zeros, N, K, group);
+  if (rc) return rc;
+  if (!packed) return MLLM_HIP_E_BADARG;
+  if (reinterpret_cast<uintptr_t>(packed) % 16) return MLLM_HIP_E_ALIGN;
+  if (mllm_hip_w4a16_packed_bytes(N, K, group) >= ((size_t)1 << 32)) return MLLM_HIP_E_SHAPE;
+  const int64_t words = w4a16_packed_qbytes(N, K) / 4;
+  hipLaunchKernelGGL(w4a16_prepack_q_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, (hipStream_t)stream, qw,
+                     reinterpret_cast<uint32_t*>(packed), (int)N, (int)K, words);
+  const int G = (int)(K / group);
+  const int64_t count = w4a16_packed_n(N) * G;
+  hipLaunchKernelGGL(w4a16_prepack_sz_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, (hipStream_t)stream, scales,
+                     zeros, reinterpret_cast<float2*>(reinterpret_cast<char*>(packed) + w4a16_packed_qbytes(N, K)), (int)N, G,
+                     count);
+  return (int)hipGetLastError();
+}
+
+MLLM_API int mllm_hip_w4a16_gemm_packed(const void* a_bf16, const void* packed, const void* bias_bf16, void* c_bf16,
+                                        int64_t M, int64_t N, int64_t K, int group, void* stream) {
+  if (!a_bf16 || !packed || !c_bf16 || M <= 0 || N <= 0 || K <= 0 || group <= 0) return MLLM_HIP_E_BADARG;
+  if (group % 64 || K % group) return MLLM_HIP_E_SHAPE;
+  if (M * K * 2 >= ((int64_t)1 << 32) || M > INT32_MAX || N > INT32_MAX ||
+      mllm_hip_w4a16_packed_bytes(N, K, group) >= ((size_t)1 << 32))
+    return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(a_bf16) % 16 || reinterpret_cast<uintptr_t>(packed) % 16) return MLLM_HIP_E_ALIGN;
+  W4A16PArgs a{(const uint16_t*)a_bf16, (const uint8_t*)packed, (const uint16_t*)bias_bf16, (uint16_t*)c_bf16,
+               (int)M, (int)N, (int)K, group};
+  return launch_w4a16_nsplit_auto(a, (hipStream_t)stream);
+}
+
+MLLM_API int mllm_hip_w4a16_dequantize_packed(const void* packed, void* w_bf16, int64_t N, int64_t K, int group, void* stream) {
+  if (!packed || !w_bf16 || N <= 0 || K <= 0 || group <= 0) return MLLM_HIP_E_BADARG;
+  if (group % 64 || K % group || N > INT32_MAX || K > INT32_MAX) return MLLM_HIP_E_SHAPE;
+  const int64_t words = N * K / 8;
+  hipLaunchKernelGGL(w4a16_dequant_packed_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     (const uint8_t*)packed, (uint16_t*)w_bf16, (int)N, (int)K, group);
   return (int)hipGetLastError();
 }

@@ -14,7 +14,6 @@ namespace mllmhip {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // =========================================================================================================
 // per-token dynamic quantization: one workgroup per row

@@ -201,6 +201,36 @@ def w4a16_gemm(a, qw, scales, zeros, bias=None, group=128, out=None):
     return y
 
 
+def w4a16_prepack(qw, scales, zeros, group=128):
+    """Checkpoint tensors -> the packed weight blob of the fast GEMM (uint8), done once per weight."""
+    assert qw.dtype == torch.uint8 and scales.dtype == torch.float16 and qw.is_contiguous() and scales.is_contiguous()
+    N, K = qw.shape[0], qw.shape[1] * 2
+    L = _lib.lib()
+    packed = torch.empty(L.mllm_hip_w4a16_packed_bytes(N, K, group), dtype=torch.uint8, device="cuda")
+    _lib.check(L.mllm_hip_w4a16_prepack(qw.data_ptr(), scales.data_ptr(), zeros.data_ptr(), N, K, group, packed.data_ptr(),
+                                        _stream()), "mllm_hip_w4a16_prepack")
+    return packed
+
+
+def w4a16_gemm_packed(a, packed, N, bias=None, group=128, out=None):
+    """a bf16 [M, K] x packed weights (w4a16_prepack) -> bf16 [M, N]."""
+    assert a.dtype == torch.bfloat16 and a.is_contiguous()
+    M, K = a.shape
+    L = _lib.lib()
+    assert packed.numel() == L.mllm_hip_w4a16_packed_bytes(N, K, group)
+    y = out if out is not None else torch.empty((M, N), dtype=torch.bfloat16, device="cuda")
+    _lib.check(L.mllm_hip_w4a16_gemm_packed(a.data_ptr(), packed.data_ptr(), _p(bias), y.data_ptr(), M, N, K, group,
+                                            _stream()), "mllm_hip_w4a16_gemm_packed")
+    return y
+
+
+def w4a16_dequantize_packed(packed, N, K, group=128):
+    w = torch.empty((N, K), dtype=torch.bfloat16, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_w4a16_dequantize_packed(packed.data_ptr(), w.data_ptr(), N, K, group, _stream()),
+               "mllm_hip_w4a16_dequantize_packed")
+    return w
+
+
 def w4a16_dequantize(qw, scales, zeros, group=128):
     N, K = qw.shape[0], qw.shape[1] * 2
     w = torch.empty((N, K), dtype=torch.bfloat16, device="cuda")

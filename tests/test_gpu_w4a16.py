@@ -76,6 +76,52 @@ def test_gemm_vs_oracle(M, N, K, group, tile):
     assert (diff == 0).mean() > 0.97
 
 
+# shapes that reach each tile of the weights-from-global kernel (128x384, 64x384, 128x128, 64x128), ragged edges, a K
+# that is not a multiple of the 128-element K step, and groups of 64 / 128 / 256
+PACKED_SHAPES = [(1, 64, 128, 128), (9, 24, 384, 128), (130, 200, 512, 128), (64, 96, 256, 64), (257, 193, 1024, 256),
+                 (33, 128, 2560, 128), (70, 100, 192, 64), (1536, 6144, 256, 128), (512, 9216, 128, 128),
+                 (1024, 3072, 128, 64)]
+
+
+@pytest.mark.parametrize("M,N,K,group", PACKED_SHAPES)
+def test_gemm_packed_vs_oracle(M, N, K, group):
+    rng = synth.rng_for(2, 3 * M + N + K + group)
+    qw, s, zp, _, _ = synth.make_w4a16(rng, N, K, group)
+    a_bits, _ = synth.make_x_bf16(rng, M, K)
+    bias = synth.fp32_to_bf16_bits((rng.standard_normal(N) * 0.1).astype(np.float32))
+    announce("w4a16 packed gemm", M, N, K, group)
+    packed = ql.w4a16_prepack(*_dev(qw, s, zp), group)
+    table = _bits(ql.w4a16_dequantize_packed(packed, N, K, group))
+    assert _same_values(table, orc.w4a16_dequant(qw, s, zp, group))
+    c = _bits(ql.w4a16_gemm_packed(bf16_dev(a_bits), packed, N, None, group))
+    cb = _bits(ql.w4a16_gemm_packed(bf16_dev(a_bits), packed, N, bf16_dev(bias), group))
+    want = orc.w4a16_gemm(a_bits, qw, s, zp, None, group)
+    wantb = orc.w4a16_gemm(a_bits, qw, s, zp, bias, group)
+    assert rel_l2(synth.bf16_bits_to_fp32(c), synth.bf16_bits_to_fp32(want)) <= TOL
+    assert rel_l2(synth.bf16_bits_to_fp32(cb), synth.bf16_bits_to_fp32(wantb)) <= TOL
+    diff = np.abs(c.astype(np.int32) - want.astype(np.int32))
+    assert diff.max() <= 1 or rel_l2(synth.bf16_bits_to_fp32(c), synth.bf16_bits_to_fp32(want)) < 1e-4
+    assert (diff == 0).mean() > 0.97
+
+
+@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 16 + 5])
+def test_gemm_packed_every_tile(tile):
+    M, N, K, group = 200, 800, 384, 128
+    rng = synth.rng_for(2, 77 + tile)
+    qw, s, zp, _, _ = synth.make_w4a16(rng, N, K, group)
+    a_bits, _ = synth.make_x_bf16(rng, M, K)
+    L = _lib.lib()
+    packed = ql.w4a16_prepack(*_dev(qw, s, zp), group)
+    try:
+        assert L.mllm_hip_w4a16_packed_set_tuning(tile) == 0
+        announce("w4a16 packed gemm tile", tile)
+        c = _bits(ql.w4a16_gemm_packed(bf16_dev(a_bits), packed, N, None, group))
+    finally:
+        L.mllm_hip_w4a16_packed_set_tuning(0)
+    want = orc.w4a16_gemm(a_bits, qw, s, zp, None, group)
+    assert rel_l2(synth.bf16_bits_to_fp32(c), synth.bf16_bits_to_fp32(want)) <= TOL
+
+
 def test_full_size_prefill():
     """A bf16 [2048,2560], W uint4 [9728,2560] g128: a row sample against the oracle, plus linearity on all rows:
     GEMM(2*A) == 2*GEMM(A) exactly (scaling by two commutes with every rounding)."""
@@ -94,6 +140,15 @@ def test_full_size_prefill():
     a2 = synth.fp32_to_bf16_bits(a * 2)
     c2 = ql.w4a16_gemm(bf16_dev(a2), *d)
     assert torch.equal(c2.float(), c.float() * 2)
+    # (this shape runs 512 full tiles and 192 half-height tiles in the packed kernel's schedule)
+    # the prepacked-weight path: table bit-exact, same row sample, same linearity, and close to the plain path everywhere
+    packed = ql.w4a16_prepack(*d)
+    assert np.array_equal(_bits(ql.w4a16_dequantize_packed(packed, N, K)), orc.w4a16_dequant(qw, s, zp))
+    cp = ql.w4a16_gemm_packed(bf16_dev(a_bits), packed, N)
+    r = rel_l2(synth.bf16_bits_to_fp32(_bits(cp)[rows]), synth.bf16_bits_to_fp32(want))
+    assert r <= TOL, r
+    assert torch.equal(ql.w4a16_gemm_packed(bf16_dev(a2), packed, N).float(), cp.float() * 2)
+    assert rel_l2(cp.float().cpu().numpy(), c.float().cpu().numpy()) <= 1e-4
     # zero-point equal to every code -> exact zeros
     z_un = rng.integers(0, 16, (64, K // 128), dtype=np.uint8)
     qz = np.repeat(z_un, 128, axis=1)
