@@ -566,6 +566,20 @@ static int launch_w4a16_nsplit_auto(const W4A16PArgs& a, hipStream_t st) {
   }
 }
 
+template <int BM, int BN, int WM, int WN>
+static int launch_w4a16(const W4A16Args& a, hipStream_t st) {
+  constexpr int NT = (BM / WM) * (BN / WN) * 64;
+  const size_t lds = 2 * (size_t)(BM + BN) * 144;
+  const unsigned grid = (unsigned)(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN));
+  auto kern = w4a16_gemm_kernel<BM, BN, WM, WN>;
+  if (lds > 64 * 1024)
+    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds, st, a);
+  return (int)hipGetLastError();
+}
+
+static int g_w4a16_tile = 0;  // 0 = heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64
+
 }  // namespace mllmhip
 
 using namespace mllmhip;
