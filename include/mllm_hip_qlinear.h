@@ -106,6 +106,31 @@ int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
 int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_per_wg);
 
 /* ---------------------------------------------------------------------------------------------------------
+ * Q4_0 / Q8_0 Linear and MoE expert FFN for many rows on the matrix cores
+ * replaces: the same reference calls as mllm_hip_linear_q / mllm_hip_moe_ffn_q (the tinyBLAS gemm branch of
+ *           llamafile_sgemm.cpp:697-743 for M > 1, and Qwen3MoE::moeInfer, modeling_qwen3_moe_fa2.hpp:175-238)
+ * Arithmetic: the activations' Q8_0 quantization is the bit-exact one; both operands then carry their block scale,
+ *   xh = fp16(dX * qX), wh = fp16(dW * qW), each product exact before its single rounding to fp16, and
+ *   y[m][n] = sum_k xh[m][k] * wh[n][k] accumulates in fp32 in v_mfma_f32_32x32x16_f16.  The two roundings (relative
+ *   error <= 2^-12 each) keep y within about 3e-4 relative L2 of the reference's fp32 block arithmetic; the entry points
+ *   above keep that arithmetic itself.  |dX*qX| and |dW*qW| must stay below 65504.
+ * Weights: "gemm-packed" once at load time from the reference blocks (codes in matrix-core operand order, N padded to
+ *   32 and K to 128; same bytes per element as the blocks).
+ * ------------------------------------------------------------------------------------------------------- */
+size_t mllm_hip_q_gemm_packed_bytes(int wtype, int64_t N, int64_t K);
+int mllm_hip_q_gemm_prepack(int wtype, const void* blocks, int weight_scale_mode, void* gemm_packed, int64_t N, int64_t K,
+                            void* stream);
+size_t mllm_hip_linear_q_gemm_workspace_bytes(int64_t M, int64_t K);
+int mllm_hip_linear_q_gemm(int wtype, const void* gemm_packed, const void* x, int x_dtype, const float* bias, float* y,
+                           int64_t M, int64_t N, int64_t K, int act_scale_mode, void* workspace, void* stream);
+/* Same arguments as mllm_hip_moe_ffn_q; the three expert arrays are E gemm-packed matrices back to back
+ * (stride mllm_hip_q_gemm_packed_bytes). */
+size_t mllm_hip_moe_gemm_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k);
+int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed,
+                            const void* x, int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T,
+                            int64_t H, int64_t I, int E, int k, int act_scale_mode, void* workspace, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------
  * W8A8 Linear (prefill): per-token dynamic int8 activations x int8 weights with per-channel scales
  * replaces: CompressedTensorsW8A8Int8Scheme.apply = per_token_quant_int8 + int8_scaled_mm
  *           pymllm/quantization/methods/compressed_tensors.py:450-468
@@ -146,6 +171,9 @@ int mllm_hip_w8a8_linear_packed(const void* x, int x_dtype, const void* W_packed
 /* GEMM tile override for tuning sweeps (plain-layout entry points): 0 heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64
  * workgroup tiles through LDS, 4 = weight operands fetched straight from global memory (K % 128 == 0, else 2). */
 int mllm_hip_w8a8_set_tuning(int tile);
+/* Tile override for the weights-from-global kernel (packed entry points and tile 4 above): 0 heuristic, 1 = 128x384,
+ * 2 = 64x384, 3 = 128x128, 4 = 64x128, 5 = 128x256. */
+int mllm_hip_w8a8_nsplit_set_tuning(int tile);
 
 /* ---------------------------------------------------------------------------------------------------------
  * W4A16 Linear (prefill): bf16 activations x uint4 weights, per-group fp16 scale and uint4 zero-point

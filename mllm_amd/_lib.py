@@ -55,6 +55,7 @@ def lib():
         L.mllm_hip_w8a8_workspace_bytes.argtypes = [i64, i64]
         L.mllm_hip_w8a8_linear.argtypes = [vp, ci, vp, vp, vp, vp, i64, i64, i64, vp, vp]
         L.mllm_hip_w8a8_set_tuning.argtypes = [ci]
+        L.mllm_hip_w8a8_nsplit_set_tuning.argtypes = [ci]
         L.mllm_hip_w8a8_packed_bytes.restype = C.c_size_t
         L.mllm_hip_w8a8_packed_bytes.argtypes = [i64, i64]
         L.mllm_hip_w8a8_prepack.argtypes = [vp, i64, i64, vp, vp]
@@ -75,6 +76,15 @@ def lib():
         L.mllm_hip_moe_workspace_bytes.restype = C.c_size_t
         L.mllm_hip_moe_workspace_bytes.argtypes = [i64, i64, i64, ci, ci]
         L.mllm_hip_moe_ffn_q.argtypes = [ci, vp, vp, vp, vp, ci, vp, vp, vp, i64, i64, i64, ci, ci, ci, vp, vp]
+        L.mllm_hip_q_gemm_packed_bytes.restype = C.c_size_t
+        L.mllm_hip_q_gemm_packed_bytes.argtypes = [ci, i64, i64]
+        L.mllm_hip_q_gemm_prepack.argtypes = [ci, vp, ci, vp, i64, i64, vp]
+        L.mllm_hip_linear_q_gemm_workspace_bytes.restype = C.c_size_t
+        L.mllm_hip_linear_q_gemm_workspace_bytes.argtypes = [i64, i64]
+        L.mllm_hip_linear_q_gemm.argtypes = [ci, vp, vp, ci, vp, vp, i64, i64, i64, ci, vp, vp]
+        L.mllm_hip_moe_gemm_workspace_bytes.restype = C.c_size_t
+        L.mllm_hip_moe_gemm_workspace_bytes.argtypes = [i64, i64, i64, ci, ci]
+        L.mllm_hip_moe_ffn_q_gemm.argtypes = [ci, vp, vp, vp, vp, ci, vp, vp, vp, i64, i64, i64, ci, ci, ci, vp, vp]
         L.mllm_hip_moe_route.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, vp]
         L.mllm_hip_matmul_f32.argtypes = [vp, vp, vp, i64, i64, i64, ci, ci, vp]
         _lib = L

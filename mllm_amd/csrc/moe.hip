@@ -34,9 +34,13 @@ struct RouteOut {
   int* ntiles;       // [1]
 };
 
-__global__ __launch_bounds__(1024) void moe_route_kernel(const int32_t* __restrict__ ids, int n, int E, RouteOut o) {
-  extern __shared__ int s_cnt[];  // [E] counts, then [E] cursors
+__global__ __launch_bounds__(1024) void moe_route_kernel(const int32_t* __restrict__ ids, int n, int E, int tile_h, RouteOut o) {
+  extern __shared__ int s_cnt[];  // [E] counts, [E] cursors, [E] scan scratch x 3
   int* s_cur = s_cnt + E;
+  int* s_off = s_cur + E;   // exclusive scan of the counts
+  int* s_full = s_off + E;  // exclusive scan of the full-tile counts
+  int* s_part = s_full + E; // exclusive scan of the partial-tile flags
+  __shared__ int s_tot[3];
   for (int e = threadIdx.x; e < E; e += blockDim.x) s_cnt[e] = 0;
   __syncthreads();
   for (int i = threadIdx.x; i < n; i += blockDim.x) {
@@ -44,31 +48,50 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const int32_t* __restri
     if (e >= 0 && e < E) atomicAdd(&s_cnt[e], 1);
   }
   __syncthreads();
-  if (threadIdx.x == 0) {
-    int off = 0, nt = 0;
-    for (int e = 0; e < E; e++) {
-      const int c = s_cnt[e];
-      o.counts[e] = c;
-      o.offsets[e] = off;
-      s_cur[e] = off;
-      off += c;
-    }
-    o.offsets[E] = off;
-    // tile list, full tiles first so that the long-running workgroups start early
-    for (int pass = 0; pass < 2; pass++)
-      for (int e = 0; e < E; e++) {
-        const int c = s_cnt[e], base = o.offsets[e];
-        for (int r = 0; r < c; r += TOK_TILE) {
-          const int rows = min(TOK_TILE, c - r);
-          if ((rows == TOK_TILE) == (pass == 0)) {
-            o.tile_expert[nt] = e;
-            o.tile_row0[nt] = base + r;
-            o.tile_rows[nt] = rows;
-            nt++;
-          }
-        }
+  // three exclusive scans over the experts, one wave each (E is at most a few thousand: 64 experts per step)
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (wave < 3) {
+    int* dst = wave == 0 ? s_off : wave == 1 ? s_full : s_part;
+    int run = 0;
+    for (int base = 0; base < E; base += 64) {
+      const int e = base + lane;
+      const int c = e < E ? s_cnt[e] : 0;
+      const int v = wave == 0 ? c : wave == 1 ? c / tile_h : (c % tile_h != 0);
+      int incl = v;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int t = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += t;
       }
-    o.ntiles[0] = nt;
+      if (e < E) dst[e] = run + incl - v;
+      run += __shfl(incl, 63, 64);
+    }
+    if (lane == 0) s_tot[wave] = run;
+  }
+  __syncthreads();
+  // tile list, full tiles first so that the long-running workgroups start early
+  for (int e = threadIdx.x; e < E; e += blockDim.x) {
+    const int c = s_cnt[e], base = s_off[e];
+    o.counts[e] = c;
+    o.offsets[e] = base;
+    s_cur[e] = base;
+    const int nf = c / tile_h;
+    for (int t = 0; t < nf; t++) {
+      const int slot = s_full[e] + t;
+      o.tile_expert[slot] = e;
+      o.tile_row0[slot] = base + t * tile_h;
+      o.tile_rows[slot] = tile_h;
+    }
+    if (c % tile_h) {
+      const int slot = s_tot[1] + s_part[e];
+      o.tile_expert[slot] = e;
+      o.tile_row0[slot] = base + nf * tile_h;
+      o.tile_rows[slot] = c % tile_h;
+    }
+  }
+  if (threadIdx.x == 0) {
+    o.offsets[E] = s_tot[0];
+    o.ntiles[0] = s_tot[1] + s_tot[2];
   }
   __syncthreads();
   // the order inside an expert does not matter: every row is computed independently of its neighbours
@@ -79,12 +102,12 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const int32_t* __restri
 }
 
 // identity routing for a plain Linear over M rows
-__global__ void identity_tiles_kernel(int M, RouteOut o) {
-  const int nt = (M + TOK_TILE - 1) / TOK_TILE;
+__global__ void identity_tiles_kernel(int M, int tile_h, RouteOut o) {
+  const int nt = (M + tile_h - 1) / tile_h;
   for (int t = threadIdx.x; t < nt; t += blockDim.x) {
     o.tile_expert[t] = 0;
-    o.tile_row0[t] = t * TOK_TILE;
-    o.tile_rows[t] = min(TOK_TILE, M - t * TOK_TILE);
+    o.tile_row0[t] = t * tile_h;
+    o.tile_rows[t] = min(tile_h, M - t * tile_h);
   }
   if (threadIdx.x == 0) o.ntiles[0] = nt;
 }
@@ -367,6 +390,448 @@ __global__ __launch_bounds__(MODE == 1 ? 512 : 256) void qgemm_tile_kernel(QGemm
   }
 }
 
+// =========================================================================================================
+// Matrix-core path for many rows: fp16 operands with the block scales folded in
+//
+//   y[row][n] = sum_k xh[row][k] * wh[n][k],   xh = fp16(dX * qX) (the Q8_0 round trip of the activations, exact product
+//   rounded once to fp16), wh = fp16(dW * qW) (likewise), fp32 accumulation in v_mfma_f32_32x32x16_f16.
+//
+// The block-dot form above needs three vector-ALU operations per (row, channel, block) to scale and add the int32 block
+// sums, which bounds it far below the matrix rate.  Folding the scales into 16-bit operands moves that work to the
+// operands: about two operations per WEIGHT element per 32*TM rows, nothing per accumulator.  Both roundings are to 11
+// significant bits (relative error <= 2^-12 each), which keeps the result within about 3e-4 relative L2 of the
+// reference's fp32 block arithmetic.  |dX*qX| and |dW*qW| must stay below 65504 (fp16).
+//
+// Weight layout ("gemm-packed", mllm_hip_q_gemm_prepack): codes in v_mfma_*_32x32x16 operand order, N padded to 32 rows
+// and K to 128 elements with zero blocks;
+//   Q4_0  q  [N/32][K/64][64 lanes][16 B]: lane l = (row l%32, half l/32); dword d of its 16 bytes holds the eight
+//            elements k = 64 kb + 16 d + 8 (l/32) + 0..7: element 2i in nibble i, element 2i+1 in nibble 4+i (so that
+//            (dword >> 4i) & 0x000f000f is the pair (2i, 2i+1) in the two halves of a register)
+//   Q8_0  q  [N/32][K/64][2][64 lanes][16 B]: plane p holds d = 2p, 2p+1; each d is two dwords of four codes in byte
+//            order e0, e2, e1, e3
+//   scales   [N/32][K/64][32 rows] dwords: fp16 scale of block 2kb | fp16 scale of block 2kb+1 << 16, after the
+//            weight_scale_mode decoding
+// Kernel structure as the W4A16 weights-from-global kernel: four waves side by side along N, activations via LDS,
+// weights straight from global memory two K steps ahead, dequantized one MFMA step ahead in the shadows of the MFMAs.
+// =========================================================================================================
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__host__ __device__ inline int64_t qg_kp(int64_t K) { return (K + 127) / 128 * 128; }
+__host__ __device__ inline int64_t qg_np(int64_t N) { return (N + 31) / 32 * 32; }
+__host__ __device__ inline int64_t qg_qbytes(int wtype, int64_t N, int64_t K) {
+  return wtype == MLLM_HIP_Q4_0 ? qg_np(N) * qg_kp(K) / 2 : qg_np(N) * qg_kp(K);
+}
+__host__ __device__ inline int64_t qg_bytes(int wtype, int64_t N, int64_t K) {
+  return qg_qbytes(wtype, N, K) + qg_np(N) * (qg_kp(K) / 64) * 4;
+}
+
+// one output dword of the code area per thread
+template <int WT>
+__global__ __launch_bounds__(256) void qg_prepack_q_kernel(const unsigned char* __restrict__ blocks, uint32_t* __restrict__ P,
+                                                           int N, int K, int64_t words) {
+  const int64_t w = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (w >= words) return;
+  const int kbs = (int)(qg_kp(K) / 64), nblk = K / QK;
+  constexpr int BS = WT == MLLM_HIP_Q4_0 ? 18 : 34;
+  uint32_t v = 0;
+  if (WT == MLLM_HIP_Q4_0) {
+    const int d = (int)(w % 4), l = (int)((w / 4) % 64);
+    const int64_t blk = w / 256;
+    const int kb = (int)(blk % kbs), nb = (int)(blk / kbs);
+    const int n = nb * 32 + (l & 31), k0 = kb * 64 + d * 16 + (l >> 5) * 8;
+    if (n < N && k0 < K) {
+      const unsigned char* qs = blocks + ((int64_t)n * nblk + k0 / QK) * BS + 2;
+      const int o = k0 % QK;  // 0, 8, 16, 24: elements o..o+7 are the low (o < 16) or high nibbles of qs[o % 16 ..]
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const uint32_t byte = qs[(o & 15) + i];
+        const uint32_t e = o < 16 ? (byte & 15u) : (byte >> 4);
+        v |= e << (4 * ((i >> 1) + 4 * (i & 1)));
+      }
+    }
+  } else {
+    const int x = (int)(w % 4), l = (int)((w / 4) % 64), pl = (int)((w / 256) % 2);
+    const int64_t blk = w / 512;
+    const int kb = (int)(blk % kbs), nb = (int)(blk / kbs);
+    const int d = 2 * pl + x / 2;
+    const int n = nb * 32 + (l & 31), k0 = kb * 64 + d * 16 + (l >> 5) * 8 + 4 * (x % 2);
+    if (n < N && k0 < K) {
+      const unsigned char* qs = blocks + ((int64_t)n * nblk + k0 / QK) * BS + 2 + k0 % QK;
+      v = (uint32_t)qs[0] | ((uint32_t)qs[2] << 8) | ((uint32_t)qs[1] << 16) | ((uint32_t)qs[3] << 24);
+    }
+  }
+  P[w] = v;
+}
+template <int WT>
+__global__ __launch_bounds__(256) void qg_prepack_s_kernel(const unsigned char* __restrict__ blocks, uint32_t* __restrict__ S,
+                                                           int N, int K, int x86_scale, int64_t count) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (nb, kb, row)
+  if (i >= count) return;
+  const int kbs = (int)(qg_kp(K) / 64), nblk = K / QK;
+  constexpr int BS = WT == MLLM_HIP_Q4_0 ? 18 : 34;
+  const int row = (int)(i % 32), kb = (int)((i / 32) % kbs), nb = (int)(i / 32 / kbs);
+  const int n = nb * 32 + row;
+  uint32_t v = 0;
+#pragma unroll
+  for (int h = 0; h < 2; h++) {
+    const int b = 2 * kb + h;
+    if (n < N && b < nblk) {
+      const unsigned char* p = blocks + ((int64_t)n * nblk + b) * BS;
+      uint16_t bits = (uint16_t)(p[0] | (p[1] << 8));
+      if (x86_scale) bits = x86_scale_bits(bits);
+      v |= (uint32_t)bits << (16 * h);
+    }
+  }
+  S[i] = v;
+}
+
+// activations: Q8_0 quantization (bit-exact codes and scale) and back to fp16 in one pass
+// (xl, when asked for: the rounding residual dX*qX - xh, exact in fp16, for the two-term gate/up path)
+__global__ void qg_act_kernel(const void* __restrict__ x, int x_dtype, uint16_t* __restrict__ xh, uint16_t* __restrict__ xl,
+                              int64_t nblocks, int x86_scale) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= nblocks) return;
+  float v[32];
+  uint32_t q[8];
+  int sum;
+  load_block_f32(x, x_dtype, i * QK, v);
+  uint16_t bits = quantize_block_q8_0(v, q, sum);
+  if (x86_scale) bits = x86_scale_bits(bits);
+  const float d = f16bits_to_f32(bits);
+  uint32_t o[16], ol[16];
+#pragma unroll
+  for (int j = 0; j < 16; j++) {
+    const float a = d * (float)(int8_t)(q[j / 2] >> (16 * (j & 1)));       // exact in fp32: 11 x 8 bits
+    const float b = d * (float)(int8_t)(q[j / 2] >> (16 * (j & 1) + 8));
+    const uint16_t ha = f32_to_f16bits(a), hb = f32_to_f16bits(b);
+    o[j] = (uint32_t)ha | ((uint32_t)hb << 16);
+    ol[j] = (uint32_t)f32_to_f16bits(a - f16bits_to_f32(ha)) | ((uint32_t)f32_to_f16bits(b - f16bits_to_f32(hb)) << 16);
+  }
+  u32x4* out = reinterpret_cast<u32x4*>(xh + i * QK);
+#pragma unroll
+  for (int j = 0; j < 4; j++) out[j] = u32x4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
+  if (xl) {
+    u32x4* outl = reinterpret_cast<u32x4*>(xl + i * QK);
+#pragma unroll
+    for (int j = 0; j < 4; j++) outl[j] = u32x4{ol[4 * j], ol[4 * j + 1], ol[4 * j + 2], ol[4 * j + 3]};
+  }
+}
+
+struct QG2Args {
+  const char* W0;        // gemm-packed weights of matrix 0 (gate, or the only matrix), expert e at W0 + e * wstride
+  const char* W1;        // gemm-packed weights of matrix 1 (up) in the fused gate/up mode
+  size_t wstride;
+  const uint16_t* xh;    // fp16 activations [a_rows][K]
+  const uint16_t* xl;    // their rounding residuals, same shape (two-term mode only)
+  const int* a_index;    // activation row of sorted position pos is a_index[pos] / a_div ; null: pos itself
+  int a_div;
+  int a_rows;
+  const int* o_index;    // output row of sorted position pos (null: pos itself)
+  float* out;            // fp32 [..][N]       (one-matrix mode)
+  const float* bias;     // [N] or null        (one-matrix mode)
+  uint16_t* hh;          // gate/up mode: fp16 Q8_0 round trip of silu(g)*u, [rows][N]
+  const int* tile_expert;
+  const int* tile_row0;
+  const int* tile_rows;
+  const int* ntiles;
+  int N, K;
+  int wtype;
+  int x86_scale;
+};
+
+// pair `b` (elements 2b, 2b+1) of the eight weights of one MFMA step, scaled: one dword of two fp16.  With PREC == 2 also
+// the rounding residual of the product (exact: the error of a product of two fp16 numbers is an fp16 number).
+template <int WT, int PREC>
+__device__ __forceinline__ uint32_t qg_pair(const u32x4 (&rq)[WT == MLLM_HIP_Q4_0 ? 1 : 2], int d, int b, f16x2 dd, uint32_t& lo) {
+  uint32_t t;
+  f16x2 off;
+  if (WT == MLLM_HIP_Q4_0) {
+    t = ((rq[0][d] >> (4 * b)) & 0x000f000fu) | 0x64006400u;       // (1024 + q) in both halves
+    off = f16x2{(_Float16)1032.f, (_Float16)1032.f};               // ... - 1032 = q - 8, exact
+  } else {
+    const uint32_t w = rq[d >> 1][2 * (d & 1) + (b >> 1)] ^ 0x80808080u;  // codes + 128, bytes e0 e2 e1 e3
+    t = ((w >> (8 * (b & 1))) & 0x00ff00ffu) | 0x64006400u;
+    off = f16x2{(_Float16)1152.f, (_Float16)1152.f};
+  }
+  const f16x2 c = __builtin_bit_cast(f16x2, t) - off;              // v_pk_add_f16, exact
+  const f16x2 r = c * dd;                                          // v_pk_mul_f16: one rounding
+  if (PREC == 2) lo = __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(c, dd, -r));  // v_pk_fma_f16
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+// One tile: `rows` (<= 32 TM) sorted positions from row0 x 128 TN channels from n0, NW weight matrices (1, or gate + up).
+// PREC == 2 carries both operands as fp16 value + fp16 residual and adds the two first-order cross terms
+// (wh*xh + wl*xh + wh*xl): the operands are then exact and the result is the fp32 sum of exact products.  The gate/up
+// stage needs it: its output is re-quantized to Q8_0, and a relative perturbation eps of the values in front of that
+// rounding step flips codes often enough to come out as about sqrt(eps/40) in relative L2.
+template <int WT, int NW, int TM, int TN, int PREC>
+__device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int row0, const int rows, const int n0,
+                                        unsigned char* smem) {
+  constexpr int BK = 64, LDK = 2 * BK + 16, KS = BK / 16;
+  constexpr int BM = TM * 32, WN = TN * 32;
+  constexpr int CA = TM;  // 16-byte activation chunks per thread and K step: 32 TM rows x 8 chunks over 256 threads
+  constexpr int STAGE = PREC * BM * LDK;  // value rows, then residual rows
+  constexpr int QW = WT == MLLM_HIP_Q4_0 ? 1 : 2;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lrow = lane & 31, hi = lane >> 5;
+  const int Kp = (int)qg_kp(a.K), kbs = Kp / 64, nbs = (int)(qg_np(a.N) / 32);
+  const int64_t qbytes = qg_qbytes(WT, a.N, a.K), wbytes = qg_bytes(WT, a.N, a.K);
+
+  const __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.xh), 0, (uint32_t)((int64_t)a.a_rows * a.K * 2), 0x00020000);
+  __amdgpu_buffer_rsrc_t rW[NW];
+  rW[0] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a.W0 + (size_t)e * a.wstride), 0, (uint32_t)wbytes, 0x00020000);
+  if (NW == 2) rW[NW - 1] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a.W1 + (size_t)e * a.wstride), 0, (uint32_t)wbytes, 0x00020000);
+
+  // activation chunk c of a thread: tile row (tid + 256 c) / 8, 16-byte column (tid + 256 c) % 8.  Rows past `rows` repeat
+  // the last one (never stored); columns past K read as zeros so that the zero-padded weight tail meets no other row.
+  uint32_t offA[CA];
+  const int colA = (tid % 8) * 8;
+#pragma unroll
+  for (int c = 0; c < CA; c++) {
+    const int pos = row0 + min((tid + c * 256) / 8, rows - 1);
+    const int arow = a.a_index ? a.a_index[pos] / a.a_div : pos;
+    offA[c] = (uint32_t)(((int64_t)arow * a.K + colA) * 2);
+  }
+  uint32_t offQ[TN], offS[TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int nb = min((n0 + wave * WN) / 32 + j, nbs - 1);
+    offQ[j] = (uint32_t)((int64_t)nb * kbs * (1024 * QW) + lane * 16);
+    offS[j] = (uint32_t)(qbytes + ((int64_t)nb * kbs * 32 + lrow) * 4);
+  }
+  const __amdgpu_buffer_rsrc_t rAl = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(PREC == 2 ? a.xl : a.xh), 0, (uint32_t)((int64_t)a.a_rows * a.K * 2), 0x00020000);
+  auto loadA = [&](int k0, u32x4 (&ga)[PREC][CA]) {
+    const bool ok = k0 + colA < a.K;
+#pragma unroll
+    for (int c = 0; c < CA; c++) {
+      ga[0][c] = __builtin_amdgcn_raw_buffer_load_b128(rA, ok ? offA[c] : 0xffffffffu, k0 * 2, 0);
+      if (PREC == 2) ga[PREC - 1][c] = __builtin_amdgcn_raw_buffer_load_b128(rAl, ok ? offA[c] : 0xffffffffu, k0 * 2, 0);
+    }
+  };
+  auto storeA = [&](int buf, const u32x4 (&ga)[PREC][CA]) {
+#pragma unroll
+    for (int p = 0; p < PREC; p++)
+#pragma unroll
+      for (int c = 0; c < CA; c++) {
+        const int idx = tid + c * 256;
+        *reinterpret_cast<u32x4*>(smem + buf * STAGE + (p * BM + idx / 8) * LDK + (idx % 8) * 16) = ga[p][c];
+      }
+  };
+  auto readA = [&](int buf, int ks, f16x8 (&fa)[PREC][TM]) {
+#pragma unroll
+    for (int p = 0; p < PREC; p++)
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+        fa[p][i] = *reinterpret_cast<const f16x8*>(smem + buf * STAGE + (p * BM + i * 32 + lrow) * LDK + ks * 32 + hi * 16);
+  };
+
+  v16f acc[NW][TN][TM];
+#pragma unroll
+  for (int w = 0; w < NW; w++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[w][j][i][r] = 0.f;
+
+  u32x4 ga[PREC][CA];
+  u32x4 rq[2][NW][TN][QW];      // packed codes of K steps kt (set kt & 1) and kt + 1
+  uint32_t rs[2][NW][TN];       // their two block scales
+  f16x8 fb[2][NW][TN][PREC];    // dequantized operands of MFMA step ks (set ks & 1): value, residual
+  f16x8 fa[2][PREC][TM];
+  auto loadW = [&](int set, int kb) {
+#pragma unroll
+    for (int w = 0; w < NW; w++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+#pragma unroll
+        for (int p = 0; p < QW; p++) rq[set][w][j][p] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], offQ[j], (kb * QW + p) * 1024, 0);
+        rs[set][w][j] = __builtin_amdgcn_raw_buffer_load_b32(rW[w], offS[j], kb * 128, 0);
+      }
+  };
+  auto scale2 = [&](uint32_t s, int d) -> f16x2 {  // the block scale of dword d in both halves
+    const uint32_t h = d < 2 ? (s & 0xffffu) : (s >> 16);
+    return __builtin_bit_cast(f16x2, h | (h << 16));
+  };
+  loadA(0, ga);
+  loadW(0, 0);
+  loadW(1, 1);
+  storeA(0, ga);
+  __syncthreads();
+  readA(0, 0, fa[0]);
+#pragma unroll
+  for (int w = 0; w < NW; w++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      const f16x2 dd = scale2(rs[0][w][j], 0);
+      uint32_t o[4], ol[4] = {0, 0, 0, 0};
+#pragma unroll
+      for (int b = 0; b < 4; b++) o[b] = qg_pair<WT, PREC>(rq[0][w][j], 0, b, dd, ol[b]);
+      fb[0][w][j][0] = __builtin_bit_cast(f16x8, u32x4{o[0], o[1], o[2], o[3]});
+      if (PREC == 2) fb[0][w][j][PREC - 1] = __builtin_bit_cast(f16x8, u32x4{ol[0], ol[1], ol[2], ol[3]});
+    }
+
+  // one K step (64 elements) with its weights in register set CUR; refills that set with K step kt + 2 when done with it
+  auto kstep = [&](auto cur_tag, int kt) {
+    constexpr int CUR = decltype(cur_tag)::value;
+    const int buf = kt & 1;
+    loadA((kt + 1) * BK, ga);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      if (ks < KS - 1) {
+        readA(buf, ks + 1, fa[(ks + 1) & 1]);  // the next step's activations while this one's MFMAs run
+      } else {
+        storeA(buf ^ 1, ga);
+        __syncthreads();
+        readA(buf ^ 1, 0, fa[(ks + 1) & 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      const int ns = ks < KS - 1 ? CUR : CUR ^ 1, nd = (ks + 1) % KS;  // register set and dword of the NEXT step's weights
+#pragma unroll
+      for (int w = 0; w < NW; w++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          // the dequantization of the next step's operand is cut into TM pieces, one pinned into the shadow of each MFMA
+          const f16x2 dd = scale2(rs[ns][w][j], nd);
+          uint32_t o[4], ol[4] = {0, 0, 0, 0};
+#pragma unroll
+          for (int i = 0; i < TM; i++) {
+            acc[w][j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ks & 1][w][j][0], fa[ks & 1][0][i], acc[w][j][i], 0, 0, 0);
+            if (PREC == 2) {
+              acc[w][j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ks & 1][w][j][PREC - 1], fa[ks & 1][0][i], acc[w][j][i], 0, 0, 0);
+              acc[w][j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ks & 1][w][j][0], fa[ks & 1][PREC - 1][i], acc[w][j][i], 0, 0, 0);
+            }
+#pragma unroll
+            for (int b = i * 4 / TM; b < (i + 1) * 4 / TM; b++) o[b] = qg_pair<WT, PREC>(rq[ns][w][j], nd, b, dd, ol[b]);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          fb[(ks + 1) & 1][w][j][0] = __builtin_bit_cast(f16x8, u32x4{o[0], o[1], o[2], o[3]});
+          if (PREC == 2) fb[(ks + 1) & 1][w][j][PREC - 1] = __builtin_bit_cast(f16x8, u32x4{ol[0], ol[1], ol[2], ol[3]});
+          if (ks == KS - 2) {  // the set's last dword is consumed: fetch K step kt + 2 into it
+#pragma unroll
+            for (int p = 0; p < QW; p++)
+              rq[CUR][w][j][p] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], offQ[j], ((kt + 2) * QW + p) * 1024, 0);
+            rs[CUR][w][j] = __builtin_amdgcn_raw_buffer_load_b32(rW[w], offS[j], (kt + 2) * 128, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+  };
+  const int KT = Kp / BK;  // even
+  for (int kt = 0; kt < KT; kt += 2) {
+    kstep(std::integral_constant<int, 0>{}, kt);
+    kstep(std::integral_constant<int, 1>{}, kt + 1);
+  }
+  __syncthreads();
+
+  // acc[w][j][i][4g+e] = result[row0 + 32i + lrow][n0 + wave*WN + 32j + 8g + 4hi + e]
+  if (NW == 1) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int r = i * 32 + lrow;
+      if (r < rows) {
+        const int pos = row0 + r;
+        float* orow = a.out + (int64_t)(a.o_index ? a.o_index[pos] : pos) * a.N;
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            const int n = n0 + wave * WN + j * 32 + 8 * g + 4 * hi;
+            f32x4 v = {acc[0][j][i][4 * g], acc[0][j][i][4 * g + 1], acc[0][j][i][4 * g + 2], acc[0][j][i][4 * g + 3]};
+            if (n + 3 < a.N && a.N % 4 == 0) {
+              if (a.bias) v += *reinterpret_cast<const f32x4*>(a.bias + n);
+              *reinterpret_cast<f32x4*>(orow + n) = v;
+            } else {
+#pragma unroll
+              for (int e2 = 0; e2 < 4; e2++)
+                if (n + e2 < a.N) orow[n + e2] = a.bias ? v[e2] + a.bias[n + e2] : v[e2];
+            }
+          }
+      }
+    }
+  } else {
+    // h = silu(gate) * up, Q8_0 round trip over each block of 32 channels (a block is one column tile j: 16 channels in
+    // this lane, 16 in lane ^ 32), written as fp16 for the next Linear
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int r = i * 32 + lrow;
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        float h[16];
+        float amax = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+          h[q] = silu_f(acc[0][j][i][q]) * acc[NW - 1][j][i][q];
+          amax = fmaxf(amax, fabsf(h[q]));
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        const float d = amax / 127.f;
+        const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
+        uint16_t bits = f32_to_f16bits(d);
+        if (a.x86_scale) bits = x86_scale_bits(bits);
+        const float deff = f16bits_to_f32(bits);
+        if (r < rows) {
+          uint16_t* hrow = a.hh + (int64_t)(row0 + r) * a.N;
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            const int n = n0 + wave * WN + j * 32 + 8 * g + 4 * hi;
+            uint32_t o[2];
+#pragma unroll
+            for (int e2 = 0; e2 < 2; e2++) {
+              const int q0 = min(127, max(-128, (int)rintf(h[4 * g + 2 * e2] * idv)));
+              const int q1 = min(127, max(-128, (int)rintf(h[4 * g + 2 * e2 + 1] * idv)));
+              o[e2] = (uint32_t)f32_to_f16bits(deff * (float)q0) | ((uint32_t)f32_to_f16bits(deff * (float)q1) << 16);
+            }
+            if (n + 3 < a.N) *reinterpret_cast<uint2*>(hrow + n) = uint2{o[0], o[1]};
+          }
+        }
+      }
+    }
+  }
+}
+
+// MODE 0: one matrix, 128 x 256 tiles, one-term operands.  MODE 1: gate and up together with two-term operands; a tile of
+// the list is cut into halves of 64 rows (blockIdx.z) x 128 channels.
+// The tile height follows the rows the tile really has: short tiles skip the MFMAs of empty row blocks.
+template <int WT, int MODE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qg_kernel(QG2Args a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int t = blockIdx.x;
+  if (t >= a.ntiles[0]) return;
+  const int e = a.tile_expert[t];
+  int row0 = a.tile_row0[t], rows = a.tile_rows[t];
+  if (MODE == 1) {
+    const int n0 = blockIdx.y * 128;
+    row0 += 64 * blockIdx.z;
+    rows -= 64 * blockIdx.z;
+    if (rows <= 0) return;
+    if (rows > 32) qg_tile<WT, 2, 2, 1, 2>(a, e, row0, min(rows, 64), n0, smem);
+    else qg_tile<WT, 2, 1, 1, 2>(a, e, row0, rows, n0, smem);
+  } else {
+    const int n0 = blockIdx.y * 256;
+    if (rows > 64) qg_tile<WT, 1, 4, 2, 1>(a, e, row0, rows, n0, smem);
+    else if (rows > 32) qg_tile<WT, 1, 2, 2, 1>(a, e, row0, rows, n0, smem);
+    else qg_tile<WT, 1, 1, 2, 1>(a, e, row0, rows, n0, smem);
+  }
+}
+
+constexpr int QG_TILE_H = 128;
+
+template <int MODE>
+static int launch_qg(const QG2Args& a, unsigned max_tiles, hipStream_t st) {
+  constexpr int TN = MODE == 1 ? 1 : 2;
+  const dim3 grid(max_tiles, (unsigned)((a.N + 128 * TN - 1) / (128 * TN)), MODE == 1 ? 2 : 1);
+  const size_t lds = 2 * (size_t)QG_TILE_H * (2 * 64 + 16);  // MODE 1: half the rows, value + residual
+  if (a.wtype == MLLM_HIP_Q4_0) hipLaunchKernelGGL((qg_kernel<MLLM_HIP_Q4_0, MODE>), grid, dim3(256), lds, st, a);
+  else hipLaunchKernelGGL((qg_kernel<MLLM_HIP_Q8_0, MODE>), grid, dim3(256), lds, st, a);
+  return (int)hipGetLastError();
+}
+
 // y[t][h] = sum_j per[t*k + j][h] * w[t][j]   (multiply, then add in j order: modeling_qwen3_moe_fa2.hpp:233-236)
 __global__ void moe_combine_kernel(const float* __restrict__ per, const float* __restrict__ w, const int32_t* __restrict__ ids,
                                    float* __restrict__ y, int64_t T, int H, int k, int E) {
@@ -453,7 +918,7 @@ MLLM_API int mllm_hip_linear_q(int wtype, const void* packed, const void* x, int
   const int64_t nblocks = M * (K / QK);
   hipLaunchKernelGGL(quant_rows_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, aq, ad, nblocks,
                      act_scale_mode == MLLM_HIP_SCALE_X86_REF);
-  hipLaunchKernelGGL(identity_tiles_kernel, dim3(1), dim3(256), 0, st, (int)M, ro);
+  hipLaunchKernelGGL(identity_tiles_kernel, dim3(1), dim3(256), 0, st, (int)M, TOK_TILE, ro);
   QGemmArgs a{};
   a.W0 = a.W1 = reinterpret_cast<const char*>(packed);
   a.wstride = 0;
@@ -482,7 +947,7 @@ MLLM_API int mllm_hip_moe_route(const int32_t* topk_ids, int64_t T, int E, int k
   hipStream_t st = (hipStream_t)stream;
   Carver c(workspace);
   RouteOut ro = carve_route(c, E, T * k);
-  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 2 * E * sizeof(int), st, topk_ids, (int)(T * k), E, ro);
+  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 5 * E * sizeof(int), st, topk_ids, (int)(T * k), E, TOK_TILE, ro);
   HIP_RET(hipGetLastError());
   if (counts) HIP_RET(hipMemcpyAsync(counts, ro.counts, E * sizeof(int), hipMemcpyDeviceToDevice, st));
   if (offsets) HIP_RET(hipMemcpyAsync(offsets, ro.offsets, (E + 1) * sizeof(int), hipMemcpyDeviceToDevice, st));
@@ -513,7 +978,7 @@ MLLM_API int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* 
   RouteOut ro = carve_route(c, E, T * k);
   const unsigned max_tiles = (unsigned)(E + (T * k) / TOK_TILE + 1);
 
-  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 2 * E * sizeof(int), st, topk_ids, (int)(T * k), E, ro);
+  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 5 * E * sizeof(int), st, topk_ids, (int)(T * k), E, TOK_TILE, ro);
   const int64_t nblocks = T * (H / QK);
   hipLaunchKernelGGL(quant_rows_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, xq, xd, nblocks, x86);
 
@@ -536,6 +1001,134 @@ MLLM_API int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* 
   a.o_index = ro.sorted_idx; a.out = per; a.bias = nullptr; a.hq = nullptr; a.hd = nullptr;
   a.N = (int)H; a.K = (int)I;
   rc = launch_tiles<0>(wtype, a, max_tiles, st);
+  if (rc) return rc;
+  const int64_t total = T * H;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
+                     (int)H, k, E);
+  return (int)hipGetLastError();
+}
+
+// ---- matrix-core path (gemm-packed weights) -------------------------------------------------------------------
+MLLM_API size_t mllm_hip_q_gemm_packed_bytes(int wtype, int64_t N, int64_t K) {
+  if ((wtype != MLLM_HIP_Q4_0 && wtype != MLLM_HIP_Q8_0) || N <= 0 || K <= 0 || K % QK) return 0;
+  return (size_t)qg_bytes(wtype, N, K);
+}
+
+MLLM_API int mllm_hip_q_gemm_prepack(int wtype, const void* blocks, int weight_scale_mode, void* packed, int64_t N, int64_t K,
+                                     void* stream) {
+  if ((wtype != MLLM_HIP_Q4_0 && wtype != MLLM_HIP_Q8_0) || !blocks || !packed || N <= 0 || K <= 0) return MLLM_HIP_E_BADARG;
+  if (weight_scale_mode != MLLM_HIP_SCALE_IEEE && weight_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
+  if (K % QK || N > INT32_MAX || K > INT32_MAX || qg_bytes(wtype, N, K) >= ((int64_t)1 << 32)) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(packed) % 16) return MLLM_HIP_E_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t words = qg_qbytes(wtype, N, K) / 4, count = qg_np(N) * (qg_kp(K) / 64);
+  const unsigned char* b = reinterpret_cast<const unsigned char*>(blocks);
+  uint32_t* q = reinterpret_cast<uint32_t*>(packed);
+  uint32_t* sc = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(packed) + qg_qbytes(wtype, N, K));
+  const int x86 = weight_scale_mode == MLLM_HIP_SCALE_X86_REF;
+  if (wtype == MLLM_HIP_Q4_0) {
+    hipLaunchKernelGGL(qg_prepack_q_kernel<MLLM_HIP_Q4_0>, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, st, b, q, (int)N, (int)K, words);
+    hipLaunchKernelGGL(qg_prepack_s_kernel<MLLM_HIP_Q4_0>, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st, b, sc, (int)N, (int)K, x86, count);
+  } else {
+    hipLaunchKernelGGL(qg_prepack_q_kernel<MLLM_HIP_Q8_0>, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, st, b, q, (int)N, (int)K, words);
+    hipLaunchKernelGGL(qg_prepack_s_kernel<MLLM_HIP_Q8_0>, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, st, b, sc, (int)N, (int)K, x86, count);
+  }
+  return (int)hipGetLastError();
+}
+
+MLLM_API size_t mllm_hip_linear_q_gemm_workspace_bytes(int64_t M, int64_t K) {
+  if (M <= 0 || K <= 0 || K % QK) return 0;
+  Carver c(nullptr);
+  c.take<uint16_t>((size_t)M * K);
+  carve_route(c, 1, M);
+  return c.used;
+}
+
+MLLM_API int mllm_hip_linear_q_gemm(int wtype, const void* gemm_packed, const void* x, int x_dtype, const float* bias,
+                                    float* y, int64_t M, int64_t N, int64_t K, int act_scale_mode, void* workspace,
+                                    void* stream) {
+  if ((wtype != MLLM_HIP_Q4_0 && wtype != MLLM_HIP_Q8_0) || !gemm_packed || !x || !y || !workspace || M <= 0 || N <= 0 || K <= 0)
+    return MLLM_HIP_E_BADARG;
+  if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
+  if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
+  if (K % QK || M * K * 2 >= ((int64_t)1 << 32) || N > INT32_MAX || qg_bytes(wtype, N, K) >= ((int64_t)1 << 32)) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16 ||
+      reinterpret_cast<uintptr_t>(gemm_packed) % 16 || reinterpret_cast<uintptr_t>(y) % 16)
+    return MLLM_HIP_E_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  Carver c(workspace);
+  uint16_t* xh = c.take<uint16_t>((size_t)M * K);
+  RouteOut ro = carve_route(c, 1, M);
+  const int64_t nblocks = M * (K / QK);
+  hipLaunchKernelGGL(qg_act_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, xh,
+                     (uint16_t*)nullptr, nblocks, act_scale_mode == MLLM_HIP_SCALE_X86_REF);
+  hipLaunchKernelGGL(identity_tiles_kernel, dim3(1), dim3(256), 0, st, (int)M, QG_TILE_H, ro);
+  QG2Args a{};
+  a.W0 = a.W1 = reinterpret_cast<const char*>(gemm_packed);
+  a.wstride = 0;
+  a.xh = xh; a.a_index = nullptr; a.a_div = 1; a.a_rows = (int)M;
+  a.o_index = nullptr; a.out = y; a.bias = bias;
+  a.tile_expert = ro.tile_expert; a.tile_row0 = ro.tile_row0; a.tile_rows = ro.tile_rows; a.ntiles = ro.ntiles;
+  a.N = (int)N; a.K = (int)K; a.wtype = wtype; a.x86_scale = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
+  return launch_qg<0>(a, (unsigned)((M + QG_TILE_H - 1) / QG_TILE_H), st);
+}
+
+MLLM_API size_t mllm_hip_moe_gemm_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k) {
+  if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || k <= 0 || H % QK || I % QK) return 0;
+  Carver c(nullptr);
+  c.take<uint16_t>((size_t)T * H);
+  c.take<uint16_t>((size_t)T * H);
+  c.take<uint16_t>((size_t)T * k * I);
+  c.take<float>((size_t)T * k * H);
+  carve_route(c, E, T * k);
+  return c.used;
+}
+
+MLLM_API int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed,
+                                     const void* x, int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y,
+                                     int64_t T, int64_t H, int64_t I, int E, int k, int act_scale_mode, void* workspace,
+                                     void* stream) {
+  if ((wtype != MLLM_HIP_Q4_0 && wtype != MLLM_HIP_Q8_0) || !gate_packed || !up_packed || !down_packed || !x || !topk_ids ||
+      !topk_w || !y || !workspace || T <= 0 || E <= 0 || E > 4096 || k <= 0)
+    return MLLM_HIP_E_BADARG;
+  if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
+  if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
+  if (H <= 0 || I <= 0 || H % QK || I % QK) return MLLM_HIP_E_SHAPE;
+  if (T * H * 2 >= ((int64_t)1 << 32) || T * k * I * 2 >= ((int64_t)1 << 32) || T * k > INT32_MAX) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  const int x86 = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
+  Carver c(workspace);
+  uint16_t* xh = c.take<uint16_t>((size_t)T * H);
+  uint16_t* xl = c.take<uint16_t>((size_t)T * H);
+  uint16_t* hh = c.take<uint16_t>((size_t)T * k * I);
+  float* per = c.take<float>((size_t)T * k * H);
+  RouteOut ro = carve_route(c, E, T * k);
+  const unsigned max_tiles = (unsigned)(E + (T * k) / QG_TILE_H + 1);
+
+  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 5 * E * sizeof(int), st, topk_ids, (int)(T * k), E, QG_TILE_H, ro);
+  const int64_t nblocks = T * (H / QK);
+  hipLaunchKernelGGL(qg_act_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, xh, xl, nblocks, x86);
+
+  QG2Args a{};
+  a.tile_expert = ro.tile_expert; a.tile_row0 = ro.tile_row0; a.tile_rows = ro.tile_rows; a.ntiles = ro.ntiles;
+  a.wtype = wtype; a.x86_scale = x86;
+  // gate & up -> silu(g)*u -> Q8_0 round trip in fp16, rows in expert-sorted order
+  a.W0 = reinterpret_cast<const char*>(gate_packed);
+  a.W1 = reinterpret_cast<const char*>(up_packed);
+  a.wstride = (size_t)qg_bytes(wtype, I, H);
+  a.xh = xh; a.xl = xl; a.a_index = ro.sorted_idx; a.a_div = k; a.a_rows = (int)T;
+  a.hh = hh;
+  a.N = (int)I; a.K = (int)H;
+  int rc = launch_qg<1>(a, max_tiles, st);
+  if (rc) return rc;
+  // down -> per-(token, slot) rows
+  a.W0 = a.W1 = reinterpret_cast<const char*>(down_packed);
+  a.wstride = (size_t)qg_bytes(wtype, H, I);
+  a.xh = hh; a.xl = nullptr; a.a_index = nullptr; a.a_div = 1; a.a_rows = (int)(T * k);
+  a.o_index = ro.sorted_idx; a.out = per; a.bias = nullptr; a.hh = nullptr;
+  a.N = (int)H; a.K = (int)I;
+  rc = launch_qg<0>(a, max_tiles, st);
   if (rc) return rc;
   const int64_t total = T * H;
   hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,

@@ -290,8 +290,9 @@ __global__ __launch_bounds__(256) void w8a8_prepack_kernel(const int8_t* __restr
 // The weights are the MFMA's first operand, so that a lane ends up with four CONSECUTIVE output columns per row.
 // Scheduling barriers pin the hand-made software pipeline: left alone, the compiler sinks all global loads to the end
 // of the loop body and exposes their latency.
-template <int TM, int TN, bool PK>
-__global__ __launch_bounds__(256) void w8a8_gemm_nsplit_kernel(W8A8Args a) {
+// WPS: waves per SIMD the register budget is held to (workgroups of 4 waves: WPS workgroups per CU).
+template <int TM, int TN, bool PK, int WPS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(WPS, WPS))) void w8a8_gemm_nsplit_kernel(W8A8Args a) {
   constexpr int BK = 128, LDK = 144, KS = BK / 32;
   constexpr int BM = TM * 32, WN = TN * 32, BN = 4 * WN;
   constexpr int CA = BM * (BK / 16) / 256;  // 16-byte activation chunks per thread and K step
@@ -481,24 +482,36 @@ __global__ __launch_bounds__(256) void w8a8_gemm_nsplit_kernel(W8A8Args a) {
   }
 }
 
-template <int TM, int TN, bool PK>
+template <int TM, int TN, bool PK, int WPS>
 static int launch_w8a8_nsplit(const W8A8Args& a, hipStream_t st) {
   constexpr int BM = TM * 32, BN = 4 * TN * 32;
   constexpr size_t stage = 2 * (size_t)BM * 144, patch = 4096 + 32 * (2 * (size_t)BN + 16);
   const size_t lds = stage > patch ? stage : patch;
   const unsigned grid = (unsigned)(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN));
-  hipLaunchKernelGGL((w8a8_gemm_nsplit_kernel<TM, TN, PK>), dim3(grid), dim3(256), lds, st, a);
+  hipLaunchKernelGGL((w8a8_gemm_nsplit_kernel<TM, TN, PK, WPS>), dim3(grid), dim3(256), lds, st, a);
   return (int)hipGetLastError();
 }
+
+static int g_w8a8_ntile = 0;  // weights-from-global kernel: 0 = heuristic, 1 = 128x384, 2 = 64x384, 3 = 128x128, 4 = 64x128, 5 = 128x256
 
 // Tile choice for the weights-from-global kernel: the biggest tile that still gives every CU work.
 template <bool PK>
 static int launch_w8a8_nsplit_auto(const W8A8Args& a, hipStream_t st) {
   auto tiles = [&](int bm, int bn) { return (int64_t)((a.M + bm - 1) / bm) * ((a.N + bn - 1) / bn); };
-  if (a.M > 64 && tiles(128, 384) >= 192) return launch_w8a8_nsplit<4, 3, PK>(a, st);
-  if (tiles(64, 384) >= 192 || a.N <= 128) return launch_w8a8_nsplit<2, 3, PK>(a, st);
-  if (a.M > 64 && tiles(128, 128) >= 192) return launch_w8a8_nsplit<4, 1, PK>(a, st);
-  return launch_w8a8_nsplit<2, 1, PK>(a, st);
+  int t = g_w8a8_ntile;
+  if (!t) {
+    if (a.M > 64 && tiles(128, 384) >= 192) t = 1;
+    else if (tiles(64, 384) >= 192 || a.N <= 128) t = 2;
+    else if (a.M > 64 && tiles(128, 128) >= 192) t = 3;
+    else t = 4;
+  }
+  switch (t) {
+    case 1: return launch_w8a8_nsplit<4, 3, PK, 1>(a, st);
+    case 2: return launch_w8a8_nsplit<2, 3, PK, 2>(a, st);
+    case 3: return launch_w8a8_nsplit<4, 1, PK, 2>(a, st);
+    case 5: return launch_w8a8_nsplit<4, 2, PK, 2>(a, st);
+    default: return launch_w8a8_nsplit<2, 1, PK, 2>(a, st);
+  }
 }
 
 template <int BM, int BN, int WM, int WN, int D>
@@ -522,6 +535,12 @@ using namespace mllmhip;
 MLLM_API int mllm_hip_w8a8_set_tuning(int tile) {
   if (tile < 0 || tile > 4) return MLLM_HIP_E_BADARG;
   g_w8a8_tile = tile;
+  return 0;
+}
+
+MLLM_API int mllm_hip_w8a8_nsplit_set_tuning(int tile) {
+  if (tile < 0 || tile > 5) return MLLM_HIP_E_BADARG;
+  g_w8a8_ntile = tile;
   return 0;
 }
 

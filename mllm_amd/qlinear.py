@@ -28,22 +28,26 @@ def _xdtype(x):
 class PackedQWeight:
     """A Q4_0 / Q8_0 weight [N, K] repacked on the device into the layout the kernels read."""
 
-    def __init__(self, wtype, blocks, weight_scale_mode=SCALE_IEEE):
-        """blocks: uint8 tensor [N, K/32, 18|34] of reference blocks (host or device)."""
+    def __init__(self, wtype, blocks, weight_scale_mode=SCALE_IEEE, layout="gemv"):
+        """blocks: uint8 tensor [N, K/32, 18|34] of reference blocks (host or device).  layout "gemv": the decode kernels'
+        structure-of-arrays form; "gemm": the matrix-core operand order of linear_q_gemm."""
         assert blocks.dtype == torch.uint8 and blocks.dim() == 3 and blocks.shape[2] == BLOCK_BYTES[wtype]
-        self.wtype, self.N, self.K = wtype, blocks.shape[0], blocks.shape[1] * 32
+        assert layout in ("gemv", "gemm")
+        self.wtype, self.N, self.K, self.layout = wtype, blocks.shape[0], blocks.shape[1] * 32, layout
         L = _lib.lib()
-        nbytes = L.mllm_hip_q_packed_bytes(wtype, self.N, self.K)
+        size_fn, pack_fn = ((L.mllm_hip_q_packed_bytes, L.mllm_hip_q_prepack) if layout == "gemv" else
+                            (L.mllm_hip_q_gemm_packed_bytes, L.mllm_hip_q_gemm_prepack))
+        nbytes = size_fn(wtype, self.N, self.K)
         if nbytes == 0:
             raise _lib.HipQLinearError("unsupported weight shape N=%d K=%d" % (self.N, self.K))
         dev_blocks = blocks.contiguous().cuda()
         self.buf = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
-        _lib.check(L.mllm_hip_q_prepack(wtype, dev_blocks.data_ptr(), weight_scale_mode, self.buf.data_ptr(), self.N,
-                                        self.K, _stream()), "mllm_hip_q_prepack")
+        _lib.check(pack_fn(wtype, dev_blocks.data_ptr(), weight_scale_mode, self.buf.data_ptr(), self.N, self.K, _stream()),
+                   "prepack")
         torch.cuda.current_stream().synchronize()  # dev_blocks may be released after this
 
     @classmethod
-    def synthetic(cls, wtype, N, K, generator=None):
+    def synthetic(cls, wtype, N, K, generator=None, layout="gemv"):
         """Random weight drawn on the device (benchmark pools): codes uniform, fp16 block scales |N(0,0.02)|/7 with the low
         three pattern bits cleared so that the IEEE and the x86 reading of the scale agree.  Goes through prepack."""
         nb = K // 32
@@ -53,7 +57,7 @@ class PackedQWeight:
         s = (torch.randn((N, nb), device="cuda", generator=generator) * 0.02).abs() / 7.0
         bits = s.to(torch.float16).view(torch.int16) & ~7
         blocks[:, :, 0:2] = bits.view(torch.uint8).view(N, nb, 2)
-        return cls(wtype, blocks)
+        return cls(wtype, blocks, layout=layout)
 
     @property
     def ptr(self):
@@ -254,24 +258,26 @@ def linear_q(w, x, bias=None, act_scale_mode=SCALE_X86_REF, workspace=None, out=
 
 
 class PackedExperts:
-    """E pre-packed [N, K] weight matrices back to back (the layout mllm_hip_moe_ffn_q takes)."""
+    """E pre-packed [N, K] weight matrices back to back: layout "gemv" for mllm_hip_moe_ffn_q, "gemm" for
+    mllm_hip_moe_ffn_q_gemm."""
 
-    def __init__(self, wtype, blocks, weight_scale_mode=SCALE_IEEE):
+    def __init__(self, wtype, blocks, weight_scale_mode=SCALE_IEEE, layout="gemv"):
         """blocks: uint8 [E, N, K/32, 18|34] (host or device)."""
-        assert blocks.dtype == torch.uint8 and blocks.dim() == 4
-        self.wtype, self.E, self.N, self.K = wtype, blocks.shape[0], blocks.shape[1], blocks.shape[2] * 32
+        assert blocks.dtype == torch.uint8 and blocks.dim() == 4 and layout in ("gemv", "gemm")
+        self.wtype, self.E, self.N, self.K, self.layout = wtype, blocks.shape[0], blocks.shape[1], blocks.shape[2] * 32, layout
         L = _lib.lib()
-        self.stride = L.mllm_hip_q_packed_bytes(wtype, self.N, self.K)
+        size_fn, pack_fn = ((L.mllm_hip_q_packed_bytes, L.mllm_hip_q_prepack) if layout == "gemv" else
+                            (L.mllm_hip_q_gemm_packed_bytes, L.mllm_hip_q_gemm_prepack))
+        self.stride = size_fn(wtype, self.N, self.K)
         self.buf = torch.empty(self.E * self.stride, dtype=torch.uint8, device="cuda")
         for e in range(self.E):
             dev = blocks[e].contiguous().cuda()
-            _lib.check(L.mllm_hip_q_prepack(wtype, dev.data_ptr(), weight_scale_mode,
-                                            self.buf.data_ptr() + e * self.stride, self.N, self.K, _stream()),
-                       "mllm_hip_q_prepack")
+            _lib.check(pack_fn(wtype, dev.data_ptr(), weight_scale_mode, self.buf.data_ptr() + e * self.stride, self.N,
+                               self.K, _stream()), "prepack")
             torch.cuda.current_stream().synchronize()
 
     @classmethod
-    def synthetic(cls, wtype, E, N, K, generator=None):
+    def synthetic(cls, wtype, E, N, K, generator=None, layout="gemv"):
         nb = K // 32
         blocks = torch.randint(0, 256, (E, N, nb, BLOCK_BYTES[wtype]), dtype=torch.uint8, device="cuda", generator=generator)
         if wtype == Q8_0:
@@ -279,7 +285,7 @@ class PackedExperts:
         s = (torch.randn((E, N, nb), device="cuda", generator=generator) * 0.02).abs() / 7.0
         bits = s.to(torch.float16).view(torch.int16) & ~7
         blocks[:, :, :, 0:2] = bits.view(torch.uint8).view(E, N, nb, 2)
-        return cls(wtype, blocks)
+        return cls(wtype, blocks, layout=layout)
 
     @property
     def ptr(self):
@@ -299,6 +305,37 @@ def moe_ffn_q(gate, up, down, x, topk_ids, topk_w, act_scale_mode=SCALE_X86_REF,
     _lib.check(L.mllm_hip_moe_ffn_q(gate.wtype, gate.ptr, up.ptr, down.ptr, x.data_ptr(), _xdtype(x), topk_ids.data_ptr(),
                                     topk_w.data_ptr(), y.data_ptr(), T, H, I, E, k, act_scale_mode, workspace.data_ptr(),
                                     _stream()), "mllm_hip_moe_ffn_q")
+    return y
+
+
+def linear_q_gemm(w, x, bias=None, act_scale_mode=SCALE_X86_REF, workspace=None, out=None):
+    """Q4_0/Q8_0 Linear for many rows on the matrix cores (fp16 operands with the block scales folded in); w in the "gemm"
+    layout."""
+    assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K and w.layout == "gemm"
+    M = x.shape[0]
+    L = _lib.lib()
+    if workspace is None:
+        workspace = torch.empty(L.mllm_hip_linear_q_gemm_workspace_bytes(M, w.K), dtype=torch.uint8, device="cuda")
+    y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")
+    _lib.check(L.mllm_hip_linear_q_gemm(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K,
+                                        act_scale_mode, workspace.data_ptr(), _stream()), "mllm_hip_linear_q_gemm")
+    return y
+
+
+def moe_ffn_q_gemm(gate, up, down, x, topk_ids, topk_w, act_scale_mode=SCALE_X86_REF, workspace=None, out=None):
+    """As moe_ffn_q on the matrix cores; gate/up/down PackedExperts in the "gemm" layout."""
+    T, H = x.shape
+    k = topk_ids.shape[1]
+    E, I = gate.E, gate.N
+    assert gate.K == H and up.N == I and down.N == H and down.K == I and topk_ids.dtype == torch.int32
+    assert gate.layout == up.layout == down.layout == "gemm"
+    L = _lib.lib()
+    if workspace is None:
+        workspace = torch.empty(L.mllm_hip_moe_gemm_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
+    y = out if out is not None else torch.empty((T, H), dtype=torch.float32, device="cuda")
+    _lib.check(L.mllm_hip_moe_ffn_q_gemm(gate.wtype, gate.ptr, up.ptr, down.ptr, x.data_ptr(), _xdtype(x),
+                                         topk_ids.data_ptr(), topk_w.data_ptr(), y.data_ptr(), T, H, I, E, k, act_scale_mode,
+                                         workspace.data_ptr(), _stream()), "mllm_hip_moe_ffn_q_gemm")
     return y
 
 

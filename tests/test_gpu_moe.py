@@ -35,6 +35,53 @@ def test_linear_q_any_m(wtype, M, N, K):
         assert rel_l2(yg, orc.linear_q(x, W, wtype)) < 2e-6
 
 
+GEMM_TOL = 5e-4  # fp16 operands: two roundings of relative error <= 2^-12 each; measured about 2e-4
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M,N,K", [(1, 32, 32), (33, 100, 96), (129, 64, 2048), (300, 768, 2048 + 64), (512, 2048, 768),
+                                    (70, 260, 160)])
+def test_linear_q_gemm_any_m(wtype, M, N, K):
+    rng = synth.rng_for(4, 5 * M + N + K + wtype)
+    W = synth.make_weight(rng, wtype, N, K)
+    w = ql.PackedQWeight(wtype, torch.from_numpy(W), layout="gemm")
+    x = synth.make_x_fp32(rng, M, K)
+    bias = rng.standard_normal(N).astype(np.float32)
+    announce("linear_q_gemm", wtype, M, N, K)
+    for mode, omode in ((ql.SCALE_X86_REF, orc.SCALE_X86_REF), (ql.SCALE_IEEE, orc.SCALE_IEEE)):
+        y = ql.linear_q_gemm(w, to_dev(x), None, mode).cpu().numpy()
+        want = orc.linear_q(x, W, wtype, None, omode)
+        assert rel_l2(y, want) < GEMM_TOL, (mode, rel_l2(y, want))
+    yb = ql.linear_q_gemm(w, to_dev(x), to_dev(bias)).cpu().numpy()
+    assert rel_l2(yb, orc.linear_q(x, W, wtype, bias)) < GEMM_TOL
+    # against the block-dot kernel on the same inputs, and bf16 activations
+    wv = ql.PackedQWeight(wtype, torch.from_numpy(W))
+    assert rel_l2(y, ql.linear_q(wv, to_dev(x), None, ql.SCALE_IEEE).cpu().numpy()) < GEMM_TOL
+    xb = synth.fp32_to_bf16_bits(x)
+    y16 = ql.linear_q_gemm(w, bf16_dev(xb)).cpu().numpy()
+    assert rel_l2(y16, orc.linear_q(synth.bf16_bits_to_fp32(xb), W, wtype)) < GEMM_TOL
+
+
+def test_linear_q_gemm_exact_when_operands_fit_fp16():
+    """Weights and activations chosen so that dW*qW and dX*qX are exactly representable in fp16 and every partial sum in
+    fp32: then the matrix-core path must equal the reference arithmetic bit for bit (a wrong nibble order, scale pairing,
+    row or column mapping cannot hide behind a tolerance)."""
+    rng = synth.rng_for(4, 99)
+    M, N, K = 150, 200, 256
+    for wtype in (0, 1):
+        W = synth.make_weight(rng, wtype, N, K)
+        Wv = W.reshape(N, K // 32, -1)
+        Wv[:, :, 0:2] = np.frombuffer(np.float16(2.0 ** rng.integers(-4, -2, (N, K // 32))).tobytes(), dtype=np.uint8).reshape(N, K // 32, 2)
+        # activations: integers in [-127, 127] with one +-127 per block, so that d = 1 and the codes are the values
+        x = rng.integers(-127, 128, (M, K)).astype(np.float32)
+        x[:, ::32] = 127.0
+        w = ql.PackedQWeight(wtype, torch.from_numpy(W), layout="gemm")
+        announce("linear_q_gemm exact", wtype)
+        y = ql.linear_q_gemm(w, to_dev(x), None, ql.SCALE_IEEE).cpu().numpy()
+        want = orc.linear_q(x, W, wtype, None, orc.SCALE_IEEE)
+        assert np.array_equal(y, want)
+
+
 def test_route_counts_and_order():
     rng = synth.rng_for(4, 1)
     T, E, k = 512, 128, 8
@@ -73,6 +120,40 @@ def test_moe_small(T, H, I, E, k, wtype):
     perm = rng.permutation(T)
     y2 = ql.moe_ffn_q(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
     assert np.array_equal(y2, y[perm])
+
+
+@pytest.mark.parametrize("T,H,I,E,k,wtype", [(16, 64, 32, 4, 2, 0), (40, 256, 96, 8, 3, 0), (200, 128, 64, 3, 2, 1),
+                                              (1, 64, 64, 4, 4, 0), (300, 192, 160, 2, 2, 0)])
+def test_moe_gemm_small(T, H, I, E, k, wtype):
+    rng = synth.rng_for(4, 3 * T + H + I + E)
+    Wg, Wu, Wd = synth.make_moe_weights(rng, E, H, I, wtype)
+    ids, w = synth.make_moe_routing(rng, T, E, k)
+    g, u, d = (ql.PackedExperts(wtype, torch.from_numpy(m), layout="gemm") for m in (Wg, Wu, Wd))
+    x = synth.make_x_fp32(rng, T, H)
+    announce("moe gemm small", T, H, I, E, k, wtype)
+    y = ql.moe_ffn_q_gemm(g, u, d, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+    want = orc.moe_ffn(x, ids, w, Wg, Wu, Wd, wtype)
+    assert rel_l2(y, want) < TOL, rel_l2(y, want)
+    perm = rng.permutation(T)
+    y2 = ql.moe_ffn_q_gemm(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
+    assert np.array_equal(y2, y[perm])
+
+
+def test_moe_gemm_full_size():
+    """The full-size case on the matrix-core path."""
+    rng = synth.rng_for(4)
+    T, H, I, E, k = 512, 2048, 768, 128, 8
+    Wg, Wu, Wd = synth.make_moe_weights(rng, E, H, I, 0)
+    ids, w = synth.make_moe_routing(rng, T, E, k)
+    g, u, d = (ql.PackedExperts(0, torch.from_numpy(m), layout="gemm") for m in (Wg, Wu, Wd))
+    bits, xf = synth.make_x_bf16(rng, T, H)
+    announce("moe gemm full size")
+    y = ql.moe_ffn_q_gemm(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
+    want = orc.moe_ffn(xf, ids, w, Wg, Wu, Wd, 0)
+    r = rel_l2(y, want)
+    assert r < TOL, r
+    y2 = ql.moe_ffn_q_gemm(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
+    assert np.array_equal(y, y2)
 
 
 def test_moe_full_size():
