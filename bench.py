@@ -37,6 +37,9 @@ def parse():
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter run: 20 launches of the dominant GEMV launch and 20 of a plain copy of the same byte count, "
                          "nothing else; meant to run under rocprofv3 --pmc FETCH_SIZE (or WRITE_SIZE)")
+    ap.add_argument("--side-only", action="store_true",
+                    help="profiling run: only the prefill GEMM / MoE side workloads (W8A8, W4A16, MoE FFN, Q4_0 prefill Linear), "
+                         "printed as one JSON object; meant to run under rocprofv3")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the M=4/8 and Q8_0 side measurements")
@@ -128,11 +131,36 @@ def side_workloads(torch, ql, synth, gen):
     wsm = torch.empty(_lib_ws(ql, "moe", T, H, I, E, k), dtype=torch.uint8, device="cuda")
     ym = torch.empty((T, H), dtype=torch.float32, device="cuda")
     tm = ev_time(lambda: ql.moe_ffn_q(gate, up, down, x, ids, tw, workspace=wsm, out=ym), 10)
+    del gate, up, down
+    from mllm_amd import _lib
+    L = _lib.lib()
+    gate2 = ql.PackedExperts.synthetic(ql.Q4_0, E, I, H, gen, layout="gemm")
+    up2 = ql.PackedExperts.synthetic(ql.Q4_0, E, I, H, gen, layout="gemm")
+    down2 = ql.PackedExperts.synthetic(ql.Q4_0, E, H, I, gen, layout="gemm")
+    wsm2 = torch.empty(L.mllm_hip_moe_gemm_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
+    tm2 = ev_time(lambda: ql.moe_ffn_q_gemm(gate2, up2, down2, x, ids, tw, workspace=wsm2, out=ym), 10)
     active = int((np.bincount(ids_np.reshape(-1), minlength=E) > 0).sum())
     wbytes = active * (2 * I * (H // 32) * 18 + H * (I // 32) * 18)
     flops = T * k * (2.0 * H * I * 2 + 2.0 * I * H)
-    out["moe_ffn_512tok_128e_top8_q4_0"] = {"us": tm * 1e6, "active_experts": active, "weight_GBps": wbytes / tm / 1e9,
-                                            "frac_of_hbm_peak": wbytes / tm / 8e12, "TOPS": flops / tm / 1e12}
+    out["moe_ffn_512tok_128e_top8_q4_0"] = {"us": tm2 * 1e6, "active_experts": active, "weight_GBps": wbytes / tm2 / 1e9,
+                                            "frac_of_hbm_peak": wbytes / tm2 / 8e12, "TFLOPS": flops / tm2 / 1e12,
+                                            "path": "matrix cores, fp16 operands with folded block scales (mllm_hip_moe_ffn_q_gemm)",
+                                            "block_dot_path": {"us": tm * 1e6, "weight_GBps": wbytes / tm / 1e9}}
+    del gate2, up2, down2
+    # Q4_0 Linear at prefill size (the reference's tinyBLAS gemm branch): gate_proj of the decode layer, 2048 rows
+    M, N, K = 2048, 9728, 2560
+    xx = torch.randn((M, K), device="cuda", generator=gen).to(torch.bfloat16)
+    yy = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    wv = ql.PackedQWeight.synthetic(ql.Q4_0, N, K, gen)
+    wg = ql.PackedQWeight.synthetic(ql.Q4_0, N, K, gen, layout="gemm")
+    ws1 = torch.empty(L.mllm_hip_linear_q_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+    ws2 = torch.empty(L.mllm_hip_linear_q_gemm_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+    t1 = ev_time(lambda: ql.linear_q(wv, xx, None, ql.SCALE_X86_REF, workspace=ws1, out=yy), 5)
+    t2 = ev_time(lambda: ql.linear_q_gemm(wg, xx, None, ql.SCALE_X86_REF, workspace=ws2, out=yy), 10)
+    fl = 2.0 * M * N * K
+    out["q4_0_linear_prefill_2048x9728x2560"] = {"us": t2 * 1e6, "TFLOPS": fl / t2 / 1e12, "frac_of_2500_TFLOPS": fl / t2 / 2.5e15,
+                                                  "path": "matrix cores (mllm_hip_linear_q_gemm)",
+                                                  "block_dot_path": {"us": t1 * 1e6, "TOPS": fl / t1 / 1e12}}
     return out
 
 
@@ -160,6 +188,9 @@ def main():
     gen.manual_seed(synth.SEED_BASE + 1)
     shapes = synth.QWEN3_4B_LAYER
     stream = torch.cuda.current_stream()
+    if args.side_only:
+        print(json.dumps({"side_only": True, "prefill_and_moe": side_workloads(torch, ql, synth, gen)}))
+        return
 
     def make_pool(wtype, layers):
         return [{name: ql.PackedQWeight.synthetic(wtype, n, k, gen) for name, (n, k) in shapes.items()}
