@@ -56,6 +56,7 @@ std::shared_ptr<HipBackend> initHipBackend() {
   if (const char* m = std::getenv("MLLM_HIP_SCALE_MODE")) {
     if (std::strcmp(m, "x86") == 0) cfg.weight_scale_mode = cfg.act_scale_mode = MLLM_HIP_SCALE_X86_REF;
   }
+  if (const char* m = std::getenv("MLLM_HIP_PREFILL")) cfg.prefill_matrix_cores = std::strcmp(m, "blockdot") != 0;
   auto backend = std::make_shared<HipBackend>(cfg);
   ctx.registerBackend(backend);
   ctx.memoryManager()->registerAllocator(kHIP, backend->allocator());
@@ -125,16 +126,26 @@ void HipLinearOp::load(const ParameterFile::ptr_t& ploader) {
       Tensor dev_blocks = onDevice(weight_);
       packed_ = Tensor::empty({(int32_t)pb}, kByte, kHIP).alloc();
       MLLM_HIP_KERNEL_CHECK(mllm_hip_q_prepack(wt, dev_blocks.ptr<void>(), be.config().weight_scale_mode, packed_.ptr<void>(), N, K, be.stream()));
+      if (be.config().prefill_matrix_cores) {
+        gemm_packed_ = Tensor::empty({(int32_t)mllm_hip_q_gemm_packed_bytes(wt, N, K)}, kByte, kHIP).alloc();
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_q_gemm_prepack(wt, dev_blocks.ptr<void>(), be.config().weight_scale_mode, gemm_packed_.ptr<void>(), N, K,
+                                                      be.stream()));
+      }
       be.synchronize();  // dev_blocks is released when it goes out of scope
       if (options_.bias) bias_dev_ = onDevice(bias_);
       break;
     }
     case kInt8: {
       scheme_ = Scheme::kW8A8;
-      weight_ = onDevice(weight_);
       weight_scale_ = onDevice(ploader->pull(getName() + ".weight.scale"));
       MLLM_RT_ASSERT_EQ(weight_scale_.dtype(), kFloat32);
       MLLM_RT_ASSERT_EQ((int64_t)weight_scale_.numel(), N);
+      {  // the load-time repack into matrix-core operand order (the reference re-lays the weight here too)
+        Tensor dev_w = onDevice(weight_);
+        packed_ = Tensor::empty({(int32_t)mllm_hip_w8a8_packed_bytes(N, K)}, kByte, kHIP).alloc();
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_w8a8_prepack(dev_w.ptr<int8_t>(), N, K, packed_.ptr<void>(), be.stream()));
+        be.synchronize();
+      }
       if (options_.bias) bias_dev_ = onDevice(bias_);
       break;
     }
@@ -142,13 +153,21 @@ void HipLinearOp::load(const ParameterFile::ptr_t& ploader) {
     case kByte: {
       scheme_ = Scheme::kW4A16;  // two uint4 codes per byte, [N][K/2]
       MLLM_RT_ASSERT_EQ((int64_t)weight_.numel(), N * K / 2);
-      weight_ = onDevice(weight_);
       weight_scale_ = onDevice(ploader->pull(getName() + ".weight.scale"));
       weight_zp_ = onDevice(ploader->pull(getName() + ".weight.zero_point"));
       MLLM_RT_ASSERT_EQ(weight_scale_.dtype(), kFloat16);
       const int64_t G = (int64_t)weight_scale_.numel() / N;
       MLLM_RT_ASSERT(G > 0 && K % G == 0);
       group_ = (int)(K / G);
+      {  // codes, scales and zero-points into one packed blob (awq_marlin.py:366-410 does the Marlin repack at this point)
+        Tensor dev_w = onDevice(weight_);
+        const size_t pb = mllm_hip_w4a16_packed_bytes(N, K, group_);
+        if (pb == 0) MLLM_ERROR_EXIT(ExitCode::kCoreError, "Linear %s: group %d must be a multiple of 64 dividing in_channels", getName().c_str(), group_);
+        packed_ = Tensor::empty({(int32_t)pb}, kByte, kHIP).alloc();
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_w4a16_prepack(dev_w.ptr<uint8_t>(), weight_scale_.ptr<uint16_t>(), weight_zp_.ptr<uint8_t>(), N, K, group_,
+                                                     packed_.ptr<void>(), be.stream()));
+        be.synchronize();
+      }
       if (options_.bias) {
         MLLM_RT_ASSERT_EQ(bias_.dtype(), kBFloat16);
         bias_dev_ = onDevice(bias_);
@@ -198,6 +217,10 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
       if (M <= 8) {
         MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), (int)M, N, K,
                                                      be.config().act_scale_mode, st));
+      } else if (!gemm_packed_.isNil()) {
+        void* ws = workspace(mllm_hip_linear_q_gemm_workspace_bytes(M, K));
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemm(wt, gemm_packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K,
+                                                     be.config().act_scale_mode, ws, st));
       } else {
         void* ws = workspace(mllm_hip_linear_q_workspace_bytes(M, K));
         MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K,
@@ -207,14 +230,14 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
     }
     case Scheme::kW8A8: {
       void* ws = workspace(mllm_hip_w8a8_workspace_bytes(M, K));
-      MLLM_HIP_KERNEL_CHECK(mllm_hip_w8a8_linear(x.ptr<void>(), xdt(), weight_.ptr<int8_t>(), weight_scale_.ptr<float>(), bias, y.ptr<void>(), M,
-                                                 N, K, ws, st));
+      MLLM_HIP_KERNEL_CHECK(mllm_hip_w8a8_linear_packed(x.ptr<void>(), xdt(), packed_.ptr<void>(), weight_scale_.ptr<float>(), bias, y.ptr<void>(),
+                                                        M, N, K, ws, st));
       break;
     }
     case Scheme::kW4A16: {
       MLLM_RT_ASSERT_EQ(x.dtype(), kBFloat16);
-      MLLM_HIP_KERNEL_CHECK(mllm_hip_w4a16_gemm(x.ptr<void>(), weight_.ptr<uint8_t>(), weight_scale_.ptr<uint16_t>(), weight_zp_.ptr<uint8_t>(),
-                                                bias_dev_.isNil() ? nullptr : bias_dev_.ptr<void>(), y.ptr<void>(), M, N, K, group_, st));
+      MLLM_HIP_KERNEL_CHECK(mllm_hip_w4a16_gemm_packed(x.ptr<void>(), packed_.ptr<void>(), bias_dev_.isNil() ? nullptr : bias_dev_.ptr<void>(),
+                                                       y.ptr<void>(), M, N, K, group_, st));
       break;
     }
     default: MLLM_ERROR_EXIT(ExitCode::kCoreError, "HipLinearOp::forward before load()");

@@ -31,6 +31,10 @@ struct HipBackendConfig {
   int weight_scale_mode = 0;
   int act_scale_mode = 0;
   int device = 0;
+  // Q4_0 / Q8_0 Linear with more than 8 rows: true = matrix-core path (fp16 operands with folded block scales, a second,
+  // gemm-packed copy of the weight is built at load()); false = the block-dot kernel, which keeps the reference's fp32
+  // block arithmetic.  MLLM_HIP_PREFILL=blockdot selects the latter.
+  bool prefill_matrix_cores = true;
 };
 
 class HipBackend final : public Backend {
@@ -64,7 +68,8 @@ class HipLinearOp final : public aops::LinearOp {
  private:
   enum class Scheme { kNone, kQ4_0, kQ8_0, kW8A8, kW4A16 };
   Scheme scheme_ = Scheme::kNone;
-  Tensor packed_;        // Q4_0 / Q8_0: the repacked device copy the kernels read
+  Tensor packed_;        // the repacked device copy the kernels read (every scheme)
+  Tensor gemm_packed_;   // Q4_0 / Q8_0: the matrix-core layout for more than 8 rows
   Tensor weight_scale_;  // "<name>.weight.scale": fp32 [N] (W8A8) or fp16 [N][K/group] (W4A16)
   Tensor weight_zp_;     // "<name>.weight.zero_point": uint8 [N][ceil(K/group/2)] (W4A16)
   Tensor bias_dev_;      // bias in the form the kernel takes (fp32; bf16 for W4A16)

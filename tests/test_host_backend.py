@@ -76,11 +76,13 @@ def test_linear_through_the_op_factory(via_plugin):
         for M in (1, 5, 20):
             x = synth.make_x_fp32(rng, M, K)
             announce("host linear", scheme, M, "plugin", via_plugin)
+            # up to 8 rows: the decode GEMV (fp32 block arithmetic); more: the matrix-core path (fp16 operands, about 2e-4)
+            tol = 2e-6 if M <= 8 else 5e-4
             y = _run(L, scheme, W, None, None, bias, x, False, M, N, K, 0, via_plugin)
-            assert rel_l2(y, orc.linear_q(x, W, wtype, bias, orc.SCALE_X86_REF)) < 2e-6
+            assert rel_l2(y, orc.linear_q(x, W, wtype, bias, orc.SCALE_X86_REF)) < tol
             bits, xf = synth.make_x_bf16(rng, M, K)
             y = _run(L, scheme, W, None, None, None, bits, True, M, N, K, 0, via_plugin)
-            assert rel_l2(y, orc.linear_q(xf, W, wtype, None, orc.SCALE_X86_REF)) < 2e-6
+            assert rel_l2(y, orc.linear_q(xf, W, wtype, None, orc.SCALE_X86_REF)) < tol
     # W8A8
     M = 40
     a_bits, W8, ws = synth.make_w8a8(rng, M, N, K)
