@@ -198,6 +198,7 @@ def main():
 
     def make_io(M):
         xs = {k: torch.randn((M, k), device="cuda", generator=gen).to(torch.bfloat16) for k in (2560, 4096, 9728)}
+        xs["workspaces"] = {k: (ql.gemv_workspace(M, k) if M >= 3 else None) for k in (2560, 4096, 9728)}
         ys = {name: torch.empty((M, n), dtype=torch.float32, device="cuda") for name, (n, _) in shapes.items()}
         return xs, ys
 
@@ -211,13 +212,15 @@ def main():
                 for name, w in layer.items():
                     ql.linear_q_gemv(w, xs[w.K], None, ql.SCALE_X86_REF, out=ys[name])
             return
+        # from three activation rows on the calls get a workspace: x is then quantized once per call by a small kernel
+        wk = xs["workspaces"]
         for l in pool:
             ql.linear_q_gemv_multi([l["q_proj"], l["k_proj"], l["v_proj"]], xs[2560], None, ql.SCALE_X86_REF,
-                                   [ys["q_proj"], ys["k_proj"], ys["v_proj"]])
-            ql.linear_q_gemv(l["o_proj"], xs[4096], None, ql.SCALE_X86_REF, out=ys["o_proj"])
+                                   [ys["q_proj"], ys["k_proj"], ys["v_proj"]], workspace=wk[2560])
+            ql.linear_q_gemv_multi([l["o_proj"]], xs[4096], None, ql.SCALE_X86_REF, [ys["o_proj"]], workspace=wk[4096])
             ql.linear_q_gemv_multi([l["gate_proj"], l["up_proj"]], xs[2560], None, ql.SCALE_X86_REF,
-                                   [ys["gate_proj"], ys["up_proj"]])
-            ql.linear_q_gemv(l["down_proj"], xs[9728], None, ql.SCALE_X86_REF, out=ys["down_proj"])
+                                   [ys["gate_proj"], ys["up_proj"]], workspace=wk[2560])
+            ql.linear_q_gemv_multi([l["down_proj"]], xs[9728], None, ql.SCALE_X86_REF, [ys["down_proj"]], workspace=wk[9728])
 
     def timed(fn, steps, warmup):
         """warmup, then `steps` calls bracketed by synchronize; returns (wall seconds, HIP-event seconds)"""
@@ -328,8 +331,9 @@ def main():
             offs = [(i * 57000000) % ((1 << 30) - n) // 256 * 256 for i in range(40)]
 
             def fl():
+                st = torch.cuda.current_stream().cuda_stream  # the capture stream while the graph is recorded
                 for o in offs:
-                    _lib.lib().mllm_hip_probe_copy(None, big.data_ptr() + o, n, stream.cuda_stream)
+                    _lib.check(_lib.lib().mllm_hip_probe_copy(None, big.data_ptr() + o, n, st), "probe_copy")
             rp = graphed(fl)
             _, ev = timed(rp, 5, 2)
             floor[str(n)] = {"us": ev / (5 * 40) * 1e6, "GBps": n / (ev / (5 * 40)) / 1e9}

@@ -79,6 +79,13 @@ typedef struct {
 int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M,
                                  int64_t K, int act_scale_mode, void* stream);
 
+/* The same with a workspace (mllm_hip_gemv_workspace_bytes): from three activation rows on, x is quantized once by a small
+ * kernel into the workspace and the GEMV copies that image instead of quantizing x again in every workgroup (two
+ * launches; same results bit for bit).  workspace may be NULL: then it is the call above. */
+size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K);
+int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M,
+                                    int64_t K, int act_scale_mode, void* workspace, void* stream);
+
 /* Same for any M: quantizes the activations with a stand-alone kernel into `workspace`
  * (mllm_hip_linear_q_workspace_bytes) and runs the tiled block-dot kernel.  Used by prefill and by the MoE path. */
 size_t mllm_hip_linear_q_workspace_bytes(int64_t M, int64_t K);

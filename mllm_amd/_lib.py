@@ -39,11 +39,14 @@ def lib():
         i64, vp, ci = C.c_int64, C.c_void_p, C.c_int
         L.mllm_hip_version.restype = C.c_char_p
         L.mllm_hip_init.argtypes = [ci]
+        L.mllm_hip_gemv_workspace_bytes.restype = C.c_size_t
+        L.mllm_hip_gemv_workspace_bytes.argtypes = [ci, i64]
         L.mllm_hip_q_packed_bytes.restype = C.c_size_t
         L.mllm_hip_q_packed_bytes.argtypes = [ci, i64, i64]
         L.mllm_hip_q_prepack.argtypes = [ci, vp, ci, vp, i64, i64, vp]
         L.mllm_hip_linear_q_gemv.argtypes = [ci, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp]
+        L.mllm_hip_linear_q_gemv_multi_ws.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp, vp]
         L.mllm_hip_quantize_q8_0.argtypes = [vp, ci, vp, vp, i64, i64, vp]
         L.mllm_hip_q_dequantize.argtypes = [ci, vp, vp, i64, i64, vp]
         L.mllm_hip_q_block_isums.argtypes = [ci, vp, vp, vp, i64, i64, i64, vp]

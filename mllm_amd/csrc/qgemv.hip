@@ -109,21 +109,18 @@ __global__ void block_isums_kernel(int wtype, PackedView w, const int8_t* __rest
 }
 
 // plain copy / read kernels of known size: the yardstick for HBM counters and for the per-launch floor of a stream
+// (buffer loads / stores: an out-of-range lane needs no branch, so all eight loads of a thread are in flight together;
+// with `if (i < n)` around each load the compiler waits for every load before the next block)
 __global__ __launch_bounds__(256) void probe_copy_kernel(u32x4* __restrict__ dst, const u32x4* __restrict__ src, size_t n16) {
-  const size_t base = (size_t)blockIdx.x * 256 * 8 + threadIdx.x;
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(src), 0, (uint32_t)(n16 * 16), 0x00020000);
+  const uint32_t base = (uint32_t)(((size_t)blockIdx.x * 256 * 8 + threadIdx.x) * 16);
   u32x4 v[8];
 #pragma unroll
-  for (int u = 0; u < 8; u++) {
-    const size_t i = base + (size_t)u * 256;
-    v[u] = u32x4{0, 0, 0, 0};
-    if (i < n16) v[u] = __builtin_nontemporal_load(&src[i]);
-  }
+  for (int u = 0; u < 8; u++) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, base + (uint32_t)u * 4096u, 0, 2);
   if (dst) {
+    const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(dst, 0, (uint32_t)(n16 * 16), 0x00020000);
 #pragma unroll
-    for (int u = 0; u < 8; u++) {
-      const size_t i = base + (size_t)u * 256;
-      if (i < n16) dst[i] = v[u];
-    }
+    for (int u = 0; u < 8; u++) __builtin_amdgcn_raw_buffer_store_b128(v[u], rd, base + (uint32_t)u * 4096u, 0, 0);
   } else {  // read only: keep the loads alive without writing
     uint32_t a = 0;
 #pragma unroll
@@ -132,7 +129,33 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(u32x4* __restrict__ dst
   }
 }
 
-// ---- launch-shape selection ------------------------------------------------------------------------------
+// The quantized image of x the GEMV kernel copies into LDS when it does not quantize itself: for MT rows (rows m >= M
+// zero) of nb blocks: 16-byte planes of elements 0..15 and 16..31, fp32 effective scales, -8 * sum(codes).
+__global__ void quant_image_kernel(const void* __restrict__ x, int x_dtype, unsigned char* __restrict__ img, int M, int MT, int nb,
+                                   int x86_scale) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;  // block index m * nb + b
+  const int mnb = MT * nb;
+  if (i >= mnb) return;
+  uint32_t q[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  float d = 0.f;
+  int sum = 0;
+  if (i < M * nb) {
+    float v[32];
+    load_block_f32(x, x_dtype, (int64_t)i * QK, v);
+    uint16_t bits = quantize_block_q8_0(v, q, sum);
+    if (x86_scale) bits = x86_scale_bits(bits);
+    d = f16bits_to_f32(bits);
+  }
+  u32x4* lo = reinterpret_cast<u32x4*>(img);
+  u32x4* hi = lo + mnb;
+  float* sd = reinterpret_cast<float*>(hi + mnb);
+  int* sn = reinterpret_cast<int*>(sd + mnb);
+  lo[i] = u32x4{q[0], q[1], q[2], q[3]};
+  hi[i] = u32x4{q[4], q[5], q[6], q[7]};
+  sd[i] = d;
+  sn[i] = -8 * sum;
+}
+
 static int g_tune_G = 0, g_tune_R = 0, g_tune_NW = 0;
 
 static GemvShape pick_shape(int MT, int64_t N, int nb) {
@@ -140,7 +163,7 @@ static GemvShape pick_shape(int MT, int64_t N, int nb) {
   // bytes per row segment) suit rows of 64..255 blocks; very long rows want the whole wave on one row and, because
   // every workgroup quantizes all of x, many waves per workgroup to share that work.
   GemvShape s;
-  s.R = MT >= 8 ? 4 : 2;
+  s.R = 2;
   s.NW = 4;
   if (nb >= 256) {
     s.G = 64;
@@ -153,7 +176,9 @@ static GemvShape pick_shape(int MT, int64_t N, int nb) {
   } else {
     s.G = 8;
   }
-  if (MT >= 4 && nb * MT >= 1024 && s.NW < 8) s.NW = 8;
+  // several activation rows: the quantization of x (done by every workgroup) grows with M, so spread it over many waves;
+  // measured best over the projection shapes: 16 waves for rows up to 255 blocks, 8 for longer rows
+  if (MT >= 4) s.NW = nb >= 256 ? 8 : (nb * MT >= 256 ? 16 : 8);
   (void)N;
   if (g_tune_G) s.G = g_tune_G;
   if (g_tune_R) s.R = g_tune_R;
@@ -184,6 +209,7 @@ MLLM_API int mllm_hip_init(int device) {
 
 MLLM_API int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream) {
   if (!src || bytes == 0 || bytes % 16) return MLLM_HIP_E_BADARG;
+  if (bytes >= ((size_t)1 << 32)) return MLLM_HIP_E_SHAPE;
   if (reinterpret_cast<uintptr_t>(src) % 16 || reinterpret_cast<uintptr_t>(dst) % 16) return MLLM_HIP_E_ALIGN;
   const size_t n16 = bytes / 16;
   hipLaunchKernelGGL(probe_copy_kernel, dim3((unsigned)((n16 + 2047) / 2048)), dim3(256), 0, (hipStream_t)stream, (u32x4*)dst,
@@ -235,13 +261,18 @@ MLLM_API int mllm_hip_q_prepack(int wtype, const void* blocks, int weight_scale_
   return (int)hipGetLastError();
 }
 
-MLLM_API int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,
-                                          int M, int64_t K, int act_scale_mode, void* stream) {
+MLLM_API size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K) {
+  if (M < 1 || M > 8 || K <= 0 || K % QK) return 0;
+  return (size_t)8 * (K / QK) * 40;
+}
+
+MLLM_API int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,
+                                             int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
   if (nparts < 1 || nparts > GEMV_MAX_PARTS || !parts) return MLLM_HIP_E_BADARG;
   if (!x || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16)) return MLLM_HIP_E_BADARG;
   if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
   if (M < 1 || M > 8) return MLLM_HIP_E_SHAPE;
-  if (reinterpret_cast<uintptr_t>(x) % 16) return MLLM_HIP_E_ALIGN;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
   GemvArgs a{};
   int64_t nmax = 0;
   for (int p = 0; p < nparts; p++) {
@@ -261,11 +292,25 @@ MLLM_API int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_
   a.nbp = (int)scale_row_stride(K);
   a.x86_scale = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8));
-  const GemvShape s = pick_shape(MT, nmax, a.nb);
+  GemvShape s = pick_shape(MT, nmax, a.nb);
   hipStream_t st = (hipStream_t)stream;
+  if (workspace && M >= 3) {
+    // several rows: quantize once for all workgroups, then the GEMV copies the quantized image instead of quantizing
+    const int mnb = MT * a.nb;
+    hipLaunchKernelGGL(quant_image_kernel, dim3((unsigned)((mnb + 127) / 128)), dim3(128), 0, st, x, x_dtype,
+                       reinterpret_cast<unsigned char*>(workspace), M, MT, a.nb, a.x86_scale);
+    a.x = workspace;
+    if (!g_tune_NW) s.NW = a.nb >= 256 ? 8 : 4;  // no quantization work to share: smaller workgroups start and finish sooner
+    return wtype == MLLM_HIP_Q4_0 ? launch_gemv_q4_preq(a, MT, s, st) : launch_gemv_q8_preq(a, MT, s, st);
+  }
   if (wtype == MLLM_HIP_Q4_0)
     return x_dtype == MLLM_HIP_F32 ? launch_gemv_q4_f32(a, MT, s, st) : launch_gemv_q4_bf16(a, MT, s, st);
   return x_dtype == MLLM_HIP_F32 ? launch_gemv_q8_f32(a, MT, s, st) : launch_gemv_q8_bf16(a, MT, s, st);
+}
+
+MLLM_API int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,
+                                          int M, int64_t K, int act_scale_mode, void* stream) {
+  return mllm_hip_linear_q_gemv_multi_ws(wtype, nparts, parts, x, x_dtype, M, K, act_scale_mode, nullptr, stream);
 }
 
 MLLM_API int mllm_hip_linear_q_gemv(int wtype, const void* packed, const void* x, int x_dtype, const float* bias,

@@ -111,6 +111,12 @@ __device__ __forceinline__ void load_chunk(WChunk<WT, R, U, SCL>& c, const WRsrc
   }
 }
 
+// XT == GEMV_PREQ: `x` is not the activations but their quantized image, laid out exactly like the kernel's LDS area
+// (code planes, scales, -8*sums; rows m >= M zero), written once by quant_image_kernel; the kernel copies it instead of
+// quantizing.  With several activation rows the quantization, which every workgroup would repeat, costs more than the
+// weights take to arrive.
+constexpr int GEMV_PREQ = 2;
+
 // Eight consecutive activation elements of one lane, raw (bf16: 16 bytes, fp32: 32 bytes) and converted.
 template <int XT>
 struct XRaw {
@@ -185,9 +191,15 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
   // item `it` = eight elements: block it/4, lanes of a quad share a block.  Addresses are clamped, validity is applied
   // when the values are used, so no branch separates these loads from the ones below.
   const int valid_items = a.M * nb * 4;
+  const int img_chunks = mnb * 5 / 2;  // 16-byte pieces of the quantized image (40 bytes per block)
   XRaw<XT> raw0, raw1;
-  load_x8<XT>(a.x, (int64_t)min(tid, valid_items - 1) * 8, raw0);
-  load_x8<XT>(a.x, (int64_t)min(tid + nthreads, valid_items - 1) * 8, raw1);
+  if (XT == GEMV_PREQ) {
+    raw0.r[0] = reinterpret_cast<const u32x4*>(a.x)[min(tid, img_chunks - 1)];
+    raw1.r[0] = reinterpret_cast<const u32x4*>(a.x)[min(tid + nthreads, img_chunks - 1)];
+  } else {
+    load_x8<XT>(a.x, (int64_t)min(tid, valid_items - 1) * 8, raw0);
+    load_x8<XT>(a.x, (int64_t)min(tid + nthreads, valid_items - 1) * 8, raw1);
+  }
 
   // ---- 2. block scales of this wave's rows: chunks of 8 scales (16 bytes), lane L takes chunks L and L+64 ------
   const WRsrc wr = make_wrsrc(pt.w, WT, N, nb, nbp);
@@ -261,12 +273,19 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
       }
     }
   };
-  quantize_item(tid, raw0);
-  quantize_item(tid + nthreads, raw1);
-  for (int it = tid + 2 * nthreads; it < mnb * 4; it += nthreads) {
-    XRaw<XT> rw;
-    load_x8<XT>(a.x, (int64_t)min(it, valid_items - 1) * 8, rw);
-    quantize_item(it, rw);
+  if (XT == GEMV_PREQ) {
+    u32x4* s16 = reinterpret_cast<u32x4*>(smem);
+    if (tid < img_chunks) s16[tid] = raw0.r[0];
+    if (tid + nthreads < img_chunks) s16[tid + nthreads] = raw1.r[0];
+    for (int c = tid + 2 * nthreads; c < img_chunks; c += nthreads) s16[c] = reinterpret_cast<const u32x4*>(a.x)[c];
+  } else {
+    quantize_item(tid, raw0);
+    quantize_item(tid + nthreads, raw1);
+    for (int it = tid + 2 * nthreads; it < mnb * 4; it += nthreads) {
+      XRaw<XT> rw;
+      load_x8<XT>(a.x, (int64_t)min(it, valid_items - 1) * 8, rw);
+      quantize_item(it, rw);
+    }
   }
   if (SCL) {
 #pragma unroll
@@ -369,16 +388,22 @@ static int launch_gemv_m(const GemvArgs& a, GemvShape s, hipStream_t st) {
 // one instance per (weight type, activation type), each in its own translation unit (compiled in parallel)
 template <int WT, int XT>
 int launch_gemv(const GemvArgs& a, int MT, GemvShape s, hipStream_t st) {
-  switch (MT) {
-    case 1: return launch_gemv_m<WT, XT, 1>(a, s, st);
-    case 2: return launch_gemv_m<WT, XT, 2>(a, s, st);
-    case 4: return launch_gemv_m<WT, XT, 4>(a, s, st);
-    default: return launch_gemv_m<WT, XT, 8>(a, s, st);
+  if constexpr (XT == GEMV_PREQ) {  // only used from three activation rows on
+    return MT == 4 ? launch_gemv_m<WT, XT, 4>(a, s, st) : launch_gemv_m<WT, XT, 8>(a, s, st);
+  } else {
+    switch (MT) {
+      case 1: return launch_gemv_m<WT, XT, 1>(a, s, st);
+      case 2: return launch_gemv_m<WT, XT, 2>(a, s, st);
+      case 4: return launch_gemv_m<WT, XT, 4>(a, s, st);
+      default: return launch_gemv_m<WT, XT, 8>(a, s, st);
+    }
   }
 }
 int launch_gemv_q4_f32(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
 int launch_gemv_q4_bf16(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
 int launch_gemv_q8_f32(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
 int launch_gemv_q8_bf16(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
+int launch_gemv_q4_preq(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
+int launch_gemv_q8_preq(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
 
 }  // namespace mllmhip

@@ -88,8 +88,14 @@ def linear_q_gemv(w, x, bias=None, act_scale_mode=SCALE_X86_REF, out=None):
     return y
 
 
-def linear_q_gemv_multi(ws, x, biases=None, act_scale_mode=SCALE_X86_REF, outs=None):
-    """Sibling projections (same x, same K) in one launch.  ws: list of PackedQWeight; returns the list of outputs."""
+def gemv_workspace(M, K):
+    """Workspace for linear_q_gemv_multi with three or more activation rows."""
+    return torch.empty(_lib.lib().mllm_hip_gemv_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+
+
+def linear_q_gemv_multi(ws, x, biases=None, act_scale_mode=SCALE_X86_REF, outs=None, workspace=None):
+    """Sibling projections (same x, same K) in one launch.  ws: list of PackedQWeight; returns the list of outputs.
+    With a workspace (gemv_workspace) and M >= 3, x is quantized once by a small kernel instead of in every workgroup."""
     assert 1 <= len(ws) <= 4 and x.is_cuda and x.is_contiguous() and x.dim() == 2
     M, K = x.shape
     if outs is None:
@@ -99,8 +105,9 @@ def linear_q_gemv_multi(ws, x, biases=None, act_scale_mode=SCALE_X86_REF, outs=N
         assert w.K == K and w.wtype == ws[0].wtype
         b = biases[i] if biases is not None else None
         parts[i] = _lib.GemvPart(w.ptr, b.data_ptr() if b is not None else None, outs[i].data_ptr(), w.N)
-    _lib.check(_lib.lib().mllm_hip_linear_q_gemv_multi(ws[0].wtype, len(ws), parts, x.data_ptr(), _xdtype(x), M, K,
-                                                       act_scale_mode, _stream()), "mllm_hip_linear_q_gemv_multi")
+    _lib.check(_lib.lib().mllm_hip_linear_q_gemv_multi_ws(ws[0].wtype, len(ws), parts, x.data_ptr(), _xdtype(x), M, K,
+                                                          act_scale_mode, _p(workspace), _stream()),
+               "mllm_hip_linear_q_gemv_multi_ws")
     return outs
 
 

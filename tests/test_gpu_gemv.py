@@ -219,3 +219,30 @@ def test_gemv_multi_equals_single(wtype, M):
     L = _lib.lib()
     assert L.mllm_hip_linear_q_gemv_multi(0, 5, None, None, 0, 1, 64, 0, None) == -1
     assert L.mllm_hip_linear_q_gemv_multi(0, 0, None, None, 0, 1, 64, 0, None) == -1
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M", [3, 4, 5, 8])
+def test_gemv_prequantized_equals_fused(wtype, M):
+    """With a workspace (three rows or more) x is quantized once by a small kernel and the GEMV copies that image: the
+    results must be the bits of the fused kernel, for fp32 and bf16 activations, both scale modes, long and ragged rows."""
+    rng = synth.rng_for(1, 90 + M + wtype)
+    for shapes in ([(9728, 2560), (9728, 2560)], [(2560, 9728)], [(40, 96), (7, 96), (33, 96)], [(65, 32)]):
+        K = shapes[0][1]
+        Ws = [synth.make_weight(rng, wtype, n, K) for n, _ in shapes]
+        ws = [ql.PackedQWeight(wtype, torch.from_numpy(W)) for W in Ws]
+        biases = [to_dev(rng.standard_normal(n).astype(np.float32)) for n, _ in shapes]
+        x = synth.make_x_fp32(rng, M, K)
+        wsp = ql.gemv_workspace(M, K)
+        announce("gemv prequantized", wtype, M, shapes)
+        for xd in (to_dev(x), bf16_dev(synth.fp32_to_bf16_bits(x))):
+            for mode in (ql.SCALE_X86_REF, ql.SCALE_IEEE):
+                fused = ql.linear_q_gemv_multi(ws, xd, biases, mode)
+                pre = ql.linear_q_gemv_multi(ws, xd, biases, mode, workspace=wsp)
+                for f, p in zip(fused, pre):
+                    assert torch.equal(f, p)
+        want = orc.linear_q(x, Ws[0], wtype, biases[0].cpu().numpy(), orc.SCALE_X86_REF)
+        got = ql.linear_q_gemv_multi(ws, to_dev(x), biases, ql.SCALE_X86_REF, workspace=wsp)[0].cpu().numpy()
+        assert rel_l2(got, want) < 2e-6
+    assert _lib.lib().mllm_hip_gemv_workspace_bytes(8, 2560) == 8 * 80 * 40
+    assert _lib.lib().mllm_hip_gemv_workspace_bytes(9, 2560) == 0
