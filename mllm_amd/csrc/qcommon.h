@@ -17,6 +17,7 @@
 namespace mllmhip {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));  // one 16-byte load
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // ---- bit casts / small conversions ---------------------------------------------------------------------
 __device__ __forceinline__ float bf16_to_f32(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }

@@ -265,7 +265,6 @@ struct W4A16PArgs {
   int M, N, K, group;
 };
 
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 // One output tile (32 TM rows from m0) x (128 TN columns from n0) by the four waves of a workgroup.
 template <int TM, int TN, int BK>
