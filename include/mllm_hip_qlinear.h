@@ -97,6 +97,14 @@ int mllm_hip_linear_q(int wtype, const void* packed, const void* x, int x_dtype,
 int mllm_hip_quantize_q8_0(const void* x, int x_dtype, int8_t* codes, uint16_t* d_bits, int64_t M, int64_t K,
                            void* stream);
 
+/* The step in front of the path: the offline weight quantizer (tools/mllm-quantizer -> quantize_row_q4_0 /
+ * quantize_row_q8_0, ggml/quantize/quantize_q4.cpp:33-68, quantize_q8.cpp:106-190).  w: fp32 [N][K] -> `blocks`: the
+ * reference's array of 18 / 34-byte structs, row-major [N][K/32] (2-byte aligned), ready for the prepack calls.
+ * weight_scale_mode says how the 2-byte scale field is STORED: IEEE = the fp16 pattern of the scale; X86_REF = what the
+ * x86 build of the reference writes (the pattern as a half-precision number; pass the same mode to prepack to read it). */
+int mllm_hip_quantize_weight_blocks(int wtype, const float* w, void* blocks, int weight_scale_mode, int64_t N, int64_t K,
+                                    void* stream);
+
 /* Parity probes (used by the tests, cheap enough to ship):
  *   dequantize: w[n][k] = code * fp32(scale)       dequantize_row_q4_0 / _q8_0 (quantize_q4.cpp:74-93, quantize_q8.cpp:197-211)
  *   block_isums: exact int32 dot product of every weight block with every activation block, [N][M][K/32] */

@@ -44,6 +44,7 @@ def lib():
         L.mllm_hip_q_packed_bytes.restype = C.c_size_t
         L.mllm_hip_q_packed_bytes.argtypes = [ci, i64, i64]
         L.mllm_hip_q_prepack.argtypes = [ci, vp, ci, vp, i64, i64, vp]
+        L.mllm_hip_quantize_weight_blocks.argtypes = [ci, vp, vp, ci, i64, i64, vp]
         L.mllm_hip_linear_q_gemv.argtypes = [ci, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi_ws.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp, vp]

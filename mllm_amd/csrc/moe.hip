@@ -480,7 +480,10 @@ __global__ __launch_bounds__(256) void qg_prepack_s_kernel(const unsigned char* 
     if (n < N && b < nblk) {
       const unsigned char* p = blocks + ((int64_t)n * nblk + b) * BS;
       uint16_t bits = (uint16_t)(p[0] | (p[1] << 8));
-      if (x86_scale) bits = x86_scale_bits(bits);
+      if (x86_scale) {  // as mllm_hip_q_prepack: the field holds the pattern as a half-precision NUMBER
+        const float num = f16bits_to_f32(bits);
+        bits = (num >= 0.f && num < 65536.f) ? (uint16_t)(uint32_t)num : (uint16_t)0;
+      }
       v |= (uint32_t)bits << (16 * h);
     }
   }

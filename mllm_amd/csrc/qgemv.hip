@@ -129,6 +129,64 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(u32x4* __restrict__ dst
   }
 }
 
+// =========================================================================================================
+// offline weight quantizers: fp32 rows -> reference blocks (one thread per block)
+//   Q4_0  quantize_row_q4_0_reference, ggml/quantize/quantize_q4.cpp:33-68
+//   Q8_0  quantize_row_q8_0, ggml/quantize/quantize_q8.cpp:106-190
+// x86_store: write the scale field as the x86 build of the reference leaves it in a file, the half-precision encoding
+// of the NUMBER equal to the fp16 pattern (mllm/core/DataTypes.hpp:26 with quantize.hpp:108-134).
+// =========================================================================================================
+__global__ void quantize_weight_blocks_kernel(int wtype, const float* __restrict__ w, uint16_t* __restrict__ blocks,
+                                              int64_t nblocks, int x86_store) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= nblocks) return;
+  float v[32];
+  load_block_f32(w, MLLM_HIP_F32, i * QK, v);
+  if (wtype == MLLM_HIP_Q4_0) {
+    float amax = 0.f, mx = 0.f;
+#pragma unroll
+    for (int j = 0; j < 32; j++)
+      if (amax < fabsf(v[j])) {
+        amax = fabsf(v[j]);
+        mx = v[j];
+      }
+    float d = mx / -8.f;
+    asm("" : "+v"(d));  // keep the product and the fp16 conversion apart: fused (v_fma_mixlo_f16 with a +0 addend) an
+                          // all-zero block would store +0 where the reference stores -0
+    const float id = d != 0.f ? 1.0f / d : 0.0f;
+    uint16_t field = f32_to_f16bits(d);
+    if (x86_store) field = f32_to_f16bits((float)field);
+    uint16_t* y = blocks + i * 9;  // 18 bytes
+    y[0] = field;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      uint32_t pair = 0;
+#pragma unroll
+      for (int b = 0; b < 2; b++) {
+        const int e = 2 * j + b;
+        int q0 = (int)(int8_t)(int)(v[e] * id + 8.5f);       // truncation toward zero, as the C cast
+        int q1 = (int)(int8_t)(int)(v[16 + e] * id + 8.5f);
+        q0 = min(15, q0);
+        q1 = min(15, q1);
+        pair |= (((uint32_t)q0 & 0xffu) | (((uint32_t)q1 << 4) & 0xf0u)) << (8 * b);
+      }
+      y[1 + j] = (uint16_t)pair;
+    }
+  } else {
+    uint32_t q[8];
+    int sum;
+    uint16_t field = quantize_block_q8_0(v, q, sum);
+    if (x86_store) field = f32_to_f16bits((float)field);
+    uint16_t* y = blocks + i * 17;  // 34 bytes
+    y[0] = field;
+#pragma unroll
+    for (int j = 0; j < 8; j++) {
+      y[1 + 2 * j] = (uint16_t)(q[j] & 0xffffu);
+      y[2 + 2 * j] = (uint16_t)(q[j] >> 16);
+    }
+  }
+}
+
 // The quantized image of x the GEMV kernel copies into LDS when it does not quantize itself: for MT rows (rows m >= M
 // zero) of nb blocks: 16-byte planes of elements 0..15 and 16..31, fp32 effective scales, -8 * sum(codes).
 __global__ void quant_image_kernel(const void* __restrict__ x, int x_dtype, unsigned char* __restrict__ img, int M, int MT, int nb,
@@ -329,6 +387,18 @@ MLLM_API int mllm_hip_quantize_q8_0(const void* x, int x_dtype, int8_t* codes, u
   const int64_t nblocks = M * (K / QK);
   hipLaunchKernelGGL(quantize_q8_0_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, (hipStream_t)stream, x,
                      x_dtype, codes, d_bits, nblocks);
+  return (int)hipGetLastError();
+}
+
+MLLM_API int mllm_hip_quantize_weight_blocks(int wtype, const float* w, void* blocks, int weight_scale_mode, int64_t N,
+                                             int64_t K, void* stream) {
+  if ((wtype != MLLM_HIP_Q4_0 && wtype != MLLM_HIP_Q8_0) || !w || !blocks || N <= 0 || K <= 0) return MLLM_HIP_E_BADARG;
+  if (weight_scale_mode != MLLM_HIP_SCALE_IEEE && weight_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
+  if (K % QK) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(w) % 16 || reinterpret_cast<uintptr_t>(blocks) % 2) return MLLM_HIP_E_ALIGN;
+  const int64_t nblocks = N * (K / QK);
+  hipLaunchKernelGGL(quantize_weight_blocks_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, (hipStream_t)stream,
+                     wtype, w, reinterpret_cast<uint16_t*>(blocks), nblocks, weight_scale_mode == MLLM_HIP_SCALE_X86_REF);
   return (int)hipGetLastError();
 }
 

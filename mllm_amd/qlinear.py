@@ -111,6 +111,16 @@ def linear_q_gemv_multi(ws, x, biases=None, act_scale_mode=SCALE_X86_REF, outs=N
     return outs
 
 
+def quantize_weight_blocks(w, wtype, weight_scale_mode=SCALE_IEEE):
+    """fp32 [N, K] on the GPU -> reference blocks uint8 [N, K/32, 18|34] (the offline quantizer's output)."""
+    assert w.is_cuda and w.is_contiguous() and w.dtype == torch.float32 and w.dim() == 2 and w.shape[1] % 32 == 0
+    N, K = w.shape
+    out = torch.empty((N, K // 32, BLOCK_BYTES[wtype]), dtype=torch.uint8, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_quantize_weight_blocks(wtype, w.data_ptr(), out.data_ptr(), weight_scale_mode, N, K,
+                                                          _stream()), "mllm_hip_quantize_weight_blocks")
+    return out
+
+
 def quantize_q8_0(x):
     """x [M, K] -> (codes int8 [M, K], scale patterns int16-viewed-as-uint16 [M, K/32])."""
     assert x.is_cuda and x.is_contiguous() and x.dim() == 2

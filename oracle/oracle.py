@@ -220,6 +220,17 @@ def moe_ffn(x, topk_ids, topk_w, Wg, Wu, Wd, wtype, scale_mode=SCALE_X86_REF):
     return y
 
 
+def quantize_weight_rows(w, wtype, scale_mode=SCALE_IEEE):
+    """fp32 [N, K] -> reference blocks uint8 [N, K/32, 18|34] (offline weight quantizer restatement)."""
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    N, K = w.shape
+    out = np.empty((N, K // 32, 18 if wtype == Q4_0 else 34), np.uint8)
+    fn = lib().orc_quantize_row_q4_0 if wtype == Q4_0 else lib().orc_quantize_row_q8_0_blocks
+    for n in range(N):
+        fn(_p(w[n], C.c_float), _p(out[n], C.c_uint8), C.c_int(K), C.c_int(scale_mode))
+    return out
+
+
 # ----------------------------------------------------------------------------- compiled reference (oracle/_ref)
 def ref_quantize_rows_q8_0(x):
     """reference quantize_row_q8_0 -> (codes int8 [M, K], EFFECTIVE scale values fp32 [M, K/32])."""

@@ -132,6 +132,59 @@ ORC_API void orc_quantize_row_q8_0(const float* x, int8_t* qs, uint16_t* d_bits,
   }
 }
 
+/* ------------------------------------------------------------------------------------------------
+ * Offline weight quantizers: fp32 rows -> reference blocks (array of 18 / 34-byte structs).
+ *   Q4_0   quantize_row_q4_0_reference, mllm/backends/cpu/kernels/common/ggml/quantize/quantize_q4.cpp:33-68
+ *          max = the element of largest magnitude, WITH its sign ; d = max / -8 ; id = d ? 1/d : 0 ;
+ *          code = min(15, (int8)(x*id + 8.5)) (truncation) ; element j in the low nibble of byte j, 16+j in the high one
+ *   Q8_0   quantize_row_q8_0 (the same routine the activations go through), quantize_q8.cpp:106-190
+ * The 2-byte scale field: scale_mode IEEE stores the fp16 pattern P of d; X86_REF stores what the x86 build of the
+ * reference leaves in the file, the half-precision ENCODING OF THE NUMBER P (DataTypes.hpp:26 with quantize.hpp:108-134),
+ * which a later x86 read turns into P rounded to 11 significant bits.  For a negative d (positive maximum) P >= 0x8000
+ * and that rounding drops up to five low bits of the scale pattern.
+ * Pinned: codes and decoded scale pattern bit-exact against the compiled reference (tests/test_oracle_vs_reference.py).
+ * ---------------------------------------------------------------------------------------------- */
+static uint16_t store_scale_field(uint16_t pattern, int scale_mode) {
+  return scale_mode == ORC_SCALE_X86_REF ? orc_fp32_to_fp16((float)pattern) : pattern;
+}
+ORC_API void orc_quantize_row_q4_0(const float* x, uint8_t* blocks, int k, int scale_mode) {
+  int nb = k / QK;
+  for (int i = 0; i < nb; i++) {
+    const float* xb = x + (size_t)i * QK;
+    uint8_t* y = blocks + (size_t)i * 18;
+    float amax = 0.0f, max = 0.0f;
+    for (int j = 0; j < QK; j++) {
+      const float v = xb[j];
+      if (amax < fabsf(v)) {
+        amax = fabsf(v);
+        max = v;
+      }
+    }
+    const float d = max / -8;
+    const float id = d ? 1.0f / d : 0.0f;
+    const uint16_t field = store_scale_field(orc_fp32_to_fp16(d), scale_mode);
+    memcpy(y, &field, 2);
+    for (int j = 0; j < QK / 2; j++) {
+      const float x0 = xb[j] * id, x1 = xb[QK / 2 + j] * id;
+      int q0 = (int8_t)(x0 + 8.5f), q1 = (int8_t)(x1 + 8.5f);
+      q0 = q0 < 15 ? q0 : 15;
+      q1 = q1 < 15 ? q1 : 15;
+      y[2 + j] = (uint8_t)((uint8_t)q0 | ((uint8_t)q1 << 4));
+    }
+  }
+}
+ORC_API void orc_quantize_row_q8_0_blocks(const float* x, uint8_t* blocks, int k, int scale_mode) {
+  int nb = k / QK;
+  for (int i = 0; i < nb; i++) {
+    int8_t qs[QK];
+    uint16_t bits;
+    orc_quantize_row_q8_0(x + (size_t)i * QK, qs, &bits, QK);
+    const uint16_t field = store_scale_field(bits, scale_mode);
+    memcpy(blocks + (size_t)i * 34, &field, 2);
+    memcpy(blocks + (size_t)i * 34 + 2, qs, QK);
+  }
+}
+
 /* Reference array-of-structures block layouts, mllm/core/DataTypes.hpp:110-121,164-170 (pack(1)):
  *   block_q4_0 = { fp16 d; uint8 qs[16] }  18 bytes; element j in the low nibble of qs[j], element j+16 in the high one
  *   block_q8_0 = { fp16 d; int8 qs[32] }   34 bytes

@@ -72,6 +72,17 @@ def main():
     W8 = synth.make_q8_0(rng, 4, 128)
     np.savez_compressed(os.path.join(OUT, "dequant_kat.npz"), W4=W4, y4=orc.ref_dequantize(W4, 0), W8=W8,
                         y8=orc.ref_dequantize(W8, 1))
+    # offline weight quantizers (quantize_row_q4_0 / quantize_row_q8_0 writing blocks on x86): inputs, the codes, and the
+    # scale pattern / value an x86 read of the written block yields
+    rq = np.random.default_rng(synth.SEED_BASE + 78)
+    w = (rq.standard_normal((12, 128)) * 0.05).astype(np.float32)
+    w[1, :32] = 0.0
+    w[2, :32] = np.float32(-0.5) * np.arange(32) / 31
+    w[3, :32] = np.float32(0.5) * np.arange(32) / 31
+    w[4, :32] = np.float32(8.0) * np.linspace(-1, 1, 32)
+    q8_codes, q8_d = orc.ref_quantize_rows_q8_0(w)
+    np.savez_compressed(os.path.join(OUT, "weight_quantizer_kat.npz"), w=w, q4_blocks=orc.ref_quantize_rows_q4_0(w),
+                        q8_codes=q8_codes, q8_d_eff=q8_d)
     for f in sorted(os.listdir(OUT)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(OUT, f)))

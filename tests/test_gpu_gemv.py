@@ -246,3 +246,37 @@ def test_gemv_prequantized_equals_fused(wtype, M):
         assert rel_l2(got, want) < 2e-6
     assert _lib.lib().mllm_hip_gemv_workspace_bytes(8, 2560) == 8 * 80 * 40
     assert _lib.lib().mllm_hip_gemv_workspace_bytes(9, 2560) == 0
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+def test_weight_quantizer_bit_exact_and_round_trip(wtype, golden_dir):
+    """The offline quantizer on the GPU: blocks equal to the oracle's byte for byte in both storage conventions (the
+    oracle is pinned against the reference's own quantizers), the reference-written golden vectors, and the round trip
+    quantize -> prepack -> GEMV against the oracle Linear on the same blocks."""
+    rng = synth.rng_for(1, 110 + wtype)
+    N, K = 200, 2560
+    w = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    w[1, :32] = 0.0
+    w[2, :32] = np.float32(-0.5) * np.arange(32) / 31
+    w[3, :32] = np.float32(0.5) * np.arange(32) / 31
+    w[4, :32] = np.float32(8.0) * np.linspace(-1, 1, 32)
+    announce("weight quantizer", wtype)
+    for mode, omode in ((ql.SCALE_IEEE, orc.SCALE_IEEE), (ql.SCALE_X86_REF, orc.SCALE_X86_REF)):
+        got = ql.quantize_weight_blocks(to_dev(w), wtype, mode).cpu().numpy()
+        assert np.array_equal(got, orc.quantize_weight_rows(w, wtype, omode)), mode
+    g = np.load(os.path.join(golden_dir, "weight_quantizer_kat.npz"))
+    gb = ql.quantize_weight_blocks(to_dev(g["w"]), wtype, ql.SCALE_X86_REF).cpu().numpy()
+    if wtype == 0:
+        assert np.array_equal(gb[:, :, 2:], g["q4_blocks"][:, :, 2:])
+    else:
+        assert np.array_equal(gb[:, :, 2:].view(np.int8).reshape(g["w"].shape[0], -1), g["q8_codes"])
+    # round trip in the x86 convention end to end
+    blocks = ql.quantize_weight_blocks(to_dev(w), wtype, ql.SCALE_X86_REF)
+    pw = ql.PackedQWeight(wtype, blocks, ql.SCALE_X86_REF)
+    x = synth.make_x_fp32(rng, 2, K)
+    y = ql.linear_q_gemv(pw, to_dev(x), None, ql.SCALE_X86_REF).cpu().numpy()
+    canon = orc.quantize_weight_rows(w, wtype, orc.SCALE_IEEE)  # raw patterns: the oracle applies the x86 reading itself
+    assert rel_l2(y, orc.linear_q(x, canon, wtype, None, orc.SCALE_X86_REF)) < 2e-6
+    L = _lib.lib()
+    assert L.mllm_hip_quantize_weight_blocks(wtype, None, blocks.data_ptr(), 0, 4, 64, None) == -1
+    assert L.mllm_hip_quantize_weight_blocks(wtype, blocks.data_ptr(), blocks.data_ptr(), 0, 4, 48, None) == -2

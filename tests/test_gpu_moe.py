@@ -82,6 +82,29 @@ def test_linear_q_gemm_exact_when_operands_fit_fp16():
         assert np.array_equal(y, want)
 
 
+@pytest.mark.parametrize("wtype", [0, 1])
+def test_gemm_layout_reads_x86_written_scales(wtype):
+    """A weight file written by the x86 quantizer holds each scale pattern as a half-precision NUMBER.  Both device
+    layouts must decode it the same way: same weights through the decode layout (dequantize probe, pinned bit-exactly
+    elsewhere) and through the matrix-core layout."""
+    rng = synth.rng_for(4, 77 + wtype)
+    M, N, K = 40, 96, 256
+    W = synth.make_weight(rng, wtype, N, K)
+    W[:, :, 0] |= 0x05  # off the grid where both readings agree
+    b = W[:, :, 0:2].copy().view(np.uint16)[:, :, 0]
+    Wx = W.copy()
+    Wx[:, :, 0:2] = b.astype(np.float32).astype(np.float16).view(np.uint16).reshape(N, -1, 1).view(np.uint8)
+    x = synth.make_x_fp32(rng, M, K)
+    announce("gemm layout x86 scales", wtype)
+    wg = ql.PackedQWeight(wtype, torch.from_numpy(Wx), ql.SCALE_X86_REF, layout="gemm")
+    y = ql.linear_q_gemm(wg, to_dev(x), None, ql.SCALE_X86_REF).cpu().numpy()
+    want = orc.linear_q(x, W, wtype, None, orc.SCALE_X86_REF)  # the oracle applies the x86 reading to the raw patterns
+    assert rel_l2(y, want) < GEMM_TOL, rel_l2(y, want)
+    wv = ql.PackedQWeight(wtype, torch.from_numpy(Wx), ql.SCALE_X86_REF)
+    yv = ql.linear_q(wv, to_dev(x), None, ql.SCALE_X86_REF).cpu().numpy()
+    assert rel_l2(yv, want) < 2e-6
+
+
 def test_route_counts_and_order():
     rng = synth.rng_for(4, 1)
     T, E, k = 512, 128, 8

@@ -59,6 +59,22 @@ def test_golden_dequant(golden_dir):
 
 
 # ------------------------------------------------------------------ fp16 / bf16 conversions vs numpy
+def test_golden_weight_quantizers(golden_dir):
+    """offline quantizers against vectors written by the reference's own quantize_row_q4_0 / quantize_row_q8_0"""
+    g = np.load(os.path.join(golden_dir, "weight_quantizer_kat.npz"))
+    w = g["w"]
+
+    def pattern(field):  # an x86 read of the stored field: the half-precision number as an integer
+        return field.view(np.float16).astype(np.float32).astype(np.uint16)
+    got = orc.quantize_weight_rows(w, orc.Q4_0, orc.SCALE_X86_REF)
+    assert np.array_equal(got[:, :, 2:], g["q4_blocks"][:, :, 2:])
+    assert np.array_equal(pattern(got[:, :, 0:2].copy().view(np.uint16)[:, :, 0]), g["q4_blocks"][:, :, 0:2].copy().view(np.uint16)[:, :, 0])
+    got8 = orc.quantize_weight_rows(w, orc.Q8_0, orc.SCALE_X86_REF)
+    assert np.array_equal(got8[:, :, 2:].view(np.int8).reshape(w.shape[0], -1), g["q8_codes"])
+    pat8 = pattern(got8[:, :, 0:2].copy().view(np.uint16)[:, :, 0])
+    assert np.array_equal(pat8.view(np.float16).astype(np.float32).view(np.uint32), g["q8_d_eff"].view(np.uint32))
+
+
 def test_fp16_vs_numpy():
     L = orc.lib()
     allb = np.arange(65536, dtype=np.uint16)

@@ -101,3 +101,51 @@ def test_q4_0_weights_from_reference_quantizer():
     # and the quantized Linear approximates the fp32 one
     ref = x @ Wf.T
     assert np.linalg.norm(y - ref) / np.linalg.norm(ref) < 0.15
+
+
+def _weight_rows(rng, N, K):
+    """rows with positive and negative maxima, zero blocks, codes landing exactly on the .5 truncation boundaries"""
+    w = (rng.standard_normal((N, K)) * 0.05).astype(np.float32)
+    w[1, :32] = 0.0                                            # all-zero block: d = 0, id = 0, every code 8
+    w[2, :32] = np.float32(-0.5) * np.arange(32) / 31          # negative maximum -> positive d
+    w[3, :32] = np.float32(0.5) * np.arange(32) / 31           # positive maximum -> negative d (pattern >= 0x8000)
+    w[4, :32] = np.float32(8.0) * np.linspace(-1, 1, 32)       # x*id lands on multiples of 1/2: the truncation boundaries
+    w[5, :64] = np.float32(1e-6)
+    return w
+
+
+def _x86_field_to_pattern(field):
+    """what a read on x86 makes of the stored field: the half-precision number, as an integer"""
+    return field.view(np.float16).astype(np.float32).astype(np.uint16)
+
+
+def test_q4_0_offline_quantizer_bit_exact():
+    rng = np.random.default_rng(21)
+    w = _weight_rows(rng, 24, 256)
+    ref = orc.ref_quantize_rows_q4_0(w)                        # codes + the scale pattern an x86 read yields
+    got = orc.quantize_weight_rows(w, orc.Q4_0, orc.SCALE_X86_REF)
+    assert np.array_equal(got[:, :, 2:], ref[:, :, 2:])
+    assert np.array_equal(_x86_field_to_pattern(got[:, :, 0:2].copy().view(np.uint16)[:, :, 0]),
+                          ref[:, :, 0:2].copy().view(np.uint16)[:, :, 0])
+    # IEEE storage: the field is the fp16 pattern of max / -8 itself; same codes
+    ieee = orc.quantize_weight_rows(w, orc.Q4_0, orc.SCALE_IEEE)
+    assert np.array_equal(ieee[:, :, 2:], ref[:, :, 2:])
+    blocks = w.reshape(24, -1, 32)
+    idx = np.abs(blocks).argmax(axis=2)
+    d = np.take_along_axis(blocks, idx[..., None], axis=2)[..., 0] / np.float32(-8)
+    assert np.array_equal(ieee[:, :, 0:2].copy().view(np.uint16)[:, :, 0], d.astype(np.float16).view(np.uint16))
+    assert ieee[3, 0, 0:2].copy().view(np.uint16)[0] >= 0x8000  # positive maximum: negative d, sign bit in the pattern
+
+
+def test_q8_0_offline_quantizer_bit_exact():
+    rng = np.random.default_rng(22)
+    w = _weight_rows(rng, 16, 128)
+    codes, d_eff = orc.ref_quantize_rows_q8_0(w)               # reference: codes + effective scale values
+    got = orc.quantize_weight_rows(w, orc.Q8_0, orc.SCALE_X86_REF)
+    assert np.array_equal(got[:, :, 2:].view(np.int8).reshape(16, -1), codes)
+    pat = _x86_field_to_pattern(got[:, :, 0:2].copy().view(np.uint16)[:, :, 0])
+    assert np.array_equal(pat.view(np.float16).astype(np.float32).view(np.uint32), d_eff.view(np.uint32))
+    ieee = orc.quantize_weight_rows(w, orc.Q8_0, orc.SCALE_IEEE)
+    qs, bits = orc.quantize_rows_q8_0(w)
+    assert np.array_equal(ieee[:, :, 0:2].copy().view(np.uint16)[:, :, 0], bits)
+    assert np.array_equal(ieee[:, :, 2:].view(np.int8).reshape(16, -1), qs)
