@@ -85,6 +85,62 @@ extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_linea
   return (int)y.dtype();
 }
 
+// ---- model files ---------------------------------------------------------------------------------------------------
+// One tensor of a model file: dtype, shape (rank entries) and, when `data` is given, its bytes.  Returns the byte count,
+// -1 if the name is missing.  Host only: touches no GPU.
+extern "C" __attribute__((visibility("default"))) int64_t mllm_hip_host_file_tensor(const char* path, int version, const char* name,
+                                                                                    int32_t* dtype, int32_t* rank, int32_t* shape,
+                                                                                    void* data, uint64_t capacity) {
+  initializeContext();
+  auto pf = load(path, static_cast<ModelFileVersion>(version));
+  if (!pf->has(name)) return -1;
+  Tensor t = pf->pull(name);
+  *dtype = (int32_t)t.dtype();
+  *rank = (int32_t)t.shape().size();
+  for (size_t i = 0; i < t.shape().size(); i++) shape[i] = t.shape()[i];
+  if (data) {
+    if (capacity < t.bytes()) return -2;
+    std::memcpy(data, t.ptr<void>(), t.bytes());
+  }
+  return (int64_t)t.bytes();
+}
+// read in one version, write in another; returns the tensor count
+extern "C" __attribute__((visibility("default"))) int mllm_hip_host_file_convert(const char* in_path, int in_version, const char* out_path,
+                                                                                 int out_version) {
+  initializeContext();
+  auto pf = load(in_path, static_cast<ModelFileVersion>(in_version));
+  save(out_path, pf, static_cast<ModelFileVersion>(out_version));
+  return (int)pf->dict().size();
+}
+// A Linear layer straight from a model file: mllm::load -> createOp(kLinear) -> load(params) -> forward.  V1 files carry
+// flat shapes; LinearOp::load views the weight as [out, in] as the reference does.
+extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_linear_file(const char* path, int version, const char* layer,
+                                                                                       int in_channels, int out_channels, int has_bias,
+                                                                                       const void* x_host, int x_is_bf16, void* y_host, int M,
+                                                                                       int weight_scale_x86, int act_scale_x86) {
+  initializeContext();
+  auto be = hip::initHipBackend();
+  be->setScaleModes(weight_scale_x86 ? MLLM_HIP_SCALE_X86_REF : MLLM_HIP_SCALE_IEEE,
+                    act_scale_x86 ? MLLM_HIP_SCALE_X86_REF : MLLM_HIP_SCALE_IEEE);
+  auto params = load(path, static_cast<ModelFileVersion>(version));
+  aops::LinearOpOptions opts;
+  opts.in_channels = in_channels;
+  opts.out_channels = out_channels;
+  opts.bias = has_bias != 0;
+  opts.impl_type = aops::LinearImplTypes::kDefault;
+  auto op = Context::instance().getBackend(kHIP)->createOp(OpTypes::kLinear, opts);
+  op->setName(layer);
+  op->load(params);
+  Tensor x = Tensor::fromExternal(const_cast<void*>(x_host), {1, M, in_channels}, x_is_bf16 ? kBFloat16 : kFloat32, kCPU).to(kHIP);
+  std::vector<Tensor> inputs{x}, outputs;
+  op->reshape(inputs, outputs);
+  op->setup(inputs, outputs);
+  op->forward(inputs, outputs);
+  Tensor y = outputs[0].to(kCPU);
+  std::memcpy(y_host, y.ptr<void>(), y.bytes());
+  return (int)y.dtype();
+}
+
 // fp32 MatMul through the kMatMul factory slot
 extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_matmul(const float* a_host, const float* b_host, float* c_host,
                                                                                   int M, int N, int K, int transpose_b) {

@@ -1,6 +1,9 @@
 // Implementation of the mllm core subset (see mllm_core.hpp for what is mirrored and from where).
 #include "mllm_core.hpp"
 
+#include <cstring>
+#include <fstream>
+
 #include <dlfcn.h>
 
 #include <cstring>
@@ -223,6 +226,149 @@ int32_t Context::lookupCustomizedOpId(DeviceTypes device, const std::string& nam
 void initializeContext() {
   auto& ctx = Context::instance();
   if (!ctx.memoryManager()->allocator(kCPU)) ctx.memoryManager()->registerAllocator(kCPU, std::make_shared<HostAllocator>());
+}
+
+// ---- model files ---------------------------------------------------------------------------------------------
+namespace {
+constexpr int32_t kV1Magic = 20012;
+constexpr int32_t kV2Magic = 0x519A, kV2Version = 2;
+constexpr size_t kV2ModelName = 512, kV2ParamName = 256, kV2ShapeLen = 16;
+struct __attribute__((packed)) V2Header {
+  int32_t magic_number, version;
+  char model_name[kV2ModelName];
+  uint32_t num_params;
+  uint64_t params_desc_offset;
+};
+struct __attribute__((packed)) V2Param {
+  uint32_t parameter_id, parameter_type;
+  uint64_t parameter_size, parameter_offset, shape_len;
+  int32_t shape[kV2ShapeLen];
+  char name[kV2ParamName];
+};
+static_assert(sizeof(V2Header) == 532 && sizeof(V2Param) == 352, "model file v2 layout");
+
+template <typename T>
+T take(const std::vector<char>& buf, size_t& pos) {
+  MLLM_RT_ASSERT(pos + sizeof(T) <= buf.size());
+  T v;
+  std::memcpy(&v, buf.data() + pos, sizeof(T));
+  pos += sizeof(T);
+  return v;
+}
+Tensor readTensor(std::ifstream& f, const std::string& name, const Tensor::shape_t& shape, DataTypes dtype, uint64_t offset,
+                  uint64_t stored_bytes) {
+  Tensor t = Tensor::empty(shape, dtype, kCPU).alloc();
+  MLLM_RT_ASSERT(stored_bytes >= t.bytes());
+  f.seekg((std::streamoff)offset, std::ios::beg);
+  f.read(t.ptr<char>(), (std::streamsize)t.bytes());
+  if (!f) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: tensor '%s' is truncated", name.c_str());
+  t.setName(name);
+  return t;
+}
+}  // namespace
+
+ParameterFile::ptr_t load(const std::string& file_name, ModelFileVersion version, DeviceTypes map_2_device, bool /*mmap*/) {
+  if (map_2_device != kCPU || (version != ModelFileVersion::kV1 && version != ModelFileVersion::kV2))
+    return ParameterFile::create();  // "return empty if not match all" (mllm/mllm.cpp:142-143)
+  std::ifstream f(file_name, std::ios::binary);
+  if (!f.is_open()) MLLM_ERROR_EXIT(ExitCode::kIOError, "Failed to open file for reading: %s", file_name.c_str());
+  auto pf = ParameterFile::create(version);
+  if (version == ModelFileVersion::kV1) {
+    int32_t magic = 0;
+    uint64_t desc_bytes = 0;
+    f.read(reinterpret_cast<char*>(&magic), 4);
+    f.read(reinterpret_cast<char*>(&desc_bytes), 8);
+    MLLM_RT_ASSERT_EQ(kV1Magic, magic);
+    std::vector<char> buf(desc_bytes);
+    f.read(buf.data(), (std::streamsize)desc_bytes);
+    if (!f) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
+    struct Item { std::string name; uint64_t len, offset; int32_t dtype; };
+    std::vector<Item> items;
+    for (size_t pos = 0; pos < buf.size();) {
+      Item it;
+      const uint32_t name_len = take<uint32_t>(buf, pos);
+      MLLM_RT_ASSERT(pos + name_len <= buf.size());
+      it.name.assign(buf.data() + pos, name_len);
+      pos += name_len;
+      it.len = take<uint64_t>(buf, pos);
+      it.offset = take<uint64_t>(buf, pos);
+      it.dtype = take<int32_t>(buf, pos);
+      items.push_back(it);
+    }
+    for (const auto& it : items) {
+      const auto dtype = static_cast<DataTypes>(it.dtype);
+      const Tensor::shape_t shape = {(int32_t)(it.len / bytesOfType(dtype) * lanesOfType(dtype))};  // flat, as the reference
+      pf->push(it.name, readTensor(f, it.name, shape, dtype, it.offset, it.len));
+    }
+  } else {
+    V2Header h{};
+    f.read(reinterpret_cast<char*>(&h), sizeof(h));
+    MLLM_RT_ASSERT_EQ(kV2Magic, h.magic_number);
+    MLLM_RT_ASSERT_EQ(kV2Version, h.version);
+    std::vector<V2Param> descs(h.num_params);
+    f.seekg((std::streamoff)h.params_desc_offset, std::ios::beg);  // an extra data segment in front of it is skipped
+    f.read(reinterpret_cast<char*>(descs.data()), (std::streamsize)(descs.size() * sizeof(V2Param)));
+    if (!f) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
+    for (const auto& d : descs) {
+      const std::string name(d.name, strnlen(d.name, sizeof(d.name)));
+      MLLM_RT_ASSERT(d.shape_len <= kV2ShapeLen);
+      Tensor::shape_t shape(d.shape, d.shape + d.shape_len);
+      pf->push(name, readTensor(f, name, shape, static_cast<DataTypes>(d.parameter_type), d.parameter_offset, d.parameter_size));
+    }
+  }
+  return pf;
+}
+
+void save(const std::string& file_name, const ParameterFile::ptr_t& parameter_file, ModelFileVersion version,
+          DeviceTypes map_2_device) {
+  if (map_2_device != kCPU || (version != ModelFileVersion::kV1 && version != ModelFileVersion::kV2)) return;
+  std::ofstream out(file_name, std::ios::binary);
+  if (!out.is_open()) MLLM_ERROR_EXIT(ExitCode::kIOError, "Failed to open file for writing: %s", file_name.c_str());
+  const auto& dict = parameter_file->dict();
+  if (version == ModelFileVersion::kV1) {
+    uint64_t desc_bytes = 0;
+    for (const auto& [name, t] : dict) desc_bytes += 4 + name.size() + 8 + 8 + 4;
+    out.write(reinterpret_cast<const char*>(&kV1Magic), 4);
+    out.write(reinterpret_cast<const char*>(&desc_bytes), 8);
+    uint64_t offset = 12 + desc_bytes;  // absolute, from the start of the file
+    for (const auto& [name, t] : dict) {
+      const uint32_t name_len = (uint32_t)name.size();
+      const uint64_t len = t.bytes();
+      const int32_t dtype = (int32_t)t.dtype();
+      out.write(reinterpret_cast<const char*>(&name_len), 4);
+      out.write(name.data(), name_len);
+      out.write(reinterpret_cast<const char*>(&len), 8);
+      out.write(reinterpret_cast<const char*>(&offset), 8);
+      out.write(reinterpret_cast<const char*>(&dtype), 4);
+      offset += len;
+    }
+  } else {
+    V2Header h{};
+    h.magic_number = kV2Magic;
+    h.version = kV2Version;
+    h.num_params = (uint32_t)dict.size();
+    h.params_desc_offset = sizeof(V2Header);
+    out.write(reinterpret_cast<const char*>(&h), sizeof(h));
+    uint64_t offset = sizeof(V2Header) + dict.size() * sizeof(V2Param);
+    uint32_t id = 0;
+    for (const auto& [name, t] : dict) {
+      V2Param d{};
+      d.parameter_id = id++;
+      d.parameter_type = (uint32_t)t.dtype();
+      d.parameter_size = t.bytes();
+      d.parameter_offset = offset;
+      d.shape_len = t.shape().size();
+      MLLM_RT_ASSERT(d.shape_len <= kV2ShapeLen);
+      for (size_t i = 0; i < t.shape().size(); i++) d.shape[i] = t.shape()[i];
+      std::strncpy(d.name, name.c_str(), kV2ParamName - 1);
+      out.write(reinterpret_cast<const char*>(&d), sizeof(d));
+      offset += t.bytes();
+    }
+  }
+  for (const auto& [name, t] : dict) {
+    MLLM_RT_ASSERT_EQ(t.device(), kCPU);
+    out.write(t.ptr<char>(), (std::streamsize)t.bytes());
+  }
 }
 
 void loadOpPackage(const std::string& path) {

@@ -344,6 +344,14 @@ class Context {
 };
 
 void initializeContext();                       // registers the host (CPU) allocator: mllm/mllm.hpp:145-164
+// Model files, mllm/mllm.cpp:135-154 with mllm/core/ParameterFile.cpp:68-440 and the schemas
+// mllm/core/schema/ModelFileV1.hpp:36-52 (magic 20012; name, byte length, offset, dtype per tensor; shapes are flat) and
+// ModelFileV2.hpp:40-62 (magic 0x519A, version 2; 352-byte descriptors with dtype, size, offset, shape, name).
+// Tensors come back as host tensors that own their memory; `mmap` is accepted and ignored (always a buffered read).
+ParameterFile::ptr_t load(const std::string& file_name, ModelFileVersion version = ModelFileVersion::kV1,
+                          DeviceTypes map_2_device = kCPU, bool mmap = false);
+void save(const std::string& file_name, const ParameterFile::ptr_t& parameter_file,
+          ModelFileVersion version = ModelFileVersion::kV1, DeviceTypes map_2_device = kCPU);
 void loadOpPackage(const std::string& path);    // dlopen + opPackageDescriptor(): mllm/backends/base/PluginSystem.cpp:37-90
 
 }  // namespace mllm

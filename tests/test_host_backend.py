@@ -116,3 +116,130 @@ def test_matmul_slot():
     bt = np.ascontiguousarray(b.T)
     assert L.mllm_hip_backend_run_matmul(p(a), p(bt), p(c), M, N, K, 0) == 0
     assert np.allclose(c, a @ b.T, rtol=1e-5, atol=1e-4)
+
+
+# ---- model files -------------------------------------------------------------------------------------------------------
+# Writers restated from the file layouts (mllm/core/schema/ModelFileV1.hpp:36-52, ModelFileV2.hpp:40-62; struct formats as
+# pymllm/mobile/convertor/model_file_v2.py:68-99 packs them).  dtype ids: mllm/core/DataTypes.hpp (kFloat32 0, kFloat16 1,
+# kGGUF_Q4_0 2, kGGUF_Q8_0 8, kInt8 16, kBFloat16 128, kUInt8 129).
+import struct
+
+_DT = {"f32": 0, "f16": 1, "q4_0": 2, "q8_0": 8, "i8": 16, "bf16": 128, "u8": 129}
+
+
+def _write_v1(path, tensors):
+    """tensors: list of (name, dtype id, shape, bytes)"""
+    desc = sum(4 + len(n.encode()) + 8 + 8 + 4 for n, _, _, _ in tensors)
+    off = 12 + desc
+    with open(path, "wb") as f:
+        f.write(struct.pack("<iQ", 20012, desc))
+        for n, dt, _, b in tensors:
+            nb = n.encode()
+            f.write(struct.pack("<I", len(nb)) + nb + struct.pack("<QQi", len(b), off, dt))
+            off += len(b)
+        for _, _, _, b in tensors:
+            f.write(b)
+
+
+def _write_v2(path, tensors, extra=b""):
+    off = 532 + len(extra) + 352 * len(tensors)
+    with open(path, "wb") as f:
+        f.write(struct.pack("<II512sIQ", 0x519A, 2, b"test-model".ljust(512, b"\0"), len(tensors), 532 + len(extra)))
+        f.write(extra)
+        for i, (n, dt, shape, b) in enumerate(tensors):
+            f.write(struct.pack("<IIQQQ16i256s", i, dt, len(b), off, len(shape), *(list(shape) + [0] * (16 - len(shape))),
+                                n.encode().ljust(256, b"\0")))
+            off += len(b)
+        for _, _, _, b in tensors:
+            f.write(b)
+
+
+def _file_tensor(L, path, version, name):
+    L.mllm_hip_host_file_tensor.restype = C.c_int64
+    dt, rank = C.c_int32(), C.c_int32()
+    shape = (C.c_int32 * 16)()
+    n = L.mllm_hip_host_file_tensor(path.encode(), version, name.encode(), C.byref(dt), C.byref(rank), shape, None,
+                                    C.c_uint64(0))
+    if n < 0:
+        return None
+    buf = (C.c_uint8 * max(n, 1))()
+    assert L.mllm_hip_host_file_tensor(path.encode(), version, name.encode(), C.byref(dt), C.byref(rank), shape, buf,
+                                       C.c_uint64(n)) == n
+    return dt.value, list(shape[:rank.value]), bytes(buf[:n])
+
+
+def _linear_file_tensors(rng, wtype, N, K):
+    W = synth.make_weight(rng, wtype, N, K)
+    bias = rng.standard_normal(N).astype(np.float32)
+    name = "model.layers.3.mlp.down_proj"
+    return W, bias, name, [(name + ".weight", _DT["q4_0"] if wtype == 0 else _DT["q8_0"], [N, K], W.tobytes()),
+                           (name + ".bias", _DT["f32"], [N], bias.tobytes()),
+                           ("model.norm.weight", _DT["f16"], [K], rng.standard_normal(K).astype(np.float16).tobytes())]
+
+
+def test_model_file_readers_and_writers(tmp_path):
+    """V1 and V2 files written here are read back tensor for tensor (dtype, shape, bytes); a file converted by the library
+    (V1 -> V2 -> V1) is parsed here and holds the same tensors; a V2 file with an extra data segment in front of the
+    descriptors is read; a missing tensor reports so."""
+    L = _host()
+    rng = synth.rng_for(5, 31)
+    W, bias, name, tensors = _linear_file_tensors(rng, 0, 48, 96)
+    p1, p2, p2x = str(tmp_path / "m1.mllm"), str(tmp_path / "m2.mllm"), str(tmp_path / "m2x.mllm")
+    _write_v1(p1, tensors)
+    _write_v2(p2, tensors)
+    _write_v2(p2x, tensors, extra=b"\xab" * 100)
+    for n, dt, shape, b in tensors:
+        got1 = _file_tensor(L, p1, 1, n)
+        numel = int(np.prod(shape))
+        assert got1 == (dt, [numel], b)                       # V1 carries no shapes: flat, element count from the byte length
+        assert _file_tensor(L, p2, 2, n) == (dt, shape, b)
+        assert _file_tensor(L, p2x, 2, n) == (dt, shape, b)
+    assert _file_tensor(L, p2, 2, "no.such.tensor") is None
+    # library-side conversion, parsed independently here
+    c2, c1 = str(tmp_path / "c2.mllm"), str(tmp_path / "c1.mllm")
+    assert L.mllm_hip_host_file_convert(p1.encode(), 1, c2.encode(), 2) == 3
+    assert L.mllm_hip_host_file_convert(c2.encode(), 2, c1.encode(), 1) == 3
+    raw = open(c2, "rb").read()
+    magic, ver, _, num, doff = struct.unpack_from("<II512sIQ", raw, 0)
+    assert (magic, ver, num, doff) == (0x519A, 2, 3, 532)
+    seen = {}
+    for i in range(num):
+        pid, dt, size, off, slen, *rest = struct.unpack_from("<IIQQQ16i256s", raw, doff + 352 * i)
+        seen[rest[16].rstrip(b"\0").decode()] = (dt, raw[off:off + size])
+    for n, dt, shape, b in tensors:
+        assert seen[n] == (dt, b)
+    raw1 = open(c1, "rb").read()
+    magic1, desc_len = struct.unpack_from("<iQ", raw1, 0)
+    assert magic1 == 20012
+    pos, names = 12, []
+    while pos < 12 + desc_len:
+        (nl,) = struct.unpack_from("<I", raw1, pos)
+        nm = raw1[pos + 4:pos + 4 + nl].decode()
+        ln, off, dt = struct.unpack_from("<QQi", raw1, pos + 4 + nl)
+        pos += 4 + nl + 20
+        names.append(nm)
+        want = {n: (d, b) for n, d, _, b in tensors}[nm]
+        assert (dt, raw1[off:off + ln]) == want
+    assert sorted(names) == sorted(n for n, _, _, _ in tensors)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("version", [1, 2])
+def test_linear_from_model_file(tmp_path, version):
+    """mllm::load -> createOp(kLinear) -> load(params) -> forward on a file holding reference Q4_0 / Q8_0 blocks"""
+    from oracle import oracle as orc
+    from gpu_util import announce, rel_l2
+    L = _host()
+    rng = synth.rng_for(5, 40 + version)
+    N, K, M = 96, 256, 3
+    for wtype in (0, 1):
+        W, bias, name, tensors = _linear_file_tensors(rng, wtype, N, K)
+        path = str(tmp_path / ("lin%d_%d.mllm" % (version, wtype)))
+        (_write_v1 if version == 1 else _write_v2)(path, tensors)
+        x = synth.make_x_fp32(rng, M, K)
+        y = np.empty((M, N), np.float32)
+        announce("linear from file", version, wtype)
+        rc = L.mllm_hip_backend_run_linear_file(path.encode(), version, name.encode(), K, N, 1, x.ctypes.data_as(C.c_void_p), 0,
+                                                y.ctypes.data_as(C.c_void_p), M, 0, 1)
+        assert rc == 0  # kFloat32
+        assert rel_l2(y, orc.linear_q(x, W, wtype, bias, orc.SCALE_X86_REF)) < 2e-6
