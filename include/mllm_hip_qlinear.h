@@ -32,6 +32,9 @@ extern "C" {
 enum { MLLM_HIP_Q4_0 = 0, MLLM_HIP_Q8_0 = 1 };
 /* activation element types */
 enum { MLLM_HIP_F32 = 0, MLLM_HIP_BF16 = 1 };
+/* instead of activations: their Q8_0 image as the decode GEMV reads it (mllm_hip_gemv_workspace_bytes, written by
+ * mllm_hip_rmsnorm / mllm_hip_silu_mul); only where an entry point says so */
+enum { MLLM_HIP_Q8_IMAGE = 2 };
 /* How a block scale is read.
  *   IEEE     the 2-byte `d` field is an IEEE fp16 bit pattern (ARM builds of the reference, GGUF files)
  *   X86_REF  the x86 build of the reference: the field is a half-precision NUMBER equal to the bit pattern
@@ -85,6 +88,14 @@ int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_gemv_part
 size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K);
 int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M,
                                     int64_t K, int act_scale_mode, void* workspace, void* stream);
+
+/* The decode GEMV with its neighbours folded in.  residual: NULL, or nparts pointers (each NULL or fp32 [M][N], may be the
+ * part's y): y = (bias + W x) + residual, the order of Linear followed by the elementwise add it replaces
+ * (mllm/models/qwen3/modeling_qwen3_fa2.hpp:233-240).  x_kind: MLLM_HIP_F32 / MLLM_HIP_BF16 activations [M][K], or
+ * MLLM_HIP_Q8_IMAGE: the image a producer kernel wrote for these M rows (act_scale_mode was applied there); the results
+ * are those of the plain call on the tensor the producer stored, bit for bit. */
+int mllm_hip_linear_q_gemv_fused(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual,
+                                 const void* x, int x_kind, int M, int64_t K, int act_scale_mode, void* stream);
 
 /* Same for any M: quantizes the activations with a stand-alone kernel into `workspace`
  * (mllm_hip_linear_q_workspace_bytes) and runs the tiled block-dot kernel.  Used by prefill and by the MoE path. */
@@ -251,6 +262,48 @@ int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed
  * replaces: the histogram + argsort at modeling_qwen3_moe_fa2.hpp:178-197 */
 int mllm_hip_moe_route(const int32_t* topk_ids, int64_t T, int E, int k, int32_t* counts, int32_t* offsets,
                        int32_t* sorted_idx, void* workspace, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * The operators either side of a quantized Linear in a decoder layer.  dtype: MLLM_HIP_F32 or MLLM_HIP_BF16 (arithmetic
+ * in fp32, results rounded to the tensor's type).  All pointers 16-byte aligned, element counts multiples of 8.
+ * q_image (may be NULL; rows <= 8, D % 32 == 0): also writes the Q8_0 image of the rows just stored, for
+ * mllm_hip_linear_q_gemv_fused(..., MLLM_HIP_Q8_IMAGE, ...); size mllm_hip_gemv_workspace_bytes(rows, D).
+ * ------------------------------------------------------------------------------------------------------- */
+
+/* y = x * (w * rms) [x * ((w + 1) * rms) with add_unit_offset], rms = 1 / sqrt(mean(x^2) + epsilon); weight fp32 [D].
+ * replaces: CPURMSNormOp::forward -> x86::rmsnorm_fp32  mllm/backends/cpu/ops/RMSNormOp.cpp:14-96,
+ *           mllm/backends/cpu/kernels/x86/rmsnorm.cpp:17-52.  D <= 16384. */
+int mllm_hip_rmsnorm(const void* x, int dtype, const float* weight, void* y, int64_t rows, int64_t D, float epsilon,
+                     int add_unit_offset, void* q_image, int act_scale_mode, void* stream);
+
+/* y = x * (1 / (1 + exp(-x))) with the reference's polynomial exp.
+ * replaces: CPUSiLUOp::forward -> x86::silu_fp32  mllm/backends/cpu/kernels/x86/silu.cpp:16-56, math.hpp:19-72 */
+int mllm_hip_silu(const void* x, void* y, int dtype, int64_t n, void* stream);
+/* y = a + b, y = a * b (same shapes).  replaces: CPUAddOp / CPUMulOp::forward  mllm/backends/cpu/ops/ElewiseOps.cpp */
+int mllm_hip_add(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream);
+int mllm_hip_mul(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream);
+/* y = silu(gate) * up in one pass (the SiLU result is rounded to the tensor's type before the product, as when the two
+ * operators run one after the other).  replaces: silu_(gate) then x * y  mllm/models/qwen3/modeling_qwen3_fa2.hpp:87-90 */
+int mllm_hip_silu_mul(const void* gate, const void* up, void* y, int dtype, int64_t rows, int64_t D, void* q_image,
+                      int act_scale_mode, void* stream);
+/* 0 (default): exp as the reference's x86 kernels compute it (math.hpp:19-72); 1: expf.  Process-wide; affects SiLU,
+ * softmax and the MoE gate. */
+int mllm_hip_set_exp_mode(int accurate);
+
+/* softmax over the last axis of fp32 [rows][len].
+ * replaces: CPUSoftmaxOp::forward -> x86::softmax_v1_fp32  mllm/backends/cpu/kernels/x86/softmax.cpp:18-76 */
+int mllm_hip_softmax(const float* x, float* y, int64_t rows, int64_t len, void* stream);
+/* k largest (or smallest) of every row of fp32 [rows][len]: values fp32 [rows][k], indices int32 [rows][k]; sorted != 0:
+ * by value, else by index; equal values are taken lowest index first.
+ * replaces: CPUTopKOp::forward  mllm/backends/cpu/ops/TopKOp.cpp:20-72 */
+int mllm_hip_topk(const float* x, float* values, int32_t* indices, int64_t rows, int64_t len, int k, int largest, int sorted,
+                  void* stream);
+/* The MoE gate in one launch: scores = softmax(x . W^T) in fp32, the k largest per token in index order, weights divided
+ * by their sum when norm_topk_prob.  x [M][H] fp32 or bf16; gate_weight fp32 [E][H]; topk_ids int32 [M][k]; topk_weights
+ * fp32 [M][k]; scores fp32 [M][E] or NULL.  H % 8 == 0.
+ * replaces: MoEGate::forward  mllm/models/qwen3_moe/modeling_qwen3_moe_fa2.hpp:121-139 */
+int mllm_hip_moe_gate(const void* x, int x_dtype, const float* gate_weight, int32_t* topk_ids, float* topk_weights, float* scores,
+                      int64_t M, int64_t H, int64_t E, int k, int norm_topk_prob, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------
  * fp32 activation x activation MatMul (the backend's kMatMul slot; not a quantized path)

@@ -48,6 +48,16 @@ def lib():
         L.mllm_hip_linear_q_gemv.argtypes = [ci, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi_ws.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp, vp]
+        L.mllm_hip_linear_q_gemv_fused.argtypes = [ci, ci, C.POINTER(GemvPart), C.POINTER(vp), vp, ci, ci, i64, ci, vp]
+        L.mllm_hip_rmsnorm.argtypes = [vp, ci, vp, vp, i64, i64, C.c_float, ci, vp, ci, vp]
+        L.mllm_hip_silu.argtypes = [vp, vp, ci, i64, vp]
+        L.mllm_hip_add.argtypes = [vp, vp, vp, ci, i64, vp]
+        L.mllm_hip_mul.argtypes = [vp, vp, vp, ci, i64, vp]
+        L.mllm_hip_silu_mul.argtypes = [vp, vp, vp, ci, i64, i64, vp, ci, vp]
+        L.mllm_hip_set_exp_mode.argtypes = [ci]
+        L.mllm_hip_softmax.argtypes = [vp, vp, i64, i64, vp]
+        L.mllm_hip_topk.argtypes = [vp, vp, vp, i64, i64, ci, ci, ci, vp]
+        L.mllm_hip_moe_gate.argtypes = [vp, ci, vp, vp, vp, vp, i64, i64, i64, ci, ci, vp]
         L.mllm_hip_quantize_q8_0.argtypes = [vp, ci, vp, vp, i64, i64, vp]
         L.mllm_hip_q_dequantize.argtypes = [ci, vp, vp, i64, i64, vp]
         L.mllm_hip_q_block_isums.argtypes = [ci, vp, vp, vp, i64, i64, i64, vp]

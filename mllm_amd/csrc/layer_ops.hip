@@ -1,0 +1,576 @@
+// The operators either side of a quantized Linear in a decoder layer, for gfx950: RMSNorm, SiLU, elementwise add / mul,
+// SiLU(gate) * up, softmax, top-k and the whole MoE gate (logits -> softmax -> top-k -> normalise).
+//
+// Arithmetic follows the reference's x86 CPU kernels:
+//   RMSNorm   mllm/backends/cpu/kernels/x86/rmsnorm.cpp:17-52      y = x * (w * rms), rms = 1 / sqrt(mean(x^2) + eps)
+//   SiLU      mllm/backends/cpu/kernels/x86/silu.cpp:16-27         x * (1 / (1 + exp_poly(-x)))
+//   exp_poly  mllm/backends/cpu/kernels/x86/math.hpp:19-72         Cephes polynomial
+//   softmax   mllm/backends/cpu/kernels/x86/softmax.cpp:18-76      exp_poly(x - max) * (1 / sum); expf for len <= 16
+//   top-k     mllm/backends/cpu/ops/TopKOp.cpp:20-72               k extreme values, by value or by index
+//   MoE gate  mllm/models/qwen3_moe/modeling_qwen3_moe_fa2.hpp:121-139
+// Sums run in a different order than the CPU's vector lanes; everything elementwise is the same fp32 operation
+// sequence.
+//
+// All of these are HBM- or latency-bound.  What they add for this GPU: the kernels that produce the input of a decode
+// GEMV (RMSNorm, SiLU*up) can also write that input's Q8_0 image in the form the GEMV kernel copies into LDS, so the
+// GEMV of every workgroup skips the quantization.
+#include "qcommon.h"
+
+namespace mllmhip {
+
+// `accurate` replaces the polynomial (whose argument reduction, as written in the reference, leaves a relative error of
+// about 2.1e-4 per unit of the binary exponent of the result) by expf.
+__device__ __forceinline__ float silu_ref(float x, bool accurate) { return x * (1.0f / (1.0f + (accurate ? expf(-x) : exp_poly(-x)))); }
+
+// ---- eight consecutive elements per lane ------------------------------------------------------------------------------
+template <int XT>
+struct Item8 {
+  u32x4 r[XT == MLLM_HIP_F32 ? 2 : 1];
+};
+template <int XT>
+__device__ __forceinline__ void item_load(const void* p, int64_t elem, Item8<XT>& it) {
+  if (XT == MLLM_HIP_F32) {
+    const u32x4* q = reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(p) + elem);
+    it.r[0] = q[0];
+    it.r[XT == MLLM_HIP_F32 ? 1 : 0] = q[1];
+  } else {
+    it.r[0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(p) + elem);
+  }
+}
+template <int XT>
+__device__ __forceinline__ void item_to_f32(const Item8<XT>& it, float (&v)[8]) {
+  if (XT == MLLM_HIP_F32) {
+    const u32x4 a = it.r[0], b = it.r[XT == MLLM_HIP_F32 ? 1 : 0];
+    v[0] = __uint_as_float(a.x); v[1] = __uint_as_float(a.y); v[2] = __uint_as_float(a.z); v[3] = __uint_as_float(a.w);
+    v[4] = __uint_as_float(b.x); v[5] = __uint_as_float(b.y); v[6] = __uint_as_float(b.z); v[7] = __uint_as_float(b.w);
+  } else {
+    const uint32_t w[4] = {it.r[0].x, it.r[0].y, it.r[0].z, it.r[0].w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      v[2 * j + 0] = __uint_as_float(w[j] << 16);
+      v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+  }
+}
+// stores v in the tensor's type and leaves in v what a reader of the tensor will see (bf16: the rounded values)
+template <int XT>
+__device__ __forceinline__ void item_store(void* p, int64_t elem, float (&v)[8]) {
+  if (XT == MLLM_HIP_F32) {
+    u32x4* q = reinterpret_cast<u32x4*>(reinterpret_cast<float*>(p) + elem);
+    q[0] = u32x4{__float_as_uint(v[0]), __float_as_uint(v[1]), __float_as_uint(v[2]), __float_as_uint(v[3])};
+    q[1] = u32x4{__float_as_uint(v[4]), __float_as_uint(v[5]), __float_as_uint(v[6]), __float_as_uint(v[7])};
+  } else {
+    u32x4 o = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+    *reinterpret_cast<u32x4*>(reinterpret_cast<uint16_t*>(p) + elem) = o;
+    const uint32_t w[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      v[2 * j + 0] = __uint_as_float(w[j] << 16);
+      v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+  }
+}
+
+// The Q8_0 image of activation rows that the decode GEMV copies into LDS: for MT rows of nb blocks, 16-byte planes of
+// elements 0..15 and 16..31 of every block, then the fp32 effective scales, then -8 * sum(codes).
+struct QImage {
+  unsigned char* base;  // null: no image wanted
+  int MT, nb, x86_scale;
+};
+// Four neighbouring lanes (a quad) hold the four eighths of one 32-element block: lane j of the quad has elements
+// 8j..8j+7.  Same arithmetic as quantize_row_q8_0 (quantize_q8.cpp:106-190), same image as quant_image_kernel writes.
+__device__ __forceinline__ void quad_quantize_to_image(const float (&v)[8], const QImage& q, int m, int blk, int j, bool write) {
+  float amax = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[e]));
+  amax = fmaxf(amax, dpp_f<0xB1>(amax));
+  amax = fmaxf(amax, dpp_f<0x4E>(amax));
+  const float d = amax / 127.f;
+  const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
+  uint32_t pk[2];
+#pragma unroll
+  for (int w = 0; w < 2; w++) {
+    uint32_t p = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      int qi = (int)rintf(v[4 * w + e] * idv);
+      qi = min(127, max(-128, qi));
+      p |= ((uint32_t)qi & 0xffu) << (8 * e);
+    }
+    pk[w] = p;
+  }
+  int sum = __builtin_amdgcn_sdot4((int)pk[0], 0x01010101, 0, false);
+  sum = __builtin_amdgcn_sdot4((int)pk[1], 0x01010101, sum, false);
+  sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xf, 0xf, true);
+  sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xf, 0xf, true);
+  if (!write) return;
+  const int mnb = q.MT * q.nb;
+  const int id = m * q.nb + blk;
+  u32x4* lo = reinterpret_cast<u32x4*>(q.base);
+  u32x4* hi = lo + mnb;
+  float* sd = reinterpret_cast<float*>(hi + mnb);
+  int* sn = reinterpret_cast<int*>(sd + mnb);
+  u32x2* dst = reinterpret_cast<u32x2*>((j < 2 ? lo : hi) + id) + (j & 1);
+  *dst = u32x2{pk[0], pk[1]};
+  if (j == 0) {
+    uint16_t bits = f32_to_f16bits(d);
+    if (q.x86_scale) bits = x86_scale_bits(bits);
+    sd[id] = f16bits_to_f32(bits);
+    sn[id] = -8 * sum;
+  }
+}
+// rows of the image beyond the real ones read as zero blocks
+__device__ __forceinline__ void image_zero_row(const QImage& q, int m, int tid, int nthreads) {
+  const int mnb = q.MT * q.nb;
+  u32x4* lo = reinterpret_cast<u32x4*>(q.base);
+  u32x4* hi = lo + mnb;
+  float* sd = reinterpret_cast<float*>(hi + mnb);
+  int* sn = reinterpret_cast<int*>(sd + mnb);
+  for (int b = tid; b < q.nb; b += nthreads) {
+    lo[m * q.nb + b] = u32x4{0, 0, 0, 0};
+    hi[m * q.nb + b] = u32x4{0, 0, 0, 0};
+    sd[m * q.nb + b] = 0.f;
+    sn[m * q.nb + b] = 0;
+  }
+}
+
+__device__ __forceinline__ float wave_sum(float v) { return group_sum<64>(v); }
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, dpp_f<0xB1>(v));
+  v = fmaxf(v, dpp_f<0x4E>(v));
+  v = fmaxf(v, dpp_f<0x141>(v));
+  v = fmaxf(v, dpp_f<0x140>(v));
+  v = fmaxf(v, __shfl_xor(v, 16, 64));
+  v = fmaxf(v, __shfl_xor(v, 32, 64));
+  return v;
+}
+
+// ---- RMSNorm ----------------------------------------------------------------------------------------------------------
+struct RmsArgs {
+  const void* x;
+  const float* w;
+  void* y;
+  int64_t rows;
+  int D;
+  float eps;
+  int add_unit_offset;
+  QImage img;
+};
+// One workgroup per row; a lane keeps NI items of eight elements in registers between the two passes.
+template <int XT, int NI>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(RmsArgs a) {
+  __shared__ float s_part[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t row = blockIdx.x;
+  if (row >= a.rows) {  // only launched for the zero rows of an image
+    image_zero_row(a.img, (int)row, tid, 256);
+    return;
+  }
+  const int nitems = a.D >> 3;
+  Item8<XT> raw[NI];
+  Item8<MLLM_HIP_F32> wraw[NI];
+#pragma unroll
+  for (int k = 0; k < NI; k++) {
+    const int it = min(tid + 256 * k, nitems - 1);
+    item_load<XT>(a.x, row * a.D + (int64_t)it * 8, raw[k]);
+  }
+#pragma unroll
+  for (int k = 0; k < NI; k++) {
+    const int it = min(tid + 256 * k, nitems - 1);
+    item_load<MLLM_HIP_F32>(a.w, (int64_t)it * 8, wraw[k]);
+  }
+  float v[NI][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NI; k++) {
+    item_to_f32<XT>(raw[k], v[k]);
+    if (tid + 256 * k < nitems) {
+#pragma unroll
+      for (int e = 0; e < 8; e++) ss = fmaf(v[k][e], v[k][e], ss);
+    }
+  }
+  ss = wave_sum(ss);
+  if (lane == 0) s_part[wave] = ss;
+  __syncthreads();
+  const float total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+  const float rms = 1.0f / sqrtf(total / (float)a.D + a.eps);
+#pragma unroll
+  for (int k = 0; k < NI; k++) {
+    const int it = tid + 256 * k;
+    const bool valid = it < nitems;
+    float wv[8], o[8];
+    item_to_f32<MLLM_HIP_F32>(wraw[k], wv);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      const float mult = (a.add_unit_offset ? wv[e] + 1.0f : wv[e]) * rms;
+      o[e] = valid ? v[k][e] * mult : 0.f;
+    }
+    if (valid) item_store<XT>(a.y, row * a.D + (int64_t)it * 8, o);
+    if (a.img.base) quad_quantize_to_image(o, a.img, (int)row, it >> 2, it & 3, valid);
+  }
+}
+
+// ---- elementwise: SiLU, SiLU(gate) * up, add, mul ---------------------------------------------------------------------
+enum { EW_SILU = 0, EW_SILU_MUL = 1, EW_ADD = 2, EW_MUL = 3 };
+struct EwArgs {
+  const void* a;
+  const void* b;
+  void* y;
+  int64_t rows;  // image: rows of D elements; without image rows * D is just the element count
+  int D;
+  int exp_accurate;
+  QImage img;
+};
+template <int XT, int OP>
+__global__ __launch_bounds__(256) void elementwise_kernel(EwArgs a) {
+  const int ipr = a.D >> 3;  // items per row
+  const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t row = it / ipr;
+  const int col = (int)(it - row * ipr);
+  const int64_t total_rows = a.img.base ? max((int64_t)a.img.MT, a.rows) : a.rows;
+  if (row >= total_rows) return;  // whole quads leave together: ipr is a multiple of 4 whenever an image is written
+  float o[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const bool valid = row < a.rows;
+  if (valid) {
+    Item8<XT> ra, rb;
+    float va[8], vb[8];
+    item_load<XT>(a.a, it * 8, ra);
+    if (OP != EW_SILU) item_load<XT>(a.b, it * 8, rb);
+    item_to_f32<XT>(ra, va);
+    if (OP != EW_SILU) item_to_f32<XT>(rb, vb);
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      if (OP == EW_SILU) o[e] = silu_ref(va[e], a.exp_accurate);
+      if (OP == EW_SILU_MUL) {
+        // the reference runs SiLU and the product as two operators: the SiLU result is stored in the tensor's type first
+        float s = silu_ref(va[e], a.exp_accurate);
+        if (XT != MLLM_HIP_F32) s = bf16_to_f32(f32_to_bf16(s));
+        o[e] = s * vb[e];
+      }
+      if (OP == EW_ADD) o[e] = va[e] + vb[e];
+      if (OP == EW_MUL) o[e] = va[e] * vb[e];
+    }
+    item_store<XT>(a.y, it * 8, o);
+  }
+  if (a.img.base) quad_quantize_to_image(o, a.img, (int)row, col >> 2, col & 3, true);
+}
+
+// ---- softmax over the last axis, one wave per row ----------------------------------------------------------------------
+// rows of at most 16 elements use expf like the reference's short-row branch (softmax.cpp:19-31); in longer rows the
+// whole vectors of eight take the polynomial and the len % 8 tail elements expf (softmax.cpp:44-57)
+__device__ __forceinline__ float softmax_exp(float x, bool poly) { return poly ? exp_poly(x) : expf(x); }
+
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const float* __restrict__ x, float* __restrict__ y, int64_t rows, int len,
+                                                           int exp_accurate) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const float* xr = x + row * len;
+  float* yr = y + row * len;
+  const bool poly = len > 16 && !exp_accurate;
+  float mx = -3.402823466e+38f;
+  for (int i = lane; i < len; i += 64) mx = fmaxf(mx, xr[i]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int i = lane; i < len; i += 64) {
+    const float e = softmax_exp(xr[i] - mx, poly && i < (len & ~7));
+    yr[i] = e;
+    sum += e;
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.f / sum;
+  for (int i = lane; i < len; i += 64) yr[i] *= inv;  // each lane re-reads what it wrote itself
+}
+
+// ---- top-k over the last axis, one wave per row -------------------------------------------------------------------------
+// Selection by repeated wave-wide extreme: round r takes the best element that comes after the one taken in round r-1
+// in the order (value descending [ascending for smallest], index ascending).  Equal values are taken lowest index
+// first (the reference's order among equal values is whatever its heap and std::sort leave).
+struct KeyIdx {
+  float v;
+  int i;
+};
+__device__ __forceinline__ bool comes_before(float va, int ia, float vb, int ib, bool largest) {
+  if (va != vb) return largest ? va > vb : va < vb;
+  return ia < ib;
+}
+__device__ __forceinline__ KeyIdx wave_best(KeyIdx k, bool largest) {
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const float ov = __shfl_xor(k.v, off, 64);
+    const int oi = __shfl_xor(k.i, off, 64);
+    if (oi >= 0 && (k.i < 0 || comes_before(ov, oi, k.v, k.i, largest))) {
+      k.v = ov;
+      k.i = oi;
+    }
+  }
+  return k;
+}
+// rows of `vals` may live in global memory or in LDS; out arrays are written by lane 0.  sorted == 0: by index.
+__device__ __forceinline__ void wave_topk(const float* vals, int len, int k, bool largest, bool sorted, float* out_v, int* out_i,
+                                          int lane) {
+  float pv = 0.f;
+  int pi = -1;  // previous pick
+  for (int r = 0; r < k; r++) {
+    KeyIdx best{0.f, -1};
+    for (int i = lane; i < len; i += 64) {
+      const float v = vals[i];
+      const bool after_prev = pi < 0 || comes_before(pv, pi, v, i, largest);
+      if (after_prev && (best.i < 0 || comes_before(v, i, best.v, best.i, largest))) {
+        best.v = v;
+        best.i = i;
+      }
+    }
+    best = wave_best(best, largest);
+    pv = best.v;
+    pi = best.i;
+    if (lane == 0) {
+      out_v[r] = best.v;
+      out_i[r] = best.i;
+    }
+  }
+  if (!sorted && lane == 0) {  // by index: insertion sort of k entries
+    for (int a = 1; a < k; a++) {
+      const float v = out_v[a];
+      const int i = out_i[a];
+      int b = a - 1;
+      while (b >= 0 && out_i[b] > i) {
+        out_v[b + 1] = out_v[b];
+        out_i[b + 1] = out_i[b];
+        b--;
+      }
+      out_v[b + 1] = v;
+      out_i[b + 1] = i;
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void topk_rows_kernel(const float* __restrict__ x, float* __restrict__ values, int32_t* __restrict__ indices,
+                                                        int64_t rows, int len, int k, int largest, int sorted) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  wave_topk(x + row * len, len, k, largest != 0, sorted != 0, values + row * k, indices + row * k, lane);
+}
+
+// ---- MoE gate: logits = x . W^T (fp32), softmax, top-k, optional normalisation ------------------------------------------
+// A workgroup of four waves takes four tokens: the tokens' activations sit in LDS, every wave walks a quarter of the
+// experts (16-byte loads along H, the four tokens share each weight load), then wave t finishes token t.
+struct GateArgs {
+  const void* x;
+  const float* w;  // [E, H]
+  int32_t* ids;    // [M, k]
+  float* weights;  // [M, k]
+  float* scores;   // [M, E] or null
+  int64_t M;
+  int H, E, k, norm, exp_accurate;
+};
+constexpr int GATE_TOK = 4;
+template <int XT>
+__global__ __launch_bounds__(256) void moe_gate_kernel(GateArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* s_x = reinterpret_cast<float*>(smem);     // [GATE_TOK][H]
+  float* s_logit = s_x + (size_t)GATE_TOK * a.H;   // [GATE_TOK][E]
+  float* s_tv = s_logit + (size_t)GATE_TOK * a.E;  // [GATE_TOK][k]
+  int* s_ti = reinterpret_cast<int*>(s_tv + (size_t)GATE_TOK * a.k);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t tok0 = (int64_t)blockIdx.x * GATE_TOK;
+  const int nitems = GATE_TOK * (a.H >> 3);
+  for (int it = tid; it < nitems; it += 256) {
+    const int t = it / (a.H >> 3), c = it - t * (a.H >> 3);
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (tok0 + t < a.M) {
+      Item8<XT> r;
+      item_load<XT>(a.x, (tok0 + t) * a.H + (int64_t)c * 8, r);
+      item_to_f32<XT>(r, v);
+    }
+    f32x4* dst = reinterpret_cast<f32x4*>(s_x + (size_t)t * a.H + c * 8);
+    dst[0] = f32x4{v[0], v[1], v[2], v[3]};
+    dst[1] = f32x4{v[4], v[5], v[6], v[7]};
+  }
+  __syncthreads();
+  for (int e = wave; e < a.E; e += 4) {
+    float acc[GATE_TOK] = {0.f, 0.f, 0.f, 0.f};
+    const f32x4* wr = reinterpret_cast<const f32x4*>(a.w + (size_t)e * a.H);
+    for (int c = lane; c < (a.H >> 2); c += 64) {
+      const f32x4 wv = wr[c];
+#pragma unroll
+      for (int t = 0; t < GATE_TOK; t++) {
+        const f32x4 xv = reinterpret_cast<const f32x4*>(s_x + (size_t)t * a.H)[c];
+        acc[t] = fmaf(xv.x, wv.x, acc[t]);
+        acc[t] = fmaf(xv.y, wv.y, acc[t]);
+        acc[t] = fmaf(xv.z, wv.z, acc[t]);
+        acc[t] = fmaf(xv.w, wv.w, acc[t]);
+      }
+    }
+#pragma unroll
+    for (int t = 0; t < GATE_TOK; t++) {
+      const float s = wave_sum(acc[t]);
+      if (lane == 0) s_logit[t * a.E + e] = s;
+    }
+  }
+  __syncthreads();
+  const int64_t tok = tok0 + wave;
+  if (tok >= a.M) return;
+  float* lg = s_logit + wave * a.E;
+  const bool poly = a.E > 16 && !a.exp_accurate;
+  float mx = -3.402823466e+38f;
+  for (int i = lane; i < a.E; i += 64) mx = fmaxf(mx, lg[i]);
+  mx = wave_max(mx);
+  float sum = 0.f;
+  for (int i = lane; i < a.E; i += 64) {
+    const float ex = softmax_exp(lg[i] - mx, poly && i < (a.E & ~7));
+    lg[i] = ex;
+    sum += ex;
+  }
+  sum = wave_sum(sum);
+  const float inv = 1.f / sum;
+  for (int i = lane; i < a.E; i += 64) {
+    const float p = lg[i] * inv;
+    lg[i] = p;
+    if (a.scores) a.scores[tok * a.E + i] = p;
+  }
+  // LDS writes of this wave are read back by other lanes of the same wave only
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  wave_topk(lg, a.E, a.k, true, false, s_tv + wave * a.k, s_ti + wave * a.k, lane);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  // topk(..., largest = true, sorted = false): by index; then weight / sum(weights) in index order
+  float tsum = 0.f;
+  for (int r = 0; r < a.k; r++) tsum += s_tv[wave * a.k + r];
+  for (int r = lane; r < a.k; r += 64) {
+    const float wv = s_tv[wave * a.k + r];
+    a.weights[tok * a.k + r] = a.norm ? wv / tsum : wv;
+    a.ids[tok * a.k + r] = s_ti[wave * a.k + r];
+  }
+}
+
+}  // namespace mllmhip
+
+using namespace mllmhip;
+
+static int g_exp_accurate = 0;
+MLLM_API int mllm_hip_set_exp_mode(int accurate) {
+  if (accurate != 0 && accurate != 1) return MLLM_HIP_E_BADARG;
+  g_exp_accurate = accurate;
+  return 0;
+}
+
+static bool dtype_ok(int t) { return t == MLLM_HIP_F32 || t == MLLM_HIP_BF16; }
+static bool al16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+// image argument checks shared by the producers: rows <= 8, D a multiple of 32
+static int make_image(void* q_image, int64_t rows, int64_t D, int act_scale_mode, QImage& q) {
+  q = QImage{nullptr, 0, 0, 0};
+  if (!q_image) return 0;
+  if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
+  if (rows < 1 || rows > 8 || D % QK) return MLLM_HIP_E_SHAPE;
+  if (!al16(q_image)) return MLLM_HIP_E_ALIGN;
+  q.base = reinterpret_cast<unsigned char*>(q_image);
+  q.MT = rows <= 1 ? 1 : (rows <= 2 ? 2 : (rows <= 4 ? 4 : 8));
+  q.nb = (int)(D / QK);
+  q.x86_scale = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
+  return 0;
+}
+
+MLLM_API int mllm_hip_rmsnorm(const void* x, int dtype, const float* weight, void* y, int64_t rows, int64_t D, float epsilon,
+                              int add_unit_offset, void* q_image, int act_scale_mode, void* stream) {
+  if (!x || !weight || !y || !dtype_ok(dtype) || rows <= 0 || D <= 0) return MLLM_HIP_E_BADARG;
+  if (D % 8 || D > 8 * 256 * 8 || rows > 0x7fffffff) return MLLM_HIP_E_SHAPE;
+  if (!al16(x) || !al16(y) || !al16(weight)) return MLLM_HIP_E_ALIGN;
+  RmsArgs a{x, weight, y, rows, (int)D, epsilon, add_unit_offset, {}};
+  int rc = make_image(q_image, rows, D, act_scale_mode, a.img);
+  if (rc) return rc;
+  const unsigned grid = (unsigned)(a.img.base ? a.img.MT : rows);
+  const int ni = (int)((D / 8 + 255) / 256);
+  hipStream_t st = (hipStream_t)stream;
+#define RMS(XT_, NI_) hipLaunchKernelGGL((rmsnorm_kernel<XT_, NI_>), dim3(grid), dim3(256), 0, st, a)
+#define RMS_T(XT_)        \
+  if (ni <= 1) RMS(XT_, 1); \
+  else if (ni <= 2) RMS(XT_, 2); \
+  else if (ni <= 4) RMS(XT_, 4); \
+  else RMS(XT_, 8)
+  if (dtype == MLLM_HIP_F32) {
+    RMS_T(MLLM_HIP_F32);
+  } else {
+    RMS_T(MLLM_HIP_BF16);
+  }
+#undef RMS_T
+#undef RMS
+  return (int)hipGetLastError();
+}
+
+template <int OP>
+static int launch_elementwise(const void* a_, const void* b_, void* y, int dtype, int64_t rows, int64_t D, void* q_image,
+                              int act_scale_mode, void* stream) {
+  if (!a_ || (OP != EW_SILU && !b_) || !y || !dtype_ok(dtype) || rows <= 0 || D <= 0) return MLLM_HIP_E_BADARG;
+  if (D % 8 || D > 0x7fffffff) return MLLM_HIP_E_SHAPE;
+  if (!al16(a_) || !al16(b_) || !al16(y)) return MLLM_HIP_E_ALIGN;
+  EwArgs a{a_, b_, y, rows, (int)D, g_exp_accurate, {}};
+  int rc = make_image(q_image, rows, D, act_scale_mode, a.img);
+  if (rc) return rc;
+  const int64_t total_rows = a.img.base ? a.img.MT : rows;
+  const int64_t items = total_rows * (D / 8);
+  if ((items + 255) / 256 > 0x7fffffff) return MLLM_HIP_E_SHAPE;
+  const unsigned grid = (unsigned)((items + 255) / 256);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MLLM_HIP_F32)
+    hipLaunchKernelGGL((elementwise_kernel<MLLM_HIP_F32, OP>), dim3(grid), dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL((elementwise_kernel<MLLM_HIP_BF16, OP>), dim3(grid), dim3(256), 0, st, a);
+  return (int)hipGetLastError();
+}
+
+MLLM_API int mllm_hip_silu(const void* x, void* y, int dtype, int64_t n, void* stream) {
+  if (n <= 0 || n % 8) return n <= 0 ? MLLM_HIP_E_BADARG : MLLM_HIP_E_SHAPE;
+  return launch_elementwise<EW_SILU>(x, nullptr, y, dtype, n / 8, 8, nullptr, 0, stream);
+}
+MLLM_API int mllm_hip_add(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream) {
+  if (n <= 0 || n % 8) return n <= 0 ? MLLM_HIP_E_BADARG : MLLM_HIP_E_SHAPE;
+  return launch_elementwise<EW_ADD>(a, b, y, dtype, n / 8, 8, nullptr, 0, stream);
+}
+MLLM_API int mllm_hip_mul(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream) {
+  if (n <= 0 || n % 8) return n <= 0 ? MLLM_HIP_E_BADARG : MLLM_HIP_E_SHAPE;
+  return launch_elementwise<EW_MUL>(a, b, y, dtype, n / 8, 8, nullptr, 0, stream);
+}
+MLLM_API int mllm_hip_silu_mul(const void* gate, const void* up, void* y, int dtype, int64_t rows, int64_t D, void* q_image,
+                               int act_scale_mode, void* stream) {
+  return launch_elementwise<EW_SILU_MUL>(gate, up, y, dtype, rows, D, q_image, act_scale_mode, stream);
+}
+
+MLLM_API int mllm_hip_softmax(const float* x, float* y, int64_t rows, int64_t len, void* stream) {
+  if (!x || !y || rows <= 0 || len <= 0) return MLLM_HIP_E_BADARG;
+  if (len > 0x7fffffff || (rows + 3) / 4 > 0x7fffffff) return MLLM_HIP_E_SHAPE;
+  hipLaunchKernelGGL(softmax_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream, x, y, rows, (int)len,
+                     g_exp_accurate);
+  return (int)hipGetLastError();
+}
+
+MLLM_API int mllm_hip_topk(const float* x, float* values, int32_t* indices, int64_t rows, int64_t len, int k, int largest,
+                           int sorted, void* stream) {
+  if (!x || !values || !indices || rows <= 0 || len <= 0) return MLLM_HIP_E_BADARG;
+  if (k < 1 || k > len || len > 0x7fffffff || (rows + 3) / 4 > 0x7fffffff) return MLLM_HIP_E_SHAPE;
+  hipLaunchKernelGGL(topk_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream, x, values, indices, rows,
+                     (int)len, k, largest, sorted);
+  return (int)hipGetLastError();
+}
+
+MLLM_API int mllm_hip_moe_gate(const void* x, int x_dtype, const float* gate_weight, int32_t* topk_ids, float* topk_weights,
+                               float* scores, int64_t M, int64_t H, int64_t E, int k, int norm_topk_prob, void* stream) {
+  if (!x || !gate_weight || !topk_ids || !topk_weights || !dtype_ok(x_dtype) || M <= 0 || H <= 0 || E <= 0) return MLLM_HIP_E_BADARG;
+  if (k < 1 || k > E || H % 8 || (M + GATE_TOK - 1) / GATE_TOK > 0x7fffffff) return MLLM_HIP_E_SHAPE;
+  if (!al16(x) || !al16(gate_weight)) return MLLM_HIP_E_ALIGN;
+  const size_t lds = ((size_t)GATE_TOK * H + (size_t)GATE_TOK * E + (size_t)2 * GATE_TOK * k) * 4;
+  if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
+  GateArgs a{x, gate_weight, topk_ids, topk_weights, scores, M, (int)H, (int)E, k, norm_topk_prob, g_exp_accurate};
+  const unsigned grid = (unsigned)((M + GATE_TOK - 1) / GATE_TOK);
+  hipStream_t st = (hipStream_t)stream;
+  auto launch = [&](auto kern) -> int {
+    if (lds > 64 * 1024)
+      HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a);
+    return (int)hipGetLastError();
+  };
+  return x_dtype == MLLM_HIP_F32 ? launch(moe_gate_kernel<MLLM_HIP_F32>) : launch(moe_gate_kernel<MLLM_HIP_BF16>);
+}

@@ -5,7 +5,7 @@
 // Reference semantics:
 //   expert loop           mllm/models/qwen3_moe/modeling_qwen3_moe_fa2.hpp:175-238 (moeInfer), :98-100 (Qwen3MoeMLP)
 //   each Linear           mllm/backends/cpu/kernels/common/ggml/matmul.cpp:148-206 (Q8_0 activations, block dots)
-//   SiLU                  mllm/backends/cpu/kernels/x86/silu.cpp:41   x / (1 + exp(-x))
+//   SiLU                  mllm/backends/cpu/kernels/x86/silu.cpp:16-27   x * (1 / (1 + exp_poly(-x))), math.hpp:19-72
 // The per-block int32 sums come from v_mfma_i32_32x32x32_i8 (K = 32 = one quantization block per instruction, exact);
 // they are scaled and accumulated in fp32 on the vector ALU.  Tokens are the MFMA rows, weight rows the MFMA columns, so
 // a lane owns one output channel: its weight scale is a scalar per block and stores are contiguous across lanes.
@@ -176,7 +176,8 @@ __device__ __forceinline__ v4i weight_operand(const u32x4& q, int hi) {
   }
 }
 
-__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+// the SiLU operator runs over whole [rows, I] tensors with I a multiple of 32: always the vector form
+__device__ __forceinline__ float silu_f(float x) { return x * (1.0f / (1.0f + exp_poly(-x))); }
 
 constexpr int PLANE = TOK_TILE * 16 + 16;          // LDS bytes of one (block, half) plane of activation codes, padded
 constexpr int SA_BYTES = KCH * 2 * PLANE;

@@ -44,6 +44,30 @@ __device__ __forceinline__ uint16_t x86_scale_bits(uint16_t b) {
   return (uint16_t)(uint32_t)(float)(_Float16)(float)(uint32_t)b;
 }
 
+// ---- exp as the reference's x86 kernels compute it ------------------------------------------------------------
+// vexpq_fast_f32, mllm/backends/cpu/kernels/x86/math.hpp:19-72 (Cephes polynomial; fmaf where the reference uses MulAdd).
+// As the reference writes the argument reduction (the full ln 2 and the Cephes correction term both subtracted), the
+// result is exp(x) * exp(n * 2.1219444e-4), n = round(x / ln 2): restated as written, not repaired.
+__device__ __forceinline__ float exp_poly(float x) {
+  x = fminf(fmaxf(x, -88.3762626647949f), 88.3762626647949f);
+  float fx = fmaf(x, 1.44269504088896341f, 0.5f);
+  const float tmp = floorf(fx);
+  fx = tmp - (tmp > fx ? 1.0f : 0.0f);
+  const float t2 = fx * 0.693147180559945309f;
+  const float z0 = fx * -2.12194440e-4f;
+  x = (x - t2) - z0;
+  const float z = x * x;
+  float y = 1.9875691500E-4f;
+  y = fmaf(y, x, 1.3981999507E-3f);
+  y = fmaf(y, x, 8.3334519073E-3f);
+  y = fmaf(y, x, 4.1665795894E-2f);
+  y = fmaf(y, x, 1.6666665459E-1f);
+  y = fmaf(y, x, 5.0000001201E-1f);
+  y = fmaf(y, z, x);
+  y = y + 1.0f;
+  const int n = (int)fx + 0x7f;
+  return y * __int_as_float(n << 23);
+}
 // ---- wavefront reductions with DPP (64-wide waves; a DPP row is 16 lanes) -------------------------------
 template <int CTRL>
 __device__ __forceinline__ float dpp_f(float v) {

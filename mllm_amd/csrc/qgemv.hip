@@ -324,10 +324,11 @@ MLLM_API size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K) {
   return (size_t)8 * (K / QK) * 40;
 }
 
-MLLM_API int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,
-                                             int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
+// x_kind: MLLM_HIP_F32 / MLLM_HIP_BF16 activations, or MLLM_HIP_Q8_IMAGE: their quantized image (act_scale_mode unused)
+static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual, const void* x,
+                           int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
   if (nparts < 1 || nparts > GEMV_MAX_PARTS || !parts) return MLLM_HIP_E_BADARG;
-  if (!x || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16)) return MLLM_HIP_E_BADARG;
+  if (!x || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16 && x_dtype != MLLM_HIP_Q8_IMAGE)) return MLLM_HIP_E_BADARG;
   if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
   if (M < 1 || M > 8) return MLLM_HIP_E_SHAPE;
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
@@ -339,6 +340,7 @@ MLLM_API int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_h
     if (!parts[p].y) return MLLM_HIP_E_BADARG;
     a.part[p].w = packed_view(wtype, parts[p].packed, parts[p].N, K);
     a.part[p].bias = parts[p].bias;
+    a.part[p].residual = residual ? residual[p] : nullptr;
     a.part[p].y = parts[p].y;
     a.part[p].N = (int)parts[p].N;
     nmax += parts[p].N;
@@ -352,6 +354,10 @@ MLLM_API int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_h
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8));
   GemvShape s = pick_shape(MT, nmax, a.nb);
   hipStream_t st = (hipStream_t)stream;
+  if (x_dtype == MLLM_HIP_Q8_IMAGE) {
+    if (!g_tune_NW) s.NW = a.nb >= 256 ? 8 : 4;
+    return wtype == MLLM_HIP_Q4_0 ? launch_gemv_q4_preq(a, MT, s, st) : launch_gemv_q8_preq(a, MT, s, st);
+  }
   if (workspace && M >= 3) {
     // several rows: quantize once for all workgroups, then the GEMV copies the quantized image instead of quantizing
     const int mnb = MT * a.nb;
@@ -364,6 +370,17 @@ MLLM_API int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_h
   if (wtype == MLLM_HIP_Q4_0)
     return x_dtype == MLLM_HIP_F32 ? launch_gemv_q4_f32(a, MT, s, st) : launch_gemv_q4_bf16(a, MT, s, st);
   return x_dtype == MLLM_HIP_F32 ? launch_gemv_q8_f32(a, MT, s, st) : launch_gemv_q8_bf16(a, MT, s, st);
+}
+
+MLLM_API int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,
+                                             int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
+  if (x_dtype == MLLM_HIP_Q8_IMAGE) return MLLM_HIP_E_BADARG;
+  return gemv_multi_impl(wtype, nparts, parts, nullptr, x, x_dtype, M, K, act_scale_mode, workspace, stream);
+}
+
+MLLM_API int mllm_hip_linear_q_gemv_fused(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual,
+                                          const void* x, int x_kind, int M, int64_t K, int act_scale_mode, void* stream) {
+  return gemv_multi_impl(wtype, nparts, parts, residual, x, x_kind, M, K, act_scale_mode, nullptr, stream);
 }
 
 MLLM_API int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,

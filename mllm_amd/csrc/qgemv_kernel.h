@@ -21,6 +21,7 @@ constexpr int GEMV_MAX_PARTS = 4;
 struct GemvPart {
   PackedView w;
   const float* bias;
+  const float* residual;  // fp32 [M][N] added to the result (may be y itself), or null
   float* y;
   int N;
 };
@@ -191,7 +192,7 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
   // item `it` = eight elements: block it/4, lanes of a quad share a block.  Addresses are clamped, validity is applied
   // when the values are used, so no branch separates these loads from the ones below.
   const int valid_items = a.M * nb * 4;
-  const int img_chunks = mnb * 5 / 2;  // 16-byte pieces of the quantized image (40 bytes per block)
+  const int img_chunks = (mnb * 5 + 1) / 2;  // 16-byte pieces of the quantized image (40 bytes per block; the buffer is sized for 8 rows)
   XRaw<XT> raw0, raw1;
   if (XT == GEMV_PREQ) {
     raw0.r[0] = reinterpret_cast<const u32x4*>(a.x)[min(tid, img_chunks - 1)];
@@ -338,7 +339,12 @@ __global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
     for (int m = 0; m < MT; m++) {
       float v = group_sum<G>(acc[r][m]);
       const int64_t row = row0 + r;
-      if (c0 == 0 && row < N && m < a.M) pt.y[(int64_t)m * N + row] = pt.bias ? pt.bias[row] + v : v;
+      if (c0 == 0 && row < N && m < a.M) {
+        // Linear first (bias + dot), then the residual: the order of the two operators it replaces
+        if (pt.bias) v = pt.bias[row] + v;
+        if (pt.residual) v = v + pt.residual[(int64_t)m * N + row];
+        pt.y[(int64_t)m * N + row] = v;
+      }
     }
 }
 
@@ -388,9 +394,7 @@ static int launch_gemv_m(const GemvArgs& a, GemvShape s, hipStream_t st) {
 // one instance per (weight type, activation type), each in its own translation unit (compiled in parallel)
 template <int WT, int XT>
 int launch_gemv(const GemvArgs& a, int MT, GemvShape s, hipStream_t st) {
-  if constexpr (XT == GEMV_PREQ) {  // only used from three activation rows on
-    return MT == 4 ? launch_gemv_m<WT, XT, 4>(a, s, st) : launch_gemv_m<WT, XT, 8>(a, s, st);
-  } else {
+  {
     switch (MT) {
       case 1: return launch_gemv_m<WT, XT, 1>(a, s, st);
       case 2: return launch_gemv_m<WT, XT, 2>(a, s, st);

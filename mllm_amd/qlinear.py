@@ -3,6 +3,8 @@
 torch is used for device memory and the current stream only; every computation is a call into
 libmllm_hip_qlinear.so.  Enumerations mirror include/mllm_hip_qlinear.h.
 """
+import ctypes as C
+
 import torch
 
 from . import _lib
@@ -108,6 +110,36 @@ def linear_q_gemv_multi(ws, x, biases=None, act_scale_mode=SCALE_X86_REF, outs=N
     _lib.check(_lib.lib().mllm_hip_linear_q_gemv_multi_ws(ws[0].wtype, len(ws), parts, x.data_ptr(), _xdtype(x), M, K,
                                                           act_scale_mode, _p(workspace), _stream()),
                "mllm_hip_linear_q_gemv_multi_ws")
+    return outs
+
+
+Q8_IMAGE = 2  # MLLM_HIP_Q8_IMAGE
+
+
+def linear_q_gemv_fused(ws, x, M=None, biases=None, residuals=None, act_scale_mode=SCALE_X86_REF, outs=None, image=False):
+    """The decode GEMV with its neighbours folded in: residuals[i] (fp32 [M, N], may be outs[i]) is added to part i, and
+    with image=True `x` is the Q8_0 image a producer (rmsnorm / silu_mul with want_image) wrote for M rows."""
+    assert 1 <= len(ws) <= 4 and x.is_cuda and x.is_contiguous()
+    K = ws[0].K
+    if not image:
+        assert x.dim() == 2 and x.shape[1] == K
+        M = x.shape[0]
+    assert M is not None
+    if outs is None:
+        outs = [torch.empty((M, w.N), dtype=torch.float32, device="cuda") for w in ws]
+    parts = (_lib.GemvPart * len(ws))()
+    res = (C.c_void_p * len(ws))()
+    for i, w in enumerate(ws):
+        assert w.K == K and w.wtype == ws[0].wtype
+        b = biases[i] if biases is not None else None
+        parts[i] = _lib.GemvPart(w.ptr, b.data_ptr() if b is not None else None, outs[i].data_ptr(), w.N)
+        r = residuals[i] if residuals is not None else None
+        if r is not None:
+            assert r.dtype == torch.float32 and r.is_contiguous() and tuple(r.shape) == (M, w.N)
+        res[i] = r.data_ptr() if r is not None else None
+    _lib.check(_lib.lib().mllm_hip_linear_q_gemv_fused(ws[0].wtype, len(ws), parts, res if residuals is not None else None,
+                                                       x.data_ptr(), Q8_IMAGE if image else _xdtype(x), M, K, act_scale_mode,
+                                                       _stream()), "mllm_hip_linear_q_gemv_fused")
     return outs
 
 
@@ -366,3 +398,86 @@ def moe_route(topk_ids, E):
     _lib.check(L.mllm_hip_moe_route(topk_ids.data_ptr(), T, E, k, counts.data_ptr(), offsets.data_ptr(), sidx.data_ptr(),
                                     ws.data_ptr(), _stream()), "mllm_hip_moe_route")
     return counts, offsets, sidx
+
+
+# ----------------------------------------------------------------------------- the operators around Linear in a layer
+def rmsnorm(x, weight, eps, add_unit_offset=False, want_image=False, act_scale_mode=SCALE_X86_REF, out=None):
+    """x [..., D] fp32 or bf16, weight fp32 [D].  want_image (rows <= 8): also returns the Q8_0 image of the result for
+    linear_q_gemv_fused(..., image=True)."""
+    assert x.is_cuda and x.is_contiguous() and weight.dtype == torch.float32 and weight.is_contiguous()
+    D = x.shape[-1]
+    rows = x.numel() // D
+    y = out if out is not None else torch.empty_like(x)
+    img = gemv_workspace(rows, D) if want_image else None
+    _lib.check(_lib.lib().mllm_hip_rmsnorm(x.data_ptr(), _xdtype(x), weight.data_ptr(), y.data_ptr(), rows, D, eps,
+                                           int(add_unit_offset), _p(img), act_scale_mode, _stream()), "mllm_hip_rmsnorm")
+    return (y, img) if want_image else y
+
+
+def _binary(fn, name, a, b):
+    assert a.is_cuda and a.is_contiguous() and b.is_contiguous() and a.shape == b.shape and a.dtype == b.dtype
+    y = torch.empty_like(a)
+    _lib.check(fn(a.data_ptr(), b.data_ptr(), y.data_ptr(), _xdtype(a), a.numel(), _stream()), name)
+    return y
+
+
+def add(a, b):
+    return _binary(_lib.lib().mllm_hip_add, "mllm_hip_add", a, b)
+
+
+def mul(a, b):
+    return _binary(_lib.lib().mllm_hip_mul, "mllm_hip_mul", a, b)
+
+
+def silu(x):
+    assert x.is_cuda and x.is_contiguous()
+    y = torch.empty_like(x)
+    _lib.check(_lib.lib().mllm_hip_silu(x.data_ptr(), y.data_ptr(), _xdtype(x), x.numel(), _stream()), "mllm_hip_silu")
+    return y
+
+
+def silu_mul(gate, up, want_image=False, act_scale_mode=SCALE_X86_REF, out=None):
+    """silu(gate) * up over [rows, D]; want_image as for rmsnorm."""
+    assert gate.is_cuda and gate.is_contiguous() and up.is_contiguous() and gate.shape == up.shape and gate.dtype == up.dtype
+    D = gate.shape[-1]
+    rows = gate.numel() // D
+    y = out if out is not None else torch.empty_like(gate)
+    img = gemv_workspace(rows, D) if want_image else None
+    _lib.check(_lib.lib().mllm_hip_silu_mul(gate.data_ptr(), up.data_ptr(), y.data_ptr(), _xdtype(gate), rows, D, _p(img),
+                                            act_scale_mode, _stream()), "mllm_hip_silu_mul")
+    return (y, img) if want_image else y
+
+
+def set_exp_mode(accurate):
+    _lib.check(_lib.lib().mllm_hip_set_exp_mode(int(accurate)), "mllm_hip_set_exp_mode")
+
+
+def softmax(x):
+    assert x.is_cuda and x.is_contiguous() and x.dtype == torch.float32
+    n = x.shape[-1]
+    y = torch.empty_like(x)
+    _lib.check(_lib.lib().mllm_hip_softmax(x.data_ptr(), y.data_ptr(), x.numel() // n, n, _stream()), "mllm_hip_softmax")
+    return y
+
+
+def topk(x, k, largest=True, sorted=True):
+    assert x.is_cuda and x.is_contiguous() and x.dtype == torch.float32
+    n = x.shape[-1]
+    v = torch.empty(x.shape[:-1] + (k,), dtype=torch.float32, device="cuda")
+    i = torch.empty(x.shape[:-1] + (k,), dtype=torch.int32, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_topk(x.data_ptr(), v.data_ptr(), i.data_ptr(), x.numel() // n, n, k, int(largest),
+                                        int(sorted), _stream()), "mllm_hip_topk")
+    return v, i
+
+
+def moe_gate(x, gate_weight, k, norm_topk_prob=True, want_scores=False):
+    """x [M, H] fp32 or bf16, gate_weight fp32 [E, H] -> (ids int32 [M, k], weights fp32 [M, k][, scores fp32 [M, E]])"""
+    assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and gate_weight.dtype == torch.float32 and gate_weight.is_contiguous()
+    M, H = x.shape
+    E = gate_weight.shape[0]
+    ids = torch.empty((M, k), dtype=torch.int32, device="cuda")
+    wt = torch.empty((M, k), dtype=torch.float32, device="cuda")
+    sc = torch.empty((M, E), dtype=torch.float32, device="cuda") if want_scores else None
+    _lib.check(_lib.lib().mllm_hip_moe_gate(x.data_ptr(), _xdtype(x), gate_weight.data_ptr(), ids.data_ptr(), wt.data_ptr(),
+                                            _p(sc), M, H, E, k, int(norm_topk_prob), _stream()), "mllm_hip_moe_gate")
+    return (ids, wt, sc) if want_scores else (ids, wt)

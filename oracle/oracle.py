@@ -46,6 +46,8 @@ def lib():
         L.orc_vec_dot.restype = C.c_float
         L.orc_silu.restype = C.c_float
         L.orc_silu.argtypes = [C.c_float]
+        L.orc_exp_poly.restype = C.c_float
+        L.orc_exp_poly.argtypes = [C.c_float]
         L.orc_linear_q.restype = C.c_int
         L.orc_w4a16_gemm.restype = C.c_int
         L.orc_moe_ffn.restype = C.c_int
@@ -272,3 +274,63 @@ def ref_quantize_rows_q4_0(x):
     for n in range(N):
         ref().ref_quantize_row_q4_0(_p(x[n], C.c_float), _p(out[n], C.c_uint8), C.c_int(K))
     return out
+
+
+# ----------------------------------------------------------------------------- neighbours of Linear in a decoder layer
+def exp_poly(x):
+    """vexpq_fast_f32 (mllm/backends/cpu/kernels/x86/math.hpp:19-72), elementwise"""
+    x = np.ascontiguousarray(x, np.float32)
+    L = lib()
+    return np.array([L.orc_exp_poly(float(v)) for v in x.ravel()], np.float32).reshape(x.shape)
+
+
+def silu(x):
+    """silu_fp32 over the flattened tensor (x86/silu.cpp:16-56)"""
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.empty_like(x)
+    lib().orc_silu_array(_p(x, C.c_float), _p(y, C.c_float), C.c_int64(x.size))
+    return y
+
+
+def rmsnorm(x, w, eps, add_unit_offset=False):
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    D = x.shape[-1]
+    assert w.shape == (D,)
+    y = np.empty_like(x)
+    lib().orc_rmsnorm(_p(x, C.c_float), _p(w, C.c_float), _p(y, C.c_float), C.c_int64(x.size // D), C.c_int(D),
+                      C.c_float(eps), C.c_int(int(add_unit_offset)))
+    return y
+
+
+def softmax(x):
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.empty_like(x)
+    n = x.shape[-1]
+    lib().orc_softmax_rows(_p(x, C.c_float), _p(y, C.c_float), C.c_int64(x.size // n), C.c_int(n))
+    return y
+
+
+def topk(x, k, largest=True, sorted=True):
+    x = np.ascontiguousarray(x, np.float32)
+    n = x.shape[-1]
+    shape = x.shape[:-1] + (k,)
+    v = np.empty(shape, np.float32)
+    i = np.empty(shape, np.int32)
+    lib().orc_topk_rows(_p(x, C.c_float), _p(v, C.c_float), _p(i, C.c_int32), C.c_int64(x.size // n), C.c_int(n), C.c_int(k),
+                        C.c_int(int(largest)), C.c_int(int(sorted)))
+    return v, i
+
+
+def moe_gate(x, w, k, norm=True):
+    """returns (ids int32 [M,k], weights fp32 [M,k], scores fp32 [M,E])"""
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    M, H = x.shape
+    E = w.shape[0]
+    ids = np.empty((M, k), np.int32)
+    wt = np.empty((M, k), np.float32)
+    sc = np.empty((M, E), np.float32)
+    lib().orc_moe_gate(_p(x, C.c_float), _p(w, C.c_float), _p(ids, C.c_int32), _p(wt, C.c_float), _p(sc, C.c_float), C.c_int64(M),
+                       C.c_int(H), C.c_int(E), C.c_int(k), C.c_int(int(norm)))
+    return ids, wt, sc

@@ -26,6 +26,13 @@
  *                                            parity unpinned by the reference; pinned here by the closed forms its tests
  *                                            state, brute force in int64/float64 and special cases
  *   orc_moe_ffn                              composition + permutation invariance + hand-built micro case
+ *   orc_exp_poly / orc_silu_array / orc_rmsnorm / orc_softmax_rows / orc_topk_rows / orc_moe_gate
+ *                                            the x86 kernels they restate need Highway, which the reference does not
+ *                                            vendor: unbuildable here.  Pinned by closed forms in float64 (exp_poly
+ *                                            against exp(x) * exp(n * 2.1219444e-4), which is what the reference's
+ *                                            reduction constants produce; rmsnorm, softmax, silu against their
+ *                                            definitions), by numpy sort for top-k, and by the properties the reference's
+ *                                            own TopK test checks (shapes of tests/cpu/KernelTest.cpp:686, descending order)
  */
 #include <math.h>
 #include <stdint.h>
@@ -401,11 +408,172 @@ ORC_API void orc_w8a8_gemm(const int8_t* xq, const float* x_scale, const int8_t*
  * MoE expert FFN over expert-sorted tokens.
  *   Qwen3MoE::moeInfer      mllm/models/qwen3_moe/modeling_qwen3_moe_fa2.hpp:175-238
  *   Qwen3MoeMLP::forward    :98-100     down(silu(gate(x)) * up(x)), every Linear = orc_linear_q
- *   SiLU scalar form        mllm/backends/cpu/kernels/x86/silu.cpp:41   x / (1 + exp(-x))
+ *   SiLU                    mllm/backends/cpu/kernels/x86/silu.cpp:16-56 (orc_silu_array, declared below)
  * x fp32 [T][H]; topk_ids int32 [T][k]; topk_w fp32 [T][k]; expert e weights: Wg,Wu blocks [I][H/32], Wd blocks [H][I/32],
  * stored per expert contiguously.  y fp32 [T][H] = sum_j topk_w[t][j] * expert_{ids[t][j]}(x[t]), j ascending.
  * ---------------------------------------------------------------------------------------------- */
 ORC_API float orc_silu(float x) { return x / (1.0f + expf(-x)); }
+ORC_API void orc_silu_array(const float* x, float* y, int64_t len);
+
+/* exp as the x86 kernels compute it: vexpq_fast_f32, mllm/backends/cpu/kernels/x86/math.hpp:19-72, one lane of it.
+ * MulAdd is a fused multiply-add on the AVX2/FMA targets the reference builds for.  Note the argument reduction as the
+ * reference writes it: C1 is the full ln 2 (std::numbers::ln2_v<float>) and the Cephes correction C2 is still
+ * subtracted, so the reduced argument is off by n * 2.1219444e-4 and the result is exp(x) * exp(n * 2.1219444e-4),
+ * n = floor(x * log2(e) + 0.5).  Restated as written. */
+ORC_API float orc_exp_poly(float x) {
+  x = fminf(fmaxf(x, -88.3762626647949f), 88.3762626647949f);
+  float fx = fmaf(x, 1.44269504088896341f, 0.5f);
+  float tmp = floorf(fx);
+  fx = tmp - (tmp > fx ? 1.0f : 0.0f);
+  float tmp2 = fx * 0.693147180559945309f;
+  float z = fx * -2.12194440e-4f;
+  x = (x - tmp2) - z;
+  z = x * x;
+  float y = 1.9875691500E-4f;
+  y = fmaf(y, x, 1.3981999507E-3f);
+  y = fmaf(y, x, 8.3334519073E-3f);
+  y = fmaf(y, x, 4.1665795894E-2f);
+  y = fmaf(y, x, 1.6666665459E-1f);
+  y = fmaf(y, x, 5.0000001201E-1f);
+  y = fmaf(y, z, x);
+  y = y + 1.0f;
+  int32_t n = (int32_t)fx + 0x7f;
+  return y * u2f((uint32_t)n << 23);
+}
+
+/* silu_fp32, mllm/backends/cpu/kernels/x86/silu.cpp:16-56: whole vectors of 8 floats (AVX2) take
+ * x * (1 / (1 + exp_poly(-x))), the remaining len % 8 elements x / (1 + exp(-x)). */
+ORC_API void orc_silu_array(const float* x, float* y, int64_t len) {
+  int64_t aligned = len - (len % 8);
+  for (int64_t i = 0; i < aligned; i++) y[i] = x[i] * (1.0f / (1.0f + orc_exp_poly(-x[i])));
+  for (int64_t i = aligned; i < len; i++) y[i] = x[i] / (1.0f + expf(-x[i]));
+}
+
+/* rmsnorm_fp32, mllm/backends/cpu/kernels/x86/rmsnorm.cpp:17-52 with vsquare_mean_fp32, math.hpp:75-90:
+ * eight partial sums (AVX2 lanes) over whole vectors, reduced, then the tail; y = x * (w * rms) in whole vectors,
+ * x * rms * w in the tail. */
+ORC_API void orc_rmsnorm(const float* x, const float* w, float* y, int64_t rows, int D, float eps, int add_unit_offset) {
+  for (int64_t r = 0; r < rows; r++) {
+    const float* xr = x + r * D;
+    float* yr = y + r * D;
+    float lanes[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    int i = 0;
+    for (; i + 8 <= D; i += 8)
+      for (int l = 0; l < 8; l++) lanes[l] = lanes[l] + xr[i + l] * xr[i + l];
+    /* hn::ReduceSum on AVX2: pairwise over the lanes */
+    float acc = ((lanes[0] + lanes[4]) + (lanes[2] + lanes[6])) + ((lanes[1] + lanes[5]) + (lanes[3] + lanes[7]));
+    for (; i < D; i++) acc += xr[i] * xr[i];
+    float rms = 1.0f / sqrtf(acc / (float)D + eps);
+    i = 0;
+    for (; i + 8 <= D; i++) {
+      float m = add_unit_offset ? (w[i] + 1.0f) * rms : w[i] * rms;
+      yr[i] = xr[i] * m;
+    }
+    for (; i < D; i++) yr[i] = add_unit_offset ? xr[i] * rms * (w[i] + 1.0f) : xr[i] * rms * w[i];
+  }
+}
+
+/* softmax_v1_fp32 over contiguous rows, mllm/backends/cpu/kernels/x86/softmax.cpp:18-76: rows of at most 16 elements
+ * use expf, longer ones exp_poly on whole vectors of 8 and expf on the tail; the sum runs in 8 lanes. */
+ORC_API void orc_softmax_rows(const float* x, float* y, int64_t rows, int len) {
+  for (int64_t r = 0; r < rows; r++) {
+    const float* xr = x + r * len;
+    float* yr = y + r * len;
+    float mx = -3.402823466e+38f;
+    for (int i = 0; i < len; i++) mx = fmaxf(mx, xr[i]);
+    float sum;
+    if (len <= 16) {
+      sum = 0.f;
+      for (int i = 0; i < len; i++) {
+        yr[i] = expf(xr[i] - mx);
+        sum += yr[i];
+      }
+    } else {
+      float lanes[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      int i = 0;
+      for (; i + 8 <= len; i += 8)
+        for (int l = 0; l < 8; l++) {
+          yr[i + l] = orc_exp_poly(xr[i + l] - mx);
+          lanes[l] += yr[i + l];
+        }
+      sum = ((lanes[0] + lanes[4]) + (lanes[2] + lanes[6])) + ((lanes[1] + lanes[5]) + (lanes[3] + lanes[7]));
+      for (; i < len; i++) {
+        yr[i] = expf(xr[i] - mx);
+        sum += yr[i];
+      }
+    }
+    sum = 1.f / sum;
+    for (int i = 0; i < len; i++) yr[i] *= sum;
+  }
+}
+
+/* topk_impl over the last axis, mllm/backends/cpu/ops/TopKOp.cpp:20-72: a candidate replaces the weakest kept element
+ * only when it is strictly better, the kept set is then ordered by value (sorted) or by index.  The order among EQUAL
+ * values is left to std::priority_queue / std::sort there; here equal values are kept lowest index first and a stable
+ * order is used (tests use rows without ties, plus tie cases checked as sets). */
+ORC_API void orc_topk_rows(const float* x, float* values, int32_t* indices, int64_t rows, int len, int k, int largest,
+                           int sorted) {
+  for (int64_t r = 0; r < rows; r++) {
+    const float* xr = x + r * len;
+    float* v = values + r * k;
+    int32_t* id = indices + r * k;
+    int n = 0;
+    for (int i = 0; i < len; i++) { /* kept set ordered best first (insertion keeps earlier indices ahead on ties) */
+      float c = xr[i];
+      int pos = n;
+      while (pos > 0 && (largest ? c > v[pos - 1] : c < v[pos - 1])) pos--;
+      if (pos >= k) continue;
+      int last = n < k ? n : k - 1;
+      for (int j = last; j > pos; j--) {
+        v[j] = v[j - 1];
+        id[j] = id[j - 1];
+      }
+      v[pos] = c;
+      id[pos] = i;
+      if (n < k) n++;
+    }
+    if (!sorted) { /* by index */
+      for (int a = 1; a < k; a++) {
+        float tv = v[a];
+        int32_t ti = id[a];
+        int b = a - 1;
+        while (b >= 0 && id[b] > ti) {
+          v[b + 1] = v[b];
+          id[b + 1] = id[b];
+          b--;
+        }
+        v[b + 1] = tv;
+        id[b + 1] = ti;
+      }
+    }
+  }
+}
+
+/* MoEGate::forward, mllm/models/qwen3_moe/modeling_qwen3_moe_fa2.hpp:121-139: logits = x . W^T in fp32, softmax, topk
+ * (largest, not sorted: index order), optionally weights / sum(weights).  The fp32 matmul's summation order on the CPU
+ * depends on the BLAS in use; here: sequential fp32 over H. */
+ORC_API void orc_moe_gate(const float* x, const float* w, int32_t* ids, float* weights, float* scores, int64_t M, int H, int E,
+                          int k, int norm) {
+  float* logit = (float*)malloc(sizeof(float) * (size_t)E);
+  float* prob = (float*)malloc(sizeof(float) * (size_t)E);
+  for (int64_t t = 0; t < M; t++) {
+    for (int e = 0; e < E; e++) {
+      float acc = 0.f;
+      for (int h = 0; h < H; h++) acc = fmaf(x[t * H + h], w[(size_t)e * H + h], acc);
+      logit[e] = acc;
+    }
+    orc_softmax_rows(logit, prob, 1, E);
+    if (scores) memcpy(scores + t * E, prob, sizeof(float) * (size_t)E);
+    orc_topk_rows(prob, weights + t * k, ids + t * k, 1, E, k, 1, 0);
+    if (norm) {
+      float s = 0.f;
+      for (int j = 0; j < k; j++) s += weights[t * k + j];
+      for (int j = 0; j < k; j++) weights[t * k + j] = weights[t * k + j] / s;
+    }
+  }
+  free(logit);
+  free(prob);
+}
 
 ORC_API int orc_moe_ffn(const float* x, const int32_t* topk_ids, const float* topk_w, const uint8_t* Wg,
                         const uint8_t* Wu, const uint8_t* Wd, int wtype, float* y, int T, int H, int I, int E, int k,
@@ -433,7 +601,8 @@ ORC_API int orc_moe_ffn(const float* x, const int32_t* topk_ids, const float* to
       }
     orc_linear_q(xe, Wg + e * gu_bytes, wtype, NULL, g, cnt, I, H, scale_mode, NULL, NULL);
     orc_linear_q(xe, Wu + e * gu_bytes, wtype, NULL, u, cnt, I, H, scale_mode, NULL, NULL);
-    for (size_t i = 0; i < (size_t)cnt * I; i++) g[i] = orc_silu(g[i]) * u[i];
+    orc_silu_array(g, g, (int64_t)cnt * I); /* the SiLU operator over the whole [cnt, I] tensor, then the product */
+    for (size_t i = 0; i < (size_t)cnt * I; i++) g[i] = g[i] * u[i];
     orc_linear_q(g, Wd + e * d_bytes, wtype, NULL, o, cnt, H, I, scale_mode, NULL, NULL);
     for (c = 0; c < cnt; c++) memcpy(per + (size_t)rows[c] * H, o + (size_t)c * H, (size_t)H * 4);
     free(rows); free(xe); free(g); free(u); free(o);

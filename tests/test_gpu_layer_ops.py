@@ -1,0 +1,252 @@
+"""GPU parity of the operators around Linear (RMSNorm, SiLU, add, mul, SiLU*up, softmax, top-k, MoE gate) and of the decode
+GEMV with those neighbours folded in (residual in the epilogue, activations handed over as a quantized image).
+
+Bars: fp32 / bf16 outputs rel-L2 <= 1e-3 against the oracle (measured: 1e-7 .. 1e-6, elementwise work is the same fp32
+operation sequence); indices, quantized images and everything derived from stored tensors bit-exact.
+"""
+import numpy as np
+import pytest
+import torch
+
+from mllm_amd import _lib, qlinear as ql, synth
+from oracle import oracle as orc
+from gpu_util import announce, bf16_dev, rel_l2, to_dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def _bf16_round(a):
+    return orc.bf16_bits_to_fp32(orc.fp32_to_bf16_bits(np.asarray(a, np.float32)))
+
+
+def _image_fields(img, M, K):
+    """splits a quantized image into (codes int8 [MT, K], scales fp32 [MT, nb], n8 int32 [MT, nb])"""
+    MT = 1 if M <= 1 else 2 if M <= 2 else 4 if M <= 4 else 8
+    nb = K // 32
+    mnb = MT * nb
+    raw = img.cpu().numpy()
+    lo = raw[:mnb * 16].view(np.int8).reshape(mnb, 16)
+    hi = raw[mnb * 16:mnb * 32].view(np.int8).reshape(mnb, 16)
+    d = raw[mnb * 32:mnb * 36].view(np.float32).reshape(MT, nb)
+    n8 = raw[mnb * 36:mnb * 40].view(np.int32).reshape(MT, nb)
+    codes = np.concatenate([lo, hi], axis=1).reshape(MT, K)
+    return codes, d, n8
+
+
+def _check_image(img, y_stored, M, K, x86):
+    """the image must be the Q8_0 quantization of the stored rows (bit-exact), zero beyond them"""
+    codes, d, n8 = _image_fields(img, M, K)
+    q, dbits = orc.quantize_rows_q8_0(np.asarray(y_stored, np.float32).reshape(M, K))
+    bits = orc.x86_scale_bits(dbits) if x86 else dbits
+    assert np.array_equal(codes[:M], q)
+    assert np.array_equal(d[:M].view(np.uint32), orc.fp16_bits_to_fp32(bits).view(np.uint32))
+    assert np.array_equal(n8[:M], -8 * q.reshape(M, K // 32, 32).astype(np.int32).sum(-1))
+    assert not codes[M:].any() and not d[M:].any() and not n8[M:].any()
+
+
+@pytest.mark.parametrize("rows,D", [(1, 2560), (5, 2560), (3, 128), (64, 4096), (2, 9728), (7, 40), (300, 128)])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_rmsnorm(rows, D, dtype):
+    rng = synth.rng_for(6, rows * 7 + D)
+    w = (1 + 0.2 * rng.standard_normal(D)).astype(np.float32)
+    if dtype == "bf16":
+        bits, xf = synth.make_x_bf16(rng, rows, D)
+        x = bf16_dev(bits)
+    else:
+        xf = synth.make_x_fp32(rng, rows, D) * 2.5
+        x = to_dev(xf)
+    for off in (False, True):
+        announce("rmsnorm", rows, D, dtype, off)
+        y = ql.rmsnorm(x, to_dev(w), 1e-6, off).float().cpu().numpy()
+        want = orc.rmsnorm(xf, w, 1e-6, off)
+        if dtype == "f32":
+            assert rel_l2(y, want) < 2e-6
+        else:  # stored as bf16: equal to the rounded oracle values up to single-ulp flips at rounding boundaries
+            assert rel_l2(y, _bf16_round(want)) < TOL
+
+
+@pytest.mark.parametrize("M,K", [(1, 2560), (2, 2560), (3, 4096), (4, 9728), (8, 2560), (1, 96), (6, 32)])
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_rmsnorm_writes_the_image_of_what_it_stored(M, K, dtype):
+    rng = synth.rng_for(6, 1000 + M * 13 + K)
+    w = (1 + 0.2 * rng.standard_normal(K)).astype(np.float32)
+    if dtype == "bf16":
+        bits, _ = synth.make_x_bf16(rng, M, K)
+        x = bf16_dev(bits)
+    else:
+        x = to_dev(synth.make_x_fp32(rng, M, K))
+    for mode, x86 in ((ql.SCALE_X86_REF, True), (ql.SCALE_IEEE, False)):
+        announce("rmsnorm image", M, K, dtype, x86)
+        y, img = ql.rmsnorm(x, to_dev(w), 1e-6, want_image=True, act_scale_mode=mode)
+        assert torch.equal(y, ql.rmsnorm(x, to_dev(w), 1e-6))
+        _check_image(img, y.float().cpu().numpy(), M, K, x86)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_elementwise(dtype):
+    rng = synth.rng_for(6, 77)
+    n = 8 * 1237
+    a = (rng.standard_normal(n) * 4).astype(np.float32)
+    b = rng.standard_normal(n).astype(np.float32)
+    if dtype == "bf16":
+        a, b = _bf16_round(a), _bf16_round(b)
+        da, db = to_dev(a).bfloat16(), to_dev(b).bfloat16()
+        rnd = _bf16_round
+    else:
+        da, db = to_dev(a), to_dev(b)
+        rnd = lambda v: v
+    announce("elementwise", dtype)
+    assert np.array_equal(ql.add(da, db).float().cpu().numpy(), rnd(a + b))
+    assert np.array_equal(ql.mul(da, db).float().cpu().numpy(), rnd(a * b))
+    s = ql.silu(da).float().cpu().numpy()
+    assert rel_l2(s, rnd(orc.silu(a))) < (2e-7 if dtype == "f32" else TOL)
+    sm = ql.silu_mul(da.view(1, n), db.view(1, n)).float().cpu().numpy().ravel()
+    assert rel_l2(sm, rnd(rnd(orc.silu(a)) * b)) < (2e-7 if dtype == "f32" else TOL)
+    # one pass equals the two operators run one after the other, bit for bit
+    assert torch.equal(ql.silu_mul(da.view(1, n), db.view(1, n)).view(-1), ql.mul(ql.silu(da), db))
+    # the reference's exp is not an accurate exp: the switch to expf moves SiLU by about 1e-4 .. 1e-3
+    if dtype == "f32":
+        ql.set_exp_mode(1)
+        try:
+            acc = ql.silu(da).cpu().numpy()
+        finally:
+            ql.set_exp_mode(0)
+        exact = a.astype(np.float64) / (1 + np.exp(-a.astype(np.float64)))
+        assert rel_l2(acc, exact) < 2e-7 and 1e-5 < rel_l2(s, exact) < 2e-3
+
+
+@pytest.mark.parametrize("M,D", [(1, 9728), (4, 9728), (8, 768), (2, 64)])
+def test_silu_mul_image(M, D):
+    rng = synth.rng_for(6, 2000 + M + D)
+    g = to_dev(synth.make_x_fp32(rng, M, D) * 2)
+    u = to_dev(synth.make_x_fp32(rng, M, D))
+    announce("silu_mul image", M, D)
+    y, img = ql.silu_mul(g, u, want_image=True, act_scale_mode=ql.SCALE_X86_REF)
+    assert torch.equal(y, ql.silu_mul(g, u))
+    _check_image(img, y.cpu().numpy(), M, D, True)
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M", [1, 2, 3, 8])
+def test_gemv_fused_equals_the_operators_it_replaces(wtype, M):
+    """rmsnorm(+image) -> gate/up GEMV from the image -> silu*up(+image) -> down GEMV from the image + residual
+    equals rmsnorm -> GEMV -> silu -> mul -> GEMV -> add, bit for bit, and the oracle's chain within tolerance"""
+    rng = synth.rng_for(6, 3000 + wtype * 10 + M)
+    H, I = 512, 1536
+    Wg, Wu, Wd = (synth.make_weight(rng, wtype, I, H), synth.make_weight(rng, wtype, I, H), synth.make_weight(rng, wtype, H, I))
+    pg, pu, pd = (ql.PackedQWeight(wtype, torch.from_numpy(W)) for W in (Wg, Wu, Wd))
+    xf = synth.make_x_fp32(rng, M, H)
+    nw = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    x, w = to_dev(xf), to_dev(nw)
+    announce("fused mlp chain", wtype, M)
+    # unfused
+    h0 = ql.rmsnorm(x, w, 1e-6)
+    g0, u0 = ql.linear_q_gemv_multi([pg, pu], h0)
+    a0 = ql.mul(ql.silu(g0), u0)
+    o0 = ql.add(ql.linear_q_gemv(pd, a0), x)
+    # fused
+    h1, img = ql.rmsnorm(x, w, 1e-6, want_image=True)
+    g1, u1 = ql.linear_q_gemv_fused([pg, pu], img, M=M, image=True)
+    a1, img2 = ql.silu_mul(g1, u1, want_image=True)
+    (o1,) = ql.linear_q_gemv_fused([pd], img2, M=M, image=True, residuals=[x])
+    assert torch.equal(g0, g1) and torch.equal(u0, u1) and torch.equal(a0, a1) and torch.equal(o0, o1)
+    # residual together with a bias, activations not pre-quantized, residual aliasing the output
+    bias = to_dev(rng.standard_normal(H).astype(np.float32))
+    o2 = x.clone()
+    ql.linear_q_gemv_fused([pd], a0, biases=[bias], residuals=[o2], outs=[o2])
+    assert torch.equal(o2, ql.add(ql.linear_q_gemv(pd, a0, bias), x))
+    # oracle chain
+    hn = orc.rmsnorm(xf, nw, 1e-6)
+    gn = orc.linear_q(hn, Wg, wtype, None, orc.SCALE_X86_REF)
+    un = orc.linear_q(hn, Wu, wtype, None, orc.SCALE_X86_REF)
+    an = orc.silu(gn) * un
+    on = orc.linear_q(an, Wd, wtype, None, orc.SCALE_X86_REF) + xf
+    assert rel_l2(g1.cpu().numpy(), gn) < TOL and rel_l2(a1.cpu().numpy(), an) < TOL and rel_l2(o1.cpu().numpy(), on) < TOL
+
+
+@pytest.mark.parametrize("rows,n", [(1, 128), (512, 128), (5, 16), (7, 13), (3, 1000), (9, 60)])
+def test_softmax(rows, n):
+    rng = synth.rng_for(6, 4000 + rows + n)
+    x = (rng.standard_normal((rows, n)) * 3).astype(np.float32)
+    announce("softmax", rows, n)
+    y = ql.softmax(to_dev(x)).cpu().numpy()
+    want = orc.softmax(x)
+    assert rel_l2(y, want) < 2e-6
+    assert np.allclose(y.sum(-1), 1.0, atol=1e-5)
+
+
+def test_topk_reference_test_shapes_and_sort():
+    rng = synth.rng_for(6, 5000)
+    for shape in [(10,), (1, 10), (5, 10), (2, 5, 10), (1, 4, 8, 16)]:  # tests/cpu/KernelTest.cpp:686
+        x = rng.uniform(-10, 10, shape).astype(np.float32)
+        announce("topk", shape)
+        v, i = ql.topk(to_dev(x), 3)
+        wv, wi = orc.topk(x, 3)
+        assert v.shape == wv.shape and i.dtype == torch.int32
+        assert np.array_equal(i.cpu().numpy(), wi) and np.array_equal(v.cpu().numpy(), wv)
+    x = rng.standard_normal((700, 128)).astype(np.float32)
+    for k, largest, srt in [(8, True, False), (8, True, True), (5, False, True), (128, True, True), (1, False, False)]:
+        announce("topk", k, largest, srt)
+        v, i = ql.topk(to_dev(x), k, largest, srt)
+        wv, wi = orc.topk(x, k, largest, srt)
+        assert np.array_equal(i.cpu().numpy(), wi) and np.array_equal(v.cpu().numpy(), wv)
+    # ties are taken lowest index first
+    t = np.float32([[1, 3, 3, 2, 3, 0, 3, 3]])
+    v, i = ql.topk(to_dev(t), 3)
+    assert i.cpu().numpy().tolist() == [[1, 2, 4]]
+    long = rng.standard_normal((3, 5000)).astype(np.float32)
+    v, i = ql.topk(to_dev(long), 20)
+    wv, wi = orc.topk(long, 20)
+    assert np.array_equal(i.cpu().numpy(), wi)
+
+
+@pytest.mark.parametrize("M,H,E,k,dtype", [(512, 2048, 128, 8, "f32"), (1, 2048, 128, 8, "f32"), (7, 256, 60, 4, "f32"),
+                                           (33, 2048, 128, 8, "bf16"), (5, 64, 8, 2, "f32")])
+def test_moe_gate(M, H, E, k, dtype):
+    rng = synth.rng_for(6, 6000 + M + E)
+    w = (rng.standard_normal((E, H)) * 0.05).astype(np.float32)
+    if dtype == "bf16":
+        bits, xf = synth.make_x_bf16(rng, M, H)
+        x = bf16_dev(bits)
+    else:
+        xf = synth.make_x_fp32(rng, M, H)
+        x = to_dev(xf)
+    for norm in (True, False):
+        announce("moe gate", M, H, E, k, dtype, norm)
+        ids, wt, sc = ql.moe_gate(x, to_dev(w), k, norm, want_scores=True)
+        ids, wt, sc = ids.cpu().numpy(), wt.cpu().numpy(), sc.cpu().numpy()
+        oi, ow, osc = orc.moe_gate(xf, w, k, norm)
+        assert rel_l2(sc, osc) < 1e-5
+        # index work is exact: the selection made on the kernel's own scores is the oracle's selection on those scores
+        sv, si = orc.topk(sc, k, True, False)
+        assert np.array_equal(ids, si)
+        want_w = sv / sv.sum(-1, keepdims=True) if norm else sv
+        assert np.max(np.abs(wt - want_w)) < 1e-6
+        # end to end the experts agree wherever the oracle's k-th and (k+1)-th scores are further apart than the
+        # rounding noise of the logits
+        srt = -np.sort(-osc, axis=-1)
+        safe = (srt[:, k - 1] - srt[:, k]) > 1e-5 * srt[:, 0] if k < E else np.ones(M, bool)
+        assert safe.mean() > 0.9
+        assert np.array_equal(ids[safe], oi[safe])
+        assert np.max(np.abs(wt[safe] - ow[safe])) < 1e-5
+
+
+def test_argument_checks():
+    L = _lib.lib()
+    x = torch.zeros(64, dtype=torch.float32, device="cuda")
+    p = x.data_ptr()
+    assert L.mllm_hip_rmsnorm(p, 0, p, p, 1, 60, 1e-6, 0, None, 0, None) == -2       # D % 8
+    assert L.mllm_hip_rmsnorm(p, 0, p, p, 1, 1 << 15, 1e-6, 0, None, 0, None) == -2  # D too long
+    assert L.mllm_hip_rmsnorm(p, 0, p, p, 9, 64, 1e-6, 0, p, 0, None) == -2          # image wants rows <= 8
+    assert L.mllm_hip_rmsnorm(p, 0, p, p, 1, 40, 1e-6, 0, p, 0, None) == -2          # image wants D % 32
+    assert L.mllm_hip_rmsnorm(p + 4, 0, p, p, 1, 8, 1e-6, 0, None, 0, None) == -3
+    assert L.mllm_hip_rmsnorm(None, 0, p, p, 1, 8, 1e-6, 0, None, 0, None) == -1
+    assert L.mllm_hip_silu(p, p, 0, 12, None) == -2
+    assert L.mllm_hip_add(p, None, p, 0, 8, None) == -1
+    assert L.mllm_hip_topk(p, p, p, 1, 8, 9, 1, 1, None) == -2
+    assert L.mllm_hip_topk(p, p, p, 1, 8, 0, 1, 1, None) == -2
+    assert L.mllm_hip_softmax(p, None, 1, 8, None) == -1
+    assert L.mllm_hip_moe_gate(p, 0, p, p, p, None, 1, 12, 4, 2, 1, None) == -2      # H % 8
+    assert L.mllm_hip_moe_gate(p, 0, p, p, p, None, 1, 8, 4, 5, 1, None) == -2       # k > E
+    assert L.mllm_hip_set_exp_mode(2) == -1

@@ -255,7 +255,7 @@ def test_moe_composition_and_invariance():
             e = ids[t, j]
             g = orc.linear_q(x[t:t + 1], Wg[e], orc.Q4_0)
             u = orc.linear_q(x[t:t + 1], Wu[e], orc.Q4_0)
-            h = (g / (np.float32(1) + np.exp(-g))).astype(np.float32) * u
+            h = orc.silu(g) * u  # the SiLU operator as the x86 build computes it (pinned in test_oracle_layer_ops.py)
             o = orc.linear_q(h, Wd[e], orc.Q4_0)
             acc = acc + o[0] * w[t, j]
         want[t] = acc
