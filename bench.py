@@ -277,6 +277,59 @@ def main():
         nbytes = sum(synth.gemv_algorithmic_bytes(wtype, M, shapes[g][0], k, 2) for g in groups) - (len(groups) - 1) * M * k * 2
         return {"us": per * 1e6, "GBps": nbytes / per / 1e9, "bytes": nbytes, "launches": reps * len(sets)}
 
+    def measure_layer_chain(pool, M, reps=5):
+        """The dependent chain of one decoder layer around its Linears (attention core left out: o_proj reads a fixed
+        buffer), fp32 residual stream, over all layers: the operators one by one (10 launches per layer) against the
+        folded form (RMSNorm and SiLU*up write the GEMV's quantized image, residual adds in the GEMV epilogue: 7)."""
+        x0 = torch.randn((M, 2560), device="cuda", generator=gen)
+        attn = torch.randn((M, 4096), device="cuda", generator=gen)
+        nw = [torch.ones(2560, device="cuda") for _ in range(2)]
+        b = {n: torch.empty((M, d), dtype=torch.float32, device="cuda")
+             for n, d in (("h", 2560), ("q", 4096), ("k", 1024), ("v", 1024), ("o", 2560), ("x1", 2560), ("h2", 2560),
+                          ("g", 9728), ("u", 9728), ("s", 9728), ("a", 9728), ("d", 2560), ("x2", 2560))}
+        img = {k: ql.gemv_workspace(M, k) for k in (2560, 9728)}
+        L = _lib.lib()
+
+        def ew(fn, a_, b_, y_):
+            _lib.check(fn(a_.data_ptr(), b_.data_ptr(), y_.data_ptr(), 0, a_.numel(), torch.cuda.current_stream().cuda_stream), "ew")
+
+        def plain():
+            x = x0
+            for l in pool:
+                ql.rmsnorm(x, nw[0], 1e-6, out=b["h"])
+                ql.linear_q_gemv_multi([l["q_proj"], l["k_proj"], l["v_proj"]], b["h"], None, ql.SCALE_X86_REF, [b["q"], b["k"], b["v"]])
+                ql.linear_q_gemv(l["o_proj"], attn, None, ql.SCALE_X86_REF, out=b["o"])
+                ew(L.mllm_hip_add, b["o"], x, b["x1"])
+                ql.rmsnorm(b["x1"], nw[1], 1e-6, out=b["h2"])
+                ql.linear_q_gemv_multi([l["gate_proj"], l["up_proj"]], b["h2"], None, ql.SCALE_X86_REF, [b["g"], b["u"]])
+                _lib.check(L.mllm_hip_silu(b["g"].data_ptr(), b["s"].data_ptr(), 0, b["g"].numel(),
+                                           torch.cuda.current_stream().cuda_stream), "silu")
+                ew(L.mllm_hip_mul, b["s"], b["u"], b["a"])
+                ql.linear_q_gemv(l["down_proj"], b["a"], None, ql.SCALE_X86_REF, out=b["d"])
+                ew(L.mllm_hip_add, b["d"], b["x1"], b["x2"])
+                x = b["x2"]
+
+        def folded():
+            x = x0
+            for l in pool:
+                st = torch.cuda.current_stream().cuda_stream
+                _lib.check(L.mllm_hip_rmsnorm(x.data_ptr(), 0, nw[0].data_ptr(), b["h"].data_ptr(), M, 2560, 1e-6, 0,
+                                              img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
+                ql.linear_q_gemv_fused([l["q_proj"], l["k_proj"], l["v_proj"]], img[2560], M=M, image=True, outs=[b["q"], b["k"], b["v"]])
+                ql.linear_q_gemv_fused([l["o_proj"]], attn, residuals=[x], outs=[b["x1"]])
+                _lib.check(L.mllm_hip_rmsnorm(b["x1"].data_ptr(), 0, nw[1].data_ptr(), b["h2"].data_ptr(), M, 2560, 1e-6, 0,
+                                              img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
+                ql.linear_q_gemv_fused([l["gate_proj"], l["up_proj"]], img[2560], M=M, image=True, outs=[b["g"], b["u"]])
+                _lib.check(L.mllm_hip_silu_mul(b["g"].data_ptr(), b["u"].data_ptr(), b["a"].data_ptr(), 0, M, 9728,
+                                               img[9728].data_ptr(), ql.SCALE_X86_REF, st), "silu_mul")
+                ql.linear_q_gemv_fused([l["down_proj"]], img[9728], M=M, image=True, residuals=[b["x1"]], outs=[b["x2"]])
+                x = b["x2"]
+        res = {}
+        for name, fn, n in (("operators_one_by_one", plain, 10), ("folded", folded, 7)):
+            _, ev = timed(graphed(fn), reps, 2)
+            res[name] = {"us_per_layer": ev / (reps * len(pool)) * 1e6, "launches_per_layer": n}
+        return res
+
     wtype = ql.Q4_0 if args.wtype == "q4_0" else ql.Q8_0
     if args.pmc_probe:
         pool = make_pool(wtype, 20)
@@ -305,6 +358,7 @@ def main():
     extra = {"per_shape": per_shape, "event_ms_per_step": head["event_ms_per_step"],
              "graph": not args.no_graph, "layers": N_LAYERS, "launches_per_step": N_LAYERS * (len(shapes) if args.per_op else 4)}
     if not args.no_extra:
+        extra["decode_layer_chain"] = {"m%d" % M: measure_layer_chain(pool, M) for M in (1, 4, 8)}
         for M in (4, 8):
             if M != args.m:
                 r = measure_workload(wtype, M, pool, max(5, args.steps // 3), 2)

@@ -16,6 +16,11 @@ class GemvPart(C.Structure):
     _fields_ = [("packed", C.c_void_p), ("bias", C.c_void_p), ("y", C.c_void_p), ("N", C.c_int64)]
 
 
+class GemvFusion(C.Structure):
+    """mllm_hip_gemv_fusion"""
+    _fields_ = [("residual", C.POINTER(C.c_void_p))]
+
+
 class HipQLinearError(RuntimeError):
     pass
 
@@ -48,7 +53,7 @@ def lib():
         L.mllm_hip_linear_q_gemv.argtypes = [ci, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi_ws.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp, vp]
-        L.mllm_hip_linear_q_gemv_fused.argtypes = [ci, ci, C.POINTER(GemvPart), C.POINTER(vp), vp, ci, ci, i64, ci, vp]
+        L.mllm_hip_linear_q_gemv_fused.argtypes = [ci, ci, C.POINTER(GemvPart), C.POINTER(GemvFusion), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_rmsnorm.argtypes = [vp, ci, vp, vp, i64, i64, C.c_float, ci, vp, ci, vp]
         L.mllm_hip_silu.argtypes = [vp, vp, ci, i64, vp]
         L.mllm_hip_add.argtypes = [vp, vp, vp, ci, i64, vp]

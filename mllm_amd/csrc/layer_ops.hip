@@ -159,7 +159,7 @@ struct RmsArgs {
 // One workgroup per row; a lane keeps NI items of eight elements in registers between the two passes.
 template <int XT, int NI>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(RmsArgs a) {
-  __shared__ float s_part[4];
+  __shared__ float s_grp[4 * NI];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t row = blockIdx.x;
   if (row >= a.rows) {  // only launched for the zero rows of an image
@@ -179,20 +179,22 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(RmsArgs a) {
     const int it = min(tid + 256 * k, nitems - 1);
     item_load<MLLM_HIP_F32>(a.w, (int64_t)it * 8, wraw[k]);
   }
+  // Sum of squares in a fixed order (per item an fma chain, the 64 items of a group through the wave butterfly, the
+  // groups one after the other): a function of the row alone, not of how rows are spread over workgroups.
   float v[NI][8];
-  float ss = 0.f;
 #pragma unroll
   for (int k = 0; k < NI; k++) {
     item_to_f32<XT>(raw[k], v[k]);
-    if (tid + 256 * k < nitems) {
+    float p = 0.f;
 #pragma unroll
-      for (int e = 0; e < 8; e++) ss = fmaf(v[k][e], v[k][e], ss);
-    }
+    for (int e = 0; e < 8; e++) p = fmaf(v[k][e], v[k][e], p);
+    p = wave_sum(tid + 256 * k < nitems ? p : 0.f);
+    if (lane == 0) s_grp[wave + 4 * k] = p;
   }
-  ss = wave_sum(ss);
-  if (lane == 0) s_part[wave] = ss;
   __syncthreads();
-  const float total = (s_part[0] + s_part[1]) + (s_part[2] + s_part[3]);
+  const int ngroups = (nitems + 63) >> 6;
+  float total = 0.f;
+  for (int g = 0; g < ngroups; g++) total += s_grp[g];
   const float rms = 1.0f / sqrtf(total / (float)a.D + a.eps);
 #pragma unroll
   for (int k = 0; k < NI; k++) {

@@ -325,8 +325,9 @@ MLLM_API size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K) {
 }
 
 // x_kind: MLLM_HIP_F32 / MLLM_HIP_BF16 activations, or MLLM_HIP_Q8_IMAGE: their quantized image (act_scale_mode unused)
-static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual, const void* x,
+static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fu, const void* x,
                            int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
+  const float* const* residual = fu ? fu->residual : nullptr;
   if (nparts < 1 || nparts > GEMV_MAX_PARTS || !parts) return MLLM_HIP_E_BADARG;
   if (!x || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16 && x_dtype != MLLM_HIP_Q8_IMAGE)) return MLLM_HIP_E_BADARG;
   if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
@@ -378,9 +379,9 @@ MLLM_API int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_h
   return gemv_multi_impl(wtype, nparts, parts, nullptr, x, x_dtype, M, K, act_scale_mode, workspace, stream);
 }
 
-MLLM_API int mllm_hip_linear_q_gemv_fused(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual,
+MLLM_API int mllm_hip_linear_q_gemv_fused(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fusion,
                                           const void* x, int x_kind, int M, int64_t K, int act_scale_mode, void* stream) {
-  return gemv_multi_impl(wtype, nparts, parts, residual, x, x_kind, M, K, act_scale_mode, nullptr, stream);
+  return gemv_multi_impl(wtype, nparts, parts, fusion, x, x_kind, M, K, act_scale_mode, nullptr, stream);
 }
 
 MLLM_API int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,

@@ -158,8 +158,11 @@ __device__ __forceinline__ void x8_to_f32(const XRaw<XT>& raw, float (&v)[8]) {
 // SCL: the fp16 scales of the wave's rows are fetched with (at most two) 16-byte loads per lane and handed out through
 // LDS instead of one 2-byte load per block.
 // U = how many block columns a lane keeps in flight per loop trip; later trips are double-buffered.
+// Register budget: with four or eight activation rows the accumulators and the weights in flight need 140..215
+// registers; the kernels are therefore built for at most eight waves per workgroup (under a 1024-thread bound the
+// compiler has 128 and spills 40..330 bytes per lane).  For one or two rows 16 waves stay possible (long rows).
 template <int WT, int XT, int MT, int G, int R, int U, bool SCL>
-__global__ __launch_bounds__(1024) void gemv_q_kernel(GemvArgs a) {
+__global__ __launch_bounds__(MT <= 2 ? 1024 : 512) void gemv_q_kernel(GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int nb = a.nb, nbp = a.nbp;
   int pidx = 0;  // uniform: which matrix this workgroup works on
@@ -353,6 +356,7 @@ template <int WT, int XT, int MT, int G, int R>
 static int launch_gemv_u(const GemvArgs& a_in, int NW, hipStream_t st) {
   constexpr int U = ((R >= 4) ? 1 : (R == 2 ? 2 : 4)) * (WT == MLLM_HIP_Q4_0 ? 2 : 1);
   constexpr int ROWS_W = (64 / G) * R;
+  if (MT > 2 && NW > 8) NW = 8;  // see the register budget note at the kernel
   const int rows_per_wg = NW * ROWS_W;
   GemvArgs a = a_in;
   unsigned grid = 0;
