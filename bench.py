@@ -291,7 +291,8 @@ def main():
         L = _lib.lib()
 
         def ew(fn, a_, b_, y_):
-            _lib.check(fn(a_.data_ptr(), b_.data_ptr(), y_.data_ptr(), 0, a_.numel(), torch.cuda.current_stream().cuda_stream), "ew")
+            _lib.check(fn(a_.data_ptr(), b_.data_ptr(), y_.data_ptr(), 0, a_.shape[0], a_.shape[1], None, 0,
+                          torch.cuda.current_stream().cuda_stream), "ew")
 
         def plain():
             x = x0

@@ -285,9 +285,12 @@ int mllm_hip_rmsnorm(const void* x, int dtype, const float* weight, void* y, int
 /* y = x * (1 / (1 + exp(-x))) with the reference's polynomial exp.
  * replaces: CPUSiLUOp::forward -> x86::silu_fp32  mllm/backends/cpu/kernels/x86/silu.cpp:16-56, math.hpp:19-72 */
 int mllm_hip_silu(const void* x, void* y, int dtype, int64_t n, void* stream);
-/* y = a + b, y = a * b (same shapes).  replaces: CPUAddOp / CPUMulOp::forward  mllm/backends/cpu/ops/ElewiseOps.cpp */
-int mllm_hip_add(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream);
-int mllm_hip_mul(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream);
+/* y = a + b, y = a * b over [rows][D] (same shapes, no broadcasting).
+ * replaces: CPUAddOp / CPUMulOp::forward  mllm/backends/cpu/ops/ElewiseOps.cpp */
+int mllm_hip_add(const void* a, const void* b, void* y, int dtype, int64_t rows, int64_t D, void* q_image, int act_scale_mode,
+                 void* stream);
+int mllm_hip_mul(const void* a, const void* b, void* y, int dtype, int64_t rows, int64_t D, void* q_image, int act_scale_mode,
+                 void* stream);
 /* y = silu(gate) * up in one pass (the SiLU result is rounded to the tensor's type before the product, as when the two
  * operators run one after the other).  replaces: silu_(gate) then x * y  mllm/models/qwen3/modeling_qwen3_fa2.hpp:87-90 */
 int mllm_hip_silu_mul(const void* gate, const void* up, void* y, int dtype, int64_t rows, int64_t D, void* q_image,

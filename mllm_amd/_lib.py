@@ -56,8 +56,8 @@ def lib():
         L.mllm_hip_linear_q_gemv_fused.argtypes = [ci, ci, C.POINTER(GemvPart), C.POINTER(GemvFusion), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_rmsnorm.argtypes = [vp, ci, vp, vp, i64, i64, C.c_float, ci, vp, ci, vp]
         L.mllm_hip_silu.argtypes = [vp, vp, ci, i64, vp]
-        L.mllm_hip_add.argtypes = [vp, vp, vp, ci, i64, vp]
-        L.mllm_hip_mul.argtypes = [vp, vp, vp, ci, i64, vp]
+        L.mllm_hip_add.argtypes = [vp, vp, vp, ci, i64, i64, vp, ci, vp]
+        L.mllm_hip_mul.argtypes = [vp, vp, vp, ci, i64, i64, vp, ci, vp]
         L.mllm_hip_silu_mul.argtypes = [vp, vp, vp, ci, i64, i64, vp, ci, vp]
         L.mllm_hip_set_exp_mode.argtypes = [ci]
         L.mllm_hip_softmax.argtypes = [vp, vp, i64, i64, vp]

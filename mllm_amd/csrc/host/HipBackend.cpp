@@ -28,6 +28,7 @@ bool HipAllocator::alloc(Storage* storage) {
   return true;
 }
 void HipAllocator::free(Storage* storage) {
+  if (storage->ptr_ && owner) owner->noteWrite(storage->ptr_, storage->size_);
   if (storage->ptr_) (void)hipFree(storage->ptr_);
   storage->ptr_ = nullptr;
 }
@@ -42,12 +43,54 @@ HipBackend::HipBackend(const HipBackendConfig& cfg) : Backend(kHIP, std::make_sh
   hipStream_t st;
   MLLM_HIP_CHECK(hipStreamCreate(&st));
   stream_ = st;
-  regOpFactory<HipLinearOpFactory, HipMatMulOpFactory, HipX2XOpFactory>();
+  std::static_pointer_cast<HipAllocator>(allocator_)->owner = this;
+  regOpFactory<HipLinearOpFactory, HipMatMulOpFactory, HipX2XOpFactory, HipRMSNormOpFactory, HipSiLUOpFactory, HipAddOpFactory,
+               HipMulOpFactory, HipSoftmaxOpFactory, HipTopKOpFactory>();
 }
 HipBackend::~HipBackend() {
+  std::static_pointer_cast<HipAllocator>(allocator_)->owner = nullptr;
+  images_.clear();
+  image_pool_.clear();
   if (stream_) (void)hipStreamDestroy((hipStream_t)stream_);
 }
 void HipBackend::synchronize() const { MLLM_HIP_CHECK(hipStreamSynchronize((hipStream_t)stream_)); }
+
+void* HipBackend::newImage(const void* tensor_ptr, size_t tensor_bytes, int rows, int64_t D) {
+  if (!cfg_.fold_images || rows < 1 || rows > 8 || D % 32) return nullptr;
+  const size_t need = mllm_hip_gemv_workspace_bytes(rows, D);
+  Tensor buf;
+  for (size_t i = 0; i < image_pool_.size(); i++)
+    if (image_pool_[i].bytes() >= need) {
+      buf = image_pool_[i];
+      image_pool_.erase(image_pool_.begin() + (long)i);
+      break;
+    }
+  if (buf.isNil()) buf = Tensor::empty({(int32_t)need}, kByte, kHIP).alloc();
+  images_.push_back(Image{tensor_ptr, tensor_bytes, rows, D, buf});
+  return buf.ptr<void>();
+}
+const void* HipBackend::findImage(const void* tensor_ptr, int rows, int64_t D) const {
+  for (const auto& im : images_)
+    if (im.tensor_ptr == tensor_ptr && im.rows == rows && im.D == D) return im.data.ptr<void>();
+  return nullptr;
+}
+void HipBackend::noteWrite(const void* ptr, size_t bytes) {
+  const char* lo = static_cast<const char*>(ptr);
+  const char* hi = lo + bytes;
+  std::vector<Tensor> dropped;  // released after the loop: freeing a buffer calls back into this function
+  for (size_t i = 0; i < images_.size();) {
+    const char* tl = static_cast<const char*>(images_[i].tensor_ptr);
+    if (tl < hi && lo < tl + images_[i].tensor_bytes) {
+      dropped.push_back(images_[i].data);
+      images_.erase(images_.begin() + (long)i);
+    } else {
+      i++;
+    }
+  }
+  // a dropped buffer may still be read by a GEMV queued on the stream; kernels that reuse it are queued behind that one
+  for (auto& t : dropped)
+    if (image_pool_.size() < 16) image_pool_.push_back(t);
+}
 
 std::shared_ptr<HipBackend> initHipBackend() {
   auto& ctx = Context::instance();
@@ -57,6 +100,7 @@ std::shared_ptr<HipBackend> initHipBackend() {
     if (std::strcmp(m, "x86") == 0) cfg.weight_scale_mode = cfg.act_scale_mode = MLLM_HIP_SCALE_X86_REF;
   }
   if (const char* m = std::getenv("MLLM_HIP_PREFILL")) cfg.prefill_matrix_cores = std::strcmp(m, "blockdot") != 0;
+  if (const char* m = std::getenv("MLLM_HIP_FOLD_IMAGES")) cfg.fold_images = std::strcmp(m, "0") != 0;
   auto backend = std::make_shared<HipBackend>(cfg);
   ctx.registerBackend(backend);
   ctx.memoryManager()->registerAllocator(kHIP, backend->allocator());
@@ -73,6 +117,7 @@ void HipX2XOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& o
   auto& out = outputs[0];
   const size_t n = in.bytes();
   auto st = (hipStream_t)backend().stream();
+  if (out.device() == kHIP) backend().noteWrite(out.ptr<void>(), out.bytes());
   if (in.device() == kCPU && out.device() == kHIP) {
     MLLM_HIP_CHECK(hipMemcpyAsync(out.ptr<void>(), in.ptr<void>(), n, hipMemcpyHostToDevice, st));
     MLLM_HIP_CHECK(hipStreamSynchronize(st));  // the host buffer may be released by the caller right after
@@ -92,6 +137,7 @@ void HipMatMulOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
   const auto& b = inputs[1];
   auto& c = outputs[0];
   if (a.dtype() != kFloat32 || b.dtype() != kFloat32) NYI("HipMatMulOp supports fp32 operands only");
+  backend().noteWrite(c.ptr<void>(), c.bytes());
   const auto& cs = c.shape();
   const int64_t M = cs[cs.size() - 2], N = cs[cs.size() - 1];
   const auto& as = a.shape();
@@ -200,6 +246,7 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
   const int64_t M = (int64_t)x.numel() / K;  // all leading dimensions are rows
   auto& be = backend();
   void* st = be.stream();
+  be.noteWrite(y.ptr<void>(), y.bytes());
   auto xdt = [&]() {
     if (x.dtype() == kFloat32) return MLLM_HIP_F32;
     if (x.dtype() == kBFloat16) return MLLM_HIP_BF16;
@@ -215,8 +262,15 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
     case Scheme::kQ8_0: {
       const int wt = scheme_ == Scheme::kQ4_0 ? MLLM_HIP_Q4_0 : MLLM_HIP_Q8_0;
       if (M <= 8) {
-        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), (int)M, N, K,
-                                                     be.config().act_scale_mode, st));
+        const void* image = be.findImage(x.ptr<void>(), (int)M, K);
+        if (image) {
+          mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
+          MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_fused(wt, 1, &part, nullptr, image, MLLM_HIP_Q8_IMAGE, (int)M, K,
+                                                             be.config().act_scale_mode, st));
+        } else {
+          MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), (int)M, N, K,
+                                                       be.config().act_scale_mode, st));
+        }
       } else if (!gemm_packed_.isNil()) {
         void* ws = workspace(mllm_hip_linear_q_gemm_workspace_bytes(M, K));
         MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemm(wt, gemm_packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K,
@@ -242,6 +296,85 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
     }
     default: MLLM_ERROR_EXIT(ExitCode::kCoreError, "HipLinearOp::forward before load()");
   }
+}
+
+// ---- the operators around Linear -----------------------------------------------------------------------------------
+static int actType(const Tensor& t, const char* who) {
+  if (t.dtype() == kFloat32) return MLLM_HIP_F32;
+  if (t.dtype() == kBFloat16) return MLLM_HIP_BF16;
+  MLLM_ERROR_EXIT(ExitCode::kCoreError, "%s: dtype %d not supported (fp32 or bf16)", who, (int)t.dtype());
+}
+static void rowsAndWidth(const Tensor& t, int64_t& rows, int64_t& D) {
+  D = t.shape().back();
+  rows = (int64_t)t.numel() / D;
+}
+
+void HipRMSNormOp::load(const ParameterFile::ptr_t& ploader) {
+  aops::RMSNormOp::load(ploader);
+  if (weight_.dtype() != kFloat32) NYI("HipRMSNormOp: weight must be fp32 (as in the reference's x86 kernel)");
+  weight_ = onDevice(weight_);
+}
+void HipRMSNormOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  const auto& x = inputs[0];
+  auto& y = outputs[0];
+  auto& be = backend();
+  int64_t rows, D;
+  rowsAndWidth(x, rows, D);
+  MLLM_RT_ASSERT_EQ((int64_t)weight_.numel(), D);
+  be.noteWrite(y.ptr<void>(), y.bytes());
+  void* image = be.newImage(y.ptr<void>(), y.bytes(), (int)std::min<int64_t>(rows, 9), D);
+  MLLM_HIP_KERNEL_CHECK(mllm_hip_rmsnorm(x.ptr<void>(), actType(x, "HipRMSNormOp"), weight_.ptr<float>(), y.ptr<void>(), rows, D,
+                                         options_.epsilon, options_.add_unit_offset, image, be.config().act_scale_mode, be.stream()));
+}
+void HipSiLUOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  auto& be = backend();
+  be.noteWrite(outputs[0].ptr<void>(), outputs[0].bytes());
+  MLLM_HIP_KERNEL_CHECK(mllm_hip_silu(inputs[0].ptr<void>(), outputs[0].ptr<void>(), actType(inputs[0], "HipSiLUOp"),
+                                      (int64_t)inputs[0].numel(), be.stream()));
+}
+template <typename Fn>
+static void binaryForward(const char* who, Fn fn, const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs, bool want_image) {
+  const auto& a = inputs[0];
+  const auto& b = inputs[1];
+  auto& y = outputs[0];
+  if (a.shape() != b.shape() || a.dtype() != b.dtype()) NYI("%s: operands must have the same shape and type (no broadcasting)", who);
+  auto& be = backend();
+  int64_t rows, D;
+  rowsAndWidth(a, rows, D);
+  be.noteWrite(y.ptr<void>(), y.bytes());
+  void* image = want_image ? be.newImage(y.ptr<void>(), y.bytes(), (int)std::min<int64_t>(rows, 9), D) : nullptr;
+  MLLM_HIP_KERNEL_CHECK(fn(a.ptr<void>(), b.ptr<void>(), y.ptr<void>(), actType(a, who), rows, D, image, be.config().act_scale_mode,
+                           be.stream()));
+}
+// the residual sum feeds the next RMSNorm, not a Linear: no image
+void HipAddOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  binaryForward("HipAddOp", mllm_hip_add, inputs, outputs, false);
+}
+// silu(gate) * up feeds down_proj
+void HipMulOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  binaryForward("HipMulOp", mllm_hip_mul, inputs, outputs, true);
+}
+void HipSoftmaxOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  const auto& x = inputs[0];
+  const int axis = options_.axis < 0 ? options_.axis + (int)x.rank() : options_.axis;
+  if (axis != (int)x.rank() - 1 || x.dtype() != kFloat32) NYI("HipSoftmaxOp: fp32 over the last axis only");
+  auto& be = backend();
+  int64_t rows, len;
+  rowsAndWidth(x, rows, len);
+  be.noteWrite(outputs[0].ptr<void>(), outputs[0].bytes());
+  MLLM_HIP_KERNEL_CHECK(mllm_hip_softmax(x.ptr<float>(), outputs[0].ptr<float>(), rows, len, be.stream()));
+}
+void HipTopKOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  const auto& x = inputs[0];
+  const int dim = options_.dim < 0 ? options_.dim + (int)x.rank() : options_.dim;
+  if (dim != (int)x.rank() - 1 || x.dtype() != kFloat32) NYI("HipTopKOp: fp32 over the last axis only");
+  auto& be = backend();
+  int64_t rows, len;
+  rowsAndWidth(x, rows, len);
+  be.noteWrite(outputs[0].ptr<void>(), outputs[0].bytes());
+  be.noteWrite(outputs[1].ptr<void>(), outputs[1].bytes());
+  MLLM_HIP_KERNEL_CHECK(mllm_hip_topk(x.ptr<float>(), outputs[0].ptr<float>(), outputs[1].ptr<int32_t>(), rows, len, options_.k,
+                                      options_.largest, options_.sorted, be.stream()));
 }
 
 ParameterFile::ptr_t HipLinearOp::getParams() {

@@ -23,6 +23,8 @@ class HipAllocator final : public Allocator {
   size_t allocSize(Storage* storage) override;
   size_t allocSize(const Storage::ptr_t& storage) override { return allocSize(storage.get()); }
   [[nodiscard]] size_t alignSize() const override { return 256; }
+  // told about every free so that the backend can drop what it keeps about that memory; cleared when the backend goes
+  class HipBackend* owner = nullptr;
 };
 
 // How fp16 block scales are read (see MLLM_HIP_SCALE_* in the C header): IEEE bit patterns, or the x86 reference build's
@@ -35,6 +37,12 @@ struct HipBackendConfig {
   // gemm-packed copy of the weight is built at load()); false = the block-dot kernel, which keeps the reference's fp32
   // block arithmetic.  MLLM_HIP_PREFILL=blockdot selects the latter.
   bool prefill_matrix_cores = true;
+  // Decode hand-over: RMSNorm and the elementwise product also write the Q8_0 image of their result (up to 8 rows), and a
+  // Q4_0 / Q8_0 Linear that then reads exactly that tensor takes the image instead of quantizing in every workgroup.
+  // Results are bit-identical either way.  The image is dropped as soon as any op of this backend writes to, or the
+  // allocator frees, the memory it describes; writes that bypass the backend (a caller's own hipMemcpy into an
+  // activation tensor) are not seen, hence the switch: MLLM_HIP_FOLD_IMAGES=0 turns it off.
+  bool fold_images = true;
 };
 
 class HipBackend final : public Backend {
@@ -46,12 +54,29 @@ class HipBackend final : public Backend {
   void setScaleModes(int weight_scale_mode, int act_scale_mode) {
     cfg_.weight_scale_mode = weight_scale_mode;
     cfg_.act_scale_mode = act_scale_mode;
+    images_.clear();  // images carry the activation-scale convention they were written with
   }
   void synchronize() const;
+  void setFoldImages(bool on) { cfg_.fold_images = on; images_.clear(); }
+
+  // quantized images of activation tensors (see HipBackendConfig::fold_images)
+  void* newImage(const void* tensor_ptr, size_t tensor_bytes, int rows, int64_t D);  // null when not applicable
+  const void* findImage(const void* tensor_ptr, int rows, int64_t D) const;
+  void noteWrite(const void* ptr, size_t bytes);  // every op calls this for its outputs before it launches
+  [[nodiscard]] size_t imageCount() const { return images_.size(); }
 
  private:
+  struct Image {
+    const void* tensor_ptr;
+    size_t tensor_bytes;
+    int rows;
+    int64_t D;
+    Tensor data;
+  };
   HipBackendConfig cfg_;
   void* stream_ = nullptr;
+  std::vector<Image> images_;
+  std::vector<Tensor> image_pool_;  // buffers of dropped images, reused (no allocation in steady state)
 };
 
 // Registers backend + allocator with the Context (idempotent).  The counterpart of initOpenCLBackend() / initAscendBackend().
@@ -89,6 +114,35 @@ class HipMatMulOp final : public aops::MatMulOp {
 class HipMatMulOpFactory final : public TypedOpFactory<OpTypes::kMatMul, aops::MatMulOpOptions> {
  public:
   std::shared_ptr<BaseOp> createOpImpl(const aops::MatMulOpOptions& options) override { return std::make_shared<HipMatMulOp>(options); }
+};
+
+// ---- the operators around Linear (kernels: mllm_hip_rmsnorm, mllm_hip_silu, mllm_hip_add / _mul, mllm_hip_softmax, mllm_hip_topk)
+#define MLLM_HIP_SIMPLE_OP(Name, Base, Options, Type)                                                                     \
+  class Name final : public aops::Base {                                                                                   \
+   public:                                                                                                                 \
+    explicit Name(const aops::Options& options) : aops::Base(options) {}                                                   \
+    void forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;                                \
+  };                                                                                                                       \
+  class Name##Factory final : public TypedOpFactory<OpTypes::Type, aops::Options> {                                        \
+   public:                                                                                                                 \
+    std::shared_ptr<BaseOp> createOpImpl(const aops::Options& options) override { return std::make_shared<Name>(options); } \
+  };
+MLLM_HIP_SIMPLE_OP(HipSiLUOp, SiLUOp, SiLUOpOptions, kSiLU)
+MLLM_HIP_SIMPLE_OP(HipAddOp, AddOp, AddOpOptions, kAdd)
+MLLM_HIP_SIMPLE_OP(HipMulOp, MulOp, MulOpOptions, kMul)
+MLLM_HIP_SIMPLE_OP(HipSoftmaxOp, SoftmaxOp, SoftmaxOpOptions, kSoftmax)
+MLLM_HIP_SIMPLE_OP(HipTopKOp, TopKOp, TopKOpOptions, kTopK)
+#undef MLLM_HIP_SIMPLE_OP
+
+class HipRMSNormOp final : public aops::RMSNormOp {
+ public:
+  explicit HipRMSNormOp(const aops::RMSNormOpOptions& options) : aops::RMSNormOp(options) {}
+  void load(const ParameterFile::ptr_t& ploader) override;  // weight -> fp32 on the device
+  void forward(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+};
+class HipRMSNormOpFactory final : public TypedOpFactory<OpTypes::kRMSNorm, aops::RMSNormOpOptions> {
+ public:
+  std::shared_ptr<BaseOp> createOpImpl(const aops::RMSNormOpOptions& options) override { return std::make_shared<HipRMSNormOp>(options); }
 };
 
 class HipX2XOp final : public aops::X2XOp {

@@ -141,6 +141,93 @@ extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_linea
   return (int)y.dtype();
 }
 
+// The MLP half of a decoder layer through the op factories, operator by operator as the reference's modules call them
+// (mllm/models/qwen3/modeling_qwen3_fa2.hpp:85-92 inside Qwen3Decoder::forward): h = rms_norm(x); g = gate(h); u = up(h);
+// a = silu(g) * u; y = x + down(a).  Returns how many Linear inputs were handed over as quantized images (0 when
+// fold_images is off); softmax / top-k run on g as a side check of those two slots (values to sm_host / tk_* when given).
+extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_decoder_mlp(
+    int is_q8, const void* Wg, const void* Wu, const void* Wd, const float* norm_w, const void* x_host, int x_is_bf16, void* y_host,
+    int M, int H, int I, float eps, int fold_images, float* softmax_host, int32_t* topk_idx_host, int topk) {
+  initializeContext();
+  auto be = hip::initHipBackend();
+  be->setScaleModes(MLLM_HIP_SCALE_IEEE, MLLM_HIP_SCALE_X86_REF);
+  be->setFoldImages(fold_images != 0);
+  auto backend = Context::instance().getBackend(kHIP);
+  const DataTypes wdt = is_q8 ? kGGUF_Q8_0 : kGGUF_Q4_0;
+  auto params = ParameterFile::create(ModelFileVersion::kV2);
+  params->push("l.norm.weight", Tensor::fromExternal(const_cast<float*>(norm_w), {H}, kFloat32, kCPU));
+  params->push("l.gate.weight", Tensor::fromExternal(const_cast<void*>(Wg), {I, H}, wdt, kCPU));
+  params->push("l.up.weight", Tensor::fromExternal(const_cast<void*>(Wu), {I, H}, wdt, kCPU));
+  params->push("l.down.weight", Tensor::fromExternal(const_cast<void*>(Wd), {H, I}, wdt, kCPU));
+  auto make = [&](OpTypes t, const BaseOpOptionsBase& o, const std::string& name) {
+    auto op = backend->createOp(t, o);
+    op->setName(name);
+    op->load(params);
+    return op;
+  };
+  auto run = [&](const BaseOp::ptr_t& op, const std::vector<Tensor>& in) {
+    std::vector<Tensor> out;
+    op->reshape(in, out);
+    op->setup(in, out);
+    op->forward(in, out);
+    return out;
+  };
+  aops::RMSNormOpOptions no;
+  no.epsilon = eps;
+  aops::LinearOpOptions gu, dn;
+  gu.in_channels = H;
+  gu.out_channels = I;
+  dn.in_channels = I;
+  dn.out_channels = H;
+  auto norm = make(OpTypes::kRMSNorm, no, "l.norm");
+  auto gate = make(OpTypes::kLinear, gu, "l.gate");
+  auto up = make(OpTypes::kLinear, gu, "l.up");
+  auto down = make(OpTypes::kLinear, dn, "l.down");
+  auto silu = make(OpTypes::kSiLU, aops::SiLUOpOptions{}, "l.act");
+  auto mul = make(OpTypes::kMul, aops::MulOpOptions{}, "l.mul");
+  auto add = make(OpTypes::kAdd, aops::AddOpOptions{}, "l.add");
+
+  Tensor x = Tensor::fromExternal(const_cast<void*>(x_host), {M, H}, x_is_bf16 ? kBFloat16 : kFloat32, kCPU).to(kHIP);
+  int handed_over = 0;
+  Tensor h = run(norm, {x})[0];
+  handed_over += be->findImage(h.ptr<void>(), M, H) != nullptr;
+  Tensor g = run(gate, {h})[0];
+  handed_over += be->findImage(h.ptr<void>(), M, H) != nullptr;  // still there for the sibling projection
+  Tensor u = run(up, {h})[0];
+  Tensor s = run(silu, {g})[0];
+  Tensor a = run(mul, {s, u})[0];
+  handed_over += be->findImage(a.ptr<void>(), M, I) != nullptr;
+  Tensor d = run(down, {a})[0];
+  // Linear yields fp32; the residual stream of this harness is fp32 whenever x is
+  Tensor y = x_is_bf16 ? d : run(add, {d, x})[0];
+  Tensor yc = y.to(kCPU);
+  std::memcpy(y_host, yc.ptr<void>(), yc.bytes());
+  if (softmax_host) {
+    aops::SoftmaxOpOptions so;
+    so.axis = -1;
+    Tensor p = run(make(OpTypes::kSoftmax, so, "l.sm"), {g})[0];
+    Tensor pc = p.to(kCPU);
+    std::memcpy(softmax_host, pc.ptr<void>(), pc.bytes());
+    if (topk_idx_host) {
+      aops::TopKOpOptions to;
+      to.k = topk;
+      to.sorted = false;
+      auto vi = run(make(OpTypes::kTopK, to, "l.topk"), {p});
+      Tensor ic = vi[1].to(kCPU);
+      std::memcpy(topk_idx_host, ic.ptr<void>(), ic.bytes());
+    }
+  }
+  // an op that overwrites a tensor must drop that tensor's image
+  std::vector<Tensor> reuse{h};
+  norm->forward({x}, reuse);
+  const bool refreshed = !fold_images || M > 8 || be->findImage(h.ptr<void>(), M, H) != nullptr;
+  std::vector<Tensor> clobber{h};
+  silu->forward({h}, clobber);  // writes h in place
+  if (be->findImage(h.ptr<void>(), M, H) != nullptr || !refreshed) return -20;
+  be->synchronize();
+  return handed_over;
+}
+
 // fp32 MatMul through the kMatMul factory slot
 extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_matmul(const float* a_host, const float* b_host, float* c_host,
                                                                                   int M, int N, int K, int transpose_b) {

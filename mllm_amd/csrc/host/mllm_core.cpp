@@ -173,6 +173,17 @@ void MatMulOp::reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& o
   outputs.emplace_back(Tensor::empty(o, inputs[0].dtype(), inputs[0].device()));
 }
 
+void RMSNormOp::reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  outputs.emplace_back(Tensor::empty(inputs[0].shape(), inputs[0].dtype(), inputs[0].device()));
+}
+void TopKOp::reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
+  auto shape = inputs[0].shape();
+  const int dim = options_.dim < 0 ? options_.dim + (int)shape.size() : options_.dim;
+  MLLM_RT_ASSERT(dim >= 0 && dim < (int)shape.size() && options_.k >= 1 && options_.k <= shape[dim]);
+  shape[dim] = options_.k;
+  outputs.emplace_back(Tensor::empty(shape, inputs[0].dtype(), inputs[0].device()));
+  outputs.emplace_back(Tensor::empty(shape, kInt32, inputs[0].device()));
+}
 void X2XOp::reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) {
   outputs.emplace_back(Tensor::empty(inputs[0].shape(), inputs[0].dtype(), options_.device));
 }

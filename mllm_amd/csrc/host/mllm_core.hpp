@@ -63,7 +63,11 @@ enum DeviceTypes : int32_t {
   kDeviceTypes_End,
 };
 
-enum class OpTypes : int32_t { kOpType_Start = 0, kMatMul = 6, kLinear = 8, kX2X = 19, kGraphBegin = 55, kGraphEnd = 56, kDynamicOp_Start = 4096 };
+// values as in mllm/core/OpTypes.hpp:13-70 (only the slots this backend fills)
+enum class OpTypes : int32_t {
+  kOpType_Start = 0, kAdd = 2, kMul = 4, kMatMul = 6, kLinear = 8, kSoftmax = 10, kRMSNorm = 14, kSiLU = 15, kX2X = 19, kTopK = 49,
+  kGraphBegin = 55, kGraphEnd = 56, kDynamicOp_Start = 4096
+};
 
 enum class ModelFileVersion : int32_t { kV1 = 1, kV2 = 2, kUserTemporary = 3 };
 
@@ -283,6 +287,60 @@ class X2XOp : public BaseOp {
 
  protected:
   X2XOpOptions options_;
+};
+
+// ---- the operators around Linear in a decoder layer (mllm/core/aops/{RMSNormOp,SiLUOp,ElewiseOps,SoftmaxOp,TopKOp}.hpp) ----
+struct RMSNormOpOptions : public BaseOpOptions<RMSNormOpOptions> {
+  float epsilon = 1e-6f;
+  bool add_unit_offset = false;  // Gemma
+};
+class RMSNormOp : public BaseOp {
+ public:
+  explicit RMSNormOp(const RMSNormOpOptions& options) : BaseOp(OpTypes::kRMSNorm), options_(options) {}
+  void load(const ParameterFile::ptr_t& ploader) override { weight_ = ploader->pull(getName() + ".weight"); }  // aops/RMSNormOp.cpp:16-30
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;
+  inline Tensor& weight() { return weight_; }
+  inline const RMSNormOpOptions& options() const { return options_; }
+
+ protected:
+  Tensor weight_;
+  RMSNormOpOptions options_;
+};
+struct SiLUOpOptions : public BaseOpOptions<SiLUOpOptions> {};
+struct AddOpOptions : public BaseOpOptions<AddOpOptions> {};
+struct MulOpOptions : public BaseOpOptions<MulOpOptions> {};
+// output = the first input's shape and type (no broadcasting in this backend: both inputs must have the same shape)
+template <OpTypes T, typename OptT>
+class SameShapeOp : public BaseOp {
+ public:
+  explicit SameShapeOp(const OptT& options) : BaseOp(T), options_(options) {}
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override {
+    outputs.emplace_back(Tensor::empty(inputs[0].shape(), inputs[0].dtype(), inputs[0].device()));
+  }
+
+ protected:
+  OptT options_;
+};
+using SiLUOp = SameShapeOp<OpTypes::kSiLU, SiLUOpOptions>;
+using AddOp = SameShapeOp<OpTypes::kAdd, AddOpOptions>;
+using MulOp = SameShapeOp<OpTypes::kMul, MulOpOptions>;
+struct SoftmaxOpOptions : public BaseOpOptions<SoftmaxOpOptions> {
+  int axis = -1;
+};
+using SoftmaxOp = SameShapeOp<OpTypes::kSoftmax, SoftmaxOpOptions>;
+struct TopKOpOptions : public BaseOpOptions<TopKOpOptions> {
+  int k = 0;
+  int dim = -1;
+  bool largest = true;
+  bool sorted = true;
+};
+class TopKOp : public BaseOp {
+ public:
+  explicit TopKOp(const TopKOpOptions& options) : BaseOp(OpTypes::kTopK), options_(options) {}
+  void reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>& outputs) override;  // values (input type), indices int32
+
+ protected:
+  TopKOpOptions options_;
 };
 
 }  // namespace aops

@@ -528,13 +528,13 @@ MLLM_API int mllm_hip_silu(const void* x, void* y, int dtype, int64_t n, void* s
   if (n <= 0 || n % 8) return n <= 0 ? MLLM_HIP_E_BADARG : MLLM_HIP_E_SHAPE;
   return launch_elementwise<EW_SILU>(x, nullptr, y, dtype, n / 8, 8, nullptr, 0, stream);
 }
-MLLM_API int mllm_hip_add(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream) {
-  if (n <= 0 || n % 8) return n <= 0 ? MLLM_HIP_E_BADARG : MLLM_HIP_E_SHAPE;
-  return launch_elementwise<EW_ADD>(a, b, y, dtype, n / 8, 8, nullptr, 0, stream);
+MLLM_API int mllm_hip_add(const void* a, const void* b, void* y, int dtype, int64_t rows, int64_t D, void* q_image,
+                          int act_scale_mode, void* stream) {
+  return launch_elementwise<EW_ADD>(a, b, y, dtype, rows, D, q_image, act_scale_mode, stream);
 }
-MLLM_API int mllm_hip_mul(const void* a, const void* b, void* y, int dtype, int64_t n, void* stream) {
-  if (n <= 0 || n % 8) return n <= 0 ? MLLM_HIP_E_BADARG : MLLM_HIP_E_SHAPE;
-  return launch_elementwise<EW_MUL>(a, b, y, dtype, n / 8, 8, nullptr, 0, stream);
+MLLM_API int mllm_hip_mul(const void* a, const void* b, void* y, int dtype, int64_t rows, int64_t D, void* q_image,
+                          int act_scale_mode, void* stream) {
+  return launch_elementwise<EW_MUL>(a, b, y, dtype, rows, D, q_image, act_scale_mode, stream);
 }
 MLLM_API int mllm_hip_silu_mul(const void* gate, const void* up, void* y, int dtype, int64_t rows, int64_t D, void* q_image,
                                int act_scale_mode, void* stream) {

@@ -415,19 +415,22 @@ def rmsnorm(x, weight, eps, add_unit_offset=False, want_image=False, act_scale_m
     return (y, img) if want_image else y
 
 
-def _binary(fn, name, a, b):
+def _binary(fn, name, a, b, want_image, act_scale_mode):
     assert a.is_cuda and a.is_contiguous() and b.is_contiguous() and a.shape == b.shape and a.dtype == b.dtype
+    D = a.shape[-1]
+    rows = a.numel() // D
     y = torch.empty_like(a)
-    _lib.check(fn(a.data_ptr(), b.data_ptr(), y.data_ptr(), _xdtype(a), a.numel(), _stream()), name)
-    return y
+    img = gemv_workspace(rows, D) if want_image else None
+    _lib.check(fn(a.data_ptr(), b.data_ptr(), y.data_ptr(), _xdtype(a), rows, D, _p(img), act_scale_mode, _stream()), name)
+    return (y, img) if want_image else y
 
 
-def add(a, b):
-    return _binary(_lib.lib().mllm_hip_add, "mllm_hip_add", a, b)
+def add(a, b, want_image=False, act_scale_mode=SCALE_X86_REF):
+    return _binary(_lib.lib().mllm_hip_add, "mllm_hip_add", a, b, want_image, act_scale_mode)
 
 
-def mul(a, b):
-    return _binary(_lib.lib().mllm_hip_mul, "mllm_hip_mul", a, b)
+def mul(a, b, want_image=False, act_scale_mode=SCALE_X86_REF):
+    return _binary(_lib.lib().mllm_hip_mul, "mllm_hip_mul", a, b, want_image, act_scale_mode)
 
 
 def silu(x):

@@ -125,6 +125,12 @@ def test_silu_mul_image(M, D):
     y, img = ql.silu_mul(g, u, want_image=True, act_scale_mode=ql.SCALE_X86_REF)
     assert torch.equal(y, ql.silu_mul(g, u))
     _check_image(img, y.cpu().numpy(), M, D, True)
+    # the product alone can write the image too (the reference runs SiLU and the product as two operators)
+    y2, img2 = ql.mul(ql.silu(g), u, want_image=True)
+    assert torch.equal(y2, y)
+    _check_image(img2, y.cpu().numpy(), M, D, True)
+    y3, img3 = ql.add(g, u, want_image=True, act_scale_mode=ql.SCALE_IEEE)
+    _check_image(img3, y3.cpu().numpy(), M, D, False)
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
@@ -243,7 +249,7 @@ def test_argument_checks():
     assert L.mllm_hip_rmsnorm(p + 4, 0, p, p, 1, 8, 1e-6, 0, None, 0, None) == -3
     assert L.mllm_hip_rmsnorm(None, 0, p, p, 1, 8, 1e-6, 0, None, 0, None) == -1
     assert L.mllm_hip_silu(p, p, 0, 12, None) == -2
-    assert L.mllm_hip_add(p, None, p, 0, 8, None) == -1
+    assert L.mllm_hip_add(p, None, p, 0, 1, 8, None, 0, None) == -1
     assert L.mllm_hip_topk(p, p, p, 1, 8, 9, 1, 1, None) == -2
     assert L.mllm_hip_topk(p, p, p, 1, 8, 0, 1, 1, None) == -2
     assert L.mllm_hip_softmax(p, None, 1, 8, None) == -1

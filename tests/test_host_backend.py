@@ -243,3 +243,45 @@ def test_linear_from_model_file(tmp_path, version):
                                                 y.ctypes.data_as(C.c_void_p), M, 0, 1)
         assert rc == 0  # kFloat32
         assert rel_l2(y, orc.linear_q(x, W, wtype, bias, orc.SCALE_X86_REF)) < 2e-6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("is_q8", [0, 1])
+def test_decoder_mlp_through_the_op_factories(is_q8):
+    """RMSNorm -> gate/up Linear -> SiLU -> Mul -> down Linear -> Add created through Backend::createOp: the oracle's chain
+    within tolerance; with the image hand-over on, three Linear inputs arrive as quantized images and the result is the
+    same bit for bit; softmax and top-k slots checked on the side"""
+    from oracle import oracle as orc
+    from gpu_util import announce, rel_l2
+    L = _host()
+    rng = synth.rng_for(5, 60 + is_q8)
+    H, I, k = 256, 512, 4
+    Wg, Wu, Wd = (synth.make_weight(rng, is_q8, I, H), synth.make_weight(rng, is_q8, I, H), synth.make_weight(rng, is_q8, H, I))
+    nw = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    vp = lambda a: a.ctypes.data_as(C.c_void_p)
+    for M in (1, 4, 8, 12):
+        x = synth.make_x_fp32(rng, M, H)
+        ys, handed = [], []
+        sm = np.empty((M, I), np.float32)
+        ti = np.empty((M, k), np.int32)
+        for fold in (0, 1):
+            y = np.empty((M, H), np.float32)
+            announce("decoder mlp", is_q8, M, "fold", fold)
+            rc = L.mllm_hip_backend_run_decoder_mlp(is_q8, vp(Wg), vp(Wu), vp(Wd), vp(nw), vp(x), 0, vp(y), M, H, I, C.c_float(1e-6), fold,
+                                                    vp(sm), vp(ti), k)
+            assert rc >= 0, rc
+            ys.append(y)
+            handed.append(rc)
+        assert handed == [0, 3 if M <= 8 else 0]
+        assert np.array_equal(ys[0], ys[1])
+        h = orc.rmsnorm(x, nw, 1e-6)
+        g = orc.linear_q(h, Wg, is_q8, None, orc.SCALE_X86_REF)
+        a = orc.silu(g) * orc.linear_q(h, Wu, is_q8, None, orc.SCALE_X86_REF)
+        want = orc.linear_q(a, Wd, is_q8, None, orc.SCALE_X86_REF) + x
+        # up to 8 rows every Linear is the fp32 block arithmetic.  More rows: the matrix-core Linear (fp16 operands, 2e-4 per
+        # Linear on identical inputs, its own test); in a CHAIN the Q8_0 re-quantization in front of down_proj turns a
+        # perturbation eps of its input into about sqrt(eps * 0.026) (codes flip at rounding boundaries), so the chain
+        # is compared at 5e-3 and MLLM_HIP_PREFILL=blockdot keeps the fp32 arithmetic where that matters
+        assert rel_l2(ys[0], want) < (1e-3 if M <= 8 else 5e-3)
+        assert rel_l2(sm, orc.softmax(g)) < 1e-3
+        assert np.array_equal(ti, orc.topk(sm, k, True, False)[1])
