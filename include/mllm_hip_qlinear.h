@@ -30,6 +30,9 @@ extern "C" {
 
 /* weight block formats: mllm/core/DataTypes.hpp:110-121 (block_q4_0, 18 B), :164-170 (block_q8_0, 34 B) */
 enum { MLLM_HIP_Q4_0 = 0, MLLM_HIP_Q8_0 = 1 };
+/* super-block formats of 256 weights: mllm/core/DataTypes.hpp:139-147 (block_q4_K, 144 B), :153-160 (block_q6_K, 210 B);
+ * only the mllm_hip_kq_* / mllm_hip_linear_kq entry points take them */
+enum { MLLM_HIP_Q4_K = 2, MLLM_HIP_Q6_K = 3 };
 /* activation element types */
 enum { MLLM_HIP_F32 = 0, MLLM_HIP_BF16 = 1 };
 /* instead of activations: their Q8_0 image as the decode GEMV reads it (mllm_hip_gemv_workspace_bytes, written by
@@ -268,6 +271,26 @@ int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed
  * replaces: the histogram + argsort at modeling_qwen3_moe_fa2.hpp:178-197 */
 int mllm_hip_moe_route(const int32_t* topk_ids, int64_t T, int E, int k, int32_t* counts, int32_t* offsets,
                        int32_t* sorted_idx, void* workspace, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------
+ * Q4_K / Q6_K Linear (weights in super-blocks of 256, activations quantized to Q8_K inside the kernel)
+ * replaces: CPULinearOp::forward -> ggml::mat_mul generic branch -> quantize_row_q8_K + vec_dot_q4_K_q8_K / vec_dot_q6_K_q8_K
+ *           mllm/backends/cpu/kernels/common/ggml/matmul.cpp:147-189,300-360, vec_dot.cpp:498-560,955-1044,
+ *           quantize/quantize_q8.cpp:215-248
+ * ------------------------------------------------------------------------------------------------------- */
+
+/* Load-time repack of reference blocks [N][K/256] (144 / 210 bytes each, any alignment) into planes of 16-byte records.
+ * weight_scale_mode as for mllm_hip_q_prepack (how the fp16 fields d / dmin are read).  packed: 256-byte aligned. */
+size_t mllm_hip_kq_packed_bytes(int wtype, int64_t N, int64_t K);
+int mllm_hip_kq_prepack(int wtype, const void* blocks, int weight_scale_mode, void* packed, int64_t N, int64_t K, void* stream);
+/* y[M][N] fp32 = x[M][K] (fp32 or bf16) * W^T + bias.  K % 256 == 0.  Up to eight rows per launch (decode); more rows run
+ * as groups of eight, each streaming the weights again. */
+int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y, int64_t M, int64_t N,
+                       int64_t K, void* stream);
+/* Parity probes.  Dequantized weights fp32 [N][K] (dequantize_row_q4_K / _q6_K, quantize_q4.cpp:284-312, quantize_q6.cpp:108-133);
+ * Q8_K activation quantization: codes int8 [M][K], d fp32 [M][K/256], sums of 16 codes int16 [M][K/16]. */
+int mllm_hip_kq_dequantize(int wtype, const void* packed, float* w, int64_t N, int64_t K, void* stream);
+int mllm_hip_quantize_q8_K(const void* x, int x_dtype, int8_t* codes, float* d, int16_t* bsums, int64_t M, int64_t K, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------
  * The operators either side of a quantized Linear in a decoder layer.  dtype: MLLM_HIP_F32 or MLLM_HIP_BF16 (arithmetic

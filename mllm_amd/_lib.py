@@ -64,6 +64,12 @@ def lib():
         L.mllm_hip_topk.argtypes = [vp, vp, vp, i64, i64, ci, ci, ci, vp]
         L.mllm_hip_moe_gate.argtypes = [vp, ci, vp, vp, vp, vp, i64, i64, i64, ci, ci, vp]
         L.mllm_hip_quantize_q8_0.argtypes = [vp, ci, vp, vp, i64, i64, vp]
+        L.mllm_hip_kq_packed_bytes.restype = C.c_size_t
+        L.mllm_hip_kq_packed_bytes.argtypes = [ci, i64, i64]
+        L.mllm_hip_kq_prepack.argtypes = [ci, vp, ci, vp, i64, i64, vp]
+        L.mllm_hip_linear_kq.argtypes = [ci, vp, vp, ci, vp, vp, i64, i64, i64, vp]
+        L.mllm_hip_kq_dequantize.argtypes = [ci, vp, vp, i64, i64, vp]
+        L.mllm_hip_quantize_q8_K.argtypes = [vp, ci, vp, vp, vp, i64, i64, vp]
         L.mllm_hip_q_dequantize.argtypes = [ci, vp, vp, i64, i64, vp]
         L.mllm_hip_q_block_isums.argtypes = [ci, vp, vp, vp, i64, i64, i64, vp]
         L.mllm_hip_probe_copy.argtypes = [vp, vp, C.c_size_t, vp]

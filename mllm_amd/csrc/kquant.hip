@@ -1,0 +1,526 @@
+// Q4_K / Q6_K Linear for gfx950: super-block formats of 256 weights with Q8_K activations (the formats the shipped
+// Qwen3-MoE recipe quantizes to).  Decode GEMV for up to eight activation rows; more rows run as groups of eight.
+//
+// Arithmetic follows the reference's x86 CPU path:
+//   activation quantization  quantize_row_q8_K_reference   mllm/backends/cpu/kernels/common/ggml/quantize/quantize_q8.cpp:215-248
+//   Q4_K dot                 vec_dot_q4_K_q8_K (AVX2)       mllm/backends/cpu/kernels/common/ggml/vec_dot.cpp:498-560
+//   Q6_K dot                 vec_dot_q6_K_q8_K (AVX2)       mllm/backends/cpu/kernels/common/ggml/vec_dot.cpp:955-1044
+//   dequantization probes    dequantize_row_q4_K / _q6_K    quantize_q4.cpp:284-312, quantize_q6.cpp:108-133
+//   call site                ggml::mat_mul generic branch    mllm/backends/cpu/kernels/common/ggml/matmul.cpp:147-189,300-360
+// The integer work (codes, sums of 16, sub-block-scaled dot products per super-block) is exact; the fp32 accumulation
+// runs per lane and is reduced over the lanes of a row, a different order than the CPU's eight lanes.
+//
+// HBM-bound like the Q4_0 / Q8_0 GEMV: a launch streams 144 (Q4_K) or 210 (Q6_K) bytes per 256 weights once, as 16-byte
+// loads that are contiguous across the lanes of a group.  The reference's array-of-structures blocks (210 is not even a
+// multiple of 4) are split at load time into planes of 16-byte records.
+#include "qcommon.h"
+
+#define QK_K 256
+
+namespace mllmhip {
+
+// ---- packed layout ---------------------------------------------------------------------------------------------------
+// Q4_K: plane A = nibbles, 128 B per super-block (eight 16-byte chunks); plane S = {fp16 d, fp16 dmin, 12 B of 6-bit scales
+//       and mins} = 16 B per super-block, fp16 fields as IEEE patterns.
+// Q6_K: plane A = low nibbles (128 B per super-block), plane H = high bit pairs (64 B), plane S = 16 int8 scales, plane D =
+//       fp16 d as IEEE pattern (2 B).
+struct KView {
+  const u32x4* a;
+  const u32x4* h;
+  const u32x4* s;
+  const uint16_t* d;
+};
+__host__ __device__ inline size_t kq_plane(size_t bytes) { return align_up(bytes, 256); }
+__host__ __device__ inline size_t kq_packed_bytes(int wtype, int64_t N, int64_t K) {
+  const size_t sb = (size_t)N * (K / QK_K);
+  if (wtype == MLLM_HIP_Q4_K) return kq_plane(sb * 128) + kq_plane(sb * 16);
+  return kq_plane(sb * 128) + kq_plane(sb * 64) + kq_plane(sb * 16) + kq_plane(sb * 2);
+}
+__host__ __device__ inline KView kq_view(int wtype, const void* packed, int64_t N, int64_t K) {
+  const size_t sb = (size_t)N * (K / QK_K);
+  const char* p = reinterpret_cast<const char*>(packed);
+  KView v{};
+  v.a = reinterpret_cast<const u32x4*>(p);
+  p += kq_plane(sb * 128);
+  if (wtype == MLLM_HIP_Q6_K) {
+    v.h = reinterpret_cast<const u32x4*>(p);
+    p += kq_plane(sb * 64);
+  }
+  v.s = reinterpret_cast<const u32x4*>(p);
+  p += kq_plane(sb * 16);
+  v.d = reinterpret_cast<const uint16_t*>(p);
+  return v;
+}
+
+// what an fp16 field reads as: the IEEE pattern itself, or (files of the x86 build) the number stored there taken as
+// the pattern
+__device__ __forceinline__ uint16_t field_bits(const uint8_t* p, int x86) {
+  const uint16_t raw = (uint16_t)p[0] | ((uint16_t)p[1] << 8);
+  if (!x86) return raw;
+  const float num = f16bits_to_f32(raw);
+  return (num >= 0.f && num < 65536.f) ? (uint16_t)(uint32_t)num : (uint16_t)0;
+}
+__device__ __forceinline__ uint32_t bytes_u32(const uint8_t* p) {
+  return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+
+// one thread per 16-byte record of plane A (Q4_K: 8 per super-block; Q6_K: 8 per super-block); thread 0 of a super-block
+// also writes the small planes
+__global__ void kq_prepack_kernel(int wtype, const uint8_t* __restrict__ blocks, int x86, KView v, int64_t nsb_total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t sb = i >> 3;
+  const int c = (int)(i & 7);
+  if (sb >= nsb_total) return;
+  u32x4* A = const_cast<u32x4*>(v.a);
+  u32x4* S = const_cast<u32x4*>(v.s);
+  if (wtype == MLLM_HIP_Q4_K) {
+    const uint8_t* b = blocks + sb * 144;
+    const uint8_t* q = b + 16 + 16 * c;
+    A[sb * 8 + c] = u32x4{bytes_u32(q), bytes_u32(q + 4), bytes_u32(q + 8), bytes_u32(q + 12)};
+    if (c == 0) {
+      const uint32_t dd = (uint32_t)field_bits(b, x86) | ((uint32_t)field_bits(b + 2, x86) << 16);
+      S[sb] = u32x4{dd, bytes_u32(b + 4), bytes_u32(b + 8), bytes_u32(b + 12)};
+    }
+  } else {
+    const uint8_t* b = blocks + sb * 210;
+    const uint8_t* q = b + 16 * c;
+    A[sb * 8 + c] = u32x4{bytes_u32(q), bytes_u32(q + 4), bytes_u32(q + 8), bytes_u32(q + 12)};
+    if (c < 4) {
+      const uint8_t* hq = b + 128 + 16 * c;
+      const_cast<u32x4*>(v.h)[sb * 4 + c] = u32x4{bytes_u32(hq), bytes_u32(hq + 4), bytes_u32(hq + 8), bytes_u32(hq + 12)};
+    }
+    if (c == 0) {
+      const uint8_t* s = b + 192;
+      S[sb] = u32x4{bytes_u32(s), bytes_u32(s + 4), bytes_u32(s + 8), bytes_u32(s + 12)};
+      const_cast<uint16_t*>(v.d)[sb] = field_bits(b + 208, x86);
+    }
+  }
+}
+
+// ---- scale decoding ----------------------------------------------------------------------------------------------------
+// the 6-bit scales and mins of a Q4_K super-block as bytes: sc[0..7] in (lo, hi) of `sc`, mins likewise
+// (get_scale_min_k4, quantize.hpp; the same bit shuffle as vec_dot.cpp:507-512)
+struct K4Scales {
+  uint32_t sc0, sc1, mn0, mn1;
+};
+__device__ __forceinline__ K4Scales k4_scales(uint32_t u0, uint32_t u1, uint32_t u2) {
+  K4Scales r;
+  r.mn1 = ((u2 >> 4) & 0x0f0f0f0fu) | (((u1 >> 6) & 0x03030303u) << 4);
+  r.mn0 = u1 & 0x3f3f3f3fu;
+  r.sc1 = (u2 & 0x0f0f0f0fu) | (((u0 >> 6) & 0x03030303u) << 4);
+  r.sc0 = u0 & 0x3f3f3f3fu;
+  return r;
+}
+__device__ __forceinline__ int byte_of(uint32_t lo, uint32_t hi, int k) {  // k = 0..7
+  return (int)(((k < 4 ? lo : hi) >> (8 * (k & 3))) & 0xffu);
+}
+
+// ---- dequantization probe ------------------------------------------------------------------------------------------------
+__global__ void kq_dequantize_kernel(int wtype, KView v, float* __restrict__ w, int64_t nsb_total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // one thread per element
+  const int64_t sb = i >> 8;
+  const int e = (int)(i & 255);
+  if (sb >= nsb_total) return;
+  const uint8_t* A = reinterpret_cast<const uint8_t*>(v.a) + sb * 128;
+  if (wtype == MLLM_HIP_Q4_K) {
+    const u32x4 s = v.s[sb];
+    const float d = f16bits_to_f32((uint16_t)(s.x & 0xffff)), mn = f16bits_to_f32((uint16_t)(s.x >> 16));
+    const K4Scales k = k4_scales(s.y, s.z, s.w);
+    const int j = e >> 5, l = e & 31;  // sub-block, element
+    const int q = (j & 1) ? (A[32 * (j >> 1) + l] >> 4) : (A[32 * (j >> 1) + l] & 0xF);
+    const float d1 = d * (float)byte_of(k.sc0, k.sc1, j), m1 = mn * (float)byte_of(k.mn0, k.mn1, j);
+    w[i] = d1 * (float)q - m1;
+  } else {
+    const uint8_t* H = reinterpret_cast<const uint8_t*>(v.h) + sb * 64;
+    const int8_t* sc = reinterpret_cast<const int8_t*>(v.s) + sb * 16;
+    const int n = e >> 7, r = e & 127, g = r >> 5, l = r & 31;
+    int lo = A[64 * n + ((g & 1) ? 32 : 0) + l];
+    lo = (g >= 2) ? (lo >> 4) : (lo & 0xF);
+    const int hi = (H[32 * n + l] >> (2 * g)) & 3;
+    const int q = (int)(int8_t)(lo | (hi << 4)) - 32;
+    const float d = f16bits_to_f32(v.d[sb]);
+    w[i] = d * (float)sc[e >> 4] * (float)q;
+  }
+}
+
+// ---- Q8_K quantization of activations ---------------------------------------------------------------------------------------
+// 32 neighbouring lanes (half a wave) hold one super-block, eight consecutive elements per lane.  The reference takes the
+// element of largest magnitude WITH its sign, the first one when several are equal: the reduction carries the lane it came
+// from.  Outputs of a lane: its eight codes (two dwords), the sum of its eight codes, the block scale.
+struct Q8KItem {
+  uint32_t q0, q1;
+  int sum8;
+  float d;
+};
+__device__ __forceinline__ Q8KItem quantize_q8k_item(const float (&v)[8], int lane) {
+  float amax = 0.f, mx = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) {
+    const float ax = fabsf(v[e]);
+    if (ax > amax) {
+      amax = ax;
+      mx = v[e];
+    }
+  }
+  int src = lane;
+#pragma unroll
+  for (int off = 1; off < 32; off <<= 1) {
+    const float oa = __shfl_xor(amax, off, 64);
+    const float om = __shfl_xor(mx, off, 64);
+    const int os = __shfl_xor(src, off, 64);
+    if (oa > amax || (oa == amax && os < src)) {
+      amax = oa;
+      mx = om;
+      src = os;
+    }
+  }
+  Q8KItem r{0u, 0u, 0, 0.f};
+  if (amax == 0.f) return r;
+  const float iscale = -128.f / mx;
+  int sum = 0;
+  uint32_t pk[2];
+#pragma unroll
+  for (int w = 0; w < 2; w++) {
+    uint32_t p = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      int q = (int)rintf(iscale * v[4 * w + e]);
+      q = min(127, q);
+      sum += q;
+      p |= ((uint32_t)q & 0xffu) << (8 * e);
+    }
+    pk[w] = p;
+  }
+  r.q0 = pk[0];
+  r.q1 = pk[1];
+  r.sum8 = sum;
+  r.d = 1.f / iscale;
+  return r;
+}
+
+template <int XT>
+__device__ __forceinline__ void load8(const void* x, int64_t elem, float (&v)[8]) {
+  if (XT == MLLM_HIP_F32) {
+    const f32x4* p = reinterpret_cast<const f32x4*>(reinterpret_cast<const float*>(x) + elem);
+    const f32x4 a = p[0], b = p[1];
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  } else {
+    const u32x4 r = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(x) + elem);
+    const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+      v[2 * j + 0] = __uint_as_float(w[j] << 16);
+      v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+    }
+  }
+}
+
+// stand-alone form (parity probe): codes int8 [M][K], d fp32 [M][K/256], sums of 16 int16 [M][K/16]
+__global__ __launch_bounds__(256) void quantize_q8k_kernel(const void* __restrict__ x, int x_dtype, int8_t* __restrict__ codes,
+                                                           float* __restrict__ d, int16_t* __restrict__ bsums, int64_t nitems) {
+  const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;  // nitems is a multiple of 32: whole half-waves
+  if (it >= nitems) return;
+  float v[8];
+  if (x_dtype == MLLM_HIP_F32) load8<MLLM_HIP_F32>(x, it * 8, v);
+  else load8<MLLM_HIP_BF16>(x, it * 8, v);
+  const Q8KItem r = quantize_q8k_item(v, threadIdx.x & 63);
+  *reinterpret_cast<u32x2*>(codes + it * 8) = u32x2{r.q0, r.q1};
+  const int s16 = r.sum8 + __builtin_amdgcn_update_dpp(0, r.sum8, 0xB1, 0xf, 0xf, true);  // with the neighbouring lane
+  if ((it & 1) == 0) bsums[it >> 1] = (int16_t)s16;
+  if ((it & 31) == 0) d[it >> 5] = r.d;
+}
+
+// ---- GEMV -------------------------------------------------------------------------------------------------------------
+struct KGemvArgs {
+  KView w;
+  const float* bias;
+  float* y;
+  const void* x;
+  int N, M, nsb;  // nsb = K / 256
+};
+#define KBUF_OOB 0xffffffffu
+#define KBUF_NT 2
+
+// A unit = what one lane takes per step.  Q4_K: one 16-byte chunk of nibbles = 32 weights (eight units per super-block).
+// Q6_K: one 16-byte chunk of high bits with its two chunks of low nibbles = 64 weights (four units per super-block).
+template <int WT>
+struct KUnit {
+  u32x4 a, b, h, s;
+  uint16_t d;
+};
+struct KRsrc {
+  __amdgpu_buffer_rsrc_t a, h, s, d;
+};
+
+template <int WT>
+__device__ __forceinline__ void load_unit(KUnit<WT>& u, const KRsrc& r, uint32_t sb_base, int unit, int units, bool row_ok) {
+  const bool ok = row_ok && unit < units;
+  if (WT == MLLM_HIP_Q4_K) {
+    const uint32_t sb = sb_base + (uint32_t)(unit >> 3);
+    u.a = __builtin_amdgcn_raw_buffer_load_b128(r.a, ok ? (sb * 8u + (uint32_t)(unit & 7)) * 16u : KBUF_OOB, 0, KBUF_NT);
+    u.s = __builtin_amdgcn_raw_buffer_load_b128(r.s, ok ? sb * 16u : KBUF_OOB, 0, KBUF_NT);
+  } else {
+    const uint32_t sb = sb_base + (uint32_t)(unit >> 2);
+    const uint32_t n = (uint32_t)(unit >> 1) & 1u, t = (uint32_t)unit & 1u;
+    u.a = __builtin_amdgcn_raw_buffer_load_b128(r.a, ok ? (sb * 8u + 4u * n + t) * 16u : KBUF_OOB, 0, KBUF_NT);
+    u.b = __builtin_amdgcn_raw_buffer_load_b128(r.a, ok ? (sb * 8u + 4u * n + 2u + t) * 16u : KBUF_OOB, 0, KBUF_NT);
+    u.h = __builtin_amdgcn_raw_buffer_load_b128(r.h, ok ? (sb * 4u + 2u * n + t) * 16u : KBUF_OOB, 0, KBUF_NT);
+    u.s = __builtin_amdgcn_raw_buffer_load_b128(r.s, ok ? sb * 16u : KBUF_OOB, 0, KBUF_NT);
+    u.d = __builtin_amdgcn_raw_buffer_load_b16(r.d, ok ? sb * 2u : KBUF_OOB, 0, KBUF_NT);
+  }
+}
+
+__device__ __forceinline__ int dot16(const u32x4& w, const u32x4& x) {
+  int acc = __builtin_amdgcn_sdot4((int)w.x, (int)x.x, 0, false);
+  acc = __builtin_amdgcn_sdot4((int)w.y, (int)x.y, acc, false);
+  acc = __builtin_amdgcn_sdot4((int)w.z, (int)x.z, acc, false);
+  acc = __builtin_amdgcn_sdot4((int)w.w, (int)x.w, acc, false);
+  return acc;
+}
+__device__ __forceinline__ int half16(uint32_t pair, int hi) { return (int)(int16_t)(hi ? (pair >> 16) : (pair & 0xffffu)); }
+
+// Workgroup = NW waves; a wave is cut into 64 / G groups of G lanes; a group owns R consecutive weight rows and its lanes
+// stride over the row's units.  x is quantized to Q8_K once per workgroup into LDS: codes [MT][K], scales [MT][nsb], sums
+// of 16 as int16 [MT][nsb][16].
+template <int WT, int XT, int MT, int G, int R>
+__global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int nsb = a.nsb;
+  const int K = nsb * QK_K;
+  u32x4* s_q = reinterpret_cast<u32x4*>(smem);                         // [MT][K / 16]
+  uint32_t* s_bs = reinterpret_cast<uint32_t*>(smem + (size_t)MT * K);  // [MT][nsb][8] pairs of int16 (sums of 16)
+  float* s_d = reinterpret_cast<float*>(s_bs + (size_t)MT * nsb * 8);   // [MT][nsb]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int GROUPS = 64 / G;
+  const int grp = lane / G, c0 = lane % G;
+  const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (GROUPS * R) + (int64_t)grp * R;
+  constexpr int UPS = WT == MLLM_HIP_Q4_K ? 8 : 4;  // units per super-block
+  const int units = nsb * UPS;
+
+  KRsrc rs;
+  {
+    const uint32_t sbt = (uint32_t)a.N * (uint32_t)nsb;
+    rs.a = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(a.w.a), 0, sbt * 128u, 0x00020000);
+    rs.h = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(WT == MLLM_HIP_Q6_K ? a.w.h : a.w.a), 0, sbt * 64u, 0x00020000);
+    rs.s = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(a.w.s), 0, sbt * 16u, 0x00020000);
+    rs.d = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.w.d), 0, sbt * 2u, 0x00020000);
+  }
+  // first trip of weight loads goes out before the activations are touched
+  KUnit<WT> cur[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) load_unit<WT>(cur[r], rs, (uint32_t)((row0 + r) * nsb), c0, units, row0 + r < a.N);
+
+  // ---- activations -> Q8_K in LDS (rows m >= M are zero) ----
+  const int nitems = MT * (K >> 3);
+  const int valid = a.M * (K >> 3);
+  for (int it = tid; it < nitems; it += 256) {  // whole half-waves: K / 8 is a multiple of 32
+    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (it < valid) load8<XT>(a.x, (int64_t)it * 8, v);
+    const Q8KItem q = quantize_q8k_item(v, lane);
+    reinterpret_cast<u32x2*>(s_q)[it] = u32x2{q.q0, q.q1};
+    const int s16 = q.sum8 + __builtin_amdgcn_update_dpp(0, q.sum8, 0xB1, 0xf, 0xf, true);
+    const int s16b = __builtin_amdgcn_update_dpp(0, s16, 0x4E, 0xf, 0xf, true);  // the other pair of the quad
+    if ((it & 3) == 0) s_bs[it >> 2] = ((uint32_t)s16 & 0xffffu) | ((uint32_t)s16b << 16);
+    if ((it & 31) == 0) s_d[it >> 5] = q.d;
+  }
+  __syncthreads();
+
+  float acc[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int m = 0; m < MT; m++) acc[r][m] = 0.f;
+
+  for (int u0 = 0; u0 < units; u0 += G) {
+    KUnit<WT> nxt[R];
+    const bool more = u0 + G < units;  // uniform
+    if (more) {
+#pragma unroll
+      for (int r = 0; r < R; r++) load_unit<WT>(nxt[r], rs, (uint32_t)((row0 + r) * nsb), u0 + G + c0, units, row0 + r < a.N);
+    }
+    const int unit = u0 + c0;
+    if (unit < units) {
+      if (WT == MLLM_HIP_Q4_K) {
+        const int sb = unit >> 3, c = unit & 7, jp = c >> 1, hh = c & 1;
+        int sc_lo[R], sc_hi[R], mn_lo[R], mn_hi[R];
+        float dw[R], dmw[R];
+        u32x4 wlo[R], whi[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          const K4Scales k = k4_scales(cur[r].s.y, cur[r].s.z, cur[r].s.w);
+          sc_lo[r] = byte_of(k.sc0, k.sc1, 2 * jp);
+          sc_hi[r] = byte_of(k.sc0, k.sc1, 2 * jp + 1);
+          mn_lo[r] = byte_of(k.mn0, k.mn1, 2 * jp);
+          mn_hi[r] = byte_of(k.mn0, k.mn1, 2 * jp + 1);
+          dw[r] = f16bits_to_f32((uint16_t)(cur[r].s.x & 0xffffu));
+          dmw[r] = f16bits_to_f32((uint16_t)(cur[r].s.x >> 16));
+          const uint32_t m4 = 0x0f0f0f0fu;
+          wlo[r] = u32x4{cur[r].a.x & m4, cur[r].a.y & m4, cur[r].a.z & m4, cur[r].a.w & m4};
+          whi[r] = u32x4{(cur[r].a.x >> 4) & m4, (cur[r].a.y >> 4) & m4, (cur[r].a.z >> 4) & m4, (cur[r].a.w >> 4) & m4};
+        }
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+          const int qb = m * (K >> 4) + sb * 16 + 4 * jp + hh;  // 16-byte chunk of the sub-block pair's low half
+          const u32x4 xlo = s_q[qb], xhi = s_q[qb + 2];
+          const float yd = s_d[m * nsb + sb];
+          const u32x2 bp = reinterpret_cast<const u32x2*>(s_bs)[(m * nsb + sb) * 4 + jp];  // sums 4jp..4jp+3
+          const int bs_lo = half16(bp.x, hh), bs_hi = half16(bp.y, hh);
+#pragma unroll
+          for (int r = 0; r < R; r++) {
+            const int isum = sc_lo[r] * dot16(wlo[r], xlo) + sc_hi[r] * dot16(whi[r], xhi);
+            const int msum = mn_lo[r] * bs_lo + mn_hi[r] * bs_hi;
+            acc[r][m] = fmaf(yd * dw[r], (float)isum, acc[r][m]);
+            acc[r][m] = fmaf(-yd * dmw[r], (float)msum, acc[r][m]);
+          }
+        }
+      } else {
+        const int sb = unit >> 2, n = (unit >> 1) & 1, t = unit & 1;
+        u32x4 wv[R][4];
+        int sc[R][4];
+        float dw[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          dw[r] = f16bits_to_f32(cur[r].d);
+          const uint32_t sw[4] = {cur[r].s.x, cur[r].s.y, cur[r].s.z, cur[r].s.w};
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            const u32x4& src = (g & 1) ? cur[r].b : cur[r].a;
+            const int sh = (g >= 2) ? 4 : 0;
+            const uint32_t m4 = 0x0f0f0f0fu, m2 = 0x03030303u;
+            wv[r][g] = u32x4{((src.x >> sh) & m4) | (((cur[r].h.x >> (2 * g)) & m2) << 4), ((src.y >> sh) & m4) | (((cur[r].h.y >> (2 * g)) & m2) << 4),
+                             ((src.z >> sh) & m4) | (((cur[r].h.z >> (2 * g)) & m2) << 4), ((src.w >> sh) & m4) | (((cur[r].h.w >> (2 * g)) & m2) << 4)};
+            const int si = 8 * n + 2 * g + t;  // scale of these 16 weights
+            sc[r][g] = (int)(int8_t)((sw[si >> 2] >> (8 * (si & 3))) & 0xffu);
+          }
+        }
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+          const float yd = s_d[m * nsb + sb];
+          const u32x4 bq = reinterpret_cast<const u32x4*>(s_bs)[(m * nsb + sb) * 2 + n];  // sums 8n..8n+7
+          const uint32_t bw[4] = {bq.x, bq.y, bq.z, bq.w};
+          int tot[R];
+#pragma unroll
+          for (int r = 0; r < R; r++) tot[r] = 0;
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            const u32x4 xq = s_q[m * (K >> 4) + sb * 16 + 8 * n + 2 * g + t];
+            const int bs = half16(bw[g], t);
+#pragma unroll
+            for (int r = 0; r < R; r++) tot[r] += sc[r][g] * (dot16(wv[r][g], xq) - 32 * bs);
+          }
+#pragma unroll
+          for (int r = 0; r < R; r++) acc[r][m] = fmaf(yd * dw[r], (float)tot[r], acc[r][m]);
+        }
+      }
+    }
+    if (more) {
+#pragma unroll
+      for (int r = 0; r < R; r++) cur[r] = nxt[r];
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < R; r++)
+#pragma unroll
+    for (int m = 0; m < MT; m++) {
+      const float v = group_sum<G>(acc[r][m]);
+      const int64_t row = row0 + r;
+      if (c0 == 0 && row < a.N && m < a.M) a.y[(int64_t)m * a.N + row] = a.bias ? v + a.bias[row] : v;
+    }
+}
+
+template <int WT, int XT, int MT, int G>
+static int launch_kq_g(const KGemvArgs& a, hipStream_t st) {
+  constexpr int R = 2;
+  constexpr int rows_per_wg = 4 * (64 / G) * R;
+  const int K = a.nsb * QK_K;
+  const size_t lds = (size_t)MT * K + (size_t)MT * a.nsb * 4 + (size_t)MT * a.nsb * 32;
+  if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
+  auto kern = kq_gemv_kernel<WT, XT, MT, G, R>;
+  if (lds > 64 * 1024)
+    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  const unsigned grid = (unsigned)((a.N + rows_per_wg - 1) / rows_per_wg);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a);
+  return (int)hipGetLastError();
+}
+template <int WT, int XT, int MT>
+static int launch_kq_m(const KGemvArgs& a, hipStream_t st) {
+  const int units = a.nsb * (WT == MLLM_HIP_Q4_K ? 8 : 4);
+  if (units >= 64) return launch_kq_g<WT, XT, MT, 64>(a, st);
+  if (units >= 32) return launch_kq_g<WT, XT, MT, 32>(a, st);
+  if (units >= 16) return launch_kq_g<WT, XT, MT, 16>(a, st);
+  return launch_kq_g<WT, XT, MT, 8>(a, st);
+}
+template <int WT, int XT>
+static int launch_kq(const KGemvArgs& a, hipStream_t st) {
+  if (a.M <= 1) return launch_kq_m<WT, XT, 1>(a, st);
+  if (a.M <= 2) return launch_kq_m<WT, XT, 2>(a, st);
+  if (a.M <= 4) return launch_kq_m<WT, XT, 4>(a, st);
+  return launch_kq_m<WT, XT, 8>(a, st);
+}
+
+}  // namespace mllmhip
+
+using namespace mllmhip;
+
+static int kq_check(int wtype, const void* packed, int64_t N, int64_t K) {
+  if (wtype != MLLM_HIP_Q4_K && wtype != MLLM_HIP_Q6_K) return MLLM_HIP_E_BADARG;
+  if (!packed || N <= 0 || K <= 0) return MLLM_HIP_E_BADARG;
+  if (K % QK_K) return MLLM_HIP_E_SHAPE;
+  if (N > INT32_MAX || N * (K / QK_K) * 128 >= ((int64_t)1 << 32)) return MLLM_HIP_E_SHAPE;  // 32-bit buffer offsets
+  if (reinterpret_cast<uintptr_t>(packed) % 256) return MLLM_HIP_E_ALIGN;
+  return 0;
+}
+
+MLLM_API size_t mllm_hip_kq_packed_bytes(int wtype, int64_t N, int64_t K) {
+  if ((wtype != MLLM_HIP_Q4_K && wtype != MLLM_HIP_Q6_K) || N <= 0 || K <= 0 || K % QK_K) return 0;
+  return kq_packed_bytes(wtype, N, K);
+}
+
+MLLM_API int mllm_hip_kq_prepack(int wtype, const void* blocks, int weight_scale_mode, void* packed, int64_t N, int64_t K, void* stream) {
+  int rc = kq_check(wtype, packed, N, K);
+  if (rc) return rc;
+  if (!blocks || (weight_scale_mode != MLLM_HIP_SCALE_IEEE && weight_scale_mode != MLLM_HIP_SCALE_X86_REF)) return MLLM_HIP_E_BADARG;
+  const int64_t nsb = N * (K / QK_K);
+  hipLaunchKernelGGL(kq_prepack_kernel, dim3((unsigned)((nsb * 8 + 255) / 256)), dim3(256), 0, (hipStream_t)stream, wtype,
+                     (const uint8_t*)blocks, weight_scale_mode == MLLM_HIP_SCALE_X86_REF, kq_view(wtype, packed, N, K), nsb);
+  return (int)hipGetLastError();
+}
+
+MLLM_API int mllm_hip_kq_dequantize(int wtype, const void* packed, float* w, int64_t N, int64_t K, void* stream) {
+  int rc = kq_check(wtype, packed, N, K);
+  if (rc) return rc;
+  if (!w) return MLLM_HIP_E_BADARG;
+  const int64_t nsb = N * (K / QK_K);
+  hipLaunchKernelGGL(kq_dequantize_kernel, dim3((unsigned)nsb), dim3(256), 0, (hipStream_t)stream, wtype, kq_view(wtype, packed, N, K), w, nsb);
+  return (int)hipGetLastError();
+}
+
+MLLM_API int mllm_hip_quantize_q8_K(const void* x, int x_dtype, int8_t* codes, float* d, int16_t* bsums, int64_t M, int64_t K, void* stream) {
+  if (!x || !codes || !d || !bsums || M <= 0 || K <= 0 || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16)) return MLLM_HIP_E_BADARG;
+  if (K % QK_K) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(codes) % 8) return MLLM_HIP_E_ALIGN;
+  const int64_t nitems = M * K / 8;
+  hipLaunchKernelGGL(quantize_q8k_kernel, dim3((unsigned)((nitems + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, x_dtype, codes, d,
+                     bsums, nitems);
+  return (int)hipGetLastError();
+}
+
+MLLM_API int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y, int64_t M,
+                                int64_t N, int64_t K, void* stream) {
+  int rc = kq_check(wtype, packed, N, K);
+  if (rc) return rc;
+  if (!x || !y || M <= 0 || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16)) return MLLM_HIP_E_BADARG;
+  if (reinterpret_cast<uintptr_t>(x) % 16) return MLLM_HIP_E_ALIGN;
+  const size_t xrow = (size_t)K * (x_dtype == MLLM_HIP_F32 ? 4 : 2);
+  for (int64_t m0 = 0; m0 < M; m0 += 8) {  // more than eight rows: groups of eight (each streams the weights again)
+    KGemvArgs a{kq_view(wtype, packed, N, K), bias, y + m0 * N, reinterpret_cast<const char*>(x) + m0 * xrow,
+                (int)N, (int)(M - m0 < 8 ? M - m0 : 8), (int)(K / QK_K)};
+    if (wtype == MLLM_HIP_Q4_K)
+      rc = x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_F32>(a, (hipStream_t)stream) : launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_BF16>(a, (hipStream_t)stream);
+    else
+      rc = x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q6_K, MLLM_HIP_F32>(a, (hipStream_t)stream) : launch_kq<MLLM_HIP_Q6_K, MLLM_HIP_BF16>(a, (hipStream_t)stream);
+    if (rc) return rc;
+  }
+  return 0;
+}

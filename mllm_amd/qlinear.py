@@ -485,3 +485,62 @@ def moe_gate(x, gate_weight, k, norm_topk_prob=True, want_scores=False):
     _lib.check(_lib.lib().mllm_hip_moe_gate(x.data_ptr(), _xdtype(x), gate_weight.data_ptr(), ids.data_ptr(), wt.data_ptr(),
                                             _p(sc), M, H, E, k, int(norm_topk_prob), _stream()), "mllm_hip_moe_gate")
     return (ids, wt, sc) if want_scores else (ids, wt)
+
+
+# ----------------------------------------------------------------------------- K-quants (Q4_K / Q6_K weights, Q8_K activations)
+Q4_K, Q6_K = 2, 3
+KBLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
+
+
+class PackedKWeight:
+    """Q4_K / Q6_K weight [N, K] repacked on the device.  blocks: uint8 [N, K/256, 144|210] (reference layout)."""
+
+    def __init__(self, wtype, blocks, weight_scale_mode=SCALE_IEEE):
+        assert blocks.dtype == torch.uint8 and blocks.dim() == 3 and blocks.shape[2] == KBLOCK_BYTES[wtype]
+        self.wtype, self.N, self.K = wtype, blocks.shape[0], blocks.shape[1] * 256
+        L = _lib.lib()
+        self.buf = torch.empty(L.mllm_hip_kq_packed_bytes(wtype, self.N, self.K), dtype=torch.uint8, device="cuda")
+        src = blocks.contiguous().cuda()
+        _lib.check(L.mllm_hip_kq_prepack(wtype, src.data_ptr(), weight_scale_mode, self.buf.data_ptr(), self.N, self.K, _stream()),
+                   "mllm_hip_kq_prepack")
+        torch.cuda.current_stream().synchronize()  # src may be released
+
+    @classmethod
+    def synthetic(cls, wtype, N, K, gen):
+        """random blocks made on the device (bench): every byte uniform, fp16 fields set to a small positive value"""
+        bb = KBLOCK_BYTES[wtype]
+        blocks = torch.randint(0, 256, (N, K // 256, bb), dtype=torch.uint8, device="cuda", generator=gen)
+        for off in ((0, 2) if wtype == Q4_K else (208,)):
+            blocks[:, :, off] = 0x00
+            blocks[:, :, off + 1] = 0x14  # 0x1400 = 9.8e-4
+        return cls(wtype, blocks)
+
+    @property
+    def ptr(self):
+        return self.buf.data_ptr()
+
+    def dequantize(self):
+        w = torch.empty((self.N, self.K), dtype=torch.float32, device="cuda")
+        _lib.check(_lib.lib().mllm_hip_kq_dequantize(self.wtype, self.ptr, w.data_ptr(), self.N, self.K, _stream()), "mllm_hip_kq_dequantize")
+        return w
+
+
+def linear_kq(w, x, bias=None, out=None):
+    assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
+    M = x.shape[0]
+    y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_linear_kq(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K, _stream()),
+               "mllm_hip_linear_kq")
+    return y
+
+
+def quantize_q8_K(x):
+    """x [M, K] -> (codes int8 [M, K], d fp32 [M, K/256], sums of 16 int16 [M, K/16])"""
+    assert x.is_cuda and x.is_contiguous() and x.dim() == 2
+    M, K = x.shape
+    codes = torch.empty((M, K), dtype=torch.int8, device="cuda")
+    d = torch.empty((M, K // 256), dtype=torch.float32, device="cuda")
+    bs = torch.empty((M, K // 16), dtype=torch.int16, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_quantize_q8_K(x.data_ptr(), _xdtype(x), codes.data_ptr(), d.data_ptr(), bs.data_ptr(), M, K, _stream()),
+               "mllm_hip_quantize_q8_K")
+    return codes, d, bs

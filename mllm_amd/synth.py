@@ -81,7 +81,31 @@ def make_q8_0(rng, N, K, sigma=0.02):
     return pack_q8_0(codes, _scales(rng, (N, K // QK), sigma))
 
 
+def make_q4_K(rng, N, K, sigma=0.02):
+    """random block_q4_K rows, uint8 [N, K/256, 144]: fp16 d and dmin on the grid both scale conventions read alike,
+    6-bit scales / mins and nibbles uniform"""
+    nb = K // 256
+    out = np.empty((N, nb, 144), np.uint8)
+    out[:, :, 0:2] = np.ascontiguousarray(_scales(rng, (N, nb), sigma / 8), dtype="<u2").reshape(N, nb, 1).view(np.uint8)
+    out[:, :, 2:4] = np.ascontiguousarray(_scales(rng, (N, nb), sigma / 8), dtype="<u2").reshape(N, nb, 1).view(np.uint8)
+    out[:, :, 4:] = rng.integers(0, 256, size=(N, nb, 140), dtype=np.uint8)
+    return out
+
+
+def make_q6_K(rng, N, K, sigma=0.02):
+    """random block_q6_K rows, uint8 [N, K/256, 210]"""
+    nb = K // 256
+    out = np.empty((N, nb, 210), np.uint8)
+    out[:, :, :208] = rng.integers(0, 256, size=(N, nb, 208), dtype=np.uint8)
+    out[:, :, 208:] = np.ascontiguousarray(_scales(rng, (N, nb), sigma / 64), dtype="<u2").reshape(N, nb, 1).view(np.uint8)
+    return out
+
+
 def make_weight(rng, wtype, N, K):
+    if wtype == 2:
+        return make_q4_K(rng, N, K)
+    if wtype == 3:
+        return make_q6_K(rng, N, K)
     return make_q4_0(rng, N, K) if wtype == 0 else make_q8_0(rng, N, K)
 
 

@@ -334,3 +334,111 @@ def moe_gate(x, w, k, norm=True):
     lib().orc_moe_gate(_p(x, C.c_float), _p(w, C.c_float), _p(ids, C.c_int32), _p(wt, C.c_float), _p(sc, C.c_float), C.c_int64(M),
                        C.c_int(H), C.c_int(E), C.c_int(k), C.c_int(int(norm)))
     return ids, wt, sc
+
+
+# ----------------------------------------------------------------------------- K-quants (Q4_K / Q6_K weights, Q8_K activations)
+Q4_K, Q6_K = 2, 3
+KBLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
+
+
+def quantize_rows_q8_K(x):
+    """x fp32 [M, K] -> (codes int8 [M, K], scales fp32 [M, K/256], sums of 16 int16 [M, K/16])"""
+    x = np.ascontiguousarray(x, np.float32)
+    M, K = x.shape
+    q = np.empty((M, K), np.int8)
+    d = np.empty((M, K // 256), np.float32)
+    bs = np.empty((M, K // 16), np.int16)
+    for m in range(M):
+        lib().orc_quantize_row_q8_K(_p(x[m], C.c_float), _p(q[m], C.c_int8), _p(d[m], C.c_float), _p(bs[m], C.c_int16), C.c_int(K))
+    return q, d, bs
+
+
+def dequantize_k(W, wtype, scale_mode=SCALE_IEEE):
+    """W uint8 [N, K/256, 144|210] -> fp32 [N, K]"""
+    W = np.ascontiguousarray(W, np.uint8)
+    N, nb, bb = W.shape
+    assert bb == KBLOCK_BYTES[wtype]
+    y = np.empty((N, nb * 256), np.float32)
+    fn = lib().orc_dequantize_row_q4_K if wtype == Q4_K else lib().orc_dequantize_row_q6_K
+    for n in range(N):
+        fn(_p(W[n], C.c_uint8), _p(y[n], C.c_float), C.c_int(nb * 256), C.c_int(scale_mode))
+    return y
+
+
+def linear_kq(x, W, wtype, bias=None, scale_mode=SCALE_X86_REF):
+    x = np.ascontiguousarray(x, np.float32)
+    W = np.ascontiguousarray(W, np.uint8)
+    M, K = x.shape
+    N, nb, bb = W.shape
+    assert nb * 256 == K and bb == KBLOCK_BYTES[wtype]
+    y = np.empty((M, N), np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    lib().orc_linear_kq.restype = C.c_int
+    rc = lib().orc_linear_kq(_p(x, C.c_float), _p(W, C.c_uint8), C.c_int(wtype), _p(b, C.c_float), _p(y, C.c_float), C.c_int(M),
+                             C.c_int(N), C.c_int(K), C.c_int(scale_mode))
+    assert rc == 0, rc
+    return y
+
+
+def kq_block_sums(W, wtype, xq, xbs):
+    """exact per-super-block integers: isum int32 [N, M, nb] (and msum for Q4_K, else None)"""
+    W = np.ascontiguousarray(W, np.uint8)
+    N, nb, bb = W.shape
+    M, K = xq.shape
+    isum = np.empty((N, M, nb), np.int32)
+    msum = np.empty((N, M, nb), np.int32) if wtype == Q4_K else None
+    xd = np.ones((M, nb), np.float32)
+    L = lib()
+    L.orc_vec_dot_q4_K_q8_K.restype = C.c_float
+    L.orc_vec_dot_q6_K_q8_K.restype = C.c_float
+    for n in range(N):
+        for m in range(M):
+            if wtype == Q4_K:
+                L.orc_vec_dot_q4_K_q8_K(_p(W[n], C.c_uint8), _p(xq[m], C.c_int8), _p(xd[m], C.c_float), _p(xbs[m], C.c_int16),
+                                        C.c_int(K), C.c_int(SCALE_IEEE), _p(isum[n, m], C.c_int32), _p(msum[n, m], C.c_int32))
+            else:
+                L.orc_vec_dot_q6_K_q8_K(_p(W[n], C.c_uint8), _p(xq[m], C.c_int8), _p(xd[m], C.c_float), C.c_int(K),
+                                        C.c_int(SCALE_IEEE), _p(isum[n, m], C.c_int32))
+    return isum, msum
+
+
+def ref_quantize_rows_q8_K(x):
+    x = np.ascontiguousarray(x, np.float32)
+    M, K = x.shape
+    q = np.empty((M, K), np.int8)
+    d = np.empty((M, K // 256), np.float32)
+    bs = np.empty((M, K // 16), np.int16)
+    for m in range(M):
+        ref().ref_quantize_row_q8_K(_p(x[m], C.c_float), _p(q[m], C.c_int8), _p(d[m], C.c_float), _p(bs[m], C.c_int16), C.c_int(K))
+    return q, d, bs
+
+
+def ref_dequantize_k(W, wtype):
+    W = np.ascontiguousarray(W, np.uint8)
+    N, nb, bb = W.shape
+    y = np.empty((N, nb * 256), np.float32)
+    for n in range(N):
+        ref().ref_dequantize_row_k(_p(W[n], C.c_uint8), C.c_int(wtype), _p(y[n], C.c_float), C.c_int(nb * 256))
+    return y
+
+
+def ref_linear_kq(x, W, wtype, bias=None):
+    x = np.ascontiguousarray(x, np.float32)
+    W = np.ascontiguousarray(W, np.uint8)
+    M, K = x.shape
+    N = W.shape[0]
+    y = np.empty((M, N), np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    ref().ref_linear_kq(_p(x, C.c_float), _p(W, C.c_uint8), C.c_int(wtype), _p(b, C.c_float), _p(y, C.c_float), C.c_int(M), C.c_int(N),
+                        C.c_int(K))
+    return y
+
+
+def ref_quantize_rows_k(w, wtype):
+    """the reference's offline quantizer -> canonical blocks uint8 [N, K/256, 144|210]"""
+    w = np.ascontiguousarray(w, np.float32)
+    N, K = w.shape
+    out = np.empty((N, K // 256, KBLOCK_BYTES[wtype]), np.uint8)
+    for n in range(N):
+        ref().ref_quantize_row_k(_p(w[n], C.c_float), _p(out[n], C.c_uint8), C.c_int(wtype), C.c_int(K))
+    return out

@@ -617,3 +617,207 @@ ORC_API int orc_moe_ffn(const float* x, const int32_t* topk_ids, const float* to
   free(per);
   return 0;
 }
+
+/* ================================================================================================
+ * K-quants: Q4_K / Q6_K weights with Q8_K activations (the formats of the shipped Qwen3-MoE recipe).
+ *   block_q4_K (144 B): fp16 d, fp16 dmin, 12 B of 6-bit scales and mins, 128 B of nibbles   mllm/core/DataTypes.hpp:139-147
+ *   block_q6_K (210 B): 128 B low nibbles, 64 B high bit pairs, 16 int8 scales, fp16 d        mllm/core/DataTypes.hpp:153-160
+ *   block_q8_K        : fp32 d, 256 int8, 16 int16 sums of 16                                 mllm/core/DataTypes.hpp:188-194
+ * Weight blocks are passed as the reference's byte layout with IEEE fp16 patterns in the fp16 fields; scale_mode
+ * X86_REF applies the x86 build's storage rounding to them where they are used (scale_value()).
+ * Pinned bit for bit against the compiled reference (quantize_row_q8_K, dequantize_row_q4_K / _q6_K, vec_dot_q4_K_q8_K,
+ * vec_dot_q6_K_q8_K) in tests/test_oracle_vs_reference.py.
+ * ============================================================================================== */
+#define QK_K 256
+enum { ORC_Q4_K = 2, ORC_Q6_K = 3 };
+static inline int kblk_bytes(int wtype) { return wtype == ORC_Q4_K ? 144 : 210; }
+
+/* quantize_row_q8_K_reference, quantize_q8.cpp:215-248.  nearest_int (quantize.hpp:261-267) is round-half-even. */
+ORC_API void orc_quantize_row_q8_K(const float* x, int8_t* qs, float* d, int16_t* bsums, int k) {
+  int nb = k / QK_K;
+  for (int i = 0; i < nb; i++) {
+    const float* xb = x + (size_t)i * QK_K;
+    int8_t* q = qs + (size_t)i * QK_K;
+    float max = 0, amax = 0;
+    for (int j = 0; j < QK_K; j++) {
+      float ax = fabsf(xb[j]);
+      if (ax > amax) {
+        amax = ax;
+        max = xb[j];
+      }
+    }
+    if (amax == 0.0f) {
+      d[i] = 0;
+      memset(q, 0, QK_K);
+      /* the reference leaves bsums of such a block untouched (uninitialised memory of a fresh tensor); zero here */
+      memset(bsums + (size_t)i * 16, 0, 32);
+      continue;
+    }
+    const float iscale = -128.f / max;
+    for (int j = 0; j < QK_K; j++) {
+      int v = (int)rintf(iscale * xb[j]);
+      q[j] = (int8_t)(v < 127 ? v : 127);
+    }
+    for (int j = 0; j < 16; j++) {
+      int sum = 0;
+      for (int ii = 0; ii < 16; ii++) sum += q[j * 16 + ii];
+      bsums[(size_t)i * 16 + j] = (int16_t)sum;
+    }
+    d[i] = 1 / iscale;
+  }
+}
+
+/* get_scale_min_k4, quantize.hpp */
+static inline void scale_min_k4(int j, const uint8_t* q, uint8_t* d, uint8_t* m) {
+  if (j < 4) {
+    *d = q[j] & 63;
+    *m = q[j + 4] & 63;
+  } else {
+    *d = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4));
+    *m = (uint8_t)((q[j + 4] >> 4) | ((q[j - 0] >> 6) << 4));
+  }
+}
+static inline uint16_t rd16(const uint8_t* p) { uint16_t v; memcpy(&v, p, 2); return v; }
+
+/* dequantize_row_q4_K, quantize_q4.cpp:284-312: y = (d * sc) * q - (dmin * m), each product rounded to fp32 */
+ORC_API void orc_dequantize_row_q4_K(const uint8_t* blocks, float* y, int k, int scale_mode) {
+  int nb = k / QK_K;
+  for (int i = 0; i < nb; i++) {
+    const uint8_t* b = blocks + (size_t)i * 144;
+    const float d = scale_value(rd16(b), scale_mode), min = scale_value(rd16(b + 2), scale_mode);
+    const uint8_t* q = b + 16;
+    int is = 0;
+    for (int j = 0; j < QK_K; j += 64) {
+      uint8_t sc, m;
+      scale_min_k4(is + 0, b + 4, &sc, &m);
+      const float d1 = d * sc, m1 = min * m;
+      scale_min_k4(is + 1, b + 4, &sc, &m);
+      const float d2 = d * sc, m2 = min * m;
+      for (int l = 0; l < 32; l++) *y++ = d1 * (q[l] & 0xF) - m1;
+      for (int l = 0; l < 32; l++) *y++ = d2 * (q[l] >> 4) - m2;
+      q += 32;
+      is += 2;
+    }
+  }
+}
+
+/* the 6-bit value (minus 32) of element e of a q6_K block, dequantize_row_q6_K, quantize_q6.cpp:108-133 */
+static inline int q6_value(const uint8_t* b, int e) {
+  const uint8_t* ql = b + 64 * (e / 128);
+  const uint8_t* qh = b + 128 + 32 * (e / 128);
+  int r = e % 128, g = r / 32, l = r % 32;
+  int lo = (g & 1) ? ql[l + 32] : ql[l];
+  lo = (g >= 2) ? (lo >> 4) : (lo & 0xF);
+  int hi = (qh[l] >> (2 * g)) & 3;
+  return (int8_t)(lo | (hi << 4)) - 32;
+}
+ORC_API void orc_dequantize_row_q6_K(const uint8_t* blocks, float* y, int k, int scale_mode) {
+  int nb = k / QK_K;
+  for (int i = 0; i < nb; i++) {
+    const uint8_t* b = blocks + (size_t)i * 210;
+    const float d = scale_value(rd16(b + 208), scale_mode);
+    const int8_t* sc = (const int8_t*)(b + 192);
+    for (int e = 0; e < QK_K; e++) y[(size_t)i * QK_K + e] = d * sc[e / 16] * q6_value(b, e);
+  }
+}
+
+static inline float hsum8(const float* a) { /* hsum_float_8 */
+  float t0 = a[4] + a[0], t1 = a[5] + a[1], t2 = a[6] + a[2], t3 = a[7] + a[3];
+  float u0 = t0 + t2, u1 = t1 + t3;
+  return u0 + u1;
+}
+
+/* vec_dot_q4_K_q8_K, AVX2 branch, vec_dot.cpp:498-560 (QK_K == 256).  Eight int32 lanes: lane u collects, over the eight
+ * sub-blocks, scale * (sum over elements 4u..4u+3 of the sub-block); acc[u] = fma(d, float(lane), acc[u]) per super-block.
+ * Mins: four lanes, lane v = m[2v] * bsum32[2v] + m[2v+1] * bsum32[2v+1], acc_m[v] = fma(dmin, float(lane), acc_m[v]),
+ * reduced as (a0 + a2) + (a1 + a3).  isum / msum (optional) receive the exact per-super-block integers. */
+ORC_API float orc_vec_dot_q4_K_q8_K(const uint8_t* wrow, const int8_t* xq, const float* xd, const int16_t* xbs, int k, int scale_mode,
+                                    int32_t* isum, int32_t* msum) {
+  int nb = k / QK_K;
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0}, acc_m[4] = {0, 0, 0, 0};
+  for (int i = 0; i < nb; i++) {
+    const uint8_t* b = wrow + (size_t)i * 144;
+    const float d = xd[i] * scale_value(rd16(b), scale_mode);
+    const float dmin = -xd[i] * scale_value(rd16(b + 2), scale_mode);
+    uint8_t sc[8], mn[8];
+    for (int j = 0; j < 8; j++) scale_min_k4(j, b + 4, &sc[j], &mn[j]);
+    const int16_t* bs = xbs + (size_t)i * 16;
+    int32_t mtot = 0;
+    for (int v = 0; v < 4; v++) {
+      int32_t p = (int32_t)mn[2 * v] * (bs[4 * v] + bs[4 * v + 1]) + (int32_t)mn[2 * v + 1] * (bs[4 * v + 2] + bs[4 * v + 3]);
+      mtot += p;
+      acc_m[v] = fmaf(dmin, (float)p, acc_m[v]);
+    }
+    int32_t lanes[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    const uint8_t* q4 = b + 16;
+    const int8_t* q8 = xq + (size_t)i * QK_K;
+    for (int j = 0; j < 4; j++) {
+      for (int u = 0; u < 8; u++) {
+        int32_t lo = 0, hi = 0;
+        for (int e = 4 * u; e < 4 * u + 4; e++) {
+          lo += (int32_t)(q4[32 * j + e] & 0xF) * q8[64 * j + e];
+          hi += (int32_t)(q4[32 * j + e] >> 4) * q8[64 * j + 32 + e];
+        }
+        lanes[u] += sc[2 * j] * lo + sc[2 * j + 1] * hi;
+      }
+    }
+    int32_t tot = 0;
+    for (int u = 0; u < 8; u++) {
+      tot += lanes[u];
+      acc[u] = fmaf(d, (float)lanes[u], acc[u]);
+    }
+    if (isum) isum[i] = tot;
+    if (msum) msum[i] = mtot;
+  }
+  float am0 = acc_m[0] + acc_m[2], am1 = acc_m[1] + acc_m[3];
+  return hsum8(acc) + (am0 + am1);
+}
+
+/* vec_dot_q6_K_q8_K, AVX2 branch, vec_dot.cpp:955-1044.  Lane u of group g covers elements 4u..4u+3 of the group's 32. */
+ORC_API float orc_vec_dot_q6_K_q8_K(const uint8_t* wrow, const int8_t* xq, const float* xd, int k, int scale_mode, int32_t* isum) {
+  int nb = k / QK_K;
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int i = 0; i < nb; i++) {
+    const uint8_t* b = wrow + (size_t)i * 210;
+    const float d = xd[i] * scale_value(rd16(b + 208), scale_mode);
+    const int8_t* sc = (const int8_t*)(b + 192);
+    const int8_t* q8 = xq + (size_t)i * QK_K;
+    int32_t lanes[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int grp = 0; grp < 8; grp++) /* 8 groups of 32 elements */
+      for (int u = 0; u < 8; u++) {
+        int32_t s = 0;
+        for (int e = 32 * grp + 4 * u; e < 32 * grp + 4 * u + 4; e++) s += q6_value(b, e) * q8[e];
+        lanes[u] += sc[2 * grp + (u >= 4)] * s;
+      }
+    int32_t tot = 0;
+    for (int u = 0; u < 8; u++) {
+      tot += lanes[u];
+      acc[u] = fmaf(d, (float)lanes[u], acc[u]);
+    }
+    if (isum) isum[i] = tot;
+  }
+  return hsum8(acc);
+}
+
+/* Linear with Q4_K / Q6_K weights: ggml::mat_mul's generic branch, matmul.cpp:147-189 (rows of x to Q8_K), :300-360
+ * (vec_dot per output element), bias added afterwards with mllm_add_fp32 (:280-290). */
+ORC_API int orc_linear_kq(const float* x, const uint8_t* W, int wtype, const float* bias, float* y, int M, int N, int K, int scale_mode) {
+  if (K % QK_K || (wtype != ORC_Q4_K && wtype != ORC_Q6_K)) return -1;
+  int nb = K / QK_K, bb = kblk_bytes(wtype);
+  int8_t* xq = (int8_t*)malloc((size_t)M * K);
+  float* xd = (float*)malloc(sizeof(float) * (size_t)M * nb);
+  int16_t* xbs = (int16_t*)malloc(sizeof(int16_t) * (size_t)M * nb * 16);
+  if (!xq || !xd || !xbs) return -2;
+  for (int m = 0; m < M; m++) orc_quantize_row_q8_K(x + (size_t)m * K, xq + (size_t)m * K, xd + (size_t)m * nb, xbs + (size_t)m * nb * 16, K);
+#pragma omp parallel for schedule(static)
+  for (int n = 0; n < N; n++)
+    for (int m = 0; m < M; m++) {
+      const uint8_t* wrow = W + (size_t)n * nb * bb;
+      float v = wtype == ORC_Q4_K
+                    ? orc_vec_dot_q4_K_q8_K(wrow, xq + (size_t)m * K, xd + (size_t)m * nb, xbs + (size_t)m * nb * 16, K, scale_mode, NULL, NULL)
+                    : orc_vec_dot_q6_K_q8_K(wrow, xq + (size_t)m * K, xd + (size_t)m * nb, K, scale_mode, NULL);
+      y[(size_t)m * N + n] = bias ? v + bias[n] : v;
+    }
+  free(xq); free(xd); free(xbs);
+  return 0;
+}

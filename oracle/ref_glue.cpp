@@ -117,3 +117,106 @@ REF_API void ref_quantize_row_q4_0(const float* x, uint8_t* canon, int k) {
     std::memcpy(canon + (size_t)i * 18 + 2, y[i].qs, 16);
   }
 }
+
+// ---- K-quants ------------------------------------------------------------------------------------------------------
+#include "mllm/backends/cpu/kernels/common/ggml/quantize/quantize_q6.hpp"
+static_assert(sizeof(block_q4_K) == 144, "block_q4_K must be 144 bytes");
+static_assert(sizeof(block_q6_K) == 210, "block_q6_K must be 210 bytes");
+
+static void to_ref_q4k(const uint8_t* canon, int nb, std::vector<block_q4_K>& out) {
+  out.resize(nb);
+  for (int i = 0; i < nb; i++) {
+    uint16_t d, m;
+    std::memcpy(&d, canon + (size_t)i * 144, 2);
+    std::memcpy(&m, canon + (size_t)i * 144 + 2, 2);
+    out[i].d = d;  // implicit conversion, as in the quantizer's `y[i].d = MLLM_FP32_TO_FP16(...)`
+    out[i].dmin = m;
+    std::memcpy(out[i].scales, canon + (size_t)i * 144 + 4, 12);
+    std::memcpy(out[i].qs, canon + (size_t)i * 144 + 16, 128);
+  }
+}
+static void to_ref_q6k(const uint8_t* canon, int nb, std::vector<block_q6_K>& out) {
+  out.resize(nb);
+  for (int i = 0; i < nb; i++) {
+    std::memcpy(out[i].ql, canon + (size_t)i * 210, 128);
+    std::memcpy(out[i].qh, canon + (size_t)i * 210 + 128, 64);
+    std::memcpy(out[i].scales, canon + (size_t)i * 210 + 192, 16);
+    uint16_t d;
+    std::memcpy(&d, canon + (size_t)i * 210 + 208, 2);
+    out[i].d = d;
+  }
+}
+
+// quantize_row_q8_K -> codes, fp32 scales, sums of 16
+REF_API void ref_quantize_row_q8_K(const float* x, int8_t* qs, float* d, int16_t* bsums, int k) {
+  int nb = k / QK_K;
+  std::vector<block_q8_K> y(nb);
+  std::memset(y.data(), 0, sizeof(block_q8_K) * nb);
+  quantize_row_q8_K(x, y.data(), k);
+  for (int i = 0; i < nb; i++) {
+    std::memcpy(qs + (size_t)i * QK_K, y[i].qs, QK_K);
+    d[i] = y[i].d;
+    std::memcpy(bsums + (size_t)i * 16, y[i].bsums, 32);
+  }
+}
+
+// wtype: 2 = Q4_K, 3 = Q6_K; canonical blocks (IEEE fp16 patterns in the fp16 fields)
+REF_API void ref_dequantize_row_k(const uint8_t* canon, int wtype, float* y, int k) {
+  int nb = k / QK_K;
+  if (wtype == 2) {
+    std::vector<block_q4_K> w;
+    to_ref_q4k(canon, nb, w);
+    dequantize_row_q4_K(w.data(), y, k);
+  } else {
+    std::vector<block_q6_K> w;
+    to_ref_q6k(canon, nb, w);
+    dequantize_row_q6_K(w.data(), y, k);
+  }
+}
+
+// Linear the way ggml::mat_mul's generic branch runs it: quantize_row_q8_K per activation row, vec_dot per output, + bias
+REF_API void ref_linear_kq(const float* x, const uint8_t* W_canon, int wtype, const float* bias, float* y, int M, int N, int K) {
+  int nb = K / QK_K;
+  std::vector<block_q8_K> xq((size_t)M * nb);
+  std::memset(xq.data(), 0, sizeof(block_q8_K) * xq.size());
+  for (int m = 0; m < M; m++) quantize_row_q8_K(x + (size_t)m * K, xq.data() + (size_t)m * nb, K);
+  std::vector<block_q4_K> w4;
+  std::vector<block_q6_K> w6;
+  for (int n = 0; n < N; n++) {
+    if (wtype == 2) to_ref_q4k(W_canon + (size_t)n * nb * 144, nb, w4);
+    else to_ref_q6k(W_canon + (size_t)n * nb * 210, nb, w6);
+    for (int m = 0; m < M; m++) {
+      float s = 0.f;
+      if (wtype == 2) vec_dot_q4_K_q8_K(K, &s, w4.data(), xq.data() + (size_t)m * nb);
+      else vec_dot_q6_K_q8_K(K, &s, w6.data(), xq.data() + (size_t)m * nb);
+      y[(size_t)m * N + n] = bias ? s + bias[n] : s;
+    }
+  }
+}
+
+// The reference's offline quantizers (quantize_q4.cpp:184-282, quantize_q6.cpp:34-106) -> canonical blocks carrying the
+// EFFECTIVE scale patterns (what an x86 read of the stored field yields), used to make realistic fixtures.
+REF_API void ref_quantize_row_k(const float* x, uint8_t* canon, int wtype, int k) {
+  int nb = k / QK_K;
+  if (wtype == 2) {
+    std::vector<block_q4_K> y(nb);
+    quantize_row_q4_K(x, y.data(), k);
+    for (int i = 0; i < nb; i++) {
+      uint16_t d = (uint16_t)(float)y[i].d, m = (uint16_t)(float)y[i].dmin;
+      std::memcpy(canon + (size_t)i * 144, &d, 2);
+      std::memcpy(canon + (size_t)i * 144 + 2, &m, 2);
+      std::memcpy(canon + (size_t)i * 144 + 4, y[i].scales, 12);
+      std::memcpy(canon + (size_t)i * 144 + 16, y[i].qs, 128);
+    }
+  } else {
+    std::vector<block_q6_K> y(nb);
+    quantize_row_q6_K(x, y.data(), k);
+    for (int i = 0; i < nb; i++) {
+      std::memcpy(canon + (size_t)i * 210, y[i].ql, 128);
+      std::memcpy(canon + (size_t)i * 210 + 128, y[i].qh, 64);
+      std::memcpy(canon + (size_t)i * 210 + 192, y[i].scales, 16);
+      uint16_t d = (uint16_t)(float)y[i].d;
+      std::memcpy(canon + (size_t)i * 210 + 208, &d, 2);
+    }
+  }
+}

@@ -1,0 +1,110 @@
+"""GPU parity of the Q4_K / Q6_K Linear against the CPU oracle (which is pinned bit for bit against the compiled reference
+kernels in tests/test_oracle_vs_reference.py).
+
+Bars: Q8_K activation codes, scales and sums of 16, and dequantized weights bit-exact; fp32 outputs rel-L2 <= 1e-3 (the
+integer part is exact, the fp32 accumulation order differs from the CPU's eight lanes; measured about 1e-7)."""
+import numpy as np
+import pytest
+import torch
+
+from mllm_amd import _lib, qlinear as ql, synth
+from oracle import oracle as orc
+from gpu_util import announce, bf16_dev, rel_l2, to_dev
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_q8_K_quantization_bit_exact(dtype):
+    rng = synth.rng_for(7, 1)
+    M, K = 7, 2560
+    if dtype == "bf16":
+        bits, xf = synth.make_x_bf16(rng, M, K)
+        x = bf16_dev(bits)
+    else:
+        xf = synth.make_x_fp32(rng, M, K) * 3
+        xf[1, 256:512] = 0                       # an all-zero super-block
+        xf[2, :256] = 0.1
+        xf[2, 9], xf[2, 200] = -4.5, 4.5         # equal magnitudes, opposite signs: the first one decides
+        xf[3, 512:768] = 0.25
+        xf[3, 767] = -0.25                       # the LAST element differs in sign only
+        x = to_dev(xf)
+    announce("q8_K quantization", dtype)
+    q, d, bs = ql.quantize_q8_K(x)
+    oq, od, obs = orc.quantize_rows_q8_K(xf)
+    assert np.array_equal(q.cpu().numpy(), oq)
+    assert np.array_equal(d.cpu().numpy().view(np.uint32), od.view(np.uint32))
+    assert np.array_equal(bs.cpu().numpy(), obs)
+
+
+@pytest.mark.parametrize("wtype", [2, 3])
+def test_prepack_and_dequantize_bit_exact(wtype):
+    rng = synth.rng_for(7, 10 + wtype)
+    N, K = 37, 1280
+    W = synth.make_weight(rng, wtype, N, K)
+    announce("kq dequantize", wtype)
+    w = ql.PackedKWeight(wtype, torch.from_numpy(W))
+    assert np.array_equal(w.dequantize().cpu().numpy().view(np.uint32), orc.dequantize_k(W, wtype, orc.SCALE_IEEE).view(np.uint32))
+    # blocks written by the x86 build: the fp16 fields hold the pattern as a NUMBER
+    Wx = W.copy()
+    for off in ((0, 2) if wtype == 2 else (208,)):
+        pat = W[:, :, off:off + 2].copy().view(np.uint16).astype(np.float32)
+        Wx[:, :, off:off + 2] = pat.astype(np.float16).view(np.uint16).reshape(N, -1, 1).view(np.uint8)
+    wx = ql.PackedKWeight(wtype, torch.from_numpy(Wx), weight_scale_mode=ql.SCALE_X86_REF)
+    assert np.array_equal(wx.dequantize().cpu().numpy().view(np.uint32), orc.dequantize_k(W, wtype, orc.SCALE_X86_REF).view(np.uint32))
+
+
+@pytest.mark.parametrize("wtype", [2, 3])
+@pytest.mark.parametrize("M,N,K", [(1, 256, 2560), (2, 100, 256), (3, 77, 768), (4, 512, 2048), (8, 130, 9728), (5, 31, 512),
+                                   (11, 64, 1024), (20, 48, 2560)])
+def test_linear_kq(wtype, M, N, K):
+    rng = synth.rng_for(7, 100 + wtype * 1000 + M * 13 + N)
+    W = synth.make_weight(rng, wtype, N, K)
+    w = ql.PackedKWeight(wtype, torch.from_numpy(W))
+    bias = rng.standard_normal(N).astype(np.float32)
+    xf = synth.make_x_fp32(rng, M, K)
+    announce("linear kq", wtype, M, N, K)
+    y = ql.linear_kq(w, to_dev(xf)).cpu().numpy()
+    assert rel_l2(y, orc.linear_kq(xf, W, wtype, None, orc.SCALE_X86_REF)) < 2e-6
+    yb = ql.linear_kq(w, to_dev(xf), to_dev(bias)).cpu().numpy()
+    assert rel_l2(yb, orc.linear_kq(xf, W, wtype, bias, orc.SCALE_X86_REF)) < 2e-6
+    bits, xb = synth.make_x_bf16(rng, M, K)
+    y2 = ql.linear_kq(w, bf16_dev(bits)).cpu().numpy()
+    assert rel_l2(y2, orc.linear_kq(xb, W, wtype, None, orc.SCALE_X86_REF)) < 2e-6
+
+
+@pytest.mark.parametrize("wtype", [2, 3])
+def test_linear_kq_exact_cases(wtype):
+    """unit scales and integer activations that quantize to themselves: every product is an integer below 2^24, so the
+    result must equal the integer matrix product exactly"""
+    rng = synth.rng_for(7, 50 + wtype)
+    N, K, M = 64, 512, 4
+    W = synth.make_weight(rng, wtype, N, K)
+    if wtype == 2:
+        W[:, :, 0:2] = np.array([0x00, 0x3c], np.uint8)
+        W[:, :, 2:4] = np.array([0x00, 0x3c], np.uint8)
+    else:
+        W[:, :, 208:210] = np.array([0x00, 0x3c], np.uint8)
+        W[:, :, 192:208] = rng.integers(-3, 4, size=(N, K // 256, 16)).astype(np.int8).view(np.uint8)
+    x = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    x[:, ::256] = -128.0  # max = -128 -> iscale = 1, d = 1: codes equal the values
+    wd = orc.dequantize_k(W, wtype, orc.SCALE_IEEE).astype(np.float64)
+    want = x.astype(np.float64) @ wd.T
+    assert np.abs(want).max() < 2 ** 24
+    announce("linear kq exact", wtype)
+    y = ql.linear_kq(ql.PackedKWeight(wtype, torch.from_numpy(W)), to_dev(x)).cpu().numpy()
+    assert np.array_equal(y.astype(np.float64), want)
+
+
+def test_argument_checks():
+    L = _lib.lib()
+    buf = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    p = buf.data_ptr()
+    assert L.mllm_hip_kq_packed_bytes(2, 4, 100) == 0
+    assert L.mllm_hip_kq_packed_bytes(0, 4, 256) == 0
+    assert L.mllm_hip_linear_kq(2, p, p, 0, None, p, 1, 4, 100, None) == -2
+    assert L.mllm_hip_linear_kq(1, p, p, 0, None, p, 1, 4, 256, None) == -1
+    assert L.mllm_hip_linear_kq(2, p + 16, p, 0, None, p, 1, 4, 256, None) == -3
+    assert L.mllm_hip_kq_prepack(3, None, 0, p, 4, 256, None) == -1
+    assert L.mllm_hip_quantize_q8_K(p, 0, p, p, p, 1, 100, None) == -2

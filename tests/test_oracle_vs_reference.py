@@ -149,3 +149,45 @@ def test_q8_0_offline_quantizer_bit_exact():
     qs, bits = orc.quantize_rows_q8_0(w)
     assert np.array_equal(ieee[:, :, 0:2].copy().view(np.uint16)[:, :, 0], bits)
     assert np.array_equal(ieee[:, :, 2:].view(np.int8).reshape(16, -1), qs)
+
+
+# ---- K-quants ------------------------------------------------------------------------------------------------------
+def test_q8_K_quantizer_bit_exact():
+    rng = np.random.default_rng(41)
+    x = (rng.standard_normal((6, 1024)) * 3).astype(np.float32)
+    x[1, 256:512] = 0                      # an all-zero super-block
+    x[2, 0], x[2, 7] = -4.5, 4.5           # equal magnitudes, opposite signs: the FIRST one sets the sign of the scale
+    x[2, 1:7] = 0.1
+    x[2, 8:256] = 0.1
+    x[3, 300] = 1e-30
+    q, d, bs = orc.quantize_rows_q8_K(x)
+    rq, rd, rbs = orc.ref_quantize_rows_q8_K(x)
+    assert np.array_equal(q, rq) and np.array_equal(d.view(np.uint32), rd.view(np.uint32))
+    nz = np.repeat(d != 0, 16, axis=1)
+    assert np.array_equal(bs[nz], rbs[nz])   # the reference leaves the sums of an all-zero block unwritten
+    assert d[2, 0] > 0 and q[2, 0] == -128 and q[2, 7] == 127
+
+
+@pytest.mark.parametrize("wtype", [2, 3])
+def test_kquant_dequantize_and_linear_bit_exact(wtype):
+    rng = np.random.default_rng(42 + wtype)
+    N, K, M = 24, 1024, 5
+    # random blocks, and blocks the reference's own offline quantizer makes from fp32 weights
+    for W in (synth.make_weight(rng, wtype, N, K), orc.ref_quantize_rows_k((rng.standard_normal((N, K)) * 0.05).astype(np.float32), wtype)):
+        assert np.array_equal(orc.dequantize_k(W, wtype, orc.SCALE_X86_REF).view(np.uint32), orc.ref_dequantize_k(W, wtype).view(np.uint32))
+        x = rng.standard_normal((M, K)).astype(np.float32)
+        bias = rng.standard_normal(N).astype(np.float32)
+        y = orc.linear_kq(x, W, wtype, bias, orc.SCALE_X86_REF)
+        assert np.array_equal(y.view(np.uint32), orc.ref_linear_kq(x, W, wtype, bias).view(np.uint32))
+        # the exact integers behind it: brute force from the dequantized codes
+        xq, xd, xbs = orc.quantize_rows_q8_K(x)
+        isum, msum = orc.kq_block_sums(W, wtype, xq, xbs)
+        unit = W.copy()
+        if wtype == 2:
+            unit[:, :, 0:2] = np.array([0x00, 0x3c], np.uint8)  # d = 1.0
+            unit[:, :, 2:4] = 0                                  # dmin = 0: codes * sub-block scales remain
+        else:
+            unit[:, :, 208:210] = np.array([0x00, 0x3c], np.uint8)
+        wq = orc.dequantize_k(unit, wtype, orc.SCALE_IEEE).astype(np.int64).reshape(N, K // 256, 256)
+        want = np.einsum("nbk,mbk->nmb", wq, xq.astype(np.int64).reshape(M, K // 256, 256))
+        assert np.array_equal(isum, want)
