@@ -378,6 +378,31 @@ def main():
         torch.cuda.empty_cache()
 
     if not args.no_extra:
+        # Q4_K / Q6_K weights (the formats of the shipped Qwen3-MoE recipe) on the same layer shapes: one launch per
+        # projection (252 per step), Q8_K activation quantization inside the kernel
+        kq = {}
+        for kname, kt, bb in (("q4_k", ql.Q4_K, 144), ("q6_k", ql.Q6_K, 210)):
+            kpool = [{name: ql.PackedKWeight.synthetic(kt, n, k, gen) for name, (n, k) in shapes.items()} for _ in range(N_LAYERS)]
+            for M in (1, 8):
+                xs, ys = make_io(M)
+                kws = {k: ql.kq_workspace(M, k) for k in (2560, 4096, 9728)}
+
+                def kstep():
+                    for layer in kpool:
+                        for name, w in layer.items():
+                            ql.linear_kq(w, xs[w.K], out=ys[name], workspace=kws[w.K])
+                wall, ev = timed(graphed(kstep), 5, 2)
+                nbytes = N_LAYERS * sum(n * (k // 256) * bb + M * k * 2 + M * n * 4 for n, k in shapes.values())
+                kq["%s_m%d" % (kname, M)] = {"GBps": nbytes * 5 / wall / 1e9, "ms_per_step": wall / 5 * 1e3, "bytes_per_step": nbytes}
+            x1 = torch.randn((1, 2560), device="cuda", generator=gen).to(torch.bfloat16)
+            y1 = torch.empty((1, 9728), dtype=torch.float32, device="cuda")
+            _, ev = timed(graphed(lambda: [ql.linear_kq(l["gate_proj"], x1, out=y1) for l in kpool]), 5, 2)
+            per = ev / (5 * N_LAYERS)
+            nb1 = 9728 * 10 * bb + 2560 * 2 + 9728 * 4
+            kq["%s_m1" % kname]["gate_proj"] = {"us": per * 1e6, "GBps": nb1 / per / 1e9, "bytes": nb1}
+            del kpool
+            torch.cuda.empty_cache()
+        extra["kquant_decode"] = kq
         # what a stream of launches of this size can reach at all: a read-only 16-byte streaming kernel over distinct buffers
         floor = {}
         big = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device="cuda", generator=gen)

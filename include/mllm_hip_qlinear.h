@@ -284,9 +284,12 @@ int mllm_hip_moe_route(const int32_t* topk_ids, int64_t T, int E, int k, int32_t
 size_t mllm_hip_kq_packed_bytes(int wtype, int64_t N, int64_t K);
 int mllm_hip_kq_prepack(int wtype, const void* blocks, int weight_scale_mode, void* packed, int64_t N, int64_t K, void* stream);
 /* y[M][N] fp32 = x[M][K] (fp32 or bf16) * W^T + bias.  K % 256 == 0.  Up to eight rows per launch (decode); more rows run
- * as groups of eight, each streaming the weights again. */
+ * as groups of eight, each streaming the weights again.  workspace (mllm_hip_kq_workspace_bytes, may be NULL): from three
+ * rows on x is quantized once by a small kernel and the GEMV copies that image instead of quantizing in every workgroup
+ * (same results bit for bit). */
+size_t mllm_hip_kq_workspace_bytes(int64_t M, int64_t K);
 int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y, int64_t M, int64_t N,
-                       int64_t K, void* stream);
+                       int64_t K, void* workspace, void* stream);
 /* Parity probes.  Dequantized weights fp32 [N][K] (dequantize_row_q4_K / _q6_K, quantize_q4.cpp:284-312, quantize_q6.cpp:108-133);
  * Q8_K activation quantization: codes int8 [M][K], d fp32 [M][K/256], sums of 16 codes int16 [M][K/16]. */
 int mllm_hip_kq_dequantize(int wtype, const void* packed, float* w, int64_t N, int64_t K, void* stream);

@@ -181,6 +181,20 @@ void HipLinearOp::load(const ParameterFile::ptr_t& ploader) {
       if (options_.bias) bias_dev_ = onDevice(bias_);
       break;
     }
+    case kGGUF_Q4_K:
+    case kGGUF_Q6_K: {
+      scheme_ = weight_.dtype() == kGGUF_Q4_K ? Scheme::kQ4_K : Scheme::kQ6_K;
+      const int wt = scheme_ == Scheme::kQ4_K ? MLLM_HIP_Q4_K : MLLM_HIP_Q6_K;
+      MLLM_RT_ASSERT_EQ((int64_t)weight_.numel(), N * K);
+      const size_t pb = mllm_hip_kq_packed_bytes(wt, N, K);
+      if (pb == 0) MLLM_ERROR_EXIT(ExitCode::kCoreError, "Linear %s: in_channels %d is not a multiple of 256", getName().c_str(), (int)K);
+      Tensor dev_blocks = onDevice(weight_);
+      packed_ = Tensor::empty({(int32_t)pb}, kByte, kHIP).alloc();
+      MLLM_HIP_KERNEL_CHECK(mllm_hip_kq_prepack(wt, dev_blocks.ptr<void>(), be.config().weight_scale_mode, packed_.ptr<void>(), N, K, be.stream()));
+      be.synchronize();
+      if (options_.bias) bias_dev_ = onDevice(bias_);
+      break;
+    }
     case kInt8: {
       scheme_ = Scheme::kW8A8;
       weight_scale_ = onDevice(ploader->pull(getName() + ".weight.scale"));
@@ -234,7 +248,8 @@ void HipLinearOp::reshape(const std::vector<Tensor>& inputs, std::vector<Tensor>
   MLLM_RT_ASSERT_EQ(o_shape[o_shape.size() - 1], options_.in_channels);
   o_shape[o_shape.size() - 1] = options_.out_channels;
   // block-quantized weights produce fp32 like the CPU backend's kGGUF path (mllm/backends/cpu/ops/LinearOp.cpp:357-360)
-  const DataTypes o_dtype = (scheme_ == Scheme::kQ4_0 || scheme_ == Scheme::kQ8_0) ? kFloat32 : kBFloat16;
+  const bool blocks = scheme_ == Scheme::kQ4_0 || scheme_ == Scheme::kQ8_0 || scheme_ == Scheme::kQ4_K || scheme_ == Scheme::kQ6_K;
+  const DataTypes o_dtype = blocks ? kFloat32 : kBFloat16;
   outputs.emplace_back(Tensor::empty(o_shape, o_dtype, i.device()));
 }
 
@@ -282,6 +297,12 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
       }
       break;
     }
+    case Scheme::kQ4_K:
+    case Scheme::kQ6_K:
+      MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_kq(scheme_ == Scheme::kQ4_K ? MLLM_HIP_Q4_K : MLLM_HIP_Q6_K, packed_.ptr<void>(), x.ptr<void>(), xdt(),
+                                               bias, y.ptr<float>(), M, N, K, M >= 3 ? workspace(mllm_hip_kq_workspace_bytes(M, K)) : nullptr,
+                                               st));
+      break;
     case Scheme::kW8A8: {
       void* ws = workspace(mllm_hip_w8a8_workspace_bytes(M, K));
       MLLM_HIP_KERNEL_CHECK(mllm_hip_w8a8_linear_packed(x.ptr<void>(), xdt(), packed_.ptr<void>(), weight_scale_.ptr<float>(), bias, y.ptr<void>(),

@@ -91,7 +91,7 @@ class HipLinearOp final : public aops::LinearOp {
   ParameterFile::ptr_t getParams() override;
 
  private:
-  enum class Scheme { kNone, kQ4_0, kQ8_0, kW8A8, kW4A16 };
+  enum class Scheme { kNone, kQ4_0, kQ8_0, kQ4_K, kQ6_K, kW8A8, kW4A16 };
   Scheme scheme_ = Scheme::kNone;
   Tensor packed_;        // the repacked device copy the kernels read (every scheme)
   Tensor gemm_packed_;   // Q4_0 / Q8_0: the matrix-core layout for more than 8 rows

@@ -15,6 +15,8 @@ namespace {
 DataTypes weight_dtype(const std::string& scheme) {
   if (scheme == "q4_0") return kGGUF_Q4_0;
   if (scheme == "q8_0") return kGGUF_Q8_0;
+  if (scheme == "q4_k") return kGGUF_Q4_K;
+  if (scheme == "q6_k") return kGGUF_Q6_K;
   if (scheme == "w8a8") return kInt8;
   if (scheme == "w4a16") return kUInt8;
   MLLM_ERROR_EXIT(ExitCode::kCoreError, "unknown scheme '%s'", scheme.c_str());

@@ -18,11 +18,13 @@ size_t bytesOfType(DataTypes t) {
     case kInt64: return 8;
     case kGGUF_Q4_0: return 18;  // block_q4_0, mllm/core/DataTypes.hpp:111-121
     case kGGUF_Q8_0: return 34;  // block_q8_0, :164-170
+    case kGGUF_Q4_K: return 144; // block_q4_K, :139-147
+    case kGGUF_Q6_K: return 210; // block_q6_K, :153-160
     case kInt8: case kUInt8: case kByte: case kUInt4: return 1;  // kUInt4 is a 1-byte placeholder (DataTypes.hpp:336-339)
   }
   MLLM_ERROR_EXIT(ExitCode::kCoreError, "bytesOfType: unknown dtype %d", (int)t);
 }
-size_t lanesOfType(DataTypes t) { return (t == kGGUF_Q4_0 || t == kGGUF_Q8_0) ? 32 : 1; }
+size_t lanesOfType(DataTypes t) { return (t == kGGUF_Q4_0 || t == kGGUF_Q8_0) ? 32 : ((t == kGGUF_Q4_K || t == kGGUF_Q6_K) ? 256 : 1); }
 
 // ---- host allocator -----------------------------------------------------------------------------------------
 namespace {

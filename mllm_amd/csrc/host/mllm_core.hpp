@@ -49,7 +49,7 @@ enum class ExitCode : int32_t { kSuccess = 0, kCoreError = 1, kAssert = 2, kIOEr
 #define NYI(...) MLLM_ERROR_EXIT(::mllm::ExitCode::kCoreError, "NYI: " __VA_ARGS__)
 
 enum DataTypes : int32_t {
-  kFloat32 = 0, kFloat16 = 1, kGGUF_Q4_0 = 2, kGGUF_Q8_0 = 8, kInt8 = 16, kInt16 = 17, kInt32 = 18,
+  kFloat32 = 0, kFloat16 = 1, kGGUF_Q4_0 = 2, kGGUF_Q8_0 = 8, kGGUF_Q4_K = 12, kGGUF_Q6_K = 14, kInt8 = 16, kInt16 = 17, kInt32 = 18,
   kBFloat16 = 128, kUInt8 = 129, kUInt16 = 130, kUInt32 = 131, kInt64 = 132, kByte = 134, kUInt4 = 137,
 };
 // bytes of one storage unit and elements ("lanes") per unit: mllm/core/DataTypes.hpp:645-648, TensorStorage.cpp:48-49

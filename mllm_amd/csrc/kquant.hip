@@ -163,17 +163,19 @@ __device__ __forceinline__ Q8KItem quantize_q8k_item(const float (&v)[8], int la
     }
   }
   int src = lane;
-#pragma unroll
-  for (int off = 1; off < 32; off <<= 1) {
-    const float oa = __shfl_xor(amax, off, 64);
-    const float om = __shfl_xor(mx, off, 64);
-    const int os = __shfl_xor(src, off, 64);
+  // butterfly over the 32 lanes: within a row of 16 lanes through DPP, the last step through a lane shuffle
+  auto take = [&](float oa, float om, int os) {
     if (oa > amax || (oa == amax && os < src)) {
       amax = oa;
       mx = om;
       src = os;
     }
-  }
+  };
+  take(dpp_f<0xB1>(amax), dpp_f<0xB1>(mx), __builtin_amdgcn_update_dpp(0, src, 0xB1, 0xf, 0xf, true));     // lane ^ 1
+  take(dpp_f<0x4E>(amax), dpp_f<0x4E>(mx), __builtin_amdgcn_update_dpp(0, src, 0x4E, 0xf, 0xf, true));     // lane ^ 2
+  take(dpp_f<0x141>(amax), dpp_f<0x141>(mx), __builtin_amdgcn_update_dpp(0, src, 0x141, 0xf, 0xf, true));  // half-row mirror
+  take(dpp_f<0x140>(amax), dpp_f<0x140>(mx), __builtin_amdgcn_update_dpp(0, src, 0x140, 0xf, 0xf, true));  // row mirror
+  take(__shfl_xor(amax, 16, 64), __shfl_xor(mx, 16, 64), __shfl_xor(src, 16, 64));
   Q8KItem r{0u, 0u, 0, 0.f};
   if (amax == 0.f) return r;
   const float iscale = -128.f / mx;
@@ -215,14 +217,20 @@ __device__ __forceinline__ void load8(const void* x, int64_t elem, float (&v)[8]
   }
 }
 
-// stand-alone form (parity probe): codes int8 [M][K], d fp32 [M][K/256], sums of 16 int16 [M][K/16]
+// stand-alone form: codes int8 [rows][K], d fp32 [rows][K/256], sums of 16 int16 [rows][K/16]; items from `valid` on
+// (rows beyond the real ones) are written as zeros.  Used as parity probe and, with the three arrays back to back, to
+// write the image the GEMV copies into LDS.
+constexpr int KQ_IMAGE = 2;  // activation "type": the quantized image instead of activations
 __global__ __launch_bounds__(256) void quantize_q8k_kernel(const void* __restrict__ x, int x_dtype, int8_t* __restrict__ codes,
-                                                           float* __restrict__ d, int16_t* __restrict__ bsums, int64_t nitems) {
+                                                           float* __restrict__ d, int16_t* __restrict__ bsums, int64_t nitems,
+                                                           int64_t valid) {
   const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;  // nitems is a multiple of 32: whole half-waves
   if (it >= nitems) return;
-  float v[8];
-  if (x_dtype == MLLM_HIP_F32) load8<MLLM_HIP_F32>(x, it * 8, v);
-  else load8<MLLM_HIP_BF16>(x, it * 8, v);
+  float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  if (it < valid) {
+    if (x_dtype == MLLM_HIP_F32) load8<MLLM_HIP_F32>(x, it * 8, v);
+    else load8<MLLM_HIP_BF16>(x, it * 8, v);
+  }
   const Q8KItem r = quantize_q8k_item(v, threadIdx.x & 63);
   *reinterpret_cast<u32x2*>(codes + it * 8) = u32x2{r.q0, r.q1};
   const int s16 = r.sum8 + __builtin_amdgcn_update_dpp(0, r.sum8, 0xB1, 0xf, 0xf, true);  // with the neighbouring lane
@@ -293,7 +301,8 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   constexpr int GROUPS = 64 / G;
   const int grp = lane / G, c0 = lane % G;
-  const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * (GROUPS * R) + (int64_t)grp * R;
+  const int nthreads = blockDim.x;  // 128 or 256
+  const int64_t row0 = ((int64_t)blockIdx.x * (nthreads >> 6) + wave) * (GROUPS * R) + (int64_t)grp * R;
   constexpr int UPS = WT == MLLM_HIP_Q4_K ? 8 : 4;  // units per super-block
   const int units = nsb * UPS;
 
@@ -313,9 +322,15 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
   // ---- activations -> Q8_K in LDS (rows m >= M are zero) ----
   const int nitems = MT * (K >> 3);
   const int valid = a.M * (K >> 3);
-  for (int it = tid; it < nitems; it += 256) {  // whole half-waves: K / 8 is a multiple of 32
+  if (XT == KQ_IMAGE) {  // codes | sums | scales, written by quantize_q8k_kernel in exactly this layout
+    const int n16 = MT * (K >> 4), n4 = MT * nsb * 9;
+    for (int c = tid; c < n16; c += nthreads) s_q[c] = reinterpret_cast<const u32x4*>(a.x)[c];
+    const uint32_t* tail = reinterpret_cast<const uint32_t*>(a.x) + (size_t)n16 * 4;
+    for (int c = tid; c < n4; c += nthreads) s_bs[c] = tail[c];
+  }
+  for (int it = tid; XT != KQ_IMAGE && it < nitems; it += nthreads) {  // whole half-waves: K / 8 is a multiple of 32
     float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (it < valid) load8<XT>(a.x, (int64_t)it * 8, v);
+    if (it < valid) load8<(XT == KQ_IMAGE ? MLLM_HIP_F32 : XT)>(a.x, (int64_t)it * 8, v);
     const Q8KItem q = quantize_q8k_item(v, lane);
     reinterpret_cast<u32x2*>(s_q)[it] = u32x2{q.q0, q.q1};
     const int s16 = q.sum8 + __builtin_amdgcn_update_dpp(0, q.sum8, 0xB1, 0xf, 0xf, true);
@@ -430,9 +445,9 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
 }
 
 template <int WT, int XT, int MT, int G>
-static int launch_kq_g(const KGemvArgs& a, hipStream_t st) {
+static int launch_kq_g(const KGemvArgs& a, int NW, hipStream_t st) {
   constexpr int R = 2;
-  constexpr int rows_per_wg = 4 * (64 / G) * R;
+  const int rows_per_wg = NW * (64 / G) * R;
   const int K = a.nsb * QK_K;
   const size_t lds = (size_t)MT * K + (size_t)MT * a.nsb * 4 + (size_t)MT * a.nsb * 32;
   if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
@@ -440,16 +455,29 @@ static int launch_kq_g(const KGemvArgs& a, hipStream_t st) {
   if (lds > 64 * 1024)
     HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   const unsigned grid = (unsigned)((a.N + rows_per_wg - 1) / rows_per_wg);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, a);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 template <int WT, int XT, int MT>
 static int launch_kq_m(const KGemvArgs& a, hipStream_t st) {
+  // Lanes per row: the width that leaves the fewest idle lane-steps over the row's units, among the widths that still
+  // give every CU a workgroup (narrow groups put many rows into one workgroup); the wider one on a tie.  Two waves per
+  // workgroup instead of four when the grid would otherwise stay below the CU count.
   const int units = a.nsb * (WT == MLLM_HIP_Q4_K ? 8 : 4);
-  if (units >= 64) return launch_kq_g<WT, XT, MT, 64>(a, st);
-  if (units >= 32) return launch_kq_g<WT, XT, MT, 32>(a, st);
-  if (units >= 16) return launch_kq_g<WT, XT, MT, 16>(a, st);
-  return launch_kq_g<WT, XT, MT, 8>(a, st);
+  auto grid_of = [&](int g, int nw) { return (a.N + nw * (64 / g) * 2 - 1) / (nw * (64 / g) * 2); };
+  int best = 64, waste = (units + 63) / 64 * 64 - units;
+  for (int g = 32; g >= 8; g >>= 1) {
+    const int w = (units + g - 1) / g * g - units;
+    if (w < waste && grid_of(g, 4) >= 256) {
+      waste = w;
+      best = g;
+    }
+  }
+  const int NW = grid_of(best, 4) >= 256 ? 4 : 2;
+  if (best == 64) return launch_kq_g<WT, XT, MT, 64>(a, NW, st);
+  if (best == 32) return launch_kq_g<WT, XT, MT, 32>(a, NW, st);
+  if (best == 16) return launch_kq_g<WT, XT, MT, 16>(a, NW, st);
+  return launch_kq_g<WT, XT, MT, 8>(a, NW, st);
 }
 template <int WT, int XT>
 static int launch_kq(const KGemvArgs& a, hipStream_t st) {
@@ -502,24 +530,43 @@ MLLM_API int mllm_hip_quantize_q8_K(const void* x, int x_dtype, int8_t* codes, f
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(codes) % 8) return MLLM_HIP_E_ALIGN;
   const int64_t nitems = M * K / 8;
   hipLaunchKernelGGL(quantize_q8k_kernel, dim3((unsigned)((nitems + 255) / 256)), dim3(256), 0, (hipStream_t)stream, x, x_dtype, codes, d,
-                     bsums, nitems);
+                     bsums, nitems, nitems);
   return (int)hipGetLastError();
 }
 
+MLLM_API size_t mllm_hip_kq_workspace_bytes(int64_t M, int64_t K) {
+  if (M <= 0 || K <= 0 || K % QK_K) return 0;
+  return (size_t)8 * K + (size_t)8 * (K / QK_K) * 36;  // one group of eight rows: codes, sums of 16, scales
+}
+
 MLLM_API int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y, int64_t M,
-                                int64_t N, int64_t K, void* stream) {
+                                int64_t N, int64_t K, void* workspace, void* stream) {
   int rc = kq_check(wtype, packed, N, K);
   if (rc) return rc;
   if (!x || !y || M <= 0 || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16)) return MLLM_HIP_E_BADARG;
-  if (reinterpret_cast<uintptr_t>(x) % 16) return MLLM_HIP_E_ALIGN;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
   const size_t xrow = (size_t)K * (x_dtype == MLLM_HIP_F32 ? 4 : 2);
+  const int nsb = (int)(K / QK_K);
+  hipStream_t st = (hipStream_t)stream;
   for (int64_t m0 = 0; m0 < M; m0 += 8) {  // more than eight rows: groups of eight (each streams the weights again)
-    KGemvArgs a{kq_view(wtype, packed, N, K), bias, y + m0 * N, reinterpret_cast<const char*>(x) + m0 * xrow,
-                (int)N, (int)(M - m0 < 8 ? M - m0 : 8), (int)(K / QK_K)};
-    if (wtype == MLLM_HIP_Q4_K)
-      rc = x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_F32>(a, (hipStream_t)stream) : launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_BF16>(a, (hipStream_t)stream);
-    else
-      rc = x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q6_K, MLLM_HIP_F32>(a, (hipStream_t)stream) : launch_kq<MLLM_HIP_Q6_K, MLLM_HIP_BF16>(a, (hipStream_t)stream);
+    const int rows = (int)(M - m0 < 8 ? M - m0 : 8);
+    const void* xg = reinterpret_cast<const char*>(x) + m0 * xrow;
+    KGemvArgs a{kq_view(wtype, packed, N, K), bias, y + m0 * N, xg, (int)N, rows, nsb};
+    if (workspace && rows >= 3) {
+      // several rows: quantize once for all workgroups; the GEMV then copies the image instead of quantizing
+      const int MT = rows <= 4 ? 4 : 8;
+      int8_t* img = reinterpret_cast<int8_t*>(workspace);
+      const int64_t nitems = (int64_t)MT * K / 8;
+      hipLaunchKernelGGL(quantize_q8k_kernel, dim3((unsigned)((nitems + 255) / 256)), dim3(256), 0, st, xg, x_dtype, img,
+                         reinterpret_cast<float*>(img + (size_t)MT * K + (size_t)MT * nsb * 32),
+                         reinterpret_cast<int16_t*>(img + (size_t)MT * K), nitems, (int64_t)rows * K / 8);
+      a.x = img;
+      rc = wtype == MLLM_HIP_Q4_K ? launch_kq<MLLM_HIP_Q4_K, KQ_IMAGE>(a, st) : launch_kq<MLLM_HIP_Q6_K, KQ_IMAGE>(a, st);
+    } else if (wtype == MLLM_HIP_Q4_K) {
+      rc = x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_F32>(a, st) : launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_BF16>(a, st);
+    } else {
+      rc = x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q6_K, MLLM_HIP_F32>(a, st) : launch_kq<MLLM_HIP_Q6_K, MLLM_HIP_BF16>(a, st);
+    }
     if (rc) return rc;
   }
   return 0;

@@ -525,12 +525,17 @@ class PackedKWeight:
         return w
 
 
-def linear_kq(w, x, bias=None, out=None):
+def kq_workspace(M, K):
+    return torch.empty(_lib.lib().mllm_hip_kq_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+
+
+def linear_kq(w, x, bias=None, out=None, workspace=None):
+    """workspace (kq_workspace): from three rows on, x is quantized once by a small kernel instead of in every workgroup"""
     assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
     M = x.shape[0]
     y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")
-    _lib.check(_lib.lib().mllm_hip_linear_kq(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K, _stream()),
-               "mllm_hip_linear_kq")
+    _lib.check(_lib.lib().mllm_hip_linear_kq(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K,
+                                             _p(workspace), _stream()), "mllm_hip_linear_kq")
     return y
 
 

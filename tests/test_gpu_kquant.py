@@ -70,8 +70,12 @@ def test_linear_kq(wtype, M, N, K):
     yb = ql.linear_kq(w, to_dev(xf), to_dev(bias)).cpu().numpy()
     assert rel_l2(yb, orc.linear_kq(xf, W, wtype, bias, orc.SCALE_X86_REF)) < 2e-6
     bits, xb = synth.make_x_bf16(rng, M, K)
-    y2 = ql.linear_kq(w, bf16_dev(bits)).cpu().numpy()
-    assert rel_l2(y2, orc.linear_kq(xb, W, wtype, None, orc.SCALE_X86_REF)) < 2e-6
+    y2 = ql.linear_kq(w, bf16_dev(bits))
+    assert rel_l2(y2.cpu().numpy(), orc.linear_kq(xb, W, wtype, None, orc.SCALE_X86_REF)) < 2e-6
+    # with a workspace (x quantized once by its own kernel): the same bits
+    ws = ql.kq_workspace(M, K)
+    assert torch.equal(ql.linear_kq(w, to_dev(xf), to_dev(bias), workspace=ws), torch.from_numpy(yb).cuda())
+    assert torch.equal(ql.linear_kq(w, bf16_dev(bits), workspace=ws), y2)
 
 
 @pytest.mark.parametrize("wtype", [2, 3])
@@ -103,8 +107,8 @@ def test_argument_checks():
     p = buf.data_ptr()
     assert L.mllm_hip_kq_packed_bytes(2, 4, 100) == 0
     assert L.mllm_hip_kq_packed_bytes(0, 4, 256) == 0
-    assert L.mllm_hip_linear_kq(2, p, p, 0, None, p, 1, 4, 100, None) == -2
-    assert L.mllm_hip_linear_kq(1, p, p, 0, None, p, 1, 4, 256, None) == -1
-    assert L.mllm_hip_linear_kq(2, p + 16, p, 0, None, p, 1, 4, 256, None) == -3
+    assert L.mllm_hip_linear_kq(2, p, p, 0, None, p, 1, 4, 100, None, None) == -2
+    assert L.mllm_hip_linear_kq(1, p, p, 0, None, p, 1, 4, 256, None, None) == -1
+    assert L.mllm_hip_linear_kq(2, p + 16, p, 0, None, p, 1, 4, 256, None, None) == -3
     assert L.mllm_hip_kq_prepack(3, None, 0, p, 4, 256, None) == -1
     assert L.mllm_hip_quantize_q8_K(p, 0, p, p, p, 1, 100, None) == -2

@@ -83,6 +83,15 @@ def test_linear_through_the_op_factory(via_plugin):
             bits, xf = synth.make_x_bf16(rng, M, K)
             y = _run(L, scheme, W, None, None, None, bits, True, M, N, K, 0, via_plugin)
             assert rel_l2(y, orc.linear_q(xf, W, wtype, None, orc.SCALE_X86_REF)) < tol
+    # K-quants
+    for scheme, wtype in (("q4_k", 2), ("q6_k", 3)):
+        W = synth.make_weight(rng, wtype, N, K)
+        bias = rng.standard_normal(N).astype(np.float32)
+        for M in (1, 5, 20):
+            x = synth.make_x_fp32(rng, M, K)
+            announce("host linear", scheme, M)
+            y = _run(L, scheme, W, None, None, bias, x, False, M, N, K, 0, via_plugin)
+            assert rel_l2(y, orc.linear_kq(x, W, wtype, bias, orc.SCALE_X86_REF)) < 2e-6
     # W8A8
     M = 40
     a_bits, W8, ws = synth.make_w8a8(rng, M, N, K)
