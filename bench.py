@@ -40,6 +40,9 @@ def parse():
     ap.add_argument("--side-only", action="store_true",
                     help="profiling run: only the prefill GEMM / MoE side workloads (W8A8, W4A16, MoE FFN, Q4_0 prefill Linear), "
                          "printed as one JSON object; meant to run under rocprofv3")
+    ap.add_argument("--layer-only", action="store_true",
+                    help="profiling run: only the decoder-layer chain (operators one by one and folded, M = 1 and 8) and the "
+                         "Q4_K / Q6_K gate projection, printed as one JSON object; meant to run under rocprofv3")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the M=4/8 and Q8_0 side measurements")
@@ -349,6 +352,17 @@ def main():
         return
     pool = make_pool(wtype, N_LAYERS)
     torch.cuda.synchronize()
+    if args.layer_only:
+        res = {"layer_only": True, "decode_layer_chain": {"m%d" % M: measure_layer_chain(pool, M, reps=3) for M in (1, 8)}}
+        x1 = torch.randn((1, 2560), device="cuda", generator=gen).to(torch.bfloat16)
+        y1 = torch.empty((1, 9728), dtype=torch.float32, device="cuda")
+        for kname, kt in (("q4_k", ql.Q4_K), ("q6_k", ql.Q6_K)):
+            ws = [ql.PackedKWeight.synthetic(kt, 9728, 2560, gen) for _ in range(N_LAYERS)]
+            _, ev = timed(graphed(lambda: [ql.linear_kq(w, x1, out=y1) for w in ws]), 3, 2)
+            res["%s_gate_proj_us" % kname] = ev / (3 * N_LAYERS) * 1e6
+            del ws
+        print(json.dumps(res))
+        return
 
     head = measure_workload(wtype, args.m, pool, args.steps, args.warmup)
     per_shape = {name: measure_shape(wtype, args.m, name, pool)

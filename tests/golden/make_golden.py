@@ -8,6 +8,9 @@ compiled unchanged) on seeded inputs; the inputs are stored next to the outputs 
   gemv_kat.npz        Q4_0 / Q8_0 Linear (quantize_row_q8_0 + vec_dot_*): N=64, K=256, M in {1,3,4,8}, with/without bias
   x86_scale_grid.npz  what a stored scale pattern reads back as on the x86 build, 4096 sampled patterns
   dequant_kat.npz     dequantize_row_q4_0 / dequantize_row_q8_0 on a few rows
+  kquant_kat.npz      Q4_K / Q6_K: blocks made by the reference's own offline quantizers from fp32 weights, their
+                      dequantized values, quantize_row_q8_K of the activations, and the Linear outputs (vec_dot_q4_K_q8_K /
+                      vec_dot_q6_K_q8_K); written alone with `--only kquant`
 """
 import os
 import sys
@@ -37,9 +40,38 @@ def actquant_rows(rng, K=256):
     return np.stack(rows)
 
 
+def kquant():
+    rk = np.random.default_rng(synth.SEED_BASE + 79)
+    N, K = 24, 512
+    out = {}
+    for name, wtype in (("q4_k", 2), ("q6_k", 3)):
+        w = (rk.standard_normal((N, K)) * 0.04).astype(np.float32)
+        w[0, :256] = 0.0                      # an all-zero super-block
+        w[1, :32] = 0.3                       # a constant sub-block
+        W = orc.ref_quantize_rows_k(w, wtype)
+        out[f"{name}_W"] = W
+        out[f"{name}_deq"] = orc.ref_dequantize_k(W, wtype)
+        bias = rk.standard_normal(N).astype(np.float32)
+        out[f"{name}_bias"] = bias
+        for M in (1, 3, 8):
+            x = rk.standard_normal((M, K)).astype(np.float32)
+            out[f"{name}_x{M}"] = x
+            out[f"{name}_y{M}"] = orc.ref_linear_kq(x, W, wtype, bias)
+    x = (rk.standard_normal((4, K)) * 2).astype(np.float32)
+    x[1, 256:] = 0.0
+    x[2, 3], x[2, 77] = 9.0, -9.0
+    q, d, bs = orc.ref_quantize_rows_q8_K(x)
+    bs[np.repeat(d == 0, 16, axis=1)] = 0     # the reference leaves the sums of an all-zero block unwritten
+    out.update(q8k_x=x, q8k_q=q, q8k_d=d, q8k_bsums=bs)
+    np.savez_compressed(os.path.join(OUT, "kquant_kat.npz"), **out)
+
+
 def main():
     if not orc.ref_available():
         raise SystemExit("oracle/_ref/libmllm_ref.so missing: run `make -C oracle ref` where the reference is mounted")
+    if sys.argv[1:] == ["--only", "kquant"]:
+        kquant()
+        return
 
     rng = np.random.default_rng(synth.SEED_BASE + 77)
     x = actquant_rows(rng)
@@ -83,6 +115,7 @@ def main():
     q8_codes, q8_d = orc.ref_quantize_rows_q8_0(w)
     np.savez_compressed(os.path.join(OUT, "weight_quantizer_kat.npz"), w=w, q4_blocks=orc.ref_quantize_rows_q4_0(w),
                         q8_codes=q8_codes, q8_d_eff=q8_d)
+    kquant()
     for f in sorted(os.listdir(OUT)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(OUT, f)))

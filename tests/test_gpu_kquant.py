@@ -112,3 +112,19 @@ def test_argument_checks():
     assert L.mllm_hip_linear_kq(2, p + 16, p, 0, None, p, 1, 4, 256, None, None) == -3
     assert L.mllm_hip_kq_prepack(3, None, 0, p, 4, 256, None) == -1
     assert L.mllm_hip_quantize_q8_K(p, 0, p, p, p, 1, 100, None) == -2
+
+
+@pytest.mark.parametrize("name,wtype", [("q4_k", 2), ("q6_k", 3)])
+def test_golden_kquant(golden_dir, name, wtype):
+    """against what the compiled reference produced on blocks written by its own offline quantizers"""
+    import os
+    g = np.load(os.path.join(golden_dir, "kquant_kat.npz"))
+    announce("golden kquant", name)
+    w = ql.PackedKWeight(wtype, torch.from_numpy(g[f"{name}_W"]))
+    assert np.array_equal(w.dequantize().cpu().numpy().view(np.uint32), g[f"{name}_deq"].view(np.uint32))
+    for M in (1, 3, 8):
+        y = ql.linear_kq(w, to_dev(g[f"{name}_x{M}"]), to_dev(g[f"{name}_bias"])).cpu().numpy()
+        assert rel_l2(y, g[f"{name}_y{M}"]) < 1e-5
+    q, d, bs = ql.quantize_q8_K(to_dev(g["q8k_x"]))
+    assert np.array_equal(q.cpu().numpy(), g["q8k_q"]) and np.array_equal(d.cpu().numpy().view(np.uint32), g["q8k_d"].view(np.uint32))
+    assert np.array_equal(bs.cpu().numpy(), g["q8k_bsums"])

@@ -267,3 +267,18 @@ def test_moe_composition_and_invariance():
     # silu special values
     L = orc.lib()
     assert L.orc_silu(0.0) == 0.0 and abs(L.orc_silu(20.0) - 20.0) < 1e-6 and abs(L.orc_silu(-20.0)) < 1e-7
+
+
+@pytest.mark.parametrize("name,wtype", [("q4_k", 2), ("q6_k", 3)])
+def test_golden_kquant(golden_dir, name, wtype):
+    """blocks written by the reference's offline quantizers, dequantized values, Q8_K activation quantization and Linear
+    outputs as the compiled reference produced them (tests/golden/make_golden.py, kquant)"""
+    g = np.load(os.path.join(golden_dir, "kquant_kat.npz"))
+    W = g[f"{name}_W"]
+    assert np.array_equal(orc.dequantize_k(W, wtype, orc.SCALE_X86_REF).view(np.uint32), g[f"{name}_deq"].view(np.uint32))
+    for M in (1, 3, 8):
+        y = orc.linear_kq(g[f"{name}_x{M}"], W, wtype, g[f"{name}_bias"], orc.SCALE_X86_REF)
+        assert np.array_equal(y.view(np.uint32), g[f"{name}_y{M}"].view(np.uint32))
+    q, d, bs = orc.quantize_rows_q8_K(g["q8k_x"])
+    assert np.array_equal(q, g["q8k_q"]) and np.array_equal(d.view(np.uint32), g["q8k_d"].view(np.uint32))
+    assert np.array_equal(bs, g["q8k_bsums"])
