@@ -392,8 +392,8 @@ def main():
         torch.cuda.empty_cache()
 
     if not args.no_extra:
-        # Q4_K / Q6_K weights (the formats of the shipped Qwen3-MoE recipe) on the same layer shapes: one launch per
-        # projection (252 per step), Q8_K activation quantization inside the kernel
+        # Q4_K / Q6_K weights (the formats of the shipped Qwen3-MoE recipe) on the same layer shapes and launch plan as the
+        # headline workload (144 launches per step), Q8_K activation quantization inside the kernel
         kq = {}
         for kname, kt, bb in (("q4_k", ql.Q4_K, 144), ("q6_k", ql.Q6_K, 210)):
             kpool = [{name: ql.PackedKWeight.synthetic(kt, n, k, gen) for name, (n, k) in shapes.items()} for _ in range(N_LAYERS)]
@@ -401,10 +401,13 @@ def main():
                 xs, ys = make_io(M)
                 kws = {k: ql.kq_workspace(M, k) for k in (2560, 4096, 9728)}
 
-                def kstep():
-                    for layer in kpool:
-                        for name, w in layer.items():
-                            ql.linear_kq(w, xs[w.K], out=ys[name], workspace=kws[w.K])
+                def kstep():  # sibling projections share a launch: qkv | o | gate+up | down
+                    for l in kpool:
+                        ql.linear_kq_multi([l["q_proj"], l["k_proj"], l["v_proj"]], xs[2560], None, [ys["q_proj"], ys["k_proj"], ys["v_proj"]],
+                                           workspace=kws[2560])
+                        ql.linear_kq(l["o_proj"], xs[4096], out=ys["o_proj"], workspace=kws[4096])
+                        ql.linear_kq_multi([l["gate_proj"], l["up_proj"]], xs[2560], None, [ys["gate_proj"], ys["up_proj"]], workspace=kws[2560])
+                        ql.linear_kq(l["down_proj"], xs[9728], out=ys["down_proj"], workspace=kws[9728])
                 wall, ev = timed(graphed(kstep), 5, 2)
                 nbytes = N_LAYERS * sum(n * (k // 256) * bb + M * k * 2 + M * n * 4 for n, k in shapes.values())
                 kq["%s_m%d" % (kname, M)] = {"GBps": nbytes * 5 / wall / 1e9, "ms_per_step": wall / 5 * 1e3, "bytes_per_step": nbytes}

@@ -288,6 +288,12 @@ int mllm_hip_kq_prepack(int wtype, const void* blocks, int weight_scale_mode, vo
  * rows on x is quantized once by a small kernel and the GEMV copies that image instead of quantizing in every workgroup
  * (same results bit for bit). */
 size_t mllm_hip_kq_workspace_bytes(int64_t M, int64_t K);
+/* Up to four Linears that share the activations and K in one launch (q/k/v, gate/up), as mllm_hip_linear_q_gemv_multi. */
+int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int64_t M, int64_t K,
+                             void* workspace, void* stream);
+/* Tuning override of the decode GEMV: lanes per weight row (8/16/32/64), waves per workgroup (1/2/4), units a lane keeps in
+ * flight per row (1/2/4; more than one only for up to two activation rows); 0 = heuristic. */
+int mllm_hip_kq_set_tuning(int lanes_per_row, int waves_per_wg, int units_in_flight);
 int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y, int64_t M, int64_t N,
                        int64_t K, void* workspace, void* stream);
 /* Parity probes.  Dequantized weights fp32 [N][K] (dequantize_row_q4_K / _q6_K, quantize_q4.cpp:284-312, quantize_q6.cpp:108-133);

@@ -13,6 +13,8 @@
 // HBM-bound like the Q4_0 / Q8_0 GEMV: a launch streams 144 (Q4_K) or 210 (Q6_K) bytes per 256 weights once, as 16-byte
 // loads that are contiguous across the lanes of a group.  The reference's array-of-structures blocks (210 is not even a
 // multiple of 4) are split at load time into planes of 16-byte records.
+#include <initializer_list>
+
 #include "qcommon.h"
 
 #define QK_K 256
@@ -239,12 +241,21 @@ __global__ __launch_bounds__(256) void quantize_q8k_kernel(const void* __restric
 }
 
 // ---- GEMV -------------------------------------------------------------------------------------------------------------
-struct KGemvArgs {
+// One launch serves up to four weight matrices that share the activations and K (sibling projections): workgroups
+// [wg_start[p], wg_start[p + 1]) belong to part p.
+constexpr int KQ_MAX_PARTS = 4;
+struct KGemvPart {
   KView w;
   const float* bias;
   float* y;
+  int N;
+};
+struct KGemvArgs {
+  KGemvPart part[KQ_MAX_PARTS];
+  int wg_start[KQ_MAX_PARTS + 1];
+  int nparts;
   const void* x;
-  int N, M, nsb;  // nsb = K / 256
+  int M, nsb;  // nsb = K / 256
 };
 #define KBUF_OOB 0xffffffffu
 #define KBUF_NT 2
@@ -290,7 +301,8 @@ __device__ __forceinline__ int half16(uint32_t pair, int hi) { return (int)(int1
 // Workgroup = NW waves; a wave is cut into 64 / G groups of G lanes; a group owns R consecutive weight rows and its lanes
 // stride over the row's units.  x is quantized to Q8_K once per workgroup into LDS: codes [MT][K], scales [MT][nsb], sums
 // of 16 as int16 [MT][nsb][16].
-template <int WT, int XT, int MT, int G, int R>
+// U = units a lane keeps in flight per row and trip.
+template <int WT, int XT, int MT, int G, int R, int U>
 __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int nsb = a.nsb;
@@ -301,42 +313,98 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   constexpr int GROUPS = 64 / G;
   const int grp = lane / G, c0 = lane % G;
-  const int nthreads = blockDim.x;  // 128 or 256
-  const int64_t row0 = ((int64_t)blockIdx.x * (nthreads >> 6) + wave) * (GROUPS * R) + (int64_t)grp * R;
+  const int nthreads = blockDim.x;  // 64, 128 or 256
+  int pidx = 0;  // uniform: which matrix this workgroup works on
+#pragma unroll
+  for (int p = 1; p < KQ_MAX_PARTS; p++)
+    if (p < a.nparts && (int)blockIdx.x >= a.wg_start[p]) pidx = p;
+  const KGemvPart& pt = a.part[pidx];
+  const int64_t row0 = ((int64_t)(blockIdx.x - a.wg_start[pidx]) * (nthreads >> 6) + wave) * (GROUPS * R) + (int64_t)grp * R;
   constexpr int UPS = WT == MLLM_HIP_Q4_K ? 8 : 4;  // units per super-block
   const int units = nsb * UPS;
 
   KRsrc rs;
   {
-    const uint32_t sbt = (uint32_t)a.N * (uint32_t)nsb;
-    rs.a = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(a.w.a), 0, sbt * 128u, 0x00020000);
-    rs.h = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(WT == MLLM_HIP_Q6_K ? a.w.h : a.w.a), 0, sbt * 64u, 0x00020000);
-    rs.s = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(a.w.s), 0, sbt * 16u, 0x00020000);
-    rs.d = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.w.d), 0, sbt * 2u, 0x00020000);
+    const uint32_t sbt = (uint32_t)pt.N * (uint32_t)nsb;
+    rs.a = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.a), 0, sbt * 128u, 0x00020000);
+    rs.h = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(WT == MLLM_HIP_Q6_K ? pt.w.h : pt.w.a), 0, sbt * 64u, 0x00020000);
+    rs.s = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.s), 0, sbt * 16u, 0x00020000);
+    rs.d = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(pt.w.d), 0, sbt * 2u, 0x00020000);
   }
-  // first trip of weight loads goes out before the activations are touched
-  KUnit<WT> cur[R];
-#pragma unroll
-  for (int r = 0; r < R; r++) load_unit<WT>(cur[r], rs, (uint32_t)((row0 + r) * nsb), c0, units, row0 + r < a.N);
-
-  // ---- activations -> Q8_K in LDS (rows m >= M are zero) ----
+  // Memory requests return in order: the activations a thread will quantize (its first two items) are requested first,
+  // then the first trip of weights, so that the quantization runs while the weights are still on their way.
   const int nitems = MT * (K >> 3);
   const int valid = a.M * (K >> 3);
+  constexpr int XL = XT == KQ_IMAGE ? MLLM_HIP_F32 : XT;
+  u32x4 raw[2][XL == MLLM_HIP_F32 ? 2 : 1];
+  if (XT != KQ_IMAGE) {
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+      const int it = min(tid + k * nthreads, valid - 1);
+      if (XL == MLLM_HIP_F32) {
+        const u32x4* p = reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(a.x) + (int64_t)it * 8);
+        raw[k][0] = p[0];
+        raw[k][XL == MLLM_HIP_F32 ? 1 : 0] = p[1];
+      } else {
+        raw[k][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(a.x) + (int64_t)it * 8);
+      }
+    }
+    __asm__ volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  KUnit<WT> cur[U][R];
+#pragma unroll
+  for (int uu = 0; uu < U; uu++)
+#pragma unroll
+    for (int r = 0; r < R; r++) load_unit<WT>(cur[uu][r], rs, (uint32_t)((row0 + r) * nsb), uu * G + c0, units, row0 + r < pt.N);
+
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+  // ---- activations -> Q8_K in LDS (rows m >= M are zero) ----
   if (XT == KQ_IMAGE) {  // codes | sums | scales, written by quantize_q8k_kernel in exactly this layout
     const int n16 = MT * (K >> 4), n4 = MT * nsb * 9;
     for (int c = tid; c < n16; c += nthreads) s_q[c] = reinterpret_cast<const u32x4*>(a.x)[c];
     const uint32_t* tail = reinterpret_cast<const uint32_t*>(a.x) + (size_t)n16 * 4;
     for (int c = tid; c < n4; c += nthreads) s_bs[c] = tail[c];
   }
-  for (int it = tid; XT != KQ_IMAGE && it < nitems; it += nthreads) {  // whole half-waves: K / 8 is a multiple of 32
-    float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (it < valid) load8<(XT == KQ_IMAGE ? MLLM_HIP_F32 : XT)>(a.x, (int64_t)it * 8, v);
+  auto quantize_to_lds = [&](int it, const float (&v)[8]) {
     const Q8KItem q = quantize_q8k_item(v, lane);
     reinterpret_cast<u32x2*>(s_q)[it] = u32x2{q.q0, q.q1};
     const int s16 = q.sum8 + __builtin_amdgcn_update_dpp(0, q.sum8, 0xB1, 0xf, 0xf, true);
     const int s16b = __builtin_amdgcn_update_dpp(0, s16, 0x4E, 0xf, 0xf, true);  // the other pair of the quad
     if ((it & 3) == 0) s_bs[it >> 2] = ((uint32_t)s16 & 0xffffu) | ((uint32_t)s16b << 16);
     if ((it & 31) == 0) s_d[it >> 5] = q.d;
+  };
+  if (XT != KQ_IMAGE) {
+#pragma unroll
+    for (int k = 0; k < 2; k++) {  // whole half-waves: nitems is a multiple of 32
+      const int it = tid + k * nthreads;
+      if (it < nitems) {
+        float v[8];
+        if (XL == MLLM_HIP_F32) {
+          const u32x4 p = raw[k][0], q = raw[k][XL == MLLM_HIP_F32 ? 1 : 0];
+          v[0] = __uint_as_float(p.x); v[1] = __uint_as_float(p.y); v[2] = __uint_as_float(p.z); v[3] = __uint_as_float(p.w);
+          v[4] = __uint_as_float(q.x); v[5] = __uint_as_float(q.y); v[6] = __uint_as_float(q.z); v[7] = __uint_as_float(q.w);
+        } else {
+          const uint32_t w[4] = {raw[k][0].x, raw[k][0].y, raw[k][0].z, raw[k][0].w};
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            v[2 * j + 0] = __uint_as_float(w[j] << 16);
+            v[2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+          }
+        }
+        if (it >= valid) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = 0.f;
+        }
+        quantize_to_lds(it, v);
+      }
+    }
+    for (int it = tid + 2 * nthreads; it < nitems; it += nthreads) {
+      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (it < valid) load8<XL>(a.x, (int64_t)it * 8, v);
+      quantize_to_lds(it, v);
+    }
   }
   __syncthreads();
 
@@ -346,14 +414,20 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
 #pragma unroll
     for (int m = 0; m < MT; m++) acc[r][m] = 0.f;
 
-  for (int u0 = 0; u0 < units; u0 += G) {
-    KUnit<WT> nxt[R];
-    const bool more = u0 + G < units;  // uniform
+  for (int u0 = 0; u0 < units; u0 += G * U) {
+    KUnit<WT> nxt[U][R];
+    const bool more = u0 + G * U < units;  // uniform
     if (more) {
 #pragma unroll
-      for (int r = 0; r < R; r++) load_unit<WT>(nxt[r], rs, (uint32_t)((row0 + r) * nsb), u0 + G + c0, units, row0 + r < a.N);
+      for (int uu = 0; uu < U; uu++)
+#pragma unroll
+        for (int r = 0; r < R; r++)
+          load_unit<WT>(nxt[uu][r], rs, (uint32_t)((row0 + r) * nsb), u0 + G * U + uu * G + c0, units, row0 + r < pt.N);
     }
-    const int unit = u0 + c0;
+#pragma unroll
+    for (int uu = 0; uu < U; uu++) {
+    const KUnit<WT>(&cu)[R] = cur[uu];
+    const int unit = u0 + uu * G + c0;
     if (unit < units) {
       if (WT == MLLM_HIP_Q4_K) {
         const int sb = unit >> 3, c = unit & 7, jp = c >> 1, hh = c & 1;
@@ -362,16 +436,16 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
         u32x4 wlo[R], whi[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
-          const K4Scales k = k4_scales(cur[r].s.y, cur[r].s.z, cur[r].s.w);
+          const K4Scales k = k4_scales(cu[r].s.y, cu[r].s.z, cu[r].s.w);
           sc_lo[r] = byte_of(k.sc0, k.sc1, 2 * jp);
           sc_hi[r] = byte_of(k.sc0, k.sc1, 2 * jp + 1);
           mn_lo[r] = byte_of(k.mn0, k.mn1, 2 * jp);
           mn_hi[r] = byte_of(k.mn0, k.mn1, 2 * jp + 1);
-          dw[r] = f16bits_to_f32((uint16_t)(cur[r].s.x & 0xffffu));
-          dmw[r] = f16bits_to_f32((uint16_t)(cur[r].s.x >> 16));
+          dw[r] = f16bits_to_f32((uint16_t)(cu[r].s.x & 0xffffu));
+          dmw[r] = f16bits_to_f32((uint16_t)(cu[r].s.x >> 16));
           const uint32_t m4 = 0x0f0f0f0fu;
-          wlo[r] = u32x4{cur[r].a.x & m4, cur[r].a.y & m4, cur[r].a.z & m4, cur[r].a.w & m4};
-          whi[r] = u32x4{(cur[r].a.x >> 4) & m4, (cur[r].a.y >> 4) & m4, (cur[r].a.z >> 4) & m4, (cur[r].a.w >> 4) & m4};
+          wlo[r] = u32x4{cu[r].a.x & m4, cu[r].a.y & m4, cu[r].a.z & m4, cu[r].a.w & m4};
+          whi[r] = u32x4{(cu[r].a.x >> 4) & m4, (cu[r].a.y >> 4) & m4, (cu[r].a.z >> 4) & m4, (cu[r].a.w >> 4) & m4};
         }
 #pragma unroll
         for (int m = 0; m < MT; m++) {
@@ -395,15 +469,15 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
         float dw[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
-          dw[r] = f16bits_to_f32(cur[r].d);
-          const uint32_t sw[4] = {cur[r].s.x, cur[r].s.y, cur[r].s.z, cur[r].s.w};
+          dw[r] = f16bits_to_f32(cu[r].d);
+          const uint32_t sw[4] = {cu[r].s.x, cu[r].s.y, cu[r].s.z, cu[r].s.w};
 #pragma unroll
           for (int g = 0; g < 4; g++) {
-            const u32x4& src = (g & 1) ? cur[r].b : cur[r].a;
+            const u32x4& src = (g & 1) ? cu[r].b : cu[r].a;
             const int sh = (g >= 2) ? 4 : 0;
             const uint32_t m4 = 0x0f0f0f0fu, m2 = 0x03030303u;
-            wv[r][g] = u32x4{((src.x >> sh) & m4) | (((cur[r].h.x >> (2 * g)) & m2) << 4), ((src.y >> sh) & m4) | (((cur[r].h.y >> (2 * g)) & m2) << 4),
-                             ((src.z >> sh) & m4) | (((cur[r].h.z >> (2 * g)) & m2) << 4), ((src.w >> sh) & m4) | (((cur[r].h.w >> (2 * g)) & m2) << 4)};
+            wv[r][g] = u32x4{((src.x >> sh) & m4) | (((cu[r].h.x >> (2 * g)) & m2) << 4), ((src.y >> sh) & m4) | (((cu[r].h.y >> (2 * g)) & m2) << 4),
+                             ((src.z >> sh) & m4) | (((cu[r].h.z >> (2 * g)) & m2) << 4), ((src.w >> sh) & m4) | (((cu[r].h.w >> (2 * g)) & m2) << 4)};
             const int si = 8 * n + 2 * g + t;  // scale of these 16 weights
             sc[r][g] = (int)(int8_t)((sw[si >> 2] >> (8 * (si & 3))) & 0xffu);
           }
@@ -428,9 +502,12 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
         }
       }
     }
+    }
     if (more) {
 #pragma unroll
-      for (int r = 0; r < R; r++) cur[r] = nxt[r];
+      for (int uu = 0; uu < U; uu++)
+#pragma unroll
+        for (int r = 0; r < R; r++) cur[uu][r] = nxt[uu][r];
     }
   }
 
@@ -440,44 +517,59 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
     for (int m = 0; m < MT; m++) {
       const float v = group_sum<G>(acc[r][m]);
       const int64_t row = row0 + r;
-      if (c0 == 0 && row < a.N && m < a.M) a.y[(int64_t)m * a.N + row] = a.bias ? v + a.bias[row] : v;
+      if (c0 == 0 && row < pt.N && m < a.M) pt.y[(int64_t)m * pt.N + row] = pt.bias ? v + pt.bias[row] : v;
     }
 }
 
-template <int WT, int XT, int MT, int G>
-static int launch_kq_g(const KGemvArgs& a, int NW, hipStream_t st) {
-  constexpr int R = 2;
+static int g_kq_G = 0, g_kq_NW = 0, g_kq_U = 0;  // tuning overrides (0 = heuristic)
+
+template <int WT, int XT, int MT, int G, int U>
+static int launch_kq_u(const KGemvArgs& a_in, int NW, hipStream_t st) {
+  constexpr int R = (WT == MLLM_HIP_Q4_K && MT >= 4) ? 4 : 2;  // wider row tiles reuse every LDS read for more weight rows
   const int rows_per_wg = NW * (64 / G) * R;
-  const int K = a.nsb * QK_K;
-  const size_t lds = (size_t)MT * K + (size_t)MT * a.nsb * 4 + (size_t)MT * a.nsb * 32;
+  const int K = a_in.nsb * QK_K;
+  const size_t lds = (size_t)MT * K + (size_t)MT * a_in.nsb * 4 + (size_t)MT * a_in.nsb * 32;
   if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
-  auto kern = kq_gemv_kernel<WT, XT, MT, G, R>;
+  KGemvArgs a = a_in;
+  unsigned grid = 0;
+  for (int p = 0; p < a.nparts; p++) {
+    a.wg_start[p] = (int)grid;
+    grid += (unsigned)((a.part[p].N + rows_per_wg - 1) / rows_per_wg);
+  }
+  a.wg_start[a.nparts] = (int)grid;
+  auto kern = kq_gemv_kernel<WT, XT, MT, G, R, U>;
   if (lds > 64 * 1024)
     HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  const unsigned grid = (unsigned)((a.N + rows_per_wg - 1) / rows_per_wg);
   hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, st, a);
   return (int)hipGetLastError();
 }
+template <int WT, int XT, int MT, int G>
+static int launch_kq_g(const KGemvArgs& a, int NW, int U, hipStream_t st) {
+  if (WT == MLLM_HIP_Q4_K && U >= 4 && MT <= 2) return launch_kq_u<WT, XT, MT, G, (WT == MLLM_HIP_Q4_K && MT <= 2) ? 4 : 1>(a, NW, st);
+  if (U >= 2 && MT <= 2) return launch_kq_u<WT, XT, MT, G, MT <= 2 ? 2 : 1>(a, NW, st);
+  return launch_kq_u<WT, XT, MT, G, 1>(a, NW, st);
+}
 template <int WT, int XT, int MT>
 static int launch_kq_m(const KGemvArgs& a, hipStream_t st) {
-  // Lanes per row: the width that leaves the fewest idle lane-steps over the row's units, among the widths that still
-  // give every CU a workgroup (narrow groups put many rows into one workgroup); the wider one on a tie.  Two waves per
-  // workgroup instead of four when the grid would otherwise stay below the CU count.
+  // Measured on MI355X over the Qwen3-4B projection shapes (lanes per row x waves x units in flight swept): Q4_K rows want 32
+  // lanes, Q6_K rows (units twice as heavy) the whole wave; four waves per workgroup share the activation quantization;
+  // a grid of about one workgroup per CU keeps four units per lane in flight, a larger grid gets its bytes in flight
+  // from occupancy and keeps one.
   const int units = a.nsb * (WT == MLLM_HIP_Q4_K ? 8 : 4);
-  auto grid_of = [&](int g, int nw) { return (a.N + nw * (64 / g) * 2 - 1) / (nw * (64 / g) * 2); };
-  int best = 64, waste = (units + 63) / 64 * 64 - units;
-  for (int g = 32; g >= 8; g >>= 1) {
-    const int w = (units + g - 1) / g * g - units;
-    if (w < waste && grid_of(g, 4) >= 256) {
-      waste = w;
-      best = g;
-    }
-  }
-  const int NW = grid_of(best, 4) >= 256 ? 4 : 2;
-  if (best == 64) return launch_kq_g<WT, XT, MT, 64>(a, NW, st);
-  if (best == 32) return launch_kq_g<WT, XT, MT, 32>(a, NW, st);
-  if (best == 16) return launch_kq_g<WT, XT, MT, 16>(a, NW, st);
-  return launch_kq_g<WT, XT, MT, 8>(a, NW, st);
+  int best = WT == MLLM_HIP_Q4_K ? 32 : 64;
+  while (best > 8 && best / 2 >= units) best >>= 1;
+  int NW = 4;
+  int64_t rows = 0;
+  for (int p = 0; p < a.nparts; p++) rows += a.part[p].N;
+  const int grid = (int)((rows + NW * (64 / best) * 2 - 1) / (NW * (64 / best) * 2));
+  int U = (WT == MLLM_HIP_Q4_K && grid < 512) ? 4 : 1;
+  if (g_kq_G) best = g_kq_G;
+  if (g_kq_NW) NW = g_kq_NW;
+  if (g_kq_U) U = g_kq_U;
+  if (best == 64) return launch_kq_g<WT, XT, MT, 64>(a, NW, U, st);
+  if (best == 32) return launch_kq_g<WT, XT, MT, 32>(a, NW, U, st);
+  if (best == 16) return launch_kq_g<WT, XT, MT, 16>(a, NW, U, st);
+  return launch_kq_g<WT, XT, MT, 8>(a, NW, U, st);
 }
 template <int WT, int XT>
 static int launch_kq(const KGemvArgs& a, hipStream_t st) {
@@ -497,6 +589,19 @@ static int kq_check(int wtype, const void* packed, int64_t N, int64_t K) {
   if (K % QK_K) return MLLM_HIP_E_SHAPE;
   if (N > INT32_MAX || N * (K / QK_K) * 128 >= ((int64_t)1 << 32)) return MLLM_HIP_E_SHAPE;  // 32-bit buffer offsets
   if (reinterpret_cast<uintptr_t>(packed) % 256) return MLLM_HIP_E_ALIGN;
+  return 0;
+}
+
+MLLM_API int mllm_hip_kq_set_tuning(int lanes_per_row, int waves_per_wg, int units_in_flight) {
+  auto ok = [](int v, std::initializer_list<int> allowed) {
+    for (int x : allowed)
+      if (v == x) return true;
+    return false;
+  };
+  if (!ok(lanes_per_row, {0, 8, 16, 32, 64}) || !ok(waves_per_wg, {0, 1, 2, 4}) || !ok(units_in_flight, {0, 1, 2, 4})) return MLLM_HIP_E_BADARG;
+  g_kq_G = lanes_per_row;
+  g_kq_NW = waves_per_wg;
+  g_kq_U = units_in_flight;
   return 0;
 }
 
@@ -539,19 +644,30 @@ MLLM_API size_t mllm_hip_kq_workspace_bytes(int64_t M, int64_t K) {
   return (size_t)8 * K + (size_t)8 * (K / QK_K) * 36;  // one group of eight rows: codes, sums of 16, scales
 }
 
-MLLM_API int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y, int64_t M,
-                                int64_t N, int64_t K, void* workspace, void* stream) {
-  int rc = kq_check(wtype, packed, N, K);
-  if (rc) return rc;
-  if (!x || !y || M <= 0 || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16)) return MLLM_HIP_E_BADARG;
+MLLM_API int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int64_t M,
+                                      int64_t K, void* workspace, void* stream) {
+  if (nparts < 1 || nparts > KQ_MAX_PARTS || !parts) return MLLM_HIP_E_BADARG;
+  if (!x || M <= 0 || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16)) return MLLM_HIP_E_BADARG;
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
+  for (int p = 0; p < nparts; p++) {
+    int rc = kq_check(wtype, parts[p].packed, parts[p].N, K);
+    if (rc) return rc;
+    if (!parts[p].y) return MLLM_HIP_E_BADARG;
+  }
   const size_t xrow = (size_t)K * (x_dtype == MLLM_HIP_F32 ? 4 : 2);
   const int nsb = (int)(K / QK_K);
   hipStream_t st = (hipStream_t)stream;
+  int rc = 0;
   for (int64_t m0 = 0; m0 < M; m0 += 8) {  // more than eight rows: groups of eight (each streams the weights again)
     const int rows = (int)(M - m0 < 8 ? M - m0 : 8);
     const void* xg = reinterpret_cast<const char*>(x) + m0 * xrow;
-    KGemvArgs a{kq_view(wtype, packed, N, K), bias, y + m0 * N, xg, (int)N, rows, nsb};
+    KGemvArgs a{};
+    for (int p = 0; p < nparts; p++)
+      a.part[p] = KGemvPart{kq_view(wtype, parts[p].packed, parts[p].N, K), parts[p].bias, parts[p].y + m0 * parts[p].N, (int)parts[p].N};
+    a.nparts = nparts;
+    a.x = xg;
+    a.M = rows;
+    a.nsb = nsb;
     if (workspace && rows >= 3) {
       // several rows: quantize once for all workgroups; the GEMV then copies the image instead of quantizing
       const int MT = rows <= 4 ? 4 : 8;
@@ -570,4 +686,11 @@ MLLM_API int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, in
     if (rc) return rc;
   }
   return 0;
+}
+
+MLLM_API int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y, int64_t M,
+                                int64_t N, int64_t K, void* workspace, void* stream) {
+  if (!y) return MLLM_HIP_E_BADARG;
+  mllm_hip_gemv_part part{packed, bias, y, N};
+  return mllm_hip_linear_kq_multi(wtype, 1, &part, x, x_dtype, M, K, workspace, stream);
 }

@@ -539,6 +539,22 @@ def linear_kq(w, x, bias=None, out=None, workspace=None):
     return y
 
 
+def linear_kq_multi(ws, x, biases=None, outs=None, workspace=None):
+    """Sibling projections (same x, same K) in one launch; ws: list of PackedKWeight."""
+    assert 1 <= len(ws) <= 4 and x.is_cuda and x.is_contiguous() and x.dim() == 2
+    M, K = x.shape
+    if outs is None:
+        outs = [torch.empty((M, w.N), dtype=torch.float32, device="cuda") for w in ws]
+    parts = (_lib.GemvPart * len(ws))()
+    for i, w in enumerate(ws):
+        assert w.K == K and w.wtype == ws[0].wtype
+        b = biases[i] if biases is not None else None
+        parts[i] = _lib.GemvPart(w.ptr, b.data_ptr() if b is not None else None, outs[i].data_ptr(), w.N)
+    _lib.check(_lib.lib().mllm_hip_linear_kq_multi(ws[0].wtype, len(ws), parts, x.data_ptr(), _xdtype(x), M, K, _p(workspace), _stream()),
+               "mllm_hip_linear_kq_multi")
+    return outs
+
+
 def quantize_q8_K(x):
     """x [M, K] -> (codes int8 [M, K], d fp32 [M, K/256], sums of 16 int16 [M, K/16])"""
     assert x.is_cuda and x.is_contiguous() and x.dim() == 2

@@ -79,6 +79,25 @@ def test_linear_kq(wtype, M, N, K):
 
 
 @pytest.mark.parametrize("wtype", [2, 3])
+@pytest.mark.parametrize("M", [1, 4, 8, 13])
+def test_linear_kq_multi_equals_single(wtype, M):
+    """sibling projections in one launch: per part the bits of the single launch"""
+    rng = synth.rng_for(7, 300 + wtype * 10 + M)
+    K = 1280
+    Ns = [96, 33, 200, 8]
+    Ws = [synth.make_weight(rng, wtype, n, K) for n in Ns]
+    ws = [ql.PackedKWeight(wtype, torch.from_numpy(W)) for W in Ws]
+    biases = [to_dev(rng.standard_normal(n).astype(np.float32)) if i % 2 == 0 else None for i, n in enumerate(Ns)]
+    x = to_dev(synth.make_x_fp32(rng, M, K))
+    announce("kq multi", wtype, M)
+    wsp = ql.kq_workspace(M, K)
+    for nparts in (2, 4):
+        outs = ql.linear_kq_multi(ws[:nparts], x, biases[:nparts], workspace=wsp if M % 2 else None)
+        for w, b, o in zip(ws, biases, outs):
+            assert torch.equal(o, ql.linear_kq(w, x, b))
+
+
+@pytest.mark.parametrize("wtype", [2, 3])
 def test_linear_kq_exact_cases(wtype):
     """unit scales and integer activations that quantize to themselves: every product is an integer below 2^24, so the
     result must equal the integer matrix product exactly"""
