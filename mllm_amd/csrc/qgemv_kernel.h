@@ -352,9 +352,13 @@ __global__ __launch_bounds__(MT <= 2 ? 1024 : 512) void gemv_q_kernel(GemvArgs a
 }
 
 // ---- launchers ---------------------------------------------------------------------------------------------------
-template <int WT, int XT, int MT, int G, int R>
+// U3: three block columns in flight instead of four.  Rows of up to 96 blocks (K = 2560: 80) are covered by one trip either
+// way, and with three the kernel fits five waves per SIMD (81 registers instead of 97): 1280 resident workgroups, so the
+// 1216 workgroups of the gate + up launch run in one round instead of 1024 + 192.
+template <int WT, int XT, int MT, int G, int R, bool U3 = false>
 static int launch_gemv_u(const GemvArgs& a_in, int NW, hipStream_t st) {
-  constexpr int U = ((R >= 4) ? 1 : (R == 2 ? 2 : 4)) * (WT == MLLM_HIP_Q4_0 ? 2 : 1);
+  constexpr int U0 = ((R >= 4) ? 1 : (R == 2 ? 2 : 4)) * (WT == MLLM_HIP_Q4_0 ? 2 : 1);
+  constexpr int U = (U3 && U0 == 4) ? 3 : U0;
   constexpr int ROWS_W = (64 / G) * R;
   if (MT > 2 && NW > 8) NW = 8;  // see the register budget note at the kernel
   const int rows_per_wg = NW * ROWS_W;
@@ -390,6 +394,9 @@ static int launch_gemv_m(const GemvArgs& a, GemvShape s, hipStream_t st) {
 #define CASE(G_)                                                                     \
   if (s.G == G_ && s.R == RL) return launch_gemv_u<WT, XT, MT, G_, RL>(a, s.NW, st); \
   if (s.G == G_ && s.R == RH) return launch_gemv_u<WT, XT, MT, G_, RH>(a, s.NW, st);
+  if constexpr (WT == MLLM_HIP_Q4_0 && MT <= 2 && RH == 2) {
+    if (s.G == 32 && s.R == 2 && a.nb <= 96) return launch_gemv_u<WT, XT, MT, 32, 2, true>(a, s.NW, st);
+  }
   CASE(8) CASE(16) CASE(32) CASE(64)
 #undef CASE
   return MLLM_HIP_E_BADARG;
