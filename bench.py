@@ -436,6 +436,24 @@ def main():
             floor[str(n)] = {"us": ev / (5 * 40) * 1e6, "GBps": n / (ev / (5 * 40)) / 1e9}
         del big
         extra["read_only_floor"] = floor
+        # the same GEMV kernel on a launch large enough to leave the fixed cost behind: gate + up of a Qwen3-32B-shaped layer
+        # (2 x 25600 x 5120, 147 MB of Q4_0 blocks), eight distinct copies
+        bigw = [[ql.PackedQWeight.synthetic(ql.Q4_0, 25600, 5120, gen) for _ in range(2)] for _ in range(8)]
+        xb = torch.randn((1, 5120), device="cuda", generator=gen).to(torch.bfloat16)
+        yb = [torch.empty((1, 25600), dtype=torch.float32, device="cuda") for _ in range(2)]
+        _, ev = timed(graphed(lambda: [ql.linear_q_gemv_multi(ws, xb, None, ql.SCALE_X86_REF, yb) for ws in bigw]), 5, 2)
+        per = ev / (5 * 8)
+        nbig = 2 * synth.gemv_algorithmic_bytes(ql.Q4_0, 1, 25600, 5120, 2) - 5120 * 2
+        # ... and with the activations handed over as the quantized image a producer kernel (RMSNorm) writes: no workgroup
+        # quantizes (with 3200 workgroups the repeated quantization is what separates the two figures)
+        _, imgb = ql.rmsnorm(xb.float(), torch.ones(5120, device="cuda"), 1e-6, want_image=True)
+        _, ev2 = timed(graphed(lambda: [ql.linear_q_gemv_fused(ws, imgb, M=1, image=True, outs=yb) for ws in bigw]), 5, 2)
+        per2 = ev2 / (5 * 8)
+        extra["large_launch_gate_up_25600x5120"] = {"us": per * 1e6, "GBps": nbig / per / 1e9, "bytes": nbig,
+                                                    "frac_of_hbm_peak": nbig / per / 1e9 / HBM_PEAK_GBS,
+                                                    "from_quantized_image": {"us": per2 * 1e6, "GBps": nbig / per2 / 1e9,
+                                                                             "frac_of_hbm_peak": nbig / per2 / 1e9 / HBM_PEAK_GBS}}
+        del bigw
         extra["prefill_and_moe"] = side_workloads(torch, ql, synth, gen)
 
     cpu = None
