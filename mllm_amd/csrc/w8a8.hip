@@ -44,7 +44,9 @@ __device__ __forceinline__ int quant1(float x, float scale) {
   return (int)r;
 }
 
-template <int XT>
+// NI > 0: the row (K <= NI * 2048, K % 8 == 0) stays in registers between the maximum and the rounding, eight elements per
+// lane and item; NI == 0: any K, the row is read twice (the second time from cache).
+template <int XT, int NI>
 __global__ __launch_bounds__(256) void per_token_quant_kernel(const void* __restrict__ x, int8_t* __restrict__ q,
                                                               float* __restrict__ scale, int K) {
   __shared__ float s_max[4];
@@ -53,7 +55,16 @@ __global__ __launch_bounds__(256) void per_token_quant_kernel(const void* __rest
   const bool vec = (K % 8) == 0;
   const int64_t base = row * K;
   float amax = 0.f;
-  if (vec) {
+  float held[NI > 0 ? NI : 1][8];
+  if (NI > 0) {
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+      const int k = (tid + 256 * i) * 8;
+      load_x8v<XT>(x, base + (k < K ? k : K - 8), held[i]);  // clamped: lanes past the row re-read its tail and are not stored
+#pragma unroll
+      for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(held[i][e]));
+    }
+  } else if (vec) {
     for (int k = tid * 8; k < K; k += 256 * 8) {
       float v[8];
       load_x8v<XT>(x, base + k, v);
@@ -76,7 +87,16 @@ __global__ __launch_bounds__(256) void per_token_quant_kernel(const void* __rest
   amax = fmaxf(amax, 1e-10f);
   const float sc = amax / 127.0f;
   if (tid == 0) scale[row] = sc;
-  if (vec) {
+  if (NI > 0) {
+#pragma unroll
+    for (int i = 0; i < NI; i++) {
+      const int k = (tid + 256 * i) * 8;
+      uint32_t pk[2] = {0, 0};
+#pragma unroll
+      for (int e = 0; e < 8; e++) pk[e >> 2] |= ((uint32_t)quant1(held[i][e], sc) & 0xffu) << (8 * (e & 3));
+      if (k < K) *reinterpret_cast<uint2*>(q + base + k) = make_uint2(pk[0], pk[1]);
+    }
+  } else if (vec) {
     for (int k = tid * 8; k < K; k += 256 * 8) {
       float v[8];
       load_x8v<XT>(x, base + k, v);
@@ -550,10 +570,21 @@ MLLM_API int mllm_hip_per_token_quant_int8(const void* x, int x_dtype, int8_t* q
     return MLLM_HIP_E_BADARG;
   if (M > INT32_MAX || K > INT32_MAX) return MLLM_HIP_E_SHAPE;
   if (K % 8 == 0 && (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(q) % 8)) return MLLM_HIP_E_ALIGN;
-  if (x_dtype == MLLM_HIP_F32)
-    hipLaunchKernelGGL(per_token_quant_kernel<MLLM_HIP_F32>, dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, x, q, scale, (int)K);
-  else
-    hipLaunchKernelGGL(per_token_quant_kernel<MLLM_HIP_BF16>, dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, x, q, scale, (int)K);
+  const int ni = (K % 8 == 0 && K >= 8 && K <= 4 * 2048) ? (K <= 2048 ? 1 : (K <= 4096 ? 2 : 4)) : 0;
+#define PTQ(XT_, NI_) \
+  hipLaunchKernelGGL((per_token_quant_kernel<XT_, NI_>), dim3((unsigned)M), dim3(256), 0, (hipStream_t)stream, x, q, scale, (int)K)
+#define PTQ_T(XT_)          \
+  if (ni == 1) PTQ(XT_, 1); \
+  else if (ni == 2) PTQ(XT_, 2); \
+  else if (ni == 4) PTQ(XT_, 4); \
+  else PTQ(XT_, 0)
+  if (x_dtype == MLLM_HIP_F32) {
+    PTQ_T(MLLM_HIP_F32);
+  } else {
+    PTQ_T(MLLM_HIP_BF16);
+  }
+#undef PTQ_T
+#undef PTQ
   return (int)hipGetLastError();
 }
 
