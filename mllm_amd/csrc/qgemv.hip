@@ -234,9 +234,15 @@ static GemvShape pick_shape(int MT, int64_t N, int nb) {
   } else {
     s.G = 8;
   }
-  // several activation rows: the quantization of x (done by every workgroup) grows with M, so spread it over many waves;
-  // measured best over the projection shapes: 16 waves for rows up to 255 blocks, 8 for longer rows
-  if (MT >= 4) s.NW = nb >= 256 ? 8 : (nb * MT >= 256 ? 16 : 8);
+  // four or eight activation rows (kernels built for at most eight waves), measured over the projection shapes with and
+  // without a pre-quantized image: eight waves, whole-wave rows from 128 blocks on.  (16 lanes per row would gain 10 % on
+  // the gate + up launch and lose as much on q + k + v; the shape is kept a function of the row length alone, so that a
+  // projection gives the same bits whether it is launched alone or with its siblings.)
+  if (MT >= 4) {
+    s.R = 2;
+    s.NW = 8;
+    if (nb >= 128) s.G = 64;
+  }
   (void)N;
   if (g_tune_G) s.G = g_tune_G;
   if (g_tune_R) s.R = g_tune_R;
@@ -356,16 +362,18 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
   GemvShape s = pick_shape(MT, nmax, a.nb);
   hipStream_t st = (hipStream_t)stream;
   if (x_dtype == MLLM_HIP_Q8_IMAGE) {
-    if (!g_tune_NW) s.NW = a.nb >= 256 ? 8 : 4;
+    if (!g_tune_NW && MT <= 2) s.NW = a.nb >= 256 ? 8 : 4;
     return wtype == MLLM_HIP_Q4_0 ? launch_gemv_q4_preq(a, MT, s, st) : launch_gemv_q8_preq(a, MT, s, st);
   }
-  if (workspace && M >= 3) {
+  // several rows and a large launch (measured: from about 600 000 block-rows, i.e. gate + up and down of the 4B shapes):
+  // quantizing x in every workgroup costs more than one more small launch
+  if (workspace && M >= 3 && nmax * a.nb >= 600000) {
     // several rows: quantize once for all workgroups, then the GEMV copies the quantized image instead of quantizing
     const int mnb = MT * a.nb;
     hipLaunchKernelGGL(quant_image_kernel, dim3((unsigned)((mnb + 127) / 128)), dim3(128), 0, st, x, x_dtype,
                        reinterpret_cast<unsigned char*>(workspace), M, MT, a.nb, a.x86_scale);
     a.x = workspace;
-    if (!g_tune_NW) s.NW = a.nb >= 256 ? 8 : 4;  // no quantization work to share: smaller workgroups start and finish sooner
+
     return wtype == MLLM_HIP_Q4_0 ? launch_gemv_q4_preq(a, MT, s, st) : launch_gemv_q8_preq(a, MT, s, st);
   }
   if (wtype == MLLM_HIP_Q4_0)
