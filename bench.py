@@ -134,6 +134,29 @@ def side_workloads(torch, ql, synth, gen):
     wsm = torch.empty(_lib_ws(ql, "moe", T, H, I, E, k), dtype=torch.uint8, device="cuda")
     ym = torch.empty((T, H), dtype=torch.float32, device="cuda")
     tm = ev_time(lambda: ql.moe_ffn_q(gate, up, down, x, ids, tw, workspace=wsm, out=ym), 10)
+    # the same layer at decode: 1 and 8 tokens, every (token, expert) pair a GEMV row, two launches; a graph of 16 calls
+    # over rotating routings (eager launches of this size would measure the host)
+    dec = {}
+    for Td in (1, 8):
+        rngd = synth.rng_for(4, 100 + Td)
+        routes = [synth.make_moe_routing(rngd, Td, E, k) for _ in range(16)]
+        idl = [torch.from_numpy(r[0]).cuda() for r in routes]
+        twl = [torch.from_numpy(r[1]).cuda() for r in routes]
+        xd = torch.randn((Td, H), device="cuda", generator=gen).to(torch.bfloat16)
+        yd = torch.empty((Td, H), dtype=torch.float32, device="cuda")
+
+        def dstep():
+            for i_, t_ in zip(idl, twl):
+                ql.moe_ffn_q(gate, up, down, xd, i_, t_, workspace=wsm, out=yd)
+        dstep()
+        torch.cuda.synchronize()
+        gd = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gd):
+            dstep()
+        td = ev_time(gd.replay, 10) / 16
+        act = float(np.mean([len(np.unique(r[0])) for r in routes]))
+        wb = act * (2 * I * (H // 32) * 18 + H * (I // 32) * 18)
+        dec["tokens_%d" % Td] = {"us": td * 1e6, "active_experts_avg": act, "weight_GBps": wb / td / 1e9, "frac_of_hbm_peak": wb / td / 8e12}
     del gate, up, down
     from mllm_amd import _lib
     L = _lib.lib()
@@ -148,7 +171,8 @@ def side_workloads(torch, ql, synth, gen):
     out["moe_ffn_512tok_128e_top8_q4_0"] = {"us": tm2 * 1e6, "active_experts": active, "weight_GBps": wbytes / tm2 / 1e9,
                                             "frac_of_hbm_peak": wbytes / tm2 / 8e12, "TFLOPS": flops / tm2 / 1e12,
                                             "path": "matrix cores, fp16 operands with folded block scales (mllm_hip_moe_ffn_q_gemm)",
-                                            "block_dot_path": {"us": tm * 1e6, "weight_GBps": wbytes / tm / 1e9}}
+                                            "block_dot_path": {"us": tm * 1e6, "weight_GBps": wbytes / tm / 1e9},
+                                            "decode": dec}
     del gate2, up2, down2
     # Q4_0 Linear at prefill size (the reference's tinyBLAS gemm branch): gate_proj of the decode layer, 2048 rows
     M, N, K = 2048, 9728, 2560

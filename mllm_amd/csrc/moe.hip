@@ -933,6 +933,15 @@ MLLM_API int mllm_hip_linear_q(int wtype, const void* packed, const void* x, int
   return launch_tiles<0>(wtype, a, (unsigned)((M + TOK_TILE - 1) / TOK_TILE), st);
 }
 
+// decode path (moe_decode.hip): up to eight tokens as GEMVs, two launches
+namespace mllmhip {
+size_t moe_decode_workspace_bytes(int64_t T, int64_t I, int k);
+bool moe_decode_applies(int64_t T, int64_t H, int64_t I, int k);
+int launch_moe_decode(int wtype, const void* gate, const void* up, const void* down, const void* x, int x_dtype, const int32_t* ids,
+                      const float* w, float* y, int64_t T, int64_t H, int64_t I, int E, int k, int x86, void* workspace,
+                      hipStream_t st);
+}  // namespace mllmhip
+
 MLLM_API size_t mllm_hip_moe_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k) {
   if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || k <= 0 || H % QK || I % QK) return 0;
   Carver c(nullptr);
@@ -942,7 +951,8 @@ MLLM_API size_t mllm_hip_moe_workspace_bytes(int64_t T, int64_t H, int64_t I, in
   c.take<float>((size_t)T * k * (I / QK));
   c.take<float>((size_t)T * k * H);
   carve_route(c, E, T * k);
-  return c.used;
+  const size_t decode = moe_decode_applies(T, H, I, k) ? moe_decode_workspace_bytes(T, I, k) : 0;
+  return c.used > decode ? c.used : decode;
 }
 
 MLLM_API int mllm_hip_moe_route(const int32_t* topk_ids, int64_t T, int E, int k, int32_t* counts, int32_t* offsets,
@@ -973,6 +983,9 @@ MLLM_API int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* 
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
   hipStream_t st = (hipStream_t)stream;
   const int x86 = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
+  // a handful of tokens: every (token, expert) pair is one GEMV row; two launches instead of five
+  if (moe_decode_applies(T, H, I, k))
+    return launch_moe_decode(wtype, gate_packed, up_packed, down_packed, x, x_dtype, topk_ids, topk_w, y, T, H, I, E, k, x86, workspace, st);
   Carver c(workspace);
   int8_t* xq = c.take<int8_t>((size_t)T * H);
   float* xd = c.take<float>((size_t)T * (H / QK));

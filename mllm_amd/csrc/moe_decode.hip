@@ -1,0 +1,244 @@
+// MoE expert FFN for a handful of tokens (decode): two launches, no routing pass.
+//
+//   reference: Qwen3MoE::moeInfer + Qwen3MoeMLP::forward, mllm/models/qwen3_moe/modeling_qwen3_moe_fa2.hpp:98-100,175-238 -- per
+//   active expert three small Linears (CPULinearOp -> quantize_row_q8_0 + block dots), SiLU and product in between, the
+//   weighted sum over the token's experts at the end.
+//
+// With up to eight tokens every (token, expert) pair is one activation row, so the path is a set of GEMVs and HBM-bound:
+// 8 experts x 3 matrices x 0.88 MB for one Qwen3-30B-A3B token.  The grouped-GEMM path spends five launches and 128-row
+// tiles on it.  Here:
+//   launch 1  one workgroup per (slot, 32 intermediate channels): quantizes the token's x (Q8_0, bit-exact), gate and up
+//             rows of the slot's expert as PAIRED rows of a lane group, h = silu(g) * u, and the Q8_0 image of those 32
+//             values of h (exactly one block) for launch 2;
+//   launch 2  one workgroup per (token, 16 output rows): copies the images of the token's k slots into LDS and walks the
+//             experts in slot order, acc += w_j * (W_down,e_j . h_j), the next expert's weights requested while the
+//             current one is multiplied.  The sum runs in the reference's order (slot j ascending), no atomics.
+// Arithmetic as in the GEMV kernel: exact int32 block dots, fp32 fma with dW * dX.
+#include "qgemv_kernel.h"
+
+namespace mllmhip {
+
+__device__ __forceinline__ float silu_vec(float x) { return x * (1.0f / (1.0f + exp_poly(-x))); }
+
+struct MoeDecodeArgs {
+  const char* gate;  // E packed [I][H] matrices back to back
+  const char* up;
+  const char* down;  // E packed [H][I]
+  size_t gu_stride, d_stride;
+  const void* x;     // [T][H]
+  const int32_t* ids;  // [T][k]
+  const float* w;      // [T][k]
+  unsigned char* img;  // per slot: Q8_0 image of h (one activation row of I elements), img_stride bytes apart
+  float* y;            // [T][H]
+  int img_stride;
+  int T, H, I, E, k, x86;
+};
+
+// ---- launch 1: gate / up / SiLU * up / re-quantization ----------------------------------------------------------------
+// 512 threads: wave w, lane group grp (16 lanes) -> intermediate channel n = n0 + 4 w + grp; row 0 of the group is the gate
+// row, row 1 the up row; lanes stride over the block columns.
+template <int WT, int XT>
+__global__ __launch_bounds__(512) void moe_decode_gateup_kernel(MoeDecodeArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int nb = a.H / QK, nbp = (int)scale_row_stride(a.H);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slot = blockIdx.y;
+  const int tok = slot / a.k;
+  const int e = a.ids[slot];
+  const int n0 = blockIdx.x * 32;
+  const QImage out{a.img + (size_t)slot * a.img_stride, 1, a.I / QK, a.x86};
+  float* s_h = reinterpret_cast<float*>(smem + align_up((size_t)nb * 40, 16));
+  if (e < 0 || e >= a.E) {  // uniform: this slot contributes nothing; its image block reads as zeros
+    if (tid < 4) {
+      const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      quad_quantize_to_image(z, out, 0, n0 / QK, tid, true);
+    }
+    return;
+  }
+  // activations of the token first, weights behind them (requests return in order)
+  const int nitems = nb * 4;
+  XRaw<XT> raw;
+  load_x8<XT>(a.x, ((int64_t)tok * nb * 4 + min(tid, nitems - 1)) * 8, raw);
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+
+  const int grp = lane >> 4, c0 = lane & 15;
+  const int n = n0 + 4 * wave + grp;
+  const PackedView wv[2] = {packed_view(WT, a.gate + (size_t)e * a.gu_stride, a.I, a.H), packed_view(WT, a.up + (size_t)e * a.gu_stride, a.I, a.H)};
+  constexpr int U = 4;  // block columns per lane and trip: 64 columns per trip
+  u32x4 w0[U][2], w1[WT == MLLM_HIP_Q8_0 ? U : 1][2];
+  uint16_t dw[U][2];
+  auto load_trip = [&](int t0) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int col = min(t0 + 16 * u + c0, nb - 1);  // clamped: columns past the row are loaded twice and not used
+#pragma unroll
+      for (int r = 0; r < 2; r++) {
+        const size_t blk = (size_t)n * nb + col;
+        w0[u][r] = wv[r].q0[blk];
+        if (WT == MLLM_HIP_Q8_0) w1[WT == MLLM_HIP_Q8_0 ? u : 0][r] = wv[r].q1[blk];
+        dw[u][r] = wv[r].d[(size_t)n * nbp + col];
+      }
+    }
+  };
+  load_trip(0);
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+
+  // x -> Q8_0 in LDS, laid out like the GEMV kernel's image (one activation row)
+  const QImage xi{smem, 1, nb, a.x86};
+  {
+    float v[8];
+    x8_to_f32<XT>(raw, v);
+    if (tid < nitems) quad_quantize_to_image(v, xi, 0, tid >> 2, tid & 3, true);  // whole quads: nitems is a multiple of 4
+    for (int it = tid + 512; it < nitems; it += 512) {
+      XRaw<XT> rw;
+      load_x8<XT>(a.x, ((int64_t)tok * nb * 4 + it) * 8, rw);
+      x8_to_f32<XT>(rw, v);
+      quad_quantize_to_image(v, xi, 0, it >> 2, it & 3, true);
+    }
+  }
+  __syncthreads();
+  const u32x4* s_lo = reinterpret_cast<const u32x4*>(smem);
+  const u32x4* s_hi = s_lo + nb;
+  const float* s_d = reinterpret_cast<const float*>(s_hi + nb);
+  const int* s_n8 = reinterpret_cast<const int*>(s_d + nb);
+
+  float acc[2] = {0.f, 0.f};
+  for (int t0 = 0; t0 < nb; t0 += 16 * U) {
+    if (t0) load_trip(t0);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int col = t0 + 16 * u + c0;
+      if (col < nb) {
+        const u32x4 xlo = s_lo[col], xhi = s_hi[col];
+        const float dx = s_d[col];
+        const int n8 = s_n8[col];
+#pragma unroll
+        for (int r = 0; r < 2; r++) {
+          const int isum = block_dot<WT>(w0[u][r], w1[WT == MLLM_HIP_Q8_0 ? u : 0][r], xlo, xhi, n8);
+          acc[r] = fmaf(f16bits_to_f32(dw[u][r]) * dx, (float)isum, acc[r]);
+        }
+      }
+    }
+  }
+  const float g = group_sum<16>(acc[0]), u = group_sum<16>(acc[1]);
+  if (c0 == 0) s_h[4 * wave + grp] = silu_vec(g) * u;
+  __syncthreads();
+  if (tid < 4) {  // one quad: the 32 values are exactly one Q8_0 block of h
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = s_h[8 * tid + i];
+    quad_quantize_to_image(v, out, 0, n0 / QK, tid, true);
+  }
+}
+
+// ---- launch 2: down projection and the weighted sum over the token's experts -------------------------------------------
+// DNW waves per workgroup: wave w, lane group grp (8 lanes) -> output row n = n0 + 8 w + grp; lanes stride over the block
+// columns (up to 32 of them: I <= 1024).
+constexpr int DNW = 2;  // measured: one wave per workgroup is 6 % slower at one and at eight tokens
+template <int WT>
+__global__ __launch_bounds__(DNW * 64) void moe_decode_down_kernel(MoeDecodeArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int nb = a.I / QK, nbp = (int)scale_row_stride(a.I);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tok = blockIdx.y;
+  const int grp = lane >> 3, c0 = lane & 7;
+  const int n = blockIdx.x * (8 * DNW) + 8 * wave + grp;
+  constexpr int U = 4;
+  struct Chunk {
+    u32x4 w0[U];
+    u32x4 w1[WT == MLLM_HIP_Q8_0 ? U : 1];
+    uint16_t dw[U];
+  };
+  auto load_expert = [&](int j, Chunk& c) {
+    int e = a.ids[tok * a.k + min(j, a.k - 1)];
+    e = min(max(e, 0), a.E - 1);  // an invalid slot loads some expert's rows and is skipped at the sum
+    const PackedView v = packed_view(WT, a.down + (size_t)e * a.d_stride, a.H, a.I);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int col = min(8 * u + c0, nb - 1);
+      const size_t blk = (size_t)n * nb + col;
+      c.w0[u] = v.q0[blk];
+      if (WT == MLLM_HIP_Q8_0) c.w1[WT == MLLM_HIP_Q8_0 ? u : 0] = v.q1[blk];
+      c.dw[u] = v.d[(size_t)n * nbp + col];
+    }
+  };
+  Chunk cur;
+  load_expert(0, cur);
+  // the images of this token's k slots are contiguous
+  const int n16 = a.k * a.img_stride / 16;
+  const u32x4* src = reinterpret_cast<const u32x4*>(a.img + (size_t)tok * a.k * a.img_stride);
+  for (int c = tid; c < n16; c += DNW * 64) reinterpret_cast<u32x4*>(smem)[c] = src[c];
+  __syncthreads();
+
+  float total = 0.f;
+  for (int j = 0; j < a.k; j++) {
+    Chunk nxt;
+    if (j + 1 < a.k) load_expert(j + 1, nxt);  // uniform
+    const unsigned char* im = smem + (size_t)j * a.img_stride;
+    const u32x4* s_lo = reinterpret_cast<const u32x4*>(im);
+    const u32x4* s_hi = s_lo + nb;
+    const float* s_d = reinterpret_cast<const float*>(s_hi + nb);
+    const int* s_n8 = reinterpret_cast<const int*>(s_d + nb);
+    float acc = 0.f;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int col = 8 * u + c0;
+      if (col < nb) {
+        const int isum = block_dot<WT>(cur.w0[u], cur.w1[WT == MLLM_HIP_Q8_0 ? u : 0], s_lo[col], s_hi[col], s_n8[col]);
+        acc = fmaf(f16bits_to_f32(cur.dw[u]) * s_d[col], (float)isum, acc);
+      }
+    }
+    const float v = group_sum<8>(acc);
+    const int e = a.ids[tok * a.k + j];
+    if (e >= 0 && e < a.E) total = total + v * a.w[tok * a.k + j];
+    if (j + 1 < a.k) cur = nxt;
+  }
+  if (c0 == 0) a.y[(size_t)tok * a.H + n] = total;
+}
+
+// image bytes of one slot, padded to 16
+__host__ __device__ inline int moe_decode_img_stride(int64_t I) { return (int)align_up((size_t)(I / QK) * 40, 16); }
+
+size_t moe_decode_workspace_bytes(int64_t T, int64_t I, int k) { return (size_t)T * k * moe_decode_img_stride(I); }
+
+bool moe_decode_applies(int64_t T, int64_t H, int64_t I, int k) {
+  return T <= 8 && I % 32 == 0 && I / QK <= 32 && H % 32 == 0 && k <= 64 && H / QK * 40 + 256 <= 64 * 1024 &&
+         (int64_t)k * moe_decode_img_stride(I) <= 64 * 1024;
+}
+
+int launch_moe_decode(int wtype, const void* gate, const void* up, const void* down, const void* x, int x_dtype, const int32_t* ids,
+                      const float* w, float* y, int64_t T, int64_t H, int64_t I, int E, int k, int x86, void* workspace,
+                      hipStream_t st) {
+  MoeDecodeArgs a{};
+  a.gate = reinterpret_cast<const char*>(gate);
+  a.up = reinterpret_cast<const char*>(up);
+  a.down = reinterpret_cast<const char*>(down);
+  a.gu_stride = packed_bytes(wtype, I, H);
+  a.d_stride = packed_bytes(wtype, H, I);
+  a.x = x;
+  a.ids = ids;
+  a.w = w;
+  a.img = reinterpret_cast<unsigned char*>(workspace);
+  a.y = y;
+  a.img_stride = moe_decode_img_stride(I);
+  a.T = (int)T; a.H = (int)H; a.I = (int)I; a.E = E; a.k = k; a.x86 = x86;
+  const size_t lds1 = align_up((size_t)(H / QK) * 40, 16) + 32 * sizeof(float);
+  const dim3 g1((unsigned)(I / 32), (unsigned)(T * k));
+#define GU(WT_, XT_) hipLaunchKernelGGL((moe_decode_gateup_kernel<WT_, XT_>), g1, dim3(512), lds1, st, a)
+  if (wtype == MLLM_HIP_Q4_0) {
+    if (x_dtype == MLLM_HIP_F32) GU(MLLM_HIP_Q4_0, MLLM_HIP_F32); else GU(MLLM_HIP_Q4_0, MLLM_HIP_BF16);
+  } else {
+    if (x_dtype == MLLM_HIP_F32) GU(MLLM_HIP_Q8_0, MLLM_HIP_F32); else GU(MLLM_HIP_Q8_0, MLLM_HIP_BF16);
+  }
+#undef GU
+  HIP_RET(hipGetLastError());
+  const size_t lds2 = (size_t)k * a.img_stride;
+  const dim3 g2((unsigned)(H / (8 * DNW)), (unsigned)T);
+  if (wtype == MLLM_HIP_Q4_0) hipLaunchKernelGGL((moe_decode_down_kernel<MLLM_HIP_Q4_0>), g2, dim3(DNW * 64), lds2, st, a);
+  else hipLaunchKernelGGL((moe_decode_down_kernel<MLLM_HIP_Q8_0>), g2, dim3(DNW * 64), lds2, st, a);
+  return (int)hipGetLastError();
+}
+
+}  // namespace mllmhip

@@ -112,6 +112,69 @@ __device__ __forceinline__ uint16_t quantize_block_q8_0(const float (&v)[32], ui
   return f32_to_f16bits(d);
 }
 
+// The Q8_0 image of activation rows that the decode GEMV copies into LDS: for MT rows of nb blocks, 16-byte planes of
+// elements 0..15 and 16..31 of every block, then the fp32 effective scales, then -8 * sum(codes).
+struct QImage {
+  unsigned char* base;  // null: no image wanted
+  int MT, nb, x86_scale;
+};
+// Four neighbouring lanes (a quad) hold the four eighths of one 32-element block: lane j of the quad has elements
+// 8j..8j+7.  Same arithmetic as quantize_row_q8_0 (quantize_q8.cpp:106-190), same image as quant_image_kernel writes.
+__device__ __forceinline__ void quad_quantize_to_image(const float (&v)[8], const QImage& q, int m, int blk, int j, bool write) {
+  float amax = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[e]));
+  amax = fmaxf(amax, dpp_f<0xB1>(amax));
+  amax = fmaxf(amax, dpp_f<0x4E>(amax));
+  const float d = amax / 127.f;
+  const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
+  uint32_t pk[2];
+#pragma unroll
+  for (int w = 0; w < 2; w++) {
+    uint32_t p = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      int qi = (int)rintf(v[4 * w + e] * idv);
+      qi = min(127, max(-128, qi));
+      p |= ((uint32_t)qi & 0xffu) << (8 * e);
+    }
+    pk[w] = p;
+  }
+  int sum = __builtin_amdgcn_sdot4((int)pk[0], 0x01010101, 0, false);
+  sum = __builtin_amdgcn_sdot4((int)pk[1], 0x01010101, sum, false);
+  sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xf, 0xf, true);
+  sum += __builtin_amdgcn_update_dpp(0, sum, 0x4E, 0xf, 0xf, true);
+  if (!write) return;
+  const int mnb = q.MT * q.nb;
+  const int id = m * q.nb + blk;
+  u32x4* lo = reinterpret_cast<u32x4*>(q.base);
+  u32x4* hi = lo + mnb;
+  float* sd = reinterpret_cast<float*>(hi + mnb);
+  int* sn = reinterpret_cast<int*>(sd + mnb);
+  u32x2* dst = reinterpret_cast<u32x2*>((j < 2 ? lo : hi) + id) + (j & 1);
+  *dst = u32x2{pk[0], pk[1]};
+  if (j == 0) {
+    uint16_t bits = f32_to_f16bits(d);
+    if (q.x86_scale) bits = x86_scale_bits(bits);
+    sd[id] = f16bits_to_f32(bits);
+    sn[id] = -8 * sum;
+  }
+}
+// rows of the image beyond the real ones read as zero blocks
+__device__ __forceinline__ void image_zero_row(const QImage& q, int m, int tid, int nthreads) {
+  const int mnb = q.MT * q.nb;
+  u32x4* lo = reinterpret_cast<u32x4*>(q.base);
+  u32x4* hi = lo + mnb;
+  float* sd = reinterpret_cast<float*>(hi + mnb);
+  int* sn = reinterpret_cast<int*>(sd + mnb);
+  for (int b = tid; b < q.nb; b += nthreads) {
+    lo[m * q.nb + b] = u32x4{0, 0, 0, 0};
+    hi[m * q.nb + b] = u32x4{0, 0, 0, 0};
+    sd[m * q.nb + b] = 0.f;
+    sn[m * q.nb + b] = 0;
+  }
+}
+
 // One 32-element activation block, raw: fp32 input = 8 x 16 B, bf16 input = 4 x 16 B.  Loading and converting are
 // separate steps so that a caller can issue other loads in between.
 template <int XT>

@@ -145,6 +145,35 @@ def test_moe_small(T, H, I, E, k, wtype):
     assert np.array_equal(y2, y[perm])
 
 
+@pytest.mark.parametrize("T,H,I,E,k,wtype", [(1, 2048, 768, 128, 8, 0), (8, 2048, 768, 128, 8, 0), (3, 256, 96, 8, 3, 1), (5, 2048, 768, 16, 8, 1),
+                                              (2, 64, 32, 4, 4, 0), (7, 128, 1024, 6, 2, 0), (8, 4096, 32, 5, 1, 0)])
+def test_moe_decode_path(T, H, I, E, k, wtype):
+    """up to eight tokens: every (token, expert) pair as a GEMV row, two launches (Qwen3-30B-A3B dimensions included);
+    fp32 block arithmetic as the CPU path, so close to the oracle; slots with an expert id outside [0, E) add nothing;
+    permuting tokens permutes outputs bit for bit; bf16 activations"""
+    rng = synth.rng_for(4, 5000 + T + H + I + E)
+    Wg, Wu, Wd, ids, w, g, u, d = _moe_case(rng, T, H, I, E, k, wtype)
+    x = synth.make_x_fp32(rng, T, H)
+    announce("moe decode", T, H, I, E, k, wtype)
+    y = ql.moe_ffn_q(g, u, d, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+    want = orc.moe_ffn(x, ids, w, Wg, Wu, Wd, wtype)
+    # fp32 summation-order noise (1e-7) in front of the Q8_0 re-quantization of h flips a code now and then: about 5e-5
+    assert rel_l2(y, want) < 2e-4, rel_l2(y, want)
+    perm = rng.permutation(T)
+    y2 = ql.moe_ffn_q(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
+    assert np.array_equal(y2, y[perm])
+    bad = ids.copy()
+    bad[0, 0] = E + 3
+    if k > 1:
+        bad[T - 1, k - 1] = -1
+    y3 = ql.moe_ffn_q(g, u, d, to_dev(x), to_dev(bad), to_dev(w)).cpu().numpy()
+    assert rel_l2(y3, orc.moe_ffn(x, bad, w, Wg, Wu, Wd, wtype)) < 2e-4
+    bits, xb = synth.make_x_bf16(rng, T, H)
+    from gpu_util import bf16_dev
+    y4 = ql.moe_ffn_q(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
+    assert rel_l2(y4, orc.moe_ffn(xb, ids, w, Wg, Wu, Wd, wtype)) < 2e-4
+
+
 @pytest.mark.parametrize("T,H,I,E,k,wtype", [(16, 64, 32, 4, 2, 0), (40, 256, 96, 8, 3, 0), (200, 128, 64, 3, 2, 1),
                                               (1, 64, 64, 4, 4, 0), (300, 192, 160, 2, 2, 0)])
 def test_moe_gemm_small(T, H, I, E, k, wtype):
