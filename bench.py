@@ -307,7 +307,8 @@ def main():
     def measure_layer_chain(pool, M, reps=5):
         """The dependent chain of one decoder layer around its Linears (attention core left out: o_proj reads a fixed
         buffer), fp32 residual stream, over all layers: the operators one by one (10 launches per layer) against the
-        folded form (RMSNorm and SiLU*up write the GEMV's quantized image, residual adds in the GEMV epilogue: 7)."""
+        folded form (RMSNorm and SiLU*up write the GEMV's quantized image, residual adds in the GEMV epilogue: 7), and with
+        gate / up / SiLU / product / image as one launch (6)."""
         x0 = torch.randn((M, 2560), device="cuda", generator=gen)
         attn = torch.randn((M, 4096), device="cuda", generator=gen)
         nw = [torch.ones(2560, device="cuda") for _ in range(2)]
@@ -352,8 +353,23 @@ def main():
                                                img[9728].data_ptr(), ql.SCALE_X86_REF, st), "silu_mul")
                 ql.linear_q_gemv_fused([l["down_proj"]], img[9728], M=M, image=True, residuals=[b["x1"]], outs=[b["x2"]])
                 x = b["x2"]
+
+        def mlp_one_launch():
+            x = x0
+            for l in pool:
+                st = torch.cuda.current_stream().cuda_stream
+                _lib.check(L.mllm_hip_rmsnorm(x.data_ptr(), 0, nw[0].data_ptr(), b["h"].data_ptr(), M, 2560, 1e-6, 0,
+                                              img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
+                ql.linear_q_gemv_fused([l["q_proj"], l["k_proj"], l["v_proj"]], img[2560], M=M, image=True, outs=[b["q"], b["k"], b["v"]])
+                ql.linear_q_gemv_fused([l["o_proj"]], attn, residuals=[x], outs=[b["x1"]])
+                _lib.check(L.mllm_hip_rmsnorm(b["x1"].data_ptr(), 0, nw[1].data_ptr(), b["h2"].data_ptr(), M, 2560, 1e-6, 0,
+                                              img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
+                _lib.check(L.mllm_hip_mlp_gate_up_q(l["gate_proj"].wtype, l["gate_proj"].ptr, l["up_proj"].ptr, img[2560].data_ptr(),
+                                                    ql.Q8_IMAGE, None, img[9728].data_ptr(), M, 9728, 2560, ql.SCALE_X86_REF, st), "mlp")
+                ql.linear_q_gemv_fused([l["down_proj"]], img[9728], M=M, image=True, residuals=[b["x1"]], outs=[b["x2"]])
+                x = b["x2"]
         res = {}
-        for name, fn, n in (("operators_one_by_one", plain, 10), ("folded", folded, 7)):
+        for name, fn, n in (("operators_one_by_one", plain, 10), ("folded", folded, 7), ("folded_mlp_one_launch", mlp_one_launch, 6)):
             _, ev = timed(graphed(fn), reps, 2)
             res[name] = {"us_per_layer": ev / (reps * len(pool)) * 1e6, "launches_per_layer": n}
         return res

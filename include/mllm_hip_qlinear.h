@@ -301,6 +301,18 @@ int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, int x_dtype
 int mllm_hip_kq_dequantize(int wtype, const void* packed, float* w, int64_t N, int64_t K, void* stream);
 int mllm_hip_quantize_q8_K(const void* x, int x_dtype, int8_t* codes, float* d, int16_t* bsums, int64_t M, int64_t K, void* stream);
 
+/* Decode MLP front half in ONE launch: h = silu(gate(x)) * up(x), M <= 8 rows, Q4_0 / Q8_0 weights [I][H].
+ *   replaces: Qwen3MLP::forward, mllm/models/qwen3/modeling_qwen3_fa2.hpp:85-92 (gate_proj, SiLU, up_proj, product: two
+ *             CPULinearOp::forward, CPUSiLUOp, CPUMulOp), fp32 tensors in between.
+ * x_kind as for mllm_hip_linear_q_gemv_fused (F32 / BF16 activations [M][H], or the Q8_0 image of M rows).  h (fp32
+ * [M][I], may be NULL) and/or h_image (may be NULL; the Q8_0 image of h for the down projection, size
+ * mllm_hip_gemv_workspace_bytes(M, I)) receive the result.  I % 32 == 0, H % 32 == 0.  SiLU follows mllm_hip_set_exp_mode.
+ * The gate and up values never reach memory; results agree with the separate calls to fp32 rounding of the row sums. */
+int mllm_hip_mlp_gate_up_q(int wtype, const void* gate_packed, const void* up_packed, const void* x, int x_kind, float* h,
+                           void* h_image, int M, int64_t I, int64_t H, int act_scale_mode, void* stream);
+/* Tuning override of that launch: block columns of a weight row a lane keeps in flight (2..5); 0 = heuristic. */
+int mllm_hip_mlp_set_tuning(int units_in_flight);
+
 /* ---------------------------------------------------------------------------------------------------------
  * The operators either side of a quantized Linear in a decoder layer.  dtype: MLLM_HIP_F32 or MLLM_HIP_BF16 (arithmetic
  * in fp32, results rounded to the tensor's type).  All pointers 16-byte aligned, element counts multiples of 8.

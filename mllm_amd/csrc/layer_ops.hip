@@ -390,6 +390,9 @@ __global__ __launch_bounds__(256) void moe_gate_kernel(GateArgs a) {
 using namespace mllmhip;
 
 static int g_exp_accurate = 0;
+namespace mllmhip {
+int exp_mode_accurate() { return g_exp_accurate; }
+}
 MLLM_API int mllm_hip_set_exp_mode(int accurate) {
   if (accurate != 0 && accurate != 1) return MLLM_HIP_E_BADARG;
   g_exp_accurate = accurate;

@@ -452,6 +452,23 @@ def silu_mul(gate, up, want_image=False, act_scale_mode=SCALE_X86_REF, out=None)
     return (y, img) if want_image else y
 
 
+def mlp_gate_up(wg, wu, x, M=None, image=False, want_h=True, want_image=False, act_scale_mode=SCALE_X86_REF):
+    """silu(x Wg^T) * (x Wu^T) for up to eight rows in one launch; `x` activations [M, H] or (image=True) their Q8_0 image.
+    Returns h (fp32 [M, I]) and/or the Q8_0 image of h for the down projection."""
+    assert wg.K == wu.K and wg.N == wu.N and wg.wtype == wu.wtype and x.is_cuda and x.is_contiguous()
+    if not image:
+        assert x.dim() == 2 and x.shape[1] == wg.K
+        M = x.shape[0]
+    assert M is not None and (want_h or want_image)
+    h = torch.empty((M, wg.N), dtype=torch.float32, device="cuda") if want_h else None
+    img = gemv_workspace(M, wg.N) if want_image else None
+    _lib.check(_lib.lib().mllm_hip_mlp_gate_up_q(wg.wtype, wg.ptr, wu.ptr, x.data_ptr(), Q8_IMAGE if image else _xdtype(x), _p(h),
+                                                 _p(img), M, wg.N, wg.K, act_scale_mode, _stream()), "mllm_hip_mlp_gate_up_q")
+    if want_h and want_image:
+        return h, img
+    return h if want_h else img
+
+
 def set_exp_mode(accurate):
     _lib.check(_lib.lib().mllm_hip_set_exp_mode(int(accurate)), "mllm_hip_set_exp_mode")
 

@@ -171,6 +171,47 @@ def test_gemv_fused_equals_the_operators_it_replaces(wtype, M):
     assert rel_l2(g1.cpu().numpy(), gn) < TOL and rel_l2(a1.cpu().numpy(), an) < TOL and rel_l2(o1.cpu().numpy(), on) < TOL
 
 
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M,H,I", [(1, 512, 1536), (2, 512, 96), (3, 2560, 9728), (4, 4096, 512), (5, 96, 64), (8, 2560, 1024), (1, 2560, 9728)])
+def test_mlp_gate_up_one_launch(wtype, M, H, I):
+    """gate / up / SiLU / product (/ Q8_0 image of the product) in one launch against the oracle's chain, and the image
+    against the Q8_0 quantization of the h the same launch stored (bit-exact); from activations and from rmsnorm's image"""
+    rng = synth.rng_for(6, 5000 + wtype * 1000 + M * 10 + H % 7)
+    Wg, Wu = synth.make_weight(rng, wtype, I, H), synth.make_weight(rng, wtype, I, H)
+    pg, pu = ql.PackedQWeight(wtype, torch.from_numpy(Wg)), ql.PackedQWeight(wtype, torch.from_numpy(Wu))
+    xf = synth.make_x_fp32(rng, M, H)
+    x = to_dev(xf)
+    announce("mlp gate/up one launch", wtype, M, H, I)
+    h, img = ql.mlp_gate_up(pg, pu, x, want_image=True)
+    gn = orc.linear_q(xf, Wg, wtype, None, orc.SCALE_X86_REF)
+    un = orc.linear_q(xf, Wu, wtype, None, orc.SCALE_X86_REF)
+    assert rel_l2(h.cpu().numpy(), orc.silu(gn) * un) < TOL
+    _check_image(img, h.cpu().numpy(), M, I, True)
+    # the separate launches it replaces: same arithmetic, row sums over other lane counts -> equal to fp32 rounding
+    g0, u0 = ql.linear_q_gemv_multi([pg, pu], x)
+    assert rel_l2(h.cpu().numpy(), ql.silu_mul(g0, u0).cpu().numpy()) < 1e-5
+    # only one of the two results asked for; bf16 activations; the image of x handed over
+    assert torch.equal(ql.mlp_gate_up(pg, pu, x), h)
+    same = lambda a, b: all(np.array_equal(p, q) for p, q in zip(_image_fields(a, M, I), _image_fields(b, M, I)))
+    assert same(ql.mlp_gate_up(pg, pu, x, want_h=False, want_image=True), img)
+    _, ximg = ql.add(x, torch.zeros_like(x), want_image=True)
+    h2, img2 = ql.mlp_gate_up(pg, pu, ximg, M=M, image=True, want_image=True)
+    assert torch.equal(h2, h) and same(img2, img)
+    xb = x.to(torch.bfloat16)
+    hb = ql.mlp_gate_up(pg, pu, xb)
+    assert torch.equal(hb, ql.mlp_gate_up(pg, pu, xb.float()))
+    # IEEE scales and the accurate exp
+    hi, imgi = ql.mlp_gate_up(pg, pu, x, want_image=True, act_scale_mode=ql.SCALE_IEEE)
+    _check_image(imgi, hi.cpu().numpy(), M, I, False)
+    ql.set_exp_mode(True)
+    try:
+        ha = ql.mlp_gate_up(pg, pu, x)
+    finally:
+        ql.set_exp_mode(False)
+    g64, u64 = gn.astype(np.float64), un.astype(np.float64)
+    assert rel_l2(ha.cpu().numpy(), g64 / (1 + np.exp(-g64)) * u64) < 1e-5
+
+
 @pytest.mark.parametrize("rows,n", [(1, 128), (512, 128), (5, 16), (7, 13), (3, 1000), (9, 60)])
 def test_softmax(rows, n):
     rng = synth.rng_for(6, 4000 + rows + n)
@@ -256,3 +297,7 @@ def test_argument_checks():
     assert L.mllm_hip_moe_gate(p, 0, p, p, p, None, 1, 12, 4, 2, 1, None) == -2      # H % 8
     assert L.mllm_hip_moe_gate(p, 0, p, p, p, None, 1, 8, 4, 5, 1, None) == -2       # k > E
     assert L.mllm_hip_set_exp_mode(2) == -1
+    assert L.mllm_hip_mlp_gate_up_q(0, p, p, p, 0, p, None, 9, 64, 64, 0, None) == -2  # at most eight rows
+    assert L.mllm_hip_mlp_gate_up_q(0, p, p, p, 0, p, None, 1, 48, 64, 0, None) == -2  # I % 32
+    assert L.mllm_hip_mlp_gate_up_q(0, p, p, p, 0, None, None, 1, 64, 64, 0, None) == -1  # no result asked for
+    assert L.mllm_hip_mlp_gate_up_q(2, p, p, p, 0, p, None, 1, 64, 64, 0, None) == -1  # Q4_0 / Q8_0 only
