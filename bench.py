@@ -188,6 +188,19 @@ def side_workloads(torch, ql, synth, gen):
     out["q4_0_linear_prefill_2048x9728x2560"] = {"us": t2 * 1e6, "TFLOPS": fl / t2 / 1e12, "frac_of_2500_TFLOPS": fl / t2 / 2.5e15,
                                                   "path": "matrix cores (mllm_hip_linear_q_gemm)",
                                                   "block_dot_path": {"us": t1 * 1e6, "TOPS": fl / t1 / 1e12}}
+    del wv, wg
+    # the same Linear with Q4_K / Q6_K weights (Q8_K activations): matrix cores against passes of the eight-row GEMV
+    for kname, kt in (("q4_k", ql.Q4_K), ("q6_k", ql.Q6_K)):
+        wkg = ql.PackedKWeight.synthetic(kt, N, K, gen, layout="gemm")
+        wsk = torch.empty(L.mllm_hip_linear_kq_gemm_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+        tk = ev_time(lambda: ql.linear_kq_gemm(wkg, xx, out=yy, workspace=wsk), 10)
+        wkv = ql.PackedKWeight.synthetic(kt, N, K, gen)
+        wsv = ql.kq_workspace(M, K)
+        tv = ev_time(lambda: ql.linear_kq(wkv, xx, out=yy, workspace=wsv), 3)
+        out["%s_linear_prefill_2048x9728x2560" % kname] = {"us": tk * 1e6, "TFLOPS": fl / tk / 1e12, "frac_of_2500_TFLOPS": fl / tk / 2.5e15,
+                                                            "path": "matrix cores (mllm_hip_linear_kq_gemm)",
+                                                            "gemv_passes_path": {"us": tv * 1e6}}
+        del wkg, wkv
     return out
 
 

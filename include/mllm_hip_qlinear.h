@@ -296,6 +296,17 @@ int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv_part* pa
 int mllm_hip_kq_set_tuning(int lanes_per_row, int waves_per_wg, int units_in_flight);
 int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y, int64_t M, int64_t N,
                        int64_t K, void* workspace, void* stream);
+/* Many rows (prefill) on the matrix cores, as mllm_hip_linear_q_gemm: fp16 operands with the scales folded in
+ * (activations: the Q8_K round trip fp16(d * q), codes and d bit-exact; weights: fma(q, fp16(d*sc), -fp16(dmin*m)) for
+ * Q4_K, (q - 32) * fp16(d*sc) for Q6_K, each rounded once), fp32 accumulation; within about 5e-4 relative L2 of the
+ * reference's arithmetic (mllm_hip_linear_kq keeps that arithmetic itself).  Weights "gemm-packed" once at load time from
+ * the reference blocks: Q4_K 0.5 byte + Q6_K 1 byte per weight, plus 8 bytes of scales per 64 weights. */
+size_t mllm_hip_kq_gemm_packed_bytes(int wtype, int64_t N, int64_t K);
+int mllm_hip_kq_gemm_prepack(int wtype, const void* blocks, int weight_scale_mode, void* gemm_packed, int64_t N, int64_t K,
+                             void* stream);
+size_t mllm_hip_linear_kq_gemm_workspace_bytes(int64_t M, int64_t K);
+int mllm_hip_linear_kq_gemm(int wtype, const void* gemm_packed, const void* x, int x_dtype, const float* bias, float* y,
+                            int64_t M, int64_t N, int64_t K, void* workspace, void* stream);
 /* Parity probes.  Dequantized weights fp32 [N][K] (dequantize_row_q4_K / _q6_K, quantize_q4.cpp:284-312, quantize_q6.cpp:108-133);
  * Q8_K activation quantization: codes int8 [M][K], d fp32 [M][K/256], sums of 16 codes int16 [M][K/16]. */
 int mllm_hip_kq_dequantize(int wtype, const void* packed, float* w, int64_t N, int64_t K, void* stream);

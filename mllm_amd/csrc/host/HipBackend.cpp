@@ -191,6 +191,11 @@ void HipLinearOp::load(const ParameterFile::ptr_t& ploader) {
       Tensor dev_blocks = onDevice(weight_);
       packed_ = Tensor::empty({(int32_t)pb}, kByte, kHIP).alloc();
       MLLM_HIP_KERNEL_CHECK(mllm_hip_kq_prepack(wt, dev_blocks.ptr<void>(), be.config().weight_scale_mode, packed_.ptr<void>(), N, K, be.stream()));
+      if (be.config().prefill_matrix_cores) {
+        gemm_packed_ = Tensor::empty({(int32_t)mllm_hip_kq_gemm_packed_bytes(wt, N, K)}, kByte, kHIP).alloc();
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_kq_gemm_prepack(wt, dev_blocks.ptr<void>(), be.config().weight_scale_mode, gemm_packed_.ptr<void>(), N, K,
+                                                       be.stream()));
+      }
       be.synchronize();
       if (options_.bias) bias_dev_ = onDevice(bias_);
       break;
@@ -298,11 +303,17 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
       break;
     }
     case Scheme::kQ4_K:
-    case Scheme::kQ6_K:
-      MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_kq(scheme_ == Scheme::kQ4_K ? MLLM_HIP_Q4_K : MLLM_HIP_Q6_K, packed_.ptr<void>(), x.ptr<void>(), xdt(),
-                                               bias, y.ptr<float>(), M, N, K, M >= 3 ? workspace(mllm_hip_kq_workspace_bytes(M, K)) : nullptr,
-                                               st));
+    case Scheme::kQ6_K: {
+      const int wt = scheme_ == Scheme::kQ4_K ? MLLM_HIP_Q4_K : MLLM_HIP_Q6_K;
+      if (M > 8 && !gemm_packed_.isNil()) {  // prefill: matrix cores
+        void* ws = workspace(mllm_hip_linear_kq_gemm_workspace_bytes(M, K));
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_kq_gemm(wt, gemm_packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K, ws, st));
+      } else {
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_kq(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K,
+                                                 M >= 3 ? workspace(mllm_hip_kq_workspace_bytes(M, K)) : nullptr, st));
+      }
       break;
+    }
     case Scheme::kW8A8: {
       void* ws = workspace(mllm_hip_w8a8_workspace_bytes(M, K));
       MLLM_HIP_KERNEL_CHECK(mllm_hip_w8a8_linear_packed(x.ptr<void>(), xdt(), packed_.ptr<void>(), weight_scale_.ptr<float>(), bias, y.ptr<void>(),

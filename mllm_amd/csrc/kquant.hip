@@ -16,6 +16,7 @@
 #include <initializer_list>
 
 #include "qcommon.h"
+#include "qgemm_layout.h"
 
 #define QK_K 256
 
@@ -579,6 +580,106 @@ static int launch_kq(const KGemvArgs& a, hipStream_t st) {
   return launch_kq_m<WT, XT, 8>(a, st);
 }
 
+
+// ---- many rows: the matrix-core GEMM of the block formats (moe.hip, qg_kernel) with these weights -------------------------
+// Same scheme as for Q4_0 / Q8_0: both operands as fp16 with their scales folded in, fp32 accumulation in
+// v_mfma_f32_32x32x16_f16.  Activations: the Q8_K round trip xh = fp16(d * q) (codes and d bit-exact, the product rounded
+// once).  Weights: Q4_K as 4-bit codes q with the sub-block's fp16(d * sc) and fp16(dmin * m), value = fma(q, ds, -dm)
+// rounded once; Q6_K as int8 codes q - 32 with fp16(d * sc) per 16 elements.  Within about 5e-4 relative L2 of the
+// reference's integer / fp32 arithmetic.
+//
+// code area, Q4_K: one output dword per thread, in the order of the Q4_0 gemm layout
+template <int WT>
+__global__ __launch_bounds__(256) void kqg_prepack_q_kernel(const uint8_t* __restrict__ blocks, uint32_t* __restrict__ P, int N, int K,
+                                                            int64_t words) {
+  const int64_t w = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (w >= words) return;
+  const int kbs = K / 64, nsb = K / QK_K;
+  uint32_t v = 0;
+  if (WT == MLLM_HIP_Q4_K) {
+    const int d = (int)(w % 4), l = (int)((w / 4) % 64);
+    const int64_t blk = w / 256;
+    const int kb = (int)(blk % kbs), nb = (int)(blk / kbs);
+    const int n = nb * 32 + (l & 31), k0 = kb * 64 + d * 16 + (l >> 5) * 8;
+    if (n < N) {
+      const uint8_t* qs = blocks + ((int64_t)n * nsb + k0 / QK_K) * 144 + 16;
+      const int e = k0 % QK_K, c = e >> 6, p = e & 63;  // 64-element chunk, position: low nibbles first, then high
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        const uint32_t byte = qs[32 * c + (p & 31) + i];
+        const uint32_t q = p < 32 ? (byte & 15u) : (byte >> 4);
+        v |= q << (4 * ((i >> 1) + 4 * (i & 1)));
+      }
+    }
+  } else {
+    const int x = (int)(w % 4), l = (int)((w / 4) % 64), pl = (int)((w / 256) % 2);
+    const int64_t blk = w / 512;
+    const int kb = (int)(blk % kbs), nb = (int)(blk / kbs);
+    const int d = 2 * pl + x / 2;
+    const int n = nb * 32 + (l & 31), k0 = kb * 64 + d * 16 + (l >> 5) * 8 + 4 * (x % 2);
+    if (n < N) {
+      const uint8_t* b = blocks + ((int64_t)n * nsb + k0 / QK_K) * 210;
+      uint32_t c[4];
+#pragma unroll
+      for (int i = 0; i < 4; i++) {  // dequantize_row_q6_K's element order: halves of 128, quarters of 32
+        const int e = k0 % QK_K + i, h = e >> 7, r = e & 127, g = r >> 5, ll = r & 31;
+        int lo = b[64 * h + ((g & 1) ? 32 : 0) + ll];
+        lo = g >= 2 ? (lo >> 4) : (lo & 15);
+        const int hi = (b[128 + 32 * h + ll] >> (2 * g)) & 3;
+        c[i] = (uint32_t)((lo | (hi << 4)) - 32) & 0xffu;
+      }
+      v = c[0] | (c[2] << 8) | (c[1] << 16) | (c[3] << 24);
+    }
+  }
+  P[w] = v;
+}
+// scale records: one thread per (32-row group, 64-element step, row)
+template <int WT>
+__global__ __launch_bounds__(256) void kqg_prepack_s_kernel(const uint8_t* __restrict__ blocks, u32x2* __restrict__ S, int N, int K, int x86,
+                                                            int64_t count) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  const int kbs = K / 64, nsb = K / QK_K;
+  const int row = (int)(i % 32), kb = (int)((i / 32) % kbs), nb = (int)(i / 32 / kbs);
+  const int n = nb * 32 + row;
+  u32x2 v{0u, 0u};
+  if (n < N) {
+    if (WT == MLLM_HIP_Q4_K) {
+      const uint8_t* b = blocks + ((int64_t)n * nsb + kb / 4) * 144;
+      const float d = f16bits_to_f32(field_bits(b, x86)), dmin = f16bits_to_f32(field_bits(b + 2, x86));
+      const K4Scales k = k4_scales(bytes_u32(b + 4), bytes_u32(b + 8), bytes_u32(b + 12));
+      const int j = 2 * (kb % 4);
+      v.x = (uint32_t)f32_to_f16bits(d * (float)byte_of(k.sc0, k.sc1, j)) | ((uint32_t)f32_to_f16bits(d * (float)byte_of(k.sc0, k.sc1, j + 1)) << 16);
+      v.y = (uint32_t)f32_to_f16bits(dmin * (float)byte_of(k.mn0, k.mn1, j)) | ((uint32_t)f32_to_f16bits(dmin * (float)byte_of(k.mn0, k.mn1, j + 1)) << 16);
+    } else {
+      const uint8_t* b = blocks + ((int64_t)n * nsb + kb / 4) * 210;
+      const float d = f16bits_to_f32(field_bits(b + 208, x86));
+      const int8_t* sc = reinterpret_cast<const int8_t*>(b + 192) + 4 * (kb % 4);
+      v.x = (uint32_t)f32_to_f16bits(d * (float)sc[0]) | ((uint32_t)f32_to_f16bits(d * (float)sc[1]) << 16);
+      v.y = (uint32_t)f32_to_f16bits(d * (float)sc[2]) | ((uint32_t)f32_to_f16bits(d * (float)sc[3]) << 16);
+    }
+  }
+  S[i] = v;
+}
+// activations: Q8_K quantization and back to fp16 in one pass, xh[rows][K]
+__global__ __launch_bounds__(256) void kq_act_f16_kernel(const void* __restrict__ x, int x_dtype, uint16_t* __restrict__ xh, int64_t nitems) {
+  const int64_t it = (int64_t)blockIdx.x * 256 + threadIdx.x;  // nitems is a multiple of 32: whole half-waves
+  if (it >= nitems) return;
+  float v[8];
+  if (x_dtype == MLLM_HIP_F32) load8<MLLM_HIP_F32>(x, it * 8, v);
+  else load8<MLLM_HIP_BF16>(x, it * 8, v);
+  const Q8KItem r = quantize_q8k_item(v, threadIdx.x & 63);
+  uint32_t o[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const uint32_t word = j < 2 ? r.q0 : r.q1;
+    const float a = r.d * (float)(int8_t)(word >> (16 * (j & 1)));
+    const float b = r.d * (float)(int8_t)(word >> (16 * (j & 1) + 8));
+    o[j] = (uint32_t)f32_to_f16bits(a) | ((uint32_t)f32_to_f16bits(b) << 16);
+  }
+  *reinterpret_cast<u32x4*>(xh + it * 8) = u32x4{o[0], o[1], o[2], o[3]};
+}
+
 }  // namespace mllmhip
 
 using namespace mllmhip;
@@ -693,4 +794,51 @@ MLLM_API int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, in
   if (!y) return MLLM_HIP_E_BADARG;
   mllm_hip_gemv_part part{packed, bias, y, N};
   return mllm_hip_linear_kq_multi(wtype, 1, &part, x, x_dtype, M, K, workspace, stream);
+}
+
+// ---- many rows on the matrix cores ------------------------------------------------------------------------------------------
+static bool kq_type(int wtype) { return wtype == MLLM_HIP_Q4_K || wtype == MLLM_HIP_Q6_K; }
+MLLM_API size_t mllm_hip_kq_gemm_packed_bytes(int wtype, int64_t N, int64_t K) {
+  if (!kq_type(wtype) || N <= 0 || K <= 0 || K % QK_K) return 0;
+  return (size_t)qg_bytes(wtype, N, K);
+}
+MLLM_API int mllm_hip_kq_gemm_prepack(int wtype, const void* blocks, int weight_scale_mode, void* gemm_packed, int64_t N, int64_t K,
+                                      void* stream) {
+  if (!kq_type(wtype) || !blocks || !gemm_packed || N <= 0 || K <= 0) return MLLM_HIP_E_BADARG;
+  if (weight_scale_mode != MLLM_HIP_SCALE_IEEE && weight_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
+  if (K % QK_K || N > INT32_MAX || K > INT32_MAX || qg_bytes(wtype, N, K) >= ((int64_t)1 << 32)) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(gemm_packed) % 16) return MLLM_HIP_E_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t words = qg_qbytes(wtype, N, K) / 4, count = qg_np(N) * (K / 64);
+  const uint8_t* b = reinterpret_cast<const uint8_t*>(blocks);
+  uint32_t* q = reinterpret_cast<uint32_t*>(gemm_packed);
+  u32x2* sc = reinterpret_cast<u32x2*>(reinterpret_cast<char*>(gemm_packed) + qg_qbytes(wtype, N, K));
+  const int x86 = weight_scale_mode == MLLM_HIP_SCALE_X86_REF;
+  const dim3 gq((unsigned)((words + 255) / 256)), gs((unsigned)((count + 255) / 256));
+  if (wtype == MLLM_HIP_Q4_K) {
+    hipLaunchKernelGGL(kqg_prepack_q_kernel<MLLM_HIP_Q4_K>, gq, dim3(256), 0, st, b, q, (int)N, (int)K, words);
+    hipLaunchKernelGGL(kqg_prepack_s_kernel<MLLM_HIP_Q4_K>, gs, dim3(256), 0, st, b, sc, (int)N, (int)K, x86, count);
+  } else {
+    hipLaunchKernelGGL(kqg_prepack_q_kernel<MLLM_HIP_Q6_K>, gq, dim3(256), 0, st, b, q, (int)N, (int)K, words);
+    hipLaunchKernelGGL(kqg_prepack_s_kernel<MLLM_HIP_Q6_K>, gs, dim3(256), 0, st, b, sc, (int)N, (int)K, x86, count);
+  }
+  return (int)hipGetLastError();
+}
+MLLM_API size_t mllm_hip_linear_kq_gemm_workspace_bytes(int64_t M, int64_t K) {
+  if (M <= 0 || K <= 0 || K % QK_K) return 0;
+  return align_up((size_t)M * K * 2, 256) + qg_route_bytes(M);
+}
+MLLM_API int mllm_hip_linear_kq_gemm(int wtype, const void* gemm_packed, const void* x, int x_dtype, const float* bias, float* y, int64_t M,
+                                     int64_t N, int64_t K, void* workspace, void* stream) {
+  if (!kq_type(wtype) || !gemm_packed || !x || !y || !workspace || M <= 0 || N <= 0 || K <= 0) return MLLM_HIP_E_BADARG;
+  if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
+  if (K % QK_K || M * K * 2 >= ((int64_t)1 << 32) || N > INT32_MAX || qg_bytes(wtype, N, K) >= ((int64_t)1 << 32)) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16 || reinterpret_cast<uintptr_t>(gemm_packed) % 16 ||
+      reinterpret_cast<uintptr_t>(y) % 16)
+    return MLLM_HIP_E_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  uint16_t* xh = reinterpret_cast<uint16_t*>(workspace);
+  const int64_t nitems = M * K / 8;
+  hipLaunchKernelGGL(kq_act_f16_kernel, dim3((unsigned)((nitems + 255) / 256)), dim3(256), 0, st, x, x_dtype, xh, nitems);
+  return qg_linear_run(wtype, gemm_packed, xh, bias, y, M, N, K, reinterpret_cast<char*>(workspace) + align_up((size_t)M * K * 2, 256), st);
 }

@@ -10,6 +10,7 @@
 // they are scaled and accumulated in fp32 on the vector ALU.  Tokens are the MFMA rows, weight rows the MFMA columns, so
 // a lane owns one output channel: its weight scale is a scalar per block and stores are contiguous across lanes.
 #include "qgemv_kernel.h"
+#include "qgemm_layout.h"
 
 namespace mllmhip {
 
@@ -419,14 +420,6 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-__host__ __device__ inline int64_t qg_kp(int64_t K) { return (K + 127) / 128 * 128; }
-__host__ __device__ inline int64_t qg_np(int64_t N) { return (N + 31) / 32 * 32; }
-__host__ __device__ inline int64_t qg_qbytes(int wtype, int64_t N, int64_t K) {
-  return wtype == MLLM_HIP_Q4_0 ? qg_np(N) * qg_kp(K) / 2 : qg_np(N) * qg_kp(K);
-}
-__host__ __device__ inline int64_t qg_bytes(int wtype, int64_t N, int64_t K) {
-  return qg_qbytes(wtype, N, K) + qg_np(N) * (qg_kp(K) / 64) * 4;
-}
 
 // one output dword of the code area per thread
 template <int WT>
@@ -547,10 +540,18 @@ struct QG2Args {
 
 // pair `b` (elements 2b, 2b+1) of the eight weights of one MFMA step, scaled: one dword of two fp16.  With PREC == 2 also
 // the rounding residual of the product (exact: the error of a product of two fp16 numbers is an fp16 number).
+// Q4_K: the sub-block's value is ds * q - dm (q = 0..15): one fused multiply-add, one rounding; Q6_K: codes widened to
+// int8 at load time, ds the scale of the step's 16 elements: the Q8_0 arithmetic.
 template <int WT, int PREC>
-__device__ __forceinline__ uint32_t qg_pair(const u32x4 (&rq)[WT == MLLM_HIP_Q4_0 ? 1 : 2], int d, int b, f16x2 dd, uint32_t& lo) {
+__device__ __forceinline__ uint32_t qg_pair(const u32x4 (&rq)[qg_nibbles(WT) ? 1 : 2], int d, int b, f16x2 dd, f16x2 dm, uint32_t& lo) {
   uint32_t t;
   f16x2 off;
+  if (WT == MLLM_HIP_Q4_K) {
+    static_assert(WT != MLLM_HIP_Q4_K || PREC == 1, "one-term operands only");
+    t = ((rq[0][d] >> (4 * b)) & 0x000f000fu) | 0x64006400u;       // (1024 + q) in both halves
+    const f16x2 c = __builtin_bit_cast(f16x2, t) - f16x2{(_Float16)1024.f, (_Float16)1024.f};  // q, exact
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(c, dd, -dm));                // v_pk_fma_f16
+  }
   if (WT == MLLM_HIP_Q4_0) {
     t = ((rq[0][d] >> (4 * b)) & 0x000f000fu) | 0x64006400u;       // (1024 + q) in both halves
     off = f16x2{(_Float16)1032.f, (_Float16)1032.f};               // ... - 1032 = q - 8, exact
@@ -577,7 +578,8 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
   constexpr int BM = TM * 32, WN = TN * 32;
   constexpr int CA = TM;  // 16-byte activation chunks per thread and K step: 32 TM rows x 8 chunks over 256 threads
   constexpr int STAGE = PREC * BM * LDK;  // value rows, then residual rows
-  constexpr int QW = WT == MLLM_HIP_Q4_0 ? 1 : 2;
+  constexpr int QW = qg_nibbles(WT) ? 1 : 2;
+  constexpr int SDW = qg_scale_dwords(WT);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int lrow = lane & 31, hi = lane >> 5;
@@ -604,7 +606,7 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
   for (int j = 0; j < TN; j++) {
     const int nb = min((n0 + wave * WN) / 32 + j, nbs - 1);
     offQ[j] = (uint32_t)((int64_t)nb * kbs * (1024 * QW) + lane * 16);
-    offS[j] = (uint32_t)(qbytes + ((int64_t)nb * kbs * 32 + lrow) * 4);
+    offS[j] = (uint32_t)(qbytes + ((int64_t)nb * kbs * 32 + lrow) * 4 * SDW);
   }
   const __amdgpu_buffer_rsrc_t rAl = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(PREC == 2 ? a.xl : a.xh), 0, (uint32_t)((int64_t)a.a_rows * a.K * 2), 0x00020000);
   auto loadA = [&](int k0, u32x4 (&ga)[PREC][CA]) {
@@ -644,9 +646,18 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
 
   u32x4 ga[PREC][CA];
   u32x4 rq[2][NW][TN][QW];      // packed codes of K steps kt (set kt & 1) and kt + 1
-  uint32_t rs[2][NW][TN];       // their two block scales
+  uint32_t rs[2][NW][TN][SDW];  // their scale records
   f16x8 fb[2][NW][TN][PREC];    // dequantized operands of MFMA step ks (set ks & 1): value, residual
   f16x8 fa[2][PREC][TM];
+  auto loadS = [&](uint32_t (&r)[SDW], int w, int j, int kb) {
+    if (SDW == 1) {
+      r[0] = __builtin_amdgcn_raw_buffer_load_b32(rW[w], offS[j], kb * 128, 0);
+    } else {
+      const u32x2 v = __builtin_amdgcn_raw_buffer_load_b64(rW[w], offS[j], kb * 256, 0);
+      r[0] = v.x;
+      r[SDW - 1] = v.y;
+    }
+  };
   auto loadW = [&](int set, int kb) {
 #pragma unroll
     for (int w = 0; w < NW; w++)
@@ -654,11 +665,22 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
       for (int j = 0; j < TN; j++) {
 #pragma unroll
         for (int p = 0; p < QW; p++) rq[set][w][j][p] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], offQ[j], (kb * QW + p) * 1024, 0);
-        rs[set][w][j] = __builtin_amdgcn_raw_buffer_load_b32(rW[w], offS[j], kb * 128, 0);
+        loadS(rs[set][w][j], w, j, kb);
       }
   };
-  auto scale2 = [&](uint32_t s, int d) -> f16x2 {  // the block scale of dword d in both halves
-    const uint32_t h = d < 2 ? (s & 0xffffu) : (s >> 16);
+  // the scale of dword d (K elements 16 d .. 16 d + 15 of the step) in both halves; for Q4_K also the offset
+  auto scale2 = [&](const uint32_t (&s)[SDW], int d) -> f16x2 {
+    uint32_t h;
+    if constexpr (WT == MLLM_HIP_Q6_K) {
+      const uint32_t v = s[d >> 1];
+      h = (d & 1) ? (v >> 16) : (v & 0xffffu);
+    } else {
+      h = d < 2 ? (s[0] & 0xffffu) : (s[0] >> 16);
+    }
+    return __builtin_bit_cast(f16x2, h | (h << 16));
+  };
+  auto offset2 = [&](const uint32_t (&s)[SDW], int d) -> f16x2 {
+    const uint32_t h = d < 2 ? (s[SDW - 1] & 0xffffu) : (s[SDW - 1] >> 16);
     return __builtin_bit_cast(f16x2, h | (h << 16));
   };
   loadA(0, ga);
@@ -671,10 +693,10 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
   for (int w = 0; w < NW; w++)
 #pragma unroll
     for (int j = 0; j < TN; j++) {
-      const f16x2 dd = scale2(rs[0][w][j], 0);
+      const f16x2 dd = scale2(rs[0][w][j], 0), dm = offset2(rs[0][w][j], 0);
       uint32_t o[4], ol[4] = {0, 0, 0, 0};
 #pragma unroll
-      for (int b = 0; b < 4; b++) o[b] = qg_pair<WT, PREC>(rq[0][w][j], 0, b, dd, ol[b]);
+      for (int b = 0; b < 4; b++) o[b] = qg_pair<WT, PREC>(rq[0][w][j], 0, b, dd, dm, ol[b]);
       fb[0][w][j][0] = __builtin_bit_cast(f16x8, u32x4{o[0], o[1], o[2], o[3]});
       if (PREC == 2) fb[0][w][j][PREC - 1] = __builtin_bit_cast(f16x8, u32x4{ol[0], ol[1], ol[2], ol[3]});
     }
@@ -701,7 +723,7 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
 #pragma unroll
         for (int j = 0; j < TN; j++) {
           // the dequantization of the next step's operand is cut into TM pieces, one pinned into the shadow of each MFMA
-          const f16x2 dd = scale2(rs[ns][w][j], nd);
+          const f16x2 dd = scale2(rs[ns][w][j], nd), dm = offset2(rs[ns][w][j], nd);
           uint32_t o[4], ol[4] = {0, 0, 0, 0};
 #pragma unroll
           for (int i = 0; i < TM; i++) {
@@ -711,7 +733,7 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
               acc[w][j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fb[ks & 1][w][j][0], fa[ks & 1][PREC - 1][i], acc[w][j][i], 0, 0, 0);
             }
 #pragma unroll
-            for (int b = i * 4 / TM; b < (i + 1) * 4 / TM; b++) o[b] = qg_pair<WT, PREC>(rq[ns][w][j], nd, b, dd, ol[b]);
+            for (int b = i * 4 / TM; b < (i + 1) * 4 / TM; b++) o[b] = qg_pair<WT, PREC>(rq[ns][w][j], nd, b, dd, dm, ol[b]);
             __builtin_amdgcn_sched_barrier(0);
           }
           fb[(ks + 1) & 1][w][j][0] = __builtin_bit_cast(f16x8, u32x4{o[0], o[1], o[2], o[3]});
@@ -720,7 +742,7 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
 #pragma unroll
             for (int p = 0; p < QW; p++)
               rq[CUR][w][j][p] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], offQ[j], ((kt + 2) * QW + p) * 1024, 0);
-            rs[CUR][w][j] = __builtin_amdgcn_raw_buffer_load_b32(rW[w], offS[j], (kt + 2) * 128, 0);
+            loadS(rs[CUR][w][j], w, j, kt + 2);
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -809,7 +831,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   if (t >= a.ntiles[0]) return;
   const int e = a.tile_expert[t];
   int row0 = a.tile_row0[t], rows = a.tile_rows[t];
-  if (MODE == 1) {
+  if constexpr (MODE == 1) {
     const int n0 = blockIdx.y * 128;
     row0 += 64 * blockIdx.z;
     rows -= 64 * blockIdx.z;
@@ -832,7 +854,11 @@ static int launch_qg(const QG2Args& a, unsigned max_tiles, hipStream_t st) {
   const dim3 grid(max_tiles, (unsigned)((a.N + 128 * TN - 1) / (128 * TN)), MODE == 1 ? 2 : 1);
   const size_t lds = 2 * (size_t)QG_TILE_H * (2 * 64 + 16);  // MODE 1: half the rows, value + residual
   if (a.wtype == MLLM_HIP_Q4_0) hipLaunchKernelGGL((qg_kernel<MLLM_HIP_Q4_0, MODE>), grid, dim3(256), lds, st, a);
-  else hipLaunchKernelGGL((qg_kernel<MLLM_HIP_Q8_0, MODE>), grid, dim3(256), lds, st, a);
+  else if (a.wtype == MLLM_HIP_Q8_0) hipLaunchKernelGGL((qg_kernel<MLLM_HIP_Q8_0, MODE>), grid, dim3(256), lds, st, a);
+  else if constexpr (MODE == 0) {  // the super-block formats: plain Linear only
+    if (a.wtype == MLLM_HIP_Q4_K) hipLaunchKernelGGL((qg_kernel<MLLM_HIP_Q4_K, 0>), grid, dim3(256), lds, st, a);
+    else hipLaunchKernelGGL((qg_kernel<MLLM_HIP_Q6_K, 0>), grid, dim3(256), lds, st, a);
+  } else return MLLM_HIP_E_BADARG;
   return (int)hipGetLastError();
 }
 
@@ -887,6 +913,26 @@ static int launch_tiles(int wtype, const QGemmArgs& a, unsigned max_tiles, hipSt
     return (int)hipGetLastError();
   };
   return wtype == MLLM_HIP_Q4_0 ? launch(qgemm_tile_kernel<MLLM_HIP_Q4_0, MODE>) : launch(qgemm_tile_kernel<MLLM_HIP_Q8_0, MODE>);
+}
+
+size_t qg_route_bytes(int64_t M) {
+  Carver c(nullptr);
+  carve_route(c, 1, M);
+  return c.used;
+}
+int qg_linear_run(int wtype, const void* gemm_packed, const uint16_t* xh, const float* bias, float* y, int64_t M, int64_t N,
+                  int64_t K, void* route_ws, hipStream_t st) {
+  Carver c(route_ws);
+  RouteOut ro = carve_route(c, 1, M);
+  hipLaunchKernelGGL(identity_tiles_kernel, dim3(1), dim3(256), 0, st, (int)M, QG_TILE_H, ro);
+  QG2Args a{};
+  a.W0 = a.W1 = reinterpret_cast<const char*>(gemm_packed);
+  a.wstride = 0;
+  a.xh = xh; a.a_index = nullptr; a.a_div = 1; a.a_rows = (int)M;
+  a.o_index = nullptr; a.out = y; a.bias = bias;
+  a.tile_expert = ro.tile_expert; a.tile_row0 = ro.tile_row0; a.tile_rows = ro.tile_rows; a.ntiles = ro.ntiles;
+  a.N = (int)N; a.K = (int)K; a.wtype = wtype; a.x86_scale = 0;
+  return launch_qg<0>(a, (unsigned)((M + QG_TILE_H - 1) / QG_TILE_H), st);
 }
 
 }  // namespace mllmhip
@@ -1075,19 +1121,10 @@ MLLM_API int mllm_hip_linear_q_gemm(int wtype, const void* gemm_packed, const vo
   hipStream_t st = (hipStream_t)stream;
   Carver c(workspace);
   uint16_t* xh = c.take<uint16_t>((size_t)M * K);
-  RouteOut ro = carve_route(c, 1, M);
   const int64_t nblocks = M * (K / QK);
   hipLaunchKernelGGL(qg_act_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, xh,
                      (uint16_t*)nullptr, nblocks, act_scale_mode == MLLM_HIP_SCALE_X86_REF);
-  hipLaunchKernelGGL(identity_tiles_kernel, dim3(1), dim3(256), 0, st, (int)M, QG_TILE_H, ro);
-  QG2Args a{};
-  a.W0 = a.W1 = reinterpret_cast<const char*>(gemm_packed);
-  a.wstride = 0;
-  a.xh = xh; a.a_index = nullptr; a.a_div = 1; a.a_rows = (int)M;
-  a.o_index = nullptr; a.out = y; a.bias = bias;
-  a.tile_expert = ro.tile_expert; a.tile_row0 = ro.tile_row0; a.tile_rows = ro.tile_rows; a.ntiles = ro.ntiles;
-  a.N = (int)N; a.K = (int)K; a.wtype = wtype; a.x86_scale = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
-  return launch_qg<0>(a, (unsigned)((M + QG_TILE_H - 1) / QG_TILE_H), st);
+  return qg_linear_run(wtype, gemm_packed, xh, bias, y, M, N, K, c.p + c.used, st);
 }
 
 MLLM_API size_t mllm_hip_moe_gemm_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k) {

@@ -512,25 +512,27 @@ KBLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
 class PackedKWeight:
     """Q4_K / Q6_K weight [N, K] repacked on the device.  blocks: uint8 [N, K/256, 144|210] (reference layout)."""
 
-    def __init__(self, wtype, blocks, weight_scale_mode=SCALE_IEEE):
+    def __init__(self, wtype, blocks, weight_scale_mode=SCALE_IEEE, layout="gemv"):
         assert blocks.dtype == torch.uint8 and blocks.dim() == 3 and blocks.shape[2] == KBLOCK_BYTES[wtype]
-        self.wtype, self.N, self.K = wtype, blocks.shape[0], blocks.shape[1] * 256
+        assert layout in ("gemv", "gemm")
+        self.wtype, self.N, self.K, self.layout = wtype, blocks.shape[0], blocks.shape[1] * 256, layout
         L = _lib.lib()
-        self.buf = torch.empty(L.mllm_hip_kq_packed_bytes(wtype, self.N, self.K), dtype=torch.uint8, device="cuda")
+        size, pack = ((L.mllm_hip_kq_packed_bytes, L.mllm_hip_kq_prepack) if layout == "gemv"
+                      else (L.mllm_hip_kq_gemm_packed_bytes, L.mllm_hip_kq_gemm_prepack))
+        self.buf = torch.empty(size(wtype, self.N, self.K), dtype=torch.uint8, device="cuda")
         src = blocks.contiguous().cuda()
-        _lib.check(L.mllm_hip_kq_prepack(wtype, src.data_ptr(), weight_scale_mode, self.buf.data_ptr(), self.N, self.K, _stream()),
-                   "mllm_hip_kq_prepack")
+        _lib.check(pack(wtype, src.data_ptr(), weight_scale_mode, self.buf.data_ptr(), self.N, self.K, _stream()), "kq prepack (%s)" % layout)
         torch.cuda.current_stream().synchronize()  # src may be released
 
     @classmethod
-    def synthetic(cls, wtype, N, K, gen):
+    def synthetic(cls, wtype, N, K, gen, layout="gemv"):
         """random blocks made on the device (bench): every byte uniform, fp16 fields set to a small positive value"""
         bb = KBLOCK_BYTES[wtype]
         blocks = torch.randint(0, 256, (N, K // 256, bb), dtype=torch.uint8, device="cuda", generator=gen)
         for off in ((0, 2) if wtype == Q4_K else (208,)):
             blocks[:, :, off] = 0x00
             blocks[:, :, off + 1] = 0x14  # 0x1400 = 9.8e-4
-        return cls(wtype, blocks)
+        return cls(wtype, blocks, layout=layout)
 
     @property
     def ptr(self):
@@ -546,9 +548,21 @@ def kq_workspace(M, K):
     return torch.empty(_lib.lib().mllm_hip_kq_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
 
 
+def linear_kq_gemm(w, x, bias=None, out=None, workspace=None):
+    """many rows on the matrix cores; w: PackedKWeight(layout="gemm")"""
+    assert w.layout == "gemm" and x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
+    M = x.shape[0]
+    L = _lib.lib()
+    y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")
+    ws = workspace if workspace is not None else torch.empty(L.mllm_hip_linear_kq_gemm_workspace_bytes(M, w.K), dtype=torch.uint8, device="cuda")
+    _lib.check(L.mllm_hip_linear_kq_gemm(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K, ws.data_ptr(),
+                                         _stream()), "mllm_hip_linear_kq_gemm")
+    return y
+
+
 def linear_kq(w, x, bias=None, out=None, workspace=None):
     """workspace (kq_workspace): from three rows on, x is quantized once by a small kernel instead of in every workgroup"""
-    assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
+    assert w.layout == "gemv" and x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
     M = x.shape[0]
     y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")
     _lib.check(_lib.lib().mllm_hip_linear_kq(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K,

@@ -120,6 +120,54 @@ def test_linear_kq_exact_cases(wtype):
     assert np.array_equal(y.astype(np.float64), want)
 
 
+@pytest.mark.parametrize("wtype", [2, 3])
+@pytest.mark.parametrize("M,N,K", [(9, 100, 256), (64, 257, 768), (130, 512, 2560), (33, 31, 512), (300, 96, 9728), (512, 300, 1024)])
+def test_linear_kq_gemm(wtype, M, N, K):
+    """many rows on the matrix cores (fp16 operands with folded scales) against the oracle's integer / fp32 arithmetic"""
+    rng = synth.rng_for(7, 700 + wtype * 1000 + M * 13 + N)
+    W = synth.make_weight(rng, wtype, N, K)
+    wg = ql.PackedKWeight(wtype, torch.from_numpy(W), layout="gemm")
+    bias = rng.standard_normal(N).astype(np.float32)
+    xf = synth.make_x_fp32(rng, M, K)
+    announce("linear kq gemm", wtype, M, N, K)
+    want = orc.linear_kq(xf, W, wtype, bias, orc.SCALE_X86_REF)
+    y = ql.linear_kq_gemm(wg, to_dev(xf), to_dev(bias)).cpu().numpy()
+    err = rel_l2(y, want)
+    print("rel-L2 %.2e" % err)
+    assert err < TOL
+    bits, xb = synth.make_x_bf16(rng, M, K)
+    y2 = ql.linear_kq_gemm(wg, bf16_dev(bits)).cpu().numpy()
+    assert rel_l2(y2, orc.linear_kq(xb, W, wtype, None, orc.SCALE_X86_REF)) < TOL
+    # and against the GEMV path (the reference arithmetic itself) on the same device
+    yv = ql.linear_kq(ql.PackedKWeight(wtype, torch.from_numpy(W)), to_dev(xf), to_dev(bias)).cpu().numpy()
+    assert rel_l2(y, yv) < TOL
+
+
+@pytest.mark.parametrize("wtype", [2, 3])
+def test_linear_kq_gemm_exact_cases(wtype):
+    """unit scales, small integer sub-block scales and integer activations that quantize to themselves: every operand is
+    an integer that fp16 holds exactly and every partial sum stays below 2^24, so the result must equal the integer
+    matrix product exactly (a misplaced code, scale or offset in the packed layout cannot pass)"""
+    rng = synth.rng_for(7, 60 + wtype)
+    N, K, M = 70, 768, 37
+    W = synth.make_weight(rng, wtype, N, K)
+    if wtype == 2:
+        W[:, :, 0:2] = np.array([0x00, 0x3c], np.uint8)
+        W[:, :, 2:4] = np.array([0x00, 0x3c], np.uint8)
+    else:
+        W[:, :, 208:210] = np.array([0x00, 0x3c], np.uint8)
+        W[:, :, 192:208] = rng.integers(-3, 4, size=(N, K // 256, 16)).astype(np.int8).view(np.uint8)
+    x = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    x[:, ::256] = -128.0  # max = -128 -> iscale = 1, d = 1: codes equal the values
+    wd = orc.dequantize_k(W, wtype, orc.SCALE_IEEE).astype(np.float64)
+    assert np.abs(wd).max() <= 2048
+    want = x.astype(np.float64) @ wd.T
+    assert (np.abs(x).astype(np.float64) @ np.abs(wd).T).max() < 2 ** 24
+    announce("linear kq gemm exact", wtype)
+    y = ql.linear_kq_gemm(ql.PackedKWeight(wtype, torch.from_numpy(W), layout="gemm"), to_dev(x)).cpu().numpy()
+    assert np.array_equal(y.astype(np.float64), want)
+
+
 def test_argument_checks():
     L = _lib.lib()
     buf = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
@@ -131,6 +179,12 @@ def test_argument_checks():
     assert L.mllm_hip_linear_kq(2, p + 16, p, 0, None, p, 1, 4, 256, None, None) == -3
     assert L.mllm_hip_kq_prepack(3, None, 0, p, 4, 256, None) == -1
     assert L.mllm_hip_quantize_q8_K(p, 0, p, p, p, 1, 100, None) == -2
+    assert L.mllm_hip_kq_gemm_packed_bytes(2, 4, 100) == 0
+    assert L.mllm_hip_kq_gemm_packed_bytes(1, 4, 256) == 0
+    assert L.mllm_hip_kq_gemm_packed_bytes(2, 33, 256) == 64 * 256 // 2 + 64 * 4 * 8
+    assert L.mllm_hip_linear_kq_gemm(2, p, p, 0, None, p, 16, 4, 100, p, None) == -2
+    assert L.mllm_hip_linear_kq_gemm(0, p, p, 0, None, p, 16, 4, 256, p, None) == -1
+    assert L.mllm_hip_linear_kq_gemm(2, p, p, 0, None, p, 16, 4, 256, None, None) == -1
 
 
 @pytest.mark.parametrize("name,wtype", [("q4_k", 2), ("q6_k", 3)])

@@ -91,7 +91,8 @@ def test_linear_through_the_op_factory(via_plugin):
             x = synth.make_x_fp32(rng, M, K)
             announce("host linear", scheme, M)
             y = _run(L, scheme, W, None, None, bias, x, False, M, N, K, 0, via_plugin)
-            assert rel_l2(y, orc.linear_kq(x, W, wtype, bias, orc.SCALE_X86_REF)) < 2e-6
+            # up to 8 rows the GEMV (integer / fp32 arithmetic), more the matrix-core path (fp16 operands, about 3.5e-4)
+            assert rel_l2(y, orc.linear_kq(x, W, wtype, bias, orc.SCALE_X86_REF)) < (2e-6 if M <= 8 else 1e-3)
     # W8A8
     M = 40
     a_bits, W8, ws = synth.make_w8a8(rng, M, N, K)
