@@ -139,6 +139,9 @@ int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
 /* GEMV launch-shape override for tuning sweeps: lanes per weight row (8/16/32/64), rows per lane group (1/2/4),
  * waves per workgroup (1..16); 0 restores the built-in heuristic. */
 int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_per_wg);
+/* Three to eight rows take their block sums from the matrix cores (v_mfma_i32_16x16x32_i8, same fp32 arithmetic around
+ * them); path = 1 keeps every launch on the vector-ALU kernel (comparison runs), 0 restores the default. */
+int mllm_hip_gemv_set_path(int path);
 
 /* ---------------------------------------------------------------------------------------------------------
  * Q4_0 / Q8_0 Linear and MoE expert FFN for many rows on the matrix cores

@@ -281,6 +281,14 @@ MLLM_API int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void*
   return (int)hipGetLastError();
 }
 
+static int g_gemv_path = 0;
+// 0: by the number of rows; 1: always the vector-ALU kernel (comparison runs and tests)
+MLLM_API int mllm_hip_gemv_set_path(int path) {
+  if (path != 0 && path != 1) return MLLM_HIP_E_BADARG;
+  g_gemv_path = path;
+  return 0;
+}
+
 MLLM_API int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_per_wg) {
   auto ok = [](int v, std::initializer_list<int> allowed) {
     for (int a : allowed)
@@ -361,6 +369,21 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8));
   GemvShape s = pick_shape(MT, nmax, a.nb);
   hipStream_t st = (hipStream_t)stream;
+  // three or more rows: block sums on the matrix cores (as long as the rows fit that kernel's LDS: 8 rows of 11 000 elements)
+  // Q8_0 (twice the code bytes per block) gains only from five rows on.  The rule looks at the weight type, the number of
+  // rows and the row length, never at the number of weight rows: a matrix takes the same kernel alone and in a multi launch.
+  if (MT >= 4 && g_gemv_path != 1 && (wtype == MLLM_HIP_Q4_0 || MT == 8) && gemv_mfma_fits(MT, a.nb)) {
+    const int waves = (g_tune_NW == 4 || g_tune_NW == 8) ? g_tune_NW : 0;
+    // a large launch (measured: from about 600 000 block-rows, i.e. gate + up and down of the 4B shapes): quantizing x in
+    // every workgroup costs more than one more small launch that quantizes it once
+    if (x_dtype != MLLM_HIP_Q8_IMAGE && workspace && nmax * a.nb >= 600000) {
+      hipLaunchKernelGGL(quant_image_kernel, dim3((unsigned)((MT * a.nb + 127) / 128)), dim3(128), 0, st, x, x_dtype,
+                         reinterpret_cast<unsigned char*>(workspace), M, MT, a.nb, a.x86_scale);
+      a.x = workspace;
+      return launch_gemv_mfma(wtype, GEMV_PREQ, MT, a, waves, st);
+    }
+    return launch_gemv_mfma(wtype, x_dtype, MT, a, waves, st);
+  }
   if (x_dtype == MLLM_HIP_Q8_IMAGE) {
     if (!g_tune_NW && MT <= 2) s.NW = a.nb >= 256 ? 8 : 4;
     return wtype == MLLM_HIP_Q4_0 ? launch_gemv_q4_preq(a, MT, s, st) : launch_gemv_q8_preq(a, MT, s, st);

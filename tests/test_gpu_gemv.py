@@ -223,6 +223,34 @@ def test_gemv_multi_equals_single(wtype, M):
 
 @pytest.mark.parametrize("wtype", [0, 1])
 @pytest.mark.parametrize("M", [3, 4, 5, 8])
+def test_gemv_matrix_core_and_vector_kernels_agree(wtype, M):
+    """three to eight rows: the matrix-core kernel (default) and the vector-ALU kernel are two independent implementations of
+    the same arithmetic (exact block sums, fp32 scaling); they differ only in the order of the fp32 sums"""
+    rng = synth.rng_for(1, 700 + M + 10 * wtype)
+    L = _lib.lib()
+    for N, K in ((9728, 2560), (2560, 9728), (100, 4096 + 64), (33, 96), (257, 8192)):
+        W = synth.make_weight(rng, wtype, N, K)
+        w = ql.PackedQWeight(wtype, torch.from_numpy(W))
+        bias = to_dev(rng.standard_normal(N).astype(np.float32))
+        xf = synth.make_x_fp32(rng, M, K)
+        xd = to_dev(xf)
+        announce("gemv both kernels", wtype, M, N, K)
+        y0 = ql.linear_q_gemv(w, xd, bias)
+        _, img = ql.add(xd, torch.zeros_like(xd), want_image=True)
+        (y0i,) = ql.linear_q_gemv_fused([w], img, M=M, image=True, biases=[bias])
+        assert torch.equal(y0, y0i)  # activations quantized in the kernel or handed over as an image: the same bits
+        assert L.mllm_hip_gemv_set_path(1) == 0
+        try:
+            y1 = ql.linear_q_gemv(w, xd, bias)
+        finally:
+            assert L.mllm_hip_gemv_set_path(0) == 0
+        assert rel_l2(y0.cpu().numpy(), y1.cpu().numpy()) < 2e-6
+        assert rel_l2(y0.cpu().numpy(), orc.linear_q(xf, W, wtype, bias.cpu().numpy(), orc.SCALE_X86_REF)) < 2e-6
+    assert L.mllm_hip_gemv_set_path(2) == -1
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M", [3, 4, 5, 8])
 def test_gemv_prequantized_equals_fused(wtype, M):
     """With a workspace (three rows or more) x is quantized once by a small kernel and the GEMV copies that image: the
     results must be the bits of the fused kernel, for fp32 and bf16 activations, both scale modes, long and ragged rows."""
