@@ -374,9 +374,10 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
   // rows and the row length, never at the number of weight rows: a matrix takes the same kernel alone and in a multi launch.
   if (MT >= 4 && g_gemv_path != 1 && (wtype == MLLM_HIP_Q4_0 || MT == 8) && gemv_mfma_fits(MT, a.nb)) {
     const int waves = (g_tune_NW == 4 || g_tune_NW == 8) ? g_tune_NW : 0;
-    // a large launch (measured: from about 600 000 block-rows, i.e. gate + up and down of the 4B shapes): quantizing x in
-    // every workgroup costs more than one more small launch that quantizes it once
-    if (x_dtype != MLLM_HIP_Q8_IMAGE && workspace && nmax * a.nb >= 600000) {
+    // quantizing x in every workgroup costs more than one more small launch that quantizes it once: with five to eight rows
+    // always (q+k+v of the 4B layer at eight rows: 11.2 us against 7.5 + 2.4), with three or four from about 600 000
+    // block-rows on (gate + up, down).  Same bits either way.
+    if (x_dtype != MLLM_HIP_Q8_IMAGE && workspace && (MT == 8 || nmax * a.nb >= 600000)) {
       hipLaunchKernelGGL(quant_image_kernel, dim3((unsigned)((MT * a.nb + 127) / 128)), dim3(128), 0, st, x, x_dtype,
                          reinterpret_cast<unsigned char*>(workspace), M, MT, a.nb, a.x86_scale);
       a.x = workspace;
