@@ -288,8 +288,11 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
           MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_fused(wt, 1, &part, nullptr, image, MLLM_HIP_Q8_IMAGE, (int)M, K,
                                                              be.config().act_scale_mode, st));
         } else {
-          MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), (int)M, N, K,
-                                                       be.config().act_scale_mode, st));
+          // from three rows on the activations are quantized once by a small kernel instead of in every workgroup (when
+          // the launch is large enough for that to pay; the library decides)
+          mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
+          void* ws = M >= 3 ? workspace(mllm_hip_gemv_workspace_bytes((int)M, K)) : nullptr;
+          MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_multi_ws(wt, 1, &part, x.ptr<void>(), xdt(), (int)M, K, be.config().act_scale_mode, ws, st));
         }
       } else if (!gemm_packed_.isNil()) {
         void* ws = workspace(mllm_hip_linear_q_gemm_workspace_bytes(M, K));
