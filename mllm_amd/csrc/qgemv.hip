@@ -373,7 +373,7 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
   // Q8_0 (twice the code bytes per block) gains only from five rows on.  The rule looks at the weight type, the number of
   // rows and the row length, never at the number of weight rows: a matrix takes the same kernel alone and in a multi launch.
   if (MT >= 4 && g_gemv_path != 1 && (wtype == MLLM_HIP_Q4_0 || MT == 8) && gemv_mfma_fits(MT, a.nb)) {
-    const int waves = (g_tune_NW == 4 || g_tune_NW == 8) ? g_tune_NW : 0;
+    const int waves = (g_tune_NW == 2 || g_tune_NW == 4 || g_tune_NW == 8) ? g_tune_NW : 0;
     // quantizing x in every workgroup costs more than one more small launch that quantizes it once: with five to eight rows
     // always (q+k+v of the 4B layer at eight rows: 11.2 us against 7.5 + 2.4), with three or four from about 600 000
     // block-rows on (gate + up, down).  Same bits either way.
@@ -381,9 +381,9 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
       hipLaunchKernelGGL(quant_image_kernel, dim3((unsigned)((MT * a.nb + 127) / 128)), dim3(128), 0, st, x, x_dtype,
                          reinterpret_cast<unsigned char*>(workspace), M, MT, a.nb, a.x86_scale);
       a.x = workspace;
-      return launch_gemv_mfma(wtype, GEMV_PREQ, MT, a, waves, st);
+      return launch_gemv_mfma(wtype, GEMV_PREQ, MT, a, waves, g_tune_R, st);
     }
-    return launch_gemv_mfma(wtype, x_dtype, MT, a, waves, st);
+    return launch_gemv_mfma(wtype, x_dtype, MT, a, waves, g_tune_R, st);
   }
   if (x_dtype == MLLM_HIP_Q8_IMAGE) {
     if (!g_tune_NW && MT <= 2) s.NW = a.nb >= 256 ? 8 : 4;

@@ -415,8 +415,8 @@ int launch_gemv(const GemvArgs& a, int MT, GemvShape s, hipStream_t st) {
   }
 }
 // three to eight rows on the matrix cores (qgemv_mfma.hip); x_kind: MLLM_HIP_F32, MLLM_HIP_BF16 or GEMV_PREQ; MT: 4 or 8;
-// waves per workgroup: 0 (by x_kind), 4 or 8
-int launch_gemv_mfma(int wtype, int x_kind, int MT, const GemvArgs& a, int waves, hipStream_t st);
+// waves per workgroup: 0 (by x_kind), 4 or 8; K slices per row tile: 0 (by row length), 1, 2 or 4 (sweeps)
+int launch_gemv_mfma(int wtype, int x_kind, int MT, const GemvArgs& a, int waves, int slices, hipStream_t st);
 bool gemv_mfma_fits(int MT, int nb);  // rows of nb blocks fit that kernel's LDS
 int launch_gemv_q4_f32(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
 int launch_gemv_q4_bf16(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);

@@ -373,9 +373,9 @@ static int mf_slices(int nb) {
 // waves per workgroup: eight when every workgroup quantizes the activations itself (twice the lanes for that, half the
 // workgroups repeating it), four when it copies their image
 template <int WT, int XT, int MT>
-static int launch_mfma_t(const GemvArgs& a_in, int waves, hipStream_t st) {
+static int launch_mfma_t(const GemvArgs& a_in, int waves, int slices, hipStream_t st) {
   GemvArgs a = a_in;
-  const int S = mf_slices(a.nb);
+  const int S = slices ? slices : mf_slices(a.nb);
   const int nbs = ((a.nb + S - 1) / S + 7) / 8 * 8;
   int nwaves = waves ? waves : (XT == GEMV_PREQ ? 4 : 8);
   if (nwaves < S) nwaves = S;
@@ -406,11 +406,12 @@ bool gemv_mfma_fits(int MT, int nb) {
 }
 
 // x_kind: MLLM_HIP_F32, MLLM_HIP_BF16 or GEMV_PREQ; MT: 4 or 8
-int launch_gemv_mfma(int wtype, int x_kind, int MT, const GemvArgs& a, int waves, hipStream_t st) {
-  if (waves != 0 && waves != 4 && waves != 8) return MLLM_HIP_E_BADARG;
+int launch_gemv_mfma(int wtype, int x_kind, int MT, const GemvArgs& a, int waves, int slices, hipStream_t st) {
+  if (waves != 0 && waves != 2 && waves != 4 && waves != 8) return MLLM_HIP_E_BADARG;
+  if (slices != 0 && slices != 1 && slices != 2 && slices != 4) return MLLM_HIP_E_BADARG;
 #define MF_CASE(WT_, XT_)                                                          \
   if (wtype == WT_ && x_kind == XT_)                                               \
-    return MT == 4 ? launch_mfma_t<WT_, XT_, 4>(a, waves, st) : launch_mfma_t<WT_, XT_, 8>(a, waves, st);
+    return MT == 4 ? launch_mfma_t<WT_, XT_, 4>(a, waves, slices, st) : launch_mfma_t<WT_, XT_, 8>(a, waves, slices, st);
   MF_CASE(MLLM_HIP_Q4_0, MLLM_HIP_F32)
   MF_CASE(MLLM_HIP_Q4_0, MLLM_HIP_BF16)
   MF_CASE(MLLM_HIP_Q4_0, GEMV_PREQ)
