@@ -581,6 +581,278 @@ static int launch_kq(const KGemvArgs& a, hipStream_t st) {
 }
 
 
+// ---- Q4_K, three to eight rows: sub-block sums on the matrix cores ---------------------------------------------------------
+// The dot4 kernel above needs the activation codes of every row from LDS for every weight unit and is bound by those reads
+// from three rows on (17 us per 9728 x 2560 projection at eight rows against 7 at one).  Here v_mfma_i32_16x16x64_i8 makes
+// the sums of one 32-element sub-block, as in the Q4_0 kernel of this kind (qgemv_mfma.hip): the instruction sums over
+// K = 64, and the sums of different sub-blocks are kept apart by the activation operand.  A 16-byte record of the nibble
+// plane holds 16 elements of sub-block 2c (low nibbles) and the same 16 of sub-block 2c+1 (high nibbles); lane group g of
+// the weight operand holds record 4j + g of the lane's weight row, so the low-nibble instruction sees sub-block 4j in
+// groups 0,1 and sub-block 4j+2 in groups 2,3 (the high-nibble instruction 4j+1 and 4j+3).  Output column 8 q + t gets the
+// codes of (that sub-block, activation row t) in groups 2q, 2q+1 and zeros in the other two: one instruction = the sums of
+// two sub-blocks for eight rows, every lane of the result useful.
+// Scaling per lane (four consecutive weight rows of one activation row):
+//   acc = fma(fp32(d*sc) * dx, float(isum), acc);  acc = fma(-(fp32(dmin*m) * dx), float(sum of the row's 32 codes), acc)
+// the reference's sum (vec_dot_q4_K_q8_K: integer sums per super-block, then d*dx and dmin*dx) regrouped; the integer parts
+// are exact, the fp32 roundings differ in order only.
+typedef int kv4i __attribute__((ext_vector_type(4)));
+constexpr int KMF_NG = 10;  // groups of four sub-blocks per trip
+
+static int kmf_slices(int nb32) {
+  int s = 1;
+  while (s < 8 && nb32 > 40 * s) s *= 2;
+  return s;
+}
+
+// blockDim = nwaves * 64; a workgroup holds nwaves / S row tiles (16 weight rows), S K-slices each; nbs = sub-blocks per slice
+// (a multiple of 8: whole super-blocks).
+// LDS: xc [nb32 + 40][MT] 32 bytes: the 32 codes of (sub-block, row); xs [nb32 + 40][MT] {dx, sum of the 32 codes};
+//      one zero record; ws per wave [whole trips][16 rows] fp32 d*sc, then the same of dmin*m; red per wave [64] four sums
+template <int XT, int MT>
+__global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, int nbs) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int TRIP = 4 * KMF_NG;
+  const int nsb = a.nsb, nb32 = nsb * 8, K = nsb * QK_K;
+  const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x, nwaves = nthreads >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int pidx = 0;
+#pragma unroll
+  for (int p = 1; p < KQ_MAX_PARTS; p++)
+    if (p < a.nparts && (int)blockIdx.x >= a.wg_start[p]) pidx = p;
+  const KGemvPart& pt = a.part[pidx];
+  const int N = pt.N;
+  const int tiles_wg = nwaves / S;
+  const int tile = ((int)blockIdx.x - a.wg_start[pidx]) * tiles_wg + wave / S;
+  const int slice = wave % S;
+  const int row0 = tile * 16;
+  const bool tile_ok = row0 < N;
+  const int b0 = slice * nbs, b1 = min(nb32, b0 + nbs);
+
+  const int wsb = (nbs + TRIP - 1) / TRIP * TRIP;
+  u32x4* xc = reinterpret_cast<u32x4*>(smem);                        // [(sb * MT + m) * 2 + half]
+  u32x4* zrec = xc + (size_t)(nb32 + TRIP) * MT * 2;
+  u32x2* xs = reinterpret_cast<u32x2*>(zrec + 1);                    // [sb * MT + m]
+  float* ws_all = reinterpret_cast<float*>(xs + (size_t)(nb32 + TRIP) * MT);
+  float* ws_ds = ws_all + (size_t)wave * 2 * wsb * 16;
+  float* ws_dm = ws_ds + (size_t)wsb * 16;
+  f32x4* red = reinterpret_cast<f32x4*>(ws_all + (size_t)nwaves * 2 * wsb * 16) + (size_t)wave * 64;
+
+  // ---- 1. weight scale records of the tile and slice: one 16-byte record per (row, super-block) --------------------------
+  const uint32_t sbt = (uint32_t)N * (uint32_t)nsb;
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.a), 0, sbt * 128u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.s), 0, sbt * 16u, 0x00020000);
+  const int spb = nbs >> 3;  // super-blocks per slice (at most 8)
+  u32x4 sc[2];
+#pragma unroll
+  for (int k = 0; k < 2; k++) {
+    const int ch = lane + 64 * k;
+    const int r = ch / spb, si = ch - r * spb;
+    const int sb256 = (b0 >> 3) + si;
+    const bool ok = tile_ok && r < 16 && row0 + r < N && sb256 < nsb;
+    sc[k] = __builtin_amdgcn_raw_buffer_load_b128(rsc, ok ? ((uint32_t)(row0 + r) * (uint32_t)nsb + (uint32_t)sb256) * 16u : KBUF_OOB, 0, KBUF_NT);
+  }
+  // ---- 2. weight codes: lane (row c, group g) takes records b0 + 4 j + g ------------------------------------------------------
+  const int c = lane & 15, g = lane >> 4;
+  const bool row_ok = tile_ok && row0 + c < N;
+  const uint32_t rbase = (uint32_t)(row0 + c) * (uint32_t)nb32;
+  u32x4 wq[KMF_NG];
+  auto load_groups = [&](int bb) {
+#pragma unroll
+    for (int j = 0; j < KMF_NG; j++) {
+      const int b = bb + 4 * j + g;
+      wq[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, (row_ok && b < b1) ? (rbase + (uint32_t)b) * 16u : KBUF_OOB, 0, KBUF_NT);
+    }
+  };
+  load_groups(b0);
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- 3. activations into LDS -------------------------------------------------------------------------------------------------
+  if (XT == KQ_IMAGE) {  // codes [MT][K], sums of 16 as int16 [MT][K/16], scales [MT][nsb]
+    const u32x4* codes = reinterpret_cast<const u32x4*>(a.x);
+    const uint32_t* pairs = reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(a.x) + (size_t)MT * K);
+    const float* dd = reinterpret_cast<const float*>(reinterpret_cast<const char*>(a.x) + (size_t)MT * K + (size_t)MT * nsb * 32);
+    for (int m = wave; m < MT; m += nwaves) {
+      for (int r = lane; r < 2 * nb32; r += 64) xc[((size_t)(r >> 1) * MT + m) * 2 + (r & 1)] = codes[(size_t)m * 2 * nb32 + r];
+      for (int sb = lane; sb < nb32; sb += 64) {
+        const uint32_t pr = pairs[(size_t)m * nb32 + sb];
+        const int bsum = (int)(int16_t)(pr & 0xffffu) + (int)(int16_t)(pr >> 16);
+        xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(dd[m * nsb + (sb >> 3)]), (uint32_t)bsum};
+      }
+    }
+  } else {
+    const int ipr = K >> 3;  // items (eight elements) per row; 32 consecutive items = one super-block
+    const int nitems = MT * ipr, valid = a.M * ipr;
+    const float inv_ipr = 1.0f / (float)ipr;
+    for (int it = tid; it < nitems; it += nthreads) {  // whole half-waves: nitems and nthreads are multiples of 32
+      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (it < valid) load8<XT == KQ_IMAGE ? MLLM_HIP_F32 : XT>(a.x, (int64_t)it * 8, v);
+      const Q8KItem qi = quantize_q8k_item(v, lane);
+      int s32 = qi.sum8 + __builtin_amdgcn_update_dpp(0, qi.sum8, 0xB1, 0xf, 0xf, true);
+      s32 += __builtin_amdgcn_update_dpp(0, s32, 0x4E, 0xf, 0xf, true);
+      const int m = (int)(((float)it + 0.5f) * inv_ipr), i = it - m * ipr;  // it / ipr: far from rounding trouble
+      const int sb = i >> 2, part = i & 3;                                   // sub-block, which 8 of its 32 codes
+      reinterpret_cast<u32x2*>(xc + ((size_t)sb * MT + m) * 2 + (part >> 1))[part & 1] = u32x2{qi.q0, qi.q1};
+      if (part == 0) xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(qi.d), (uint32_t)s32};
+    }
+  }
+  if (tid == 0) zrec[0] = u32x4{0u, 0u, 0u, 0u};
+  for (int i = tid; i < TRIP * MT * 2; i += nthreads) xc[(size_t)nb32 * MT * 2 + i] = u32x4{0u, 0u, 0u, 0u};
+  for (int i = tid; i < TRIP * MT; i += nthreads) xs[(size_t)nb32 * MT + i] = u32x2{0u, 0u};
+  // weight scales: fp32 d*sc and dmin*m per (sub-block of the slice, row); zero past the row and in the rest of the last trip
+#pragma unroll
+  for (int k = 0; k < 2; k++) {
+    const int ch = lane + 64 * k;
+    const int r = ch / spb, si = ch - r * spb;
+    if (r < 16) {
+      const bool in = (b0 >> 3) + si < nsb;
+      const float d = f16bits_to_f32((uint16_t)(sc[k].x & 0xffffu)), dmin = f16bits_to_f32((uint16_t)(sc[k].x >> 16));
+      const K4Scales ks = k4_scales(sc[k].y, sc[k].z, sc[k].w);
+#pragma unroll
+      for (int j = 0; j < 8; j++) {
+        ws_ds[(8 * si + j) * 16 + r] = in ? d * (float)byte_of(ks.sc0, ks.sc1, j) : 0.f;
+        ws_dm[(8 * si + j) * 16 + r] = in ? dmin * (float)byte_of(ks.mn0, ks.mn1, j) : 0.f;
+      }
+    }
+  }
+  for (int i = nbs * 16 + lane; i < wsb * 16; i += 64) {
+    ws_ds[i] = 0.f;
+    ws_dm[i] = 0.f;
+  }
+  __syncthreads();
+
+  // ---- 4. sub-block sums on the matrix cores, scaling on the vector ALU (software-pipelined over groups of four) --------------
+  const int q2 = (lane & 15) >> 3, t = lane & 7, tm = t & (MT - 1);
+  const bool mine = (g >> 1) == q2;  // the lane groups that supply this column's codes
+  const int half = g & 1;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int bb = b0; bb < b1; bb += TRIP) {
+    if (bb != b0) load_groups(bb);
+    const u32x4* bl = mine ? xc + ((size_t)(bb + 2 * q2) * MT + tm) * 2 + half : zrec;
+    const int bstep = mine ? 8 * MT : 0;  // four sub-blocks further per group
+    const u32x2* xsl = xs + (size_t)(bb + 2 * q2) * MT + tm;
+    const float* dsl = ws_ds + (bb - b0 + 2 * q2) * 16 + 4 * g;
+    const float* dml = ws_dm + (bb - b0 + 2 * q2) * 16 + 4 * g;
+    u32x4 Bl[2], Bh[2];
+    u32x2 sx[2][2];
+    f32x4 ds[2][2], dm[2][2];
+    kv4i D[2][2];
+    auto fetch_b = [&](int set, int j) {
+      Bl[set] = bl[j * bstep];
+      Bh[set] = bl[j * bstep + (mine ? 2 * MT : 0)];
+    };
+    auto fetch_s = [&](int set, int j) {
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        sx[set][h] = xsl[(4 * j + h) * MT];
+        ds[set][h] = *reinterpret_cast<const f32x4*>(dsl + (4 * j + h) * 16);
+        dm[set][h] = *reinterpret_cast<const f32x4*>(dml + (4 * j + h) * 16);
+      }
+    };
+    auto issue = [&](int set, int j) {
+      const u32x4 w = wq[j];
+      const kv4i Al = {(int)(w.x & 0x0f0f0f0fu), (int)(w.y & 0x0f0f0f0fu), (int)(w.z & 0x0f0f0f0fu), (int)(w.w & 0x0f0f0f0fu)};
+      const kv4i Ah = {(int)((w.x >> 4) & 0x0f0f0f0fu), (int)((w.y >> 4) & 0x0f0f0f0fu), (int)((w.z >> 4) & 0x0f0f0f0fu),
+                       (int)((w.w >> 4) & 0x0f0f0f0fu)};
+      D[set][0] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Al, __builtin_bit_cast(kv4i, Bl[set]), kv4i{0, 0, 0, 0}, 0, 0, 0);
+      D[set][1] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ah, __builtin_bit_cast(kv4i, Bh[set]), kv4i{0, 0, 0, 0}, 0, 0, 0);
+    };
+    auto scale = [&](int set, int j) {
+#pragma unroll
+      for (int h = 0; h < 2; h++) {
+        const bool live = bb + 4 * j + 2 * q2 + h < b1;
+        const float dx = live ? __uint_as_float(sx[set][h].x) : 0.f;
+        const float bs = (float)(int)sx[set][h].y;
+        acc.x = fmaf(ds[set][h].x * dx, (float)D[set][h].x, acc.x);
+        acc.y = fmaf(ds[set][h].y * dx, (float)D[set][h].y, acc.y);
+        acc.z = fmaf(ds[set][h].z * dx, (float)D[set][h].z, acc.z);
+        acc.w = fmaf(ds[set][h].w * dx, (float)D[set][h].w, acc.w);
+        acc.x = fmaf(-(dm[set][h].x * dx), bs, acc.x);
+        acc.y = fmaf(-(dm[set][h].y * dx), bs, acc.y);
+        acc.z = fmaf(-(dm[set][h].z * dx), bs, acc.z);
+        acc.w = fmaf(-(dm[set][h].w * dx), bs, acc.w);
+      }
+    };
+    fetch_b(0, 0);
+#pragma unroll
+    for (int j = 0; j < KMF_NG; j++) {
+      issue(j & 1, j);
+      if (j + 1 < KMF_NG) fetch_b((j + 1) & 1, j + 1);
+      fetch_s(j & 1, j);
+      __builtin_amdgcn_sched_barrier(0);
+      if (j > 0) scale((j - 1) & 1, j - 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    scale((KMF_NG - 1) & 1, KMF_NG - 1);
+  }
+  {  // the two lanes of an activation row (sub-blocks = 0,1 and 2,3 mod 4)
+    acc.x += __shfl_xor(acc.x, 8, 64);
+    acc.y += __shfl_xor(acc.y, 8, 64);
+    acc.z += __shfl_xor(acc.z, 8, 64);
+    acc.w += __shfl_xor(acc.w, 8, 64);
+  }
+
+  // ---- 5. slices of a tile in slice order, bias ------------------------------------------------------------------------------
+  if (S > 1) {
+    red[lane] = acc;
+    __syncthreads();
+    if (slice != 0) return;
+    for (int s = 1; s < S; s++) {
+      const f32x4 o = red[(size_t)s * 64 + lane];
+      acc.x += o.x; acc.y += o.y; acc.z += o.z; acc.w += o.w;
+    }
+  }
+  if (!tile_ok || q2 != 0 || t >= MT || t >= a.M) return;
+  const int n = row0 + 4 * g;
+  const float v[4] = {acc.x, acc.y, acc.z, acc.w};
+#pragma unroll
+  for (int e = 0; e < 4; e++)
+    if (n + e < N) pt.y[(int64_t)t * N + n + e] = pt.bias ? v[e] + pt.bias[n + e] : v[e];
+}
+
+template <int MT>
+static size_t kmf_lds_bytes(int nb32, int nbs, int nwaves) {
+  const int trip = 4 * KMF_NG;
+  const int wsb = (nbs + trip - 1) / trip * trip;
+  return (size_t)(nb32 + trip) * MT * 32 + 16 + (size_t)(nb32 + trip) * MT * 8 + (size_t)nwaves * 2 * wsb * 64 + (size_t)nwaves * 1024;
+}
+static bool kq4_mfma_fits(int MT, int nsb) {
+  const int nb32 = nsb * 8;
+  if (nb32 > 512) return false;  // scale records: at most 128 per wave
+  const int S = kmf_slices(nb32);
+  const int nbs = ((nb32 + S - 1) / S + 7) / 8 * 8;
+  return (MT == 4 ? kmf_lds_bytes<4>(nb32, nbs, 8) : kmf_lds_bytes<8>(nb32, nbs, 8)) <= 160 * 1024;
+}
+template <int XT, int MT>
+static int launch_kq4_mfma_t(const KGemvArgs& a_in, hipStream_t st) {
+  KGemvArgs a = a_in;
+  const int nb32 = a.nsb * 8;
+  const int S = kmf_slices(nb32);
+  const int nbs = ((nb32 + S - 1) / S + 7) / 8 * 8;
+  int nwaves = XT == KQ_IMAGE ? 4 : 8;
+  if (nwaves < S) nwaves = S;
+  const int tiles_wg = nwaves / S;
+  unsigned grid = 0;
+  for (int p = 0; p < a.nparts; p++) {
+    a.wg_start[p] = (int)grid;
+    grid += (unsigned)(((a.part[p].N + 15) / 16 + tiles_wg - 1) / tiles_wg);
+  }
+  a.wg_start[a.nparts] = (int)grid;
+  const size_t lds = kmf_lds_bytes<MT>(nb32, nbs, nwaves);
+  if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
+  auto kern = kq4_gemv_mfma_kernel<XT, MT>;
+  if (lds > 64 * 1024)
+    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(nwaves * 64), lds, st, a, S, nbs);
+  return (int)hipGetLastError();
+}
+template <int XT>
+static int launch_kq4_mfma(const KGemvArgs& a, hipStream_t st) {
+  return a.M <= 4 ? launch_kq4_mfma_t<XT, 4>(a, st) : launch_kq4_mfma_t<XT, 8>(a, st);
+}
+static int g_kq_path = 0;  // 1: always the dot4 kernel (comparison runs and tests)
+
+
 // ---- many rows: the matrix-core GEMM of the block formats (moe.hip, qg_kernel) with these weights -------------------------
 // Same scheme as for Q4_0 / Q8_0: both operands as fp16 with their scales folded in, fp32 accumulation in
 // v_mfma_f32_32x32x16_f16.  Activations: the Q8_K round trip xh = fp16(d * q) (codes and d bit-exact, the product rounded
@@ -693,6 +965,11 @@ static int kq_check(int wtype, const void* packed, int64_t N, int64_t K) {
   return 0;
 }
 
+MLLM_API int mllm_hip_kq_set_path(int path) {
+  if (path != 0 && path != 1) return MLLM_HIP_E_BADARG;
+  g_kq_path = path;
+  return 0;
+}
 MLLM_API int mllm_hip_kq_set_tuning(int lanes_per_row, int waves_per_wg, int units_in_flight) {
   auto ok = [](int v, std::initializer_list<int> allowed) {
     for (int x : allowed)
@@ -769,6 +1046,7 @@ MLLM_API int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv
     a.x = xg;
     a.M = rows;
     a.nsb = nsb;
+    const bool mfma = wtype == MLLM_HIP_Q4_K && rows >= 3 && g_kq_path != 1 && kq4_mfma_fits(rows <= 4 ? 4 : 8, nsb);
     if (workspace && rows >= 3) {
       // several rows: quantize once for all workgroups; the GEMV then copies the image instead of quantizing
       const int MT = rows <= 4 ? 4 : 8;
@@ -778,7 +1056,10 @@ MLLM_API int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv
                          reinterpret_cast<float*>(img + (size_t)MT * K + (size_t)MT * nsb * 32),
                          reinterpret_cast<int16_t*>(img + (size_t)MT * K), nitems, (int64_t)rows * K / 8);
       a.x = img;
-      rc = wtype == MLLM_HIP_Q4_K ? launch_kq<MLLM_HIP_Q4_K, KQ_IMAGE>(a, st) : launch_kq<MLLM_HIP_Q6_K, KQ_IMAGE>(a, st);
+      if (mfma) rc = launch_kq4_mfma<KQ_IMAGE>(a, st);
+      else rc = wtype == MLLM_HIP_Q4_K ? launch_kq<MLLM_HIP_Q4_K, KQ_IMAGE>(a, st) : launch_kq<MLLM_HIP_Q6_K, KQ_IMAGE>(a, st);
+    } else if (mfma) {
+      rc = x_dtype == MLLM_HIP_F32 ? launch_kq4_mfma<MLLM_HIP_F32>(a, st) : launch_kq4_mfma<MLLM_HIP_BF16>(a, st);
     } else if (wtype == MLLM_HIP_Q4_K) {
       rc = x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_F32>(a, st) : launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_BF16>(a, st);
     } else {
