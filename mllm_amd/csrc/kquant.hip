@@ -850,7 +850,299 @@ template <int XT>
 static int launch_kq4_mfma(const KGemvArgs& a, hipStream_t st) {
   return a.M <= 4 ? launch_kq4_mfma_t<XT, 4>(a, st) : launch_kq4_mfma_t<XT, 8>(a, st);
 }
-static int g_kq_path = 0;  // 1: always the dot4 kernel (comparison runs and tests)
+// ---- Q6_K, three to eight rows: the same on 16-element units -------------------------------------------------------------------
+// Q6_K scales 16 elements at a time, which is exactly what one lane supplies to the K = 64 instruction: lane group g of the
+// weight operand holds one 16-element unit, and output column 4 q + t gets the codes of (unit q of the four, activation row
+// t) in lane group q and zeros elsewhere: one instruction = the sums of four units for four rows.  A 16-byte record of the
+// low-nibble plane serves two units (low and high nibbles) with the matching 16 bytes of the bit-pair plane; the codes stay
+// unsigned (0..63) and the offset of 32 goes into the sum as -32 * (sum of the unit's 16 activation codes), which the Q8_K
+// quantization delivers anyway.  Scaling per lane: acc = fma(fp32(d * sc) * dx, float(isum - 32 * bsum), acc).
+// Step st of a trip = half a super-block (records 4 (st & 1) + g of super-block st / 2): low nibbles are units 8 (st & 1) + g,
+// high nibbles units 8 (st & 1) + 4 + g.
+constexpr int K6_ST = 10;  // steps per trip: five super-blocks
+template <int XT, int MT>
+__global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, int sps) {  // sps = super-blocks per slice
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int TH = MT / 4;
+  constexpr int TSB = K6_ST / 2;  // super-blocks per trip
+  const int nsb = a.nsb, nu = nsb * 16, K = nsb * QK_K;
+  const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x, nwaves = nthreads >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int pidx = 0;
+#pragma unroll
+  for (int p = 1; p < KQ_MAX_PARTS; p++)
+    if (p < a.nparts && (int)blockIdx.x >= a.wg_start[p]) pidx = p;
+  const KGemvPart& pt = a.part[pidx];
+  const int N = pt.N;
+  const int tiles_wg = nwaves / S;
+  const int tile = ((int)blockIdx.x - a.wg_start[pidx]) * tiles_wg + wave / S;
+  const int slice = wave % S;
+  const int row0 = tile * 16;
+  const bool tile_ok = row0 < N;
+  const int s0 = slice * sps, s1 = min(nsb, s0 + sps);  // this wave's super-blocks
+
+  const int wsu = (sps + TSB - 1) / TSB * TSB * 16;  // units of weight scales per wave: whole trips
+  u32x4* xc = reinterpret_cast<u32x4*>(smem);                     // [unit * MT + m] the unit's 16 codes
+  u32x4* zrec = xc + (size_t)(nu + TSB * 16) * MT;
+  int* bs16 = reinterpret_cast<int*>(zrec + 1);                   // [unit * MT + m] sum of the unit's codes
+  float* dxs = reinterpret_cast<float*>(bs16 + (size_t)(nu + TSB * 16) * MT);  // [super-block * MT + m]
+  float* ws_all = dxs + (size_t)(nsb + TSB) * MT;
+  float* ws = ws_all + (size_t)wave * wsu * 16;
+  f32x4* red = reinterpret_cast<f32x4*>(smem) + (size_t)wave * TH * 64;  // takes the place of the codes once every wave is done with them
+
+  const uint32_t sbt = (uint32_t)N * (uint32_t)nsb;
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.a), 0, sbt * 128u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.h), 0, sbt * 64u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.s), 0, sbt * 16u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(pt.w.d), 0, sbt * 2u, 0x00020000);
+  // ---- 1. weight scales of the tile and slice: 16 int8 and one fp16 per (row, super-block) -------------------------------------
+  u32x4 sc[2];
+  uint16_t scd[2];
+#pragma unroll
+  for (int k = 0; k < 2; k++) {
+    const int ch = lane + 64 * k;
+    const int r = ch / sps, si = ch - r * sps;
+    const bool ok = tile_ok && r < 16 && row0 + r < N && s0 + si < nsb;
+    const uint32_t idx = (uint32_t)(row0 + r) * (uint32_t)nsb + (uint32_t)(s0 + si);
+    sc[k] = __builtin_amdgcn_raw_buffer_load_b128(rsc, ok ? idx * 16u : KBUF_OOB, 0, KBUF_NT);
+    scd[k] = __builtin_amdgcn_raw_buffer_load_b16(rd, ok ? idx * 2u : KBUF_OOB, 0, KBUF_NT);
+  }
+  // ---- 2. weight codes: lane (row c, group g), step st: low-nibble record 4 (st & 1) + g and bit-pair record 2 (st & 1) + (g & 1)
+  const int c = lane & 15, g = lane >> 4;
+  const bool row_ok = tile_ok && row0 + c < N;
+  const uint32_t rbase = (uint32_t)(row0 + c) * (uint32_t)nsb;
+  u32x4 wl[K6_ST], wh[K6_ST];
+  auto load_steps = [&](int sb0) {
+#pragma unroll
+    for (int st = 0; st < K6_ST; st++) {
+      const int sb = sb0 + (st >> 1);
+      const bool ok = row_ok && sb < s1;
+      wl[st] = __builtin_amdgcn_raw_buffer_load_b128(ra, ok ? ((rbase + (uint32_t)sb) * 8u + 4u * (st & 1) + (uint32_t)g) * 16u : KBUF_OOB, 0, KBUF_NT);
+      wh[st] = __builtin_amdgcn_raw_buffer_load_b128(rh, ok ? ((rbase + (uint32_t)sb) * 4u + 2u * (st & 1) + (uint32_t)(g & 1)) * 16u : KBUF_OOB, 0, KBUF_NT);
+    }
+  };
+  load_steps(s0);
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- 3. activations into LDS -------------------------------------------------------------------------------------------------
+  if (XT == KQ_IMAGE) {  // codes [MT][K], sums of 16 as int16 [MT][K/16], scales [MT][nsb]
+    const u32x4* codes = reinterpret_cast<const u32x4*>(a.x);
+    const int16_t* sums = reinterpret_cast<const int16_t*>(reinterpret_cast<const char*>(a.x) + (size_t)MT * K);
+    const float* dd = reinterpret_cast<const float*>(reinterpret_cast<const char*>(a.x) + (size_t)MT * K + (size_t)MT * nsb * 32);
+    for (int m = wave; m < MT; m += nwaves) {
+      for (int u = lane; u < nu; u += 64) {
+        xc[(size_t)u * MT + m] = codes[(size_t)m * nu + u];
+        bs16[(size_t)u * MT + m] = (int)sums[(size_t)m * nu + u];
+      }
+      for (int sb = lane; sb < nsb; sb += 64) dxs[sb * MT + m] = dd[m * nsb + sb];
+    }
+  } else {
+    const int ipr = K >> 3;
+    const int nitems = MT * ipr, valid = a.M * ipr;
+    const float inv_ipr = 1.0f / (float)ipr;
+    for (int it = tid; it < nitems; it += nthreads) {  // whole half-waves
+      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+      if (it < valid) load8<XT == KQ_IMAGE ? MLLM_HIP_F32 : XT>(a.x, (int64_t)it * 8, v);
+      const Q8KItem qi = quantize_q8k_item(v, lane);
+      const int s16 = qi.sum8 + __builtin_amdgcn_update_dpp(0, qi.sum8, 0xB1, 0xf, 0xf, true);
+      const int m = (int)(((float)it + 0.5f) * inv_ipr), i = it - m * ipr;
+      const int u = i >> 1;
+      reinterpret_cast<u32x2*>(xc + (size_t)u * MT + m)[i & 1] = u32x2{qi.q0, qi.q1};
+      if ((i & 1) == 0) bs16[(size_t)u * MT + m] = s16;
+      if ((i & 31) == 0) dxs[(i >> 5) * MT + m] = qi.d;
+    }
+  }
+  if (tid == 0) zrec[0] = u32x4{0u, 0u, 0u, 0u};
+  for (int i = tid; i < TSB * 16 * MT; i += nthreads) {
+    xc[(size_t)nu * MT + i] = u32x4{0u, 0u, 0u, 0u};
+    bs16[(size_t)nu * MT + i] = 0;
+  }
+  for (int i = tid; i < TSB * MT; i += nthreads) dxs[nsb * MT + i] = 0.f;
+#pragma unroll
+  for (int k = 0; k < 2; k++) {
+    const int ch = lane + 64 * k;
+    const int r = ch / sps, si = ch - r * sps;
+    if (r < 16) {
+      const float d = (s0 + si < nsb) ? f16bits_to_f32(scd[k]) : 0.f;
+      const uint32_t wds[4] = {sc[k].x, sc[k].y, sc[k].z, sc[k].w};
+#pragma unroll
+      for (int j = 0; j < 16; j++) ws[(16 * si + j) * 16 + r] = d * (float)(int8_t)(wds[j >> 2] >> (8 * (j & 3)));
+    }
+  }
+  for (int i = sps * 256 + lane; i < wsu * 16; i += 64) ws[i] = 0.f;
+  __syncthreads();
+
+  // ---- 4. unit sums on the matrix cores, scaling on the vector ALU ----------------------------------------------------------------
+  const int q = (lane & 15) >> 2, tt = lane & 3;
+  const bool mine = g == q;
+  const int shl = 2 * (g >> 1);  // this lane's low-nibble units take bit pair g / 2 of the high plane, its high-nibble units g / 2 + 2
+  f32x4 acc[TH];
+#pragma unroll
+  for (int h = 0; h < TH; h++) acc[h] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int sb0 = s0; sb0 < s1; sb0 += TSB) {
+    if (sb0 != s0) load_steps(sb0);
+    const int u0 = sb0 * 16;
+    const u32x4* bl[TH];
+    const int* bsl[TH];
+    const float* dxl[TH];
+#pragma unroll
+    for (int h = 0; h < TH; h++) {
+      bl[h] = mine ? xc + (size_t)(u0 + q) * MT + 4 * h + tt : zrec;
+      bsl[h] = bs16 + (size_t)(u0 + q) * MT + 4 * h + tt;
+      dxl[h] = dxs + sb0 * MT + 4 * h + tt;
+    }
+    const int bstep = mine ? MT : 0;
+    const float* wsl = ws + (size_t)(u0 - s0 * 16 + q) * 16 + 4 * g;
+    u32x4 B[2][2][TH];
+    int bs[2][2][TH];
+    float dxv[2][TH];
+    f32x4 dsv[2][2];
+    kv4i D[2][2][TH];
+    auto fetch_b = [&](int set, int st) {  // units 8 st + q (low nibbles) and 8 st + 4 + q (high)
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        B[set][0][h] = bl[h][(8 * st) * bstep];
+        B[set][1][h] = bl[h][(8 * st + 4) * bstep];
+      }
+    };
+    auto fetch_s = [&](int set, int st) {
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        bs[set][0][h] = bsl[h][(8 * st) * MT];
+        bs[set][1][h] = bsl[h][(8 * st + 4) * MT];
+        dxv[set][h] = dxl[h][(st >> 1) * MT];
+      }
+      dsv[set][0] = *reinterpret_cast<const f32x4*>(wsl + (8 * st) * 16);
+      dsv[set][1] = *reinterpret_cast<const f32x4*>(wsl + (8 * st + 4) * 16);
+    };
+    auto issue = [&](int set, int st) {
+      const uint32_t l4[4] = {wl[st].x, wl[st].y, wl[st].z, wl[st].w};
+      const uint32_t h4[4] = {wh[st].x, wh[st].y, wh[st].z, wh[st].w};
+      kv4i Alo, Ahi;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const uint32_t hs = h4[e] >> shl;
+        Alo[e] = (int)((l4[e] & 0x0f0f0f0fu) | ((hs & 0x03030303u) << 4));
+        Ahi[e] = (int)(((l4[e] >> 4) & 0x0f0f0f0fu) | (((hs >> 4) & 0x03030303u) << 4));
+      }
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        D[set][0][h] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Alo, __builtin_bit_cast(kv4i, B[set][0][h]), kv4i{0, 0, 0, 0}, 0, 0, 0);
+        D[set][1][h] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ahi, __builtin_bit_cast(kv4i, B[set][1][h]), kv4i{0, 0, 0, 0}, 0, 0, 0);
+      }
+    };
+    auto scale = [&](int set, int st) {
+      const bool live = sb0 + (st >> 1) < s1;  // uniform
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        const float dx = live ? dxv[set][h] : 0.f;
+#pragma unroll
+        for (int w = 0; w < 2; w++) {
+          const int corr = -32 * bs[set][w][h];  // the codes went in as 0..63
+          acc[h].x = fmaf(dsv[set][w].x * dx, (float)(D[set][w][h].x + corr), acc[h].x);
+          acc[h].y = fmaf(dsv[set][w].y * dx, (float)(D[set][w][h].y + corr), acc[h].y);
+          acc[h].z = fmaf(dsv[set][w].z * dx, (float)(D[set][w][h].z + corr), acc[h].z);
+          acc[h].w = fmaf(dsv[set][w].w * dx, (float)(D[set][w][h].w + corr), acc[h].w);
+        }
+      }
+    };
+    fetch_b(0, 0);
+#pragma unroll
+    for (int st = 0; st < K6_ST; st++) {
+      issue(st & 1, st);
+      if (st + 1 < K6_ST) fetch_b((st + 1) & 1, st + 1);
+      fetch_s(st & 1, st);
+      __builtin_amdgcn_sched_barrier(0);
+      if (st > 0) scale((st - 1) & 1, st - 1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    scale((K6_ST - 1) & 1, K6_ST - 1);
+  }
+#pragma unroll
+  for (int h = 0; h < TH; h++) {  // the four lanes of an activation row (units = 0..3 mod 4)
+    float v[4] = {acc[h].x, acc[h].y, acc[h].z, acc[h].w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      v[e] += __shfl_xor(v[e], 4, 64);
+      v[e] += __shfl_xor(v[e], 8, 64);
+    }
+    acc[h] = f32x4{v[0], v[1], v[2], v[3]};
+  }
+
+  // ---- 5. slices of a tile in slice order, bias ------------------------------------------------------------------------------
+  if (S > 1) {
+    __syncthreads();
+#pragma unroll
+    for (int h = 0; h < TH; h++) red[h * 64 + lane] = acc[h];
+    __syncthreads();
+    if (slice != 0) return;
+    for (int s = 1; s < S; s++)
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        const f32x4 o = red[(size_t)s * TH * 64 + h * 64 + lane];
+        acc[h].x += o.x; acc[h].y += o.y; acc[h].z += o.z; acc[h].w += o.w;
+      }
+  }
+  if (!tile_ok || q != 0) return;
+  const int n = row0 + 4 * g;
+#pragma unroll
+  for (int h = 0; h < TH; h++) {
+    const int t = 4 * h + tt;
+    if (t >= a.M) continue;
+    const float v[4] = {acc[h].x, acc[h].y, acc[h].z, acc[h].w};
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      if (n + e < N) pt.y[(int64_t)t * N + n + e] = pt.bias ? v[e] + pt.bias[n + e] : v[e];
+  }
+}
+
+template <int MT>
+static size_t k6mf_lds_bytes(int nsb, int sps, int nwaves) {
+  const int tsb = K6_ST / 2;
+  const int wsu = (sps + tsb - 1) / tsb * tsb * 16;
+  return (size_t)(nsb * 16 + tsb * 16) * MT * 16 + 16 + (size_t)(nsb * 16 + tsb * 16) * MT * 4 + (size_t)(nsb + tsb) * MT * 4 +
+         (size_t)nwaves * wsu * 64;  // the partial sums of the slices reuse the code area
+}
+static void k6mf_split(int nsb, int& S, int& sps) {
+  S = 1;
+  while (S < 8 && nsb > 5 * S) S *= 2;
+  sps = (nsb + S - 1) / S;
+}
+static bool kq6_mfma_fits(int MT, int nsb) {
+  int S, sps;
+  k6mf_split(nsb, S, sps);
+  if (sps > 8) return false;  // scale records: at most 128 per wave
+  return (MT == 4 ? k6mf_lds_bytes<4>(nsb, sps, 8) : k6mf_lds_bytes<8>(nsb, sps, 8)) <= 160 * 1024;
+}
+template <int XT, int MT>
+static int launch_kq6_mfma_t(const KGemvArgs& a_in, hipStream_t st) {
+  KGemvArgs a = a_in;
+  int S, sps;
+  k6mf_split(a.nsb, S, sps);
+  int nwaves = XT == KQ_IMAGE ? 4 : 8;
+  if (nwaves < S) nwaves = S;
+  const int tiles_wg = nwaves / S;
+  unsigned grid = 0;
+  for (int p = 0; p < a.nparts; p++) {
+    a.wg_start[p] = (int)grid;
+    grid += (unsigned)(((a.part[p].N + 15) / 16 + tiles_wg - 1) / tiles_wg);
+  }
+  a.wg_start[a.nparts] = (int)grid;
+  const size_t lds = k6mf_lds_bytes<MT>(a.nsb, sps, nwaves);
+  if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
+  auto kern = kq6_gemv_mfma_kernel<XT, MT>;
+  if (lds > 64 * 1024)
+    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(nwaves * 64), lds, st, a, S, sps);
+  return (int)hipGetLastError();
+}
+template <int XT>
+static int launch_kq6_mfma(const KGemvArgs& a, hipStream_t st) {
+  return a.M <= 4 ? launch_kq6_mfma_t<XT, 4>(a, st) : launch_kq6_mfma_t<XT, 8>(a, st);
+}
+
+static int g_kq_path = 0;  // 1: always the dot4 kernel, 2: the matrix-core kernels wherever they fit (comparison runs and tests)
 
 
 // ---- many rows: the matrix-core GEMM of the block formats (moe.hip, qg_kernel) with these weights -------------------------
@@ -966,7 +1258,7 @@ static int kq_check(int wtype, const void* packed, int64_t N, int64_t K) {
 }
 
 MLLM_API int mllm_hip_kq_set_path(int path) {
-  if (path != 0 && path != 1) return MLLM_HIP_E_BADARG;
+  if (path != 0 && path != 1 && path != 2) return MLLM_HIP_E_BADARG;
   g_kq_path = path;
   return 0;
 }
@@ -1046,7 +1338,12 @@ MLLM_API int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv
     a.x = xg;
     a.M = rows;
     a.nsb = nsb;
-    const bool mfma = wtype == MLLM_HIP_Q4_K && rows >= 3 && g_kq_path != 1 && kq4_mfma_fits(rows <= 4 ? 4 : 8, nsb);
+    // Q4_K: from three rows on.  Q6_K (heavier unpacking, 200 registers): measured faster only with five to eight rows of more
+    // than 4096 elements (down projection 9728: 37.6 -> 20.7 us at eight rows; a 2560-element row ties, q and o lose).
+    // The rule looks at the weight type, the number of rows and the row length only.
+    const bool mfma = rows >= 3 && g_kq_path != 1 &&
+                      (wtype == MLLM_HIP_Q4_K ? kq4_mfma_fits(rows <= 4 ? 4 : 8, nsb)
+                                              : ((rows > 4 && nsb > 16) || g_kq_path == 2) && kq6_mfma_fits(rows <= 4 ? 4 : 8, nsb));
     if (workspace && rows >= 3) {
       // several rows: quantize once for all workgroups; the GEMV then copies the image instead of quantizing
       const int MT = rows <= 4 ? 4 : 8;
@@ -1056,10 +1353,12 @@ MLLM_API int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv
                          reinterpret_cast<float*>(img + (size_t)MT * K + (size_t)MT * nsb * 32),
                          reinterpret_cast<int16_t*>(img + (size_t)MT * K), nitems, (int64_t)rows * K / 8);
       a.x = img;
-      if (mfma) rc = launch_kq4_mfma<KQ_IMAGE>(a, st);
+      if (mfma) rc = wtype == MLLM_HIP_Q4_K ? launch_kq4_mfma<KQ_IMAGE>(a, st) : launch_kq6_mfma<KQ_IMAGE>(a, st);
       else rc = wtype == MLLM_HIP_Q4_K ? launch_kq<MLLM_HIP_Q4_K, KQ_IMAGE>(a, st) : launch_kq<MLLM_HIP_Q6_K, KQ_IMAGE>(a, st);
-    } else if (mfma) {
+    } else if (mfma && wtype == MLLM_HIP_Q4_K) {
       rc = x_dtype == MLLM_HIP_F32 ? launch_kq4_mfma<MLLM_HIP_F32>(a, st) : launch_kq4_mfma<MLLM_HIP_BF16>(a, st);
+    } else if (mfma) {
+      rc = x_dtype == MLLM_HIP_F32 ? launch_kq6_mfma<MLLM_HIP_F32>(a, st) : launch_kq6_mfma<MLLM_HIP_BF16>(a, st);
     } else if (wtype == MLLM_HIP_Q4_K) {
       rc = x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_F32>(a, st) : launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_BF16>(a, st);
     } else {

@@ -168,29 +168,34 @@ def test_linear_kq_gemm_exact_cases(wtype):
     assert np.array_equal(y.astype(np.float64), want)
 
 
+@pytest.mark.parametrize("wtype", [2, 3])
 @pytest.mark.parametrize("M", [3, 4, 5, 8, 11])
-def test_q4_K_matrix_core_and_dot4_kernels_agree(M):
-    """three to eight rows of Q4_K: the matrix-core kernel (default) and the dot4 kernel are independent implementations of the
-    same arithmetic (exact integer sums, fp32 scaling in another order)"""
-    rng = synth.rng_for(7, 900 + M)
+def test_matrix_core_and_dot4_kernels_agree(wtype, M):
+    """three to eight rows: the matrix-core kernels (default) and the dot4 kernel are independent implementations of the same
+    arithmetic (exact integer sums, fp32 scaling in another order)"""
+    rng = synth.rng_for(7, 900 + M + 100 * wtype)
     L = _lib.lib()
     for N, K in ((9728, 2560), (2560, 9728), (77, 768), (130, 4096 + 256), (33, 256)):
-        W = synth.make_weight(rng, 2, N, K)
-        w = ql.PackedKWeight(2, torch.from_numpy(W))
+        W = synth.make_weight(rng, wtype, N, K)
+        w = ql.PackedKWeight(wtype, torch.from_numpy(W))
         bias = to_dev(rng.standard_normal(N).astype(np.float32))
         xf = synth.make_x_fp32(rng, M, K)
         xd = to_dev(xf)
-        announce("q4_K both kernels", M, N, K)
-        y0 = ql.linear_kq(w, xd, bias)
-        assert torch.equal(y0, ql.linear_kq(w, xd, bias, workspace=ql.kq_workspace(M, K)))
-        assert L.mllm_hip_kq_set_path(1) == 0
+        announce("kq both kernels", wtype, M, N, K)
+        assert L.mllm_hip_kq_set_path(2) == 0  # the matrix-core kernel also where the default keeps the dot4 kernel
         try:
+            y0 = ql.linear_kq(w, xd, bias)
+            assert torch.equal(y0, ql.linear_kq(w, xd, bias, workspace=ql.kq_workspace(M, K)))
+            assert L.mllm_hip_kq_set_path(1) == 0
             y1 = ql.linear_kq(w, xd, bias)
         finally:
             assert L.mllm_hip_kq_set_path(0) == 0
+        yd = ql.linear_kq(w, xd, bias)  # whatever the default picks per group of eight rows: one of the two, bit for bit
+        for lo in range(0, M, 8):
+            assert torch.equal(yd[lo:lo + 8], y0[lo:lo + 8]) or torch.equal(yd[lo:lo + 8], y1[lo:lo + 8])
         assert rel_l2(y0.cpu().numpy(), y1.cpu().numpy()) < 2e-6
-        assert rel_l2(y0.cpu().numpy(), orc.linear_kq(xf, W, 2, bias.cpu().numpy(), orc.SCALE_X86_REF)) < 2e-6
-    assert L.mllm_hip_kq_set_path(2) == -1
+        assert rel_l2(y0.cpu().numpy(), orc.linear_kq(xf, W, wtype, bias.cpu().numpy(), orc.SCALE_X86_REF)) < 2e-6
+    assert L.mllm_hip_kq_set_path(3) == -1
 
 
 def test_argument_checks():
