@@ -329,6 +329,7 @@ def main():
              for n, d in (("h", 2560), ("q", 4096), ("k", 1024), ("v", 1024), ("o", 2560), ("x1", 2560), ("h2", 2560),
                           ("g", 9728), ("u", 9728), ("s", 9728), ("a", 9728), ("d", 2560), ("x2", 2560))}
         img = {k: ql.gemv_workspace(M, k) for k in (2560, 9728)}
+        ws_o = ql.gemv_workspace(M, 4096)  # o_proj reads the attention output raw: quantized once per launch from three rows on
         L = _lib.lib()
 
         def ew(fn, a_, b_, y_):
@@ -358,7 +359,7 @@ def main():
                 _lib.check(L.mllm_hip_rmsnorm(x.data_ptr(), 0, nw[0].data_ptr(), b["h"].data_ptr(), M, 2560, 1e-6, 0,
                                               img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
                 ql.linear_q_gemv_fused([l["q_proj"], l["k_proj"], l["v_proj"]], img[2560], M=M, image=True, outs=[b["q"], b["k"], b["v"]])
-                ql.linear_q_gemv_fused([l["o_proj"]], attn, residuals=[x], outs=[b["x1"]])
+                ql.linear_q_gemv_fused([l["o_proj"]], attn, residuals=[x], outs=[b["x1"]], workspace=ws_o)
                 _lib.check(L.mllm_hip_rmsnorm(b["x1"].data_ptr(), 0, nw[1].data_ptr(), b["h2"].data_ptr(), M, 2560, 1e-6, 0,
                                               img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
                 ql.linear_q_gemv_fused([l["gate_proj"], l["up_proj"]], img[2560], M=M, image=True, outs=[b["g"], b["u"]])
@@ -374,7 +375,7 @@ def main():
                 _lib.check(L.mllm_hip_rmsnorm(x.data_ptr(), 0, nw[0].data_ptr(), b["h"].data_ptr(), M, 2560, 1e-6, 0,
                                               img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
                 ql.linear_q_gemv_fused([l["q_proj"], l["k_proj"], l["v_proj"]], img[2560], M=M, image=True, outs=[b["q"], b["k"], b["v"]])
-                ql.linear_q_gemv_fused([l["o_proj"]], attn, residuals=[x], outs=[b["x1"]])
+                ql.linear_q_gemv_fused([l["o_proj"]], attn, residuals=[x], outs=[b["x1"]], workspace=ws_o)
                 _lib.check(L.mllm_hip_rmsnorm(b["x1"].data_ptr(), 0, nw[1].data_ptr(), b["h2"].data_ptr(), M, 2560, 1e-6, 0,
                                               img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
                 _lib.check(L.mllm_hip_mlp_gate_up_q(l["gate_proj"].wtype, l["gate_proj"].ptr, l["up_proj"].ptr, img[2560].data_ptr(),

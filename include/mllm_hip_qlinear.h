@@ -102,6 +102,8 @@ int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_hip_gemv_p
  * workgroup quantizes. */
 typedef struct {
   const float* const* residual;
+  void* workspace; /* NULL, or mllm_hip_gemv_workspace_bytes(M, K) bytes for raw activations: as in
+                      mllm_hip_linear_q_gemv_multi_ws (same results bit for bit) */
 } mllm_hip_gemv_fusion;
 int mllm_hip_linear_q_gemv_fused(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fusion,
                                  const void* x, int x_kind, int M, int64_t K, int act_scale_mode, void* stream);

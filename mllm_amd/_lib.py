@@ -18,7 +18,7 @@ class GemvPart(C.Structure):
 
 class GemvFusion(C.Structure):
     """mllm_hip_gemv_fusion"""
-    _fields_ = [("residual", C.POINTER(C.c_void_p))]
+    _fields_ = [("residual", C.POINTER(C.c_void_p)), ("workspace", C.c_void_p)]
 
 
 class HipQLinearError(RuntimeError):

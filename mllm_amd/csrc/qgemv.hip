@@ -413,7 +413,7 @@ MLLM_API int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_h
 
 MLLM_API int mllm_hip_linear_q_gemv_fused(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fusion,
                                           const void* x, int x_kind, int M, int64_t K, int act_scale_mode, void* stream) {
-  return gemv_multi_impl(wtype, nparts, parts, fusion, x, x_kind, M, K, act_scale_mode, nullptr, stream);
+  return gemv_multi_impl(wtype, nparts, parts, fusion, x, x_kind, M, K, act_scale_mode, fusion ? fusion->workspace : nullptr, stream);
 }
 
 MLLM_API int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,

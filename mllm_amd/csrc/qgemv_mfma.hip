@@ -375,7 +375,8 @@ static int mf_slices(int nb) {
 template <int WT, int XT, int MT>
 static int launch_mfma_t(const GemvArgs& a_in, int waves, int slices, hipStream_t st) {
   GemvArgs a = a_in;
-  const int S = slices ? slices : mf_slices(a.nb);
+  int S = slices ? slices : mf_slices(a.nb);
+  if (((a.nb + S - 1) / S + 7) / 8 * 8 > 64) S = mf_slices(a.nb);  // an override that leaves slices too long for the scale staging
   const int nbs = ((a.nb + S - 1) / S + 7) / 8 * 8;
   int nwaves = waves ? waves : (XT == GEMV_PREQ ? 4 : 8);
   if (nwaves < S) nwaves = S;

@@ -116,7 +116,8 @@ def linear_q_gemv_multi(ws, x, biases=None, act_scale_mode=SCALE_X86_REF, outs=N
 Q8_IMAGE = 2  # MLLM_HIP_Q8_IMAGE
 
 
-def linear_q_gemv_fused(ws, x, M=None, biases=None, residuals=None, act_scale_mode=SCALE_X86_REF, outs=None, image=False):
+def linear_q_gemv_fused(ws, x, M=None, biases=None, residuals=None, act_scale_mode=SCALE_X86_REF, outs=None, image=False,
+                        workspace=None):
     """The decode GEMV with its neighbours folded in: residuals[i] (fp32 [M, N], may be outs[i]) is added to part i;
     with image=True `x` is the Q8_0 image a producer (rmsnorm / silu_mul with want_image) wrote for M rows."""
     assert 1 <= len(ws) <= 4 and x.is_cuda and x.is_contiguous()
@@ -137,7 +138,7 @@ def linear_q_gemv_fused(ws, x, M=None, biases=None, residuals=None, act_scale_mo
         if r is not None:
             assert r.dtype == torch.float32 and r.is_contiguous() and tuple(r.shape) == (M, w.N)
         res[i] = r.data_ptr() if r is not None else None
-    fu = _lib.GemvFusion(res if residuals is not None else None)
+    fu = _lib.GemvFusion(res if residuals is not None else None, _p(workspace))
     _lib.check(_lib.lib().mllm_hip_linear_q_gemv_fused(ws[0].wtype, len(ws), parts, C.byref(fu), x.data_ptr(),
                                                        Q8_IMAGE if image else _xdtype(x), M, K, act_scale_mode, _stream()),
                "mllm_hip_linear_q_gemv_fused")

@@ -133,9 +133,11 @@ def test_gemv_ragged(N, K, M):
 
 
 def test_gemv_every_launch_shape():
+    """the dot4 kernel in every launch shape it is compiled for (with three rows or more it is the comparison path: path 1)"""
     rng = synth.rng_for(1, 99)
     N, K = 520, 2560
     L = _lib.lib()
+    assert L.mllm_hip_gemv_set_path(1) == 0
     try:
         for wtype in (0, 1):
             W = synth.make_weight(rng, wtype, N, K)
@@ -151,8 +153,21 @@ def test_gemv_every_launch_shape():
                             assert L.mllm_hip_gemv_set_tuning(G, R, NW) == 0
                             y = ql.linear_q_gemv(w, xd, None, ql.SCALE_X86_REF).cpu().numpy()
                             assert rel_l2(y, want) < 2e-6, (wtype, M, G, R, NW)
+        # the matrix-core kernel with its own sweep knobs: K slices (second argument) and waves per workgroup (third)
+        assert L.mllm_hip_gemv_set_path(0) == 0
+        W = synth.make_weight(rng, 0, N, K)
+        w = ql.PackedQWeight(0, torch.from_numpy(W))
+        for M in (3, 8):
+            xf = synth.make_x_fp32(rng, M, K)
+            want = orc.linear_q(xf, W, 0, None, orc.SCALE_X86_REF)
+            for S in (0, 1, 2, 4):
+                for NW in (0, 2, 4, 8):
+                    announce("matrix-core launch shape", M, S, NW)
+                    assert L.mllm_hip_gemv_set_tuning(0, S, NW) == 0
+                    assert rel_l2(ql.linear_q_gemv(w, to_dev(xf), None, ql.SCALE_X86_REF).cpu().numpy(), want) < 2e-6, (M, S, NW)
     finally:
         L.mllm_hip_gemv_set_tuning(0, 0, 0)
+        L.mllm_hip_gemv_set_path(0)
 
 
 def test_gemv_special_inputs():

@@ -157,6 +157,9 @@ def test_gemv_fused_equals_the_operators_it_replaces(wtype, M):
     a1, img2 = ql.silu_mul(g1, u1, want_image=True)
     (o1,) = ql.linear_q_gemv_fused([pd], img2, M=M, image=True, residuals=[x])
     assert torch.equal(g0, g1) and torch.equal(u0, u1) and torch.equal(a0, a1) and torch.equal(o0, o1)
+    # raw activations with a workspace (quantized once per launch from three rows on): the same bits
+    (o1w,) = ql.linear_q_gemv_fused([pd], a0, residuals=[x], workspace=ql.gemv_workspace(M, I))
+    assert torch.equal(o1w, o0)
     # residual together with a bias, activations not pre-quantized, residual aliasing the output
     bias = to_dev(rng.standard_normal(H).astype(np.float32))
     o2 = x.clone()
