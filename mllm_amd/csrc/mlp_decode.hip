@@ -14,6 +14,10 @@
 namespace mllmhip {
 
 int exp_mode_accurate();  // layer_ops.hip: the setting of mllm_hip_set_exp_mode
+// three to eight rows of Q4_0: the matrix-core form (mlp_mfma.hip)
+bool mlp_mfma_fits(int MT, int nb);
+int launch_mlp_mfma(int x_kind, const PackedView& gate, const PackedView& up, const void* x, float* h, unsigned char* image, int M, int I,
+                    int nb, int nbp, int x86_scale, int exp_accurate, hipStream_t st);
 
 __device__ __forceinline__ float silu_sel(float x, int accurate) { return x * (1.0f / (1.0f + (accurate ? expf(-x) : exp_poly(-x)))); }
 
@@ -244,6 +248,8 @@ MLLM_API int mllm_hip_mlp_gate_up_q(int wtype, const void* gate_packed, const vo
   MlpArgs a{packed_view(wtype, gate_packed, I, H), packed_view(wtype, up_packed, I, H), x, h, reinterpret_cast<unsigned char*>(h_image),
             M, (int)H, (int)I, act_scale_mode == MLLM_HIP_SCALE_X86_REF, exp_mode_accurate()};
   hipStream_t st = (hipStream_t)stream;
+  if (wtype == MLLM_HIP_Q4_0 && M >= 3 && g_mlp_U == 0 && mlp_mfma_fits(M <= 4 ? 4 : 8, (int)(H / QK)))
+    return launch_mlp_mfma(x_kind, a.gate, a.up, x, h, a.h_image, M, (int)I, (int)(H / QK), (int)scale_row_stride(H), a.x86, a.exp_accurate, st);
   if (wtype == MLLM_HIP_Q4_0) {
     if (x_kind == MLLM_HIP_F32) return launch_mlp_m<MLLM_HIP_Q4_0, MLLM_HIP_F32>(a, st);
     if (x_kind == MLLM_HIP_BF16) return launch_mlp_m<MLLM_HIP_Q4_0, MLLM_HIP_BF16>(a, st);
