@@ -52,7 +52,7 @@ const char* mllm_hip_version(void);
 int mllm_hip_init(int device);
 
 /* ---------------------------------------------------------------------------------------------------------
- * Q4_0 / Q8_0 Linear  (decode GEMV, M = 1..8)
+ * Q4_0 / Q8_0 Linear  (decode GEMV: one launch per eight rows)
  * replaces: CPULinearOp::forward -> ggml::mat_mul -> quantize_row_q8_0 + llamafile_sgemm
  *           mllm/backends/cpu/ops/LinearOp.cpp:100-128,282-288 ; ggml/matmul.cpp:148-206 ;
  *           ggml/quantize/quantize_q8.cpp:106-190 ; llamafile/llamafile_sgemm.cpp:697-743
@@ -68,8 +68,10 @@ int mllm_hip_q_prepack(int wtype, const void* blocks, int weight_scale_mode, voi
                        void* stream);
 
 /* y[m][n] = bias[n] + sum_b fp32(dW[n][b] * dX[m][b]) * int32(sum_32 qW * qX),   qX,dX = Q8_0 quantization of x[m]
- * x: [M][K] fp32 or bf16 (x_dtype), y: fp32 [M][N], bias: fp32 [N] or NULL, 1 <= M <= 8, K % 32 == 0.
- * The activation quantization is fused into the kernel. */
+ * x: [M][K] fp32 or bf16 (x_dtype), y: fp32 [M][N], bias: fp32 [N] or NULL, M >= 1, K % 32 == 0.
+ * The activation quantization is fused into the kernel.  One launch serves up to eight rows; more rows run as passes of
+ * eight over the same weights (up to about 32 rows that is faster than the matrix-core path below, whose 128-row tiles
+ * leave most of the chip idle).  A quantized image (MLLM_HIP_Q8_IMAGE) holds at most eight rows. */
 int mllm_hip_linear_q_gemv(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y,
                            int M, int64_t N, int64_t K, int act_scale_mode, void* stream);
 

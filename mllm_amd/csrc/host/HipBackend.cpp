@@ -281,8 +281,8 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
     case Scheme::kQ4_0:
     case Scheme::kQ8_0: {
       const int wt = scheme_ == Scheme::kQ4_0 ? MLLM_HIP_Q4_0 : MLLM_HIP_Q8_0;
-      if (M <= 8) {
-        const void* image = be.findImage(x.ptr<void>(), (int)M, K);
+      if (M <= 32) {  // decode and small batches: the GEMV (passes of eight rows beat the 128-row tiles of the matrix-core path)
+        const void* image = M <= 8 ? be.findImage(x.ptr<void>(), (int)M, K) : nullptr;
         if (image) {
           mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
           MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_fused(wt, 1, &part, nullptr, image, MLLM_HIP_Q8_IMAGE, (int)M, K,
@@ -291,7 +291,7 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
           // from three rows on the activations are quantized once by a small kernel instead of in every workgroup (when
           // the launch is large enough for that to pay; the library decides)
           mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
-          void* ws = M >= 3 ? workspace(mllm_hip_gemv_workspace_bytes((int)M, K)) : nullptr;
+          void* ws = M >= 3 ? workspace(mllm_hip_gemv_workspace_bytes(8, K)) : nullptr;
           MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_multi_ws(wt, 1, &part, x.ptr<void>(), xdt(), (int)M, K, be.config().act_scale_mode, ws, st));
         }
       } else if (!gemm_packed_.isNil()) {

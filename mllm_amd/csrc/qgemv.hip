@@ -334,14 +334,40 @@ MLLM_API int mllm_hip_q_prepack(int wtype, const void* blocks, int weight_scale_
 }
 
 MLLM_API size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K) {
-  if (M < 1 || M > 8 || K <= 0 || K % QK) return 0;
-  return (size_t)8 * (K / QK) * 40;
+  if (M < 1 || K <= 0 || K % QK) return 0;
+  return (size_t)8 * (K / QK) * 40;  // one pass of eight rows at a time
 }
 
 // x_kind: MLLM_HIP_F32 / MLLM_HIP_BF16 activations, or MLLM_HIP_Q8_IMAGE: their quantized image (act_scale_mode unused)
+static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual, const void* x,
+                           int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, void* stream);
+
+// More than eight rows of raw activations: passes of eight rows, each streaming the weights again (the same arithmetic row by
+// row; up to about 32 rows this is faster than the matrix-core GEMM path, whose 128-row tiles leave most of the chip idle).
 static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fu, const void* x,
                            int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
   const float* const* residual = fu ? fu->residual : nullptr;
+  if (M <= 8 || x_dtype == MLLM_HIP_Q8_IMAGE || nparts < 1 || nparts > GEMV_MAX_PARTS || !parts || !x)
+    return gemv_multi_pass(wtype, nparts, parts, residual, x, x_dtype, M, K, act_scale_mode, workspace, stream);
+  if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
+  const size_t xrow = (size_t)K * (x_dtype == MLLM_HIP_F32 ? 4 : 2);
+  for (int m0 = 0; m0 < M; m0 += 8) {
+    mllm_hip_gemv_part pp[GEMV_MAX_PARTS];
+    const float* rr[GEMV_MAX_PARTS];
+    for (int p = 0; p < nparts; p++) {
+      pp[p] = parts[p];
+      if (pp[p].y) pp[p].y += (size_t)m0 * parts[p].N;
+      rr[p] = (residual && residual[p]) ? residual[p] + (size_t)m0 * parts[p].N : nullptr;
+    }
+    const int rc = gemv_multi_pass(wtype, nparts, pp, residual ? rr : nullptr, reinterpret_cast<const char*>(x) + (size_t)m0 * xrow, x_dtype,
+                                   M - m0 < 8 ? M - m0 : 8, K, act_scale_mode, workspace, stream);
+    if (rc) return rc;
+  }
+  return 0;
+}
+
+static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual, const void* x,
+                           int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
   if (nparts < 1 || nparts > GEMV_MAX_PARTS || !parts) return MLLM_HIP_E_BADARG;
   if (!x || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16 && x_dtype != MLLM_HIP_Q8_IMAGE)) return MLLM_HIP_E_BADARG;
   if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;

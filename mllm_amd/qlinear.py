@@ -80,7 +80,7 @@ class PackedQWeight:
 
 
 def linear_q_gemv(w, x, bias=None, act_scale_mode=SCALE_X86_REF, out=None):
-    """y = Linear(x) with Q4_0/Q8_0 weights, 1 <= M <= 8.  x [M, K] fp32/bf16 on the GPU -> y fp32 [M, N]."""
+    """y = Linear(x) with Q4_0/Q8_0 weights (more than eight rows: passes of eight).  x [M, K] fp32/bf16 on the GPU -> y fp32 [M, N]."""
     assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
     M = x.shape[0]
     y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")

@@ -5,6 +5,8 @@ Bars: activation codes, scale patterns, dequantized weights and int32 block sums
 """
 import os
 
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
@@ -192,6 +194,27 @@ def test_gemv_special_inputs():
     assert np.allclose(y[0], col * (np.float32(127) * d), rtol=1e-6, atol=0)
 
 
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M", [9, 16, 21])
+def test_gemv_more_than_eight_rows_runs_as_passes(wtype, M):
+    """rows beyond eight are passes of eight over the same weights: row by row the bits of an eight-row call"""
+    rng = synth.rng_for(1, 800 + M + wtype)
+    N, K = 300, 1024
+    W = synth.make_weight(rng, wtype, N, K)
+    w = ql.PackedQWeight(wtype, torch.from_numpy(W))
+    bias = to_dev(rng.standard_normal(N).astype(np.float32))
+    xf = synth.make_x_fp32(rng, M, K)
+    xd = to_dev(xf)
+    announce("gemv passes", wtype, M)
+    y = ql.linear_q_gemv(w, xd, bias)
+    for m0 in range(0, M, 8):
+        assert torch.equal(y[m0:m0 + 8], ql.linear_q_gemv(w, xd[m0:m0 + 8].contiguous(), bias))
+    assert rel_l2(y.cpu().numpy(), orc.linear_q(xf, W, wtype, bias.cpu().numpy(), orc.SCALE_X86_REF)) < 2e-6
+    r = to_dev(rng.standard_normal((M, N)).astype(np.float32))
+    (yr,) = ql.linear_q_gemv_fused([w], xd, biases=[bias], residuals=[r], workspace=ql.gemv_workspace(8, K))
+    assert torch.equal(yr, y + r)
+
+
 def test_gemv_argument_errors():
     L = _lib.lib()
     rng = synth.rng_for(1, 6)
@@ -201,7 +224,9 @@ def test_gemv_argument_errors():
     y = torch.zeros((8, 8), device="cuda")
     f = L.mllm_hip_linear_q_gemv
     assert f(0, w.ptr, x.data_ptr(), 0, None, y.data_ptr(), 0, 8, 64, 0, None) == -2   # M = 0
-    assert f(0, w.ptr, x.data_ptr(), 0, None, y.data_ptr(), 9, 8, 64, 0, None) == -2   # M = 9
+    fu = _lib.GemvFusion(None, None)  # an image holds at most eight rows
+    part = (_lib.GemvPart * 1)(_lib.GemvPart(w.ptr, None, y.data_ptr(), 8))
+    assert L.mllm_hip_linear_q_gemv_fused(0, 1, part, C.byref(fu), x.data_ptr(), ql.Q8_IMAGE, 9, 64, 0, None) == -2
     assert f(0, w.ptr, x.data_ptr(), 0, None, y.data_ptr(), 1, 8, 48, 0, None) == -2   # K % 32
     assert f(5, w.ptr, x.data_ptr(), 0, None, y.data_ptr(), 1, 8, 64, 0, None) == -1   # weight type
     assert f(0, None, x.data_ptr(), 0, None, y.data_ptr(), 1, 8, 64, 0, None) == -1    # null weight
@@ -288,7 +313,8 @@ def test_gemv_prequantized_equals_fused(wtype, M):
         got = ql.linear_q_gemv_multi(ws, to_dev(x), biases, ql.SCALE_X86_REF, workspace=wsp)[0].cpu().numpy()
         assert rel_l2(got, want) < 2e-6
     assert _lib.lib().mllm_hip_gemv_workspace_bytes(8, 2560) == 8 * 80 * 40
-    assert _lib.lib().mllm_hip_gemv_workspace_bytes(9, 2560) == 0
+    assert _lib.lib().mllm_hip_gemv_workspace_bytes(9, 2560) == 8 * 80 * 40  # more rows run as passes of eight
+    assert _lib.lib().mllm_hip_gemv_workspace_bytes(0, 2560) == 0
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
