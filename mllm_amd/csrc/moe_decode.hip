@@ -11,8 +11,8 @@
 //             rows of the slot's expert as PAIRED rows of a lane group, h = silu(g) * u, and the Q8_0 image of those 32
 //             values of h (exactly one block) for launch 2;
 //   launch 2  one workgroup per (token, 16 output rows): copies the images of the token's k slots into LDS and walks the
-//             experts in slot order, acc += w_j * (W_down,e_j . h_j), the next expert's weights requested while the
-//             current one is multiplied.  The sum runs in the reference's order (slot j ascending), no atomics.
+//             experts in slot order, acc += w_j * (W_down,e_j . h_j), the weights of the next eight experts in flight
+//             while one is multiplied.  The sum runs in the reference's order (slot j ascending), no atomics.
 // Arithmetic as in the GEMV kernel: exact int32 block dots, fp32 fma with dW * dX.
 #include "qgemv_kernel.h"
 
@@ -164,8 +164,12 @@ __global__ __launch_bounds__(DNW * 64) void moe_decode_down_kernel(MoeDecodeArgs
       c.dw[u] = v.d[(size_t)n * nbp + col];
     }
   };
-  Chunk cur;
-  load_expert(0, cur);
+  // the weights of the next PF experts are in flight while one is multiplied: with only the next one requested the walk over a
+  // token's experts is a chain of exposed load latencies (8.8 us for eight experts, 7 MB)
+  constexpr int PF = WT == MLLM_HIP_Q4_0 ? 8 : 4;
+  Chunk buf[PF];
+#pragma unroll
+  for (int p = 0; p < PF; p++) load_expert(p, buf[p]);  // slots past k load the last expert again and are not used
   // the images of this token's k slots are contiguous
   const int n16 = a.k * a.img_stride / 16;
   const u32x4* src = reinterpret_cast<const u32x4*>(a.img + (size_t)tok * a.k * a.img_stride);
@@ -173,27 +177,31 @@ __global__ __launch_bounds__(DNW * 64) void moe_decode_down_kernel(MoeDecodeArgs
   __syncthreads();
 
   float total = 0.f;
-  for (int j = 0; j < a.k; j++) {
-    Chunk nxt;
-    if (j + 1 < a.k) load_expert(j + 1, nxt);  // uniform
-    const unsigned char* im = smem + (size_t)j * a.img_stride;
-    const u32x4* s_lo = reinterpret_cast<const u32x4*>(im);
-    const u32x4* s_hi = s_lo + nb;
-    const float* s_d = reinterpret_cast<const float*>(s_hi + nb);
-    const int* s_n8 = reinterpret_cast<const int*>(s_d + nb);
-    float acc = 0.f;
+  for (int j0 = 0; j0 < a.k; j0 += PF) {
 #pragma unroll
-    for (int u = 0; u < U; u++) {
-      const int col = 8 * u + c0;
-      if (col < nb) {
-        const int isum = block_dot<WT>(cur.w0[u], cur.w1[WT == MLLM_HIP_Q8_0 ? u : 0], s_lo[col], s_hi[col], s_n8[col]);
-        acc = fmaf(f16bits_to_f32(cur.dw[u]) * s_d[col], (float)isum, acc);
+    for (int p = 0; p < PF; p++) {
+      const int j = j0 + p;
+      if (j < a.k) {  // uniform
+        const unsigned char* im = smem + (size_t)j * a.img_stride;
+        const u32x4* s_lo = reinterpret_cast<const u32x4*>(im);
+        const u32x4* s_hi = s_lo + nb;
+        const float* s_d = reinterpret_cast<const float*>(s_hi + nb);
+        const int* s_n8 = reinterpret_cast<const int*>(s_d + nb);
+        float acc = 0.f;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+          const int col = 8 * u + c0;
+          if (col < nb) {
+            const int isum = block_dot<WT>(buf[p].w0[u], buf[p].w1[WT == MLLM_HIP_Q8_0 ? u : 0], s_lo[col], s_hi[col], s_n8[col]);
+            acc = fmaf(f16bits_to_f32(buf[p].dw[u]) * s_d[col], (float)isum, acc);
+          }
+        }
+        const float v = group_sum<8>(acc);
+        const int e = a.ids[tok * a.k + j];
+        if (e >= 0 && e < a.E) total = total + v * a.w[tok * a.k + j];
+        if (j + PF < a.k) load_expert(j + PF, buf[p]);  // uniform: refill the slot just used
       }
     }
-    const float v = group_sum<8>(acc);
-    const int e = a.ids[tok * a.k + j];
-    if (e >= 0 && e < a.E) total = total + v * a.w[tok * a.k + j];
-    if (j + 1 < a.k) cur = nxt;
   }
   if (c0 == 0) a.y[(size_t)tok * a.H + n] = total;
 }
