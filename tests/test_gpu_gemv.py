@@ -215,6 +215,23 @@ def test_gemv_more_than_eight_rows_runs_as_passes(wtype, M):
     assert torch.equal(yr, y + r)
 
 
+@pytest.mark.parametrize("M", [1, 2, 5])
+def test_gemv_vocabulary_sized_matrix(M):
+    """the lm_head of the reference's Qwen3 recipes: 151936 rows (quant_cfg_30B_q4_k.json lists [151936, 2048]); checked on
+    sampled rows, the first and the last ones included"""
+    rng = synth.rng_for(1, 950 + M)
+    N, K = 151936, 2048
+    W = synth.make_weight(rng, 0, N, K)
+    w = ql.PackedQWeight(0, torch.from_numpy(W))
+    xf = synth.make_x_fp32(rng, M, K)
+    announce("gemv vocabulary rows", M)
+    y = ql.linear_q_gemv(w, to_dev(xf)).cpu().numpy()
+    rows = np.unique(np.concatenate([np.arange(40), np.arange(N - 40, N), rng.integers(0, N, 2000)]))
+    want = orc.linear_q(xf, W[rows], 0, None, orc.SCALE_X86_REF)
+    assert rel_l2(y[:, rows], want) < 2e-6
+    assert np.isfinite(y).all()
+
+
 def test_gemv_argument_errors():
     L = _lib.lib()
     rng = synth.rng_for(1, 6)
