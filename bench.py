@@ -188,7 +188,20 @@ def side_workloads(torch, ql, synth, gen):
     out["q4_0_linear_prefill_2048x9728x2560"] = {"us": t2 * 1e6, "TFLOPS": fl / t2 / 1e12, "frac_of_2500_TFLOPS": fl / t2 / 2.5e15,
                                                   "path": "matrix cores (mllm_hip_linear_q_gemm)",
                                                   "block_dot_path": {"us": t1 * 1e6, "TOPS": fl / t1 / 1e12}}
-    del wv, wg
+    del wv
+    # a short prompt: 128 rows through the gate and the down projection of the layer; K cut into ranges (the _short entry point)
+    # against one workgroup per tile
+    sp = {}
+    for nm, (n_, k_) in (("gate_9728x2560", (9728, 2560)), ("down_2560x9728", (2560, 9728))):
+        wsg = wg if (n_, k_) == (N, K) else ql.PackedQWeight.synthetic(ql.Q4_0, n_, k_, gen, layout="gemm")
+        xs_ = torch.randn((128, k_), device="cuda", generator=gen).to(torch.bfloat16)
+        ys_ = torch.empty((128, n_), dtype=torch.float32, device="cuda")
+        wss = torch.empty(L.mllm_hip_linear_q_gemm_short_workspace_bytes(128, n_, k_), dtype=torch.uint8, device="cuda")
+        ta = ev_time(lambda: ql.linear_q_gemm(wsg, xs_, None, ql.SCALE_X86_REF, workspace=wss, out=ys_), 10)
+        tb = ev_time(lambda: ql.linear_q_gemm(wsg, xs_, None, ql.SCALE_X86_REF, workspace=wss, out=ys_, short=True), 10)
+        sp[nm] = {"us": tb * 1e6, "one_workgroup_per_tile_us": ta * 1e6}
+    out["q4_0_linear_short_prompt_128_rows"] = sp
+    del wg
     # the same Linear with Q4_K / Q6_K weights (Q8_K activations): matrix cores against passes of the eight-row GEMV
     for kname, kt in (("q4_k", ql.Q4_K), ("q6_k", ql.Q6_K)):
         wkg = ql.PackedKWeight.synthetic(kt, N, K, gen, layout="gemm")

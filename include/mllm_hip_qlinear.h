@@ -70,8 +70,8 @@ int mllm_hip_q_prepack(int wtype, const void* blocks, int weight_scale_mode, voi
 /* y[m][n] = bias[n] + sum_b fp32(dW[n][b] * dX[m][b]) * int32(sum_32 qW * qX),   qX,dX = Q8_0 quantization of x[m]
  * x: [M][K] fp32 or bf16 (x_dtype), y: fp32 [M][N], bias: fp32 [N] or NULL, M >= 1, K % 32 == 0.
  * The activation quantization is fused into the kernel.  One launch serves up to eight rows; more rows run as passes of
- * eight over the same weights (up to about 32 rows that is faster than the matrix-core path below, whose 128-row tiles
- * leave most of the chip idle).  A quantized image (MLLM_HIP_Q8_IMAGE) holds at most eight rows. */
+ * eight over the same weights (the reference arithmetic for any number of rows; from nine rows on
+ * mllm_hip_linear_q_gemm_short is faster).  A quantized image (MLLM_HIP_Q8_IMAGE) holds at most eight rows. */
 int mllm_hip_linear_q_gemv(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y,
                            int M, int64_t N, int64_t K, int act_scale_mode, void* stream);
 
@@ -165,6 +165,13 @@ int mllm_hip_q_gemm_prepack(int wtype, const void* blocks, int weight_scale_mode
 size_t mllm_hip_linear_q_gemm_workspace_bytes(int64_t M, int64_t K);
 int mllm_hip_linear_q_gemm(int wtype, const void* gemm_packed, const void* x, int x_dtype, const float* bias, float* y,
                            int64_t M, int64_t N, int64_t K, int act_scale_mode, void* workspace, void* stream);
+/* The same Linear for short batches (a prompt of up to 1024 rows): its M/128 x N/256 tiles would occupy a fraction of the chip,
+ * so K is cut into up to eight ranges that run as separate workgroups and a small second kernel adds their partial results
+ * in range order (deterministic).  Same operands and arithmetic; the fp32 sum over K is grouped by range.  Any M is
+ * accepted (where cutting K does not pay it is the call above).  workspace: 256-byte aligned. */
+size_t mllm_hip_linear_q_gemm_short_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mllm_hip_linear_q_gemm_short(int wtype, const void* gemm_packed, const void* x, int x_dtype, const float* bias, float* y,
+                                 int64_t M, int64_t N, int64_t K, int act_scale_mode, void* workspace, void* stream);
 /* Same arguments as mllm_hip_moe_ffn_q; the three expert arrays are E gemm-packed matrices back to back
  * (stride mllm_hip_q_gemm_packed_bytes). */
 size_t mllm_hip_moe_gemm_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k);
@@ -318,6 +325,10 @@ int mllm_hip_kq_gemm_prepack(int wtype, const void* blocks, int weight_scale_mod
 size_t mllm_hip_linear_kq_gemm_workspace_bytes(int64_t M, int64_t K);
 int mllm_hip_linear_kq_gemm(int wtype, const void* gemm_packed, const void* x, int x_dtype, const float* bias, float* y,
                             int64_t M, int64_t N, int64_t K, void* workspace, void* stream);
+/* The same for short batches, as mllm_hip_linear_q_gemm_short. */
+size_t mllm_hip_linear_kq_gemm_short_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int mllm_hip_linear_kq_gemm_short(int wtype, const void* gemm_packed, const void* x, int x_dtype, const float* bias, float* y,
+                                  int64_t M, int64_t N, int64_t K, void* workspace, void* stream);
 /* Parity probes.  Dequantized weights fp32 [N][K] (dequantize_row_q4_K / _q6_K, quantize_q4.cpp:284-312, quantize_q6.cpp:108-133);
  * Q8_K activation quantization: codes int8 [M][K], d fp32 [M][K/256], sums of 16 codes int16 [M][K/16]. */
 int mllm_hip_kq_dequantize(int wtype, const void* packed, float* w, int64_t N, int64_t K, void* stream);

@@ -74,6 +74,12 @@ def lib():
         L.mllm_hip_linear_kq_gemm_workspace_bytes.restype = C.c_size_t
         L.mllm_hip_linear_kq_gemm_workspace_bytes.argtypes = [i64, i64]
         L.mllm_hip_linear_kq_gemm.argtypes = [ci, vp, vp, ci, vp, vp, i64, i64, i64, vp, vp]
+        L.mllm_hip_linear_q_gemm_short_workspace_bytes.restype = C.c_size_t
+        L.mllm_hip_linear_q_gemm_short_workspace_bytes.argtypes = [i64, i64, i64]
+        L.mllm_hip_linear_q_gemm_short.argtypes = [ci, vp, vp, ci, vp, vp, i64, i64, i64, ci, vp, vp]
+        L.mllm_hip_linear_kq_gemm_short_workspace_bytes.restype = C.c_size_t
+        L.mllm_hip_linear_kq_gemm_short_workspace_bytes.argtypes = [i64, i64, i64]
+        L.mllm_hip_linear_kq_gemm_short.argtypes = [ci, vp, vp, ci, vp, vp, i64, i64, i64, vp, vp]
         L.mllm_hip_kq_packed_bytes.restype = C.c_size_t
         L.mllm_hip_kq_packed_bytes.argtypes = [ci, i64, i64]
         L.mllm_hip_kq_prepack.argtypes = [ci, vp, ci, vp, i64, i64, vp]

@@ -281,8 +281,8 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
     case Scheme::kQ4_0:
     case Scheme::kQ8_0: {
       const int wt = scheme_ == Scheme::kQ4_0 ? MLLM_HIP_Q4_0 : MLLM_HIP_Q8_0;
-      if (M <= 32) {  // decode and small batches: the GEMV (passes of eight rows beat the 128-row tiles of the matrix-core path)
-        const void* image = M <= 8 ? be.findImage(x.ptr<void>(), (int)M, K) : nullptr;
+      if (M <= 8) {  // decode: the GEMV
+        const void* image = be.findImage(x.ptr<void>(), (int)M, K);
         if (image) {
           mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
           MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_fused(wt, 1, &part, nullptr, image, MLLM_HIP_Q8_IMAGE, (int)M, K,
@@ -295,9 +295,10 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
           MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_multi_ws(wt, 1, &part, x.ptr<void>(), xdt(), (int)M, K, be.config().act_scale_mode, ws, st));
         }
       } else if (!gemm_packed_.isNil()) {
-        void* ws = workspace(mllm_hip_linear_q_gemm_workspace_bytes(M, K));
-        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemm(wt, gemm_packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K,
-                                                     be.config().act_scale_mode, ws, st));
+        // (the short-batch entry point cuts K into ranges up to 256 rows and is the plain call beyond)
+        void* ws = workspace(mllm_hip_linear_q_gemm_short_workspace_bytes(M, N, K));
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemm_short(wt, gemm_packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K,
+                                                           be.config().act_scale_mode, ws, st));
       } else {
         void* ws = workspace(mllm_hip_linear_q_workspace_bytes(M, K));
         MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K,
@@ -309,8 +310,8 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
     case Scheme::kQ6_K: {
       const int wt = scheme_ == Scheme::kQ4_K ? MLLM_HIP_Q4_K : MLLM_HIP_Q6_K;
       if (M > 8 && !gemm_packed_.isNil()) {  // prefill: matrix cores
-        void* ws = workspace(mllm_hip_linear_kq_gemm_workspace_bytes(M, K));
-        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_kq_gemm(wt, gemm_packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K, ws, st));
+        void* ws = workspace(mllm_hip_linear_kq_gemm_short_workspace_bytes(M, N, K));
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_kq_gemm_short(wt, gemm_packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K, ws, st));
       } else {
         MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_kq(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K,
                                                  M >= 3 ? workspace(mllm_hip_kq_workspace_bytes(M, K)) : nullptr, st));

@@ -1420,5 +1420,27 @@ MLLM_API int mllm_hip_linear_kq_gemm(int wtype, const void* gemm_packed, const v
   uint16_t* xh = reinterpret_cast<uint16_t*>(workspace);
   const int64_t nitems = M * K / 8;
   hipLaunchKernelGGL(kq_act_f16_kernel, dim3((unsigned)((nitems + 255) / 256)), dim3(256), 0, st, x, x_dtype, xh, nitems);
-  return qg_linear_run(wtype, gemm_packed, xh, bias, y, M, N, K, reinterpret_cast<char*>(workspace) + align_up((size_t)M * K * 2, 256), st);
+  return qg_linear_run(wtype, gemm_packed, xh, bias, y, M, N, K, reinterpret_cast<char*>(workspace) + align_up((size_t)M * K * 2, 256), nullptr, st);
+}
+
+// the same for short batches (M <= 256 gains; any M is accepted): K cut into ranges that run as separate workgroups
+MLLM_API size_t mllm_hip_linear_kq_gemm_short_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % QK_K) return 0;
+  return align_up(mllm_hip_linear_kq_gemm_workspace_bytes(M, K), 256) + qg_partial_bytes(M, N, K);
+}
+MLLM_API int mllm_hip_linear_kq_gemm_short(int wtype, const void* gemm_packed, const void* x, int x_dtype, const float* bias, float* y,
+                                           int64_t M, int64_t N, int64_t K, void* workspace, void* stream) {
+  if (!kq_type(wtype) || !gemm_packed || !x || !y || !workspace || M <= 0 || N <= 0 || K <= 0) return MLLM_HIP_E_BADARG;
+  if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
+  if (K % QK_K || M * K * 2 >= ((int64_t)1 << 32) || N > INT32_MAX || qg_bytes(wtype, N, K) >= ((int64_t)1 << 32)) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 256 || reinterpret_cast<uintptr_t>(gemm_packed) % 16 ||
+      reinterpret_cast<uintptr_t>(y) % 16)
+    return MLLM_HIP_E_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  uint16_t* xh = reinterpret_cast<uint16_t*>(workspace);
+  const int64_t nitems = M * K / 8;
+  hipLaunchKernelGGL(kq_act_f16_kernel, dim3((unsigned)((nitems + 255) / 256)), dim3(256), 0, st, x, x_dtype, xh, nitems);
+  char* base = reinterpret_cast<char*>(workspace);
+  void* partial = qg_partial_bytes(M, N, K) ? base + align_up(mllm_hip_linear_kq_gemm_workspace_bytes(M, K), 256) : nullptr;
+  return qg_linear_run(wtype, gemm_packed, xh, bias, y, M, N, K, base + align_up((size_t)M * K * 2, 256), partial, st);
 }

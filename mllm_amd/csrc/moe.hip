@@ -536,6 +536,8 @@ struct QG2Args {
   int N, K;
   int wtype;
   int x86_scale;
+  int ksplit;            // one-matrix mode: K is cut into this many ranges (blockIdx.z), each writing its own partial result
+  float* partial;        // [ksplit][a_rows][N] when ksplit > 1
 };
 
 // pair `b` (elements 2b, 2b+1) of the eight weights of one MFMA step, scaled: one dword of two fp16.  With PREC == 2 also
@@ -683,9 +685,21 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
     const uint32_t h = d < 2 ? (s[SDW - 1] & 0xffffu) : (s[SDW - 1] >> 16);
     return __builtin_bit_cast(f16x2, h | (h << 16));
   };
-  loadA(0, ga);
-  loadW(0, 0);
-  loadW(1, 1);
+  // K range of this workgroup: all of it, or (short batches, one matrix) range blockIdx.z of a.ksplit, written to its own
+  // partial result; the ranges start at even K steps
+  int kt0 = 0, kt1 = Kp / BK;  // even
+  float* outp = a.out;
+  const float* biasp = a.bias;
+  if (NW == 1 && a.ksplit > 1) {
+    const int per = ((kt1 + a.ksplit - 1) / a.ksplit + 1) / 2 * 2;
+    kt0 = (int)blockIdx.z * per;
+    kt1 = min(kt1, kt0 + per);
+    outp = a.partial + (size_t)blockIdx.z * a.a_rows * a.N;
+    biasp = nullptr;
+  }
+  loadA(kt0 * BK, ga);
+  loadW(0, kt0);
+  loadW(1, kt0 + 1);
   storeA(0, ga);
   __syncthreads();
   readA(0, 0, fa[0]);
@@ -748,8 +762,7 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
         }
     }
   };
-  const int KT = Kp / BK;  // even
-  for (int kt = 0; kt < KT; kt += 2) {
+  for (int kt = kt0; kt < kt1; kt += 2) {
     kstep(std::integral_constant<int, 0>{}, kt);
     kstep(std::integral_constant<int, 1>{}, kt + 1);
   }
@@ -762,7 +775,7 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
       const int r = i * 32 + lrow;
       if (r < rows) {
         const int pos = row0 + r;
-        float* orow = a.out + (int64_t)(a.o_index ? a.o_index[pos] : pos) * a.N;
+        float* orow = outp + (int64_t)(a.o_index ? a.o_index[pos] : pos) * a.N;
 #pragma unroll
         for (int j = 0; j < TN; j++)
 #pragma unroll
@@ -770,12 +783,12 @@ __device__ __forceinline__ void qg_tile(const QG2Args& a, const int e, const int
             const int n = n0 + wave * WN + j * 32 + 8 * g + 4 * hi;
             f32x4 v = {acc[0][j][i][4 * g], acc[0][j][i][4 * g + 1], acc[0][j][i][4 * g + 2], acc[0][j][i][4 * g + 3]};
             if (n + 3 < a.N && a.N % 4 == 0) {
-              if (a.bias) v += *reinterpret_cast<const f32x4*>(a.bias + n);
+              if (biasp) v += *reinterpret_cast<const f32x4*>(biasp + n);
               *reinterpret_cast<f32x4*>(orow + n) = v;
             } else {
 #pragma unroll
               for (int e2 = 0; e2 < 4; e2++)
-                if (n + e2 < a.N) orow[n + e2] = a.bias ? v[e2] + a.bias[n + e2] : v[e2];
+                if (n + e2 < a.N) orow[n + e2] = biasp ? v[e2] + biasp[n + e2] : v[e2];
             }
           }
       }
@@ -851,7 +864,7 @@ constexpr int QG_TILE_H = 128;
 template <int MODE>
 static int launch_qg(const QG2Args& a, unsigned max_tiles, hipStream_t st) {
   constexpr int TN = MODE == 1 ? 1 : 2;
-  const dim3 grid(max_tiles, (unsigned)((a.N + 128 * TN - 1) / (128 * TN)), MODE == 1 ? 2 : 1);
+  const dim3 grid(max_tiles, (unsigned)((a.N + 128 * TN - 1) / (128 * TN)), MODE == 1 ? 2 : (unsigned)(a.ksplit > 1 ? a.ksplit : 1));
   const size_t lds = 2 * (size_t)QG_TILE_H * (2 * 64 + 16);  // MODE 1: half the rows, value + residual
   if (a.wtype == MLLM_HIP_Q4_0) hipLaunchKernelGGL((qg_kernel<MLLM_HIP_Q4_0, MODE>), grid, dim3(256), lds, st, a);
   else if (a.wtype == MLLM_HIP_Q8_0) hipLaunchKernelGGL((qg_kernel<MLLM_HIP_Q8_0, MODE>), grid, dim3(256), lds, st, a);
@@ -915,13 +928,44 @@ static int launch_tiles(int wtype, const QGemmArgs& a, unsigned max_tiles, hipSt
   return wtype == MLLM_HIP_Q4_0 ? launch(qgemm_tile_kernel<MLLM_HIP_Q4_0, MODE>) : launch(qgemm_tile_kernel<MLLM_HIP_Q8_0, MODE>);
 }
 
+// y = sum over the K ranges of their partial results (in range order) + bias
+__global__ __launch_bounds__(256) void qg_reduce_kernel(const float* __restrict__ partial, int Z, int64_t MN, int N, const float* __restrict__ bias,
+                                                        float* __restrict__ y) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;  // N % 4 == 0 on this path
+  if (i >= MN) return;
+  f32x4 v = *reinterpret_cast<const f32x4*>(partial + i);
+  for (int z = 1; z < Z; z++) v += *reinterpret_cast<const f32x4*>(partial + (size_t)z * MN + i);
+  if (bias) v += *reinterpret_cast<const f32x4*>(bias + i % N);
+  *reinterpret_cast<f32x4*>(y + i) = v;
+}
+
+// Short batches: a Linear of a few hundred rows has M/128 x N/256 tiles, far fewer than the chip has CUs (gate projection of
+// the 4B layer at 128 rows: 38 workgroups, down: 10), and each streams its weights two K steps ahead only.  K is therefore
+// cut into up to eight ranges that run as separate workgroups and leave partial results, summed by a small second kernel
+// in range order.  Number of ranges: enough for about one workgroup per CU, at most 24 MB of partial results (their round trip through memory is what the second kernel costs); up to 1024 rows.
+int qg_short_splits(int64_t M, int64_t N, int64_t K) {
+  if (M > 1024 || N % 4) return 1;
+  const int64_t tiles = ((M + QG_TILE_H - 1) / QG_TILE_H) * ((N + 255) / 256);
+  const int KT = (int)(qg_kp(K) / 64);
+  int z = (int)((256 + tiles - 1) / tiles);
+  if (z > 8) z = 8;
+  while (z > 1 && (int64_t)z * M * N * 4 > (24 << 20)) z--;
+  if (z <= 1) return 1;
+  const int per = ((KT + z - 1) / z + 1) / 2 * 2;
+  return (KT + per - 1) / per;  // no empty range
+}
+size_t qg_partial_bytes(int64_t M, int64_t N, int64_t K) {
+  const int z = qg_short_splits(M, N, K);
+  return z > 1 ? align_up((size_t)z * M * N * 4, 256) : 0;
+}
+
 size_t qg_route_bytes(int64_t M) {
   Carver c(nullptr);
   carve_route(c, 1, M);
   return c.used;
 }
 int qg_linear_run(int wtype, const void* gemm_packed, const uint16_t* xh, const float* bias, float* y, int64_t M, int64_t N,
-                  int64_t K, void* route_ws, hipStream_t st) {
+                  int64_t K, void* route_ws, void* partial_ws, hipStream_t st) {
   Carver c(route_ws);
   RouteOut ro = carve_route(c, 1, M);
   hipLaunchKernelGGL(identity_tiles_kernel, dim3(1), dim3(256), 0, st, (int)M, QG_TILE_H, ro);
@@ -932,7 +976,12 @@ int qg_linear_run(int wtype, const void* gemm_packed, const uint16_t* xh, const 
   a.o_index = nullptr; a.out = y; a.bias = bias;
   a.tile_expert = ro.tile_expert; a.tile_row0 = ro.tile_row0; a.tile_rows = ro.tile_rows; a.ntiles = ro.ntiles;
   a.N = (int)N; a.K = (int)K; a.wtype = wtype; a.x86_scale = 0;
-  return launch_qg<0>(a, (unsigned)((M + QG_TILE_H - 1) / QG_TILE_H), st);
+  a.ksplit = partial_ws ? qg_short_splits(M, N, K) : 1;
+  a.partial = reinterpret_cast<float*>(partial_ws);
+  const int rc = launch_qg<0>(a, (unsigned)((M + QG_TILE_H - 1) / QG_TILE_H), st);
+  if (rc || a.ksplit <= 1) return rc;
+  hipLaunchKernelGGL(qg_reduce_kernel, dim3((unsigned)((M * N / 4 + 255) / 256)), dim3(256), 0, st, a.partial, a.ksplit, M * N, (int)N, bias, y);
+  return (int)hipGetLastError();
 }
 
 }  // namespace mllmhip
@@ -1124,7 +1173,33 @@ MLLM_API int mllm_hip_linear_q_gemm(int wtype, const void* gemm_packed, const vo
   const int64_t nblocks = M * (K / QK);
   hipLaunchKernelGGL(qg_act_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, xh,
                      (uint16_t*)nullptr, nblocks, act_scale_mode == MLLM_HIP_SCALE_X86_REF);
-  return qg_linear_run(wtype, gemm_packed, xh, bias, y, M, N, K, c.p + c.used, st);
+  return qg_linear_run(wtype, gemm_packed, xh, bias, y, M, N, K, c.p + c.used, nullptr, st);
+}
+
+// the same for short batches (M <= 256 gains; any M is accepted): K cut into ranges, see qg_short_splits
+MLLM_API size_t mllm_hip_linear_q_gemm_short_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % QK) return 0;
+  return mllm_hip_linear_q_gemm_workspace_bytes(M, K) + qg_partial_bytes(M, N, K);
+}
+MLLM_API int mllm_hip_linear_q_gemm_short(int wtype, const void* gemm_packed, const void* x, int x_dtype, const float* bias, float* y,
+                                          int64_t M, int64_t N, int64_t K, int act_scale_mode, void* workspace, void* stream) {
+  if ((wtype != MLLM_HIP_Q4_0 && wtype != MLLM_HIP_Q8_0) || !gemm_packed || !x || !y || !workspace || M <= 0 || N <= 0 || K <= 0)
+    return MLLM_HIP_E_BADARG;
+  if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
+  if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
+  if (K % QK || M * K * 2 >= ((int64_t)1 << 32) || N > INT32_MAX || qg_bytes(wtype, N, K) >= ((int64_t)1 << 32)) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 256 ||
+      reinterpret_cast<uintptr_t>(gemm_packed) % 16 || reinterpret_cast<uintptr_t>(y) % 16)
+    return MLLM_HIP_E_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  Carver c(workspace);
+  uint16_t* xh = c.take<uint16_t>((size_t)M * K);
+  const int64_t nblocks = M * (K / QK);
+  hipLaunchKernelGGL(qg_act_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, xh,
+                     (uint16_t*)nullptr, nblocks, act_scale_mode == MLLM_HIP_SCALE_X86_REF);
+  void* route = c.p + c.used;
+  void* partial = qg_partial_bytes(M, N, K) ? c.p + mllm_hip_linear_q_gemm_workspace_bytes(M, K) : nullptr;
+  return qg_linear_run(wtype, gemm_packed, xh, bias, y, M, N, K, route, partial, st);
 }
 
 MLLM_API size_t mllm_hip_moe_gemm_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k) {

@@ -22,8 +22,11 @@ __host__ __device__ inline int64_t qg_bytes(int wtype, int64_t N, int64_t K) {
 }
 
 // y[M][N] fp32 = xh[M][K] (fp16) * W^T + bias on the matrix cores; route_ws: qg_route_bytes(M) bytes, 16-byte aligned
+// partial_ws: null, or qg_partial_bytes(M, N, K) bytes (256-byte aligned) for short batches: K is then cut into ranges that
+// run as separate workgroups (qg_partial_bytes returns 0 where that does not pay; pass null then)
 size_t qg_route_bytes(int64_t M);
+size_t qg_partial_bytes(int64_t M, int64_t N, int64_t K);
 int qg_linear_run(int wtype, const void* gemm_packed, const uint16_t* xh, const float* bias, float* y, int64_t M, int64_t N,
-                  int64_t K, void* route_ws, hipStream_t st);
+                  int64_t K, void* route_ws, void* partial_ws, hipStream_t st);
 
 }  // namespace mllmhip

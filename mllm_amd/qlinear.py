@@ -359,17 +359,19 @@ def moe_ffn_q(gate, up, down, x, topk_ids, topk_w, act_scale_mode=SCALE_X86_REF,
     return y
 
 
-def linear_q_gemm(w, x, bias=None, act_scale_mode=SCALE_X86_REF, workspace=None, out=None):
+def linear_q_gemm(w, x, bias=None, act_scale_mode=SCALE_X86_REF, workspace=None, out=None, short=False):
     """Q4_0/Q8_0 Linear for many rows on the matrix cores (fp16 operands with the block scales folded in); w in the "gemm"
-    layout."""
+    layout.  short=True: the entry point for short batches (K cut into ranges that run as separate workgroups)."""
     assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K and w.layout == "gemm"
     M = x.shape[0]
     L = _lib.lib()
     if workspace is None:
-        workspace = torch.empty(L.mllm_hip_linear_q_gemm_workspace_bytes(M, w.K), dtype=torch.uint8, device="cuda")
+        size = L.mllm_hip_linear_q_gemm_short_workspace_bytes(M, w.N, w.K) if short else L.mllm_hip_linear_q_gemm_workspace_bytes(M, w.K)
+        workspace = torch.empty(size, dtype=torch.uint8, device="cuda")
     y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")
-    _lib.check(L.mllm_hip_linear_q_gemm(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K,
-                                        act_scale_mode, workspace.data_ptr(), _stream()), "mllm_hip_linear_q_gemm")
+    fn = L.mllm_hip_linear_q_gemm_short if short else L.mllm_hip_linear_q_gemm
+    _lib.check(fn(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K, act_scale_mode, workspace.data_ptr(),
+                  _stream()), "mllm_hip_linear_q_gemm")
     return y
 
 
@@ -549,15 +551,18 @@ def kq_workspace(M, K):
     return torch.empty(_lib.lib().mllm_hip_kq_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
 
 
-def linear_kq_gemm(w, x, bias=None, out=None, workspace=None):
-    """many rows on the matrix cores; w: PackedKWeight(layout="gemm")"""
+def linear_kq_gemm(w, x, bias=None, out=None, workspace=None, short=False):
+    """many rows on the matrix cores; w: PackedKWeight(layout="gemm"); short=True: the entry point for short batches"""
     assert w.layout == "gemm" and x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
     M = x.shape[0]
     L = _lib.lib()
     y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")
-    ws = workspace if workspace is not None else torch.empty(L.mllm_hip_linear_kq_gemm_workspace_bytes(M, w.K), dtype=torch.uint8, device="cuda")
-    _lib.check(L.mllm_hip_linear_kq_gemm(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K, ws.data_ptr(),
-                                         _stream()), "mllm_hip_linear_kq_gemm")
+    if workspace is None:
+        size = L.mllm_hip_linear_kq_gemm_short_workspace_bytes(M, w.N, w.K) if short else L.mllm_hip_linear_kq_gemm_workspace_bytes(M, w.K)
+        workspace = torch.empty(size, dtype=torch.uint8, device="cuda")
+    fn = L.mllm_hip_linear_kq_gemm_short if short else L.mllm_hip_linear_kq_gemm
+    _lib.check(fn(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K, workspace.data_ptr(), _stream()),
+               "mllm_hip_linear_kq_gemm")
     return y
 
 

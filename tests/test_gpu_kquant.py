@@ -138,6 +138,8 @@ def test_linear_kq_gemm(wtype, M, N, K):
     bits, xb = synth.make_x_bf16(rng, M, K)
     y2 = ql.linear_kq_gemm(wg, bf16_dev(bits)).cpu().numpy()
     assert rel_l2(y2, orc.linear_kq(xb, W, wtype, None, orc.SCALE_X86_REF)) < TOL
+    ys = ql.linear_kq_gemm(wg, to_dev(xf), to_dev(bias), short=True).cpu().numpy()  # K ranges as separate workgroups
+    assert rel_l2(ys, y) < 2e-6
     # and against the GEMV path (the reference arithmetic itself) on the same device
     yv = ql.linear_kq(ql.PackedKWeight(wtype, torch.from_numpy(W)), to_dev(xf), to_dev(bias)).cpu().numpy()
     assert rel_l2(y, yv) < TOL

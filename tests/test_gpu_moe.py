@@ -60,6 +60,29 @@ def test_linear_q_gemm_any_m(wtype, M, N, K):
     xb = synth.fp32_to_bf16_bits(x)
     y16 = ql.linear_q_gemm(w, bf16_dev(xb)).cpu().numpy()
     assert rel_l2(y16, orc.linear_q(synth.bf16_bits_to_fp32(xb), W, wtype)) < GEMM_TOL
+    # the entry point for short batches (K cut into ranges, partial results added in range order): same operands, the fp32
+    # sum over K grouped differently; deterministic
+    ys = ql.linear_q_gemm(w, to_dev(x), to_dev(bias), short=True)
+    assert rel_l2(ys.cpu().numpy(), yb) < 2e-6
+    assert torch.equal(ys, ql.linear_q_gemm(w, to_dev(x), to_dev(bias), short=True))
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M,N,K", [(16, 9728, 2560), (128, 2560, 9728), (200, 1024, 640), (256, 6144, 2560), (40, 132, 4096 + 128)])
+def test_linear_q_gemm_short_batches(wtype, M, N, K):
+    """short prompts: K ranges as separate workgroups + reduction, against the oracle and the unsplit call"""
+    rng = synth.rng_for(4, 600 + M + N % 97 + wtype)
+    W = synth.make_weight(rng, wtype, N, K)
+    w = ql.PackedQWeight(wtype, torch.from_numpy(W), layout="gemm")
+    x = synth.make_x_fp32(rng, M, K)
+    bias = rng.standard_normal(N).astype(np.float32)
+    announce("linear_q_gemm short", wtype, M, N, K)
+    assert _lib.lib().mllm_hip_linear_q_gemm_short_workspace_bytes(M, N, K) > _lib.lib().mllm_hip_linear_q_gemm_workspace_bytes(M, K)
+    ys = ql.linear_q_gemm(w, to_dev(x), to_dev(bias), short=True).cpu().numpy()
+    rows = rng.integers(0, M, 8)
+    want = orc.linear_q(x[rows], W, wtype, bias)
+    assert rel_l2(ys[rows], want) < GEMM_TOL
+    assert rel_l2(ys, ql.linear_q_gemm(w, to_dev(x), to_dev(bias)).cpu().numpy()) < 2e-6
 
 
 def test_linear_q_gemm_exact_when_operands_fit_fp16():
@@ -80,6 +103,7 @@ def test_linear_q_gemm_exact_when_operands_fit_fp16():
         y = ql.linear_q_gemm(w, to_dev(x), None, ql.SCALE_IEEE).cpu().numpy()
         want = orc.linear_q(x, W, wtype, None, orc.SCALE_IEEE)
         assert np.array_equal(y, want)
+        assert np.array_equal(ql.linear_q_gemm(w, to_dev(x), None, ql.SCALE_IEEE, short=True).cpu().numpy(), want)
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
