@@ -175,7 +175,8 @@ def test_gemv_fused_equals_the_operators_it_replaces(wtype, M):
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
-@pytest.mark.parametrize("M,H,I", [(1, 512, 1536), (2, 512, 96), (3, 2560, 9728), (4, 4096, 512), (5, 96, 64), (8, 2560, 1024), (1, 2560, 9728)])
+@pytest.mark.parametrize("M,H,I", [(1, 512, 1536), (2, 512, 96), (3, 2560, 9728), (4, 4096, 512), (5, 96, 64), (8, 2560, 1024), (1, 2560, 9728),
+                                   (6, 4096, 256), (7, 5120, 160), (3, 8192, 64)])
 def test_mlp_gate_up_one_launch(wtype, M, H, I):
     """gate / up / SiLU / product (/ Q8_0 image of the product) in one launch against the oracle's chain, and the image
     against the Q8_0 quantization of the h the same launch stored (bit-exact); from activations and from rmsnorm's image"""
