@@ -648,8 +648,10 @@ MLLM_API size_t mllm_hip_w8a8_workspace_bytes(int64_t M, int64_t K) {
 
 MLLM_API int mllm_hip_w8a8_linear(const void* x, int x_dtype, const int8_t* W, const float* w_scale, const float* bias,
                                   void* out_bf16, int64_t M, int64_t N, int64_t K, void* workspace, void* stream) {
-  if (!workspace) return MLLM_HIP_E_BADARG;
-  if (reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
+  // everything the second step would reject is rejected before the first one is launched
+  if (!workspace || !W || !w_scale || !out_bf16 || N <= 0) return MLLM_HIP_E_BADARG;
+  if (K > 0 && K % 16) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(workspace) % 16 || reinterpret_cast<uintptr_t>(W) % 16) return MLLM_HIP_E_ALIGN;
   int8_t* q = reinterpret_cast<int8_t*>(workspace);
   float* xs = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + align_up((size_t)M * K, 256));
   int rc = mllm_hip_per_token_quant_int8(x, x_dtype, q, xs, M, K, stream);
@@ -660,8 +662,10 @@ MLLM_API int mllm_hip_w8a8_linear(const void* x, int x_dtype, const int8_t* W, c
 MLLM_API int mllm_hip_w8a8_linear_packed(const void* x, int x_dtype, const void* W_packed, const float* w_scale,
                                          const float* bias, void* out_bf16, int64_t M, int64_t N, int64_t K,
                                          void* workspace, void* stream) {
-  if (!workspace) return MLLM_HIP_E_BADARG;
-  if (reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
+  // everything the second step would reject is rejected before the first one is launched
+  if (!workspace || !W_packed || !w_scale || !out_bf16 || N <= 0) return MLLM_HIP_E_BADARG;
+  if (K > 0 && K % 16) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(workspace) % 16 || reinterpret_cast<uintptr_t>(W_packed) % 16) return MLLM_HIP_E_ALIGN;
   int8_t* q = reinterpret_cast<int8_t*>(workspace);
   float* xs = reinterpret_cast<float*>(reinterpret_cast<char*>(workspace) + align_up((size_t)M * K, 256));
   int rc = mllm_hip_per_token_quant_int8(x, x_dtype, q, xs, M, K, stream);
