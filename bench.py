@@ -134,10 +134,11 @@ def side_workloads(torch, ql, synth, gen):
     wsm = torch.empty(_lib_ws(ql, "moe", T, H, I, E, k), dtype=torch.uint8, device="cuda")
     ym = torch.empty((T, H), dtype=torch.float32, device="cuda")
     tm = ev_time(lambda: ql.moe_ffn_q(gate, up, down, x, ids, tw, workspace=wsm, out=ym), 10)
-    # the same layer at decode: 1 and 8 tokens, every (token, expert) pair a GEMV row, two launches; a graph of 16 calls
-    # over rotating routings (eager launches of this size would measure the host)
+    # the same layer with few tokens (1 and 8: decode; 16 and 32: short batches, still at most three pairs per expert): every
+    # (token, expert) pair a GEMV row, two launches; a graph of 16 calls over rotating routings (eager launches of this size
+    # would measure the host)
     dec = {}
-    for Td in (1, 8):
+    for Td in (1, 8, 16, 32):
         rngd = synth.rng_for(4, 100 + Td)
         routes = [synth.make_moe_routing(rngd, Td, E, k) for _ in range(16)]
         idl = [torch.from_numpy(r[0]).cuda() for r in routes]

@@ -902,9 +902,9 @@ struct Carver {
     return r;
   }
 };
-static RouteOut carve_route(Carver& c, int E, int64_t entries) {
+static RouteOut carve_route(Carver& c, int E, int64_t entries, int tile_h = TOK_TILE) {
   RouteOut o;
-  const size_t max_tiles = (size_t)E + (size_t)(entries / TOK_TILE) + 1;
+  const size_t max_tiles = (size_t)E + (size_t)(entries / tile_h) + 1;
   o.counts = c.take<int>(E);
   o.offsets = c.take<int>(E + 1);
   o.sorted_idx = c.take<int>(entries);
@@ -1031,7 +1031,28 @@ MLLM_API int mllm_hip_linear_q(int wtype, const void* packed, const void* x, int
 // decode path (moe_decode.hip): up to eight tokens as GEMVs, two launches
 namespace mllmhip {
 size_t moe_decode_workspace_bytes(int64_t T, int64_t I, int k);
-bool moe_decode_applies(int64_t T, int64_t H, int64_t I, int k);
+bool moe_decode_applies(int64_t T, int64_t H, int64_t I, int E, int k);
+int moe_decode_set_tokens(int tokens);
+bool moe_rows_applies(int64_t T, int64_t H, int64_t I, int E, int k);
+int moe_rows_set_tokens(int tokens);
+int moe_rows_tile();
+int launch_moe_rows(int wtype, const void* gate, const void* up, const void* down, const void* x, int x_dtype, const int* tile_expert,
+                    const int* tile_row0, const int* tile_rows, const int* ntiles, const int* sorted_idx, void* img, float* per,
+                    int64_t T, int64_t H, int64_t I, int E, int k, int x86, unsigned max_tiles, hipStream_t st);
+
+// workspace of the row-tile path: images of h, one down result per pair, routing with tiles of moe_rows_tile() rows
+struct RowsCarve {
+  unsigned char* img;
+  float* per;
+  RouteOut ro;
+};
+static RowsCarve carve_rows(Carver& c, int64_t T, int64_t H, int64_t I, int E, int k) {
+  RowsCarve r;
+  r.img = c.take<unsigned char>(moe_decode_workspace_bytes(T, I, k));
+  r.per = c.take<float>((size_t)T * k * H);
+  r.ro = carve_route(c, E, T * k, moe_rows_tile());
+  return r;
+}
 int launch_moe_decode(int wtype, const void* gate, const void* up, const void* down, const void* x, int x_dtype, const int32_t* ids,
                       const float* w, float* y, int64_t T, int64_t H, int64_t I, int E, int k, int x86, void* workspace,
                       hipStream_t st);
@@ -1046,8 +1067,19 @@ MLLM_API size_t mllm_hip_moe_workspace_bytes(int64_t T, int64_t H, int64_t I, in
   c.take<float>((size_t)T * k * (I / QK));
   c.take<float>((size_t)T * k * H);
   carve_route(c, E, T * k);
-  const size_t decode = moe_decode_applies(T, H, I, k) ? moe_decode_workspace_bytes(T, I, k) : 0;
-  return c.used > decode ? c.used : decode;
+  // whichever path the call then takes
+  const size_t decode = moe_decode_workspace_bytes(T, I, k);
+  Carver cr(nullptr);
+  carve_rows(cr, T, H, I, E, k);
+  const size_t most = c.used > cr.used ? c.used : cr.used;
+  return most > decode ? most : decode;
+}
+
+MLLM_API int mllm_hip_moe_set_tuning(int pair_tokens, int row_tokens) {
+  if (pair_tokens < 0 || pair_tokens > 4096 || row_tokens < 0 || row_tokens > 65536) return MLLM_HIP_E_BADARG;
+  moe_decode_set_tokens(pair_tokens);
+  moe_rows_set_tokens(row_tokens);
+  return 0;
 }
 
 MLLM_API int mllm_hip_moe_route(const int32_t* topk_ids, int64_t T, int E, int k, int32_t* counts, int32_t* offsets,
@@ -1078,9 +1110,24 @@ MLLM_API int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* 
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
   hipStream_t st = (hipStream_t)stream;
   const int x86 = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
-  // a handful of tokens: every (token, expert) pair is one GEMV row; two launches instead of five
-  if (moe_decode_applies(T, H, I, k))
+  // few pairs per expert: every (token, expert) pair is one GEMV row; two launches instead of five
+  if (moe_decode_applies(T, H, I, E, k))
     return launch_moe_decode(wtype, gate_packed, up_packed, down_packed, x, x_dtype, topk_ids, topk_w, y, T, H, I, E, k, x86, workspace, st);
+  // a few pairs per expert: the pairs sorted by expert, tiles of eight rows that share the expert's weights
+  if (moe_rows_applies(T, H, I, E, k)) {
+    Carver cr(workspace);
+    RowsCarve rc = carve_rows(cr, T, H, I, E, k);
+    const unsigned max_tiles = (unsigned)(E + (T * k) / moe_rows_tile() + 1);
+    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 5 * E * sizeof(int), st, topk_ids, (int)(T * k), E, moe_rows_tile(), rc.ro);
+    HIP_RET(hipGetLastError());
+    int r = launch_moe_rows(wtype, gate_packed, up_packed, down_packed, x, x_dtype, rc.ro.tile_expert, rc.ro.tile_row0, rc.ro.tile_rows,
+                            rc.ro.ntiles, rc.ro.sorted_idx, rc.img, rc.per, T, H, I, E, k, x86, max_tiles, st);
+    if (r) return r;
+    const int64_t total = T * H;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, rc.per, topk_w, topk_ids, y, T,
+                       (int)H, k, E);
+    return (int)hipGetLastError();
+  }
   Carver c(workspace);
   int8_t* xq = c.take<int8_t>((size_t)T * H);
   float* xd = c.take<float>((size_t)T * (H / QK));

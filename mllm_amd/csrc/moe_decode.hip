@@ -211,9 +211,21 @@ __host__ __device__ inline int moe_decode_img_stride(int64_t I) { return (int)al
 
 size_t moe_decode_workspace_bytes(int64_t T, int64_t I, int k) { return (size_t)T * k * moe_decode_img_stride(I); }
 
-bool moe_decode_applies(int64_t T, int64_t H, int64_t I, int k) {
-  return T <= 8 && I % 32 == 0 && I / QK <= 32 && H % 32 == 0 && k <= 64 && H / QK * 40 + 256 <= 64 * 1024 &&
-         (int64_t)k * moe_decode_img_stride(I) <= 64 * 1024;
+// Whether the per-pair kernels run.  They read an expert's matrices once per pair that uses it; measured at 128 experts,
+// top-8 (2048 x 768) they are the fastest form up to one pair per expert (16 tokens: 54 us; the eight-row tiles below 53 us, the
+// grouped 64-row tiles 144 us), and the row tiles from there on (32 tokens: 97 vs 76 us).
+// g_moe_decode_tokens > 0 replaces the rule by a token limit (comparison runs, tests).
+static int g_moe_decode_tokens = 0;
+int moe_decode_set_tokens(int tokens) {
+  if (tokens < 0 || tokens > 4096) return MLLM_HIP_E_BADARG;
+  g_moe_decode_tokens = tokens;
+  return 0;
+}
+
+bool moe_decode_applies(int64_t T, int64_t H, int64_t I, int E, int k) {
+  const bool few = g_moe_decode_tokens > 0 ? T <= g_moe_decode_tokens : (T <= 8 || (T <= 4096 && T * k <= (int64_t)E));
+  return few && I % 32 == 0 && I / QK <= 32 && H % 32 == 0 && k <= 64 && H / QK * 40 + 256 <= 64 * 1024 &&
+         (int64_t)k * moe_decode_img_stride(I) <= 64 * 1024 && T * k <= 65535;
 }
 
 int launch_moe_decode(int wtype, const void* gate, const void* up, const void* down, const void* x, int x_dtype, const int32_t* ids,
@@ -246,6 +258,238 @@ int launch_moe_decode(int wtype, const void* gate, const void* up, const void* d
   const dim3 g2((unsigned)(H / (8 * DNW)), (unsigned)T);
   if (wtype == MLLM_HIP_Q4_0) hipLaunchKernelGGL((moe_decode_down_kernel<MLLM_HIP_Q4_0>), g2, dim3(DNW * 64), lds2, st, a);
   else hipLaunchKernelGGL((moe_decode_down_kernel<MLLM_HIP_Q8_0>), g2, dim3(DNW * 64), lds2, st, a);
+  return (int)hipGetLastError();
+}
+
+// ---- a few rows per expert ------------------------------------------------------------------------------------------------
+// Between decode and prefill (up to about eight pairs per expert) the per-pair kernels read an expert's matrices once per
+// pair and the 64-row tiles of the grouped path are mostly empty.  Here the pairs are sorted by expert (the routing pass of
+// the grouped path with tiles of eight rows) and one workgroup serves the rows of one tile: the weights are read once per
+// tile, each row has its own Q8_0 image in LDS and its own accumulators.  Same block arithmetic and the same two stages as
+// above; the down stage writes one row per pair and the weighted sum over a token's slots is the grouped path's combine pass
+// (slot order, no atomics).
+constexpr int MOE_ROWS = 8;  // rows of a tile
+
+struct MoeRowsArgs {
+  MoeDecodeArgs d;
+  const int* tile_expert;
+  const int* tile_row0;
+  const int* tile_rows;
+  const int* ntiles;
+  const int* sorted_idx;  // flat index t*k + j at every expert-sorted position
+  float* per;             // [T*k][H] down results by flat index
+  int x_stride;           // bytes of one row's image of x in LDS
+};
+
+// gate / up / SiLU * up / re-quantization for the R (>= rows) rows of one tile; thread roles as in moe_decode_gateup_kernel
+template <int WT, int XT, int R>
+__device__ __forceinline__ void moe_rows_gateup(const MoeRowsArgs& b, const int e, const int row0, const int rows, unsigned char* smem) {
+  const MoeDecodeArgs& a = b.d;
+  const int nb = a.H / QK, nbp = (int)scale_row_stride(a.H);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * 32;
+  const int grp = lane >> 4, c0 = lane & 15;
+  const int n = n0 + 4 * wave + grp;
+  float* s_h = reinterpret_cast<float*>(smem + (size_t)MOE_ROWS * b.x_stride);
+
+  const PackedView wv[2] = {packed_view(WT, a.gate + (size_t)e * a.gu_stride, a.I, a.H), packed_view(WT, a.up + (size_t)e * a.gu_stride, a.I, a.H)};
+  constexpr int U = 2;  // block columns per lane and trip: with more, the unpacked codes of a trip no longer fit 128 registers
+  u32x4 w0[U][2], w1[WT == MLLM_HIP_Q8_0 ? U : 1][2];
+  uint16_t dw[U][2];
+  auto load_trip = [&](int t0) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int col = min(t0 + 16 * u + c0, nb - 1);
+#pragma unroll
+      for (int r = 0; r < 2; r++) {
+        const size_t blk = (size_t)n * nb + col;
+        w0[u][r] = wv[r].q0[blk];
+        if (WT == MLLM_HIP_Q8_0) w1[WT == MLLM_HIP_Q8_0 ? u : 0][r] = wv[r].q1[blk];
+        dw[u][r] = wv[r].d[(size_t)n * nbp + col];
+      }
+    }
+  };
+  load_trip(0);
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+
+  // the rows' activations -> Q8_0 images in LDS, four requests in flight per thread; items are eighths of a block, so the four
+  // lanes of a quad always hold one block of one row
+  const int nitems = nb * 4, total = rows * nitems;
+  for (int it0 = tid; it0 < total; it0 += 512 * 4) {
+    XRaw<XT> raw[4];
+    int rr[4], ii[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      const int it = min(it0 + 512 * q, total - 1);
+      rr[q] = it / nitems;
+      ii[q] = it - rr[q] * nitems;
+      const int tok = b.sorted_idx[row0 + rr[q]] / a.k;
+      load_x8<XT>(a.x, ((int64_t)tok * nitems + ii[q]) * 8, raw[q]);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+      if (it0 + 512 * q < total) {  // the same answer in the four lanes of a quad: total and the strides are multiples of 4
+        float v[8];
+        x8_to_f32<XT>(raw[q], v);
+        quad_quantize_to_image(v, QImage{smem + (size_t)rr[q] * b.x_stride, 1, nb, a.x86}, 0, ii[q] >> 2, ii[q] & 3, true);
+      }
+    }
+  }
+  __syncthreads();
+
+  float acc[R][2];
+#pragma unroll
+  for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = 0.f;
+  for (int t0 = 0; t0 < nb; t0 += 16 * U) {
+    if (t0) load_trip(t0);
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int col = t0 + 16 * u + c0;
+      if (col < nb) {
+        const float dg = f16bits_to_f32(dw[u][0]), du = f16bits_to_f32(dw[u][1]);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+          if (r < rows) {  // uniform
+            const unsigned char* im = smem + (size_t)r * b.x_stride;
+            const u32x4* s_lo = reinterpret_cast<const u32x4*>(im);
+            const u32x4 xlo = s_lo[col], xhi = s_lo[nb + col];
+            const float dx = reinterpret_cast<const float*>(s_lo + 2 * nb)[col];
+            const int n8 = reinterpret_cast<const int*>(s_lo + 2 * nb)[nb + col];
+            const int ig = block_dot<WT>(w0[u][0], w1[WT == MLLM_HIP_Q8_0 ? u : 0][0], xlo, xhi, n8);
+            const int iu = block_dot<WT>(w0[u][1], w1[WT == MLLM_HIP_Q8_0 ? u : 0][1], xlo, xhi, n8);
+            acc[r][0] = fmaf(dg * dx, (float)ig, acc[r][0]);
+            acc[r][1] = fmaf(du * dx, (float)iu, acc[r][1]);
+          }
+          __builtin_amdgcn_sched_barrier(0);  // one row's image block in registers at a time: two workgroups fit a CU
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    if (r < rows) {
+      const float g = group_sum<16>(acc[r][0]), u = group_sum<16>(acc[r][1]);
+      if (c0 == 0) s_h[r * 32 + 4 * wave + grp] = silu_vec(g) * u;
+    }
+  }
+  __syncthreads();
+  if (tid < 4 * rows) {  // one quad per row: the 32 values are exactly one Q8_0 block of that row's h
+    const int r = tid >> 2, j = tid & 3;
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) v[i] = s_h[r * 32 + 8 * j + i];
+    quad_quantize_to_image(v, QImage{a.img + (size_t)(row0 + r) * a.img_stride, 1, a.I / QK, a.x86}, 0, n0 / QK, j, true);
+  }
+}
+
+template <int WT, int XT>
+__global__ __launch_bounds__(512, 4) void moe_rows_gateup_kernel(MoeRowsArgs b) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int t = blockIdx.y;
+  if (t >= b.ntiles[0]) return;
+  const int e = b.tile_expert[t], row0 = b.tile_row0[t], rows = b.tile_rows[t];
+  if (rows <= 2) moe_rows_gateup<WT, XT, 2>(b, e, row0, rows, smem);
+  else if (rows <= 4) moe_rows_gateup<WT, XT, 4>(b, e, row0, rows, smem);
+  else moe_rows_gateup<WT, XT, MOE_ROWS>(b, e, row0, rows, smem);
+}
+
+// down projection of the rows of one tile: wave w, lane group grp (8 lanes) -> output row n = n0 + 8 w + grp
+template <int WT>
+__global__ __launch_bounds__(DNW * 64) void moe_rows_down_kernel(MoeRowsArgs b) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const MoeDecodeArgs& a = b.d;
+  const int t = blockIdx.y;
+  if (t >= b.ntiles[0]) return;
+  const int e = b.tile_expert[t], row0 = b.tile_row0[t], rows = b.tile_rows[t];
+  const int nb = a.I / QK, nbp = (int)scale_row_stride(a.I);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int grp = lane >> 3, c0 = lane & 7;
+  const int n = blockIdx.x * (8 * DNW) + 8 * wave + grp;
+  constexpr int U = 4;
+  u32x4 w0[U], w1[WT == MLLM_HIP_Q8_0 ? U : 1];
+  uint16_t dw[U];
+  const PackedView v = packed_view(WT, a.down + (size_t)e * a.d_stride, a.H, a.I);
+#pragma unroll
+  for (int u = 0; u < U; u++) {
+    const int col = min(8 * u + c0, nb - 1);
+    const size_t blk = (size_t)n * nb + col;
+    w0[u] = v.q0[blk];
+    if (WT == MLLM_HIP_Q8_0) w1[WT == MLLM_HIP_Q8_0 ? u : 0] = v.q1[blk];
+    dw[u] = v.d[(size_t)n * nbp + col];
+  }
+  // the images of the tile's rows are contiguous (sorted positions row0 .. row0 + rows - 1)
+  const int n16 = rows * a.img_stride / 16;
+  const u32x4* src = reinterpret_cast<const u32x4*>(a.img + (size_t)row0 * a.img_stride);
+  for (int c = tid; c < n16; c += DNW * 64) reinterpret_cast<u32x4*>(smem)[c] = src[c];
+  __syncthreads();
+  for (int r = 0; r < rows; r++) {  // uniform
+    const unsigned char* im = smem + (size_t)r * a.img_stride;
+    const u32x4* s_lo = reinterpret_cast<const u32x4*>(im);
+    const float* s_d = reinterpret_cast<const float*>(s_lo + 2 * nb);
+    const int* s_n8 = reinterpret_cast<const int*>(s_d + nb);
+    float acc = 0.f;
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int col = 8 * u + c0;
+      if (col < nb) {
+        const int isum = block_dot<WT>(w0[u], w1[WT == MLLM_HIP_Q8_0 ? u : 0], s_lo[col], s_lo[nb + col], s_n8[col]);
+        acc = fmaf(f16bits_to_f32(dw[u]) * s_d[col], (float)isum, acc);
+      }
+    }
+    const float val = group_sum<8>(acc);
+    if (c0 == 0) b.per[(size_t)b.sorted_idx[row0 + r] * a.H + n] = val;
+  }
+}
+
+// The row tiles run up to seven pairs per expert (measured as above: 64 tokens 116 us against 173 us for the grouped 64-row
+// tiles, 128 tokens 184 against 189 us); a token limit > 0 replaces the rule.
+static int g_moe_rows_tokens = 0;
+int moe_rows_set_tokens(int tokens) {
+  if (tokens < 0 || tokens > 65536) return MLLM_HIP_E_BADARG;
+  g_moe_rows_tokens = tokens;
+  return 0;
+}
+static size_t moe_rows_x_stride(int64_t H) { return align_up((size_t)(H / QK) * 40, 16); }
+bool moe_rows_applies(int64_t T, int64_t H, int64_t I, int E, int k) {
+  const bool few = g_moe_rows_tokens > 0 ? T <= g_moe_rows_tokens : T * k <= 7 * (int64_t)E;
+  return few && I % 32 == 0 && I / QK <= 32 && H % 32 == 0 && MOE_ROWS * moe_rows_x_stride(H) + MOE_ROWS * 32 * 4 <= 64 * 1024 &&
+         E + T * k / MOE_ROWS + 1 <= 65535;
+}
+int moe_rows_tile() { return MOE_ROWS; }
+
+// the two stages between the routing pass and the combine pass; img: T*k images of h (moe_decode_workspace_bytes)
+int launch_moe_rows(int wtype, const void* gate, const void* up, const void* down, const void* x, int x_dtype, const int* tile_expert,
+                    const int* tile_row0, const int* tile_rows, const int* ntiles, const int* sorted_idx, void* img, float* per,
+                    int64_t T, int64_t H, int64_t I, int E, int k, int x86, unsigned max_tiles, hipStream_t st) {
+  MoeRowsArgs b{};
+  MoeDecodeArgs& a = b.d;
+  a.gate = reinterpret_cast<const char*>(gate);
+  a.up = reinterpret_cast<const char*>(up);
+  a.down = reinterpret_cast<const char*>(down);
+  a.gu_stride = packed_bytes(wtype, I, H);
+  a.d_stride = packed_bytes(wtype, H, I);
+  a.x = x;
+  a.img = reinterpret_cast<unsigned char*>(img);
+  a.img_stride = moe_decode_img_stride(I);
+  a.T = (int)T; a.H = (int)H; a.I = (int)I; a.E = E; a.k = k; a.x86 = x86;
+  b.tile_expert = tile_expert; b.tile_row0 = tile_row0; b.tile_rows = tile_rows; b.ntiles = ntiles; b.sorted_idx = sorted_idx;
+  b.per = per;
+  b.x_stride = (int)moe_rows_x_stride(H);
+  const size_t lds1 = (size_t)MOE_ROWS * b.x_stride + MOE_ROWS * 32 * sizeof(float);
+  const dim3 g1((unsigned)(I / 32), max_tiles);
+#define GU(WT_, XT_) hipLaunchKernelGGL((moe_rows_gateup_kernel<WT_, XT_>), g1, dim3(512), lds1, st, b)
+  if (wtype == MLLM_HIP_Q4_0) {
+    if (x_dtype == MLLM_HIP_F32) GU(MLLM_HIP_Q4_0, MLLM_HIP_F32); else GU(MLLM_HIP_Q4_0, MLLM_HIP_BF16);
+  } else {
+    if (x_dtype == MLLM_HIP_F32) GU(MLLM_HIP_Q8_0, MLLM_HIP_F32); else GU(MLLM_HIP_Q8_0, MLLM_HIP_BF16);
+  }
+#undef GU
+  HIP_RET(hipGetLastError());
+  const size_t lds2 = (size_t)MOE_ROWS * a.img_stride;
+  const dim3 g2((unsigned)(H / (8 * DNW)), max_tiles);
+  if (wtype == MLLM_HIP_Q4_0) hipLaunchKernelGGL((moe_rows_down_kernel<MLLM_HIP_Q4_0>), g2, dim3(DNW * 64), lds2, st, b);
+  else hipLaunchKernelGGL((moe_rows_down_kernel<MLLM_HIP_Q8_0>), g2, dim3(DNW * 64), lds2, st, b);
   return (int)hipGetLastError();
 }
 

@@ -170,9 +170,11 @@ def test_moe_small(T, H, I, E, k, wtype):
 
 
 @pytest.mark.parametrize("T,H,I,E,k,wtype", [(1, 2048, 768, 128, 8, 0), (8, 2048, 768, 128, 8, 0), (3, 256, 96, 8, 3, 1), (5, 2048, 768, 16, 8, 1),
-                                              (2, 64, 32, 4, 4, 0), (7, 128, 1024, 6, 2, 0), (8, 4096, 32, 5, 1, 0)])
+                                              (2, 64, 32, 4, 4, 0), (7, 128, 1024, 6, 2, 0), (8, 4096, 32, 5, 1, 0),
+                                              (20, 2048, 768, 128, 8, 0), (12, 256, 96, 64, 4, 1), (48, 512, 64, 128, 8, 0)])
 def test_moe_decode_path(T, H, I, E, k, wtype):
-    """up to eight tokens: every (token, expert) pair as a GEMV row, two launches (Qwen3-30B-A3B dimensions included);
+    """few tokens under the default rule: up to eight tokens, or up to one pair per expert, every (token, expert) pair is a GEMV
+    row (two launches, Qwen3-30B-A3B dimensions included); the larger cases here run as eight-row tiles;
     fp32 block arithmetic as the CPU path, so close to the oracle; slots with an expert id outside [0, E) add nothing;
     permuting tokens permutes outputs bit for bit; bf16 activations"""
     rng = synth.rng_for(4, 5000 + T + H + I + E)
@@ -213,6 +215,57 @@ def test_moe_gemm_small(T, H, I, E, k, wtype):
     perm = rng.permutation(T)
     y2 = ql.moe_ffn_q_gemm(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
     assert np.array_equal(y2, y[perm])
+
+
+@pytest.mark.parametrize("T,wtype", [(6, 0), (24, 0), (40, 1), (100, 0)])
+def test_moe_pair_row_and_tile_kernels_agree(T, wtype):
+    """the per-pair kernels, the eight-row tiles and the grouped 64-row tiles follow the same block arithmetic: forced one way
+    or the other by the tuning override they agree to fp32 summation order (plus the odd flipped Q8_0 code of h), and all
+    match the oracle; slots with an expert id outside [0, E) add nothing on any of them"""
+    L = _lib.lib()
+    H, I, E, k = 512, 128, 32, 4
+    rng = synth.rng_for(4, 5300 + T)
+    Wg, Wu, Wd, ids, w, g, u, d = _moe_case(rng, T, H, I, E, k, wtype)
+    ids[0, 0] = E + 3
+    ids[T - 1, k - 1] = -1
+    x = synth.make_x_fp32(rng, T, H)
+    announce("moe pairs vs rows vs tiles", T, wtype)
+    ys = {}
+    try:
+        for name, (pt, rt) in {"pairs": (4096, 1), "rows": (1, 65536), "tiles": (1, 1)}.items():
+            assert L.mllm_hip_moe_set_tuning(pt, rt) == 0
+            ys[name] = ql.moe_ffn_q(g, u, d, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+    finally:
+        L.mllm_hip_moe_set_tuning(0, 0)
+    want = orc.moe_ffn(x, ids, w, Wg, Wu, Wd, wtype)
+    for name, y in ys.items():
+        assert rel_l2(y, want) < 2e-4, (name, rel_l2(y, want))
+    assert rel_l2(ys["pairs"], ys["tiles"]) < 2e-4 and rel_l2(ys["rows"], ys["tiles"]) < 2e-4
+    assert L.mllm_hip_moe_set_tuning(-1, 0) == -1
+
+
+@pytest.mark.parametrize("T,H,I,E,k,wtype", [(64, 2048, 768, 128, 8, 0), (100, 2048, 768, 128, 8, 1), (9, 64, 32, 2, 2, 0),
+                                              (33, 256, 1024, 7, 3, 1), (150, 4096 + 32, 96, 128, 8, 0)])
+def test_moe_row_tiles(T, H, I, E, k, wtype):
+    """a few pairs per expert (Qwen3-30B-A3B dimensions at 64 and 100 tokens; one expert with many tiles; ragged last tiles): the
+    pairs sorted by expert, eight rows per workgroup; permuting tokens permutes outputs bit for bit; bf16 activations"""
+    rng = synth.rng_for(4, 5600 + T + H + I + E)
+    Wg, Wu, Wd, ids, w, g, u, d = _moe_case(rng, T, H, I, E, k, wtype)
+    x = synth.make_x_fp32(rng, T, H)
+    announce("moe row tiles", T, H, I, E, k, wtype)
+    L = _lib.lib()
+    try:
+        assert L.mllm_hip_moe_set_tuning(1, 65536) == 0
+        y = ql.moe_ffn_q(g, u, d, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+        perm = rng.permutation(T)
+        y2 = ql.moe_ffn_q(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
+        bits, xb = synth.make_x_bf16(rng, T, H)
+        y4 = ql.moe_ffn_q(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
+    finally:
+        L.mllm_hip_moe_set_tuning(0, 0)
+    assert rel_l2(y, orc.moe_ffn(x, ids, w, Wg, Wu, Wd, wtype)) < 2e-4
+    assert np.array_equal(y2, y[perm])
+    assert rel_l2(y4, orc.moe_ffn(xb, ids, w, Wg, Wu, Wd, wtype)) < 2e-4
 
 
 def test_moe_gemm_full_size():
