@@ -281,7 +281,7 @@ int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed
                        int64_t I, int E, int k, int act_scale_mode, void* workspace, void* stream);
 
 /* mllm_hip_moe_ffn_q has three forms: every (token, expert) pair as GEMV rows (up to eight tokens or one pair per
- * expert), the pairs sorted by expert in tiles of eight rows that share the expert's weights (up to seven pairs per expert), and
+ * expert), the pairs sorted by expert in tiles of eight rows that share the expert's weights (up to ten pairs per expert), and
  * the grouped 64-row tiles.  Tuning override: token counts up to which the first and the second run (0 = the rule above; 1
  * keeps a form to single-token calls).  No counterpart in the reference (its loop over experts is the same for any T). */
 int mllm_hip_moe_set_tuning(int pair_tokens, int row_tokens);

@@ -293,9 +293,10 @@ __device__ __forceinline__ void moe_rows_gateup(const MoeRowsArgs& b, const int 
   float* s_h = reinterpret_cast<float*>(smem + (size_t)MOE_ROWS * b.x_stride);
 
   const PackedView wv[2] = {packed_view(WT, a.gate + (size_t)e * a.gu_stride, a.I, a.H), packed_view(WT, a.up + (size_t)e * a.gu_stride, a.I, a.H)};
-  constexpr int U = 2;  // block columns per lane and trip: with more, the unpacked codes of a trip no longer fit 128 registers
-  u32x4 w0[U][2], w1[WT == MLLM_HIP_Q8_0 ? U : 1][2];
-  uint16_t dw[U][2];
+  constexpr int U = (R > 4 || (R > 2 && WT == MLLM_HIP_Q8_0)) ? 1 : 2;  // block columns per lane and trip, as 128 registers allow
+  // two register sets: the next trip's weights are requested before the current trip is multiplied
+  u32x4 w0[U][2], w1[WT == MLLM_HIP_Q8_0 ? U : 1][2], w0n[U][2], w1n[WT == MLLM_HIP_Q8_0 ? U : 1][2];
+  uint16_t dw[U][2], dwn[U][2];
   auto load_trip = [&](int t0) {
 #pragma unroll
     for (int u = 0; u < U; u++) {
@@ -303,9 +304,9 @@ __device__ __forceinline__ void moe_rows_gateup(const MoeRowsArgs& b, const int 
 #pragma unroll
       for (int r = 0; r < 2; r++) {
         const size_t blk = (size_t)n * nb + col;
-        w0[u][r] = wv[r].q0[blk];
-        if (WT == MLLM_HIP_Q8_0) w1[WT == MLLM_HIP_Q8_0 ? u : 0][r] = wv[r].q1[blk];
-        dw[u][r] = wv[r].d[(size_t)n * nbp + col];
+        w0n[u][r] = wv[r].q0[blk];
+        if (WT == MLLM_HIP_Q8_0) w1n[WT == MLLM_HIP_Q8_0 ? u : 0][r] = wv[r].q1[blk];
+        dwn[u][r] = wv[r].d[(size_t)n * nbp + col];
       }
     }
   };
@@ -342,7 +343,15 @@ __device__ __forceinline__ void moe_rows_gateup(const MoeRowsArgs& b, const int 
 #pragma unroll
   for (int r = 0; r < R; r++) acc[r][0] = acc[r][1] = 0.f;
   for (int t0 = 0; t0 < nb; t0 += 16 * U) {
-    if (t0) load_trip(t0);
+#pragma unroll
+    for (int u = 0; u < U; u++)
+#pragma unroll
+      for (int r = 0; r < 2; r++) {
+        w0[u][r] = w0n[u][r];
+        if (WT == MLLM_HIP_Q8_0) w1[WT == MLLM_HIP_Q8_0 ? u : 0][r] = w1n[WT == MLLM_HIP_Q8_0 ? u : 0][r];
+        dw[u][r] = dwn[u][r];
+      }
+    if (t0 + 16 * U < nb) load_trip(t0 + 16 * U);  // uniform
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const int col = t0 + 16 * u + c0;
@@ -394,9 +403,9 @@ __global__ __launch_bounds__(512, 4) void moe_rows_gateup_kernel(MoeRowsArgs b) 
   else moe_rows_gateup<WT, XT, MOE_ROWS>(b, e, row0, rows, smem);
 }
 
-// down projection of the rows of one tile: wave w, lane group grp (8 lanes) -> output row n = n0 + 8 w + grp
-template <int WT>
-__global__ __launch_bounds__(DNW * 64) void moe_rows_down_kernel(MoeRowsArgs b) {
+// down projection of the rows of one tile: NW waves, wave w, lane group grp (8 lanes) -> output row n = n0 + 8 w + grp
+template <int WT, int NW>
+__global__ __launch_bounds__(NW * 64) void moe_rows_down_kernel(MoeRowsArgs b) {
   extern __shared__ __align__(16) unsigned char smem[];
   const MoeDecodeArgs& a = b.d;
   const int t = blockIdx.y;
@@ -405,7 +414,7 @@ __global__ __launch_bounds__(DNW * 64) void moe_rows_down_kernel(MoeRowsArgs b) 
   const int nb = a.I / QK, nbp = (int)scale_row_stride(a.I);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int grp = lane >> 3, c0 = lane & 7;
-  const int n = blockIdx.x * (8 * DNW) + 8 * wave + grp;
+  const int n = blockIdx.x * (8 * NW) + 8 * wave + grp;
   constexpr int U = 4;
   u32x4 w0[U], w1[WT == MLLM_HIP_Q8_0 ? U : 1];
   uint16_t dw[U];
@@ -421,7 +430,7 @@ __global__ __launch_bounds__(DNW * 64) void moe_rows_down_kernel(MoeRowsArgs b) 
   // the images of the tile's rows are contiguous (sorted positions row0 .. row0 + rows - 1)
   const int n16 = rows * a.img_stride / 16;
   const u32x4* src = reinterpret_cast<const u32x4*>(a.img + (size_t)row0 * a.img_stride);
-  for (int c = tid; c < n16; c += DNW * 64) reinterpret_cast<u32x4*>(smem)[c] = src[c];
+  for (int c = tid; c < n16; c += NW * 64) reinterpret_cast<u32x4*>(smem)[c] = src[c];
   __syncthreads();
   for (int r = 0; r < rows; r++) {  // uniform
     const unsigned char* im = smem + (size_t)r * a.img_stride;
@@ -442,8 +451,8 @@ __global__ __launch_bounds__(DNW * 64) void moe_rows_down_kernel(MoeRowsArgs b) 
   }
 }
 
-// The row tiles run up to seven pairs per expert (measured as above: 64 tokens 116 us against 173 us for the grouped 64-row
-// tiles, 128 tokens 184 against 189 us); a token limit > 0 replaces the rule.
+// The row tiles run up to ten pairs per expert (measured as above: 64 tokens 105 us against 175 us for the grouped 64-row
+// tiles, 160 tokens 181 against 194 us, 192 tokens 215 against 198 us); a token limit > 0 replaces the rule.
 static int g_moe_rows_tokens = 0;
 int moe_rows_set_tokens(int tokens) {
   if (tokens < 0 || tokens > 65536) return MLLM_HIP_E_BADARG;
@@ -452,7 +461,7 @@ int moe_rows_set_tokens(int tokens) {
 }
 static size_t moe_rows_x_stride(int64_t H) { return align_up((size_t)(H / QK) * 40, 16); }
 bool moe_rows_applies(int64_t T, int64_t H, int64_t I, int E, int k) {
-  const bool few = g_moe_rows_tokens > 0 ? T <= g_moe_rows_tokens : T * k <= 7 * (int64_t)E;
+  const bool few = g_moe_rows_tokens > 0 ? T <= g_moe_rows_tokens : T * k <= 10 * (int64_t)E;
   return few && I % 32 == 0 && I / QK <= 32 && H % 32 == 0 && MOE_ROWS * moe_rows_x_stride(H) + MOE_ROWS * 32 * 4 <= 64 * 1024 &&
          E + T * k / MOE_ROWS + 1 <= 65535;
 }
@@ -487,9 +496,17 @@ int launch_moe_rows(int wtype, const void* gate, const void* up, const void* dow
 #undef GU
   HIP_RET(hipGetLastError());
   const size_t lds2 = (size_t)MOE_ROWS * a.img_stride;
-  const dim3 g2((unsigned)(H / (8 * DNW)), max_tiles);
-  if (wtype == MLLM_HIP_Q4_0) hipLaunchKernelGGL((moe_rows_down_kernel<MLLM_HIP_Q4_0>), g2, dim3(DNW * 64), lds2, st, b);
-  else hipLaunchKernelGGL((moe_rows_down_kernel<MLLM_HIP_Q8_0>), g2, dim3(DNW * 64), lds2, st, b);
+  // 64 output rows per workgroup where H allows (a tile's images are copied into LDS once per workgroup, and eight times
+  // fewer workgroups are dispatched), else 16
+  if (H % 64 == 0) {
+    const dim3 g2((unsigned)(H / 64), max_tiles);
+    if (wtype == MLLM_HIP_Q4_0) hipLaunchKernelGGL((moe_rows_down_kernel<MLLM_HIP_Q4_0, 8>), g2, dim3(512), lds2, st, b);
+    else hipLaunchKernelGGL((moe_rows_down_kernel<MLLM_HIP_Q8_0, 8>), g2, dim3(512), lds2, st, b);
+  } else {
+    const dim3 g2((unsigned)(H / 16), max_tiles);
+    if (wtype == MLLM_HIP_Q4_0) hipLaunchKernelGGL((moe_rows_down_kernel<MLLM_HIP_Q4_0, 2>), g2, dim3(128), lds2, st, b);
+    else hipLaunchKernelGGL((moe_rows_down_kernel<MLLM_HIP_Q8_0, 2>), g2, dim3(128), lds2, st, b);
+  }
   return (int)hipGetLastError();
 }
 
