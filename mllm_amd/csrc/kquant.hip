@@ -23,8 +23,10 @@
 namespace mllmhip {
 
 // ---- packed layout ---------------------------------------------------------------------------------------------------
-// Q4_K: plane A = nibbles, 128 B per super-block (eight 16-byte chunks); plane S = {fp16 d, fp16 dmin, 12 B of 6-bit scales
-//       and mins} = 16 B per super-block, fp16 fields as IEEE patterns.
+// Q4_K: plane A = nibbles, 128 B per super-block (eight 16-byte chunks); plane S = the 6-bit scales and mins decoded to bytes
+//       at load time, one dword per pair of sub-blocks {sc[2p], sc[2p+1], m[2p], m[2p+1]} = 16 B per super-block (a lane of
+//       the GEMV needs exactly the dword of its chunk's pair: no bit shuffle per chunk); plane D = {fp16 d, fp16 dmin} as
+//       IEEE patterns, 4 B per super-block.
 // Q6_K: plane A = low nibbles (128 B per super-block), plane H = high bit pairs (64 B), plane S = 16 int8 scales, plane D =
 //       fp16 d as IEEE pattern (2 B).
 struct KView {
@@ -36,7 +38,7 @@ struct KView {
 __host__ __device__ inline size_t kq_plane(size_t bytes) { return align_up(bytes, 256); }
 __host__ __device__ inline size_t kq_packed_bytes(int wtype, int64_t N, int64_t K) {
   const size_t sb = (size_t)N * (K / QK_K);
-  if (wtype == MLLM_HIP_Q4_K) return kq_plane(sb * 128) + kq_plane(sb * 16);
+  if (wtype == MLLM_HIP_Q4_K) return kq_plane(sb * 128) + kq_plane(sb * 16) + kq_plane(sb * 4);
   return kq_plane(sb * 128) + kq_plane(sb * 64) + kq_plane(sb * 16) + kq_plane(sb * 2);
 }
 __host__ __device__ inline KView kq_view(int wtype, const void* packed, int64_t N, int64_t K) {
@@ -67,39 +69,6 @@ __device__ __forceinline__ uint32_t bytes_u32(const uint8_t* p) {
   return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
 }
 
-// one thread per 16-byte record of plane A (Q4_K: 8 per super-block; Q6_K: 8 per super-block); thread 0 of a super-block
-// also writes the small planes
-__global__ void kq_prepack_kernel(int wtype, const uint8_t* __restrict__ blocks, int x86, KView v, int64_t nsb_total) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t sb = i >> 3;
-  const int c = (int)(i & 7);
-  if (sb >= nsb_total) return;
-  u32x4* A = const_cast<u32x4*>(v.a);
-  u32x4* S = const_cast<u32x4*>(v.s);
-  if (wtype == MLLM_HIP_Q4_K) {
-    const uint8_t* b = blocks + sb * 144;
-    const uint8_t* q = b + 16 + 16 * c;
-    A[sb * 8 + c] = u32x4{bytes_u32(q), bytes_u32(q + 4), bytes_u32(q + 8), bytes_u32(q + 12)};
-    if (c == 0) {
-      const uint32_t dd = (uint32_t)field_bits(b, x86) | ((uint32_t)field_bits(b + 2, x86) << 16);
-      S[sb] = u32x4{dd, bytes_u32(b + 4), bytes_u32(b + 8), bytes_u32(b + 12)};
-    }
-  } else {
-    const uint8_t* b = blocks + sb * 210;
-    const uint8_t* q = b + 16 * c;
-    A[sb * 8 + c] = u32x4{bytes_u32(q), bytes_u32(q + 4), bytes_u32(q + 8), bytes_u32(q + 12)};
-    if (c < 4) {
-      const uint8_t* hq = b + 128 + 16 * c;
-      const_cast<u32x4*>(v.h)[sb * 4 + c] = u32x4{bytes_u32(hq), bytes_u32(hq + 4), bytes_u32(hq + 8), bytes_u32(hq + 12)};
-    }
-    if (c == 0) {
-      const uint8_t* s = b + 192;
-      S[sb] = u32x4{bytes_u32(s), bytes_u32(s + 4), bytes_u32(s + 8), bytes_u32(s + 12)};
-      const_cast<uint16_t*>(v.d)[sb] = field_bits(b + 208, x86);
-    }
-  }
-}
-
 // ---- scale decoding ----------------------------------------------------------------------------------------------------
 // the 6-bit scales and mins of a Q4_K super-block as bytes: sc[0..7] in (lo, hi) of `sc`, mins likewise
 // (get_scale_min_k4, quantize.hpp; the same bit shuffle as vec_dot.cpp:507-512)
@@ -118,6 +87,45 @@ __device__ __forceinline__ int byte_of(uint32_t lo, uint32_t hi, int k) {  // k 
   return (int)(((k < 4 ? lo : hi) >> (8 * (k & 3))) & 0xffu);
 }
 
+// one thread per 16-byte record of plane A (Q4_K: 8 per super-block; Q6_K: 8 per super-block); thread 0 of a super-block
+// also writes the small planes
+__global__ void kq_prepack_kernel(int wtype, const uint8_t* __restrict__ blocks, int x86, KView v, int64_t nsb_total) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t sb = i >> 3;
+  const int c = (int)(i & 7);
+  if (sb >= nsb_total) return;
+  u32x4* A = const_cast<u32x4*>(v.a);
+  u32x4* S = const_cast<u32x4*>(v.s);
+  if (wtype == MLLM_HIP_Q4_K) {
+    const uint8_t* b = blocks + sb * 144;
+    const uint8_t* q = b + 16 + 16 * c;
+    A[sb * 8 + c] = u32x4{bytes_u32(q), bytes_u32(q + 4), bytes_u32(q + 8), bytes_u32(q + 12)};
+    if (c == 0) {
+      const K4Scales k = k4_scales(bytes_u32(b + 4), bytes_u32(b + 8), bytes_u32(b + 12));
+      uint32_t rec[4];
+#pragma unroll
+      for (int p = 0; p < 4; p++)
+        rec[p] = (uint32_t)byte_of(k.sc0, k.sc1, 2 * p) | ((uint32_t)byte_of(k.sc0, k.sc1, 2 * p + 1) << 8) |
+                 ((uint32_t)byte_of(k.mn0, k.mn1, 2 * p) << 16) | ((uint32_t)byte_of(k.mn0, k.mn1, 2 * p + 1) << 24);
+      S[sb] = u32x4{rec[0], rec[1], rec[2], rec[3]};
+      reinterpret_cast<uint32_t*>(const_cast<uint16_t*>(v.d))[sb] = (uint32_t)field_bits(b, x86) | ((uint32_t)field_bits(b + 2, x86) << 16);
+    }
+  } else {
+    const uint8_t* b = blocks + sb * 210;
+    const uint8_t* q = b + 16 * c;
+    A[sb * 8 + c] = u32x4{bytes_u32(q), bytes_u32(q + 4), bytes_u32(q + 8), bytes_u32(q + 12)};
+    if (c < 4) {
+      const uint8_t* hq = b + 128 + 16 * c;
+      const_cast<u32x4*>(v.h)[sb * 4 + c] = u32x4{bytes_u32(hq), bytes_u32(hq + 4), bytes_u32(hq + 8), bytes_u32(hq + 12)};
+    }
+    if (c == 0) {
+      const uint8_t* s = b + 192;
+      S[sb] = u32x4{bytes_u32(s), bytes_u32(s + 4), bytes_u32(s + 8), bytes_u32(s + 12)};
+      const_cast<uint16_t*>(v.d)[sb] = field_bits(b + 208, x86);
+    }
+  }
+}
+
 // ---- dequantization probe ------------------------------------------------------------------------------------------------
 __global__ void kq_dequantize_kernel(int wtype, KView v, float* __restrict__ w, int64_t nsb_total) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;  // one thread per element
@@ -126,12 +134,12 @@ __global__ void kq_dequantize_kernel(int wtype, KView v, float* __restrict__ w, 
   if (sb >= nsb_total) return;
   const uint8_t* A = reinterpret_cast<const uint8_t*>(v.a) + sb * 128;
   if (wtype == MLLM_HIP_Q4_K) {
-    const u32x4 s = v.s[sb];
-    const float d = f16bits_to_f32((uint16_t)(s.x & 0xffff)), mn = f16bits_to_f32((uint16_t)(s.x >> 16));
-    const K4Scales k = k4_scales(s.y, s.z, s.w);
+    const uint32_t dd = reinterpret_cast<const uint32_t*>(v.d)[sb];
+    const float d = f16bits_to_f32((uint16_t)(dd & 0xffff)), mn = f16bits_to_f32((uint16_t)(dd >> 16));
     const int j = e >> 5, l = e & 31;  // sub-block, element
+    const uint32_t rec = reinterpret_cast<const uint32_t*>(v.s)[sb * 4 + (j >> 1)];
     const int q = (j & 1) ? (A[32 * (j >> 1) + l] >> 4) : (A[32 * (j >> 1) + l] & 0xF);
-    const float d1 = d * (float)byte_of(k.sc0, k.sc1, j), m1 = mn * (float)byte_of(k.mn0, k.mn1, j);
+    const float d1 = d * (float)((rec >> (8 * (j & 1))) & 0xffu), m1 = mn * (float)((rec >> (16 + 8 * (j & 1))) & 0xffu);
     w[i] = d1 * (float)q - m1;
   } else {
     const uint8_t* H = reinterpret_cast<const uint8_t*>(v.h) + sb * 64;
@@ -278,7 +286,8 @@ __device__ __forceinline__ void load_unit(KUnit<WT>& u, const KRsrc& r, uint32_t
   if (WT == MLLM_HIP_Q4_K) {
     const uint32_t sb = sb_base + (uint32_t)(unit >> 3);
     u.a = __builtin_amdgcn_raw_buffer_load_b128(r.a, ok ? (sb * 8u + (uint32_t)(unit & 7)) * 16u : KBUF_OOB, 0, KBUF_NT);
-    u.s = __builtin_amdgcn_raw_buffer_load_b128(r.s, ok ? sb * 16u : KBUF_OOB, 0, KBUF_NT);
+    u.s.x = __builtin_amdgcn_raw_buffer_load_b32(r.s, ok ? sb * 16u + (uint32_t)((unit >> 1) & 3) * 4u : KBUF_OOB, 0, KBUF_NT);  // its pair's scales
+    u.s.y = __builtin_amdgcn_raw_buffer_load_b32(r.d, ok ? sb * 4u : KBUF_OOB, 0, KBUF_NT);                                      // d, dmin
   } else {
     const uint32_t sb = sb_base + (uint32_t)(unit >> 2);
     const uint32_t n = (uint32_t)(unit >> 1) & 1u, t = (uint32_t)unit & 1u;
@@ -303,8 +312,8 @@ __device__ __forceinline__ int half16(uint32_t pair, int hi) { return (int)(int1
 // stride over the row's units.  x is quantized to Q8_K once per workgroup into LDS: codes [MT][K], scales [MT][nsb], sums
 // of 16 as int16 [MT][nsb][16].
 // U = units a lane keeps in flight per row and trip.
-template <int WT, int XT, int MT, int G, int R, int U>
-__global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
+template <int WT, int XT, int MT, int G, int R, int U, int LB = 256>
+__global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int nsb = a.nsb;
   const int K = nsb * QK_K;
@@ -314,7 +323,7 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   constexpr int GROUPS = 64 / G;
   const int grp = lane / G, c0 = lane % G;
-  const int nthreads = blockDim.x;  // 64, 128 or 256
+  const int nthreads = blockDim.x;  // 64 .. LB
   int pidx = 0;  // uniform: which matrix this workgroup works on
 #pragma unroll
   for (int p = 1; p < KQ_MAX_PARTS; p++)
@@ -330,7 +339,7 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
     rs.a = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.a), 0, sbt * 128u, 0x00020000);
     rs.h = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(WT == MLLM_HIP_Q6_K ? pt.w.h : pt.w.a), 0, sbt * 64u, 0x00020000);
     rs.s = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.s), 0, sbt * 16u, 0x00020000);
-    rs.d = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(pt.w.d), 0, sbt * 2u, 0x00020000);
+    rs.d = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(pt.w.d), 0, sbt * (WT == MLLM_HIP_Q4_K ? 4u : 2u), 0x00020000);
   }
   // Memory requests return in order: the activations a thread will quantize (its first two items) are requested first,
   // then the first trip of weights, so that the quantization runs while the weights are still on their way.
@@ -437,13 +446,13 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
         u32x4 wlo[R], whi[R];
 #pragma unroll
         for (int r = 0; r < R; r++) {
-          const K4Scales k = k4_scales(cu[r].s.y, cu[r].s.z, cu[r].s.w);
-          sc_lo[r] = byte_of(k.sc0, k.sc1, 2 * jp);
-          sc_hi[r] = byte_of(k.sc0, k.sc1, 2 * jp + 1);
-          mn_lo[r] = byte_of(k.mn0, k.mn1, 2 * jp);
-          mn_hi[r] = byte_of(k.mn0, k.mn1, 2 * jp + 1);
-          dw[r] = f16bits_to_f32((uint16_t)(cu[r].s.x & 0xffffu));
-          dmw[r] = f16bits_to_f32((uint16_t)(cu[r].s.x >> 16));
+          const uint32_t rec = cu[r].s.x;  // {sc[2jp], sc[2jp+1], m[2jp], m[2jp+1]}
+          sc_lo[r] = (int)(rec & 0xffu);
+          sc_hi[r] = (int)((rec >> 8) & 0xffu);
+          mn_lo[r] = (int)((rec >> 16) & 0xffu);
+          mn_hi[r] = (int)(rec >> 24);
+          dw[r] = f16bits_to_f32((uint16_t)(cu[r].s.y & 0xffffu));
+          dmw[r] = f16bits_to_f32((uint16_t)(cu[r].s.y >> 16));
           const uint32_t m4 = 0x0f0f0f0fu;
           wlo[r] = u32x4{cu[r].a.x & m4, cu[r].a.y & m4, cu[r].a.z & m4, cu[r].a.w & m4};
           whi[r] = u32x4{(cu[r].a.x >> 4) & m4, (cu[r].a.y >> 4) & m4, (cu[r].a.z >> 4) & m4, (cu[r].a.w >> 4) & m4};
@@ -524,9 +533,13 @@ __global__ __launch_bounds__(256) void kq_gemv_kernel(KGemvArgs a) {
 
 static int g_kq_G = 0, g_kq_NW = 0, g_kq_U = 0;  // tuning overrides (0 = heuristic)
 
-template <int WT, int XT, int MT, int G, int U>
+// R1: one weight row per lane group and up to 16 waves per workgroup (few rows of many units: o_proj, down_proj).  The
+// quantization of x is the long part of such a workgroup, so it is shared by as many rows as still fill the CUs.
+template <int WT, int XT, int MT, int G, int U, bool R1 = false>
 static int launch_kq_u(const KGemvArgs& a_in, int NW, hipStream_t st) {
-  constexpr int R = (WT == MLLM_HIP_Q4_K && MT >= 4) ? 4 : 2;  // wider row tiles reuse every LDS read for more weight rows
+  constexpr int R = R1 ? 1 : (WT == MLLM_HIP_Q4_K && MT >= 4) ? 4 : 2;  // wider row tiles reuse every LDS read for more weight rows
+  constexpr int LB = R1 ? 1024 : 256;
+  if (NW < 1 || NW * 64 > LB) return MLLM_HIP_E_BADARG;  // the kernel is compiled for at most LB threads
   const int rows_per_wg = NW * (64 / G) * R;
   const int K = a_in.nsb * QK_K;
   const size_t lds = (size_t)MT * K + (size_t)MT * a_in.nsb * 4 + (size_t)MT * a_in.nsb * 32;
@@ -538,14 +551,15 @@ static int launch_kq_u(const KGemvArgs& a_in, int NW, hipStream_t st) {
     grid += (unsigned)((a.part[p].N + rows_per_wg - 1) / rows_per_wg);
   }
   a.wg_start[a.nparts] = (int)grid;
-  auto kern = kq_gemv_kernel<WT, XT, MT, G, R, U>;
+  auto kern = kq_gemv_kernel<WT, XT, MT, G, R, U, LB>;
   if (lds > 64 * 1024)
     HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 template <int WT, int XT, int MT, int G>
-static int launch_kq_g(const KGemvArgs& a, int NW, int U, hipStream_t st) {
+static int launch_kq_g(const KGemvArgs& a, int NW, int U, bool r1, hipStream_t st) {
+  if (r1 && MT <= 2 && G >= 32) return launch_kq_u<WT, XT, MT, G, (MT <= 2 && G >= 32 && WT == MLLM_HIP_Q4_K) ? 4 : 1, (MT <= 2 && G >= 32)>(a, NW, st);
   if (WT == MLLM_HIP_Q4_K && U >= 4 && MT <= 2) return launch_kq_u<WT, XT, MT, G, (WT == MLLM_HIP_Q4_K && MT <= 2) ? 4 : 1>(a, NW, st);
   if (U >= 2 && MT <= 2) return launch_kq_u<WT, XT, MT, G, MT <= 2 ? 2 : 1>(a, NW, st);
   return launch_kq_u<WT, XT, MT, G, 1>(a, NW, st);
@@ -564,13 +578,21 @@ static int launch_kq_m(const KGemvArgs& a, hipStream_t st) {
   for (int p = 0; p < a.nparts; p++) rows += a.part[p].N;
   const int grid = (int)((rows + NW * (64 / best) * 2 - 1) / (NW * (64 / best) * 2));
   int U = (WT == MLLM_HIP_Q4_K && grid < 512) ? 4 : 1;
+  // few rows of many units (o_proj, down_proj): large workgroups of one row per lane group, the whole wave on a row when it is
+  // long enough to keep 64 lanes busy for a trip
+  // (only with at least 32 lanes per row: the narrower shapes have no such variant and keep their 256-thread workgroups)
+  const bool r1 = MT <= 2 && grid < (WT == MLLM_HIP_Q4_K ? 256 : 512) && best >= 32 && !g_kq_NW && !g_kq_G;
+  if (r1) {
+    if (units >= 64 * 4) best = 64;
+    NW = best == 64 ? 16 : 8;  // 16 rows per workgroup either way
+  }  // (many rows, K = 2560: eight waves per workgroup measured slower than four, 11.0 against 9.6 us for gate + up)
   if (g_kq_G) best = g_kq_G;
   if (g_kq_NW) NW = g_kq_NW;
   if (g_kq_U) U = g_kq_U;
-  if (best == 64) return launch_kq_g<WT, XT, MT, 64>(a, NW, U, st);
-  if (best == 32) return launch_kq_g<WT, XT, MT, 32>(a, NW, U, st);
-  if (best == 16) return launch_kq_g<WT, XT, MT, 16>(a, NW, U, st);
-  return launch_kq_g<WT, XT, MT, 8>(a, NW, U, st);
+  if (best == 64) return launch_kq_g<WT, XT, MT, 64>(a, NW, U, r1, st);
+  if (best == 32) return launch_kq_g<WT, XT, MT, 32>(a, NW, U, r1, st);
+  if (best == 16) return launch_kq_g<WT, XT, MT, 16>(a, NW, U, r1, st);
+  return launch_kq_g<WT, XT, MT, 8>(a, NW, U, r1, st);
 }
 template <int WT, int XT>
 static int launch_kq(const KGemvArgs& a, hipStream_t st) {
@@ -642,14 +664,18 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
   const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.a), 0, sbt * 128u, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.s), 0, sbt * 16u, 0x00020000);
   const int spb = nbs >> 3;  // super-blocks per slice (at most 8)
+  const __amdgpu_buffer_rsrc_t rdd = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(pt.w.d), 0, sbt * 4u, 0x00020000);
   u32x4 sc[2];
+  uint32_t scd[2];
 #pragma unroll
   for (int k = 0; k < 2; k++) {
     const int ch = lane + 64 * k;
     const int r = ch / spb, si = ch - r * spb;
     const int sb256 = (b0 >> 3) + si;
     const bool ok = tile_ok && r < 16 && row0 + r < N && sb256 < nsb;
-    sc[k] = __builtin_amdgcn_raw_buffer_load_b128(rsc, ok ? ((uint32_t)(row0 + r) * (uint32_t)nsb + (uint32_t)sb256) * 16u : KBUF_OOB, 0, KBUF_NT);
+    const uint32_t rec = (uint32_t)(row0 + r) * (uint32_t)nsb + (uint32_t)sb256;
+    sc[k] = __builtin_amdgcn_raw_buffer_load_b128(rsc, ok ? rec * 16u : KBUF_OOB, 0, KBUF_NT);
+    scd[k] = __builtin_amdgcn_raw_buffer_load_b32(rdd, ok ? rec * 4u : KBUF_OOB, 0, KBUF_NT);
   }
   // ---- 2. weight codes: lane (row c, group g) takes records b0 + 4 j + g ------------------------------------------------------
   const int c = lane & 15, g = lane >> 4;
@@ -706,12 +732,12 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
     const int r = ch / spb, si = ch - r * spb;
     if (r < 16) {
       const bool in = (b0 >> 3) + si < nsb;
-      const float d = f16bits_to_f32((uint16_t)(sc[k].x & 0xffffu)), dmin = f16bits_to_f32((uint16_t)(sc[k].x >> 16));
-      const K4Scales ks = k4_scales(sc[k].y, sc[k].z, sc[k].w);
+      const float d = f16bits_to_f32((uint16_t)(scd[k] & 0xffffu)), dmin = f16bits_to_f32((uint16_t)(scd[k] >> 16));
+      const uint32_t rec[4] = {sc[k].x, sc[k].y, sc[k].z, sc[k].w};  // per pair of sub-blocks {sc, sc, m, m}
 #pragma unroll
       for (int j = 0; j < 8; j++) {
-        ws_ds[(8 * si + j) * 16 + r] = in ? d * (float)byte_of(ks.sc0, ks.sc1, j) : 0.f;
-        ws_dm[(8 * si + j) * 16 + r] = in ? dmin * (float)byte_of(ks.mn0, ks.mn1, j) : 0.f;
+        ws_ds[(8 * si + j) * 16 + r] = in ? d * (float)((rec[j >> 1] >> (8 * (j & 1))) & 0xffu) : 0.f;
+        ws_dm[(8 * si + j) * 16 + r] = in ? dmin * (float)((rec[j >> 1] >> (16 + 8 * (j & 1))) & 0xffu) : 0.f;
       }
     }
   }
