@@ -577,7 +577,8 @@ static int launch_kq_m(const KGemvArgs& a, hipStream_t st) {
   int64_t rows = 0;
   for (int p = 0; p < a.nparts; p++) rows += a.part[p].N;
   const int grid = (int)((rows + NW * (64 / best) * 2 - 1) / (NW * (64 / best) * 2));
-  int U = (WT == MLLM_HIP_Q4_K && grid < 512) ? 4 : 1;
+  int U = 1;  // (four units in flight only in the large workgroups below: the 384-workgroup q/k/v launch measured 5.8 us with
+              // one unit against 6.4 us with four)
   // few rows of many units (o_proj, down_proj): large workgroups of one row per lane group, the whole wave on a row when it is
   // long enough to keep 64 lanes busy for a trip
   // (only with at least 32 lanes per row: the narrower shapes have no such variant and keep their 256-thread workgroups)
@@ -586,6 +587,13 @@ static int launch_kq_m(const KGemvArgs& a, hipStream_t st) {
     if (units >= 64 * 4) best = 64;
     NW = best == 64 ? 16 : 8;  // 16 rows per workgroup either way
   }  // (many rows, K = 2560: eight waves per workgroup measured slower than four, 11.0 against 9.6 us for gate + up)
+  // Q6_K rows whose units leave most of a 64-lane trip idle (K = 2560: 40 units): 16 lanes per row, two waves, where that still
+  // makes a thousand workgroups (gate + up 15.8 -> 13.5 us; the smaller q/k/v launch stays faster with the whole wave)
+  if (WT == MLLM_HIP_Q6_K && MT <= 2 && !r1 && !g_kq_G && !g_kq_NW && best == 64 && rows / 16 >= 1024 &&
+      2 * ((units + 15) / 16 * 16 - units) < (units + 63) / 64 * 64 - units) {
+    best = 16;
+    NW = 2;
+  }
   if (g_kq_G) best = g_kq_G;
   if (g_kq_NW) NW = g_kq_NW;
   if (g_kq_U) U = g_kq_U;
