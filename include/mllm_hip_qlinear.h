@@ -280,6 +280,17 @@ int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed
                        int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H,
                        int64_t I, int E, int k, int act_scale_mode, void* workspace, void* stream);
 
+/* The same expert FFN with the experts in the super-block formats (MLLM_HIP_Q4_K / MLLM_HIP_Q6_K, the formats the shipped
+ * Qwen3-MoE recipe quantizes to; activations Q8_K in front of every projection): gate_packed / up_packed / down_packed are E
+ * matrices packed by mllm_hip_kq_prepack back to back, mllm_hip_kq_packed_bytes(wtype, I, H) resp. (wtype, H, I) apart.
+ * H % 256 == 0, I % 256 == 0, T * k <= 65535.  Every (token, expert) pair runs as one GEMV row (four launches for any T): the
+ * decode form; an expert's weights are read once per pair that uses it.
+ * replaces: the same loop over experts with Q4_K / Q6_K Linear ops, modeling_qwen3_moe_fa2.hpp:98-100,175-238 */
+size_t mllm_hip_moe_kq_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k);
+int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x,
+                        int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H, int64_t I,
+                        int E, int k, void* workspace, void* stream);
+
 /* mllm_hip_moe_ffn_q has three forms: every (token, expert) pair as GEMV rows (up to eight tokens or one pair per
  * expert), the pairs sorted by expert in tiles of eight rows that share the expert's weights (up to ten pairs per expert), and
  * the grouped 64-row tiles.  Tuning override: token counts up to which the first and the second run (0 = the rule above; 1

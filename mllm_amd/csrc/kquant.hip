@@ -265,6 +265,11 @@ struct KGemvArgs {
   int nparts;
   const void* x;
   int M, nsb;  // nsb = K / 256
+  // MoE slots (M = 1 only): blockIdx.y = slot; its expert's matrices lie slot_ids[slot] * estride bytes further in every plane,
+  // its activation row is slot / slot_div, its output row is the slot.  slot_ids == null: a plain Linear.
+  const int32_t* slot_ids;
+  int slot_E, slot_div, slot_div_slots;  // experts, pairs per activation row, number of slots (grid y)
+  size_t estride;
 };
 #define KBUF_OOB 0xffffffffu
 #define KBUF_NT 2
@@ -333,13 +338,26 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
   constexpr int UPS = WT == MLLM_HIP_Q4_K ? 8 : 4;  // units per super-block
   const int units = nsb * UPS;
 
+  // MoE slot (uniform): expert offset of the weight planes, activation row, output row.  A slot whose expert id is outside
+  // [0, E) computes with expert 0 and its row is never read (the combine pass skips it).
+  size_t eoff = 0;
+  int64_t xrow = 0, yrow = 0;
+  if (MT == 1 && a.slot_ids) {
+    const int slot = blockIdx.y;
+    const int e = a.slot_ids[slot];
+    eoff = (size_t)((e >= 0 && e < a.slot_E) ? e : 0) * a.estride;
+    xrow = slot / a.slot_div;
+    yrow = slot;
+  }
+  const char* xp = reinterpret_cast<const char*>(a.x) + xrow * K * (XT == MLLM_HIP_BF16 ? 2 : 4);
   KRsrc rs;
   {
     const uint32_t sbt = (uint32_t)pt.N * (uint32_t)nsb;
-    rs.a = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.a), 0, sbt * 128u, 0x00020000);
-    rs.h = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(WT == MLLM_HIP_Q6_K ? pt.w.h : pt.w.a), 0, sbt * 64u, 0x00020000);
-    rs.s = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.s), 0, sbt * 16u, 0x00020000);
-    rs.d = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(pt.w.d), 0, sbt * (WT == MLLM_HIP_Q4_K ? 4u : 2u), 0x00020000);
+    auto at = [&](const void* base) { return const_cast<char*>(reinterpret_cast<const char*>(base) + eoff); };
+    rs.a = __builtin_amdgcn_make_buffer_rsrc(at(pt.w.a), 0, sbt * 128u, 0x00020000);
+    rs.h = __builtin_amdgcn_make_buffer_rsrc(at(WT == MLLM_HIP_Q6_K ? pt.w.h : pt.w.a), 0, sbt * 64u, 0x00020000);
+    rs.s = __builtin_amdgcn_make_buffer_rsrc(at(pt.w.s), 0, sbt * 16u, 0x00020000);
+    rs.d = __builtin_amdgcn_make_buffer_rsrc(at(pt.w.d), 0, sbt * (WT == MLLM_HIP_Q4_K ? 4u : 2u), 0x00020000);
   }
   // Memory requests return in order: the activations a thread will quantize (its first two items) are requested first,
   // then the first trip of weights, so that the quantization runs while the weights are still on their way.
@@ -352,11 +370,11 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
     for (int k = 0; k < 2; k++) {
       const int it = min(tid + k * nthreads, valid - 1);
       if (XL == MLLM_HIP_F32) {
-        const u32x4* p = reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(a.x) + (int64_t)it * 8);
+        const u32x4* p = reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(xp) + (int64_t)it * 8);
         raw[k][0] = p[0];
         raw[k][XL == MLLM_HIP_F32 ? 1 : 0] = p[1];
       } else {
-        raw[k][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(a.x) + (int64_t)it * 8);
+        raw[k][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(xp) + (int64_t)it * 8);
       }
     }
     __asm__ volatile("" ::: "memory");
@@ -412,7 +430,7 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
     }
     for (int it = tid + 2 * nthreads; it < nitems; it += nthreads) {
       float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      if (it < valid) load8<XL>(a.x, (int64_t)it * 8, v);
+      if (it < valid) load8<XL>(xp, (int64_t)it * 8, v);
       quantize_to_lds(it, v);
     }
   }
@@ -527,7 +545,7 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
     for (int m = 0; m < MT; m++) {
       const float v = group_sum<G>(acc[r][m]);
       const int64_t row = row0 + r;
-      if (c0 == 0 && row < pt.N && m < a.M) pt.y[(int64_t)m * pt.N + row] = pt.bias ? v + pt.bias[row] : v;
+      if (c0 == 0 && row < pt.N && m < a.M) pt.y[(yrow + m) * pt.N + row] = pt.bias ? v + pt.bias[row] : v;
     }
 }
 
@@ -554,7 +572,8 @@ static int launch_kq_u(const KGemvArgs& a_in, int NW, hipStream_t st) {
   auto kern = kq_gemv_kernel<WT, XT, MT, G, R, U, LB>;
   if (lds > 64 * 1024)
     HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, st, a);
+  const unsigned slots = (MT == 1 && a.slot_ids) ? (unsigned)a.slot_div_slots : 1u;
+  hipLaunchKernelGGL(kern, dim3(grid, slots), dim3(NW * 64), lds, st, a);
   return (int)hipGetLastError();
 }
 template <int WT, int XT, int MT, int G>
@@ -1409,6 +1428,31 @@ MLLM_API int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, in
   mllm_hip_gemv_part part{packed, bias, y, N};
   return mllm_hip_linear_kq_multi(wtype, 1, &part, x, x_dtype, M, K, workspace, stream);
 }
+
+// ---- MoE slots: one GEMV row per (token, expert) pair ---------------------------------------------------------------------------
+// nparts sibling matrices per expert (gate and up, or down alone), packed0[p] = expert 0's matrix of part p, the experts'
+// matrices mllm_hip_kq_packed_bytes(wtype, N, K) apart; slot s multiplies activation row s / slot_div by the matrices of
+// expert ids[s] and writes row s of ys[p] ([slots][N]).
+namespace mllmhip {
+int kq_moe_gemv(int wtype, int nparts, const void* const* packed0, float* const* ys, int64_t N, int64_t K, const void* x, int x_dtype,
+                const int32_t* ids, int E, int slots, int slot_div, hipStream_t st) {
+  if (nparts < 1 || nparts > KQ_MAX_PARTS || slots < 1 || slots > 65535) return MLLM_HIP_E_SHAPE;
+  KGemvArgs a{};
+  for (int p = 0; p < nparts; p++) a.part[p] = KGemvPart{kq_view(wtype, packed0[p], N, K), nullptr, ys[p], (int)N};
+  a.nparts = nparts;
+  a.x = x;
+  a.M = 1;
+  a.nsb = (int)(K / QK_K);
+  a.slot_ids = ids;
+  a.slot_E = E;
+  a.slot_div = slot_div;
+  a.slot_div_slots = slots;
+  a.estride = kq_packed_bytes(wtype, N, K);
+  if (wtype == MLLM_HIP_Q4_K)
+    return x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_F32>(a, st) : launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_BF16>(a, st);
+  return x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q6_K, MLLM_HIP_F32>(a, st) : launch_kq<MLLM_HIP_Q6_K, MLLM_HIP_BF16>(a, st);
+}
+}  // namespace mllmhip
 
 // ---- many rows on the matrix cores ------------------------------------------------------------------------------------------
 static bool kq_type(int wtype) { return wtype == MLLM_HIP_Q4_K || wtype == MLLM_HIP_Q6_K; }

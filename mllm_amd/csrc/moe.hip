@@ -1311,3 +1311,57 @@ MLLM_API int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const v
                      (int)H, k, E);
   return (int)hipGetLastError();
 }
+
+// ---- experts in the super-block formats (kquant.hip) ----------------------------------------------------------------------
+// The shipped Qwen3-MoE recipe quantizes the experts to Q4_K / Q6_K.  Every (token, expert) pair is one row of the K-quant
+// GEMV: gate and up in one launch (the workgroup quantizes the token's x to Q8_K), silu(g) * u, the down GEMV (quantizing h),
+// the weighted sum in slot order.  Four launches for any T; the weights of an expert are read once per pair that uses it,
+// so this is the decode form (prefill wants the experts grouped, which this format does not have yet).
+namespace mllmhip {
+int kq_moe_gemv(int wtype, int nparts, const void* const* packed0, float* const* ys, int64_t N, int64_t K, const void* x, int x_dtype,
+                const int32_t* ids, int E, int slots, int slot_div, hipStream_t st);
+}
+MLLM_API size_t mllm_hip_moe_kq_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k) {
+  if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || k <= 0 || H % 256 || I % 256) return 0;
+  Carver c(nullptr);
+  c.take<float>((size_t)T * k * I);
+  c.take<float>((size_t)T * k * I);
+  c.take<float>((size_t)T * k * I);
+  c.take<float>((size_t)T * k * H);
+  return c.used;
+}
+
+MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x,
+                                 int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H,
+                                 int64_t I, int E, int k, void* workspace, void* stream) {
+  if ((wtype != MLLM_HIP_Q4_K && wtype != MLLM_HIP_Q6_K) || !gate_packed || !up_packed || !down_packed || !x || !topk_ids ||
+      !topk_w || !y || !workspace || T <= 0 || E <= 0 || E > 4096 || k <= 0)
+    return MLLM_HIP_E_BADARG;
+  if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
+  if (H <= 0 || I <= 0 || H % 256 || I % 256 || T * k > 65535) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16 ||
+      reinterpret_cast<uintptr_t>(gate_packed) % 16 || reinterpret_cast<uintptr_t>(up_packed) % 16 ||
+      reinterpret_cast<uintptr_t>(down_packed) % 16)
+    return MLLM_HIP_E_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  const int slots = (int)(T * k);
+  Carver c(workspace);
+  float* g = c.take<float>((size_t)slots * I);
+  float* u = c.take<float>((size_t)slots * I);
+  float* h = c.take<float>((size_t)slots * I);
+  float* per = c.take<float>((size_t)slots * H);
+  const void* gu[2] = {gate_packed, up_packed};
+  float* guy[2] = {g, u};
+  int rc = kq_moe_gemv(wtype, 2, gu, guy, I, H, x, x_dtype, topk_ids, E, slots, k, st);
+  if (rc) return rc;
+  rc = mllm_hip_silu_mul(g, u, h, MLLM_HIP_F32, slots, I, nullptr, MLLM_HIP_SCALE_IEEE, stream);
+  if (rc) return rc;
+  const void* dn[1] = {down_packed};
+  float* dny[1] = {per};
+  rc = kq_moe_gemv(wtype, 1, dn, dny, H, I, h, MLLM_HIP_F32, topk_ids, E, slots, 1, st);
+  if (rc) return rc;
+  const int64_t total = T * H;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
+                     (int)H, k, E);
+  return (int)hipGetLastError();
+}

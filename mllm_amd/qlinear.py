@@ -547,6 +547,51 @@ class PackedKWeight:
         return w
 
 
+class PackedKExperts:
+    """E Q4_K / Q6_K matrices [N, K] packed back to back for mllm_hip_moe_ffn_kq.  blocks: uint8 [E, N, K/256, 144|210]."""
+
+    def __init__(self, wtype, blocks, weight_scale_mode=SCALE_IEEE):
+        assert blocks.dtype == torch.uint8 and blocks.dim() == 4 and blocks.shape[3] == KBLOCK_BYTES[wtype]
+        self.wtype, self.E, self.N, self.K = wtype, blocks.shape[0], blocks.shape[1], blocks.shape[2] * 256
+        L = _lib.lib()
+        self.stride = L.mllm_hip_kq_packed_bytes(wtype, self.N, self.K)
+        self.buf = torch.empty(self.E * self.stride, dtype=torch.uint8, device="cuda")
+        for e in range(self.E):
+            src = blocks[e].contiguous().cuda()
+            _lib.check(L.mllm_hip_kq_prepack(wtype, src.data_ptr(), weight_scale_mode, self.buf.data_ptr() + e * self.stride, self.N,
+                                             self.K, _stream()), "kq prepack")
+            torch.cuda.current_stream().synchronize()
+
+    @classmethod
+    def synthetic(cls, wtype, E, N, K, gen):
+        bb = KBLOCK_BYTES[wtype]
+        blocks = torch.randint(0, 256, (E, N, K // 256, bb), dtype=torch.uint8, device="cuda", generator=gen)
+        for off in ((0, 2) if wtype == Q4_K else (208,)):
+            blocks[..., off] = 0x00
+            blocks[..., off + 1] = 0x14
+        return cls(wtype, blocks)
+
+    @property
+    def ptr(self):
+        return self.buf.data_ptr()
+
+
+def moe_ffn_kq(gate, up, down, x, topk_ids, topk_w, workspace=None, out=None):
+    """The MoE expert FFN with Q4_K / Q6_K experts (PackedKExperts): x [T, H], topk_ids int32 [T, k], topk_w fp32 [T, k]."""
+    T, H = x.shape
+    k = topk_ids.shape[1]
+    E, I = gate.E, gate.N
+    assert gate.K == H and up.N == I and down.N == H and down.K == I and topk_ids.dtype == torch.int32
+    L = _lib.lib()
+    if workspace is None:
+        workspace = torch.empty(L.mllm_hip_moe_kq_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
+    y = out if out is not None else torch.empty((T, H), dtype=torch.float32, device="cuda")
+    _lib.check(L.mllm_hip_moe_ffn_kq(gate.wtype, gate.ptr, up.ptr, down.ptr, x.data_ptr(), _xdtype(x), topk_ids.data_ptr(),
+                                     topk_w.data_ptr(), y.data_ptr(), T, H, I, E, k, workspace.data_ptr(), _stream()),
+               "mllm_hip_moe_ffn_kq")
+    return y
+
+
 def kq_workspace(M, K):
     return torch.empty(_lib.lib().mllm_hip_kq_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
 

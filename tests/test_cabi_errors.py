@@ -58,6 +58,9 @@ def _cases():
         "mllm_hip_moe_ffn_q_gemm": ([Q4_0, P, P, P, P, F32, P, P, P, 4, 64, 64, 8, 2, 0, P, None],
                                     [(2, None, BADARG), (3, None, BADARG), (15, None, BADARG), (10, 48, SHAPE), (11, 48, SHAPE),
                                      (4, ODD, ALIGN), (0, Q4_K, BADARG)]),
+        "mllm_hip_moe_ffn_kq": ([Q4_K, P, P, P, P, F32, P, P, P, 4, 256, 256, 8, 2, P, None],
+                                [(0, Q4_0, BADARG), (1, None, BADARG), (3, None, BADARG), (4, None, BADARG), (6, None, BADARG),
+                                 (14, None, BADARG), (10, 128, SHAPE), (11, 320, SHAPE), (9, 40000, SHAPE), (4, ODD, ALIGN)]),
         "mllm_hip_kq_prepack": ([Q4_K, P, 0, P, 8, 256, None], [(0, Q4_0, BADARG), (1, None, BADARG), (3, None, BADARG), (5, 128, SHAPE)]),
         "mllm_hip_linear_kq": ([Q6_K, P, P, F32, None, P, 1, 8, 256, P, None],
                                [(0, Q8_0, BADARG), (1, None, BADARG), (2, None, BADARG), (5, None, BADARG), (9, ODD, ALIGN),
@@ -122,3 +125,4 @@ def test_size_helpers_return_zero_for_shapes_they_do_not_take():
     assert L.mllm_hip_moe_workspace_bytes(4, 48, 64, 8, 2) == 0
     assert L.mllm_hip_moe_gemm_workspace_bytes(4, 64, 64, 0, 2) == 0
     assert L.mllm_hip_w4a16_packed_bytes(64, 256, 100) == 0
+    assert L.mllm_hip_moe_kq_workspace_bytes(4, 128, 256, 8, 2) == 0

@@ -233,3 +233,34 @@ def test_golden_kquant(golden_dir, name, wtype):
     q, d, bs = ql.quantize_q8_K(to_dev(g["q8k_x"]))
     assert np.array_equal(q.cpu().numpy(), g["q8k_q"]) and np.array_equal(d.cpu().numpy().view(np.uint32), g["q8k_d"].view(np.uint32))
     assert np.array_equal(bs.cpu().numpy(), g["q8k_bsums"])
+
+
+@pytest.mark.parametrize("wtype,T,H,I,E,k", [(2, 1, 2048, 768, 16, 8), (3, 1, 2048, 768, 16, 8), (2, 5, 512, 256, 6, 3), (3, 9, 256, 512, 4, 2),
+                                            (2, 8, 2048, 768, 128, 8)])
+def test_moe_ffn_with_k_quant_experts(wtype, T, H, I, E, k):
+    """Q4_K / Q6_K experts (Qwen3-30B-A3B dimensions included): every (token, expert) pair one K-quant GEMV row, SiLU and product,
+    down GEMV, weighted sum in slot order, against the oracle's composition of the same Linears; slots with an expert id
+    outside [0, E) add nothing; permuting tokens permutes outputs bit for bit; bf16 activations"""
+    rng = synth.rng_for(9, 7000 + wtype + T + H + I + E)
+    Wg = synth.make_weight(rng, wtype, E * I, H).reshape(E, I, H // 256, -1)
+    Wu = synth.make_weight(rng, wtype, E * I, H).reshape(E, I, H // 256, -1)
+    Wd = synth.make_weight(rng, wtype, E * H, I).reshape(E, H, I // 256, -1)
+    ids, w = synth.make_moe_routing(rng, T, E, k)
+    g, u, d = (ql.PackedKExperts(wtype, torch.from_numpy(W)) for W in (Wg, Wu, Wd))
+    x = synth.make_x_fp32(rng, T, H)
+    announce("moe k-quant", wtype, T, H, I, E, k)
+    y = ql.moe_ffn_kq(g, u, d, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+    want = orc.moe_ffn_kq(x, ids, w, Wg, Wu, Wd, wtype)
+    assert rel_l2(y, want) < 1e-3, rel_l2(y, want)
+    perm = rng.permutation(T)
+    y2 = ql.moe_ffn_kq(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
+    assert np.array_equal(y2, y[perm])
+    bad = ids.copy()
+    bad[0, 0] = E + 3
+    if k > 1:
+        bad[T - 1, k - 1] = -1
+    y3 = ql.moe_ffn_kq(g, u, d, to_dev(x), to_dev(bad), to_dev(w)).cpu().numpy()
+    assert rel_l2(y3, orc.moe_ffn_kq(x, bad, w, Wg, Wu, Wd, wtype)) < 1e-3
+    bits, xb = synth.make_x_bf16(rng, T, H)
+    y4 = ql.moe_ffn_kq(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
+    assert rel_l2(y4, orc.moe_ffn_kq(xb, ids, w, Wg, Wu, Wd, wtype)) < 1e-3

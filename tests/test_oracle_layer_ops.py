@@ -130,3 +130,32 @@ def test_moe_gate_composition():
     assert np.allclose(wt.sum(-1), 1.0, atol=1e-6)
     _, wt2, _ = orc.moe_gate(x, w, k, norm=False)
     assert np.max(np.abs(wt2 - pw)) < 2e-6
+
+
+def test_moe_ffn_kq_composition_against_float64_model():
+    """The K-quant MoE oracle is a composition of linear_kq and silu (each pinned on its own).  What the composition adds --
+    which expert serves which slot, gate against up, the weighted sum -- is checked against a float64 model on the dequantized
+    weights; the two differ by the Q8_K activation noise only (under one percent), while a swapped operand, a wrong expert
+    or a dropped slot would show as tens of percent.  Slots with an expert id outside [0, E) contribute nothing."""
+    from mllm_amd import synth
+    rng = synth.rng_for(9, 1)
+    for wt in (2, 3):
+        T, H, I, E, k = 3, 256, 256, 4, 2
+        Wg = synth.make_weight(rng, wt, E * I, H).reshape(E, I, H // 256, -1)
+        Wu = synth.make_weight(rng, wt, E * I, H).reshape(E, I, H // 256, -1)
+        Wd = synth.make_weight(rng, wt, E * H, I).reshape(E, H, I // 256, -1)
+        ids, w = synth.make_moe_routing(rng, T, E, k)
+        ids[1, 1] = E + 2
+        x = synth.make_x_fp32(rng, T, H)
+        y = orc.moe_ffn_kq(x, ids, w, Wg, Wu, Wd, wt)
+        Dg = [orc.dequantize_k(Wg[e], wt).astype(np.float64) for e in range(E)]
+        Du = [orc.dequantize_k(Wu[e], wt).astype(np.float64) for e in range(E)]
+        Dd = [orc.dequantize_k(Wd[e], wt).astype(np.float64) for e in range(E)]
+        ref = np.zeros((T, H))
+        for t in range(T):
+            for j in range(k):
+                e = ids[t, j]
+                if 0 <= e < E:
+                    g, u = Dg[e] @ x[t], Du[e] @ x[t]
+                    ref[t] += w[t, j] * (Dd[e] @ (g / (1 + np.exp(-g)) * u))
+        assert np.linalg.norm(y - ref) / np.linalg.norm(ref) < 0.03
