@@ -159,6 +159,34 @@ def side_workloads(torch, ql, synth, gen):
         wb = act * (2 * I * (H // 32) * 18 + H * (I // 32) * 18)
         dec["tokens_%d" % Td] = {"us": td * 1e6, "active_experts_avg": act, "weight_GBps": wb / td / 1e9, "frac_of_hbm_peak": wb / td / 8e12}
     del gate, up, down
+    # the same layer with Q4_K experts (the format of the shipped Qwen3-MoE recipe), 1 and 8 tokens: pairs as K-quant GEMV rows
+    gk = ql.PackedKExperts.synthetic(ql.Q4_K, E, I, H, gen)
+    uk = ql.PackedKExperts.synthetic(ql.Q4_K, E, I, H, gen)
+    dk = ql.PackedKExperts.synthetic(ql.Q4_K, E, H, I, gen)
+    deck = {}
+    for Td in (1, 8):
+        rngd = synth.rng_for(4, 100 + Td)
+        routes = [synth.make_moe_routing(rngd, Td, E, k) for _ in range(16)]
+        idl = [torch.from_numpy(r[0]).cuda() for r in routes]
+        twl = [torch.from_numpy(r[1]).cuda() for r in routes]
+        xd = torch.randn((Td, H), device="cuda", generator=gen).to(torch.bfloat16)
+        yd = torch.empty((Td, H), dtype=torch.float32, device="cuda")
+        from mllm_amd import _lib as _l
+        wsk = torch.empty(_l.lib().mllm_hip_moe_kq_workspace_bytes(Td, H, I, E, k), dtype=torch.uint8, device="cuda")
+
+        def kstep():
+            for i_, t_ in zip(idl, twl):
+                ql.moe_ffn_kq(gk, uk, dk, xd, i_, t_, workspace=wsk, out=yd)
+        kstep()
+        torch.cuda.synchronize()
+        gd = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gd):
+            kstep()
+        td = ev_time(gd.replay, 10) / 16
+        act = float(np.mean([len(np.unique(r[0])) for r in routes]))
+        wb = act * 3 * I * (H // 256) * 144
+        deck["tokens_%d" % Td] = {"us": td * 1e6, "active_experts_avg": act, "weight_GBps": wb / td / 1e9, "frac_of_hbm_peak": wb / td / 8e12}
+    del gk, uk, dk
     from mllm_amd import _lib
     L = _lib.lib()
     gate2 = ql.PackedExperts.synthetic(ql.Q4_0, E, I, H, gen, layout="gemm")
@@ -173,7 +201,7 @@ def side_workloads(torch, ql, synth, gen):
                                             "frac_of_hbm_peak": wbytes / tm2 / 8e12, "TFLOPS": flops / tm2 / 1e12,
                                             "path": "matrix cores, fp16 operands with folded block scales (mllm_hip_moe_ffn_q_gemm)",
                                             "block_dot_path": {"us": tm * 1e6, "weight_GBps": wbytes / tm / 1e9},
-                                            "decode": dec}
+                                            "decode": dec, "decode_q4_k_experts": deck}
     del gate2, up2, down2
     # Q4_0 Linear at prefill size (the reference's tinyBLAS gemm branch): gate_proj of the decode layer, 2048 rows
     M, N, K = 2048, 9728, 2560

@@ -595,7 +595,8 @@ static int launch_kq_m(const KGemvArgs& a, hipStream_t st) {
   int NW = 4;
   int64_t rows = 0;
   for (int p = 0; p < a.nparts; p++) rows += a.part[p].N;
-  const int grid = (int)((rows + NW * (64 / best) * 2 - 1) / (NW * (64 / best) * 2));
+  // (MoE slots multiply the grid: the shape rules below look at the whole launch)
+  const int grid = (int)((rows + NW * (64 / best) * 2 - 1) / (NW * (64 / best) * 2)) * ((MT == 1 && a.slot_ids) ? a.slot_div_slots : 1);
   int U = 1;  // (four units in flight only in the large workgroups below: the 384-workgroup q/k/v launch measured 5.8 us with
               // one unit against 6.4 us with four)
   // few rows of many units (o_proj, down_proj): large workgroups of one row per lane group, the whole wave on a row when it is
