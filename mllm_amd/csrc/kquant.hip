@@ -614,6 +614,12 @@ static int launch_kq_m(const KGemvArgs& a, hipStream_t st) {
     best = 16;
     NW = 2;
   }
+  // MoE slots (thousands of small workgroups, each quantizing its token's x): 16 lanes per row make the workgroups twice as
+  // tall, two units in flight (Qwen3-30B-A3B experts, eight tokens: 54.6 -> 45.1 us for the layer)
+  if (MT == 1 && a.slot_ids && a.slot_div_slots > 1 && best >= 16 && !r1) {
+    best = 16;
+    U = 2;
+  }
   if (g_kq_G) best = g_kq_G;
   if (g_kq_NW) NW = g_kq_NW;
   if (g_kq_U) U = g_kq_U;
