@@ -283,7 +283,7 @@ int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed
 /* The same expert FFN with the experts in the super-block formats (MLLM_HIP_Q4_K / MLLM_HIP_Q6_K, the formats the shipped
  * Qwen3-MoE recipe quantizes to; activations Q8_K in front of every projection): gate_packed / up_packed / down_packed are E
  * matrices packed by mllm_hip_kq_prepack back to back, mllm_hip_kq_packed_bytes(wtype, I, H) resp. (wtype, H, I) apart.
- * H % 256 == 0, I % 256 == 0, T * k <= 65535.  Every (token, expert) pair runs as one GEMV row (four launches for any T): the
+ * H % 256 == 0, I % 256 == 0, T * k <= 65535.  Every (token, expert) pair runs as one GEMV row (three or four launches for any T): the
  * decode form; an expert's weights are read once per pair that uses it.
  * replaces: the same loop over experts with Q4_K / Q6_K Linear ops, modeling_qwen3_moe_fa2.hpp:98-100,175-238 */
 size_t mllm_hip_moe_kq_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k);

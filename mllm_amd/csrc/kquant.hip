@@ -268,6 +268,8 @@ struct KGemvArgs {
   // MoE slots (M = 1 only): blockIdx.y = slot; its expert's matrices lie slot_ids[slot] * estride bytes further in every plane,
   // its activation row is slot / slot_div, its output row is the slot.  slot_ids == null: a plain Linear.
   const int32_t* slot_ids;
+  const float* x2;       // slots with fp32 x only: the activation is silu(x) * x2 (the MLP's product folded into the down GEMV)
+  int silu_accurate;     // expf instead of the reference's polynomial (mllm_hip_set_exp_mode)
   int slot_E, slot_div, slot_div_slots;  // experts, pairs per activation row, number of slots (grid y)
   size_t estride;
 };
@@ -313,6 +315,13 @@ __device__ __forceinline__ int dot16(const u32x4& w, const u32x4& x) {
 }
 __device__ __forceinline__ int half16(uint32_t pair, int hi) { return (int)(int16_t)(hi ? (pair >> 16) : (pair & 0xffffu)); }
 
+__device__ __forceinline__ void silu_mul8(float (&v)[8], const float* u, bool accurate) {
+  const f32x4 a = reinterpret_cast<const f32x4*>(u)[0], b = reinterpret_cast<const f32x4*>(u)[1];
+  const float uu[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+  for (int e = 0; e < 8; e++) v[e] = v[e] * (1.0f / (1.0f + (accurate ? expf(-v[e]) : exp_poly(-v[e])))) * uu[e];
+}
+
 // Workgroup = NW waves; a wave is cut into 64 / G groups of G lanes; a group owns R consecutive weight rows and its lanes
 // stride over the row's units.  x is quantized to Q8_K once per workgroup into LDS: codes [MT][K], scales [MT][nsb], sums
 // of 16 as int16 [MT][nsb][16].
@@ -350,6 +359,7 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
     yrow = slot;
   }
   const char* xp = reinterpret_cast<const char*>(a.x) + xrow * K * (XT == MLLM_HIP_BF16 ? 2 : 4);
+  const float* x2p = (XT == MLLM_HIP_F32 && MT == 1 && a.x2) ? a.x2 + xrow * K : nullptr;  // uniform
   KRsrc rs;
   {
     const uint32_t sbt = (uint32_t)pt.N * (uint32_t)nsb;
@@ -365,6 +375,7 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
   const int valid = a.M * (K >> 3);
   constexpr int XL = XT == KQ_IMAGE ? MLLM_HIP_F32 : XT;
   u32x4 raw[2][XL == MLLM_HIP_F32 ? 2 : 1];
+  u32x4 raw2[2][2];
   if (XT != KQ_IMAGE) {
 #pragma unroll
     for (int k = 0; k < 2; k++) {
@@ -375,6 +386,14 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
         raw[k][XL == MLLM_HIP_F32 ? 1 : 0] = p[1];
       } else {
         raw[k][0] = *reinterpret_cast<const u32x4*>(reinterpret_cast<const uint16_t*>(xp) + (int64_t)it * 8);
+      }
+    }
+    if (XT == MLLM_HIP_F32 && MT == 1 && x2p) {  // the second factor with the first (ahead of the weights: requests return in order)
+#pragma unroll
+      for (int k = 0; k < 2; k++) {
+        const u32x4* p = reinterpret_cast<const u32x4*>(x2p + (int64_t)min(tid + k * nthreads, valid - 1) * 8);
+        raw2[k][0] = p[0];
+        raw2[k][1] = p[1];
       }
     }
     __asm__ volatile("" ::: "memory");
@@ -425,12 +444,14 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
 #pragma unroll
           for (int e = 0; e < 8; e++) v[e] = 0.f;
         }
+        if (XT == MLLM_HIP_F32 && MT == 1 && x2p) silu_mul8(v, reinterpret_cast<const float*>(&raw2[k][0]), a.silu_accurate);
         quantize_to_lds(it, v);
       }
     }
     for (int it = tid + 2 * nthreads; it < nitems; it += nthreads) {
       float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       if (it < valid) load8<XL>(xp, (int64_t)it * 8, v);
+      if (XT == MLLM_HIP_F32 && MT == 1 && x2p) silu_mul8(v, x2p + (int64_t)min(it, valid - 1) * 8, a.silu_accurate);
       quantize_to_lds(it, v);
     }
   }
@@ -1439,10 +1460,12 @@ MLLM_API int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, in
 // ---- MoE slots: one GEMV row per (token, expert) pair ---------------------------------------------------------------------------
 // nparts sibling matrices per expert (gate and up, or down alone), packed0[p] = expert 0's matrix of part p, the experts'
 // matrices mllm_hip_kq_packed_bytes(wtype, N, K) apart; slot s multiplies activation row s / slot_div by the matrices of
-// expert ids[s] and writes row s of ys[p] ([slots][N]).
+// expert ids[s] and writes row s of ys[p] ([slots][N]).  x2 (fp32, same rows as x): the activation is silu(x) * x2.
 namespace mllmhip {
+int exp_mode_accurate();  // layer_ops.hip: the setting of mllm_hip_set_exp_mode
 int kq_moe_gemv(int wtype, int nparts, const void* const* packed0, float* const* ys, int64_t N, int64_t K, const void* x, int x_dtype,
-                const int32_t* ids, int E, int slots, int slot_div, hipStream_t st) {
+                const float* x2, const int32_t* ids, int E, int slots, int slot_div, hipStream_t st) {
+  if (x2 && x_dtype != MLLM_HIP_F32) return MLLM_HIP_E_BADARG;
   if (nparts < 1 || nparts > KQ_MAX_PARTS || slots < 1 || slots > 65535) return MLLM_HIP_E_SHAPE;
   KGemvArgs a{};
   for (int p = 0; p < nparts; p++) a.part[p] = KGemvPart{kq_view(wtype, packed0[p], N, K), nullptr, ys[p], (int)N};
@@ -1451,6 +1474,8 @@ int kq_moe_gemv(int wtype, int nparts, const void* const* packed0, float* const*
   a.M = 1;
   a.nsb = (int)(K / QK_K);
   a.slot_ids = ids;
+  a.x2 = x2;
+  a.silu_accurate = exp_mode_accurate();
   a.slot_E = E;
   a.slot_div = slot_div;
   a.slot_div_slots = slots;
