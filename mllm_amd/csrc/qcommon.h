@@ -112,6 +112,17 @@ __device__ __forceinline__ uint16_t quantize_block_q8_0(const float (&v)[32], ui
   return f32_to_f16bits(d);
 }
 
+// Four Q8_0 codes rint(v[e] * idv) packed into a dword, for |v[e] * idv| <= 127 (idv = 127 / amax of the block): adding
+// 1.5 * 2^23 rounds to nearest-even exactly as rintf does and leaves the two's-complement code in the low byte of the sum,
+// so round / convert / clamp / shift-or become one add and three byte permutes.  The product is rounded to fp32 first, as
+// in the reference (the build never contracts a * b + c).
+__device__ __forceinline__ uint32_t q8_pack4(const float* v, float idv) {
+  uint32_t b[4];
+#pragma unroll
+  for (int e = 0; e < 4; e++) b[e] = __float_as_uint(v[e] * idv + 12582912.0f);
+  return __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u) | __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+}
+
 // The Q8_0 image of activation rows that the decode GEMV copies into LDS: for MT rows of nb blocks, 16-byte planes of
 // elements 0..15 and 16..31 of every block, then the fp32 effective scales, then -8 * sum(codes).
 struct QImage {
@@ -128,18 +139,7 @@ __device__ __forceinline__ void quad_quantize_to_image(const float (&v)[8], cons
   amax = fmaxf(amax, dpp_f<0x4E>(amax));
   const float d = amax / 127.f;
   const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
-  uint32_t pk[2];
-#pragma unroll
-  for (int w = 0; w < 2; w++) {
-    uint32_t p = 0;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      int qi = (int)rintf(v[4 * w + e] * idv);
-      qi = min(127, max(-128, qi));
-      p |= ((uint32_t)qi & 0xffu) << (8 * e);
-    }
-    pk[w] = p;
-  }
+  const uint32_t pk[2] = {q8_pack4(&v[0], idv), q8_pack4(&v[4], idv)};
   int sum = __builtin_amdgcn_sdot4((int)pk[0], 0x01010101, 0, false);
   sum = __builtin_amdgcn_sdot4((int)pk[1], 0x01010101, sum, false);
   sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xf, 0xf, true);

@@ -250,17 +250,7 @@ __global__ __launch_bounds__(MT <= 2 ? 1024 : 512) void gemv_q_kernel(GemvArgs a
     amax = fmaxf(amax, dpp_f<0x4E>(amax));
     const float d = amax / 127.f;
     const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
-    // code = rint(v * idv), |v * idv| <= 127 by construction: adding 1.5 * 2^23 rounds to nearest-even exactly as rintf does and
-    // leaves the two's-complement code in the low byte of the sum (one add instead of round, convert and clamp); the
-    // product is rounded to fp32 first, as in the reference (no fused multiply-add)
-    uint32_t pk[2];
-#pragma unroll
-    for (int w = 0; w < 2; w++) {
-      uint32_t b[4];
-#pragma unroll
-      for (int e = 0; e < 4; e++) b[e] = __float_as_uint(v[4 * w + e] * idv + 12582912.0f);
-      pk[w] = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u) | __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
-    }
+    const uint32_t pk[2] = {q8_pack4(&v[0], idv), q8_pack4(&v[4], idv)};
     int sum = __builtin_amdgcn_sdot4((int)pk[0], 0x01010101, 0, false);
     sum = __builtin_amdgcn_sdot4((int)pk[1], 0x01010101, sum, false);
     sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xf, 0xf, true);

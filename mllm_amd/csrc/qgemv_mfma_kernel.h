@@ -39,16 +39,8 @@ __device__ __forceinline__ void quad_quantize(const float (&v)[8], int x86, uint
   amax = fmaxf(amax, dpp_f<0x4E>(amax));
   const float d = amax / 127.f;
   const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
-#pragma unroll
-  for (int w = 0; w < 2; w++) {
-    uint32_t p = 0;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      const int qi = (int)rintf(v[4 * w + e] * idv);  // |v| <= amax: within -127 .. 127, the reference's saturation never acts
-      p |= ((uint32_t)qi & 0xffu) << (8 * e);
-    }
-    pk[w] = p;
-  }
+  pk[0] = q8_pack4(&v[0], idv);  // |v| <= amax: within -127 .. 127, the reference's saturation never acts
+  pk[1] = q8_pack4(&v[4], idv);
   int sum = __builtin_amdgcn_sdot4((int)pk[0], 0x01010101, 0, false);
   sum = __builtin_amdgcn_sdot4((int)pk[1], 0x01010101, sum, false);
   sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xf, 0xf, true);
