@@ -274,7 +274,7 @@ int mllm_hip_w4a16_packed_set_tuning(int tile);
  * gate_packed / up_packed: E pre-packed [I][H] matrices back to back, expert e at + e * mllm_hip_q_packed_bytes(wtype, I, H);
  * down_packed: E pre-packed [H][I] matrices, stride mllm_hip_q_packed_bytes(wtype, H, I).
  * x [T][H] fp32 or bf16; topk_ids int32 [T][k] (entries outside [0, E) contribute nothing); topk_w fp32 [T][k];
- * y fp32 [T][H].  H % 32 == 0, I % 32 == 0, E <= 4096.  workspace: mllm_hip_moe_workspace_bytes. */
+ * y fp32 [T][H].  H % 32 == 0, I % 32 == 0, E <= 3072 (more: MLLM_HIP_E_SHAPE).  workspace: mllm_hip_moe_workspace_bytes. */
 size_t mllm_hip_moe_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k);
 int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x,
                        int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H,

@@ -25,11 +25,22 @@ bool HipAllocator::alloc(Storage* storage) {
   void* p = nullptr;
   if (hipMalloc(&p, storage->size_ ? storage->size_ : 256) != hipSuccess) return false;
   storage->ptr_ = p;
+  live_[static_cast<const char*>(p)] = storage->size_ ? storage->size_ : 256;
   return true;
+}
+bool HipAllocator::owns(const void* ptr, size_t bytes) const {
+  const char* p = static_cast<const char*>(ptr);
+  auto it = live_.upper_bound(p);
+  if (it == live_.begin()) return false;
+  --it;
+  return p >= it->first && p + bytes <= it->first + it->second;
 }
 void HipAllocator::free(Storage* storage) {
   if (storage->ptr_ && owner) owner->noteWrite(storage->ptr_, storage->size_);
-  if (storage->ptr_) (void)hipFree(storage->ptr_);
+  if (storage->ptr_) {
+    live_.erase(static_cast<const char*>(storage->ptr_));
+    (void)hipFree(storage->ptr_);
+  }
   storage->ptr_ = nullptr;
 }
 bool HipAllocator::generalAlloc(void** ptr, size_t cap, size_t) { return hipMalloc(ptr, cap) == hipSuccess; }
@@ -57,6 +68,12 @@ void HipBackend::synchronize() const { MLLM_HIP_CHECK(hipStreamSynchronize((hipS
 
 void* HipBackend::newImage(const void* tensor_ptr, size_t tensor_bytes, int rows, int64_t D) {
   if (!cfg_.fold_images || rows < 1 || rows > 8 || D % 32) return nullptr;
+  // only for memory whose every free this backend sees; an external buffer could be reused behind its back
+  if (!std::static_pointer_cast<HipAllocator>(allocator_)->owns(tensor_ptr, tensor_bytes)) return nullptr;
+  if (images_.size() >= kMaxImages) {  // oldest first; its buffer goes back to the pool like any dropped image
+    if (image_pool_.size() < 16) image_pool_.push_back(images_.front().data);
+    images_.erase(images_.begin());
+  }
   const size_t need = mllm_hip_gemv_workspace_bytes(rows, D);
   Tensor buf;
   for (size_t i = 0; i < image_pool_.size(); i++)
@@ -100,7 +117,7 @@ std::shared_ptr<HipBackend> initHipBackend() {
     if (std::strcmp(m, "x86") == 0) cfg.weight_scale_mode = cfg.act_scale_mode = MLLM_HIP_SCALE_X86_REF;
   }
   if (const char* m = std::getenv("MLLM_HIP_PREFILL")) cfg.prefill_matrix_cores = std::strcmp(m, "blockdot") != 0;
-  if (const char* m = std::getenv("MLLM_HIP_FOLD_IMAGES")) cfg.fold_images = std::strcmp(m, "0") != 0;
+  if (const char* m = std::getenv("MLLM_HIP_FOLD_IMAGES")) cfg.fold_images = std::strcmp(m, "1") == 0;
   auto backend = std::make_shared<HipBackend>(cfg);
   ctx.registerBackend(backend);
   ctx.memoryManager()->registerAllocator(kHIP, backend->allocator());

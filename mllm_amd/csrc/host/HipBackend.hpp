@@ -7,6 +7,8 @@
 //   device allocator  mllm/backends/cuda/CudaAllocator.cpp:10-65
 //   weight-side names mllm/backends/ascend/ops/AscendLinearOp.cpp:42-48 ("<name>.weight.scale")
 #pragma once
+#include <map>
+
 #include "mllm_core.hpp"
 
 namespace mllm::hip {
@@ -25,6 +27,11 @@ class HipAllocator final : public Allocator {
   [[nodiscard]] size_t alignSize() const override { return 256; }
   // told about every free so that the backend can drop what it keeps about that memory; cleared when the backend goes
   class HipBackend* owner = nullptr;
+  // true when [ptr, ptr + bytes) lies inside an allocation this allocator made through alloc() and has not freed
+  [[nodiscard]] bool owns(const void* ptr, size_t bytes) const;
+
+ private:
+  std::map<const char*, size_t> live_;  // start -> size of every Storage allocation
 };
 
 // How fp16 block scales are read (see MLLM_HIP_SCALE_* in the C header): IEEE bit patterns, or the x86 reference build's
@@ -40,9 +47,12 @@ struct HipBackendConfig {
   // Decode hand-over: RMSNorm and the elementwise product also write the Q8_0 image of their result (up to 8 rows), and a
   // Q4_0 / Q8_0 Linear that then reads exactly that tensor takes the image instead of quantizing in every workgroup.
   // Results are bit-identical either way.  The image is dropped as soon as any op of this backend writes to, or the
-  // allocator frees, the memory it describes; writes that bypass the backend (a caller's own hipMemcpy into an
-  // activation tensor) are not seen, hence the switch: MLLM_HIP_FOLD_IMAGES=0 turns it off.
-  bool fold_images = true;
+  // allocator frees, the memory it describes.  Writes that bypass the backend (another backend's op, a caller's own
+  // hipMemcpy into an activation tensor) are NOT seen and would leave a stale image behind, so the hand-over is opt-in:
+  // off by default, MLLM_HIP_FOLD_IMAGES=1 (or setFoldImages) turns it on for graphs in which every writer of an
+  // activation tensor is an op of this backend.  Images are only kept for memory this backend's allocator handed out
+  // (never for external buffers, whose lifetime it cannot see) and at most kMaxImages at a time (oldest dropped first).
+  bool fold_images = false;
 };
 
 class HipBackend final : public Backend {
@@ -64,6 +74,7 @@ class HipBackend final : public Backend {
   const void* findImage(const void* tensor_ptr, int rows, int64_t D) const;
   void noteWrite(const void* ptr, size_t bytes);  // every op calls this for its outputs before it launches
   [[nodiscard]] size_t imageCount() const { return images_.size(); }
+  static constexpr size_t kMaxImages = 64;
 
  private:
   struct Image {

@@ -3,6 +3,8 @@
 //   initializeContext + initHipBackend -> Backend::createOp(kLinear, LinearOpOptions) -> load(ParameterFile)
 //   -> Tensor::to(kHIP) (X2X) -> reshape -> setup -> forward -> Tensor::to(kCPU)
 // (mllm/nn/Layer.cpp:13-34,53-82, mllm/backends/cpu/CPUDispatcher.cpp:56-62).
+#include <hip/hip_runtime_api.h>
+
 #include <cstring>
 #include <string>
 
@@ -228,6 +230,65 @@ extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_decod
   if (be->findImage(h.ptr<void>(), M, H) != nullptr || !refreshed) return -20;
   be->synchronize();
   return handed_over;
+}
+
+// A writer the backend cannot see: RMSNorm -> Linear, then the activation tensor is overwritten with a plain hipMemcpy
+// (what another backend's op or an integrator's own kernel would do) and the Linear runs again on the same tensor.
+// y1_host / y2_host receive the two Linear results; returns the number of images the backend holds for the tensor at the
+// second call (with the backend's default configuration that is 0 and the second result follows the new contents),
+// or a negative code.  `external` != 0 runs the Linear on a caller-owned device buffer instead of a backend tensor, with
+// the hand-over switched on: no image may be made for memory the backend's allocator does not own.
+extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_rewrite_behind_backend(
+    int is_q8, const void* W, const float* norm_w, const float* x_host, const float* h2_host, float* y1_host, float* y2_host, int M,
+    int H, int N, int external) {
+  initializeContext();
+  auto be = hip::initHipBackend();
+  be->setScaleModes(MLLM_HIP_SCALE_IEEE, MLLM_HIP_SCALE_X86_REF);
+  be->setFoldImages(external != 0 ? true : hip::HipBackendConfig().fold_images);  // the default, whatever ran before
+  auto backend = Context::instance().getBackend(kHIP);
+  auto params = ParameterFile::create(ModelFileVersion::kV2);
+  params->push("l.norm.weight", Tensor::fromExternal(const_cast<float*>(norm_w), {H}, kFloat32, kCPU));
+  params->push("l.proj.weight", Tensor::fromExternal(const_cast<void*>(W), {N, H}, is_q8 ? kGGUF_Q8_0 : kGGUF_Q4_0, kCPU));
+  aops::RMSNormOpOptions no;
+  no.epsilon = 1e-6f;
+  aops::LinearOpOptions lo;
+  lo.in_channels = H;
+  lo.out_channels = N;
+  auto norm = backend->createOp(OpTypes::kRMSNorm, no);
+  norm->setName("l.norm");
+  norm->load(params);
+  auto proj = backend->createOp(OpTypes::kLinear, lo);
+  proj->setName("l.proj");
+  proj->load(params);
+  auto run = [&](const BaseOp::ptr_t& op, const std::vector<Tensor>& in, std::vector<Tensor> out = {}) {
+    if (out.empty()) {
+      op->reshape(in, out);
+      op->setup(in, out);
+    }
+    op->forward(in, out);
+    return out;
+  };
+  Tensor x = Tensor::fromExternal(const_cast<float*>(x_host), {M, H}, kFloat32, kCPU).to(kHIP);
+  Tensor h;
+  void* ext = nullptr;
+  if (external) {
+    if (hipMalloc(&ext, (size_t)M * H * 4) != hipSuccess) return -30;
+    h = Tensor::fromExternal(ext, {M, H}, kFloat32, kHIP);
+    run(norm, {x}, {h});
+  } else {
+    h = run(norm, {x})[0];
+  }
+  Tensor y1 = run(proj, {h})[0].to(kCPU);
+  std::memcpy(y1_host, y1.ptr<void>(), y1.bytes());
+  be->synchronize();
+  if (hipMemcpy(h.ptr<void>(), h2_host, (size_t)M * H * 4, hipMemcpyHostToDevice) != hipSuccess) return -31;
+  const int images = be->findImage(h.ptr<void>(), M, H) != nullptr;
+  Tensor y2 = run(proj, {h})[0].to(kCPU);
+  std::memcpy(y2_host, y2.ptr<void>(), y2.bytes());
+  be->synchronize();
+  be->setFoldImages(hip::HipBackendConfig().fold_images);
+  if (ext) (void)hipFree(ext);
+  return images;
 }
 
 // fp32 MatMul through the kMatMul factory slot

@@ -113,6 +113,20 @@ __global__ void identity_tiles_kernel(int M, int tile_h, RouteOut o) {
   if (threadIdx.x == 0) o.ntiles[0] = nt;
 }
 
+// The routing pass keeps five int arrays of E entries in LDS: E is limited to what fits the 64 KB a launch gets without
+// raising the kernel's dynamic-LDS attribute.  The launch status is read before anything that consumes the tile list is
+// queued: a consumer must never walk a list the routing pass did not write.
+constexpr int MOE_MAX_EXPERTS = 3072;
+static int launch_route(const int32_t* ids, int64_t entries, int E, int tile_h, const RouteOut& ro, hipStream_t st) {
+  if (E <= 0 || E > MOE_MAX_EXPERTS) return MLLM_HIP_E_SHAPE;
+  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 5 * (size_t)E * sizeof(int), st, ids, (int)entries, E, tile_h, ro);
+  return (int)hipGetLastError();
+}
+static int launch_identity_tiles(int64_t M, int tile_h, const RouteOut& ro, hipStream_t st) {
+  hipLaunchKernelGGL(identity_tiles_kernel, dim3(1), dim3(256), 0, st, (int)M, tile_h, ro);
+  return (int)hipGetLastError();
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // Q8_0 activation quantization to codes + the fp32 scale that takes part in the arithmetic
 // (quantize_row_q8_0, AVX2 branch, ggml/quantize/quantize_q8.cpp:106-190)
@@ -206,7 +220,7 @@ __global__ __launch_bounds__(MODE == 1 ? 512 : 256) void qgemm_tile_kernel(QGemm
   float* sU = reinterpret_cast<float*>(smem);  // MODE 1 hand-over tile, reuses the staging area after the last chunk
 
   const int tile = blockIdx.x;
-  if (tile >= a.ntiles[0]) return;
+  if (tile >= min(a.ntiles[0], (int)gridDim.x)) return;
   const int e = a.tile_expert[tile], row0 = a.tile_row0[tile], rows = a.tile_rows[tile];
   const int ntt = (rows + 31) >> 5;
   const int last_njg = (rows - 32 * (ntt - 1) + 7) >> 3;  // 8-row groups in the last 32-row tile
@@ -841,7 +855,7 @@ template <int WT, int MODE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qg_kernel(QG2Args a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int t = blockIdx.x;
-  if (t >= a.ntiles[0]) return;
+  if (t >= min(a.ntiles[0], (int)gridDim.x)) return;
   const int e = a.tile_expert[t];
   int row0 = a.tile_row0[t], rows = a.tile_rows[t];
   if constexpr (MODE == 1) {
@@ -968,7 +982,7 @@ int qg_linear_run(int wtype, const void* gemm_packed, const uint16_t* xh, const 
                   int64_t K, void* route_ws, void* partial_ws, hipStream_t st) {
   Carver c(route_ws);
   RouteOut ro = carve_route(c, 1, M);
-  hipLaunchKernelGGL(identity_tiles_kernel, dim3(1), dim3(256), 0, st, (int)M, QG_TILE_H, ro);
+  RC_RET(launch_identity_tiles(M, QG_TILE_H, ro, st));
   QG2Args a{};
   a.W0 = a.W1 = reinterpret_cast<const char*>(gemm_packed);
   a.wstride = 0;
@@ -1017,7 +1031,7 @@ MLLM_API int mllm_hip_linear_q(int wtype, const void* packed, const void* x, int
   const int64_t nblocks = M * (K / QK);
   hipLaunchKernelGGL(quant_rows_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, aq, ad, nblocks,
                      act_scale_mode == MLLM_HIP_SCALE_X86_REF);
-  hipLaunchKernelGGL(identity_tiles_kernel, dim3(1), dim3(256), 0, st, (int)M, TOK_TILE, ro);
+  RC_RET(launch_identity_tiles(M, TOK_TILE, ro, st));
   QGemmArgs a{};
   a.W0 = a.W1 = reinterpret_cast<const char*>(packed);
   a.wstride = 0;
@@ -1084,12 +1098,11 @@ MLLM_API int mllm_hip_moe_set_tuning(int pair_tokens, int row_tokens) {
 
 MLLM_API int mllm_hip_moe_route(const int32_t* topk_ids, int64_t T, int E, int k, int32_t* counts, int32_t* offsets,
                                 int32_t* sorted_idx, void* workspace, void* stream) {
-  if (!topk_ids || !workspace || T <= 0 || E <= 0 || E > 4096 || k <= 0) return MLLM_HIP_E_BADARG;
+  if (!topk_ids || !workspace || T <= 0 || E <= 0 || k <= 0) return MLLM_HIP_E_BADARG;
   hipStream_t st = (hipStream_t)stream;
   Carver c(workspace);
   RouteOut ro = carve_route(c, E, T * k);
-  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 5 * E * sizeof(int), st, topk_ids, (int)(T * k), E, TOK_TILE, ro);
-  HIP_RET(hipGetLastError());
+  RC_RET(launch_route(topk_ids, T * k, E, TOK_TILE, ro, st));
   if (counts) HIP_RET(hipMemcpyAsync(counts, ro.counts, E * sizeof(int), hipMemcpyDeviceToDevice, st));
   if (offsets) HIP_RET(hipMemcpyAsync(offsets, ro.offsets, (E + 1) * sizeof(int), hipMemcpyDeviceToDevice, st));
   if (sorted_idx) HIP_RET(hipMemcpyAsync(sorted_idx, ro.sorted_idx, T * k * sizeof(int), hipMemcpyDeviceToDevice, st));
@@ -1101,11 +1114,11 @@ MLLM_API int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* 
                                 int64_t T, int64_t H, int64_t I, int E, int k, int act_scale_mode, void* workspace,
                                 void* stream) {
   if ((wtype != MLLM_HIP_Q4_0 && wtype != MLLM_HIP_Q8_0) || !gate_packed || !up_packed || !down_packed || !x || !topk_ids ||
-      !topk_w || !y || !workspace || T <= 0 || E <= 0 || E > 4096 || k <= 0)
+      !topk_w || !y || !workspace || T <= 0 || E <= 0 || k <= 0)
     return MLLM_HIP_E_BADARG;
   if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
   if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
-  if (H <= 0 || I <= 0 || H % QK || I % QK) return MLLM_HIP_E_SHAPE;
+  if (H <= 0 || I <= 0 || H % QK || I % QK || E > MOE_MAX_EXPERTS) return MLLM_HIP_E_SHAPE;
   if (T * H >= ((int64_t)1 << 32) || T * k * I >= ((int64_t)1 << 32) || T * k > INT32_MAX) return MLLM_HIP_E_SHAPE;
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
   hipStream_t st = (hipStream_t)stream;
@@ -1118,8 +1131,7 @@ MLLM_API int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* 
     Carver cr(workspace);
     RowsCarve rc = carve_rows(cr, T, H, I, E, k);
     const unsigned max_tiles = (unsigned)(E + (T * k) / moe_rows_tile() + 1);
-    hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 5 * E * sizeof(int), st, topk_ids, (int)(T * k), E, moe_rows_tile(), rc.ro);
-    HIP_RET(hipGetLastError());
+    RC_RET(launch_route(topk_ids, T * k, E, moe_rows_tile(), rc.ro, st));
     int r = launch_moe_rows(wtype, gate_packed, up_packed, down_packed, x, x_dtype, rc.ro.tile_expert, rc.ro.tile_row0, rc.ro.tile_rows,
                             rc.ro.ntiles, rc.ro.sorted_idx, rc.img, rc.per, T, H, I, E, k, x86, max_tiles, st);
     if (r) return r;
@@ -1137,7 +1149,7 @@ MLLM_API int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* 
   RouteOut ro = carve_route(c, E, T * k);
   const unsigned max_tiles = (unsigned)(E + (T * k) / TOK_TILE + 1);
 
-  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 5 * E * sizeof(int), st, topk_ids, (int)(T * k), E, TOK_TILE, ro);
+  RC_RET(launch_route(topk_ids, T * k, E, TOK_TILE, ro, st));
   const int64_t nblocks = T * (H / QK);
   hipLaunchKernelGGL(quant_rows_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, xq, xd, nblocks, x86);
 
@@ -1265,11 +1277,11 @@ MLLM_API int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const v
                                      int64_t T, int64_t H, int64_t I, int E, int k, int act_scale_mode, void* workspace,
                                      void* stream) {
   if ((wtype != MLLM_HIP_Q4_0 && wtype != MLLM_HIP_Q8_0) || !gate_packed || !up_packed || !down_packed || !x || !topk_ids ||
-      !topk_w || !y || !workspace || T <= 0 || E <= 0 || E > 4096 || k <= 0)
+      !topk_w || !y || !workspace || T <= 0 || E <= 0 || k <= 0)
     return MLLM_HIP_E_BADARG;
   if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
   if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
-  if (H <= 0 || I <= 0 || H % QK || I % QK) return MLLM_HIP_E_SHAPE;
+  if (H <= 0 || I <= 0 || H % QK || I % QK || E > MOE_MAX_EXPERTS) return MLLM_HIP_E_SHAPE;
   if (T * H * 2 >= ((int64_t)1 << 32) || T * k * I * 2 >= ((int64_t)1 << 32) || T * k > INT32_MAX) return MLLM_HIP_E_SHAPE;
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
   hipStream_t st = (hipStream_t)stream;
@@ -1282,7 +1294,7 @@ MLLM_API int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const v
   RouteOut ro = carve_route(c, E, T * k);
   const unsigned max_tiles = (unsigned)(E + (T * k) / QG_TILE_H + 1);
 
-  hipLaunchKernelGGL(moe_route_kernel, dim3(1), dim3(1024), 5 * E * sizeof(int), st, topk_ids, (int)(T * k), E, QG_TILE_H, ro);
+  RC_RET(launch_route(topk_ids, T * k, E, QG_TILE_H, ro, st));
   const int64_t nblocks = T * (H / QK);
   hipLaunchKernelGGL(qg_act_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, xh, xl, nblocks, x86);
 
@@ -1335,7 +1347,7 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
                                  int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H,
                                  int64_t I, int E, int k, void* workspace, void* stream) {
   if ((wtype != MLLM_HIP_Q4_K && wtype != MLLM_HIP_Q6_K) || !gate_packed || !up_packed || !down_packed || !x || !topk_ids ||
-      !topk_w || !y || !workspace || T <= 0 || E <= 0 || E > 4096 || k <= 0)
+      !topk_w || !y || !workspace || T <= 0 || E <= 0 || k <= 0)
     return MLLM_HIP_E_BADARG;
   if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
   if (H <= 0 || I <= 0 || H % 256 || I % 256 || T * k > 65535) return MLLM_HIP_E_SHAPE;

@@ -13,6 +13,12 @@
     hipError_t e__ = (expr);             \
     if (e__ != hipSuccess) return (int)e__; \
   } while (0)
+// the same for calls of this library that return its own int codes (0 = success)
+#define RC_RET(expr)         \
+  do {                       \
+    int rc__ = (expr);       \
+    if (rc__ != 0) return rc__; \
+  } while (0)
 
 namespace mllmhip {
 

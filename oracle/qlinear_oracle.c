@@ -465,10 +465,11 @@ ORC_API void orc_rmsnorm(const float* x, const float* w, float* y, int64_t rows,
     for (; i < D; i++) acc += xr[i] * xr[i];
     float rms = 1.0f / sqrtf(acc / (float)D + eps);
     i = 0;
-    for (; i + 8 <= D; i++) {
-      float m = add_unit_offset ? (w[i] + 1.0f) * rms : w[i] * rms;
-      yr[i] = xr[i] * m;
-    }
+    for (; i + 8 <= D; i += 8)
+      for (int l = 0; l < 8; l++) {
+        float m = add_unit_offset ? (w[i + l] + 1.0f) * rms : w[i + l] * rms;
+        yr[i + l] = xr[i + l] * m;
+      }
     for (; i < D; i++) yr[i] = add_unit_offset ? xr[i] * rms * (w[i] + 1.0f) : xr[i] * rms * w[i];
   }
 }

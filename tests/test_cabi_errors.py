@@ -54,10 +54,12 @@ def _cases():
                                     (8, 48, SHAPE), (9, 48, SHAPE), (0, Q6_K, BADARG)]),
         "mllm_hip_moe_ffn_q": ([Q4_0, P, P, P, P, F32, P, P, P, 4, 64, 64, 8, 2, 0, P, None],
                                [(1, None, BADARG), (4, None, BADARG), (6, None, BADARG), (7, None, BADARG), (8, None, BADARG),
-                                (15, None, BADARG), (10, 48, SHAPE), (11, 48, SHAPE), (12, 0, BADARG), (13, 0, BADARG)]),
+                                (15, None, BADARG), (10, 48, SHAPE), (11, 48, SHAPE), (12, 0, BADARG), (13, 0, BADARG), (12, 3073, SHAPE)]),
         "mllm_hip_moe_ffn_q_gemm": ([Q4_0, P, P, P, P, F32, P, P, P, 4, 64, 64, 8, 2, 0, P, None],
                                     [(2, None, BADARG), (3, None, BADARG), (15, None, BADARG), (10, 48, SHAPE), (11, 48, SHAPE),
-                                     (4, ODD, ALIGN), (0, Q4_K, BADARG)]),
+                                     (4, ODD, ALIGN), (0, Q4_K, BADARG), (12, 3073, SHAPE)]),
+        # the routing pass keeps five int arrays of E entries in 64 KB of LDS
+        "mllm_hip_moe_route": ([P, 4, 8, 2, None, None, None, P, None], [(0, None, BADARG), (7, None, BADARG), (2, 3073, SHAPE), (2, 0, BADARG)]),
         "mllm_hip_moe_ffn_kq": ([Q4_K, P, P, P, P, F32, P, P, P, 4, 256, 256, 8, 2, P, None],
                                 [(0, Q4_0, BADARG), (1, None, BADARG), (3, None, BADARG), (4, None, BADARG), (6, None, BADARG),
                                  (14, None, BADARG), (10, 128, SHAPE), (11, 320, SHAPE), (9, 40000, SHAPE), (4, ODD, ALIGN)]),

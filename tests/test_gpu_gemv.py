@@ -105,7 +105,7 @@ SHAPES = [("c1", 6144, 2048)] + [(k, n, kk) for k, (n, kk) in synth.QWEN3_4B_LAY
 @pytest.mark.parametrize("name,N,K", SHAPES)
 @pytest.mark.parametrize("wtype", [0, 1])
 def test_gemv_full_shapes(name, N, K, wtype):
-    rng = synth.rng_for(1, hash((name, wtype)) % 1000)
+    rng = synth.rng_for(1, 2 * [s[0] for s in SHAPES].index(name) + wtype)  # fixed: the same inputs in every run
     W = synth.make_weight(rng, wtype, N, K)
     w = ql.PackedQWeight(wtype, torch.from_numpy(W))
     bias = rng.standard_normal(N).astype(np.float32)

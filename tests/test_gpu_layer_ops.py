@@ -66,6 +66,21 @@ def test_rmsnorm(rows, D, dtype):
             assert rel_l2(y, _bf16_round(want)) < TOL
 
 
+@pytest.mark.parametrize("rows,D", [(1, 2560), (3, 128), (4, 4096), (2, 40)])
+def test_rmsnorm_fp32_bit_for_bit(rows, D):
+    """x * (w * rms) in the reference's operation order (x86/rmsnorm.cpp:29-47), compared bit for bit: the rows hold small
+    integers, so the sum of squares is exact in fp32 whatever the order of its additions and rms is the same number on
+    both sides; every difference left would be an operation-order difference in the elementwise part."""
+    rng = synth.rng_for(6, 50000 + rows * 7 + D)
+    xf = rng.integers(-15, 16, (rows, D)).astype(np.float32)
+    w = (1 + 0.2 * rng.standard_normal(D)).astype(np.float32)
+    for off in (False, True):
+        announce("rmsnorm bit-exact", rows, D, off)
+        y = ql.rmsnorm(to_dev(xf), to_dev(w), 1e-6, off).cpu().numpy()
+        want = orc.rmsnorm(xf, w, 1e-6, off)
+        assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+
+
 @pytest.mark.parametrize("M,K", [(1, 2560), (2, 2560), (3, 4096), (4, 9728), (8, 2560), (1, 96), (6, 32)])
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_rmsnorm_writes_the_image_of_what_it_stored(M, K, dtype):

@@ -295,3 +295,27 @@ def test_decoder_mlp_through_the_op_factories(is_q8):
         assert rel_l2(ys[0], want) < (1e-3 if M <= 8 else 5e-3)
         assert rel_l2(sm, orc.softmax(g)) < 1e-3
         assert np.array_equal(ti, orc.topk(sm, k, True, False)[1])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("external", [0, 1])
+def test_linear_requantizes_after_a_write_the_backend_cannot_see(external):
+    """RMSNorm -> Linear, then the activation tensor is overwritten by a plain hipMemcpy and the Linear runs again: the
+    second result must follow the new contents.  With the backend's defaults no quantized image is kept at all (the
+    hand-over is opt-in); with the hand-over on, a caller-owned buffer (external) never gets one either."""
+    from oracle import oracle as orc
+    from gpu_util import announce, rel_l2
+    L = _host()
+    rng = synth.rng_for(5, 90 + external)
+    M, H, N = 4, 256, 320
+    W = synth.make_weight(rng, 0, N, H)
+    nw = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
+    x = synth.make_x_fp32(rng, M, H)
+    h2 = synth.make_x_fp32(rng, M, H) * 3
+    y1, y2 = np.empty((M, N), np.float32), np.empty((M, N), np.float32)
+    vp = lambda a: a.ctypes.data_as(C.c_void_p)
+    announce("rewrite behind the backend", external)
+    rc = L.mllm_hip_backend_run_rewrite_behind_backend(0, vp(W), vp(nw), vp(x), vp(h2), vp(y1), vp(y2), M, H, N, external)
+    assert rc == 0, rc  # no image for the tensor at the second call
+    assert rel_l2(y1, orc.linear_q(orc.rmsnorm(x, nw, 1e-6), W, 0, None, orc.SCALE_X86_REF)) < 2e-6
+    assert rel_l2(y2, orc.linear_q(h2, W, 0, None, orc.SCALE_X86_REF)) < 2e-6

@@ -69,6 +69,32 @@ def test_rmsnorm_definition():
     assert np.allclose(y, 3.0, rtol=1e-6)
 
 
+def test_rmsnorm_operation_order_in_whole_vectors_and_tail():
+    """x86/rmsnorm.cpp:29-36,41-47: every whole vector of eight takes x * (w * rms), only the D % 8 tail takes
+    x * rms * w.  The two orders differ in the last bit for many elements; both are computed here with numpy's fp32
+    scalars (one IEEE rounding per operation, nothing shared with the C restatement)."""
+    f = np.float32
+    for D in (16, 64, 37, 2560):
+        rng = np.random.default_rng(100 + D)
+        # small integers: the sum of squares is exact in fp32 in any order, so rms is the same number for everybody
+        x = rng.integers(-15, 16, (1, D)).astype(np.float32)
+        x[0, -8:] = [3, -5, 7, 9, -11, 13, 14, -15]
+        w = (1 + 0.2 * rng.standard_normal(D)).astype(np.float32)
+        eps = f(1e-6)
+        rms = f(1.0) / np.sqrt(f(np.sum(x.astype(np.float64) ** 2)) / f(D) + eps, dtype=np.float32)
+        for off in (False, True):
+            ww = w + f(1.0) if off else w
+            vec_form = x[0] * (ww * rms)          # fp32 throughout
+            tail_form = (x[0] * rms) * ww
+            n_vec = D - D % 8
+            want = np.concatenate([vec_form[:n_vec], tail_form[n_vec:]])
+            got = orc.rmsnorm(x, w, 1e-6, off)[0]
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (D, off)
+            # the case must be able to tell the orders apart in the last seven elements of the vector part
+            lo, hi = max(0, n_vec - 7), n_vec
+            assert np.any(vec_form[lo:hi].view(np.uint32) != tail_form[lo:hi].view(np.uint32)), (D, off)
+
+
 def test_softmax_definition():
     rng = np.random.default_rng(3)
     for n in (4, 16, 17, 128, 133):
