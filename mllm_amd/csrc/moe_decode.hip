@@ -396,7 +396,7 @@ template <int WT, int XT>
 __global__ __launch_bounds__(512, 4) void moe_rows_gateup_kernel(MoeRowsArgs b) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int t = blockIdx.y;
-  if (t >= min(b.ntiles[0], (int)gridDim.x)) return;
+  if (t >= min(b.ntiles[0], (int)gridDim.y)) return;
   const int e = b.tile_expert[t], row0 = b.tile_row0[t], rows = b.tile_rows[t];
   if (rows <= 2) moe_rows_gateup<WT, XT, 2>(b, e, row0, rows, smem);
   else if (rows <= 4) moe_rows_gateup<WT, XT, 4>(b, e, row0, rows, smem);
@@ -409,7 +409,7 @@ __global__ __launch_bounds__(NW * 64) void moe_rows_down_kernel(MoeRowsArgs b) {
   extern __shared__ __align__(16) unsigned char smem[];
   const MoeDecodeArgs& a = b.d;
   const int t = blockIdx.y;
-  if (t >= min(b.ntiles[0], (int)gridDim.x)) return;
+  if (t >= min(b.ntiles[0], (int)gridDim.y)) return;
   const int e = b.tile_expert[t], row0 = b.tile_row0[t], rows = b.tile_rows[t];
   const int nb = a.I / QK, nbp = (int)scale_row_stride(a.I);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
