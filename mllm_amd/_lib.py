@@ -53,6 +53,7 @@ def lib():
         L.mllm_hip_linear_q_gemv.argtypes = [ci, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi_ws.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp, vp]
+        L.mllm_hip_linear_q_gemv_multi_static.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_fused.argtypes = [ci, ci, C.POINTER(GemvPart), C.POINTER(GemvFusion), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_mlp_gate_up_q.argtypes = [ci, vp, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]
         L.mllm_hip_mlp_set_tuning.argtypes = [ci]

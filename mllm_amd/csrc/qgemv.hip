@@ -261,6 +261,29 @@ using namespace mllmhip;
 // =========================================================================================================
 MLLM_API const char* mllm_hip_version(void) { return "mllm-hip-qlinear 0.1 (gfx950)"; }
 
+// Scratch of mllm_hip_linear_q_gemv_multi_static: the quantized image of up to eight activation rows, in device memory
+// that belongs to the loaded code object (one copy per GPU, held until the process ends).  The name below is a host-side
+// stand-in only; the device address is looked up once per device (static_scratch) and only that pointer is ever handed
+// to a kernel.
+constexpr int64_t GEMV_STATIC_MAX_K = 32768;
+constexpr size_t GEMV_STATIC_BYTES = (size_t)8 * (GEMV_STATIC_MAX_K / QK) * 40;  // 320 KB
+static __device__ __align__(256) unsigned char scratch[GEMV_STATIC_BYTES];
+constexpr int MAX_DEVICES = 64;
+static void* g_scratch_ptr[MAX_DEVICES];
+
+// device address of the scratch array on `device`, which must be the current device; 0 + *out on success
+static int static_scratch(int device, void** out) {
+  if (device < 0 || device >= MAX_DEVICES) return MLLM_HIP_E_NODEVICE;
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    HIP_RET(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return MLLM_HIP_E_NODEVICE;
+    g_scratch_ptr[device] = p;
+  }
+  *out = g_scratch_ptr[device];
+  return 0;
+}
+
 MLLM_API int mllm_hip_init(int device) {
   int count = 0;
   HIP_RET(hipGetDeviceCount(&count));
@@ -268,7 +291,14 @@ MLLM_API int mllm_hip_init(int device) {
   hipDeviceProp_t prop;
   HIP_RET(hipGetDeviceProperties(&prop, device));
   if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return MLLM_HIP_E_NODEVICE;
-  return 0;
+  // the per-device address of the static scratch array, looked up with that device current and put back afterwards
+  int cur = 0;
+  HIP_RET(hipGetDevice(&cur));
+  if (cur != device) HIP_RET(hipSetDevice(device));
+  void* p = nullptr;
+  const int rc = static_scratch(device, &p);
+  if (cur != device) HIP_RET(hipSetDevice(cur));
+  return rc;
 }
 
 MLLM_API int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream) {
@@ -342,6 +372,21 @@ MLLM_API size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K) {
 static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual, const void* x,
                            int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, void* stream);
 
+// everything that can be refused without touching the device
+static int gemv_check_args(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M, int64_t K,
+                           int act_scale_mode, const void* workspace) {
+  if (nparts < 1 || nparts > GEMV_MAX_PARTS || !parts) return MLLM_HIP_E_BADARG;
+  if (!x || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16 && x_dtype != MLLM_HIP_Q8_IMAGE)) return MLLM_HIP_E_BADARG;
+  if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
+  if (M < 1) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
+  for (int p = 0; p < nparts; p++) {
+    RC_RET(check_w(wtype, parts[p].packed, parts[p].N, K));
+    if (!parts[p].y) return MLLM_HIP_E_BADARG;
+  }
+  return 0;
+}
+
 // More than eight rows of raw activations: passes of eight rows, each streaming the weights again (the same arithmetic row by
 // row; up to about 32 rows this is faster than the matrix-core GEMM path, whose 128-row tiles leave most of the chip idle).
 static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fu, const void* x,
@@ -368,17 +413,11 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
 
 static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual, const void* x,
                            int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
-  if (nparts < 1 || nparts > GEMV_MAX_PARTS || !parts) return MLLM_HIP_E_BADARG;
-  if (!x || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16 && x_dtype != MLLM_HIP_Q8_IMAGE)) return MLLM_HIP_E_BADARG;
-  if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
-  if (M < 1 || M > 8) return MLLM_HIP_E_SHAPE;
-  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
+  RC_RET(gemv_check_args(wtype, nparts, parts, x, x_dtype, M, K, act_scale_mode, workspace));
+  if (M > 8) return MLLM_HIP_E_SHAPE;
   GemvArgs a{};
   int64_t nmax = 0;
   for (int p = 0; p < nparts; p++) {
-    int rc = check_w(wtype, parts[p].packed, parts[p].N, K);
-    if (rc) return rc;
-    if (!parts[p].y) return MLLM_HIP_E_BADARG;
     a.part[p].w = packed_view(wtype, parts[p].packed, parts[p].N, K);
     a.part[p].bias = parts[p].bias;
     a.part[p].residual = residual ? residual[p] : nullptr;
@@ -435,6 +474,20 @@ MLLM_API int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_h
                                              int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
   if (x_dtype == MLLM_HIP_Q8_IMAGE) return MLLM_HIP_E_BADARG;
   return gemv_multi_impl(wtype, nparts, parts, nullptr, x, x_dtype, M, K, act_scale_mode, workspace, stream);
+}
+
+// The call above for callers that cannot allocate or pass a workspace: the image lives in the static scratch array of the
+// current device.  Calls that overlap on one GPU (two streams) would share it and race.
+MLLM_API int mllm_hip_linear_q_gemv_multi_static(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,
+                                                 int M, int64_t K, int act_scale_mode, void* stream) {
+  if (x_dtype == MLLM_HIP_Q8_IMAGE) return MLLM_HIP_E_BADARG;
+  RC_RET(gemv_check_args(wtype, nparts, parts, x, x_dtype, M, K, act_scale_mode, nullptr));
+  if (K > GEMV_STATIC_MAX_K) return MLLM_HIP_E_SHAPE;  // the image of eight rows would not fit the array
+  int dev = 0;
+  HIP_RET(hipGetDevice(&dev));
+  void* ws = nullptr;
+  RC_RET(static_scratch(dev, &ws));
+  return gemv_multi_impl(wtype, nparts, parts, nullptr, x, x_dtype, M, K, act_scale_mode, ws, stream);
 }
 
 MLLM_API int mllm_hip_linear_q_gemv_fused(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fusion,

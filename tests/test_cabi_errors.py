@@ -35,6 +35,9 @@ def _cases():
                                           (6, 40, SHAPE), (3, ODD, ALIGN)]),
         "mllm_hip_linear_q_gemv_multi_ws": ([Q8_0, 1, part, P, BF16, 4, 64, 0, P, None],
                                             [(3, None, BADARG), (6, 40, SHAPE), (8, ODD, ALIGN)]),
+        # the variant that allocates nothing: rows longer than its static array hold are refused
+        "mllm_hip_linear_q_gemv_multi_static": ([Q8_0, 1, part, P, BF16, 4, 64, 0, None],
+                                                [(3, None, BADARG), (4, IMAGE, BADARG), (6, 32768 + 32, SHAPE), (6, 40, SHAPE)]),
         "mllm_hip_linear_q": ([Q4_0, P, P, F32, None, P, 16, 64, 64, 0, P, None],
                               [(1, None, BADARG), (2, None, BADARG), (5, None, BADARG), (10, None, BADARG), (8, 50, SHAPE),
                                (6, 0, BADARG)]),
