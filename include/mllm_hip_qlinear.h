@@ -189,6 +189,12 @@ int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const void* up_p
                             const void* x, int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T,
                             int64_t H, int64_t I, int E, int k, int act_scale_mode, void* workspace, void* stream);
 
+/* mllm_hip_moe_ffn_q_gemm has two forms.  0 (default): the reference's block arithmetic itself on the matrix cores: the
+ * exact integer sum of every 32-element block (fp16 MFMAs on the integer codes), the exact product dW * dX of its two
+ * scales (a third MFMA), one fp32 fused multiply-add per block; only the order in which blocks are added differs from the
+ * CPU path.  1: fp16 operands with the block scales folded in as in mllm_hip_linear_q_gemm (about 2e-4 relative L2). */
+int mllm_hip_moe_gemm_set_path(int path);
+
 /* ---------------------------------------------------------------------------------------------------------
  * W8A8 Linear (prefill): per-token dynamic int8 activations x int8 weights with per-channel scales
  * replaces: CompressedTensorsW8A8Int8Scheme.apply = per_token_quant_int8 + int8_scaled_mm
@@ -284,7 +290,7 @@ int mllm_hip_w4a16_packed_set_tuning(int tile);
  * gate_packed / up_packed: E pre-packed [I][H] matrices back to back, expert e at + e * mllm_hip_q_packed_bytes(wtype, I, H);
  * down_packed: E pre-packed [H][I] matrices, stride mllm_hip_q_packed_bytes(wtype, H, I).
  * x [T][H] fp32 or bf16; topk_ids int32 [T][k] (entries outside [0, E) contribute nothing); topk_w fp32 [T][k];
- * y fp32 [T][H].  H % 32 == 0, I % 32 == 0, E <= 3072 (more: MLLM_HIP_E_SHAPE).  workspace: mllm_hip_moe_workspace_bytes. */
+ * y fp32 [T][H], 16-byte aligned like x and the workspace.  H % 32 == 0, I % 32 == 0, E <= 3072 (more: MLLM_HIP_E_SHAPE).  workspace: mllm_hip_moe_workspace_bytes. */
 size_t mllm_hip_moe_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k);
 int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x,
                        int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H,

@@ -889,19 +889,482 @@ static int launch_qg(const QG2Args& a, unsigned max_tiles, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
-// y[t][h] = sum_j per[t*k + j][h] * w[t][j]   (multiply, then add in j order: modeling_qwen3_moe_fa2.hpp:233-236)
-__global__ void moe_combine_kernel(const float* __restrict__ per, const float* __restrict__ w, const int32_t* __restrict__ ids,
-                                   float* __restrict__ y, int64_t T, int H, int k, int E) {
+// =========================================================================================================
+// Exact block sums on the matrix cores ("qx"): the reference's arithmetic itself for many rows
+//
+//   y[row][n] = sum_b fp32(dW[n][b] * dX[row][b]) * float(sum_32 qW * qX)
+//
+// (llamafile_sgemm.cpp:697-743: Cv += set1(dW * dX) * float(int32 block sum)).  Per 32-row x 32-channel tile and block,
+// four v_mfma_f32_32x32x16_f16 and sixteen fp32 FMAs:
+//   * the block sum: two MFMAs whose operands are integers held as fp16 numbers.  The activation codes are stored that
+//     way; a weight code is OR-ed into the mantissa of 1024.0 (nibble at bits 0..3 of a half-word) or of 64.0 (bits
+//     4..7), i.e. it enters as 1024 + q or 64 + q (q = 0..15; Q8_0: 1024 + 128 + q), which costs five operations per
+//     eight 4-bit codes.  A third MFMA puts the correction in front: its operands are the constants -(1024 + 8),
+//     -(64 + 8) and the sums of the activation codes that meet each constant (two per row and block, from the producer
+//     of the activations), so the chain starts at -sum(offset * qX) and ends at sum((q - 8) * qX).  Every product and
+//     every partial sum is an integer below 2^24: the fp32 result IS the int32 block sum, already a float.
+//   * the 32 x 32 scale products dW[n] * dX[row]: a fourth MFMA, an outer product of the two fp16 scales sitting in one
+//     K slot of otherwise zero operands; an 11-bit by 11-bit product is exact in fp32.
+//   * acc = fma(dW * dX, block sum, acc): the reference's operation.  Only the order in which blocks are added differs
+//     from the CPU path.
+// Same gemm-packed weights and tile list as the fp16-operand kernel.  Activations: Q8_0 codes as fp16 integers
+// [rows][K] and one record of three dwords per row and K step of 64: the fp16 scales of the step's two blocks, then per
+// block the two partial code sums (elements with bit 1 of k clear | set) as fp16 integers.
+// =========================================================================================================
+struct QXArgs {
+  const char* W0;        // gemm-packed weights of matrix 0 (gate, or the only matrix), expert e at W0 + e * wstride
+  const char* W1;        // matrix 1 (up) in the gate/up mode
+  size_t wstride;
+  const uint16_t* xq;    // Q8_0 codes of the activations as fp16 integers [a_rows][K]
+  const uint32_t* xd;    // [a_rows][KD][3] dwords: fp16 scales of blocks 2j | 2j+1, then per block fp16(sum of the codes
+                         // with (k & 2) == 0) | fp16(sum of the others) << 16; zeros past the end
+  const int* a_index;    // activation row of sorted position pos is a_index[pos] / a_div ; null: pos itself
+  int a_div;
+  int a_rows;
+  const int* o_index;    // output row of sorted position pos (null: pos itself)
+  float* out;            // fp32 [..][N]       (one-matrix mode)
+  const float* bias;     // [N] or null        (one-matrix mode)
+  uint16_t* hq;          // gate/up mode: Q8_0 codes of silu(g)*u as fp16 integers [rows][N]
+  uint32_t* hd;          // gate/up mode: their records [rows][ceil(N/64)][3], as xd
+  const int* tile_expert;
+  const int* tile_row0;
+  const int* tile_rows;
+  const int* ntiles;
+  int N, K;
+  int x86_scale;
+};
+
+// masks and exponent patterns of qx_codes, kept in registers (v_and_or_b32 takes no literal constants)
+struct QXConst {
+  uint32_t m_lo, m_hi, e_1024, e_64;
+};
+__device__ __forceinline__ QXConst qx_const(int wtype) {
+  QXConst c{wtype == MLLM_HIP_Q4_0 ? 0x000f000fu : 0x00ff00ffu, 0x00f000f0u, 0x64006400u, 0x54005400u};
+  asm volatile("" : "+v"(c.m_lo), "+v"(c.m_hi), "+v"(c.e_1024), "+v"(c.e_64));
+  return c;
+}
+// the eight weight codes of MFMA step d (16 K elements, this lane's half) as fp16 numbers offset + code:
+// Q4_0: 1024 + q for the elements with (k & 2) == 0, 64 + q for the others (q = 0..15); Q8_0: 1152 + q (q = -128..127)
+template <int WT>
+__device__ __forceinline__ f16x8 qx_codes(const u32x4 (&rq)[WT == MLLM_HIP_Q4_0 ? 1 : 2], int d, const QXConst& c) {
+  uint32_t o[4];
+  if (WT == MLLM_HIP_Q4_0) {
+    // pair i of the dword sits in nibbles i and 4 + i.  Nibbles at bits 0..3 of a half-word land in the mantissa of 1024.0
+    // (unit 1), nibbles at bits 4..7 in the mantissa of 64.0 (unit 1/16): pairs 0 and 1 need no shift, pairs 2 and 3 one
+    // shift by 8 for both.
+    const uint32_t v = rq[0][d], t = v >> 8;
+    o[0] = (v & c.m_lo) | c.e_1024;
+    o[1] = (v & c.m_hi) | c.e_64;
+    o[2] = (t & c.m_lo) | c.e_1024;
+    o[3] = (t & c.m_hi) | c.e_64;
+  } else {
+    // two dwords of four codes each in byte order e0 e2 e1 e3; + 128 makes them unsigned
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+      const uint32_t w = rq[d >> 1][2 * (d & 1) + h] ^ 0x80808080u;
+      o[2 * h] = (w & c.m_lo) | c.e_1024;
+      o[2 * h + 1] = ((w >> 8) & c.m_lo) | c.e_1024;
+    }
+  }
+  return __builtin_bit_cast(f16x8, u32x4{o[0], o[1], o[2], o[3]});
+}
+// fp16 pair (-offset of the elements with (k & 2) == 0, -offset of the others) including the 8 of Q4_0's code offset
+__host__ __device__ constexpr uint32_t qx_offsets(int wtype) { return wtype == MLLM_HIP_Q4_0 ? 0xD480E408u : 0xE480E480u; }
+
+// One tile: `rows` (<= 32 TM) sorted positions from row0 x 128 TN channels from n0, NW weight matrices (1, or gate + up).
+template <int WT, int NW, int TM, int TN>
+__device__ __forceinline__ void qx_tile(const QXArgs& a, const int e, const int row0, const int rows, const int n0,
+                                        unsigned char* smem) {
+  constexpr int BK = 64, LDK = 2 * BK + 16;
+  constexpr int BM = TM * 32, WN = TN * 32;
+  constexpr int CA = TM;                      // 16-byte activation chunks per thread and K step
+  constexpr int STAGE = BM * LDK + BM * 48;   // code rows, then per row the record's three dwords, each the first of a
+                                              // 16-byte MFMA operand whose other K slots are zero
+  constexpr int QW = WT == MLLM_HIP_Q4_0 ? 1 : 2;
+  constexpr int ST = 4;                       // K steps of weights in flight per wave
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lrow = lane & 31, hi = lane >> 5;
+  const int Kp = (int)qg_kp(a.K), kbs = Kp / 64, nbs = (int)(qg_np(a.N) / 32), KD = (a.K + 63) / 64;
+  const int64_t qbytes = qg_qbytes(WT, a.N, a.K), wbytes = qg_bytes(WT, a.N, a.K);
+
+  const __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.xq), 0, (uint32_t)((int64_t)a.a_rows * a.K * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rD = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(a.xd), 0, (uint32_t)((int64_t)a.a_rows * KD * 12), 0x00020000);
+  __amdgpu_buffer_rsrc_t rW[NW];
+  rW[0] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a.W0 + (size_t)e * a.wstride), 0, (uint32_t)wbytes, 0x00020000);
+  if (NW == 2) rW[NW - 1] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a.W1 + (size_t)e * a.wstride), 0, (uint32_t)wbytes, 0x00020000);
+
+  // activation chunk c of a thread: tile row (tid + 256 c) / 8, 16-byte column (tid + 256 c) % 8.  Rows past `rows` repeat
+  // the last one (never stored); columns past K read as zeros (out-of-range buffer offsets).
+  uint32_t offA[CA];
+  const int colA = (tid % 8) * 8;
+#pragma unroll
+  for (int c = 0; c < CA; c++) {
+    const int pos = row0 + min((tid + c * 256) / 8, rows - 1);
+    const int arow = a.a_index ? a.a_index[pos] / a.a_div : pos;
+    offA[c] = (uint32_t)(((int64_t)arow * a.K + colA) * 2);
+  }
+  // the record of a row and K step: threads 0 .. BM-1, one row each
+  uint32_t offD = 0xffffffffu;
+  if (tid < BM) {
+    const int pos = row0 + min(tid, rows - 1);
+    const int arow = a.a_index ? a.a_index[pos] / a.a_div : pos;
+    offD = (uint32_t)((int64_t)arow * KD * 12);
+  }
+  uint32_t offQ[TN], offS[TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int nb = min((n0 + wave * WN) / 32 + j, nbs - 1);
+    offQ[j] = (uint32_t)((int64_t)nb * kbs * (1024 * QW) + lane * 16);
+    offS[j] = (uint32_t)(qbytes + ((int64_t)nb * kbs * 32 + lrow) * 4);
+  }
+  typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+  // Activations travel two K steps ahead of their use, in two register sets.  Vector memory returns in order: the wait for
+  // a step's activations also waits for every load issued before them, so loading them only one step ahead would cut
+  // the weights' lead (ST steps) down to one step as well.
+  u32x4 ga[2][CA];
+  u32x3 gd[2] = {{0u, 0u, 0u}, {0u, 0u, 0u}};
+  auto loadA = [&](int set, int kt) {
+    const bool ok = kt * BK + colA < a.K;
+#pragma unroll
+    for (int c = 0; c < CA; c++) ga[set][c] = __builtin_amdgcn_raw_buffer_load_b128(rA, ok ? offA[c] : 0xffffffffu, kt * BK * 2, 0);
+    if (tid < BM) gd[set] = __builtin_amdgcn_raw_buffer_load_b96(rD, kt < KD ? offD : 0xffffffffu, kt * 12, 0);
+  };
+  auto storeA = [&](int set, int buf) {
+#pragma unroll
+    for (int c = 0; c < CA; c++) {
+      const int idx = tid + c * 256;
+      *reinterpret_cast<u32x4*>(smem + buf * STAGE + (idx / 8) * LDK + (idx % 8) * 16) = ga[set][c];
+    }
+    if (tid < BM) {
+      u32x4* rec = reinterpret_cast<u32x4*>(smem + buf * STAGE + BM * LDK + tid * 48);
+      rec[0] = u32x4{gd[set].x, 0u, 0u, 0u};
+      rec[1] = u32x4{gd[set].y, 0u, 0u, 0u};
+      rec[2] = u32x4{gd[set].z, 0u, 0u, 0u};
+    }
+  };
+
+  v16f acc[NW][TN][TM];
+#pragma unroll
+  for (int w = 0; w < NW; w++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[w][j][i][r] = 0.f;
+
+  u32x4 rq[ST][NW][TN][QW];  // packed codes of the K steps in flight (ring, slot = step % ST)
+  uint32_t rs[ST][NW][TN];   // their scale dwords
+  auto loadW = [&](int slot, int kt) {
+    const bool ok = kt < kbs;  // steps past the end read nothing (zeros): the ring is always full
+#pragma unroll
+    for (int w = 0; w < NW; w++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+#pragma unroll
+        for (int p = 0; p < QW; p++)
+          rq[slot][w][j][p] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], ok ? offQ[j] : 0xffffffffu, (kt * QW + p) * 1024, 0);
+        rs[slot][w][j] = __builtin_amdgcn_raw_buffer_load_b32(rW[w], ok ? offS[j] : 0xffffffffu, kt * 128, 0);
+      }
+  };
+  // Scale operand of the weights: the fp16 scale of the step's first block in K slot 0 (low half of the first register), of
+  // its second block in K slot 1 (high half), in the lanes of the low K half only; every other K slot is zero.  The
+  // activations' scale pair and code sums are used as they come (first register of an otherwise zero operand): what a K
+  // slot holds does not matter where the other operand is zero.
+  static_assert(TM == 1, "one row tile per workgroup");
+  const uint32_t msk0 = hi ? 0u : 0x0000ffffu, msk1 = hi ? 0u : 0xffff0000u;
+  const v16f zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const QXConst kc = qx_const(WT);
+  const f16x8 off_op = __builtin_bit_cast(f16x8, u32x4{hi ? 0u : qx_offsets(WT), 0u, 0u, 0u});
+
+  // A "group" is one (block, matrix, column tile): four MFMAs (offset correction, shared by the matrices of a block; two
+  // for the block sum; the scale product) and sixteen FMAs.  A wave issues in order and a dependent MFMA holds it until its
+  // input is ready, so everything else is slotted between the MFMAs of one group: the unpacking of the NEXT group's weight
+  // codes and the FMAs of the PREVIOUS group (whose MFMA results sit in the other of two register sets).  The matrix pipe
+  // then runs back to back while the vector ALU works in its shadow, within one wave.
+  constexpr int G = 2 * NW * TN;  // groups per K step: block-major, then matrix, then column tile
+  f16x8 fw[2][2];                 // unpacked codes of the current / next group (two MFMA steps each)
+  u32x4 sw[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};  // their scale operands
+  v16f T[2], S[2];                // block sums and scale products of the current / previous group
+  T[1] = zero16;
+  S[1] = zero16;
+
+  const int nsteps = (kbs + ST - 1) / ST * ST;
+  loadA(0, 0);
+  loadA(1, 1);
+#pragma unroll
+  for (int s = 0; s < ST; s++) loadW(s, s);
+  storeA(0, 0);
+  // the first group's operands
+  fw[0][0] = qx_codes<WT>(rq[0][0][0], 0, kc);
+  fw[0][1] = qx_codes<WT>(rq[0][0][0], 1, kc);
+  sw[0].x = rs[0][0][0] & msk0;
+  __syncthreads();
+
+  // one K step (64 elements = two blocks) with its weights in ring slot SLOT; refills the slot with step kt + ST
+  auto kstep = [&](auto slot_tag, int kt) {
+    constexpr int SLOT = decltype(slot_tag)::value;
+    constexpr int NSLOT = (SLOT + 1) % ST;
+    const int buf = kt & 1;
+    loadA(SLOT & 1, kt + 2);  // the set whose step (kt) is in LDS already
+    f16x8 fb[2][2];
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+#pragma unroll
+      for (int d = 0; d < 2; d++)
+        fb[b][d] = *reinterpret_cast<const f16x8*>(smem + buf * STAGE + lrow * LDK + (2 * b + d) * 32 + hi * 16);
+    // the row's scale pair (both scales: the weight operand is zero in the other block's K slot) and its two code-sum pairs,
+    // each already an operand
+    f16x8 rec[3];
+#pragma unroll
+    for (int q = 0; q < 3; q++) rec[q] = *reinterpret_cast<const f16x8*>(smem + buf * STAGE + BM * LDK + lrow * 48 + q * 16);
+    v16f tc = zero16;
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+      constexpr int cur = 0;  // the register sets alternate by the parity of g (G is even)
+      const int c = (g + cur) & 1, n = c ^ 1;
+      const int b = g / (NW * TN), w = (g / TN) % NW, j = g % TN;
+      // the next group: (b', w', j') in this step, or the first group of the next step (ring slot NSLOT)
+      const bool last = g == G - 1;
+      const int gn = last ? 0 : g + 1;
+      const int bn = gn / (NW * TN), wn = (gn / TN) % NW, jn = gn % TN;
+      __builtin_amdgcn_sched_barrier(0);
+      if (w == 0 && j == 0) {  // the block's correction, shared by all its groups
+        tc = __builtin_amdgcn_mfma_f32_32x32x16_f16(off_op, rec[1 + b], zero16, 0, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (last) fw[n][0] = qx_codes<WT>(rq[NSLOT][wn][jn], 2 * bn, kc);
+      else fw[n][0] = qx_codes<WT>(rq[SLOT][wn][jn], 2 * bn, kc);
+      __builtin_amdgcn_sched_barrier(0);
+      T[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[c][0], fb[b][0], tc, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (last) {
+        fw[n][1] = qx_codes<WT>(rq[NSLOT][wn][jn], 2 * bn + 1, kc);
+        sw[n].x = rs[NSLOT][wn][jn] & msk0;
+      } else {
+        fw[n][1] = qx_codes<WT>(rq[SLOT][wn][jn], 2 * bn + 1, kc);
+        sw[n].x = rs[SLOT][wn][jn] & (bn ? msk1 : msk0);
+        if (bn == 1) {  // both blocks of (wn, jn) are unpacked: its ring registers are free, fetch K step kt + ST into them
+#pragma unroll
+          for (int p = 0; p < QW; p++)
+            rq[SLOT][wn][jn][p] = __builtin_amdgcn_raw_buffer_load_b128(rW[wn], kt + ST < kbs ? offQ[jn] : 0xffffffffu, ((kt + ST) * QW + p) * 1024, 0);
+          rs[SLOT][wn][jn] = __builtin_amdgcn_raw_buffer_load_b32(rW[wn], kt + ST < kbs ? offS[jn] : 0xffffffffu, (kt + ST) * 128, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      S[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, sw[c]), rec[0], zero16, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // the FMAs of the previous group (of the previous step's last group when g == 0): first half
+      const int pg = g == 0 ? G - 1 : g - 1;
+      const int pw = (pg / TN) % NW, pj = pg % TN;
+#pragma unroll
+      for (int r = 0; r < 8; r++) acc[pw][pj][0][r] = fmaf(S[n][r], T[n][r], acc[pw][pj][0][r]);
+      asm volatile("" : "+v"(acc[pw][pj][0]));  // pins the FMAs here (the compiler otherwise sinks them to the end of the body)
+      __builtin_amdgcn_sched_barrier(0);
+      T[c] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fw[c][1], fb[b][1], T[c], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 8; r < 16; r++) acc[pw][pj][0][r] = fmaf(S[n][r], T[n][r], acc[pw][pj][0][r]);
+      asm volatile("" : "+v"(acc[pw][pj][0]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    storeA((SLOT & 1) ^ 1, buf ^ 1);
+    __syncthreads();
+  };
+  for (int kt = 0; kt < nsteps; kt += ST) {
+    kstep(std::integral_constant<int, 0>{}, kt);
+    kstep(std::integral_constant<int, 1>{}, kt + 1);
+    kstep(std::integral_constant<int, 2>{}, kt + 2);
+    kstep(std::integral_constant<int, 3>{}, kt + 3);
+  }
+  // the last group's FMAs (G even: its results are in set 1)
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[NW - 1][TN - 1][0][r] = fmaf(S[1][r], T[1][r], acc[NW - 1][TN - 1][0][r]);
+
+  // acc[w][j][i][4g+e] = result[row0 + 32i + lrow][n0 + wave*WN + 32j + 8g + 4hi + e]
+  if (NW == 1) {
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int r = i * 32 + lrow;
+      if (r < rows) {
+        const int pos = row0 + r;
+        float* orow = a.out + (int64_t)(a.o_index ? a.o_index[pos] : pos) * a.N;
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            const int n = n0 + wave * WN + j * 32 + 8 * g + 4 * hi;
+            f32x4 v = {acc[0][j][i][4 * g], acc[0][j][i][4 * g + 1], acc[0][j][i][4 * g + 2], acc[0][j][i][4 * g + 3]};
+            if (n + 3 < a.N && a.N % 4 == 0) {
+              if (a.bias) v += *reinterpret_cast<const f32x4*>(a.bias + n);
+              *reinterpret_cast<f32x4*>(orow + n) = v;
+            } else {
+#pragma unroll
+              for (int e2 = 0; e2 < 4; e2++)
+                if (n + e2 < a.N) orow[n + e2] = a.bias ? v[e2] + a.bias[n + e2] : v[e2];
+            }
+          }
+      }
+    }
+  } else {
+    // h = silu(gate) * up, quantized to Q8_0 over each block of 32 channels (a block is one column tile j: 16 channels in
+    // this lane, 16 in lane ^ 32): codes as fp16 integers and the fp16 scale, the next Linear's activation format
+    const int nblk = a.N / QK, KDo = (a.N + 63) / 64;
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+      const int r = i * 32 + lrow;
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        float h[16];
+        float amax = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+          h[q] = silu_f(acc[0][j][i][q]) * acc[NW - 1][j][i][q];
+          amax = fmaxf(amax, fabsf(h[q]));
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        const float d = amax / 127.f;
+        const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
+        uint16_t bits = f32_to_f16bits(d);
+        if (a.x86_scale) bits = x86_scale_bits(bits);
+        const int blk = (n0 + wave * WN) / 32 + j;
+        // element 8g + 4hi + e of the block: bit 1 of its index is bit 1 of e
+        int qv[16], sa = 0, sb = 0;
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+          qv[q] = min(127, max(-128, (int)rintf(h[q] * idv)));
+          if (q & 2) sb += qv[q];
+          else sa += qv[q];
+        }
+        sa += __shfl_xor(sa, 32, 64);
+        sb += __shfl_xor(sb, 32, 64);
+        if (r < rows && blk < nblk) {
+          uint16_t* hrow = a.hq + (int64_t)(row0 + r) * a.N;
+#pragma unroll
+          for (int g = 0; g < 4; g++) {
+            const int n = n0 + wave * WN + j * 32 + 8 * g + 4 * hi;
+            uint32_t o[2];
+#pragma unroll
+            for (int e2 = 0; e2 < 2; e2++)
+              o[e2] = (uint32_t)f32_to_f16bits((float)qv[4 * g + 2 * e2]) | ((uint32_t)f32_to_f16bits((float)qv[4 * g + 2 * e2 + 1]) << 16);
+            *reinterpret_cast<uint2*>(hrow + n) = uint2{o[0], o[1]};
+          }
+          if (hi == 0) {
+            uint32_t* recp = a.hd + ((int64_t)(row0 + r) * KDo + (blk >> 1)) * 3;
+            reinterpret_cast<uint16_t*>(recp)[blk & 1] = bits;
+            recp[1 + (blk & 1)] = (uint32_t)f32_to_f16bits((float)sa) | ((uint32_t)f32_to_f16bits((float)sb) << 16);
+            if (blk == nblk - 1 && (nblk & 1)) {  // the unused half of the last record
+              reinterpret_cast<uint16_t*>(recp)[1] = 0;
+              recp[2] = 0;
+            }
+          }
+        }
+      }
+    }
+  }
+}
+
+constexpr int QX_TILE_H = 32;
+constexpr int QX_DOWN_TN = 2;  // column tiles per wave in the one-matrix mode
+// MODE 0: one matrix, up to 32 rows x 256 channels per workgroup.  MODE 1: gate and up together, 32 rows x 128 channels.
+template <int WT, int MODE>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qx_kernel(QXArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int t = blockIdx.x;
+  if (t >= min(a.ntiles[0], (int)gridDim.x)) return;
+  const int e = a.tile_expert[t], row0 = a.tile_row0[t], rows = a.tile_rows[t];
+  if constexpr (MODE == 1) {
+    const int n0 = blockIdx.y * 128;
+    qx_tile<WT, 2, 1, 1>(a, e, row0, rows, n0, smem);
+  } else {
+    const int n0 = blockIdx.y * (128 * QX_DOWN_TN);
+    qx_tile<WT, 1, 1, QX_DOWN_TN>(a, e, row0, rows, n0, smem);
+  }
+}
+
+
+
+template <int MODE>
+static int launch_qx(int wtype, const QXArgs& a, unsigned max_tiles, hipStream_t st) {
+  const int wg_n = MODE == 1 ? 128 : 128 * QX_DOWN_TN;
+  const dim3 grid(max_tiles, (unsigned)((a.N + wg_n - 1) / wg_n));
+  const size_t lds = 2 * (size_t)(QX_TILE_H * (2 * 64 + 16) + QX_TILE_H * 48);
+  if (wtype == MLLM_HIP_Q4_0) hipLaunchKernelGGL((qx_kernel<MLLM_HIP_Q4_0, MODE>), grid, dim3(256), lds, st, a);
+  else hipLaunchKernelGGL((qx_kernel<MLLM_HIP_Q8_0, MODE>), grid, dim3(256), lds, st, a);
+  return (int)hipGetLastError();
+}
+
+// activations for the kernel above: Q8_0 quantization (bit-exact codes and scale); codes as fp16 integers, and per row and K
+// step of 64 a record of three dwords: the two blocks' fp16 scales, then per block the code sums over the elements with
+// bit 1 of k clear | set, as fp16 integers (at most 16 x 127 each: exact).  The second half of a last, incomplete record is zero.
+__global__ void qx_act_kernel(const void* __restrict__ x, int x_dtype, uint16_t* __restrict__ xq, uint32_t* __restrict__ xd,
+                              int64_t nblocks, int nb, int x86_scale) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= nblocks) return;
+  float v[32];
+  uint32_t q[8];
+  int sum;
+  load_block_f32(x, x_dtype, i * QK, v);
+  uint16_t bits = quantize_block_q8_0(v, q, sum);
+  if (x86_scale) bits = x86_scale_bits(bits);
+  uint32_t o[16];
+  int sa = 0, sb = 0;
+#pragma unroll
+  for (int j = 0; j < 16; j++) {  // elements 2j, 2j+1
+    const int c0 = (int8_t)(q[j / 2] >> (16 * (j & 1))), c1 = (int8_t)(q[j / 2] >> (16 * (j & 1) + 8));
+    o[j] = (uint32_t)f32_to_f16bits((float)c0) | ((uint32_t)f32_to_f16bits((float)c1) << 16);
+    if (j & 1) sb += c0 + c1;
+    else sa += c0 + c1;
+  }
+  u32x4* out = reinterpret_cast<u32x4*>(xq + i * QK);
+#pragma unroll
+  for (int j = 0; j < 4; j++) out[j] = u32x4{o[4 * j], o[4 * j + 1], o[4 * j + 2], o[4 * j + 3]};
+  const int64_t row = i / nb;
+  const int b = (int)(i - row * nb), KD = (nb + 1) / 2;
+  uint32_t* rec = xd + (row * KD + (b >> 1)) * 3;
+  reinterpret_cast<uint16_t*>(rec)[b & 1] = bits;
+  rec[1 + (b & 1)] = (uint32_t)f32_to_f16bits((float)sa) | ((uint32_t)f32_to_f16bits((float)sb) << 16);
+  if (b == nb - 1 && (nb & 1)) {
+    reinterpret_cast<uint16_t*>(rec)[1] = 0;
+    rec[2] = 0;
+  }
+}
+
+// y[t][h] = sum_j per[t*k + j][h] * w[t][j]   (multiply, then add in j order: modeling_qwen3_moe_fa2.hpp:233-236)
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ per, const float* __restrict__ w, const int32_t* __restrict__ ids,
+                                                          float* __restrict__ y, int64_t T, int H, int k, int E) {
+  // four consecutive channels per thread (H % 4 == 0: H is a multiple of the block size), all k rows requested before the
+  // first is used; the sum itself runs in slot order
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
   if (i >= T * H) return;
   const int64_t t = i / H;
-  const int h = (int)(i % H);
-  float acc = 0.f;
-  for (int j = 0; j < k; j++) {
-    const int e = ids[t * k + j];
-    if (e >= 0 && e < E) acc = acc + per[(t * k + j) * H + h] * w[t * k + j];
+  const int h = (int)(i - t * H);
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int j0 = 0; j0 < k; j0 += 8) {
+    // every load is unconditional (slots past k repeat the last one; the row of a slot without expert was never written
+    // but is readable memory): nothing waits on a branch, and what must not count is dropped by a select
+    int e[8];
+    float wj[8];
+    f32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const int64_t s = t * k + min(j0 + u, k - 1);
+      e[u] = ids[s];
+      wj[u] = w[s];
+      v[u] = *reinterpret_cast<const f32x4*>(per + s * H + h);
+    }
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+      const f32x4 nx = acc + v[u] * wj[u];
+      const bool ok = j0 + u < k && e[u] >= 0 && e[u] < E;
+      acc.x = ok ? nx.x : acc.x;
+      acc.y = ok ? nx.y : acc.y;
+      acc.z = ok ? nx.z : acc.z;
+      acc.w = ok ? nx.w : acc.w;
+    }
   }
-  y[i] = acc;
+  *reinterpret_cast<f32x4*>(y + i) = acc;
 }
 
 // ---- workspace carving ---------------------------------------------------------------------------------------
@@ -1120,7 +1583,7 @@ MLLM_API int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* 
   if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
   if (H <= 0 || I <= 0 || H % QK || I % QK || E > MOE_MAX_EXPERTS) return MLLM_HIP_E_SHAPE;
   if (T * H >= ((int64_t)1 << 32) || T * k * I >= ((int64_t)1 << 32) || T * k > INT32_MAX) return MLLM_HIP_E_SHAPE;
-  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16 || reinterpret_cast<uintptr_t>(y) % 16) return MLLM_HIP_E_ALIGN;
   hipStream_t st = (hipStream_t)stream;
   const int x86 = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
   // few pairs per expert: every (token, expert) pair is one GEMV row; two launches instead of five
@@ -1136,7 +1599,7 @@ MLLM_API int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* 
                             rc.ro.ntiles, rc.ro.sorted_idx, rc.img, rc.per, T, H, I, E, k, x86, max_tiles, st);
     if (r) return r;
     const int64_t total = T * H;
-    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, rc.per, topk_w, topk_ids, y, T,
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st, rc.per, topk_w, topk_ids, y, T,
                        (int)H, k, E);
     return (int)hipGetLastError();
   }
@@ -1174,7 +1637,7 @@ MLLM_API int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* 
   rc = launch_tiles<0>(wtype, a, max_tiles, st);
   if (rc) return rc;
   const int64_t total = T * H;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
                      (int)H, k, E);
   return (int)hipGetLastError();
 }
@@ -1261,6 +1724,69 @@ MLLM_API int mllm_hip_linear_q_gemm_short(int wtype, const void* gemm_packed, co
   return qg_linear_run(wtype, gemm_packed, xh, bias, y, M, N, K, route, partial, st);
 }
 
+namespace mllmhip {
+struct QXCarve {
+  uint16_t* xq;
+  uint32_t* xd;
+  uint16_t* hq;
+  uint32_t* hd;
+  float* per;
+  RouteOut ro;
+};
+static QXCarve carve_qx(Carver& c, int64_t T, int64_t H, int64_t I, int E, int k) {
+  QXCarve r;
+  r.xq = c.take<uint16_t>((size_t)T * H);
+  r.xd = c.take<uint32_t>((size_t)T * 3 * ((H + 63) / 64));
+  r.hq = c.take<uint16_t>((size_t)T * k * I);
+  r.hd = c.take<uint32_t>((size_t)T * k * 3 * ((I + 63) / 64));
+  r.per = c.take<float>((size_t)T * k * H);
+  r.ro = carve_route(c, E, T * k, QX_TILE_H);
+  return r;
+}
+static int g_moe_gemm_path = 0;  // 0: exact block sums (qx_kernel); 1: fp16 operands with the block scales folded in (qg_kernel)
+}  // namespace mllmhip
+
+MLLM_API int mllm_hip_moe_gemm_set_path(int path) {
+  if (path != 0 && path != 1) return MLLM_HIP_E_BADARG;
+  g_moe_gemm_path = path;
+  return 0;
+}
+
+// The grouped expert FFN with the reference's own block arithmetic on the matrix cores (qx_kernel): route, quantize x,
+// gate + up + SiLU * up + re-quantization in one launch, down, weighted sum in slot order.
+static int moe_ffn_qx(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x, int x_dtype,
+                      const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H, int64_t I, int E, int k, int x86,
+                      void* workspace, hipStream_t st) {
+  Carver c(workspace);
+  QXCarve w = carve_qx(c, T, H, I, E, k);
+  const unsigned max_tiles = (unsigned)(E + (T * k) / QX_TILE_H + 1);
+  RC_RET(launch_route(topk_ids, T * k, E, QX_TILE_H, w.ro, st));
+  const int64_t nblocks = T * (H / QK);
+  hipLaunchKernelGGL(qx_act_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, w.xq, w.xd, nblocks,
+                     (int)(H / QK), x86);
+  HIP_RET(hipGetLastError());
+  QXArgs a{};
+  a.tile_expert = w.ro.tile_expert; a.tile_row0 = w.ro.tile_row0; a.tile_rows = w.ro.tile_rows; a.ntiles = w.ro.ntiles;
+  a.x86_scale = x86;
+  a.W0 = reinterpret_cast<const char*>(gate_packed);
+  a.W1 = reinterpret_cast<const char*>(up_packed);
+  a.wstride = (size_t)qg_bytes(wtype, I, H);
+  a.xq = w.xq; a.xd = w.xd; a.a_index = w.ro.sorted_idx; a.a_div = k; a.a_rows = (int)T;
+  a.hq = w.hq; a.hd = w.hd;
+  a.N = (int)I; a.K = (int)H;
+  RC_RET(launch_qx<1>(wtype, a, max_tiles, st));
+  a.W0 = a.W1 = reinterpret_cast<const char*>(down_packed);
+  a.wstride = (size_t)qg_bytes(wtype, H, I);
+  a.xq = w.hq; a.xd = w.hd; a.a_index = nullptr; a.a_div = 1; a.a_rows = (int)(T * k);
+  a.o_index = w.ro.sorted_idx; a.out = w.per; a.bias = nullptr; a.hq = nullptr; a.hd = nullptr;
+  a.N = (int)H; a.K = (int)I;
+  RC_RET(launch_qx<0>(wtype, a, max_tiles, st));
+  const int64_t total = T * H;
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st, w.per, topk_w, topk_ids, y, T,
+                     (int)H, k, E);
+  return (int)hipGetLastError();
+}
+
 MLLM_API size_t mllm_hip_moe_gemm_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k) {
   if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || k <= 0 || H % QK || I % QK) return 0;
   Carver c(nullptr);
@@ -1269,7 +1795,10 @@ MLLM_API size_t mllm_hip_moe_gemm_workspace_bytes(int64_t T, int64_t H, int64_t 
   c.take<uint16_t>((size_t)T * k * I);
   c.take<float>((size_t)T * k * H);
   carve_route(c, E, T * k);
-  return c.used;
+  // the exact form: codes as fp16 integers + scale pairs for x and for h, the per-pair rows, routing
+  Carver cx(nullptr);
+  carve_qx(cx, T, H, I, E, k);
+  return c.used > cx.used ? c.used : cx.used;
 }
 
 MLLM_API int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed,
@@ -1283,9 +1812,11 @@ MLLM_API int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const v
   if (act_scale_mode != MLLM_HIP_SCALE_IEEE && act_scale_mode != MLLM_HIP_SCALE_X86_REF) return MLLM_HIP_E_BADARG;
   if (H <= 0 || I <= 0 || H % QK || I % QK || E > MOE_MAX_EXPERTS) return MLLM_HIP_E_SHAPE;
   if (T * H * 2 >= ((int64_t)1 << 32) || T * k * I * 2 >= ((int64_t)1 << 32) || T * k > INT32_MAX) return MLLM_HIP_E_SHAPE;
-  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
+  if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16 || reinterpret_cast<uintptr_t>(y) % 16) return MLLM_HIP_E_ALIGN;
   hipStream_t st = (hipStream_t)stream;
   const int x86 = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
+  if (g_moe_gemm_path == 0)
+    return moe_ffn_qx(wtype, gate_packed, up_packed, down_packed, x, x_dtype, topk_ids, topk_w, y, T, H, I, E, k, x86, workspace, st);
   Carver c(workspace);
   uint16_t* xh = c.take<uint16_t>((size_t)T * H);
   uint16_t* xl = c.take<uint16_t>((size_t)T * H);
@@ -1319,7 +1850,7 @@ MLLM_API int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const v
   rc = launch_qg<0>(a, max_tiles, st);
   if (rc) return rc;
   const int64_t total = T * H;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
                      (int)H, k, E);
   return (int)hipGetLastError();
 }
@@ -1353,7 +1884,7 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
   if (H <= 0 || I <= 0 || H % 256 || I % 256 || T * k > 65535) return MLLM_HIP_E_SHAPE;
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16 ||
       reinterpret_cast<uintptr_t>(gate_packed) % 16 || reinterpret_cast<uintptr_t>(up_packed) % 16 ||
-      reinterpret_cast<uintptr_t>(down_packed) % 16)
+      reinterpret_cast<uintptr_t>(down_packed) % 16 || reinterpret_cast<uintptr_t>(y) % 16)
     return MLLM_HIP_E_ALIGN;
   hipStream_t st = (hipStream_t)stream;
   const int slots = (int)(T * k);
@@ -1380,7 +1911,7 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
   }
   if (rc) return rc;
   const int64_t total = T * H;
-  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
+  hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
                      (int)H, k, E);
   return (int)hipGetLastError();
 }

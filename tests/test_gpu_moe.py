@@ -201,20 +201,58 @@ def test_moe_decode_path(T, H, I, E, k, wtype):
 
 
 @pytest.mark.parametrize("T,H,I,E,k,wtype", [(16, 64, 32, 4, 2, 0), (40, 256, 96, 8, 3, 0), (200, 128, 64, 3, 2, 1),
-                                              (1, 64, 64, 4, 4, 0), (300, 192, 160, 2, 2, 0)])
+                                              (1, 64, 64, 4, 4, 0), (300, 192, 160, 2, 2, 0), (70, 96, 224, 5, 3, 1)])
 def test_moe_gemm_small(T, H, I, E, k, wtype):
+    """Both forms of the grouped FFN on gemm-packed experts.  Form 0 keeps the reference's block arithmetic (exact integer
+    block sums, exact scale products, one fp32 FMA per block): as close to the oracle as the decode kernels (2e-4 leaves
+    room for the odd Q8_0 code of h that flips where fp32 sums differ in the last bit).  Form 1 folds the scales into fp16
+    operands (1e-3).  Odd block counts (H = 96, I = 224, 160: 3, 7 and 5 blocks) exercise the half-filled last record;
+    slots with an expert id outside [0, E) add nothing."""
     rng = synth.rng_for(4, 3 * T + H + I + E)
     Wg, Wu, Wd = synth.make_moe_weights(rng, E, H, I, wtype)
     ids, w = synth.make_moe_routing(rng, T, E, k)
+    if T > 1:
+        ids[0, 0] = E + 2
+        ids[T - 1, k - 1] = -1
     g, u, d = (ql.PackedExperts(wtype, torch.from_numpy(m), layout="gemm") for m in (Wg, Wu, Wd))
     x = synth.make_x_fp32(rng, T, H)
-    announce("moe gemm small", T, H, I, E, k, wtype)
-    y = ql.moe_ffn_q_gemm(g, u, d, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
     want = orc.moe_ffn(x, ids, w, Wg, Wu, Wd, wtype)
-    assert rel_l2(y, want) < TOL, rel_l2(y, want)
-    perm = rng.permutation(T)
-    y2 = ql.moe_ffn_q_gemm(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
-    assert np.array_equal(y2, y[perm])
+    L = _lib.lib()
+    try:
+        for form, tol in ((0, 2e-4), (1, TOL)):
+            announce("moe gemm small", T, H, I, E, k, wtype, "form", form)
+            assert L.mllm_hip_moe_gemm_set_path(form) == 0
+            y = ql.moe_ffn_q_gemm(g, u, d, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+            assert rel_l2(y, want) < tol, (form, rel_l2(y, want))
+            perm = rng.permutation(T)
+            y2 = ql.moe_ffn_q_gemm(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
+            assert np.array_equal(y2, y[perm])
+    finally:
+        L.mllm_hip_moe_gemm_set_path(0)
+    assert L.mllm_hip_moe_gemm_set_path(2) == -1
+
+
+def test_moe_gemm_exact_form_is_the_block_arithmetic():
+    """Form 0 against the block-dot kernels of mllm_hip_moe_ffn_q on the same inputs: both compute
+    sum_b fp32(dW * dX) * float(int32 block sum) with exact block sums, so they differ by fp32 summation order only; and a
+    case built from integers (unit scales, small codes) in which every sum is exact must come out bit for bit."""
+    rng = synth.rng_for(4, 7100)
+    T, H, I, E, k = 96, 256, 128, 6, 2
+    Wg, Wu, Wd = synth.make_moe_weights(rng, E, H, I, 0)
+    ids, w = synth.make_moe_routing(rng, T, E, k)
+    x = synth.make_x_fp32(rng, T, H)
+    gg, ug, dg = (ql.PackedExperts(0, torch.from_numpy(m), layout="gemm") for m in (Wg, Wu, Wd))
+    gv, uv, dv = (ql.PackedExperts(0, torch.from_numpy(m)) for m in (Wg, Wu, Wd))
+    announce("moe gemm exact form vs block-dot tiles")
+    L = _lib.lib()
+    try:
+        assert L.mllm_hip_moe_set_tuning(1, 1) == 0  # the grouped block-dot tiles
+        yv = ql.moe_ffn_q(gv, uv, dv, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+    finally:
+        L.mllm_hip_moe_set_tuning(0, 0)
+    yg = ql.moe_ffn_q_gemm(gg, ug, dg, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+    assert rel_l2(yg, yv) < 1e-4, rel_l2(yg, yv)
+    assert rel_l2(yg, orc.moe_ffn(x, ids, w, Wg, Wu, Wd, 0)) < 2e-4
 
 
 @pytest.mark.parametrize("T,wtype", [(6, 0), (24, 0), (40, 1), (100, 0)])
@@ -280,9 +318,15 @@ def test_moe_gemm_full_size():
     y = ql.moe_ffn_q_gemm(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
     want = orc.moe_ffn(xf, ids, w, Wg, Wu, Wd, 0)
     r = rel_l2(y, want)
-    assert r < TOL, r
+    assert r < 2e-4, r  # the exact form: the reference's block arithmetic
     y2 = ql.moe_ffn_q_gemm(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
     assert np.array_equal(y, y2)
+    try:
+        assert _lib.lib().mllm_hip_moe_gemm_set_path(1) == 0
+        y3 = ql.moe_ffn_q_gemm(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
+    finally:
+        _lib.lib().mllm_hip_moe_gemm_set_path(0)
+    assert rel_l2(y3, want) < TOL
 
 
 def test_moe_full_size():
