@@ -35,8 +35,8 @@ struct RouteOut {
   int* ntiles;       // [1]
 };
 
-__global__ __launch_bounds__(1024) void moe_route_kernel(const int32_t* __restrict__ ids, int n, int E, int tile_h, RouteOut o) {
-  extern __shared__ int s_cnt[];  // [E] counts, [E] cursors, [E] scan scratch x 3
+__device__ __forceinline__ void moe_route_body(const int32_t* __restrict__ ids, int n, int E, int tile_h, const RouteOut& o, int* s_cnt) {
+  // s_cnt: [E] counts, [E] cursors, [E] scan scratch x 3
   int* s_cur = s_cnt + E;
   int* s_off = s_cur + E;   // exclusive scan of the counts
   int* s_full = s_off + E;  // exclusive scan of the full-tile counts
@@ -100,6 +100,11 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const int32_t* __restri
     const int e = ids[i];
     if (e >= 0 && e < E) o.sorted_idx[atomicAdd(&s_cur[e], 1)] = i;
   }
+}
+
+__global__ __launch_bounds__(1024) void moe_route_kernel(const int32_t* __restrict__ ids, int n, int E, int tile_h, RouteOut o) {
+  extern __shared__ int s_route[];
+  moe_route_body(ids, n, E, tile_h, o, s_route);
 }
 
 // identity routing for a plain Linear over M rows
@@ -1298,10 +1303,8 @@ static int launch_qx(int wtype, const QXArgs& a, unsigned max_tiles, hipStream_t
 // activations for the kernel above: Q8_0 quantization (bit-exact codes and scale); codes as fp16 integers, and per row and K
 // step of 64 a record of three dwords: the two blocks' fp16 scales, then per block the code sums over the elements with
 // bit 1 of k clear | set, as fp16 integers (at most 16 x 127 each: exact).  The second half of a last, incomplete record is zero.
-__global__ void qx_act_kernel(const void* __restrict__ x, int x_dtype, uint16_t* __restrict__ xq, uint32_t* __restrict__ xd,
-                              int64_t nblocks, int nb, int x86_scale) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= nblocks) return;
+__device__ __forceinline__ void qx_act_block(const void* __restrict__ x, int x_dtype, uint16_t* __restrict__ xq, uint32_t* __restrict__ xd,
+                                             int64_t i, int nb, int x86_scale) {
   float v[32];
   uint32_t q[8];
   int sum;
@@ -1329,6 +1332,19 @@ __global__ void qx_act_kernel(const void* __restrict__ x, int x_dtype, uint16_t*
     reinterpret_cast<uint16_t*>(rec)[1] = 0;
     rec[2] = 0;
   }
+}
+
+// the two independent preparations of the grouped FFN in one launch: workgroup 0 routes, the others quantize x
+__global__ __launch_bounds__(1024) void qx_prepare_kernel(const int32_t* __restrict__ ids, int n, int E, int tile_h, RouteOut o,
+                                                          const void* __restrict__ x, int x_dtype, uint16_t* __restrict__ xq,
+                                                          uint32_t* __restrict__ xd, int64_t nblocks, int nb, int x86_scale) {
+  extern __shared__ int s_route[];
+  if (blockIdx.x == 0) {
+    moe_route_body(ids, n, E, tile_h, o, s_route);
+    return;
+  }
+  const int64_t i = (int64_t)(blockIdx.x - 1) * 1024 + threadIdx.x;
+  if (i < nblocks) qx_act_block(x, x_dtype, xq, xd, i, nb, x86_scale);
 }
 
 // y[t][h] = sum_j per[t*k + j][h] * w[t][j]   (multiply, then add in j order: modeling_qwen3_moe_fa2.hpp:233-236)
@@ -1760,10 +1776,10 @@ static int moe_ffn_qx(int wtype, const void* gate_packed, const void* up_packed,
   Carver c(workspace);
   QXCarve w = carve_qx(c, T, H, I, E, k);
   const unsigned max_tiles = (unsigned)(E + (T * k) / QX_TILE_H + 1);
-  RC_RET(launch_route(topk_ids, T * k, E, QX_TILE_H, w.ro, st));
+  if (E > MOE_MAX_EXPERTS) return MLLM_HIP_E_SHAPE;
   const int64_t nblocks = T * (H / QK);
-  hipLaunchKernelGGL(qx_act_kernel, dim3((unsigned)((nblocks + 127) / 128)), dim3(128), 0, st, x, x_dtype, w.xq, w.xd, nblocks,
-                     (int)(H / QK), x86);
+  hipLaunchKernelGGL(qx_prepare_kernel, dim3((unsigned)(1 + (nblocks + 1023) / 1024)), dim3(1024), 5 * (size_t)E * sizeof(int), st,
+                     topk_ids, (int)(T * k), E, QX_TILE_H, w.ro, x, x_dtype, w.xq, w.xd, nblocks, (int)(H / QK), x86);
   HIP_RET(hipGetLastError());
   QXArgs a{};
   a.tile_expert = w.ro.tile_expert; a.tile_row0 = w.ro.tile_row0; a.tile_rows = w.ro.tile_rows; a.ntiles = w.ro.ntiles;
