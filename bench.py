@@ -23,6 +23,22 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 N_LAYERS = 36
+# counter summary of the dominant launch (two rocprofv3 --pmc runs of `bench.py --pmc-probe`); its "total" line is what
+# roofline.traffic reports, so the figure and its evidence cannot drift apart
+TRAFFIC_PROFILE = "profiles/gemv_q4_0_gate_up_m1_pmc_hbm_traffic.txt"
+
+
+def traffic_from_profile():
+    """bytes per launch from the committed counter summary (line `total  <bytes> B  vs algorithmic ...`), or None"""
+    import re
+    try:
+        for line in open(os.path.join(ROOT, TRAFFIC_PROFILE)):
+            m = re.match(r"\s*total\s+([0-9 ]+) B\s+vs algorithmic", line)
+            if m:
+                return int(m.group(1).replace(" ", ""))
+    except OSError:
+        pass
+    return None
 
 
 def parse():
@@ -194,13 +210,22 @@ def side_workloads(torch, ql, synth, gen):
     down2 = ql.PackedExperts.synthetic(ql.Q4_0, E, H, I, gen, layout="gemm")
     wsm2 = torch.empty(L.mllm_hip_moe_gemm_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
     tm2 = ev_time(lambda: ql.moe_ffn_q_gemm(gate2, up2, down2, x, ids, tw, workspace=wsm2, out=ym), 10)
+    L.mllm_hip_moe_gemm_set_path(1)
+    tm3 = ev_time(lambda: ql.moe_ffn_q_gemm(gate2, up2, down2, x, ids, tw, workspace=wsm2, out=ym), 10)
+    L.mllm_hip_moe_gemm_set_path(0)
     active = int((np.bincount(ids_np.reshape(-1), minlength=E) > 0).sum())
     wbytes = active * (2 * I * (H // 32) * 18 + H * (I // 32) * 18)
     flops = T * k * (2.0 * H * I * 2 + 2.0 * I * H)
     out["moe_ffn_512tok_128e_top8_q4_0"] = {"us": tm2 * 1e6, "active_experts": active, "weight_GBps": wbytes / tm2 / 1e9,
                                             "frac_of_hbm_peak": wbytes / tm2 / 8e12, "TFLOPS": flops / tm2 / 1e12,
-                                            "path": "matrix cores, fp16 operands with folded block scales (mllm_hip_moe_ffn_q_gemm)",
-                                            "block_dot_path": {"us": tm * 1e6, "weight_GBps": wbytes / tm / 1e9},
+                                            "path": "mllm_hip_moe_ffn_q_gemm, default form: the reference's block arithmetic on the matrix "
+                                                    "cores (exact integer block sums and exact scale products from fp16 MFMAs, one fp32 FMA "
+                                                    "per block; 4 launches: route + quantize, gate + up + SiLU*up + re-quantize, down, weighted sum)",
+                                            "fp16_operand_form": {"us": tm3 * 1e6, "weight_GBps": wbytes / tm3 / 1e9,
+                                                                  "note": "mllm_hip_moe_gemm_set_path(1): block scales folded into fp16 "
+                                                                          "operands, no exact block sums (about 2e-4 from the oracle)"},
+                                            "block_dot_path": {"us": tm * 1e6, "weight_GBps": wbytes / tm / 1e9,
+                                                               "note": "mllm_hip_moe_ffn_q: int8 MFMA block sums scaled on the vector ALU"},
                                             "decode": dec, "decode_q4_k_experts": deck}
     del gate2, up2, down2
     # Q4_0 Linear at prefill size (the reference's tinyBLAS gemm branch): gate_proj of the decode layer, 2048 rows
@@ -465,6 +490,15 @@ def main():
                  for name in ("gate_up", "qkv", "gate_proj", "down_proj", "q_proj", "o_proj", "k_proj")}
     dom_name = "gate_proj" if args.per_op else "gate_up"
     dom = per_shape[dom_name]
+    # BASELINE configs[0]: the single Q4_0 Linear [1,2048] x [6144,2048]^T with fp32 activations, over 80 distinct copies of the
+    # weight (566 MB: every launch streams from HBM), one launch each
+    c1w = [ql.PackedQWeight.synthetic(ql.Q4_0, 6144, 2048, gen) for _ in range(80)]
+    c1x = torch.randn((1, 2048), device="cuda", generator=gen)
+    c1y = torch.empty((1, 6144), dtype=torch.float32, device="cuda")
+    _, ev = timed(graphed(lambda: [ql.linear_q_gemv(w, c1x, None, ql.SCALE_X86_REF, out=c1y) for w in c1w]), 5, 2)
+    c1b = synth.gemv_algorithmic_bytes(ql.Q4_0, 1, 6144, 2048, 4)
+    per_shape["c1_6144x2048_fp32_x"] = {"us": ev / (5 * 80) * 1e6, "GBps": c1b / (ev / (5 * 80)) / 1e9, "bytes": c1b, "launches": 400}
+    del c1w
 
     extra = {"per_shape": per_shape, "event_ms_per_step": head["event_ms_per_step"],
              "graph": not args.no_graph, "layers": N_LAYERS, "launches_per_step": N_LAYERS * (len(shapes) if args.per_op else 4)}
@@ -519,7 +553,7 @@ def main():
         # what a stream of launches of this size can reach at all: a read-only 16-byte streaming kernel over distinct buffers
         floor = {}
         big = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device="cuda", generator=gen)
-        for nb_ in (1483776, 5919744, 14052352, 28099584, 56199168):
+        for nb_ in sorted({v["bytes"] for v in per_shape.values()} | {56199168}):
             n = nb_ // 16 * 16
             offs = [(i * 57000000) % ((1 << 30) - n) // 256 * 256 for i in range(40)]
 
@@ -532,6 +566,8 @@ def main():
             floor[str(n)] = {"us": ev / (5 * 40) * 1e6, "GBps": n / (ev / (5 * 40)) / 1e9}
         del big
         extra["read_only_floor"] = floor
+        # every launch shape against the read-only floor of its own byte count (1.0 = as fast as merely reading the bytes)
+        extra["floor_over_launch"] = {name: round(floor[str(v["bytes"] // 16 * 16)]["us"] / v["us"], 3) for name, v in per_shape.items()}
         # the same GEMV kernel on a launch large enough to leave the fixed cost behind: gate + up of a Qwen3-32B-shaped layer
         # (2 x 25600 x 5120, 147 MB of Q4_0 blocks), eight distinct copies
         bigw = [[ql.PackedQWeight.synthetic(ql.Q4_0, 25600, 5120, gen) for _ in range(2)] for _ in range(8)]
@@ -560,20 +596,27 @@ def main():
         Ws = {name: synth.make_weight(rng, otype, n, k) for name, (n, k) in shapes.items()}
         xsf = {k: synth.make_x_bf16(rng, args.m, k)[1] for k in (2560, 4096, 9728)}
         cores = len(os.sched_getaffinity(0))
-        threads = int(os.environ.get("OMP_NUM_THREADS", cores))
-        for name, W in Ws.items():  # warm-up pass
-            orc.linear_q(xsf[W.shape[1] * 32], W, otype)
-        passes, t0 = 0, time.perf_counter()
-        while time.perf_counter() - t0 < 10.0 and passes < 200:
-            for name, W in Ws.items():
-                orc.linear_q(xsf[W.shape[1] * 32], W, otype)
-            passes += 1
-        dt = time.perf_counter() - t0
         layer_bytes = step_bytes(wtype, args.m) / N_LAYERS
-        cpu = {"value": layer_bytes * passes / dt / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-               "sample": "%d passes over ONE decoder layer (7 GEMVs, %.1f MB) with the C oracle "
-                         "(scalar restatement of quantize_row_q8_0 + tinyBLAS block dots, OpenMP over output rows)"
-                         % (passes, layer_bytes / 1e6)}
+
+        def cpu_rate(threads, budget_s):
+            """passes over one decoder layer with the AVX2 tile form of the reference's x86 path (tinyBLAS_Q0_AVX tiles, jobs
+            split over `threads` as the op's threads option does), bit-identical to the scalar oracle"""
+            for W in Ws.values():  # warm-up pass
+                orc.linear_q_tiles(xsf[W.shape[1] * 32], W, otype, None, orc.SCALE_X86_REF, threads)
+            passes, t0 = 0, time.perf_counter()
+            while time.perf_counter() - t0 < budget_s and passes < 400:
+                for W in Ws.values():
+                    orc.linear_q_tiles(xsf[W.shape[1] * 32], W, otype, None, orc.SCALE_X86_REF, threads)
+                passes += 1
+            return layer_bytes * passes / (time.perf_counter() - t0) / 1e9, passes
+        v_all, p_all = cpu_rate(cores, 10.0)
+        v_8, p_8 = cpu_rate(min(8, cores), 8.0)
+        cpu = {"value": v_all, "unit": "GB/s", "cores": cores, "kind": "port",
+               "sample": "%d passes over ONE decoder layer (7 GEMVs, %.1f MB, M=%d) with the oracle's AVX2 tile form of the "
+                         "reference's x86 path (quantize_row_q8_0 + tinyBLAS_Q0_AVX tiles with maddubs/madd block dots, jobs "
+                         "split over the threads as llamafile_sgemm does), %d threads = every core this process may use; "
+                         "bit-identical to the scalar oracle" % (p_all, layer_bytes / 1e6, args.m, cores),
+               "at_reference_default_8_threads": {"value": v_8, "unit": "GB/s", "cores": min(8, cores), "passes": p_8}}
 
     out = {
         "metric": "W4 decode GEMV HBM GB/s" if wtype == ql.Q4_0 else "W8 decode GEMV HBM GB/s",
@@ -591,7 +634,8 @@ def main():
                      "frac": round(dom["GBps"] / HBM_PEAK_GBS, 4),
                      # FETCH_SIZE + WRITE_SIZE per dispatch from two rocprofv3 --pmc runs of `bench.py --pmc-probe`, each scaled
                      # by what the counter reads for the library's plain copy kernel of the same size
-                     "traffic": 28159986 if (wtype == ql.Q4_0 and args.m == 1 and not args.per_op) else None,
+                     "traffic": traffic_from_profile() if (wtype == ql.Q4_0 and args.m == 1 and not args.per_op) else None,
+                     "traffic_source": TRAFFIC_PROFILE if (wtype == ql.Q4_0 and args.m == 1 and not args.per_op) else None,
                      "kernel": ("gemv_q_kernel gate_proj N=9728 K=2560 M=%d" if args.per_op else
                                 "gemv_q_kernel gate+up in one launch, 2 x (N=9728 K=2560), M=%d") % args.m, "us_per_launch": round(dom["us"], 3),
                      "algorithmic_bytes_per_launch": dom["bytes"]},

@@ -147,6 +147,22 @@ def linear_q(x, W, wtype, bias=None, scale_mode=SCALE_X86_REF, return_xq=False):
     return (y, xq, xd) if return_xq else y
 
 
+def linear_q_tiles(x, W, wtype, bias=None, scale_mode=SCALE_X86_REF, threads=8):
+    """The same Linear through the AVX2 tile form of the reference's x86 path (tinyBLAS tiles, jobs split over `threads` as
+    the op's threads option does); bit-identical to linear_q."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    W = np.ascontiguousarray(W, dtype=np.uint8)
+    M, K = x.shape
+    N, nb, bb = W.shape
+    assert nb * 32 == K and bb == BLOCK_BYTES[wtype]
+    y = np.empty((M, N), np.float32)
+    b = None if bias is None else np.ascontiguousarray(bias, dtype=np.float32)
+    rc = lib().orc_linear_q_tiles(_p(x, C.c_float), _p(W, C.c_uint8), C.c_int(wtype), _p(b, C.c_float), _p(y, C.c_float),
+                                  C.c_int(M), C.c_int(N), C.c_int(K), C.c_int(scale_mode), C.c_int(threads), None)
+    assert rc == 0, rc
+    return y
+
+
 # ----------------------------------------------------------------------------- W4A16
 def w4a16_dequant(qw, s_bits, zp, group=128):
     """qw uint8 [N, K/2], s uint16 [N, G], zp uint8 [N, ceil(G/2)] -> bf16 bit patterns [N, K]."""

@@ -301,6 +301,145 @@ ORC_API int orc_linear_q(const float* x, const uint8_t* W, int wtype, const floa
 }
 
 /* ------------------------------------------------------------------------------------------------
+ * The same Linear with the vector instructions and the work split of the reference's x86 path: the form whose
+ * speed stands for "the reference's CPU path" when it is timed next to the GPU.
+ *   tinyBLAS_Q0_AVX<block_q4_0 | block_q8_0, block_q8_0, float>   llamafile/llamafile_sgemm.cpp:579-790
+ *     mnpack (tile shapes of a 16-register build, VECTOR_REGISTERS == 16)      :588-695
+ *     gemm<RM, RN>: jobs = tiles, duty = ceil(tiles / nth), thread ith takes jobs [duty * ith, duty * (ith + 1))   :697-705
+ *       per block l:  Cv[j][i] = fmadd(set1(dW * dX), cvtepi32_ps(madd_epi16(1, maddubs_epi16(|w|, sign(x, w)))), Cv[j][i])
+ *       C[ldc * (jj + j) + ii + i] = bias[ii + i] + hsum(Cv[j][i])                                                 :706-741
+ *     loaders: Q4_0 nibbles -> bytes - 8 (denibble), Q8_0 as stored          :745-778
+ *   called once per thread id under an OpenMP parallel-for over [0, threads)  ggml/matmul.cpp:197-206
+ * Weights and activations are arrays of blocks as in the reference (the activations are repacked from this file's
+ * structure-of-arrays quantizer output into block_q8_0 records first).  The scale of a block is read through
+ * scale_value(), i.e. with the x86 build's storage rounding when scale_mode says so.
+ * Every output goes through exactly the operations of dot_row() above (same eight lanes, same fused multiply-add, same
+ * horizontal sum), so the two must agree bit for bit: tests/test_oracle_golden.py checks that.
+ * ---------------------------------------------------------------------------------------------- */
+#if defined(__AVX2__) && defined(__FMA__)
+#include <immintrin.h>
+#include <omp.h>
+
+typedef struct {
+  const uint8_t* A; /* weight blocks [m rows][k blocks] */
+  const uint8_t* B; /* activation blocks (34 bytes each) [n rows][k blocks] */
+  const float* bias;
+  float* C;
+  int64_t k, lda, ldb, ldc;
+  int ith, nth, wtype, scale_mode, abytes;
+} tb_q0;
+
+static inline float tb_hsum(__m256 x) { /* llamafile_sgemm.cpp:161-177 */
+  __m128 v = _mm_add_ps(_mm256_extractf128_ps(x, 1), _mm256_castps256_ps128(x));
+  v = _mm_add_ps(v, _mm_movehl_ps(v, v));
+  v = _mm_add_ss(v, _mm_movehdup_ps(v));
+  return _mm_cvtss_f32(v);
+}
+static inline __m256i tb_load_w(const tb_q0* t, const uint8_t* blk) {
+  if (t->wtype == ORC_Q4_0) { /* denibble(qs) - 8, :757,774-777 */
+    __m128i x = _mm_loadu_si128((const __m128i*)(blk + 2));
+    __m256i n = _mm256_and_si256(_mm256_set1_epi8(15), _mm256_insertf128_si256(_mm256_castsi128_si256(x), _mm_srli_epi16(x, 4), 1));
+    return _mm256_sub_epi8(n, _mm256_set1_epi8(8));
+  }
+  return _mm256_loadu_si256((const __m256i*)(blk + 2));
+}
+static inline __m256 tb_updot(__m256i u, __m256i s) { /* :762-772, the branch without VNNI */
+  return _mm256_cvtepi32_ps(_mm256_madd_epi16(_mm256_set1_epi16(1), _mm256_maddubs_epi16(u, s)));
+}
+
+#define TB_GEMM(RM, RN)                                                                                                  \
+  static void tb_gemm_##RM##x##RN(const tb_q0* t, int64_t m0, int64_t m, int64_t n0, int64_t n) {                        \
+    const int64_t ytiles = (m - m0) / RM, xtiles = (n - n0) / RN, tiles = xtiles * ytiles;                               \
+    const int64_t duty = (tiles + t->nth - 1) / t->nth, start = duty * t->ith;                                           \
+    int64_t end = start + duty;                                                                                          \
+    if (end > tiles) end = tiles;                                                                                        \
+    for (int64_t job = start; job < end; ++job) {                                                                        \
+      const int64_t ii = m0 + job / xtiles * RM, jj = n0 + job % xtiles * RN;                                            \
+      __m256 Cv[RN][RM];                                                                                                 \
+      for (int j = 0; j < RN; ++j)                                                                                       \
+        for (int i = 0; i < RM; ++i) Cv[j][i] = _mm256_setzero_ps();                                                     \
+      for (int64_t l = 0; l < t->k; ++l)                                                                                 \
+        for (int j = 0; j < RN; ++j)                                                                                     \
+          for (int i = 0; i < RM; ++i) {                                                                                 \
+            const uint8_t* ab = t->A + (t->lda * (ii + i) + l) * t->abytes;                                              \
+            const uint8_t* bb = t->B + (t->ldb * (jj + j) + l) * 34;                                                     \
+            const __m256i a = tb_load_w(t, ab), b = _mm256_loadu_si256((const __m256i*)(bb + 2));                        \
+            const __m256 ud = tb_updot(_mm256_sign_epi8(a, a), _mm256_sign_epi8(b, a));                                  \
+            const float d = scale_value(blk_d(ab), t->scale_mode) * scale_value(blk_d(bb), t->scale_mode);               \
+            Cv[j][i] = _mm256_fmadd_ps(_mm256_set1_ps(d), ud, Cv[j][i]);                                                 \
+          }                                                                                                              \
+      for (int j = 0; j < RN; ++j)                                                                                       \
+        for (int i = 0; i < RM; ++i) {                                                                                   \
+          const float v = tb_hsum(Cv[j][i]);                                                                             \
+          t->C[t->ldc * (jj + j) + (ii + i)] = t->bias ? t->bias[ii + i] + v : v;                                        \
+        }                                                                                                                \
+    }                                                                                                                    \
+  }
+TB_GEMM(4, 2) TB_GEMM(2, 4) TB_GEMM(3, 2) TB_GEMM(2, 3) TB_GEMM(4, 1) TB_GEMM(2, 2) TB_GEMM(1, 4) TB_GEMM(3, 1)
+TB_GEMM(1, 3) TB_GEMM(2, 1) TB_GEMM(1, 2) TB_GEMM(1, 1)
+#undef TB_GEMM
+
+static void tb_mnpack(const tb_q0* t, int64_t m0, int64_t m, int64_t n0, int64_t n) { /* :588-695, VECTOR_REGISTERS == 16 */
+  int64_t mc, nc;
+  const int64_t dm = m - m0 < 4 ? m - m0 : 4, dn = n - n0 < 4 ? n - n0 : 4;
+  switch ((int)((dm << 4) | dn)) {
+    case 0x44: case 0x43: case 0x42: mc = 4; nc = 2; tb_gemm_4x2(t, m0, m, n0, n); break;
+    case 0x34: case 0x24: mc = 2; nc = 4; tb_gemm_2x4(t, m0, m, n0, n); break;
+    case 0x33: case 0x32: mc = 3; nc = 2; tb_gemm_3x2(t, m0, m, n0, n); break;
+    case 0x23: mc = 2; nc = 3; tb_gemm_2x3(t, m0, m, n0, n); break;
+    case 0x41: mc = 4; nc = 1; tb_gemm_4x1(t, m0, m, n0, n); break;
+    case 0x22: mc = 2; nc = 2; tb_gemm_2x2(t, m0, m, n0, n); break;
+    case 0x14: mc = 1; nc = 4; tb_gemm_1x4(t, m0, m, n0, n); break;
+    case 0x31: mc = 3; nc = 1; tb_gemm_3x1(t, m0, m, n0, n); break;
+    case 0x13: mc = 1; nc = 3; tb_gemm_1x3(t, m0, m, n0, n); break;
+    case 0x21: mc = 2; nc = 1; tb_gemm_2x1(t, m0, m, n0, n); break;
+    case 0x12: mc = 1; nc = 2; tb_gemm_1x2(t, m0, m, n0, n); break;
+    case 0x11: mc = 1; nc = 1; tb_gemm_1x1(t, m0, m, n0, n); break;
+    default: return;
+  }
+  const int64_t mp = m0 + (m - m0) / mc * mc, np = n0 + (n - n0) / nc * nc;
+  tb_mnpack(t, mp, m, n0, np);
+  tb_mnpack(t, m0, m, np, n);
+}
+
+/* x fp32 [M][K]; W reference blocks [N][K/32]; y fp32 [M][N]; nth threads as the op's `threads` option (default 8,
+ * mllm/core/BaseOp.hpp:77).  work: M * (K/32) * 34 bytes for the activation blocks, or NULL (allocated per call, as
+ * mat_mul allocates its temporary, ggml/matmul.cpp:148-153). */
+ORC_API int orc_linear_q_tiles(const float* x, const uint8_t* W, int wtype, const float* bias, float* y, int M, int N, int K,
+                               int scale_mode, int nth, uint8_t* work) {
+  if (K % QK != 0 || M < 0 || N < 0 || nth < 1) return -1;
+  const int nb = K / QK;
+  uint8_t* B = work ? work : (uint8_t*)malloc((size_t)M * nb * 34 + 64);
+  if (!B) return -2;
+  /* quantize_row_q8_0 per activation row, rows spread over the threads (ggml/matmul.cpp:173-187) */
+#pragma omp parallel for schedule(static) num_threads(nth)
+  for (int mrow = 0; mrow < M; mrow++) {
+    int8_t q[QK];
+    uint16_t d;
+    for (int b = 0; b < nb; b++) {
+      orc_quantize_row_q8_0(x + (size_t)mrow * K + (size_t)b * QK, q, &d, QK);
+      uint8_t* blk = B + ((size_t)mrow * nb + b) * 34;
+      memcpy(blk, &d, 2);
+      memcpy(blk + 2, q, QK);
+    }
+  }
+#pragma omp parallel num_threads(nth)
+  {
+    tb_q0 t = {W, B, bias, y, nb, nb, nb, N, omp_get_thread_num(), omp_get_num_threads(), wtype, scale_mode, blk_bytes(wtype)};
+    tb_mnpack(&t, 0, N, 0, M);
+  }
+  if (!work) free(B);
+  return 0;
+}
+#else
+ORC_API int orc_linear_q_tiles(const float* x, const uint8_t* W, int wtype, const float* bias, float* y, int M, int N, int K,
+                               int scale_mode, int nth, uint8_t* work) {
+  (void)nth; (void)work;
+  return orc_linear_q(x, W, wtype, bias, y, M, N, K, scale_mode, NULL, NULL);
+}
+#endif
+
+/* ------------------------------------------------------------------------------------------------
  * W4A16, group 128 along K, uint4 codes with uint4 zero-points and fp16 scales (AWQ/Marlin semantics):
  *   w = (q - zp) * scale, computed in the activation dtype   mllm-kernel/mllm_kernel/cuda/csrc/gemm/marlin/dequant.h:18-26,
  *                                                            marlin_template.h:153-168

@@ -282,3 +282,25 @@ def test_golden_kquant(golden_dir, name, wtype):
     q, d, bs = orc.quantize_rows_q8_K(g["q8k_x"])
     assert np.array_equal(q, g["q8k_q"]) and np.array_equal(d.view(np.uint32), g["q8k_d"].view(np.uint32))
     assert np.array_equal(bs, g["q8k_bsums"])
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+def test_avx2_tile_form_equals_the_scalar_restatement_bit_for_bit(wtype):
+    """orc_linear_q_tiles (the vector instructions, tile shapes and job split of tinyBLAS_Q0_AVX, llamafile_sgemm.cpp:579-790)
+    against orc_linear_q (scalar, pinned against the compiled vec_dot_* of the reference): every output goes through the same
+    eight lanes, fused multiply-adds and horizontal sum, so the bits must agree for every tile shape of mnpack (rows 1..9
+    exercise 4x2, 2x4, 3x2, 2x3, 4x1, ... down to 1x1 with ragged edges), with and without bias, for any thread count."""
+    from mllm_amd import synth
+    from oracle import oracle as orc
+    rng = synth.rng_for(2, 800 + wtype)
+    for M, N, K in [(1, 64, 256), (2, 37, 96), (3, 50, 64), (4, 33, 128), (5, 7, 32), (7, 130, 160), (9, 23, 96)]:
+        W = synth.make_weight(rng, wtype, N, K)
+        x = synth.make_x_fp32(rng, M, K)
+        bias = rng.standard_normal(N).astype(np.float32)
+        for mode in (orc.SCALE_X86_REF, orc.SCALE_IEEE):
+            want = orc.linear_q(x, W, wtype, None, mode)
+            for threads in (1, 3, 8):
+                got = orc.linear_q_tiles(x, W, wtype, None, mode, threads)
+                assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (M, N, K, mode, threads)
+        wb = orc.linear_q(x, W, wtype, bias, orc.SCALE_X86_REF)
+        assert np.array_equal(orc.linear_q_tiles(x, W, wtype, bias, orc.SCALE_X86_REF, 4).view(np.uint32), wb.view(np.uint32))
