@@ -258,6 +258,17 @@ int mllm_hip_w4a16_gemm(const void* a_bf16, const uint8_t* qw, const uint16_t* s
 int mllm_hip_w4a16_dequantize(const uint8_t* qw, const uint16_t* scales, const uint8_t* zeros, void* w_bf16, int64_t N,
                               int64_t K, int group, void* stream);
 
+/* AWQ checkpoint tensors -> the row-major tensors mllm_hip_w4a16_gemm / mllm_hip_w4a16_prepack take.
+ * replaces: the unpacking half of AWQMarlinLinearMethod.process_weights_after_loading
+ *           pymllm/quantization/methods/awq_marlin.py:366-410 (awq_marlin_repack, awq_to_marlin_zero_points :237-259,
+ *           unpack_cols :202-213), mllm-kernel/mllm_kernel/cuda/csrc/gemm/marlin/awq_marlin_repack.cuh:106-126
+ * qweight int32 [K][N/8] and qzeros int32 [K/group][N/8] hold eight 4-bit codes per dword, nibble position p = output
+ * column 8 j + {0,2,4,6,1,3,5,7}[p]; scales fp16 [K/group][N] (create_weights, awq_marlin.py:284-364).
+ * Writes qw uint8 [N][K/2], scales_out fp16 [N][K/group], zeros_out uint8 [N][ceil(K/group/2)].
+ * N % 8 == 0, K % 8 == 0, K % group == 0. */
+int mllm_hip_w4a16_from_awq(const int32_t* qweight, const int32_t* qzeros, const uint16_t* scales, int64_t N, int64_t K,
+                            int group, uint8_t* qw, uint16_t* scales_out, uint8_t* zeros_out, void* stream);
+
 /* GEMM tile override for tuning sweeps: 0 heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64 workgroup tiles. */
 int mllm_hip_w4a16_set_tuning(int tile);
 

@@ -109,6 +109,7 @@ def lib():
         L.mllm_hip_w8a8_linear_packed.argtypes = [vp, ci, vp, vp, vp, vp, i64, i64, i64, vp, vp]
         L.mllm_hip_w4a16_gemm.argtypes = [vp, vp, vp, vp, vp, vp, i64, i64, i64, ci, vp]
         L.mllm_hip_w4a16_dequantize.argtypes = [vp, vp, vp, vp, i64, i64, ci, vp]
+        L.mllm_hip_w4a16_from_awq.argtypes = [vp, vp, vp, i64, i64, ci, vp, vp, vp, vp]
         L.mllm_hip_w4a16_set_tuning.argtypes = [ci]
         L.mllm_hip_w4a16_packed_set_tuning.argtypes = [ci]
         L.mllm_hip_w4a16_packed_bytes.restype = C.c_size_t

@@ -6,6 +6,8 @@
 //   block dot + scaling       mllm/backends/cpu/kernels/common/llamafile/llamafile_sgemm.cpp:697-743
 //   flow                      mllm/backends/cpu/kernels/common/ggml/matmul.cpp:148-206
 // The int32 block sums are exact; the fp32 accumulation order differs from the CPU's 8-lane order (tolerance 1e-3 rel-L2).
+#include <algorithm>
+
 #include "qgemv_kernel.h"
 
 #include <string.h>
@@ -227,6 +229,10 @@ static GemvShape pick_shape(int MT, int64_t N, int nb) {
     s.G = 64;
     if (MT <= 2) s.R = 1;
     s.NW = 16;
+    // one row per wave: the waves per workgroup only decide how many workgroups there are (not the arithmetic).  With sixteen
+    // the 2560 rows of a down projection make 160 workgroups on 256 CUs; about one workgroup per CU measured best
+    // (N = 2560, 304 blocks: 16 waves 5.84 us, 11 waves 5.27 us, 8 waves 6.4 us)
+    if (MT <= 2) s.NW = (int)std::min<int64_t>(16, std::max<int64_t>(8, (N + 239) / 240));
   } else if (nb >= 64) {
     s.G = 32;
   } else if (nb >= 16) {
@@ -243,7 +249,6 @@ static GemvShape pick_shape(int MT, int64_t N, int nb) {
     s.NW = 8;
     if (nb >= 128) s.G = 64;
   }
-  (void)N;
   if (g_tune_G) s.G = g_tune_G;
   if (g_tune_R) s.R = g_tune_R;
   if (g_tune_NW) s.NW = g_tune_NW;

@@ -640,6 +640,73 @@ MLLM_API int mllm_hip_w4a16_dequantize(const uint8_t* qw, const uint16_t* scales
   return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// AWQ checkpoint tensors -> the row-major layout of this file (the unpacking half of what the reference does in
+// AWQMarlinLinearMethod.process_weights_after_loading, pymllm/quantization/methods/awq_marlin.py:366-410).
+//   qweight int32 [K][N/8], qzeros int32 [K/group][N/8]: eight 4-bit codes of eight neighbouring output columns per dword,
+//   nibble position p holding column 8 j + {0,2,4,6,1,3,5,7}[p] (awq_marlin.py:202-213 unpack_cols followed by the
+//   undo_interleave of :248-257; awq_marlin_repack.cuh:108-110 reads column c from nibble {0,4,1,5,2,6,3,7}[c]);
+//   scales fp16 [K/group][N].
+// The weight codes are transposed through LDS in 64 x 64 tiles so that both the checkpoint reads and the [N][K/2] writes
+// are whole 32-byte runs.
+__device__ __forceinline__ int awq_nibble_of_column(int c) { return ((c & 1) << 2) | (c >> 1); }  // {0,4,1,5,2,6,3,7}[c]
+
+__global__ __launch_bounds__(256) void awq_unpack_q_kernel(const uint32_t* __restrict__ qweight, uint32_t* __restrict__ qw,
+                                                           int N, int K) {
+  __shared__ uint32_t tile[64][9];  // [k][column dword], one pad dword against bank conflicts of the column reads
+  const int n0 = blockIdx.x * 64, k0 = blockIdx.y * 64, t = threadIdx.x;
+  const int nd = N / 8;
+  for (int i = t; i < 512; i += 256) {
+    const int k = k0 + i / 8, j = n0 / 8 + i % 8;
+    tile[i / 8][i % 8] = (k < K && j < nd) ? qweight[(int64_t)k * nd + j] : 0u;
+  }
+  __syncthreads();
+  for (int i = t; i < 512; i += 256) {
+    const int r = i / 8, kd = i % 8;  // output row n0 + r, its dword of elements k0 + 8 kd .. + 7
+    const int n = n0 + r, k = k0 + kd * 8;
+    if (n >= N || k >= K) continue;
+    const int sh = 4 * awq_nibble_of_column(r & 7);
+    uint32_t v = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v |= ((tile[kd * 8 + e][r >> 3] >> sh) & 15u) << (4 * e);
+    qw[((int64_t)n * K + k) / 8] = v;
+  }
+}
+
+__global__ __launch_bounds__(256) void awq_unpack_sz_kernel(const uint32_t* __restrict__ qzeros, const uint16_t* __restrict__ s_in,
+                                                            uint16_t* __restrict__ s_out, uint8_t* __restrict__ z_out, int N,
+                                                            int G) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (group, n): neighbouring threads read neighbouring columns
+  if (i >= (int64_t)N * G) return;
+  const int n = (int)(i % N), g = (int)(i / N);
+  s_out[(int64_t)n * G + g] = s_in[(int64_t)g * N + n];
+  if (g & 1) return;  // one thread per byte of zero points: groups g (low nibble) and g + 1 (high nibble)
+  const int sh = 4 * awq_nibble_of_column(n & 7), nd = N / 8;
+  uint32_t z = (qzeros[(int64_t)g * nd + n / 8] >> sh) & 15u;
+  if (g + 1 < G) z |= ((qzeros[(int64_t)(g + 1) * nd + n / 8] >> sh) & 15u) << 4;
+  z_out[(int64_t)n * ((G + 1) / 2) + g / 2] = (uint8_t)z;
+}
+
+MLLM_API int mllm_hip_w4a16_from_awq(const int32_t* qweight, const int32_t* qzeros, const uint16_t* scales, int64_t N,
+                                     int64_t K, int group, uint8_t* qw, uint16_t* scales_out, uint8_t* zeros_out,
+                                     void* stream) {
+  if (!qweight || !qzeros || !scales || !qw || !scales_out || !zeros_out || N <= 0 || K <= 0 || group <= 0)
+    return MLLM_HIP_E_BADARG;
+  if (N % 8 || K % 8 || K % group) return MLLM_HIP_E_SHAPE;
+  if (N * K / 2 >= ((int64_t)1 << 32) || N > INT32_MAX || K > INT32_MAX) return MLLM_HIP_E_SHAPE;
+  if (reinterpret_cast<uintptr_t>(qw) % 4 || reinterpret_cast<uintptr_t>(qweight) % 4 ||
+      reinterpret_cast<uintptr_t>(qzeros) % 4)
+    return MLLM_HIP_E_ALIGN;
+  const int G = (int)(K / group);
+  if ((K + 63) / 64 > 65535) return MLLM_HIP_E_SHAPE;
+  hipLaunchKernelGGL(awq_unpack_q_kernel, dim3((unsigned)((N + 63) / 64), (unsigned)((K + 63) / 64)), dim3(256), 0,
+                     (hipStream_t)stream, reinterpret_cast<const uint32_t*>(qweight), reinterpret_cast<uint32_t*>(qw), (int)N,
+                     (int)K);
+  hipLaunchKernelGGL(awq_unpack_sz_kernel, dim3((unsigned)((N * G + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                     reinterpret_cast<const uint32_t*>(qzeros), scales, scales_out, zeros_out, (int)N, G);
+  return (int)hipGetLastError();
+}
+
 MLLM_API size_t mllm_hip_w4a16_packed_bytes(int64_t N, int64_t K, int group) {
   if (N <= 0 || K <= 0 || group <= 0 || group % 64 || K % group) return 0;
   return (size_t)(w4a16_packed_qbytes(N, K) + w4a16_packed_n(N) * (K / group) * 8);

@@ -256,6 +256,24 @@ def w4a16_gemm(a, qw, scales, zeros, bias=None, group=128, out=None):
     return y
 
 
+def w4a16_from_awq(qweight, qzeros, scales, group=128):
+    """AWQ checkpoint tensors (qweight int32 [K, N/8], qzeros int32 [K/group, N/8], scales fp16 [K/group, N]) ->
+    (qw uint8 [N, K/2], scales fp16 [N, K/group], zeros uint8 [N, ceil(K/group/2)]), the inputs of w4a16_gemm / w4a16_prepack.
+    pymllm/quantization/methods/awq_marlin.py:284-410."""
+    assert qweight.dtype == torch.int32 and qzeros.dtype == torch.int32 and scales.dtype == torch.float16
+    assert qweight.is_contiguous() and qzeros.is_contiguous() and scales.is_contiguous()
+    K, N = qweight.shape[0], qweight.shape[1] * 8
+    G = K // group
+    assert qzeros.shape == (G, N // 8) and scales.shape == (G, N)
+    qw = torch.empty((N, K // 2), dtype=torch.uint8, device="cuda")
+    s = torch.empty((N, G), dtype=torch.float16, device="cuda")
+    z = torch.empty((N, (G + 1) // 2), dtype=torch.uint8, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_w4a16_from_awq(qweight.data_ptr(), qzeros.data_ptr(), scales.data_ptr(), N, K, group,
+                                                  qw.data_ptr(), s.data_ptr(), z.data_ptr(), _stream()),
+               "mllm_hip_w4a16_from_awq")
+    return qw, s, z
+
+
 def w4a16_prepack(qw, scales, zeros, group=128):
     """Checkpoint tensors -> the packed weight blob of the fast GEMM (uint8), done once per weight."""
     assert qw.dtype == torch.uint8 and scales.dtype == torch.float16 and qw.is_contiguous() and scales.is_contiguous()

@@ -154,6 +154,29 @@ def make_w4a16(rng, N, K, group=128, sigma=0.01):
     return pack_nibbles(q), s, pack_nibbles(z), q, z
 
 
+def pack_awq_cols(codes):
+    """codes [R, N] in [0, 15] -> int32 [R, N/8] as an AWQ checkpoint stores them: each run of eight columns reordered to
+    (0, 2, 4, 6, 1, 3, 5, 7) and then packed column i of the run into bits 4 i .. 4 i + 3 (the pack_cols of
+    pymllm/quantization/methods/awq_marlin.py:188-199 applied to the interleaved columns)."""
+    codes = np.asarray(codes, dtype=np.uint32)
+    R, N = codes.shape
+    assert N % 8 == 0
+    inter = codes.reshape(-1, 8)[:, [0, 2, 4, 6, 1, 3, 5, 7]].reshape(R, N)
+    out = np.zeros((R, N // 8), np.uint32)
+    for i in range(8):
+        out |= inter[:, i::8] << np.uint32(4 * i)
+    return out.view(np.int32)
+
+
+def make_awq(rng, N, K, group=128, sigma=0.01):
+    """returns (qweight int32 [K, N/8], qzeros int32 [G, N/8], scales fp16 bits [G, N], q [N, K], z [N, G], s bits [N, G])."""
+    G = K // group
+    q = rng.integers(0, 16, size=(N, K), dtype=np.uint8)
+    z = rng.integers(0, 16, size=(N, G), dtype=np.uint8)
+    s = np.abs(rng.normal(0.0, sigma, size=(N, G))).astype(np.float32).astype(np.float16).view(np.uint16)
+    return pack_awq_cols(q.T), pack_awq_cols(z.T), np.ascontiguousarray(s.T), q, z, s
+
+
 # ----------------------------------------------------------------------------- W8A8
 def make_w8a8(rng, M, N, K):
     """A bf16 bits [M, K] ~N(0,1) with 1 % of entries x20; W int8 [N, K]; w_scale fp32 [N]."""

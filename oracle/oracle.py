@@ -176,6 +176,32 @@ def w4a16_dequant(qw, s_bits, zp, group=128):
     return w
 
 
+AWQ_ORDER = np.array([0, 2, 4, 6, 1, 3, 5, 7])  # nibble position p of a checkpoint dword holds column 8 j + AWQ_ORDER[p]
+
+
+def awq_unpack_cols(packed):
+    """int32 [R, N/8] -> codes [R, N] in true column order: unpack_cols (pymllm/quantization/methods/awq_marlin.py:202-213)
+    followed by the undo_interleave step of awq_to_marlin_zero_points (:248-257)."""
+    packed = np.ascontiguousarray(packed).view(np.uint32)
+    R, nd = packed.shape
+    out = np.zeros((R, nd * 8), np.uint8)
+    for i in range(8):
+        out[:, i::8] = (packed >> np.uint32(4 * i)) & np.uint32(15)
+    undo = np.argsort(AWQ_ORDER)
+    return out.reshape(-1, 8)[:, undo].reshape(R, nd * 8)
+
+
+def awq_unpack(qweight, qzeros, scales_bits):
+    """AWQ checkpoint tensors (qweight int32 [K, N/8], qzeros int32 [G, N/8], scales fp16 bits [G, N]) -> the row-major
+    tensors of w4a16_dequant / w4a16_gemm: (qw uint8 [N, K/2], scales uint16 [N, G], zeros uint8 [N, ceil(G/2)])."""
+    q = awq_unpack_cols(qweight).T  # [N, K]
+    z = awq_unpack_cols(qzeros).T  # [N, G]
+    if z.shape[1] % 2:
+        z = np.concatenate([z, np.zeros((z.shape[0], 1), np.uint8)], axis=1)
+    return ((q[:, 0::2] | (q[:, 1::2] << 4)).astype(np.uint8), np.ascontiguousarray(np.asarray(scales_bits, np.uint16).T),
+            (z[:, 0::2] | (z[:, 1::2] << 4)).astype(np.uint8))
+
+
 def w4a16_gemm(a_bits, qw, s_bits, zp, bias_bits=None, group=128):
     """A bf16 bits [M, K] -> C bf16 bits [M, N]."""
     a_bits = np.ascontiguousarray(a_bits, dtype=np.uint16)

@@ -90,6 +90,9 @@ def _cases():
         "mllm_hip_w4a16_gemm": ([P, P, P, P, None, P, 16, 64, 256, 128, None],
                                 [(0, None, BADARG), (1, None, BADARG), (2, None, BADARG), (5, None, BADARG), (9, 100, SHAPE),
                                  (8, 200, SHAPE)]),
+        "mllm_hip_w4a16_from_awq": ([P, P, P, 64, 256, 128, P, P, P, None],
+                                    [(0, None, BADARG), (1, None, BADARG), (2, None, BADARG), (6, None, BADARG), (7, None, BADARG),
+                                     (8, None, BADARG), (3, 60, SHAPE), (4, 100, SHAPE), (5, 96, SHAPE), (6, ODD, ALIGN)]),
         "mllm_hip_w4a16_gemm_packed": ([P, P, None, P, 16, 64, 256, 128, None],
                                        [(0, None, BADARG), (1, None, BADARG), (3, None, BADARG), (7, 100, SHAPE)]),
         "mllm_hip_rmsnorm": ([P, F32, P, P, 1, 64, C.c_float(1e-6), 0, None, 0, None],

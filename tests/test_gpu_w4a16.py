@@ -167,3 +167,28 @@ def test_argument_errors():
     assert g(None, p, p, p, None, p, 8, 8, 128, 128, None) == -1
     assert g(p, p + 1, p, p, None, p, 8, 8, 128, 128, None) == -3
     assert L.mllm_hip_w4a16_set_tuning(-1) == -1
+
+
+@pytest.mark.parametrize("N,K,group", [(8, 128, 128), (24, 384, 128), (200, 512, 64), (72, 1000, 200), (9728, 2560, 128)])
+def test_awq_checkpoint_unpack_bit_exact_and_gemm(N, K, group):
+    """AWQ int32 tensors -> row-major tensors byte for byte (against the known codes and against the oracle's unpack of the
+    same dwords), then the packed GEMM on them against the oracle."""
+    rng = synth.rng_for(2, N + K + group + 5)
+    qweight, qzeros, scales, q, z, s = synth.make_awq(rng, N, K, group)
+    announce("w4a16 from awq N=%d K=%d group=%d" % (N, K, group))
+    qw_d, s_d, z_d = ql.w4a16_from_awq(torch.from_numpy(qweight).cuda(), torch.from_numpy(qzeros).cuda(),
+                                       torch.from_numpy(scales.view(np.float16).copy()).cuda(), group)
+    torch.cuda.synchronize()
+    assert np.array_equal(qw_d.cpu().numpy(), synth.pack_nibbles(q))
+    assert np.array_equal(z_d.cpu().numpy(), synth.pack_nibbles(z))
+    assert np.array_equal(_bits(s_d), s)
+    oq, osb, oz = orc.awq_unpack(qweight, qzeros, scales)
+    assert np.array_equal(qw_d.cpu().numpy(), oq) and np.array_equal(z_d.cpu().numpy(), oz) and np.array_equal(_bits(s_d), osb)
+    if group % 64 or N > 1000:
+        return
+    M = 37
+    a_bits, _ = synth.make_x_bf16(rng, M, K)
+    packed = ql.w4a16_prepack(qw_d, s_d, z_d, group)
+    got = _bits(ql.w4a16_gemm_packed(bf16_dev(a_bits), packed, N, None, group))
+    want = orc.w4a16_gemm(a_bits, oq, osb, oz, None, group)
+    assert rel_l2(synth.bf16_bits_to_fp32(got), synth.bf16_bits_to_fp32(want)) <= TOL

@@ -304,3 +304,17 @@ def test_avx2_tile_form_equals_the_scalar_restatement_bit_for_bit(wtype):
                 assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (M, N, K, mode, threads)
         wb = orc.linear_q(x, W, wtype, bias, orc.SCALE_X86_REF)
         assert np.array_equal(orc.linear_q_tiles(x, W, wtype, bias, orc.SCALE_X86_REF, 4).view(np.uint32), wb.view(np.uint32))
+
+
+def test_awq_checkpoint_order_known_answer_and_round_trip():
+    """A dword whose nibble p holds the value p: the reference reads column c of the run from nibble (0, 4, 1, 5, 2, 6, 3, 7)[c]
+    (mllm-kernel/mllm_kernel/cuda/csrc/gemm/marlin/awq_marlin_repack.cuh:108-110), so the columns read 0 4 1 5 2 6 3 7."""
+    one = np.array([[0x76543210]], np.uint32).view(np.int32)
+    assert orc.awq_unpack_cols(one).tolist() == [[0, 4, 1, 5, 2, 6, 3, 7]]
+    # second dword of a row = columns 8..15; value 0xF in nibble 1 only -> column 2 of that run
+    two = np.array([[0, 0x000000F0]], np.uint32).view(np.int32)
+    assert np.flatnonzero(orc.awq_unpack_cols(two)[0]).tolist() == [10]
+    rng = synth.rng_for(2, 77)
+    qweight, qzeros, scales, q, z, s = synth.make_awq(rng, 24, 384, 128)
+    qw, s2, zp = orc.awq_unpack(qweight, qzeros, scales)
+    assert np.array_equal(qw, synth.pack_nibbles(q)) and np.array_equal(zp, synth.pack_nibbles(z)) and np.array_equal(s2, s)
