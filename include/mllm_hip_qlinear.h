@@ -38,6 +38,8 @@ enum { MLLM_HIP_F32 = 0, MLLM_HIP_BF16 = 1 };
 /* instead of activations: their Q8_0 image as the decode GEMV reads it (mllm_hip_gemv_workspace_bytes, written by
  * mllm_hip_rmsnorm / mllm_hip_silu_mul); only where an entry point says so */
 enum { MLLM_HIP_Q8_IMAGE = 2 };
+/* IEEE half precision; only where an entry point says so (mllm_hip_matmul_batched) */
+enum { MLLM_HIP_F16 = 3 };
 /* How a block scale is read.
  *   IEEE     the 2-byte `d` field is an IEEE fp16 bit pattern (ARM builds of the reference, GGUF files)
  *   X86_REF  the x86 build of the reference: the field is a half-precision NUMBER equal to the bit pattern
@@ -436,10 +438,17 @@ int mllm_hip_moe_gate(const void* x, int x_dtype, const float* gate_weight, int3
                       int64_t M, int64_t H, int64_t E, int k, int norm_topk_prob, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------
- * fp32 activation x activation MatMul (the backend's kMatMul slot; not a quantized path)
- * replaces: CPUMatMulOp::forward  mllm/backends/cpu/ops/MatMulOp.cpp:47-61
- * C[M][N] = op(A) * op(B), op(X) = X or X^T; A is [M][K] ([K][M] when transposed), B is [K][N] ([N][K] when transposed).
+ * Activation x activation MatMul on the matrix cores (the backend's kMatMul slot; not a quantized path)
+ * replaces: CPUMatMulOp::forward  mllm/backends/cpu/ops/MatMulOp.cpp:19-90 (shapes :30-44, default kernel choice :47-61)
+ * C[b][M][N] = op(A[b]) * op(B[b]), op(X) = X or X^T; A[b] is [M][K] ([K][M] when transposed), B[b] is [K][N] ([N][K]
+ * when transposed).  dtype MLLM_HIP_F32, MLLM_HIP_BF16 or MLLM_HIP_F16 for all three tensors; products are exact and
+ * summed in fp32, 16-bit results are rounded once to nearest even.  Batch entry b starts stride_x * b elements after
+ * entry 0 (stride_b = 0 multiplies every A[b] by the same B); the whole batch is one launch.
  * ------------------------------------------------------------------------------------------------------- */
+int mllm_hip_matmul_batched(const void* A, const void* B, void* C, int dtype, int64_t batch, int64_t M, int64_t N, int64_t K,
+                            int64_t stride_a, int64_t stride_b, int64_t stride_c, int transpose_a, int transpose_b,
+                            void* stream);
+/* batch = 1, fp32 */
 int mllm_hip_matmul_f32(const float* A, const float* B, float* C, int64_t M, int64_t N, int64_t K, int transpose_a,
                         int transpose_b, void* stream);
 

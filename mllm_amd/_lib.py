@@ -139,6 +139,7 @@ def lib():
         L.mllm_hip_moe_gemm_set_path.argtypes = [ci]
         L.mllm_hip_moe_route.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, vp]
         L.mllm_hip_matmul_f32.argtypes = [vp, vp, vp, i64, i64, i64, ci, ci, vp]
+        L.mllm_hip_matmul_batched.argtypes = [vp, vp, vp, ci, i64, i64, i64, i64, i64, i64, i64, ci, ci, vp]
         _lib = L
     return _lib
 

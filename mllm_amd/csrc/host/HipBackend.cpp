@@ -153,20 +153,29 @@ void HipMatMulOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
   const auto& a = inputs[0];
   const auto& b = inputs[1];
   auto& c = outputs[0];
-  if (a.dtype() != kFloat32 || b.dtype() != kFloat32) NYI("HipMatMulOp supports fp32 operands only");
+  int dtype;
+  switch (a.dtype()) {
+    case kFloat32: dtype = MLLM_HIP_F32; break;
+    case kFloat16: dtype = MLLM_HIP_F16; break;
+    case kBFloat16: dtype = MLLM_HIP_BF16; break;
+    default: NYI("HipMatMulOp takes fp32, fp16 or bf16 operands"); return;
+  }
+  if (b.dtype() != a.dtype() || c.dtype() != a.dtype()) NYI("HipMatMulOp: both operands and the output share one element type");
   backend().noteWrite(c.ptr<void>(), c.bytes());
   const auto& cs = c.shape();
   const int64_t M = cs[cs.size() - 2], N = cs[cs.size() - 1];
   const auto& as = a.shape();
   const int64_t K = options_.transpose_a ? as[as.size() - 2] : as[as.size() - 1];
-  int64_t batch = 1;
+  int64_t batch = 1, b_batch = 1;
   for (size_t i = 0; i + 2 < cs.size(); i++) batch *= cs[i];
-  const bool b_batched = b.rank() == a.rank() && b.rank() > 2;
-  for (int64_t i = 0; i < batch; i++) {
-    MLLM_HIP_KERNEL_CHECK(mllm_hip_matmul_f32(a.ptr<float>() + i * M * K, b.ptr<float>() + (b_batched ? i * N * K : 0),
-                                              c.ptr<float>() + i * M * N, M, N, K, options_.transpose_a, options_.transpose_b,
-                                              backend().stream()));
-  }
+  for (size_t i = 0; i + 2 < b.shape().size(); i++) b_batch *= b.shape()[i];
+  // the reference wants equal batch counts (mllm/backends/cpu/ops/MatMulOp.cpp:40-44); a single right-hand matrix is
+  // additionally taken as shared by every batch entry
+  if (b_batch != batch && b_batch != 1) NYI("HipMatMulOp: batch counts of the operands differ");
+  // the whole batch is one launch
+  MLLM_HIP_KERNEL_CHECK(mllm_hip_matmul_batched(a.ptr<void>(), b.ptr<void>(), c.ptr<void>(), dtype, batch, M, N, K, M * K,
+                                                b_batch == batch ? N * K : 0, M * N, options_.transpose_a, options_.transpose_b,
+                                                backend().stream()));
 }
 
 // ---- Linear ------------------------------------------------------------------------------------------------------

@@ -307,6 +307,30 @@ extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_matmu
   return 0;
 }
 
+// batched MatMul of any of the three element types (mllm DataTypes id: 0 fp32, 1 fp16, 128 bf16) through the same slot;
+// a is [batch][M][K] ([batch][K][M] transposed), b is [batch][K][N] ([batch][N][K] transposed) or one matrix for all
+extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_run_matmul_batched(const void* a_host, const void* b_host,
+                                                                                          void* c_host, int dtype, int batch, int M,
+                                                                                          int N, int K, int transpose_a,
+                                                                                          int transpose_b, int b_batched) {
+  initializeContext();
+  hip::initHipBackend();
+  auto& ctx = Context::instance();
+  const DataTypes dt = (DataTypes)dtype;
+  Tensor::shape_t sa = transpose_a ? Tensor::shape_t{batch, K, M} : Tensor::shape_t{batch, M, K};
+  Tensor::shape_t sb = transpose_b ? Tensor::shape_t{N, K} : Tensor::shape_t{K, N};
+  if (b_batched) sb.insert(sb.begin(), batch);
+  Tensor a = Tensor::fromExternal(const_cast<void*>(a_host), sa, dt, kCPU).to(kHIP);
+  Tensor b = Tensor::fromExternal(const_cast<void*>(b_host), sb, dt, kCPU).to(kHIP);
+  aops::MatMulOpOptions o;
+  o.transpose_a = transpose_a != 0;
+  o.transpose_b = transpose_b != 0;
+  auto outs = ctx.buildOpAndSubmitTask(OpTypes::kMatMul, o, {a, b});
+  Tensor c = outs[0].to(kCPU);
+  std::memcpy(c_host, c.ptr<void>(), c.bytes());
+  return 0;
+}
+
 // error-path probe for the CPU tests: asks a backend that was never registered for an op (the runtime's behaviour is to
 // terminate the process, mllm/engine/Context.cpp:37-42) -- run in a child process.
 extern "C" __attribute__((visibility("default"))) int mllm_hip_backend_probe_missing_backend() {

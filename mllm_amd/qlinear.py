@@ -665,3 +665,28 @@ def quantize_q8_K(x):
     _lib.check(_lib.lib().mllm_hip_quantize_q8_K(x.data_ptr(), _xdtype(x), codes.data_ptr(), d.data_ptr(), bs.data_ptr(), M, K, _stream()),
                "mllm_hip_quantize_q8_K")
     return codes, d, bs
+
+
+# ----------------------------------------------------------------------------- MatMul (activation x activation)
+_MM_DTYPE = {torch.float32: 0, torch.bfloat16: 1, torch.float16: 3}
+
+
+def matmul(a, b, transpose_a=False, transpose_b=False, out=None):
+    """C[..., M, N] = op(a) @ op(b) for fp32 / bf16 / fp16 tensors of rank >= 2, the whole batch in one launch; b may be a
+    single matrix shared by every batch entry.  mllm/backends/cpu/ops/MatMulOp.cpp:19-90."""
+    assert a.dtype == b.dtype and a.dtype in _MM_DTYPE and a.is_contiguous() and b.is_contiguous()
+    M, K = (a.shape[-1], a.shape[-2]) if transpose_a else (a.shape[-2], a.shape[-1])
+    N, Kb = (b.shape[-2], b.shape[-1]) if transpose_b else (b.shape[-1], b.shape[-2])
+    assert K == Kb
+    batch = 1
+    for d in a.shape[:-2]:
+        batch *= d
+    b_batch = 1
+    for d in b.shape[:-2]:
+        b_batch *= d
+    assert b_batch in (1, batch)
+    c = out if out is not None else torch.empty(tuple(a.shape[:-2]) + (M, N), dtype=a.dtype, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_matmul_batched(a.data_ptr(), b.data_ptr(), c.data_ptr(), _MM_DTYPE[a.dtype], batch, M, N, K,
+                                                  M * K, N * K if b_batch == batch and batch > 1 else 0, M * N,
+                                                  int(transpose_a), int(transpose_b), _stream()), "mllm_hip_matmul_batched")
+    return c

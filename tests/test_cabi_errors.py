@@ -102,6 +102,9 @@ def _cases():
         "mllm_hip_softmax": ([P, P, 2, 16, None], [(0, None, BADARG), (1, None, BADARG), (2, 0, BADARG)]),
         "mllm_hip_topk": ([P, P, P, 2, 16, 4, 1, 1, None], [(0, None, BADARG), (1, None, BADARG), (2, None, BADARG), (5, 0, SHAPE),
                                                             (5, 17, SHAPE)]),
+        "mllm_hip_matmul_batched": ([P, P, P, 0, 2, 4, 4, 4, 16, 16, 16, 0, 0, None],
+                                    [(0, None, BADARG), (1, None, BADARG), (2, None, BADARG), (3, 2, BADARG), (3, 7, BADARG),
+                                     (4, 0, BADARG), (5, 0, BADARG), (8, -1, BADARG), (10, 8, SHAPE), (0, P + 2, ALIGN)]),
         "mllm_hip_matmul_f32": ([P, P, P, 4, 4, 4, 0, 0, None], [(0, None, BADARG), (1, None, BADARG), (2, None, BADARG), (3, 0, BADARG)]),
     }
     return cases

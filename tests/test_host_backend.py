@@ -128,6 +128,31 @@ def test_matmul_slot():
     assert np.allclose(c, a @ b.T, rtol=1e-5, atol=1e-4)
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["fp32", "bf16", "fp16"])
+def test_matmul_slot_batched_in_one_launch(dtype):
+    """[batch][M][K] x [batch][K][N] (attention probabilities x values) and a transposed left operand through the kMatMul slot"""
+    import torch
+    from gpu_util import announce
+    L = _host()
+    rng = synth.rng_for(5, 10)
+    batch, M, N, K = 6, 40, 64, 50
+    td, tid = {"fp32": (torch.float32, 0), "bf16": (torch.bfloat16, 128), "fp16": (torch.float16, 1)}[dtype]
+    a = torch.from_numpy(rng.standard_normal((batch, M, K)).astype(np.float32)).to(td)
+    b = torch.from_numpy(rng.standard_normal((batch, K, N)).astype(np.float32)).to(td)
+    c = torch.empty((batch, M, N), dtype=td)
+    want = (a.double() @ b.double()).numpy()
+    tol = {"fp32": 2e-6, "bf16": 3e-3, "fp16": 4e-4}[dtype]
+    vp = lambda t: C.c_void_p(t.data_ptr())
+    announce("host matmul batched " + dtype)
+    assert L.mllm_hip_backend_run_matmul_batched(vp(a), vp(b), vp(c), tid, batch, M, N, K, 0, 0, 1) == 0
+    assert np.linalg.norm(c.double().numpy() - want) / np.linalg.norm(want) <= tol
+    at = a.transpose(1, 2).contiguous()
+    c.zero_()
+    assert L.mllm_hip_backend_run_matmul_batched(vp(at), vp(b), vp(c), tid, batch, M, N, K, 1, 0, 1) == 0
+    assert np.linalg.norm(c.double().numpy() - want) / np.linalg.norm(want) <= tol
+
+
 # ---- model files -------------------------------------------------------------------------------------------------------
 # Writers restated from the file layouts (mllm/core/schema/ModelFileV1.hpp:36-52, ModelFileV2.hpp:40-62; struct formats as
 # pymllm/mobile/convertor/model_file_v2.py:68-99 packs them).  dtype ids: mllm/core/DataTypes.hpp (kFloat32 0, kFloat16 1,
