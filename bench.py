@@ -324,7 +324,9 @@ def main():
 
     def make_io(M):
         xs = {k: torch.randn((M, k), device="cuda", generator=gen).to(torch.bfloat16) for k in (2560, 4096, 9728)}
-        xs["workspaces"] = {k: (ql.gemv_workspace(M, k) if M >= 3 else None) for k in (2560, 4096, 9728)}
+        # room for the K slices' partial sums of the widest launch that reads x of this length (gate + up: 2 x 9728 rows)
+        n_total = {2560: 2 * 9728, 4096: 2560, 9728: 2560}
+        xs["workspaces"] = {k: (ql.gemv_workspace(M, k, n_total[k]) if M >= 3 else None) for k in (2560, 4096, 9728)}
         ys = {name: torch.empty((M, n), dtype=torch.float32, device="cuda") for name, (n, _) in shapes.items()}
         return xs, ys
 
@@ -338,7 +340,7 @@ def main():
                 for name, w in layer.items():
                     ql.linear_q_gemv(w, xs[w.K], None, ql.SCALE_X86_REF, out=ys[name])
             return
-        # from three activation rows on the calls get a workspace: x is then quantized once per call by a small kernel
+        # from three activation rows on the calls get a workspace with room for the partial sums of the K slices
         wk = xs["workspaces"]
         for l in pool:
             ql.linear_q_gemv_multi([l["q_proj"], l["k_proj"], l["v_proj"]], xs[2560], None, ql.SCALE_X86_REF,
@@ -415,7 +417,9 @@ def main():
              for n, d in (("h", 2560), ("q", 4096), ("k", 1024), ("v", 1024), ("o", 2560), ("x1", 2560), ("h2", 2560),
                           ("g", 9728), ("u", 9728), ("s", 9728), ("a", 9728), ("d", 2560), ("x2", 2560))}
         img = {k: ql.gemv_workspace(M, k) for k in (2560, 9728)}
-        ws_o = ql.gemv_workspace(M, 4096)  # o_proj reads the attention output raw: quantized once per launch from three rows on
+        ws_o = ql.gemv_workspace(M, 4096, 2560)  # o_proj reads the attention output raw
+        # room for the partial sums of the K slices (three rows or more: the slices of a row tile are separate workgroups)
+        wsp = {2560: ql.gemv_workspace(M, 2560, 2 * 9728), 9728: ql.gemv_workspace(M, 9728, 2560)} if M >= 3 else {2560: None, 9728: None}
         L = _lib.lib()
 
         def ew(fn, a_, b_, y_):
@@ -444,14 +448,15 @@ def main():
                 st = torch.cuda.current_stream().cuda_stream
                 _lib.check(L.mllm_hip_rmsnorm(x.data_ptr(), 0, nw[0].data_ptr(), b["h"].data_ptr(), M, 2560, 1e-6, 0,
                                               img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
-                ql.linear_q_gemv_fused([l["q_proj"], l["k_proj"], l["v_proj"]], img[2560], M=M, image=True, outs=[b["q"], b["k"], b["v"]])
+                ql.linear_q_gemv_fused([l["q_proj"], l["k_proj"], l["v_proj"]], img[2560], M=M, image=True, outs=[b["q"], b["k"], b["v"]],
+                                       workspace=wsp[2560])
                 ql.linear_q_gemv_fused([l["o_proj"]], attn, residuals=[x], outs=[b["x1"]], workspace=ws_o)
                 _lib.check(L.mllm_hip_rmsnorm(b["x1"].data_ptr(), 0, nw[1].data_ptr(), b["h2"].data_ptr(), M, 2560, 1e-6, 0,
                                               img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
-                ql.linear_q_gemv_fused([l["gate_proj"], l["up_proj"]], img[2560], M=M, image=True, outs=[b["g"], b["u"]])
+                ql.linear_q_gemv_fused([l["gate_proj"], l["up_proj"]], img[2560], M=M, image=True, outs=[b["g"], b["u"]], workspace=wsp[2560])
                 _lib.check(L.mllm_hip_silu_mul(b["g"].data_ptr(), b["u"].data_ptr(), b["a"].data_ptr(), 0, M, 9728,
                                                img[9728].data_ptr(), ql.SCALE_X86_REF, st), "silu_mul")
-                ql.linear_q_gemv_fused([l["down_proj"]], img[9728], M=M, image=True, residuals=[b["x1"]], outs=[b["x2"]])
+                ql.linear_q_gemv_fused([l["down_proj"]], img[9728], M=M, image=True, residuals=[b["x1"]], outs=[b["x2"]], workspace=wsp[9728])
                 x = b["x2"]
 
         def mlp_one_launch():
@@ -460,13 +465,14 @@ def main():
                 st = torch.cuda.current_stream().cuda_stream
                 _lib.check(L.mllm_hip_rmsnorm(x.data_ptr(), 0, nw[0].data_ptr(), b["h"].data_ptr(), M, 2560, 1e-6, 0,
                                               img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
-                ql.linear_q_gemv_fused([l["q_proj"], l["k_proj"], l["v_proj"]], img[2560], M=M, image=True, outs=[b["q"], b["k"], b["v"]])
+                ql.linear_q_gemv_fused([l["q_proj"], l["k_proj"], l["v_proj"]], img[2560], M=M, image=True, outs=[b["q"], b["k"], b["v"]],
+                                       workspace=wsp[2560])
                 ql.linear_q_gemv_fused([l["o_proj"]], attn, residuals=[x], outs=[b["x1"]], workspace=ws_o)
                 _lib.check(L.mllm_hip_rmsnorm(b["x1"].data_ptr(), 0, nw[1].data_ptr(), b["h2"].data_ptr(), M, 2560, 1e-6, 0,
                                               img[2560].data_ptr(), ql.SCALE_X86_REF, st), "rmsnorm")
                 _lib.check(L.mllm_hip_mlp_gate_up_q(l["gate_proj"].wtype, l["gate_proj"].ptr, l["up_proj"].ptr, img[2560].data_ptr(),
                                                     ql.Q8_IMAGE, None, img[9728].data_ptr(), M, 9728, 2560, ql.SCALE_X86_REF, st), "mlp")
-                ql.linear_q_gemv_fused([l["down_proj"]], img[9728], M=M, image=True, residuals=[b["x1"]], outs=[b["x2"]])
+                ql.linear_q_gemv_fused([l["down_proj"]], img[9728], M=M, image=True, residuals=[b["x1"]], outs=[b["x2"]], workspace=wsp[9728])
                 x = b["x2"]
         res = {}
         for name, fn, n in (("operators_one_by_one", plain, 10), ("folded", folded, 7), ("folded_mlp_one_launch", mlp_one_launch, 6)):

@@ -96,6 +96,15 @@ size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K);
 int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M,
                                     int64_t K, int act_scale_mode, void* workspace, void* stream);
 
+/* The same with a workspace of stated size.  With room behind the image for the partial sums of the K slices
+ * (mllm_hip_gemv_splitk_workspace_bytes; N_total = the rows of all parts together) three to eight activation rows take one
+ * launch whose workgroups each quantize only their K slice of x and whose slices meet through the workspace: same results
+ * bit for bit, about two thirds of the time at eight rows.  With less room it is the call above.  Calls that may overlap
+ * on a GPU need workspaces of their own (the first 1024 different workspace addresses per GPU take this form). */
+size_t mllm_hip_gemv_splitk_workspace_bytes(int M, int64_t K, int64_t N_total);
+int mllm_hip_linear_q_gemv_multi_wsn(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M,
+                                     int64_t K, int act_scale_mode, void* workspace, size_t workspace_bytes, void* stream);
+
 /* mllm_hip_linear_q_gemv_multi_ws without a workspace argument and without any allocation.  No counterpart in the
  * reference; it exists for callers that cannot allocate device memory or carry a workspace around: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  The quantized image of the activations lives in a
@@ -118,6 +127,8 @@ typedef struct {
   const float* const* residual;
   void* workspace; /* NULL, or mllm_hip_gemv_workspace_bytes(M, K) bytes for raw activations: as in
                       mllm_hip_linear_q_gemv_multi_ws (same results bit for bit) */
+  size_t workspace_bytes; /* 0 = mllm_hip_gemv_workspace_bytes(M, K); more (mllm_hip_gemv_splitk_workspace_bytes): as in
+                             mllm_hip_linear_q_gemv_multi_wsn, for raw activations and for images alike */
 } mllm_hip_gemv_fusion;
 int mllm_hip_linear_q_gemv_fused(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fusion,
                                  const void* x, int x_kind, int M, int64_t K, int act_scale_mode, void* stream);

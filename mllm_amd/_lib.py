@@ -18,7 +18,7 @@ class GemvPart(C.Structure):
 
 class GemvFusion(C.Structure):
     """mllm_hip_gemv_fusion"""
-    _fields_ = [("residual", C.POINTER(C.c_void_p)), ("workspace", C.c_void_p)]
+    _fields_ = [("residual", C.POINTER(C.c_void_p)), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t)]
 
 
 class HipQLinearError(RuntimeError):
@@ -53,6 +53,9 @@ def lib():
         L.mllm_hip_linear_q_gemv.argtypes = [ci, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_multi_ws.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp, vp]
+        L.mllm_hip_linear_q_gemv_multi_wsn.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp, C.c_size_t, vp]
+        L.mllm_hip_gemv_splitk_workspace_bytes.restype = C.c_size_t
+        L.mllm_hip_gemv_splitk_workspace_bytes.argtypes = [ci, i64, i64]
         L.mllm_hip_linear_q_gemv_multi_static.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_fused.argtypes = [ci, ci, C.POINTER(GemvPart), C.POINTER(GemvFusion), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_mlp_gate_up_q.argtypes = [ci, vp, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]

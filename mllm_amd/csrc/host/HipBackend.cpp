@@ -309,16 +309,18 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
       const int wt = scheme_ == Scheme::kQ4_0 ? MLLM_HIP_Q4_0 : MLLM_HIP_Q8_0;
       if (M <= 8) {  // decode: the GEMV
         const void* image = be.findImage(x.ptr<void>(), (int)M, K);
+        mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
+        // from three rows on: room for the partial sums of the K slices, which lets the rows run as one launch whose
+        // workgroups each quantize (or copy) only their slice of the activations; the library decides
+        const size_t ws_bytes = M >= 3 ? mllm_hip_gemv_splitk_workspace_bytes(8, K, N) : 0;
+        void* ws = ws_bytes ? workspace(ws_bytes) : nullptr;
         if (image) {
-          mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
-          MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_fused(wt, 1, &part, nullptr, image, MLLM_HIP_Q8_IMAGE, (int)M, K,
+          const mllm_hip_gemv_fusion fu{nullptr, ws, ws_bytes};
+          MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_fused(wt, 1, &part, ws ? &fu : nullptr, image, MLLM_HIP_Q8_IMAGE, (int)M, K,
                                                              be.config().act_scale_mode, st));
         } else {
-          // from three rows on the activations are quantized once by a small kernel instead of in every workgroup (when
-          // the launch is large enough for that to pay; the library decides)
-          mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
-          void* ws = M >= 3 ? workspace(mllm_hip_gemv_workspace_bytes(8, K)) : nullptr;
-          MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_multi_ws(wt, 1, &part, x.ptr<void>(), xdt(), (int)M, K, be.config().act_scale_mode, ws, st));
+          MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_q_gemv_multi_wsn(wt, 1, &part, x.ptr<void>(), xdt(), (int)M, K,
+                                                                 be.config().act_scale_mode, ws, ws_bytes, st));
         }
       } else if (!gemm_packed_.isNil()) {
         // (the short-batch entry point cuts K into ranges up to 256 rows and is the plain call beyond)

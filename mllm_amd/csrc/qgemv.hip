@@ -317,9 +317,10 @@ MLLM_API int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void*
 }
 
 static int g_gemv_path = 0;
-// 0: by the number of rows; 1: always the vector-ALU kernel (comparison runs and tests)
+// 0: by the number of rows; 1: always the vector-ALU kernel; 2: as 0 without the K-slices-as-workgroups form of the
+// matrix-core kernel (comparison runs and tests)
 MLLM_API int mllm_hip_gemv_set_path(int path) {
-  if (path != 0 && path != 1) return MLLM_HIP_E_BADARG;
+  if (path != 0 && path != 1 && path != 2) return MLLM_HIP_E_BADARG;
   g_gemv_path = path;
   return 0;
 }
@@ -368,14 +369,23 @@ MLLM_API int mllm_hip_q_prepack(int wtype, const void* blocks, int weight_scale_
   return (int)hipGetLastError();
 }
 
+// the quantized image of one pass of eight rows: 40 bytes per block
+static size_t gemv_image_bytes(int64_t K) { return (size_t)8 * (K / QK) * 40; }
+
 MLLM_API size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K) {
   if (M < 1 || K <= 0 || K % QK) return 0;
-  return (size_t)8 * (K / QK) * 40;  // one pass of eight rows at a time
+  return gemv_image_bytes(K);
+}
+
+// image, then the partial sums of the K slices of one pass of eight rows (each part's rows rounded up to 16)
+MLLM_API size_t mllm_hip_gemv_splitk_workspace_bytes(int M, int64_t K, int64_t N_total) {
+  if (M < 1 || K <= 0 || K % QK || N_total <= 0) return 0;
+  return gemv_image_bytes(K) + (size_t)gemv_mfk_slices((int)(K / QK)) * 8 * (size_t)(N_total + 16 * GEMV_MAX_PARTS) * 4;
 }
 
 // x_kind: MLLM_HIP_F32 / MLLM_HIP_BF16 activations, or MLLM_HIP_Q8_IMAGE: their quantized image (act_scale_mode unused)
 static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual, const void* x,
-                           int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, void* stream);
+                           int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, size_t ws_bytes, void* stream);
 
 // everything that can be refused without touching the device
 static int gemv_check_args(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M, int64_t K,
@@ -395,10 +405,10 @@ static int gemv_check_args(int wtype, int nparts, const mllm_hip_gemv_part* part
 // More than eight rows of raw activations: passes of eight rows, each streaming the weights again (the same arithmetic row by
 // row; up to about 32 rows this is faster than the matrix-core GEMM path, whose 128-row tiles leave most of the chip idle).
 static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fu, const void* x,
-                           int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
+                           int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, size_t ws_bytes, void* stream) {
   const float* const* residual = fu ? fu->residual : nullptr;
   if (M <= 8 || x_dtype == MLLM_HIP_Q8_IMAGE || nparts < 1 || nparts > GEMV_MAX_PARTS || !parts || !x)
-    return gemv_multi_pass(wtype, nparts, parts, residual, x, x_dtype, M, K, act_scale_mode, workspace, stream);
+    return gemv_multi_pass(wtype, nparts, parts, residual, x, x_dtype, M, K, act_scale_mode, workspace, ws_bytes, stream);
   if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
   const size_t xrow = (size_t)K * (x_dtype == MLLM_HIP_F32 ? 4 : 2);
   for (int m0 = 0; m0 < M; m0 += 8) {
@@ -410,14 +420,14 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
       rr[p] = (residual && residual[p]) ? residual[p] + (size_t)m0 * parts[p].N : nullptr;
     }
     const int rc = gemv_multi_pass(wtype, nparts, pp, residual ? rr : nullptr, reinterpret_cast<const char*>(x) + (size_t)m0 * xrow, x_dtype,
-                                   M - m0 < 8 ? M - m0 : 8, K, act_scale_mode, workspace, stream);
+                                   M - m0 < 8 ? M - m0 : 8, K, act_scale_mode, workspace, ws_bytes, stream);
     if (rc) return rc;
   }
   return 0;
 }
 
 static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual, const void* x,
-                           int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
+                           int x_dtype, int M, int64_t K, int act_scale_mode, void* workspace, size_t ws_bytes, void* stream) {
   RC_RET(gemv_check_args(wtype, nparts, parts, x, x_dtype, M, K, act_scale_mode, workspace));
   if (M > 8) return MLLM_HIP_E_SHAPE;
   GemvArgs a{};
@@ -442,8 +452,21 @@ static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* part
   // three or more rows: block sums on the matrix cores (as long as the rows fit that kernel's LDS: 8 rows of 11 000 elements)
   // Q8_0 (twice the code bytes per block) gains only from five rows on.  The rule looks at the weight type, the number of
   // rows and the row length, never at the number of weight rows: a matrix takes the same kernel alone and in a multi launch.
-  if (MT >= 4 && g_gemv_path != 1 && (wtype == MLLM_HIP_Q4_0 || MT == 8) && gemv_mfma_fits(MT, a.nb)) {
-    const int waves = (g_tune_NW == 2 || g_tune_NW == 4 || g_tune_NW == 8) ? g_tune_NW : 0;
+  // Q8_0 with three or four rows is faster on the vector ALU as long as the rows fit its LDS image (40 bytes per block and row)
+  const bool long_rows = (size_t)MT * a.nb * 40 > 140 * 1024;
+  const bool mfma_rows = MT >= 4 && g_gemv_path != 1 && (wtype == MLLM_HIP_Q4_0 || MT == 8 || long_rows);
+  const int waves = (g_tune_NW == 2 || g_tune_NW == 4 || g_tune_NW == 8) ? g_tune_NW : 0;
+  // K slices as separate workgroups, each quantizing only its slice of x (one launch, same bits, no limit on the row length
+  // from LDS): needs room for the slices' partial sums behind the image area of the workspace; falls through where that
+  // room is missing
+  if (mfma_rows && g_gemv_path != 2) {
+    const size_t img = gemv_image_bytes(K);
+    char* part = (workspace && ws_bytes > img) ? reinterpret_cast<char*>(workspace) + img : nullptr;
+    const int rc = launch_gemv_mfk(wtype, x_dtype == MLLM_HIP_Q8_IMAGE ? GEMV_PREQ : x_dtype, MT, a, workspace, part,
+                                   part ? ws_bytes - img : 0, waves, st);
+    if (rc != MFK_NOT_TAKEN) return rc;
+  }
+  if (mfma_rows && gemv_mfma_fits(MT, a.nb)) {
     // quantizing x in every workgroup costs more than one more small launch that quantizes it once: with five to eight rows
     // always (q+k+v of the 4B layer at eight rows: 11.2 us against 7.5 + 2.4), with three or four from about 600 000
     // block-rows on (gate + up, down).  Same bits either way.
@@ -478,7 +501,17 @@ static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* part
 MLLM_API int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,
                                              int M, int64_t K, int act_scale_mode, void* workspace, void* stream) {
   if (x_dtype == MLLM_HIP_Q8_IMAGE) return MLLM_HIP_E_BADARG;
-  return gemv_multi_impl(wtype, nparts, parts, nullptr, x, x_dtype, M, K, act_scale_mode, workspace, stream);
+  return gemv_multi_impl(wtype, nparts, parts, nullptr, x, x_dtype, M, K, act_scale_mode, workspace,
+                         workspace && K > 0 && K % QK == 0 ? gemv_image_bytes(K) : 0, stream);
+}
+
+MLLM_API int mllm_hip_linear_q_gemv_multi_wsn(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,
+                                              int M, int64_t K, int act_scale_mode, void* workspace, size_t workspace_bytes,
+                                              void* stream) {
+  if (x_dtype == MLLM_HIP_Q8_IMAGE) return MLLM_HIP_E_BADARG;
+  if (workspace && K > 0 && K % QK == 0 && workspace_bytes < gemv_image_bytes(K)) return MLLM_HIP_E_SHAPE;
+  return gemv_multi_impl(wtype, nparts, parts, nullptr, x, x_dtype, M, K, act_scale_mode, workspace, workspace ? workspace_bytes : 0,
+                         stream);
 }
 
 // The call above for callers that cannot allocate or pass a workspace: the image lives in the static scratch array of the
@@ -492,12 +525,18 @@ MLLM_API int mllm_hip_linear_q_gemv_multi_static(int wtype, int nparts, const ml
   HIP_RET(hipGetDevice(&dev));
   void* ws = nullptr;
   RC_RET(static_scratch(dev, &ws));
-  return gemv_multi_impl(wtype, nparts, parts, nullptr, x, x_dtype, M, K, act_scale_mode, ws, stream);
+  return gemv_multi_impl(wtype, nparts, parts, nullptr, x, x_dtype, M, K, act_scale_mode, ws, GEMV_STATIC_BYTES, stream);
 }
 
 MLLM_API int mllm_hip_linear_q_gemv_fused(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fusion,
                                           const void* x, int x_kind, int M, int64_t K, int act_scale_mode, void* stream) {
-  return gemv_multi_impl(wtype, nparts, parts, fusion, x, x_kind, M, K, act_scale_mode, fusion ? fusion->workspace : nullptr, stream);
+  void* ws = fusion ? fusion->workspace : nullptr;
+  size_t ws_bytes = 0;
+  if (ws && K > 0 && K % QK == 0) {
+    ws_bytes = fusion->workspace_bytes ? fusion->workspace_bytes : gemv_image_bytes(K);
+    if (ws_bytes < gemv_image_bytes(K)) return MLLM_HIP_E_SHAPE;
+  }
+  return gemv_multi_impl(wtype, nparts, parts, fusion, x, x_kind, M, K, act_scale_mode, ws, ws_bytes, stream);
 }
 
 MLLM_API int mllm_hip_linear_q_gemv_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,

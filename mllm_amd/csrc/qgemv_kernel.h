@@ -407,6 +407,13 @@ int launch_gemv(const GemvArgs& a, int MT, GemvShape s, hipStream_t st) {
 // waves per workgroup: 0 (by x_kind), 4 or 8; K slices per row tile: 0 (by row length), 1, 2 or 4 (sweeps)
 int launch_gemv_mfma(int wtype, int x_kind, int MT, const GemvArgs& a, int waves, int slices, hipStream_t st);
 bool gemv_mfma_fits(int MT, int nb);  // rows of nb blocks fit that kernel's LDS
+// The matrix-core kernel with the K slices as separate workgroups.  image_ws: where a raw x could be quantized first (unused
+// so far); part / part_bytes: room for the slices' partial sums (may be null / 0).  Returns MFK_NOT_TAKEN when the launch
+// does not fit (no room for the partial sums, no free counter block, slices too long): the caller takes another kernel.
+constexpr int MFK_NOT_TAKEN = 1;
+int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a, const void* workspace, void* part, size_t part_bytes, int waves,
+                    hipStream_t st);
+int gemv_mfk_slices(int nb);
 int launch_gemv_q4_f32(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
 int launch_gemv_q4_bf16(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
 int launch_gemv_q8_f32(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);

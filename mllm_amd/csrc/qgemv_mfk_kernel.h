@@ -1,0 +1,352 @@
+// Q4_0 / Q8_0 decode GEMV for three to eight activation rows on the matrix cores, K cut into slices that are separate
+// WORKGROUPS (qgemv_mfma_kernel.h keeps the slices of a row tile inside one workgroup).
+//
+// Same arithmetic and the same order of additions as that kernel (block sums with v_mfma_i32_16x16x64_i8, one fused
+// multiply-add per block into the lane that owns blocks = q mod 4, the four lanes as (0 + 1) + (2 + 3), then the slices
+// in slice order), so both give the same bits.  What differs is who does which part:
+//   * a workgroup holds `nwaves` row tiles of 16 weight rows and ONE K slice of at most 64 blocks.  It quantizes (or copies
+//     from the quantized image) only its slice of the activations: with eight rows of 9728 elements that is 320 blocks per
+//     workgroup instead of 2432, and the LDS footprint no longer grows with K;
+//   * weight codes are requested as 8 rows x 128 contiguous bytes per load instruction (the operand layout of the MFMA,
+//     16 rows x 64 bytes per instruction, measured 25 % slower on the 4B shapes) and turned into the operand layout
+//     through a 2 KB LDS stage that belongs to the wave (no barrier: LDS operations of one wave execute in order);
+//   * the slices of a row tile meet in global memory: every workgroup stores its partial sums, the one that arrives last
+//     at the tile's counter adds them up in slice order, applies bias / residual and stores y.  The counter goes back to
+//     zero, so the counters are zero between launches.
+#pragma once
+#include "qgemv_mfma_kernel.h"
+
+namespace mllmhip {
+
+constexpr int MFK_CH = 6;             // chunks of 8 blocks requested up front per trip
+constexpr int MFK_TRIP = 8 * MFK_CH;
+constexpr int MFK_STG = 16 * 9;       // 16-byte pieces of one stage: 16 rows, stride 9 (reads of 16 rows hit 16 bank groups)
+constexpr int MFK_MAX_NBS = 64;       // blocks per slice (weight scales of a slice: two 16-byte loads per lane)
+
+struct MfkArgs {
+  float* part;         // [S][MT][NP] partial sums (S > 1)
+  unsigned* counters;  // one per workgroup column (blockIdx.x), zero between launches (S > 1)
+  int NP;              // columns of a partial row: every part's rows rounded up to 16
+  int S, nbs;          // K slices; blocks per slice (a multiple of 8, at most MFK_MAX_NBS)
+  int col0[GEMV_MAX_PARTS];  // first column of each part within a partial row
+  int ipr_magic;             // ceil(2^20 / (4 nbs)): item / (items per row) as a multiply and a shift
+};
+
+template <int MT>
+static size_t mfk_lds_bytes(int wtype, int nbs, int nwaves) {
+  const int rs = mf_row_stride(nbs);
+  return ((size_t)2 * MT * rs + nbs) * 16 + (size_t)MT * nbs * 8 +
+         (size_t)nwaves * ((size_t)nbs * 64 + (size_t)MFK_STG * 16 * (wtype == MLLM_HIP_Q8_0 ? 2 : 1)) + 16;
+}
+
+// blockDim = 256 or 512 (four or eight row tiles per workgroup)
+template <int WT, int XT, int MT>
+__global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  constexpr int TH = MT / 4;
+  constexpr int NPL = WT == MLLM_HIP_Q8_0 ? 2 : 1;  // code planes
+  constexpr int XTT = XT == GEMV_PREQ ? MLLM_HIP_BF16 : XT;
+  const int nb = a.nb, nbp = a.nbp, nbs = k.nbs, S = k.S;
+  const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x, nwaves = nthreads >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  int pidx = 0;  // uniform: which matrix this workgroup works on
+#pragma unroll
+  for (int p = 1; p < GEMV_MAX_PARTS; p++)
+    if (p < a.nparts && (int)blockIdx.x >= a.wg_start[p]) pidx = p;
+  const GemvPart& pt = a.part[pidx];
+  const int wg0 = a.wg_start[pidx], pcol0 = k.col0[pidx];
+  const void* const xptr = a.x;
+  const int aM = a.M, x86 = a.x86_scale;
+  float* const kpart = k.part;
+  unsigned* const kcnt = k.counters;
+  const int kNP = k.NP;
+  const int N = pt.N;
+  const int tile = ((int)blockIdx.x - wg0) * nwaves + wave;
+  const int slice = blockIdx.y;
+  const int row0 = tile * 16;
+  const bool tile_ok = row0 < N;
+  const int b0 = slice * nbs, b1 = min(nb, b0 + nbs);  // this workgroup's blocks (possibly none: b1 <= b0)
+
+  const int rs = mf_row_stride(nbs);
+  u32x4* xlo = reinterpret_cast<u32x4*>(smem);  // [MT][rs] codes of elements 0..15 of (row, block of the slice)
+  u32x4* xhi = xlo + (size_t)MT * rs;           // likewise elements 16..31
+  u32x4* zrow = xhi + (size_t)MT * rs;          // [nbs] zeros: the operand of the lane groups that must not contribute
+  u32x2* xs = reinterpret_cast<u32x2*>(zrow + nbs);  // [MT][nbs] {effective scale, -8 * sum}
+  float* ws_all = reinterpret_cast<float*>(xs + (size_t)MT * nbs);
+  float* ws = ws_all + (size_t)wave * nbs * 16;  // per wave [block][16 rows]
+  u32x4* stg_all = reinterpret_cast<u32x4*>(ws_all + (size_t)nwaves * nbs * 16);
+  u32x4* stg = stg_all + (size_t)wave * MFK_STG * NPL;
+  int* s_flag = reinterpret_cast<int*>(stg_all + (size_t)nwaves * MFK_STG * NPL);
+
+  // ---- 1. activation requests (they return first; nothing here divides: the weight requests below must leave early) ------
+  // raw activations: item it = tid + i * blockDim = eight elements, the four lanes of a quad share a block;
+  // image: thread (row tid / 64 + i * nwaves, block tid % 64)
+  const int ipr = nbs * 4;            // items of eight elements per row of the slice
+  const int nitems = MT * ipr;        // item it: row it / ipr, column it % ipr (the quads stay whole: ipr % 4 == 0)
+  XRaw<XTT> raw[MT];
+  const int mnb = MT * nb;
+  const u32x4* img_lo = reinterpret_cast<const u32x4*>(xptr);
+  const u32x4* img_hi = img_lo + mnb;
+  const float* img_d = reinterpret_cast<const float*>(img_hi + mnb);
+  const int* img_n8 = reinterpret_cast<const int*>(img_d + mnb);
+  constexpr int NIMG = MT / 4;
+  const int ib = tid & 63, im = tid >> 6;
+  u32x4 plo[NIMG], phi[NIMG];
+  float pd[NIMG];
+  int pn[NIMG];
+  if (XT == GEMV_PREQ) {
+#pragma unroll
+    for (int i = 0; i < NIMG; i++) {
+      const int it = min(im + i * nwaves, MT - 1) * nb + min(b0 + ib, nb - 1);
+      plo[i] = img_lo[it]; phi[i] = img_hi[it]; pd[i] = img_d[it]; pn[i] = img_n8[it];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < MT; i++) {
+      if (i * nthreads < nitems) {  // uniform
+        const int it = min(tid + i * nthreads, nitems - 1);
+        const int m = (int)(((uint32_t)it * (uint32_t)k.ipr_magic) >> 20), xc = it - m * ipr;
+        // clamped addresses: validity is applied when the values are used
+        load_x8<XTT>(xptr, ((int64_t)min(m, aM - 1) * nb * 4 + min(b0 * 4 + xc, nb * 4 - 1)) * 8, raw[i]);
+      }
+    }
+  }
+
+  // ---- 2. weight scales of the tile and slice: 16-byte pieces of eight, lane (row lane / 8 + 8 i, piece lane % 8) -------
+  const WRsrc wr = make_wrsrc(pt.w, WT, N, nb, nbp);
+  u32x4 sc[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int r = (lane >> 3) + 8 * i, cc = lane & 7;
+    const bool ok = tile_ok && row0 + r < N && 8 * cc < nbs && b0 + 8 * cc < nbp;
+    sc[i] = __builtin_amdgcn_raw_buffer_load_b128(wr.d, ok ? (uint32_t)(((int64_t)(row0 + r) * nbp + b0 + 8 * cc) * 2) : BUF_OOB, 0, BUF_NT);
+  }
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- 3. weight codes of a trip: chunk ch = 8 blocks, instruction i of it = rows 8 i .. 8 i + 7, 128 bytes of each --------
+  const int lr = lane >> 3, lp = lane & 7;
+  u32x4 wq[MFK_CH][2][NPL];
+  auto load_trip = [&](int bb) {
+#pragma unroll
+    for (int ch = 0; ch < MFK_CH; ch++)
+#pragma unroll
+      for (int i = 0; i < 2; i++) {
+        const int r = row0 + 8 * i + lr, b = bb + 8 * ch + lp;
+        const uint32_t off = (tile_ok && r < N && b < b1) ? ((uint32_t)r * (uint32_t)nb + (uint32_t)b) * 16u : BUF_OOB;
+        wq[ch][i][0] = __builtin_amdgcn_raw_buffer_load_b128(wr.q0, off, 0, BUF_NT);
+        if (WT == MLLM_HIP_Q8_0) wq[ch][i][NPL - 1] = __builtin_amdgcn_raw_buffer_load_b128(wr.q1, off, 0, BUF_NT);
+      }
+  };
+  load_trip(b0);
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- 4. the slice of the activations into LDS ------------------------------------------------------------------------
+  if (XT == GEMV_PREQ) {
+#pragma unroll
+    for (int i = 0; i < NIMG; i++) {
+      const int m = im + i * nwaves;
+      if (m < MT && ib < nbs) {
+        const bool live = b0 + ib < nb;  // the image has no blocks past the row
+        xlo[(size_t)m * rs + ib] = live ? plo[i] : u32x4{0u, 0u, 0u, 0u};
+        xhi[(size_t)m * rs + ib] = live ? phi[i] : u32x4{0u, 0u, 0u, 0u};
+        xs[(size_t)m * nbs + ib] = live ? u32x2{__float_as_uint(pd[i]), (uint32_t)pn[i]} : u32x2{0u, 0u};
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < MT; i++) {
+      const int it = tid + i * nthreads;
+      if (it < nitems) {  // whole quads: nitems and nthreads are multiples of 4
+        const int m = (int)(((uint32_t)it * (uint32_t)k.ipr_magic) >> 20), xc = it - m * ipr;
+        float v[8];
+        x8_to_f32<XTT>(raw[i], v);
+        const int b = xc >> 2, j = xc & 3;
+        if (m >= aM || b0 + b >= nb) {
+#pragma unroll
+          for (int e = 0; e < 8; e++) v[e] = 0.f;
+        }
+        uint32_t pk[2];
+        float deff;
+        int n8;
+        quad_quantize(v, x86, pk, deff, n8);
+        u32x2* dst = reinterpret_cast<u32x2*>((j < 2 ? xlo : xhi) + (size_t)m * rs + b) + (j & 1);
+        *dst = u32x2{pk[0], pk[1]};
+        if (j == 0) xs[(size_t)m * nbs + b] = u32x2{__float_as_uint(deff), (uint32_t)n8};
+      }
+    }
+  }
+  for (int i = tid; i < nbs; i += nthreads) zrow[i] = u32x4{0u, 0u, 0u, 0u};
+  // weight scales -> fp32 [block of the slice][row]; blocks past the row are zero
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int r = (lane >> 3) + 8 * i, cc = lane & 7;
+    if (8 * cc < nbs) {
+      const uint32_t wds[4] = {sc[i].x, sc[i].y, sc[i].z, sc[i].w};
+#pragma unroll
+      for (int e = 0; e < 8; e++)
+        ws[(8 * cc + e) * 16 + r] = (b0 + 8 * cc + e < nb) ? f16bits_to_f32((uint16_t)(wds[e >> 1] >> (16 * (e & 1)))) : 0.f;
+    }
+  }
+  __syncthreads();
+
+  // ---- 5. block sums on the matrix cores, scaling on the vector ALU -----------------------------------------------------------
+  // chunk by chunk as the weights arrive: its 8 blocks through the wave's LDS stage into the operand layout, then its two
+  // groups of four blocks with all operands requested before the first instruction issues
+  const int c = lane & 15, g = lane >> 4;        // operand layout: weight row c, block 4 j + g of a group of four
+  const int q = (lane & 15) >> 2, tt = lane & 3;  // this lane's result column: block 4 j + q, activation row 4 h + tt
+  const bool mine = g == q;                      // the lane group that supplies this column's activation codes
+  f32x4 acc[TH];
+#pragma unroll
+  for (int h = 0; h < TH; h++) acc[h] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int bb = b0; bb < b1; bb += MFK_TRIP) {
+    if (bb != b0) load_trip(bb);
+#pragma unroll
+    for (int ch = 0; ch < MFK_CH; ch++) {
+      const int cb = bb + 8 * ch;  // first block of the chunk
+      if (cb >= b1) break;         // uniform
+#pragma unroll
+      for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int p = 0; p < NPL; p++) stg[p * MFK_STG + (8 * i + lr) * 9 + lp] = wq[ch][i][p];
+      u32x4 Aw[2][NPL], Bl[2][TH], Bh[2][TH];
+      u32x2 sx[2][TH];
+      f32x4 dw[2];
+      bool live[2];
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++) {
+        const int lb = cb - b0 + 4 * jj + q;  // this lane's block within the slice (inside the slice's LDS rows even when dead)
+        live[jj] = cb + 4 * jj + q < b1;
+#pragma unroll
+        for (int p = 0; p < NPL; p++) Aw[jj][p] = stg[p * MFK_STG + c * 9 + 4 * jj + g];
+        dw[jj] = *reinterpret_cast<const f32x4*>(ws + lb * 16 + 4 * g);
+#pragma unroll
+        for (int h = 0; h < TH; h++) {
+          const int m = 4 * h + tt;
+          Bl[jj][h] = mine ? xlo[(size_t)m * rs + lb] : zrow[lb];
+          Bh[jj][h] = mine ? xhi[(size_t)m * rs + lb] : zrow[lb];
+          sx[jj][h] = xs[(size_t)m * nbs + lb];
+        }
+      }
+      v4i_t D[2][TH];
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++) {
+        v4i_t Al, Ah;
+        if (WT == MLLM_HIP_Q4_0) {
+          const u32x4 w = Aw[jj][0];
+          Al = v4i_t{(int)(w.x & 0x0f0f0f0fu), (int)(w.y & 0x0f0f0f0fu), (int)(w.z & 0x0f0f0f0fu), (int)(w.w & 0x0f0f0f0fu)};
+          Ah = v4i_t{(int)((w.x >> 4) & 0x0f0f0f0fu), (int)((w.y >> 4) & 0x0f0f0f0fu), (int)((w.z >> 4) & 0x0f0f0f0fu),
+                     (int)((w.w >> 4) & 0x0f0f0f0fu)};
+        } else {
+          Al = __builtin_bit_cast(v4i_t, Aw[jj][0]);
+          Ah = __builtin_bit_cast(v4i_t, Aw[jj][NPL - 1]);
+        }
+#pragma unroll
+        for (int h = 0; h < TH; h++) {
+          const v4i_t d = __builtin_amdgcn_mfma_i32_16x16x64_i8(Al, __builtin_bit_cast(v4i_t, Bl[jj][h]), v4i_t{0, 0, 0, 0}, 0, 0, 0);
+          D[jj][h] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ah, __builtin_bit_cast(v4i_t, Bh[jj][h]), d, 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+        for (int h = 0; h < TH; h++) {
+          const float dx = live[jj] ? __uint_as_float(sx[jj][h].x) : 0.f;
+          const int n8 = WT == MLLM_HIP_Q4_0 ? (int)sx[jj][h].y : 0;  // nibbles are unsigned: sum((q - 8) x) = sum(q x) - 8 sum(x)
+          acc[h].x = fmaf(dw[jj].x * dx, (float)(D[jj][h].x + n8), acc[h].x);
+          acc[h].y = fmaf(dw[jj].y * dx, (float)(D[jj][h].y + n8), acc[h].y);
+          acc[h].z = fmaf(dw[jj].z * dx, (float)(D[jj][h].z + n8), acc[h].z);
+          acc[h].w = fmaf(dw[jj].w * dx, (float)(D[jj][h].w + n8), acc[h].w);
+        }
+    }
+  }
+  // the four lanes of an activation row (blocks = 0, 1, 2, 3 mod 4): (0 + 1) + (2 + 3) on every lane
+#pragma unroll
+  for (int h = 0; h < TH; h++) {
+    float v[4] = {acc[h].x, acc[h].y, acc[h].z, acc[h].w};
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      v[e] += __shfl_xor(v[e], 4, 64);
+      v[e] += __shfl_xor(v[e], 8, 64);
+    }
+    acc[h] = f32x4{v[0], v[1], v[2], v[3]};
+  }
+
+  const int n = row0 + 4 * g;  // lanes with q == 0 hold rows n .. n + 3 of activation row 4 h + tt
+  if (S == 1) {
+    if (!tile_ok || q != 0) return;
+#pragma unroll
+    for (int h = 0; h < TH; h++) {
+      const int t = 4 * h + tt;
+      if (t >= aM) continue;
+      const float v[4] = {acc[h].x, acc[h].y, acc[h].z, acc[h].w};
+      float* yrow = pt.y + (int64_t)t * N;
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        if (n + e < N) {
+          float o = v[e];
+          if (pt.bias) o = pt.bias[n + e] + o;
+          if (pt.residual) o = o + pt.residual[(int64_t)t * N + n + e];
+          yrow[n + e] = o;
+        }
+      }
+    }
+    return;
+  }
+
+  // ---- 6. the slices of a tile meet in global memory ------------------------------------------------------------------------------
+  // Partial sums leave with device-scope stores (written through this chip-let's L2); the barrier makes every wave wait until
+  // its stores are acknowledged; then thread 0 counts the workgroup in.  A release fence in every wave (or even one per
+  // workgroup) makes the hardware look through the whole L2 for dirty lines and cost 5 to 50 us per launch; nothing but these
+  // stores has to be visible to the workgroup that arrives last, and it reads them with device-scope loads.
+  const int col = pcol0 + n;
+  if (tile_ok && q == 0) {
+#pragma unroll
+    for (int h = 0; h < TH; h++) {
+      float* dst = kpart + ((size_t)slice * MT + 4 * h + tt) * kNP + col;
+      __hip_atomic_store(dst + 0, acc[h].x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(dst + 1, acc[h].y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(dst + 2, acc[h].z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(dst + 3, acc[h].w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    const unsigned old = atomicAdd(kcnt + blockIdx.x, 1u);
+    const int last = old == (unsigned)(S - 1);
+    if (last) kcnt[blockIdx.x] = 0u;  // every slice has arrived: ready for the next launch
+    *s_flag = last;
+  }
+  __syncthreads();
+  if (!*s_flag || !tile_ok) return;
+  // the workgroup that arrived last: lane l of a wave sums outputs (activation row l / 16 + 4 i, weight row l % 16) of its
+  // tile over the slices, slice 0 first; the loads of up to eight slices are in flight together
+  const int r = lane & 15;
+#pragma unroll
+  for (int i = 0; i < TH; i++) {
+    const int t = (lane >> 4) + 4 * i;
+    const float* src = kpart + (size_t)t * kNP + pcol0 + row0 + r;
+    const size_t sstride = (size_t)MT * kNP;
+    float sum = 0.f;
+    for (int s0 = 0; s0 < S; s0 += 8) {
+      float pv[8];
+#pragma unroll
+      for (int u = 0; u < 8; u++)
+        pv[u] = __hip_atomic_load(src + (size_t)min(s0 + u, S - 1) * sstride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        if (s0 + u == 0) sum = pv[0];
+        else if (s0 + u < S) sum += pv[u];
+      }
+    }
+    if (t < aM && row0 + r < N) {
+      float o = sum;
+      if (pt.bias) o = pt.bias[row0 + r] + o;
+      if (pt.residual) o = o + pt.residual[(int64_t)t * N + row0 + r];
+      pt.y[(int64_t)t * N + row0 + r] = o;
+    }
+  }
+}
+
+}  // namespace mllmhip

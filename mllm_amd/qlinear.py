@@ -90,9 +90,13 @@ def linear_q_gemv(w, x, bias=None, act_scale_mode=SCALE_X86_REF, out=None):
     return y
 
 
-def gemv_workspace(M, K):
-    """Workspace for linear_q_gemv_multi with three or more activation rows."""
-    return torch.empty(_lib.lib().mllm_hip_gemv_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+def gemv_workspace(M, K, n_total=None):
+    """Workspace for linear_q_gemv_multi with three or more activation rows (also the size of a quantized image of x).
+    n_total = rows of all weight matrices of a launch together: room for the partial sums of the K slices as well, which
+    lets three to eight rows run as one launch."""
+    L = _lib.lib()
+    size = L.mllm_hip_gemv_workspace_bytes(M, K) if n_total is None else L.mllm_hip_gemv_splitk_workspace_bytes(M, K, n_total)
+    return torch.empty(size, dtype=torch.uint8, device="cuda")
 
 
 def linear_q_gemv_multi(ws, x, biases=None, act_scale_mode=SCALE_X86_REF, outs=None, workspace=None):
@@ -107,9 +111,10 @@ def linear_q_gemv_multi(ws, x, biases=None, act_scale_mode=SCALE_X86_REF, outs=N
         assert w.K == K and w.wtype == ws[0].wtype
         b = biases[i] if biases is not None else None
         parts[i] = _lib.GemvPart(w.ptr, b.data_ptr() if b is not None else None, outs[i].data_ptr(), w.N)
-    _lib.check(_lib.lib().mllm_hip_linear_q_gemv_multi_ws(ws[0].wtype, len(ws), parts, x.data_ptr(), _xdtype(x), M, K,
-                                                          act_scale_mode, _p(workspace), _stream()),
-               "mllm_hip_linear_q_gemv_multi_ws")
+    _lib.check(_lib.lib().mllm_hip_linear_q_gemv_multi_wsn(ws[0].wtype, len(ws), parts, x.data_ptr(), _xdtype(x), M, K,
+                                                           act_scale_mode, _p(workspace),
+                                                           workspace.numel() if workspace is not None else 0, _stream()),
+               "mllm_hip_linear_q_gemv_multi_wsn")
     return outs
 
 
@@ -138,7 +143,7 @@ def linear_q_gemv_fused(ws, x, M=None, biases=None, residuals=None, act_scale_mo
         if r is not None:
             assert r.dtype == torch.float32 and r.is_contiguous() and tuple(r.shape) == (M, w.N)
         res[i] = r.data_ptr() if r is not None else None
-    fu = _lib.GemvFusion(res if residuals is not None else None, _p(workspace))
+    fu = _lib.GemvFusion(res if residuals is not None else None, _p(workspace), workspace.numel() if workspace is not None else 0)
     _lib.check(_lib.lib().mllm_hip_linear_q_gemv_fused(ws[0].wtype, len(ws), parts, C.byref(fu), x.data_ptr(),
                                                        Q8_IMAGE if image else _xdtype(x), M, K, act_scale_mode, _stream()),
                "mllm_hip_linear_q_gemv_fused")

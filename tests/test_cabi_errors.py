@@ -35,6 +35,10 @@ def _cases():
                                           (6, 40, SHAPE), (3, ODD, ALIGN)]),
         "mllm_hip_linear_q_gemv_multi_ws": ([Q8_0, 1, part, P, BF16, 4, 64, 0, P, None],
                                             [(3, None, BADARG), (6, 40, SHAPE), (8, ODD, ALIGN)]),
+        # the workspace of stated size: one smaller than the image of eight rows is refused
+        "mllm_hip_linear_q_gemv_multi_wsn": ([Q8_0, 1, part, P, BF16, 4, 64, 0, P, 8 * 2 * 40, None],
+                                             [(3, None, BADARG), (4, IMAGE, BADARG), (6, 40, SHAPE), (8, ODD, ALIGN),
+                                              (9, 8 * 2 * 40 - 1, SHAPE)]),
         # the variant that allocates nothing: rows longer than its static array hold are refused
         "mllm_hip_linear_q_gemv_multi_static": ([Q8_0, 1, part, P, BF16, 4, 64, 0, None],
                                                 [(3, None, BADARG), (4, IMAGE, BADARG), (6, 32768 + 32, SHAPE), (6, 40, SHAPE)]),

@@ -303,7 +303,77 @@ def test_gemv_matrix_core_and_vector_kernels_agree(wtype, M):
             assert L.mllm_hip_gemv_set_path(0) == 0
         assert rel_l2(y0.cpu().numpy(), y1.cpu().numpy()) < 2e-6
         assert rel_l2(y0.cpu().numpy(), orc.linear_q(xf, W, wtype, bias.cpu().numpy(), orc.SCALE_X86_REF)) < 2e-6
-    assert L.mllm_hip_gemv_set_path(2) == -1
+    assert L.mllm_hip_gemv_set_path(3) == -1
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M", [3, 4, 5, 8])
+def test_gemv_k_slices_as_workgroups_give_the_same_bits(wtype, M):
+    """With room for partial sums in the workspace the K slices of a row tile are separate workgroups that meet through
+    global memory (one launch, every workgroup quantizes its slice of x).  Same partial sums added in the same order as the
+    form that keeps the slices in one workgroup (path 2), so the outputs must be equal bit for bit: fp32 and bf16
+    activations, both scale modes, bias, several matrices per launch, ragged N, rows whose last slice is empty (161 blocks),
+    one to eight slices; and against the oracle."""
+    rng = synth.rng_for(1, 900 + M + 10 * wtype)
+    L = _lib.lib()
+    for shapes in ([(9728, 2560), (9728, 2560)], [(2560, 9728)], [(4096, 2560), (1024, 2560), (1024, 2560)], [(2560, 4096)],
+                   [(40, 96), (7, 96), (33, 96)], [(65, 32)], [(50, 161 * 32)], [(129, 41 * 32), (16, 41 * 32)],
+                   # the longest rows the one-workgroup matrix-core kernel holds (two trips per slice at four rows)
+                   [(31, (512 if M <= 4 else 320) * 32)]):
+        K = shapes[0][1]
+        Ws = [synth.make_weight(rng, wtype, n, K) for n, _ in shapes]
+        ws = [ql.PackedQWeight(wtype, torch.from_numpy(W)) for W in Ws]
+        biases = [to_dev(rng.standard_normal(n).astype(np.float32)) for n, _ in shapes]
+        x = synth.make_x_fp32(rng, M, K)
+        wsp = ql.gemv_workspace(M, K, sum(n for n, _ in shapes))
+        announce("gemv k slices as workgroups", wtype, M, shapes)
+        for xd in (to_dev(x), bf16_dev(synth.fp32_to_bf16_bits(x))):
+            for mode in (ql.SCALE_X86_REF, ql.SCALE_IEEE):
+                assert L.mllm_hip_gemv_set_path(2) == 0
+                try:
+                    one_wg = ql.linear_q_gemv_multi(ws, xd, biases, mode, workspace=wsp)
+                finally:
+                    assert L.mllm_hip_gemv_set_path(0) == 0
+                for rep in range(2):  # twice: the arrival counters must be back at zero after a launch
+                    outs = [torch.full((M, n), float("nan"), device="cuda") for n, _ in shapes]
+                    ql.linear_q_gemv_multi(ws, xd, biases, mode, outs=outs, workspace=wsp)
+                    for f, p in zip(one_wg, outs):
+                        assert torch.equal(f, p)
+        # residual added in the epilogue, and the quantized image as input
+        xd = to_dev(x)
+        res = [to_dev(rng.standard_normal((M, n)).astype(np.float32)) for n, _ in shapes]
+        _, img = ql.add(xd, torch.zeros_like(xd), want_image=True)
+        assert L.mllm_hip_gemv_set_path(2) == 0
+        try:
+            r0 = ql.linear_q_gemv_fused(ws, xd, biases=biases, residuals=res, workspace=wsp)
+        finally:
+            assert L.mllm_hip_gemv_set_path(0) == 0
+        r1 = ql.linear_q_gemv_fused(ws, xd, biases=biases, residuals=res, workspace=wsp)
+        r2 = ql.linear_q_gemv_fused(ws, img, M=M, image=True, biases=biases, residuals=res, workspace=wsp)
+        for f, p, i in zip(r0, r1, r2):
+            assert torch.equal(f, p) and torch.equal(f, i)
+        want = orc.linear_q(x, Ws[0], wtype, biases[0].cpu().numpy(), orc.SCALE_X86_REF)
+        got = ql.linear_q_gemv_multi(ws, to_dev(x), biases, ql.SCALE_X86_REF, workspace=wsp)[0].cpu().numpy()
+        assert rel_l2(got, want) < 2e-6
+    assert L.mllm_hip_gemv_splitk_workspace_bytes(8, 9728, 2560) == 8 * 304 * 40 + 8 * 8 * (2560 + 64) * 4
+    assert L.mllm_hip_gemv_splitk_workspace_bytes(8, 96, 100) == 8 * 3 * 40 + 1 * 8 * (100 + 64) * 4
+    assert L.mllm_hip_gemv_splitk_workspace_bytes(0, 96, 100) == 0
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M", [4, 8])
+def test_gemv_k_slices_as_workgroups_take_rows_of_any_length(wtype, M):
+    """rows beyond what the one-workgroup kernels hold in LDS (eight rows: about 11 000 elements): the slice form has no such
+    limit; against the oracle"""
+    rng = synth.rng_for(1, 950 + M + 10 * wtype)
+    for N, K in ((31, 512 * 32), (20, 1030 * 32)):
+        W = synth.make_weight(rng, wtype, N, K)
+        w = ql.PackedQWeight(wtype, torch.from_numpy(W))
+        x = synth.make_x_fp32(rng, M, K)
+        bias = rng.standard_normal(N).astype(np.float32)
+        announce("gemv long rows", wtype, M, N, K)
+        (got,) = ql.linear_q_gemv_multi([w], to_dev(x), [to_dev(bias)], ql.SCALE_X86_REF, workspace=ql.gemv_workspace(M, K, N))
+        assert rel_l2(got.cpu().numpy(), orc.linear_q(x, W, wtype, bias, orc.SCALE_X86_REF)) < 2e-6
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
