@@ -35,6 +35,8 @@ struct RouteOut {
   int* ntiles;       // [1]
 };
 
+// GROUPED: an expert's tiles are neighbours in the list (full tiles, then its partial tile); otherwise all full tiles come first
+template <bool GROUPED = false>
 __device__ __forceinline__ void moe_route_body(const int32_t* __restrict__ ids, int n, int E, int tile_h, const RouteOut& o, int* s_cnt) {
   // s_cnt: [E] counts, [E] cursors, [E] scan scratch x 3
   int* s_cur = s_cnt + E;
@@ -70,7 +72,7 @@ __device__ __forceinline__ void moe_route_body(const int32_t* __restrict__ ids, 
     if (lane == 0) s_tot[wave] = run;
   }
   __syncthreads();
-  // tile list, full tiles first so that the long-running workgroups start early
+  // tile list, full tiles first so that the long-running workgroups start early (GROUPED: expert by expert)
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
     const int c = s_cnt[e], base = s_off[e];
     o.counts[e] = c;
@@ -78,13 +80,13 @@ __device__ __forceinline__ void moe_route_body(const int32_t* __restrict__ ids, 
     s_cur[e] = base;
     const int nf = c / tile_h;
     for (int t = 0; t < nf; t++) {
-      const int slot = s_full[e] + t;
+      const int slot = s_full[e] + t + (GROUPED ? s_part[e] : 0);
       o.tile_expert[slot] = e;
       o.tile_row0[slot] = base + t * tile_h;
       o.tile_rows[slot] = tile_h;
     }
     if (c % tile_h) {
-      const int slot = s_tot[1] + s_part[e];
+      const int slot = GROUPED ? s_full[e] + nf + s_part[e] : s_tot[1] + s_part[e];
       o.tile_expert[slot] = e;
       o.tile_row0[slot] = base + nf * tile_h;
       o.tile_rows[slot] = c % tile_h;
@@ -1276,14 +1278,23 @@ constexpr int QX_DOWN_TN = 2;  // column tiles per wave in the one-matrix mode
 template <int WT, int MODE>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void qx_kernel(QXArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
-  const int t = blockIdx.x;
-  if (t >= min(a.ntiles[0], (int)gridDim.x)) return;
+  // Work item w = (column block, tile), tiles in list order (an expert's tiles are neighbours).  Workgroup L runs on XCD
+  // L % 8, and every XCD has its own L2: XCD x takes a contiguous eighth of the work items, so that the tiles
+  // of one expert and column block -- which read the same weights -- run on one XCD at about the same time and the weights
+  // come from memory once instead of once per tile.
+  const int nt = min(a.ntiles[0], (int)gridDim.x), ny = (int)gridDim.y;
+  const int L = (int)(blockIdx.x + gridDim.x * blockIdx.y);
+  const int nw = nt * ny, base = nw >> 3, rem = nw & 7;  // XCD x takes base + (x < rem) items
+  const int xcd = L & 7, seq = L >> 3;
+  if (seq >= base + (xcd < rem)) return;
+  const int w = xcd * base + min(xcd, rem) + seq;
+  const int by = w / nt, t = w - by * nt;
   const int e = a.tile_expert[t], row0 = a.tile_row0[t], rows = a.tile_rows[t];
   if constexpr (MODE == 1) {
-    const int n0 = blockIdx.y * 128;
+    const int n0 = by * 128;
     qx_tile<WT, 2, 1, 1>(a, e, row0, rows, n0, smem);
   } else {
-    const int n0 = blockIdx.y * (128 * QX_DOWN_TN);
+    const int n0 = by * (128 * QX_DOWN_TN);
     qx_tile<WT, 1, 1, QX_DOWN_TN>(a, e, row0, rows, n0, smem);
   }
 }
@@ -1340,7 +1351,7 @@ __global__ __launch_bounds__(1024) void qx_prepare_kernel(const int32_t* __restr
                                                           uint32_t* __restrict__ xd, int64_t nblocks, int nb, int x86_scale) {
   extern __shared__ int s_route[];
   if (blockIdx.x == 0) {
-    moe_route_body(ids, n, E, tile_h, o, s_route);
+    moe_route_body<true>(ids, n, E, tile_h, o, s_route);
     return;
   }
   const int64_t i = (int64_t)(blockIdx.x - 1) * 1024 + threadIdx.x;
