@@ -393,12 +393,15 @@ def main():
         if name == "gate_proj":
             sets += [[layer["up_proj"]] for layer in pool]
 
+        # three rows or more: with the workspace the step uses (room for the partial sums of the K slices)
+        wsp = ql.gemv_workspace(M, k, sum(shapes[g][0] for g in groups)) if M >= 3 else None
+
         def fn():
             for ws in sets:
-                if len(ws) == 1:
+                if len(ws) == 1 and wsp is None:
                     ql.linear_q_gemv(ws[0], x, None, ql.SCALE_X86_REF, out=ys[0])
                 else:
-                    ql.linear_q_gemv_multi(ws, x, None, ql.SCALE_X86_REF, ys)
+                    ql.linear_q_gemv_multi(ws, x, None, ql.SCALE_X86_REF, ys, workspace=wsp)
         replay = graphed(fn)
         _, ev = timed(replay, reps, 2)
         per = ev / (reps * len(sets))
