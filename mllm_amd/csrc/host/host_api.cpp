@@ -108,6 +108,23 @@ extern "C" __attribute__((visibility("default"))) int64_t mllm_hip_host_file_ten
   }
   return (int64_t)t.bytes();
 }
+// The two ways of reading a model file: 1 when, read with mmap = true, the tensor is a view into the file's mapping (nothing
+// copied) AND holds the same bytes as the copy that mmap = false reads; 0 otherwise, -1 if the name is missing.
+extern "C" __attribute__((visibility("default"))) int mllm_hip_host_file_tensor_is_mapped_view(const char* path, int version,
+                                                                                               const char* name) {
+  initializeContext();
+  auto mapped = load(path, static_cast<ModelFileVersion>(version), kCPU, true);
+  auto copied = load(path, static_cast<ModelFileVersion>(version), kCPU, false);
+  if (!mapped->has(name) || !copied->has(name)) return -1;
+  Tensor a = mapped->pull(name), b = copied->pull(name);
+  const auto& mf = mapped->getMappedFile();
+  if (!mf || copied->getMappedFile()) return 0;
+  const char* p = a.ptr<char>();
+  const char* base = static_cast<const char*>(mf->data());
+  const bool inside = p >= base && p + a.bytes() <= base + mf->size();
+  const bool outside = !(b.ptr<char>() >= base && b.ptr<char>() < base + mf->size());
+  return inside && outside && a.bytes() == b.bytes() && std::memcmp(p, b.ptr<void>(), a.bytes()) == 0 ? 1 : 0;
+}
 // read in one version, write in another; returns the tensor count
 extern "C" __attribute__((visibility("default"))) int mllm_hip_host_file_convert(const char* in_path, int in_version, const char* out_path,
                                                                                  int out_version) {

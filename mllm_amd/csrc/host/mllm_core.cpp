@@ -2,6 +2,11 @@
 #include "mllm_core.hpp"
 
 #include <cstring>
+#include <fcntl.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
 #include <fstream>
 
 #include <dlfcn.h>
@@ -280,21 +285,19 @@ Tensor readTensor(std::ifstream& f, const std::string& name, const Tensor::shape
 }
 }  // namespace
 
-ParameterFile::ptr_t load(const std::string& file_name, ModelFileVersion version, DeviceTypes map_2_device, bool /*mmap*/) {
-  if (map_2_device != kCPU || (version != ModelFileVersion::kV1 && version != ModelFileVersion::kV2))
-    return ParameterFile::create();  // "return empty if not match all" (mllm/mllm.cpp:142-143)
-  std::ifstream f(file_name, std::ios::binary);
-  if (!f.is_open()) MLLM_ERROR_EXIT(ExitCode::kIOError, "Failed to open file for reading: %s", file_name.c_str());
-  auto pf = ParameterFile::create(version);
+// The parsing is the same for a mapped file and for one that is read tensor by tensor: `bytes(offset, n)` hands out the
+// descriptor bytes, `tensor(...)` makes the tensor (a view into the mapping, or a copy read from the stream).
+template <typename Bytes, typename MakeTensor>
+static void parseModelFile(const std::string& file_name, ModelFileVersion version, const ParameterFile::ptr_t& pf, Bytes&& bytes,
+                           MakeTensor&& tensor) {
   if (version == ModelFileVersion::kV1) {
     int32_t magic = 0;
     uint64_t desc_bytes = 0;
-    f.read(reinterpret_cast<char*>(&magic), 4);
-    f.read(reinterpret_cast<char*>(&desc_bytes), 8);
+    bytes(0, 4, &magic);
+    bytes(4, 8, &desc_bytes);
     MLLM_RT_ASSERT_EQ(kV1Magic, magic);
     std::vector<char> buf(desc_bytes);
-    f.read(buf.data(), (std::streamsize)desc_bytes);
-    if (!f) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
+    bytes(12, desc_bytes, buf.data());
     struct Item { std::string name; uint64_t len, offset; int32_t dtype; };
     std::vector<Item> items;
     for (size_t pos = 0; pos < buf.size();) {
@@ -311,24 +314,78 @@ ParameterFile::ptr_t load(const std::string& file_name, ModelFileVersion version
     for (const auto& it : items) {
       const auto dtype = static_cast<DataTypes>(it.dtype);
       const Tensor::shape_t shape = {(int32_t)(it.len / bytesOfType(dtype) * lanesOfType(dtype))};  // flat, as the reference
-      pf->push(it.name, readTensor(f, it.name, shape, dtype, it.offset, it.len));
+      pf->push(it.name, tensor(it.name, shape, dtype, it.offset, it.len));
     }
   } else {
     V2Header h{};
-    f.read(reinterpret_cast<char*>(&h), sizeof(h));
+    bytes(0, sizeof(h), &h);
     MLLM_RT_ASSERT_EQ(kV2Magic, h.magic_number);
     MLLM_RT_ASSERT_EQ(kV2Version, h.version);
     std::vector<V2Param> descs(h.num_params);
-    f.seekg((std::streamoff)h.params_desc_offset, std::ios::beg);  // an extra data segment in front of it is skipped
-    f.read(reinterpret_cast<char*>(descs.data()), (std::streamsize)(descs.size() * sizeof(V2Param)));
-    if (!f) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
+    bytes(h.params_desc_offset, descs.size() * sizeof(V2Param), descs.data());  // an extra data segment in front of it is skipped
     for (const auto& d : descs) {
       const std::string name(d.name, strnlen(d.name, sizeof(d.name)));
       MLLM_RT_ASSERT(d.shape_len <= kV2ShapeLen);
       Tensor::shape_t shape(d.shape, d.shape + d.shape_len);
-      pf->push(name, readTensor(f, name, shape, static_cast<DataTypes>(d.parameter_type), d.parameter_offset, d.parameter_size));
+      pf->push(name, tensor(name, shape, static_cast<DataTypes>(d.parameter_type), d.parameter_offset, d.parameter_size));
     }
   }
+  (void)file_name;
+}
+
+MappedFile::MappedFile(const std::string& filename) {
+  fd_ = ::open(filename.c_str(), O_RDONLY);
+  if (fd_ < 0) MLLM_ERROR_EXIT(ExitCode::kIOError, "Failed to open file for reading: %s", filename.c_str());
+  struct stat st {};
+  if (::fstat(fd_, &st) != 0 || st.st_size <= 0) MLLM_ERROR_EXIT(ExitCode::kIOError, "Failed to stat file: %s", filename.c_str());
+  size_ = (size_t)st.st_size;
+  mapping_ = ::mmap(nullptr, size_, PROT_READ, MAP_PRIVATE, fd_, 0);
+  if (mapping_ == MAP_FAILED) MLLM_ERROR_EXIT(ExitCode::kIOError, "Failed to map file: %s", filename.c_str());
+}
+MappedFile::~MappedFile() {
+  if (mapping_ && mapping_ != MAP_FAILED) ::munmap(mapping_, size_);
+  if (fd_ >= 0) ::close(fd_);
+}
+
+// mmap = true (the reference's default, mllm/mllm.hpp:210-211; mllm/core/ParameterFile.cpp:68-116): tensors are views into
+// the read-only mapping -- nothing is copied into host memory, pages come in when the upload reads them, and the
+// ParameterFile keeps the mapping alive.  mmap = false reads every tensor into memory of its own.
+ParameterFile::ptr_t load(const std::string& file_name, ModelFileVersion version, DeviceTypes map_2_device, bool mmap) {
+  if (map_2_device != kCPU || (version != ModelFileVersion::kV1 && version != ModelFileVersion::kV2))
+    return ParameterFile::create();  // "return empty if not match all" (mllm/mllm.cpp:142-143)
+  auto pf = ParameterFile::create(version);
+  if (mmap) {
+    auto mf = MappedFile::create(file_name);
+    pf->setMappedFile(mf);
+    char* base = static_cast<char*>(mf->data());
+    const size_t size = mf->size();
+    parseModelFile(
+        file_name, version, pf,
+        [&](uint64_t off, uint64_t n, void* dst) {
+          if (off + n > size) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
+          std::memcpy(dst, base + off, n);
+        },
+        [&](const std::string& name, const Tensor::shape_t& shape, DataTypes dtype, uint64_t offset, uint64_t stored_bytes) {
+          Tensor t = Tensor::fromExternal(base + offset, shape, dtype, kCPU);
+          MLLM_RT_ASSERT(stored_bytes >= t.bytes());
+          if (offset + t.bytes() > size) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: tensor '%s' is truncated", name.c_str());
+          t.setName(name);
+          return t;
+        });
+    return pf;
+  }
+  std::ifstream f(file_name, std::ios::binary);
+  if (!f.is_open()) MLLM_ERROR_EXIT(ExitCode::kIOError, "Failed to open file for reading: %s", file_name.c_str());
+  parseModelFile(
+      file_name, version, pf,
+      [&](uint64_t off, uint64_t n, void* dst) {
+        f.seekg((std::streamoff)off, std::ios::beg);
+        f.read(static_cast<char*>(dst), (std::streamsize)n);
+        if (!f) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
+      },
+      [&](const std::string& name, const Tensor::shape_t& shape, DataTypes dtype, uint64_t offset, uint64_t stored_bytes) {
+        return readTensor(f, name, shape, dtype, offset, stored_bytes);
+      });
   return pf;
 }
 

@@ -132,6 +132,25 @@ class Tensor {
   std::string name_;
 };
 
+// A model file mapped read-only into the address space (mllm/core/MappedFile.hpp:21-44): tensors of a ParameterFile read
+// with mmap = true point into the mapping, which the ParameterFile keeps alive.
+class MappedFile {
+ public:
+  using ptr_t = std::shared_ptr<MappedFile>;
+  explicit MappedFile(const std::string& filename);
+  static ptr_t create(const std::string& filename) { return std::make_shared<MappedFile>(filename); }
+  ~MappedFile();
+  MappedFile(const MappedFile&) = delete;
+  MappedFile& operator=(const MappedFile&) = delete;
+  [[nodiscard]] void* data() const { return mapping_; }
+  [[nodiscard]] size_t size() const { return size_; }
+
+ private:
+  int fd_ = -1;
+  size_t size_ = 0;
+  void* mapping_ = nullptr;
+};
+
 class ParameterFile {
  public:
   using ptr_t = std::shared_ptr<ParameterFile>;
@@ -142,9 +161,12 @@ class ParameterFile {
   [[nodiscard]] bool has(const std::string& name) const { return data_.count(name) != 0; }
   [[nodiscard]] ModelFileVersion version() const { return version_; }
   [[nodiscard]] const std::map<std::string, Tensor>& dict() const { return data_; }
+  void setMappedFile(const MappedFile::ptr_t& f) { mapped_file_ = f; }  // mllm/core/ParameterFile.cpp:75-78
+  [[nodiscard]] const MappedFile::ptr_t& getMappedFile() const { return mapped_file_; }
 
  private:
   ModelFileVersion version_;
+  MappedFile::ptr_t mapped_file_;
   std::map<std::string, Tensor> data_;
 };
 
@@ -407,7 +429,7 @@ void initializeContext();                       // registers the host (CPU) allo
 // ModelFileV2.hpp:40-62 (magic 0x519A, version 2; 352-byte descriptors with dtype, size, offset, shape, name).
 // Tensors come back as host tensors that own their memory; `mmap` is accepted and ignored (always a buffered read).
 ParameterFile::ptr_t load(const std::string& file_name, ModelFileVersion version = ModelFileVersion::kV1,
-                          DeviceTypes map_2_device = kCPU, bool mmap = false);
+                          DeviceTypes map_2_device = kCPU, bool mmap = true);
 void save(const std::string& file_name, const ParameterFile::ptr_t& parameter_file,
           ModelFileVersion version = ModelFileVersion::kV1, DeviceTypes map_2_device = kCPU);
 void loadOpPackage(const std::string& path);    // dlopen + opPackageDescriptor(): mllm/backends/base/PluginSystem.cpp:37-90

@@ -232,6 +232,11 @@ def test_model_file_readers_and_writers(tmp_path):
     assert _file_tensor(L, p2, 2, "no.such.tensor") is None
     # library-side conversion, parsed independently here
     c2, c1 = str(tmp_path / "c2.mllm"), str(tmp_path / "c1.mllm")
+    # read with mmap (the reference's default) the tensors are views into the mapping, with the bytes a plain read gives
+    for path, version in ((p1, 1), (p2, 2)):
+        for tname, _, _, _ in tensors:
+            assert L.mllm_hip_host_file_tensor_is_mapped_view(path.encode(), version, tname.encode()) == 1
+        assert L.mllm_hip_host_file_tensor_is_mapped_view(path.encode(), version, b"no.such.tensor") == -1
     assert L.mllm_hip_host_file_convert(p1.encode(), 1, c2.encode(), 2) == 3
     assert L.mllm_hip_host_file_convert(c2.encode(), 2, c1.encode(), 1) == 3
     raw = open(c2, "rb").read()
