@@ -221,7 +221,18 @@ def side_workloads(torch, ql, synth, gen):
         act = float(np.mean([len(np.unique(r[0])) for r in routes]))
         wb = act * 3 * I * (H // 256) * 144
         deck["tokens_%d" % Td] = {"us": td * 1e6, "active_experts_avg": act, "weight_GBps": wb / td / 1e9, "frac_of_hbm_peak": wb / td / 8e12}
-    del gk, uk, dk
+    # the 512-token layer with Q4_K experts: pairs sorted by expert, tiles of eight rows on the matrix cores (the grouped form),
+    # against one GEMV row per pair
+    from mllm_amd import _lib as _l
+    wsk = torch.empty(_l.lib().mllm_hip_moe_kq_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
+    tk2 = ev_time(lambda: ql.moe_ffn_kq(gk, uk, dk, x, ids, tw, workspace=wsk, out=ym), 5)
+    _l.lib().mllm_hip_moe_kq_set_path(1)
+    tk1 = ev_time(lambda: ql.moe_ffn_kq(gk, uk, dk, x, ids, tw, workspace=wsk, out=ym), 3)
+    _l.lib().mllm_hip_moe_kq_set_path(0)
+    wbk = int((np.bincount(ids_np.reshape(-1), minlength=E) > 0).sum()) * 3 * I * (H // 256) * 144
+    deck["tokens_512_grouped"] = {"us": tk2 * 1e6, "weight_GBps": wbk / tk2 / 1e9, "frac_of_hbm_peak": wbk / tk2 / 8e12,
+                                  "pairs_as_gemv_rows_us": tk1 * 1e6}
+    del gk, uk, dk, wsk
     from mllm_amd import _lib
     L = _lib.lib()
     gate2 = ql.PackedExperts.synthetic(ql.Q4_0, E, I, H, gen, layout="gemm")

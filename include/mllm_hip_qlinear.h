@@ -323,10 +323,14 @@ int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed
 /* The same expert FFN with the experts in the super-block formats (MLLM_HIP_Q4_K / MLLM_HIP_Q6_K, the formats the shipped
  * Qwen3-MoE recipe quantizes to; activations Q8_K in front of every projection): gate_packed / up_packed / down_packed are E
  * matrices packed by mllm_hip_kq_prepack back to back, mllm_hip_kq_packed_bytes(wtype, I, H) resp. (wtype, H, I) apart.
- * H % 256 == 0, I % 256 == 0, T * k <= 65535.  Every (token, expert) pair runs as one GEMV row (three or four launches for any T): the
- * decode form; an expert's weights are read once per pair that uses it.
+ * H % 256 == 0, I % 256 == 0, T * k <= 65535, E <= 3072.  Up to two (token, expert) pairs per expert every pair runs as one
+ * GEMV row (three or four launches; the decode form, an expert's weights are read once per pair that uses it).  Beyond that
+ * the pairs are sorted by expert and run as tiles of eight rows on the matrix cores (the grouped form: x and h quantized
+ * to Q8_K once, an expert's weights read once per eight pairs; seven launches), same arithmetic.
  * replaces: the same loop over experts with Q4_K / Q6_K Linear ops, modeling_qwen3_moe_fa2.hpp:98-100,175-238 */
 size_t mllm_hip_moe_kq_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k);
+/* 0: by the number of pairs per expert (default); 1: always pairs as GEMV rows; 2: always tiles of eight rows (comparison runs and tests) */
+int mllm_hip_moe_kq_set_path(int path);
 int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x,
                         int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H, int64_t I,
                         int E, int k, void* workspace, void* stream);

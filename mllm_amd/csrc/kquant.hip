@@ -272,7 +272,51 @@ struct KGemvArgs {
   int silu_accurate;     // expf instead of the reference's polynomial (mllm_hip_set_exp_mode)
   int slot_E, slot_div, slot_div_slots;  // experts, pairs per activation row, number of slots (grid y)
   size_t estride;
+  // MoE row tiles (matrix-core kernels, quantized image as input): blockIdx.y = a tile of up to eight expert-sorted positions
+  // that share an expert.  The image holds img_rows rows; tile row m reads image row row_ids[row0 + m] / row_div (row_ids
+  // null: row0 + m) and writes output row out_ids[row0 + m] (null: row0 + m).  tile_expert == null: a plain Linear.
+  const int* tile_expert;
+  const int* tile_row0;
+  const int* tile_rows;
+  const int* ntiles;
+  const int* row_ids;
+  const int* out_ids;
+  int row_div;
+  int img_rows;  // rows of the image (0: the kernel's row tile MT)
 };
+// the tile of this workgroup: how many rows it has, where they start, where the expert's matrices lie
+struct KTile {
+  int rows, row0;
+  size_t eoff;
+  bool active;
+};
+__device__ __forceinline__ KTile kq_tile(const KGemvArgs& a) {
+  KTile t{a.M, 0, 0, true};
+  if (a.tile_expert) {
+    const int ti = blockIdx.y;
+    if (ti >= min(a.ntiles[0], (int)gridDim.y)) {
+      t.active = false;
+      return t;
+    }
+    t.rows = a.tile_rows[ti];
+    t.row0 = a.tile_row0[ti];
+    t.eoff = (size_t)a.tile_expert[ti] * a.estride;
+  }
+  return t;
+}
+__device__ __forceinline__ int kq_tile_in_row(const KGemvArgs& a, const KTile& t, int m) {
+  if (!a.tile_expert) return m;
+  const int pos = t.row0 + min(m, t.rows - 1);  // rows past the tile repeat its last row; their results are dropped
+  return a.row_ids ? a.row_ids[pos] / a.row_div : pos;
+}
+__device__ __forceinline__ int kq_tile_out_row(const KGemvArgs& a, const KTile& t, int m) {
+  if (!a.tile_expert) return m;
+  return a.out_ids ? a.out_ids[t.row0 + m] : t.row0 + m;
+}
+template <typename T>
+__device__ __forceinline__ const T* kq_at(const T* p, size_t byte_offset) {
+  return reinterpret_cast<const T*>(reinterpret_cast<const char*>(p) + byte_offset);
+}
 #define KBUF_OOB 0xffffffffu
 #define KBUF_NT 2
 
@@ -697,6 +741,8 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
   for (int p = 1; p < KQ_MAX_PARTS; p++)
     if (p < a.nparts && (int)blockIdx.x >= a.wg_start[p]) pidx = p;
   const KGemvPart& pt = a.part[pidx];
+  const KTile mt = kq_tile(a);
+  if (!mt.active) return;  // uniform, ahead of every barrier
   const int N = pt.N;
   const int tiles_wg = nwaves / S;
   const int tile = ((int)blockIdx.x - a.wg_start[pidx]) * tiles_wg + wave / S;
@@ -716,10 +762,10 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
 
   // ---- 1. weight scale records of the tile and slice: one 16-byte record per (row, super-block) --------------------------
   const uint32_t sbt = (uint32_t)N * (uint32_t)nsb;
-  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.a), 0, sbt * 128u, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.s), 0, sbt * 16u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(kq_at(pt.w.a, mt.eoff)), 0, sbt * 128u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(kq_at(pt.w.s, mt.eoff)), 0, sbt * 16u, 0x00020000);
   const int spb = nbs >> 3;  // super-blocks per slice (at most 8)
-  const __amdgpu_buffer_rsrc_t rdd = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(pt.w.d), 0, sbt * 4u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rdd = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(kq_at(pt.w.d, mt.eoff)), 0, sbt * 4u, 0x00020000);
   u32x4 sc[2];
   uint32_t scd[2];
 #pragma unroll
@@ -749,16 +795,18 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- 3. activations into LDS -------------------------------------------------------------------------------------------------
-  if (XT == KQ_IMAGE) {  // codes [MT][K], sums of 16 as int16 [MT][K/16], scales [MT][nsb]
+  if (XT == KQ_IMAGE) {  // codes [R][K], sums of 16 as int16 [R][K/16], scales [R][nsb]; R = MT, or the rows of a MoE image
+    const size_t R = a.img_rows ? (size_t)a.img_rows : (size_t)MT;
     const u32x4* codes = reinterpret_cast<const u32x4*>(a.x);
-    const uint32_t* pairs = reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(a.x) + (size_t)MT * K);
-    const float* dd = reinterpret_cast<const float*>(reinterpret_cast<const char*>(a.x) + (size_t)MT * K + (size_t)MT * nsb * 32);
+    const uint32_t* pairs = reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(a.x) + R * K);
+    const float* dd = reinterpret_cast<const float*>(reinterpret_cast<const char*>(a.x) + R * K + R * nsb * 32);
     for (int m = wave; m < MT; m += nwaves) {
-      for (int r = lane; r < 2 * nb32; r += 64) xc[((size_t)(r >> 1) * MT + m) * 2 + (r & 1)] = codes[(size_t)m * 2 * nb32 + r];
+      const size_t src = (size_t)kq_tile_in_row(a, mt, m);
+      for (int r = lane; r < 2 * nb32; r += 64) xc[((size_t)(r >> 1) * MT + m) * 2 + (r & 1)] = codes[src * 2 * nb32 + r];
       for (int sb = lane; sb < nb32; sb += 64) {
-        const uint32_t pr = pairs[(size_t)m * nb32 + sb];
+        const uint32_t pr = pairs[src * nb32 + sb];
         const int bsum = (int)(int16_t)(pr & 0xffffu) + (int)(int16_t)(pr >> 16);
-        xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(dd[m * nsb + (sb >> 3)]), (uint32_t)bsum};
+        xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(dd[src * nsb + (sb >> 3)]), (uint32_t)bsum};
       }
     }
   } else {
@@ -883,12 +931,13 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
       acc.x += o.x; acc.y += o.y; acc.z += o.z; acc.w += o.w;
     }
   }
-  if (!tile_ok || q2 != 0 || t >= MT || t >= a.M) return;
+  if (!tile_ok || q2 != 0 || t >= MT || t >= mt.rows) return;
   const int n = row0 + 4 * g;
   const float v[4] = {acc.x, acc.y, acc.z, acc.w};
+  float* yrow = pt.y + (int64_t)kq_tile_out_row(a, mt, t) * N;
 #pragma unroll
   for (int e = 0; e < 4; e++)
-    if (n + e < N) pt.y[(int64_t)t * N + n + e] = pt.bias ? v[e] + pt.bias[n + e] : v[e];
+    if (n + e < N) yrow[n + e] = pt.bias ? v[e] + pt.bias[n + e] : v[e];
 }
 
 template <int MT>
@@ -905,7 +954,7 @@ static bool kq4_mfma_fits(int MT, int nsb) {
   return (MT == 4 ? kmf_lds_bytes<4>(nb32, nbs, 8) : kmf_lds_bytes<8>(nb32, nbs, 8)) <= 160 * 1024;
 }
 template <int XT, int MT>
-static int launch_kq4_mfma_t(const KGemvArgs& a_in, hipStream_t st) {
+static int launch_kq4_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned grid_y = 1) {
   KGemvArgs a = a_in;
   const int nb32 = a.nsb * 8;
   const int S = kmf_slices(nb32);
@@ -924,7 +973,7 @@ static int launch_kq4_mfma_t(const KGemvArgs& a_in, hipStream_t st) {
   auto kern = kq4_gemv_mfma_kernel<XT, MT>;
   if (lds > 64 * 1024)
     HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(nwaves * 64), lds, st, a, S, nbs);
+  hipLaunchKernelGGL(kern, dim3(grid, grid_y), dim3(nwaves * 64), lds, st, a, S, nbs);
   return (int)hipGetLastError();
 }
 template <int XT>
@@ -954,6 +1003,8 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
   for (int p = 1; p < KQ_MAX_PARTS; p++)
     if (p < a.nparts && (int)blockIdx.x >= a.wg_start[p]) pidx = p;
   const KGemvPart& pt = a.part[pidx];
+  const KTile mt = kq_tile(a);
+  if (!mt.active) return;  // uniform, ahead of every barrier
   const int N = pt.N;
   const int tiles_wg = nwaves / S;
   const int tile = ((int)blockIdx.x - a.wg_start[pidx]) * tiles_wg + wave / S;
@@ -972,10 +1023,10 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
   f32x4* red = reinterpret_cast<f32x4*>(smem) + (size_t)wave * TH * 64;  // takes the place of the codes once every wave is done with them
 
   const uint32_t sbt = (uint32_t)N * (uint32_t)nsb;
-  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.a), 0, sbt * 128u, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.h), 0, sbt * 64u, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(pt.w.s), 0, sbt * 16u, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(pt.w.d), 0, sbt * 2u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(kq_at(pt.w.a, mt.eoff)), 0, sbt * 128u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rh = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(kq_at(pt.w.h, mt.eoff)), 0, sbt * 64u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(kq_at(pt.w.s, mt.eoff)), 0, sbt * 16u, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rd = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(kq_at(pt.w.d, mt.eoff)), 0, sbt * 2u, 0x00020000);
   // ---- 1. weight scales of the tile and slice: 16 int8 and one fp16 per (row, super-block) -------------------------------------
   u32x4 sc[2];
   uint16_t scd[2];
@@ -1007,16 +1058,18 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
   __builtin_amdgcn_sched_barrier(0);
 
   // ---- 3. activations into LDS -------------------------------------------------------------------------------------------------
-  if (XT == KQ_IMAGE) {  // codes [MT][K], sums of 16 as int16 [MT][K/16], scales [MT][nsb]
+  if (XT == KQ_IMAGE) {  // codes [R][K], sums of 16 as int16 [R][K/16], scales [R][nsb]; R = MT, or the rows of a MoE image
+    const size_t R = a.img_rows ? (size_t)a.img_rows : (size_t)MT;
     const u32x4* codes = reinterpret_cast<const u32x4*>(a.x);
-    const int16_t* sums = reinterpret_cast<const int16_t*>(reinterpret_cast<const char*>(a.x) + (size_t)MT * K);
-    const float* dd = reinterpret_cast<const float*>(reinterpret_cast<const char*>(a.x) + (size_t)MT * K + (size_t)MT * nsb * 32);
+    const int16_t* sums = reinterpret_cast<const int16_t*>(reinterpret_cast<const char*>(a.x) + R * K);
+    const float* dd = reinterpret_cast<const float*>(reinterpret_cast<const char*>(a.x) + R * K + R * nsb * 32);
     for (int m = wave; m < MT; m += nwaves) {
+      const size_t src = (size_t)kq_tile_in_row(a, mt, m);
       for (int u = lane; u < nu; u += 64) {
-        xc[(size_t)u * MT + m] = codes[(size_t)m * nu + u];
-        bs16[(size_t)u * MT + m] = (int)sums[(size_t)m * nu + u];
+        xc[(size_t)u * MT + m] = codes[src * nu + u];
+        bs16[(size_t)u * MT + m] = (int)sums[src * nu + u];
       }
-      for (int sb = lane; sb < nsb; sb += 64) dxs[sb * MT + m] = dd[m * nsb + sb];
+      for (int sb = lane; sb < nsb; sb += 64) dxs[sb * MT + m] = dd[src * nsb + sb];
     }
   } else {
     const int ipr = K >> 3;
@@ -1170,11 +1223,12 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
 #pragma unroll
   for (int h = 0; h < TH; h++) {
     const int t = 4 * h + tt;
-    if (t >= a.M) continue;
+    if (t >= mt.rows) continue;
     const float v[4] = {acc[h].x, acc[h].y, acc[h].z, acc[h].w};
+    float* yrow = pt.y + (int64_t)kq_tile_out_row(a, mt, t) * N;
 #pragma unroll
     for (int e = 0; e < 4; e++)
-      if (n + e < N) pt.y[(int64_t)t * N + n + e] = pt.bias ? v[e] + pt.bias[n + e] : v[e];
+      if (n + e < N) yrow[n + e] = pt.bias ? v[e] + pt.bias[n + e] : v[e];
   }
 }
 
@@ -1197,7 +1251,7 @@ static bool kq6_mfma_fits(int MT, int nsb) {
   return (MT == 4 ? k6mf_lds_bytes<4>(nsb, sps, 8) : k6mf_lds_bytes<8>(nsb, sps, 8)) <= 160 * 1024;
 }
 template <int XT, int MT>
-static int launch_kq6_mfma_t(const KGemvArgs& a_in, hipStream_t st) {
+static int launch_kq6_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned grid_y = 1) {
   KGemvArgs a = a_in;
   int S, sps;
   k6mf_split(a.nsb, S, sps);
@@ -1215,7 +1269,7 @@ static int launch_kq6_mfma_t(const KGemvArgs& a_in, hipStream_t st) {
   auto kern = kq6_gemv_mfma_kernel<XT, MT>;
   if (lds > 64 * 1024)
     HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(nwaves * 64), lds, st, a, S, sps);
+  hipLaunchKernelGGL(kern, dim3(grid, grid_y), dim3(nwaves * 64), lds, st, a, S, sps);
   return (int)hipGetLastError();
 }
 template <int XT>
@@ -1483,6 +1537,40 @@ int kq_moe_gemv(int wtype, int nparts, const void* const* packed0, float* const*
   if (wtype == MLLM_HIP_Q4_K)
     return x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_F32>(a, st) : launch_kq<MLLM_HIP_Q4_K, MLLM_HIP_BF16>(a, st);
   return x_dtype == MLLM_HIP_F32 ? launch_kq<MLLM_HIP_Q6_K, MLLM_HIP_F32>(a, st) : launch_kq<MLLM_HIP_Q6_K, MLLM_HIP_BF16>(a, st);
+}
+
+// The Q8_K image of `rows` activation rows of K elements (codes [rows][K], sums of 16 [rows][K/16] int16, scales
+// [rows][K/256]) at `image`: what the matrix-core kernels copy into LDS.
+size_t kq_image_bytes(int64_t rows, int64_t K) { return (size_t)rows * K + (size_t)rows * (K / 16) * 2 + (size_t)rows * (K / QK_K) * 4; }
+int kq_quantize_image(const void* x, int x_dtype, void* image, int64_t rows, int64_t K, hipStream_t st) {
+  const int64_t nitems = rows * K / 8;
+  int8_t* codes = reinterpret_cast<int8_t*>(image);
+  int16_t* bsums = reinterpret_cast<int16_t*>(codes + rows * K);
+  float* d = reinterpret_cast<float*>(codes + rows * K + rows * (K / 16) * 2);
+  hipLaunchKernelGGL(quantize_q8k_kernel, dim3((unsigned)((nitems + 255) / 256)), dim3(256), 0, st, x, x_dtype, codes, d, bsums, nitems,
+                     nitems);
+  return (int)hipGetLastError();
+}
+bool kq_moe_tiles_fit(int wtype, int64_t K) {
+  return wtype == MLLM_HIP_Q4_K ? kq4_mfma_fits(8, (int)(K / QK_K)) : kq6_mfma_fits(8, (int)(K / QK_K));
+}
+// MoE row tiles on the matrix-core kernels: tile t (blockIdx.y) = up to eight expert-sorted positions of expert tile_expert[t];
+// its rows read image rows row_ids[pos] / row_div (null: pos) and write rows out_ids[pos] (null: pos) of ys[p].
+int kq_moe_tiles_gemv(int wtype, int nparts, const void* const* packed0, float* const* ys, int64_t N, int64_t K, const void* image,
+                      int64_t img_rows, const int* tile_expert, const int* tile_row0, const int* tile_rows, const int* ntiles,
+                      unsigned max_tiles, const int* row_ids, int row_div, const int* out_ids, hipStream_t st) {
+  if (nparts < 1 || nparts > KQ_MAX_PARTS || max_tiles < 1 || max_tiles > 65535) return MLLM_HIP_E_SHAPE;
+  KGemvArgs a{};
+  for (int p = 0; p < nparts; p++) a.part[p] = KGemvPart{kq_view(wtype, packed0[p], N, K), nullptr, ys[p], (int)N};
+  a.nparts = nparts;
+  a.x = image;
+  a.M = 8;
+  a.nsb = (int)(K / QK_K);
+  a.estride = kq_packed_bytes(wtype, N, K);
+  a.tile_expert = tile_expert; a.tile_row0 = tile_row0; a.tile_rows = tile_rows; a.ntiles = ntiles;
+  a.row_ids = row_ids; a.out_ids = out_ids; a.row_div = row_div > 0 ? row_div : 1;
+  a.img_rows = (int)img_rows;
+  return wtype == MLLM_HIP_Q4_K ? launch_kq4_mfma_t<KQ_IMAGE, 8>(a, st, max_tiles) : launch_kq6_mfma_t<KQ_IMAGE, 8>(a, st, max_tiles);
 }
 }  // namespace mllmhip
 

@@ -1886,18 +1886,48 @@ MLLM_API int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const v
 // The shipped Qwen3-MoE recipe quantizes the experts to Q4_K / Q6_K.  Every (token, expert) pair is one row of the K-quant
 // GEMV: gate and up in one launch (the workgroup quantizes the token's x to Q8_K), silu(g) * u, the down GEMV (quantizing h),
 // the weighted sum in slot order.  Three or four launches for any T; the weights of an expert are read once per pair that uses it,
-// so this is the decode form (prefill wants the experts grouped, which this format does not have yet).
+// so this is the decode form.  With more than two pairs per expert the pairs are sorted by expert and run as tiles of eight
+// rows on the matrix-core kernels instead (the grouped form).
 namespace mllmhip {
 int kq_moe_gemv(int wtype, int nparts, const void* const* packed0, float* const* ys, int64_t N, int64_t K, const void* x, int x_dtype,
                 const float* x2, const int32_t* ids, int E, int slots, int slot_div, hipStream_t st);
+size_t kq_image_bytes(int64_t rows, int64_t K);
+int kq_quantize_image(const void* x, int x_dtype, void* image, int64_t rows, int64_t K, hipStream_t st);
+bool kq_moe_tiles_fit(int wtype, int64_t K);
+int kq_moe_tiles_gemv(int wtype, int nparts, const void* const* packed0, float* const* ys, int64_t N, int64_t K, const void* image,
+                      int64_t img_rows, const int* tile_expert, const int* tile_row0, const int* tile_rows, const int* ntiles,
+                      unsigned max_tiles, const int* row_ids, int row_div, const int* out_ids, hipStream_t st);
+static int g_moe_kq_path = 0;  // 0: by the number of pairs per expert; 1: always pairs as GEMV rows; 2: always tiles of eight rows
+constexpr int KQ_MOE_TILE = 8;
+struct KqMoeCarve {
+  float *g, *u, *h, *per;
+  char *ximg, *himg;
+  RouteOut ro;
+};
+static KqMoeCarve carve_kq_moe(Carver& c, int64_t T, int64_t H, int64_t I, int E, int k) {
+  KqMoeCarve r;
+  const size_t slots = (size_t)T * k;
+  r.g = c.take<float>(slots * I);
+  r.u = c.take<float>(slots * I);
+  r.h = c.take<float>(slots * I);
+  r.per = c.take<float>(slots * H);
+  r.ximg = c.take<char>(kq_image_bytes(T, H));
+  r.himg = c.take<char>(kq_image_bytes((int64_t)slots, I));
+  r.ro = carve_route(c, E, (int64_t)slots, KQ_MOE_TILE);
+  return r;
 }
+}  // namespace mllmhip
+
+MLLM_API int mllm_hip_moe_kq_set_path(int path) {
+  if (path < 0 || path > 2) return MLLM_HIP_E_BADARG;
+  g_moe_kq_path = path;
+  return 0;
+}
+
 MLLM_API size_t mllm_hip_moe_kq_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k) {
   if (T <= 0 || H <= 0 || I <= 0 || E <= 0 || k <= 0 || H % 256 || I % 256) return 0;
   Carver c(nullptr);
-  c.take<float>((size_t)T * k * I);
-  c.take<float>((size_t)T * k * I);
-  c.take<float>((size_t)T * k * I);
-  c.take<float>((size_t)T * k * H);
+  carve_kq_moe(c, T, H, I, E, k);
   return c.used;
 }
 
@@ -1916,10 +1946,36 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
   hipStream_t st = (hipStream_t)stream;
   const int slots = (int)(T * k);
   Carver c(workspace);
-  float* g = c.take<float>((size_t)slots * I);
-  float* u = c.take<float>((size_t)slots * I);
-  float* h = c.take<float>((size_t)slots * I);
-  float* per = c.take<float>((size_t)slots * H);
+  const KqMoeCarve w = carve_kq_moe(c, T, H, I, E, k);
+  float *g = w.g, *u = w.u, *h = w.h, *per = w.per;
+  // More than about two pairs per expert (Q6_K: one): the pairs are sorted by expert and run as tiles of eight rows on the matrix-core
+  // kernels, so an expert's matrices are streamed once per eight pairs instead of once per pair (the grouped form).
+  // x and h are quantized to Q8_K once (bit-exact images), the tiles gather their rows from the images.
+  const bool tiles_ok = E <= MOE_MAX_EXPERTS && kq_moe_tiles_fit(wtype, H) && kq_moe_tiles_fit(wtype, I) &&
+                        (size_t)E + (size_t)slots / KQ_MOE_TILE + 1 <= 65535;
+  // measured at 128 experts, top-8 (pairs -> tiles, us): Q4_K 32 tokens 140 -> 143, 64: 273 -> 192, 512: 2149 -> 649;
+  // Q6_K 16 tokens 142 -> 140, 32: 264 -> 187, 512: 3976 -> 887
+  const int per_expert = wtype == MLLM_HIP_Q4_K ? 2 : 1;
+  if (tiles_ok && (g_moe_kq_path == 2 || (g_moe_kq_path == 0 && slots > per_expert * E))) {
+    const unsigned max_tiles = (unsigned)(E + slots / KQ_MOE_TILE + 1);
+    RC_RET(launch_route(topk_ids, slots, E, KQ_MOE_TILE, w.ro, st));
+    RC_RET(kq_quantize_image(x, x_dtype, w.ximg, T, H, st));
+    const void* gu2[2] = {gate_packed, up_packed};
+    float* guy2[2] = {g, u};  // rows in expert-sorted order
+    RC_RET(kq_moe_tiles_gemv(wtype, 2, gu2, guy2, I, H, w.ximg, T, w.ro.tile_expert, w.ro.tile_row0, w.ro.tile_rows, w.ro.ntiles,
+                             max_tiles, w.ro.sorted_idx, k, nullptr, st));
+    // positions past the last valid pair (invalid expert ids) are never written nor read: the tiles cover offsets[E] rows
+    RC_RET(mllm_hip_silu_mul(g, u, h, MLLM_HIP_F32, slots, I, nullptr, MLLM_HIP_SCALE_IEEE, stream));
+    RC_RET(kq_quantize_image(h, MLLM_HIP_F32, w.himg, slots, I, st));
+    const void* dn2[1] = {down_packed};
+    float* dny2[1] = {per};  // row t * k + j
+    RC_RET(kq_moe_tiles_gemv(wtype, 1, dn2, dny2, H, I, w.himg, slots, w.ro.tile_expert, w.ro.tile_row0, w.ro.tile_rows,
+                             w.ro.ntiles, max_tiles, nullptr, 1, w.ro.sorted_idx, st));
+    const int64_t total2 = T * H;
+    hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total2 / 4 + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
+                       (int)H, k, E);
+    return (int)hipGetLastError();
+  }
   const void* gu[2] = {gate_packed, up_packed};
   float* guy[2] = {g, u};
   int rc = kq_moe_gemv(wtype, 2, gu, guy, I, H, x, x_dtype, nullptr, topk_ids, E, slots, k, st);

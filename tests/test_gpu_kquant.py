@@ -264,3 +264,42 @@ def test_moe_ffn_with_k_quant_experts(wtype, T, H, I, E, k):
     bits, xb = synth.make_x_bf16(rng, T, H)
     y4 = ql.moe_ffn_kq(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
     assert rel_l2(y4, orc.moe_ffn_kq(xb, ids, w, Wg, Wu, Wd, wtype)) < 1e-3
+
+
+@pytest.mark.parametrize("wtype,T,H,I,E,k", [(2, 40, 512, 256, 6, 3), (3, 33, 256, 512, 4, 2), (2, 96, 2048, 768, 16, 4),
+                                            (3, 64, 2048, 768, 8, 2), (2, 9, 256, 256, 3, 1)])
+def test_moe_ffn_k_quant_grouped_form_equals_the_pair_form(wtype, T, H, I, E, k):
+    """Many pairs per expert: the pairs sorted by expert run as tiles of eight rows on the matrix-core kernels (x and h
+    quantized to Q8_K once, tiles gather their rows).  Same arithmetic as one GEMV row per pair (exact integer sums, fp32
+    scaling in another order): the two forms agree to 1e-5, both meet the oracle; invalid expert ids add nothing; a permutation
+    of the tokens permutes the outputs bit for bit; bf16 activations."""
+    rng = synth.rng_for(9, 7100 + wtype + T + H + I + E)
+    L = _lib.lib()
+    Wg = synth.make_weight(rng, wtype, E * I, H).reshape(E, I, H // 256, -1)
+    Wu = synth.make_weight(rng, wtype, E * I, H).reshape(E, I, H // 256, -1)
+    Wd = synth.make_weight(rng, wtype, E * H, I).reshape(E, H, I // 256, -1)
+    ids, w = synth.make_moe_routing(rng, T, E, k)
+    ids[1, 0] = E + 2          # an expert id out of range
+    if k > 1:
+        ids[T - 1, k - 1] = -1
+    g, u, d = (ql.PackedKExperts(wtype, torch.from_numpy(W)) for W in (Wg, Wu, Wd))
+    x = synth.make_x_fp32(rng, T, H)
+    announce("moe k-quant grouped", wtype, T, H, I, E, k)
+    outs = {}
+    for path in (1, 2):
+        assert L.mllm_hip_moe_kq_set_path(path) == 0
+        try:
+            outs[path] = ql.moe_ffn_kq(g, u, d, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+            if path == 2:
+                perm = rng.permutation(T)
+                y2 = ql.moe_ffn_kq(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
+                bits, xb = synth.make_x_bf16(rng, T, H)
+                y4 = ql.moe_ffn_kq(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
+        finally:
+            assert L.mllm_hip_moe_kq_set_path(0) == 0
+    want = orc.moe_ffn_kq(x, ids, w, Wg, Wu, Wd, wtype)
+    assert rel_l2(outs[2], want) < 1e-3, rel_l2(outs[2], want)
+    assert rel_l2(outs[2], outs[1]) < 1e-5, rel_l2(outs[2], outs[1])
+    assert np.array_equal(y2, outs[2][perm])
+    assert rel_l2(y4, orc.moe_ffn_kq(xb, ids, w, Wg, Wu, Wd, wtype)) < 1e-3
+    assert L.mllm_hip_moe_kq_set_path(3) == -1
