@@ -452,18 +452,20 @@ static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* part
   // three or more rows: block sums on the matrix cores (as long as the rows fit that kernel's LDS: 8 rows of 11 000 elements)
   // Q8_0 (twice the code bytes per block) gains only from five rows on.  The rule looks at the weight type, the number of
   // rows and the row length, never at the number of weight rows: a matrix takes the same kernel alone and in a multi launch.
-  // Q8_0 with three or four rows is faster on the vector ALU as long as the rows fit its LDS image (40 bytes per block and row)
-  const bool long_rows = (size_t)MT * a.nb * 40 > 140 * 1024;
-  const bool mfma_rows = MT >= 4 && g_gemv_path != 1 && (wtype == MLLM_HIP_Q4_0 || MT == 8 || long_rows);
+  // Q8_0 with three or four rows is faster on the vector ALU for rows of up to a few thousand elements (gate + up of the 4B
+  // layer 16.7 against 17.9 us, q+k+v 8.1 / 8.5) and slower for long ones (down, 9728 elements: 13.0 / 10.0)
+  const bool long_rows = a.nb >= 256;
+  const bool mfma_rows = MT >= 4 && g_gemv_path != 1 && (wtype == MLLM_HIP_Q4_0 || MT == 8);
+  const bool mfk_rows = mfma_rows || (MT >= 4 && g_gemv_path != 1 && long_rows);
   const int waves = (g_tune_NW == 2 || g_tune_NW == 4 || g_tune_NW == 8) ? g_tune_NW : 0;
   // K slices as separate workgroups, each quantizing only its slice of x (one launch, same bits, no limit on the row length
   // from LDS): needs room for the slices' partial sums behind the image area of the workspace; falls through where that
   // room is missing
-  if (mfma_rows && g_gemv_path != 2) {
+  if (mfk_rows && g_gemv_path != 2) {
     const size_t img = gemv_image_bytes(K);
     char* part = (workspace && ws_bytes > img) ? reinterpret_cast<char*>(workspace) + img : nullptr;
     const int rc = launch_gemv_mfk(wtype, x_dtype == MLLM_HIP_Q8_IMAGE ? GEMV_PREQ : x_dtype, MT, a, workspace, part,
-                                   part ? ws_bytes - img : 0, waves, st);
+                                   part ? ws_bytes - img : 0, g_tune_NW, st);
     if (rc != MFK_NOT_TAKEN) return rc;
   }
   if (mfma_rows && gemv_mfma_fits(MT, a.nb)) {

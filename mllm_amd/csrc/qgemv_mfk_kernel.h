@@ -39,7 +39,8 @@ static size_t mfk_lds_bytes(int wtype, int nbs, int nwaves) {
          (size_t)nwaves * ((size_t)nbs * 64 + (size_t)MFK_STG * 16 * (wtype == MLLM_HIP_Q8_0 ? 2 : 1)) + 16;
 }
 
-// blockDim = 256 or 512 (four or eight row tiles per workgroup)
+// blockDim = 64 x (row tiles per workgroup): three to eight waves, at least nbs / 16 (the threads hold one pass of
+// quantization items per activation row)
 template <int WT, int XT, int MT>
 __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -89,7 +90,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   const u32x4* img_hi = img_lo + mnb;
   const float* img_d = reinterpret_cast<const float*>(img_hi + mnb);
   const int* img_n8 = reinterpret_cast<const int*>(img_d + mnb);
-  constexpr int NIMG = MT / 4;
+  constexpr int NIMG = (MT + 2) / 3;  // passes of one image row per wave (at least three waves)
   const int ib = tid & 63, im = tid >> 6;
   u32x4 plo[NIMG], phi[NIMG];
   float pd[NIMG];

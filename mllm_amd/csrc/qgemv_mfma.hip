@@ -1,4 +1,5 @@
 // Launchers of the matrix-core decode GEMV (three to eight activation rows); the kernel is in qgemv_mfma_kernel.h.
+#include <algorithm>
 #include <mutex>
 
 #include "qgemv_mfk_kernel.h"
@@ -63,9 +64,27 @@ int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const v
   k.nbs = ((a.nb + k.S - 1) / k.S + 7) / 8 * 8;
   if (k.nbs > MFK_MAX_NBS || k.S > 65535) return MFK_NOT_TAKEN;
   k.ipr_magic = ((1 << 20) + 4 * k.nbs - 1) / (4 * k.nbs);
-  // four row tiles per workgroup; eight where eight activation rows meet long rows (measured on the 4B shapes: the down
-  // projection at eight rows 11.2 against 12.1 us, everything else 0.2 to 1.1 us slower with eight)
-  const int nwaves = waves == 8 || (!waves && MT == 8 && k.S >= 8) ? 8 : 4;
+  // Row tiles (= waves) per workgroup.  All workgroups are resident at once and every one costs vector-ALU time (its
+  // quantization of the slice of x, then per tile the MFMA / scaling loop), so what counts is the work of the busiest CU:
+  // rounds = ceil(workgroups / 256 CUs), each round costing (tiles per workgroup x loop + quantization).  Measured ratio of
+  // the two on the 4B shapes at eight rows: quantization of a slice = about two tiles' loops.  E.g. gate + up (1216 tiles x 2
+  // slices): four tiles per workgroup -> 608 workgroups, three on some CUs (12 tile loops + 3 quantizations), five -> 488
+  // workgroups, two per CU (10 + 2); the down projection (160 tiles x 8 slices): five -> exactly 256 workgroups.
+  const int nw_min = std::max(3, (k.nbs + 15) / 16);
+  int nwaves = waves;
+  if (nwaves < nw_min || nwaves > 8) {
+    double best = 1e30;
+    for (int nw = nw_min; nw <= 8; nw++) {
+      int64_t wgs = 0;
+      for (int p = 0; p < a.nparts; p++) wgs += ((a.part[p].N + 15) / 16 + nw - 1) / nw;
+      wgs *= k.S;
+      const double cost = (double)((wgs + 255) / 256) * (nw + 2.0);
+      if (cost < best - 1e-9) {
+        best = cost;
+        nwaves = nw;
+      }
+    }
+  }
   unsigned grid = 0;
   int np = 0;
   for (int p = 0; p < a.nparts; p++) {

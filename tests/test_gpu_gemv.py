@@ -316,6 +316,9 @@ def test_gemv_k_slices_as_workgroups_give_the_same_bits(wtype, M):
     one to eight slices; and against the oracle."""
     rng = synth.rng_for(1, 900 + M + 10 * wtype)
     L = _lib.lib()
+    # Q8_0 at three or four rows: the comparison path is the vector-ALU kernel there (another order of the fp32 sums), and the
+    # slice form is only taken for long rows
+    same_bits = not (wtype == 1 and M <= 4)
     for shapes in ([(9728, 2560), (9728, 2560)], [(2560, 9728)], [(4096, 2560), (1024, 2560), (1024, 2560)], [(2560, 4096)],
                    [(40, 96), (7, 96), (33, 96)], [(65, 32)], [(50, 161 * 32)], [(129, 41 * 32), (16, 41 * 32)],
                    # the longest rows the one-workgroup matrix-core kernel holds (two trips per slice at four rows)
@@ -338,7 +341,10 @@ def test_gemv_k_slices_as_workgroups_give_the_same_bits(wtype, M):
                     outs = [torch.full((M, n), float("nan"), device="cuda") for n, _ in shapes]
                     ql.linear_q_gemv_multi(ws, xd, biases, mode, outs=outs, workspace=wsp)
                     for f, p in zip(one_wg, outs):
-                        assert torch.equal(f, p)
+                        if same_bits:
+                            assert torch.equal(f, p)
+                        else:
+                            assert rel_l2(p.cpu().numpy(), f.cpu().numpy()) < 2e-6
         # residual added in the epilogue, and the quantized image as input
         xd = to_dev(x)
         res = [to_dev(rng.standard_normal((M, n)).astype(np.float32)) for n, _ in shapes]
@@ -351,7 +357,8 @@ def test_gemv_k_slices_as_workgroups_give_the_same_bits(wtype, M):
         r1 = ql.linear_q_gemv_fused(ws, xd, biases=biases, residuals=res, workspace=wsp)
         r2 = ql.linear_q_gemv_fused(ws, img, M=M, image=True, biases=biases, residuals=res, workspace=wsp)
         for f, p, i in zip(r0, r1, r2):
-            assert torch.equal(f, p) and torch.equal(f, i)
+            assert torch.equal(p, i)
+            assert torch.equal(f, p) if same_bits else rel_l2(p.cpu().numpy(), f.cpu().numpy()) < 2e-6
         want = orc.linear_q(x, Ws[0], wtype, biases[0].cpu().numpy(), orc.SCALE_X86_REF)
         got = ql.linear_q_gemv_multi(ws, to_dev(x), biases, ql.SCALE_X86_REF, workspace=wsp)[0].cpu().numpy()
         assert rel_l2(got, want) < 2e-6
