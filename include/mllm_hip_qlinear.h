@@ -164,10 +164,12 @@ int mllm_hip_q_block_isums(int wtype, const void* packed, const int8_t* codes, i
 int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
 
 /* GEMV launch-shape override for tuning sweeps: lanes per weight row (8/16/32/64), rows per lane group (1/2/4),
- * waves per workgroup (1..16); 0 restores the built-in heuristic. */
+ * waves per workgroup (1..16; the three- to eight-row kernel with K slices as workgroups takes 3..8); 0 restores the built-in
+ * heuristic. */
 int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_per_wg);
 /* Three to eight rows take their block sums from the matrix cores (v_mfma_i32_16x16x32_i8, same fp32 arithmetic around
- * them); path = 1 keeps every launch on the vector-ALU kernel (comparison runs), 0 restores the default. */
+ * them); path = 1 keeps every launch on the vector-ALU kernel, path = 2 keeps the K slices of a row tile in one workgroup
+ * (comparison runs), 0 restores the default. */
 int mllm_hip_gemv_set_path(int path);
 
 /* ---------------------------------------------------------------------------------------------------------
