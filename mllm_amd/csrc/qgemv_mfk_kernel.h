@@ -23,13 +23,38 @@ constexpr int MFK_TRIP = 8 * MFK_CH;
 constexpr int MFK_STG = 16 * 9;       // 16-byte pieces of one stage: 16 rows, stride 9 (reads of 16 rows hit 16 bank groups)
 constexpr int MFK_MAX_NBS = 64;       // blocks per slice (weight scales of a slice: two 16-byte loads per lane)
 
+// Quantization of sixteen elements (half a block) by one lane of a pair; lanes 2 b and 2 b + 1 share block b.  The same
+// operations on the same values as quad_quantize (maximum of 32 magnitudes, the two IEEE divisions, v * id rounded to
+// nearest even, integer sums): same codes, same scale, half as many instructions per element.  `ok` false = an element past
+// the row or a row past M: zeros (v then holds finite or non-finite values of the last valid row, whose codes a scale of
+// zero multiplies away).
+__device__ __forceinline__ void pair_quantize(const float (&v)[16], bool ok, int x86, u32x4& codes, float& deff, int& n8) {
+  float amax = 0.f;
+#pragma unroll
+  for (int e = 0; e < 16; e++) amax = fmaxf(amax, fabsf(v[e]));
+  amax = ok ? amax : 0.f;  // with amax = 0 the inverse scale is 0 and every code comes out 0, whatever v holds
+  amax = fmaxf(amax, dpp_f<0xB1>(amax));
+  const float d = amax / 127.f;
+  const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
+  codes = u32x4{q8_pack4(&v[0], idv), q8_pack4(&v[4], idv), q8_pack4(&v[8], idv), q8_pack4(&v[12], idv)};
+  int sum = __builtin_amdgcn_sdot4((int)codes.x, 0x01010101, 0, false);
+  sum = __builtin_amdgcn_sdot4((int)codes.y, 0x01010101, sum, false);
+  sum = __builtin_amdgcn_sdot4((int)codes.z, 0x01010101, sum, false);
+  sum = __builtin_amdgcn_sdot4((int)codes.w, 0x01010101, sum, false);
+  sum += __builtin_amdgcn_update_dpp(0, sum, 0xB1, 0xf, 0xf, true);
+  uint16_t bits = f32_to_f16bits(d);
+  if (x86) bits = x86_scale_bits(bits);
+  deff = f16bits_to_f32(bits);
+  n8 = -8 * sum;
+}
+
 struct MfkArgs {
   float* part;         // [S][MT][NP] partial sums (S > 1)
   unsigned* counters;  // one per workgroup column (blockIdx.x), zero between launches (S > 1)
   int NP;              // columns of a partial row: every part's rows rounded up to 16
   int S, nbs;          // K slices; blocks per slice (a multiple of 8, at most MFK_MAX_NBS)
   int col0[GEMV_MAX_PARTS];  // first column of each part within a partial row
-  int ipr_magic;             // ceil(2^20 / (4 nbs)): item / (items per row) as a multiply and a shift
+  int ipr_magic;             // ceil(2^20 / (2 nbs)): item / (items per row) as a multiply and a shift
 };
 
 template <int MT>
@@ -80,11 +105,12 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   int* s_flag = reinterpret_cast<int*>(stg_all + (size_t)nwaves * MFK_STG * NPL);
 
   // ---- 1. activation requests (they return first; nothing here divides: the weight requests below must leave early) ------
-  // raw activations: item it = tid + i * blockDim = eight elements, the four lanes of a quad share a block;
+  // raw activations: item it = tid + i * blockDim = sixteen elements, two neighbouring lanes share a block;
   // image: thread (row tid / 64 + i * nwaves, block tid % 64)
-  const int ipr = nbs * 4;            // items of eight elements per row of the slice
-  const int nitems = MT * ipr;        // item it: row it / ipr, column it % ipr (the quads stay whole: ipr % 4 == 0)
-  XRaw<XTT> raw[MT];
+  const int ipr = nbs * 2;            // items of sixteen elements (half a block) per row of the slice
+  const int nitems = MT * ipr;        // item it: row it / ipr, half block it % ipr (pairs of lanes stay whole: ipr % 2 == 0)
+  constexpr int NXP = MT / 2;         // passes: the threads number at least 4 nbs (launcher), so MT * ipr / blockDim <= MT / 2
+  XRaw<XTT> raw[NXP][2];
   const int mnb = MT * nb;
   const u32x4* img_lo = reinterpret_cast<const u32x4*>(xptr);
   const u32x4* img_hi = img_lo + mnb;
@@ -103,12 +129,14 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < MT; i++) {
+    for (int i = 0; i < NXP; i++) {
       if (i * nthreads < nitems) {  // uniform
         const int it = min(tid + i * nthreads, nitems - 1);
         const int m = (int)(((uint32_t)it * (uint32_t)k.ipr_magic) >> 20), xc = it - m * ipr;
         // clamped addresses: validity is applied when the values are used
-        load_x8<XTT>(xptr, ((int64_t)min(m, aM - 1) * nb * 4 + min(b0 * 4 + xc, nb * 4 - 1)) * 8, raw[i]);
+        const int64_t e0 = ((int64_t)min(m, aM - 1) * nb * 2 + min(b0 * 2 + xc, nb * 2 - 1)) * 16;
+        load_x8<XTT>(xptr, e0, raw[i][0]);
+        load_x8<XTT>(xptr, e0 + 8, raw[i][1]);
       }
     }
   }
@@ -157,23 +185,27 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < MT; i++) {
+    for (int i = 0; i < NXP; i++) {
       const int it = tid + i * nthreads;
-      if (it < nitems) {  // whole quads: nitems and nthreads are multiples of 4
+      if (it < nitems) {  // whole pairs: nitems and nthreads are even
         const int m = (int)(((uint32_t)it * (uint32_t)k.ipr_magic) >> 20), xc = it - m * ipr;
-        float v[8];
-        x8_to_f32<XTT>(raw[i], v);
-        const int b = xc >> 2, j = xc & 3;
-        if (m >= aM || b0 + b >= nb) {
+        float v[16], v1[8];
+        {
+          float v0[8];
+          x8_to_f32<XTT>(raw[i][0], v0);
+          x8_to_f32<XTT>(raw[i][1], v1);
 #pragma unroll
-          for (int e = 0; e < 8; e++) v[e] = 0.f;
+          for (int e = 0; e < 8; e++) {
+            v[e] = v0[e];
+            v[8 + e] = v1[e];
+          }
         }
-        uint32_t pk[2];
+        const int b = xc >> 1, j = xc & 1;
+        u32x4 codes;
         float deff;
         int n8;
-        quad_quantize(v, x86, pk, deff, n8);
-        u32x2* dst = reinterpret_cast<u32x2*>((j < 2 ? xlo : xhi) + (size_t)m * rs + b) + (j & 1);
-        *dst = u32x2{pk[0], pk[1]};
+        pair_quantize(v, m < aM && b0 + b < nb, x86, codes, deff, n8);
+        (j == 0 ? xlo : xhi)[(size_t)m * rs + b] = codes;
         if (j == 0) xs[(size_t)m * nbs + b] = u32x2{__float_as_uint(deff), (uint32_t)n8};
       }
     }

@@ -63,7 +63,7 @@ int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const v
   k.S = gemv_mfk_slices(a.nb);
   k.nbs = ((a.nb + k.S - 1) / k.S + 7) / 8 * 8;
   if (k.nbs > MFK_MAX_NBS || k.S > 65535) return MFK_NOT_TAKEN;
-  k.ipr_magic = ((1 << 20) + 4 * k.nbs - 1) / (4 * k.nbs);
+  k.ipr_magic = ((1 << 20) + 2 * k.nbs - 1) / (2 * k.nbs);
   // Row tiles (= waves) per workgroup.  All workgroups are resident at once and every one costs vector-ALU time (its
   // quantization of the slice of x, then per tile the MFMA / scaling loop), so what counts is the work of the busiest CU:
   // rounds = ceil(workgroups / 256 CUs), each round costing (tiles per workgroup x loop + quantization).  Measured ratio of
