@@ -163,9 +163,10 @@ int mllm_hip_q_block_isums(int wtype, const void* packed, const int8_t* codes, i
  * dst is NULL.  Used to calibrate HBM traffic counters and to measure the fixed cost of a launch of a given size. */
 int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
 
-/* GEMV launch-shape override for tuning sweeps: lanes per weight row (8/16/32/64), rows per lane group (1/2/4),
- * waves per workgroup (1..16; the three- to eight-row kernel with K slices as workgroups takes 3..8); 0 restores the built-in
- * heuristic. */
+/* GEMV launch-shape override for tuning sweeps: lanes per weight row (8/16/32/64), rows per lane group (1/2/4; the
+ * three- to eight-row kernel with K slices as workgroups reads it as: 1 = keep rows of up to 128 blocks whole, 2 = always cut
+ * them; the result bits are the same either way), waves per workgroup (1..16; that kernel takes 3..8); 0 restores the
+ * built-in heuristic. */
 int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_per_wg);
 /* Three to eight rows take their block sums from the matrix cores (v_mfma_i32_16x16x32_i8, same fp32 arithmetic around
  * them); path = 1 keeps every launch on the vector-ALU kernel, path = 2 keeps the K slices of a row tile in one workgroup

@@ -465,7 +465,7 @@ static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* part
     const size_t img = gemv_image_bytes(K);
     char* part = (workspace && ws_bytes > img) ? reinterpret_cast<char*>(workspace) + img : nullptr;
     const int rc = launch_gemv_mfk(wtype, x_dtype == MLLM_HIP_Q8_IMAGE ? GEMV_PREQ : x_dtype, MT, a, workspace, part,
-                                   part ? ws_bytes - img : 0, g_tune_NW, st);
+                                   part ? ws_bytes - img : 0, g_tune_NW, g_tune_R, st);
     if (rc != MFK_NOT_TAKEN) return rc;
   }
   if (mfma_rows && gemv_mfma_fits(MT, a.nb)) {

@@ -4,9 +4,13 @@
 // Same arithmetic and the same order of additions as that kernel (block sums with v_mfma_i32_16x16x64_i8, one fused
 // multiply-add per block into the lane that owns blocks = q mod 4, the four lanes as (0 + 1) + (2 + 3), then the slices
 // in slice order), so both give the same bits.  What differs is who does which part:
-//   * a workgroup holds `nwaves` row tiles of 16 weight rows and ONE K slice of at most 64 blocks.  It quantizes (or copies
-//     from the quantized image) only its slice of the activations: with eight rows of 9728 elements that is 320 blocks per
-//     workgroup instead of 2432, and the LDS footprint no longer grows with K;
+//   * a workgroup holds `nwaves` row tiles of 16 weight rows and ONE K slice (rows that are cut: at most 64 blocks).  It
+//     quantizes (or copies from the quantized image) only its slice of the activations: with eight rows of 9728 elements
+//     that is 320 blocks per workgroup instead of 2432, and the LDS footprint no longer grows with K;
+//   * a launch with enough row tiles to fill the chip by themselves keeps rows of up to 128 blocks whole (one slice, no
+//     partial sums): the workgroup then sums the row in the chains the slices would have been and adds them in slice order;
+//   * weight codes stream through a ring of MFK_CH chunk slots per wave: a slot is requested again as soon as its chunk has
+//     been staged, so a slice of any length keeps MFK_CH chunks of loads ahead of the arithmetic;
 //   * weight codes are requested as 8 rows x 128 contiguous bytes per load instruction (the operand layout of the MFMA,
 //     16 rows x 64 bytes per instruction, measured 25 % slower on the 4B shapes) and turned into the operand layout
 //     through a 2 KB LDS stage that belongs to the wave (no barrier: LDS operations of one wave execute in order);
@@ -18,10 +22,10 @@
 
 namespace mllmhip {
 
-constexpr int MFK_CH = 6;             // chunks of 8 blocks requested up front per trip
+constexpr int MFK_CH = 6;             // chunks of 8 blocks in flight per wave (a trip = one turn of the ring)
 constexpr int MFK_TRIP = 8 * MFK_CH;
 constexpr int MFK_STG = 16 * 9;       // 16-byte pieces of one stage: 16 rows, stride 9 (reads of 16 rows hit 16 bank groups)
-constexpr int MFK_MAX_NBS = 64;       // blocks per slice (weight scales of a slice: two 16-byte loads per lane)
+constexpr int MFK_MAX_NBS = 128;      // blocks per slice (weight scales of a slice: four 16-byte loads per lane)
 
 // Quantization of sixteen elements (half a block) by one lane of a pair; lanes 2 b and 2 b + 1 share block b.  The same
 // operations on the same values as quad_quantize (maximum of 32 magnitudes, the two IEEE divisions, v * id rounded to
@@ -53,6 +57,8 @@ struct MfkArgs {
   unsigned* counters;  // one per workgroup column (blockIdx.x), zero between launches (S > 1)
   int NP;              // columns of a partial row: every part's rows rounded up to 16
   int S, nbs;          // K slices; blocks per slice (a multiple of 8, at most MFK_MAX_NBS)
+  int vs;              // blocks per summation chain (a multiple of 8): S > 1: nbs; S == 1: the length the slices would have
+                       // had -- the chains of a whole row are added in slice order, so the bits do not depend on S
   int col0[GEMV_MAX_PARTS];  // first column of each part within a partial row
   int ipr_magic;             // ceil(2^20 / (2 nbs)): item / (items per row) as a multiply and a shift
 };
@@ -60,7 +66,7 @@ struct MfkArgs {
 template <int MT>
 static size_t mfk_lds_bytes(int wtype, int nbs, int nwaves) {
   const int rs = mf_row_stride(nbs);
-  return ((size_t)2 * MT * rs + nbs) * 16 + (size_t)MT * nbs * 8 +
+  return ((size_t)2 * MT * rs + nbs) * 16 + (size_t)MT * nbs * 20 +
          (size_t)nwaves * ((size_t)nbs * 64 + (size_t)MFK_STG * 16 * (wtype == MLLM_HIP_Q8_0 ? 2 : 1)) + 16;
 }
 
@@ -97,8 +103,9 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   u32x4* xlo = reinterpret_cast<u32x4*>(smem);  // [MT][rs] codes of elements 0..15 of (row, block of the slice)
   u32x4* xhi = xlo + (size_t)MT * rs;           // likewise elements 16..31
   u32x4* zrow = xhi + (size_t)MT * rs;          // [nbs] zeros: the operand of the lane groups that must not contribute
-  u32x2* xs = reinterpret_cast<u32x2*>(zrow + nbs);  // [MT][nbs] {effective scale, -8 * sum}
-  float* ws_all = reinterpret_cast<float*>(xs + (size_t)MT * nbs);
+  v4i_t* xn = reinterpret_cast<v4i_t*>(zrow + nbs);  // [MT][nbs] -8 * sum of the codes, four times: the MFMA's addend as it is read
+  float* xd = reinterpret_cast<float*>(xn + (size_t)MT * nbs);  // [MT][nbs] effective scale
+  float* ws_all = xd + (size_t)MT * nbs;
   float* ws = ws_all + (size_t)wave * nbs * 16;  // per wave [block][16 rows]
   u32x4* stg_all = reinterpret_cast<u32x4*>(ws_all + (size_t)nwaves * nbs * 16);
   u32x4* stg = stg_all + (size_t)wave * MFK_STG * NPL;
@@ -106,7 +113,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
 
   // ---- 1. activation requests (they return first; nothing here divides: the weight requests below must leave early) ------
   // raw activations: item it = tid + i * blockDim = sixteen elements, two neighbouring lanes share a block;
-  // image: thread (row tid / 64 + i * nwaves, block tid % 64)
+  // image: item it = tid + i * blockDim = (row it / 64, block it % 64) of the slice; slices of more than 64 blocks: 128
   const int ipr = nbs * 2;            // items of sixteen elements (half a block) per row of the slice
   const int nitems = MT * ipr;        // item it: row it / ipr, half block it % ipr (pairs of lanes stay whole: ipr % 2 == 0)
   constexpr int NXP = MT / 2;         // passes: the threads number at least 4 nbs (launcher), so MT * ipr / blockDim <= MT / 2
@@ -116,16 +123,19 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   const u32x4* img_hi = img_lo + mnb;
   const float* img_d = reinterpret_cast<const float*>(img_hi + mnb);
   const int* img_n8 = reinterpret_cast<const int*>(img_d + mnb);
-  constexpr int NIMG = (MT + 2) / 3;  // passes of one image row per wave (at least three waves)
-  const int ib = tid & 63, im = tid >> 6;
+  constexpr int NIMG = MT / 2;  // passes: at least three waves for up to 64 blocks, at least five for up to 128
+  const int imsh = nbs > 64 ? 7 : 6, nimg = MT << imsh;  // uniform
   u32x4 plo[NIMG], phi[NIMG];
   float pd[NIMG];
   int pn[NIMG];
   if (XT == GEMV_PREQ) {
 #pragma unroll
     for (int i = 0; i < NIMG; i++) {
-      const int it = min(im + i * nwaves, MT - 1) * nb + min(b0 + ib, nb - 1);
-      plo[i] = img_lo[it]; phi[i] = img_hi[it]; pd[i] = img_d[it]; pn[i] = img_n8[it];
+      if (i * nthreads < nimg) {  // uniform
+        const int item = tid + i * nthreads, im = item >> imsh, ib = item & ((1 << imsh) - 1);
+        const int it = min(im, MT - 1) * nb + min(b0 + ib, nb - 1);
+        plo[i] = img_lo[it]; phi[i] = img_hi[it]; pd[i] = img_d[it]; pn[i] = img_n8[it];
+      }
     }
   } else {
 #pragma unroll
@@ -141,12 +151,15 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
     }
   }
 
-  // ---- 2. weight scales of the tile and slice: 16-byte pieces of eight, lane (row lane / 8 + 8 i, piece lane % 8) -------
+  // ---- 2. weight scales of the tile and slice: 16-byte pieces of eight blocks, a row's pieces on neighbouring lanes ------
   const WRsrc wr = make_wrsrc(pt.w, WT, N, nb, nbp);
-  u32x4 sc[2];
+  // (slices of up to 64 blocks: 8 pieces per row, two loads; longer ones: 16 pieces per row, four loads)
+  const int scsh = nbs > 64 ? 4 : 3, nsc = nbs > 64 ? 4 : 2;  // uniform
+  u32x4 sc[4];
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
-    const int r = (lane >> 3) + 8 * i, cc = lane & 7;
+  for (int i = 0; i < 4; i++) {
+    if (i >= nsc) break;
+    const int r = (lane >> scsh) + (64 >> scsh) * i, cc = lane & ((1 << scsh) - 1);
     const bool ok = tile_ok && row0 + r < N && 8 * cc < nbs && b0 + 8 * cc < nbp;
     sc[i] = __builtin_amdgcn_raw_buffer_load_b128(wr.d, ok ? (uint32_t)(((int64_t)(row0 + r) * nbp + b0 + 8 * cc) * 2) : BUF_OOB, 0, BUF_NT);
   }
@@ -156,18 +169,17 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   // ---- 3. weight codes of a trip: chunk ch = 8 blocks, instruction i of it = rows 8 i .. 8 i + 7, 128 bytes of each --------
   const int lr = lane >> 3, lp = lane & 7;
   u32x4 wq[MFK_CH][2][NPL];
-  auto load_trip = [&](int bb) {
+  auto load_chunk = [&](int ch, int cb) {  // chunk slot ch <- the eight blocks from cb on (nothing is fetched past the slice)
 #pragma unroll
-    for (int ch = 0; ch < MFK_CH; ch++)
-#pragma unroll
-      for (int i = 0; i < 2; i++) {
-        const int r = row0 + 8 * i + lr, b = bb + 8 * ch + lp;
-        const uint32_t off = (tile_ok && r < N && b < b1) ? ((uint32_t)r * (uint32_t)nb + (uint32_t)b) * 16u : BUF_OOB;
-        wq[ch][i][0] = __builtin_amdgcn_raw_buffer_load_b128(wr.q0, off, 0, BUF_NT);
-        if (WT == MLLM_HIP_Q8_0) wq[ch][i][NPL - 1] = __builtin_amdgcn_raw_buffer_load_b128(wr.q1, off, 0, BUF_NT);
-      }
+    for (int i = 0; i < 2; i++) {
+      const int r = row0 + 8 * i + lr, b = cb + lp;
+      const uint32_t off = (tile_ok && r < N && b < b1) ? ((uint32_t)r * (uint32_t)nb + (uint32_t)b) * 16u : BUF_OOB;
+      wq[ch][i][0] = __builtin_amdgcn_raw_buffer_load_b128(wr.q0, off, 0, BUF_NT);
+      if (WT == MLLM_HIP_Q8_0) wq[ch][i][NPL - 1] = __builtin_amdgcn_raw_buffer_load_b128(wr.q1, off, 0, BUF_NT);
+    }
   };
-  load_trip(b0);
+#pragma unroll
+  for (int ch = 0; ch < MFK_CH; ch++) load_chunk(ch, b0 + 8 * ch);
   __asm__ volatile("" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
@@ -175,12 +187,14 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   if (XT == GEMV_PREQ) {
 #pragma unroll
     for (int i = 0; i < NIMG; i++) {
-      const int m = im + i * nwaves;
-      if (m < MT && ib < nbs) {
+      const int item = tid + i * nthreads, m = item >> imsh, ib = item & ((1 << imsh) - 1);
+      if (i * nthreads < nimg && m < MT && ib < nbs) {
         const bool live = b0 + ib < nb;  // the image has no blocks past the row
         xlo[(size_t)m * rs + ib] = live ? plo[i] : u32x4{0u, 0u, 0u, 0u};
         xhi[(size_t)m * rs + ib] = live ? phi[i] : u32x4{0u, 0u, 0u, 0u};
-        xs[(size_t)m * nbs + ib] = live ? u32x2{__float_as_uint(pd[i]), (uint32_t)pn[i]} : u32x2{0u, 0u};
+        const int n8 = (live && WT == MLLM_HIP_Q4_0) ? pn[i] : 0;
+        xn[(size_t)m * nbs + ib] = v4i_t{n8, n8, n8, n8};
+        xd[(size_t)m * nbs + ib] = live ? pd[i] : 0.f;
       }
     }
   } else {
@@ -206,15 +220,20 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
         int n8;
         pair_quantize(v, m < aM && b0 + b < nb, x86, codes, deff, n8);
         (j == 0 ? xlo : xhi)[(size_t)m * rs + b] = codes;
-        if (j == 0) xs[(size_t)m * nbs + b] = u32x2{__float_as_uint(deff), (uint32_t)n8};
+        if (j == 0) {
+          if (WT != MLLM_HIP_Q4_0) n8 = 0;  // nibbles are unsigned: sum((q - 8) x) = sum(q x) - 8 sum(x); Q8_0 codes are signed
+          xn[(size_t)m * nbs + b] = v4i_t{n8, n8, n8, n8};
+          xd[(size_t)m * nbs + b] = deff;
+        }
       }
     }
   }
   for (int i = tid; i < nbs; i += nthreads) zrow[i] = u32x4{0u, 0u, 0u, 0u};
   // weight scales -> fp32 [block of the slice][row]; blocks past the row are zero
 #pragma unroll
-  for (int i = 0; i < 2; i++) {
-    const int r = (lane >> 3) + 8 * i, cc = lane & 7;
+  for (int i = 0; i < 4; i++) {
+    if (i >= nsc) break;
+    const int r = (lane >> scsh) + (64 >> scsh) * i, cc = lane & ((1 << scsh) - 1);
     if (8 * cc < nbs) {
       const uint32_t wds[4] = {sc[i].x, sc[i].y, sc[i].z, sc[i].w};
 #pragma unroll
@@ -233,24 +252,54 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   f32x4 acc[TH];
 #pragma unroll
   for (int h = 0; h < TH; h++) acc[h] = f32x4{0.f, 0.f, 0.f, 0.f};
+  // the four lanes of an activation row (lane l + 4 j of a row of 16 lanes: blocks = j mod 4): (0 + 1) + (2 + 3), complete on
+  // the lanes with j == 0, the ones that store.  Shifts within the row of 16 on the vector ALU (lane l takes lane l + 4, then
+  // l + 8; a shuffle would be an LDS instruction in a loop that keeps LDS reads in flight)
+  auto across_lanes = [&]() {
+#pragma unroll
+    for (int h = 0; h < TH; h++) {
+      float v[4] = {acc[h].x, acc[h].y, acc[h].z, acc[h].w};
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        v[e] += dpp_f<0x104>(v[e]);  // row_shl:4
+        v[e] += dpp_f<0x108>(v[e]);  // row_shl:8
+      }
+      acc[h] = f32x4{v[0], v[1], v[2], v[3]};
+    }
+  };
+  f32x4 tot[TH];       // sum of the chains that are complete
+  bool have_tot = false;
+  int chain_end = b0 + k.vs;
   for (int bb = b0; bb < b1; bb += MFK_TRIP) {
-    if (bb != b0) load_trip(bb);
 #pragma unroll
     for (int ch = 0; ch < MFK_CH; ch++) {
       const int cb = bb + 8 * ch;  // first block of the chunk
       if (cb >= b1) break;         // uniform
+      if (cb == chain_end) {       // uniform; only whole rows (S == 1) get here
+        across_lanes();
+#pragma unroll
+        for (int h = 0; h < TH; h++) {
+          tot[h] = have_tot ? f32x4{tot[h].x + acc[h].x, tot[h].y + acc[h].y, tot[h].z + acc[h].z, tot[h].w + acc[h].w} : acc[h];
+          acc[h] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        have_tot = true;
+        chain_end += k.vs;
+      }
 #pragma unroll
       for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int p = 0; p < NPL; p++) stg[p * MFK_STG + (8 * i + lr) * 9 + lp] = wq[ch][i][p];
+        for (int p = 0; p < NPL; p++) {
+          stg[p * MFK_STG + (8 * i + lr) * 9 + lp] = wq[ch][i][p];
+        }
+      // the slot is free: the same chunk of the next trip takes it, MFK_CH chunks ahead of the arithmetic
+      if (cb + MFK_TRIP < b1) load_chunk(ch, cb + MFK_TRIP);  // uniform
       u32x4 Aw[2][NPL], Bl[2][TH], Bh[2][TH];
-      u32x2 sx[2][TH];
+      v4i_t nx[2][TH];
+      float dxs[2][TH];
       f32x4 dw[2];
-      bool live[2];
 #pragma unroll
       for (int jj = 0; jj < 2; jj++) {
         const int lb = cb - b0 + 4 * jj + q;  // this lane's block within the slice (inside the slice's LDS rows even when dead)
-        live[jj] = cb + 4 * jj + q < b1;
 #pragma unroll
         for (int p = 0; p < NPL; p++) Aw[jj][p] = stg[p * MFK_STG + c * 9 + 4 * jj + g];
         dw[jj] = *reinterpret_cast<const f32x4*>(ws + lb * 16 + 4 * g);
@@ -259,7 +308,8 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
           const int m = 4 * h + tt;
           Bl[jj][h] = mine ? xlo[(size_t)m * rs + lb] : zrow[lb];
           Bh[jj][h] = mine ? xhi[(size_t)m * rs + lb] : zrow[lb];
-          sx[jj][h] = xs[(size_t)m * nbs + lb];
+          nx[jj][h] = xn[(size_t)m * nbs + lb];
+          dxs[jj][h] = xd[(size_t)m * nbs + lb];
         }
       }
       v4i_t D[2][TH];
@@ -277,7 +327,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
         }
 #pragma unroll
         for (int h = 0; h < TH; h++) {
-          const v4i_t d = __builtin_amdgcn_mfma_i32_16x16x64_i8(Al, __builtin_bit_cast(v4i_t, Bl[jj][h]), v4i_t{0, 0, 0, 0}, 0, 0, 0);
+          const v4i_t d = __builtin_amdgcn_mfma_i32_16x16x64_i8(Al, __builtin_bit_cast(v4i_t, Bl[jj][h]), nx[jj][h], 0, 0, 0);
           D[jj][h] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ah, __builtin_bit_cast(v4i_t, Bh[jj][h]), d, 0, 0, 0);
         }
       }
@@ -285,25 +335,20 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
       for (int jj = 0; jj < 2; jj++)
 #pragma unroll
         for (int h = 0; h < TH; h++) {
-          const float dx = live[jj] ? __uint_as_float(sx[jj][h].x) : 0.f;
-          const int n8 = WT == MLLM_HIP_Q4_0 ? (int)sx[jj][h].y : 0;  // nibbles are unsigned: sum((q - 8) x) = sum(q x) - 8 sum(x)
-          acc[h].x = fmaf(dw[jj].x * dx, (float)(D[jj][h].x + n8), acc[h].x);
-          acc[h].y = fmaf(dw[jj].y * dx, (float)(D[jj][h].y + n8), acc[h].y);
-          acc[h].z = fmaf(dw[jj].z * dx, (float)(D[jj][h].z + n8), acc[h].z);
-          acc[h].w = fmaf(dw[jj].w * dx, (float)(D[jj][h].w + n8), acc[h].w);
+          // blocks past the row carry zero scales on both sides (sections 4), blocks past the slice are never in a chunk
+          const float dx = dxs[jj][h];
+          acc[h].x = fmaf(dw[jj].x * dx, (float)D[jj][h].x, acc[h].x);
+          acc[h].y = fmaf(dw[jj].y * dx, (float)D[jj][h].y, acc[h].y);
+          acc[h].z = fmaf(dw[jj].z * dx, (float)D[jj][h].z, acc[h].z);
+          acc[h].w = fmaf(dw[jj].w * dx, (float)D[jj][h].w, acc[h].w);
         }
     }
   }
-  // the four lanes of an activation row (blocks = 0, 1, 2, 3 mod 4): (0 + 1) + (2 + 3) on every lane
+  across_lanes();
+  if (have_tot) {
 #pragma unroll
-  for (int h = 0; h < TH; h++) {
-    float v[4] = {acc[h].x, acc[h].y, acc[h].z, acc[h].w};
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      v[e] += __shfl_xor(v[e], 4, 64);
-      v[e] += __shfl_xor(v[e], 8, 64);
-    }
-    acc[h] = f32x4{v[0], v[1], v[2], v[3]};
+    for (int h = 0; h < TH; h++)
+      acc[h] = f32x4{tot[h].x + acc[h].x, tot[h].y + acc[h].y, tot[h].z + acc[h].z, tot[h].w + acc[h].w};
   }
 
   const int n = row0 + 4 * g;  // lanes with q == 0 hold rows n .. n + 3 of activation row 4 h + tt

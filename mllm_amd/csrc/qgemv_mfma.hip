@@ -43,7 +43,8 @@ static int mfk_counter_block(const void* workspace, unsigned** out) {
   return MFK_NOT_TAKEN;
 }
 
-int gemv_mfk_slices(int nb) { return nb <= 8 * MFK_MAX_NBS ? mf_slices(nb) : (nb + MFK_MAX_NBS - 1) / MFK_MAX_NBS; }
+// slices of a row when it is cut: the ones of the one-workgroup kernel (at most eight) up to 512 blocks, then slices of 64
+int gemv_mfk_slices(int nb) { return nb <= 8 * 64 ? mf_slices(nb) : (nb + 63) / 64; }
 
 template <int WT, int XT, int MT>
 static int launch_mfk_t(const GemvArgs& a_in, const MfkArgs& k, int nwaves, unsigned grid_x, hipStream_t st) {
@@ -57,11 +58,22 @@ static int launch_mfk_t(const GemvArgs& a_in, const MfkArgs& k, int nwaves, unsi
 }
 
 int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const void* workspace, void* part, size_t part_bytes,
-                    int waves, hipStream_t st) {
+                    int waves, int slices, hipStream_t st) {
   GemvArgs a = a_in;
   MfkArgs k{};
+  int tiles_total = 0;
+  for (int p = 0; p < a.nparts; p++) tiles_total += (a.part[p].N + 15) / 16;
   k.S = gemv_mfk_slices(a.nb);
   k.nbs = ((a.nb + k.S - 1) / k.S + 7) / 8 * 8;
+  k.vs = k.nbs;
+  // a launch whose row tiles alone fill the chip keeps its rows whole where a slice may be that long: no partial sums, no
+  // second pass (gate + up of the 4B layer, 1216 tiles x 80 blocks: 10.6 -> 9.3 us at four rows, 12.7 -> 12.3 at eight;
+  // q+k+v, 384 tiles, is slower whole: 6.5 -> 8.6 / 8.2 -> 11.6).  The kernel still sums the row in chains of k.vs blocks
+  // and adds the chains in slice order: the same bits either way.  (slices: 1 = whole rows, 2 = never, for measurements)
+  if (a.nb <= MFK_MAX_NBS && (slices == 1 || (slices <= 0 && tiles_total >= 1024))) {
+    k.S = 1;
+    k.nbs = (a.nb + 7) / 8 * 8;
+  }
   if (k.nbs > MFK_MAX_NBS || k.S > 65535) return MFK_NOT_TAKEN;
   k.ipr_magic = ((1 << 20) + 2 * k.nbs - 1) / (2 * k.nbs);
   // Row tiles (= waves) per workgroup.  All workgroups are resident at once and every one costs vector-ALU time (its

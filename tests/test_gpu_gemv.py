@@ -318,12 +318,16 @@ def test_gemv_k_slices_as_workgroups_give_the_same_bits(wtype, M):
     L = _lib.lib()
     # Q8_0 at three or four rows: the comparison path is the vector-ALU kernel there (another order of the fp32 sums), and the
     # slice form is only taken for long rows
-    same_bits = not (wtype == 1 and M <= 4)
     for shapes in ([(9728, 2560), (9728, 2560)], [(2560, 9728)], [(4096, 2560), (1024, 2560), (1024, 2560)], [(2560, 4096)],
                    [(40, 96), (7, 96), (33, 96)], [(65, 32)], [(50, 161 * 32)], [(129, 41 * 32), (16, 41 * 32)],
                    # the longest rows the one-workgroup matrix-core kernel holds (two trips per slice at four rows)
-                   [(31, (512 if M <= 4 else 320) * 32)]):
+                   [(31, (512 if M <= 4 else 320) * 32)],
+                   # whole rows (below), ragged: 97 blocks, the last row tile with one row
+                   [(8200, 97 * 32), (8193, 97 * 32)]):
         K = shapes[0][1]
+        # (a launch of 1024 row tiles or more with rows of up to 128 blocks keeps its rows whole: one workgroup sums the
+        # chains the slices would have summed and adds them in slice order)
+        same_bits = not (wtype == 1 and M <= 4)
         Ws = [synth.make_weight(rng, wtype, n, K) for n, _ in shapes]
         ws = [ql.PackedQWeight(wtype, torch.from_numpy(W)) for W in Ws]
         biases = [to_dev(rng.standard_normal(n).astype(np.float32)) for n, _ in shapes]
