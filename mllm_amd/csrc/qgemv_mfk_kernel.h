@@ -22,7 +22,7 @@
 
 namespace mllmhip {
 
-constexpr int MFK_CH = 6;             // chunks of 8 blocks in flight per wave (a trip = one turn of the ring)
+constexpr int MFK_CH = 4;             // chunks of 8 blocks in flight per wave (a trip = one turn of the ring)
 constexpr int MFK_TRIP = 8 * MFK_CH;
 constexpr int MFK_STG = 16 * 9;       // 16-byte pieces of one stage: 16 rows, stride 9 (reads of 16 rows hit 16 bank groups)
 constexpr int MFK_MAX_NBS = 128;      // blocks per slice (weight scales of a slice: four 16-byte loads per lane)
@@ -66,7 +66,7 @@ struct MfkArgs {
 template <int MT>
 static size_t mfk_lds_bytes(int wtype, int nbs, int nwaves) {
   const int rs = mf_row_stride(nbs);
-  return ((size_t)2 * MT * rs + nbs) * 16 + (size_t)MT * nbs * 20 +
+  return ((size_t)2 * MT * rs + nbs) * 16 + (size_t)MT * nbs * 8 +
          (size_t)nwaves * ((size_t)nbs * 64 + (size_t)MFK_STG * 16 * (wtype == MLLM_HIP_Q8_0 ? 2 : 1)) + 16;
 }
 
@@ -103,9 +103,8 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   u32x4* xlo = reinterpret_cast<u32x4*>(smem);  // [MT][rs] codes of elements 0..15 of (row, block of the slice)
   u32x4* xhi = xlo + (size_t)MT * rs;           // likewise elements 16..31
   u32x4* zrow = xhi + (size_t)MT * rs;          // [nbs] zeros: the operand of the lane groups that must not contribute
-  v4i_t* xn = reinterpret_cast<v4i_t*>(zrow + nbs);  // [MT][nbs] -8 * sum of the codes, four times: the MFMA's addend as it is read
-  float* xd = reinterpret_cast<float*>(xn + (size_t)MT * nbs);  // [MT][nbs] effective scale
-  float* ws_all = xd + (size_t)MT * nbs;
+  u32x2* xs = reinterpret_cast<u32x2*>(zrow + nbs);  // [MT][nbs] {effective scale, -8 * sum of the codes (Q8_0: 0)}
+  float* ws_all = reinterpret_cast<float*>(xs + (size_t)MT * nbs);
   float* ws = ws_all + (size_t)wave * nbs * 16;  // per wave [block][16 rows]
   u32x4* stg_all = reinterpret_cast<u32x4*>(ws_all + (size_t)nwaves * nbs * 16);
   u32x4* stg = stg_all + (size_t)wave * MFK_STG * NPL;
@@ -154,11 +153,12 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   // ---- 2. weight scales of the tile and slice: 16-byte pieces of eight blocks, a row's pieces on neighbouring lanes ------
   const WRsrc wr = make_wrsrc(pt.w, WT, N, nb, nbp);
   // (slices of up to 64 blocks: 8 pieces per row, two loads; longer ones: 16 pieces per row, four loads)
-  const int scsh = nbs > 64 ? 4 : 3, nsc = nbs > 64 ? 4 : 2;  // uniform
+  const int nsc = nbs > 64 ? 4 : 2;  // uniform
   u32x4 sc[4];
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     if (i >= nsc) break;
+    const int scsh = nbs > 64 ? 4 : 3;
     const int r = (lane >> scsh) + (64 >> scsh) * i, cc = lane & ((1 << scsh) - 1);
     const bool ok = tile_ok && row0 + r < N && 8 * cc < nbs && b0 + 8 * cc < nbp;
     sc[i] = __builtin_amdgcn_raw_buffer_load_b128(wr.d, ok ? (uint32_t)(((int64_t)(row0 + r) * nbp + b0 + 8 * cc) * 2) : BUF_OOB, 0, BUF_NT);
@@ -193,8 +193,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
         xlo[(size_t)m * rs + ib] = live ? plo[i] : u32x4{0u, 0u, 0u, 0u};
         xhi[(size_t)m * rs + ib] = live ? phi[i] : u32x4{0u, 0u, 0u, 0u};
         const int n8 = (live && WT == MLLM_HIP_Q4_0) ? pn[i] : 0;
-        xn[(size_t)m * nbs + ib] = v4i_t{n8, n8, n8, n8};
-        xd[(size_t)m * nbs + ib] = live ? pd[i] : 0.f;
+        xs[(size_t)m * nbs + ib] = u32x2{live ? __float_as_uint(pd[i]) : 0u, (uint32_t)n8};
       }
     }
   } else {
@@ -222,8 +221,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
         (j == 0 ? xlo : xhi)[(size_t)m * rs + b] = codes;
         if (j == 0) {
           if (WT != MLLM_HIP_Q4_0) n8 = 0;  // nibbles are unsigned: sum((q - 8) x) = sum(q x) - 8 sum(x); Q8_0 codes are signed
-          xn[(size_t)m * nbs + b] = v4i_t{n8, n8, n8, n8};
-          xd[(size_t)m * nbs + b] = deff;
+          xs[(size_t)m * nbs + b] = u32x2{__float_as_uint(deff), (uint32_t)n8};
         }
       }
     }
@@ -233,6 +231,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
 #pragma unroll
   for (int i = 0; i < 4; i++) {
     if (i >= nsc) break;
+    const int scsh = nbs > 64 ? 4 : 3;
     const int r = (lane >> scsh) + (64 >> scsh) * i, cc = lane & ((1 << scsh) - 1);
     if (8 * cc < nbs) {
       const uint32_t wds[4] = {sc[i].x, sc[i].y, sc[i].z, sc[i].w};
@@ -294,8 +293,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
       // the slot is free: the same chunk of the next trip takes it, MFK_CH chunks ahead of the arithmetic
       if (cb + MFK_TRIP < b1) load_chunk(ch, cb + MFK_TRIP);  // uniform
       u32x4 Aw[2][NPL], Bl[2][TH], Bh[2][TH];
-      v4i_t nx[2][TH];
-      float dxs[2][TH];
+      u32x2 sx[2][TH];
       f32x4 dw[2];
 #pragma unroll
       for (int jj = 0; jj < 2; jj++) {
@@ -306,10 +304,11 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
 #pragma unroll
         for (int h = 0; h < TH; h++) {
           const int m = 4 * h + tt;
+          // (selecting the address costs less than reading under a lane mask: the branches that takes cut the chunk into
+          // pieces the instruction scheduler cannot mix; measured 3 % slower)
           Bl[jj][h] = mine ? xlo[(size_t)m * rs + lb] : zrow[lb];
           Bh[jj][h] = mine ? xhi[(size_t)m * rs + lb] : zrow[lb];
-          nx[jj][h] = xn[(size_t)m * nbs + lb];
-          dxs[jj][h] = xd[(size_t)m * nbs + lb];
+          sx[jj][h] = xs[(size_t)m * nbs + lb];
         }
       }
       v4i_t D[2][TH];
@@ -327,7 +326,8 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
         }
 #pragma unroll
         for (int h = 0; h < TH; h++) {
-          const v4i_t d = __builtin_amdgcn_mfma_i32_16x16x64_i8(Al, __builtin_bit_cast(v4i_t, Bl[jj][h]), nx[jj][h], 0, 0, 0);
+          const int n8 = (int)sx[jj][h].y;  // nibbles are unsigned: sum((q - 8) x) = sum(q x) - 8 sum(x)
+          const v4i_t d = __builtin_amdgcn_mfma_i32_16x16x64_i8(Al, __builtin_bit_cast(v4i_t, Bl[jj][h]), v4i_t{n8, n8, n8, n8}, 0, 0, 0);
           D[jj][h] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ah, __builtin_bit_cast(v4i_t, Bh[jj][h]), d, 0, 0, 0);
         }
       }
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
 #pragma unroll
         for (int h = 0; h < TH; h++) {
           // blocks past the row carry zero scales on both sides (sections 4), blocks past the slice are never in a chunk
-          const float dx = dxs[jj][h];
+          const float dx = __uint_as_float(sx[jj][h].x);
           acc[h].x = fmaf(dw[jj].x * dx, (float)D[jj][h].x, acc[h].x);
           acc[h].y = fmaf(dw[jj].y * dx, (float)D[jj][h].y, acc[h].y);
           acc[h].z = fmaf(dw[jj].z * dx, (float)D[jj][h].z, acc[h].z);
@@ -354,10 +354,28 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   const int n = row0 + 4 * g;  // lanes with q == 0 hold rows n .. n + 3 of activation row 4 h + tt
   if (S == 1) {
     if (!tile_ok || q != 0) return;
+    // rows of a multiple of four outputs, 16-byte aligned pointers: 16 bytes per lane, the four lanes of an activation row
+    // write one 64-byte line
+    const bool vec = (N & 3) == 0 && ((reinterpret_cast<uintptr_t>(pt.y) | reinterpret_cast<uintptr_t>(pt.bias) |
+                                       reinterpret_cast<uintptr_t>(pt.residual)) & 15) == 0;  // uniform
 #pragma unroll
     for (int h = 0; h < TH; h++) {
       const int t = 4 * h + tt;
       if (t >= aM) continue;
+      if (vec) {
+        if (n >= N) continue;  // (n and N are multiples of four: n < N means n + 3 < N)
+        f32x4 o = acc[h];
+        if (pt.bias) {
+          const f32x4 bv = *reinterpret_cast<const f32x4*>(pt.bias + n);
+          o = f32x4{bv.x + o.x, bv.y + o.y, bv.z + o.z, bv.w + o.w};
+        }
+        if (pt.residual) {
+          const f32x4 rv = *reinterpret_cast<const f32x4*>(pt.residual + (int64_t)t * N + n);
+          o = f32x4{o.x + rv.x, o.y + rv.y, o.z + rv.z, o.w + rv.w};
+        }
+        *reinterpret_cast<f32x4*>(pt.y + (int64_t)t * N + n) = o;
+        continue;
+      }
       const float v[4] = {acc[h].x, acc[h].y, acc[h].z, acc[h].w};
       float* yrow = pt.y + (int64_t)t * N;
 #pragma unroll
