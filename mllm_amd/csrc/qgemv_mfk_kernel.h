@@ -71,7 +71,8 @@ static size_t mfk_lds_bytes(int wtype, int nbs, int nwaves) {
 }
 
 // blockDim = 64 x (row tiles per workgroup): three to eight waves, at least nbs / 16 (the threads hold one pass of
-// quantization items per activation row)
+// quantization items per activation row).  Waves beyond the row tiles that only help to quantize were measured: slower
+// (gate + up of the 4B layer at eight rows 11.6 -> 12.2 us with ten waves instead of five).
 template <int WT, int XT, int MT>
 __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   extern __shared__ __align__(16) unsigned char smem[];
@@ -269,81 +270,91 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   f32x4 tot[TH];       // sum of the chains that are complete
   bool have_tot = false;
   int chain_end = b0 + k.vs;
-  for (int bb = b0; bb < b1; bb += MFK_TRIP) {
+  const int we = tile_ok ? b1 : b0;                    // a wave without a row tile has no chunks
+  const int b1r = b0 + (max(we - b0, 0) + 7) / 8 * 8;  // the end of the wave's blocks rounded up to whole chunks
+  // One chunk: slot ch of the ring holds blocks cb .. cb + 7.  The loop below runs whole trips with nothing conditional
+  // between the requests, and the chunks of a last, partial trip follow as straight-line code: the compiler's wait counts have
+  // to hold for every path that reaches a wait, and with an exit (or a skipped request) inside the loop body they came out as
+  // "wait for all loads" at the head of every trip.
+  auto chunk = [&](const int ch, const int cb, const bool refill) {
+    if (cb == chain_end) {       // uniform; only whole rows (S == 1) get here
+      across_lanes();
 #pragma unroll
-    for (int ch = 0; ch < MFK_CH; ch++) {
-      const int cb = bb + 8 * ch;  // first block of the chunk
-      if (cb >= b1) break;         // uniform
-      if (cb == chain_end) {       // uniform; only whole rows (S == 1) get here
-        across_lanes();
-#pragma unroll
-        for (int h = 0; h < TH; h++) {
-          tot[h] = have_tot ? f32x4{tot[h].x + acc[h].x, tot[h].y + acc[h].y, tot[h].z + acc[h].z, tot[h].w + acc[h].w} : acc[h];
-          acc[h] = f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-        have_tot = true;
-        chain_end += k.vs;
+      for (int h = 0; h < TH; h++) {
+        tot[h] = have_tot ? f32x4{tot[h].x + acc[h].x, tot[h].y + acc[h].y, tot[h].z + acc[h].z, tot[h].w + acc[h].w} : acc[h];
+        acc[h] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
-#pragma unroll
-      for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int p = 0; p < NPL; p++) {
-          stg[p * MFK_STG + (8 * i + lr) * 9 + lp] = wq[ch][i][p];
-        }
-      // the slot is free: the same chunk of the next trip takes it, MFK_CH chunks ahead of the arithmetic
-      if (cb + MFK_TRIP < b1) load_chunk(ch, cb + MFK_TRIP);  // uniform
-      u32x4 Aw[2][NPL], Bl[2][TH], Bh[2][TH];
-      u32x2 sx[2][TH];
-      f32x4 dw[2];
-#pragma unroll
-      for (int jj = 0; jj < 2; jj++) {
-        const int lb = cb - b0 + 4 * jj + q;  // this lane's block within the slice (inside the slice's LDS rows even when dead)
-#pragma unroll
-        for (int p = 0; p < NPL; p++) Aw[jj][p] = stg[p * MFK_STG + c * 9 + 4 * jj + g];
-        dw[jj] = *reinterpret_cast<const f32x4*>(ws + lb * 16 + 4 * g);
-#pragma unroll
-        for (int h = 0; h < TH; h++) {
-          const int m = 4 * h + tt;
-          // (selecting the address costs less than reading under a lane mask: the branches that takes cut the chunk into
-          // pieces the instruction scheduler cannot mix; measured 3 % slower)
-          Bl[jj][h] = mine ? xlo[(size_t)m * rs + lb] : zrow[lb];
-          Bh[jj][h] = mine ? xhi[(size_t)m * rs + lb] : zrow[lb];
-          sx[jj][h] = xs[(size_t)m * nbs + lb];
-        }
-      }
-      v4i_t D[2][TH];
-#pragma unroll
-      for (int jj = 0; jj < 2; jj++) {
-        v4i_t Al, Ah;
-        if (WT == MLLM_HIP_Q4_0) {
-          const u32x4 w = Aw[jj][0];
-          Al = v4i_t{(int)(w.x & 0x0f0f0f0fu), (int)(w.y & 0x0f0f0f0fu), (int)(w.z & 0x0f0f0f0fu), (int)(w.w & 0x0f0f0f0fu)};
-          Ah = v4i_t{(int)((w.x >> 4) & 0x0f0f0f0fu), (int)((w.y >> 4) & 0x0f0f0f0fu), (int)((w.z >> 4) & 0x0f0f0f0fu),
-                     (int)((w.w >> 4) & 0x0f0f0f0fu)};
-        } else {
-          Al = __builtin_bit_cast(v4i_t, Aw[jj][0]);
-          Ah = __builtin_bit_cast(v4i_t, Aw[jj][NPL - 1]);
-        }
-#pragma unroll
-        for (int h = 0; h < TH; h++) {
-          const int n8 = (int)sx[jj][h].y;  // nibbles are unsigned: sum((q - 8) x) = sum(q x) - 8 sum(x)
-          const v4i_t d = __builtin_amdgcn_mfma_i32_16x16x64_i8(Al, __builtin_bit_cast(v4i_t, Bl[jj][h]), v4i_t{n8, n8, n8, n8}, 0, 0, 0);
-          D[jj][h] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ah, __builtin_bit_cast(v4i_t, Bh[jj][h]), d, 0, 0, 0);
-        }
-      }
-#pragma unroll
-      for (int jj = 0; jj < 2; jj++)
-#pragma unroll
-        for (int h = 0; h < TH; h++) {
-          // blocks past the row carry zero scales on both sides (sections 4), blocks past the slice are never in a chunk
-          const float dx = __uint_as_float(sx[jj][h].x);
-          acc[h].x = fmaf(dw[jj].x * dx, (float)D[jj][h].x, acc[h].x);
-          acc[h].y = fmaf(dw[jj].y * dx, (float)D[jj][h].y, acc[h].y);
-          acc[h].z = fmaf(dw[jj].z * dx, (float)D[jj][h].z, acc[h].z);
-          acc[h].w = fmaf(dw[jj].w * dx, (float)D[jj][h].w, acc[h].w);
-        }
+      have_tot = true;
+      chain_end += k.vs;
     }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+      for (int p = 0; p < NPL; p++) {
+        stg[p * MFK_STG + (8 * i + lr) * 9 + lp] = wq[ch][i][p];
+      }
+    // the slot is free: the same chunk of the next trip takes it, MFK_CH chunks ahead of the arithmetic (past the slice the
+    // offsets are out of range and nothing is fetched)
+    if (refill) load_chunk(ch, cb + MFK_TRIP);
+    u32x4 Aw[2][NPL], Bl[2][TH], Bh[2][TH];
+    u32x2 sx[2][TH];
+    f32x4 dw[2];
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++) {
+      const int lb = cb - b0 + 4 * jj + q;  // this lane's block within the slice (inside the slice's LDS rows even when dead)
+#pragma unroll
+      for (int p = 0; p < NPL; p++) Aw[jj][p] = stg[p * MFK_STG + c * 9 + 4 * jj + g];
+      dw[jj] = *reinterpret_cast<const f32x4*>(ws + lb * 16 + 4 * g);
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        const int m = 4 * h + tt;
+        // (selecting the address costs less than reading under a lane mask: the branches that takes cut the chunk into
+        // pieces the instruction scheduler cannot mix; measured 3 % slower)
+        Bl[jj][h] = mine ? xlo[(size_t)m * rs + lb] : zrow[lb];
+        Bh[jj][h] = mine ? xhi[(size_t)m * rs + lb] : zrow[lb];
+        sx[jj][h] = xs[(size_t)m * nbs + lb];
+      }
+    }
+    v4i_t D[2][TH];
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++) {
+      v4i_t Al, Ah;
+      if (WT == MLLM_HIP_Q4_0) {
+        const u32x4 w = Aw[jj][0];
+        Al = v4i_t{(int)(w.x & 0x0f0f0f0fu), (int)(w.y & 0x0f0f0f0fu), (int)(w.z & 0x0f0f0f0fu), (int)(w.w & 0x0f0f0f0fu)};
+        Ah = v4i_t{(int)((w.x >> 4) & 0x0f0f0f0fu), (int)((w.y >> 4) & 0x0f0f0f0fu), (int)((w.z >> 4) & 0x0f0f0f0fu),
+                   (int)((w.w >> 4) & 0x0f0f0f0fu)};
+      } else {
+        Al = __builtin_bit_cast(v4i_t, Aw[jj][0]);
+        Ah = __builtin_bit_cast(v4i_t, Aw[jj][NPL - 1]);
+      }
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        const int n8 = (int)sx[jj][h].y;  // nibbles are unsigned: sum((q - 8) x) = sum(q x) - 8 sum(x)
+        const v4i_t d = __builtin_amdgcn_mfma_i32_16x16x64_i8(Al, __builtin_bit_cast(v4i_t, Bl[jj][h]), v4i_t{n8, n8, n8, n8}, 0, 0, 0);
+        D[jj][h] = __builtin_amdgcn_mfma_i32_16x16x64_i8(Ah, __builtin_bit_cast(v4i_t, Bh[jj][h]), d, 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int jj = 0; jj < 2; jj++)
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        // blocks past the row carry zero scales on both sides (sections 4), blocks past the slice are never in a chunk
+        const float dx = __uint_as_float(sx[jj][h].x);
+        acc[h].x = fmaf(dw[jj].x * dx, (float)D[jj][h].x, acc[h].x);
+        acc[h].y = fmaf(dw[jj].y * dx, (float)D[jj][h].y, acc[h].y);
+        acc[h].z = fmaf(dw[jj].z * dx, (float)D[jj][h].z, acc[h].z);
+        acc[h].w = fmaf(dw[jj].w * dx, (float)D[jj][h].w, acc[h].w);
+      }
+  };
+  int cb0 = b0;
+  for (; cb0 + MFK_TRIP <= b1r; cb0 += MFK_TRIP) {
+#pragma unroll
+    for (int ch = 0; ch < MFK_CH; ch++) chunk(ch, cb0 + 8 * ch, true);
   }
+#pragma unroll
+  for (int ch = 0; ch < MFK_CH - 1; ch++)
+    if (cb0 + 8 * ch < we) chunk(ch, cb0 + 8 * ch, false);  // uniform
   across_lanes();
   if (have_tot) {
 #pragma unroll
