@@ -105,13 +105,14 @@ size_t mllm_hip_gemv_splitk_workspace_bytes(int M, int64_t K, int64_t N_total);
 int mllm_hip_linear_q_gemv_multi_wsn(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M,
                                      int64_t K, int act_scale_mode, void* workspace, size_t workspace_bytes, void* stream);
 
-/* mllm_hip_linear_q_gemv_multi_ws without a workspace argument and without any allocation.  No counterpart in the
+/* mllm_hip_linear_q_gemv_multi_wsn without a workspace argument and without any allocation.  No counterpart in the
  * reference; it exists for callers that cannot allocate device memory or carry a workspace around: code under HIP graph
- * capture, tight serving loops, harnesses that forbid hipMalloc.  The quantized image of the activations lives in a
- * static device array of the library (320 KB per GPU, held until the process ends), whose per-device address
- * mllm_hip_init(device) looks up (otherwise the first call on a device does, which is not allowed during capture).
- * Same arguments, same results bit for bit.  K <= 32768, else MLLM_HIP_E_SHAPE.  Every call on a GPU shares that GPU's
- * array: calls that overlap on one GPU (different streams) race; calls on one stream are ordered and safe. */
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  The workspace is a static device array of the library
+ * (327 680 bytes per GPU, held until the process ends: the quantized image of the activations and, where they fit behind
+ * it, the partial sums of the K slices), whose per-device address mllm_hip_init(device) looks up (otherwise the first call
+ * on a device does, which is not allowed during capture).  Same arguments otherwise, same results bit for bit as that call
+ * with a workspace of 327 680 bytes.  K <= 32768, else MLLM_HIP_E_SHAPE.  Every call on a GPU shares that GPU's array:
+ * calls that overlap on one GPU (different streams) race; calls on one stream are ordered and safe. */
 int mllm_hip_linear_q_gemv_multi_static(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,
                                         int M, int64_t K, int act_scale_mode, void* stream);
 

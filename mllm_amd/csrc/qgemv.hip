@@ -449,21 +449,24 @@ static int gemv_multi_pass(int wtype, int nparts, const mllm_hip_gemv_part* part
   const int MT = M <= 1 ? 1 : (M <= 2 ? 2 : (M <= 4 ? 4 : 8));
   GemvShape s = pick_shape(MT, nmax, a.nb);
   hipStream_t st = (hipStream_t)stream;
-  // three or more rows: block sums on the matrix cores (as long as the rows fit that kernel's LDS: 8 rows of 11 000 elements)
-  // Q8_0 (twice the code bytes per block) gains only from five rows on.  The rule looks at the weight type, the number of
-  // rows and the row length, never at the number of weight rows: a matrix takes the same kernel alone and in a multi launch.
-  // Q8_0 with three or four rows is faster on the vector ALU for rows of up to a few thousand elements (gate + up of the 4B
-  // layer 16.7 against 17.9 us, q+k+v 8.1 / 8.5) and slower for long ones (down, 9728 elements: 13.0 / 10.0)
-  const bool long_rows = a.nb >= 256;
-  const bool mfma_rows = MT >= 4 && g_gemv_path != 1 && (wtype == MLLM_HIP_Q4_0 || MT == 8);
-  const bool mfk_rows = mfma_rows || (MT >= 4 && g_gemv_path != 1 && long_rows);
+  // three or more rows: block sums on the matrix cores.  The rule looks at the weight type, the number of rows and the row
+  // length, never at the number of weight rows: a matrix takes the same kernel alone and in a multi launch.
+  // The form with K slices as workgroups (below) is the fastest for both formats wherever it can run (Q8_0 at four rows, 4B
+  // layer: gate + up 12.2 us against 16.6 on the vector ALU, down 9.2 / 13.0, q+k+v 7.5 / 7.9, o 6.9 / 7.5).  Where it cannot
+  // (no room for partial sums), Q4_0 and Q8_0 at five rows or more take the one-workgroup matrix-core kernel (as long as the
+  // rows fit its LDS: 8 rows of 11 000 elements), Q8_0 at three or four rows the vector-ALU kernel (down 13.0 against 15.4).
+  const bool mfk_rows = MT >= 4 && g_gemv_path != 1;
+  const bool mfma_rows = mfk_rows && (wtype == MLLM_HIP_Q4_0 || MT == 8);
   const int waves = (g_tune_NW == 2 || g_tune_NW == 4 || g_tune_NW == 8) ? g_tune_NW : 0;
   // K slices as separate workgroups, each quantizing only its slice of x (one launch, same bits, no limit on the row length
   // from LDS): needs room for the slices' partial sums behind the image area of the workspace; falls through where that
   // room is missing
-  if (mfk_rows && g_gemv_path != 2) {
-    const size_t img = gemv_image_bytes(K);
-    char* part = (workspace && ws_bytes > img) ? reinterpret_cast<char*>(workspace) + img : nullptr;
+  // (Q8_0 at three or four rows only when the caller has given that room, also for a launch that would not need it: its
+  // other kernel, the vector-ALU one, adds the blocks in another order, and the bits of a matrix must not depend on what
+  // else is in the launch)
+  const size_t img = gemv_image_bytes(K);
+  char* part = (workspace && ws_bytes > img) ? reinterpret_cast<char*>(workspace) + img : nullptr;
+  if (mfk_rows && g_gemv_path != 2 && (mfma_rows || part)) {
     const int rc = launch_gemv_mfk(wtype, x_dtype == MLLM_HIP_Q8_IMAGE ? GEMV_PREQ : x_dtype, MT, a, workspace, part,
                                    part ? ws_bytes - img : 0, g_tune_NW, g_tune_R, st);
     if (rc != MFK_NOT_TAKEN) return rc;

@@ -316,8 +316,8 @@ def test_gemv_k_slices_as_workgroups_give_the_same_bits(wtype, M):
     one to eight slices; and against the oracle."""
     rng = synth.rng_for(1, 900 + M + 10 * wtype)
     L = _lib.lib()
-    # Q8_0 at three or four rows: the comparison path is the vector-ALU kernel there (another order of the fp32 sums), and the
-    # slice form is only taken for long rows
+    # Q8_0 at three or four rows: the comparison path (no slice form) is the vector-ALU kernel there, which adds the blocks
+    # of a row in another order
     for shapes in ([(9728, 2560), (9728, 2560)], [(2560, 9728)], [(4096, 2560), (1024, 2560), (1024, 2560)], [(2560, 4096)],
                    [(40, 96), (7, 96), (33, 96)], [(65, 32)], [(50, 161 * 32)], [(129, 41 * 32), (16, 41 * 32)],
                    # the longest rows the one-workgroup matrix-core kernel holds (two trips per slice at four rows)

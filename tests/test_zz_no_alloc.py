@@ -1,7 +1,8 @@
-"""The entry point that allocates nothing (mllm_hip_linear_q_gemv_multi_static): its quantized-activation image lives in
-a static device array of the library instead of a caller-provided workspace.  Called through the C ABI and compared bit
-for bit with the entry point it is a variant of (mllm_hip_linear_q_gemv_multi_ws), on two calls in a row, the second
-with a smaller input, which must not see anything the first one left in the array."""
+"""The entry point that allocates nothing (mllm_hip_linear_q_gemv_multi_static): its workspace (the quantized-activation
+image and, where they fit, the partial sums of the K slices) is a static device array of the library instead of a
+caller-provided buffer.  Called through the C ABI and compared bit for bit with the entry point it is a variant of
+(mllm_hip_linear_q_gemv_multi_wsn with a workspace of the array's size), on two calls in a row, the second with a smaller
+input, which must not see anything the first one left in the array."""
 import ctypes as C
 
 import numpy as np
@@ -12,6 +13,8 @@ from mllm_amd import _lib, qlinear as ql, synth
 from gpu_util import announce, bf16_dev, to_dev
 
 pytestmark = pytest.mark.gpu
+
+STATIC_BYTES = 327680  # the library's static array (include/mllm_hip_qlinear.h)
 
 
 def _both(wtype, Ws, bits_or_x, M, K, is_bf16):
@@ -30,9 +33,9 @@ def _both(wtype, Ws, bits_or_x, M, K, is_bf16):
             rc = L.mllm_hip_linear_q_gemv_multi_static(wtype, len(ws), parts, x.data_ptr(), 1 if is_bf16 else 0, M, K,
                                                        ql.SCALE_X86_REF, stream)
         else:
-            work = ql.gemv_workspace(M, K)
-            rc = L.mllm_hip_linear_q_gemv_multi_ws(wtype, len(ws), parts, x.data_ptr(), 1 if is_bf16 else 0, M, K,
-                                                   ql.SCALE_X86_REF, work.data_ptr(), stream)
+            work = torch.empty(STATIC_BYTES, dtype=torch.uint8, device="cuda")  # the size of the library's static array
+            rc = L.mllm_hip_linear_q_gemv_multi_wsn(wtype, len(ws), parts, x.data_ptr(), 1 if is_bf16 else 0, M, K,
+                                                    ql.SCALE_X86_REF, work.data_ptr(), STATIC_BYTES, stream)
         assert rc == 0, rc
         torch.cuda.synchronize()
         outs.append([y.cpu().numpy() for y in ys])
