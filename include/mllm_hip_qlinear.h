@@ -327,7 +327,7 @@ int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed
 /* The same expert FFN with the experts in the super-block formats (MLLM_HIP_Q4_K / MLLM_HIP_Q6_K, the formats the shipped
  * Qwen3-MoE recipe quantizes to; activations Q8_K in front of every projection): gate_packed / up_packed / down_packed are E
  * matrices packed by mllm_hip_kq_prepack back to back, mllm_hip_kq_packed_bytes(wtype, I, H) resp. (wtype, H, I) apart.
- * H % 256 == 0, I % 256 == 0, T * k <= 65535, E <= 3072.  Up to two (token, expert) pairs per expert every pair runs as one
+ * H % 256 == 0, I % 256 == 0, T * k <= 65535, E <= 3072.  Up to one (token, expert) pair per expert (Q6_K: half) every pair runs as one
  * GEMV row (three or four launches; the decode form, an expert's weights are read once per pair that uses it).  Beyond that
  * the pairs are sorted by expert and run as tiles of eight rows on the matrix cores (the grouped form: x and h quantized
  * to Q8_K once, an expert's weights read once per eight pairs; seven launches), same arithmetic.

@@ -717,7 +717,7 @@ static int launch_kq(const KGemvArgs& a, hipStream_t st) {
 // the reference's sum (vec_dot_q4_K_q8_K: integer sums per super-block, then d*dx and dmin*dx) regrouped; the integer parts
 // are exact, the fp32 roundings differ in order only.
 typedef int kv4i __attribute__((ext_vector_type(4)));
-constexpr int KMF_NG = 10;  // groups of four sub-blocks per trip
+constexpr int KMF_NG = 10;  // groups of four sub-blocks per trip, at most (the launcher takes 6 or 8 for shorter slices)
 
 static int kmf_slices(int nb32) {
   int s = 1;
@@ -727,12 +727,16 @@ static int kmf_slices(int nb32) {
 
 // blockDim = nwaves * 64; a workgroup holds nwaves / S row tiles (16 weight rows), S K-slices each; nbs = sub-blocks per slice
 // (a multiple of 8: whole super-blocks).
-// LDS: xc [nb32 + 40][MT] 32 bytes: the 32 codes of (sub-block, row); xs [nb32 + 40][MT] {dx, sum of the 32 codes};
-//      one zero record; ws per wave [whole trips][16 rows] fp32 d*sc, then the same of dmin*m; red per wave [64] four sums
-template <int XT, int MT>
-__global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, int nbs) {
+// LDS: xc [nb32 + xpad][MT] 32 bytes: the 32 codes of (sub-block, row); xs [nb32 + xpad][MT] {dx, sum of the 32 codes}
+//      (xpad = how far the last trip of the last slice reaches past the row: zeros); one zero record;
+//      ws per wave [whole trips][16 rows] fp32 d*sc, then the same of dmin*m (after the loop: the wave's four sums for the
+//      wave of slice 0).
+// NG = groups of four sub-blocks per trip: the slice in one trip where it fits (6, 8 or 10), so that neither registers nor
+// LDS rows are held for sub-blocks the slice does not have -- with K = 2048 three workgroups fit a CU instead of two.
+template <int XT, int MT, int NG = KMF_NG>
+__global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, int nbs, int xpad) {
   extern __shared__ __align__(16) unsigned char smem[];
-  constexpr int TRIP = 4 * KMF_NG;
+  constexpr int TRIP = 4 * NG;
   const int nsb = a.nsb, nb32 = nsb * 8, K = nsb * QK_K;
   const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x, nwaves = nthreads >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -753,12 +757,12 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
 
   const int wsb = (nbs + TRIP - 1) / TRIP * TRIP;
   u32x4* xc = reinterpret_cast<u32x4*>(smem);                        // [(sb * MT + m) * 2 + half]
-  u32x4* zrec = xc + (size_t)(nb32 + TRIP) * MT * 2;
+  u32x4* zrec = xc + (size_t)(nb32 + xpad) * MT * 2;
   u32x2* xs = reinterpret_cast<u32x2*>(zrec + 1);                    // [sb * MT + m]
-  float* ws_all = reinterpret_cast<float*>(xs + (size_t)(nb32 + TRIP) * MT);
+  float* ws_all = reinterpret_cast<float*>(xs + (size_t)(nb32 + xpad) * MT);
   float* ws_ds = ws_all + (size_t)wave * 2 * wsb * 16;
   float* ws_dm = ws_ds + (size_t)wsb * 16;
-  f32x4* red = reinterpret_cast<f32x4*>(ws_all + (size_t)nwaves * 2 * wsb * 16) + (size_t)wave * 64;
+  f32x4* red = reinterpret_cast<f32x4*>(ws_ds);  // the wave's scale table, dead after the loop (2 wsb x 64 bytes >= 1 KB)
 
   // ---- 1. weight scale records of the tile and slice: one 16-byte record per (row, super-block) --------------------------
   const uint32_t sbt = (uint32_t)N * (uint32_t)nsb;
@@ -782,10 +786,10 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
   const int c = lane & 15, g = lane >> 4;
   const bool row_ok = tile_ok && row0 + c < N;
   const uint32_t rbase = (uint32_t)(row0 + c) * (uint32_t)nb32;
-  u32x4 wq[KMF_NG];
+  u32x4 wq[NG];
   auto load_groups = [&](int bb) {
 #pragma unroll
-    for (int j = 0; j < KMF_NG; j++) {
+    for (int j = 0; j < NG; j++) {
       const int b = bb + 4 * j + g;
       wq[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, (row_ok && b < b1) ? (rbase + (uint32_t)b) * 16u : KBUF_OOB, 0, KBUF_NT);
     }
@@ -826,8 +830,8 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
     }
   }
   if (tid == 0) zrec[0] = u32x4{0u, 0u, 0u, 0u};
-  for (int i = tid; i < TRIP * MT * 2; i += nthreads) xc[(size_t)nb32 * MT * 2 + i] = u32x4{0u, 0u, 0u, 0u};
-  for (int i = tid; i < TRIP * MT; i += nthreads) xs[(size_t)nb32 * MT + i] = u32x2{0u, 0u};
+  for (int i = tid; i < xpad * MT * 2; i += nthreads) xc[(size_t)nb32 * MT * 2 + i] = u32x4{0u, 0u, 0u, 0u};
+  for (int i = tid; i < xpad * MT; i += nthreads) xs[(size_t)nb32 * MT + i] = u32x2{0u, 0u};
   // weight scales: fp32 d*sc and dmin*m per (sub-block of the slice, row); zero past the row and in the rest of the last trip
 #pragma unroll
   for (int k = 0; k < 2; k++) {
@@ -904,15 +908,15 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
     };
     fetch_b(0, 0);
 #pragma unroll
-    for (int j = 0; j < KMF_NG; j++) {
+    for (int j = 0; j < NG; j++) {
       issue(j & 1, j);
-      if (j + 1 < KMF_NG) fetch_b((j + 1) & 1, j + 1);
+      if (j + 1 < NG) fetch_b((j + 1) & 1, j + 1);
       fetch_s(j & 1, j);
       __builtin_amdgcn_sched_barrier(0);
       if (j > 0) scale((j - 1) & 1, j - 1);
       __builtin_amdgcn_sched_barrier(0);
     }
-    scale((KMF_NG - 1) & 1, KMF_NG - 1);
+    scale((NG - 1) & 1, NG - 1);
   }
   {  // the two lanes of an activation row (sub-blocks = 0,1 and 2,3 mod 4)
     acc.x += __shfl_xor(acc.x, 8, 64);
@@ -927,7 +931,7 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
     __syncthreads();
     if (slice != 0) return;
     for (int s = 1; s < S; s++) {
-      const f32x4 o = red[(size_t)s * 64 + lane];
+      const f32x4 o = reinterpret_cast<const f32x4*>(ws_ds + (size_t)s * 2 * wsb * 16)[lane];  // the table of wave + s
       acc.x += o.x; acc.y += o.y; acc.z += o.z; acc.w += o.w;
     }
   }
@@ -940,18 +944,29 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
     if (n + e < N) yrow[n + e] = pt.bias ? v[e] + pt.bias[n + e] : v[e];
 }
 
+static int kmf_groups(int nbs) { return nbs <= 24 ? 6 : (nbs <= 32 ? 8 : KMF_NG); }
+// how far the last trip of a slice reads past the row's nb32 sub-blocks (whole trips from the slice's first sub-block)
+static int kmf_xpad(int nb32, int S, int nbs) {
+  const int trip = 4 * kmf_groups(nbs);
+  int pad = 0;
+  for (int s = 0; s < S; s++) {
+    const int b0 = s * nbs, b1 = std::min(nb32, b0 + nbs);
+    if (b1 > b0) pad = std::max(pad, b0 + ((b1 - b0 - 1) / trip + 1) * trip - nb32);
+  }
+  return pad;
+}
 template <int MT>
-static size_t kmf_lds_bytes(int nb32, int nbs, int nwaves) {
-  const int trip = 4 * KMF_NG;
-  const int wsb = (nbs + trip - 1) / trip * trip;
-  return (size_t)(nb32 + trip) * MT * 32 + 16 + (size_t)(nb32 + trip) * MT * 8 + (size_t)nwaves * 2 * wsb * 64 + (size_t)nwaves * 1024;
+static size_t kmf_lds_bytes(int nb32, int nbs, int nwaves, int S) {
+  const int trip = 4 * kmf_groups(nbs);
+  const int wsb = (nbs + trip - 1) / trip * trip, rows = nb32 + kmf_xpad(nb32, S, nbs);
+  return (size_t)rows * MT * 32 + 16 + (size_t)rows * MT * 8 + (size_t)nwaves * 2 * wsb * 64;
 }
 static bool kq4_mfma_fits(int MT, int nsb) {
   const int nb32 = nsb * 8;
   if (nb32 > 512) return false;  // scale records: at most 128 per wave
   const int S = kmf_slices(nb32);
   const int nbs = ((nb32 + S - 1) / S + 7) / 8 * 8;
-  return (MT == 4 ? kmf_lds_bytes<4>(nb32, nbs, 8) : kmf_lds_bytes<8>(nb32, nbs, 8)) <= 160 * 1024;
+  return (MT == 4 ? kmf_lds_bytes<4>(nb32, nbs, 8, S) : kmf_lds_bytes<8>(nb32, nbs, 8, S)) <= 160 * 1024;
 }
 template <int XT, int MT>
 static int launch_kq4_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned grid_y = 1) {
@@ -968,13 +983,20 @@ static int launch_kq4_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned gri
     grid += (unsigned)(((a.part[p].N + 15) / 16 + tiles_wg - 1) / tiles_wg);
   }
   a.wg_start[a.nparts] = (int)grid;
-  const size_t lds = kmf_lds_bytes<MT>(nb32, nbs, nwaves);
+  const size_t lds = kmf_lds_bytes<MT>(nb32, nbs, nwaves, S);
   if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
-  auto kern = kq4_gemv_mfma_kernel<XT, MT>;
-  if (lds > 64 * 1024)
-    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kern, dim3(grid, grid_y), dim3(nwaves * 64), lds, st, a, S, nbs);
-  return (int)hipGetLastError();
+  const int xpad = kmf_xpad(nb32, S, nbs);
+  auto go = [&](auto kern) {
+    if (lds > 64 * 1024)
+      HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3(grid, grid_y), dim3(nwaves * 64), lds, st, a, S, nbs, xpad);
+    return (int)hipGetLastError();
+  };
+  switch (kmf_groups(nbs)) {
+    case 6: return go(kq4_gemv_mfma_kernel<XT, MT, 6>);
+    case 8: return go(kq4_gemv_mfma_kernel<XT, MT, 8>);
+    default: return go(kq4_gemv_mfma_kernel<XT, MT, KMF_NG>);
+  }
 }
 template <int XT>
 static int launch_kq4_mfma(const KGemvArgs& a, hipStream_t st) {
@@ -989,12 +1011,14 @@ static int launch_kq4_mfma(const KGemvArgs& a, hipStream_t st) {
 // quantization delivers anyway.  Scaling per lane: acc = fma(fp32(d * sc) * dx, float(isum - 32 * bsum), acc).
 // Step st of a trip = half a super-block (records 4 (st & 1) + g of super-block st / 2): low nibbles are units 8 (st & 1) + g,
 // high nibbles units 8 (st & 1) + 4 + g.
-constexpr int K6_ST = 10;  // steps per trip: five super-blocks
-template <int XT, int MT>
-__global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, int sps) {  // sps = super-blocks per slice
+constexpr int K6_ST = 10;  // steps per trip, at most: five super-blocks (the launcher takes fewer for shorter slices)
+// ST = steps per trip: the slice in one trip where it fits (6, 8 or 10); xpad = super-blocks the last trip of a slice reaches
+// past the row (zeros in LDS)
+template <int XT, int MT, int ST = K6_ST>
+__global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, int sps, int xpad) {  // sps = super-blocks per slice
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int TH = MT / 4;
-  constexpr int TSB = K6_ST / 2;  // super-blocks per trip
+  constexpr int TSB = ST / 2;  // super-blocks per trip
   const int nsb = a.nsb, nu = nsb * 16, K = nsb * QK_K;
   const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x, nwaves = nthreads >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1015,10 +1039,10 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
 
   const int wsu = (sps + TSB - 1) / TSB * TSB * 16;  // units of weight scales per wave: whole trips
   u32x4* xc = reinterpret_cast<u32x4*>(smem);                     // [unit * MT + m] the unit's 16 codes
-  u32x4* zrec = xc + (size_t)(nu + TSB * 16) * MT;
+  u32x4* zrec = xc + (size_t)(nu + xpad * 16) * MT;
   int* bs16 = reinterpret_cast<int*>(zrec + 1);                   // [unit * MT + m] sum of the unit's codes
-  float* dxs = reinterpret_cast<float*>(bs16 + (size_t)(nu + TSB * 16) * MT);  // [super-block * MT + m]
-  float* ws_all = dxs + (size_t)(nsb + TSB) * MT;
+  float* dxs = reinterpret_cast<float*>(bs16 + (size_t)(nu + xpad * 16) * MT);  // [super-block * MT + m]
+  float* ws_all = dxs + (size_t)(nsb + xpad) * MT;
   float* ws = ws_all + (size_t)wave * wsu * 16;
   f32x4* red = reinterpret_cast<f32x4*>(smem) + (size_t)wave * TH * 64;  // takes the place of the codes once every wave is done with them
 
@@ -1043,10 +1067,10 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
   const int c = lane & 15, g = lane >> 4;
   const bool row_ok = tile_ok && row0 + c < N;
   const uint32_t rbase = (uint32_t)(row0 + c) * (uint32_t)nsb;
-  u32x4 wl[K6_ST], wh[K6_ST];
+  u32x4 wl[ST], wh[ST];
   auto load_steps = [&](int sb0) {
 #pragma unroll
-    for (int st = 0; st < K6_ST; st++) {
+    for (int st = 0; st < ST; st++) {
       const int sb = sb0 + (st >> 1);
       const bool ok = row_ok && sb < s1;
       wl[st] = __builtin_amdgcn_raw_buffer_load_b128(ra, ok ? ((rbase + (uint32_t)sb) * 8u + 4u * (st & 1) + (uint32_t)g) * 16u : KBUF_OOB, 0, KBUF_NT);
@@ -1088,11 +1112,11 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
     }
   }
   if (tid == 0) zrec[0] = u32x4{0u, 0u, 0u, 0u};
-  for (int i = tid; i < TSB * 16 * MT; i += nthreads) {
+  for (int i = tid; i < xpad * 16 * MT; i += nthreads) {
     xc[(size_t)nu * MT + i] = u32x4{0u, 0u, 0u, 0u};
     bs16[(size_t)nu * MT + i] = 0;
   }
-  for (int i = tid; i < TSB * MT; i += nthreads) dxs[nsb * MT + i] = 0.f;
+  for (int i = tid; i < xpad * MT; i += nthreads) dxs[nsb * MT + i] = 0.f;
 #pragma unroll
   for (int k = 0; k < 2; k++) {
     const int ch = lane + 64 * k;
@@ -1183,15 +1207,15 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
     };
     fetch_b(0, 0);
 #pragma unroll
-    for (int st = 0; st < K6_ST; st++) {
+    for (int st = 0; st < ST; st++) {
       issue(st & 1, st);
-      if (st + 1 < K6_ST) fetch_b((st + 1) & 1, st + 1);
+      if (st + 1 < ST) fetch_b((st + 1) & 1, st + 1);
       fetch_s(st & 1, st);
       __builtin_amdgcn_sched_barrier(0);
       if (st > 0) scale((st - 1) & 1, st - 1);
       __builtin_amdgcn_sched_barrier(0);
     }
-    scale((K6_ST - 1) & 1, K6_ST - 1);
+    scale((ST - 1) & 1, ST - 1);
   }
 #pragma unroll
   for (int h = 0; h < TH; h++) {  // the four lanes of an activation row (units = 0..3 mod 4)
@@ -1232,12 +1256,24 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
   }
 }
 
+static int k6mf_steps(int sps) { return sps <= 3 ? 6 : (sps <= 4 ? 8 : K6_ST); }
+// super-blocks the last trip of a slice reads past the row (whole trips from the slice's first super-block)
+static int k6mf_xpad(int nsb, int S, int sps) {
+  const int tsb = k6mf_steps(sps) / 2;
+  int pad = 0;
+  for (int s = 0; s < S; s++) {
+    const int s0 = s * sps, s1 = std::min(nsb, s0 + sps);
+    if (s1 > s0) pad = std::max(pad, s0 + ((s1 - s0 - 1) / tsb + 1) * tsb - nsb);
+  }
+  return pad;
+}
 template <int MT>
-static size_t k6mf_lds_bytes(int nsb, int sps, int nwaves) {
-  const int tsb = K6_ST / 2;
+static size_t k6mf_lds_bytes(int nsb, int sps, int nwaves, int S) {
+  const int tsb = k6mf_steps(sps) / 2, rows = nsb + k6mf_xpad(nsb, S, sps);
   const int wsu = (sps + tsb - 1) / tsb * tsb * 16;
-  return (size_t)(nsb * 16 + tsb * 16) * MT * 16 + 16 + (size_t)(nsb * 16 + tsb * 16) * MT * 4 + (size_t)(nsb + tsb) * MT * 4 +
-         (size_t)nwaves * wsu * 64;  // the partial sums of the slices reuse the code area
+  const size_t need = (size_t)rows * 16 * MT * 16 + 16 + (size_t)rows * 16 * MT * 4 + (size_t)rows * MT * 4 + (size_t)nwaves * wsu * 64;
+  // the partial sums of the slices reuse the code area: it must hold them
+  return std::max(need, (size_t)nwaves * (MT / 4) * 1024);
 }
 static void k6mf_split(int nsb, int& S, int& sps) {
   S = 1;
@@ -1248,7 +1284,7 @@ static bool kq6_mfma_fits(int MT, int nsb) {
   int S, sps;
   k6mf_split(nsb, S, sps);
   if (sps > 8) return false;  // scale records: at most 128 per wave
-  return (MT == 4 ? k6mf_lds_bytes<4>(nsb, sps, 8) : k6mf_lds_bytes<8>(nsb, sps, 8)) <= 160 * 1024;
+  return (MT == 4 ? k6mf_lds_bytes<4>(nsb, sps, 8, S) : k6mf_lds_bytes<8>(nsb, sps, 8, S)) <= 160 * 1024;
 }
 template <int XT, int MT>
 static int launch_kq6_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned grid_y = 1) {
@@ -1264,13 +1300,20 @@ static int launch_kq6_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned gri
     grid += (unsigned)(((a.part[p].N + 15) / 16 + tiles_wg - 1) / tiles_wg);
   }
   a.wg_start[a.nparts] = (int)grid;
-  const size_t lds = k6mf_lds_bytes<MT>(a.nsb, sps, nwaves);
+  const size_t lds = k6mf_lds_bytes<MT>(a.nsb, sps, nwaves, S);
   if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
-  auto kern = kq6_gemv_mfma_kernel<XT, MT>;
-  if (lds > 64 * 1024)
-    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kern, dim3(grid, grid_y), dim3(nwaves * 64), lds, st, a, S, sps);
-  return (int)hipGetLastError();
+  const int xpad = k6mf_xpad(a.nsb, S, sps);
+  auto go = [&](auto kern) {
+    if (lds > 64 * 1024)
+      HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3(grid, grid_y), dim3(nwaves * 64), lds, st, a, S, sps, xpad);
+    return (int)hipGetLastError();
+  };
+  switch (k6mf_steps(sps)) {
+    case 6: return go(kq6_gemv_mfma_kernel<XT, MT, 6>);
+    case 8: return go(kq6_gemv_mfma_kernel<XT, MT, 8>);
+    default: return go(kq6_gemv_mfma_kernel<XT, MT, K6_ST>);
+  }
 }
 template <int XT>
 static int launch_kq6_mfma(const KGemvArgs& a, hipStream_t st) {

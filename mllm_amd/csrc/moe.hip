@@ -1948,15 +1948,15 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
   Carver c(workspace);
   const KqMoeCarve w = carve_kq_moe(c, T, H, I, E, k);
   float *g = w.g, *u = w.u, *h = w.h, *per = w.per;
-  // More than about two pairs per expert (Q6_K: one): the pairs are sorted by expert and run as tiles of eight rows on the matrix-core
+  // More than about one pair per expert (Q6_K: half a pair): the pairs are sorted by expert and run as tiles of eight rows on the matrix-core
   // kernels, so an expert's matrices are streamed once per eight pairs instead of once per pair (the grouped form).
   // x and h are quantized to Q8_K once (bit-exact images), the tiles gather their rows from the images.
   const bool tiles_ok = E <= MOE_MAX_EXPERTS && kq_moe_tiles_fit(wtype, H) && kq_moe_tiles_fit(wtype, I) &&
                         (size_t)E + (size_t)slots / KQ_MOE_TILE + 1 <= 65535;
-  // measured at 128 experts, top-8 (pairs -> tiles, us): Q4_K 32 tokens 140 -> 143, 64: 273 -> 192, 512: 2149 -> 649;
-  // Q6_K 16 tokens 142 -> 140, 32: 264 -> 187, 512: 3976 -> 887
-  const int per_expert = wtype == MLLM_HIP_Q4_K ? 2 : 1;
-  if (tiles_ok && (g_moe_kq_path == 2 || (g_moe_kq_path == 0 && slots > per_expert * E))) {
+  // measured at 128 experts, top-8 (pairs / tiles, us): Q4_K 16 tokens 80 / 84, 24: 112 / 97, 32: 145 / 112, 64: 289 / 153,
+  // 512: 2182 / 480; Q6_K 8 tokens 79 / 77, 16: 142 / 126, 32: 260 / 165, 512: 3976 / 760
+  const bool many = wtype == MLLM_HIP_Q4_K ? slots > E : 2 * slots > E;
+  if (tiles_ok && (g_moe_kq_path == 2 || (g_moe_kq_path == 0 && many))) {
     const unsigned max_tiles = (unsigned)(E + slots / KQ_MOE_TILE + 1);
     RC_RET(launch_route(topk_ids, slots, E, KQ_MOE_TILE, w.ro, st));
     RC_RET(kq_quantize_image(x, x_dtype, w.ximg, T, H, st));
