@@ -974,7 +974,9 @@ static int launch_kq4_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned gri
   const int nb32 = a.nsb * 8;
   const int S = kmf_slices(nb32);
   const int nbs = ((nb32 + S - 1) / S + 7) / 8 * 8;
-  int nwaves = XT == KQ_IMAGE ? 4 : 8;
+  // (MoE row tiles, grid_y > 1: the tile's eight image rows are staged once per workgroup; eight waves = 64 weight rows per
+  // staging instead of 32: Q4_K 512 tokens 491 -> 458 us.  The Q6_K kernel, with two waves per SIMD, loses with eight: 780 -> 915)
+  int nwaves = XT == KQ_IMAGE ? (grid_y > 1 ? (g_kq_NW ? g_kq_NW : 8) : 4) : 8;
   if (nwaves < S) nwaves = S;
   const int tiles_wg = nwaves / S;
   unsigned grid = 0;
