@@ -671,6 +671,11 @@ static int launch_kq_m(const KGemvArgs& a, hipStream_t st) {
   if (r1) {
     if (units >= 64 * 4) best = 64;
     NW = best == 64 ? 16 : 8;  // 16 rows per workgroup either way
+    // ... or fewer, so that the grid is about one workgroup per CU (the Q4_0 kernel's finding: 2560 rows of 9728 elements
+    // as 160 workgroups of 16 waves or as 256 of 10)
+    const int rpw = 64 / best;  // rows per wave
+    const int want = (int)((rows / rpw + 255) / 256);
+    if (want >= 4 && want < NW) NW = want;
   }  // (many rows, K = 2560: eight waves per workgroup measured slower than four, 11.0 against 9.6 us for gate + up)
   // Q6_K rows whose units leave most of a 64-lane trip idle (K = 2560: 40 units): 16 lanes per row, two waves, where that still
   // makes a thousand workgroups (gate + up 15.8 -> 13.5 us; the smaller q/k/v launch stays faster with the whole wave)
