@@ -220,7 +220,7 @@ static int g_tune_G = 0, g_tune_R = 0, g_tune_NW = 0;
 
 static GemvShape pick_shape(int MT, int64_t N, int nb) {
   // Measured on MI355X over the Qwen3-4B projection shapes: groups of 32 lanes with two rows each (512 contiguous
-  // bytes per row segment) suit rows of 64..255 blocks; very long rows want the whole wave on one row and, because
+  // bytes per row segment) suit rows of 65..255 blocks; very long rows want the whole wave on one row and, because
   // every workgroup quantizes all of x, many waves per workgroup to share that work.
   GemvShape s;
   s.R = 2;
@@ -233,9 +233,10 @@ static GemvShape pick_shape(int MT, int64_t N, int nb) {
     // the 2560 rows of a down projection make 160 workgroups on 256 CUs; about one workgroup per CU measured best
     // (N = 2560, 304 blocks: 16 waves 5.84 us, 11 waves 5.27 us, 8 waves 6.4 us)
     if (MT <= 2) s.NW = (int)std::min<int64_t>(16, std::max<int64_t>(8, (N + 239) / 240));
-  } else if (nb >= 64) {
+  } else if (nb > 64) {
     s.G = 32;
   } else if (nb >= 16) {
+    // (rows of exactly 64 blocks, 6144 of them: 16 lanes per row 3.48 us, 32 lanes 3.80)
     s.G = 16;
   } else {
     s.G = 8;
