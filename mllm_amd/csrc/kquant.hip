@@ -155,58 +155,46 @@ __global__ void kq_dequantize_kernel(int wtype, KView v, float* __restrict__ w, 
 }
 
 // ---- Q8_K quantization of activations ---------------------------------------------------------------------------------------
-// 32 neighbouring lanes (half a wave) hold one super-block, eight consecutive elements per lane.  The reference takes the
-// element of largest magnitude WITH its sign, the first one when several are equal: the reduction carries the lane it came
-// from.  Outputs of a lane: its eight codes (two dwords), the sum of its eight codes, the block scale.
+// 32 neighbouring lanes (half a wave) hold one super-block, eight consecutive elements per lane; both halves of the wave
+// must be active or idle as a whole.  The reference takes the element of largest magnitude WITH its sign, the first one
+// when several are equal: the magnitude goes through a plain max butterfly, the sign comes from the first lane (lowest set
+// bit of a ballot) that holds an element of that magnitude and, in it, the first such element.  Codes: the product is
+// rounded to fp32, then adding 1.5 * 2^23 rounds to nearest-even as rintf does and leaves the two's-complement code in the
+// low byte; the clamp to 127 is an integer min on the bits of that (positive) sum.  Outputs of a lane: its eight codes (two dwords), the sum of its
+// eight codes, the block scale.
 struct Q8KItem {
   uint32_t q0, q1;
   int sum8;
   float d;
 };
 __device__ __forceinline__ Q8KItem quantize_q8k_item(const float (&v)[8], int lane) {
-  float amax = 0.f, mx = 0.f;
+  // magnitudes compare as their bit patterns: the butterfly runs on unsigned integers
+  uint32_t am = 0u;
 #pragma unroll
-  for (int e = 0; e < 8; e++) {
-    const float ax = fabsf(v[e]);
-    if (ax > amax) {
-      amax = ax;
-      mx = v[e];
-    }
-  }
-  int src = lane;
-  // butterfly over the 32 lanes: within a row of 16 lanes through DPP, the last step through a lane shuffle
-  auto take = [&](float oa, float om, int os) {
-    if (oa > amax || (oa == amax && os < src)) {
-      amax = oa;
-      mx = om;
-      src = os;
-    }
-  };
-  take(dpp_f<0xB1>(amax), dpp_f<0xB1>(mx), __builtin_amdgcn_update_dpp(0, src, 0xB1, 0xf, 0xf, true));     // lane ^ 1
-  take(dpp_f<0x4E>(amax), dpp_f<0x4E>(mx), __builtin_amdgcn_update_dpp(0, src, 0x4E, 0xf, 0xf, true));     // lane ^ 2
-  take(dpp_f<0x141>(amax), dpp_f<0x141>(mx), __builtin_amdgcn_update_dpp(0, src, 0x141, 0xf, 0xf, true));  // half-row mirror
-  take(dpp_f<0x140>(amax), dpp_f<0x140>(mx), __builtin_amdgcn_update_dpp(0, src, 0x140, 0xf, 0xf, true));  // row mirror
-  take(__shfl_xor(amax, 16, 64), __shfl_xor(mx, 16, 64), __shfl_xor(src, 16, 64));
+  for (int e = 0; e < 8; e++) am = max(am, __float_as_uint(v[e]) & 0x7fffffffu);
+  am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0xB1, 0xf, 0xf, true));   // lane ^ 1
+  am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0x4E, 0xf, 0xf, true));   // lane ^ 2
+  am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0x141, 0xf, 0xf, true));  // half-row mirror
+  am = max(am, (uint32_t)__builtin_amdgcn_update_dpp(0, (int)am, 0x140, 0xf, 0xf, true));  // row mirror
+  am = max(am, (uint32_t)__shfl_xor((int)am, 16, 64));
+  const float amax = __uint_as_float(am);
+  float sel = 0.f;  // the lane's first element of that magnitude
+#pragma unroll
+  for (int e = 7; e >= 0; e--) sel = ((__float_as_uint(v[e]) & 0x7fffffffu) == am) ? v[e] : sel;
+  const bool hit = (__float_as_uint(sel) & 0x7fffffffu) == am, neg = (__float_as_uint(sel) >> 31) != 0u;
+  const unsigned long long mh = __ballot(hit), mn = __ballot(hit && neg);
+  const uint32_t h32 = (lane & 32) ? (uint32_t)(mh >> 32) : (uint32_t)mh;
+  const uint32_t n32 = (lane & 32) ? (uint32_t)(mn >> 32) : (uint32_t)mn;
+  const bool negative = (n32 & (h32 & (0u - h32))) != 0u;
   Q8KItem r{0u, 0u, 0, 0.f};
   if (amax == 0.f) return r;
-  const float iscale = -128.f / mx;
-  int sum = 0;
-  uint32_t pk[2];
+  const float iscale = -128.f / (negative ? -amax : amax);
+  uint32_t b[8];
 #pragma unroll
-  for (int w = 0; w < 2; w++) {
-    uint32_t p = 0;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-      int q = (int)rintf(iscale * v[4 * w + e]);
-      q = min(127, q);
-      sum += q;
-      p |= ((uint32_t)q & 0xffu) << (8 * e);
-    }
-    pk[w] = p;
-  }
-  r.q0 = pk[0];
-  r.q1 = pk[1];
-  r.sum8 = sum;
+  for (int e = 0; e < 8; e++) b[e] = (uint32_t)min((int)__float_as_uint(iscale * v[e] + 12582912.0f), 0x4B40007F);  // bits of 1.5 * 2^23 + 127
+  r.q0 = __builtin_amdgcn_perm(b[1], b[0], 0x0c0c0400u) | __builtin_amdgcn_perm(b[3], b[2], 0x04000c0cu);
+  r.q1 = __builtin_amdgcn_perm(b[5], b[4], 0x0c0c0400u) | __builtin_amdgcn_perm(b[7], b[6], 0x04000c0cu);
+  r.sum8 = __builtin_amdgcn_sdot4((int)r.q1, 0x01010101, __builtin_amdgcn_sdot4((int)r.q0, 0x01010101, 0, false), false);
   r.d = 1.f / iscale;
   return r;
 }

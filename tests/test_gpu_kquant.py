@@ -29,6 +29,12 @@ def test_q8_K_quantization_bit_exact(dtype):
         xf[2, 9], xf[2, 200] = -4.5, 4.5         # equal magnitudes, opposite signs: the first one decides
         xf[3, 512:768] = 0.25
         xf[3, 767] = -0.25                       # the LAST element differs in sign only
+        xf[4, :256] = 0.1
+        xf[4, 16], xf[4, 17] = 5.0, -5.0         # the tie inside one lane's eight elements, positive first
+        xf[5, :256] = 0.1
+        xf[5, 18], xf[5, 21] = -5.0, 5.0         # ... negative first
+        xf[6, 256:512] = 0.1
+        xf[6, 256 + 128], xf[6, 256 + 255] = 6.0, -6.0  # the tie across the two 16-lane rows of an odd super-block
         x = to_dev(xf)
     announce("q8_K quantization", dtype)
     q, d, bs = ql.quantize_q8_K(x)
