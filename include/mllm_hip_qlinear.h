@@ -135,7 +135,9 @@ int mllm_hip_linear_q_gemv_fused(int wtype, int nparts, const mllm_hip_gemv_part
                                  const void* x, int x_kind, int M, int64_t K, int act_scale_mode, void* stream);
 
 /* Same for any M: quantizes the activations with a stand-alone kernel into `workspace`
- * (mllm_hip_linear_q_workspace_bytes) and runs the tiled block-dot kernel.  Used by prefill and by the MoE path. */
+ * (mllm_hip_linear_q_workspace_bytes) and runs the tiled block-dot kernel; up to 16 rows run as passes of the eight-row
+ * GEMV above instead (the same block arithmetic, the weights streamed once per eight rows).  Used by prefill and by the
+ * MoE path. */
 size_t mllm_hip_linear_q_workspace_bytes(int64_t M, int64_t K);
 int mllm_hip_linear_q(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y,
                       int64_t M, int64_t N, int64_t K, int act_scale_mode, void* workspace, void* stream);

@@ -319,7 +319,8 @@ def w4a16_dequantize(qw, scales, zeros, group=128):
 
 # ----------------------------------------------------------------------------- any-M quantized Linear and the MoE FFN
 def linear_q(w, x, bias=None, act_scale_mode=SCALE_X86_REF, workspace=None, out=None):
-    """Q4_0/Q8_0 Linear for any number of rows: stand-alone Q8_0 activation quantization + MFMA block-dot tiles."""
+    """Q4_0/Q8_0 Linear for any number of rows: stand-alone Q8_0 activation quantization + MFMA block-dot tiles (up to 16 rows:
+    passes of the eight-row GEMV, the same arithmetic)."""
     assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
     M = x.shape[0]
     L = _lib.lib()

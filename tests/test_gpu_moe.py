@@ -16,7 +16,8 @@ TOL = 1e-3
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
-@pytest.mark.parametrize("M,N,K", [(1, 32, 32), (33, 100, 96), (129, 64, 2048), (300, 768, 2048 + 64), (512, 2048, 768)])
+@pytest.mark.parametrize("M,N,K", [(1, 32, 32), (9, 100, 96), (16, 768, 2048 + 64), (17, 64, 2048), (33, 100, 96), (129, 64, 2048),
+                                   (300, 768, 2048 + 64), (512, 2048, 768)])
 def test_linear_q_any_m(wtype, M, N, K):
     rng = synth.rng_for(4, M + N + K + wtype)
     W = synth.make_weight(rng, wtype, N, K)
