@@ -307,15 +307,16 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
     case Scheme::kQ4_0:
     case Scheme::kQ8_0: {
       const int wt = scheme_ == Scheme::kQ4_0 ? MLLM_HIP_Q4_0 : MLLM_HIP_Q8_0;
-      // decode, and short batches as passes of eight rows over the same weights: measured on the Qwen3-4B projections the
-      // passes beat the short-batch matrix-core entry up to 16 rows (9 rows: 11-14 us against 15-24) and the exact tile
-      // kernel up to 32 (32 rows: 30-36 us against 46-149)
-      if (M <= 16 || (gemm_packed_.isNil() && M <= 32)) {
+      // decode, and short batches as groups of eight rows over the same weights (from sixteen rows on the whole groups share
+      // one launch): measured on the Qwen3-4B projections against the short-batch matrix-core entry, 16 rows 8-15 us against
+      // 15-23, 32 rows 9-24 against 16-24 (a layer's seven projections together 108 against 128), 64 rows 171 against 154;
+      // against the exact tile kernel 64 rows 17-39 us against 70-235
+      if (M <= 32 || (gemm_packed_.isNil() && M <= 64)) {
         const void* image = be.findImage(x.ptr<void>(), (int)M, K);
         mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
         // from three rows on: room for the partial sums of the K slices, which lets the rows run as one launch whose
         // workgroups each quantize (or copy) only their slice of the activations; the library decides
-        const size_t ws_bytes = M >= 3 ? mllm_hip_gemv_splitk_workspace_bytes(8, K, N) : 0;
+        const size_t ws_bytes = M >= 3 ? mllm_hip_gemv_splitk_workspace_bytes((int)M, K, N) : 0;
         void* ws = ws_bytes ? workspace(ws_bytes) : nullptr;
         if (image) {
           const mllm_hip_gemv_fusion fu{nullptr, ws, ws_bytes};

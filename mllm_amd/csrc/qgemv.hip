@@ -378,10 +378,12 @@ MLLM_API size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K) {
   return gemv_image_bytes(K);
 }
 
-// image, then the partial sums of the K slices of one pass of eight rows (each part's rows rounded up to 16)
+// image, then the partial sums of the K slices of eight rows (each part's rows rounded up to 16), for every whole group of
+// eight rows from sixteen rows on
 MLLM_API size_t mllm_hip_gemv_splitk_workspace_bytes(int M, int64_t K, int64_t N_total) {
   if (M < 1 || K <= 0 || K % QK || N_total <= 0) return 0;
-  return gemv_image_bytes(K) + (size_t)gemv_mfk_slices((int)(K / QK)) * 8 * (size_t)(N_total + 16 * GEMV_MAX_PARTS) * 4;
+  const size_t groups = M >= 16 ? (size_t)(M / 8) : 1;  // whole groups of eight rows share a launch
+  return gemv_image_bytes(K) + groups * (size_t)gemv_mfk_slices((int)(K / QK)) * 8 * (size_t)(N_total + 16 * GEMV_MAX_PARTS) * 4;
 }
 
 // x_kind: MLLM_HIP_F32 / MLLM_HIP_BF16 activations, or MLLM_HIP_Q8_IMAGE: their quantized image (act_scale_mode unused)
@@ -403,6 +405,32 @@ static int gemv_check_args(int wtype, int nparts, const mllm_hip_gemv_part* part
   return 0;
 }
 
+// `groups` groups of eight rows of raw activations in one launch of the K-slice kernel; MFK_NOT_TAKEN where that kernel does
+// not apply (the caller then runs passes)
+static int gemv_multi_groups(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual, const void* x,
+                             int x_dtype, int groups, int64_t K, int act_scale_mode, void* workspace, size_t ws_bytes, void* stream) {
+  RC_RET(gemv_check_args(wtype, nparts, parts, x, x_dtype, 8 * groups, K, act_scale_mode, workspace));
+  if (g_gemv_path == 1 || g_gemv_path == 2 || !workspace) return MFK_NOT_TAKEN;
+  const size_t img = gemv_image_bytes(K);
+  if (ws_bytes <= img) return MFK_NOT_TAKEN;
+  GemvArgs a{};
+  for (int p = 0; p < nparts; p++) {
+    a.part[p].w = packed_view(wtype, parts[p].packed, parts[p].N, K);
+    a.part[p].bias = parts[p].bias;
+    a.part[p].residual = residual ? residual[p] : nullptr;
+    a.part[p].y = parts[p].y;
+    a.part[p].N = (int)parts[p].N;
+  }
+  a.nparts = nparts;
+  a.x = x;
+  a.M = 8 * groups;
+  a.nb = (int)(K / QK);
+  a.nbp = (int)scale_row_stride(K);
+  a.x86_scale = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
+  return launch_gemv_mfk(wtype, x_dtype, 8, a, workspace, reinterpret_cast<char*>(workspace) + img, ws_bytes - img, g_tune_NW, g_tune_R,
+                         (hipStream_t)stream, groups);
+}
+
 // More than eight rows of raw activations: passes of eight rows, each streaming the weights again (the same arithmetic row by
 // row; up to about 32 rows this is faster than the matrix-core GEMM path, whose 128-row tiles leave most of the chip idle).
 static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* parts, const mllm_hip_gemv_fusion* fu, const void* x,
@@ -412,7 +440,15 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
     return gemv_multi_pass(wtype, nparts, parts, residual, x, x_dtype, M, K, act_scale_mode, workspace, ws_bytes, stream);
   if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
   const size_t xrow = (size_t)K * (x_dtype == MLLM_HIP_F32 ? 4 : 2);
-  for (int m0 = 0; m0 < M; m0 += 8) {
+  int m_first = 0;
+  if (M >= 16) {
+    // the whole groups of eight rows in one launch of the K-slice kernel where it applies (room for every group's partial
+    // sums): the groups share one pass over the weights.  Row by row the bits of an eight-row call.
+    const int rc = gemv_multi_groups(wtype, nparts, parts, residual, x, x_dtype, M / 8, K, act_scale_mode, workspace, ws_bytes, stream);
+    if (rc == 0) m_first = M / 8 * 8;
+    else if (rc != MFK_NOT_TAKEN) return rc;
+  }
+  for (int m0 = m_first; m0 < M; m0 += 8) {
     mllm_hip_gemv_part pp[GEMV_MAX_PARTS];
     const float* rr[GEMV_MAX_PARTS];
     for (int p = 0; p < nparts; p++) {

@@ -412,7 +412,7 @@ bool gemv_mfma_fits(int MT, int nb);  // rows of nb blocks fit that kernel's LDS
 // does not fit (no room for the partial sums, no free counter block, slices too long): the caller takes another kernel.
 constexpr int MFK_NOT_TAKEN = 1;
 int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a, const void* workspace, void* part, size_t part_bytes, int waves,
-                    int slices, hipStream_t st);
+                    int slices, hipStream_t st, int groups = 1);
 int gemv_mfk_slices(int nb);
 int launch_gemv_q4_f32(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
 int launch_gemv_q4_bf16(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);

@@ -88,12 +88,18 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
     if (p < a.nparts && (int)blockIdx.x >= a.wg_start[p]) pidx = p;
   const GemvPart& pt = a.part[pidx];
   const int wg0 = a.wg_start[pidx], pcol0 = k.col0[pidx];
-  const void* const xptr = a.x;
-  const int aM = a.M, x86 = a.x86_scale;
-  float* const kpart = k.part;
-  unsigned* const kcnt = k.counters;
+  // blockIdx.z: group of MT activation rows (raw activations; an image is always one group).  A group has its own rows of x
+  // and y, its own partial sums and counters, and reads the same weights as its siblings.
+  const int rg = blockIdx.z;
+  const void* const xptr =
+      XT == GEMV_PREQ ? a.x : static_cast<const void*>(reinterpret_cast<const char*>(a.x) + (size_t)rg * MT * nb * QK * (XT == MLLM_HIP_F32 ? 4 : 2));
+  const int aM = min(a.M - rg * MT, MT), x86 = a.x86_scale;
   const int kNP = k.NP;
+  float* const kpart = k.part + (size_t)rg * gridDim.y * MT * kNP;
+  unsigned* const kcnt = k.counters + rg * gridDim.x;
   const int N = pt.N;
+  float* const ybase = pt.y + (int64_t)rg * MT * N;
+  const float* const rbase = pt.residual ? pt.residual + (int64_t)rg * MT * N : nullptr;
   const int tile = ((int)blockIdx.x - wg0) * nwaves + wave;
   const int slice = blockIdx.y;
   const int row0 = tile * 16;
@@ -367,8 +373,8 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
     if (!tile_ok || q != 0) return;
     // rows of a multiple of four outputs, 16-byte aligned pointers: 16 bytes per lane, the four lanes of an activation row
     // write one 64-byte line
-    const bool vec = (N & 3) == 0 && ((reinterpret_cast<uintptr_t>(pt.y) | reinterpret_cast<uintptr_t>(pt.bias) |
-                                       reinterpret_cast<uintptr_t>(pt.residual)) & 15) == 0;  // uniform
+    const bool vec = (N & 3) == 0 && ((reinterpret_cast<uintptr_t>(ybase) | reinterpret_cast<uintptr_t>(pt.bias) |
+                                       reinterpret_cast<uintptr_t>(rbase)) & 15) == 0;  // uniform
 #pragma unroll
     for (int h = 0; h < TH; h++) {
       const int t = 4 * h + tt;
@@ -380,21 +386,21 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
           const f32x4 bv = *reinterpret_cast<const f32x4*>(pt.bias + n);
           o = f32x4{bv.x + o.x, bv.y + o.y, bv.z + o.z, bv.w + o.w};
         }
-        if (pt.residual) {
-          const f32x4 rv = *reinterpret_cast<const f32x4*>(pt.residual + (int64_t)t * N + n);
+        if (rbase) {
+          const f32x4 rv = *reinterpret_cast<const f32x4*>(rbase + (int64_t)t * N + n);
           o = f32x4{o.x + rv.x, o.y + rv.y, o.z + rv.z, o.w + rv.w};
         }
-        *reinterpret_cast<f32x4*>(pt.y + (int64_t)t * N + n) = o;
+        *reinterpret_cast<f32x4*>(ybase + (int64_t)t * N + n) = o;
         continue;
       }
       const float v[4] = {acc[h].x, acc[h].y, acc[h].z, acc[h].w};
-      float* yrow = pt.y + (int64_t)t * N;
+      float* yrow = ybase + (int64_t)t * N;
 #pragma unroll
       for (int e = 0; e < 4; e++) {
         if (n + e < N) {
           float o = v[e];
           if (pt.bias) o = pt.bias[n + e] + o;
-          if (pt.residual) o = o + pt.residual[(int64_t)t * N + n + e];
+          if (rbase) o = o + rbase[(int64_t)t * N + n + e];
           yrow[n + e] = o;
         }
       }
@@ -450,8 +456,8 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
     if (t < aM && row0 + r < N) {
       float o = sum;
       if (pt.bias) o = pt.bias[row0 + r] + o;
-      if (pt.residual) o = o + pt.residual[(int64_t)t * N + row0 + r];
-      pt.y[(int64_t)t * N + row0 + r] = o;
+      if (rbase) o = o + rbase[(int64_t)t * N + row0 + r];
+      ybase[(int64_t)t * N + row0 + r] = o;
     }
   }
 }

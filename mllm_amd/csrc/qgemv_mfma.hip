@@ -47,18 +47,21 @@ static int mfk_counter_block(const void* workspace, unsigned** out) {
 int gemv_mfk_slices(int nb) { return nb <= 8 * 64 ? mf_slices(nb) : (nb + 63) / 64; }
 
 template <int WT, int XT, int MT>
-static int launch_mfk_t(const GemvArgs& a_in, const MfkArgs& k, int nwaves, unsigned grid_x, hipStream_t st) {
+static int launch_mfk_t(const GemvArgs& a_in, const MfkArgs& k, int nwaves, unsigned grid_x, unsigned groups, hipStream_t st) {
   const size_t lds = mfk_lds_bytes<MT>(WT, k.nbs, nwaves);
   if (lds > 160 * 1024) return MFK_NOT_TAKEN;
   auto kern = gemv_mfk_kernel<WT, XT, MT>;
   if (lds > 64 * 1024)
     HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kern, dim3(grid_x, (unsigned)k.S), dim3(nwaves * 64), lds, st, a_in, k);
+  hipLaunchKernelGGL(kern, dim3(grid_x, (unsigned)k.S, groups), dim3(nwaves * 64), lds, st, a_in, k);
   return (int)hipGetLastError();
 }
 
+// groups > 1: a_in.M = 8 * groups rows of raw activations, every group of eight a workgroup of its own per (row tiles, slice)
+// in the same launch (the groups read the same weights: once from memory, then from the caches)
 int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const void* workspace, void* part, size_t part_bytes,
-                    int waves, int slices, hipStream_t st) {
+                    int waves, int slices, hipStream_t st, int groups) {
+  if (groups < 1 || groups > 65535 || (groups > 1 && (MT != 8 || x_kind == GEMV_PREQ || a_in.M != 8 * groups))) return MFK_NOT_TAKEN;
   GemvArgs a = a_in;
   MfkArgs k{};
   int tiles_total = 0;
@@ -70,7 +73,9 @@ int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const v
   // second pass (gate + up of the 4B layer, 1216 tiles x 80 blocks: 10.6 -> 9.3 us at four rows, 12.7 -> 12.3 at eight;
   // q+k+v, 384 tiles, is slower whole: 6.5 -> 8.6 / 8.2 -> 11.6).  The kernel still sums the row in chains of k.vs blocks
   // and adds the chains in slice order: the same bits either way.  (slices: 1 = whole rows, 2 = never, for measurements)
-  if (a.nb <= MFK_MAX_NBS && (slices == 1 || (slices <= 0 && tiles_total >= 1024))) {
+  // (Row groups count like more tiles, for matrices of at least 512 tiles: 9728 x 2560 with two groups 16.0 -> 12.3 us whole;
+  // 4096 x 2560 with four groups is slower whole, 9.4 -> 12.1.)
+  if (a.nb <= MFK_MAX_NBS && (slices == 1 || (slices <= 0 && (int64_t)tiles_total * groups >= 1024 && tiles_total >= 512))) {
     k.S = 1;
     k.nbs = (a.nb + 7) / 8 * 8;
   }
@@ -89,7 +94,7 @@ int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const v
     for (int nw = nw_min; nw <= 8; nw++) {
       int64_t wgs = 0;
       for (int p = 0; p < a.nparts; p++) wgs += ((a.part[p].N + 15) / 16 + nw - 1) / nw;
-      wgs *= k.S;
+      wgs *= (int64_t)k.S * groups;
       const double cost = (double)((wgs + 255) / 256) * (nw + 2.0);
       if (cost < best - 1e-9) {
         best = cost;
@@ -109,13 +114,13 @@ int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const v
   a.wg_start[a.nparts] = (int)grid;
   k.NP = np;
   if (k.S > 1) {
-    if (!workspace || !part || (size_t)k.S * MT * np * 4 > part_bytes || grid > (unsigned)MFK_COUNTERS) return MFK_NOT_TAKEN;
+    if (!workspace || !part || (size_t)groups * k.S * MT * np * 4 > part_bytes || (size_t)grid * groups > (size_t)MFK_COUNTERS) return MFK_NOT_TAKEN;
     RC_RET(mfk_counter_block(workspace, &k.counters));
     k.part = static_cast<float*>(part);
   }
 #define MFK_CASE(WT_, XT_)                                                         \
   if (wtype == WT_ && x_kind == XT_)                                               \
-    return MT == 4 ? launch_mfk_t<WT_, XT_, 4>(a, k, nwaves, grid, st) : launch_mfk_t<WT_, XT_, 8>(a, k, nwaves, grid, st);
+    return MT == 4 ? launch_mfk_t<WT_, XT_, 4>(a, k, nwaves, grid, (unsigned)groups, st) : launch_mfk_t<WT_, XT_, 8>(a, k, nwaves, grid, (unsigned)groups, st);
   MFK_CASE(MLLM_HIP_Q4_0, MLLM_HIP_F32)
   MFK_CASE(MLLM_HIP_Q4_0, MLLM_HIP_BF16)
   MFK_CASE(MLLM_HIP_Q4_0, GEMV_PREQ)

@@ -256,6 +256,53 @@ def test_gemv_argument_errors():
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M", [16, 21, 32])
+def test_gemv_groups_of_eight_rows_share_a_launch(wtype, M):
+    """from sixteen rows on, with room in the workspace for every group's partial sums, the whole groups of eight rows run in
+    one launch (the remaining rows as a pass of their own): row by row the bits of an eight-row call with the same kind of
+    workspace; cut rows, whole rows, several matrices, ragged N, a last slice that is empty"""
+    rng = synth.rng_for(1, 900 + M + wtype)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(900 + M + wtype)
+    for shapes, oracle_too in (([(300, 1024)], True), ([(50, 161 * 32)], True), ([(2560, 9728)], False),
+                               ([(4096, 2560), (1024, 2560), (1024, 2560)], False), ([(9728, 2560), (9728, 2560)], False),
+                               ([(8200, 97 * 32), (8193, 97 * 32)], False)):
+        K = shapes[0][1]
+        n_total = sum(n for n, _ in shapes)
+        if oracle_too:
+            Ws = [synth.make_weight(rng, wtype, n, K) for n, _ in shapes]
+            ws = [ql.PackedQWeight(wtype, torch.from_numpy(W)) for W in Ws]
+        else:
+            ws = [ql.PackedQWeight.synthetic(wtype, n, K, gen) for n, _ in shapes]
+        biases = [to_dev(rng.standard_normal(n).astype(np.float32)) for n, _ in shapes]
+        for bf16 in (True, False):
+            if bf16:
+                bits, xf = synth.make_x_bf16(rng, M, K)
+                xd = bf16_dev(bits)
+            else:
+                xf = synth.make_x_fp32(rng, M, K)
+                xd = to_dev(xf)
+            announce("gemv row groups", wtype, M, shapes, "bf16" if bf16 else "fp32")
+            outs = ql.linear_q_gemv_multi(ws, xd, biases, workspace=ql.gemv_workspace(M, K, n_total))
+            ws8 = ql.gemv_workspace(8, K, n_total)
+            for m0 in range(0, M, 8):
+                part = ql.linear_q_gemv_multi(ws, xd[m0:m0 + 8].contiguous(), biases, workspace=ws8)
+                for o, pr in zip(outs, part):
+                    assert torch.equal(o[m0:m0 + 8], pr), (shapes, m0)
+            if oracle_too:
+                for W, b, o in zip(Ws, biases, outs):
+                    assert rel_l2(o.cpu().numpy(), orc.linear_q(xf, W, wtype, b.cpu().numpy(), orc.SCALE_X86_REF)) < 2e-6
+    # with residuals (the fused entry point), the same groups
+    K, N = 1024, 300
+    w = ql.PackedQWeight.synthetic(wtype, N, K, gen)
+    xd = to_dev(synth.make_x_fp32(rng, M, K))
+    r = to_dev(rng.standard_normal((M, N)).astype(np.float32))
+    (y,) = ql.linear_q_gemv_multi([w], xd, None, workspace=ql.gemv_workspace(M, K, N))
+    (yr,) = ql.linear_q_gemv_fused([w], xd, residuals=[r], workspace=ql.gemv_workspace(M, K, N))
+    assert torch.equal(yr, y + r)
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
 @pytest.mark.parametrize("M", [1, 3, 8])
 def test_gemv_multi_equals_single(wtype, M):
     """sibling projections in one launch give exactly the bits of one launch each (q/k/v and gate/up shapes)"""
