@@ -60,6 +60,7 @@ struct MfkArgs {
   int vs;              // blocks per summation chain (a multiple of 8): S > 1: nbs; S == 1: the length the slices would have
                        // had -- the chains of a whole row are added in slice order, so the bits do not depend on S
   int col0[GEMV_MAX_PARTS];  // first column of each part within a partial row
+  int gx, groups;            // groups > 1 (row groups of eight): a 1-D grid over (workgroup column < gx, slice, group), see the kernel
   int ipr_magic;             // ceil(2^20 / (2 nbs)): item / (items per row) as a multiply and a shift
 };
 
@@ -82,26 +83,38 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   const int nb = a.nb, nbp = a.nbp, nbs = k.nbs, S = k.S;
   const int tid = threadIdx.x, lane = tid & 63, nthreads = blockDim.x, nwaves = nthreads >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // Work item = (workgroup column bx, K slice, row group rg).  One row group: the grid is (columns, slices).  Several: a
+  // 1-D grid in which the groups of one (column, slice) are neighbours ON ONE XCD (workgroup L runs on XCD L % 8, every XCD
+  // has its own L2): they read the same weights at about the same time, so the weights come from memory once.  The grid is
+  // padded to whole eights of (column, slice) items; the padding leaves at once.
+  int bx = blockIdx.x, slice = blockIdx.y, rg = 0, gx = gridDim.x;
+  if (k.groups > 1) {
+    const int L = blockIdx.x, seq = L >> 3;
+    rg = seq % k.groups;
+    const int item = (seq / k.groups) * 8 + (L & 7);
+    if (item >= k.gx * S) return;
+    gx = k.gx;
+    slice = item / gx;
+    bx = item - slice * gx;
+  }
   int pidx = 0;  // uniform: which matrix this workgroup works on
 #pragma unroll
   for (int p = 1; p < GEMV_MAX_PARTS; p++)
-    if (p < a.nparts && (int)blockIdx.x >= a.wg_start[p]) pidx = p;
+    if (p < a.nparts && bx >= a.wg_start[p]) pidx = p;
   const GemvPart& pt = a.part[pidx];
   const int wg0 = a.wg_start[pidx], pcol0 = k.col0[pidx];
-  // blockIdx.z: group of MT activation rows (raw activations; an image is always one group).  A group has its own rows of x
-  // and y, its own partial sums and counters, and reads the same weights as its siblings.
-  const int rg = blockIdx.z;
+  // rg: group of MT activation rows (raw activations; an image is always one group).  A group has its own rows of x and y,
+  // its own partial sums and counters, and reads the same weights as its siblings.
   const void* const xptr =
       XT == GEMV_PREQ ? a.x : static_cast<const void*>(reinterpret_cast<const char*>(a.x) + (size_t)rg * MT * nb * QK * (XT == MLLM_HIP_F32 ? 4 : 2));
   const int aM = min(a.M - rg * MT, MT), x86 = a.x86_scale;
   const int kNP = k.NP;
-  float* const kpart = k.part + (size_t)rg * gridDim.y * MT * kNP;
-  unsigned* const kcnt = k.counters + rg * gridDim.x;
+  float* const kpart = k.part + (size_t)rg * S * MT * kNP;
+  unsigned* const kcnt = k.counters + rg * gx;
   const int N = pt.N;
   float* const ybase = pt.y + (int64_t)rg * MT * N;
   const float* const rbase = pt.residual ? pt.residual + (int64_t)rg * MT * N : nullptr;
-  const int tile = ((int)blockIdx.x - wg0) * nwaves + wave;
-  const int slice = blockIdx.y;
+  const int tile = (bx - wg0) * nwaves + wave;
   const int row0 = tile * 16;
   const bool tile_ok = row0 < N;
   const int b0 = slice * nbs, b1 = min(nb, b0 + nbs);  // this workgroup's blocks (possibly none: b1 <= b0)
@@ -426,9 +439,9 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   }
   __syncthreads();
   if (tid == 0) {
-    const unsigned old = atomicAdd(kcnt + blockIdx.x, 1u);
+    const unsigned old = atomicAdd(kcnt + bx, 1u);
     const int last = old == (unsigned)(S - 1);
-    if (last) kcnt[blockIdx.x] = 0u;  // every slice has arrived: ready for the next launch
+    if (last) kcnt[bx] = 0u;  // every slice has arrived: ready for the next launch
     *s_flag = last;
   }
   __syncthreads();

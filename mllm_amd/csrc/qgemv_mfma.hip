@@ -47,13 +47,18 @@ static int mfk_counter_block(const void* workspace, unsigned** out) {
 int gemv_mfk_slices(int nb) { return nb <= 8 * 64 ? mf_slices(nb) : (nb + 63) / 64; }
 
 template <int WT, int XT, int MT>
-static int launch_mfk_t(const GemvArgs& a_in, const MfkArgs& k, int nwaves, unsigned grid_x, unsigned groups, hipStream_t st) {
+static int launch_mfk_t(const GemvArgs& a_in, const MfkArgs& k_in, int nwaves, unsigned grid_x, unsigned groups, hipStream_t st) {
+  MfkArgs k = k_in;
+  k.gx = (int)grid_x;
+  k.groups = (int)groups;
   const size_t lds = mfk_lds_bytes<MT>(WT, k.nbs, nwaves);
   if (lds > 160 * 1024) return MFK_NOT_TAKEN;
   auto kern = gemv_mfk_kernel<WT, XT, MT>;
   if (lds > 64 * 1024)
     HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL(kern, dim3(grid_x, (unsigned)k.S, groups), dim3(nwaves * 64), lds, st, a_in, k);
+  // several row groups: a 1-D grid, (column, slice) items padded to whole eights, the groups of an item next to each other
+  const dim3 grid = groups > 1 ? dim3((grid_x * (unsigned)k.S + 7) / 8 * 8 * groups) : dim3(grid_x, (unsigned)k.S);
+  hipLaunchKernelGGL(kern, grid, dim3(nwaves * 64), lds, st, a_in, k);
   return (int)hipGetLastError();
 }
 
