@@ -548,6 +548,12 @@ def main():
                 r = measure_workload(wtype, M, pool, max(5, args.steps // 3), 2)
                 extra["%s_m%d" % (args.wtype, M)] = {"GBps": r["GBps"], "ms_per_step": r["ms_per_step"],
                                                      dom_name: measure_shape(wtype, M, dom_name, pool, 3)}
+        # short batches: the whole groups of eight rows share a launch (weights read from memory once per launch)
+        for M in (16, 32):
+            if M != args.m:
+                r = measure_workload(wtype, M, pool, max(5, args.steps // 3), 2)
+                extra["%s_m%d" % (args.wtype, M)] = {"GBps": r["GBps"], "ms_per_step": r["ms_per_step"],
+                                                     "rows_per_ms": M / r["ms_per_step"]}
         del pool
         torch.cuda.empty_cache()
         other = ql.Q8_0 if wtype == ql.Q4_0 else ql.Q4_0

@@ -74,7 +74,7 @@ static size_t mfk_lds_bytes(int wtype, int nbs, int nwaves) {
 // blockDim = 64 x (row tiles per workgroup): three to eight waves, at least nbs / 16 (the threads hold one pass of
 // quantization items per activation row).  Waves beyond the row tiles that only help to quantize were measured: slower
 // (gate + up of the 4B layer at eight rows 11.6 -> 12.2 us with ten waves instead of five).
-template <int WT, int XT, int MT>
+template <int WT, int XT, int MT, bool GR = false>  // GR: several row groups in the launch
 __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int TH = MT / 4;
@@ -88,7 +88,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   // has its own L2): they read the same weights at about the same time, so the weights come from memory once.  The grid is
   // padded to whole eights of (column, slice) items; the padding leaves at once.
   int bx = blockIdx.x, slice = blockIdx.y, rg = 0, gx = gridDim.x;
-  if (k.groups > 1) {
+  if (GR) {
     const int L = blockIdx.x, seq = L >> 3;
     rg = seq % k.groups;
     const int item = (seq / k.groups) * 8 + (L & 7);
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   // its own partial sums and counters, and reads the same weights as its siblings.
   const void* const xptr =
       XT == GEMV_PREQ ? a.x : static_cast<const void*>(reinterpret_cast<const char*>(a.x) + (size_t)rg * MT * nb * QK * (XT == MLLM_HIP_F32 ? 4 : 2));
-  const int aM = min(a.M - rg * MT, MT), x86 = a.x86_scale;
+  const int aM = GR ? min(a.M - rg * MT, MT) : a.M, x86 = a.x86_scale;
   const int kNP = k.NP;
   float* const kpart = k.part + (size_t)rg * S * MT * kNP;
   unsigned* const kcnt = k.counters + rg * gx;

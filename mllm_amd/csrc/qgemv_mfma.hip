@@ -53,7 +53,9 @@ static int launch_mfk_t(const GemvArgs& a_in, const MfkArgs& k_in, int nwaves, u
   k.groups = (int)groups;
   const size_t lds = mfk_lds_bytes<MT>(WT, k.nbs, nwaves);
   if (lds > 160 * 1024) return MFK_NOT_TAKEN;
-  auto kern = gemv_mfk_kernel<WT, XT, MT>;
+  constexpr bool CAN_GROUP = MT == 8 && XT != GEMV_PREQ;  // the only form the launcher lets through with several groups
+  if (groups > 1 && !CAN_GROUP) return MFK_NOT_TAKEN;
+  auto kern = groups > 1 ? gemv_mfk_kernel<WT, XT, MT, CAN_GROUP> : gemv_mfk_kernel<WT, XT, MT, false>;
   if (lds > 64 * 1024)
     HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   // several row groups: a 1-D grid, (column, slice) items padded to whole eights, the groups of an item next to each other
