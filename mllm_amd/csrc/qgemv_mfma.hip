@@ -96,6 +96,10 @@ int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const v
   // workgroups, two per CU (10 + 2); the down projection (160 tiles x 8 slices): five -> exactly 256 workgroups.
   const int nw_min = std::max(3, (k.nbs + 15) / 16);
   int nwaves = waves;
+  // several row groups: four waves (measured over the 4B shapes with two to four groups against the model below, which counts
+  // rounds of workgroups although all of them are resident: down 15.7 -> 12.6 us at 16 rows and 21.7 -> 17.8 at 32, o at 32
+  // rows 13.5 -> 11.1, q+k+v at 24 rows 15.5 -> 12.2; q+k+v and o at 16 rows lose 0.8 us)
+  if ((nwaves < nw_min || nwaves > 8) && groups > 1) nwaves = std::max(nw_min, 4);
   if (nwaves < nw_min || nwaves > 8) {
     double best = 1e30;
     for (int nw = nw_min; nw <= 8; nw++) {
