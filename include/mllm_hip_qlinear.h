@@ -101,9 +101,10 @@ int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_hip_gemv_p
  * launch whose workgroups each quantize only their K slice of x and whose slices meet through the workspace: same results
  * bit for bit, about two thirds of the time at eight rows.  With less room it is the call above.  Calls that may overlap
  * on a GPU need workspaces of their own (the first 1024 different workspace addresses per GPU take this form).
- * From sixteen rows on, the whole groups of eight rows run in ONE such launch when the workspace has room for every
+ * With more than eight rows the groups of eight rows run in ONE such launch when the workspace has room for every
  * group's partial sums (mllm_hip_gemv_splitk_workspace_bytes with the real M): the groups share one pass over the
- * weights; row by row the bits of an eight-row call. */
+ * weights.  A last group of three to seven rows joins them; one or two remaining rows run as a pass of their own.  Row
+ * by row the bits of a call with that group of rows alone. */
 size_t mllm_hip_gemv_splitk_workspace_bytes(int M, int64_t K, int64_t N_total);
 int mllm_hip_linear_q_gemv_multi_wsn(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M,
                                      int64_t K, int act_scale_mode, void* workspace, size_t workspace_bytes, void* stream);

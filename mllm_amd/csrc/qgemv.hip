@@ -378,11 +378,11 @@ MLLM_API size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K) {
   return gemv_image_bytes(K);
 }
 
-// image, then the partial sums of the K slices of eight rows (each part's rows rounded up to 16), for every whole group of
-// eight rows from sixteen rows on
+// image, then the partial sums of the K slices of eight rows (each part's rows rounded up to 16), for every group of eight
+// rows
 MLLM_API size_t mllm_hip_gemv_splitk_workspace_bytes(int M, int64_t K, int64_t N_total) {
   if (M < 1 || K <= 0 || K % QK || N_total <= 0) return 0;
-  const size_t groups = M >= 16 ? (size_t)(M / 8) : 1;  // whole groups of eight rows share a launch
+  const size_t groups = (size_t)(M + 7) / 8;  // the groups of eight rows share a launch
   return gemv_image_bytes(K) + groups * (size_t)gemv_mfk_slices((int)(K / QK)) * 8 * (size_t)(N_total + 16 * GEMV_MAX_PARTS) * 4;
 }
 
@@ -405,11 +405,12 @@ static int gemv_check_args(int wtype, int nparts, const mllm_hip_gemv_part* part
   return 0;
 }
 
-// `groups` groups of eight rows of raw activations in one launch of the K-slice kernel; MFK_NOT_TAKEN where that kernel does
+// `rows` rows of raw activations as `groups` groups of eight (the last one may be shorter) in one launch of the K-slice kernel; MFK_NOT_TAKEN where that kernel does
 // not apply (the caller then runs passes)
 static int gemv_multi_groups(int wtype, int nparts, const mllm_hip_gemv_part* parts, const float* const* residual, const void* x,
-                             int x_dtype, int groups, int64_t K, int act_scale_mode, void* workspace, size_t ws_bytes, void* stream) {
-  RC_RET(gemv_check_args(wtype, nparts, parts, x, x_dtype, 8 * groups, K, act_scale_mode, workspace));
+                             int x_dtype, int rows, int groups, int64_t K, int act_scale_mode, void* workspace, size_t ws_bytes,
+                             void* stream) {
+  RC_RET(gemv_check_args(wtype, nparts, parts, x, x_dtype, rows, K, act_scale_mode, workspace));
   if (g_gemv_path == 1 || g_gemv_path == 2 || !workspace) return MFK_NOT_TAKEN;
   const size_t img = gemv_image_bytes(K);
   if (ws_bytes <= img) return MFK_NOT_TAKEN;
@@ -423,7 +424,7 @@ static int gemv_multi_groups(int wtype, int nparts, const mllm_hip_gemv_part* pa
   }
   a.nparts = nparts;
   a.x = x;
-  a.M = 8 * groups;
+  a.M = rows;
   a.nb = (int)(K / QK);
   a.nbp = (int)scale_row_stride(K);
   a.x86_scale = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
@@ -441,11 +442,15 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
   if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
   const size_t xrow = (size_t)K * (x_dtype == MLLM_HIP_F32 ? 4 : 2);
   int m_first = 0;
-  if (M >= 16) {
-    // the whole groups of eight rows in one launch of the K-slice kernel where it applies (room for every group's partial
-    // sums): the groups share one pass over the weights.  Row by row the bits of an eight-row call.
-    const int rc = gemv_multi_groups(wtype, nparts, parts, residual, x, x_dtype, M / 8, K, act_scale_mode, workspace, ws_bytes, stream);
-    if (rc == 0) m_first = M / 8 * 8;
+  // Groups of eight rows in one launch of the K-slice kernel where it applies (room for every group's partial sums): the
+  // groups share one pass over the weights.  A last group of three to seven rows joins them (the kernel it would run alone,
+  // with fewer rows filled); one or two remaining rows stay a pass of their own, on the kernel one or two rows always take.
+  // Row by row the bits of a call with that group alone.
+  const int rem = M % 8, groups = M / 8 + (rem >= 3 ? 1 : 0);
+  if (groups >= 2) {
+    const int rows = rem >= 3 ? M : M - rem;
+    const int rc = gemv_multi_groups(wtype, nparts, parts, residual, x, x_dtype, rows, groups, K, act_scale_mode, workspace, ws_bytes, stream);
+    if (rc == 0) m_first = rows;
     else if (rc != MFK_NOT_TAKEN) return rc;
   }
   for (int m0 = m_first; m0 < M; m0 += 8) {

@@ -64,11 +64,11 @@ static int launch_mfk_t(const GemvArgs& a_in, const MfkArgs& k_in, int nwaves, u
   return (int)hipGetLastError();
 }
 
-// groups > 1: a_in.M = 8 * groups rows of raw activations, every group of eight a workgroup of its own per (row tiles, slice)
+// groups > 1: a_in.M rows of raw activations in groups of eight (the last may be shorter), every group a workgroup of its own per (row tiles, slice)
 // in the same launch (the groups read the same weights: once from memory, then from the caches)
 int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const void* workspace, void* part, size_t part_bytes,
                     int waves, int slices, hipStream_t st, int groups) {
-  if (groups < 1 || groups > 65535 || (groups > 1 && (MT != 8 || x_kind == GEMV_PREQ || a_in.M != 8 * groups))) return MFK_NOT_TAKEN;
+  if (groups < 1 || groups > 65535 || (groups > 1 && (MT != 8 || x_kind == GEMV_PREQ || a_in.M <= 8 * (groups - 1) || a_in.M > 8 * groups))) return MFK_NOT_TAKEN;
   GemvArgs a = a_in;
   MfkArgs k{};
   int tiles_total = 0;
@@ -99,7 +99,9 @@ int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const v
   // several row groups: four waves (measured over the 4B shapes with two to four groups against the model below, which counts
   // rounds of workgroups although all of them are resident: down 15.7 -> 12.6 us at 16 rows and 21.7 -> 17.8 at 32, o at 32
   // rows 13.5 -> 11.1, q+k+v at 24 rows 15.5 -> 12.2; q+k+v and o at 16 rows lose 0.8 us)
-  if ((nwaves < nw_min || nwaves > 8) && groups > 1) nwaves = std::max(nw_min, 4);
+  // (cut rows only: whole rows want one workgroup per CU, which the model finds: 9728 x 2560 at 24 rows 13.6 us with eight
+  // waves = 228 workgroups, 21.4 with five = 366)
+  if ((nwaves < nw_min || nwaves > 8) && groups > 1 && k.S > 1) nwaves = std::max(nw_min, 4);
   if (nwaves < nw_min || nwaves > 8) {
     double best = 1e30;
     for (int nw = nw_min; nw <= 8; nw++) {

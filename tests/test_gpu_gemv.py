@@ -256,11 +256,12 @@ def test_gemv_argument_errors():
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
-@pytest.mark.parametrize("M", [16, 21, 32])
+@pytest.mark.parametrize("M", [11, 16, 18, 20, 21, 32])
 def test_gemv_groups_of_eight_rows_share_a_launch(wtype, M):
-    """from sixteen rows on, with room in the workspace for every group's partial sums, the whole groups of eight rows run in
-    one launch (the remaining rows as a pass of their own): row by row the bits of an eight-row call with the same kind of
-    workspace; cut rows, whole rows, several matrices, ragged N, a last slice that is empty"""
+    """more than eight rows, with room in the workspace for every group's partial sums: the groups of eight rows run in one
+    launch, a last group of three to seven rows with them (one or two remaining rows as a pass of their own): row by row the
+    bits of a call with that group alone and the same kind of workspace (a group of three or four rows alone runs the
+    four-row build of the kernel: same bits); cut rows, whole rows, several matrices, ragged N, a last slice that is empty"""
     rng = synth.rng_for(1, 900 + M + wtype)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(900 + M + wtype)
