@@ -307,11 +307,12 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
     case Scheme::kQ4_0:
     case Scheme::kQ8_0: {
       const int wt = scheme_ == Scheme::kQ4_0 ? MLLM_HIP_Q4_0 : MLLM_HIP_Q8_0;
-      // decode, and short batches as groups of eight rows over the same weights (from sixteen rows on the whole groups share
-      // one launch): measured on the Qwen3-4B projections against the short-batch matrix-core entry, 16 rows 8-15 us against
-      // 15-23, 32 rows 9-24 against 16-24 (a layer's seven projections together 108 against 128), 64 rows 171 against 154;
-      // against the exact tile kernel 64 rows 17-39 us against 70-235
-      if (M <= 32 || (gemm_packed_.isNil() && M <= 64)) {
+      // decode, and short batches as groups of eight rows over the same weights (the groups share one launch): measured on
+      // the Qwen3-4B projections against the short-batch matrix-core entry (gate / down / q / o, us): 16 rows 12.0 / 12.3 /
+      // 8.5 / 9.4 against 17.2 / 22.6 / 15.2 / 16.3; 48 rows 25.5 / 26.0 / 12.7 / 14.4 against 24.6 / 27.7 / 18.9 / 19.5;
+      // 64 rows 34.3 / 31.8 / 16.3 / 16.8 against 25.1 / 28.3 / 19.7 / 20.5 (a layer's seven projections: a tie).  Against
+      // the exact tile kernel: 128 rows 59.9 / 60.1 / 27.6 / 28.9 against 71.5 / 236.5 / 70.7 / 103.3
+      if (M <= 48 || (gemm_packed_.isNil() && M <= 128)) {
         const void* image = be.findImage(x.ptr<void>(), (int)M, K);
         mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
         // from three rows on: room for the partial sums of the K slices, which lets the rows run as one launch whose

@@ -73,12 +73,12 @@ def test_linear_through_the_op_factory(via_plugin):
     for scheme, wtype in (("q4_0", 0), ("q8_0", 1)):
         W = synth.make_weight(rng, wtype, N, K)
         bias = rng.standard_normal(N).astype(np.float32)
-        for M in (1, 5, 12, 20, 40):
+        for M in (1, 5, 12, 20, 40, 60):
             x = synth.make_x_fp32(rng, M, K)
             announce("host linear", scheme, M, "plugin", via_plugin)
-            # up to 32 rows: the decode GEMV, in groups of eight (fp32 block arithmetic); more: the matrix-core path (fp16
+            # up to 48 rows: the decode GEMV, in groups of eight (fp32 block arithmetic); more: the matrix-core path (fp16
             # operands, about 2e-4)
-            tol = 2e-6 if M <= 32 else 5e-4
+            tol = 2e-6 if M <= 48 else 5e-4
             y = _run(L, scheme, W, None, None, bias, x, False, M, N, K, 0, via_plugin)
             assert rel_l2(y, orc.linear_q(x, W, wtype, bias, orc.SCALE_X86_REF)) < tol
             bits, xf = synth.make_x_bf16(rng, M, K)
@@ -300,7 +300,7 @@ def test_decoder_mlp_through_the_op_factories(is_q8):
     Wg, Wu, Wd = (synth.make_weight(rng, is_q8, I, H), synth.make_weight(rng, is_q8, I, H), synth.make_weight(rng, is_q8, H, I))
     nw = (1 + 0.1 * rng.standard_normal(H)).astype(np.float32)
     vp = lambda a: a.ctypes.data_as(C.c_void_p)
-    for M in (1, 4, 8, 12, 24, 40):
+    for M in (1, 4, 8, 12, 24, 40, 60):
         x = synth.make_x_fp32(rng, M, H)
         ys, handed = [], []
         sm = np.empty((M, I), np.float32)
@@ -319,11 +319,11 @@ def test_decoder_mlp_through_the_op_factories(is_q8):
         g = orc.linear_q(h, Wg, is_q8, None, orc.SCALE_X86_REF)
         a = orc.silu(g) * orc.linear_q(h, Wu, is_q8, None, orc.SCALE_X86_REF)
         want = orc.linear_q(a, Wd, is_q8, None, orc.SCALE_X86_REF) + x
-        # up to 32 rows every Linear is the fp32 block arithmetic.  More rows: the matrix-core Linear (fp16 operands, 2e-4 per
+        # up to 48 rows every Linear is the fp32 block arithmetic.  More rows: the matrix-core Linear (fp16 operands, 2e-4 per
         # Linear on identical inputs, its own test); in a CHAIN the Q8_0 re-quantization in front of down_proj turns a
         # perturbation eps of its input into about sqrt(eps * 0.026) (codes flip at rounding boundaries), so the chain
         # is compared at 5e-3 and MLLM_HIP_PREFILL=blockdot keeps the fp32 arithmetic where that matters
-        assert rel_l2(ys[0], want) < (1e-3 if M <= 32 else 5e-3)
+        assert rel_l2(ys[0], want) < (1e-3 if M <= 48 else 5e-3)
         assert rel_l2(sm, orc.softmax(g)) < 1e-3
         assert np.array_equal(ti, orc.topk(sm, k, True, False)[1])
 
