@@ -445,13 +445,28 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
   // Groups of eight rows in one launch of the K-slice kernel where it applies (room for every group's partial sums): the
   // groups share one pass over the weights.  A last group of three to seven rows joins them (the kernel it would run alone,
   // with fewer rows filled); one or two remaining rows stay a pass of their own, on the kernel one or two rows always take.
-  // Row by row the bits of a call with that group alone.
-  const int rem = M % 8, groups = M / 8 + (rem >= 3 ? 1 : 0);
-  if (groups >= 2) {
-    const int rows = rem >= 3 ? M : M - rem;
-    const int rc = gemv_multi_groups(wtype, nparts, parts, residual, x, x_dtype, rows, groups, K, act_scale_mode, workspace, ws_bytes, stream);
-    if (rc == 0) m_first = rows;
-    else if (rc != MFK_NOT_TAKEN) return rc;
+  // Row by row the bits of a call with that group alone.  Where all groups together are refused (arrival counters or room
+  // for partial sums), halves of them are tried, and so on down to two groups per launch.
+  const int rem = M % 8, rows = rem >= 3 ? M : M - rem;
+  auto offset_parts = [&](int m0, mllm_hip_gemv_part* pp, const float** rr) {
+    for (int p = 0; p < nparts; p++) {
+      pp[p] = parts[p];
+      if (pp[p].y) pp[p].y += (size_t)m0 * parts[p].N;
+      rr[p] = (residual && residual[p]) ? residual[p] + (size_t)m0 * parts[p].N : nullptr;
+    }
+  };
+  for (int chunk = (rows + 7) / 8; chunk >= 2 && m_first == 0; chunk = chunk > 2 ? (chunk + 1) / 2 : 0) {
+    while (rows - m_first > 8) {  // at least two groups left
+      const int r = rows - m_first < chunk * 8 ? rows - m_first : chunk * 8;
+      mllm_hip_gemv_part pp[GEMV_MAX_PARTS];
+      const float* rr[GEMV_MAX_PARTS];
+      offset_parts(m_first, pp, rr);
+      const int rc = gemv_multi_groups(wtype, nparts, pp, residual ? rr : nullptr, reinterpret_cast<const char*>(x) + (size_t)m_first * xrow,
+                                       x_dtype, r, (r + 7) / 8, K, act_scale_mode, workspace, ws_bytes, stream);
+      if (rc == MFK_NOT_TAKEN) break;  // (the first launch of a chunk size decides: the later ones are no larger)
+      if (rc) return rc;
+      m_first += r;
+    }
   }
   for (int m0 = m_first; m0 < M; m0 += 8) {
     mllm_hip_gemv_part pp[GEMV_MAX_PARTS];

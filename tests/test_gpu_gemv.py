@@ -303,6 +303,24 @@ def test_gemv_groups_of_eight_rows_share_a_launch(wtype, M):
     assert torch.equal(yr, y + r)
 
 
+def test_gemv_groups_run_in_several_launches_when_one_is_refused():
+    """all groups of a batch in one launch need room for every group's partial sums and an arrival counter per (workgroup
+    column, group): with less of either the groups run as halves (quarters, ...) of the batch per launch, same bits"""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(77)
+    rng = synth.rng_for(1, 977)
+    # 8192 x 8192: rows of 256 blocks are always cut, 128 workgroup columns x 16 groups = 2048 counters > 1024
+    for (N, K, M, ws_rows) in ((8192, 8192, 128, 128), (300, 1024, 37, 16), (2560, 9728, 32, 16)):
+        w = ql.PackedQWeight.synthetic(0, N, K, gen)
+        xd = to_dev(synth.make_x_fp32(rng, M, K))
+        announce("gemv row groups in several launches", N, K, M, ws_rows)
+        (y,) = ql.linear_q_gemv_multi([w], xd, None, workspace=ql.gemv_workspace(ws_rows, K, N))
+        ws8 = ql.gemv_workspace(8, K, N)
+        for m0 in range(0, M, 8):
+            (part,) = ql.linear_q_gemv_multi([w], xd[m0:m0 + 8].contiguous(), None, workspace=ws8)
+            assert torch.equal(y[m0:m0 + 8], part), (N, K, M, m0)
+
+
 @pytest.mark.parametrize("wtype", [0, 1])
 @pytest.mark.parametrize("M", [1, 3, 8])
 def test_gemv_multi_equals_single(wtype, M):
