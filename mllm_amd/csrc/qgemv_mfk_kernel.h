@@ -1,4 +1,4 @@
-// Q4_0 / Q8_0 decode GEMV for three to eight activation rows on the matrix cores, K cut into slices that are separate
+// Q4_0 / Q8_0 decode GEMV for three to eight activation rows (and groups of such rows) on the matrix cores, K cut into slices that are separate
 // WORKGROUPS (qgemv_mfma_kernel.h keeps the slices of a row tile inside one workgroup).
 //
 // Same arithmetic and the same order of additions as that kernel (block sums with v_mfma_i32_16x16x64_i8, one fused
@@ -16,7 +16,10 @@
 //     through a 2 KB LDS stage that belongs to the wave (no barrier: LDS operations of one wave execute in order);
 //   * the slices of a row tile meet in global memory: every workgroup stores its partial sums, the one that arrives last
 //     at the tile's counter adds them up in slice order, applies bias / residual and stores y.  The counter goes back to
-//     zero, so the counters are zero between launches.
+//     zero, so the counters are zero between launches;
+//   * more than eight activation rows: groups of eight rows are further workgroups of the same launch (template parameter
+//     GR), each with its own rows of x and y, partial sums and counters; the groups of a (workgroup column, slice) item are
+//     neighbours on one XCD and read the same weights.
 #pragma once
 #include "qgemv_mfma_kernel.h"
 
@@ -53,8 +56,8 @@ __device__ __forceinline__ void pair_quantize(const float (&v)[16], bool ok, int
 }
 
 struct MfkArgs {
-  float* part;         // [S][MT][NP] partial sums (S > 1)
-  unsigned* counters;  // one per workgroup column (blockIdx.x), zero between launches (S > 1)
+  float* part;         // [row groups][S][MT][NP] partial sums (S > 1)
+  unsigned* counters;  // one per (workgroup column, row group), zero between launches (S > 1)
   int NP;              // columns of a partial row: every part's rows rounded up to 16
   int S, nbs;          // K slices; blocks per slice (a multiple of 8, at most MFK_MAX_NBS)
   int vs;              // blocks per summation chain (a multiple of 8): S > 1: nbs; S == 1: the length the slices would have
