@@ -50,7 +50,9 @@ enum { MLLM_HIP_SCALE_IEEE = 0, MLLM_HIP_SCALE_X86_REF = 1 };
 
 /* library / device ------------------------------------------------------------------------------------ */
 const char* mllm_hip_version(void);
-/* Selects nothing and allocates nothing; returns 0 when device `device` is a gfx950 part and the kernels load. */
+/* Selects nothing and allocates nothing; returns 0 when device `device` is a gfx950 part and the kernels load.  Also looks up
+ * the per-device addresses of the library's own device arrays and sets the kernels' LDS limits, so that later launches
+ * (e.g. under stream capture) make no such runtime call. */
 int mllm_hip_init(int device);
 
 /* ---------------------------------------------------------------------------------------------------------
@@ -100,7 +102,11 @@ int mllm_hip_linear_q_gemv_multi_ws(int wtype, int nparts, const mllm_hip_gemv_p
  * (mllm_hip_gemv_splitk_workspace_bytes; N_total = the rows of all parts together) three to eight activation rows take one
  * launch whose workgroups each quantize only their K slice of x and whose slices meet through the workspace: same results
  * bit for bit, about two thirds of the time at eight rows.  With less room it is the call above.  Calls that may overlap
- * on a GPU need workspaces of their own (the first 1024 different workspace addresses per GPU take this form).
+ * on a GPU need workspaces of their own.  The library keeps a block of arrival counters per workspace ADDRESS (1024 blocks
+ * per GPU, in its own device memory, zero between launches): give an address back with mllm_hip_gemv_workspace_release when
+ * the workspace is freed.  A caller that never does and walks through more than 1024 addresses pays one device
+ * synchronisation per 1024 new addresses (the blocks are then handed out afresh; said once on stderr); only under stream
+ * capture, where the device cannot be synchronised, does such a launch take the slower kernels instead.
  * With more than eight rows the groups of eight rows run in ONE such launch when the workspace has room for every
  * group's partial sums (mllm_hip_gemv_splitk_workspace_bytes with the real M): the groups share one pass over the
  * weights.  A last group of three to seven rows joins them; one or two remaining rows run as a pass of their own.  Row
@@ -109,12 +115,20 @@ size_t mllm_hip_gemv_splitk_workspace_bytes(int M, int64_t K, int64_t N_total);
 int mllm_hip_linear_q_gemv_multi_wsn(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int M,
                                      int64_t K, int act_scale_mode, void* workspace, size_t workspace_bytes, void* stream);
 
+/* Gives the counter block of a workspace address back (call it where the workspace is freed, after the work that used it has
+ * finished -- the rule of hipFree).  Unknown addresses are fine.  No counterpart in the reference. */
+int mllm_hip_gemv_workspace_release(const void* workspace);
+/* Counter blocks in use on `device`, their number, how often they were handed out afresh and how many launches were
+ * refused the K-slice kernel (any pointer may be NULL).  For tests and monitoring. */
+int mllm_hip_gemv_workspace_stats(int device, int* owned, int* capacity, long long* recycles, long long* refused);
+
 /* mllm_hip_linear_q_gemv_multi_wsn without a workspace argument and without any allocation.  No counterpart in the
  * reference; it exists for callers that cannot allocate device memory or carry a workspace around: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  The workspace is a static device array of the library
  * (327 680 bytes per GPU, held until the process ends: the quantized image of the activations and, where they fit behind
- * it, the partial sums of the K slices), whose per-device address mllm_hip_init(device) looks up (otherwise the first call
- * on a device does, which is not allowed during capture).  Same arguments otherwise, same results bit for bit as that call
+ * it, the partial sums of the K slices), whose per-device address mllm_hip_init(device) looks up together with the arrival
+ * counters and the LDS limits of the kernels (otherwise the first call on a device does, which is not allowed during
+ * capture).  Same arguments otherwise, same results bit for bit as that call
  * with a workspace of 327 680 bytes.  K <= 32768, else MLLM_HIP_E_SHAPE.  Every call on a GPU shares that GPU's array:
  * calls that overlap on one GPU (different streams) race; calls on one stream are ordered and safe. */
 int mllm_hip_linear_q_gemv_multi_static(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype,

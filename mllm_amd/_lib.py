@@ -56,6 +56,8 @@ def lib():
         L.mllm_hip_linear_q_gemv_multi_wsn.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp, C.c_size_t, vp]
         L.mllm_hip_gemv_splitk_workspace_bytes.restype = C.c_size_t
         L.mllm_hip_gemv_splitk_workspace_bytes.argtypes = [ci, i64, i64]
+        L.mllm_hip_gemv_workspace_release.argtypes = [vp]
+        L.mllm_hip_gemv_workspace_stats.argtypes = [ci, C.POINTER(ci), C.POINTER(ci), C.POINTER(C.c_longlong), C.POINTER(C.c_longlong)]
         L.mllm_hip_linear_q_gemv_multi_static.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_linear_q_gemv_fused.argtypes = [ci, ci, C.POINTER(GemvPart), C.POINTER(GemvFusion), vp, ci, ci, i64, ci, vp]
         L.mllm_hip_mlp_gate_up_q.argtypes = [ci, vp, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]

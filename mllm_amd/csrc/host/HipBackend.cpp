@@ -39,7 +39,9 @@ void HipAllocator::free(Storage* storage) {
   if (storage->ptr_ && owner) owner->noteWrite(storage->ptr_, storage->size_);
   if (storage->ptr_) {
     live_.erase(static_cast<const char*>(storage->ptr_));
-    (void)hipFree(storage->ptr_);
+    (void)hipFree(storage->ptr_);  // (waits for the device: nothing uses the memory any more)
+    // the memory may have been a decode-GEMV workspace: its address gives the block of arrival counters back
+    (void)mllm_hip_gemv_workspace_release(storage->ptr_);
   }
   storage->ptr_ = nullptr;
 }

@@ -265,18 +265,35 @@ struct __attribute__((packed)) V2Param {
 };
 static_assert(sizeof(V2Header) == 532 && sizeof(V2Param) == 352, "model file v2 layout");
 
+// Offsets and lengths come from the file: every range check is written so that it cannot wrap (n > size || off > size - n),
+// and nothing is allocated from a length that exceeds the file.
+bool rangeInside(uint64_t off, uint64_t n, uint64_t size) { return n <= size && off <= size - n; }
+
 template <typename T>
 T take(const std::vector<char>& buf, size_t& pos) {
-  MLLM_RT_ASSERT(pos + sizeof(T) <= buf.size());
+  MLLM_RT_ASSERT(pos <= buf.size() && sizeof(T) <= buf.size() - pos);
   T v;
   std::memcpy(&v, buf.data() + pos, sizeof(T));
   pos += sizeof(T);
   return v;
 }
-Tensor readTensor(std::ifstream& f, const std::string& name, const Tensor::shape_t& shape, DataTypes dtype, uint64_t offset,
-                  uint64_t stored_bytes) {
+// bytes a tensor of this shape and type occupies, without allocating it; UINT64_MAX for a negative extent or an overflow
+uint64_t shapeBytes(const Tensor::shape_t& shape, DataTypes dtype) {
+  uint64_t numel = 1;
+  for (int32_t d : shape) {
+    if (d < 0) return UINT64_MAX;
+    if (d != 0 && numel > (UINT64_MAX / 64) / (uint64_t)d) return UINT64_MAX;
+    numel *= (uint64_t)d;
+  }
+  return numel / lanesOfType(dtype) * bytesOfType(dtype);
+}
+Tensor readTensor(std::ifstream& f, uint64_t file_size, const std::string& name, const Tensor::shape_t& shape, DataTypes dtype,
+                  uint64_t offset, uint64_t stored_bytes) {
+  const uint64_t need = shapeBytes(shape, dtype);
+  if (stored_bytes < need || !rangeInside(offset, need, file_size))
+    MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: tensor '%s' is truncated", name.c_str());
   Tensor t = Tensor::empty(shape, dtype, kCPU).alloc();
-  MLLM_RT_ASSERT(stored_bytes >= t.bytes());
+  MLLM_RT_ASSERT(need == t.bytes());
   f.seekg((std::streamoff)offset, std::ios::beg);
   f.read(t.ptr<char>(), (std::streamsize)t.bytes());
   if (!f) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: tensor '%s' is truncated", name.c_str());
@@ -288,14 +305,16 @@ Tensor readTensor(std::ifstream& f, const std::string& name, const Tensor::shape
 // The parsing is the same for a mapped file and for one that is read tensor by tensor: `bytes(offset, n)` hands out the
 // descriptor bytes, `tensor(...)` makes the tensor (a view into the mapping, or a copy read from the stream).
 template <typename Bytes, typename MakeTensor>
-static void parseModelFile(const std::string& file_name, ModelFileVersion version, const ParameterFile::ptr_t& pf, Bytes&& bytes,
-                           MakeTensor&& tensor) {
+static void parseModelFile(const std::string& file_name, ModelFileVersion version, uint64_t file_size, const ParameterFile::ptr_t& pf,
+                           Bytes&& bytes, MakeTensor&& tensor) {
   if (version == ModelFileVersion::kV1) {
     int32_t magic = 0;
     uint64_t desc_bytes = 0;
     bytes(0, 4, &magic);
     bytes(4, 8, &desc_bytes);
     MLLM_RT_ASSERT_EQ(kV1Magic, magic);
+    if (!rangeInside(12, desc_bytes, file_size))
+      MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
     std::vector<char> buf(desc_bytes);
     bytes(12, desc_bytes, buf.data());
     struct Item { std::string name; uint64_t len, offset; int32_t dtype; };
@@ -303,7 +322,7 @@ static void parseModelFile(const std::string& file_name, ModelFileVersion versio
     for (size_t pos = 0; pos < buf.size();) {
       Item it;
       const uint32_t name_len = take<uint32_t>(buf, pos);
-      MLLM_RT_ASSERT(pos + name_len <= buf.size());
+      MLLM_RT_ASSERT(name_len <= buf.size() - pos);
       it.name.assign(buf.data() + pos, name_len);
       pos += name_len;
       it.len = take<uint64_t>(buf, pos);
@@ -321,6 +340,8 @@ static void parseModelFile(const std::string& file_name, ModelFileVersion versio
     bytes(0, sizeof(h), &h);
     MLLM_RT_ASSERT_EQ(kV2Magic, h.magic_number);
     MLLM_RT_ASSERT_EQ(kV2Version, h.version);
+    if (!rangeInside(h.params_desc_offset, (uint64_t)h.num_params * sizeof(V2Param), file_size))
+      MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
     std::vector<V2Param> descs(h.num_params);
     bytes(h.params_desc_offset, descs.size() * sizeof(V2Param), descs.data());  // an extra data segment in front of it is skipped
     for (const auto& d : descs) {
@@ -360,15 +381,17 @@ ParameterFile::ptr_t load(const std::string& file_name, ModelFileVersion version
     char* base = static_cast<char*>(mf->data());
     const size_t size = mf->size();
     parseModelFile(
-        file_name, version, pf,
+        file_name, version, size, pf,
         [&](uint64_t off, uint64_t n, void* dst) {
-          if (off + n > size) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
+          if (!rangeInside(off, n, size)) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
           std::memcpy(dst, base + off, n);
         },
         [&](const std::string& name, const Tensor::shape_t& shape, DataTypes dtype, uint64_t offset, uint64_t stored_bytes) {
+          const uint64_t need = shapeBytes(shape, dtype);
+          if (stored_bytes < need || !rangeInside(offset, need, size))
+            MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: tensor '%s' is truncated", name.c_str());
           Tensor t = Tensor::fromExternal(base + offset, shape, dtype, kCPU);
-          MLLM_RT_ASSERT(stored_bytes >= t.bytes());
-          if (offset + t.bytes() > size) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: tensor '%s' is truncated", name.c_str());
+          MLLM_RT_ASSERT(need == t.bytes());
           t.setName(name);
           return t;
         });
@@ -376,15 +399,18 @@ ParameterFile::ptr_t load(const std::string& file_name, ModelFileVersion version
   }
   std::ifstream f(file_name, std::ios::binary);
   if (!f.is_open()) MLLM_ERROR_EXIT(ExitCode::kIOError, "Failed to open file for reading: %s", file_name.c_str());
+  f.seekg(0, std::ios::end);
+  const uint64_t fsize = (uint64_t)std::max<std::streamoff>(0, f.tellg());
   parseModelFile(
-      file_name, version, pf,
+      file_name, version, fsize, pf,
       [&](uint64_t off, uint64_t n, void* dst) {
+        if (!rangeInside(off, n, fsize)) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
         f.seekg((std::streamoff)off, std::ios::beg);
         f.read(static_cast<char*>(dst), (std::streamsize)n);
         if (!f) MLLM_ERROR_EXIT(ExitCode::kIOError, "model file: descriptor section truncated: %s", file_name.c_str());
       },
       [&](const std::string& name, const Tensor::shape_t& shape, DataTypes dtype, uint64_t offset, uint64_t stored_bytes) {
-        return readTensor(f, name, shape, dtype, offset, stored_bytes);
+        return readTensor(f, fsize, name, shape, dtype, offset, stored_bytes);
       });
   return pf;
 }

@@ -427,7 +427,10 @@ void initializeContext();                       // registers the host (CPU) allo
 // Model files, mllm/mllm.cpp:135-154 with mllm/core/ParameterFile.cpp:68-440 and the schemas
 // mllm/core/schema/ModelFileV1.hpp:36-52 (magic 20012; name, byte length, offset, dtype per tensor; shapes are flat) and
 // ModelFileV2.hpp:40-62 (magic 0x519A, version 2; 352-byte descriptors with dtype, size, offset, shape, name).
-// Tensors come back as host tensors that own their memory; `mmap` is accepted and ignored (always a buffered read).
+// mmap = true (the reference's default): the file is mapped read-only and the tensors are views into the mapping, which the
+// ParameterFile keeps alive; mmap = false: every tensor is read into host memory of its own.  Offsets and lengths read from
+// the file are checked against the file size in a form that cannot wrap; a file that fails a check ends the process as any
+// other load error does.
 ParameterFile::ptr_t load(const std::string& file_name, ModelFileVersion version = ModelFileVersion::kV1,
                           DeviceTypes map_2_device = kCPU, bool mmap = true);
 void save(const std::string& file_name, const ParameterFile::ptr_t& parameter_file,

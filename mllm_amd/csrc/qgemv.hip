@@ -13,6 +13,7 @@
 #include <string.h>
 
 #include <initializer_list>
+#include <mutex>
 
 namespace mllmhip {
 
@@ -276,10 +277,12 @@ constexpr size_t GEMV_STATIC_BYTES = (size_t)8 * (GEMV_STATIC_MAX_K / QK) * 40; 
 static __device__ __align__(256) unsigned char scratch[GEMV_STATIC_BYTES];
 constexpr int MAX_DEVICES = 64;
 static void* g_scratch_ptr[MAX_DEVICES];
+static std::mutex g_scratch_mutex;
 
 // device address of the scratch array on `device`, which must be the current device; 0 + *out on success
 static int static_scratch(int device, void** out) {
   if (device < 0 || device >= MAX_DEVICES) return MLLM_HIP_E_NODEVICE;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (!g_scratch_ptr[device]) {
     void* p = nullptr;
     HIP_RET(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
@@ -301,10 +304,24 @@ MLLM_API int mllm_hip_init(int device) {
   int cur = 0;
   HIP_RET(hipGetDevice(&cur));
   if (cur != device) HIP_RET(hipSetDevice(device));
+  // ... and everything else a first launch would otherwise look up or set: the arrival counters of the K-slice kernels and
+  // the dynamic-LDS limits of the matrix-core GEMV kernels, so that a launch under stream capture makes no such call
   void* p = nullptr;
-  const int rc = static_scratch(device, &p);
+  int rc = static_scratch(device, &p);
+  if (!rc) rc = gemv_mfk_prepare_device();
   if (cur != device) HIP_RET(hipSetDevice(cur));
   return rc;
+}
+
+MLLM_API int mllm_hip_gemv_workspace_release(const void* workspace) {
+  if (!workspace) return MLLM_HIP_E_BADARG;
+  return gemv_mfk_release(workspace);
+}
+
+MLLM_API int mllm_hip_gemv_workspace_stats(int device, int* owned, int* capacity, long long* recycles, long long* refused) {
+  if (device < 0) return MLLM_HIP_E_BADARG;
+  gemv_mfk_stats(device, owned, capacity, recycles, refused);
+  return 0;
 }
 
 MLLM_API int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream) {

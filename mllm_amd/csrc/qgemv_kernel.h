@@ -409,11 +409,15 @@ int launch_gemv_mfma(int wtype, int x_kind, int MT, const GemvArgs& a, int waves
 bool gemv_mfma_fits(int MT, int nb);  // rows of nb blocks fit that kernel's LDS
 // The matrix-core kernel with the K slices as separate workgroups.  image_ws: where a raw x could be quantized first (unused
 // so far); part / part_bytes: room for the slices' partial sums (may be null / 0).  Returns MFK_NOT_TAKEN when the launch
-// does not fit (no room for the partial sums, no free counter block, slices too long): the caller takes another kernel.
+// does not fit (no room for the partial sums, no counter block to be had under stream capture, slices too long): the caller
+// takes another kernel.
 constexpr int MFK_NOT_TAKEN = 1;
 int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a, const void* workspace, void* part, size_t part_bytes, int waves,
                     int slices, hipStream_t st, int groups = 1);
 int gemv_mfk_slices(int nb);
+int gemv_mfk_prepare_device();                 // counter table and kernel attributes of the current device (mllm_hip_init)
+int gemv_mfk_release(const void* workspace);   // the workspace address gives its counter block back
+void gemv_mfk_stats(int device, int* owned, int* capacity, long long* recycles, long long* refused);
 int launch_gemv_q4_f32(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
 int launch_gemv_q4_bf16(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);
 int launch_gemv_q8_f32(const GemvArgs& a, int MT, GemvShape s, hipStream_t st);

@@ -425,10 +425,17 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   }
 
   // ---- 6. the slices of a tile meet in global memory ------------------------------------------------------------------------------
-  // Partial sums leave with device-scope stores (written through this chip-let's L2); the barrier makes every wave wait until
-  // its stores are acknowledged; then thread 0 counts the workgroup in.  A release fence in every wave (or even one per
-  // workgroup) makes the hardware look through the whole L2 for dirty lines and cost 5 to 50 us per launch; nothing but these
-  // stores has to be visible to the workgroup that arrives last, and it reads them with device-scope loads.
+  // Ordering between workgroups, stated step by step (nothing here is left to what a barrier happens to wait for):
+  //   producer  (a) partial sums leave with device-scope stores (written through this chip-let's L2 to where the other
+  //                 chip-lets read them);
+  //             (b) every wave waits until the memory system has acknowledged all its stores (s_waitcnt vmcnt(0): on this
+  //                 chip stores count in vmcnt until they are acknowledged);
+  //             (c) the workgroup barrier: all waves have passed (b);
+  //             (d) thread 0 counts the workgroup in with a device-scope atomic add.
+  //   consumer  (e) thread 0 of the workgroup that sees the last count tells its workgroup through LDS and a barrier;
+  //             (f) its waves read the partial sums with device-scope loads, issued after that barrier.
+  // A release fence in place of (b) (in every wave, or even one per workgroup) makes the hardware write back this
+  // chip-let's whole L2 and cost 5 to 50 us per launch; nothing but these stores has to be visible to the consumer.
   const int col = pcol0 + n;
   if (tile_ok && q == 0) {
 #pragma unroll
@@ -440,14 +447,16 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
       __hip_atomic_store(dst + 3, acc[h].w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
-  __syncthreads();
+  __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (b)
+  __syncthreads();                                       // (c)
   if (tid == 0) {
-    const unsigned old = atomicAdd(kcnt + bx, 1u);
+    const unsigned old = __hip_atomic_fetch_add(kcnt + bx, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (d)
     const int last = old == (unsigned)(S - 1);
-    if (last) kcnt[bx] = 0u;  // every slice has arrived: ready for the next launch
+    // every slice has arrived: ready for the next launch
+    if (last) __hip_atomic_store(kcnt + bx, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     *s_flag = last;
   }
-  __syncthreads();
+  __syncthreads();  // (e)
   if (!*s_flag || !tile_ok) return;
   // the workgroup that arrived last: lane l of a wave sums outputs (activation row l / 16 + 4 i, weight row l % 16) of its
   // tile over the slices, slice 0 first; the loads of up to eight slices are in flight together

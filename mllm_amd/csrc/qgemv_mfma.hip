@@ -1,6 +1,10 @@
 // Launchers of the matrix-core decode GEMV (three to eight activation rows); the kernel is in qgemv_mfma_kernel.h.
+#include <stdio.h>
+
 #include <algorithm>
 #include <mutex>
+#include <unordered_map>
+#include <vector>
 
 #include "qgemv_mfk_kernel.h"
 
@@ -10,37 +14,137 @@ namespace mllmhip {
 // Arrival counters of the row tiles: device memory of the loaded code object, zero when the code object is loaded and put
 // back to zero by every launch that uses them.  The name below is a host-side stand-in; kernels get the device address that
 // hipGetSymbolAddress returned for the current device.  Launches that may run at the same time must not share counters:
-// the array is cut into blocks and a block belongs to one workspace address for good (callers already keep one workspace
-// per concurrent call).  A workspace that finds no free block (1024 addresses per GPU) takes the other kernels.
+// the array is cut into blocks and a block belongs to one workspace address (callers already keep one workspace per
+// concurrent call) until that address is released (mllm_hip_gemv_workspace_release) or the table is recycled: when a new
+// address finds every block taken, the device is synchronised -- after which no launch is in flight and every counter is
+// zero -- and all blocks are handed out afresh.  A caller that walks through ever new workspace addresses therefore pays one
+// device synchronisation per MFK_BLOCKS new addresses instead of losing this kernel.  Only a stream under capture cannot
+// synchronise: that launch takes the other kernels (MFK_NOT_TAKEN) and the library says so once on stderr.
 constexpr int MFK_BLOCKS = 1024, MFK_COUNTERS = 1024, MFK_MAX_DEVICES = 64;
 static __device__ __align__(256) unsigned mfk_counters[MFK_BLOCKS * MFK_COUNTERS];  // 4 MB per GPU
-static unsigned* g_mfk_ptr[MFK_MAX_DEVICES];
-static const void* g_mfk_owner[MFK_MAX_DEVICES][MFK_BLOCKS];
+struct MfkTable {
+  unsigned* base = nullptr;                     // device address of mfk_counters on this device
+  std::unordered_map<const void*, int> block;   // workspace address -> block
+  std::vector<int> free_blocks;
+  bool prepared = false;                        // dynamic-LDS attributes of the kernels set on this device
+  uint64_t recycles = 0, refused = 0;
+};
+static MfkTable g_mfk[MFK_MAX_DEVICES];
 static std::mutex g_mfk_mutex;
+static bool g_mfk_said_recycle = false, g_mfk_said_refused = false;
 
-// 0 and *out = the counter block of `workspace` on the current device; MFK_NOT_TAKEN when every block has another owner
-static int mfk_counter_block(const void* workspace, unsigned** out) {
+// every instantiation the launchers below can pick: the limit of dynamic LDS is a per-device attribute of a kernel and is
+// set once here instead of in front of every launch (a launch under stream capture then makes no other runtime call)
+template <int WT, int XT, int MT>
+static int mfk_set_lds_attr() {
+  HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mfk_kernel<WT, XT, MT, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mfma_kernel<WT, XT, MT, false>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  if constexpr (MT == 8 && XT != GEMV_PREQ)
+    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mfk_kernel<WT, XT, MT, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  return 0;
+}
+template <int WT>
+static int mfk_set_lds_attr_w() {
+  RC_RET((mfk_set_lds_attr<WT, MLLM_HIP_F32, 4>()));
+  RC_RET((mfk_set_lds_attr<WT, MLLM_HIP_F32, 8>()));
+  RC_RET((mfk_set_lds_attr<WT, MLLM_HIP_BF16, 4>()));
+  RC_RET((mfk_set_lds_attr<WT, MLLM_HIP_BF16, 8>()));
+  RC_RET((mfk_set_lds_attr<WT, GEMV_PREQ, 4>()));
+  RC_RET((mfk_set_lds_attr<WT, GEMV_PREQ, 8>()));
+  return 0;
+}
+
+// the table of the current device, ready for launches (counter address looked up, kernel attributes set); g_mfk_mutex held
+static int mfk_table_locked(MfkTable** out) {
   int dev = 0;
   HIP_RET(hipGetDevice(&dev));
-  if (dev < 0 || dev >= MFK_MAX_DEVICES) return MFK_NOT_TAKEN;
-  std::lock_guard<std::mutex> lock(g_mfk_mutex);
-  if (!g_mfk_ptr[dev]) {
+  if (dev < 0 || dev >= MFK_MAX_DEVICES) return MLLM_HIP_E_NODEVICE;
+  MfkTable& t = g_mfk[dev];
+  if (!t.base) {
     void* p = nullptr;
     HIP_RET(hipGetSymbolAddress(&p, HIP_SYMBOL(mfk_counters)));
     if (!p) return MLLM_HIP_E_NODEVICE;
-    g_mfk_ptr[dev] = static_cast<unsigned*>(p);
+    t.base = static_cast<unsigned*>(p);
+    t.free_blocks.reserve(MFK_BLOCKS);
+    for (int b = MFK_BLOCKS - 1; b >= 0; b--) t.free_blocks.push_back(b);
   }
-  // open addressing from a hash of the address; an address keeps its block for the life of the process
-  const size_t h0 = (reinterpret_cast<uintptr_t>(workspace) >> 8) * 0x9E3779B97F4A7C15ull >> 40;
-  for (int i = 0; i < MFK_BLOCKS; i++) {
-    const int b = (int)((h0 + i) % MFK_BLOCKS);
-    if (g_mfk_owner[dev][b] == workspace || !g_mfk_owner[dev][b]) {
-      g_mfk_owner[dev][b] = workspace;
-      *out = g_mfk_ptr[dev] + (size_t)b * MFK_COUNTERS;
-      return 0;
+  if (!t.prepared) {
+    RC_RET(mfk_set_lds_attr_w<MLLM_HIP_Q4_0>());
+    RC_RET(mfk_set_lds_attr_w<MLLM_HIP_Q8_0>());
+    t.prepared = true;
+  }
+  *out = &t;
+  return 0;
+}
+
+// what mllm_hip_init does for these kernels on the device that is current
+int gemv_mfk_prepare_device() {
+  std::lock_guard<std::mutex> lock(g_mfk_mutex);
+  MfkTable* t = nullptr;
+  return mfk_table_locked(&t);
+}
+
+// 0 and *out = the counter block of `workspace` on the current device; MFK_NOT_TAKEN when every block has an owner and the
+// device cannot be synchronised now (stream capture)
+static int mfk_counter_block(const void* workspace, hipStream_t st, unsigned** out) {
+  std::lock_guard<std::mutex> lock(g_mfk_mutex);
+  MfkTable* t = nullptr;
+  RC_RET(mfk_table_locked(&t));
+  auto it = t->block.find(workspace);
+  if (it == t->block.end()) {
+    if (t->free_blocks.empty()) {
+      // every block has an owner.  Once the device is idle no launch uses any counter and all of them are zero, so every
+      // owner can lose its block (an owner that comes back simply takes a new one).
+      hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+      const bool capturing = hipStreamIsCapturing(st, &cs) != hipSuccess || cs != hipStreamCaptureStatusNone;
+      if (capturing || hipDeviceSynchronize() != hipSuccess) {
+        (void)hipGetLastError();
+        t->refused++;
+        if (!g_mfk_said_refused) {
+          g_mfk_said_refused = true;
+          fprintf(stderr, "mllm_hip: all %d counter blocks of the K-slice decode GEMV belong to other workspaces and the device cannot be "
+                          "synchronised during stream capture; this launch takes the slower kernels (release workspaces with "
+                          "mllm_hip_gemv_workspace_release, or reuse them)\n", MFK_BLOCKS);
+        }
+        return MFK_NOT_TAKEN;
+      }
+      t->block.clear();
+      t->free_blocks.clear();
+      for (int b = MFK_BLOCKS - 1; b >= 0; b--) t->free_blocks.push_back(b);
+      t->recycles++;
+      if (!g_mfk_said_recycle) {
+        g_mfk_said_recycle = true;
+        fprintf(stderr, "mllm_hip: more than %d workspace addresses have used the K-slice decode GEMV; the device was synchronised to "
+                        "hand its counter blocks out afresh (release workspaces with mllm_hip_gemv_workspace_release, or reuse them, "
+                        "to avoid this)\n", MFK_BLOCKS);
+      }
     }
+    const int b = t->free_blocks.back();
+    t->free_blocks.pop_back();
+    it = t->block.emplace(workspace, b).first;
   }
-  return MFK_NOT_TAKEN;
+  *out = t->base + (size_t)it->second * MFK_COUNTERS;
+  return 0;
+}
+
+int gemv_mfk_release(const void* workspace) {
+  std::lock_guard<std::mutex> lock(g_mfk_mutex);
+  for (MfkTable& t : g_mfk) {
+    auto it = t.block.find(workspace);
+    if (it == t.block.end()) continue;
+    t.free_blocks.push_back(it->second);
+    t.block.erase(it);
+  }
+  return 0;
+}
+
+void gemv_mfk_stats(int device, int* owned, int* capacity, long long* recycles, long long* refused) {
+  std::lock_guard<std::mutex> lock(g_mfk_mutex);
+  const bool ok = device >= 0 && device < MFK_MAX_DEVICES;
+  if (owned) *owned = ok ? (int)g_mfk[device].block.size() : 0;
+  if (capacity) *capacity = MFK_BLOCKS;
+  if (recycles) *recycles = ok ? (long long)g_mfk[device].recycles : 0;
+  if (refused) *refused = ok ? (long long)g_mfk[device].refused : 0;
 }
 
 // slices of a row when it is cut: the ones of the one-workgroup kernel (at most eight) up to 512 blocks, then slices of 64
@@ -56,8 +160,7 @@ static int launch_mfk_t(const GemvArgs& a_in, const MfkArgs& k_in, int nwaves, u
   constexpr bool CAN_GROUP = MT == 8 && XT != GEMV_PREQ;  // the only form the launcher lets through with several groups
   if (groups > 1 && !CAN_GROUP) return MFK_NOT_TAKEN;
   auto kern = groups > 1 ? gemv_mfk_kernel<WT, XT, MT, CAN_GROUP> : gemv_mfk_kernel<WT, XT, MT, false>;
-  if (lds > 64 * 1024)
-    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  if (lds > 64 * 1024) RC_RET(gemv_mfk_prepare_device());  // (sets the kernels' dynamic-LDS limit once per device)
   // several row groups: a 1-D grid, (column, slice) items padded to whole eights, the groups of an item next to each other
   const dim3 grid = groups > 1 ? dim3((grid_x * (unsigned)k.S + 7) / 8 * 8 * groups) : dim3(grid_x, (unsigned)k.S);
   hipLaunchKernelGGL(kern, grid, dim3(nwaves * 64), lds, st, a_in, k);
@@ -128,7 +231,7 @@ int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const v
   k.NP = np;
   if (k.S > 1) {
     if (!workspace || !part || (size_t)groups * k.S * MT * np * 4 > part_bytes || (size_t)grid * groups > (size_t)MFK_COUNTERS) return MFK_NOT_TAKEN;
-    RC_RET(mfk_counter_block(workspace, &k.counters));
+    RC_RET(mfk_counter_block(workspace, st, &k.counters));
     k.part = static_cast<float*>(part);
   }
 #define MFK_CASE(WT_, XT_)                                                         \
@@ -163,8 +266,7 @@ static int launch_mfma_t(const GemvArgs& a_in, int waves, int slices, hipStream_
   const size_t lds = mf_lds_bytes<MT>(a.nb, nbs, nwaves);
   if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
   auto kern = gemv_mfma_kernel<WT, XT, MT, false>;
-  if (lds > 64 * 1024)
-    HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  if (lds > 64 * 1024) RC_RET(gemv_mfk_prepare_device());
   hipLaunchKernelGGL(kern, dim3(grid), dim3(nwaves * 64), lds, st, a, S, nbs, MfmaMlpOut{nullptr, nullptr, 0});
   return (int)hipGetLastError();
 }

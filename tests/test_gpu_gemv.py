@@ -437,6 +437,62 @@ def test_gemv_k_slices_as_workgroups_give_the_same_bits(wtype, M):
     assert L.mllm_hip_gemv_splitk_workspace_bytes(0, 96, 100) == 0
 
 
+def _counter_stats():
+    import ctypes as C
+    owned, cap = C.c_int(), C.c_int()
+    rec, ref = C.c_longlong(), C.c_longlong()
+    assert _lib.lib().mllm_hip_gemv_workspace_stats(0, C.byref(owned), C.byref(cap), C.byref(rec), C.byref(ref)) == 0
+    return owned.value, cap.value, rec.value, ref.value
+
+
+def test_gemv_k_slices_keep_their_kernel_over_more_workspace_addresses_than_counter_blocks():
+    """The K-slice kernel keeps one block of arrival counters per workspace ADDRESS.  A caller that walks through more
+    addresses than there are blocks must still get that kernel: same bits as the first call (Q8_0 at four rows, where the
+    kernels that would otherwise run add the blocks in another order and give other bits), nothing refused, the blocks handed
+    out afresh at least once, and about the same time per call.  A released address gives its block back."""
+    import time
+    rng = synth.rng_for(1, 4242)
+    L = _lib.lib()
+    M, N, K = 4, 200, 64 * 32
+    W = synth.make_weight(rng, 1, N, K)
+    w = ql.PackedQWeight(1, torch.from_numpy(W))
+    x = to_dev(synth.make_x_fp32(rng, M, K))
+    need = L.mllm_hip_gemv_splitk_workspace_bytes(M, K, N)
+    stride = (need + 255) // 256 * 256
+    _, cap, rec0, ref0 = _counter_stats()
+    count = cap + 76
+    pool = torch.empty(stride * count, dtype=torch.uint8, device="cuda")
+    announce("gemv k slices: workspace addresses", count, "counter blocks", cap)
+    first = ql.linear_q_gemv_multi([w], x, workspace=pool[:need])[0]
+    want = orc.linear_q(x.cpu().numpy(), W, 1, None, orc.SCALE_X86_REF)
+    assert rel_l2(first.cpu().numpy(), want) < 2e-6
+    assert L.mllm_hip_gemv_set_path(2) == 0  # without the K-slice kernel: the bits differ (that is what makes this a test)
+    try:
+        other = ql.linear_q_gemv_multi([w], x, workspace=pool[:need])[0]
+    finally:
+        assert L.mllm_hip_gemv_set_path(0) == 0
+    assert not torch.equal(first, other)
+    torch.cuda.synchronize()
+    times = []
+    for i in range(count):
+        wsp = pool[i * stride:i * stride + need]
+        t0 = time.perf_counter()
+        y = ql.linear_q_gemv_multi([w], x, workspace=wsp)[0]
+        times.append(time.perf_counter() - t0)
+        assert torch.equal(y, first), i
+    torch.cuda.synchronize()
+    owned, _, rec1, ref1 = _counter_stats()
+    assert ref1 == ref0 and rec1 >= rec0 + 1 and 1 <= owned <= cap
+    # the calls after the table was handed out afresh cost what the early ones did (host time per call, median)
+    early, late = sorted(times[10:110])[50], sorted(times[-60:])[30]
+    assert late < 3 * early + 20e-6, (early, late)
+    # release: the address of the last call gives its block back, an unknown address is fine
+    assert L.mllm_hip_gemv_workspace_release(wsp.data_ptr()) == 0
+    assert _counter_stats()[0] == owned - 1
+    assert L.mllm_hip_gemv_workspace_release(wsp.data_ptr()) == 0
+    assert L.mllm_hip_gemv_workspace_release(None) == -1
+
+
 @pytest.mark.parametrize("wtype", [0, 1])
 @pytest.mark.parametrize("M", [4, 8])
 def test_gemv_k_slices_as_workgroups_take_rows_of_any_length(wtype, M):

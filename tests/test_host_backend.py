@@ -264,6 +264,66 @@ def test_model_file_readers_and_writers(tmp_path):
     assert sorted(names) == sorted(n for n, _, _, _ in tensors)
 
 
+def _load_in_child(path, version, name, mmap):
+    """mllm::load ends the process on a bad file (as the reference's MLLM_ERROR_EXIT does): run it in a child"""
+    fn = "mllm_hip_host_file_tensor_is_mapped_view" if mmap else "mllm_hip_host_file_tensor"
+    if mmap:
+        call = "L.%s(%r, %d, %r)" % (fn, path.encode(), version, name.encode())
+    else:
+        call = ("L.%s(%r, %d, %r, ctypes.byref(ctypes.c_int32()), ctypes.byref(ctypes.c_int32()), (ctypes.c_int32 * 16)(), None, 0)"
+                % (fn, path.encode(), version, name.encode()))
+    code = "import ctypes; L = ctypes.CDLL(%r); L.%s.restype = ctypes.c_int64; print('rc', %s)" % (HOST_LIB, fn, call)
+    return subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+
+
+@pytest.mark.parametrize("mmap", [True, False])
+def test_model_file_with_bad_offsets_is_refused(tmp_path, mmap):
+    """Offsets and lengths in a model file are untrusted: a truncated file, an offset + length that wraps around 2^64, a
+    descriptor count or descriptor length beyond the file, and a shape whose byte count overflows all end in the load
+    error, never in a read outside the file."""
+    rng = synth.rng_for(5, 77)
+    _, _, name, tensors = _linear_file_tensors(rng, 0, 48, 96)
+    wname = name + ".weight"
+    good1, good2 = str(tmp_path / "g1.mllm"), str(tmp_path / "g2.mllm")
+    _write_v1(good1, tensors)
+    _write_v2(good2, tensors)
+    for path, version in ((good1, 1), (good2, 2)):
+        r = _load_in_child(path, version, wname, mmap)
+        assert r.returncode == 0 and "rc" in r.stdout, r.stderr
+    raw1, raw2 = open(good1, "rb").read(), open(good2, "rb").read()
+    cases = []
+    # truncated in the tensor data
+    cases.append(("v1 truncated", 1, raw1[:len(raw1) - 40]))
+    cases.append(("v2 truncated", 2, raw2[:len(raw2) - 40]))
+    # V1: descriptor length beyond the file / enormous
+    cases.append(("v1 desc_bytes huge", 1, raw1[:4] + struct.pack("<Q", 2**63) + raw1[12:]))
+    cases.append(("v1 desc_bytes wraps", 1, raw1[:4] + struct.pack("<Q", 2**64 - 8) + raw1[12:]))
+    # V1: first tensor's offset such that offset + length wraps to a small number
+    (nl,) = struct.unpack_from("<I", raw1, 12)
+    off_pos = 12 + 4 + nl + 8
+    (ln,) = struct.unpack_from("<Q", raw1, 12 + 4 + nl)
+    cases.append(("v1 offset wraps", 1, raw1[:off_pos] + struct.pack("<Q", 2**64 - ln + 16) + raw1[off_pos + 8:]))
+    # V2: descriptor table offset wraps / count too large
+    cases.append(("v2 desc offset wraps", 2, raw2[:524] + struct.pack("<Q", 2**64 - 352) + raw2[532:]))
+    cases.append(("v2 count huge", 2, raw2[:520] + struct.pack("<I", 2**32 - 1) + raw2[524:]))
+    # V2: every tensor's data offset wraps; every tensor's shape overflows the byte count
+    bad = bytearray(raw2)
+    for i in range(3):
+        struct.pack_into("<Q", bad, 532 + 352 * i + 16, 2**64 - 64)
+    cases.append(("v2 offset wraps", 2, bytes(bad)))
+    bad = bytearray(raw2)
+    for i in range(3):
+        struct.pack_into("<Q", bad, 532 + 352 * i + 24, 16)
+        struct.pack_into("<16i", bad, 532 + 352 * i + 32, *([2**31 - 1] * 16))
+    cases.append(("v2 shape overflows", 2, bytes(bad)))
+    for what, version, data in cases:
+        path = str(tmp_path / "bad.mllm")
+        open(path, "wb").write(data)
+        r = _load_in_child(path, version, wname, mmap)
+        assert r.returncode > 0 and "rc" not in r.stdout, (what, r.returncode, r.stdout, r.stderr)  # the exit code of the load error, not a signal
+        assert "truncated" in r.stderr or "assertion failed" in r.stderr, (what, r.stderr)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("version", [1, 2])
 def test_linear_from_model_file(tmp_path, version):
