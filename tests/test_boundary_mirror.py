@@ -197,3 +197,99 @@ def test_plugin_descriptor_fields_match_the_reference():
     # both pack the struct to 4 bytes
     assert re.search(r"#pragma\s+pack\(push,\s*4\)\s*struct\s+PluginOpPackageDescriptor", rtxt)
     assert re.search(r"#pragma\s+pack\(push,\s*4\)\s*struct\s+PluginOpPackageDescriptor", MIR)
+
+
+# ---- model-file schema ---------------------------------------------------------------------------------------------
+# The V1 / V2 reader and writer (mllm_amd/csrc/host/mllm_core.cpp) restate the reference's packed structs; the tests of the
+# reader otherwise only see files that this repository's own tests write.  Here the reference's schema headers are read as
+# text: magic numbers, version, array lengths, the field lists (type, name, order) and the sizes their static_asserts state.
+CORE_CPP = os.path.join(ROOT, "mllm_amd", "csrc", "host", "mllm_core.cpp")
+_WIDTH = {"int32_t": 4, "uint32_t": 4, "uint64_t": 8, "size_t": 8, "char": 1}
+
+
+def _macros(txt):
+    return {m.group(1): int(m.group(2), 0) for m in re.finditer(r"#define\s+(\w+)\s+(0x[0-9A-Fa-f]+|\d+)\b", txt)}
+
+
+def _struct_body(txt, struct):
+    """like _body, for `struct [__attribute__((packed))] name { ... }`; also returns the text between `struct` and the name"""
+    m = re.search(r"\bstruct\s+((?:__attribute__\s*\(\(\s*packed\s*\)\)\s*)?)%s\s*\{" % re.escape(struct), txt)
+    assert m, "struct %s not found" % struct
+    depth, i = 1, m.end()
+    while depth and i < len(txt):
+        depth += {"{": 1, "}": -1}.get(txt[i], 0)
+        i += 1
+    return txt[m.end():i - 1], m.group(1)
+
+
+def _fields(txt, struct, macros=None):
+    """[(type, name, array length or None)] of a packed struct's data members, in order"""
+    out = []
+    for st in _statements(_struct_body(txt, struct)[0]):
+        m = re.fullmatch(r"(\w+)\s+(\w+(?:\[\w+\])?(?:\s*,\s*\w+(?:\[\w+\])?)*)", st)
+        if not m:
+            continue  # member functions
+        for decl in m.group(2).split(","):  # `int32_t magic_number, version;` declares two members
+            d = re.fullmatch(r"\s*(\w+)(?:\[(\w+)\])?\s*", decl)
+            n = d.group(2)
+            if n is not None:
+                n = int(n, 0) if re.fullmatch(r"0x[0-9A-Fa-f]+|\d+", n) else (macros or {})[n]
+            out.append((m.group(1), d.group(1), n))
+    return out
+
+
+def _sizeof(fields):
+    return sum(_WIDTH[t] * (n or 1) for t, _, n in fields)
+
+
+def _asserted_sizes(txt):
+    return {m.group(1): int(m.group(2)) for m in re.finditer(r"static_assert\(sizeof\((\w+)\)\s*==\s*(\d+)", txt)}
+
+
+def test_model_file_v2_schema_matches_the_reference_header():
+    ref = _strip_comments(open(os.path.join(REF, "mllm/core/schema/ModelFileV2.hpp")).read())
+    mine = _strip_comments(open(CORE_CPP).read())
+    mac = _macros(ref)
+    consts = {m.group(1): int(m.group(2), 0) for m in re.finditer(r"\b(k\w+)\s*=\s*(0x[0-9A-Fa-f]+|\d+)", mine)}
+    assert consts["kV2Magic"] == mac["MLLM_MODEL_FILE_V2_MAGIC_NUMBER"] == 0x519A
+    assert consts["kV2Version"] == mac["MLLM_MODEL_FILE_V2_VERSION"]
+    assert consts["kV2ModelName"] == mac["MLLM_MODEL_FILE_V2_MODEL_NAME_LENGTH"]
+    assert consts["kV2ParamName"] == mac["MLLM_MODEL_FILE_V2_PARAMS_NAME_LENGTH"]
+    assert consts["kV2ShapeLen"] == mac["MLLM_MODEL_FILE_V2_TENSOR_SHAPE_LENGTH"]
+    sizes_ref, sizes_mine = _asserted_sizes(ref), {}
+    m = re.search(r"static_assert\(sizeof\(V2Header\)\s*==\s*(\d+)\s*&&\s*sizeof\(V2Param\)\s*==\s*(\d+)", mine)
+    assert m, "the mirror states its struct sizes"
+    sizes_mine = {"V2Header": int(m.group(1)), "V2Param": int(m.group(2))}
+    for theirs, ours in (("ModelFileV2Descriptor", "V2Header"), ("ModelFileV2ParamsDescriptor", "V2Param")):
+        fr, fm = _fields(ref, theirs, mac), _fields(mine, ours, consts)
+        assert "packed" in _struct_body(ref, theirs)[1] and "packed" in _struct_body(mine, ours)[1]
+        # same names in the same order, same widths (size_t in the reference is 8 bytes on every 64-bit target it builds for)
+        assert [(n, _WIDTH[t], a) for t, n, a in fr] == [(n, _WIDTH[t], a) for t, n, a in fm], (theirs, fr, fm)
+        assert _sizeof(fr) == sizes_ref[theirs] == sizes_mine[ours] == _sizeof(fm)
+
+
+def test_model_file_v1_schema_matches_the_reference_header():
+    ref = _strip_comments(open(os.path.join(REF, "mllm/core/schema/ModelFileV1.hpp")).read())
+    mine = _strip_comments(open(CORE_CPP).read())
+    assert _macros(ref)["MLLM_MODEL_FILE_V1_MAGIC_NUMBER"] == int(re.search(r"kV1Magic\s*=\s*(\d+)", mine).group(1)) == 20012
+    assert "packed" in _struct_body(ref, "ModelFileV1Descriptor")[1] and "packed" in _struct_body(ref, "ModelFileV1ParamsDescriptor")[1]
+    head = _fields(ref, "ModelFileV1Descriptor")
+    assert [(n, _WIDTH[t]) for t, n, _ in head] == [("magic_number", 4), ("parameter_desc_offset", 8)]
+    assert _sizeof(head) == _asserted_sizes(ref)["ModelFileV1Descriptor"] == 12
+    # the reader takes the header as 4 + 8 bytes at offsets 0 and 4 and the descriptors from byte 12 on
+    assert re.search(r"bytes\(0,\s*4,\s*&magic\)", mine) and re.search(r"bytes\(4,\s*8,\s*&desc_bytes\)", mine)
+    assert re.search(r"bytes\(12,\s*desc_bytes", mine)
+    # per tensor: name_len, the name, then data_len, offset, dtype with the reference's widths, in the reference's order
+    per = _fields(ref, "ModelFileV1ParamsDescriptor")
+    assert [(n, _WIDTH[t]) for t, n, _ in per] == [("name_len", 4), ("data_len", 8), ("offset", 8), ("dtype", 4)]
+    v1 = mine[mine.index("version == ModelFileVersion::kV1"):]
+    v1 = v1[:v1.index("items.push_back")]
+    takes = re.findall(r"(\w+)\s*=\s*take<(\w+)>", v1)
+    assert [(_WIDTH[t]) for _, t in takes] == [4, 8, 8, 4], takes
+    assert [n.split(".")[-1] for n, _ in takes] == ["name_len", "len", "offset", "dtype"]
+    # ... and the writer emits the same sequence
+    sv = mine[mine.index("void save("):]
+    sv = sv[sv.index("version == ModelFileVersion::kV1"):sv.index("} else {")]
+    writes = re.findall(r"out\.write\((?:reinterpret_cast<const char\*>\(&(\w+)\)|(\w+)\.data\(\)),\s*(\w+)\)", sv)
+    assert [(a or b, n) for a, b, n in writes] == [("kV1Magic", "4"), ("desc_bytes", "8"), ("name_len", "4"), ("name", "name_len"),
+                                                    ("len", "8"), ("offset", "8"), ("dtype", "4")], writes
