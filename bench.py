@@ -631,6 +631,23 @@ def main():
                                                     "from_quantized_image": {"us": per2 * 1e6, "GBps": nbig / per2 / 1e9,
                                                                              "frac_of_hbm_peak": nbig / per2 / 1e9 / HBM_PEAK_GBS}}
         del bigw
+        # the Linear that ends every decode token of the model: lm_head, 151 936 x 2560 (mllm/models/qwen3/modeling_qwen3_fa2.hpp:264-265),
+        # Q4_0, one row; four distinct copies (875 MB), one launch each, the kernel and launch shape the layer GEMVs take
+        lmw = [ql.PackedQWeight.synthetic(ql.Q4_0, 151936, 2560, gen) for _ in range(4)]
+        xl = torch.randn((1, 2560), device="cuda", generator=gen).to(torch.bfloat16)
+        yl = torch.empty((1, 151936), dtype=torch.float32, device="cuda")
+        _, ev = timed(graphed(lambda: [ql.linear_q_gemv(w, xl, None, ql.SCALE_X86_REF, out=yl) for w in lmw]), 5, 2)
+        per = ev / (5 * 4)
+        nlm = synth.gemv_algorithmic_bytes(ql.Q4_0, 1, 151936, 2560, 2)
+        extra["lm_head_151936x2560"] = {"us": per * 1e6, "GBps": nlm / per / 1e9, "bytes": nlm,
+                                        "frac_of_hbm_peak": nlm / per / 1e9 / HBM_PEAK_GBS}
+        if wtype == ql.Q4_0 and args.m == 1:
+            tok_s = head["ms_per_step"] * 1e-3 + per
+            tok_b = head["bytes_per_step"] + nlm
+            extra["decode_token_36_layers_plus_lm_head"] = {"ms": tok_s * 1e3, "GBps": tok_b / tok_s / 1e9, "bytes": tok_b,
+                                                            "frac_of_hbm_peak": tok_b / tok_s / 1e9 / HBM_PEAK_GBS,
+                                                            "note": "the measured step plus one lm_head launch (sum of the two times)"}
+        del lmw
         extra["prefill_and_moe"] = side_workloads(torch, ql, synth, gen)
 
     cpu = None

@@ -382,6 +382,15 @@ int mllm_hip_moe_route(const int32_t* topk_ids, int64_t T, int E, int k, int32_t
  * weight_scale_mode as for mllm_hip_q_prepack (how the fp16 fields d / dmin are read).  packed: 256-byte aligned. */
 size_t mllm_hip_kq_packed_bytes(int wtype, int64_t N, int64_t K);
 int mllm_hip_kq_prepack(int wtype, const void* blocks, int weight_scale_mode, void* packed, int64_t N, int64_t K, void* stream);
+
+/* Offline K-quant quantizers on the GPU: w fp32 [N][K] (K % 256 == 0) -> reference super-blocks [N][K/256] of 144 (Q4_K) or 210
+ * (Q6_K) bytes, byte for byte what the reference's converter writes.  weight_scale_mode says how the fp16 fields d / dmin are
+ * stored and read back inside the quantizer (IEEE pattern, or the x86 build's form; see MLLM_HIP_SCALE_*).  `blocks`: 16-byte
+ * aligned for Q4_K, 2-byte aligned for Q6_K.
+ * replaces: quantize_row_q4_K / quantize_row_q6_K, mllm/backends/cpu/kernels/common/ggml/quantize/quantize_q4.cpp:97-168,184-282,325 ;
+ *           quantize_q6.cpp:34-106,153 with quantize.hpp:261-325 ; called from tools/mllm-quantizer/schema/gguf.cpp:211-250 */
+int mllm_hip_kq_quantize_weight_blocks(int wtype, const float* w, void* blocks, int weight_scale_mode, int64_t N, int64_t K,
+                                       void* stream);
 /* y[M][N] fp32 = x[M][K] (fp32 or bf16) * W^T + bias.  K % 256 == 0.  Up to eight rows per launch (decode); more rows run
  * as groups of eight, each streaming the weights again.  workspace (mllm_hip_kq_workspace_bytes, may be NULL): from three
  * rows on x is quantized once by a small kernel and the GEMV copies that image instead of quantizing in every workgroup

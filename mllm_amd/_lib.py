@@ -90,6 +90,7 @@ def lib():
         L.mllm_hip_kq_packed_bytes.restype = C.c_size_t
         L.mllm_hip_kq_packed_bytes.argtypes = [ci, i64, i64]
         L.mllm_hip_kq_prepack.argtypes = [ci, vp, ci, vp, i64, i64, vp]
+        L.mllm_hip_kq_quantize_weight_blocks.argtypes = [ci, vp, vp, ci, i64, i64, vp]
         L.mllm_hip_linear_kq.argtypes = [ci, vp, vp, ci, vp, vp, i64, i64, i64, vp, vp]
         L.mllm_hip_kq_set_tuning.argtypes = [ci, ci, ci]
         L.mllm_hip_linear_kq_multi.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, i64, i64, vp, vp]

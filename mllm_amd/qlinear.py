@@ -536,6 +536,16 @@ Q4_K, Q6_K = 2, 3
 KBLOCK_BYTES = {Q4_K: 144, Q6_K: 210}
 
 
+def kq_quantize_weight_blocks(w, wtype, weight_scale_mode=SCALE_IEEE):
+    """fp32 [N, K] on the GPU -> reference super-blocks uint8 [N, K/256, 144|210] (the offline K-quant quantizers' output)."""
+    assert w.is_cuda and w.is_contiguous() and w.dtype == torch.float32 and w.dim() == 2 and w.shape[1] % 256 == 0
+    N, K = w.shape
+    out = torch.empty((N, K // 256, KBLOCK_BYTES[wtype]), dtype=torch.uint8, device="cuda")
+    _lib.check(_lib.lib().mllm_hip_kq_quantize_weight_blocks(wtype, w.data_ptr(), out.data_ptr(), weight_scale_mode, N, K, _stream()),
+               "mllm_hip_kq_quantize_weight_blocks")
+    return out
+
+
 class PackedKWeight:
     """Q4_K / Q6_K weight [N, K] repacked on the device.  blocks: uint8 [N, K/256, 144|210] (reference layout)."""
 

@@ -507,6 +507,19 @@ def ref_linear_kq(x, W, wtype, bias=None):
     return y
 
 
+def quantize_weight_rows_k(w, wtype, scale_mode=SCALE_IEEE):
+    """fp32 [N, K] -> reference super-blocks uint8 [N, K/256, 144|210] (offline K-quant quantizer restatement); the fp16
+    fields are stored as scale_mode says (IEEE pattern, or the x86 build's encoding of the pattern as a number)"""
+    w = np.ascontiguousarray(w, np.float32)
+    N, K = w.shape
+    assert K % 256 == 0
+    out = np.empty((N, K // 256, KBLOCK_BYTES[wtype]), np.uint8)
+    fn = lib().orc_quantize_row_q4_K if wtype == Q4_K else lib().orc_quantize_row_q6_K
+    for n in range(N):
+        fn(_p(w[n], C.c_float), _p(out[n], C.c_uint8), C.c_int(K), C.c_int(scale_mode))
+    return out
+
+
 def ref_quantize_rows_k(w, wtype):
     """the reference's offline quantizer -> canonical blocks uint8 [N, K/256, 144|210]"""
     w = np.ascontiguousarray(w, np.float32)

@@ -961,3 +961,251 @@ ORC_API int orc_linear_kq(const float* x, const uint8_t* W, int wtype, const flo
   free(xq); free(xd); free(xbs);
   return 0;
 }
+
+/* ================================================================================================
+ * Offline K-quant weight quantizers: fp32 rows -> reference super-blocks
+ *   Q4_K  quantize_row_q4_K_reference with make_qkx2_quants(32, 15, ..., rmin -1, rdelta 0.1, nstep 20, squared error),
+ *         mllm/backends/cpu/kernels/common/ggml/quantize/quantize_q4.cpp:97-168 (the search), :184-282 (the super-block)
+ *   Q6_K  quantize_row_q6_K_reference with make_qx_quants(16, 32, ..., rmse_type 1), quantize_q6.cpp:34-106,
+ *         quantize.hpp:268-325 (the search); nearest_int quantize.hpp:261-267
+ * Every fp32 operation is written in the reference's order (no contraction in either build): sums run element by element,
+ * `w * l * l` is (w * l) * l, and so on.  The fp16 fields d / dmin: scale_mode IEEE stores the fp16 pattern P and the final
+ * code pass reads its value; X86_REF stores what the x86 build leaves in the file, the half-precision encoding of the NUMBER P,
+ * and the final code pass reads what that build reads back, P rounded to 11 significant bits (orc_x86_scale_bits) -- so
+ * the codes themselves can differ between the two modes.
+ * Pinned: bytes (codes, 6-bit / int8 scales) and decoded d / dmin patterns bit-exact against the compiled reference
+ * quantizers in X86_REF mode (tests/test_oracle_vs_reference.py); the IEEE mode differs only in the two lines named above.
+ * ============================================================================================== */
+static inline int orc_nearest_int(float fval) {
+  float val = fval + 12582912.f;
+  int i;
+  memcpy(&i, &val, sizeof(int));
+  return (i & 0x007fffff) - 0x00400000;
+}
+
+/* one sub-block of n weights -> codes L (0..nmax), returns the scale, *the_min = -offset (>= 0) */
+static float orc_qkx2_search(int n, int nmax, const float* x, const float* weights, uint8_t* L, float* the_min, uint8_t* Laux,
+                             float rmin, float rdelta, int nstep) {
+  float min = x[0], max = x[0];
+  float sum_w = weights[0];
+  float sum_x = sum_w * x[0];
+  for (int i = 1; i < n; i++) {
+    if (x[i] < min) min = x[i];
+    if (x[i] > max) max = x[i];
+    const float w = weights[i];
+    sum_w += w;
+    sum_x += w * x[i];
+  }
+  if (min > 0) min = 0;
+  if (max == min) {
+    for (int i = 0; i < n; i++) L[i] = 0;
+    *the_min = -min;
+    return 0.f;
+  }
+  float iscale = nmax / (max - min);
+  float scale = 1 / iscale;
+  float best = 0;
+  for (int i = 0; i < n; i++) {
+    int l = orc_nearest_int(iscale * (x[i] - min));
+    l = l < 0 ? 0 : (l > nmax ? nmax : l);
+    L[i] = (uint8_t)l;
+    float diff = scale * L[i] + min - x[i];
+    diff = diff * diff;
+    best += weights[i] * diff;
+  }
+  for (int is = 0; is <= nstep; is++) {
+    iscale = (rmin + rdelta * is + nmax) / (max - min);
+    float sum_l = 0, sum_l2 = 0, sum_xl = 0;
+    for (int i = 0; i < n; i++) {
+      int l = orc_nearest_int(iscale * (x[i] - min));
+      l = l < 0 ? 0 : (l > nmax ? nmax : l);
+      Laux[i] = (uint8_t)l;
+      const float w = weights[i];
+      sum_l += w * l;
+      sum_l2 += w * l * l;
+      sum_xl += w * l * x[i];
+    }
+    const float D = sum_w * sum_l2 - sum_l * sum_l;
+    if (D > 0) {
+      float this_scale = (sum_w * sum_xl - sum_x * sum_l) / D;
+      float this_min = (sum_l2 * sum_x - sum_l * sum_xl) / D;
+      if (this_min > 0) {
+        this_min = 0;
+        this_scale = sum_xl / sum_l2;
+      }
+      float err = 0;
+      for (int i = 0; i < n; i++) {
+        float diff = this_scale * Laux[i] + this_min - x[i];
+        diff = diff * diff;
+        err += weights[i] * diff;
+      }
+      if (err < best) {
+        for (int i = 0; i < n; i++) L[i] = Laux[i];
+        best = err;
+        scale = this_scale;
+        min = this_min;
+      }
+    }
+  }
+  *the_min = -min;
+  return scale;
+}
+
+ORC_API void orc_quantize_row_q4_K(const float* x, uint8_t* blocks, int k, int scale_mode) {
+  const int nb = k / QK_K;
+  for (int i = 0; i < nb; i++, x += QK_K) {
+    uint8_t* y = blocks + (size_t)i * 144;
+    uint8_t L[QK_K], Laux[32];
+    float weights[32], mins[8], scales[8];
+    float max_scale = 0, max_min = 0;
+    for (int j = 0; j < 8; j++) {
+      const float* xs = x + 32 * j;
+      float sum_x2 = 0;
+      for (int l = 0; l < 32; l++) sum_x2 += xs[l] * xs[l];
+      const float av_x = sqrtf(sum_x2 / 32);
+      for (int l = 0; l < 32; l++) weights[l] = av_x + fabsf(xs[l]);
+      scales[j] = orc_qkx2_search(32, 15, xs, weights, L + 32 * j, &mins[j], Laux, -1.f, 0.1f, 20);
+      if (scales[j] > max_scale) max_scale = scales[j];
+      if (mins[j] > max_min) max_min = mins[j];
+    }
+    const float inv_scale = max_scale > 0 ? 63.f / max_scale : 0.f;
+    const float inv_min = max_min > 0 ? 63.f / max_min : 0.f;
+    uint8_t* sc12 = y + 4;
+    memset(sc12, 0, 12);
+    uint8_t ls6[8], lm6[8];
+    for (int j = 0; j < 8; j++) {
+      uint8_t ls = (uint8_t)orc_nearest_int(inv_scale * scales[j]);
+      uint8_t lm = (uint8_t)orc_nearest_int(inv_min * mins[j]);
+      ls = ls < 63 ? ls : 63;
+      lm = lm < 63 ? lm : 63;
+      ls6[j] = ls;
+      lm6[j] = lm;
+      if (j < 4) {
+        sc12[j] = ls;
+        sc12[j + 4] = lm;
+      } else {
+        sc12[j + 4] = (uint8_t)((ls & 0xF) | ((lm & 0xF) << 4));
+        sc12[j - 4] |= (uint8_t)((ls >> 4) << 6);
+        sc12[j] |= (uint8_t)((lm >> 4) << 6);
+      }
+    }
+    const uint16_t pd = orc_fp32_to_fp16(max_scale / 63.f), pm = orc_fp32_to_fp16(max_min / 63.f);
+    const uint16_t fd = store_scale_field(pd, scale_mode), fm = store_scale_field(pm, scale_mode);
+    memcpy(y, &fd, 2);
+    memcpy(y + 2, &fm, 2);
+    const float dv = scale_value(pd, scale_mode), mv = scale_value(pm, scale_mode);
+    for (int j = 0; j < 8; j++) {
+      const float d = dv * ls6[j];  /* the 6-bit values read back (get_scale_min_k4) are the ones just packed */
+      if (d == 0.0f) continue;
+      const float dm = mv * lm6[j];
+      for (int ii = 0; ii < 32; ii++) {
+        int l = orc_nearest_int((x[32 * j + ii] + dm) / d);
+        L[32 * j + ii] = (uint8_t)(l < 0 ? 0 : (l > 15 ? 15 : l));
+      }
+    }
+    uint8_t* q = y + 16;
+    for (int j = 0; j < QK_K; j += 64, q += 32)
+      for (int l = 0; l < 32; l++) q[l] = (uint8_t)(L[j + l] | (L[j + l + 32] << 4));
+  }
+}
+
+/* one group of n weights -> codes L (0 .. 2 nmax - 1, offset nmax), returns the scale; weights x^2 (rmse_type 1) */
+static float orc_qx_search(int n, int nmax, const float* x, int8_t* L) {
+  float max = 0, amax = 0;
+  for (int i = 0; i < n; i++) {
+    const float ax = fabsf(x[i]);
+    if (ax > amax) {
+      amax = ax;
+      max = x[i];
+    }
+  }
+  if (amax < 1e-30f) {
+    for (int i = 0; i < n; i++) L[i] = 0;
+    return 0.f;
+  }
+  float iscale = -nmax / max;
+  float sumlx = 0, suml2 = 0;
+  for (int i = 0; i < n; i++) {
+    int l = orc_nearest_int(iscale * x[i]);
+    l = l < -nmax ? -nmax : (l > nmax - 1 ? nmax - 1 : l);
+    L[i] = (int8_t)(l + nmax);
+    const float w = x[i] * x[i];
+    sumlx += w * x[i] * l;
+    suml2 += w * l * l;
+  }
+  float scale = sumlx / suml2;
+  float best = scale * sumlx;
+  for (int is = -9; is <= 9; is++) {
+    if (is == 0) continue;
+    iscale = -(nmax + 0.1f * is) / max;
+    sumlx = suml2 = 0;
+    for (int i = 0; i < n; i++) {
+      int l = orc_nearest_int(iscale * x[i]);
+      l = l < -nmax ? -nmax : (l > nmax - 1 ? nmax - 1 : l);
+      const float w = x[i] * x[i];
+      sumlx += w * x[i] * l;
+      suml2 += w * l * l;
+    }
+    if (suml2 > 0 && sumlx * sumlx > best * suml2) {
+      for (int i = 0; i < n; i++) {
+        int l = orc_nearest_int(iscale * x[i]);
+        l = l < -nmax ? -nmax : (l > nmax - 1 ? nmax - 1 : l);
+        L[i] = (int8_t)(nmax + l);
+      }
+      scale = sumlx / suml2;
+      best = scale * sumlx;
+    }
+  }
+  return scale;
+}
+
+ORC_API void orc_quantize_row_q6_K(const float* x, uint8_t* blocks, int k, int scale_mode) {
+  const int nb = k / QK_K;
+  for (int i = 0; i < nb; i++, x += QK_K) {
+    uint8_t* y = blocks + (size_t)i * 210;
+    int8_t L[QK_K];
+    float scales[16];
+    float max_scale = 0, max_abs_scale = 0;
+    for (int ib = 0; ib < 16; ib++) {
+      const float scale = orc_qx_search(16, 32, x + 16 * ib, L + 16 * ib);
+      scales[ib] = scale;
+      const float a = fabsf(scale);
+      if (a > max_abs_scale) {
+        max_abs_scale = a;
+        max_scale = scale;
+      }
+    }
+    if (!max_abs_scale) {
+      memset(y, 0, 210);  /* the fp16 pattern of 0.0 is 0 in either storage mode */
+      continue;
+    }
+    const float iscale = -128.f / max_scale;
+    const uint16_t pd = orc_fp32_to_fp16(1 / iscale);
+    const uint16_t fd = store_scale_field(pd, scale_mode);
+    memcpy(y + 208, &fd, 2);
+    int8_t* sc = (int8_t*)(y + 192);
+    for (int ib = 0; ib < 16; ib++) {
+      const int v = orc_nearest_int(iscale * scales[ib]);
+      sc[ib] = (int8_t)(v < 127 ? v : 127);
+    }
+    const float dv = scale_value(pd, scale_mode);
+    for (int j = 0; j < 16; j++) {
+      const float d = dv * sc[j];
+      if (!d) continue;
+      for (int ii = 0; ii < 16; ii++) {
+        int l = orc_nearest_int(x[16 * j + ii] / d);
+        l = l < -32 ? -32 : (l > 31 ? 31 : l);
+        L[16 * j + ii] = (int8_t)(l + 32);
+      }
+    }
+    uint8_t* ql = y;
+    uint8_t* qh = y + 128;
+    for (int j = 0; j < QK_K; j += 128, ql += 64, qh += 32)
+      for (int l = 0; l < 32; l++) {
+        const uint8_t q1 = L[j + l] & 0xF, q2 = L[j + l + 32] & 0xF, q3 = L[j + l + 64] & 0xF, q4 = L[j + l + 96] & 0xF;
+        ql[l] = (uint8_t)(q1 | (q3 << 4));
+        ql[l + 32] = (uint8_t)(q2 | (q4 << 4));
+        qh[l] = (uint8_t)((L[j + l] >> 4) | ((L[j + l + 32] >> 4) << 2) | ((L[j + l + 64] >> 4) << 4) | ((L[j + l + 96] >> 4) << 6));
+      }
+  }
+}

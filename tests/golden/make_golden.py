@@ -11,6 +11,8 @@ compiled unchanged) on seeded inputs; the inputs are stored next to the outputs 
   kquant_kat.npz      Q4_K / Q6_K: blocks made by the reference's own offline quantizers from fp32 weights, their
                       dequantized values, quantize_row_q8_K of the activations, and the Linear outputs (vec_dot_q4_K_q8_K /
                       vec_dot_q6_K_q8_K); written alone with `--only kquant`
+  kquant_quantizer_kat.npz  fp32 weights and the super-blocks the reference's offline Q4_K / Q6_K quantizers make of them; written
+                      alone with `--only kquant_quantizer`
 """
 import os
 import sys
@@ -66,11 +68,32 @@ def kquant():
     np.savez_compressed(os.path.join(OUT, "kquant_kat.npz"), **out)
 
 
+def kquant_quantizer():
+    """inputs and outputs of the reference's offline Q4_K / Q6_K quantizers (quantize_row_q4_K / _q6_K compiled from the
+    reference's sources): canonical super-blocks whose fp16 fields hold the patterns an x86 read of the written block yields"""
+    rq = np.random.default_rng(synth.SEED_BASE + 80)
+    N, K = 16, 512
+    w = (rq.standard_normal((N, K)) * 0.04).astype(np.float32)
+    w[0, :256] = 0.0                                         # an all-zero super-block
+    w[1, :32] = 0.3                                          # constant sub-blocks, positive and negative
+    w[1, 32:64] = -0.3
+    w[2, :256] = np.abs(w[2, :256])                          # all positive: every offset is zero
+    w[3, :256] *= 50
+    w[4, :16] = 0.0                                          # an all-zero group of 16 inside a live super-block
+    w[5, :256] = np.float32(1e-3) * rq.integers(-8, 8, 256)  # few distinct values
+    w[6, 0], w[6, 5] = 0.9, -0.9                             # equal magnitudes, opposite signs
+    np.savez_compressed(os.path.join(OUT, "kquant_quantizer_kat.npz"), w=w, q4_k_blocks=orc.ref_quantize_rows_k(w, 2),
+                        q6_k_blocks=orc.ref_quantize_rows_k(w, 3))
+
+
 def main():
     if not orc.ref_available():
         raise SystemExit("oracle/_ref/libmllm_ref.so missing: run `make -C oracle ref` where the reference is mounted")
     if sys.argv[1:] == ["--only", "kquant"]:
         kquant()
+        return
+    if sys.argv[1:] == ["--only", "kquant_quantizer"]:
+        kquant_quantizer()
         return
 
     rng = np.random.default_rng(synth.SEED_BASE + 77)
@@ -116,6 +139,7 @@ def main():
     np.savez_compressed(os.path.join(OUT, "weight_quantizer_kat.npz"), w=w, q4_blocks=orc.ref_quantize_rows_q4_0(w),
                         q8_codes=q8_codes, q8_d_eff=q8_d)
     kquant()
+    kquant_quantizer()
     for f in sorted(os.listdir(OUT)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(OUT, f)))

@@ -309,3 +309,56 @@ def test_moe_ffn_k_quant_grouped_form_equals_the_pair_form(wtype, T, H, I, E, k)
     assert np.array_equal(y2, outs[2][perm])
     assert rel_l2(y4, orc.moe_ffn_kq(xb, ids, w, Wg, Wu, Wd, wtype)) < 1e-3
     assert L.mllm_hip_moe_kq_set_path(3) == -1
+
+
+def _x86_field_to_pattern(field):
+    """what a read on x86 makes of a stored fp16 field: the half-precision number, as an integer"""
+    return field.view(np.float16).astype(np.float32).astype(np.uint16)
+
+
+@pytest.mark.parametrize("wtype", [2, 3])
+def test_offline_k_quant_quantizers_byte_exact(wtype, golden_dir):
+    """mllm_hip_kq_quantize_weight_blocks against the oracle (pinned byte for byte to the compiled reference quantizers) in both
+    storage modes, against the fixture the compiled reference wrote, and through the library's own Linear."""
+    import os
+    rng = synth.rng_for(7, 300 + wtype)
+    N, K = 48, 1024
+    w = (rng.standard_normal((N, K)) * 0.04).astype(np.float32)
+    w[0, :256] = 0.0
+    w[1, :32], w[1, 32:64] = 0.3, -0.3
+    w[2, :256] = np.abs(w[2, :256])
+    w[3, :512] *= 80
+    w[4, :16] = 0.0
+    w[5, :256] = np.float32(1e-3) * rng.integers(-8, 8, 256)
+    w[6, 0], w[6, 5] = 0.9, -0.9
+    w[7, :] = 1e-20                                      # below the all-zero threshold of the Q6_K search, not of the Q4_K one
+    announce("offline k-quant quantizer", wtype)
+    for mode, omode in ((ql.SCALE_X86_REF, orc.SCALE_X86_REF), (ql.SCALE_IEEE, orc.SCALE_IEEE)):
+        got = ql.kq_quantize_weight_blocks(to_dev(w), wtype, mode).cpu().numpy()
+        want = orc.quantize_weight_rows_k(w, wtype, omode)
+        assert np.array_equal(got, want), (mode, np.argwhere(got != want)[:5])
+    # the fixture of the compiled reference: codes and sub-block scales byte for byte, the fp16 fields as an x86 read decodes them
+    g = np.load(os.path.join(golden_dir, "kquant_quantizer_kat.npz"))
+    ref = g["q4_k_blocks" if wtype == 2 else "q6_k_blocks"]
+    gb = ql.kq_quantize_weight_blocks(to_dev(g["w"]), wtype, ql.SCALE_X86_REF).cpu().numpy()
+    body = np.ones(gb.shape[2], bool)
+    for a, b in ([(0, 2), (2, 4)] if wtype == 2 else [(208, 210)]):
+        body[a:b] = False
+        assert np.array_equal(_x86_field_to_pattern(gb[:, :, a:b].copy().view(np.uint16)[:, :, 0]), ref[:, :, a:b].copy().view(np.uint16)[:, :, 0])
+    assert np.array_equal(gb[:, :, body], ref[:, :, body])
+    # quantize -> prepack -> Linear on the GPU equals the oracle's Linear on the oracle's blocks
+    blocks = ql.kq_quantize_weight_blocks(to_dev(w), wtype, ql.SCALE_IEEE)
+    pw = ql.PackedKWeight(wtype, blocks)
+    x = synth.make_x_fp32(rng, 3, K)
+    y = ql.linear_kq(pw, to_dev(x)).cpu().numpy()
+    assert rel_l2(y, orc.linear_kq(x, orc.quantize_weight_rows_k(w, wtype, orc.SCALE_IEEE), wtype, None, orc.SCALE_IEEE)) < 2e-6
+    # and the blocks reproduce the weights to the format's resolution
+    deq = pw.dequantize().cpu().numpy()
+    assert np.abs(deq - w).max() <= (0.08 if wtype == 2 else 0.05) * np.abs(w).max()
+    L = _lib.lib()
+    p = blocks.data_ptr()
+    assert L.mllm_hip_kq_quantize_weight_blocks(wtype, None, p, 0, 4, 256, None) == -1
+    assert L.mllm_hip_kq_quantize_weight_blocks(0, p, p, 0, 4, 256, None) == -1
+    assert L.mllm_hip_kq_quantize_weight_blocks(wtype, p, p, 2, 4, 256, None) == -1
+    assert L.mllm_hip_kq_quantize_weight_blocks(wtype, p, p, 0, 4, 128, None) == -2
+    assert L.mllm_hip_kq_quantize_weight_blocks(wtype, p + 4, p, 0, 4, 256, None) == -3

@@ -284,6 +284,20 @@ def test_golden_kquant(golden_dir, name, wtype):
     assert np.array_equal(bs, g["q8k_bsums"])
 
 
+@pytest.mark.parametrize("name,wtype", [("q4_k", 2), ("q6_k", 3)])
+def test_golden_kquant_quantizers(golden_dir, name, wtype):
+    """the offline Q4_K / Q6_K quantizers against super-blocks the compiled reference wrote (make_golden.py, kquant_quantizer)"""
+    g = np.load(os.path.join(golden_dir, "kquant_quantizer_kat.npz"))
+    ref = g[f"{name}_blocks"]
+    got = orc.quantize_weight_rows_k(g["w"], wtype, orc.SCALE_X86_REF)
+    body = np.ones(got.shape[2], bool)
+    for a, b in ([(0, 2), (2, 4)] if wtype == 2 else [(208, 210)]):
+        body[a:b] = False
+        pat = got[:, :, a:b].copy().view(np.uint16)[:, :, 0].view(np.float16).astype(np.float32).astype(np.uint16)  # an x86 read
+        assert np.array_equal(pat, ref[:, :, a:b].copy().view(np.uint16)[:, :, 0])
+    assert np.array_equal(got[:, :, body], ref[:, :, body])
+
+
 @pytest.mark.parametrize("wtype", [0, 1])
 def test_avx2_tile_form_equals_the_scalar_restatement_bit_for_bit(wtype):
     """orc_linear_q_tiles (the vector instructions, tile shapes and job split of tinyBLAS_Q0_AVX, llamafile_sgemm.cpp:579-790)

@@ -191,3 +191,48 @@ def test_kquant_dequantize_and_linear_bit_exact(wtype):
         wq = orc.dequantize_k(unit, wtype, orc.SCALE_IEEE).astype(np.int64).reshape(N, K // 256, 256)
         want = np.einsum("nbk,mbk->nmb", wq, xq.astype(np.int64).reshape(M, K // 256, 256))
         assert np.array_equal(isum, want)
+
+
+def _kq_weight_rows(rng, N, K):
+    w = (rng.standard_normal((N, K)) * 0.04).astype(np.float32)
+    w[0, :256] = 0.0                                        # an all-zero super-block
+    w[1, :32] = 0.3                                         # a constant positive sub-block (its minimum is clamped to 0)
+    w[1, 32:64] = -0.3                                      # a constant negative sub-block: max == min
+    w[2, :256] = np.abs(w[2, :256])                         # all positive: every offset is zero
+    w[3, :256] *= 50                                        # large values
+    w[4, :16] = 0.0                                         # an all-zero group of 16 (Q6_K) inside a live super-block
+    w[5, :256] = np.float32(1e-3) * rng.integers(-8, 8, 256)  # few distinct values, many ties in the search
+    w[6, 0], w[6, 5] = 0.9, -0.9                            # equal magnitudes, opposite signs: the first one decides
+    return w
+
+
+@pytest.mark.parametrize("wtype", [orc.Q4_K, orc.Q6_K])
+def test_k_quant_offline_quantizers_bit_exact(wtype):
+    """orc_quantize_row_q4_K / _q6_K against the compiled reference quantizers (quantize_q4.cpp:184-282 with the search of
+    :97-168; quantize_q6.cpp:34-106 with quantize.hpp:268-325): every byte of codes and sub-block scales equal, and the fp16
+    fields decode -- the way an x86 read decodes them -- to the patterns the reference holds."""
+    rng = np.random.default_rng(61 + wtype)
+    w = _kq_weight_rows(rng, 20, 768)
+    ref = orc.ref_quantize_rows_k(w, wtype)                 # canonical: effective patterns in the fp16 fields
+    got = orc.quantize_weight_rows_k(w, wtype, orc.SCALE_X86_REF)
+    fields = [(0, 2), (2, 4)] if wtype == orc.Q4_K else [(208, 210)]
+    body = np.ones(got.shape[2], bool)
+    for a, b in fields:
+        body[a:b] = False
+        assert np.array_equal(_x86_field_to_pattern(got[:, :, a:b].copy().view(np.uint16)[:, :, 0]),
+                              ref[:, :, a:b].copy().view(np.uint16)[:, :, 0])
+    assert np.array_equal(got[:, :, body], ref[:, :, body])
+    # IEEE storage: the field is the fp16 pattern itself; the codes may differ from the x86 form only in super-blocks whose d
+    # or dmin pattern the x86 read rounds (patterns of more than 11 significant bits)
+    ieee = orc.quantize_weight_rows_k(w, wtype, orc.SCALE_IEEE)
+    same = np.ones(got.shape[:2], bool)
+    for a, b in fields:
+        pat = ieee[:, :, a:b].copy().view(np.uint16)[:, :, 0]
+        rounded = np.array([[orc.lib().orc_x86_scale_bits(int(v)) for v in row] for row in pat], np.uint16)
+        same &= rounded == pat
+    assert same.any() and (~same).any()
+    assert np.array_equal(ieee[same][:, body], ref[same][:, body])
+    # and the dequantized values of the blocks reproduce the weights to the formats' resolution
+    deq = orc.dequantize_k(ref, wtype)
+    err = np.abs(deq - w).max(axis=1) / (np.abs(w).max(axis=1) + 1e-12)
+    assert (err < (0.08 if wtype == orc.Q4_K else 0.05)).all(), err
