@@ -335,11 +335,13 @@ MLLM_API int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void*
 }
 
 static int g_gemv_path = 0;
+static int g_gemv_many_rows = 1;  // 0: nine rows and more as groups of eight (comparison runs and tests)
 // 0: by the number of rows; 1: always the vector-ALU kernel; 2: as 0 without the K-slices-as-workgroups form of the
 // matrix-core kernel (comparison runs and tests)
 MLLM_API int mllm_hip_gemv_set_path(int path) {
-  if (path != 0 && path != 1 && path != 2) return MLLM_HIP_E_BADARG;
-  g_gemv_path = path;
+  if (path != 0 && path != 1 && path != 2 && path != 3) return MLLM_HIP_E_BADARG;
+  g_gemv_many_rows = path != 3;  // 3: as 0, nine rows and more as groups of eight rows (the form without the many-row kernel)
+  g_gemv_path = path == 3 ? 0 : path;
   return 0;
 }
 
@@ -389,6 +391,8 @@ MLLM_API int mllm_hip_q_prepack(int wtype, const void* blocks, int weight_scale_
 
 // the quantized image of one pass of eight rows: 40 bytes per block
 static size_t gemv_image_bytes(int64_t K) { return (size_t)8 * (K / QK) * 40; }
+// ... of all rows of a call with nine rows or more (the many-row kernel reads whole groups of 16 or 32 rows)
+static size_t gemv_mr_image_bytes(int M, int64_t K) { return (size_t)gemv_mr_image_rows(M) * (K / QK) * 40; }
 
 MLLM_API size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K) {
   if (M < 1 || K <= 0 || K % QK) return 0;
@@ -400,7 +404,11 @@ MLLM_API size_t mllm_hip_gemv_workspace_bytes(int M, int64_t K) {
 MLLM_API size_t mllm_hip_gemv_splitk_workspace_bytes(int M, int64_t K, int64_t N_total) {
   if (M < 1 || K <= 0 || K % QK || N_total <= 0) return 0;
   const size_t groups = (size_t)(M + 7) / 8;  // the groups of eight rows share a launch
-  return gemv_image_bytes(K) + groups * (size_t)gemv_mfk_slices((int)(K / QK)) * 8 * (size_t)(N_total + 16 * GEMV_MAX_PARTS) * 4;
+  const size_t eight = gemv_image_bytes(K) + groups * (size_t)gemv_mfk_slices((int)(K / QK)) * 8 * (size_t)(N_total + 16 * GEMV_MAX_PARTS) * 4;
+  if (M <= 8) return eight;
+  // nine rows and more: the image of all rows (whole groups of 16 or 32), then every group's partial sums
+  const size_t many = gemv_mr_image_bytes(M, K) + gemv_mr_part_bytes(M, (int)(K / QK), N_total + 16 * GEMV_MAX_PARTS);
+  return std::max(eight, many);
 }
 
 // x_kind: MLLM_HIP_F32 / MLLM_HIP_BF16 activations, or MLLM_HIP_Q8_IMAGE: their quantized image (act_scale_mode unused)
@@ -457,6 +465,40 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
   if (M <= 8 || x_dtype == MLLM_HIP_Q8_IMAGE || nparts < 1 || nparts > GEMV_MAX_PARTS || !parts || !x)
     return gemv_multi_pass(wtype, nparts, parts, residual, x, x_dtype, M, K, act_scale_mode, workspace, ws_bytes, stream);
   if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
+  // Nine rows and more with room in the workspace for the image of all rows and the partial sums: one small launch quantizes
+  // x once, one launch of the many-row kernel reads the weights once for up to 32 rows (qgemv_mr_kernel.h).
+  if (g_gemv_many_rows && g_gemv_path == 0 && workspace && K > 0 && K % QK == 0 && ws_bytes >= gemv_mr_image_bytes(M, K)) {
+    RC_RET(gemv_check_args(wtype, nparts, parts, x, x_dtype, M, K, act_scale_mode, workspace));
+    const size_t img = gemv_mr_image_bytes(M, K);
+    GemvArgs a{};
+    for (int p = 0; p < nparts; p++) {
+      a.part[p].w = packed_view(wtype, parts[p].packed, parts[p].N, K);
+      a.part[p].bias = parts[p].bias;
+      a.part[p].residual = residual ? residual[p] : nullptr;
+      a.part[p].y = parts[p].y;
+      a.part[p].N = (int)parts[p].N;
+    }
+    a.nparts = nparts;
+    a.x = workspace;
+    a.M = M;
+    a.nb = (int)(K / QK);
+    a.nbp = (int)scale_row_stride(K);
+    a.x86_scale = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
+    // (refusals are decided before anything is queued: the quantization launch goes out only when the kernel will follow)
+    const int rows_img = gemv_mr_image_rows(M);
+    const int64_t mnb = (int64_t)rows_img * a.nb;
+    if (mnb < ((int64_t)1 << 31)) {
+      int np = 0;
+      for (int p = 0; p < nparts; p++) np += ((int)parts[p].N + 15) / 16 * 16;
+      const size_t need = gemv_mr_part_bytes(M, a.nb, np);
+      if (ws_bytes - img >= need) {
+        hipLaunchKernelGGL(quant_image_kernel, dim3((unsigned)((mnb + 127) / 128)), dim3(128), 0, (hipStream_t)stream, x, x_dtype,
+                           reinterpret_cast<unsigned char*>(workspace), M, rows_img, a.nb, a.x86_scale);
+        const int rc = launch_gemv_mr(wtype, a, workspace, reinterpret_cast<char*>(workspace) + img, ws_bytes - img, g_tune_NW, g_tune_R, (hipStream_t)stream);
+        if (rc != MFK_NOT_TAKEN) return rc;
+      }
+    }
+  }
   const size_t xrow = (size_t)K * (x_dtype == MLLM_HIP_F32 ? 4 : 2);
   int m_first = 0;
   // Groups of eight rows in one launch of the K-slice kernel where it applies (room for every group's partial sums): the

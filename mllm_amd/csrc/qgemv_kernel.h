@@ -415,6 +415,11 @@ constexpr int MFK_NOT_TAKEN = 1;
 int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a, const void* workspace, void* part, size_t part_bytes, int waves,
                     int slices, hipStream_t st, int groups = 1);
 int gemv_mfk_slices(int nb);
+// nine rows and more: the many-row kernel (qgemv_mr.hip).  a.x = the quantized image of gemv_mr_image_rows(a.M) rows; MFK_NOT_TAKEN
+// where it does not fit (room for partial sums, counters)
+int gemv_mr_image_rows(int M);
+size_t gemv_mr_part_bytes(int M, int nb, int64_t n_total_padded);
+int launch_gemv_mr(int wtype, const GemvArgs& a, const void* workspace, void* part, size_t part_bytes, int waves, int slices, hipStream_t st);
 int gemv_mfk_prepare_device();                 // counter table and kernel attributes of the current device (mllm_hip_init)
 int gemv_mfk_release(const void* workspace);   // the workspace address gives its counter block back
 void gemv_mfk_stats(int device, int* owned, int* capacity, long long* recycles, long long* refused);

@@ -127,6 +127,9 @@ static int mfk_counter_block(const void* workspace, hipStream_t st, unsigned** o
   return 0;
 }
 
+// the same blocks for the many-row kernel (qgemv_mr.hip): a workspace runs one launch at a time
+int gemv_counter_block(const void* workspace, hipStream_t st, unsigned** out) { return mfk_counter_block(workspace, st, out); }
+
 int gemv_mfk_release(const void* workspace) {
   std::lock_guard<std::mutex> lock(g_mfk_mutex);
   for (MfkTable& t : g_mfk) {

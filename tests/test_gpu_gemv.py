@@ -265,6 +265,14 @@ def test_gemv_groups_of_eight_rows_share_a_launch(wtype, M):
     rng = synth.rng_for(1, 900 + M + wtype)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(900 + M + wtype)
+    assert _lib.lib().mllm_hip_gemv_set_path(3) == 0  # this form, not the many-row kernel that nine rows and more take by default
+    try:
+        _groups_of_eight_rows_share_a_launch(wtype, M, rng, gen)
+    finally:
+        assert _lib.lib().mllm_hip_gemv_set_path(0) == 0
+
+
+def _groups_of_eight_rows_share_a_launch(wtype, M, rng, gen):
     for shapes, oracle_too in (([(300, 1024)], True), ([(50, 161 * 32)], True), ([(2560, 9728)], False),
                                ([(4096, 2560), (1024, 2560), (1024, 2560)], False), ([(9728, 2560), (9728, 2560)], False),
                                ([(8200, 97 * 32), (8193, 97 * 32)], False)):
@@ -309,16 +317,107 @@ def test_gemv_groups_run_in_several_launches_when_one_is_refused():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(77)
     rng = synth.rng_for(1, 977)
-    # 8192 x 8192: rows of 256 blocks are always cut, 128 workgroup columns x 16 groups = 2048 counters > 1024
-    for (N, K, M, ws_rows) in ((8192, 8192, 128, 128), (300, 1024, 37, 16), (2560, 9728, 32, 16)):
-        w = ql.PackedQWeight.synthetic(0, N, K, gen)
-        xd = to_dev(synth.make_x_fp32(rng, M, K))
-        announce("gemv row groups in several launches", N, K, M, ws_rows)
-        (y,) = ql.linear_q_gemv_multi([w], xd, None, workspace=ql.gemv_workspace(ws_rows, K, N))
-        ws8 = ql.gemv_workspace(8, K, N)
-        for m0 in range(0, M, 8):
-            (part,) = ql.linear_q_gemv_multi([w], xd[m0:m0 + 8].contiguous(), None, workspace=ws8)
-            assert torch.equal(y[m0:m0 + 8], part), (N, K, M, m0)
+    assert _lib.lib().mllm_hip_gemv_set_path(3) == 0  # the form of groups of eight rows
+    try:
+        # 8192 x 8192: rows of 256 blocks are always cut, 128 workgroup columns x 16 groups = 2048 counters > 1024
+        for (N, K, M, ws_rows) in ((8192, 8192, 128, 128), (300, 1024, 37, 16), (2560, 9728, 32, 16)):
+            w = ql.PackedQWeight.synthetic(0, N, K, gen)
+            xd = to_dev(synth.make_x_fp32(rng, M, K))
+            announce("gemv row groups in several launches", N, K, M, ws_rows)
+            (y,) = ql.linear_q_gemv_multi([w], xd, None, workspace=ql.gemv_workspace(ws_rows, K, N))
+            ws8 = ql.gemv_workspace(8, K, N)
+            for m0 in range(0, M, 8):
+                (part,) = ql.linear_q_gemv_multi([w], xd[m0:m0 + 8].contiguous(), None, workspace=ws8)
+                assert torch.equal(y[m0:m0 + 8], part), (N, K, M, m0)
+    finally:
+        assert _lib.lib().mllm_hip_gemv_set_path(0) == 0
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M", [9, 12, 16, 17, 24, 32, 33, 40, 64, 70])
+def test_gemv_many_rows_read_the_weights_once(wtype, M):
+    """Nine rows and more with room in the workspace for the image of all rows: one launch quantizes x, one launch of the
+    many-row kernel (16 x 16 x 32 integer matrix instruction = one block, 16 or 32 activation rows per workgroup) produces every
+    row.  Against the oracle (the reference's arithmetic, 2e-6: the fp32 additions run in another order), against the form of
+    groups of eight rows, twice in a row (the arrival counters go back to zero), and row by row the same bits whatever else is
+    in the call: cut rows, whole rows, several matrices, ragged N, a last slice that is empty, bias and residual."""
+    rng = synth.rng_for(1, 1900 + M + wtype)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1900 + M + wtype)
+    L = _lib.lib()
+    for shapes, oracle_too in (([(300, 1024)], True), ([(50, 161 * 32)], True), ([(37, 96), (7, 96)], True), ([(65, 32)], True),
+                               ([(2560, 9728)], False), ([(4096, 2560), (1024, 2560), (1024, 2560)], False),
+                               ([(9728, 2560), (9728, 2560)], False), ([(8200, 97 * 32), (8193, 97 * 32)], False)):
+        K = shapes[0][1]
+        n_total = sum(n for n, _ in shapes)
+        if oracle_too:
+            Ws = [synth.make_weight(rng, wtype, n, K) for n, _ in shapes]
+            ws = [ql.PackedQWeight(wtype, torch.from_numpy(W)) for W in Ws]
+        else:
+            ws = [ql.PackedQWeight.synthetic(wtype, n, K, gen) for n, _ in shapes]
+        biases = [to_dev(rng.standard_normal(n).astype(np.float32)) for n, _ in shapes]
+        wsp = ql.gemv_workspace(M, K, n_total)
+        for bf16 in (True, False):
+            if bf16:
+                bits, xf = synth.make_x_bf16(rng, M, K)
+                xd = bf16_dev(bits)
+            else:
+                xf = synth.make_x_fp32(rng, M, K)
+                xd = to_dev(xf)
+            announce("gemv many rows", wtype, M, shapes, "bf16" if bf16 else "fp32")
+            # by default the kernel takes the launches whose rows stay whole (many row tiles, rows of up to 128 blocks) and leaves
+            # the others to the groups of eight rows; the second tuning value 2 makes it take every launch (rows cut into K
+            # slices that meet in memory), 1 keeps rows whole wherever they fit
+            outs = [torch.full((M, n), float("nan"), device="cuda") for n, _ in shapes]
+            ql.linear_q_gemv_multi(ws, xd, biases, outs=outs, workspace=wsp)
+            assert L.mllm_hip_gemv_set_tuning(0, 2, 0) == 0
+            try:
+                forced = [torch.full((M, n), float("nan"), device="cuda") for n, _ in shapes]
+                ql.linear_q_gemv_multi(ws, xd, biases, outs=forced, workspace=wsp)
+                again = ql.linear_q_gemv_multi(ws, xd, biases, workspace=wsp)  # (the arrival counters are back at zero)
+                if M > 9:  # a row's bits do not depend on the other rows of the call
+                    tail = ql.linear_q_gemv_multi(ws, xd[M - 9:].contiguous(), biases, workspace=wsp)
+                    for o, t in zip(forced, tail):
+                        assert torch.equal(o[M - 9:], t)
+                assert L.mllm_hip_gemv_set_tuning(0, 1, 0) == 0
+                whole = ql.linear_q_gemv_multi(ws, xd, biases, workspace=wsp)
+            finally:
+                assert L.mllm_hip_gemv_set_tuning(0, 0, 0) == 0
+            for o, f, o2, wh in zip(outs, forced, again, whole):
+                assert torch.equal(f, o2)
+                assert rel_l2(f.cpu().numpy(), o.cpu().numpy()) < 2e-6 and rel_l2(wh.cpu().numpy(), o.cpu().numpy()) < 2e-6
+            if oracle_too:
+                for W, b, f, wh in zip(Ws, biases, forced, whole):
+                    want = orc.linear_q(xf, W, wtype, b.cpu().numpy(), orc.SCALE_X86_REF)
+                    assert rel_l2(f.cpu().numpy(), want) < 2e-6 and rel_l2(wh.cpu().numpy(), want) < 2e-6
+            assert L.mllm_hip_gemv_set_path(3) == 0
+            try:
+                eights = ql.linear_q_gemv_multi(ws, xd, biases, workspace=wsp)
+            finally:
+                assert L.mllm_hip_gemv_set_path(0) == 0
+            for o, e in zip(outs, eights):
+                assert rel_l2(o.cpu().numpy(), e.cpu().numpy()) < 2e-6  # another kernel: another order of additions of the same terms
+            if oracle_too:
+                for W, b, o in zip(Ws, biases, outs):
+                    assert rel_l2(o.cpu().numpy(), orc.linear_q(xf, W, wtype, b.cpu().numpy(), orc.SCALE_X86_REF)) < 2e-6
+    # residuals (the fused entry point)
+    K, N = 1024, 300
+    w = ql.PackedQWeight.synthetic(wtype, N, K, gen)
+    xd = to_dev(synth.make_x_fp32(rng, M, K))
+    r = to_dev(rng.standard_normal((M, N)).astype(np.float32))
+    wsp = ql.gemv_workspace(M, K, N)
+    (y,) = ql.linear_q_gemv_multi([w], xd, None, workspace=wsp)
+    (yr,) = ql.linear_q_gemv_fused([w], xd, residuals=[r], workspace=wsp)
+    assert torch.equal(yr, y + r)
+    # a workspace without room for the image of all rows: the groups of eight rows, as before
+    (y8,) = ql.linear_q_gemv_multi([w], xd, None, workspace=ql.gemv_workspace(8, K))
+    assert L.mllm_hip_gemv_set_path(3) == 0
+    try:
+        (y3,) = ql.linear_q_gemv_multi([w], xd, None, workspace=ql.gemv_workspace(8, K))
+    finally:
+        assert L.mllm_hip_gemv_set_path(0) == 0
+    assert torch.equal(y8, y3)
+    assert L.mllm_hip_gemv_splitk_workspace_bytes(32, 2560, 19456) >= 32 * 80 * 40 + 2 * 32 * (19456 + 32) * 4
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
@@ -369,7 +468,7 @@ def test_gemv_matrix_core_and_vector_kernels_agree(wtype, M):
             assert L.mllm_hip_gemv_set_path(0) == 0
         assert rel_l2(y0.cpu().numpy(), y1.cpu().numpy()) < 2e-6
         assert rel_l2(y0.cpu().numpy(), orc.linear_q(xf, W, wtype, bias.cpu().numpy(), orc.SCALE_X86_REF)) < 2e-6
-    assert L.mllm_hip_gemv_set_path(3) == -1
+    assert L.mllm_hip_gemv_set_path(4) == -1
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
