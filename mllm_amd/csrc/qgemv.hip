@@ -491,10 +491,12 @@ static int gemv_multi_impl(int wtype, int nparts, const mllm_hip_gemv_part* part
       int np = 0;
       for (int p = 0; p < nparts; p++) np += ((int)parts[p].N + 15) / 16 * 16;
       const size_t need = gemv_mr_part_bytes(M, a.nb, np);
-      if (ws_bytes - img >= need) {
+      char* part = reinterpret_cast<char*>(workspace) + img;
+      if (ws_bytes - img >= need &&
+          launch_gemv_mr(wtype, a, workspace, part, ws_bytes - img, g_tune_NW, g_tune_R, (hipStream_t)stream, true) == 0) {
         hipLaunchKernelGGL(quant_image_kernel, dim3((unsigned)((mnb + 127) / 128)), dim3(128), 0, (hipStream_t)stream, x, x_dtype,
                            reinterpret_cast<unsigned char*>(workspace), M, rows_img, a.nb, a.x86_scale);
-        const int rc = launch_gemv_mr(wtype, a, workspace, reinterpret_cast<char*>(workspace) + img, ws_bytes - img, g_tune_NW, g_tune_R, (hipStream_t)stream);
+        const int rc = launch_gemv_mr(wtype, a, workspace, part, ws_bytes - img, g_tune_NW, g_tune_R, (hipStream_t)stream);
         if (rc != MFK_NOT_TAKEN) return rc;
       }
     }

@@ -419,7 +419,8 @@ int gemv_mfk_slices(int nb);
 // where it does not fit (room for partial sums, counters)
 int gemv_mr_image_rows(int M);
 size_t gemv_mr_part_bytes(int M, int nb, int64_t n_total_padded);
-int launch_gemv_mr(int wtype, const GemvArgs& a, const void* workspace, void* part, size_t part_bytes, int waves, int slices, hipStream_t st);
+int launch_gemv_mr(int wtype, const GemvArgs& a, const void* workspace, void* part, size_t part_bytes, int waves, int slices, hipStream_t st,
+                   bool dry = false);
 int gemv_mfk_prepare_device();                 // counter table and kernel attributes of the current device (mllm_hip_init)
 int gemv_mfk_release(const void* workspace);   // the workspace address gives its counter block back
 void gemv_mfk_stats(int device, int* owned, int* capacity, long long* recycles, long long* refused);

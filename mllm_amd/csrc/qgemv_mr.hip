@@ -39,8 +39,10 @@ static int launch_mr_t(const GemvArgs& a, const MrArgs& k, int nwaves, hipStream
 }
 
 // a_in.x = the quantized image of gemv_mr_image_rows(a_in.M) rows (rows past a_in.M zero); part / part_bytes: room for the partial
-// sums.  MFK_NOT_TAKEN where the launch does not fit (room, counters): the caller takes the eight-row kernels.
-int launch_gemv_mr(int wtype, const GemvArgs& a_in, const void* workspace, void* part, size_t part_bytes, int waves, int slices, hipStream_t st) {
+// sums.  MFK_NOT_TAKEN where the launch does not fit (room, counters) or the kernel is not the faster one: the caller takes the
+// eight-row kernels.  dry: decide only (0 = the launch would go out), so that the caller queues the quantization of x first.
+int launch_gemv_mr(int wtype, const GemvArgs& a_in, const void* workspace, void* part, size_t part_bytes, int waves, int slices, hipStream_t st,
+                   bool dry) {
   GemvArgs a = a_in;
   MrArgs k{};
   const int AG = a.M <= 16 ? 1 : 2, MT = 16 * AG;
@@ -105,9 +107,10 @@ int launch_gemv_mr(int wtype, const GemvArgs& a_in, const void* workspace, void*
   if ((size_t)grid * k.S * k.groups > 0x7fffffffu / 8) return MFK_NOT_TAKEN;
   if (k.S > 1) {
     if (!workspace || !part || (size_t)k.groups * k.S * MT * np * 4 > part_bytes || (size_t)grid * k.groups > 1024) return MFK_NOT_TAKEN;
-    RC_RET(gemv_counter_block(workspace, st, &k.counters));
+    if (!dry) RC_RET(gemv_counter_block(workspace, st, &k.counters));
     k.part = static_cast<float*>(part);
   }
+  if (dry) return (wtype == MLLM_HIP_Q4_0 || wtype == MLLM_HIP_Q8_0) ? 0 : MLLM_HIP_E_BADARG;
   if (wtype == MLLM_HIP_Q4_0) return AG == 1 ? launch_mr_t<MLLM_HIP_Q4_0, 1>(a, k, nwaves, st) : launch_mr_t<MLLM_HIP_Q4_0, 2>(a, k, nwaves, st);
   if (wtype == MLLM_HIP_Q8_0) return AG == 1 ? launch_mr_t<MLLM_HIP_Q8_0, 1>(a, k, nwaves, st) : launch_mr_t<MLLM_HIP_Q8_0, 2>(a, k, nwaves, st);
   return MLLM_HIP_E_BADARG;
