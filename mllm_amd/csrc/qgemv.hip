@@ -309,6 +309,7 @@ MLLM_API int mllm_hip_init(int device) {
   void* p = nullptr;
   int rc = static_scratch(device, &p);
   if (!rc) rc = gemv_mfk_prepare_device();
+  if (!rc) rc = gemv_mr_prepare_device();
   if (cur != device) HIP_RET(hipSetDevice(cur));
   return rc;
 }

@@ -418,6 +418,7 @@ int gemv_mfk_slices(int nb);
 // nine rows and more: the many-row kernel (qgemv_mr.hip).  a.x = the quantized image of gemv_mr_image_rows(a.M) rows; MFK_NOT_TAKEN
 // where it does not fit (room for partial sums, counters)
 int gemv_mr_image_rows(int M);
+int gemv_mr_prepare_device();  // kernel attributes of the current device (mllm_hip_init)
 size_t gemv_mr_part_bytes(int M, int nb, int64_t n_total_padded);
 int launch_gemv_mr(int wtype, const GemvArgs& a, const void* workspace, void* part, size_t part_bytes, int waves, int slices, hipStream_t st,
                    bool dry = false);

@@ -19,22 +19,29 @@ size_t gemv_mr_part_bytes(int M, int nb, int64_t n_total_padded) {
   return S > 1 ? (size_t)gemv_mr_image_rows(M) * S * (size_t)n_total_padded * 4 : 0;
 }
 
+// the limit of dynamic LDS is a per-device attribute of a kernel: set once per device for every instantiation (mllm_hip_init
+// calls this, so that a launch under stream capture makes no other runtime call)
+static bool g_mr_prepared[64];
+int gemv_mr_prepare_device() {
+  int dev = 0;
+  HIP_RET(hipGetDevice(&dev));
+  if (dev < 0 || dev >= 64) return MLLM_HIP_E_NODEVICE;
+  if (g_mr_prepared[dev]) return 0;
+  HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mr_kernel<MLLM_HIP_Q4_0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mr_kernel<MLLM_HIP_Q4_0, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mr_kernel<MLLM_HIP_Q8_0, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_mr_kernel<MLLM_HIP_Q8_0, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+  g_mr_prepared[dev] = true;
+  return 0;
+}
+
 template <int WT, int AG>
 static int launch_mr_t(const GemvArgs& a, const MrArgs& k, int nwaves, hipStream_t st) {
   const size_t lds = mr_lds_bytes<AG>(WT, k.nbs, nwaves);
   if (lds > 160 * 1024) return MFK_NOT_TAKEN;
-  auto kern = gemv_mr_kernel<WT, AG>;
-  if (lds > 64 * 1024) {
-    static bool done[64][2][2];  // per device: the limit of dynamic LDS is an attribute of the kernel on that device
-    int dev = 0;
-    HIP_RET(hipGetDevice(&dev));
-    if (dev >= 0 && dev < 64 && !done[dev][WT][AG - 1]) {
-      HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-      done[dev][WT][AG - 1] = true;
-    }
-  }
+  if (lds > 64 * 1024) RC_RET(gemv_mr_prepare_device());
   const unsigned grid = (unsigned)(((size_t)k.gx * k.S + 7) / 8 * 8 * k.groups);
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(nwaves * 64), lds, st, a, k);
+  hipLaunchKernelGGL((gemv_mr_kernel<WT, AG>), dim3(grid), dim3(nwaves * 64), lds, st, a, k);
   return (int)hipGetLastError();
 }
 
