@@ -229,7 +229,9 @@ int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const void* up_p
 /* mllm_hip_moe_ffn_q_gemm has two forms.  0 (default): the reference's block arithmetic itself on the matrix cores: the
  * exact integer sum of every 32-element block (fp16 MFMAs on the integer codes), the exact product dW * dX of its two
  * scales (a third MFMA), one fp32 fused multiply-add per block; only the order in which blocks are added differs from the
- * CPU path.  1: fp16 operands with the block scales folded in as in mllm_hip_linear_q_gemm (about 2e-4 relative L2). */
+ * CPU path; an expert's last tile of at most sixteen rows takes instructions of 16 rows (half the matrix time, same
+ * bits).  1: fp16 operands with the block scales folded in as in mllm_hip_linear_q_gemm (about 2e-4 relative L2).
+ * 2: as 0 with every tile in the 32-row form (comparison runs and tests). */
 int mllm_hip_moe_gemm_set_path(int path);
 
 /* ---------------------------------------------------------------------------------------------------------

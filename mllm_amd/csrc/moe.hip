@@ -35,7 +35,10 @@ struct RouteOut {
   int* ntiles;       // [1]
 };
 
-// GROUPED: an expert's tiles are neighbours in the list (full tiles, then its partial tile); otherwise all full tiles come first
+// GROUPED: an expert's tiles are neighbours in the list (full tiles, then its partial tile), the experts in the order of
+// their numbers; otherwise all full tiles come first.  (Measured and dropped for the grouped list: experts in order of
+// falling row counts, so that the short tiles end a launch: 4 % slower on 512 tokens x 8 of 128 experts -- the heavy
+// experts' tiles are bound by arithmetic and the light ones by memory, and a list that mixes them overlaps the two.)
 template <bool GROUPED = false>
 __device__ __forceinline__ void moe_route_body(const int32_t* __restrict__ ids, int n, int E, int tile_h, const RouteOut& o, int* s_cnt) {
   // s_cnt: [E] counts, [E] cursors, [E] scan scratch x 3
@@ -939,6 +942,7 @@ struct QXArgs {
   const int* ntiles;
   int N, K;
   int x86_scale;
+  int half_tiles;        // tiles of at most sixteen rows take the 16-row form (same bits; 0: comparison runs and tests)
 };
 
 // masks and exponent patterns of qx_codes, kept in registers (v_and_or_b32 takes no literal constants)
@@ -952,28 +956,33 @@ __device__ __forceinline__ QXConst qx_const(int wtype) {
 }
 // the eight weight codes of MFMA step d (16 K elements, this lane's half) as fp16 numbers offset + code:
 // Q4_0: 1024 + q for the elements with (k & 2) == 0, 64 + q for the others (q = 0..15); Q8_0: 1152 + q (q = -128..127)
+// ... from the dwords themselves: Q4_0 one dword (v1 unused), Q8_0 two
 template <int WT>
-__device__ __forceinline__ f16x8 qx_codes(const u32x4 (&rq)[WT == MLLM_HIP_Q4_0 ? 1 : 2], int d, const QXConst& c) {
+__device__ __forceinline__ f16x8 qx_codes_dw(uint32_t v0, uint32_t v1, const QXConst& c) {
   uint32_t o[4];
   if (WT == MLLM_HIP_Q4_0) {
     // pair i of the dword sits in nibbles i and 4 + i.  Nibbles at bits 0..3 of a half-word land in the mantissa of 1024.0
     // (unit 1), nibbles at bits 4..7 in the mantissa of 64.0 (unit 1/16): pairs 0 and 1 need no shift, pairs 2 and 3 one
     // shift by 8 for both.
-    const uint32_t v = rq[0][d], t = v >> 8;
-    o[0] = (v & c.m_lo) | c.e_1024;
-    o[1] = (v & c.m_hi) | c.e_64;
+    const uint32_t t = v0 >> 8;
+    o[0] = (v0 & c.m_lo) | c.e_1024;
+    o[1] = (v0 & c.m_hi) | c.e_64;
     o[2] = (t & c.m_lo) | c.e_1024;
     o[3] = (t & c.m_hi) | c.e_64;
   } else {
     // two dwords of four codes each in byte order e0 e2 e1 e3; + 128 makes them unsigned
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-      const uint32_t w = rq[d >> 1][2 * (d & 1) + h] ^ 0x80808080u;
-      o[2 * h] = (w & c.m_lo) | c.e_1024;
-      o[2 * h + 1] = ((w >> 8) & c.m_lo) | c.e_1024;
-    }
+    const uint32_t w0 = v0 ^ 0x80808080u, w1 = v1 ^ 0x80808080u;
+    o[0] = (w0 & c.m_lo) | c.e_1024;
+    o[1] = ((w0 >> 8) & c.m_lo) | c.e_1024;
+    o[2] = (w1 & c.m_lo) | c.e_1024;
+    o[3] = ((w1 >> 8) & c.m_lo) | c.e_1024;
   }
   return __builtin_bit_cast(f16x8, u32x4{o[0], o[1], o[2], o[3]});
+}
+template <int WT>
+__device__ __forceinline__ f16x8 qx_codes(const u32x4 (&rq)[WT == MLLM_HIP_Q4_0 ? 1 : 2], int d, const QXConst& c) {
+  if (WT == MLLM_HIP_Q4_0) return qx_codes_dw<WT>(rq[0][d], 0u, c);
+  return qx_codes_dw<WT>(rq[d >> 1][2 * (d & 1)], rq[d >> 1][2 * (d & 1) + 1], c);
 }
 // fp16 pair (-offset of the elements with (k & 2) == 0, -offset of the others) including the 8 of Q4_0's code offset
 __host__ __device__ constexpr uint32_t qx_offsets(int wtype) { return wtype == MLLM_HIP_Q4_0 ? 0xD480E408u : 0xE480E480u; }
@@ -1272,6 +1281,293 @@ __device__ __forceinline__ void qx_tile(const QXArgs& a, const int e, const int 
   }
 }
 
+
+// The same tile for at most SIXTEEN sorted positions: v_mfma_f32_16x16x32_f16 takes a whole block of 32 elements per
+// instruction for 16 channels x 16 rows, so a tile of up to 16 rows costs half the matrix time (and half the FMAs) of the
+// 32-row form above, which would pad it to 32.  Same packed weights: a lane of the 32-row layout holds, of channel lane % 32,
+// the block's elements 8 hi .. 8 hi + 7 (MFMA step 0) and 16 + 8 hi .. (step 1); the 16-row operand wants, in lane
+// (channel c, K group kg), eight elements of channel c [+ 16].  v_permlane16_swap on the PACKED dwords (step 0 as first
+// operand, step 1 as second) leaves in the first the channels 0..15 and in the second the channels 16..31, each with K
+// groups (hi 0, step 0), (hi 0, step 1), (hi 1, step 0), (hi 1, step 1); the activation operand is read from LDS in that
+// order of K, so the products that meet are the same and every sum is the same exact integer.  Same scale products,
+// same FMAs per block, same order of blocks: the same bits as the 32-row form row by row.
+template <int WT, int NW, int TN>
+__device__ __forceinline__ void qx_tile16(const QXArgs& a, const int e, const int row0, const int rows, const int n0,
+                                          unsigned char* smem) {
+  constexpr int BK = 64, LDK = 2 * BK + 16;
+  constexpr int BM = 16, WN = TN * 32;
+  constexpr int STAGE = BM * LDK + BM * 48;
+  constexpr int QW = WT == MLLM_HIP_Q4_0 ? 1 : 2;
+  constexpr int ST = 4;  // K steps of weights in flight per wave
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lrow = lane & 31;             // channel of this lane in the packed layout
+  const int c16 = lane & 15, kg = lane >> 4;  // 16-row operands: channel / row c16, K group kg
+  const int Kp = (int)qg_kp(a.K), kbs = Kp / 64, nbs = (int)(qg_np(a.N) / 32), KD = (a.K + 63) / 64;
+  const int64_t qbytes = qg_qbytes(WT, a.N, a.K), wbytes = qg_bytes(WT, a.N, a.K);
+
+  const __amdgpu_buffer_rsrc_t rA = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(a.xq), 0, (uint32_t)((int64_t)a.a_rows * a.K * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rD = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(a.xd), 0, (uint32_t)((int64_t)a.a_rows * KD * 12), 0x00020000);
+  __amdgpu_buffer_rsrc_t rW[NW];
+  rW[0] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a.W0 + (size_t)e * a.wstride), 0, (uint32_t)wbytes, 0x00020000);
+  if (NW == 2) rW[NW - 1] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a.W1 + (size_t)e * a.wstride), 0, (uint32_t)wbytes, 0x00020000);
+
+  // activation chunk of threads 0 .. 127: tile row tid / 8, 16-byte column tid % 8; record of a row: threads 0 .. 15.
+  // Rows past `rows` repeat the last one (never stored); columns past K read as zeros.
+  const bool ldA = tid < BM * 8;
+  const int colA = (tid % 8) * 8;
+  uint32_t offA = 0xffffffffu, offD = 0xffffffffu;
+  if (ldA) {
+    const int pos = row0 + min(tid / 8, rows - 1);
+    const int arow = a.a_index ? a.a_index[pos] / a.a_div : pos;
+    offA = (uint32_t)(((int64_t)arow * a.K + colA) * 2);
+  }
+  if (tid < BM) {
+    const int pos = row0 + min(tid, rows - 1);
+    const int arow = a.a_index ? a.a_index[pos] / a.a_div : pos;
+    offD = (uint32_t)((int64_t)arow * KD * 12);
+  }
+  uint32_t offQ[TN], offS[TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int nb = min((n0 + wave * WN) / 32 + j, nbs - 1);
+    offQ[j] = (uint32_t)((int64_t)nb * kbs * (1024 * QW) + lane * 16);
+    offS[j] = (uint32_t)(qbytes + ((int64_t)nb * kbs * 32 + lrow) * 4);
+  }
+  typedef uint32_t u32x3 __attribute__((ext_vector_type(3)));
+  u32x4 ga[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+  u32x3 gd[2] = {{0u, 0u, 0u}, {0u, 0u, 0u}};
+  auto loadA = [&](int set, int kt) {  // two K steps ahead of their use, as in the 32-row form
+    if (ldA) ga[set] = __builtin_amdgcn_raw_buffer_load_b128(rA, kt * BK + colA < a.K ? offA : 0xffffffffu, kt * BK * 2, 0);
+    if (tid < BM) gd[set] = __builtin_amdgcn_raw_buffer_load_b96(rD, kt < KD ? offD : 0xffffffffu, kt * 12, 0);
+  };
+  auto storeA = [&](int set, int buf) {
+    if (ldA) *reinterpret_cast<u32x4*>(smem + buf * STAGE + (tid / 8) * LDK + (tid % 8) * 16) = ga[set];
+    if (tid < BM) {
+      u32x4* rec = reinterpret_cast<u32x4*>(smem + buf * STAGE + BM * LDK + tid * 48);
+      rec[0] = u32x4{gd[set].x, 0u, 0u, 0u};
+      rec[1] = u32x4{gd[set].y, 0u, 0u, 0u};
+      rec[2] = u32x4{gd[set].z, 0u, 0u, 0u};
+    }
+  };
+
+  f32x4 acc[NW][TN][2];  // [matrix][column tile][channel half]
+#pragma unroll
+  for (int w = 0; w < NW; w++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int h = 0; h < 2; h++) acc[w][j][h] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  u32x4 rq[ST][NW][TN][QW];
+  uint32_t rs[ST][NW][TN];
+  auto loadW = [&](int slot, int kt) {
+    const bool ok = kt < kbs;
+#pragma unroll
+    for (int w = 0; w < NW; w++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+#pragma unroll
+        for (int p = 0; p < QW; p++)
+          rq[slot][w][j][p] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], ok ? offQ[j] : 0xffffffffu, (kt * QW + p) * 1024, 0);
+        rs[slot][w][j] = __builtin_amdgcn_raw_buffer_load_b32(rW[w], ok ? offS[j] : 0xffffffffu, kt * 128, 0);
+      }
+  };
+  // scale operands: the fp16 scale of the step's first block in K slot 0, of its second block in K slot 1, in the lanes of K
+  // group 0; everything else zero
+  const uint32_t msk0 = kg ? 0u : 0x0000ffffu, msk1 = kg ? 0u : 0xffff0000u;
+  const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  const QXConst kc = qx_const(WT);
+  const f16x8 off_op = __builtin_bit_cast(f16x8, u32x4{kg ? 0u : qx_offsets(WT), 0u, 0u, 0u});
+
+  // the operands of one (block, matrix, column tile) from the packed registers: codes of the channels 0..15 | 16..31
+  auto unpack = [&](const u32x4 (&q)[QW], int b, f16x8 (&fw)[2]) {
+    if (WT == MLLM_HIP_Q4_0) {
+      const auto r = __builtin_amdgcn_permlane16_swap(q[0][2 * b], q[0][2 * b + 1], false, false);
+      fw[0] = qx_codes_dw<WT>(r[0], 0u, kc);
+      fw[1] = qx_codes_dw<WT>(r[1], 0u, kc);
+    } else {
+      // block b: steps 2b (dwords 0, 1 of register b) and 2b + 1 (dwords 2, 3)
+      const auto r0 = __builtin_amdgcn_permlane16_swap(q[QW - 1 ? b : 0][0], q[QW - 1 ? b : 0][2], false, false);
+      const auto r1 = __builtin_amdgcn_permlane16_swap(q[QW - 1 ? b : 0][1], q[QW - 1 ? b : 0][3], false, false);
+      fw[0] = qx_codes_dw<WT>(r0[0], r1[0], kc);
+      fw[1] = qx_codes_dw<WT>(r0[1], r1[1], kc);
+    }
+  };
+  auto scales = [&](uint32_t s, int b, u32x4 (&sw)[2]) {
+    const uint32_t up = __builtin_amdgcn_permlane16_swap(s, s, false, false)[1];  // lanes 0..15 <- lanes 16..31
+    const uint32_t m = b ? msk1 : msk0;
+    sw[0].x = s & m;
+    sw[1].x = up & m;
+  };
+
+  constexpr int G = 2 * NW * TN;  // groups per K step: block-major, then matrix, then column tile
+  f16x8 fw[2][2];                 // [current | next group][channel half]
+  u32x4 sw[2][2] = {{{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}}, {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}}};
+  f32x4 T[2][2], S[2][2];         // block sums and scale products of the current / previous group
+  T[1][0] = T[1][1] = S[1][0] = S[1][1] = zero4;
+
+  const int nsteps = (kbs + ST - 1) / ST * ST;
+  loadA(0, 0);
+  loadA(1, 1);
+#pragma unroll
+  for (int s = 0; s < ST; s++) loadW(s, s);
+  storeA(0, 0);
+  unpack(rq[0][0][0], 0, fw[0]);
+  scales(rs[0][0][0], 0, sw[0]);
+  __syncthreads();
+
+  auto kstep = [&](auto slot_tag, int kt) {
+    constexpr int SLOT = decltype(slot_tag)::value;
+    constexpr int NSLOT = (SLOT + 1) % ST;
+    const int buf = kt & 1;
+    loadA(SLOT & 1, kt + 2);
+    f16x8 fb[2];
+#pragma unroll
+    for (int b = 0; b < 2; b++)
+      fb[b] = *reinterpret_cast<const f16x8*>(smem + buf * STAGE + c16 * LDK + (2 * b + (kg & 1)) * 32 + (kg >> 1) * 16);
+    f16x8 rec[3];
+#pragma unroll
+    for (int q = 0; q < 3; q++) rec[q] = *reinterpret_cast<const f16x8*>(smem + buf * STAGE + BM * LDK + c16 * 48 + q * 16);
+    f32x4 tc = zero4;
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+      const int c = g & 1, n = c ^ 1;  // the register sets alternate (G is even)
+      const int b = g / (NW * TN);
+      const bool last = g == G - 1;
+      const int gn = last ? 0 : g + 1;
+      const int bn = gn / (NW * TN), wn = (gn / TN) % NW, jn = gn % TN;
+      const int pg = g == 0 ? G - 1 : g - 1;
+      const int pw = (pg / TN) % NW, pj = pg % TN;
+      __builtin_amdgcn_sched_barrier(0);
+      if (g % (NW * TN) == 0) tc = __builtin_amdgcn_mfma_f32_16x16x32_f16(off_op, rec[1 + b], zero4, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (last) unpack(rq[NSLOT][wn][jn], bn, fw[n]);
+      else unpack(rq[SLOT][wn][jn], bn, fw[n]);
+      __builtin_amdgcn_sched_barrier(0);
+      T[c][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[c][0], fb[b], tc, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      S[c][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, sw[c][0]), rec[0], zero4, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (last) {
+        scales(rs[NSLOT][wn][jn], bn, sw[n]);
+      } else {
+        scales(rs[SLOT][wn][jn], bn, sw[n]);
+        if (bn == 1) {  // both blocks of (wn, jn) are unpacked: fetch K step kt + ST into its ring registers
+#pragma unroll
+          for (int p = 0; p < QW; p++)
+            rq[SLOT][wn][jn][p] = __builtin_amdgcn_raw_buffer_load_b128(rW[wn], kt + ST < kbs ? offQ[jn] : 0xffffffffu, ((kt + ST) * QW + p) * 1024, 0);
+          rs[SLOT][wn][jn] = __builtin_amdgcn_raw_buffer_load_b32(rW[wn], kt + ST < kbs ? offS[jn] : 0xffffffffu, (kt + ST) * 128, 0);
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      T[c][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fw[c][1], fb[b], tc, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      // the FMAs of the previous group (of the previous step's last group when g == 0)
+#pragma unroll
+      for (int r = 0; r < 4; r++) acc[pw][pj][0][r] = fmaf(S[n][0][r], T[n][0][r], acc[pw][pj][0][r]);
+      asm volatile("" : "+v"(acc[pw][pj][0]));
+      __builtin_amdgcn_sched_barrier(0);
+      S[c][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, sw[c][1]), rec[0], zero4, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < 4; r++) acc[pw][pj][1][r] = fmaf(S[n][1][r], T[n][1][r], acc[pw][pj][1][r]);
+      asm volatile("" : "+v"(acc[pw][pj][1]));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    storeA((SLOT & 1) ^ 1, buf ^ 1);
+    __syncthreads();
+  };
+  for (int kt = 0; kt < nsteps; kt += ST) {
+    kstep(std::integral_constant<int, 0>{}, kt);
+    kstep(std::integral_constant<int, 1>{}, kt + 1);
+    kstep(std::integral_constant<int, 2>{}, kt + 2);
+    kstep(std::integral_constant<int, 3>{}, kt + 3);
+  }
+  // the last group's FMAs (G even: its results are in set 1)
+#pragma unroll
+  for (int h = 0; h < 2; h++)
+#pragma unroll
+    for (int r = 0; r < 4; r++) acc[NW - 1][TN - 1][h][r] = fmaf(S[1][h][r], T[1][h][r], acc[NW - 1][TN - 1][h][r]);
+
+  // acc[w][j][h][e] = result[row0 + c16][n0 + wave*WN + 32j + 16h + 4kg + e]
+  if (NW == 1) {
+    if (c16 < rows) {
+      const int pos = row0 + c16;
+      float* orow = a.out + (int64_t)(a.o_index ? a.o_index[pos] : pos) * a.N;
+#pragma unroll
+      for (int j = 0; j < TN; j++)
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const int n = n0 + wave * WN + j * 32 + 16 * h + 4 * kg;
+          f32x4 v = acc[0][j][h];
+          if (n + 3 < a.N && a.N % 4 == 0) {
+            if (a.bias) v += *reinterpret_cast<const f32x4*>(a.bias + n);
+            *reinterpret_cast<f32x4*>(orow + n) = v;
+          } else {
+#pragma unroll
+            for (int e2 = 0; e2 < 4; e2++)
+              if (n + e2 < a.N) orow[n + e2] = a.bias ? v[e2] + a.bias[n + e2] : v[e2];
+          }
+        }
+    }
+  } else {
+    // h = silu(gate) * up, quantized to Q8_0 over each block of 32 channels (one column tile j: eight channels in each of the
+    // four lanes of a row), written in the next Linear's activation format
+    const int nblk = a.N / QK, KDo = (a.N + 63) / 64;
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+      float hv[8];
+      float amax = 0.f;
+#pragma unroll
+      for (int q = 0; q < 8; q++) {
+        hv[q] = silu_f(acc[0][j][q >> 2][q & 3]) * acc[NW - 1][j][q >> 2][q & 3];
+        amax = fmaxf(amax, fabsf(hv[q]));
+      }
+      amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+      amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+      const float d = amax / 127.f;
+      const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
+      uint16_t bits = f32_to_f16bits(d);
+      if (a.x86_scale) bits = x86_scale_bits(bits);
+      const int blk = (n0 + wave * WN) / 32 + j;
+      // element 16h + 4kg + e of the block: bit 1 of its index is bit 1 of e
+      int qv[8], sa = 0, sb = 0;
+#pragma unroll
+      for (int q = 0; q < 8; q++) {
+        qv[q] = min(127, max(-128, (int)rintf(hv[q] * idv)));
+        if (q & 2) sb += qv[q];
+        else sa += qv[q];
+      }
+      sa += __shfl_xor(sa, 16, 64);
+      sa += __shfl_xor(sa, 32, 64);
+      sb += __shfl_xor(sb, 16, 64);
+      sb += __shfl_xor(sb, 32, 64);
+      if (c16 < rows && blk < nblk) {
+        uint16_t* hrow = a.hq + (int64_t)(row0 + c16) * a.N;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+          const int n = n0 + wave * WN + j * 32 + 16 * h + 4 * kg;
+          uint32_t o[2];
+#pragma unroll
+          for (int e2 = 0; e2 < 2; e2++)
+            o[e2] = (uint32_t)f32_to_f16bits((float)qv[4 * h + 2 * e2]) | ((uint32_t)f32_to_f16bits((float)qv[4 * h + 2 * e2 + 1]) << 16);
+          *reinterpret_cast<uint2*>(hrow + n) = uint2{o[0], o[1]};
+        }
+        if (kg == 0) {
+          uint32_t* recp = a.hd + ((int64_t)(row0 + c16) * KDo + (blk >> 1)) * 3;
+          reinterpret_cast<uint16_t*>(recp)[blk & 1] = bits;
+          recp[1 + (blk & 1)] = (uint32_t)f32_to_f16bits((float)sa) | ((uint32_t)f32_to_f16bits((float)sb) << 16);
+          if (blk == nblk - 1 && (nblk & 1)) {  // the unused half of the last record
+            reinterpret_cast<uint16_t*>(recp)[1] = 0;
+            recp[2] = 0;
+          }
+        }
+      }
+    }
+  }
+}
+
 constexpr int QX_TILE_H = 32;
 constexpr int QX_DOWN_TN = 2;  // column tiles per wave in the one-matrix mode
 constexpr int QX_GROUP = 8;    // tiles per group of work items (see qx_kernel)
@@ -1297,10 +1593,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   const int e = a.tile_expert[t], row0 = a.tile_row0[t], rows = a.tile_rows[t];
   if constexpr (MODE == 1) {
     const int n0 = by * 128;
-    qx_tile<WT, 2, 1, 1>(a, e, row0, rows, n0, smem);
+    if (rows <= 16 && a.half_tiles) qx_tile16<WT, 2, 1>(a, e, row0, rows, n0, smem);
+    else qx_tile<WT, 2, 1, 1>(a, e, row0, rows, n0, smem);
   } else {
     const int n0 = by * (128 * QX_DOWN_TN);
-    qx_tile<WT, 1, 1, QX_DOWN_TN>(a, e, row0, rows, n0, smem);
+    if (rows <= 16 && a.half_tiles) qx_tile16<WT, 1, QX_DOWN_TN>(a, e, row0, rows, n0, smem);
+    else qx_tile<WT, 1, 1, QX_DOWN_TN>(a, e, row0, rows, n0, smem);
   }
 }
 
@@ -1787,11 +2085,13 @@ static QXCarve carve_qx(Carver& c, int64_t T, int64_t H, int64_t I, int E, int k
   r.ro = carve_route(c, E, T * k, QX_TILE_H);
   return r;
 }
-static int g_moe_gemm_path = 0;  // 0: exact block sums (qx_kernel); 1: fp16 operands with the block scales folded in (qg_kernel)
+// 0: exact block sums (qx_kernel); 1: fp16 operands with the block scales folded in (qg_kernel); 2: as 0 with every tile in
+// the 32-row form (the comparison for the 16-row form: same bits)
+static int g_moe_gemm_path = 0;
 }  // namespace mllmhip
 
 MLLM_API int mllm_hip_moe_gemm_set_path(int path) {
-  if (path != 0 && path != 1) return MLLM_HIP_E_BADARG;
+  if (path < 0 || path > 2) return MLLM_HIP_E_BADARG;
   g_moe_gemm_path = path;
   return 0;
 }
@@ -1812,6 +2112,7 @@ static int moe_ffn_qx(int wtype, const void* gate_packed, const void* up_packed,
   QXArgs a{};
   a.tile_expert = w.ro.tile_expert; a.tile_row0 = w.ro.tile_row0; a.tile_rows = w.ro.tile_rows; a.ntiles = w.ro.ntiles;
   a.x86_scale = x86;
+  a.half_tiles = g_moe_gemm_path != 2;
   a.W0 = reinterpret_cast<const char*>(gate_packed);
   a.W1 = reinterpret_cast<const char*>(up_packed);
   a.wstride = (size_t)qg_bytes(wtype, I, H);
@@ -1859,7 +2160,7 @@ MLLM_API int mllm_hip_moe_ffn_q_gemm(int wtype, const void* gate_packed, const v
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16 || reinterpret_cast<uintptr_t>(y) % 16) return MLLM_HIP_E_ALIGN;
   hipStream_t st = (hipStream_t)stream;
   const int x86 = act_scale_mode == MLLM_HIP_SCALE_X86_REF;
-  if (g_moe_gemm_path == 0)
+  if (g_moe_gemm_path != 1)
     return moe_ffn_qx(wtype, gate_packed, up_packed, down_packed, x, x_dtype, topk_ids, topk_w, y, T, H, I, E, k, x86, workspace, st);
   Carver c(workspace);
   uint16_t* xh = c.take<uint16_t>((size_t)T * H);

@@ -228,9 +228,13 @@ def test_moe_gemm_small(T, H, I, E, k, wtype):
             perm = rng.permutation(T)
             y2 = ql.moe_ffn_q_gemm(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
             assert np.array_equal(y2, y[perm])
+            if form == 0:  # tiles of at most sixteen rows in their own form or padded to 32 rows: the same bits
+                assert L.mllm_hip_moe_gemm_set_path(2) == 0
+                y32 = ql.moe_ffn_q_gemm(g, u, d, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+                assert np.array_equal(y32, y)
     finally:
         L.mllm_hip_moe_gemm_set_path(0)
-    assert L.mllm_hip_moe_gemm_set_path(2) == -1
+    assert L.mllm_hip_moe_gemm_set_path(3) == -1
 
 
 def test_moe_gemm_exact_form_is_the_block_arithmetic():
@@ -323,6 +327,9 @@ def test_moe_gemm_full_size():
     y2 = ql.moe_ffn_q_gemm(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
     assert np.array_equal(y, y2)
     try:
+        assert _lib.lib().mllm_hip_moe_gemm_set_path(2) == 0  # every tile padded to 32 rows: the same bits
+        y32 = ql.moe_ffn_q_gemm(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
+        assert np.array_equal(y, y32)
         assert _lib.lib().mllm_hip_moe_gemm_set_path(1) == 0
         y3 = ql.moe_ffn_q_gemm(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
     finally:
