@@ -221,17 +221,25 @@ def side_workloads(torch, ql, synth, gen):
         act = float(np.mean([len(np.unique(r[0])) for r in routes]))
         wb = act * 3 * I * (H // 256) * 144
         deck["tokens_%d" % Td] = {"us": td * 1e6, "active_experts_avg": act, "weight_GBps": wb / td / 1e9, "frac_of_hbm_peak": wb / td / 8e12}
-    # the 512-token layer with Q4_K experts: pairs sorted by expert, tiles of eight rows on the matrix cores (the grouped form),
-    # against one GEMV row per pair
+    # the 512-token layer with Q4_K experts: pairs sorted by expert, tiles of 32 rows on the matrix cores (the grouped form),
+    # against tiles of eight rows (the decode kernels) and one GEMV row per pair
     from mllm_amd import _lib as _l
     wsk = torch.empty(_l.lib().mllm_hip_moe_kq_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
     tk2 = ev_time(lambda: ql.moe_ffn_kq(gk, uk, dk, x, ids, tw, workspace=wsk, out=ym), 5)
+    gkq = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gkq):
+        for _ in range(10):
+            ql.moe_ffn_kq(gk, uk, dk, x, ids, tw, workspace=wsk, out=ym)
+    tk2g = ev_replay(gkq, 10) / 10
+    del gkq
+    _l.lib().mllm_hip_moe_kq_set_path(2)
+    tk8 = ev_time(lambda: ql.moe_ffn_kq(gk, uk, dk, x, ids, tw, workspace=wsk, out=ym), 5)
     _l.lib().mllm_hip_moe_kq_set_path(1)
     tk1 = ev_time(lambda: ql.moe_ffn_kq(gk, uk, dk, x, ids, tw, workspace=wsk, out=ym), 3)
     _l.lib().mllm_hip_moe_kq_set_path(0)
     wbk = int((np.bincount(ids_np.reshape(-1), minlength=E) > 0).sum()) * 3 * I * (H // 256) * 144
     deck["tokens_512_grouped"] = {"us": tk2 * 1e6, "weight_GBps": wbk / tk2 / 1e9, "frac_of_hbm_peak": wbk / tk2 / 8e12,
-                                  "pairs_as_gemv_rows_us": tk1 * 1e6}
+                                  "in_a_graph_us": tk2g * 1e6, "tiles_of_8_rows_us": tk8 * 1e6, "pairs_as_gemv_rows_us": tk1 * 1e6}
     del gk, uk, dk, wsk
     from mllm_amd import _lib
     L = _lib.lib()
@@ -240,6 +248,14 @@ def side_workloads(torch, ql, synth, gen):
     down2 = ql.PackedExperts.synthetic(ql.Q4_0, E, H, I, gen, layout="gemm")
     wsm2 = torch.empty(L.mllm_hip_moe_gemm_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
     tm2 = ev_time(lambda: ql.moe_ffn_q_gemm(gate2, up2, down2, x, ids, tw, workspace=wsm2, out=ym), 10)
+    # the same call captured ten times in a graph (how a serving loop would issue it): without the gaps that four eager
+    # launches per call leave between their kernels
+    gm = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gm):
+        for _ in range(10):
+            ql.moe_ffn_q_gemm(gate2, up2, down2, x, ids, tw, workspace=wsm2, out=ym)
+    tm2g = ev_replay(gm, 10) / 10
+    del gm
     L.mllm_hip_moe_gemm_set_path(1)
     tm3 = ev_time(lambda: ql.moe_ffn_q_gemm(gate2, up2, down2, x, ids, tw, workspace=wsm2, out=ym), 10)
     L.mllm_hip_moe_gemm_set_path(0)
@@ -248,6 +264,10 @@ def side_workloads(torch, ql, synth, gen):
     flops = T * k * (2.0 * H * I * 2 + 2.0 * I * H)
     out["moe_ffn_512tok_128e_top8_q4_0"] = {"us": tm2 * 1e6, "active_experts": active, "weight_GBps": wbytes / tm2 / 1e9,
                                             "frac_of_hbm_peak": wbytes / tm2 / 8e12, "TFLOPS": flops / tm2 / 1e12,
+                                            "in_a_graph": {"us": tm2g * 1e6, "weight_GBps": wbytes / tm2g / 1e9,
+                                                           "frac_of_hbm_peak": wbytes / tm2g / 8e12,
+                                                           "note": "ten calls captured in one HIP graph; 'us' above is the same call "
+                                                                   "launched eagerly (four launches, gaps between their kernels)"},
                                             "path": "mllm_hip_moe_ffn_q_gemm, default form: the reference's block arithmetic on the matrix "
                                                     "cores (exact integer block sums and exact scale products from fp16 MFMAs, one fp32 FMA "
                                                     "per block; 4 launches: route + quantize, gate + up + SiLU*up + re-quantize, down, weighted sum)",

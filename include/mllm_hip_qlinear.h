@@ -352,10 +352,13 @@ int mllm_hip_moe_ffn_q(int wtype, const void* gate_packed, const void* up_packed
  * H % 256 == 0, I % 256 == 0, T * k <= 65535, E <= 3072.  Up to one (token, expert) pair per expert (Q6_K: half) every pair runs as one
  * GEMV row (three or four launches; the decode form, an expert's weights are read once per pair that uses it).  Beyond that
  * the pairs are sorted by expert and run as tiles of eight rows on the matrix cores (the grouped form: x and h quantized
- * to Q8_K once, an expert's weights read once per eight pairs; seven launches), same arithmetic.
+ * to Q8_K once, an expert's weights read once per eight pairs; seven launches), same arithmetic; from four pairs per expert
+ * on (Q4_K) as tiles of 32 rows, the weights as the second operand of 32 x 32 matrix instructions (an expert's weights read
+ * and unpacked once per 32 pairs), the same integers.
  * replaces: the same loop over experts with Q4_K / Q6_K Linear ops, modeling_qwen3_moe_fa2.hpp:98-100,175-238 */
 size_t mllm_hip_moe_kq_workspace_bytes(int64_t T, int64_t H, int64_t I, int E, int k);
-/* 0: by the number of pairs per expert (default); 1: always pairs as GEMV rows; 2: always tiles of eight rows (comparison runs and tests) */
+/* 0: by the number of pairs per expert (default); 1: always pairs as GEMV rows; 2: always tiles of eight rows; 3: always tiles
+ * of 32 rows where the format has them (comparison runs and tests) */
 int mllm_hip_moe_kq_set_path(int path);
 int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x,
                         int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H, int64_t I,

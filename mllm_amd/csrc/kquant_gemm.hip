@@ -1,0 +1,284 @@
+// Q4_K / Q6_K experts with many rows each: tiles of 32 expert-sorted rows on the matrix cores, the reference's integer
+// arithmetic kept exact.
+//
+// The decode kernels (kquant.hip) stream an expert's weights once per eight rows.  With tens of rows per expert the same
+// weights would be streamed several times and every eight rows pay the whole unpacking, so here a workgroup takes 32 rows x
+// 128 (two matrices) or 256 (one matrix) channels and walks K one super-block of 256 elements at a time:
+//   * activations: the Q8_K image (codes, sums of 16, scale per super-block; bit-exact, written once per call by
+//     quantize_q8k_kernel) goes through LDS, 32 rows x one super-block per stage, double-buffered;
+//   * weights: from the packed planes of mllm_hip_kq_prepack into registers, one super-block ahead, as whole 128-byte
+//     lines (a load instruction = 8 channels x the 128 bytes of their super-block; one channel per lane and 16 bytes of it,
+//     the operand's own layout, touches 32 lines per instruction and was bound by the L1's tag rate: gate + up at 512 tokens
+//     110 us), then through a 4.5 KB LDS patch that belongs to the wave into the operand layout.  The weights are the SECOND
+//     operand of the matrix instruction, so a lane owns ONE channel (lane % 32) and sixteen rows: the channel's sub-block
+//     scales are then per-lane values and scaling a sub-block's sums costs one integer multiply-add per output;
+//   * Q4_K: per sub-block of 32 elements one v_mfma_i32_32x32x32_i8 (codes 0..15 as they are: the format's minimum is a
+//     separate term), I += sc * T in int32; the minimum term sum_j m_j * bsum_j is one v_mfma_f32_32x32x16_f16 per super-block
+//     on the sixteen sums of 16 as fp16 integers (at most 2048: exact) and the 6-bit minima (every product and sum below
+//     2^24: exact); per super-block and output then y += (dX * d) * float(I) and y += -(dX * dmin) * float(M), the products
+//     and the FMAs of vec_dot_q4_K_q8_K (mllm/backends/cpu/kernels/common/ggml/vec_dot.cpp:498-560).
+// What differs from the CPU path is the order of the fp32 additions only (the CPU keeps eight lanes per output and a
+// separate accumulator for the minimum term; here one accumulator per output takes both terms super-block by super-block).
+#include <type_traits>
+
+#include "kquant_layout.h"
+
+namespace mllmhip {
+
+typedef int kx4i __attribute__((ext_vector_type(4)));
+typedef int kx16i __attribute__((ext_vector_type(16)));
+typedef float kx16f __attribute__((ext_vector_type(16)));
+typedef _Float16 kxh8 __attribute__((ext_vector_type(8)));
+
+struct KXArgs {
+  const char* W[2];      // packed experts (mllm_hip_kq_prepack layout), expert e at W[w] + e * estride
+  size_t estride;
+  const char* image;     // Q8_K image of the activations: codes [img_rows][K], sums of 16 int16 [img_rows][K/16], d [img_rows][K/256]
+  int img_rows;
+  const int* row_ids;    // image row of sorted position pos: row_ids[pos] / row_div (null: pos)
+  int row_div;
+  const int* out_ids;    // output row of sorted position pos (null: pos)
+  float* y[2];           // fp32 [..][N] per matrix
+  const int* tile_expert;
+  const int* tile_row0;
+  const int* tile_rows;
+  const int* ntiles;
+  int N, K;
+};
+
+constexpr int KX_LDC = 256 + 16;                           // code row of a super-block, padded: 16-byte reads of 16 rows hit 16 bank groups
+constexpr int KX_BS = 48;                                   // the row's sixteen sums of 16 as fp16, padded likewise
+constexpr int KX_OFF_BS = 32 * KX_LDC;
+constexpr int KX_OFF_DX = KX_OFF_BS + 32 * KX_BS;
+constexpr int KX_STAGE = KX_OFF_DX + 32 * 4;
+constexpr int KX_WROW = 128 + 16;                           // a channel's line in the wave's patch, padded likewise
+constexpr int KX_PATCH = 32 * KX_WROW;
+
+// NW matrices (gate and up share the activations) x TN column tiles of 32 channels per wave
+template <int NW, int TN>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void kx4_kernel(KXArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int t = blockIdx.x;
+  if (t >= a.ntiles[0]) return;
+  const int e = a.tile_expert[t], row0 = a.tile_row0[t], rows = a.tile_rows[t];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c32 = lane & 31, hi = lane >> 5;
+  const int nsb = a.K / QK_K;
+  const int n0 = blockIdx.y * (128 * TN) + wave * (32 * TN);
+
+  // ---- the image: this thread's pieces of a stage ---------------------------------------------------------------------------
+  const size_t img_codes = (size_t)a.img_rows * a.K, img_bs = (size_t)a.img_rows * (a.K / 16) * 2;
+  const __amdgpu_buffer_rsrc_t rI = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a.image), 0,
+                                                                    (uint32_t)(img_codes + img_bs + (size_t)a.img_rows * nsb * 4), 0x00020000);
+  auto image_row = [&](int m) {  // rows past the tile repeat its last row; their results are dropped
+    const int pos = row0 + min(m, rows - 1);
+    return a.row_ids ? a.row_ids[pos] / a.row_div : pos;
+  };
+  // codes: chunk c = tid + 256 i of 16 bytes: row c / 16, column c % 16
+  uint32_t offC[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) offC[i] = (uint32_t)((size_t)image_row((tid >> 4) + 16 * i) * a.K + (tid & 15) * 16);
+  // sums of 16: threads 0..63, row tid / 2, eight sums each; scale: threads 64..95, one row each
+  uint32_t offB = 0xffffffffu;
+  if (tid < 64) offB = (uint32_t)(img_codes + ((size_t)image_row(tid >> 1) * (a.K / 16) + (tid & 1) * 8) * 2);
+  else if (tid < 96) offB = (uint32_t)(img_codes + img_bs + (size_t)image_row(tid - 64) * nsb * 4);
+  u32x4 gc[2], gb;
+  auto load_stage = [&](int sb) {
+    const bool ok = sb < nsb;
+#pragma unroll
+    for (int i = 0; i < 2; i++) gc[i] = __builtin_amdgcn_raw_buffer_load_b128(rI, ok ? offC[i] : 0xffffffffu, sb * 256, 0);
+    if (tid < 64) gb = __builtin_amdgcn_raw_buffer_load_b128(rI, ok ? offB : 0xffffffffu, sb * 32, 0);
+    else if (tid < 96) gb.x = __builtin_amdgcn_raw_buffer_load_b32(rI, ok ? offB : 0xffffffffu, sb * 4, 0);
+  };
+  auto store_stage = [&](int buf) {
+    unsigned char* st = smem + buf * KX_STAGE;
+#pragma unroll
+    for (int i = 0; i < 2; i++) *reinterpret_cast<u32x4*>(st + ((tid >> 4) + 16 * i) * KX_LDC + (tid & 15) * 16) = gc[i];
+    if (tid < 64) {
+      // int16 sums (at most 16 * 128 in magnitude) as fp16 integers: exact
+      const uint32_t w[4] = {gb.x, gb.y, gb.z, gb.w};
+      uint32_t o[4];
+#pragma unroll
+      for (int q = 0; q < 4; q++) {
+        const _Float16 lo = (_Float16)(short)(w[q] & 0xffffu), hi16 = (_Float16)(short)(w[q] >> 16);
+        o[q] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi16) << 16);
+      }
+      *reinterpret_cast<u32x4*>(st + KX_OFF_BS + (tid >> 1) * KX_BS + (tid & 1) * 16) = u32x4{o[0], o[1], o[2], o[3]};
+    } else if (tid < 96) {
+      *reinterpret_cast<uint32_t*>(st + KX_OFF_DX + (tid - 64) * 4) = gb.x;
+    }
+  };
+
+  // ---- the weights: lane (channel c32 of a column tile, K half hi) -----------------------------------------------------------
+  const size_t sbt = (size_t)a.N * nsb;
+  const uint32_t oS = (uint32_t)kq_plane(sbt * 128), oD = oS + (uint32_t)kq_plane(sbt * 16);
+  __amdgpu_buffer_rsrc_t rW[NW];
+#pragma unroll
+  for (int w = 0; w < NW; w++)
+    rW[w] = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(a.W[w] + (size_t)e * a.estride), 0, (uint32_t)a.estride, 0x00020000);
+  uint32_t offS[TN], offD[TN];
+#pragma unroll
+  for (int j = 0; j < TN; j++) {
+    const int n = n0 + 32 * j + c32;
+    const bool ok = n < a.N;
+    offS[j] = ok ? oS + (uint32_t)((size_t)n * nsb * 16) : 0xffffffffu;
+    offD[j] = ok ? oD + (uint32_t)((size_t)n * nsb * 4) : 0xffffffffu;
+  }
+  // one register set: a chunk's registers are requested again for the next super-block as soon as the chunk is unpacked
+  u32x4 wq[NW][TN][4], ws[NW][TN];
+  uint32_t wd[NW][TN];
+  // request i of a column tile: channels 8 i .. 8 i + 7, lane l takes 16-byte chunk l % 8 of channel 8 i + l / 8
+  const int lr = lane >> 3, lc = lane & 7;
+  auto load_chunk = [&](int w, int j, int i, int sb) {
+    const int n = n0 + 32 * j + 8 * i + lr;
+    const uint32_t off = (n < a.N && sb < nsb) ? (uint32_t)(((size_t)n * nsb * 8 + lc) * 16) : 0xffffffffu;
+    wq[w][j][i] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], off, sb * 128, 0);
+  };
+  auto load_scales = [&](int w, int j, int sb) {
+    ws[w][j] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], sb < nsb ? offS[j] : 0xffffffffu, sb * 16, 0);
+    wd[w][j] = __builtin_amdgcn_raw_buffer_load_b32(rW[w], sb < nsb ? offD[j] : 0xffffffffu, sb * 4, 0);
+  };
+
+  float acc[NW][TN][16];
+#pragma unroll
+  for (int w = 0; w < NW; w++)
+#pragma unroll
+    for (int j = 0; j < TN; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[w][j][r] = 0.f;
+  const kx16i zi = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  const kx16f zf = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  // one super-block from LDS buffer `buf`
+  auto compute = [&](int sb, int buf) {
+    const unsigned char* st = smem + buf * KX_STAGE;
+    unsigned char* patch = smem + 2 * KX_STAGE + wave * KX_PATCH;
+    // output r of this lane = tile row 8 (r / 4) + 4 hi + r % 4
+    f32x4 dxv[4];
+#pragma unroll
+    for (int g = 0; g < 4; g++) dxv[g] = *reinterpret_cast<const f32x4*>(st + KX_OFF_DX + (8 * g + 4 * hi) * 4);
+    const kxh8 Am = *reinterpret_cast<const kxh8*>(st + KX_OFF_BS + c32 * KX_BS + hi * 16);
+#pragma unroll
+    for (int w = 0; w < NW; w++)
+#pragma unroll
+      for (int j = 0; j < TN; j++) {
+        int I[16];
+#pragma unroll
+        for (int r = 0; r < 16; r++) I[r] = 0;
+        const uint32_t srec[4] = {ws[w][j].x, ws[w][j].y, ws[w][j].z, ws[w][j].w};
+        const uint32_t dd = wd[w][j];
+        // into the operand layout through the wave's patch (LDS operations of one wave execute in order: no barrier); the
+        // registers are then free for the next super-block, whose lines are requested in consecutive instructions
+#pragma unroll
+        for (int i = 0; i < 4; i++) *reinterpret_cast<u32x4*>(patch + (8 * i + lr) * KX_WROW + lc * 16) = wq[w][j][i];
+#pragma unroll
+        for (int i = 0; i < 4; i++) load_chunk(w, j, i, sb + 1);
+#pragma unroll
+        for (int p = 0; p < 4; p++) {
+          const kx4i A0 = *reinterpret_cast<const kx4i*>(st + c32 * KX_LDC + (2 * p) * 32 + hi * 16);
+          const kx4i A1 = *reinterpret_cast<const kx4i*>(st + c32 * KX_LDC + (2 * p + 1) * 32 + hi * 16);
+          // chunk 2 p + hi of the channel: low nibbles = elements 16 hi .. 16 hi + 15 of sub-block 2 p, high nibbles of 2 p + 1
+          const u32x4 q = *reinterpret_cast<const u32x4*>(patch + c32 * KX_WROW + (2 * p + hi) * 16);
+          const kx4i lo = {(int)(q.x & 0x0f0f0f0fu), (int)(q.y & 0x0f0f0f0fu), (int)(q.z & 0x0f0f0f0fu), (int)(q.w & 0x0f0f0f0fu)};
+          const kx4i up = {(int)((q.x >> 4) & 0x0f0f0f0fu), (int)((q.y >> 4) & 0x0f0f0f0fu), (int)((q.z >> 4) & 0x0f0f0f0fu),
+                           (int)((q.w >> 4) & 0x0f0f0f0fu)};
+          const kx16i T0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(A0, lo, zi, 0, 0, 0);
+          const kx16i T1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(A1, up, zi, 0, 0, 0);
+          const int sc0 = (int)(srec[p] & 0xffu), sc1 = (int)((srec[p] >> 8) & 0xffu);
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            // one multiply-add per sub-block and output (|T| < 2^16, sc < 2^6), and one pair of sub-blocks at a time: written
+            // as C the sums reassociate, the compiler forms all eight sub-block results (128 registers) before it scales the
+            // first and adds with separate multiplies
+            I[r] = __mul24(T0[r], sc0) + I[r];
+            asm volatile("" : "+v"(I[r]));
+            I[r] = __mul24(T1[r], sc1) + I[r];
+            asm volatile("" : "+v"(I[r]));
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        load_scales(w, j, sb + 1);
+        // the minimum term: K slot 8 hi + i of the instruction = sum of 16 number 8 hi + i, which belongs to sub-block 4 hi + i / 2
+        const uint32_t sA = hi ? srec[2] : srec[0], sB = hi ? srec[3] : srec[1];
+        const _Float16 m0 = (_Float16)(float)((sA >> 16) & 0xffu), m1 = (_Float16)(float)(sA >> 24);
+        const _Float16 m2 = (_Float16)(float)((sB >> 16) & 0xffu), m3 = (_Float16)(float)(sB >> 24);
+        const kxh8 Bm = {m0, m0, m1, m1, m2, m2, m3, m3};
+        const kx16f Mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(Am, Bm, zf, 0, 0, 0);
+        const float dW = f16bits_to_f32((uint16_t)(dd & 0xffffu)), dmW = f16bits_to_f32((uint16_t)(dd >> 16));
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const float dx = dxv[r >> 2][r & 3];
+          acc[w][j][r] = fmaf(dx * dW, (float)I[r], acc[w][j][r]);
+          acc[w][j][r] = fmaf(-dx * dmW, Mn[r], acc[w][j][r]);
+        }
+      }
+  };
+
+  load_stage(0);
+#pragma unroll
+  for (int w = 0; w < NW; w++)
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+#pragma unroll
+      for (int p = 0; p < 4; p++) load_chunk(w, j, p, 0);
+      load_scales(w, j, 0);
+    }
+  store_stage(0);
+  __syncthreads();
+  for (int sb = 0; sb < nsb; sb++) {
+    load_stage(sb + 1);
+    compute(sb, sb & 1);
+    store_stage((sb + 1) & 1);  // free since the barrier that ended super-block sb - 1
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int r = 0; r < 16; r++) {
+    const int m = 8 * (r >> 2) + 4 * hi + (r & 3);
+    if (m < rows) {
+      const int pos = row0 + m;
+      const int64_t orow = a.out_ids ? a.out_ids[pos] : pos;
+#pragma unroll
+      for (int w = 0; w < NW; w++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          const int n = n0 + 32 * j + c32;
+          if (n < a.N) a.y[w][orow * a.N + n] = acc[w][j][r];
+        }
+    }
+  }
+}
+
+constexpr int KX_TILE = 32;
+bool kx_moe_tiles_fit(int wtype, int64_t N, int64_t K) {
+  return wtype == MLLM_HIP_Q4_K && K % QK_K == 0 && kq_packed_bytes(wtype, N, K) < ((size_t)1 << 32);
+}
+int kx_tile_rows() { return KX_TILE; }
+// MoE row tiles of up to 32 expert-sorted positions: tile t = rows tile_row0[t] .. of expert tile_expert[t]; its rows read
+// image rows row_ids[pos] / row_div (null: pos) and write rows out_ids[pos] (null: pos) of ys[p].
+int kx_moe_tiles(int wtype, int nparts, const void* const* packed0, float* const* ys, int64_t N, int64_t K, const void* image,
+                 int64_t img_rows, const int* tile_expert, const int* tile_row0, const int* tile_rows, const int* ntiles,
+                 unsigned max_tiles, const int* row_ids, int row_div, const int* out_ids, hipStream_t st) {
+  if (!kx_moe_tiles_fit(wtype, N, K) || nparts < 1 || nparts > 2 || max_tiles < 1) return MLLM_HIP_E_SHAPE;
+  if ((size_t)img_rows * K + (size_t)img_rows * (K / 16) * 2 + (size_t)img_rows * (K / QK_K) * 4 >= ((size_t)1 << 32)) return MLLM_HIP_E_SHAPE;
+  KXArgs a{};
+  for (int p = 0; p < nparts; p++) {
+    a.W[p] = reinterpret_cast<const char*>(packed0[p]);
+    a.y[p] = ys[p];
+  }
+  a.estride = kq_packed_bytes(wtype, N, K);
+  a.image = reinterpret_cast<const char*>(image);
+  a.img_rows = (int)img_rows;
+  a.row_ids = row_ids; a.row_div = row_div > 0 ? row_div : 1; a.out_ids = out_ids;
+  a.tile_expert = tile_expert; a.tile_row0 = tile_row0; a.tile_rows = tile_rows; a.ntiles = ntiles;
+  a.N = (int)N; a.K = (int)K;
+  const size_t lds = 2 * (size_t)KX_STAGE + 4 * (size_t)KX_PATCH;
+  if (nparts == 2) {
+    hipLaunchKernelGGL((kx4_kernel<2, 1>), dim3(max_tiles, (unsigned)((N + 127) / 128)), dim3(256), lds, st, a);
+  } else {
+    hipLaunchKernelGGL((kx4_kernel<1, 2>), dim3(max_tiles, (unsigned)((N + 255) / 256)), dim3(256), lds, st, a);
+  }
+  return (int)hipGetLastError();
+}
+
+}  // namespace mllmhip

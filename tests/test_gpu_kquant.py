@@ -308,7 +308,47 @@ def test_moe_ffn_k_quant_grouped_form_equals_the_pair_form(wtype, T, H, I, E, k)
     assert rel_l2(outs[2], outs[1]) < 1e-5, rel_l2(outs[2], outs[1])
     assert np.array_equal(y2, outs[2][perm])
     assert rel_l2(y4, orc.moe_ffn_kq(xb, ids, w, Wg, Wu, Wd, wtype)) < 1e-3
-    assert L.mllm_hip_moe_kq_set_path(3) == -1
+    assert L.mllm_hip_moe_kq_set_path(4) == -1
+
+
+@pytest.mark.parametrize("wtype,T,H,I,E,k", [(2, 40, 512, 256, 6, 3), (2, 96, 2048, 768, 16, 4), (2, 200, 1024, 512, 5, 2),
+                                            (2, 33, 256, 256, 1, 1), (2, 70, 768, 2048, 9, 4), (2, 300, 256, 512, 64, 8)])
+def test_moe_ffn_k_quant_tiles_of_32_rows(wtype, T, H, I, E, k):
+    """Four pairs per expert and more: tiles of 32 expert-sorted rows, the weights as the second operand of 32 x 32 matrix
+    instructions, integer sub-block sums scaled in int32 (experts with one row, 32, 33 rows, none at all; channel counts that
+    end inside a workgroup's 128 or 256).  Same integers as one GEMV row per pair, fp32 scaling in another order: the forms
+    agree to 1e-5 and meet the oracle; invalid expert ids add nothing; a permutation of the tokens permutes the outputs bit
+    for bit; bf16 activations."""
+    rng = synth.rng_for(9, 7300 + wtype + T + H + I + E)
+    L = _lib.lib()
+    Wg = synth.make_weight(rng, wtype, E * I, H).reshape(E, I, H // 256, -1)
+    Wu = synth.make_weight(rng, wtype, E * I, H).reshape(E, I, H // 256, -1)
+    Wd = synth.make_weight(rng, wtype, E * H, I).reshape(E, H, I // 256, -1)
+    ids, w = synth.make_moe_routing(rng, T, E, k)
+    if E > 2:
+        ids[1, 0] = E + 2          # an expert id out of range
+        if k > 1:
+            ids[T - 1, k - 1] = -1
+    g, u, d = (ql.PackedKExperts(wtype, torch.from_numpy(W)) for W in (Wg, Wu, Wd))
+    x = synth.make_x_fp32(rng, T, H)
+    announce("moe k-quant tiles of 32 rows", wtype, T, H, I, E, k)
+    outs = {}
+    for path in (1, 3):
+        assert L.mllm_hip_moe_kq_set_path(path) == 0
+        try:
+            outs[path] = ql.moe_ffn_kq(g, u, d, to_dev(x), to_dev(ids), to_dev(w)).cpu().numpy()
+            if path == 3:
+                perm = rng.permutation(T)
+                y2 = ql.moe_ffn_kq(g, u, d, to_dev(x[perm]), to_dev(ids[perm]), to_dev(w[perm])).cpu().numpy()
+                bits, xb = synth.make_x_bf16(rng, T, H)
+                y4 = ql.moe_ffn_kq(g, u, d, bf16_dev(bits), to_dev(ids), to_dev(w)).cpu().numpy()
+        finally:
+            assert L.mllm_hip_moe_kq_set_path(0) == 0
+    want = orc.moe_ffn_kq(x, ids, w, Wg, Wu, Wd, wtype)
+    assert rel_l2(outs[3], want) < 1e-3, rel_l2(outs[3], want)
+    assert rel_l2(outs[3], outs[1]) < 1e-5, rel_l2(outs[3], outs[1])
+    assert np.array_equal(y2, outs[3][perm])
+    assert rel_l2(y4, orc.moe_ffn_kq(xb, ids, w, Wg, Wu, Wd, wtype)) < 1e-3
 
 
 def _x86_field_to_pattern(field):
