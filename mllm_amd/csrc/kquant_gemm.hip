@@ -44,6 +44,8 @@ struct KXArgs {
   const int* tile_rows;
   const int* ntiles;
   int N, K;
+  int silu_mul;          // two matrices: write silu(y0) * y1 to y[0] instead of both results (the expert MLP's product)
+  int exp_accurate;      // expf instead of the reference's polynomial (mllm_hip_set_exp_mode)
 };
 
 constexpr int KX_LDC = 256 + 16;                           // code row of a super-block, padded: 16-byte reads of 16 rows hit 16 bank groups
@@ -53,18 +55,30 @@ constexpr int KX_OFF_DX = KX_OFF_BS + 32 * KX_BS;
 constexpr int KX_STAGE = KX_OFF_DX + 32 * 4;
 constexpr int KX_WROW = 128 + 16;                           // a channel's line in the wave's patch, padded likewise
 constexpr int KX_PATCH = 32 * KX_WROW;
+constexpr int KX_GROUP = 8;                                 // tiles per group of work items (see the kernel)
 
 // NW matrices (gate and up share the activations) x TN column tiles of 32 channels per wave
 template <int NW, int TN>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void kx4_kernel(KXArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
-  const int t = blockIdx.x;
-  if (t >= a.ntiles[0]) return;
+  // Work items in groups of KX_GROUP tiles (list order: an expert's tiles are neighbours) x all column blocks, inside a group
+  // the tile index fastest.  Workgroup L runs on XCD L % 8, and every XCD has its own L2: XCD x takes a contiguous eighth of
+  // the work items, so that the tiles of one expert and column block, which read the same weights, and the column blocks of
+  // one tile, which read the same activation rows, run on one XCD at about the same time.
+  const int nt = min(a.ntiles[0], (int)gridDim.x), ny = (int)gridDim.y;
+  const int L = (int)(blockIdx.x + gridDim.x * blockIdx.y);
+  const int nw = nt * ny, base = nw >> 3, rem = nw & 7;  // XCD x takes base + (x < rem) items
+  const int xcd = L & 7, seq = L >> 3;
+  if (seq >= base + (xcd < rem)) return;
+  const int wi = xcd * base + min(xcd, rem) + seq;
+  const int per = KX_GROUP * ny, grp = wi / per, r0 = wi - grp * per;
+  const int gt = min(KX_GROUP, nt - grp * KX_GROUP);  // tiles in this group (the last one may be short)
+  const int by = r0 / gt, t = grp * KX_GROUP + (r0 - by * gt);
   const int e = a.tile_expert[t], row0 = a.tile_row0[t], rows = a.tile_rows[t];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c32 = lane & 31, hi = lane >> 5;
   const int nsb = a.K / QK_K;
-  const int n0 = blockIdx.y * (128 * TN) + wave * (32 * TN);
+  const int n0 = by * (128 * TN) + wave * (32 * TN);
 
   // ---- the image: this thread's pieces of a stage ---------------------------------------------------------------------------
   const size_t img_codes = (size_t)a.img_rows * a.K, img_bs = (size_t)a.img_rows * (a.K / 16) * 2;
@@ -238,6 +252,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     if (m < rows) {
       const int pos = row0 + m;
       const int64_t orow = a.out_ids ? a.out_ids[pos] : pos;
+      if (NW == 2 && a.silu_mul) {
+        // SiLU as mllm/backends/cpu/kernels/x86/silu.cpp:16-27 (x * (1 / (1 + exp(-x)))), then the product with the up projection
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          const int n = n0 + 32 * j + c32;
+          const float gv = acc[0][j][r], uv = acc[NW - 1][j][r];
+          if (n < a.N) a.y[0][orow * a.N + n] = gv * (1.0f / (1.0f + (a.exp_accurate ? expf(-gv) : exp_poly(-gv)))) * uv;
+        }
+        continue;
+      }
 #pragma unroll
       for (int w = 0; w < NW; w++)
 #pragma unroll
@@ -256,9 +280,11 @@ bool kx_moe_tiles_fit(int wtype, int64_t N, int64_t K) {
 int kx_tile_rows() { return KX_TILE; }
 // MoE row tiles of up to 32 expert-sorted positions: tile t = rows tile_row0[t] .. of expert tile_expert[t]; its rows read
 // image rows row_ids[pos] / row_div (null: pos) and write rows out_ids[pos] (null: pos) of ys[p].
+// silu_mul (two matrices): ys[0] receives silu(first) * second, ys[1] is not written.
+int exp_mode_accurate();  // layer_ops.hip: the setting of mllm_hip_set_exp_mode
 int kx_moe_tiles(int wtype, int nparts, const void* const* packed0, float* const* ys, int64_t N, int64_t K, const void* image,
                  int64_t img_rows, const int* tile_expert, const int* tile_row0, const int* tile_rows, const int* ntiles,
-                 unsigned max_tiles, const int* row_ids, int row_div, const int* out_ids, hipStream_t st) {
+                 unsigned max_tiles, const int* row_ids, int row_div, const int* out_ids, int silu_mul, hipStream_t st) {
   if (!kx_moe_tiles_fit(wtype, N, K) || nparts < 1 || nparts > 2 || max_tiles < 1) return MLLM_HIP_E_SHAPE;
   if ((size_t)img_rows * K + (size_t)img_rows * (K / 16) * 2 + (size_t)img_rows * (K / QK_K) * 4 >= ((size_t)1 << 32)) return MLLM_HIP_E_SHAPE;
   KXArgs a{};
@@ -272,6 +298,8 @@ int kx_moe_tiles(int wtype, int nparts, const void* const* packed0, float* const
   a.row_ids = row_ids; a.row_div = row_div > 0 ? row_div : 1; a.out_ids = out_ids;
   a.tile_expert = tile_expert; a.tile_row0 = tile_row0; a.tile_rows = tile_rows; a.ntiles = ntiles;
   a.N = (int)N; a.K = (int)K;
+  a.silu_mul = nparts == 2 && silu_mul;
+  a.exp_accurate = exp_mode_accurate();
   const size_t lds = 2 * (size_t)KX_STAGE + 4 * (size_t)KX_PATCH;
   if (nparts == 2) {
     hipLaunchKernelGGL((kx4_kernel<2, 1>), dim3(max_tiles, (unsigned)((N + 127) / 128)), dim3(256), lds, st, a);

@@ -2219,7 +2219,7 @@ bool kx_moe_tiles_fit(int wtype, int64_t N, int64_t K);
 int kx_tile_rows();
 int kx_moe_tiles(int wtype, int nparts, const void* const* packed0, float* const* ys, int64_t N, int64_t K, const void* image,
                  int64_t img_rows, const int* tile_expert, const int* tile_row0, const int* tile_rows, const int* ntiles,
-                 unsigned max_tiles, const int* row_ids, int row_div, const int* out_ids, hipStream_t st);
+                 unsigned max_tiles, const int* row_ids, int row_div, const int* out_ids, int silu_mul, hipStream_t st);
 // 0: by the number of pairs per expert; 1: always pairs as GEMV rows; 2: always tiles of eight rows; 3: always tiles of 32 rows
 // (where the format has them)
 static int g_moe_kq_path = 0;
@@ -2282,7 +2282,8 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
   // 512: 2182 / 480; Q6_K 8 tokens 79 / 77, 16: 142 / 126, 32: 260 / 165, 512: 3976 / 760
   const bool many = wtype == MLLM_HIP_Q4_K ? slots > E : 2 * slots > E;
   // Four pairs per expert and more: tiles of 32 rows, weights as the second operand of 32 x 32 matrix instructions (one pass
-  // over an expert's weights per 32 pairs, one unpacking per 32 rows).  Same integer arithmetic, same launches.
+  // over an expert's weights per 32 pairs, one unpacking per 32 rows).  Same integer arithmetic; silu(gate) * up is formed where
+  // the two results leave their kernel (six launches).
   const bool tiles32_ok = E <= MOE_MAX_EXPERTS && kx_moe_tiles_fit(wtype, I, H) && kx_moe_tiles_fit(wtype, H, I);
   if (tiles32_ok && (g_moe_kq_path == 3 || (g_moe_kq_path == 0 && slots >= 4 * E))) {
     const int th = kx_tile_rows();
@@ -2290,15 +2291,14 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
     RC_RET(launch_route(topk_ids, slots, E, th, w.ro, st));
     RC_RET(kq_quantize_image(x, x_dtype, w.ximg, T, H, st));
     const void* gu2[2] = {gate_packed, up_packed};
-    float* guy2[2] = {g, u};  // rows in expert-sorted order
+    float* guy2[2] = {h, u};  // silu(gate) * up, rows in expert-sorted order
     RC_RET(kx_moe_tiles(wtype, 2, gu2, guy2, I, H, w.ximg, T, w.ro.tile_expert, w.ro.tile_row0, w.ro.tile_rows, w.ro.ntiles, max_tiles,
-                        w.ro.sorted_idx, k, nullptr, st));
-    RC_RET(mllm_hip_silu_mul(g, u, h, MLLM_HIP_F32, slots, I, nullptr, MLLM_HIP_SCALE_IEEE, stream));
+                        w.ro.sorted_idx, k, nullptr, 1, st));
     RC_RET(kq_quantize_image(h, MLLM_HIP_F32, w.himg, slots, I, st));
     const void* dn2[1] = {down_packed};
     float* dny2[1] = {per};  // row t * k + j
     RC_RET(kx_moe_tiles(wtype, 1, dn2, dny2, H, I, w.himg, slots, w.ro.tile_expert, w.ro.tile_row0, w.ro.tile_rows, w.ro.ntiles,
-                        max_tiles, nullptr, 1, w.ro.sorted_idx, st));
+                        max_tiles, nullptr, 1, w.ro.sorted_idx, 0, st));
     const int64_t total2 = T * H;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total2 / 4 + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
                        (int)H, k, E);
