@@ -363,6 +363,12 @@ int mllm_hip_moe_kq_set_path(int path);
 int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x,
                         int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H, int64_t I,
                         int E, int k, void* workspace, void* stream);
+/* The same with the down projections in the other super-block format: wtype for gate and up, wtype_down for down (the shipped
+ * recipe quantizes the experts' gate / up to Q4_K and down to Q6_K, examples/qwen3_moe/quant_cfg_30B_q4_k.json; down_packed then
+ * holds E matrices mllm_hip_kq_packed_bytes(wtype_down, H, I) apart).  Same workspace. */
+int mllm_hip_moe_ffn_kq2(int wtype, int wtype_down, const void* gate_packed, const void* up_packed, const void* down_packed,
+                         const void* x, int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H,
+                         int64_t I, int E, int k, void* workspace, void* stream);
 
 /* mllm_hip_moe_ffn_q has three forms: every (token, expert) pair as GEMV rows (up to eight tokens or one pair per
  * expert), the pairs sorted by expert in tiles of eight rows that share the expert's weights (up to ten pairs per expert), and

@@ -143,6 +143,7 @@ def lib():
         L.mllm_hip_moe_kq_workspace_bytes.restype = C.c_size_t
         L.mllm_hip_moe_kq_workspace_bytes.argtypes = [i64, i64, i64, ci, ci]
         L.mllm_hip_moe_ffn_kq.argtypes = [ci, vp, vp, vp, vp, ci, vp, vp, vp, i64, i64, i64, ci, ci, vp, vp]
+        L.mllm_hip_moe_ffn_kq2.argtypes = [ci, ci, vp, vp, vp, vp, ci, vp, vp, vp, i64, i64, i64, ci, ci, vp, vp]
         L.mllm_hip_moe_gemm_set_path.argtypes = [ci]
         L.mllm_hip_moe_route.argtypes = [vp, i64, ci, ci, vp, vp, vp, vp, vp]
         L.mllm_hip_matmul_f32.argtypes = [vp, vp, vp, i64, i64, i64, ci, ci, vp]

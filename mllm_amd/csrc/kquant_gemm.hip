@@ -17,6 +17,10 @@
 //     on the sixteen sums of 16 as fp16 integers (at most 2048: exact) and the 6-bit minima (every product and sum below
 //     2^24: exact); per super-block and output then y += (dX * d) * float(I) and y += -(dX * dmin) * float(M), the products
 //     and the FMAs of vec_dot_q4_K_q8_K (mllm/backends/cpu/kernels/common/ggml/vec_dot.cpp:498-560).
+//   * Q6_K: the scales belong to groups of 16 elements, so a group is one v_mfma_i32_32x32x16_i8; the 6-bit codes enter
+//     unsigned (low nibble | two high bits << 4, three to four operations per four codes) and the format's offset of 32 leaves
+//     through the sums of 16: I = sum_g sc_g * T_g - 32 * sum_g sc_g * bsum_g, the second sum again one fp16 instruction per
+//     super-block (at most 128 * 2048 * 16: exact); y += (dX * d) * float(I), vec_dot_q6_K_q8_K (vec_dot.cpp:955-1044).
 // What differs from the CPU path is the order of the fp32 additions only (the CPU keeps eight lanes per output and a
 // separate accumulator for the minimum term; here one accumulator per output takes both terms super-block by super-block).
 #include <type_traits>
@@ -55,11 +59,14 @@ constexpr int KX_OFF_DX = KX_OFF_BS + 32 * KX_BS;
 constexpr int KX_STAGE = KX_OFF_DX + 32 * 4;
 constexpr int KX_WROW = 128 + 16;                           // a channel's line in the wave's patch, padded likewise
 constexpr int KX_PATCH = 32 * KX_WROW;
+constexpr int KX6_WROW = 128 + 64 + 16;                     // Q6_K: low nibbles, high bit pairs, padding
+constexpr int KX6_PATCH = 32 * KX6_WROW;
 constexpr int KX_GROUP = 8;                                 // tiles per group of work items (see the kernel)
 
 // NW matrices (gate and up share the activations) x TN column tiles of 32 channels per wave
-template <int NW, int TN>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void kx4_kernel(KXArgs a) {
+template <int WT, int NW, int TN>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void kx_kernel(KXArgs a) {
+  constexpr bool K4 = WT == MLLM_HIP_Q4_K;
   extern __shared__ __align__(16) unsigned char smem[];
   // Work items in groups of KX_GROUP tiles (list order: an expert's tiles are neighbours) x all column blocks, inside a group
   // the tile index fastest.  Workgroup L runs on XCD L % 8, and every XCD has its own L2: XCD x takes a contiguous eighth of
@@ -125,7 +132,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
   // ---- the weights: lane (channel c32 of a column tile, K half hi) -----------------------------------------------------------
   const size_t sbt = (size_t)a.N * nsb;
-  const uint32_t oS = (uint32_t)kq_plane(sbt * 128), oD = oS + (uint32_t)kq_plane(sbt * 16);
+  const uint32_t oH = (uint32_t)kq_plane(sbt * 128);                            // Q6_K: high bit pairs
+  const uint32_t oS = K4 ? oH : oH + (uint32_t)kq_plane(sbt * 64), oD = oS + (uint32_t)kq_plane(sbt * 16);
+  constexpr int DB = K4 ? 4 : 2;                                                // bytes of plane D per super-block
   __amdgpu_buffer_rsrc_t rW[NW];
 #pragma unroll
   for (int w = 0; w < NW; w++)
@@ -136,10 +145,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int n = n0 + 32 * j + c32;
     const bool ok = n < a.N;
     offS[j] = ok ? oS + (uint32_t)((size_t)n * nsb * 16) : 0xffffffffu;
-    offD[j] = ok ? oD + (uint32_t)((size_t)n * nsb * 4) : 0xffffffffu;
+    offD[j] = ok ? oD + (uint32_t)((size_t)n * nsb * DB) : 0xffffffffu;
   }
   // one register set: a chunk's registers are requested again for the next super-block as soon as the chunk is unpacked
-  u32x4 wq[NW][TN][4], ws[NW][TN];
+  u32x4 wq[NW][TN][4], wh[NW][TN][K4 ? 1 : 2], ws[NW][TN];
   uint32_t wd[NW][TN];
   // request i of a column tile: channels 8 i .. 8 i + 7, lane l takes 16-byte chunk l % 8 of channel 8 i + l / 8
   const int lr = lane >> 3, lc = lane & 7;
@@ -148,9 +157,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const uint32_t off = (n < a.N && sb < nsb) ? (uint32_t)(((size_t)n * nsb * 8 + lc) * 16) : 0xffffffffu;
     wq[w][j][i] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], off, sb * 128, 0);
   };
+  // Q6_K, high bit pairs: request i = channels 16 i .. 16 i + 15, lane l takes chunk l % 4 of channel 16 i + l / 4
+  auto load_high = [&](int w, int j, int i, int sb) {
+    const int n = n0 + 32 * j + 16 * i + (lane >> 2);
+    const uint32_t off = (n < a.N && sb < nsb) ? oH + (uint32_t)(((size_t)n * nsb * 4 + (lane & 3)) * 16) : 0xffffffffu;
+    wh[w][j][K4 ? 0 : i] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], off, sb * 64, 0);
+  };
   auto load_scales = [&](int w, int j, int sb) {
     ws[w][j] = __builtin_amdgcn_raw_buffer_load_b128(rW[w], sb < nsb ? offS[j] : 0xffffffffu, sb * 16, 0);
-    wd[w][j] = __builtin_amdgcn_raw_buffer_load_b32(rW[w], sb < nsb ? offD[j] : 0xffffffffu, sb * 4, 0);
+    if (K4) wd[w][j] = __builtin_amdgcn_raw_buffer_load_b32(rW[w], sb < nsb ? offD[j] : 0xffffffffu, sb * 4, 0);
+    else wd[w][j] = (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rW[w], sb < nsb ? offD[j] : 0xffffffffu, sb * 2, 0);
   };
 
   float acc[NW][TN][16];
@@ -166,12 +182,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   // one super-block from LDS buffer `buf`
   auto compute = [&](int sb, int buf) {
     const unsigned char* st = smem + buf * KX_STAGE;
-    unsigned char* patch = smem + 2 * KX_STAGE + wave * KX_PATCH;
+    unsigned char* patch = smem + 2 * KX_STAGE + wave * (K4 ? KX_PATCH : KX6_PATCH);
     // output r of this lane = tile row 8 (r / 4) + 4 hi + r % 4
     f32x4 dxv[4];
 #pragma unroll
     for (int g = 0; g < 4; g++) dxv[g] = *reinterpret_cast<const f32x4*>(st + KX_OFF_DX + (8 * g + 4 * hi) * 4);
     const kxh8 Am = *reinterpret_cast<const kxh8*>(st + KX_OFF_BS + c32 * KX_BS + hi * 16);
+    if constexpr (K4) {
 #pragma unroll
     for (int w = 0; w < NW; w++)
 #pragma unroll
@@ -226,6 +243,72 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           acc[w][j][r] = fmaf(-dx * dmW, Mn[r], acc[w][j][r]);
         }
       }
+      } else {
+#pragma unroll
+      for (int w = 0; w < NW; w++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+          int I[16];
+#pragma unroll
+          for (int r = 0; r < 16; r++) I[r] = 0;
+          const uint32_t srec[4] = {ws[w][j].x, ws[w][j].y, ws[w][j].z, ws[w][j].w};
+          const uint32_t dd = wd[w][j];
+#pragma unroll
+          for (int i = 0; i < 4; i++) *reinterpret_cast<u32x4*>(patch + (8 * i + lr) * KX6_WROW + lc * 16) = wq[w][j][i];
+#pragma unroll
+          for (int i = 0; i < 2; i++) *reinterpret_cast<u32x4*>(patch + (16 * i + (lane >> 2)) * KX6_WROW + 128 + (lane & 3) * 16) = wh[w][j][i];
+#pragma unroll
+          for (int i = 0; i < 4; i++) load_chunk(w, j, i, sb + 1);
+#pragma unroll
+          for (int i = 0; i < 2; i++) load_high(w, j, i, sb + 1);
+          // group g of 16 elements = half h = g / 8, quarter qd = g % 8 / 2, l = 16 (g % 2) + 8 hi + (0..7) (dequantize_row_q6_K,
+          // quantize_q6.cpp:108-133): low nibbles from ql[64 h + 32 (qd % 2) + l] (high nibble for qd >= 2), bits 2 qd, 2 qd + 1 of qh[32 h + l]
+#pragma unroll
+          for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int par = 0; par < 2; par++) {
+              const u32x2 QH = *reinterpret_cast<const u32x2*>(patch + c32 * KX6_WROW + 128 + 32 * h + 16 * par + 8 * hi);
+#pragma unroll
+              for (int ql01 = 0; ql01 < 2; ql01++) {
+                const u32x2 QL = *reinterpret_cast<const u32x2*>(patch + c32 * KX6_WROW + 64 * h + 32 * ql01 + 16 * par + 8 * hi);
+#pragma unroll
+                for (int nib = 0; nib < 2; nib++) {
+                  const int qd = 2 * nib + ql01, g = 8 * h + 2 * qd + par;
+                  uint32_t b[2];
+#pragma unroll
+                  for (int d2 = 0; d2 < 2; d2++) {
+                    const uint32_t lbits = nib ? (QL[d2] >> 4) & 0x0f0f0f0fu : QL[d2] & 0x0f0f0f0fu;
+                    const uint32_t hs = qd == 0 ? QH[d2] << 4 : qd == 1 ? QH[d2] << 2 : qd == 2 ? QH[d2] : QH[d2] >> 2;
+                    b[d2] = (hs & 0x30303030u) | lbits;
+                  }
+                  const long B = (long)(((unsigned long)b[1] << 32) | b[0]);
+                  const long A = *reinterpret_cast<const long*>(st + c32 * KX_LDC + 16 * g + 8 * hi);
+                  const kx16i T = __builtin_amdgcn_mfma_i32_32x32x16_i8(A, B, zi, 0, 0, 0);
+                  const int sc = (int)(int8_t)(srec[g >> 2] >> (8 * (g & 3)));
+#pragma unroll
+                  for (int r = 0; r < 16; r++) {
+                    I[r] = __mul24(T[r], sc) + I[r];
+                    asm volatile("" : "+v"(I[r]));
+                  }
+                  __builtin_amdgcn_sched_barrier(0);
+                }
+              }
+            }
+          load_scales(w, j, sb + 1);
+          // the offset of 32: K slot 8 hi + i of the instruction = sum of 16 number 8 hi + i = group 8 hi + i
+          kxh8 Bs;
+#pragma unroll
+          for (int i = 0; i < 8; i++) Bs[i] = (_Float16)(float)(int)(int8_t)((hi ? srec[2 + (i >> 2)] : srec[i >> 2]) >> (8 * (i & 3)));
+          const kx16f Mn = __builtin_amdgcn_mfma_f32_32x32x16_f16(Am, Bs, zf, 0, 0, 0);
+          const float dW = f16bits_to_f32((uint16_t)dd);
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            const float dx = dxv[r >> 2][r & 3];
+            const int tot = I[r] - 32 * (int)Mn[r];
+            acc[w][j][r] = fmaf(dx * dW, (float)tot, acc[w][j][r]);
+          }
+        }
+    }
   };
 
   load_stage(0);
@@ -235,6 +318,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     for (int j = 0; j < TN; j++) {
 #pragma unroll
       for (int p = 0; p < 4; p++) load_chunk(w, j, p, 0);
+      if (!K4) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) load_high(w, j, p, 0);
+      }
       load_scales(w, j, 0);
     }
   store_stage(0);
@@ -275,7 +362,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 
 constexpr int KX_TILE = 32;
 bool kx_moe_tiles_fit(int wtype, int64_t N, int64_t K) {
-  return wtype == MLLM_HIP_Q4_K && K % QK_K == 0 && kq_packed_bytes(wtype, N, K) < ((size_t)1 << 32);
+  return (wtype == MLLM_HIP_Q4_K || wtype == MLLM_HIP_Q6_K) && K % QK_K == 0 && kq_packed_bytes(wtype, N, K) < ((size_t)1 << 32);
 }
 int kx_tile_rows() { return KX_TILE; }
 // MoE row tiles of up to 32 expert-sorted positions: tile t = rows tile_row0[t] .. of expert tile_expert[t]; its rows read
@@ -300,11 +387,15 @@ int kx_moe_tiles(int wtype, int nparts, const void* const* packed0, float* const
   a.N = (int)N; a.K = (int)K;
   a.silu_mul = nparts == 2 && silu_mul;
   a.exp_accurate = exp_mode_accurate();
-  const size_t lds = 2 * (size_t)KX_STAGE + 4 * (size_t)KX_PATCH;
+  const bool k4 = wtype == MLLM_HIP_Q4_K;
+  const size_t lds = 2 * (size_t)KX_STAGE + 4 * (size_t)(k4 ? KX_PATCH : KX6_PATCH);
+  const dim3 g2(max_tiles, (unsigned)((N + 127) / 128)), g1(max_tiles, (unsigned)((N + 255) / 256));
   if (nparts == 2) {
-    hipLaunchKernelGGL((kx4_kernel<2, 1>), dim3(max_tiles, (unsigned)((N + 127) / 128)), dim3(256), lds, st, a);
+    if (k4) hipLaunchKernelGGL((kx_kernel<MLLM_HIP_Q4_K, 2, 1>), g2, dim3(256), lds, st, a);
+    else hipLaunchKernelGGL((kx_kernel<MLLM_HIP_Q6_K, 2, 1>), g2, dim3(256), lds, st, a);
   } else {
-    hipLaunchKernelGGL((kx4_kernel<1, 2>), dim3(max_tiles, (unsigned)((N + 255) / 256)), dim3(256), lds, st, a);
+    if (k4) hipLaunchKernelGGL((kx_kernel<MLLM_HIP_Q4_K, 1, 2>), g1, dim3(256), lds, st, a);
+    else hipLaunchKernelGGL((kx_kernel<MLLM_HIP_Q6_K, 1, 2>), g1, dim3(256), lds, st, a);
   }
   return (int)hipGetLastError();
 }

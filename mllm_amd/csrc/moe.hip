@@ -2256,10 +2256,10 @@ MLLM_API size_t mllm_hip_moe_kq_workspace_bytes(int64_t T, int64_t H, int64_t I,
   return c.used;
 }
 
-MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x,
-                                 int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H,
-                                 int64_t I, int E, int k, void* workspace, void* stream) {
-  if ((wtype != MLLM_HIP_Q4_K && wtype != MLLM_HIP_Q6_K) || !gate_packed || !up_packed || !down_packed || !x || !topk_ids ||
+MLLM_API int mllm_hip_moe_ffn_kq2(int wtype, int wtype_down, const void* gate_packed, const void* up_packed, const void* down_packed,
+                                  const void* x, int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T,
+                                  int64_t H, int64_t I, int E, int k, void* workspace, void* stream) {
+  if ((wtype != MLLM_HIP_Q4_K && wtype != MLLM_HIP_Q6_K) || (wtype_down != MLLM_HIP_Q4_K && wtype_down != MLLM_HIP_Q6_K) || !gate_packed || !up_packed || !down_packed || !x || !topk_ids ||
       !topk_w || !y || !workspace || T <= 0 || E <= 0 || k <= 0)
     return MLLM_HIP_E_BADARG;
   if (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16) return MLLM_HIP_E_BADARG;
@@ -2276,15 +2276,15 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
   // More than about one pair per expert (Q6_K: half a pair): the pairs are sorted by expert and run as tiles of eight rows on the matrix-core
   // kernels, so an expert's matrices are streamed once per eight pairs instead of once per pair (the grouped form).
   // x and h are quantized to Q8_K once (bit-exact images), the tiles gather their rows from the images.
-  const bool tiles_ok = E <= MOE_MAX_EXPERTS && kq_moe_tiles_fit(wtype, H) && kq_moe_tiles_fit(wtype, I) &&
+  const bool tiles_ok = E <= MOE_MAX_EXPERTS && kq_moe_tiles_fit(wtype, H) && kq_moe_tiles_fit(wtype_down, I) &&
                         (size_t)E + (size_t)slots / KQ_MOE_TILE + 1 <= 65535;
   // measured at 128 experts, top-8 (pairs / tiles, us): Q4_K 16 tokens 80 / 84, 24: 112 / 97, 32: 145 / 112, 64: 289 / 153,
   // 512: 2182 / 480; Q6_K 8 tokens 79 / 77, 16: 142 / 126, 32: 260 / 165, 512: 3976 / 760
-  const bool many = wtype == MLLM_HIP_Q4_K ? slots > E : 2 * slots > E;
+  const bool many = (wtype == MLLM_HIP_Q4_K && wtype_down == MLLM_HIP_Q4_K) ? slots > E : 2 * slots > E;
   // Four pairs per expert and more: tiles of 32 rows, weights as the second operand of 32 x 32 matrix instructions (one pass
   // over an expert's weights per 32 pairs, one unpacking per 32 rows).  Same integer arithmetic; silu(gate) * up is formed where
   // the two results leave their kernel (six launches).
-  const bool tiles32_ok = E <= MOE_MAX_EXPERTS && kx_moe_tiles_fit(wtype, I, H) && kx_moe_tiles_fit(wtype, H, I);
+  const bool tiles32_ok = E <= MOE_MAX_EXPERTS && kx_moe_tiles_fit(wtype, I, H) && kx_moe_tiles_fit(wtype_down, H, I);
   if (tiles32_ok && (g_moe_kq_path == 3 || (g_moe_kq_path == 0 && slots >= 4 * E))) {
     const int th = kx_tile_rows();
     const unsigned max_tiles = (unsigned)(E + slots / th + 1);
@@ -2297,7 +2297,7 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
     RC_RET(kq_quantize_image(h, MLLM_HIP_F32, w.himg, slots, I, st));
     const void* dn2[1] = {down_packed};
     float* dny2[1] = {per};  // row t * k + j
-    RC_RET(kx_moe_tiles(wtype, 1, dn2, dny2, H, I, w.himg, slots, w.ro.tile_expert, w.ro.tile_row0, w.ro.tile_rows, w.ro.ntiles,
+    RC_RET(kx_moe_tiles(wtype_down, 1, dn2, dny2, H, I, w.himg, slots, w.ro.tile_expert, w.ro.tile_row0, w.ro.tile_rows, w.ro.ntiles,
                         max_tiles, nullptr, 1, w.ro.sorted_idx, 0, st));
     const int64_t total2 = T * H;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total2 / 4 + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
@@ -2317,7 +2317,7 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
     RC_RET(kq_quantize_image(h, MLLM_HIP_F32, w.himg, slots, I, st));
     const void* dn2[1] = {down_packed};
     float* dny2[1] = {per};  // row t * k + j
-    RC_RET(kq_moe_tiles_gemv(wtype, 1, dn2, dny2, H, I, w.himg, slots, w.ro.tile_expert, w.ro.tile_row0, w.ro.tile_rows,
+    RC_RET(kq_moe_tiles_gemv(wtype_down, 1, dn2, dny2, H, I, w.himg, slots, w.ro.tile_expert, w.ro.tile_row0, w.ro.tile_rows,
                              w.ro.ntiles, max_tiles, nullptr, 1, w.ro.sorted_idx, st));
     const int64_t total2 = T * H;
     hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total2 / 4 + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
@@ -2334,15 +2334,22 @@ MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void*
   const void* dn[1] = {down_packed};
   float* dny[1] = {per};
   if (slots <= 32) {
-    rc = kq_moe_gemv(wtype, 1, dn, dny, H, I, g, MLLM_HIP_F32, u, topk_ids, E, slots, 1, st);
+    rc = kq_moe_gemv(wtype_down, 1, dn, dny, H, I, g, MLLM_HIP_F32, u, topk_ids, E, slots, 1, st);
   } else {
     rc = mllm_hip_silu_mul(g, u, h, MLLM_HIP_F32, slots, I, nullptr, MLLM_HIP_SCALE_IEEE, stream);
     if (rc) return rc;
-    rc = kq_moe_gemv(wtype, 1, dn, dny, H, I, h, MLLM_HIP_F32, nullptr, topk_ids, E, slots, 1, st);
+    rc = kq_moe_gemv(wtype_down, 1, dn, dny, H, I, h, MLLM_HIP_F32, nullptr, topk_ids, E, slots, 1, st);
   }
   if (rc) return rc;
   const int64_t total = T * H;
   hipLaunchKernelGGL(moe_combine_kernel, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st, per, topk_w, topk_ids, y, T,
                      (int)H, k, E);
   return (int)hipGetLastError();
+}
+
+MLLM_API int mllm_hip_moe_ffn_kq(int wtype, const void* gate_packed, const void* up_packed, const void* down_packed, const void* x,
+                                 int x_dtype, const int32_t* topk_ids, const float* topk_w, float* y, int64_t T, int64_t H,
+                                 int64_t I, int E, int k, void* workspace, void* stream) {
+  return mllm_hip_moe_ffn_kq2(wtype, wtype, gate_packed, up_packed, down_packed, x, x_dtype, topk_ids, topk_w, y, T, H, I, E, k, workspace,
+                              stream);
 }

@@ -611,18 +611,25 @@ class PackedKExperts:
 
 
 def moe_ffn_kq(gate, up, down, x, topk_ids, topk_w, workspace=None, out=None):
-    """The MoE expert FFN with Q4_K / Q6_K experts (PackedKExperts): x [T, H], topk_ids int32 [T, k], topk_w fp32 [T, k]."""
+    """The MoE expert FFN with Q4_K / Q6_K experts (PackedKExperts): x [T, H], topk_ids int32 [T, k], topk_w fp32 [T, k].
+    gate and up share a format; down may have the other one (the shipped recipe: Q4_K gate / up, Q6_K down)."""
     T, H = x.shape
     k = topk_ids.shape[1]
     E, I = gate.E, gate.N
     assert gate.K == H and up.N == I and down.N == H and down.K == I and topk_ids.dtype == torch.int32
+    assert gate.wtype == up.wtype
     L = _lib.lib()
     if workspace is None:
         workspace = torch.empty(L.mllm_hip_moe_kq_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
     y = out if out is not None else torch.empty((T, H), dtype=torch.float32, device="cuda")
-    _lib.check(L.mllm_hip_moe_ffn_kq(gate.wtype, gate.ptr, up.ptr, down.ptr, x.data_ptr(), _xdtype(x), topk_ids.data_ptr(),
-                                     topk_w.data_ptr(), y.data_ptr(), T, H, I, E, k, workspace.data_ptr(), _stream()),
-               "mllm_hip_moe_ffn_kq")
+    if down.wtype == gate.wtype:
+        _lib.check(L.mllm_hip_moe_ffn_kq(gate.wtype, gate.ptr, up.ptr, down.ptr, x.data_ptr(), _xdtype(x), topk_ids.data_ptr(),
+                                         topk_w.data_ptr(), y.data_ptr(), T, H, I, E, k, workspace.data_ptr(), _stream()),
+                   "mllm_hip_moe_ffn_kq")
+    else:
+        _lib.check(L.mllm_hip_moe_ffn_kq2(gate.wtype, down.wtype, gate.ptr, up.ptr, down.ptr, x.data_ptr(), _xdtype(x),
+                                          topk_ids.data_ptr(), topk_w.data_ptr(), y.data_ptr(), T, H, I, E, k, workspace.data_ptr(),
+                                          _stream()), "mllm_hip_moe_ffn_kq2")
     return y
 
 

@@ -422,18 +422,20 @@ def linear_kq(x, W, wtype, bias=None, scale_mode=SCALE_X86_REF):
     return y
 
 
-def moe_ffn_kq(x, topk_ids, topk_w, Wg, Wu, Wd, wtype, scale_mode=SCALE_X86_REF):
+def moe_ffn_kq(x, topk_ids, topk_w, Wg, Wu, Wd, wtype, scale_mode=SCALE_X86_REF, wtype_down=None):
     """The expert FFN of moe_ffn with Q4_K / Q6_K experts (the formats the shipped Qwen3-MoE recipe quantizes to): per active
     expert three linear_kq calls (each quantizes its input rows to Q8_K), silu over the gathered [cnt, I] tensor and the
     product in between, then acc += per * w in slot order (modeling_qwen3_moe_fa2.hpp:98-100,175-238).  A composition of
     functions pinned on their own (linear_kq, silu); x fp32 [T, H]; Wg/Wu uint8 [E, I, H/256, blk]; Wd uint8 [E, H, I/256, blk];
-    slots with an expert id outside [0, E) contribute nothing."""
+    slots with an expert id outside [0, E) contribute nothing.  wtype_down: the format of the down projections where it
+    differs (the shipped recipe: Q4_K gate / up, Q6_K down, examples/qwen3_moe/quant_cfg_30B_q4_k.json)."""
     x = np.ascontiguousarray(x, dtype=np.float32)
     ids = np.ascontiguousarray(topk_ids, dtype=np.int32)
     tw = np.ascontiguousarray(topk_w, dtype=np.float32)
     T, H = x.shape
     E = Wg.shape[0]
     k = ids.shape[1]
+    wtype_down = wtype if wtype_down is None else wtype_down
     per = np.zeros((T * k, H), np.float32)
     flat = ids.reshape(-1)
     for e in range(E):
@@ -444,7 +446,7 @@ def moe_ffn_kq(x, topk_ids, topk_w, Wg, Wu, Wd, wtype, scale_mode=SCALE_X86_REF)
         g = linear_kq(xe, Wg[e], wtype, scale_mode=scale_mode)
         u = linear_kq(xe, Wu[e], wtype, scale_mode=scale_mode)
         h = silu(g) * u
-        per[pos] = linear_kq(h, Wd[e], wtype, scale_mode=scale_mode)
+        per[pos] = linear_kq(h, Wd[e], wtype_down, scale_mode=scale_mode)
     y = np.zeros((T, H), np.float32)
     per = per.reshape(T, k, H)
     valid = (ids >= 0) & (ids < E)

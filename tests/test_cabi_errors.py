@@ -70,6 +70,9 @@ def _cases():
         "mllm_hip_moe_ffn_kq": ([Q4_K, P, P, P, P, F32, P, P, P, 4, 256, 256, 8, 2, P, None],
                                 [(0, Q4_0, BADARG), (1, None, BADARG), (3, None, BADARG), (4, None, BADARG), (6, None, BADARG),
                                  (14, None, BADARG), (10, 128, SHAPE), (11, 320, SHAPE), (9, 40000, SHAPE), (4, ODD, ALIGN)]),
+        "mllm_hip_moe_ffn_kq2": ([Q4_K, Q6_K, P, P, P, P, F32, P, P, P, 4, 256, 256, 8, 2, P, None],
+                                 [(0, Q4_0, BADARG), (1, Q8_0, BADARG), (2, None, BADARG), (5, None, BADARG), (11, 128, SHAPE),
+                                  (12, 320, SHAPE), (10, 40000, SHAPE), (5, ODD, ALIGN)]),
         "mllm_hip_kq_quantize_weight_blocks": ([Q6_K, P, P, 0, 8, 256, None], [(0, Q8_0, BADARG), (1, None, BADARG), (2, None, BADARG),
                                                                               (3, 7, BADARG), (5, 128, SHAPE), (4, 0, BADARG)]),
         "mllm_hip_kq_prepack": ([Q4_K, P, 0, P, 8, 256, None], [(0, Q4_0, BADARG), (1, None, BADARG), (3, None, BADARG), (5, 128, SHAPE)]),
