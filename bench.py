@@ -69,25 +69,28 @@ def side_workloads(torch, ql, synth, gen):
     """The other configurations of the metric: W8A8 / W4A16 prefill GEMMs (MFMA-bound) and the MoE expert FFN."""
     def ev_time(fn, reps):
         """seconds per call: `reps` calls captured in one HIP graph (a few microseconds of Python per eager call would otherwise
-        be counted as kernel time of the small launches), replayed three times between HIP events"""
+        be counted as kernel time of the small launches), replayed ten times between HIP events after three untimed replays
+        (the first replays of a graph run 5 to 10 % slower than the steady state the headline's warm-up steps reach)"""
         fn()
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             for _ in range(reps):
                 fn()
-        g.replay()
+        for _ in range(3):
+            g.replay()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(3):
+        for _ in range(10):
             g.replay()
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / (3 * reps)
+        return e0.elapsed_time(e1) * 1e-3 / (10 * reps)
 
     def ev_replay(g, reps):
-        g.replay()
+        for _ in range(3):
+            g.replay()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -226,12 +229,6 @@ def side_workloads(torch, ql, synth, gen):
     from mllm_amd import _lib as _l
     wsk = torch.empty(_l.lib().mllm_hip_moe_kq_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
     tk2 = ev_time(lambda: ql.moe_ffn_kq(gk, uk, dk, x, ids, tw, workspace=wsk, out=ym), 5)
-    gkq = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(gkq):
-        for _ in range(10):
-            ql.moe_ffn_kq(gk, uk, dk, x, ids, tw, workspace=wsk, out=ym)
-    tk2g = ev_replay(gkq, 10) / 10
-    del gkq
     _l.lib().mllm_hip_moe_kq_set_path(2)
     tk8 = ev_time(lambda: ql.moe_ffn_kq(gk, uk, dk, x, ids, tw, workspace=wsk, out=ym), 5)
     _l.lib().mllm_hip_moe_kq_set_path(1)
@@ -240,21 +237,13 @@ def side_workloads(torch, ql, synth, gen):
     wbk = int((np.bincount(ids_np.reshape(-1), minlength=E) > 0).sum()) * 3 * I * (H // 256) * 144
     # the shipped recipe's formats: gate / up Q4_K, down Q6_K (examples/qwen3_moe/quant_cfg_30B_q4_k.json)
     dk6 = ql.PackedKExperts.synthetic(ql.Q6_K, E, H, I, gen)
-    gk6 = torch.cuda.CUDAGraph()
-    ql.moe_ffn_kq(gk, uk, dk6, x, ids, tw, workspace=wsk, out=ym)
-    torch.cuda.synchronize()
-    with torch.cuda.graph(gk6):
-        for _ in range(10):
-            ql.moe_ffn_kq(gk, uk, dk6, x, ids, tw, workspace=wsk, out=ym)
-    tk6g = ev_replay(gk6, 10) / 10
-    del gk6
     tk6 = ev_time(lambda: ql.moe_ffn_kq(gk, uk, dk6, x, ids, tw, workspace=wsk, out=ym), 5)
     wbk6 = wbk // 3 * 2 + int((np.bincount(ids_np.reshape(-1), minlength=E) > 0).sum()) * H * (I // 256) * 210
-    deck["tokens_512_grouped_q4_k_gate_up_q6_k_down"] = {"us": tk6 * 1e6, "in_a_graph_us": tk6g * 1e6, "weight_GBps": wbk6 / tk6g / 1e9,
-                                                         "frac_of_hbm_peak_in_a_graph": wbk6 / tk6g / 8e12}
+    deck["tokens_512_grouped_q4_k_gate_up_q6_k_down"] = {"us": tk6 * 1e6, "weight_GBps": wbk6 / tk6 / 1e9,
+                                                         "frac_of_hbm_peak": wbk6 / tk6 / 8e12}
     del dk6
     deck["tokens_512_grouped"] = {"us": tk2 * 1e6, "weight_GBps": wbk / tk2 / 1e9, "frac_of_hbm_peak": wbk / tk2 / 8e12,
-                                  "in_a_graph_us": tk2g * 1e6, "tiles_of_8_rows_us": tk8 * 1e6, "pairs_as_gemv_rows_us": tk1 * 1e6}
+                                  "tiles_of_8_rows_us": tk8 * 1e6, "pairs_as_gemv_rows_us": tk1 * 1e6}
     del gk, uk, dk, wsk
     from mllm_amd import _lib
     L = _lib.lib()
@@ -263,14 +252,6 @@ def side_workloads(torch, ql, synth, gen):
     down2 = ql.PackedExperts.synthetic(ql.Q4_0, E, H, I, gen, layout="gemm")
     wsm2 = torch.empty(L.mllm_hip_moe_gemm_workspace_bytes(T, H, I, E, k), dtype=torch.uint8, device="cuda")
     tm2 = ev_time(lambda: ql.moe_ffn_q_gemm(gate2, up2, down2, x, ids, tw, workspace=wsm2, out=ym), 10)
-    # the same call captured ten times in a graph (how a serving loop would issue it): without the gaps that four eager
-    # launches per call leave between their kernels
-    gm = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(gm):
-        for _ in range(10):
-            ql.moe_ffn_q_gemm(gate2, up2, down2, x, ids, tw, workspace=wsm2, out=ym)
-    tm2g = ev_replay(gm, 10) / 10
-    del gm
     L.mllm_hip_moe_gemm_set_path(1)
     tm3 = ev_time(lambda: ql.moe_ffn_q_gemm(gate2, up2, down2, x, ids, tw, workspace=wsm2, out=ym), 10)
     L.mllm_hip_moe_gemm_set_path(0)
@@ -279,10 +260,6 @@ def side_workloads(torch, ql, synth, gen):
     flops = T * k * (2.0 * H * I * 2 + 2.0 * I * H)
     out["moe_ffn_512tok_128e_top8_q4_0"] = {"us": tm2 * 1e6, "active_experts": active, "weight_GBps": wbytes / tm2 / 1e9,
                                             "frac_of_hbm_peak": wbytes / tm2 / 8e12, "TFLOPS": flops / tm2 / 1e12,
-                                            "in_a_graph": {"us": tm2g * 1e6, "weight_GBps": wbytes / tm2g / 1e9,
-                                                           "frac_of_hbm_peak": wbytes / tm2g / 8e12,
-                                                           "note": "ten calls captured in one HIP graph; 'us' above is the same call "
-                                                                   "launched eagerly (four launches, gaps between their kernels)"},
                                             "path": "mllm_hip_moe_ffn_q_gemm, default form: the reference's block arithmetic on the matrix "
                                                     "cores (exact integer block sums and exact scale products from fp16 MFMAs, one fp32 FMA "
                                                     "per block; 4 launches: route + quantize, gate + up + SiLU*up + re-quantize, down, weighted sum)",
