@@ -56,6 +56,8 @@ def parse():
     ap.add_argument("--side-only", action="store_true",
                     help="profiling run: only the prefill GEMM / MoE side workloads (W8A8, W4A16, MoE FFN, Q4_0 prefill Linear), "
                          "printed as one JSON object; meant to run under rocprofv3")
+    ap.add_argument("--brief", action="store_true",
+                    help="with --side-only: one untimed and one timed replay per workload (counter runs: fewer dispatches to record)")
     ap.add_argument("--layer-only", action="store_true",
                     help="profiling run: only the decoder-layer chain (operators one by one and folded, M = 1 and 8) and the "
                          "Q4_K / Q6_K gate projection, printed as one JSON object; meant to run under rocprofv3")
@@ -65,8 +67,10 @@ def parse():
     return ap.parse_args()
 
 
-def side_workloads(torch, ql, synth, gen):
+def side_workloads(torch, ql, synth, gen, brief=False):
     """The other configurations of the metric: W8A8 / W4A16 prefill GEMMs (MFMA-bound) and the MoE expert FFN."""
+    WARM, TIMED = (1, 1) if brief else (3, 10)
+
     def ev_time(fn, reps):
         """seconds per call: `reps` calls captured in one HIP graph (a few microseconds of Python per eager call would otherwise
         be counted as kernel time of the small launches), replayed ten times between HIP events after three untimed replays
@@ -77,19 +81,21 @@ def side_workloads(torch, ql, synth, gen):
         with torch.cuda.graph(g):
             for _ in range(reps):
                 fn()
-        for _ in range(3):
+        for _ in range(WARM):
             g.replay()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(10):
+        for _ in range(TIMED):
             g.replay()
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / (10 * reps)
+        return e0.elapsed_time(e1) * 1e-3 / (TIMED * reps)
 
     def ev_replay(g, reps):
-        for _ in range(3):
+        if brief:
+            reps = 1
+        for _ in range(WARM):
             g.replay()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -338,7 +344,7 @@ def main():
     shapes = synth.QWEN3_4B_LAYER
     stream = torch.cuda.current_stream()
     if args.side_only:
-        print(json.dumps({"side_only": True, "prefill_and_moe": side_workloads(torch, ql, synth, gen)}))
+        print(json.dumps({"side_only": True, "prefill_and_moe": side_workloads(torch, ql, synth, gen, brief=args.brief)}))
         return
 
     def make_pool(wtype, layers):

@@ -114,7 +114,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
   auto store_stage = [&](int buf) {
     unsigned char* st = smem + buf * KX_STAGE;
 #pragma unroll
-    for (int i = 0; i < 2; i++) *reinterpret_cast<u32x4*>(st + ((tid >> 4) + 16 * i) * KX_LDC + (tid & 15) * 16) = gc[i];
+    for (int i = 0; i < 2; i++) {
+      // Q6_K reads this stage (and its patch) 8 bytes per lane: rows r and r + 16 would meet in the same banks, so rows 16..31
+      // keep the two halves of every 16-byte piece swapped (the reads swap them back by address)
+      const u32x4 v = (!K4 && i == 1) ? u32x4{gc[i].z, gc[i].w, gc[i].x, gc[i].y} : gc[i];
+      *reinterpret_cast<u32x4*>(st + ((tid >> 4) + 16 * i) * KX_LDC + (tid & 15) * 16) = v;
+    }
     if (tid < 64) {
       // int16 sums (at most 16 * 128 in magnitude) as fp16 integers: exact
       const uint32_t w[4] = {gb.x, gb.y, gb.z, gb.w};
@@ -254,9 +259,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           const uint32_t srec[4] = {ws[w][j].x, ws[w][j].y, ws[w][j].z, ws[w][j].w};
           const uint32_t dd = wd[w][j];
 #pragma unroll
-          for (int i = 0; i < 4; i++) *reinterpret_cast<u32x4*>(patch + (8 * i + lr) * KX6_WROW + lc * 16) = wq[w][j][i];
+          for (int i = 0; i < 4; i++) {
+            const u32x4 v = i >= 2 ? u32x4{wq[w][j][i].z, wq[w][j][i].w, wq[w][j][i].x, wq[w][j][i].y} : wq[w][j][i];
+            *reinterpret_cast<u32x4*>(patch + (8 * i + lr) * KX6_WROW + lc * 16) = v;
+          }
 #pragma unroll
-          for (int i = 0; i < 2; i++) *reinterpret_cast<u32x4*>(patch + (16 * i + (lane >> 2)) * KX6_WROW + 128 + (lane & 3) * 16) = wh[w][j][i];
+          for (int i = 0; i < 2; i++) {
+            const u32x4 v = i == 1 ? u32x4{wh[w][j][i].z, wh[w][j][i].w, wh[w][j][i].x, wh[w][j][i].y} : wh[w][j][i];
+            *reinterpret_cast<u32x4*>(patch + (16 * i + (lane >> 2)) * KX6_WROW + 128 + (lane & 3) * 16) = v;
+          }
+          const int hs = hi ^ (c32 >> 4);  // which half of a 16-byte piece holds this lane's eight bytes
 #pragma unroll
           for (int i = 0; i < 4; i++) load_chunk(w, j, i, sb + 1);
 #pragma unroll
@@ -267,10 +279,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
           for (int h = 0; h < 2; h++)
 #pragma unroll
             for (int par = 0; par < 2; par++) {
-              const u32x2 QH = *reinterpret_cast<const u32x2*>(patch + c32 * KX6_WROW + 128 + 32 * h + 16 * par + 8 * hi);
+              const u32x2 QH = *reinterpret_cast<const u32x2*>(patch + c32 * KX6_WROW + 128 + 32 * h + 16 * par + 8 * hs);
 #pragma unroll
               for (int ql01 = 0; ql01 < 2; ql01++) {
-                const u32x2 QL = *reinterpret_cast<const u32x2*>(patch + c32 * KX6_WROW + 64 * h + 32 * ql01 + 16 * par + 8 * hi);
+                const u32x2 QL = *reinterpret_cast<const u32x2*>(patch + c32 * KX6_WROW + 64 * h + 32 * ql01 + 16 * par + 8 * hs);
 #pragma unroll
                 for (int nib = 0; nib < 2; nib++) {
                   const int qd = 2 * nib + ql01, g = 8 * h + 2 * qd + par;
@@ -282,7 +294,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
                     b[d2] = (hs & 0x30303030u) | lbits;
                   }
                   const long B = (long)(((unsigned long)b[1] << 32) | b[0]);
-                  const long A = *reinterpret_cast<const long*>(st + c32 * KX_LDC + 16 * g + 8 * hi);
+                  const long A = *reinterpret_cast<const long*>(st + c32 * KX_LDC + 16 * g + 8 * hs);
                   const kx16i T = __builtin_amdgcn_mfma_i32_32x32x16_i8(A, B, zi, 0, 0, 0);
                   const int sc = (int)(int8_t)(srec[g >> 2] >> (8 * (g & 3)));
 #pragma unroll
