@@ -41,8 +41,8 @@ __device__ __forceinline__ void pair_quantize(const float (&v)[16], bool ok, int
   for (int e = 0; e < 16; e++) amax = fmaxf(amax, fabsf(v[e]));
   amax = ok ? amax : 0.f;  // with amax = 0 the inverse scale is 0 and every code comes out 0, whatever v holds
   amax = fmaxf(amax, dpp_f<0xB1>(amax));
-  const float d = amax / 127.f;
-  const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
+  float d, idv;
+  q8_scales(amax, d, idv);
   codes = u32x4{q8_pack4(&v[0], idv), q8_pack4(&v[4], idv), q8_pack4(&v[8], idv), q8_pack4(&v[12], idv)};
   int sum = __builtin_amdgcn_sdot4((int)codes.x, 0x01010101, 0, false);
   sum = __builtin_amdgcn_sdot4((int)codes.y, 0x01010101, sum, false);

@@ -37,8 +37,8 @@ __device__ __forceinline__ void quad_quantize(const float (&v)[8], int x86, uint
   for (int e = 0; e < 8; e++) amax = fmaxf(amax, fabsf(v[e]));
   amax = fmaxf(amax, dpp_f<0xB1>(amax));
   amax = fmaxf(amax, dpp_f<0x4E>(amax));
-  const float d = amax / 127.f;
-  const float idv = (amax != 0.f) ? 127.f / amax : 0.f;
+  float d, idv;
+  q8_scales(amax, d, idv);
   pk[0] = q8_pack4(&v[0], idv);  // |v| <= amax: within -127 .. 127, the reference's saturation never acts
   pk[1] = q8_pack4(&v[4], idv);
   int sum = __builtin_amdgcn_sdot4((int)pk[0], 0x01010101, 0, false);
