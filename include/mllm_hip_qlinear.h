@@ -184,6 +184,13 @@ int mllm_hip_q_block_isums(int wtype, const void* packed, const int8_t* codes, i
  * dst is NULL.  Used to calibrate HBM traffic counters and to measure the fixed cost of a launch of a given size. */
 int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream);
 
+/* Parity probe for the two divisions of quantize_row_q8_0 (d = amax / 127, id = 127 / amax,
+ * mllm/backends/cpu/kernels/common/ggml/quantize/quantize_q8.cpp:106-190): the kernels for three to eight activation rows
+ * form them from short sequences; this runs those sequences on every fp32 bit pattern in [first_bits, last_bits] taken as
+ * amax and ADDS to *mismatches (device memory, 8 bytes, set to zero by the caller) the number of patterns on which either
+ * result differs from IEEE division.  Zero over 0 .. 0x7fffffff. */
+int mllm_hip_probe_q8_scales(uint32_t first_bits, uint32_t last_bits, unsigned long long* mismatches, void* stream);
+
 /* GEMV launch-shape override for tuning sweeps: lanes per weight row (8/16/32/64), rows per lane group (1/2/4; the
  * three- to eight-row kernel with K slices as workgroups reads it as: 1 = keep rows of up to 128 blocks whole, 2 = always cut
  * them; the result bits are the same either way), waves per workgroup (1..16; that kernel takes 3..8); 0 restores the

@@ -101,6 +101,7 @@ def lib():
         L.mllm_hip_q_dequantize.argtypes = [ci, vp, vp, i64, i64, vp]
         L.mllm_hip_q_block_isums.argtypes = [ci, vp, vp, vp, i64, i64, i64, vp]
         L.mllm_hip_probe_copy.argtypes = [vp, vp, C.c_size_t, vp]
+        L.mllm_hip_probe_q8_scales.argtypes = [C.c_uint32, C.c_uint32, vp, vp]
         L.mllm_hip_gemv_set_tuning.argtypes = [ci, ci, ci]
         L.mllm_hip_per_token_quant_int8.argtypes = [vp, ci, vp, vp, i64, i64, vp]
         L.mllm_hip_w8a8_gemm.argtypes = [vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, vp]

@@ -325,6 +325,28 @@ MLLM_API int mllm_hip_gemv_workspace_stats(int device, int* owned, int* capacity
   return 0;
 }
 
+// every fp32 bit pattern in [first, last] as amax: the scale and inverse scale of q8_scales against IEEE division
+__global__ void probe_q8_scales_kernel(uint32_t first, uint32_t last, unsigned long long* mismatches) {
+  unsigned long long bad = 0;
+  const uint64_t step = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t b = (uint64_t)first + (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; b <= last; b += step) {
+    const float amax = __uint_as_float((uint32_t)b);
+    float d, id;
+    q8_scales(amax, d, id);
+    const float dref = amax / 127.f, iref = (amax != 0.f) ? 127.f / amax : 0.f;
+    // (a NaN has no single pattern: both sides NaN counts as equal)
+    bad += !((__float_as_uint(d) == __float_as_uint(dref) || (d != d && dref != dref)) &&
+             (__float_as_uint(id) == __float_as_uint(iref) || (id != id && iref != iref)));
+  }
+  if (bad) atomicAdd(mismatches, bad);
+}
+
+MLLM_API int mllm_hip_probe_q8_scales(uint32_t first_bits, uint32_t last_bits, unsigned long long* mismatches, void* stream) {
+  if (!mismatches || first_bits > last_bits) return MLLM_HIP_E_BADARG;
+  hipLaunchKernelGGL(probe_q8_scales_kernel, dim3(4096), dim3(256), 0, (hipStream_t)stream, first_bits, last_bits, mismatches);
+  return (int)hipGetLastError();
+}
+
 MLLM_API int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void* stream) {
   if (!src || bytes == 0 || bytes % 16) return MLLM_HIP_E_BADARG;
   if (bytes >= ((size_t)1 << 32)) return MLLM_HIP_E_SHAPE;

@@ -668,3 +668,18 @@ def test_weight_quantizer_bit_exact_and_round_trip(wtype, golden_dir):
     L = _lib.lib()
     assert L.mllm_hip_quantize_weight_blocks(wtype, None, blocks.data_ptr(), 0, 4, 64, None) == -1
     assert L.mllm_hip_quantize_weight_blocks(wtype, blocks.data_ptr(), blocks.data_ptr(), 0, 4, 48, None) == -2
+
+
+def test_q8_scale_divisions_equal_ieee_division_for_every_amax():
+    """The kernels for three to eight rows form d = amax / 127 and id = 127 / amax from short sequences (a multiply by
+    RN(1/127) or v_rcp_f32, one residual, one correction; a wave with an amax outside [2^-100, 2^100] takes the compiler's
+    division).  Every fp32 bit pattern from +0 through the positive finite numbers, +inf and the positive NaNs, taken as
+    amax, must give the bits of IEEE division (amax is a maximum of magnitudes: never negative)."""
+    L = _lib.lib()
+    bad = torch.zeros(1, dtype=torch.int64, device="cuda")
+    announce("q8 scale divisions, all non-negative bit patterns")
+    for first, last in ((0x00000000, 0x3fffffff), (0x40000000, 0x7fffffff)):
+        _lib.check(L.mllm_hip_probe_q8_scales(first, last, bad.data_ptr(), None), "mllm_hip_probe_q8_scales")
+    torch.cuda.synchronize()
+    assert int(bad.item()) == 0
+    assert L.mllm_hip_probe_q8_scales(5, 4, bad.data_ptr(), None) == -1  # an empty range is refused
