@@ -65,13 +65,21 @@ struct MfkArgs {
   int col0[GEMV_MAX_PARTS];  // first column of each part within a partial row
   int gx, groups;            // groups > 1 (row groups of eight): a 1-D grid over (workgroup column < gx, slice, group), see the kernel
   int ipr_magic;             // ceil(2^20 / (2 nbs)): item / (items per row) as a multiply and a shift
+  int cstride;               // counters from column to column: up to 32 (a cache line each) where the block has room, so that
+                             // the arrivals of different columns do not queue on one line
 };
+
+// A wave's table of weight scales in LDS: fp32 [block of the slice][16 rows], with eight floats of padding after every eight
+// blocks.  A lane writes the eight scales of one 16-byte piece (blocks 8 cc .. 8 cc + 7 of row r); without the padding the
+// pieces of a row lie 128 dwords apart and all lanes of a row hit one bank (8 or 16 lanes per bank and instruction).
+__host__ __device__ inline int mfk_ws_index(int lb) { return lb * 16 + (lb >> 3) * 8; }
+__host__ __device__ inline int mfk_ws_floats(int nbs) { return nbs * 16 + (nbs + 7) / 8 * 8; }
 
 template <int MT>
 static size_t mfk_lds_bytes(int wtype, int nbs, int nwaves) {
   const int rs = mf_row_stride(nbs);
   return ((size_t)2 * MT * rs + nbs) * 16 + (size_t)MT * nbs * 8 +
-         (size_t)nwaves * ((size_t)nbs * 64 + (size_t)MFK_STG * 16 * (wtype == MLLM_HIP_Q8_0 ? 2 : 1)) + 16;
+         (size_t)nwaves * ((size_t)mfk_ws_floats(nbs) * 4 + (size_t)MFK_STG * 16 * (wtype == MLLM_HIP_Q8_0 ? 2 : 1)) + 16;
 }
 
 // blockDim = 64 x (row tiles per workgroup): three to eight waves, at least nbs / 16 (the threads hold one pass of
@@ -113,7 +121,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   const int aM = GR ? min(a.M - rg * MT, MT) : a.M, x86 = a.x86_scale;
   const int kNP = k.NP;
   float* const kpart = k.part + (size_t)rg * S * MT * kNP;
-  unsigned* const kcnt = k.counters + rg * gx;
+  unsigned* const kcnt = k.counters + (size_t)rg * gx * k.cstride;  // (column bx: kcnt[bx * k.cstride])
   const int N = pt.N;
   float* const ybase = pt.y + (int64_t)rg * MT * N;
   const float* const rbase = pt.residual ? pt.residual + (int64_t)rg * MT * N : nullptr;
@@ -128,8 +136,8 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   u32x4* zrow = xhi + (size_t)MT * rs;          // [nbs] zeros: the operand of the lane groups that must not contribute
   u32x2* xs = reinterpret_cast<u32x2*>(zrow + nbs);  // [MT][nbs] {effective scale, -8 * sum of the codes (Q8_0: 0)}
   float* ws_all = reinterpret_cast<float*>(xs + (size_t)MT * nbs);
-  float* ws = ws_all + (size_t)wave * nbs * 16;  // per wave [block][16 rows]
-  u32x4* stg_all = reinterpret_cast<u32x4*>(ws_all + (size_t)nwaves * nbs * 16);
+  float* ws = ws_all + (size_t)wave * mfk_ws_floats(nbs);  // per wave [block][16 rows], padded: mfk_ws_index
+  u32x4* stg_all = reinterpret_cast<u32x4*>(ws_all + (size_t)nwaves * mfk_ws_floats(nbs));
   u32x4* stg = stg_all + (size_t)wave * MFK_STG * NPL;
   int* s_flag = reinterpret_cast<int*>(stg_all + (size_t)nwaves * MFK_STG * NPL);
 
@@ -260,7 +268,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
       const uint32_t wds[4] = {sc[i].x, sc[i].y, sc[i].z, sc[i].w};
 #pragma unroll
       for (int e = 0; e < 8; e++)
-        ws[(8 * cc + e) * 16 + r] = (b0 + 8 * cc + e < nb) ? f16bits_to_f32((uint16_t)(wds[e >> 1] >> (16 * (e & 1)))) : 0.f;
+        ws[mfk_ws_index(8 * cc + e) + r] = (b0 + 8 * cc + e < nb) ? f16bits_to_f32((uint16_t)(wds[e >> 1] >> (16 * (e & 1)))) : 0.f;
     }
   }
   __syncthreads();
@@ -326,7 +334,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
       const int lb = cb - b0 + 4 * jj + q;  // this lane's block within the slice (inside the slice's LDS rows even when dead)
 #pragma unroll
       for (int p = 0; p < NPL; p++) Aw[jj][p] = stg[p * MFK_STG + c * 9 + 4 * jj + g];
-      dw[jj] = *reinterpret_cast<const f32x4*>(ws + lb * 16 + 4 * g);
+      dw[jj] = *reinterpret_cast<const f32x4*>(ws + mfk_ws_index(lb) + 4 * g);
 #pragma unroll
       for (int h = 0; h < TH; h++) {
         const int m = 4 * h + tt;
@@ -450,10 +458,10 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
   __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (b)
   __syncthreads();                                       // (c)
   if (tid == 0) {
-    const unsigned old = __hip_atomic_fetch_add(kcnt + bx, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (d)
+    const unsigned old = __hip_atomic_fetch_add(kcnt + bx * k.cstride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (d)
     const int last = old == (unsigned)(S - 1);
     // every slice has arrived: ready for the next launch
-    if (last) __hip_atomic_store(kcnt + bx, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (last) __hip_atomic_store(kcnt + bx * k.cstride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     *s_flag = last;
   }
   __syncthreads();  // (e)

@@ -236,6 +236,11 @@ int launch_gemv_mfk(int wtype, int x_kind, int MT, const GemvArgs& a_in, const v
     if (!workspace || !part || (size_t)groups * k.S * MT * np * 4 > part_bytes || (size_t)grid * groups > (size_t)MFK_COUNTERS) return MFK_NOT_TAKEN;
     RC_RET(mfk_counter_block(workspace, st, &k.counters));
     k.part = static_cast<float*>(part);
+    // the columns' counters up to a cache line apart where the block has room: the workgroups of different columns arrive at
+    // about the same time, and arrivals on one line queue behind each other (the step of the 4B layers at four rows
+    // 1.078 -> 1.002 ms, at eight 1.351 -> 1.281; a block four times the size, a line per counter throughout: no further gain)
+    k.cstride = 1;
+    while (k.cstride < 32 && (size_t)grid * groups * k.cstride * 2 <= (size_t)MFK_COUNTERS) k.cstride *= 2;
   }
 #define MFK_CASE(WT_, XT_)                                                         \
   if (wtype == WT_ && x_kind == XT_)                                               \

@@ -116,6 +116,8 @@ int launch_gemv_mr(int wtype, const GemvArgs& a_in, const void* workspace, void*
     if (!workspace || !part || (size_t)k.groups * k.S * MT * np * 4 > part_bytes || (size_t)grid * k.groups > 1024) return MFK_NOT_TAKEN;
     if (!dry) RC_RET(gemv_counter_block(workspace, st, &k.counters));
     k.part = static_cast<float*>(part);
+    k.cstride = 1;  // the columns' counters up to a cache line apart where the block of 1024 has room (see the K-slice kernel)
+    while (k.cstride < 32 && (size_t)grid * k.groups * k.cstride * 2 <= 1024) k.cstride *= 2;
   }
   if (dry) return (wtype == MLLM_HIP_Q4_0 || wtype == MLLM_HIP_Q8_0) ? 0 : MLLM_HIP_E_BADARG;
   if (wtype == MLLM_HIP_Q4_0) return AG == 1 ? launch_mr_t<MLLM_HIP_Q4_0, 1>(a, k, nwaves, st) : launch_mr_t<MLLM_HIP_Q4_0, 2>(a, k, nwaves, st);

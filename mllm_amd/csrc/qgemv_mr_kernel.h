@@ -24,7 +24,8 @@ typedef int64_t mr_i64;
 
 struct MrArgs {
   float* part;         // [row groups][S][MT][NP] partial sums (S > 1)
-  unsigned* counters;  // one per (workgroup column, row group), zero between launches (S > 1)
+  unsigned* counters;  // one per (workgroup column, row group), zero between launches (S > 1), cstride counters apart
+  int cstride;
   int NP;              // columns of a partial row: every part's rows rounded up to 16
   int S, nbs;          // K slices; blocks per slice (a multiple of 8, at most MR_MAX_NBS)
   int col0[GEMV_MAX_PARTS];
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(512) void gemv_mr_kernel(GemvArgs a, MrArgs k) {
   const int m0 = rg * MT;                       // first activation row of this group
   const int aM = min(a.M - m0, MT);             // its valid rows (the image is zero past a.M)
   float* const kpart = k.part + (size_t)rg * S * MT * kNP;
-  unsigned* const kcnt = k.counters + rg * gx;
+  unsigned* const kcnt = k.counters + (size_t)rg * gx * k.cstride;
   float* const ybase = pt.y + (int64_t)m0 * N;
   const float* const rbase = pt.residual ? pt.residual + (int64_t)m0 * N : nullptr;
   const int tile = (bx - wg0) * nwaves + wave;
@@ -281,9 +282,9 @@ __global__ __launch_bounds__(512) void gemv_mr_kernel(GemvArgs a, MrArgs k) {
   __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (b)
   __syncthreads();                                       // (c)
   if (tid == 0) {
-    const unsigned old = __hip_atomic_fetch_add(kcnt + bx, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (d)
+    const unsigned old = __hip_atomic_fetch_add(kcnt + bx * k.cstride, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (d)
     const int last = old == (unsigned)(S - 1);
-    if (last) __hip_atomic_store(kcnt + bx, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+    if (last) __hip_atomic_store(kcnt + bx * k.cstride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
     *s_flag = last;
   }
   __syncthreads();  // (e)
