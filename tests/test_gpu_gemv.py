@@ -536,6 +536,37 @@ def test_gemv_k_slices_as_workgroups_give_the_same_bits(wtype, M):
     assert L.mllm_hip_gemv_splitk_workspace_bytes(0, 96, 100) == 0
 
 
+@pytest.mark.parametrize("wtype", [0, 1])
+def test_gemv_k_slices_share_a_workspace_across_launch_shapes(wtype):
+    """The columns' arrival counters of a launch lie up to a cache line apart inside the workspace's block of counters, the
+    distance depending on how many columns the launch has: launches of different shapes on ONE workspace (32 columns: a
+    line per counter; hundreds of columns and several row groups: neighbouring counters) must find every counter at zero
+    whatever the launch before used.  Three rounds over the shapes, eight and 24 rows, each output equal bit for bit to the
+    form that keeps the slices in one workgroup (eight rows) or to the same call on a workspace of its own (24 rows)."""
+    rng = synth.rng_for(1, 977 + wtype)
+    L = _lib.lib()
+    shapes = [(2560, 9728), (6144, 2560), (100, 161 * 32), (9000, 4096)]
+    Ws = [ql.PackedQWeight(wtype, torch.from_numpy(synth.make_weight(rng, wtype, n, k))) for n, k in shapes]
+    for M in (8, 24):
+        xs = [bf16_dev(synth.fp32_to_bf16_bits(synth.make_x_fp32(rng, M, k))) for _, k in shapes]
+        shared = ql.gemv_workspace(M, max(k for _, k in shapes), max(n for n, _ in shapes))
+        refs = []
+        for w, x, (n, k) in zip(Ws, xs, shapes):
+            own = ql.gemv_workspace(M, k, n)
+            if M <= 8:
+                assert L.mllm_hip_gemv_set_path(2) == 0
+            try:
+                refs.append(ql.linear_q_gemv_multi([w], x, None, ql.SCALE_X86_REF, workspace=own)[0])
+            finally:
+                assert L.mllm_hip_gemv_set_path(0) == 0
+        announce("gemv k slices, one workspace, several launch shapes", wtype, M)
+        for rnd in range(3):
+            for w, x, ref in zip(Ws, xs, refs):
+                y = torch.full_like(ref, float("nan"))
+                ql.linear_q_gemv_multi([w], x, None, ql.SCALE_X86_REF, outs=[y], workspace=shared)
+                assert torch.equal(y, ref)
+
+
 def _counter_stats():
     import ctypes as C
     owned, cap = C.c_int(), C.c_int()
