@@ -9,8 +9,8 @@
 //     that is 320 blocks per workgroup instead of 2432, and the LDS footprint no longer grows with K;
 //   * a launch with enough row tiles to fill the chip by themselves keeps rows of up to 128 blocks whole (one slice, no
 //     partial sums): the workgroup then sums the row in the chains the slices would have been and adds them in slice order;
-//   * weight codes stream through a ring of MFK_CH chunk slots per wave: a slot is requested again as soon as its chunk has
-//     been staged, so a slice of any length keeps MFK_CH chunks of loads ahead of the arithmetic;
+//   * weight codes stream through a ring of chunk slots per wave (mfk_ring): a slot is requested again as soon as its chunk has
+//     been staged, so a slice of any length keeps that many chunks of loads ahead of the arithmetic;
 //   * weight codes are requested as 8 rows x 128 contiguous bytes per load instruction (the operand layout of the MFMA,
 //     16 rows x 64 bytes per instruction, measured 25 % slower on the 4B shapes) and turned into the operand layout
 //     through a 2 KB LDS stage that belongs to the wave (no barrier: LDS operations of one wave execute in order);
@@ -25,8 +25,14 @@
 
 namespace mllmhip {
 
-constexpr int MFK_CH = 4;             // chunks of 8 blocks in flight per wave (a trip = one turn of the ring)
-constexpr int MFK_TRIP = 8 * MFK_CH;
+// chunks of 8 blocks in flight per wave (a trip = one turn of the ring).  Measured on the 4B decode shapes (ms per step of 36
+// layers at 3 / 4 / 8 rows, one row group; at 16 rows, two groups): four slots 0.999 / 1.001 / 1.280 and 1.765, three
+// 0.972 / 0.975 / 1.264 and 1.773, two 0.979 / 0.984 / 1.297 and 1.746 (six and more were slower before that): what a launch
+// asks for at its start delays the activations that every workgroup needs first.
+// (Q8_0, two planes of codes per chunk: 1.265 / 1.509 -> 1.214 / 1.433 at four / eight rows with three slots, 2.075 -> 1.875 at 16
+// rows with two; Q4_0 with several row groups is no faster with fewer than four.)
+constexpr int mfk_ring(int wtype, bool groups) { return groups ? (wtype == MLLM_HIP_Q8_0 ? 2 : 4) : 3; }
+constexpr int MR_CH = 2;  // the many-row kernel (qgemv_mr_kernel.h)
 constexpr int MFK_STG = 16 * 9;       // 16-byte pieces of one stage: 16 rows, stride 9 (reads of 16 rows hit 16 bank groups)
 constexpr int MFK_MAX_NBS = 128;      // blocks per slice (weight scales of a slice: four 16-byte loads per lane)
 
@@ -199,7 +205,8 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
 
   // ---- 3. weight codes of a trip: chunk ch = 8 blocks, instruction i of it = rows 8 i .. 8 i + 7, 128 bytes of each --------
   const int lr = lane >> 3, lp = lane & 7;
-  u32x4 wq[MFK_CH][2][NPL];
+  constexpr int CH = mfk_ring(WT, GR), TRIP = 8 * CH;
+  u32x4 wq[CH][2][NPL];
   auto load_chunk = [&](int ch, int cb) {  // chunk slot ch <- the eight blocks from cb on (nothing is fetched past the slice)
 #pragma unroll
     for (int i = 0; i < 2; i++) {
@@ -210,7 +217,7 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
     }
   };
 #pragma unroll
-  for (int ch = 0; ch < MFK_CH; ch++) load_chunk(ch, b0 + 8 * ch);
+  for (int ch = 0; ch < CH; ch++) load_chunk(ch, b0 + 8 * ch);
   __asm__ volatile("" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
@@ -323,9 +330,9 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
       for (int p = 0; p < NPL; p++) {
         stg[p * MFK_STG + (8 * i + lr) * 9 + lp] = wq[ch][i][p];
       }
-    // the slot is free: the same chunk of the next trip takes it, MFK_CH chunks ahead of the arithmetic (past the slice the
+    // the slot is free: the same chunk of the next trip takes it, CH chunks ahead of the arithmetic (past the slice the
     // offsets are out of range and nothing is fetched)
-    if (refill) load_chunk(ch, cb + MFK_TRIP);
+    if (refill) load_chunk(ch, cb + TRIP);
     u32x4 Aw[2][NPL], Bl[2][TH], Bh[2][TH];
     u32x2 sx[2][TH];
     f32x4 dw[2];
@@ -378,12 +385,12 @@ __global__ __launch_bounds__(512) void gemv_mfk_kernel(GemvArgs a, MfkArgs k) {
       }
   };
   int cb0 = b0;
-  for (; cb0 + MFK_TRIP <= b1r; cb0 += MFK_TRIP) {
+  for (; cb0 + TRIP <= b1r; cb0 += TRIP) {
 #pragma unroll
-    for (int ch = 0; ch < MFK_CH; ch++) chunk(ch, cb0 + 8 * ch, true);
+    for (int ch = 0; ch < CH; ch++) chunk(ch, cb0 + 8 * ch, true);
   }
 #pragma unroll
-  for (int ch = 0; ch < MFK_CH - 1; ch++)
+  for (int ch = 0; ch < CH - 1; ch++)
     if (cb0 + 8 * ch < we) chunk(ch, cb0 + 8 * ch, false);  // uniform
   across_lanes();
   if (have_tot) {

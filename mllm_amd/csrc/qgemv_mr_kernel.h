@@ -130,7 +130,7 @@ __global__ __launch_bounds__(512) void gemv_mr_kernel(GemvArgs a, MrArgs k) {
   __builtin_amdgcn_sched_barrier(0);
   // ---- 3. weight codes: the ring's first turn (chunk = 8 blocks; instruction i of it = rows 8 i .. 8 i + 7, 128 bytes of each) ----
   const int lr = lane >> 3, lp = lane & 7;
-  u32x4 wq[MFK_CH][2][NPL];
+  u32x4 wq[MR_CH][2][NPL];
   auto load_chunk = [&](int ch, int cb) {
 #pragma unroll
     for (int i = 0; i < 2; i++) {
@@ -141,7 +141,7 @@ __global__ __launch_bounds__(512) void gemv_mr_kernel(GemvArgs a, MrArgs k) {
     }
   };
 #pragma unroll
-  for (int ch = 0; ch < MFK_CH; ch++) load_chunk(ch, b0 + 8 * ch);
+  for (int ch = 0; ch < MR_CH; ch++) load_chunk(ch, b0 + 8 * ch);
   __asm__ volatile("" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(512) void gemv_mr_kernel(GemvArgs a, MrArgs k) {
     for (int i = 0; i < 2; i++)
 #pragma unroll
       for (int p = 0; p < NPL; p++) stg[p * MFK_STG + (8 * i + lr) * 9 + lp] = wq[ch][i][p];
-    if (refill) load_chunk(ch, cb + MFK_TRIP);
+    if (refill) load_chunk(ch, cb + (8 * MR_CH));
 #pragma unroll
     for (int jb = 0; jb < 8; jb++) {
       const int lb = cb - b0 + jb;  // block within the slice (inside the slice's LDS rows even when past the row: zero scales)
@@ -218,12 +218,12 @@ __global__ __launch_bounds__(512) void gemv_mr_kernel(GemvArgs a, MrArgs k) {
     }
   };
   int cb0 = b0;
-  for (; cb0 + MFK_TRIP <= b1r; cb0 += MFK_TRIP) {
+  for (; cb0 + (8 * MR_CH) <= b1r; cb0 += (8 * MR_CH)) {
 #pragma unroll
-    for (int ch = 0; ch < MFK_CH; ch++) chunk(ch, cb0 + 8 * ch, true);
+    for (int ch = 0; ch < MR_CH; ch++) chunk(ch, cb0 + 8 * ch, true);
   }
 #pragma unroll
-  for (int ch = 0; ch < MFK_CH - 1; ch++)
+  for (int ch = 0; ch < MR_CH - 1; ch++)
     if (cb0 + 8 * ch < we) chunk(ch, cb0 + 8 * ch, false);  // uniform
 
   // lane: activation rows 16 h + c, weight rows n .. n + 3
