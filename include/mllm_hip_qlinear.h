@@ -200,6 +200,11 @@ int mllm_hip_gemv_set_tuning(int lanes_per_row, int rows_per_group, int waves_pe
  * them); path = 1 keeps every launch on the vector-ALU kernel, path = 2 keeps the K slices of a row tile in one workgroup
  * (comparison runs), 0 restores the default. */
 int mllm_hip_gemv_set_path(int path);
+/* One or two rows: the kernel asks for the first block column of its weights at once and for the others of its first trip
+ * behind the quantization of x (what all workgroups of a launch ask for at their start delays the activations each of
+ * them needs first).  mode = -1: launches of 8 MB (Q8_0: 14 MB) and more with rows of 80 blocks and more, at two rows every
+ * launch with such rows (the default); 0: never; 1: always (comparison runs and tests; the bits are the same). */
+int mllm_hip_gemv_set_request_order(int mode);
 
 /* ---------------------------------------------------------------------------------------------------------
  * Q4_0 / Q8_0 Linear and MoE expert FFN for many rows on the matrix cores

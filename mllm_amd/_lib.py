@@ -63,6 +63,7 @@ def lib():
         L.mllm_hip_mlp_gate_up_q.argtypes = [ci, vp, vp, vp, ci, vp, vp, ci, i64, i64, ci, vp]
         L.mllm_hip_mlp_set_tuning.argtypes = [ci]
         L.mllm_hip_gemv_set_path.argtypes = [ci]
+        L.mllm_hip_gemv_set_request_order.argtypes = [ci]
         L.mllm_hip_kq_set_path.argtypes = [ci]
         L.mllm_hip_moe_kq_set_path.argtypes = [ci]
         L.mllm_hip_rmsnorm.argtypes = [vp, ci, vp, vp, i64, i64, C.c_float, ci, vp, ci, vp]

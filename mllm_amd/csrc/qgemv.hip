@@ -357,6 +357,7 @@ MLLM_API int mllm_hip_probe_copy(void* dst, const void* src, size_t bytes, void*
   return (int)hipGetLastError();
 }
 
+namespace mllmhip { int g_gemv_defer = -1; }
 static int g_gemv_path = 0;
 static int g_gemv_many_rows = 1;  // 0: nine rows and more as groups of eight (comparison runs and tests)
 // 0: by the number of rows; 1: always the vector-ALU kernel; 2: as 0 without the K-slices-as-workgroups form of the
@@ -365,6 +366,12 @@ MLLM_API int mllm_hip_gemv_set_path(int path) {
   if (path != 0 && path != 1 && path != 2 && path != 3) return MLLM_HIP_E_BADARG;
   g_gemv_many_rows = path != 3;  // 3: as 0, nine rows and more as groups of eight rows (the form without the many-row kernel)
   g_gemv_path = path == 3 ? 0 : path;
+  return 0;
+}
+
+MLLM_API int mllm_hip_gemv_set_request_order(int mode) {
+  if (mode < -1 || mode > 1) return MLLM_HIP_E_BADARG;
+  mllmhip::g_gemv_defer = mode;
   return 0;
 }
 

@@ -35,6 +35,7 @@ struct GemvArgs {
   int nbp;        // scale row stride (nb rounded up to 8)
   int x86_scale;  // reproduce the x86 storage rounding of the activation scale
 };
+extern int g_gemv_defer;  // the deferred form of the one- and two-row kernel: -1 by the launch's size (default); 0 / 1: never / always (comparison runs)
 struct GemvShape {
   int G, R, NW;  // lanes per weight row, rows per lane group, waves per workgroup
 };
@@ -95,11 +96,11 @@ __device__ __forceinline__ WRsrc make_wrsrc(const PackedView& w, int wtype, int6
   return r;
 }
 
-template <int WT, int G, int R, int U, bool SCL>
+template <int WT, int G, int R, int U, bool SCL, int ULO = 0, int UHI = U>
 __device__ __forceinline__ void load_chunk(WChunk<WT, R, U, SCL>& c, const WRsrc& w, const uint32_t (&rbase)[R],
                                            const uint32_t (&dbase)[R], int t0, int c0, int nb) {
 #pragma unroll
-  for (int u = 0; u < U; u++) {
+  for (int u = ULO; u < UHI; u++) {
     const int col = t0 + u * G + c0;
 #pragma unroll
     for (int r = 0; r < R; r++) {
@@ -161,7 +162,7 @@ __device__ __forceinline__ void x8_to_f32(const XRaw<XT>& raw, float (&v)[8]) {
 // Register budget: with four or eight activation rows the accumulators and the weights in flight need 140..215
 // registers; the kernels are therefore built for at most eight waves per workgroup (under a 1024-thread bound the
 // compiler has 128 and spills 40..330 bytes per lane).  For one or two rows 16 waves stay possible (long rows).
-template <int WT, int XT, int MT, int G, int R, int U, bool SCL>
+template <int WT, int XT, int MT, int G, int R, int U, bool SCL, bool DEFER = false>
 __global__ __launch_bounds__(MT <= 2 ? 1024 : 512) void gemv_q_kernel(GemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int nb = a.nb, nbp = a.nbp;
@@ -230,7 +231,12 @@ __global__ __launch_bounds__(MT <= 2 ? 1024 : 512) void gemv_q_kernel(GemvArgs a
     dbase[r] = (uint32_t)((row0 + r) * nbp);
   }
   WChunk<WT, R, U, SCL> cur;
-  load_chunk<WT, G, R, U, SCL>(cur, wr, rbase, dbase, 0, c0, nb);
+  // One or two rows: only the first block column of the trip is requested here, the others behind the quantization of x.
+  // Every workgroup of a launch starts within a microsecond and needs its activations first; what all of them ask for at
+  // that moment is in the way of exactly those answers (the step of the 4B layers: 0.698 -> 0.686 ms at one row, 0.981 ->
+  // 0.960 at two; nothing here: 0.745; the others right after the activations have arrived: 0.697; behind the barrier: 0.729).
+  constexpr int UFIRST = DEFER ? 1 : U;
+  load_chunk<WT, G, R, U, SCL, 0, UFIRST>(cur, wr, rbase, dbase, 0, c0, nb);
   __asm__ volatile("" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
@@ -287,6 +293,8 @@ __global__ __launch_bounds__(MT <= 2 ? 1024 : 512) void gemv_q_kernel(GemvArgs a
       if (ch < ROWS_W * cpr) *reinterpret_cast<u32x4*>(s_ws + ch * 8) = sc[k];
     }
   }
+  // the rest of the first trip's weights (see UFIRST above)
+  load_chunk<WT, G, R, U, SCL, UFIRST, U>(cur, wr, rbase, dbase, 0, c0, nb);  // the rest of the first trip's weights (DEFER)
   __syncthreads();
 
   // ---- 5. block dots ------------------------------------------------------------------------------------------------
@@ -367,6 +375,18 @@ static int launch_gemv_u(const GemvArgs& a_in, int NW, hipStream_t st) {
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NW * 64), lds, st, a);
     return (int)hipGetLastError();
   };
+  if constexpr (MT <= 2 && U >= 2) {
+    // Measured per shape (us per launch, all at once -> deferred, one row, Q4_0): 1024 x 2560 3.23 -> 3.39, 2560 x 4096 3.61 -> 3.93,
+    // 4096 x 2560 3.50 -> 3.68, 6144 x 2048 3.57 -> 3.90, 8192 x 2048 3.82 -> 4.08, q+k+v 6144 x 2560 4.15 -> 3.93, 9728 x 2560
+    // 5.19 -> 4.68, 2560 x 9728 5.20 -> 4.80, gate + up 7.00 -> 6.92, 2 x 25600 x 5120 27.7 -> 26.9; Q8_0 wins from q+k+v
+    // (15.9 MB) on.  So: launches of 8 MB (Q8_0: 14 MB) and more with rows of 80 blocks and more.
+    int64_t blocks = 0;
+    for (int p = 0; p < a.nparts; p++) blocks += (int64_t)a.part[p].N * a.nb;
+    // (two rows: every shape with rows of 80 blocks and more wins, 2560 x 4096 5.50 -> 5.22, 4096 x 2560 4.75 -> 4.42)
+    const bool big = a.nb >= 80 && (MT == 2 || blocks * (WT == MLLM_HIP_Q4_0 ? 18 : 34) >= (int64_t)(WT == MLLM_HIP_Q4_0 ? 8 : 14) << 20);
+    if (g_gemv_defer < 0 ? big : g_gemv_defer != 0)
+      return scl ? launch(gemv_q_kernel<WT, XT, MT, G, R, U, true, true>) : launch(gemv_q_kernel<WT, XT, MT, G, R, U, false, true>);
+  }
   return scl ? launch(gemv_q_kernel<WT, XT, MT, G, R, U, true>) : launch(gemv_q_kernel<WT, XT, MT, G, R, U, false>);
 }
 

@@ -444,6 +444,47 @@ def test_gemv_multi_equals_single(wtype, M):
 
 
 @pytest.mark.parametrize("wtype", [0, 1])
+@pytest.mark.parametrize("M", [1, 2])
+def test_gemv_request_order_does_not_change_the_bits(wtype, M):
+    """One or two rows: the kernel that asks for all weights of its first trip at once and the one that asks for all but the
+    first block column behind the quantization of x (the default for large launches) compute the same sums in the same
+    order: equal bit for bit, whichever the size rule would pick.  Raw activations (fp32, bf16), both scale modes, bias,
+    sibling matrices, ragged N, rows of one to 304 blocks, and the quantized image as input."""
+    rng = synth.rng_for(1, 430 + M + 10 * wtype)
+    L = _lib.lib()
+    assert L.mllm_hip_gemv_set_request_order(2) == -1 and L.mllm_hip_gemv_set_request_order(-2) == -1
+    for shapes in ([(4096, 2560), (1024, 2560), (1024, 2560)], [(2560, 9728)], [(257, 4096)], [(40, 96), (7, 96), (33, 96)],
+                   [(65, 32)], [(300, 2048), (9, 2048)], [(129, 161 * 32)]):
+        K = shapes[0][1]
+        ws = [ql.PackedQWeight(wtype, torch.from_numpy(synth.make_weight(rng, wtype, n, K))) for n, _ in shapes]
+        biases = [to_dev(rng.standard_normal(n).astype(np.float32)) for n, _ in shapes]
+        x = synth.make_x_fp32(rng, M, K)
+        announce("gemv request order", wtype, M, shapes)
+        for xd in (to_dev(x), bf16_dev(synth.fp32_to_bf16_bits(x))):
+            for mode in (ql.SCALE_X86_REF, ql.SCALE_IEEE):
+                outs = {}
+                for order in (0, 1):
+                    assert L.mllm_hip_gemv_set_request_order(order) == 0
+                    try:
+                        outs[order] = ql.linear_q_gemv_multi(ws, xd, biases, mode)
+                    finally:
+                        assert L.mllm_hip_gemv_set_request_order(-1) == 0
+                for a_, b_ in zip(outs[0], outs[1]):
+                    assert torch.equal(a_, b_)
+        xd = to_dev(x)
+        _, img = ql.add(xd, torch.zeros_like(xd), want_image=True)
+        outs = {}
+        for order in (0, 1):
+            assert L.mllm_hip_gemv_set_request_order(order) == 0
+            try:
+                outs[order] = ql.linear_q_gemv_fused(ws, img, M=M, image=True, biases=biases)
+            finally:
+                assert L.mllm_hip_gemv_set_request_order(-1) == 0
+        for a_, b_ in zip(outs[0], outs[1]):
+            assert torch.equal(a_, b_)
+
+
+@pytest.mark.parametrize("wtype", [0, 1])
 @pytest.mark.parametrize("M", [3, 4, 5, 8])
 def test_gemv_matrix_core_and_vector_kernels_agree(wtype, M):
     """three to eight rows: the matrix-core kernel (default) and the vector-ALU kernel are two independent implementations of
