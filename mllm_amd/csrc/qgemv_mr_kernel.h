@@ -140,8 +140,7 @@ __global__ __launch_bounds__(512) void gemv_mr_kernel(GemvArgs a, MrArgs k) {
       if (WT == MLLM_HIP_Q8_0) wq[ch][i][NPL - 1] = __builtin_amdgcn_raw_buffer_load_b128(wr.q1, off, 0, BUF_NT);
     }
   };
-#pragma unroll
-  for (int ch = 0; ch < MR_CH; ch++) load_chunk(ch, b0 + 8 * ch);
+  load_chunk(0, b0);  // (the other chunks of the ring: behind the image copy, see below)
   __asm__ volatile("" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
@@ -158,6 +157,8 @@ __global__ __launch_bounds__(512) void gemv_mr_kernel(GemvArgs a, MrArgs k) {
       xs[(size_t)m * rx + ib] = u32x2{live ? __float_as_uint(pd[i]) : 0u, (uint32_t)n8};
     }
   }
+#pragma unroll
+  for (int ch = 1; ch < MR_CH; ch++) load_chunk(ch, b0 + 8 * ch);
   // weight scales -> fp32 [block of the slice][row]; blocks past the row are zero
 #pragma unroll
   for (int i = 0; i < 4; i++) {
