@@ -9,6 +9,7 @@
 // any exchange between workgroups.  x comes as activations (quantized here, once per workgroup) or as the image a
 // producer (RMSNorm) wrote.  Same arithmetic as the stand-alone operators: results equal gate/up GEMV -> SiLU -> mul
 // (-> quantization) bit for bit when the GEMV sums a row over the same 16 lanes, and agree to rounding otherwise.
+#include <type_traits>
 #include "qgemv_kernel.h"
 
 namespace mllmhip {
@@ -77,9 +78,9 @@ __global__ __launch_bounds__(32 * G) void mlp_gateup_kernel(MlpArgs a) {
   __builtin_amdgcn_sched_barrier(0);
 
   const uint32_t rbase = (uint32_t)n * (uint32_t)nb, dbase = (uint32_t)n * (uint32_t)nbp;
-  auto load_trip = [&](PairChunk<WT, U, SCL>& c, int t0) {
+  auto load_trip = [&](PairChunk<WT, U, SCL>& c, int t0, auto ulo, auto uhi) {
 #pragma unroll
-    for (int u = 0; u < U; u++) {
+    for (int u = decltype(ulo)::value; u < decltype(uhi)::value; u++) {
       const int col = t0 + G * u + c0;
       const bool ok = col < nb;
 #pragma unroll
@@ -91,8 +92,11 @@ __global__ __launch_bounds__(32 * G) void mlp_gateup_kernel(MlpArgs a) {
       }
     }
   };
+  // (only the first block column of the first trip here, the others behind the quantization of x: what every workgroup of
+  // the launch asks for at its start delays the activations each of them needs first)
   PairChunk<WT, U, SCL> cur;
-  load_trip(cur, 0);
+  constexpr int UFIRST = U >= 2 ? 1 : U;
+  load_trip(cur, 0, std::integral_constant<int, 0>{}, std::integral_constant<int, UFIRST>{});
   __asm__ volatile("" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
@@ -124,6 +128,7 @@ __global__ __launch_bounds__(32 * G) void mlp_gateup_kernel(MlpArgs a) {
     *reinterpret_cast<u32x4*>(s_ws + lane * 8) = sc[0];
     *reinterpret_cast<u32x4*>(s_ws + (GROUPS * cpr + lane) * 8) = sc[1];
   }
+  load_trip(cur, 0, std::integral_constant<int, UFIRST>{}, std::integral_constant<int, U>{});
   __syncthreads();
   const u32x4* s_lo = reinterpret_cast<const u32x4*>(smem);
   const u32x4* s_hi = s_lo + mnb;
@@ -138,7 +143,7 @@ __global__ __launch_bounds__(32 * G) void mlp_gateup_kernel(MlpArgs a) {
   for (int t0 = 0; t0 < nb; t0 += G * U) {
     PairChunk<WT, U, SCL> nxt;
     const bool more = t0 + G * U < nb;  // uniform
-    if (more) load_trip(nxt, t0 + G * U);
+    if (more) load_trip(nxt, t0 + G * U, std::integral_constant<int, 0>{}, std::integral_constant<int, U>{});
 #pragma unroll
     for (int u = 0; u < U; u++) {
       const int col = t0 + G * u + c0;
