@@ -62,6 +62,8 @@ def parse():
                     help="profiling run: only the decoder-layer chain (operators one by one and folded, M = 1 and 8) and the "
                          "Q4_K / Q6_K gate projection, printed as one JSON object; meant to run under rocprofv3")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--request-order", type=int, default=-1, choices=[-1, 0, 1],
+                    help="mllm_hip_gemv_set_request_order: -1 the library's rule (default), 0 / 1 never / always deferred (comparison runs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the M=4/8 and Q8_0 side measurements")
     return ap.parse_args()
@@ -338,6 +340,7 @@ def main():
     from mllm_amd import _lib, qlinear as ql, synth
 
     _lib.check(_lib.lib().mllm_hip_init(0), "mllm_hip_init")
+    _lib.check(_lib.lib().mllm_hip_gemv_set_request_order(args.request_order), "mllm_hip_gemv_set_request_order")
     torch.cuda.set_device(0)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(synth.SEED_BASE + 1)
