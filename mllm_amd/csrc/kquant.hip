@@ -674,6 +674,12 @@ static int launch_kq(const KGemvArgs& a, hipStream_t st) {
 //   acc = fma(fp32(d*sc) * dx, float(isum), acc);  acc = fma(-(fp32(dmin*m) * dx), float(sum of the row's 32 codes), acc)
 // the reference's sum (vec_dot_q4_K_q8_K: integer sums per super-block, then d*dx and dmin*dx) regrouped; the integer parts
 // are exact, the fp32 roundings differ in order only.
+#ifndef KMF_WEIGHTS_FIRST
+#define KMF_WEIGHTS_FIRST 0
+#endif
+#ifndef KMF_COPY_UNROLL
+#define KMF_COPY_UNROLL 5
+#endif
 typedef int kv4i __attribute__((ext_vector_type(4)));
 constexpr int KMF_NG = 10;  // groups of four sub-blocks per trip, at most (the launcher takes 6 or 8 for shorter slices)
 
@@ -752,7 +758,7 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
       wq[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, (row_ok && b < b1) ? (rbase + (uint32_t)b) * 16u : KBUF_OOB, 0, KBUF_NT);
     }
   };
-  load_groups(b0);
+  if (KMF_WEIGHTS_FIRST) load_groups(b0);
   __asm__ volatile("" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
@@ -764,6 +770,7 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
     const float* dd = reinterpret_cast<const float*>(reinterpret_cast<const char*>(a.x) + R * K + R * nsb * 32);
     for (int m = wave; m < MT; m += nwaves) {
       const size_t src = (size_t)kq_tile_in_row(a, mt, m);
+#pragma unroll KMF_COPY_UNROLL
       for (int r = lane; r < 2 * nb32; r += 64) xc[((size_t)(r >> 1) * MT + m) * 2 + (r & 1)] = codes[src * 2 * nb32 + r];
       for (int sb = lane; sb < nb32; sb += 64) {
         const uint32_t pr = pairs[src * nb32 + sb];
@@ -787,6 +794,7 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
       if (part == 0) xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(qi.d), (uint32_t)s32};
     }
   }
+  if (!KMF_WEIGHTS_FIRST) load_groups(b0);
   if (tid == 0) zrec[0] = u32x4{0u, 0u, 0u, 0u};
   for (int i = tid; i < xpad * MT * 2; i += nthreads) xc[(size_t)nb32 * MT * 2 + i] = u32x4{0u, 0u, 0u, 0u};
   for (int i = tid; i < xpad * MT; i += nthreads) xs[(size_t)nb32 * MT + i] = u32x2{0u, 0u};
@@ -1037,7 +1045,7 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
       wh[st] = __builtin_amdgcn_raw_buffer_load_b128(rh, ok ? ((rbase + (uint32_t)sb) * 4u + 2u * (st & 1) + (uint32_t)(g & 1)) * 16u : KBUF_OOB, 0, KBUF_NT);
     }
   };
-  load_steps(s0);
+  if (KMF_WEIGHTS_FIRST) load_steps(s0);
   __asm__ volatile("" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
@@ -1049,6 +1057,7 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
     const float* dd = reinterpret_cast<const float*>(reinterpret_cast<const char*>(a.x) + R * K + R * nsb * 32);
     for (int m = wave; m < MT; m += nwaves) {
       const size_t src = (size_t)kq_tile_in_row(a, mt, m);
+#pragma unroll KMF_COPY_UNROLL
       for (int u = lane; u < nu; u += 64) {
         xc[(size_t)u * MT + m] = codes[src * nu + u];
         bs16[(size_t)u * MT + m] = (int)sums[src * nu + u];
@@ -1071,6 +1080,7 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
       if ((i & 31) == 0) dxs[(i >> 5) * MT + m] = qi.d;
     }
   }
+  if (!KMF_WEIGHTS_FIRST) load_steps(s0);
   if (tid == 0) zrec[0] = u32x4{0u, 0u, 0u, 0u};
   for (int i = tid; i < xpad * 16 * MT; i += nthreads) {
     xc[(size_t)nu * MT + i] = u32x4{0u, 0u, 0u, 0u};
