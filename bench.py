@@ -312,7 +312,7 @@ def side_workloads(torch, ql, synth, gen, brief=False):
         wsk = torch.empty(L.mllm_hip_linear_kq_gemm_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
         tk = ev_time(lambda: ql.linear_kq_gemm(wkg, xx, out=yy, workspace=wsk), 10)
         wkv = ql.PackedKWeight.synthetic(kt, N, K, gen)
-        wsv = ql.kq_workspace(M, K)
+        wsv = ql.kq_workspace(M, K, N)
         tv = ev_time(lambda: ql.linear_kq(wkv, xx, out=yy, workspace=wsv), 3)
         out["%s_linear_prefill_2048x9728x2560" % kname] = {"us": tk * 1e6, "TFLOPS": fl / tk / 1e12, "frac_of_2500_TFLOPS": fl / tk / 2.5e15,
                                                             "path": "matrix cores (mllm_hip_linear_kq_gemm)",
@@ -595,7 +595,7 @@ def main():
             kpool = [{name: ql.PackedKWeight.synthetic(kt, n, k, gen) for name, (n, k) in shapes.items()} for _ in range(N_LAYERS)]
             for M in (1, 8):
                 xs, ys = make_io(M)
-                kws = {k: ql.kq_workspace(M, k) for k in (2560, 4096, 9728)}
+                kws = {k: ql.kq_workspace(M, k, 2 * 9728) for k in (2560, 4096, 9728)}  # (with room for partial sums of K slices)
 
                 def kstep():  # sibling projections share a launch: qkv | o | gate+up | down
                     for l in kpool:

@@ -97,6 +97,10 @@ def lib():
         L.mllm_hip_linear_kq_multi.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, i64, i64, vp, vp]
         L.mllm_hip_kq_workspace_bytes.restype = C.c_size_t
         L.mllm_hip_kq_workspace_bytes.argtypes = [i64, i64]
+        L.mllm_hip_kq_set_slice_meeting.argtypes = [ci, ci]
+        L.mllm_hip_kq_workspace_bytes_n.restype = C.c_size_t
+        L.mllm_hip_kq_workspace_bytes_n.argtypes = [i64, i64, i64]
+        L.mllm_hip_linear_kq_multi_ws.argtypes = [ci, ci, C.POINTER(GemvPart), vp, ci, i64, i64, vp, C.c_size_t, vp]
         L.mllm_hip_kq_dequantize.argtypes = [ci, vp, vp, i64, i64, vp]
         L.mllm_hip_quantize_q8_K.argtypes = [vp, ci, vp, vp, vp, i64, i64, vp]
         L.mllm_hip_q_dequantize.argtypes = [ci, vp, vp, i64, i64, vp]

@@ -348,8 +348,11 @@ void HipLinearOp::forward(const std::vector<Tensor>& inputs, std::vector<Tensor>
         void* ws = workspace(mllm_hip_linear_kq_gemm_short_workspace_bytes(M, N, K));
         MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_kq_gemm_short(wt, gemm_packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K, ws, st));
       } else {
-        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_kq(wt, packed_.ptr<void>(), x.ptr<void>(), xdt(), bias, y.ptr<float>(), M, N, K,
-                                                 M >= 3 ? workspace(mllm_hip_kq_workspace_bytes(M, K)) : nullptr, st));
+        // (from three rows on: room for the quantized image of x and for the partial sums of K slices that meet in memory)
+        const size_t ws_bytes = M >= 3 ? mllm_hip_kq_workspace_bytes_n(M, K, N) : 0;
+        const mllm_hip_gemv_part part{packed_.ptr<void>(), bias, y.ptr<float>(), N};
+        MLLM_HIP_KERNEL_CHECK(mllm_hip_linear_kq_multi_ws(wt, 1, &part, x.ptr<void>(), xdt(), M, K, ws_bytes ? workspace(ws_bytes) : nullptr,
+                                                          ws_bytes, st));
       }
       break;
     }

@@ -697,8 +697,24 @@ static int kmf_slices(int nb32) {
 //      wave of slice 0).
 // NG = groups of four sub-blocks per trip: the slice in one trip where it fits (6, 8 or 10), so that neither registers nor
 // LDS rows are held for sub-blocks the slice does not have -- with K = 2048 three workgroups fit a CU instead of two.
+// K slices spread over workgroups (blockIdx.z = slice group): where they meet.  SG = 1: all slices of a tile in one workgroup.
+struct KMeet {
+  int SG;              // slice groups (= gridDim.z); a workgroup holds slices [z S, z S + S)
+  int lrows;           // sub-blocks a workgroup keeps in LDS: its slices' plus what their last trips reach past them
+  float* part;         // [x column of the grid][wave][slice group][32 lanes] four partial sums
+  unsigned* counters;  // one per x column (cstride counters apart), zero between launches
+  int cstride;
+};
+// host side: what a caller's workspace offers for it (key = the workspace address that owns the counter block)
+struct KMeetRoom {
+  const void* key;
+  void* part;
+  size_t part_bytes;
+};
+int gemv_counter_block(const void* workspace, hipStream_t st, unsigned** out);  // qgemv_mfma.hip
+constexpr int KQ_NOT_TAKEN = 1;  // a launcher's answer when the launch does not suit it (also gemv_counter_block's when no block is free)
 template <int XT, int MT, int NG = KMF_NG>
-__global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, int nbs, int xpad) {
+__global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, int nbs, KMeet km) {
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int TRIP = 4 * NG;
   const int nsb = a.nsb, nb32 = nsb * 8, K = nsb * QK_K;
@@ -714,19 +730,23 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
   const int N = pt.N;
   const int tiles_wg = nwaves / S;
   const int tile = ((int)blockIdx.x - a.wg_start[pidx]) * tiles_wg + wave / S;
-  const int slice = wave % S;
+  const int sg = km.SG > 1 ? (int)blockIdx.z : 0;
+  const int slice = sg * S + wave % S;
   const int row0 = tile * 16;
   const bool tile_ok = row0 < N;
   const int b0 = slice * nbs, b1 = min(nb32, b0 + nbs);
+  const int kb0 = min(nb32, sg * S * nbs), kb1 = min(nb32, kb0 + S * nbs);  // the workgroup's sub-blocks; LDS rows count from kb0
+  const int nloc = kb1 - kb0, lrows = km.lrows;
 
   const int wsb = (nbs + TRIP - 1) / TRIP * TRIP;
-  u32x4* xc = reinterpret_cast<u32x4*>(smem);                        // [(sb * MT + m) * 2 + half]
-  u32x4* zrec = xc + (size_t)(nb32 + xpad) * MT * 2;
-  u32x2* xs = reinterpret_cast<u32x2*>(zrec + 1);                    // [sb * MT + m]
-  float* ws_all = reinterpret_cast<float*>(xs + (size_t)(nb32 + xpad) * MT);
+  u32x4* xc = reinterpret_cast<u32x4*>(smem);                        // [((sb - kb0) * MT + m) * 2 + half]
+  u32x4* zrec = xc + (size_t)lrows * MT * 2;
+  u32x2* xs = reinterpret_cast<u32x2*>(zrec + 1);                    // [(sb - kb0) * MT + m]
+  float* ws_all = reinterpret_cast<float*>(xs + (size_t)lrows * MT);
   float* ws_ds = ws_all + (size_t)wave * 2 * wsb * 16;
   float* ws_dm = ws_ds + (size_t)wsb * 16;
   f32x4* red = reinterpret_cast<f32x4*>(ws_ds);  // the wave's scale table, dead after the loop (2 wsb x 64 bytes >= 1 KB)
+  int* s_flag = reinterpret_cast<int*>(ws_all + (size_t)nwaves * 2 * wsb * 16);
 
   // ---- 1. weight scale records of the tile and slice: one 16-byte record per (row, super-block) --------------------------
   const uint32_t sbt = (uint32_t)N * (uint32_t)nsb;
@@ -771,33 +791,34 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
     for (int m = wave; m < MT; m += nwaves) {
       const size_t src = (size_t)kq_tile_in_row(a, mt, m);
 #pragma unroll KMF_COPY_UNROLL
-      for (int r = lane; r < 2 * nb32; r += 64) xc[((size_t)(r >> 1) * MT + m) * 2 + (r & 1)] = codes[src * 2 * nb32 + r];
-      for (int sb = lane; sb < nb32; sb += 64) {
-        const uint32_t pr = pairs[src * nb32 + sb];
+      for (int r = lane; r < 2 * nloc; r += 64) xc[((size_t)(r >> 1) * MT + m) * 2 + (r & 1)] = codes[(src * nb32 + kb0) * 2 + r];
+      for (int sb = lane; sb < nloc; sb += 64) {
+        const uint32_t pr = pairs[src * nb32 + kb0 + sb];
         const int bsum = (int)(int16_t)(pr & 0xffffu) + (int)(int16_t)(pr >> 16);
-        xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(dd[src * nsb + (sb >> 3)]), (uint32_t)bsum};
+        xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(dd[src * nsb + ((kb0 + sb) >> 3)]), (uint32_t)bsum};
       }
     }
   } else {
-    const int ipr = K >> 3;  // items (eight elements) per row; 32 consecutive items = one super-block
-    const int nitems = MT * ipr, valid = a.M * ipr;
-    const float inv_ipr = 1.0f / (float)ipr;
+    const int ipr = K >> 3;     // items (eight elements) per row; 32 consecutive items = one super-block
+    const int iwg = nloc << 2;  // of them in this workgroup's sub-blocks (whole super-blocks)
+    const int nitems = MT * iwg;
+    const float inv_iwg = 1.0f / (float)iwg;
     for (int it = tid; it < nitems; it += nthreads) {  // whole half-waves: nitems and nthreads are multiples of 32
+      const int m = (int)(((float)it + 0.5f) * inv_iwg), i = it - m * iwg;  // it / iwg: far from rounding trouble
       float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      if (it < valid) load8<XT == KQ_IMAGE ? MLLM_HIP_F32 : XT>(a.x, (int64_t)it * 8, v);
+      if (m < a.M) load8<XT == KQ_IMAGE ? MLLM_HIP_F32 : XT>(a.x, ((int64_t)m * ipr + 4 * kb0 + i) * 8, v);
       const Q8KItem qi = quantize_q8k_item(v, lane);
       int s32 = qi.sum8 + __builtin_amdgcn_update_dpp(0, qi.sum8, 0xB1, 0xf, 0xf, true);
       s32 += __builtin_amdgcn_update_dpp(0, s32, 0x4E, 0xf, 0xf, true);
-      const int m = (int)(((float)it + 0.5f) * inv_ipr), i = it - m * ipr;  // it / ipr: far from rounding trouble
-      const int sb = i >> 2, part = i & 3;                                   // sub-block, which 8 of its 32 codes
+      const int sb = i >> 2, part = i & 3;  // sub-block (from kb0), which 8 of its 32 codes
       reinterpret_cast<u32x2*>(xc + ((size_t)sb * MT + m) * 2 + (part >> 1))[part & 1] = u32x2{qi.q0, qi.q1};
       if (part == 0) xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(qi.d), (uint32_t)s32};
     }
   }
   if (!KMF_WEIGHTS_FIRST) load_groups(b0);
   if (tid == 0) zrec[0] = u32x4{0u, 0u, 0u, 0u};
-  for (int i = tid; i < xpad * MT * 2; i += nthreads) xc[(size_t)nb32 * MT * 2 + i] = u32x4{0u, 0u, 0u, 0u};
-  for (int i = tid; i < xpad * MT; i += nthreads) xs[(size_t)nb32 * MT + i] = u32x2{0u, 0u};
+  for (int i = tid; i < (lrows - nloc) * MT * 2; i += nthreads) xc[(size_t)nloc * MT * 2 + i] = u32x4{0u, 0u, 0u, 0u};
+  for (int i = tid; i < (lrows - nloc) * MT; i += nthreads) xs[(size_t)nloc * MT + i] = u32x2{0u, 0u};
   // weight scales: fp32 d*sc and dmin*m per (sub-block of the slice, row); zero past the row and in the rest of the last trip
 #pragma unroll
   for (int k = 0; k < 2; k++) {
@@ -827,9 +848,9 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
   f32x4 acc = {0.f, 0.f, 0.f, 0.f};
   for (int bb = b0; bb < b1; bb += TRIP) {
     if (bb != b0) load_groups(bb);
-    const u32x4* bl = mine ? xc + ((size_t)(bb + 2 * q2) * MT + tm) * 2 + half : zrec;
+    const u32x4* bl = mine ? xc + ((size_t)(bb - kb0 + 2 * q2) * MT + tm) * 2 + half : zrec;
     const int bstep = mine ? 8 * MT : 0;  // four sub-blocks further per group
-    const u32x2* xsl = xs + (size_t)(bb + 2 * q2) * MT + tm;
+    const u32x2* xsl = xs + (size_t)(bb - kb0 + 2 * q2) * MT + tm;
     const float* dsl = ws_ds + (bb - b0 + 2 * q2) * 16 + 4 * g;
     const float* dml = ws_dm + (bb - b0 + 2 * q2) * 16 + 4 * g;
     u32x4 Bl[2], Bh[2];
@@ -895,10 +916,51 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
   if (S > 1) {
     red[lane] = acc;
     __syncthreads();
-    if (slice != 0) return;
+    if (wave % S != 0) return;
     for (int s = 1; s < S; s++) {
       const f32x4 o = reinterpret_cast<const f32x4*>(ws_ds + (size_t)s * 2 * wsb * 16)[lane];  // the table of wave + s
       acc.x += o.x; acc.y += o.y; acc.z += o.z; acc.w += o.w;
+    }
+  }
+  if (km.SG > 1) {
+    // The slice groups of a grid column meet in global memory (S = 1 here: every wave is a tile).  Ordering, step by step:
+    // partial sums leave with device-scope stores; every wave waits until the memory system has acknowledged its stores
+    // (s_waitcnt vmcnt(0): stores count in vmcnt until acknowledged); the workgroup barrier; thread 0 counts the workgroup
+    // in with a device-scope atomic add; the workgroup that sees the last count reads all partial sums with device-scope
+    // loads issued after a second barrier, and adds them in slice order: the bits of the one-workgroup form.
+    const int SG = km.SG;
+    const int li = 8 * g + t;
+    float* pbase = km.part + (((size_t)blockIdx.x * nwaves + wave) * SG) * 128;
+    if (q2 == 0) {
+      float* dst = pbase + (size_t)sg * 128 + 4 * li;
+      __hip_atomic_store(dst + 0, acc.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(dst + 1, acc.y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(dst + 2, acc.z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(dst + 3, acc.w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+      unsigned* cnt = km.counters + (size_t)blockIdx.x * km.cstride;
+      const unsigned old = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int last = old == (unsigned)(SG - 1);
+      if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+      *s_flag = last;
+    }
+    __syncthreads();
+    if (!*s_flag) return;
+    if (q2 == 0) {  // (at most eight slice groups; their loads are in flight together)
+      float pv[8][4];
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        const float* src = pbase + (size_t)min(u, SG - 1) * 128 + 4 * li;
+#pragma unroll
+        for (int e = 0; e < 4; e++) pv[u][e] = __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      acc = f32x4{pv[0][0], pv[0][1], pv[0][2], pv[0][3]};
+#pragma unroll
+      for (int u = 1; u < 8; u++)
+        if (u < SG) { acc.x += pv[u][0]; acc.y += pv[u][1]; acc.z += pv[u][2]; acc.w += pv[u][3]; }
     }
   }
   if (!tile_ok || q2 != 0 || t >= MT || t >= mt.rows) return;
@@ -925,7 +987,14 @@ template <int MT>
 static size_t kmf_lds_bytes(int nb32, int nbs, int nwaves, int S) {
   const int trip = 4 * kmf_groups(nbs);
   const int wsb = (nbs + trip - 1) / trip * trip, rows = nb32 + kmf_xpad(nb32, S, nbs);
-  return (size_t)rows * MT * 32 + 16 + (size_t)rows * MT * 8 + (size_t)nwaves * 2 * wsb * 64;
+  return (size_t)rows * MT * 32 + 16 + (size_t)rows * MT * 8 + (size_t)nwaves * 2 * wsb * 64 + 16;
+}
+// the same with one slice per workgroup (slice groups over the grid's z): the slice's sub-blocks in whole trips
+template <int MT>
+static size_t kmf_lds_bytes_z(int nbs, int nwaves) {
+  const int trip = 4 * kmf_groups(nbs);
+  const int wsb = (nbs + trip - 1) / trip * trip;
+  return (size_t)wsb * MT * 32 + 16 + (size_t)wsb * MT * 8 + (size_t)nwaves * 2 * wsb * 64 + 16;
 }
 static bool kq4_mfma_fits(int MT, int nsb) {
   const int nb32 = nsb * 8;
@@ -933,6 +1002,63 @@ static bool kq4_mfma_fits(int MT, int nsb) {
   const int S = kmf_slices(nb32);
   const int nbs = ((nb32 + S - 1) / S + 7) / 8 * 8;
   return (MT == 4 ? kmf_lds_bytes<4>(nb32, nbs, 8, S) : kmf_lds_bytes<8>(nb32, nbs, 8, S)) <= 160 * 1024;
+}
+// room for the partial sums of a launch whose slices meet in global memory (0: its slices share a workgroup anyway)
+static size_t kmf_part_bytes(int nsb, int64_t n_total, int nparts) {
+  const int S = kmf_slices(nsb * 8);
+  if (S < 2) return 0;
+  return (size_t)((n_total + 15) / 16 + (int64_t)nparts * 8) * S * 512;
+}
+int g_kq_meet = -1, g_kq_meet_waves = 0, g_kq_meet_min = 4;  // (mllm_hip_kq_set_slice_meeting)
+template <int XT, int MT>
+static int launch_kq4_mfma_z(const KGemvArgs& a_in, const KMeetRoom& room, hipStream_t st) {
+  KGemvArgs a = a_in;
+  const int nb32 = a.nsb * 8;
+  const int SG = kmf_slices(nb32);
+  const int nbs = ((nb32 + SG - 1) / SG + 7) / 8 * 8;
+  // row tiles (= waves) per workgroup: four to six, the first that needs the fewest rounds of 256 workgroups (measured on
+  // 2560 x 9728 with eight slices: 12.6 / 11.4 / 12.4 us with four / five / six at four rows, five = exactly 256 workgroups;
+  // 2560 x 4096 with four slices: 8.8 / 8.9 / 9.8, and 9.2 with three)
+  int nwaves = g_kq_meet_waves;
+  if (!nwaves) {
+    int64_t best = 0;
+    for (int nw = 4; nw <= 6; nw++) {
+      int64_t wgs = 0;
+      for (int p = 0; p < a.nparts; p++) wgs += ((a.part[p].N + 15) / 16 + nw - 1) / nw;
+      const int64_t rounds = (wgs * SG + 255) / 256;
+      if (!best || rounds < best) {
+        best = rounds;
+        nwaves = nw;
+      }
+    }
+  }
+  unsigned grid = 0;
+  for (int p = 0; p < a.nparts; p++) {
+    a.wg_start[p] = (int)grid;
+    grid += (unsigned)(((a.part[p].N + 15) / 16 + nwaves - 1) / nwaves);
+  }
+  a.wg_start[a.nparts] = (int)grid;
+  if (SG < 2 || g_kq_meet == 0 || !room.part || (size_t)grid * nwaves * SG * 512 > room.part_bytes || grid > 1024u) return KQ_NOT_TAKEN;
+  KMeet km{};
+  km.SG = SG;
+  const int trip = 4 * kmf_groups(nbs);
+  km.lrows = (nbs + trip - 1) / trip * trip;
+  km.part = static_cast<float*>(room.part);
+  RC_RET(gemv_counter_block(room.key, st, &km.counters));
+  km.cstride = 1;
+  while (km.cstride < 32 && (size_t)grid * km.cstride * 2 <= 1024u) km.cstride *= 2;
+  const size_t lds = kmf_lds_bytes_z<MT>(nbs, nwaves);
+  auto go = [&](auto kern) {
+    if (lds > 64 * 1024)
+      HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3(grid, 1, (unsigned)SG), dim3(nwaves * 64), lds, st, a, 1, nbs, km);
+    return (int)hipGetLastError();
+  };
+  switch (kmf_groups(nbs)) {
+    case 6: return go(kq4_gemv_mfma_kernel<XT, MT, 6>);
+    case 8: return go(kq4_gemv_mfma_kernel<XT, MT, 8>);
+    default: return go(kq4_gemv_mfma_kernel<XT, MT, KMF_NG>);
+  }
 }
 template <int XT, int MT>
 static int launch_kq4_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned grid_y = 1) {
@@ -953,11 +1079,13 @@ static int launch_kq4_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned gri
   a.wg_start[a.nparts] = (int)grid;
   const size_t lds = kmf_lds_bytes<MT>(nb32, nbs, nwaves, S);
   if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
-  const int xpad = kmf_xpad(nb32, S, nbs);
+  KMeet km{};
+  km.SG = 1;
+  km.lrows = nb32 + kmf_xpad(nb32, S, nbs);
   auto go = [&](auto kern) {
     if (lds > 64 * 1024)
       HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kern, dim3(grid, grid_y), dim3(nwaves * 64), lds, st, a, S, nbs, xpad);
+    hipLaunchKernelGGL(kern, dim3(grid, grid_y), dim3(nwaves * 64), lds, st, a, S, nbs, km);
     return (int)hipGetLastError();
   };
   switch (kmf_groups(nbs)) {
@@ -1410,6 +1538,14 @@ MLLM_API int mllm_hip_kq_set_path(int path) {
   g_kq_path = path;
   return 0;
 }
+MLLM_API int mllm_hip_kq_set_slice_meeting(int mode, int waves_per_wg) {
+  if (mode < -1 || mode > 1 || (waves_per_wg != 0 && (waves_per_wg < 1 || waves_per_wg > 8))) return MLLM_HIP_E_BADARG;
+  g_kq_meet = mode;
+  g_kq_meet_min = mode == 1 ? 2 : 4;
+  g_kq_meet_waves = waves_per_wg;
+  return 0;
+}
+
 MLLM_API int mllm_hip_kq_set_tuning(int lanes_per_row, int waves_per_wg, int units_in_flight) {
   auto ok = [](int v, std::initializer_list<int> allowed) {
     for (int x : allowed)
@@ -1462,8 +1598,20 @@ MLLM_API size_t mllm_hip_kq_workspace_bytes(int64_t M, int64_t K) {
   return (size_t)8 * K + (size_t)8 * (K / QK_K) * 36;  // one group of eight rows: codes, sums of 16, scales
 }
 
+MLLM_API size_t mllm_hip_kq_workspace_bytes_n(int64_t M, int64_t K, int64_t N_total) {
+  const size_t img = mllm_hip_kq_workspace_bytes(M, K);
+  if (!img || N_total <= 0) return img;
+  return align_up(img, 256) + kmf_part_bytes((int)(K / QK_K), N_total, KQ_MAX_PARTS);
+}
+
 MLLM_API int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int64_t M,
                                       int64_t K, void* workspace, void* stream) {
+  return mllm_hip_linear_kq_multi_ws(wtype, nparts, parts, x, x_dtype, M, K, workspace, workspace ? mllm_hip_kq_workspace_bytes(M, K) : 0,
+                                     stream);
+}
+
+MLLM_API int mllm_hip_linear_kq_multi_ws(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int64_t M,
+                                         int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
   if (nparts < 1 || nparts > KQ_MAX_PARTS || !parts) return MLLM_HIP_E_BADARG;
   if (!x || M <= 0 || (x_dtype != MLLM_HIP_F32 && x_dtype != MLLM_HIP_BF16)) return MLLM_HIP_E_BADARG;
   if (reinterpret_cast<uintptr_t>(x) % 16 || reinterpret_cast<uintptr_t>(workspace) % 16) return MLLM_HIP_E_ALIGN;
@@ -1476,6 +1624,14 @@ MLLM_API int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv
   const int nsb = (int)(K / QK_K);
   hipStream_t st = (hipStream_t)stream;
   int rc = 0;
+  const size_t img_bytes = mllm_hip_kq_workspace_bytes(M, K);
+  if (workspace && workspace_bytes < img_bytes) return MLLM_HIP_E_BADARG;
+  // what lies behind the image serves the partial sums of K slices that meet in global memory
+  KMeetRoom room{workspace, nullptr, 0};
+  if (workspace && workspace_bytes > align_up(img_bytes, 256)) {
+    room.part = reinterpret_cast<char*>(workspace) + align_up(img_bytes, 256);
+    room.part_bytes = workspace_bytes - align_up(img_bytes, 256);
+  }
   for (int64_t m0 = 0; m0 < M; m0 += 8) {  // more than eight rows: groups of eight (each streams the weights again)
     const int rows = (int)(M - m0 < 8 ? M - m0 : 8);
     const void* xg = reinterpret_cast<const char*>(x) + m0 * xrow;
@@ -1492,6 +1648,13 @@ MLLM_API int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv
     const bool mfma = rows >= 3 && g_kq_path != 1 &&
                       (wtype == MLLM_HIP_Q4_K ? kq4_mfma_fits(rows <= 4 ? 4 : 8, nsb)
                                               : ((rows > 4 && nsb > 16) || g_kq_path == 2) && kq6_mfma_fits(rows <= 4 ? 4 : 8, nsb));
+    if (mfma && wtype == MLLM_HIP_Q4_K && room.part && g_kq_meet != 0 && kmf_slices(nsb * 8) >= g_kq_meet_min) {
+      // long rows: every workgroup takes one K slice and quantizes just that part of x itself; the slices meet in the workspace
+      if (rows <= 4) rc = x_dtype == MLLM_HIP_F32 ? launch_kq4_mfma_z<MLLM_HIP_F32, 4>(a, room, st) : launch_kq4_mfma_z<MLLM_HIP_BF16, 4>(a, room, st);
+      else rc = x_dtype == MLLM_HIP_F32 ? launch_kq4_mfma_z<MLLM_HIP_F32, 8>(a, room, st) : launch_kq4_mfma_z<MLLM_HIP_BF16, 8>(a, room, st);
+      if (rc == 0) continue;
+      if (rc != KQ_NOT_TAKEN) return rc;
+    }
     if (workspace && rows >= 3) {
       // several rows: quantize once for all workgroups; the GEMV then copies the image instead of quantizing
       const int MT = rows <= 4 ? 4 : 8;

@@ -633,8 +633,11 @@ def moe_ffn_kq(gate, up, down, x, topk_ids, topk_w, workspace=None, out=None):
     return y
 
 
-def kq_workspace(M, K):
-    return torch.empty(_lib.lib().mllm_hip_kq_workspace_bytes(M, K), dtype=torch.uint8, device="cuda")
+def kq_workspace(M, K, N_total=0):
+    """N_total (the sum of the N of a launch's parts) > 0: with room for the partial sums of K slices that meet in global memory"""
+    L = _lib.lib()
+    size = L.mllm_hip_kq_workspace_bytes_n(M, K, N_total) if N_total else L.mllm_hip_kq_workspace_bytes(M, K)
+    return torch.empty(size, dtype=torch.uint8, device="cuda")
 
 
 def linear_kq_gemm(w, x, bias=None, out=None, workspace=None, short=False):
@@ -653,10 +656,13 @@ def linear_kq_gemm(w, x, bias=None, out=None, workspace=None, short=False):
 
 
 def linear_kq(w, x, bias=None, out=None, workspace=None):
-    """workspace (kq_workspace): from three rows on, x is quantized once by a small kernel instead of in every workgroup"""
+    """workspace (kq_workspace): from three rows on, x is quantized once by a small kernel instead of in every workgroup;
+    with room for partial sums (kq_workspace(M, K, N)), long Q4_K rows are cut into K slices with a workgroup each"""
     assert w.layout == "gemv" and x.is_cuda and x.is_contiguous() and x.dim() == 2 and x.shape[1] == w.K
     M = x.shape[0]
     y = out if out is not None else torch.empty((M, w.N), dtype=torch.float32, device="cuda")
+    if workspace is not None and workspace.numel() > _lib.lib().mllm_hip_kq_workspace_bytes(M, w.K):
+        return linear_kq_multi([w], x, [bias], [y], workspace=workspace)[0]  # (the entry point that is told the workspace's size)
     _lib.check(_lib.lib().mllm_hip_linear_kq(w.wtype, w.ptr, x.data_ptr(), _xdtype(x), _p(bias), y.data_ptr(), M, w.N, w.K,
                                              _p(workspace), _stream()), "mllm_hip_linear_kq")
     return y
@@ -673,7 +679,11 @@ def linear_kq_multi(ws, x, biases=None, outs=None, workspace=None):
         assert w.K == K and w.wtype == ws[0].wtype
         b = biases[i] if biases is not None else None
         parts[i] = _lib.GemvPart(w.ptr, b.data_ptr() if b is not None else None, outs[i].data_ptr(), w.N)
-    _lib.check(_lib.lib().mllm_hip_linear_kq_multi(ws[0].wtype, len(ws), parts, x.data_ptr(), _xdtype(x), M, K, _p(workspace), _stream()),
+    if workspace is not None:
+        _lib.check(_lib.lib().mllm_hip_linear_kq_multi_ws(ws[0].wtype, len(ws), parts, x.data_ptr(), _xdtype(x), M, K, workspace.data_ptr(),
+                                                          workspace.numel(), _stream()), "mllm_hip_linear_kq_multi_ws")
+        return outs
+    _lib.check(_lib.lib().mllm_hip_linear_kq_multi(ws[0].wtype, len(ws), parts, x.data_ptr(), _xdtype(x), M, K, None, _stream()),
                "mllm_hip_linear_kq_multi")
     return outs
 

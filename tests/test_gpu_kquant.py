@@ -206,6 +206,40 @@ def test_matrix_core_and_dot4_kernels_agree(wtype, M):
     assert L.mllm_hip_kq_set_path(3) == -1
 
 
+@pytest.mark.parametrize("M", [3, 4, 7, 8, 19])
+def test_q4_k_slices_that_meet_in_the_workspace_give_the_same_bits(M):
+    """a workspace with room for partial sums: rows of more than 2560 elements are cut into K slices with a workgroup each, which
+    quantize their own part of x and meet through arrival counters; the sum runs in slice order as in the one-workgroup form.
+    Ragged N, several parts, bias, fp32 and bf16 activations, every workgroup shape, the workspace used again and again."""
+    wtype = 2
+    rng = synth.rng_for(7, 1300 + M)
+    L = _lib.lib()
+    for Ns, K in (((2560,), 9728), ((2560,), 4096), ((77, 130), 4096 + 256), ((33, 16, 50, 200), 3072), ((700, 90), 2560), ((40,), 256)):
+        ws = [ql.PackedKWeight(wtype, torch.from_numpy(synth.make_weight(rng, wtype, N, K))) for N in Ns]
+        biases = [to_dev(rng.standard_normal(N).astype(np.float32)) if i % 2 == 0 else None for i, N in enumerate(Ns)]
+        xf = synth.make_x_fp32(rng, M, K)
+        for x in (to_dev(xf), to_dev(xf).to(torch.bfloat16)):
+            announce("kq4 slices meet", M, Ns, K, x.dtype)
+            want = ql.linear_kq_multi(ws, x, biases)                                        # no workspace
+            small = ql.linear_kq_multi(ws, x, biases, workspace=ql.kq_workspace(M, K))       # image only
+            room = ql.kq_workspace(M, K, sum(Ns))
+            assert room.numel() >= ql.kq_workspace(M, K).numel()
+            try:
+                for mode, waves in ((-1, 0), (-1, 0), (1, 0), (1, 1), (1, 3), (-1, 5), (1, 8), (0, 0)):
+                    assert L.mllm_hip_kq_set_slice_meeting(mode, waves) == 0
+                    got = ql.linear_kq_multi(ws, x, biases, workspace=room)
+                    for a, b, c in zip(want, small, got):
+                        assert torch.equal(a, b) and torch.equal(a, c), (mode, waves)
+            finally:
+                assert L.mllm_hip_kq_set_slice_meeting(-1, 0) == 0
+            assert L.mllm_hip_gemv_workspace_release(room.data_ptr()) == 0
+    assert L.mllm_hip_kq_set_slice_meeting(2, 0) == -1 and L.mllm_hip_kq_set_slice_meeting(0, 9) == -1
+    # a workspace smaller than the image is an error, stated size or not
+    p = ws[0].ptr
+    part = (_lib.GemvPart * 1)(_lib.GemvPart(p, None, want[0].data_ptr(), 40))
+    assert L.mllm_hip_linear_kq_multi_ws(wtype, 1, part, x.data_ptr(), ql._xdtype(x), M, 256, room.data_ptr(), 16, None) == -1
+
+
 def test_argument_checks():
     L = _lib.lib()
     buf = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
