@@ -677,6 +677,9 @@ static int launch_kq(const KGemvArgs& a, hipStream_t st) {
 #ifndef KMF_WEIGHTS_FIRST
 #define KMF_WEIGHTS_FIRST 0
 #endif
+#ifndef KMF_QUANT_BATCH
+#define KMF_QUANT_BATCH 4
+#endif
 #ifndef KMF_COPY_UNROLL
 #define KMF_COPY_UNROLL 5
 #endif
@@ -778,7 +781,7 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
       wq[j] = __builtin_amdgcn_raw_buffer_load_b128(ra, (row_ok && b < b1) ? (rbase + (uint32_t)b) * 16u : KBUF_OOB, 0, KBUF_NT);
     }
   };
-  if (KMF_WEIGHTS_FIRST) load_groups(b0);
+  if (KMF_WEIGHTS_FIRST && XT == KQ_IMAGE) load_groups(b0);
   __asm__ volatile("" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
@@ -788,34 +791,77 @@ __global__ __launch_bounds__(512) void kq4_gemv_mfma_kernel(KGemvArgs a, int S, 
     const u32x4* codes = reinterpret_cast<const u32x4*>(a.x);
     const uint32_t* pairs = reinterpret_cast<const uint32_t*>(reinterpret_cast<const char*>(a.x) + R * K);
     const float* dd = reinterpret_cast<const float*>(reinterpret_cast<const char*>(a.x) + R * K + R * nsb * 32);
-    for (int m = wave; m < MT; m += nwaves) {
-      const size_t src = (size_t)kq_tile_in_row(a, mt, m);
-#pragma unroll KMF_COPY_UNROLL
-      for (int r = lane; r < 2 * nloc; r += 64) xc[((size_t)(r >> 1) * MT + m) * 2 + (r & 1)] = codes[(src * nb32 + kb0) * 2 + r];
-      for (int sb = lane; sb < nloc; sb += 64) {
-        const uint32_t pr = pairs[src * nb32 + kb0 + sb];
-        const int bsum = (int)(int16_t)(pr & 0xffffu) + (int)(int16_t)(pr >> 16);
-        xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(dd[src * nsb + ((kb0 + sb) >> 3)]), (uint32_t)bsum};
+    // Thread (row m = tid % MT, piece tid / MT): a wave reads 128 contiguous bytes of each of its rows and writes 1 KB of
+    // contiguous LDS.  The pieces of a batch are all requested before the first is stored, and the sums and scales before
+    // the codes: one round trip to memory per batch, where a copy row by row and pass by pass took one per pass.
+    const int m = tid & (MT - 1), p0 = tid / MT, pstep = nthreads / MT;
+    const size_t src = (size_t)kq_tile_in_row(a, mt, m);
+    constexpr int CS = 3;
+    uint32_t pr[CS];
+    float dv[CS];
+#pragma unroll
+    for (int u = 0; u < CS; u++) {
+      const int sb = p0 + u * pstep;
+      if (sb < nloc) {
+        pr[u] = pairs[src * nb32 + kb0 + sb];
+        dv[u] = dd[src * nsb + ((kb0 + sb) >> 3)];
       }
     }
+    for (int r0 = p0; r0 < 2 * nloc; r0 += pstep * KMF_COPY_UNROLL) {
+      u32x4 cv[KMF_COPY_UNROLL];
+#pragma unroll
+      for (int u = 0; u < KMF_COPY_UNROLL; u++) {
+        const int r = r0 + u * pstep;
+        if (r < 2 * nloc) cv[u] = codes[(src * nb32 + kb0) * 2 + r];
+      }
+#pragma unroll
+      for (int u = 0; u < KMF_COPY_UNROLL; u++) {
+        const int r = r0 + u * pstep;
+        if (r < 2 * nloc) xc[((size_t)(r >> 1) * MT + m) * 2 + (r & 1)] = cv[u];
+      }
+    }
+    auto put_sums = [&](int sb, uint32_t pair, float d) {
+      const int bsum = (int)(int16_t)(pair & 0xffffu) + (int)(int16_t)(pair >> 16);
+      xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(d), (uint32_t)bsum};
+    };
+#pragma unroll
+    for (int u = 0; u < CS; u++)
+      if (p0 + u * pstep < nloc) put_sums(p0 + u * pstep, pr[u], dv[u]);
+    for (int sb = p0 + CS * pstep; sb < nloc; sb += pstep) put_sums(sb, pairs[src * nb32 + kb0 + sb], dd[src * nsb + ((kb0 + sb) >> 3)]);
   } else {
     const int ipr = K >> 3;     // items (eight elements) per row; 32 consecutive items = one super-block
     const int iwg = nloc << 2;  // of them in this workgroup's sub-blocks (whole super-blocks)
     const int nitems = MT * iwg;
     const float inv_iwg = 1.0f / (float)iwg;
-    for (int it = tid; it < nitems; it += nthreads) {  // whole half-waves: nitems and nthreads are multiples of 32
-      const int m = (int)(((float)it + 0.5f) * inv_iwg), i = it - m * iwg;  // it / iwg: far from rounding trouble
-      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      if (m < a.M) load8<XT == KQ_IMAGE ? MLLM_HIP_F32 : XT>(a.x, ((int64_t)m * ipr + 4 * kb0 + i) * 8, v);
-      const Q8KItem qi = quantize_q8k_item(v, lane);
-      int s32 = qi.sum8 + __builtin_amdgcn_update_dpp(0, qi.sum8, 0xB1, 0xf, 0xf, true);
-      s32 += __builtin_amdgcn_update_dpp(0, s32, 0x4E, 0xf, 0xf, true);
-      const int sb = i >> 2, part = i & 3;  // sub-block (from kb0), which 8 of its 32 codes
-      reinterpret_cast<u32x2*>(xc + ((size_t)sb * MT + m) * 2 + (part >> 1))[part & 1] = u32x2{qi.q0, qi.q1};
-      if (part == 0) xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(qi.d), (uint32_t)s32};
+    // (the items of a batch are all requested before the first is quantized: one round trip to memory per batch)
+    constexpr int QI = KMF_QUANT_BATCH;
+    for (int it0 = tid; it0 < nitems; it0 += nthreads * QI) {  // whole half-waves: nitems and nthreads are multiples of 32
+      float v[QI][8];
+#pragma unroll
+      for (int u = 0; u < QI; u++) {
+        const int it = it0 + u * nthreads;
+        const int m = (int)(((float)it + 0.5f) * inv_iwg), i = it - m * iwg;  // it / iwg: far from rounding trouble
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[u][e] = 0.f;
+        if (it < nitems && m < a.M) load8<XT == KQ_IMAGE ? MLLM_HIP_F32 : XT>(a.x, ((int64_t)m * ipr + 4 * kb0 + i) * 8, v[u]);
+      }
+      if (it0 == tid) load_groups(b0);  // the weights right behind the first batch: they arrive while it is quantized
+#pragma unroll
+      for (int u = 0; u < QI; u++) {
+        const int it = it0 + u * nthreads;
+        if (it >= nitems) break;
+        const int m = (int)(((float)it + 0.5f) * inv_iwg), i = it - m * iwg;
+        const Q8KItem qi = quantize_q8k_item(v[u], lane);
+        int s32 = qi.sum8 + __builtin_amdgcn_update_dpp(0, qi.sum8, 0xB1, 0xf, 0xf, true);
+        s32 += __builtin_amdgcn_update_dpp(0, s32, 0x4E, 0xf, 0xf, true);
+        const int sb = i >> 2, part = i & 3;  // sub-block (from kb0), which 8 of its 32 codes
+        reinterpret_cast<u32x2*>(xc + ((size_t)sb * MT + m) * 2 + (part >> 1))[part & 1] = u32x2{qi.q0, qi.q1};
+        if (part == 0) xs[(size_t)sb * MT + m] = u32x2{__float_as_uint(qi.d), (uint32_t)s32};
+      }
     }
   }
-  if (!KMF_WEIGHTS_FIRST) load_groups(b0);
+  if (!KMF_WEIGHTS_FIRST && XT == KQ_IMAGE) load_groups(b0);
+  if (XT != KQ_IMAGE && tid >= (nloc << 2) * MT) load_groups(b0);  // (threads without an item to quantize)
   if (tid == 0) zrec[0] = u32x4{0u, 0u, 0u, 0u};
   for (int i = tid; i < (lrows - nloc) * MT * 2; i += nthreads) xc[(size_t)nloc * MT * 2 + i] = u32x4{0u, 0u, 0u, 0u};
   for (int i = tid; i < (lrows - nloc) * MT; i += nthreads) xs[(size_t)nloc * MT + i] = u32x2{0u, 0u};
