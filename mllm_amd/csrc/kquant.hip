@@ -1229,29 +1229,63 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
     const u32x4* codes = reinterpret_cast<const u32x4*>(a.x);
     const int16_t* sums = reinterpret_cast<const int16_t*>(reinterpret_cast<const char*>(a.x) + R * K);
     const float* dd = reinterpret_cast<const float*>(reinterpret_cast<const char*>(a.x) + R * K + R * nsb * 32);
-    for (int m = wave; m < MT; m += nwaves) {
-      const size_t src = (size_t)kq_tile_in_row(a, mt, m);
-#pragma unroll KMF_COPY_UNROLL
-      for (int u = lane; u < nu; u += 64) {
-        xc[(size_t)u * MT + m] = codes[src * nu + u];
-        bs16[(size_t)u * MT + m] = (int)sums[src * nu + u];
+    // thread (row m = tid % MT, unit tid / MT), a batch of units requested before the first is stored, as in the Q4_K kernel
+    const int m = tid & (MT - 1), p0 = tid / MT, pstep = nthreads / MT;
+    const size_t src = (size_t)kq_tile_in_row(a, mt, m);
+    float dv[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+      if (p0 + i * pstep < nsb) dv[i] = dd[src * nsb + p0 + i * pstep];
+    for (int u0 = p0; u0 < nu; u0 += pstep * KMF_COPY_UNROLL) {
+      u32x4 cv[KMF_COPY_UNROLL];
+      int16_t sv[KMF_COPY_UNROLL];
+#pragma unroll
+      for (int i = 0; i < KMF_COPY_UNROLL; i++) {
+        const int u = u0 + i * pstep;
+        if (u < nu) {
+          cv[i] = codes[src * nu + u];
+          sv[i] = sums[src * nu + u];
+        }
       }
-      for (int sb = lane; sb < nsb; sb += 64) dxs[sb * MT + m] = dd[src * nsb + sb];
+#pragma unroll
+      for (int i = 0; i < KMF_COPY_UNROLL; i++) {
+        const int u = u0 + i * pstep;
+        if (u < nu) {
+          xc[(size_t)u * MT + m] = cv[i];
+          bs16[(size_t)u * MT + m] = (int)sv[i];
+        }
+      }
     }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+      if (p0 + i * pstep < nsb) dxs[(p0 + i * pstep) * MT + m] = dv[i];
+    for (int sb = p0 + 2 * pstep; sb < nsb; sb += pstep) dxs[sb * MT + m] = dd[src * nsb + sb];
   } else {
     const int ipr = K >> 3;
     const int nitems = MT * ipr, valid = a.M * ipr;
     const float inv_ipr = 1.0f / (float)ipr;
-    for (int it = tid; it < nitems; it += nthreads) {  // whole half-waves
-      float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-      if (it < valid) load8<XT == KQ_IMAGE ? MLLM_HIP_F32 : XT>(a.x, (int64_t)it * 8, v);
-      const Q8KItem qi = quantize_q8k_item(v, lane);
-      const int s16 = qi.sum8 + __builtin_amdgcn_update_dpp(0, qi.sum8, 0xB1, 0xf, 0xf, true);
-      const int m = (int)(((float)it + 0.5f) * inv_ipr), i = it - m * ipr;
-      const int u = i >> 1;
-      reinterpret_cast<u32x2*>(xc + (size_t)u * MT + m)[i & 1] = u32x2{qi.q0, qi.q1};
-      if ((i & 1) == 0) bs16[(size_t)u * MT + m] = s16;
-      if ((i & 31) == 0) dxs[(i >> 5) * MT + m] = qi.d;
+    constexpr int QI = KMF_QUANT_BATCH;  // (a batch of items is requested before the first is quantized)
+    for (int it0 = tid; it0 < nitems; it0 += nthreads * QI) {  // whole half-waves
+      float v[QI][8];
+#pragma unroll
+      for (int b = 0; b < QI; b++) {
+        const int it = it0 + b * nthreads;
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[b][e] = 0.f;
+        if (it < valid) load8<XT == KQ_IMAGE ? MLLM_HIP_F32 : XT>(a.x, (int64_t)it * 8, v[b]);
+      }
+#pragma unroll
+      for (int b = 0; b < QI; b++) {
+        const int it = it0 + b * nthreads;
+        if (it >= nitems) break;
+        const Q8KItem qi = quantize_q8k_item(v[b], lane);
+        const int s16 = qi.sum8 + __builtin_amdgcn_update_dpp(0, qi.sum8, 0xB1, 0xf, 0xf, true);
+        const int m = (int)(((float)it + 0.5f) * inv_ipr), i = it - m * ipr;
+        const int u = i >> 1;
+        reinterpret_cast<u32x2*>(xc + (size_t)u * MT + m)[i & 1] = u32x2{qi.q0, qi.q1};
+        if ((i & 1) == 0) bs16[(size_t)u * MT + m] = s16;
+        if ((i & 31) == 0) dxs[(i >> 5) * MT + m] = qi.d;
+      }
     }
   }
   if (!KMF_WEIGHTS_FIRST) load_steps(s0);
