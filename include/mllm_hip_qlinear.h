@@ -442,7 +442,7 @@ int mllm_hip_kq_set_slice_meeting(int mode, int waves_per_wg);
  * flight per row (1/2/4; more than one only for up to two activation rows); 0 = heuristic. */
 int mllm_hip_kq_set_tuning(int lanes_per_row, int waves_per_wg, int units_in_flight);
 /* Three to eight rows take their sub-block sums from the matrix cores as the Q4_0 kernel of that kind does (Q4_K always, Q6_K
- * with five to eight rows of more than 4096 elements, where it measured faster).  path = 1 keeps every launch on the dot4
+ * with five to eight rows, and with three or four rows of more than 4096 elements, where it measured faster).  path = 1 keeps every launch on the dot4
  * kernel, 2 uses the matrix-core kernels wherever they fit (comparison runs, tests), 0 restores the default. */
 int mllm_hip_kq_set_path(int path);
 int mllm_hip_linear_kq(int wtype, const void* packed, const void* x, int x_dtype, const float* bias, float* y, int64_t M, int64_t N,

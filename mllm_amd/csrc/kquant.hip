@@ -1722,12 +1722,14 @@ MLLM_API int mllm_hip_linear_kq_multi_ws(int wtype, int nparts, const mllm_hip_g
     a.x = xg;
     a.M = rows;
     a.nsb = nsb;
-    // Q4_K: from three rows on.  Q6_K (heavier unpacking, 200 registers): measured faster only with five to eight rows of more
-    // than 4096 elements (down projection 9728: 37.6 -> 20.7 us at eight rows; a 2560-element row ties, q and o lose).
-    // The rule looks at the weight type, the number of rows and the row length only.
+    // Q4_K: from three rows on.  Q6_K (heavier unpacking, 200 registers): from five rows on, and with three or four rows of
+    // more than 4096 elements (4B layer shapes q+k+v / o / gate+up / down, dot4 -> matrix cores: eight rows 14.8 / 13.8 / 33.3 /
+    // 19.7 -> 13.8 / 12.6 / 25.0 / 19.7 us; four rows 11.1 / 10.1 / 24.1 / 17.8 -> 12.1 / 10.6 / 21.3 / 16.2).
+    // The rule looks at the weight type, the number of rows and the row length only: a projection gives the same bits alone
+    // and as a part of a launch.
     const bool mfma = rows >= 3 && g_kq_path != 1 &&
                       (wtype == MLLM_HIP_Q4_K ? kq4_mfma_fits(rows <= 4 ? 4 : 8, nsb)
-                                              : ((rows > 4 && nsb > 16) || g_kq_path == 2) && kq6_mfma_fits(rows <= 4 ? 4 : 8, nsb));
+                                              : (rows > 4 || nsb > 16 || g_kq_path == 2) && kq6_mfma_fits(rows <= 4 ? 4 : 8, nsb));
     if (mfma && wtype == MLLM_HIP_Q4_K && room.part && g_kq_meet != 0 && kmf_slices(nsb * 8) >= g_kq_meet_min) {
       // long rows: every workgroup takes one K slice and quantizes just that part of x itself; the slices meet in the workspace
       if (rows <= 4) rc = x_dtype == MLLM_HIP_F32 ? launch_kq4_mfma_z<MLLM_HIP_F32, 4>(a, room, st) : launch_kq4_mfma_z<MLLM_HIP_BF16, 4>(a, room, st);
