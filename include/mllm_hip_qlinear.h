@@ -423,9 +423,9 @@ size_t mllm_hip_kq_workspace_bytes(int64_t M, int64_t K);
 int mllm_hip_linear_kq_multi(int wtype, int nparts, const mllm_hip_gemv_part* parts, const void* x, int x_dtype, int64_t M, int64_t K,
                              void* workspace, void* stream);
 /* The same with the size of the workspace stated.  A workspace of mllm_hip_kq_workspace_bytes_n(M, K, N_total) bytes (N_total =
- * the sum of the parts' N) also has room for partial sums: Q4_K launches of three to eight rows whose rows have more than
- * 2560 elements (four K slices and more) then give every slice a workgroup of its own, which quantizes just its part of x
- * (no separate quantization launch), and the slices meet in that room.  Same results bit for bit.  The arrival counters
+ * the sum of the parts' N) also has room for partial sums: launches of three to eight rows on the matrix-core kernels whose
+ * rows have more than 2560 elements (Q6_K: more than 5120) then give every K slice a workgroup of its own, which quantizes
+ * just its part of x (no separate quantization launch), and the slices meet in that room.  Same results bit for bit.  The arrival counters
  * belong to the workspace address as for mllm_hip_linear_q_gemv_multi: one launch at a time per workspace, and
  * mllm_hip_gemv_workspace_release before the memory is freed.  A smaller workspace (at least mllm_hip_kq_workspace_bytes)
  * is used as by mllm_hip_linear_kq_multi; less than that is MLLM_HIP_E_BADARG.
@@ -435,7 +435,7 @@ int mllm_hip_linear_kq_multi_ws(int wtype, int nparts, const mllm_hip_gemv_part*
                                 void* workspace, size_t workspace_bytes, void* stream);
 /* Comparison runs and tests: mode 0 keeps the K slices of every launch in one workgroup even where the workspace has room
  * for partial sums; -1 (the default) lets them meet in global memory where a row has at least four slices (more than
- * 2560 elements), 1 from two slices on; waves_per_wg = row tiles of a workgroup in that form (1..8, 0 = chosen per launch).
+ * 2560 elements; Q6_K: eight slices, more than 5120 elements), 1 from two slices on; waves_per_wg = row tiles of a workgroup in that form (1..8, 0 = chosen per launch).
  * Same results bit for bit in every setting. */
 int mllm_hip_kq_set_slice_meeting(int mode, int waves_per_wg);
 /* Tuning override of the decode GEMV: lanes per weight row (8/16/32/64), waves per workgroup (1/2/4), units a lane keeps in

@@ -1051,20 +1051,15 @@ static bool kq4_mfma_fits(int MT, int nsb) {
 }
 // room for the partial sums of a launch whose slices meet in global memory (0: its slices share a workgroup anyway)
 static size_t kmf_part_bytes(int nsb, int64_t n_total, int nparts) {
-  const int S = kmf_slices(nsb * 8);
+  const int S = std::max(kmf_slices(nsb * 8), nsb > 5 ? (nsb > 10 ? (nsb > 20 ? 8 : 4) : 2) : 1);  // (Q4_K's slices, Q6_K's: k6mf_split)
   if (S < 2) return 0;
   return (size_t)((n_total + 15) / 16 + (int64_t)nparts * 8) * S * 512;
 }
 int g_kq_meet = -1, g_kq_meet_waves = 0, g_kq_meet_min = 4;  // (mllm_hip_kq_set_slice_meeting)
-template <int XT, int MT>
-static int launch_kq4_mfma_z(const KGemvArgs& a_in, const KMeetRoom& room, hipStream_t st) {
-  KGemvArgs a = a_in;
-  const int nb32 = a.nsb * 8;
-  const int SG = kmf_slices(nb32);
-  const int nbs = ((nb32 + SG - 1) / SG + 7) / 8 * 8;
-  // row tiles (= waves) per workgroup: four to six, the first that needs the fewest rounds of 256 workgroups (measured on
-  // 2560 x 9728 with eight slices: 12.6 / 11.4 / 12.4 us with four / five / six at four rows, five = exactly 256 workgroups;
-  // 2560 x 4096 with four slices: 8.8 / 8.9 / 9.8, and 9.2 with three)
+// row tiles (= waves) per workgroup of a launch whose K slices meet in memory: four to six, the first that needs the fewest
+// rounds of 256 workgroups (measured with Q4_K on 2560 x 9728 with eight slices: 12.6 / 11.4 / 12.4 us with four / five /
+// six at four rows, five = exactly 256 workgroups; 2560 x 4096 with four slices: 8.8 / 8.9 / 9.8, and 9.2 with three)
+static int kq_meet_waves(const KGemvArgs& a, int SG) {
   int nwaves = g_kq_meet_waves;
   if (!nwaves) {
     int64_t best = 0;
@@ -1078,6 +1073,15 @@ static int launch_kq4_mfma_z(const KGemvArgs& a_in, const KMeetRoom& room, hipSt
       }
     }
   }
+  return nwaves;
+}
+template <int XT, int MT>
+static int launch_kq4_mfma_z(const KGemvArgs& a_in, const KMeetRoom& room, hipStream_t st) {
+  KGemvArgs a = a_in;
+  const int nb32 = a.nsb * 8;
+  const int SG = kmf_slices(nb32);
+  const int nbs = ((nb32 + SG - 1) / SG + 7) / 8 * 8;
+  const int nwaves = kq_meet_waves(a, SG);
   unsigned grid = 0;
   for (int p = 0; p < a.nparts; p++) {
     a.wg_start[p] = (int)grid;
@@ -1157,7 +1161,7 @@ constexpr int K6_ST = 10;  // steps per trip, at most: five super-blocks (the la
 // ST = steps per trip: the slice in one trip where it fits (6, 8 or 10); xpad = super-blocks the last trip of a slice reaches
 // past the row (zeros in LDS)
 template <int XT, int MT, int ST = K6_ST>
-__global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, int sps, int xpad) {  // sps = super-blocks per slice
+__global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, int sps, KMeet km) {  // sps = super-blocks per slice; km.lrows in super-blocks
   extern __shared__ __align__(16) unsigned char smem[];
   constexpr int TH = MT / 4;
   constexpr int TSB = ST / 2;  // super-blocks per trip
@@ -1174,18 +1178,22 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
   const int N = pt.N;
   const int tiles_wg = nwaves / S;
   const int tile = ((int)blockIdx.x - a.wg_start[pidx]) * tiles_wg + wave / S;
-  const int slice = wave % S;
+  const int sg = km.SG > 1 ? (int)blockIdx.z : 0;  // slice group: the workgroup's slices are [sg S, sg S + S)
+  const int slice = sg * S + wave % S;
   const int row0 = tile * 16;
   const bool tile_ok = row0 < N;
   const int s0 = slice * sps, s1 = min(nsb, s0 + sps);  // this wave's super-blocks
+  const int ks0 = min(nsb, sg * S * sps), ks1 = min(nsb, ks0 + S * sps);  // the workgroup's; LDS rows count from ks0
+  const int nloc = ks1 - ks0, lsb = km.lrows, nul = nloc * 16;
 
   const int wsu = (sps + TSB - 1) / TSB * TSB * 16;  // units of weight scales per wave: whole trips
-  u32x4* xc = reinterpret_cast<u32x4*>(smem);                     // [unit * MT + m] the unit's 16 codes
-  u32x4* zrec = xc + (size_t)(nu + xpad * 16) * MT;
-  int* bs16 = reinterpret_cast<int*>(zrec + 1);                   // [unit * MT + m] sum of the unit's codes
-  float* dxs = reinterpret_cast<float*>(bs16 + (size_t)(nu + xpad * 16) * MT);  // [super-block * MT + m]
-  float* ws_all = dxs + (size_t)(nsb + xpad) * MT;
+  u32x4* xc = reinterpret_cast<u32x4*>(smem);                     // [(unit - 16 ks0) * MT + m] the unit's 16 codes
+  u32x4* zrec = xc + (size_t)lsb * 16 * MT;
+  int* bs16 = reinterpret_cast<int*>(zrec + 1);                   // [(unit - 16 ks0) * MT + m] sum of the unit's codes
+  float* dxs = reinterpret_cast<float*>(bs16 + (size_t)lsb * 16 * MT);  // [(super-block - ks0) * MT + m]
+  float* ws_all = dxs + (size_t)lsb * MT;
   float* ws = ws_all + (size_t)wave * wsu * 16;
+  int* s_flag = reinterpret_cast<int*>(ws_all + (size_t)nwaves * wsu * 16);
   f32x4* red = reinterpret_cast<f32x4*>(smem) + (size_t)wave * TH * 64;  // takes the place of the codes once every wave is done with them
 
   const uint32_t sbt = (uint32_t)N * (uint32_t)nsb;
@@ -1219,7 +1227,7 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
       wh[st] = __builtin_amdgcn_raw_buffer_load_b128(rh, ok ? ((rbase + (uint32_t)sb) * 4u + 2u * (st & 1) + (uint32_t)(g & 1)) * 16u : KBUF_OOB, 0, KBUF_NT);
     }
   };
-  if (KMF_WEIGHTS_FIRST) load_steps(s0);
+  if (KMF_WEIGHTS_FIRST && XT == KQ_IMAGE) load_steps(s0);
   __asm__ volatile("" ::: "memory");
   __builtin_amdgcn_sched_barrier(0);
 
@@ -1235,22 +1243,22 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
     float dv[2];
 #pragma unroll
     for (int i = 0; i < 2; i++)
-      if (p0 + i * pstep < nsb) dv[i] = dd[src * nsb + p0 + i * pstep];
-    for (int u0 = p0; u0 < nu; u0 += pstep * KMF_COPY_UNROLL) {
+      if (p0 + i * pstep < nloc) dv[i] = dd[src * nsb + ks0 + p0 + i * pstep];
+    for (int u0 = p0; u0 < nul; u0 += pstep * KMF_COPY_UNROLL) {
       u32x4 cv[KMF_COPY_UNROLL];
       int16_t sv[KMF_COPY_UNROLL];
 #pragma unroll
       for (int i = 0; i < KMF_COPY_UNROLL; i++) {
         const int u = u0 + i * pstep;
-        if (u < nu) {
-          cv[i] = codes[src * nu + u];
-          sv[i] = sums[src * nu + u];
+        if (u < nul) {
+          cv[i] = codes[src * nu + ks0 * 16 + u];
+          sv[i] = sums[src * nu + ks0 * 16 + u];
         }
       }
 #pragma unroll
       for (int i = 0; i < KMF_COPY_UNROLL; i++) {
         const int u = u0 + i * pstep;
-        if (u < nu) {
+        if (u < nul) {
           xc[(size_t)u * MT + m] = cv[i];
           bs16[(size_t)u * MT + m] = (int)sv[i];
         }
@@ -1258,29 +1266,32 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
     }
 #pragma unroll
     for (int i = 0; i < 2; i++)
-      if (p0 + i * pstep < nsb) dxs[(p0 + i * pstep) * MT + m] = dv[i];
-    for (int sb = p0 + 2 * pstep; sb < nsb; sb += pstep) dxs[sb * MT + m] = dd[src * nsb + sb];
+      if (p0 + i * pstep < nloc) dxs[(p0 + i * pstep) * MT + m] = dv[i];
+    for (int sb = p0 + 2 * pstep; sb < nloc; sb += pstep) dxs[sb * MT + m] = dd[src * nsb + ks0 + sb];
   } else {
-    const int ipr = K >> 3;
-    const int nitems = MT * ipr, valid = a.M * ipr;
-    const float inv_ipr = 1.0f / (float)ipr;
+    const int ipr = K >> 3;      // items (eight elements) per row
+    const int iwg = nloc << 5;   // of them in this workgroup's super-blocks
+    const int nitems = MT * iwg;
+    const float inv_iwg = 1.0f / (float)iwg;
     constexpr int QI = KMF_QUANT_BATCH;  // (a batch of items is requested before the first is quantized)
     for (int it0 = tid; it0 < nitems; it0 += nthreads * QI) {  // whole half-waves
       float v[QI][8];
 #pragma unroll
       for (int b = 0; b < QI; b++) {
         const int it = it0 + b * nthreads;
+        const int m = (int)(((float)it + 0.5f) * inv_iwg), i = it - m * iwg;
 #pragma unroll
         for (int e = 0; e < 8; e++) v[b][e] = 0.f;
-        if (it < valid) load8<XT == KQ_IMAGE ? MLLM_HIP_F32 : XT>(a.x, (int64_t)it * 8, v[b]);
+        if (it < nitems && m < a.M) load8<XT == KQ_IMAGE ? MLLM_HIP_F32 : XT>(a.x, ((int64_t)m * ipr + 32 * ks0 + i) * 8, v[b]);
       }
+      if (it0 == tid) load_steps(s0);  // the weights right behind the first batch: they arrive while it is quantized
 #pragma unroll
       for (int b = 0; b < QI; b++) {
         const int it = it0 + b * nthreads;
         if (it >= nitems) break;
         const Q8KItem qi = quantize_q8k_item(v[b], lane);
         const int s16 = qi.sum8 + __builtin_amdgcn_update_dpp(0, qi.sum8, 0xB1, 0xf, 0xf, true);
-        const int m = (int)(((float)it + 0.5f) * inv_ipr), i = it - m * ipr;
+        const int m = (int)(((float)it + 0.5f) * inv_iwg), i = it - m * iwg;
         const int u = i >> 1;
         reinterpret_cast<u32x2*>(xc + (size_t)u * MT + m)[i & 1] = u32x2{qi.q0, qi.q1};
         if ((i & 1) == 0) bs16[(size_t)u * MT + m] = s16;
@@ -1288,13 +1299,14 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
       }
     }
   }
-  if (!KMF_WEIGHTS_FIRST) load_steps(s0);
+  if (!KMF_WEIGHTS_FIRST && XT == KQ_IMAGE) load_steps(s0);
+  if (XT != KQ_IMAGE && tid >= (nloc << 5) * MT) load_steps(s0);  // (threads without an item to quantize)
   if (tid == 0) zrec[0] = u32x4{0u, 0u, 0u, 0u};
-  for (int i = tid; i < xpad * 16 * MT; i += nthreads) {
-    xc[(size_t)nu * MT + i] = u32x4{0u, 0u, 0u, 0u};
-    bs16[(size_t)nu * MT + i] = 0;
+  for (int i = tid; i < (lsb - nloc) * 16 * MT; i += nthreads) {
+    xc[(size_t)nul * MT + i] = u32x4{0u, 0u, 0u, 0u};
+    bs16[(size_t)nul * MT + i] = 0;
   }
-  for (int i = tid; i < xpad * MT; i += nthreads) dxs[nsb * MT + i] = 0.f;
+  for (int i = tid; i < (lsb - nloc) * MT; i += nthreads) dxs[nloc * MT + i] = 0.f;
 #pragma unroll
   for (int k = 0; k < 2; k++) {
     const int ch = lane + 64 * k;
@@ -1318,7 +1330,7 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
   for (int h = 0; h < TH; h++) acc[h] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int sb0 = s0; sb0 < s1; sb0 += TSB) {
     if (sb0 != s0) load_steps(sb0);
-    const int u0 = sb0 * 16;
+    const int u0 = (sb0 - ks0) * 16;  // first unit of the trip in LDS
     const u32x4* bl[TH];
     const int* bsl[TH];
     const float* dxl[TH];
@@ -1326,10 +1338,10 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
     for (int h = 0; h < TH; h++) {
       bl[h] = mine ? xc + (size_t)(u0 + q) * MT + 4 * h + tt : zrec;
       bsl[h] = bs16 + (size_t)(u0 + q) * MT + 4 * h + tt;
-      dxl[h] = dxs + sb0 * MT + 4 * h + tt;
+      dxl[h] = dxs + (sb0 - ks0) * MT + 4 * h + tt;
     }
     const int bstep = mine ? MT : 0;
-    const float* wsl = ws + (size_t)(u0 - s0 * 16 + q) * 16 + 4 * g;
+    const float* wsl = ws + (size_t)((sb0 - s0) * 16 + q) * 16 + 4 * g;
     u32x4 B[2][2][TH];
     int bs[2][2][TH];
     float dxv[2][TH];
@@ -1412,13 +1424,55 @@ __global__ __launch_bounds__(512) void kq6_gemv_mfma_kernel(KGemvArgs a, int S, 
 #pragma unroll
     for (int h = 0; h < TH; h++) red[h * 64 + lane] = acc[h];
     __syncthreads();
-    if (slice != 0) return;
+    if (wave % S != 0) return;
     for (int s = 1; s < S; s++)
 #pragma unroll
       for (int h = 0; h < TH; h++) {
         const f32x4 o = red[(size_t)s * TH * 64 + h * 64 + lane];
         acc[h].x += o.x; acc[h].y += o.y; acc[h].z += o.z; acc[h].w += o.w;
       }
+  }
+  if (km.SG > 1) {  // the slice groups of a grid column meet in global memory, as in the Q4_K kernel (S = 1 here: every wave is a tile)
+    const int SG = km.SG;
+    const int li = 4 * g + tt;
+    float* pbase = km.part + (((size_t)blockIdx.x * nwaves + wave) * SG) * 128;
+    if (q == 0) {
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        float* dst = pbase + (size_t)sg * 128 + (16 * h + li) * 4;
+        __hip_atomic_store(dst + 0, acc[h].x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(dst + 1, acc[h].y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(dst + 2, acc[h].z, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(dst + 3, acc[h].w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    __asm__ volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+      unsigned* cnt = km.counters + (size_t)blockIdx.x * km.cstride;
+      const unsigned old = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int last = old == (unsigned)(SG - 1);
+      if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+      *s_flag = last;
+    }
+    __syncthreads();
+    if (!*s_flag) return;
+    if (q == 0) {
+#pragma unroll
+      for (int h = 0; h < TH; h++) {
+        float pv[8][4];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+          const float* src = pbase + (size_t)min(u, SG - 1) * 128 + (16 * h + li) * 4;
+#pragma unroll
+          for (int e = 0; e < 4; e++) pv[u][e] = __hip_atomic_load(src + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        acc[h] = f32x4{pv[0][0], pv[0][1], pv[0][2], pv[0][3]};
+#pragma unroll
+        for (int u = 1; u < 8; u++)
+          if (u < SG) { acc[h].x += pv[u][0]; acc[h].y += pv[u][1]; acc[h].z += pv[u][2]; acc[h].w += pv[u][3]; }
+      }
+    }
   }
   if (!tile_ok || q != 0) return;
   const int n = row0 + 4 * g;
@@ -1449,9 +1503,15 @@ template <int MT>
 static size_t k6mf_lds_bytes(int nsb, int sps, int nwaves, int S) {
   const int tsb = k6mf_steps(sps) / 2, rows = nsb + k6mf_xpad(nsb, S, sps);
   const int wsu = (sps + tsb - 1) / tsb * tsb * 16;
-  const size_t need = (size_t)rows * 16 * MT * 16 + 16 + (size_t)rows * 16 * MT * 4 + (size_t)rows * MT * 4 + (size_t)nwaves * wsu * 64;
+  const size_t need = (size_t)rows * 16 * MT * 16 + 16 + (size_t)rows * 16 * MT * 4 + (size_t)rows * MT * 4 + (size_t)nwaves * wsu * 64 + 16;
   // the partial sums of the slices reuse the code area: it must hold them
   return std::max(need, (size_t)nwaves * (MT / 4) * 1024);
+}
+// the same with one slice per workgroup (slice groups over the grid's z): the slice's super-blocks in whole trips
+template <int MT>
+static size_t k6mf_lds_bytes_z(int sps, int nwaves) {
+  const int tsb = k6mf_steps(sps) / 2, rows = (sps + tsb - 1) / tsb * tsb;
+  return (size_t)rows * 16 * MT * 16 + 16 + (size_t)rows * 16 * MT * 4 + (size_t)rows * MT * 4 + (size_t)nwaves * rows * 16 * 64 + 16;
 }
 static void k6mf_split(int nsb, int& S, int& sps) {
   S = 1;
@@ -1463,6 +1523,42 @@ static bool kq6_mfma_fits(int MT, int nsb) {
   k6mf_split(nsb, S, sps);
   if (sps > 8) return false;  // scale records: at most 128 per wave
   return (MT == 4 ? k6mf_lds_bytes<4>(nsb, sps, 8, S) : k6mf_lds_bytes<8>(nsb, sps, 8, S)) <= 160 * 1024;
+}
+static int kq_meet_waves(const KGemvArgs& a, int SG);
+// every K slice a workgroup of its own (four to six row tiles), meeting in the caller's workspace: as launch_kq4_mfma_z
+template <int XT, int MT>
+static int launch_kq6_mfma_z(const KGemvArgs& a_in, const KMeetRoom& room, hipStream_t st) {
+  KGemvArgs a = a_in;
+  int SG, sps;
+  k6mf_split(a.nsb, SG, sps);
+  const int nwaves = kq_meet_waves(a, SG);
+  unsigned grid = 0;
+  for (int p = 0; p < a.nparts; p++) {
+    a.wg_start[p] = (int)grid;
+    grid += (unsigned)(((a.part[p].N + 15) / 16 + nwaves - 1) / nwaves);
+  }
+  a.wg_start[a.nparts] = (int)grid;
+  if (SG < 2 || sps > 8 || g_kq_meet == 0 || !room.part || (size_t)grid * nwaves * SG * 512 > room.part_bytes || grid > 1024u) return KQ_NOT_TAKEN;
+  KMeet km{};
+  km.SG = SG;
+  const int tsb = k6mf_steps(sps) / 2;
+  km.lrows = (sps + tsb - 1) / tsb * tsb;
+  km.part = static_cast<float*>(room.part);
+  RC_RET(gemv_counter_block(room.key, st, &km.counters));
+  km.cstride = 1;
+  while (km.cstride < 32 && (size_t)grid * km.cstride * 2 <= 1024u) km.cstride *= 2;
+  const size_t lds = k6mf_lds_bytes_z<MT>(sps, nwaves);
+  auto go = [&](auto kern) {
+    if (lds > 64 * 1024)
+      HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    hipLaunchKernelGGL(kern, dim3(grid, 1, (unsigned)SG), dim3(nwaves * 64), lds, st, a, 1, sps, km);
+    return (int)hipGetLastError();
+  };
+  switch (k6mf_steps(sps)) {
+    case 6: return go(kq6_gemv_mfma_kernel<XT, MT, 6>);
+    case 8: return go(kq6_gemv_mfma_kernel<XT, MT, 8>);
+    default: return go(kq6_gemv_mfma_kernel<XT, MT, K6_ST>);
+  }
 }
 template <int XT, int MT>
 static int launch_kq6_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned grid_y = 1) {
@@ -1480,11 +1576,13 @@ static int launch_kq6_mfma_t(const KGemvArgs& a_in, hipStream_t st, unsigned gri
   a.wg_start[a.nparts] = (int)grid;
   const size_t lds = k6mf_lds_bytes<MT>(a.nsb, sps, nwaves, S);
   if (lds > 160 * 1024) return MLLM_HIP_E_SHAPE;
-  const int xpad = k6mf_xpad(a.nsb, S, sps);
+  KMeet km{};
+  km.SG = 1;
+  km.lrows = a.nsb + k6mf_xpad(a.nsb, S, sps);
   auto go = [&](auto kern) {
     if (lds > 64 * 1024)
       HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    hipLaunchKernelGGL(kern, dim3(grid, grid_y), dim3(nwaves * 64), lds, st, a, S, sps, xpad);
+    hipLaunchKernelGGL(kern, dim3(grid, grid_y), dim3(nwaves * 64), lds, st, a, S, sps, km);
     return (int)hipGetLastError();
   };
   switch (k6mf_steps(sps)) {
@@ -1730,10 +1828,19 @@ MLLM_API int mllm_hip_linear_kq_multi_ws(int wtype, int nparts, const mllm_hip_g
     const bool mfma = rows >= 3 && g_kq_path != 1 &&
                       (wtype == MLLM_HIP_Q4_K ? kq4_mfma_fits(rows <= 4 ? 4 : 8, nsb)
                                               : (rows > 4 || nsb > 16 || g_kq_path == 2) && kq6_mfma_fits(rows <= 4 ? 4 : 8, nsb));
-    if (mfma && wtype == MLLM_HIP_Q4_K && room.part && g_kq_meet != 0 && kmf_slices(nsb * 8) >= g_kq_meet_min) {
+    int k6S = 1, k6sps = 0;
+    k6mf_split(nsb, k6S, k6sps);
+    // (Q6_K: from eight slices on; with four, 2560 x 4096 at eight rows, the one-workgroup form measured 12.7 us against 13.4)
+    if (mfma && room.part && g_kq_meet != 0 &&
+        (wtype == MLLM_HIP_Q4_K ? kmf_slices(nsb * 8) >= g_kq_meet_min : k6S >= (g_kq_meet == 1 ? 2 : 8))) {
       // long rows: every workgroup takes one K slice and quantizes just that part of x itself; the slices meet in the workspace
-      if (rows <= 4) rc = x_dtype == MLLM_HIP_F32 ? launch_kq4_mfma_z<MLLM_HIP_F32, 4>(a, room, st) : launch_kq4_mfma_z<MLLM_HIP_BF16, 4>(a, room, st);
-      else rc = x_dtype == MLLM_HIP_F32 ? launch_kq4_mfma_z<MLLM_HIP_F32, 8>(a, room, st) : launch_kq4_mfma_z<MLLM_HIP_BF16, 8>(a, room, st);
+      const bool f32 = x_dtype == MLLM_HIP_F32, r4 = rows <= 4;
+      if (wtype == MLLM_HIP_Q4_K)
+        rc = r4 ? (f32 ? launch_kq4_mfma_z<MLLM_HIP_F32, 4>(a, room, st) : launch_kq4_mfma_z<MLLM_HIP_BF16, 4>(a, room, st))
+                : (f32 ? launch_kq4_mfma_z<MLLM_HIP_F32, 8>(a, room, st) : launch_kq4_mfma_z<MLLM_HIP_BF16, 8>(a, room, st));
+      else
+        rc = r4 ? (f32 ? launch_kq6_mfma_z<MLLM_HIP_F32, 4>(a, room, st) : launch_kq6_mfma_z<MLLM_HIP_BF16, 4>(a, room, st))
+                : (f32 ? launch_kq6_mfma_z<MLLM_HIP_F32, 8>(a, room, st) : launch_kq6_mfma_z<MLLM_HIP_BF16, 8>(a, room, st));
       if (rc == 0) continue;
       if (rc != KQ_NOT_TAKEN) return rc;
     }

@@ -206,20 +206,20 @@ def test_matrix_core_and_dot4_kernels_agree(wtype, M):
     assert L.mllm_hip_kq_set_path(3) == -1
 
 
+@pytest.mark.parametrize("wtype", [2, 3])
 @pytest.mark.parametrize("M", [3, 4, 7, 8, 19])
-def test_q4_k_slices_that_meet_in_the_workspace_give_the_same_bits(M):
+def test_k_slices_that_meet_in_the_workspace_give_the_same_bits(wtype, M):
     """a workspace with room for partial sums: rows of more than 2560 elements are cut into K slices with a workgroup each, which
     quantize their own part of x and meet through arrival counters; the sum runs in slice order as in the one-workgroup form.
     Ragged N, several parts, bias, fp32 and bf16 activations, every workgroup shape, the workspace used again and again."""
-    wtype = 2
-    rng = synth.rng_for(7, 1300 + M)
+    rng = synth.rng_for(7, 1300 + M + 50 * wtype)
     L = _lib.lib()
     for Ns, K in (((2560,), 9728), ((2560,), 4096), ((77, 130), 4096 + 256), ((33, 16, 50, 200), 3072), ((700, 90), 2560), ((40,), 256)):
         ws = [ql.PackedKWeight(wtype, torch.from_numpy(synth.make_weight(rng, wtype, N, K))) for N in Ns]
         biases = [to_dev(rng.standard_normal(N).astype(np.float32)) if i % 2 == 0 else None for i, N in enumerate(Ns)]
         xf = synth.make_x_fp32(rng, M, K)
         for x in (to_dev(xf), to_dev(xf).to(torch.bfloat16)):
-            announce("kq4 slices meet", M, Ns, K, x.dtype)
+            announce("kq slices meet", wtype, M, Ns, K, x.dtype)
             want = ql.linear_kq_multi(ws, x, biases)                                        # no workspace
             small = ql.linear_kq_multi(ws, x, biases, workspace=ql.kq_workspace(M, K))       # image only
             room = ql.kq_workspace(M, K, sum(Ns))
