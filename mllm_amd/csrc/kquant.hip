@@ -323,7 +323,8 @@ __device__ __forceinline__ void silu_mul8(float (&v)[8], const float* u, bool ac
 // stride over the row's units.  x is quantized to Q8_K once per workgroup into LDS: codes [MT][K], scales [MT][nsb], sums
 // of 16 as int16 [MT][nsb][16].
 // U = units a lane keeps in flight per row and trip.
-template <int WT, int XT, int MT, int G, int R, int U, int LB = 256>
+// ONE: the row's units fit one trip (units <= G U): no second set of registers for the next trip.
+template <int WT, int XT, int MT, int G, int R, int U, int LB = 256, bool ONE = false>
 __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
   extern __shared__ __align__(16) unsigned char smem[];
   const int nsb = a.nsb;
@@ -462,7 +463,7 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
 
   for (int u0 = 0; u0 < units; u0 += G * U) {
     KUnit<WT> nxt[U][R];
-    const bool more = u0 + G * U < units;  // uniform
+    const bool more = !ONE && u0 + G * U < units;  // uniform
     if (more) {
 #pragma unroll
       for (int uu = 0; uu < U; uu++)
@@ -571,7 +572,7 @@ static int g_kq_G = 0, g_kq_NW = 0, g_kq_U = 0;  // tuning overrides (0 = heuris
 
 // R1: one weight row per lane group and up to 16 waves per workgroup (few rows of many units: o_proj, down_proj).  The
 // quantization of x is the long part of such a workgroup, so it is shared by as many rows as still fill the CUs.
-template <int WT, int XT, int MT, int G, int U, bool R1 = false>
+template <int WT, int XT, int MT, int G, int U, bool R1 = false, bool ONE = false>
 static int launch_kq_u(const KGemvArgs& a_in, int NW, hipStream_t st) {
   constexpr int R = R1 ? 1 : (WT == MLLM_HIP_Q4_K && MT >= 4) ? 4 : 2;  // wider row tiles reuse every LDS read for more weight rows
   constexpr int LB = R1 ? 1024 : 256;
@@ -587,7 +588,8 @@ static int launch_kq_u(const KGemvArgs& a_in, int NW, hipStream_t st) {
     grid += (unsigned)((a.part[p].N + rows_per_wg - 1) / rows_per_wg);
   }
   a.wg_start[a.nparts] = (int)grid;
-  auto kern = kq_gemv_kernel<WT, XT, MT, G, R, U, LB>;
+  if (ONE && a_in.nsb * (WT == MLLM_HIP_Q4_K ? 8 : 4) > G * U) return MLLM_HIP_E_BADARG;
+  auto kern = kq_gemv_kernel<WT, XT, MT, G, R, U, LB, ONE>;
   if (lds > 64 * 1024)
     HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
   const unsigned slots = (MT == 1 && a.slot_ids) ? (unsigned)a.slot_div_slots : 1u;
@@ -596,6 +598,19 @@ static int launch_kq_u(const KGemvArgs& a_in, int NW, hipStream_t st) {
 }
 template <int WT, int XT, int MT, int G>
 static int launch_kq_g(const KGemvArgs& a, int NW, int U, bool r1, hipStream_t st) {
+  // Q4_K, one or two rows, 32 lanes per weight row: a row of up to 96 (128 in the large workgroups) units is requested whole
+  // before the quantization of x, three (four) units per lane, instead of one trip ahead of the dot loop -- time stamps put
+  // a round trip to memory into every further trip (2560-element rows: 2.0 to 2.9 us of loop for three trips)
+  if constexpr (WT == MLLM_HIP_Q4_K && MT <= 2 && G == 32) {
+    const int units = a.nsb * 8;
+    if (!g_kq_U) {  // (a tuning override of the units in flight keeps the trips)
+      if (r1 && units <= 4 * G) return launch_kq_u<WT, XT, MT, G, 4, true, true>(a, NW, st);
+      // (one row only: with two, no gain.  117 registers = four waves per SIMD, so the 1216 workgroups of gate + up come in
+      // two rounds; asking the compiler for five waves, 96 registers, measured slower: gate + up 8.7 -> 9.1 us, q+k+v 5.35 -> 5.65)
+      if constexpr (MT == 1)
+        if (!r1 && units > 2 * G && units <= 3 * G) return launch_kq_u<WT, XT, MT, G, 3, false, true>(a, NW, st);
+    }
+  }
   if (r1 && MT <= 2 && G >= 32) return launch_kq_u<WT, XT, MT, G, (MT <= 2 && G >= 32 && WT == MLLM_HIP_Q4_K) ? 4 : 1, (MT <= 2 && G >= 32)>(a, NW, st);
   if (WT == MLLM_HIP_Q4_K && U >= 4 && MT <= 2) return launch_kq_u<WT, XT, MT, G, (WT == MLLM_HIP_Q4_K && MT <= 2) ? 4 : 1>(a, NW, st);
   if (U >= 2 && MT <= 2) return launch_kq_u<WT, XT, MT, G, MT <= 2 ? 2 : 1>(a, NW, st);

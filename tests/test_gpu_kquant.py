@@ -240,6 +240,26 @@ def test_k_slices_that_meet_in_the_workspace_give_the_same_bits(wtype, M):
     assert L.mllm_hip_linear_kq_multi_ws(wtype, 1, part, x.data_ptr(), ql._xdtype(x), M, 256, room.data_ptr(), 16, None) == -1
 
 
+@pytest.mark.parametrize("wtype", [2, 3])
+def test_units_in_flight_do_not_change_the_bits(wtype):
+    """one or two rows: a lane adds its units in the same order whether the row is requested whole before the quantization of
+    x (the default for Q4_K rows of up to 96 / 128 units) or trip by trip (mllm_hip_kq_set_tuning with units in flight)"""
+    rng = synth.rng_for(7, 1500 + wtype)
+    L = _lib.lib()
+    for M in (1, 2):
+        for N, K in ((1000, 2560), (300, 4096), (70, 768), (2560, 2560 + 512)):
+            w = ql.PackedKWeight(wtype, torch.from_numpy(synth.make_weight(rng, wtype, N, K)))
+            x = to_dev(synth.make_x_fp32(rng, M, K)).to(torch.bfloat16)
+            announce("kq units in flight", wtype, M, N, K)
+            want = ql.linear_kq(w, x)
+            try:
+                for u in (1, 2, 4):
+                    assert L.mllm_hip_kq_set_tuning(0, 0, u) == 0
+                    assert torch.equal(want, ql.linear_kq(w, x)), u
+            finally:
+                assert L.mllm_hip_kq_set_tuning(0, 0, 0) == 0
+
+
 def test_argument_checks():
     L = _lib.lib()
     buf = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
