@@ -48,6 +48,13 @@ __global__ __launch_bounds__(512) void moe_decode_gateup_kernel(MoeDecodeArgs a)
   const int n0 = blockIdx.x * 32;
   const QImage out{a.img + (size_t)slot * a.img_stride, 1, a.I / QK, a.x86};
   float* s_h = reinterpret_cast<float*>(smem + align_up((size_t)nb * 40, 16));
+  // activations of the token first, weights behind them (requests return in order); the activations do not wait for the
+  // slot's expert id either, which the weight addresses need
+  const int nitems = nb * 4;
+  XRaw<XT> raw;
+  load_x8<XT>(a.x, ((int64_t)tok * nb * 4 + min(tid, nitems - 1)) * 8, raw);
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
   if (e < 0 || e >= a.E) {  // uniform: this slot contributes nothing; its image block reads as zeros
     if (tid < 4) {
       const float z[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
@@ -55,12 +62,6 @@ __global__ __launch_bounds__(512) void moe_decode_gateup_kernel(MoeDecodeArgs a)
     }
     return;
   }
-  // activations of the token first, weights behind them (requests return in order)
-  const int nitems = nb * 4;
-  XRaw<XT> raw;
-  load_x8<XT>(a.x, ((int64_t)tok * nb * 4 + min(tid, nitems - 1)) * 8, raw);
-  __asm__ volatile("" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
 
   const int grp = lane >> 4, c0 = lane & 15;
   const int n = n0 + 4 * wave + grp;
@@ -168,12 +169,25 @@ __global__ __launch_bounds__(DNW * 64) void moe_decode_down_kernel(MoeDecodeArgs
   // token's experts is a chain of exposed load latencies (8.8 us for eight experts, 7 MB)
   constexpr int PF = WT == MLLM_HIP_Q4_0 ? 8 : 4;
   Chunk buf[PF];
-#pragma unroll
-  for (int p = 0; p < PF; p++) load_expert(p, buf[p]);  // slots past k load the last expert again and are not used
-  // the images of this token's k slots are contiguous
+  // the images of this token's k slots are contiguous; their first pieces are requested ahead of the weights (requests
+  // return in order, and the addresses of the weights wait for the expert ids)
   const int n16 = a.k * a.img_stride / 16;
   const u32x4* src = reinterpret_cast<const u32x4*>(a.img + (size_t)tok * a.k * a.img_stride);
-  for (int c = tid; c < n16; c += DNW * 64) reinterpret_cast<u32x4*>(smem)[c] = src[c];
+  constexpr int IP = 4;
+  u32x4 ip[IP];
+#pragma unroll
+  for (int i = 0; i < IP; i++)
+    if (tid + i * DNW * 64 < n16) ip[i] = src[tid + i * DNW * 64];
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int p = 0; p < PF; p++) load_expert(p, buf[p]);  // slots past k load the last expert again and are not used
+  __asm__ volatile("" ::: "memory");
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int i = 0; i < IP; i++)
+    if (tid + i * DNW * 64 < n16) reinterpret_cast<u32x4*>(smem)[tid + i * DNW * 64] = ip[i];
+  for (int c = tid + IP * DNW * 64; c < n16; c += DNW * 64) reinterpret_cast<u32x4*>(smem)[c] = src[c];
   __syncthreads();
 
   float total = 0.f;
