@@ -59,8 +59,8 @@ def parse():
     ap.add_argument("--brief", action="store_true",
                     help="with --side-only: one untimed and one timed replay per workload (counter runs: fewer dispatches to record)")
     ap.add_argument("--layer-only", action="store_true",
-                    help="profiling run: only the decoder-layer chain (operators one by one and folded, M = 1 and 8) and the "
-                         "Q4_K / Q6_K gate projection, printed as one JSON object; meant to run under rocprofv3")
+                    help="profiling run: only the decoder-layer chain (operators one by one and folded, M = 1 and 8), the "
+                         "Q4_K / Q6_K gate projection at one row and the four launches of a Q4_K / Q6_K layer at eight, printed as one JSON object; meant to run under rocprofv3")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--request-order", type=int, default=-1, choices=[-1, 0, 1],
                     help="mllm_hip_gemv_set_request_order: -1 the library's rule (default), 0 / 1 never / always deferred (comparison runs)")
@@ -542,6 +542,23 @@ def main():
             _, ev = timed(graphed(lambda: [ql.linear_kq(w, x1, out=y1) for w in ws]), 3, 2)
             res["%s_gate_proj_us" % kname] = ev / (3 * N_LAYERS) * 1e6
             del ws
+            # the four launches of a layer (q+k+v | o | gate+up | down) at eight rows over 12 layers' weights, with workspaces
+            # that have room for the partial sums of K slices
+            kpool = [{name: ql.PackedKWeight.synthetic(kt, n, k, gen) for name, (n, k) in shapes.items()} for _ in range(12)]
+            xs8 = {k: torch.randn((8, k), device="cuda", generator=gen).to(torch.bfloat16) for k in (2560, 4096, 9728)}
+            ys8 = {name: torch.empty((8, n), dtype=torch.float32, device="cuda") for name, (n, _) in shapes.items()}
+            kws = {k: ql.kq_workspace(8, k, 2 * 9728) for k in (2560, 4096, 9728)}
+
+            def klayers():
+                for l in kpool:
+                    ql.linear_kq_multi([l["q_proj"], l["k_proj"], l["v_proj"]], xs8[2560], None, [ys8["q_proj"], ys8["k_proj"], ys8["v_proj"]],
+                                       workspace=kws[2560])
+                    ql.linear_kq(l["o_proj"], xs8[4096], out=ys8["o_proj"], workspace=kws[4096])
+                    ql.linear_kq_multi([l["gate_proj"], l["up_proj"]], xs8[2560], None, [ys8["gate_proj"], ys8["up_proj"]], workspace=kws[2560])
+                    ql.linear_kq(l["down_proj"], xs8[9728], out=ys8["down_proj"], workspace=kws[9728])
+            _, ev = timed(graphed(klayers), 3, 2)
+            res["%s_layer_m8_us" % kname] = ev / (3 * 12) * 1e6
+            del kpool
         print(json.dumps(res))
         return
 
