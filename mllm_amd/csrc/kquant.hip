@@ -372,11 +372,14 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
   const int nitems = MT * (K >> 3);
   const int valid = a.M * (K >> 3);
   constexpr int XL = XT == KQ_IMAGE ? MLLM_HIP_F32 : XT;
-  u32x4 raw[2][XL == MLLM_HIP_F32 ? 2 : 1];
+  // (two rows: four items, or rows of 2560 elements leave half an item per thread to the loop further down, where it comes
+  // back behind the weights)
+  constexpr int NPRE = MT == 2 ? 4 : 2;
+  u32x4 raw[NPRE][XL == MLLM_HIP_F32 ? 2 : 1];
   u32x4 raw2[2][2];
   if (XT != KQ_IMAGE) {
 #pragma unroll
-    for (int k = 0; k < 2; k++) {
+    for (int k = 0; k < NPRE; k++) {
       const int it = min(tid + k * nthreads, valid - 1);
       if (XL == MLLM_HIP_F32) {
         const u32x4* p = reinterpret_cast<const u32x4*>(reinterpret_cast<const float*>(xp) + (int64_t)it * 8);
@@ -422,7 +425,7 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
   };
   if (XT != KQ_IMAGE) {
 #pragma unroll
-    for (int k = 0; k < 2; k++) {  // whole half-waves: nitems is a multiple of 32
+    for (int k = 0; k < NPRE; k++) {  // whole half-waves: nitems is a multiple of 32
       const int it = tid + k * nthreads;
       if (it < nitems) {
         float v[8];
@@ -442,11 +445,11 @@ __global__ __launch_bounds__(LB) void kq_gemv_kernel(KGemvArgs a) {
 #pragma unroll
           for (int e = 0; e < 8; e++) v[e] = 0.f;
         }
-        if (XT == MLLM_HIP_F32 && MT == 1 && x2p) silu_mul8(v, reinterpret_cast<const float*>(&raw2[k][0]), a.silu_accurate);
+        if (XT == MLLM_HIP_F32 && MT == 1 && x2p) silu_mul8(v, reinterpret_cast<const float*>(&raw2[k < 2 ? k : 0][0]), a.silu_accurate);
         quantize_to_lds(it, v);
       }
     }
-    for (int it = tid + 2 * nthreads; it < nitems; it += nthreads) {
+    for (int it = tid + NPRE * nthreads; it < nitems; it += nthreads) {
       float v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
       if (it < valid) load8<XL>(xp, (int64_t)it * 8, v);
       if (XT == MLLM_HIP_F32 && MT == 1 && x2p) silu_mul8(v, x2p + (int64_t)min(it, valid - 1) * 8, a.silu_accurate);

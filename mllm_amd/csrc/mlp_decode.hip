@@ -58,9 +58,16 @@ __global__ __launch_bounds__(32 * G) void mlp_gateup_kernel(MlpArgs a) {
   // requests return in order: activations first, then the scales, then the weights
   const int nitems = mnb * 4, valid = a.M * nb * 4;
   const int img_chunks = (mnb * 5 + 1) / 2;
-  XRaw<XT> raw;
+  // (two rows: a second item per thread is requested here too -- one requested in the quantization loop comes back behind
+  // the weights)
+  constexpr int NPRE = MT == 1 ? 1 : 2;
+  XRaw<XT> raw, raw2;
   if (XT == GEMV_PREQ) raw.r[0] = reinterpret_cast<const u32x4*>(a.x)[min(tid, img_chunks - 1)];
   else load_x8<XT>(a.x, (int64_t)min(tid, valid - 1) * 8, raw);
+  if (NPRE > 1) {
+    if (XT == GEMV_PREQ) raw2.r[0] = reinterpret_cast<const u32x4*>(a.x)[min(tid + NTHR, img_chunks - 1)];
+    else load_x8<XT>(a.x, (int64_t)min(tid + NTHR, valid - 1) * 8, raw2);
+  }
 
   const int grp = lane / G, c0 = lane % G;
   const int nw0 = n0 + GROUPS * wave;  // first channel of this wave
@@ -103,7 +110,8 @@ __global__ __launch_bounds__(32 * G) void mlp_gateup_kernel(MlpArgs a) {
   if (XT == GEMV_PREQ) {
     u32x4* s16 = reinterpret_cast<u32x4*>(smem);
     if (tid < img_chunks) s16[tid] = raw.r[0];
-    for (int c = tid + NTHR; c < img_chunks; c += NTHR) s16[c] = reinterpret_cast<const u32x4*>(a.x)[c];
+    if (NPRE > 1 && tid + NTHR < img_chunks) s16[tid + NTHR] = raw2.r[0];
+    for (int c = tid + NPRE * NTHR; c < img_chunks; c += NTHR) s16[c] = reinterpret_cast<const u32x4*>(a.x)[c];
   } else {
     const QImage xi{smem, MT, nb, a.x86};
     float v[8];
@@ -113,7 +121,16 @@ __global__ __launch_bounds__(32 * G) void mlp_gateup_kernel(MlpArgs a) {
       for (int e = 0; e < 8; e++) v[e] = 0.f;
     }
     if (tid < nitems) quad_quantize_to_image(v, xi, 0, tid >> 2, tid & 3, true);  // block index runs over m * nb + b
-    for (int it = tid + NTHR; it < nitems; it += NTHR) {
+    if (NPRE > 1) {
+      const int it = tid + NTHR;
+      x8_to_f32<XT>(raw2, v);
+      if (it >= valid) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) v[e] = 0.f;
+      }
+      if (it < nitems) quad_quantize_to_image(v, xi, 0, it >> 2, it & 3, true);  // whole quads: nitems and NTHR are multiples of 4
+    }
+    for (int it = tid + NPRE * NTHR; it < nitems; it += NTHR) {
       XRaw<XT> rw;
       load_x8<XT>(a.x, (int64_t)min(it, valid - 1) * 8, rw);
       x8_to_f32<XT>(rw, v);
