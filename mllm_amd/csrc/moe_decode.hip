@@ -324,13 +324,12 @@ __device__ __forceinline__ void moe_rows_gateup(const MoeRowsArgs& b, const int 
       }
     }
   };
-  load_trip(0);
-  __asm__ volatile("" ::: "memory");
-  __builtin_amdgcn_sched_barrier(0);
-
   // the rows' activations -> Q8_0 images in LDS, four requests in flight per thread; items are eighths of a block, so the four
-  // lanes of a quad always hold one block of one row
+  // lanes of a quad always hold one block of one row.  The first trip of weights is requested right behind the first batch
+  // of activations (requests return in order: ahead of them it would hold the activations back, whose addresses already
+  // wait for the sorted positions; 32 / 64 tokens of the 128-expert layer: 63.0 / 93.0 -> 61.4 / 90.5 us)
   const int nitems = nb * 4, total = rows * nitems;
+  if (tid >= total) load_trip(0);  // (threads without an item)
   for (int it0 = tid; it0 < total; it0 += 512 * 4) {
     XRaw<XT> raw[4];
     int rr[4], ii[4];
@@ -342,6 +341,7 @@ __device__ __forceinline__ void moe_rows_gateup(const MoeRowsArgs& b, const int 
       const int tok = b.sorted_idx[row0 + rr[q]] / a.k;
       load_x8<XT>(a.x, ((int64_t)tok * nitems + ii[q]) * 8, raw[q]);
     }
+    if (it0 == tid) load_trip(0);
 #pragma unroll
     for (int q = 0; q < 4; q++) {
       if (it0 + 512 * q < total) {  // the same answer in the four lanes of a quad: total and the strides are multiples of 4
