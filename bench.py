@@ -581,7 +581,7 @@ def main():
              "graph": not args.no_graph, "layers": N_LAYERS, "launches_per_step": N_LAYERS * (len(shapes) if args.per_op else 4)}
     if not args.no_extra:
         extra["decode_layer_chain"] = {"m%d" % M: measure_layer_chain(pool, M) for M in (1, 4, 8)}
-        for M in (4, 8):
+        for M in (2, 4, 8):
             if M != args.m:
                 r = measure_workload(wtype, M, pool, max(5, args.steps // 3), 2)
                 extra["%s_m%d" % (args.wtype, M)] = {"GBps": r["GBps"], "ms_per_step": r["ms_per_step"],
@@ -597,7 +597,7 @@ def main():
         other = ql.Q8_0 if wtype == ql.Q4_0 else ql.Q4_0
         oname = "q8_0" if wtype == ql.Q4_0 else "q4_0"
         pool2 = make_pool(other, N_LAYERS)
-        for M in (1, 4, 8):
+        for M in (1, 2, 4, 8):
             r = measure_workload(other, M, pool2, max(5, args.steps // 3), 2)
             extra["%s_m%d" % (oname, M)] = {"GBps": r["GBps"], "ms_per_step": r["ms_per_step"],
                                             dom_name: measure_shape(other, M, dom_name, pool2, 3)}
