@@ -79,6 +79,11 @@ def _cases():
         "mllm_hip_linear_kq": ([Q6_K, P, P, F32, None, P, 1, 8, 256, P, None],
                                [(0, Q8_0, BADARG), (1, None, BADARG), (2, None, BADARG), (5, None, BADARG), (9, ODD, ALIGN),
                                 (8, 320, SHAPE), (6, 0, BADARG)]),
+        # the workspace of stated size: one smaller than the Q8_K image of eight rows is refused
+        "mllm_hip_linear_kq_multi_ws": ([Q4_K, 1, part, P, BF16, 4, 256, P, 8 * 256 + 8 * 36, None],
+                                        [(0, Q4_0, BADARG), (1, 0, BADARG), (1, 5, BADARG), (2, None, BADARG), (3, None, BADARG),
+                                         (4, IMAGE, BADARG), (5, 0, BADARG), (6, 320, SHAPE), (7, ODD, ALIGN), (8, 8 * 256 + 8 * 36 - 1, BADARG)]),
+        "mllm_hip_kq_set_slice_meeting": ([-1, 0], [(0, 2, BADARG), (0, -2, BADARG), (1, 9, BADARG), (1, -1, BADARG)]),
         "mllm_hip_kq_gemm_prepack": ([Q4_K, P, 0, P, 8, 256, None], [(0, Q8_0, BADARG), (1, None, BADARG), (5, 96, SHAPE)]),
         "mllm_hip_linear_kq_gemm": ([Q4_K, P, P, F32, None, P, 16, 8, 256, P, None],
                                     [(0, Q4_0, BADARG), (1, None, BADARG), (5, None, BADARG), (9, None, BADARG), (8, 100, SHAPE)]),
@@ -146,3 +151,8 @@ def test_size_helpers_return_zero_for_shapes_they_do_not_take():
     assert L.mllm_hip_moe_gemm_workspace_bytes(4, 64, 64, 0, 2) == 0
     assert L.mllm_hip_w4a16_packed_bytes(64, 256, 100) == 0
     assert L.mllm_hip_moe_kq_workspace_bytes(4, 128, 256, 8, 2) == 0
+    assert L.mllm_hip_kq_workspace_bytes_n(4, 128, 64) == 0
+    # room for partial sums only where a row has K slices: 256 elements have none, 4096 have four
+    assert 0 <= L.mllm_hip_kq_workspace_bytes_n(4, 256, 64) - L.mllm_hip_kq_workspace_bytes(4, 256) < 256
+    assert L.mllm_hip_kq_workspace_bytes_n(4, 4096, 64) >= L.mllm_hip_kq_workspace_bytes(4, 4096) + 4 * 4 * 512
+    assert L.mllm_hip_kq_workspace_bytes_n(4, 4096, 0) == L.mllm_hip_kq_workspace_bytes(4, 4096)
