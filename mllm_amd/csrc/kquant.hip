@@ -692,6 +692,11 @@ static int launch_kq(const KGemvArgs& a, hipStream_t st) {
 //   acc = fma(fp32(d*sc) * dx, float(isum), acc);  acc = fma(-(fp32(dmin*m) * dx), float(sum of the row's 32 codes), acc)
 // the reference's sum (vec_dot_q4_K_q8_K: integer sums per super-block, then d*dx and dmin*dx) regrouped; the integer parts
 // are exact, the fp32 roundings differ in order only.
+// Order and batching of the requests in front of the loop (measured on the 4B layer shapes; the values compiled in are the
+// fastest): KMF_WEIGHTS_FIRST 1 asks for the slice's weights before the quantized image is copied -- the image, which every
+// wave needs before the first barrier, then comes back behind them (layer at eight rows 58.3 us against 54.2);
+// KMF_COPY_UNROLL = image pieces a thread requests before it stores the first (10: the down projection gets slower);
+// KMF_QUANT_BATCH = activation items a thread requests before it quantizes the first.
 #ifndef KMF_WEIGHTS_FIRST
 #define KMF_WEIGHTS_FIRST 0
 #endif
