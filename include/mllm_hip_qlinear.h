@@ -517,12 +517,17 @@ int mllm_hip_softmax(const float* x, float* y, int64_t rows, int64_t len, void* 
  * replaces: CPUTopKOp::forward  mllm/backends/cpu/ops/TopKOp.cpp:20-72 */
 int mllm_hip_topk(const float* x, float* values, int32_t* indices, int64_t rows, int64_t len, int k, int largest, int sorted,
                   void* stream);
-/* The MoE gate in one launch: scores = softmax(x . W^T) in fp32, the k largest per token in index order, weights divided
- * by their sum when norm_topk_prob.  x [M][H] fp32 or bf16; gate_weight fp32 [E][H]; topk_ids int32 [M][k]; topk_weights
- * fp32 [M][k]; scores fp32 [M][E] or NULL.  H % 8 == 0.
+/* The MoE gate: scores = softmax(x . W^T) in fp32, the k largest per token in index order, weights divided by their sum
+ * when norm_topk_prob.  x [M][H] fp32 or bf16; gate_weight fp32 [E][H]; topk_ids int32 [M][k]; topk_weights fp32 [M][k];
+ * scores fp32 [M][E] or NULL.  H % 8 == 0.  With a scores buffer the call is two launches -- the logits with the experts
+ * spread over the grid (the buffer holds them in between), then one wave per token for softmax and selection -- which is
+ * what a decode token wants (1 MB of gate weights for 128 experts: 6 us against 26 through the single workgroup of the
+ * one-launch form, which callers without a scores buffer get).  Same logits, scores and selection either way.
  * replaces: MoEGate::forward  mllm/models/qwen3_moe/modeling_qwen3_moe_fa2.hpp:121-139 */
 int mllm_hip_moe_gate(const void* x, int x_dtype, const float* gate_weight, int32_t* topk_ids, float* topk_weights, float* scores,
                       int64_t M, int64_t H, int64_t E, int k, int norm_topk_prob, void* stream);
+/* 0: the one-launch form also where a scores buffer is given (comparison runs and tests); 1: the default */
+int mllm_hip_moe_gate_set_form(int two_launches);
 
 /* ---------------------------------------------------------------------------------------------------------
  * Activation x activation MatMul on the matrix cores (the backend's kMatMul slot; not a quantized path)

@@ -284,6 +284,40 @@ __device__ __forceinline__ void wave_topk(const float* vals, int len, int k, boo
   }
 }
 
+// The same selection for a row of up to 64 R elements in LDS, by rank: a lane keeps its R elements (index lane + 64 j) and counts,
+// over one pass of broadcast reads, how many elements of the row come before each of them in the order above; the elements
+// of rank < k are the selection, rank = place by value, and the place by index is a count over ballots.  One pass instead of
+// k rounds of wave-wide extremes (each six exchanges through the LDS pipe): the gate's 8 of 128 take a fifth of the time.
+template <int R>
+__device__ __forceinline__ void wave_topk_ranked(const float* vals, int len, int k, bool largest, bool sorted, float* out_v, int* out_i,
+                                                 int lane) {
+  float v[R];
+  int rank[R];
+#pragma unroll
+  for (int j = 0; j < R; j++) {
+    v[j] = lane + 64 * j < len ? vals[lane + 64 * j] : 0.f;
+    rank[j] = 0;
+  }
+  for (int o = 0; o < len; o++) {
+    const float ov = vals[o];  // every lane the same address
+#pragma unroll
+    for (int j = 0; j < R; j++) rank[j] += comes_before(ov, o, v[j], lane + 64 * j, largest) ? 1 : 0;
+  }
+  unsigned long long m[R];
+#pragma unroll
+  for (int j = 0; j < R; j++) m[j] = __ballot(lane + 64 * j < len && rank[j] < k);
+  int before = 0;  // selected elements of the lower sixty-fours
+#pragma unroll
+  for (int j = 0; j < R; j++) {
+    if (lane + 64 * j < len && rank[j] < k) {
+      const int pos = sorted ? rank[j] : before + __popcll(m[j] & ((1ull << lane) - 1ull));
+      out_v[pos] = v[j];
+      out_i[pos] = lane + 64 * j;
+    }
+    before += __popcll(m[j]);
+  }
+}
+
 __global__ __launch_bounds__(256) void topk_rows_kernel(const float* __restrict__ x, float* __restrict__ values, int32_t* __restrict__ indices,
                                                         int64_t rows, int len, int k, int largest, int sorted) {
   const int lane = threadIdx.x & 63;
@@ -310,18 +344,11 @@ struct GateArgs {
 };
 constexpr int GATE_TOK = 4;
 constexpr int GATE_WAVES = 16;
+// x of the workgroup's ntok tokens -> fp32 in LDS
 template <int XT>
-__global__ __launch_bounds__(GATE_WAVES * 64) void moe_gate_kernel(GateArgs a) {
-  extern __shared__ __align__(16) unsigned char smem[];
-  float* s_x = reinterpret_cast<float*>(smem);     // [GATE_TOK][H]
-  float* s_logit = s_x + (size_t)GATE_TOK * a.H;   // [GATE_TOK][E]
-  float* s_tv = s_logit + (size_t)GATE_TOK * a.E;  // [GATE_TOK][k]
-  int* s_ti = reinterpret_cast<int*>(s_tv + (size_t)GATE_TOK * a.k);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t tok0 = (int64_t)blockIdx.x * GATE_TOK;
-  const int ntok = (int)min((int64_t)GATE_TOK, a.M - tok0);  // uniform
+__device__ __forceinline__ void gate_stage_x(const GateArgs& a, int64_t tok0, int ntok, float* s_x, int tid, int nthreads) {
   const int ipr = a.H >> 3, nitems = ntok * ipr;
-  for (int it = tid; it < nitems; it += GATE_WAVES * 64) {  // (four tokens of 2048 elements: one item per thread)
+  for (int it = tid; it < nitems; it += nthreads) {  // (four tokens of 2048 elements, 1024 threads: one item per thread)
     const int t = it / ipr, c = it - t * ipr;
     float v[8];
     Item8<XT> r;
@@ -331,10 +358,13 @@ __global__ __launch_bounds__(GATE_WAVES * 64) void moe_gate_kernel(GateArgs a) {
     dst[0] = f32x4{v[0], v[1], v[2], v[3]};
     dst[1] = f32x4{v[4], v[5], v[6], v[7]};
   }
-  __syncthreads();
+}
+// logits of experts e0 + wave, e0 + wave + nwaves, ... < e1 for the ntok tokens in s_x; out[t * ostride + e]
+__device__ __forceinline__ void gate_logits(const GateArgs& a, const float* s_x, int ntok, int e0, int e1, int wave, int nwaves, int lane,
+                                            float* out, size_t ostride) {
   constexpr int CB = 8;  // pieces of a row a lane requests before it multiplies the first
   const int nc = a.H >> 2;
-  for (int e = wave; e < a.E; e += GATE_WAVES) {
+  for (int e = e0 + wave; e < e1; e += nwaves) {
     float acc[GATE_TOK] = {0.f, 0.f, 0.f, 0.f};
     const f32x4* wr = reinterpret_cast<const f32x4*>(a.w + (size_t)e * a.H);
     for (int c0 = lane; c0 < nc; c0 += 64 * CB) {
@@ -363,14 +393,13 @@ __global__ __launch_bounds__(GATE_WAVES * 64) void moe_gate_kernel(GateArgs a) {
     for (int t = 0; t < GATE_TOK; t++) {
       if (t < ntok) {
         const float s = wave_sum(acc[t]);
-        if (lane == 0) s_logit[t * a.E + e] = s;
+        if (lane == 0) out[t * ostride + e] = s;
       }
     }
   }
-  __syncthreads();
-  const int64_t tok = tok0 + wave;
-  if (wave >= ntok) return;
-  float* lg = s_logit + wave * a.E;
+}
+// one wave finishes one token: softmax over its E logits in lg (LDS, overwritten), the k largest in index order, weights
+__device__ __forceinline__ void gate_select(const GateArgs& a, float* lg, int64_t tok, float* tv, int* ti, int lane) {
   const bool poly = a.E > 16 && !a.exp_accurate;
   float mx = -3.402823466e+38f;
   for (int i = lane; i < a.E; i += 64) mx = fmaxf(mx, lg[i]);
@@ -391,17 +420,67 @@ __global__ __launch_bounds__(GATE_WAVES * 64) void moe_gate_kernel(GateArgs a) {
   // LDS writes of this wave are read back by other lanes of the same wave only
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
-  wave_topk(lg, a.E, a.k, true, false, s_tv + wave * a.k, s_ti + wave * a.k, lane);
+  if (a.E <= 128) wave_topk_ranked<2>(lg, a.E, a.k, true, false, tv, ti, lane);
+  else if (a.E <= 256) wave_topk_ranked<4>(lg, a.E, a.k, true, false, tv, ti, lane);
+  else wave_topk(lg, a.E, a.k, true, false, tv, ti, lane);
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   // topk(..., largest = true, sorted = false): by index; then weight / sum(weights) in index order
   float tsum = 0.f;
-  for (int r = 0; r < a.k; r++) tsum += s_tv[wave * a.k + r];
+  for (int r = 0; r < a.k; r++) tsum += tv[r];
   for (int r = lane; r < a.k; r += 64) {
-    const float wv = s_tv[wave * a.k + r];
+    const float wv = tv[r];
     a.weights[tok * a.k + r] = a.norm ? wv / tsum : wv;
-    a.ids[tok * a.k + r] = s_ti[wave * a.k + r];
+    a.ids[tok * a.k + r] = ti[r];
   }
+}
+// everything in one launch: a workgroup per four tokens (callers that pass no scores buffer)
+template <int XT>
+__global__ __launch_bounds__(GATE_WAVES * 64) void moe_gate_kernel(GateArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* s_x = reinterpret_cast<float*>(smem);     // [GATE_TOK][H]
+  float* s_logit = s_x + (size_t)GATE_TOK * a.H;   // [GATE_TOK][E]
+  float* s_tv = s_logit + (size_t)GATE_TOK * a.E;  // [GATE_TOK][k]
+  int* s_ti = reinterpret_cast<int*>(s_tv + (size_t)GATE_TOK * a.k);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t tok0 = (int64_t)blockIdx.x * GATE_TOK;
+  const int ntok = (int)min((int64_t)GATE_TOK, a.M - tok0);  // uniform
+  gate_stage_x<XT>(a, tok0, ntok, s_x, tid, GATE_WAVES * 64);
+  __syncthreads();
+  gate_logits(a, s_x, ntok, 0, a.E, wave, GATE_WAVES, lane, s_logit, (size_t)a.E);
+  __syncthreads();
+  if (wave >= ntok) return;
+  gate_select(a, s_logit + wave * a.E, tok0 + wave, s_tv + wave * a.k, s_ti + wave * a.k, lane);
+}
+// The same in two launches for callers that pass a scores buffer, which holds the logits in between: with few tokens one
+// workgroup per four tokens leaves the chip to one CU (a decode token: 1 MB of gate weights through one workgroup), so the
+// experts are spread over the grid's y -- epg experts and as many waves per workgroup -- and a second, small launch
+// finishes each token.  Same logits, same selection.
+template <int XT>
+__global__ __launch_bounds__(GATE_WAVES * 64) void moe_gate_logits_kernel(GateArgs a, int epg) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* s_x = reinterpret_cast<float*>(smem);  // [GATE_TOK][H]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x;
+  const int64_t tok0 = (int64_t)blockIdx.x * GATE_TOK;
+  const int ntok = (int)min((int64_t)GATE_TOK, a.M - tok0);  // uniform
+  gate_stage_x<XT>(a, tok0, ntok, s_x, tid, nthreads);
+  __syncthreads();
+  const int e0 = (int)blockIdx.y * epg;
+  gate_logits(a, s_x, ntok, e0, min(a.E, e0 + epg), wave, nthreads >> 6, lane, a.scores + tok0 * a.E, (size_t)a.E);
+}
+__global__ __launch_bounds__(GATE_TOK * 64) void moe_gate_select_kernel(GateArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  float* s_logit = reinterpret_cast<float*>(smem);  // [GATE_TOK][E]
+  float* s_tv = s_logit + (size_t)GATE_TOK * a.E;   // [GATE_TOK][k]
+  int* s_ti = reinterpret_cast<int*>(s_tv + (size_t)GATE_TOK * a.k);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t tok = (int64_t)blockIdx.x * GATE_TOK + wave;
+  if (tok >= a.M) return;  // (no workgroup barrier below)
+  float* lg = s_logit + wave * a.E;
+  for (int i = lane; i < a.E; i += 64) lg[i] = a.scores[tok * a.E + i];
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  gate_select(a, lg, tok, s_tv + wave * a.k, s_ti + wave * a.k, lane);
 }
 
 }  // namespace mllmhip
@@ -517,6 +596,13 @@ MLLM_API int mllm_hip_topk(const float* x, float* values, int32_t* indices, int6
   return (int)hipGetLastError();
 }
 
+static int g_gate_two_launches = 1;  // 0: the one-launch form also where a scores buffer is given (comparison runs and tests)
+MLLM_API int mllm_hip_moe_gate_set_form(int two_launches) {
+  if (two_launches != 0 && two_launches != 1) return MLLM_HIP_E_BADARG;
+  g_gate_two_launches = two_launches;
+  return 0;
+}
+
 MLLM_API int mllm_hip_moe_gate(const void* x, int x_dtype, const float* gate_weight, int32_t* topk_ids, float* topk_weights,
                                float* scores, int64_t M, int64_t H, int64_t E, int k, int norm_topk_prob, void* stream) {
   if (!x || !gate_weight || !topk_ids || !topk_weights || !dtype_ok(x_dtype) || M <= 0 || H <= 0 || E <= 0) return MLLM_HIP_E_BADARG;
@@ -527,6 +613,22 @@ MLLM_API int mllm_hip_moe_gate(const void* x, int x_dtype, const float* gate_wei
   GateArgs a{x, gate_weight, topk_ids, topk_weights, scores, M, (int)H, (int)E, k, norm_topk_prob, g_exp_accurate};
   const unsigned grid = (unsigned)((M + GATE_TOK - 1) / GATE_TOK);
   hipStream_t st = (hipStream_t)stream;
+  if (scores && g_gate_two_launches) {
+    // experts per workgroup: four (one per wave) while the token groups alone do not fill the chip, else sixteen
+    const int epg = grid >= 64 ? 16 : 4;
+    const size_t lds1 = (size_t)GATE_TOK * H * 4, lds2 = ((size_t)GATE_TOK * E + (size_t)2 * GATE_TOK * k) * 4;
+    auto go = [&](auto kern) -> int {
+      if (lds1 > 64 * 1024)
+        HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds1));
+      hipLaunchKernelGGL(kern, dim3(grid, (unsigned)((E + epg - 1) / epg)), dim3(64 * epg), lds1, st, a, epg);
+      return (int)hipGetLastError();
+    };
+    RC_RET(x_dtype == MLLM_HIP_F32 ? go(moe_gate_logits_kernel<MLLM_HIP_F32>) : go(moe_gate_logits_kernel<MLLM_HIP_BF16>));
+    if (lds2 > 64 * 1024)
+      HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(moe_gate_select_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds2));
+    hipLaunchKernelGGL(moe_gate_select_kernel, dim3(grid), dim3(GATE_TOK * 64), lds2, st, a);
+    return (int)hipGetLastError();
+  }
   auto launch = [&](auto kern) -> int {
     if (lds > 64 * 1024)
       HIP_RET(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));

@@ -518,14 +518,15 @@ def topk(x, k, largest=True, sorted=True):
     return v, i
 
 
-def moe_gate(x, gate_weight, k, norm_topk_prob=True, want_scores=False):
-    """x [M, H] fp32 or bf16, gate_weight fp32 [E, H] -> (ids int32 [M, k], weights fp32 [M, k][, scores fp32 [M, E]])"""
+def moe_gate(x, gate_weight, k, norm_topk_prob=True, want_scores=False, scores=None):
+    """x [M, H] fp32 or bf16, gate_weight fp32 [E, H] -> (ids int32 [M, k], weights fp32 [M, k][, scores fp32 [M, E]]).
+    scores: a buffer fp32 [M, E] to use (with one -- want_scores allocates it -- the call takes the two-launch form)"""
     assert x.is_cuda and x.is_contiguous() and x.dim() == 2 and gate_weight.dtype == torch.float32 and gate_weight.is_contiguous()
     M, H = x.shape
     E = gate_weight.shape[0]
     ids = torch.empty((M, k), dtype=torch.int32, device="cuda")
     wt = torch.empty((M, k), dtype=torch.float32, device="cuda")
-    sc = torch.empty((M, E), dtype=torch.float32, device="cuda") if want_scores else None
+    sc = scores if scores is not None else (torch.empty((M, E), dtype=torch.float32, device="cuda") if want_scores else None)
     _lib.check(_lib.lib().mllm_hip_moe_gate(x.data_ptr(), _xdtype(x), gate_weight.data_ptr(), ids.data_ptr(), wt.data_ptr(),
                                             _p(sc), M, H, E, k, int(norm_topk_prob), _stream()), "mllm_hip_moe_gate")
     return (ids, wt, sc) if want_scores else (ids, wt)

@@ -281,6 +281,16 @@ def test_moe_gate(M, H, E, k, dtype):
     for norm in (True, False):
         announce("moe gate", M, H, E, k, dtype, norm)
         ids, wt, sc = ql.moe_gate(x, to_dev(w), k, norm, want_scores=True)
+        # the two forms -- logits with the experts spread over the grid and a second launch per token (with a scores buffer),
+        # everything in one workgroup per four tokens (without, or forced) -- give the same bits
+        L = _lib.lib()
+        i1, w1 = ql.moe_gate(x, to_dev(w), k, norm)
+        assert L.mllm_hip_moe_gate_set_form(0) == 0
+        try:
+            i0, w0, s0 = ql.moe_gate(x, to_dev(w), k, norm, want_scores=True)
+        finally:
+            assert L.mllm_hip_moe_gate_set_form(1) == 0
+        assert torch.equal(ids, i1) and torch.equal(wt, w1) and torch.equal(ids, i0) and torch.equal(wt, w0) and torch.equal(sc, s0)
         ids, wt, sc = ids.cpu().numpy(), wt.cpu().numpy(), sc.cpu().numpy()
         oi, ow, osc = orc.moe_gate(xf, w, k, norm)
         assert rel_l2(sc, osc) < 1e-5
@@ -313,6 +323,7 @@ def test_argument_checks():
     assert L.mllm_hip_topk(p, p, p, 1, 8, 9, 1, 1, None) == -2
     assert L.mllm_hip_topk(p, p, p, 1, 8, 0, 1, 1, None) == -2
     assert L.mllm_hip_softmax(p, None, 1, 8, None) == -1
+    assert L.mllm_hip_moe_gate_set_form(2) == -1
     assert L.mllm_hip_moe_gate(p, 0, p, p, p, None, 1, 12, 4, 2, 1, None) == -2      # H % 8
     assert L.mllm_hip_moe_gate(p, 0, p, p, p, None, 1, 8, 4, 5, 1, None) == -2       # k > E
     assert L.mllm_hip_set_exp_mode(2) == -1
