@@ -205,6 +205,17 @@ def side_workloads(torch, ql, synth, gen, brief=False):
         wb = act * (2 * I * (H // 32) * 18 + H * (I // 32) * 18)
         dec["tokens_%d" % Td] = {"us": td * 1e6, "active_experts_avg": act, "weight_GBps": wb / td / 1e9, "frac_of_hbm_peak": wb / td / 8e12}
     del gate, up, down
+    # the router gate of that layer (MoEGate::forward: logits, softmax, the k largest, weights): fp32 gate weights [E, H], 16
+    # distinct copies, with a scores buffer (two launches) and without (one workgroup per four tokens)
+    gws = [torch.randn((E, H), device="cuda", generator=gen) * 0.05 for _ in range(16)]
+    gatet = {}
+    for Tg in (1, 8, 512):
+        xg = torch.randn((Tg, H), device="cuda", generator=gen).to(torch.bfloat16)
+        scb = torch.empty((Tg, E), dtype=torch.float32, device="cuda")
+        t2 = ev_time(lambda: [ql.moe_gate(xg, w_, k, scores=scb) for w_ in gws], 1) / 16
+        t1 = ev_time(lambda: [ql.moe_gate(xg, w_, k) for w_ in gws], 1) / 16
+        gatet["tokens_%d" % Tg] = {"us": t2 * 1e6, "one_launch_us": t1 * 1e6}
+    del gws
     # the same layer with Q4_K experts (the format of the shipped Qwen3-MoE recipe), 1 and 8 tokens: pairs as K-quant GEMV rows
     gk = ql.PackedKExperts.synthetic(ql.Q4_K, E, I, H, gen)
     uk = ql.PackedKExperts.synthetic(ql.Q4_K, E, I, H, gen)
@@ -276,7 +287,7 @@ def side_workloads(torch, ql, synth, gen, brief=False):
                                                                           "operands, no exact block sums (about 2e-4 from the oracle)"},
                                             "block_dot_path": {"us": tm * 1e6, "weight_GBps": wbytes / tm / 1e9,
                                                                "note": "mllm_hip_moe_ffn_q: int8 MFMA block sums scaled on the vector ALU"},
-                                            "decode": dec, "decode_q4_k_experts": deck}
+                                            "decode": dec, "decode_q4_k_experts": deck, "router_gate": gatet}
     del gate2, up2, down2
     # Q4_0 Linear at prefill size (the reference's tinyBLAS gemm branch): gate_proj of the decode layer, 2048 rows
     M, N, K = 2048, 9728, 2560
