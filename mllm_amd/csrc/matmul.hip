@@ -204,8 +204,111 @@ __global__ __launch_bounds__(256) void matmul_kernel(MMArgs a) {
   }
 }
 
+// Up to four rows of A [M][K] against B [K][N] (attention probabilities x values of a decode token): a GEMV per row, bound by
+// reading B once, which the tile kernel above walks with one workgroup per 64 columns and a K step at a time (32 heads x
+// 8192 x 128 bf16: 158 us, 0.43 TB/s).  Here a workgroup of sixteen waves takes 2^lpr_log2 x VE columns (VE elements = 16
+// bytes per lane); a wave reads 64 >> lpr_log2 rows of B per pass, the waves stride over K, four passes requested before the
+// first is multiplied; fp32 sums per lane, then over the lanes of a column (wave shuffles), then over the waves in order
+// through LDS.  Exact products, fp32 sums in another order than the tile kernel's.
+template <int DT>
+__device__ __forceinline__ float mm_to_f32(typename MMElem<DT>::type e) {
+  if constexpr (DT == MLLM_HIP_F32) return e;
+  else if constexpr (DT == MLLM_HIP_BF16) return bf16_to_f32(e);
+  else return f16bits_to_f32(e);
+}
+constexpr int MMR_WAVES = 16;
+template <int DT, int MR>
+__global__ __launch_bounds__(MMR_WAVES * 64) void matmul_rows_kernel(MMArgs a, int lpr_log2) {
+  using E = typename MMElem<DT>::type;
+  constexpr int VE = 16 / (int)sizeof(E);
+  extern __shared__ __align__(16) unsigned char mmr_smem[];
+  float* s_part = reinterpret_cast<float*>(mmr_smem);  // [wave][row][column of the workgroup]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lpr = 1 << lpr_log2, rpw = 64 >> lpr_log2, ncols = lpr * VE;
+  const int col = (lane & (lpr - 1)) * VE, sub = lane >> lpr_log2;
+  const int n0 = (int)blockIdx.x * ncols + col;
+  const int kstep = MMR_WAVES * rpw;
+  constexpr int UB = 4;
+  for (int z = blockIdx.y; z < a.batch; z += gridDim.y) {
+    const E* A = reinterpret_cast<const E*>(a.A) + z * a.sA;
+    const E* B = reinterpret_cast<const E*>(a.B) + z * a.sB;
+    E* C = reinterpret_cast<E*>(a.C) + z * a.sC;
+    float acc[MR][VE];
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+#pragma unroll
+      for (int j = 0; j < VE; j++) acc[m][j] = 0.f;
+    for (int k0 = wave * rpw + sub; k0 < a.K; k0 += kstep * UB) {
+      u32x4 bv[UB];
+      E av[UB][MR];
+#pragma unroll
+      for (int u = 0; u < UB; u++) {
+        const int k = k0 + u * kstep;
+        const bool ok = k < a.K && n0 < a.N;  // (N is a multiple of VE here: a lane's columns are all inside or all outside)
+        bv[u] = u32x4{0u, 0u, 0u, 0u};
+        if (ok) bv[u] = *reinterpret_cast<const u32x4*>(B + (int64_t)k * a.N + n0);
+#pragma unroll
+        for (int m = 0; m < MR; m++) av[u][m] = (ok && m < a.M) ? A[(int64_t)m * a.K + k] : (E)0;
+      }
+#pragma unroll
+      for (int u = 0; u < UB; u++)
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+          const float am = mm_to_f32<DT>(av[u][m]);
+#pragma unroll
+          for (int j = 0; j < VE; j++) acc[m][j] = fmaf(am, mm_to_f32<DT>(MMTile<E, 64, true>::elem(bv[u], j)), acc[m][j]);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; m++)
+#pragma unroll
+      for (int j = 0; j < VE; j++) {
+        float v = acc[m][j];
+        for (int off = lpr; off < 64; off <<= 1) v += __shfl_xor(v, off, 64);
+        if (sub == 0) s_part[((size_t)wave * MR + m) * ncols + col + j] = v;
+      }
+    __syncthreads();
+    for (int i = tid; i < MR * ncols; i += MMR_WAVES * 64) {
+      const int m = i / ncols, c = i - m * ncols, n = (int)blockIdx.x * ncols + c;
+      if (m < a.M && n < a.N) {
+        float f = 0.f;
+#pragma unroll
+        for (int w = 0; w < MMR_WAVES; w++) f += s_part[((size_t)w * MR + m) * ncols + c];
+        if constexpr (DT == MLLM_HIP_F32) C[(int64_t)m * a.N + n] = f;
+        else if constexpr (DT == MLLM_HIP_BF16) C[(int64_t)m * a.N + n] = f32_to_bf16(f);
+        else C[(int64_t)m * a.N + n] = f32_to_f16bits(f);
+      }
+    }
+    __syncthreads();
+  }
+}
+// the launch shape of the kernel above; false where it does not apply (the tile kernel then)
+template <int DT>
+static bool launch_matmul_rows(const MMArgs& a, hipStream_t st, int* rc) {
+  constexpr int VE = 16 / (int)sizeof(typename MMElem<DT>::type);
+  if (a.M > 4 || !a.vecB || a.N % VE || a.K < 256) return false;
+  int lg = 0;
+  while (lg < 6 && (VE << lg) < a.N) lg++;
+  // narrower column blocks while the launch has fewer than 128 workgroups, down to 64 bytes of a row per workgroup
+  while (lg > 2 && (int64_t)a.batch * ((a.N + (VE << lg) - 1) / (VE << lg)) < 128) lg--;
+  const int mr = a.M <= 1 ? 1 : (a.M <= 2 ? 2 : 4);
+  while (lg > 0 && (size_t)MMR_WAVES * mr * (VE << lg) * sizeof(float) > 64 * 1024) lg--;  // the waves' partial sums fit 64 KB of LDS
+  const int ncols = VE << lg;
+  const dim3 grid((unsigned)((a.N + ncols - 1) / ncols), (unsigned)std::min(a.batch, 65535));
+  const size_t lds = (size_t)MMR_WAVES * 4 * ncols * sizeof(float);
+  if (a.M <= 1) hipLaunchKernelGGL((matmul_rows_kernel<DT, 1>), grid, dim3(MMR_WAVES * 64), lds / 4, st, a, lg);
+  else if (a.M <= 2) hipLaunchKernelGGL((matmul_rows_kernel<DT, 2>), grid, dim3(MMR_WAVES * 64), lds / 2, st, a, lg);
+  else hipLaunchKernelGGL((matmul_rows_kernel<DT, 4>), grid, dim3(MMR_WAVES * 64), lds, st, a, lg);
+  *rc = (int)hipGetLastError();
+  return true;
+}
+
 template <int DT, bool TA, bool TB>
 static int launch_matmul(const MMArgs& a, hipStream_t st) {
+  if constexpr (!TA && !TB) {
+    int rc = 0;
+    if (launch_matmul_rows<DT>(a, st, &rc)) return rc;
+  }
   // the small tile where the large one would leave most of the 256 CUs without a workgroup
   const int64_t big = (int64_t)((a.M + 127) / 128) * ((a.N + 127) / 128) * a.batch;
   const unsigned gz = (unsigned)std::min(a.batch, 65535);

@@ -24,7 +24,9 @@ def _ref(a, b, ta, tb):
 
 
 SHAPES = [(1, 1, 1, 1), (1, 70, 130, 96), (3, 33, 65, 31), (2, 128, 128, 128), (5, 1, 257, 64), (2, 200, 7, 40),
-          (4, 129, 131, 250), (1, 64, 64, 2049)]
+          (4, 129, 131, 250), (1, 64, 64, 2049),
+          # up to four rows against [K][N] (a decode token's probabilities x values): the GEMV form when not transposed
+          (32, 1, 128, 1024), (3, 2, 136, 300), (2, 4, 1024, 257), (1, 3, 2052, 512), (5, 1, 8, 4096)]
 
 
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
@@ -68,7 +70,8 @@ def test_matmul_unaligned_views_take_the_element_path():
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])
 @pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
-@pytest.mark.parametrize("batch,M,N,K", [(1, 70, 130, 96), (3, 33, 65, 31), (2, 256, 128, 128), (16, 128, 256, 64), (2, 9, 200, 1000)])
+@pytest.mark.parametrize("batch,M,N,K", [(1, 70, 130, 96), (3, 33, 65, 31), (2, 256, 128, 128), (16, 128, 256, 64), (2, 9, 200, 1000),
+                                          (32, 1, 128, 1024), (3, 2, 136, 300), (2, 4, 1024, 264), (1, 3, 4104, 512)])
 def test_matmul_16_bit(batch, M, N, K, ta, tb, dtype):
     rng = synth.rng_for(6, 1000 + batch + M + N + K + 2 * ta + tb)
     td = torch.bfloat16 if dtype == "bf16" else torch.float16
