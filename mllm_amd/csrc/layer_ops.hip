@@ -443,6 +443,77 @@ __global__ __launch_bounds__(256) void topk_rows_kernel(const float* __restrict_
   wave_topk(x + row * len, len, k, largest != 0, sorted != 0, values + row * k, indices + row * k, lane);
 }
 
+// Long rows (a vocabulary): a workgroup of sixteen waves per row runs the same k rounds, every thread scanning its share of
+// the row with eight loads in flight, the waves' candidates meeting in LDS.  20 of 151 936: 11.3 ms with one wave -> 0.2 ms.
+constexpr int TOPK_WG = 1024;
+__global__ __launch_bounds__(TOPK_WG) void topk_long_rows_kernel(const float* __restrict__ x, float* __restrict__ values,
+                                                                int32_t* __restrict__ indices, int len, int k, int largest, int sorted) {
+  __shared__ float s_v[TOPK_WG / 64];
+  __shared__ int s_i[TOPK_WG / 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t row = blockIdx.x;
+  const float* xr = x + row * len;
+  float* out_v = values + row * k;
+  int32_t* out_i = indices + row * k;
+  const bool lg = largest != 0;
+  float pv = 0.f;
+  int pi = -1;  // previous pick
+  constexpr int UB = 8;
+  for (int r = 0; r < k; r++) {
+    KeyIdx best{0.f, -1};
+    for (int i0 = tid; i0 < len; i0 += TOPK_WG * UB) {
+      float v[UB];
+#pragma unroll
+      for (int u = 0; u < UB; u++) v[u] = i0 + TOPK_WG * u < len ? xr[i0 + TOPK_WG * u] : 0.f;
+#pragma unroll
+      for (int u = 0; u < UB; u++) {
+        const int i = i0 + TOPK_WG * u;
+        if (i < len) {
+          const bool after_prev = pi < 0 || comes_before(pv, pi, v[u], i, lg);
+          if (after_prev && (best.i < 0 || comes_before(v[u], i, best.v, best.i, lg))) {
+            best.v = v[u];
+            best.i = i;
+          }
+        }
+      }
+    }
+    best = wave_best(best, lg);
+    if (lane == 0) {
+      s_v[wave] = best.v;
+      s_i[wave] = best.i;
+    }
+    __syncthreads();
+    best = KeyIdx{s_v[0], s_i[0]};
+#pragma unroll
+    for (int w = 1; w < TOPK_WG / 64; w++) {
+      const float ov = s_v[w];
+      const int oi = s_i[w];
+      if (oi >= 0 && (best.i < 0 || comes_before(ov, oi, best.v, best.i, lg))) best = KeyIdx{ov, oi};
+    }
+    __syncthreads();
+    pv = best.v;
+    pi = best.i;
+    if (tid == 0) {
+      out_v[r] = best.v;
+      out_i[r] = best.i;
+    }
+  }
+  if (!sorted && tid == 0) {  // by index: insertion sort of k entries (thread 0 wrote them itself)
+    for (int a = 1; a < k; a++) {
+      const float v = out_v[a];
+      const int i = out_i[a];
+      int b = a - 1;
+      while (b >= 0 && out_i[b] > i) {
+        out_v[b + 1] = out_v[b];
+        out_i[b + 1] = out_i[b];
+        b--;
+      }
+      out_v[b + 1] = v;
+      out_i[b + 1] = i;
+    }
+  }
+}
+
 // ---- MoE gate: logits = x . W^T (fp32), softmax, top-k, optional normalisation ------------------------------------------
 // A workgroup of sixteen waves takes four tokens: the tokens' activations sit in LDS, every wave walks a sixteenth of the
 // experts (16-byte loads along H, the tokens share each weight load), then wave t finishes token t.
@@ -713,8 +784,12 @@ MLLM_API int mllm_hip_topk(const float* x, float* values, int32_t* indices, int6
                            int sorted, void* stream) {
   if (!x || !values || !indices || rows <= 0 || len <= 0) return MLLM_HIP_E_BADARG;
   if (k < 1 || k > len || len > 0x7fffffff || (rows + 3) / 4 > 0x7fffffff) return MLLM_HIP_E_SHAPE;
-  hipLaunchKernelGGL(topk_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream, x, values, indices, rows,
-                     (int)len, k, largest, sorted);
+  if (len >= 8192 && rows <= 0x7fffffff)
+    hipLaunchKernelGGL(topk_long_rows_kernel, dim3((unsigned)rows), dim3(TOPK_WG), 0, (hipStream_t)stream, x, values, indices, (int)len, k,
+                       largest, sorted);
+  else
+    hipLaunchKernelGGL(topk_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream, x, values, indices, rows,
+                       (int)len, k, largest, sorted);
   return (int)hipGetLastError();
 }
 

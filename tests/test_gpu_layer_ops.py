@@ -265,6 +265,13 @@ def test_topk_reference_test_shapes_and_sort():
     v, i = ql.topk(to_dev(long), 20)
     wv, wi = orc.topk(long, 20)
     assert np.array_equal(i.cpu().numpy(), wi)
+    # rows long enough for the workgroup-per-row kernel, with repeated values (ties go lowest index first), both orders
+    vocab = np.round(rng.standard_normal((3, 20011)) * 50).astype(np.float32)
+    for k, largest, srt in [(20, True, True), (7, False, False), (50, True, False)]:
+        announce("topk long rows", k, largest, srt)
+        v, i = ql.topk(to_dev(vocab), k, largest, srt)
+        wv, wi = orc.topk(vocab, k, largest, srt)
+        assert np.array_equal(i.cpu().numpy(), wi) and np.array_equal(v.cpu().numpy(), wv)
 
 
 @pytest.mark.parametrize("M,H,E,k,dtype", [(512, 2048, 128, 8, "f32"), (1, 2048, 128, 8, "f32"), (7, 256, 60, 4, "f32"),
