@@ -558,6 +558,109 @@ MLLM_API int mllm_hip_w8a8_set_tuning(int tile) {
   return 0;
 }
 
+// ---- decode: up to eight tokens against the prepacked weights --------------------------------------------------------------
+// The tile kernels above spend a 128-row tile on a decode token and leave most CUs idle (9728 x 2560 at one token: 16 us;
+// 2560 x 9728: 41 us).  Here a workgroup takes one block row of the packed matrix (32 weight rows) and its waves stride over
+// the K blocks, eight 1 KB blocks requested per wave before the first is multiplied (the first batch ahead of the copy of
+// the tokens' codes into LDS, which it does not depend on); v_dot4_i32_i8 sums, the two K halves of a block met by a wave
+// shuffle, the waves through LDS.  Integer sums are exact: the epilogue is the tile kernels' and so are the bits.
+constexpr int W8G_MAXW = 16;
+template <int MT>
+__global__ __launch_bounds__(W8G_MAXW * 64) void w8a8_gemv_packed_kernel(W8A8Args a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int Kp = (int)w8a8_packed_k(a.K), kbs = Kp / 32;
+  u32x4* sx = reinterpret_cast<u32x4*>(smem);                          // [MT][Kp / 16] the tokens' codes, zero past K and M
+  int* s_part = reinterpret_cast<int*>(smem + (size_t)MT * Kp);        // [wave][MT][32]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x, nwaves = nthreads >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int nb = blockIdx.x;
+  const u32x4* P = reinterpret_cast<const u32x4*>(a.W) + (size_t)nb * kbs * 64 + lane;
+  constexpr int UB = 8;
+  u32x4 wv[UB];
+  auto load_batch = [&](int kb0) {
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+      const int kb = kb0 + u * nwaves;
+      wv[u] = u32x4{0u, 0u, 0u, 0u};
+      if (kb < kbs) wv[u] = P[(size_t)kb * 64];
+    }
+  };
+  load_batch(wave);
+  const int cpr = Kp / 16;  // 16-byte pieces per token
+  for (int i = tid; i < MT * cpr; i += nthreads) {
+    const int m = i / cpr, c = i - m * cpr;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (m < a.M && c * 16 < a.K) v = *reinterpret_cast<const u32x4*>(a.A + (size_t)m * a.K + c * 16);  // K % 16 == 0
+    sx[i] = v;
+  }
+  __syncthreads();
+  int acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; m++) acc[m] = 0;
+  for (int kb0 = wave; kb0 < kbs; kb0 += nwaves * UB) {
+    if (kb0 != wave) load_batch(kb0);
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+      const int kb = kb0 + u * nwaves;
+      if (kb < kbs) {  // uniform
+#pragma unroll
+        for (int m = 0; m < MT; m++) {
+          const u32x4 xv = sx[m * cpr + kb * 2 + h];
+          int s = acc[m];
+          s = __builtin_amdgcn_sdot4((int)wv[u].x, (int)xv.x, s, false);
+          s = __builtin_amdgcn_sdot4((int)wv[u].y, (int)xv.y, s, false);
+          s = __builtin_amdgcn_sdot4((int)wv[u].z, (int)xv.z, s, false);
+          s = __builtin_amdgcn_sdot4((int)wv[u].w, (int)xv.w, s, false);
+          acc[m] = s;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MT; m++) {
+    acc[m] += __shfl_xor(acc[m], 32, 64);
+    if (h == 0) s_part[(wave * MT + m) * 32 + r] = acc[m];
+  }
+  __syncthreads();
+  for (int i = tid; i < MT * 32; i += nthreads) {
+    const int m = i >> 5, n = nb * 32 + (i & 31);
+    if (m < a.M && n < a.N) {
+      int v = 0;
+      for (int w = 0; w < nwaves; w++) v += s_part[(w * MT + m) * 32 + (i & 31)];
+      if (a.acc) a.acc[(int64_t)m * a.N + n] = v;
+      if (a.C) {
+        float f = (float)v * (a.ws[n] * a.xs[m]);
+        if (a.bias) f += a.bias[n];
+        a.C[(int64_t)m * a.N + n] = (uint16_t)pack_bf16(f, 0.f);
+      }
+    }
+  }
+}
+// false where the kernel above does not apply (more than eight tokens, or rows too long for its LDS)
+static int g_w8a8_decode = 1;  // 0: the tile kernels also for a few tokens (comparison runs and tests)
+static bool launch_w8a8_gemv_packed(const W8A8Args& a, hipStream_t st, int* rc) {
+  if (a.M > 8 || !g_w8a8_decode) return false;
+  const int MT = a.M <= 1 ? 1 : (a.M <= 2 ? 2 : (a.M <= 4 ? 4 : 8));
+  const int Kp = (int)w8a8_packed_k(a.K), kbs = Kp / 32;
+  const int nwaves = kbs >= 32 ? W8G_MAXW : 4;
+  const size_t lds = (size_t)MT * Kp + (size_t)nwaves * MT * 32 * 4;
+  if (lds > 160 * 1024) return false;
+  const dim3 grid((unsigned)(w8a8_packed_n(a.N) / 32));
+  auto go = [&](auto kern) {
+    if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return (int)hipGetLastError();
+    hipLaunchKernelGGL(kern, grid, dim3(nwaves * 64), lds, st, a);
+    return (int)hipGetLastError();
+  };
+  *rc = MT == 1 ? go(w8a8_gemv_packed_kernel<1>) : MT == 2 ? go(w8a8_gemv_packed_kernel<2>) : MT == 4 ? go(w8a8_gemv_packed_kernel<4>) : go(w8a8_gemv_packed_kernel<8>);
+  return true;
+}
+MLLM_API int mllm_hip_w8a8_set_decode(int gemv) {
+  if (gemv != 0 && gemv != 1) return MLLM_HIP_E_BADARG;
+  g_w8a8_decode = gemv;
+  return 0;
+}
+
 MLLM_API int mllm_hip_w8a8_nsplit_set_tuning(int tile) {
   if (tile < 0 || tile > 5) return MLLM_HIP_E_BADARG;
   g_w8a8_ntile = tile;
@@ -638,6 +741,8 @@ MLLM_API int mllm_hip_w8a8_gemm_packed(const int8_t* xq, const float* x_scale, c
     return MLLM_HIP_E_SHAPE;
   if (reinterpret_cast<uintptr_t>(xq) % 16 || reinterpret_cast<uintptr_t>(W_packed) % 16) return MLLM_HIP_E_ALIGN;
   W8A8Args a{xq, reinterpret_cast<const int8_t*>(W_packed), x_scale, w_scale, bias, (uint16_t*)out_bf16, acc_out, (int)M, (int)N, (int)K};
+  int rc = 0;
+  if (launch_w8a8_gemv_packed(a, (hipStream_t)stream, &rc)) return rc;  // up to eight tokens
   return launch_w8a8_nsplit_auto<true>(a, (hipStream_t)stream);
 }
 

@@ -110,6 +110,35 @@ def test_gemm_packed_bit_exact(M, N, K):
     assert np.array_equal(_bits(yb), wyb)
 
 
+@pytest.mark.parametrize("M", [1, 2, 3, 5, 8])
+def test_decode_gemv_packed_bit_exact(M):
+    """up to eight tokens take the GEMV kernel (a block row of the packed matrix per workgroup): the oracle's bits, and the tile
+    kernels' bits; ragged N and K (zero padding of the packed layout), long rows, bias"""
+    L = _lib.lib()
+    for N, K in ((9728, 2560), (2560, 9728), (77, 48), (200, 144), (33, 4096 + 16)):
+        rng = synth.rng_for(3, 700 + M * 11 + N + K)
+        xq = rng.integers(-127, 128, (M, K), dtype=np.int8)
+        W = rng.integers(-127, 128, (N, K), dtype=np.int8)
+        xs = ((rng.random(M) + 0.01) * 0.01).astype(np.float32)
+        ws = ((rng.random(N) + 0.01) * 0.01).astype(np.float32)
+        bias = (rng.standard_normal(N) * 0.01).astype(np.float32)
+        announce("w8a8 decode gemv", M, N, K)
+        Wp = ql.w8a8_prepack(to_dev(W))
+        y, acc = ql.w8a8_gemm_packed(to_dev(xq), to_dev(xs), Wp, N, to_dev(ws), None, want_acc=True)
+        yb = ql.w8a8_gemm_packed(to_dev(xq), to_dev(xs), Wp, N, to_dev(ws), to_dev(bias))
+        wacc, wy = orc.w8a8_gemm(xq, xs, W, ws, None)
+        _, wyb = orc.w8a8_gemm(xq, xs, W, ws, bias)
+        assert np.array_equal(acc.cpu().numpy(), wacc)
+        assert np.array_equal(_bits(y), wy) and np.array_equal(_bits(yb), wyb)
+        assert L.mllm_hip_w8a8_set_decode(0) == 0
+        try:
+            yt = ql.w8a8_gemm_packed(to_dev(xq), to_dev(xs), Wp, N, to_dev(ws), to_dev(bias))
+        finally:
+            assert L.mllm_hip_w8a8_set_decode(1) == 0
+        assert np.array_equal(_bits(yt), wyb)
+    assert L.mllm_hip_w8a8_set_decode(2) == -1
+
+
 def test_full_size_prefill():
     """A bf16 [2048,2048] with outliers, W int8 [6144,2048]: quantization bit-exact on every row; accumulators checked on a
     row sample against the oracle and on ALL rows through the column-sum identity
