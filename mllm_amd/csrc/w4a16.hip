@@ -748,6 +748,122 @@ MLLM_API int mllm_hip_w4a16_prepack(const uint8_t* qw, const uint16_t* scales, c
   return (int)hipGetLastError();
 }
 
+// ---- decode: up to eight tokens against the packed weights ------------------------------------------------------------------
+// The tile kernels spend a 128-row tile on a decode token (9728 x 2560 at one token: 20 us; 2560 x 9728: 65 us).  Here a
+// workgroup takes one block row of the packed matrix (32 weight rows), its waves stride over the 64-element K blocks, eight
+// blocks requested per wave before the first is dequantized (the first batch ahead of the copy of the tokens' activations
+// into LDS); weights go to bf16 exactly as in the tile kernels (dequant8), the products (exact in fp32) are added by fp32
+// FMAs, the two K halves of a block meet through a wave shuffle, the waves through LDS.  Same rounding points as the tile
+// kernels (weights to bf16, the sum + bias to bf16), fp32 sums in another order.  The kernel is bound by its vector ALU
+// work, which grows with the tokens: it is used up to four (9728 x 2560: 12.5 / 14.0 / 17.9 us at one / two / four tokens
+// against 20 us for the tile kernels, 25.5 at eight).
+constexpr int W4G_MAXW = 16;
+template <int MT>
+__global__ __launch_bounds__(W4G_MAXW * 64) void w4a16_gemv_packed_kernel(W4A16PArgs a) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int Kp = (int)w4a16_packed_k(a.K), kbs = Kp / 64, G = a.K / a.group, g64 = a.group / 64;
+  u32x4* sx = reinterpret_cast<u32x4*>(smem);                         // [MT][Kp / 8] bf16 activations, zero past K and M
+  float* s_part = reinterpret_cast<float*>(smem + (size_t)MT * Kp * 2);  // [wave][MT][32]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x, nwaves = nthreads >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int nb = blockIdx.x;
+  const int64_t qbytes = w4a16_packed_qbytes(a.N, a.K);
+  const u32x4* Q = reinterpret_cast<const u32x4*>(a.P) + (size_t)nb * kbs * 64 + lane;
+  const float2* SZ = reinterpret_cast<const float2*>(a.P + qbytes) + (size_t)nb * G * 32 + r;
+  constexpr int UB = 8;
+  u32x4 wv[UB];
+  float2 sz[UB];
+  auto load_batch = [&](int kb0) {
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+      const int kb = kb0 + u * nwaves;
+      wv[u] = u32x4{0u, 0u, 0u, 0u};
+      sz[u] = float2{0.f, 0.f};
+      if (kb < kbs) {
+        wv[u] = Q[(size_t)kb * 64];
+        sz[u] = SZ[(size_t)min(kb / g64, G - 1) * 32];  // (blocks of the zero padding past K: their codes are zero, as are the activations)
+      }
+    }
+  };
+  load_batch(wave);
+  const int cpr = Kp / 8;  // 16-byte pieces (eight elements) per token
+  for (int i = tid; i < MT * cpr; i += nthreads) {
+    const int m = i / cpr, c = i - m * cpr;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (m < a.M && c * 8 < a.K) v = *reinterpret_cast<const u32x4*>(a.A + (size_t)m * a.K + c * 8);  // K % 64 == 0
+    sx[i] = v;
+  }
+  __syncthreads();
+  float acc[MT];
+#pragma unroll
+  for (int m = 0; m < MT; m++) acc[m] = 0.f;
+  for (int kb0 = wave; kb0 < kbs; kb0 += nwaves * UB) {
+    if (kb0 != wave) load_batch(kb0);
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+      const int kb = kb0 + u * nwaves;
+      if (kb < kbs) {  // uniform
+        const uint32_t wd[4] = {wv[u].x, wv[u].y, wv[u].z, wv[u].w};
+#pragma unroll
+        for (int d = 0; d < 4; d++) {  // elements k = 64 kb + 16 d + 8 h + 0..7
+          uint32_t wb[4];
+          dequant8(wd[d], sz[u].x, sz[u].y, wb);
+#pragma unroll
+          for (int m = 0; m < MT; m++) {
+            const u32x4 xv = sx[m * cpr + kb * 8 + 2 * d + h];
+            float s = acc[m];
+            const uint32_t xw[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+            for (int p = 0; p < 4; p++) {
+              s = fmaf(__uint_as_float(wb[p] << 16), __uint_as_float(xw[p] << 16), s);
+              s = fmaf(__uint_as_float(wb[p] & 0xffff0000u), __uint_as_float(xw[p] & 0xffff0000u), s);
+            }
+            acc[m] = s;
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int m = 0; m < MT; m++) {
+    acc[m] += __shfl_xor(acc[m], 32, 64);
+    if (h == 0) s_part[(wave * MT + m) * 32 + r] = acc[m];
+  }
+  __syncthreads();
+  for (int i = tid; i < MT * 32; i += nthreads) {
+    const int m = i >> 5, n = nb * 32 + (i & 31);
+    if (m < a.M && n < a.N) {
+      float f = 0.f;
+      for (int w = 0; w < nwaves; w++) f += s_part[(w * MT + m) * 32 + (i & 31)];
+      if (a.bias) f += bf16_to_f32(a.bias[n]);
+      a.C[(int64_t)m * a.N + n] = (uint16_t)pack_bf16(f, 0.f);
+    }
+  }
+}
+static int g_w4a16_decode = 1;  // 0: the tile kernels also for a few tokens (comparison runs and tests)
+static bool launch_w4a16_gemv_packed(const W4A16PArgs& a, hipStream_t st, int* rc) {
+  if (a.M > 4 || !g_w4a16_decode) return false;
+  const int MT = a.M <= 1 ? 1 : (a.M <= 2 ? 2 : 4);
+  const int Kp = (int)w4a16_packed_k(a.K), kbs = Kp / 64;
+  const int nwaves = kbs >= 32 ? W4G_MAXW : 4;
+  const size_t lds = (size_t)MT * Kp * 2 + (size_t)nwaves * MT * 32 * 4;
+  if (lds > 160 * 1024) return false;
+  const dim3 grid((unsigned)(w4a16_packed_n(a.N) / 32));
+  auto go = [&](auto kern) {
+    if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return (int)hipGetLastError();
+    hipLaunchKernelGGL(kern, grid, dim3(nwaves * 64), lds, st, a);
+    return (int)hipGetLastError();
+  };
+  *rc = MT == 1 ? go(w4a16_gemv_packed_kernel<1>) : MT == 2 ? go(w4a16_gemv_packed_kernel<2>) : go(w4a16_gemv_packed_kernel<4>);
+  return true;
+}
+MLLM_API int mllm_hip_w4a16_set_decode(int gemv) {
+  if (gemv != 0 && gemv != 1) return MLLM_HIP_E_BADARG;
+  g_w4a16_decode = gemv;
+  return 0;
+}
+
 MLLM_API int mllm_hip_w4a16_gemm_packed(const void* a_bf16, const void* packed, const void* bias_bf16, void* c_bf16,
                                         int64_t M, int64_t N, int64_t K, int group, void* stream) {
   if (!a_bf16 || !packed || !c_bf16 || M <= 0 || N <= 0 || K <= 0 || group <= 0) return MLLM_HIP_E_BADARG;
@@ -758,6 +874,8 @@ MLLM_API int mllm_hip_w4a16_gemm_packed(const void* a_bf16, const void* packed, 
   if (reinterpret_cast<uintptr_t>(a_bf16) % 16 || reinterpret_cast<uintptr_t>(packed) % 16) return MLLM_HIP_E_ALIGN;
   W4A16PArgs a{(const uint16_t*)a_bf16, (const uint8_t*)packed, (const uint16_t*)bias_bf16, (uint16_t*)c_bf16,
                (int)M, (int)N, (int)K, group};
+  int rc = 0;
+  if (launch_w4a16_gemv_packed(a, (hipStream_t)stream, &rc)) return rc;  // up to four tokens
   return launch_w4a16_nsplit_auto(a, (hipStream_t)stream);
 }
 

@@ -104,6 +104,35 @@ def test_gemm_packed_vs_oracle(M, N, K, group):
     assert (diff == 0).mean() > 0.97
 
 
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+def test_decode_gemv_packed_vs_oracle_and_tiles(M):
+    """up to four tokens take the GEMV kernel (a block row of the packed matrix per workgroup): the oracle within the GEMM's
+    tolerance, nearly every output the tile kernels' bits; ragged N, K not a multiple of 128, groups of 64 / 128 / 256, bias"""
+    L = _lib.lib()
+    for N, K, group in ((9728, 2560, 128), (2560, 9728, 128), (77, 192, 64), (200, 1024, 256), (33, 4096 + 64, 64)):
+        rng = synth.rng_for(2, 900 + 3 * M + N + K + group)
+        qw, s, zp, _, _ = synth.make_w4a16(rng, N, K, group)
+        a_bits, _ = synth.make_x_bf16(rng, M, K)
+        bias = synth.fp32_to_bf16_bits((rng.standard_normal(N) * 0.1).astype(np.float32))
+        announce("w4a16 decode gemv", M, N, K, group)
+        packed = ql.w4a16_prepack(*_dev(qw, s, zp), group)
+        c = _bits(ql.w4a16_gemm_packed(bf16_dev(a_bits), packed, N, None, group))
+        cb = _bits(ql.w4a16_gemm_packed(bf16_dev(a_bits), packed, N, bf16_dev(bias), group))
+        want = orc.w4a16_gemm(a_bits, qw, s, zp, None, group)
+        wantb = orc.w4a16_gemm(a_bits, qw, s, zp, bias, group)
+        assert rel_l2(synth.bf16_bits_to_fp32(c), synth.bf16_bits_to_fp32(want)) <= TOL
+        assert rel_l2(synth.bf16_bits_to_fp32(cb), synth.bf16_bits_to_fp32(wantb)) <= TOL
+        assert L.mllm_hip_w4a16_set_decode(0) == 0
+        try:
+            ct = _bits(ql.w4a16_gemm_packed(bf16_dev(a_bits), packed, N, bf16_dev(bias), group))
+        finally:
+            assert L.mllm_hip_w4a16_set_decode(1) == 0
+        diff = np.abs(cb.astype(np.int32) - ct.astype(np.int32))
+        assert diff.max() <= 1 or rel_l2(synth.bf16_bits_to_fp32(cb), synth.bf16_bits_to_fp32(ct)) < 1e-4
+        assert (diff == 0).mean() > 0.95
+    assert L.mllm_hip_w4a16_set_decode(2) == -1
+
+
 @pytest.mark.parametrize("tile", [1, 2, 3, 4, 5, 16 + 5])
 def test_gemm_packed_every_tile(tile):
     M, N, K, group = 200, 800, 384, 128
