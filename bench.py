@@ -329,6 +329,50 @@ def side_workloads(torch, ql, synth, gen, brief=False):
                                                             "path": "matrix cores (mllm_hip_linear_kq_gemm)",
                                                             "gemv_passes_path": {"us": tv * 1e6}}
         del wkg, wkv
+    # W8A8 / W4A16 at decode size (the GEMV kernels against packed weights; W8A8 with its per-token quantization) and the
+    # operators of a decode token around the Linears
+    dec_ops = {}
+    for nm, (n_, k_) in (("gate_9728x2560", (9728, 2560)), ("down_2560x9728", (2560, 9728))):
+        Wp8 = [ql.w8a8_prepack(torch.randint(-127, 128, (n_, k_), dtype=torch.int8, device="cuda", generator=gen)) for _ in range(4)]
+        ws8 = (torch.rand(n_, device="cuda", generator=gen) + 0.01) * 0.01
+        s4 = (torch.randn((n_, k_ // 128), device="cuda", generator=gen).abs() * 0.01).to(torch.float16)
+        zp = torch.randint(0, 256, (n_, k_ // 256), dtype=torch.uint8, device="cuda", generator=gen)
+        Wp4 = [ql.w4a16_prepack(torch.randint(0, 256, (n_, k_ // 2), dtype=torch.uint8, device="cuda", generator=gen), s4, zp, 128)
+               for _ in range(4)]
+        for m_ in (1, 4):
+            a_ = torch.randn((m_, k_), device="cuda", generator=gen).to(torch.bfloat16)
+            y_ = torch.empty((m_, n_), dtype=torch.bfloat16, device="cuda")
+            wq = torch.empty(_lib_ws(ql, "w8a8", m_, k_), dtype=torch.uint8, device="cuda")
+            j = [0]
+
+            def f8():
+                ql.w8a8_linear_packed(a_, Wp8[j[0] % 4], n_, ws8, None, workspace=wq, out=y_)
+                j[0] += 1
+
+            def f4():
+                ql.w4a16_gemm_packed(a_, Wp4[j[0] % 4], n_, None, 128, out=y_)
+                j[0] += 1
+            t8, t4 = ev_time(f8, 8), ev_time(f4, 8)
+            dec_ops["%s_tokens_%d" % (nm, m_)] = {"w8a8_us": t8 * 1e6, "w8a8_weight_GBps": n_ * k_ / t8 / 1e9,
+                                                  "w4a16_us": t4 * 1e6, "w4a16_weight_GBps": n_ * k_ / 2 / t4 / 1e9}
+        del Wp8, Wp4
+    xs_ = torch.randn((8, 151936), device="cuda", generator=gen)
+    dec_ops["softmax_8x151936_us"] = ev_time(lambda: ql.softmax(xs_), 2) * 1e6
+    dec_ops["topk_20_of_151936_us"] = ev_time(lambda: ql.topk(xs_[:1], 20), 2) * 1e6
+    xs_ = torch.randn((32 * 512, 512), device="cuda", generator=gen)
+    dec_ops["softmax_16384x512_us"] = ev_time(lambda: ql.softmax(xs_), 8) * 1e6
+    xs_ = torch.randn((512, 128), device="cuda", generator=gen)
+    dec_ops["topk_8_of_128_rows_512_us"] = ev_time(lambda: ql.topk(xs_, 8), 8) * 1e6
+    p_ = torch.randn((32, 1, 8192), device="cuda", generator=gen).to(torch.bfloat16)
+    v_ = torch.randn((32, 8192, 128), device="cuda", generator=gen).to(torch.bfloat16)
+    o_ = torch.empty((32, 1, 128), dtype=torch.bfloat16, device="cuda")
+    tpv = ev_time(lambda: ql.matmul(p_, v_, out=o_), 8)
+    dec_ops["matmul_scores_x_values_32x1x8192x128_bf16"] = {"us": tpv * 1e6, "GBps": v_.numel() * 2 / tpv / 1e9}
+    s_ = torch.empty((32, 1, 8192), dtype=torch.bfloat16, device="cuda")
+    q_ = torch.randn((32, 1, 128), device="cuda", generator=gen).to(torch.bfloat16)
+    tqk = ev_time(lambda: ql.matmul(q_, v_, transpose_b=True, out=s_), 8)
+    dec_ops["matmul_query_x_keys_32x1x128x8192_bf16"] = {"us": tqk * 1e6, "GBps": v_.numel() * 2 / tqk / 1e9}
+    out["decode_size_w8a8_w4a16_and_operators"] = dec_ops
     return out
 
 

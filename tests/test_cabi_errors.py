@@ -84,6 +84,10 @@ def _cases():
                                         [(0, Q4_0, BADARG), (1, 0, BADARG), (1, 5, BADARG), (2, None, BADARG), (3, None, BADARG),
                                          (4, IMAGE, BADARG), (5, 0, BADARG), (6, 320, SHAPE), (7, ODD, ALIGN), (8, 8 * 256 + 8 * 36 - 1, BADARG)]),
         "mllm_hip_kq_set_slice_meeting": ([-1, 0], [(0, 2, BADARG), (0, -2, BADARG), (1, 9, BADARG), (1, -1, BADARG)]),
+        # switches for comparison runs: anything but 0 and 1 is refused and leaves the setting alone
+        "mllm_hip_w8a8_set_decode": ([1], [(0, 2, BADARG), (0, -1, BADARG)]),
+        "mllm_hip_w4a16_set_decode": ([1], [(0, 2, BADARG), (0, -1, BADARG)]),
+        "mllm_hip_moe_gate_set_form": ([1], [(0, 2, BADARG), (0, -1, BADARG)]),
         "mllm_hip_kq_gemm_prepack": ([Q4_K, P, 0, P, 8, 256, None], [(0, Q8_0, BADARG), (1, None, BADARG), (5, 96, SHAPE)]),
         "mllm_hip_linear_kq_gemm": ([Q4_K, P, P, F32, None, P, 16, 8, 256, P, None],
                                     [(0, Q4_0, BADARG), (1, None, BADARG), (5, None, BADARG), (9, None, BADARG), (8, 100, SHAPE)]),
