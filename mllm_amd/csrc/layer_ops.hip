@@ -514,6 +514,186 @@ __global__ __launch_bounds__(TOPK_WG) void topk_long_rows_kernel(const float* __
   }
 }
 
+// Rows longer than 256 elements, k up to TOPK_SEL_MAX: radix select.  (value, index) pairs are ordered by order_key(); the
+// key of the k-th pair is found a digit at a time (four bytes, or 12, 12 and 8 bits), highest first: a histogram of that digit
+// over the elements that agree with the digits found so far (LDS counters; lanes of a wave that hold the same digit add once),
+// then the bin in which the k-th falls.  These counting passes give the value's key; where more elements share that value
+// than are still wanted, as many again over the inverted index choose the lowest indices among them.  Every pair at or above the k-th key is then collected
+// in LDS and placed by its rank among the k.  The passes read the row again (eight 16-byte loads in flight per thread) or,
+// for rows of up to eight such loads per thread, keep the keys in registers.  The cost does not depend on k.
+constexpr int TOPK_SEL_MAX = 2048;
+#ifndef TOPK_LEADERS
+#define TOPK_LEADERS 2
+#endif
+template <int VEC> struct TopkVec;
+template <> struct TopkVec<1> { typedef float T; };
+template <> struct TopkVec<4> { typedef float4 T; };
+template <int NT, int VEC, int R, bool WIDE>
+__global__ __launch_bounds__(NT) void topk_select_rows_kernel(const float* __restrict__ x, float* __restrict__ values,
+                                                              int32_t* __restrict__ indices, int len, int k, int largest, int sorted) {
+  typedef typename TopkVec<VEC>::T VT;
+  __shared__ unsigned s_hist[WIDE ? 4096 : 256];
+  __shared__ unsigned s_pick[4];  // chosen digit, pairs still wanted inside its bin, the bin's count; [3]: pairs collected
+  __shared__ unsigned long long s_sel[TOPK_SEL_MAX];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int64_t row = blockIdx.x;
+  const float* xr = x + row * len;
+  const bool lg = largest != 0;
+  const int nunits = len / VEC;  // (VEC divides len)
+  const bool inreg = nunits <= NT * R;
+  uint32_t kreg[R][VEC];
+  auto vkey = [&](float v) {
+    uint32_t b = __float_as_uint(v + 0.f);
+    b = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+    return lg ? b : ~b;
+  };
+  auto load_keys = [&](int base, uint32_t (&kk)[R][VEC]) {
+    VT v[R];
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+      const int u = base + tid + NT * j;
+      if (u < nunits) v[j] = reinterpret_cast<const VT*>(xr)[u];
+      else v[j] = VT{};
+    }
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+      const float* f = reinterpret_cast<const float*>(&v[j]);
+#pragma unroll
+      for (int e = 0; e < VEC; e++) kk[j][e] = vkey(f[e]);
+    }
+  };
+  if (inreg) load_keys(0, kreg);
+  // f(key, index, valid) for every element of the row, by all lanes of every wave together (f holds wave-wide operations)
+  auto scan = [&](auto&& f) {
+    if (inreg) {
+#pragma unroll
+      for (int j = 0; j < R; j++) {
+        const int u = tid + NT * j;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) f(kreg[j][e], u * VEC + e, u < nunits);
+      }
+    } else {
+      for (int base = 0; base < nunits; base += NT * R) {
+        uint32_t kk[R][VEC];
+        load_keys(base, kk);
+#pragma unroll
+        for (int j = 0; j < R; j++) {
+          const int u = base + tid + NT * j;
+#pragma unroll
+          for (int e = 0; e < VEC; e++) f(kk[j][e], u * VEC + e, u < nunits);
+        }
+      }
+    }
+  };
+  auto hist_add = [&](bool match, uint32_t digit) {
+    unsigned long long m = __ballot(match);
+    for (int it = 0; it < TOPK_LEADERS && m; it++) {  // (m is the same in every lane)
+      const int leader = __ffsll((long long)m) - 1;
+      const uint32_t d0 = (uint32_t)__builtin_amdgcn_readlane((int)digit, leader);
+      const bool mine = match && digit == d0;
+      const unsigned long long same = __ballot(mine);
+      if (lane == leader) atomicAdd(&s_hist[d0], (unsigned)__popcll(same));
+      match = match && !mine;
+      m &= ~same;
+    }
+    if (match) atomicAdd(&s_hist[digit], 1u);
+  };
+  // the bin of the `need`-th largest digit among nb bins: wave 0, a lane per nb / 64 bins
+  auto pick = [&](uint32_t need, int nb) {
+    if (tid < 64) {
+      const int per = nb >> 6, b0 = lane * per;
+      uint32_t tot = 0;
+      for (int q = 0; q < per; q++) tot += s_hist[b0 + ((q + lane) & (per - 1))];  // (the lanes on different banks)
+      uint32_t incl = tot;  // this lane's bins and all higher ones
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const uint32_t o = (uint32_t)__shfl_down((int)incl, off, 64);
+        if (lane + off < 64) incl += o;
+      }
+      uint32_t a = incl - tot;
+      if (a < need && need <= incl) {
+        for (int q = per - 1; q >= 0; q--) {
+          const uint32_t c = s_hist[b0 + q];
+          if (a + c >= need) {
+            s_pick[0] = (uint32_t)(b0 + q);
+            s_pick[1] = need - a;
+            s_pick[2] = c;
+            break;
+          }
+          a += c;
+        }
+      }
+    }
+  };
+  // one counting pass over the digit of `bits` bits at `shift`: keyof(key, index, valid, &k32) says whether the element still
+  // agrees with the digits found so far and gives the 32 bits the digit is taken from
+  auto count_pass = [&](int shift, int bits, uint32_t need, auto&& keyof) {
+    const int nb = 1 << bits;
+    for (int b = tid; b < nb; b += NT) s_hist[b] = 0;
+    __syncthreads();
+    scan([&](uint32_t key, int idx, bool ok) {
+      uint32_t k32;
+      const bool mt = keyof(key, idx, ok, k32);
+      hist_add(mt, (k32 >> shift) & (uint32_t)(nb - 1));
+    });
+    __syncthreads();
+    pick(need, nb);
+    __syncthreads();
+  };
+  // rows read again per pass: 12 + 12 + 8 bits (a pass over memory less); rows in registers: four bytes (256 counters to clear
+  // and to walk per pass instead of 4096)
+  constexpr int NPASS = WIDE ? 3 : 4;
+  const int p_shift[4] = {WIDE ? 20 : 24, WIDE ? 8 : 16, WIDE ? 0 : 8, 0}, p_bits[4] = {WIDE ? 12 : 8, WIDE ? 12 : 8, 8, 8};
+  uint32_t need = (uint32_t)k, t_val = 0, mask = 0, ties = 0;
+  if (tid == 0) s_pick[3] = 0;
+#pragma unroll
+  for (int p = 0; p < NPASS; p++) {
+    count_pass(p_shift[p], p_bits[p], need, [&](uint32_t key, int, bool ok, uint32_t& k32) {
+      k32 = key;
+      return ok && (key & mask) == t_val;
+    });
+    t_val |= s_pick[0] << p_shift[p];
+    mask |= ((1u << p_bits[p]) - 1u) << p_shift[p];
+    need = s_pick[1];
+    ties = s_pick[2];
+  }
+  uint32_t t_idx = 0;  // pairs of the k-th value are taken down to this inverted index
+  if (ties != need) {   // (the same in every thread)
+    mask = 0;
+#pragma unroll
+    for (int p = 0; p < NPASS; p++) {
+      count_pass(p_shift[p], p_bits[p], need, [&](uint32_t key, int idx, bool ok, uint32_t& k32) {
+        k32 = ~(uint32_t)idx;
+        return ok && key == t_val && (k32 & mask) == t_idx;
+      });
+      t_idx |= s_pick[0] << p_shift[p];
+      mask |= ((1u << p_bits[p]) - 1u) << p_shift[p];
+      need = s_pick[1];
+    }
+  }
+  scan([&](uint32_t key, int idx, bool ok) {
+    const uint32_t ni = ~(uint32_t)idx;
+    if (ok && (key > t_val || (key == t_val && ni >= t_idx))) {
+      const unsigned pos = atomicAdd(&s_pick[3], 1u);
+      if (pos < (unsigned)TOPK_SEL_MAX) s_sel[pos] = ((unsigned long long)key << 32) | ni;
+    }
+  });
+  __syncthreads();
+  const bool by_value = sorted != 0;
+  for (int t = tid; t < k; t += NT) {
+    const unsigned long long my = s_sel[t];
+    const unsigned long long mc = by_value ? my : (my << 32);  // by index: the inverted index alone, larger = earlier
+    int rank = 0;
+    for (int j = 0; j < k; j++) {
+      const unsigned long long o = s_sel[j];
+      rank += (by_value ? o : (o << 32)) > mc ? 1 : 0;
+    }
+    const int idx = (int)~(uint32_t)my;
+    values[row * k + rank] = xr[idx];
+    indices[row * k + rank] = idx;
+  }
+}
+
 // ---- MoE gate: logits = x . W^T (fp32), softmax, top-k, optional normalisation ------------------------------------------
 // A workgroup of sixteen waves takes four tokens: the tokens' activations sit in LDS, every wave walks a sixteenth of the
 // experts (16-byte loads along H, the tokens share each weight load), then wave t finishes token t.
@@ -784,7 +964,25 @@ MLLM_API int mllm_hip_topk(const float* x, float* values, int32_t* indices, int6
                            int sorted, void* stream) {
   if (!x || !values || !indices || rows <= 0 || len <= 0) return MLLM_HIP_E_BADARG;
   if (k < 1 || k > len || len > 0x7fffffff || (rows + 3) / 4 > 0x7fffffff) return MLLM_HIP_E_SHAPE;
-  if (len >= 8192 && rows <= 0x7fffffff)
+  if (len > 256 && k <= TOPK_SEL_MAX && rows <= 0x7fffffff) {
+    const bool vec = len % 4 == 0 && ((uintptr_t)x & 15) == 0;
+    const int64_t units = vec ? len / 4 : len;
+    const dim3 grid((unsigned)rows);
+    hipStream_t st = (hipStream_t)stream;
+#define TOPK_SELECT(NT, R, WIDE) \
+  do { \
+    if (vec) hipLaunchKernelGGL((topk_select_rows_kernel<NT, 4, R, WIDE>), grid, dim3(NT), 0, st, x, values, indices, (int)len, k, largest, sorted); \
+    else hipLaunchKernelGGL((topk_select_rows_kernel<NT, 1, R, WIDE>), grid, dim3(NT), 0, st, x, values, indices, (int)len, k, largest, sorted); \
+  } while (0)
+    if (units <= 256) TOPK_SELECT(256, 1, false);  // (loads per thread that hold the row: no empty slots to step over)
+    else if (units <= 512) TOPK_SELECT(256, 2, false);
+    else if (units <= 1024) TOPK_SELECT(256, 4, false);
+    else if (units <= 2048) TOPK_SELECT(256, 8, false);
+    else if (units <= 4096) TOPK_SELECT(1024, 4, false);
+    else if (units <= 8192) TOPK_SELECT(1024, 8, false);
+    else TOPK_SELECT(1024, 8, true);
+#undef TOPK_SELECT
+  } else if (len >= 8192 && rows <= 0x7fffffff)
     hipLaunchKernelGGL(topk_long_rows_kernel, dim3((unsigned)rows), dim3(TOPK_WG), 0, (hipStream_t)stream, x, values, indices, (int)len, k,
                        largest, sorted);
   else

@@ -274,6 +274,26 @@ def test_topk_reference_test_shapes_and_sort():
         assert np.array_equal(i.cpu().numpy(), wi) and np.array_equal(v.cpu().numpy(), wv)
 
 
+@pytest.mark.parametrize("rows,ln", [(5, 257), (3, 1000), (4, 2048), (3, 2051), (2, 8192), (2, 9001), (2, 33000), (1, 151936)])
+def test_topk_by_radix_select(rows, ln):
+    """rows longer than 256 elements: every selection equals the oracle's (ties lowest index first), whatever the row's length
+    (whole 16-byte loads or single elements, keys in registers or read again per pass), k, order and kind of ties"""
+    rng = synth.rng_for(6, 5100 + ln)
+    smooth = rng.standard_normal((rows, ln)).astype(np.float32)
+    coarse = np.round(rng.standard_normal((rows, ln)) * 3).astype(np.float32)  # a few dozen distinct values, signed zeros among them
+    coarse[:, ::7] *= -1.0
+    flat = np.full((rows, ln), 2.5, np.float32)  # every element ties
+    flat[:, ln // 2] = 7.0
+    for nm, x in (("smooth", smooth), ("coarse", coarse), ("flat", flat)):
+        for k, largest, srt in [(1, True, True), (8, True, False), (50, True, True), (33, False, True), (min(ln, 2048), True, False),
+                                (257, False, False)]:
+            announce("topk radix", nm, rows, ln, k, largest, srt)
+            v, i = ql.topk(to_dev(x), k, largest, srt)
+            wv, wi = orc.topk(x, k, largest, srt)
+            assert np.array_equal(i.cpu().numpy(), wi)
+            assert np.array_equal(v.cpu().numpy().view(np.uint32), wv.view(np.uint32))
+
+
 @pytest.mark.parametrize("M,H,E,k,dtype", [(512, 2048, 128, 8, "f32"), (1, 2048, 128, 8, "f32"), (7, 256, 60, 4, "f32"),
                                            (33, 2048, 128, 8, "bf16"), (5, 64, 8, 2, "f32")])
 def test_moe_gate(M, H, E, k, dtype):
