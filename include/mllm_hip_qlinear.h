@@ -341,10 +341,14 @@ int mllm_hip_w4a16_gemm_packed(const void* a_bf16, const void* packed, const voi
                                int64_t N, int64_t K, int group, void* stream);
 /* Parity probe: the dequantized weight table w_bf16 [N][K] exactly as the packed GEMM forms it. */
 int mllm_hip_w4a16_dequantize_packed(const void* packed, void* w_bf16, int64_t N, int64_t K, int group, void* stream);
-/* Up to four tokens against packed weights run as a GEMV kernel (a block row of the packed matrix per workgroup, waves striding
- * over K; weights rounded to bf16 and the sum + bias rounded to bf16 as in the tile kernels, fp32 sums in another order).
+/* Up to 32 tokens against packed weights run as GEMV kernels (a block row of the packed matrix per workgroup, waves striding
+ * over K; weights rounded to bf16 and the sum + bias rounded to bf16 as in the tile kernels, fp32 sums in another order): fp32
+ * FMAs for one token, the matrix cores from two (17 to 32 tokens only where N <= 8192).
  * 0 keeps the tile kernels also there (comparison runs and tests), 1 restores the default. */
 int mllm_hip_w4a16_set_decode(int gemv);
+/* The token count from which the decode kernels use the matrix cores (1..33, 33 = never; default 2): comparison runs and tests.
+ * No counterpart in the reference. */
+int mllm_hip_w4a16_set_decode_mfma_from(int tokens);
 /* Tile override for the packed GEMM: 0 heuristic, 1 = 128x384, 2 = 64x384, 3 = 128x128, 4 = 64x128, 5 = 128x256;
  * + 16 switches off the half-height tiles that shorten a partly filled last round. */
 int mllm_hip_w4a16_packed_set_tuning(int tile);

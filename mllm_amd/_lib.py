@@ -78,6 +78,7 @@ def lib():
         L.mllm_hip_moe_gate_set_form.argtypes = [ci]
         L.mllm_hip_w8a8_set_decode.argtypes = [ci]
         L.mllm_hip_w4a16_set_decode.argtypes = [ci]
+        L.mllm_hip_w4a16_set_decode_mfma_from.argtypes = [ci]
         L.mllm_hip_quantize_q8_0.argtypes = [vp, ci, vp, vp, i64, i64, vp]
         L.mllm_hip_kq_gemm_packed_bytes.restype = C.c_size_t
         L.mllm_hip_kq_gemm_packed_bytes.argtypes = [ci, i64, i64]

@@ -748,15 +748,15 @@ MLLM_API int mllm_hip_w4a16_prepack(const uint8_t* qw, const uint16_t* scales, c
   return (int)hipGetLastError();
 }
 
-// ---- decode: up to eight tokens against the packed weights ------------------------------------------------------------------
+// ---- decode: up to 32 tokens against the packed weights ------------------------------------------------------------------
 // The tile kernels spend a 128-row tile on a decode token (9728 x 2560 at one token: 20 us; 2560 x 9728: 65 us).  Here a
 // workgroup takes one block row of the packed matrix (32 weight rows), its waves stride over the 64-element K blocks, eight
 // blocks requested per wave before the first is dequantized (the first batch ahead of the copy of the tokens' activations
 // into LDS); weights go to bf16 exactly as in the tile kernels (dequant8), the products (exact in fp32) are added by fp32
 // FMAs, the two K halves of a block meet through a wave shuffle, the waves through LDS.  Same rounding points as the tile
 // kernels (weights to bf16, the sum + bias to bf16), fp32 sums in another order.  The kernel is bound by its vector ALU
-// work, which grows with the tokens: it is used up to four (9728 x 2560: 12.5 / 14.0 / 17.9 us at one / two / four tokens
-// against 20 us for the tile kernels, 25.5 at eight).
+// work, which grows with the tokens (9728 x 2560: 12.5 / 14.0 / 17.9 / 25.5 us at one / two / four / eight tokens against 20 us
+// for the tile kernels): it serves one token, the matrix-core form below two and more.
 constexpr int W4G_MAXW = 16;
 template <int MT>
 __global__ __launch_bounds__(W4G_MAXW * 64) void w4a16_gemv_packed_kernel(W4A16PArgs a) {
@@ -840,15 +840,122 @@ __global__ __launch_bounds__(W4G_MAXW * 64) void w4a16_gemv_packed_kernel(W4A16P
     }
   }
 }
+// The same walk with the products on the matrix cores: the packed dword d of a lane IS its operand of the d-th
+// v_mfma_f32_32x32x16_bf16 of the block (row l % 32, eight consecutive k of half l / 32), the other operand the same eight k of
+// token l % 32 from LDS (lanes past the MT tokens staged pass zeros), so a block costs four matrix instructions whatever the
+// token count and the vector ALU does the dequantization only.  acc[4g + e] = C[token l % 32][row 8g + 4 (l / 32) + e]; the
+// waves' sums meet in LDS where the activations were (after a barrier).
+template <int MT>
+__global__ __launch_bounds__(W4G_MAXW * 64) void w4a16_gemv_mfma_packed_kernel(W4A16PArgs a, int cb) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int Kp = (int)w4a16_packed_k(a.K), kbs = Kp / 64, G = a.K / a.group, g64 = a.group / 64;
+  u32x4* sx = reinterpret_cast<u32x4*>(smem);       // [MT][8 cb] bf16 activations of the cb blocks in work, zero past K and M
+  float* s_part = reinterpret_cast<float*>(smem);   // [wave][MT][32], after the loop
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x, nwaves = nthreads >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int nb = blockIdx.x;
+  const int64_t qbytes = w4a16_packed_qbytes(a.N, a.K);
+  const u32x4* Q = reinterpret_cast<const u32x4*>(a.P) + (size_t)nb * kbs * 64 + lane;
+  const float2* SZ = reinterpret_cast<const float2*>(a.P + qbytes) + (size_t)nb * G * 32 + r;
+  constexpr int UB = 8;
+  u32x4 wv[UB];
+  float2 sz[UB];
+  auto load_batch = [&](int kb0, int c1) {
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+      const int kb = kb0 + u * nwaves;
+      wv[u] = u32x4{0u, 0u, 0u, 0u};
+      sz[u] = float2{0.f, 0.f};
+      if (kb < c1) {
+        wv[u] = Q[(size_t)kb * 64];
+        sz[u] = SZ[(size_t)min(kb / g64, G - 1) * 32];
+      }
+    }
+  };
+  const int cpr = cb * 8;  // 16-byte pieces (eight elements) per token in LDS
+  v16f acc;
+#pragma unroll
+  for (int j = 0; j < 16; j++) acc[j] = 0.f;
+  const bool staged = r < MT;
+  const u32x4* sxr = sx + (size_t)(staged ? r : 0) * cpr + h;
+  // the K blocks in runs of cb (all of them where the tokens' rows fit LDS whole)
+  for (int c0 = 0; c0 < kbs; c0 += cb) {
+  const int c1 = min(c0 + cb, kbs);
+  load_batch(c0 + wave, c1);  // ahead of the copy of the activations
+  if (c0) __syncthreads();    // every wave is done with the previous run's activations
+  for (int i = tid; i < MT * cpr; i += nthreads) {
+    const int m = i / cpr, c = i - m * cpr, gc = c0 * 8 + c;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (m < a.M && gc * 8 < a.K) v = *reinterpret_cast<const u32x4*>(a.A + (size_t)m * a.K + gc * 8);
+    sx[i] = v;
+  }
+  __syncthreads();
+  for (int kb0 = c0 + wave; kb0 < c1; kb0 += nwaves * UB) {
+    if (kb0 != c0 + wave) load_batch(kb0, c1);
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+      const int kb = kb0 + u * nwaves;
+      if (kb < c1) {  // uniform
+        const uint32_t wd[4] = {wv[u].x, wv[u].y, wv[u].z, wv[u].w};
+#pragma unroll
+        for (int d = 0; d < 4; d++) {  // elements k = 64 kb + 16 d + 8 h + 0..7
+          uint32_t wb[4];
+          dequant8(wd[d], sz[u].x, sz[u].y, wb);
+          u32x4 xv = {0u, 0u, 0u, 0u};
+          if (staged) xv = sxr[(kb - c0) * 8 + 2 * d];
+          acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, u32x4{wb[0], wb[1], wb[2], wb[3]}),
+                                                        __builtin_bit_cast(bf16x8, xv), acc, 0, 0, 0);
+        }
+      }
+    }
+  }
+  }
+  __syncthreads();  // every wave is done with the activations
+  if (staged) {
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+      *reinterpret_cast<f32x4*>(&s_part[(wave * MT + r) * 32 + 8 * g + 4 * h]) = f32x4{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+  }
+  __syncthreads();
+  for (int i = tid; i < MT * 32; i += nthreads) {
+    const int m = i >> 5, n = nb * 32 + (i & 31);
+    if (m < a.M && n < a.N) {
+      float f = 0.f;
+      for (int w = 0; w < nwaves; w++) f += s_part[(w * MT + m) * 32 + (i & 31)];
+      if (a.bias) f += bf16_to_f32(a.bias[n]);
+      a.C[(int64_t)m * a.N + n] = (uint16_t)pack_bf16(f, 0.f);
+    }
+  }
+}
 static int g_w4a16_decode = 1;  // 0: the tile kernels also for a few tokens (comparison runs and tests)
+static int g_w4a16_decode_mfma_from = 2;  // token counts from this one up take the matrix-core form
 static bool launch_w4a16_gemv_packed(const W4A16PArgs& a, hipStream_t st, int* rc) {
-  if (a.M > 4 || !g_w4a16_decode) return false;
-  const int MT = a.M <= 1 ? 1 : (a.M <= 2 ? 2 : 4);
+  if (a.M > 32 || !g_w4a16_decode) return false;
   const int Kp = (int)w4a16_packed_k(a.K), kbs = Kp / 64;
   const int nwaves = kbs >= 32 ? W4G_MAXW : 4;
+  const dim3 grid((unsigned)(w4a16_packed_n(a.N) / 32));
+  if (a.M >= g_w4a16_decode_mfma_from) {
+    // 17 to 32 tokens: every lane reads its own token's activations from LDS, and the tile kernels win where N gives them
+    // enough tiles (9728 x 2560 at 32 tokens: 24 us here, 20 there; 6144 x 2048: 11.6 against 16.9)
+    if (a.M > 16 && a.N > 8192) return false;
+    const int MT = a.M <= 8 ? 8 : (a.M <= 16 ? 16 : 32);
+    const int cap = 152 * 1024 / (MT * 128);  // K blocks of MT tokens in 152 KB
+    const int cb = kbs < cap ? kbs : cap;
+    const size_t x_bytes = (size_t)MT * cb * 128, part_bytes = (size_t)nwaves * MT * 32 * 4;
+    const size_t lds = x_bytes > part_bytes ? x_bytes : part_bytes;
+    auto go = [&](auto kern) {
+      if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return (int)hipGetLastError();
+      hipLaunchKernelGGL(kern, grid, dim3(nwaves * 64), lds, st, a, cb);
+      return (int)hipGetLastError();
+    };
+    *rc = MT == 8 ? go(w4a16_gemv_mfma_packed_kernel<8>) : MT == 16 ? go(w4a16_gemv_mfma_packed_kernel<16>) : go(w4a16_gemv_mfma_packed_kernel<32>);
+    return true;
+  }
+  if (a.M > 4) return false;
+  const int MT = a.M <= 1 ? 1 : (a.M <= 2 ? 2 : 4);
   const size_t lds = (size_t)MT * Kp * 2 + (size_t)nwaves * MT * 32 * 4;
   if (lds > 160 * 1024) return false;
-  const dim3 grid((unsigned)(w4a16_packed_n(a.N) / 32));
   auto go = [&](auto kern) {
     if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return (int)hipGetLastError();
@@ -863,6 +970,11 @@ MLLM_API int mllm_hip_w4a16_set_decode(int gemv) {
   g_w4a16_decode = gemv;
   return 0;
 }
+MLLM_API int mllm_hip_w4a16_set_decode_mfma_from(int tokens) {
+  if (tokens < 1 || tokens > 33) return MLLM_HIP_E_BADARG;
+  g_w4a16_decode_mfma_from = tokens;
+  return 0;
+}
 
 MLLM_API int mllm_hip_w4a16_gemm_packed(const void* a_bf16, const void* packed, const void* bias_bf16, void* c_bf16,
                                         int64_t M, int64_t N, int64_t K, int group, void* stream) {
@@ -875,7 +987,7 @@ MLLM_API int mllm_hip_w4a16_gemm_packed(const void* a_bf16, const void* packed, 
   W4A16PArgs a{(const uint16_t*)a_bf16, (const uint8_t*)packed, (const uint16_t*)bias_bf16, (uint16_t*)c_bf16,
                (int)M, (int)N, (int)K, group};
   int rc = 0;
-  if (launch_w4a16_gemv_packed(a, (hipStream_t)stream, &rc)) return rc;  // up to four tokens
+  if (launch_w4a16_gemv_packed(a, (hipStream_t)stream, &rc)) return rc;  // up to 32 tokens
   return launch_w4a16_nsplit_auto(a, (hipStream_t)stream);
 }
 

@@ -87,6 +87,7 @@ def _cases():
         # switches for comparison runs: anything but 0 and 1 is refused and leaves the setting alone
         "mllm_hip_w8a8_set_decode": ([1], [(0, 2, BADARG), (0, -1, BADARG)]),
         "mllm_hip_w4a16_set_decode": ([1], [(0, 2, BADARG), (0, -1, BADARG)]),
+        "mllm_hip_w4a16_set_decode_mfma_from": ([2], [(0, 0, BADARG), (0, 34, BADARG)]),
         "mllm_hip_moe_gate_set_form": ([1], [(0, 2, BADARG), (0, -1, BADARG)]),
         "mllm_hip_kq_gemm_prepack": ([Q4_K, P, 0, P, 8, 256, None], [(0, Q8_0, BADARG), (1, None, BADARG), (5, 96, SHAPE)]),
         "mllm_hip_linear_kq_gemm": ([Q4_K, P, P, F32, None, P, 16, 8, 256, P, None],

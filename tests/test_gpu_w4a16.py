@@ -104,11 +104,21 @@ def test_gemm_packed_vs_oracle(M, N, K, group):
     assert (diff == 0).mean() > 0.97
 
 
-@pytest.mark.parametrize("M", [1, 2, 3, 4])
-def test_decode_gemv_packed_vs_oracle_and_tiles(M):
-    """up to four tokens take the GEMV kernel (a block row of the packed matrix per workgroup): the oracle within the GEMM's
-    tolerance, nearly every output the tile kernels' bits; ragged N, K not a multiple of 128, groups of 64 / 128 / 256, bias"""
+@pytest.mark.parametrize("M,mfma_from", [(1, 2), (2, 5), (3, 5), (4, 5), (1, 1), (2, 2), (3, 2), (5, 2), (8, 2), (13, 2), (16, 2), (27, 2), (32, 2)])
+def test_decode_gemv_packed_vs_oracle_and_tiles(M, mfma_from):
+    """a few tokens take the GEMV kernels (a block row of the packed matrix per workgroup; fp32 FMAs up to four tokens, the matrix
+    cores from `mfma_from`): the oracle within the GEMM's tolerance, nearly every output the tile kernels' bits; ragged N, K not
+    a multiple of 128, groups of 64 / 128 / 256, bias.  (Where the tokens' activations do not fit LDS the tile kernels run.)"""
     L = _lib.lib()
+    assert L.mllm_hip_w4a16_set_decode_mfma_from(mfma_from) == 0
+    try:
+        _decode_gemv_cases(L, M)
+    finally:
+        assert L.mllm_hip_w4a16_set_decode_mfma_from(2) == 0
+    assert L.mllm_hip_w4a16_set_decode_mfma_from(0) == -1 and L.mllm_hip_w4a16_set_decode_mfma_from(34) == -1
+
+
+def _decode_gemv_cases(L, M):
     for N, K, group in ((9728, 2560, 128), (2560, 9728, 128), (77, 192, 64), (200, 1024, 256), (33, 4096 + 64, 64)):
         rng = synth.rng_for(2, 900 + 3 * M + N + K + group)
         qw, s, zp, _, _ = synth.make_w4a16(rng, N, K, group)
