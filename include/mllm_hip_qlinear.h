@@ -287,10 +287,13 @@ int mllm_hip_w8a8_linear_packed(const void* x, int x_dtype, const void* W_packed
 /* GEMM tile override for tuning sweeps (plain-layout entry points): 0 heuristic, 1 = 256x192, 2 = 128x128, 3 = 64x64
  * workgroup tiles through LDS, 4 = weight operands fetched straight from global memory (K % 128 == 0, else 2). */
 int mllm_hip_w8a8_set_tuning(int tile);
-/* Up to eight tokens against prepacked weights run as a GEMV kernel (one block row of the packed matrix per workgroup, its
- * waves striding over K; same integer sums and epilogue, so the same bits as the tile kernels).  0 keeps the tile kernels
- * also there (comparison runs and tests), 1 restores the default. */
+/* Up to 32 tokens against prepacked weights run as GEMV kernels (one block row of the packed matrix per workgroup, its
+ * waves striding over K; dot instructions up to four tokens, the matrix cores from five, 17 to 32 tokens only where N <= 8192;
+ * same integer sums and epilogue, so the same bits as the tile kernels).  0 keeps the tile kernels also there (comparison runs and tests), 1 restores the default. */
 int mllm_hip_w8a8_set_decode(int gemv);
+/* The token count from which the decode kernels use the matrix cores (1..33, 33 = never: then up to eight tokens take the dot
+ * form; default 5): comparison runs and tests.  No counterpart in the reference. */
+int mllm_hip_w8a8_set_decode_mfma_from(int tokens);
 /* Tile override for the weights-from-global kernel (packed entry points and tile 4 above): 0 heuristic, 1 = 128x384,
  * 2 = 64x384, 3 = 128x128, 4 = 64x128, 5 = 128x256. */
 int mllm_hip_w8a8_nsplit_set_tuning(int tile);

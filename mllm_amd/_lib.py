@@ -77,6 +77,7 @@ def lib():
         L.mllm_hip_moe_gate.argtypes = [vp, ci, vp, vp, vp, vp, i64, i64, i64, ci, ci, vp]
         L.mllm_hip_moe_gate_set_form.argtypes = [ci]
         L.mllm_hip_w8a8_set_decode.argtypes = [ci]
+        L.mllm_hip_w8a8_set_decode_mfma_from.argtypes = [ci]
         L.mllm_hip_w4a16_set_decode.argtypes = [ci]
         L.mllm_hip_w4a16_set_decode_mfma_from.argtypes = [ci]
         L.mllm_hip_quantize_q8_0.argtypes = [vp, ci, vp, vp, i64, i64, vp]

@@ -636,13 +636,111 @@ __global__ __launch_bounds__(W8G_MAXW * 64) void w8a8_gemv_packed_kernel(W8A8Arg
     }
   }
 }
-// false where the kernel above does not apply (more than eight tokens, or rows too long for its LDS)
+// The same walk with the sums on the matrix cores: the 16 bytes a lane holds of a packed block ARE its operand of one
+// v_mfma_i32_32x32x32_i8 (row l % 32, sixteen consecutive k of half l / 32), the other operand the same sixteen k of token
+// l % 32 from LDS (lanes past the MT tokens staged pass zeros): one matrix instruction per block whatever the token count, no
+// vector arithmetic in the loop.  The tokens' codes sit in LDS in runs of cb K blocks (all of them where the rows fit whole).
+// acc[4g + e] = C[token l % 32][row 8g + 4 (l / 32) + e]; integer sums, so the same bits as every other form.
+template <int MT>
+__global__ __launch_bounds__(W8G_MAXW * 64) void w8a8_gemv_mfma_packed_kernel(W8A8Args a, int cb) {
+  extern __shared__ __align__(16) unsigned char smem[];
+  const int Kp = (int)w8a8_packed_k(a.K), kbs = Kp / 32;
+  u32x4* sx = reinterpret_cast<u32x4*>(smem);   // [MT][2 cb] the tokens' codes of the cb blocks in work, zero past K and M
+  int* s_part = reinterpret_cast<int*>(smem);   // [wave][MT][32], after the loop
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nthreads = blockDim.x, nwaves = nthreads >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int nb = blockIdx.x;
+  const u32x4* P = reinterpret_cast<const u32x4*>(a.W) + (size_t)nb * kbs * 64 + lane;
+  constexpr int UB = 8;
+  u32x4 wv[UB];
+  auto load_batch = [&](int kb0, int c1) {
+#pragma unroll
+    for (int u = 0; u < UB; u++) {
+      const int kb = kb0 + u * nwaves;
+      wv[u] = u32x4{0u, 0u, 0u, 0u};
+      if (kb < c1) wv[u] = P[(size_t)kb * 64];
+    }
+  };
+  const int cpr = cb * 2;  // 16-byte pieces per token in LDS
+  v16i acc;
+#pragma unroll
+  for (int j = 0; j < 16; j++) acc[j] = 0;
+  const bool staged = r < MT;
+  const u32x4* sxr = sx + (size_t)(staged ? r : 0) * cpr + h;
+  for (int c0 = 0; c0 < kbs; c0 += cb) {
+    const int c1 = min(c0 + cb, kbs);
+    load_batch(c0 + wave, c1);  // ahead of the copy of the codes
+    if (c0) __syncthreads();    // every wave is done with the previous run's codes
+    for (int i = tid; i < MT * cpr; i += nthreads) {
+      const int m = i / cpr, c = i - m * cpr, gc = c0 * 2 + c;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (m < a.M && gc * 16 < a.K) v = *reinterpret_cast<const u32x4*>(a.A + (size_t)m * a.K + gc * 16);  // K % 16 == 0
+      sx[i] = v;
+    }
+    __syncthreads();
+    for (int kb0 = c0 + wave; kb0 < c1; kb0 += nwaves * UB) {
+      if (kb0 != c0 + wave) load_batch(kb0, c1);
+#pragma unroll
+      for (int u = 0; u < UB; u++) {
+        const int kb = kb0 + u * nwaves;
+        if (kb < c1) {  // uniform
+          u32x4 xv = {0u, 0u, 0u, 0u};
+          if (staged) xv = sxr[(kb - c0) * 2];
+          acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(__builtin_bit_cast(v4i, wv[u]), __builtin_bit_cast(v4i, xv), acc, 0, 0, 0);
+        }
+      }
+    }
+  }
+  __syncthreads();  // every wave is done with the codes
+  if (staged) {
+#pragma unroll
+    for (int g = 0; g < 4; g++)
+      *reinterpret_cast<v4i*>(&s_part[(wave * MT + r) * 32 + 8 * g + 4 * h]) = v4i{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+  }
+  __syncthreads();
+  for (int i = tid; i < MT * 32; i += nthreads) {
+    const int m = i >> 5, n = nb * 32 + (i & 31);
+    if (m < a.M && n < a.N) {
+      int v = 0;
+      for (int w = 0; w < nwaves; w++) v += s_part[(w * MT + m) * 32 + (i & 31)];
+      if (a.acc) a.acc[(int64_t)m * a.N + n] = v;
+      if (a.C) {
+        float f = (float)v * (a.ws[n] * a.xs[m]);
+        if (a.bias) f += a.bias[n];
+        a.C[(int64_t)m * a.N + n] = (uint16_t)pack_bf16(f, 0.f);
+      }
+    }
+  }
+}
+// false where the kernels above do not apply
 static int g_w8a8_decode = 1;  // 0: the tile kernels also for a few tokens (comparison runs and tests)
+static int g_w8a8_decode_mfma_from = 5;  // token counts from this one up take the matrix-core form (two to four: the dot form is
+                                         // faster, 9728 x 2560 at four tokens 11.3 against 12.9 us)
 static bool launch_w8a8_gemv_packed(const W8A8Args& a, hipStream_t st, int* rc) {
-  if (a.M > 8 || !g_w8a8_decode) return false;
-  const int MT = a.M <= 1 ? 1 : (a.M <= 2 ? 2 : (a.M <= 4 ? 4 : 8));
+  if (a.M > 32 || !g_w8a8_decode) return false;
   const int Kp = (int)w8a8_packed_k(a.K), kbs = Kp / 32;
   const int nwaves = kbs >= 32 ? W8G_MAXW : 4;
+  if (a.M >= g_w8a8_decode_mfma_from) {
+    // 17 to 32 tokens: every lane reads its own token's codes from LDS, and the tile kernels win where N gives them enough
+    // tiles (9728 x 2560 at 32 tokens: 21.6 us here, 17.1 there; 2560 x 9728: 28.4 against 43.5)
+    if (a.M > 16 && a.N > 8192) return false;
+    const int MT = a.M <= 8 ? 8 : (a.M <= 16 ? 16 : 32);
+    const int cap = 152 * 1024 / (MT * 32);  // K blocks of MT tokens in 152 KB
+    const int cb = kbs < cap ? kbs : cap;
+    const size_t x_bytes = (size_t)MT * cb * 32, part_bytes = (size_t)nwaves * MT * 32 * 4;
+    const size_t lds = x_bytes > part_bytes ? x_bytes : part_bytes;
+    const dim3 grid((unsigned)(w8a8_packed_n(a.N) / 32));
+    auto go = [&](auto kern) {
+      if (lds > 64 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+        return (int)hipGetLastError();
+      hipLaunchKernelGGL(kern, grid, dim3(nwaves * 64), lds, st, a, cb);
+      return (int)hipGetLastError();
+    };
+    *rc = MT == 8 ? go(w8a8_gemv_mfma_packed_kernel<8>) : MT == 16 ? go(w8a8_gemv_mfma_packed_kernel<16>) : go(w8a8_gemv_mfma_packed_kernel<32>);
+    return true;
+  }
+  if (a.M > 8) return false;
+  const int MT = a.M <= 1 ? 1 : (a.M <= 2 ? 2 : (a.M <= 4 ? 4 : 8));
   const size_t lds = (size_t)MT * Kp + (size_t)nwaves * MT * 32 * 4;
   if (lds > 160 * 1024) return false;
   const dim3 grid((unsigned)(w8a8_packed_n(a.N) / 32));
@@ -658,6 +756,11 @@ static bool launch_w8a8_gemv_packed(const W8A8Args& a, hipStream_t st, int* rc) 
 MLLM_API int mllm_hip_w8a8_set_decode(int gemv) {
   if (gemv != 0 && gemv != 1) return MLLM_HIP_E_BADARG;
   g_w8a8_decode = gemv;
+  return 0;
+}
+MLLM_API int mllm_hip_w8a8_set_decode_mfma_from(int tokens) {
+  if (tokens < 1 || tokens > 33) return MLLM_HIP_E_BADARG;
+  g_w8a8_decode_mfma_from = tokens;
   return 0;
 }
 
@@ -742,7 +845,7 @@ MLLM_API int mllm_hip_w8a8_gemm_packed(const int8_t* xq, const float* x_scale, c
   if (reinterpret_cast<uintptr_t>(xq) % 16 || reinterpret_cast<uintptr_t>(W_packed) % 16) return MLLM_HIP_E_ALIGN;
   W8A8Args a{xq, reinterpret_cast<const int8_t*>(W_packed), x_scale, w_scale, bias, (uint16_t*)out_bf16, acc_out, (int)M, (int)N, (int)K};
   int rc = 0;
-  if (launch_w8a8_gemv_packed(a, (hipStream_t)stream, &rc)) return rc;  // up to eight tokens
+  if (launch_w8a8_gemv_packed(a, (hipStream_t)stream, &rc)) return rc;  // up to 32 tokens
   return launch_w8a8_nsplit_auto<true>(a, (hipStream_t)stream);
 }
 

@@ -86,6 +86,7 @@ def _cases():
         "mllm_hip_kq_set_slice_meeting": ([-1, 0], [(0, 2, BADARG), (0, -2, BADARG), (1, 9, BADARG), (1, -1, BADARG)]),
         # switches for comparison runs: anything but 0 and 1 is refused and leaves the setting alone
         "mllm_hip_w8a8_set_decode": ([1], [(0, 2, BADARG), (0, -1, BADARG)]),
+        "mllm_hip_w8a8_set_decode_mfma_from": ([5], [(0, 0, BADARG), (0, 34, BADARG)]),
         "mllm_hip_w4a16_set_decode": ([1], [(0, 2, BADARG), (0, -1, BADARG)]),
         "mllm_hip_w4a16_set_decode_mfma_from": ([2], [(0, 0, BADARG), (0, 34, BADARG)]),
         "mllm_hip_moe_gate_set_form": ([1], [(0, 2, BADARG), (0, -1, BADARG)]),

@@ -110,11 +110,22 @@ def test_gemm_packed_bit_exact(M, N, K):
     assert np.array_equal(_bits(yb), wyb)
 
 
-@pytest.mark.parametrize("M", [1, 2, 3, 5, 8])
-def test_decode_gemv_packed_bit_exact(M):
-    """up to eight tokens take the GEMV kernel (a block row of the packed matrix per workgroup): the oracle's bits, and the tile
-    kernels' bits; ragged N and K (zero padding of the packed layout), long rows, bias"""
+@pytest.mark.parametrize("M,mfma_from", [(1, 5), (2, 5), (3, 5), (5, 33), (8, 33), (1, 1), (2, 2), (3, 2), (5, 5), (8, 5), (13, 5), (16, 5),
+                                         (27, 5), (32, 5)])
+def test_decode_gemv_packed_bit_exact(M, mfma_from):
+    """up to 32 tokens take the GEMV kernels (a block row of the packed matrix per workgroup; dot instructions, or the matrix
+    cores from `mfma_from` tokens): the oracle's bits, and the tile kernels' bits; ragged N and K (zero padding of the packed
+    layout), rows long enough to pass through LDS in several runs, bias"""
     L = _lib.lib()
+    assert L.mllm_hip_w8a8_set_decode_mfma_from(mfma_from) == 0
+    try:
+        _decode_gemv_cases(L, M)
+    finally:
+        assert L.mllm_hip_w8a8_set_decode_mfma_from(5) == 0
+    assert L.mllm_hip_w8a8_set_decode_mfma_from(0) == -1 and L.mllm_hip_w8a8_set_decode_mfma_from(34) == -1
+
+
+def _decode_gemv_cases(L, M):
     for N, K in ((9728, 2560), (2560, 9728), (77, 48), (200, 144), (33, 4096 + 16)):
         rng = synth.rng_for(3, 700 + M * 11 + N + K)
         xq = rng.integers(-127, 128, (M, K), dtype=np.int8)
