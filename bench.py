@@ -339,7 +339,7 @@ def side_workloads(torch, ql, synth, gen, brief=False):
         zp = torch.randint(0, 256, (n_, k_ // 256), dtype=torch.uint8, device="cuda", generator=gen)
         Wp4 = [ql.w4a16_prepack(torch.randint(0, 256, (n_, k_ // 2), dtype=torch.uint8, device="cuda", generator=gen), s4, zp, 128)
                for _ in range(4)]
-        for m_ in (1, 4):
+        for m_ in (1, 4, 8, 16):
             a_ = torch.randn((m_, k_), device="cuda", generator=gen).to(torch.bfloat16)
             y_ = torch.empty((m_, n_), dtype=torch.bfloat16, device="cuda")
             wq = torch.empty(_lib_ws(ql, "w8a8", m_, k_), dtype=torch.uint8, device="cuda")
