@@ -313,6 +313,44 @@ __global__ __launch_bounds__(SOFTMAX_WG) void softmax_long_rows_kernel(const flo
   }
 }
 
+// Rows between the two (2049 to 16 384 elements: the keys of an attention row): a workgroup of four waves per row, the row in
+// registers (16, 32 or 64 elements per thread), one pass over memory; maxima and sums meet in LDS.
+template <int R>
+__global__ __launch_bounds__(256) void softmax_wg_rows_kernel(const float* __restrict__ x, float* __restrict__ y, int len, int exp_accurate) {
+  __shared__ float s_red[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const float* xr = x + (int64_t)blockIdx.x * len;
+  float* yr = y + (int64_t)blockIdx.x * len;
+  const bool poly = !exp_accurate;
+  float v[R];
+#pragma unroll
+  for (int j = 0; j < R; j++) v[j] = tid + 256 * j < len ? xr[tid + 256 * j] : -3.402823466e+38f;
+  float mx = v[0];
+#pragma unroll
+  for (int j = 1; j < R; j++) mx = fmaxf(mx, v[j]);
+  mx = wave_max(mx);
+  if (lane == 0) s_red[wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+  __syncthreads();
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < R; j++) {
+    const int i = tid + 256 * j;
+    if (i < len) {
+      v[j] = softmax_exp(v[j] - mx, poly && i < (len & ~7));
+      sum += v[j];
+    }
+  }
+  sum = wave_sum(sum);
+  if (lane == 0) s_red[wave] = sum;
+  __syncthreads();
+  const float inv = 1.f / (((s_red[0] + s_red[1]) + s_red[2]) + s_red[3]);
+#pragma unroll
+  for (int j = 0; j < R; j++)
+    if (tid + 256 * j < len) yr[tid + 256 * j] = v[j] * inv;
+}
+
 // ---- top-k over the last axis, one wave per row -------------------------------------------------------------------------
 // Selection by repeated wave-wide extreme: round r takes the best element that comes after the one taken in round r-1
 // in the order (value descending [ascending for smallest], index ascending).  Equal values are taken lowest index
@@ -955,6 +993,9 @@ MLLM_API int mllm_hip_softmax(const float* x, float* y, int64_t rows, int64_t le
   if (len <= 256) hipLaunchKernelGGL(softmax_rows_reg_kernel<4>, grid4, dim3(256), 0, st, x, y, rows, (int)len, g_exp_accurate);
   else if (len <= 1024) hipLaunchKernelGGL(softmax_rows_reg_kernel<16>, grid4, dim3(256), 0, st, x, y, rows, (int)len, g_exp_accurate);
   else if (len <= 2048) hipLaunchKernelGGL(softmax_rows_reg_kernel<32>, grid4, dim3(256), 0, st, x, y, rows, (int)len, g_exp_accurate);
+  else if (len <= 4096 && rows <= 0x7fffffff) hipLaunchKernelGGL(softmax_wg_rows_kernel<16>, dim3((unsigned)rows), dim3(256), 0, st, x, y, (int)len, g_exp_accurate);
+  else if (len <= 8192 && rows <= 0x7fffffff) hipLaunchKernelGGL(softmax_wg_rows_kernel<32>, dim3((unsigned)rows), dim3(256), 0, st, x, y, (int)len, g_exp_accurate);
+  else if (len <= 16384 && rows <= 0x7fffffff) hipLaunchKernelGGL(softmax_wg_rows_kernel<64>, dim3((unsigned)rows), dim3(256), 0, st, x, y, (int)len, g_exp_accurate);
   else if (len >= 16384 && rows <= 0x7fffffff) hipLaunchKernelGGL(softmax_long_rows_kernel, dim3((unsigned)rows), dim3(SOFTMAX_WG), 0, st, x, y, (int)len, g_exp_accurate);
   else hipLaunchKernelGGL(softmax_rows_kernel, grid4, dim3(256), 0, st, x, y, rows, (int)len, g_exp_accurate);
   return (int)hipGetLastError();

@@ -231,14 +231,16 @@ def test_mlp_gate_up_one_launch(wtype, M, H, I):
     assert rel_l2(ha.cpu().numpy(), g64 / (1 + np.exp(-g64)) * u64) < 1e-5
 
 
-@pytest.mark.parametrize("rows,n", [(1, 128), (512, 128), (5, 16), (7, 13), (3, 1000), (9, 60)])
+@pytest.mark.parametrize("rows,n", [(1, 128), (512, 128), (5, 16), (7, 13), (3, 1000), (9, 60), (3, 2048), (5, 2049), (3, 4099), (2, 8192),
+                                    (3, 12003), (2, 16384), (2, 16391), (1, 40003)])
 def test_softmax(rows, n):
     rng = synth.rng_for(6, 4000 + rows + n)
     x = (rng.standard_normal((rows, n)) * 3).astype(np.float32)
     announce("softmax", rows, n)
     y = ql.softmax(to_dev(x)).cpu().numpy()
     want = orc.softmax(x)
-    assert rel_l2(y, want) < 2e-6
+    # (the oracle adds a row's terms one after another in fp32: over tens of thousands of terms its own sum is the less exact one)
+    assert rel_l2(y, want) < (2e-6 if n <= 16384 else 4e-6)
     assert np.allclose(y.sum(-1), 1.0, atol=1e-5)
 
 
